@@ -1,0 +1,106 @@
+/* zkllm_hip.h -- C ABI of the MI355X (gfx950) prover kernels.
+ *
+ * This is the boundary a host program binds to (the C++ class layer in
+ * zkllm-ccs2024_amd/host does; so do the ctypes tests).  Plain pointers and sizes only.
+ *
+ * Conventions
+ *   - Every function returns 0 on success, a hipError_t value or a code >= 10001 otherwise;
+ *     zk_last_error() returns the message of the calling thread's last failure.  Nothing throws.
+ *   - Pointers named out/a/b/in/table/... are DEVICE pointers unless the name ends in _host
+ *     or the parameter is a `const uint32_t*` scalar/challenge (8 limbs per Fr, host memory).
+ *   - Fr element: 8 little-endian u32 limbs, 32 bytes, standard (non-Montgomery) form -- the
+ *     reference's Fr_t as stored by FrTensor (fr-tensor.cuh:15, fr-tensor.cu:181-184).
+ *   - G1 point: Jacobian (x,y,z), 3 x 12 u32 limbs, Montgomery form, 144 bytes -- the reference's
+ *     G1Jacobian_t as stored by G1TensorJacobian (bls12-381.cuh:429-433, g1-tensor.cu:174-183).
+ *     Any z == 0 is the point at infinity.
+ *   - `stream` is a hipStream_t passed as void* (NULL = default stream).  Launches are
+ *     asynchronous; functions that return host values synchronise that stream.
+ *   - Scratch memory comes from the library's caching allocator (zk_malloc/zk_free); all work
+ *     is expected on one stream at a time.
+ */
+#ifndef ZKLLM_HIP_H
+#define ZKLLM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- runtime ------------------------------------------------------------------------------- */
+const char* zk_last_error(void);
+int zk_init(int device);                                   /* hipSetDevice; fails if no GPU */
+int zk_device_info(char* name, int name_len, int* compute_units, int* clock_khz, size_t* total_mem);
+/* replaces the cudaMalloc/cudaFree pair of every FrTensor/G1Tensor ctor/dtor (fr-tensor.cu:158-179) */
+int zk_malloc(void** out, size_t bytes);
+int zk_free(void* p);
+int zk_pool_trim(void);                                    /* return cached blocks to the driver */
+int zk_pool_stats(size_t* live_bytes, size_t* cached_bytes);
+/* replace cudaMemcpy in ctors, operator()(idx), savebin/loadbin (ioutils.cu:3-45) */
+int zk_memcpy_h2d(void* dst, const void* src_host, size_t bytes, void* stream);
+int zk_memcpy_d2h(void* dst_host, const void* src, size_t bytes, void* stream);
+int zk_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream);
+int zk_memset(void* dst, int value, size_t bytes, void* stream);
+int zk_sync(void* stream);
+int zk_event_create(void** ev);
+int zk_event_destroy(void* ev);
+int zk_event_record(void* ev, void* stream);
+int zk_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* ---- Fr elementwise (Fr_elementwise_* / Fr_broadcast_*, fr-tensor.cu:71-153, :257-373) ------- */
+int zk_fr_add(void* out, const void* a, const void* b, size_t n, void* stream);
+int zk_fr_sub(void* out, const void* a, const void* b, size_t n, void* stream);
+int zk_fr_mul(void* out, const void* a, const void* b, size_t n, void* stream);       /* a*b (Fr_elementwise_mul) */
+int zk_fr_montmul(void* out, const void* a, const void* b, size_t n, void* stream);   /* a*b*R^-1 (Fr_elementwise_mont_mul) */
+int zk_fr_neg(void* out, const void* a, size_t n, void* stream);
+int zk_fr_add_s(void* out, const void* a, const uint32_t* s, size_t n, void* stream);
+int zk_fr_sub_s(void* out, const void* a, const uint32_t* s, size_t n, void* stream);
+int zk_fr_mul_s(void* out, const void* a, const uint32_t* s, size_t n, void* stream);
+int zk_fr_mont(void* out, const void* a, size_t n, void* stream);                     /* a*R  */
+int zk_fr_unmont(void* out, const void* a, size_t n, void* stream);                   /* a/R  */
+int zk_fr_fill(void* out, const uint32_t* s, size_t n, void* stream);
+int zk_fr_bias_add(void* z, const void* bias, size_t rows, uint32_t cols, void* stream);   /* fcAddBiasKernel zkfc.cu:36-41 */
+
+/* ---- conversions (fr-tensor.cu:186-248, :691-798, :922-945) ------------------------------------ */
+int zk_fr_from_i32(void* out, const void* in_i32, size_t n, void* stream);
+int zk_fr_from_i64(void* out, const void* in_i64, size_t n, void* stream);
+int zk_fr_from_u32(void* out, const void* in_u32, size_t n, void* stream);             /* count_to_m tlookup.cu:17-20 */
+int zk_fr_from_f32(void* out, const void* in_f32, uint64_t scaling_factor, size_t n, void* stream);
+int zk_fr_from_f64(void* out, const void* in_f64, uint64_t scaling_factor, size_t n, void* stream);
+int zk_fr_to_i32(void* out_i32, const void* in, size_t n, void* stream);
+int zk_fr_to_i64(void* out_i64, const void* in, size_t n, void* stream);
+
+/* ---- layout (pad fr-tensor.cu:800-828, transpose :885-900, gather tlookup.cu:446-453) ----------- */
+int zk_fr_pad(void* out, const void* in, size_t rows, uint32_t last_in, uint32_t last_out, const uint32_t* pad, void* stream);
+int zk_fr_transpose(void* out, const void* in, uint32_t M, uint32_t N, void* stream);
+int zk_fr_gather(void* out, const void* table, const void* idx_u32, size_t n, void* stream);
+
+/* ---- reductions and folds ------------------------------------------------------------------------ */
+/* FrTensor::sum (fr-tensor.cu:382-434) */
+int zk_fr_sum(uint32_t* out_host, const void* a, size_t n, void* stream);
+/* sum_i a_i*b_i; replaces (a*b).sum() at tlookup.cu:360 */
+int zk_fr_dot(uint32_t* out_host, const void* a, const void* b, size_t n, void* stream);
+/* 1..3 levels of Fr_multi_dim_partial_me_step / Fr_me_step / Fr_partial_me_step in one pass over
+ * in[other][cur][window] (fr-tensor.cu:518-560, :588-641).  u: `levels` standard-form challenges. */
+int zk_fr_fold_axis(void* out, const void* in, const uint32_t* u, int levels, size_t other, uint32_t cur, size_t window, void* stream);
+/* FrTensor::operator()(u) / Fr_me (fr-tensor.cu:437-442, :602-609): whole evaluation, fused */
+int zk_fr_me(uint32_t* out_host, const void* a, size_t n, const uint32_t* u, int k, void* stream);
+/* zkip_reduce_kernel / tLookup reduce kernels / hadamard_reduce_kernel on one tensor */
+int zk_fr_fold_halves(void* out, const void* a, const uint32_t* v, size_t n_in, size_t n_out, void* stream);
+
+/* ---- matmul (matrixMultiplyOptimized fr-tensor.cu:831-881) ---------------------------------------- */
+int zk_fr_matmul_generic(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, void* stream);
+/* mode 0: pick the small-integer path when a device-side bound check proves it exact; 1: generic
+ * Montgomery only; 2: small-integer only (error if the bound fails).  path_used: 1 generic, 2 small-int. */
+int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used_host, void* stream);
+
+/* ---- inner-product sumcheck (zkip_poly_kernel + 3 sums, zkfc.cu:94-138) ----------------------------- */
+int zk_ip_round(uint32_t* poly3_host, const void* a, const void* b, size_t n_in, size_t n_out, void* stream);
+/* all rounds of zkip (zkfc.cu:140-151) in one launch, n <= 8192 */
+int zk_ip_sumcheck_small(uint32_t* polys_host, uint32_t* fin_host, const void* a, const void* b, uint32_t n, const uint32_t* u, int k, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,257 @@
+"""ctypes front-ends of the product libraries for tests, smoke and bench.
+
+Hip     raw C ABI (include/zkllm_hip.h): device buffers are plain integers (addresses)
+Prover  class-layer harness (zkp_* in libzkllm_prover.so): tensors are opaque handles
+Both fail loudly when the libraries are missing or no GPU is visible; neither has a CPU path.
+"""
+import ctypes
+import importlib
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+pkg = importlib.import_module("zkllm-ccs2024_amd")
+
+c_void_p, c_size_t, c_int, c_uint, c_u64 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint64
+
+
+def _np_ptr(a):
+    assert isinstance(a, np.ndarray) and a.flags["C_CONTIGUOUS"]
+    return c_void_p(a.ctypes.data)
+
+
+class Hip:
+    def __init__(self, device=0):
+        self.lib = pkg.load_hip()
+        self.check(self.lib.zk_init(c_int(device)))
+
+    def check(self, rc):
+        if rc != 0:
+            raise RuntimeError(f"zk error {rc}: {self.lib.zk_last_error().decode()}")
+
+    # ---- memory ----
+    def malloc(self, nbytes):
+        p = c_void_p()
+        self.check(self.lib.zk_malloc(ctypes.byref(p), c_size_t(nbytes)))
+        return p.value
+
+    def free(self, p):
+        self.check(self.lib.zk_free(c_void_p(p)))
+
+    def upload(self, arr):
+        arr = np.ascontiguousarray(arr)
+        p = self.malloc(max(arr.nbytes, 1))
+        self.check(self.lib.zk_memcpy_h2d(c_void_p(p), _np_ptr(arr), c_size_t(arr.nbytes), None))
+        return p
+
+    def download(self, p, shape, dtype):
+        out = np.zeros(shape, dtype=dtype)
+        self.check(self.lib.zk_memcpy_d2h(_np_ptr(out), c_void_p(p), c_size_t(out.nbytes), None))
+        return out
+
+    def sync(self):
+        self.check(self.lib.zk_sync(None))
+
+    # ---- generic call: device addresses as ints, numpy arrays as host pointers ----
+    def call(self, name, *args):
+        fn = getattr(self.lib, name)
+        conv = []
+        for a in args:
+            if isinstance(a, np.ndarray):
+                conv.append(_np_ptr(a))
+            elif a is None:
+                conv.append(c_void_p(None))
+            elif isinstance(a, (ctypes._SimpleCData, ctypes._Pointer)) or type(a).__name__ == "CArgObject":
+                conv.append(a)
+            else:
+                conv.append(a)
+        self.check(fn(*conv))
+
+    def fr_binary(self, name, a, b):
+        n = a.shape[0]
+        da, db, do = self.upload(a), self.upload(b), self.malloc(32 * max(n, 1))
+        self.call(name, c_void_p(do), c_void_p(da), c_void_p(db), c_size_t(n), None)
+        out = self.download(do, (n, 8), np.uint32)
+        for p in (da, db, do):
+            self.free(p)
+        return out
+
+    def fr_unary(self, name, a):
+        n = a.shape[0]
+        da, do = self.upload(a), self.malloc(32 * max(n, 1))
+        self.call(name, c_void_p(do), c_void_p(da), c_size_t(n), None)
+        out = self.download(do, (n, 8), np.uint32)
+        self.free(da)
+        self.free(do)
+        return out
+
+    def fr_scalar(self, name, a, s):
+        n = a.shape[0]
+        da, do = self.upload(a), self.malloc(32 * max(n, 1))
+        s = np.ascontiguousarray(s, dtype=np.uint32)
+        self.call(name, c_void_p(do), c_void_p(da), s, c_size_t(n), None)
+        out = self.download(do, (n, 8), np.uint32)
+        self.free(da)
+        self.free(do)
+        return out
+
+
+class FrHandle:
+    def __init__(self, pv, h):
+        if not h:
+            raise RuntimeError("prover error: " + pv.lib.zkp_last_error().decode())
+        self.pv, self.h = pv, h
+
+    @property
+    def size(self):
+        return self.pv.lib.zkp_fr_size(c_void_p(self.h))
+
+    @property
+    def devptr(self):
+        return self.pv.lib.zkp_fr_devptr(c_void_p(self.h))
+
+    def host(self):
+        out = np.zeros((self.size, 8), dtype=np.uint32)
+        self.pv.check(self.pv.lib.zkp_fr_to_host(c_void_p(self.h), _np_ptr(out)))
+        return out
+
+    def __del__(self):
+        try:
+            self.pv.lib.zkp_fr_free(c_void_p(self.h))
+        except Exception:
+            pass
+
+
+class Prover:
+    def __init__(self, device=0):
+        self.lib = pkg.load_prover()
+        L = self.lib
+        for name in ("zkp_fr_from_i32", "zkp_fr_from_i64", "zkp_fr_from_fr", "zkp_fr_from_f32", "zkp_fr_from_f64", "zkp_fr_from_file",
+                     "zkp_fr_devptr", "zkp_fr_binop", "zkp_fr_scalarop", "zkp_fr_partial_me", "zkp_fr_partial_me_window",
+                     "zkp_fr_pad", "zkp_fr_transpose", "zkp_fr_matmul"):
+            getattr(L, name).restype = c_void_p
+        L.zkp_transcript_size.restype = ctypes.c_long
+        L.zkp_fr_size.restype = c_uint
+        self.check(L.zkp_init(c_int(device)))
+
+    def check(self, rc):
+        if rc != 0:
+            raise RuntimeError("prover error: " + self.lib.zkp_last_error().decode())
+
+    def H(self, h):
+        return FrHandle(self, h)
+
+    # ---- tensors ----
+    def from_i32(self, a):
+        a = np.ascontiguousarray(a, dtype=np.int32)
+        return self.H(self.lib.zkp_fr_from_i32(_np_ptr(a), c_uint(a.size)))
+
+    def from_i64(self, a):
+        a = np.ascontiguousarray(a, dtype=np.int64)
+        return self.H(self.lib.zkp_fr_from_i64(_np_ptr(a), c_uint(a.size)))
+
+    def from_fr(self, a):
+        a = np.ascontiguousarray(a, dtype=np.uint32).reshape(-1, 8)
+        return self.H(self.lib.zkp_fr_from_fr(_np_ptr(a), c_uint(a.shape[0])))
+
+    def from_f32(self, a, sf):
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        return self.H(self.lib.zkp_fr_from_f32(_np_ptr(a), c_uint(a.size), c_u64(sf)))
+
+    def from_f64(self, a, sf):
+        a = np.ascontiguousarray(a, dtype=np.float64)
+        return self.H(self.lib.zkp_fr_from_f64(_np_ptr(a), c_uint(a.size), c_u64(sf)))
+
+    def binop(self, op, a, b):
+        return self.H(self.lib.zkp_fr_binop(c_int(op), c_void_p(a.h), c_void_p(b.h)))
+
+    def scalarop(self, op, a, s=None):
+        s = np.zeros(8, np.uint32) if s is None else np.ascontiguousarray(s, dtype=np.uint32)
+        return self.H(self.lib.zkp_fr_scalarop(c_int(op), c_void_p(a.h), _np_ptr(s)))
+
+    def sum(self, a):
+        out = np.zeros(8, np.uint32)
+        self.check(self.lib.zkp_fr_sum(c_void_p(a.h), _np_ptr(out)))
+        return out
+
+    def me(self, a, u):
+        u = np.ascontiguousarray(u, dtype=np.uint32).reshape(-1, 8)
+        out = np.zeros(8, np.uint32)
+        self.check(self.lib.zkp_fr_me(c_void_p(a.h), _np_ptr(u), c_int(u.shape[0]), _np_ptr(out)))
+        return out
+
+    def partial_me(self, a, u, cur_dim, window):
+        u = np.ascontiguousarray(u, dtype=np.uint32).reshape(-1, 8)
+        return self.H(self.lib.zkp_fr_partial_me(c_void_p(a.h), _np_ptr(u), c_int(u.shape[0]), c_uint(cur_dim), c_uint(window)))
+
+    def partial_me_window(self, a, u, window):
+        u = np.ascontiguousarray(u, dtype=np.uint32).reshape(-1, 8)
+        return self.H(self.lib.zkp_fr_partial_me_window(c_void_p(a.h), _np_ptr(u), c_int(u.shape[0]), c_uint(window)))
+
+    def multi_dim_me(self, a, us, shape):
+        cat = np.ascontiguousarray(np.concatenate([np.asarray(u, dtype=np.uint32).reshape(-1, 8) for u in us]) if us else np.zeros((0, 8), np.uint32))
+        lens = np.array([np.asarray(u).reshape(-1, 8).shape[0] for u in us], dtype=np.uint32)
+        shp = np.array(shape, dtype=np.uint32)
+        out = np.zeros(8, np.uint32)
+        self.check(self.lib.zkp_fr_multi_dim_me(c_void_p(a.h), _np_ptr(cat), _np_ptr(lens), _np_ptr(shp), c_int(len(shape)), _np_ptr(out)))
+        return out
+
+    def pad(self, a, shape, pad_val=None):
+        pv = np.zeros(8, np.uint32) if pad_val is None else np.ascontiguousarray(pad_val, dtype=np.uint32)
+        shp = np.array(shape, dtype=np.uint32)
+        return self.H(self.lib.zkp_fr_pad(c_void_p(a.h), _np_ptr(shp), c_int(len(shape)), _np_ptr(pv)))
+
+    def transpose(self, a, M, N):
+        return self.H(self.lib.zkp_fr_transpose(c_void_p(a.h), c_uint(M), c_uint(N)))
+
+    def matmul(self, a, b, M, N, P):
+        return self.H(self.lib.zkp_fr_matmul(c_void_p(a.h), c_void_p(b.h), c_uint(M), c_uint(N), c_uint(P)))
+
+    # ---- transcript / challenges ----
+    def seed(self, s):
+        self.lib.zkp_seed(c_uint(s))
+
+    def transcript_begin(self):
+        self.lib.zkp_transcript_begin()
+
+    def transcript(self):
+        n = self.lib.zkp_transcript_size()
+        out = np.zeros((n, 8), dtype=np.uint32)
+        if n:
+            self.lib.zkp_transcript_get(_np_ptr(out))
+        return out
+
+    def sync(self):
+        self.check(self.lib.zkp_sync())
+
+    # ---- protocols ----
+    def zkip(self, claim, a, b, u):
+        u = np.ascontiguousarray(u, dtype=np.uint32).reshape(-1, 8)
+        k = u.shape[0]
+        proof = np.zeros((k, 3, 8), np.uint32)
+        fin = np.zeros(8, np.uint32)
+        claim = np.ascontiguousarray(claim, dtype=np.uint32)
+        self.check(self.lib.zkp_zkip(_np_ptr(claim), c_void_p(a.h), c_void_p(b.h), _np_ptr(u), c_int(k), _np_ptr(proof), _np_ptr(fin)))
+        return proof, fin
+
+    def zkfc_prove(self, X, W, Y, in_dim, out_dim):
+        cw = np.zeros(8, np.uint32)
+        self.check(self.lib.zkp_zkfc_prove(c_void_p(X.h), c_void_p(W.h), c_void_p(Y.h), c_uint(in_dim), c_uint(out_dim), _np_ptr(cw)))
+        return cw
+
+    def zkfc_scenario(self, X, W, seed, matmul_mode=0):
+        """forward + prove on int32 inputs; returns (Y as Fr limbs, transcript)"""
+        B, I = X.shape
+        O = W.shape[1]
+        self.lib.zkp_set_matmul_mode(c_int(matmul_mode))
+        hX, hW = self.from_i32(X), self.from_i32(W)
+        hY = self.matmul(hX, hW, B, I, O)
+        self.seed(seed)
+        self.transcript_begin()
+        self.zkfc_prove(hX, hW, hY, I, O)
+        self.lib.zkp_transcript_end()
+        return hY.host(), self.transcript()

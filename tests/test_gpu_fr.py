@@ -1,0 +1,270 @@
+"""GPU parity: FrTensor kernels, folds, matmul, inner-product sumcheck and zkFC::prove, through the
+C ABI / class layer, bit-exact against the CPU oracle on the same seeded inputs."""
+import ctypes
+import random
+
+import numpy as np
+import pytest
+
+from zkhelp import FR_R, R_MOD, fr_array, fr_ints, load_oracle, me_bruteforce, mt_random_vec, orc_check, orc_transcript
+
+pytestmark = pytest.mark.gpu
+
+EDGE = [0, 1, 2, R_MOD - 1, R_MOD - 2, FR_R, FR_R * FR_R % R_MOD, (1 << 32) - 1, ((1 << 32) - 1) << 32,
+        (1944954706 << 224) | ((1 << 224) - 1), 1 << 254, R_MOD >> 1]
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from gpuhelp import Hip
+    return Hip()
+
+
+@pytest.fixture(scope="module")
+def pv():
+    from gpuhelp import Prover
+    return Prover()
+
+
+@pytest.fixture(scope="module")
+def orc():
+    return load_oracle()
+
+
+def seeded(n, seed):
+    """n field elements from the seeded challenge generator (plus the edge set in front)"""
+    raw = mt_random_vec(np.random.RandomState(seed), n)
+    return np.concatenate([fr_array(EDGE), raw])
+
+
+def test_elementwise_ops_bit_exact(hip, orc):
+    n = 1 << 16
+    A, B = seeded(n, 1), seeded(n, 2)[::-1].copy()
+    N = A.shape[0]
+    exp = np.zeros_like(A)
+    for name, op in (("zk_fr_add", 0), ("zk_fr_sub", 1), ("zk_fr_montmul", 2), ("zk_fr_mul", 7)):
+        print("case", name, flush=True)
+        got = hip.fr_binary(name, A, B)
+        orc_check(orc.orc_fr_op(op, A, B, exp, N))
+        assert (got == exp).all(), name
+    for name, op in (("zk_fr_neg", 9), ("zk_fr_mont", 4), ("zk_fr_unmont", 5)):
+        print("case", name, flush=True)
+        got = hip.fr_unary(name, A)
+        orc_check(orc.orc_fr_op(op, A, A, exp, N))
+        assert (got == exp).all(), name
+    s = fr_array([R_MOD - 12345])[0]
+    S = np.tile(s, (N, 1))
+    for name, op in (("zk_fr_add_s", 0), ("zk_fr_sub_s", 1), ("zk_fr_mul_s", 7)):
+        print("case", name, flush=True)
+        got = hip.fr_scalar(name, A, s)
+        orc_check(orc.orc_fr_op(op, A, S, exp, N))
+        assert (got == exp).all(), name
+
+
+def test_empty_and_single_element(hip, pv):
+    empty = np.zeros((0, 8), np.uint32)
+    assert hip.fr_binary("zk_fr_add", empty, empty).shape == (0, 8)
+    one = fr_array([5])
+    assert fr_ints(hip.fr_binary("zk_fr_mul", one, fr_array([7]))) == [35]
+    h = pv.from_fr(one)
+    assert fr_ints(pv.sum(h)) == [5]
+    assert fr_ints(pv.me(h, np.zeros((0, 8), np.uint32))) == [5]
+
+
+def test_conversions(hip, pv, orc):
+    xs = np.array([0, 1, -1, 2 ** 15, -(2 ** 15), 2 ** 31 - 1, -(2 ** 31) + 1] + list(np.random.default_rng(3).integers(-2 ** 31 + 1, 2 ** 31 - 1, 1000)), dtype=np.int32)
+    h = pv.from_i32(xs)
+    assert fr_ints(h.host()) == [int(x) % R_MOD for x in xs]
+    ls = np.array([0, 1, -1, 2 ** 40, -(2 ** 40), 2 ** 62, -(2 ** 62)] + list(np.random.default_rng(4).integers(-2 ** 62, 2 ** 62, 1000)), dtype=np.int64)
+    hl = pv.from_i64(ls)
+    assert fr_ints(hl.host()) == [int(x) % R_MOD for x in ls]
+    # back to integers through the C ABI
+    from gpuhelp import c_void_p, c_size_t
+    d = hip.malloc(4 * len(xs))
+    hip.call("zk_fr_to_i32", c_void_p(d), c_void_p(h.devptr), c_size_t(len(xs)), None)
+    assert (hip.download(d, (len(xs),), np.int32) == xs).all()
+    hip.free(d)
+    d = hip.malloc(8 * len(ls))
+    hip.call("zk_fr_to_i64", c_void_p(d), c_void_p(hl.devptr), c_size_t(len(ls)), None)
+    assert (hip.download(d, (len(ls),), np.int64) == ls).all()
+    hip.free(d)
+    fl = np.random.default_rng(5).normal(0, 0.02, 4096)
+    fl[:6] = [0.0, 0.5 / 65536, -0.5 / 65536, 1.5 / 65536, -1.5 / 65536, 0.49999 / 65536]
+    exp = np.zeros((len(fl), 8), np.uint32)
+    orc.orc_fr_from_f64(fl, 1 << 16, exp, len(fl))
+    assert (pv.from_f64(fl, 1 << 16).host() == exp).all()
+    f32 = fl.astype(np.float32)
+    orc.orc_fr_from_f32(f32, 1 << 16, exp, len(fl))
+    assert (pv.from_f32(f32, 1 << 16).host() == exp).all()
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 255, 256, 257, 1000, 1024, 1025, 4096, 50000, (1 << 20) + 3])
+def test_sum_and_me(pv, orc, n):
+    print("case n", n, flush=True)
+    A = mt_random_vec(np.random.RandomState(100 + n % 97), n)
+    h = pv.from_fr(A)
+    exp = np.zeros(8, np.uint32)
+    orc_check(orc.orc_fr_sum(A, n, exp))
+    assert (pv.sum(h) == exp).all()
+    k = max(0, (n - 1).bit_length())
+    u = mt_random_vec(np.random.RandomState(7), k)
+    orc_check(orc.orc_fr_me(A, n, u, k, exp))
+    assert (pv.me(h, u) == exp).all()
+
+
+def test_me_boolean_points_and_bruteforce(pv):
+    rng = random.Random(5)
+    t = [rng.randrange(R_MOD) for _ in range(13)]
+    h = pv.from_fr(fr_array(t))
+    u = [rng.randrange(R_MOD) for _ in range(4)]
+    assert fr_ints(pv.me(h, fr_array(u))) == [me_bruteforce(t, u)]
+    for i in (0, 5, 12, 15):
+        pt = [(i >> j) & 1 for j in range(4)]
+        assert fr_ints(pv.me(h, fr_array(pt))) == [t[i] if i < 13 else 0]
+
+
+@pytest.mark.parametrize("other,cur,win", [(1, 8, 1), (3, 4, 5), (2, 5, 3), (4, 11, 1), (1, 6, 7), (7, 43, 1), (1, 16, 64), (5, 1000, 3), (1, 2048, 33), (64, 4096, 1)])
+def test_partial_me(pv, orc, other, cur, win):
+    print("case", other, cur, win, flush=True)
+    n = other * cur * win
+    A = mt_random_vec(np.random.RandomState(cur), n)
+    k = (cur - 1).bit_length()
+    u = mt_random_vec(np.random.RandomState(8), k)
+    exp = np.zeros((n, 8), np.uint32)
+    out_n = np.zeros(1, np.int64)
+    orc_check(orc.orc_fr_partial_me(A, n, u, k, cur, win, exp, out_n))
+    got = pv.partial_me(pv.from_fr(A), u, cur, win).host()
+    assert got.shape[0] == out_n[0] == other * win
+    assert (got == exp[:out_n[0]]).all()
+    # fewer levels than bits: the axis is only partly folded
+    if k >= 2:
+        kk = k - 1
+        # legal only when 2^(kk-1) < cur <= 2^kk fails -> use the raw step count via a sub-axis
+        sub = 1 << kk
+        if cur >= sub:
+            A2 = A[: other * sub * win].copy()
+            orc_check(orc.orc_fr_partial_me(A2, other * sub * win, u[:kk].copy(), kk, sub, win, exp, out_n))
+            got = pv.partial_me(pv.from_fr(A2), u[:kk].copy(), sub, win).host()
+            assert (got == exp[:out_n[0]]).all()
+
+
+@pytest.mark.parametrize("n,win,k", [(32, 4, 3), (15, 3, 3), (18, 4, 3), (4096 * 16, 4096, 4), (11008 * 8, 8, 14)])
+def test_window_fold(pv, orc, n, win, k):
+    A = mt_random_vec(np.random.RandomState(n % 1000), n)
+    u = mt_random_vec(np.random.RandomState(9), k)
+    exp = np.zeros((n + 2 * win, 8), np.uint32)
+    out_n = np.zeros(1, np.int64)
+    orc_check(orc.orc_fr_partial_me_window(A, n, u, k, win, exp, out_n))
+    got = pv.partial_me_window(pv.from_fr(A), u, win).host()
+    assert got.shape[0] == out_n[0]
+    assert (got == exp[:out_n[0]]).all()
+
+
+def test_multi_dim_me(pv, orc):
+    for shape in ((4, 8), (16, 64), (3, 5, 7), (2048, 33)):
+        n = int(np.prod(shape))
+        A = mt_random_vec(np.random.RandomState(n % 991), n)
+        us = [mt_random_vec(np.random.RandomState(10 + i), max(0, (d - 1).bit_length())) for i, d in enumerate(shape)]
+        cat = np.ascontiguousarray(np.concatenate(us))
+        lens = np.array([u.shape[0] for u in us], np.uint32)
+        exp = np.zeros(8, np.uint32)
+        orc_check(orc.orc_fr_multi_dim_me(A, n, cat, lens, np.array(shape, np.uint32), len(shape), exp))
+        assert (pv.multi_dim_me(pv.from_fr(A), us, shape) == exp).all(), shape
+
+
+def test_pad_and_transpose(pv, orc):
+    for shape in ((3, 5), (11, 43), (1, 7), (16, 16), (5, 3, 6)):
+        n = int(np.prod(shape))
+        A = mt_random_vec(np.random.RandomState(n), n)
+        padv = fr_array([R_MOD - 3])[0]
+        exp = np.zeros((n * 8 + 64, 8), np.uint32)
+        out_n = np.zeros(1, np.int64)
+        orc_check(orc.orc_fr_pad(A, n, np.array(shape, np.uint32), len(shape), padv, exp, out_n))
+        got = pv.pad(pv.from_fr(A), shape, padv).host()
+        assert got.shape[0] == out_n[0] and (got == exp[:out_n[0]]).all(), shape
+    for M, N in ((3, 5), (32, 32), (33, 65), (1, 100), (100, 1), (257, 130)):
+        A = mt_random_vec(np.random.RandomState(M * N), M * N)
+        exp = np.zeros_like(A)
+        orc_check(orc.orc_fr_transpose(A, M, N, exp))
+        assert (pv.transpose(pv.from_fr(A), M, N).host() == exp).all(), (M, N)
+
+
+@pytest.mark.parametrize("M,N,P", [(1, 1, 1), (3, 4, 5), (16, 64, 64), (17, 9, 33), (40, 100, 24)])
+def test_matmul_generic_matches_oracle(pv, orc, M, N, P):
+    print("case", M, N, P, flush=True)
+    A = mt_random_vec(np.random.RandomState(M), M * N)
+    B = mt_random_vec(np.random.RandomState(P + 50), N * P)
+    exp = np.zeros((M * P, 8), np.uint32)
+    orc_check(orc.orc_fr_matmul(A, B, M, N, P, exp))
+    pv.lib.zkp_set_matmul_mode(ctypes.c_int(1))
+    got = pv.matmul(pv.from_fr(A), pv.from_fr(B), M, N, P).host()
+    assert pv.lib.zkp_last_matmul_path() == 1
+    assert (got == exp).all()
+    pv.lib.zkp_set_matmul_mode(ctypes.c_int(0))
+    got = pv.matmul(pv.from_fr(A), pv.from_fr(B), M, N, P).host()   # full-width residues: the bound check must refuse the integer path
+    assert pv.lib.zkp_last_matmul_path() == 1 and (got == exp).all()
+
+
+def test_matmul_small_integer_path_equals_generic(pv):
+    rng = np.random.default_rng(31)
+    M, N, P = 70, 130, 50
+    A = np.round(rng.normal(0, 1, (M, N)) * 65536).astype(np.int32)
+    B = np.round(rng.normal(0, 0.02, (N, P)) * 65536).astype(np.int32)
+    exp = [int(v) % R_MOD for v in (A.astype(object) @ B.astype(object)).reshape(-1)]
+    for mode, path in ((0, 2), (1, 1)):
+        pv.lib.zkp_set_matmul_mode(ctypes.c_int(mode))
+        got = pv.matmul(pv.from_i32(A), pv.from_i32(B), M, N, P).host()
+        assert pv.lib.zkp_last_matmul_path() == path
+        assert fr_ints(got) == exp
+    # int64-range operands (softmax outputs are ~2^40): still exact, or falls back when the bound fails
+    A64 = rng.integers(-2 ** 40, 2 ** 40, (8, 16)).astype(np.int64)
+    B64 = rng.integers(-2 ** 15, 2 ** 15, (16, 8)).astype(np.int64)
+    exp = [int(v) % R_MOD for v in (A64.astype(object) @ B64.astype(object)).reshape(-1)]
+    pv.lib.zkp_set_matmul_mode(ctypes.c_int(0))
+    got = pv.matmul(pv.from_i64(A64), pv.from_i64(B64), 8, 16, 8).host()
+    assert pv.lib.zkp_last_matmul_path() == 2 and fr_ints(got) == exp
+    A64 = rng.integers(-2 ** 50, 2 ** 50, (8, 16)).astype(np.int64)
+    exp = [int(v) % R_MOD for v in (A64.astype(object) @ B64.astype(object)).reshape(-1)]
+    got = pv.matmul(pv.from_i64(A64), pv.from_i64(B64), 8, 16, 8).host()
+    assert pv.lib.zkp_last_matmul_path() == 1 and fr_ints(got) == exp
+    pv.lib.zkp_set_matmul_mode(ctypes.c_int(0))
+
+
+@pytest.mark.parametrize("n", [2, 3, 8, 11, 64, 1000, 4096, 8192, 8193, 40000, 1 << 17])
+def test_zkip_matches_oracle(pv, orc, n):
+    print("case n", n, flush=True)
+    a = mt_random_vec(np.random.RandomState(n % 89), n)
+    b = mt_random_vec(np.random.RandomState(n % 83 + 200), n)
+    k = (n - 1).bit_length()
+    u = mt_random_vec(np.random.RandomState(12), k)
+    claim = np.zeros(8, np.uint32)
+    ha, hb = pv.from_fr(a), pv.from_fr(b)
+    # the claim is <a,b>
+    orc_check(orc.orc_fr_op(7, a, b, prod := np.zeros_like(a), n))
+    orc_check(orc.orc_fr_sum(prod, n, claim))
+    exp_proof = np.zeros((k, 3, 8), np.uint32)
+    exp_fin = np.zeros(8, np.uint32)
+    orc_check(orc.orc_zkip(claim, a, b, n, u, k, exp_proof, exp_fin))
+    proof, fin = pv.zkip(claim, ha, hb, u)
+    assert (proof == exp_proof).all() and (fin == exp_fin).all()
+    # a wrong claim is rejected exactly like the reference does
+    bad = claim.copy()
+    bad[0] ^= 1
+    with pytest.raises(RuntimeError, match="claim != p"):
+        pv.zkip(bad, ha, hb, u)
+
+
+@pytest.mark.parametrize("B,I,O,mode", [(16, 64, 64, 1), (16, 64, 64, 0), (5, 24, 10, 1), (64, 256, 128, 0)])
+def test_zkfc_forward_and_proof_transcript(pv, orc, B, I, O, mode):
+    rng = np.random.default_rng(B * I + O)
+    X = np.round(rng.normal(0, 0.02, (B, I)) * 65536).astype(np.int32)
+    W = np.round(rng.normal(0, 0.02, (I, O)) * 65536).astype(np.int32)
+    got_Y, got_t = pv.zkfc_scenario(X, W, seed=4242, matmul_mode=mode)
+    orc.orc_seed(4242)
+    orc.orc_transcript_clear()
+    exp_Y = np.zeros((B * O, 8), np.uint32)
+    orc_check(orc.orc_zkfc(X, W, B, I, O, exp_Y, np.zeros(8, np.uint32)))
+    exp_t = orc_transcript(orc)
+    assert (got_Y == exp_Y).all()
+    assert got_t.shape == exp_t.shape and (got_t == exp_t).all()
+    pv.lib.zkp_set_matmul_mode(ctypes.c_int(0))

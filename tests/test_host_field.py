@@ -1,0 +1,68 @@
+"""The product's own limb arithmetic (zkllm-ccs2024_amd/csrc/field.hpp -- one source for the GPU kernels
+and the prover's host-side scalar work), run on the CPU through the class-layer library and compared
+with python big-int closed forms and with the oracle.  No GPU needed."""
+import random
+
+import numpy as np
+
+from gpuhelp import _np_ptr, pkg
+from zkhelp import FP_R, FR_R, P_MOD, R_MOD, fp_array, fp_ints, fr_array, fr_ints, load_oracle, orc_check
+
+import ctypes
+
+
+def _lib():
+    return pkg.load_prover()
+
+
+def test_host_fr_ops_match_bigint_and_oracle():
+    lib, orc = _lib(), load_oracle()
+    rng = random.Random(11)
+    edge = [0, 1, 2, R_MOD - 1, R_MOD - 2, FR_R, (1 << 32) - 1, 1 << 254, (1944954706 << 224) | ((1 << 224) - 1)]
+    a = edge + [rng.randrange(R_MOD) for _ in range(500)]
+    b = list(reversed(a))
+    A, B = fr_array(a), fr_array(b)
+    got, exp = np.zeros_like(A), np.zeros_like(A)
+    rinv = pow(FR_R, -1, R_MOD)
+    closed = {0: lambda x, y: (x + y) % R_MOD, 1: lambda x, y: (x - y) % R_MOD, 2: lambda x, y: x * y * rinv % R_MOD,
+              3: lambda x, y: 2 * x % R_MOD, 4: lambda x, y: x * FR_R % R_MOD, 5: lambda x, y: x * rinv % R_MOD,
+              7: lambda x, y: x * y % R_MOD, 8: lambda x, y: pow(x, -1, R_MOD) if x else 0, 9: lambda x, y: (-x) % R_MOD}
+    for op, f in closed.items():
+        assert lib.zkp_host_fr_op(ctypes.c_int(op), _np_ptr(A), _np_ptr(B), _np_ptr(got), ctypes.c_long(len(a))) == 0
+        assert fr_ints(got) == [f(x, y) for x, y in zip(a, b)], f"host fr op {op}"
+        orc_check(orc.orc_fr_op(op, A, B, exp, len(a)))
+        assert (got == exp).all(), f"host fr op {op} vs oracle"
+    assert lib.zkp_host_fr_op(ctypes.c_int(6), _np_ptr(A), _np_ptr(B), _np_ptr(got), ctypes.c_long(64)) == 0
+    orc_check(orc.orc_fr_op(6, A, B, exp, 64))
+    assert (got[:64] == exp[:64]).all()
+
+
+def test_host_fp_ops_match_bigint_and_oracle():
+    lib, orc = _lib(), load_oracle()
+    rng = random.Random(12)
+    a = [0, 1, P_MOD - 1, FP_R, 1 << 380] + [rng.randrange(P_MOD) for _ in range(300)]
+    b = list(reversed(a))
+    A, B = fp_array(a), fp_array(b)
+    got, exp = np.zeros_like(A), np.zeros_like(A)
+    rinv = pow(FP_R, -1, P_MOD)
+    closed = {0: lambda x, y: (x + y) % P_MOD, 1: lambda x, y: (x - y) % P_MOD, 2: lambda x, y: x * y * rinv % P_MOD,
+              3: lambda x, y: 2 * x % P_MOD, 4: lambda x, y: x * FP_R % P_MOD, 5: lambda x, y: x * rinv % P_MOD}
+    for op, f in closed.items():
+        assert lib.zkp_host_fp_op(ctypes.c_int(op), _np_ptr(A), _np_ptr(B), _np_ptr(got), ctypes.c_long(len(a))) == 0
+        assert fp_ints(got) == [f(x, y) for x, y in zip(a, b)], f"host fp op {op}"
+        orc_check(orc.orc_fp_op(op, A, B, exp, len(a)))
+        assert (got == exp).all()
+    assert lib.zkp_host_fp_op(ctypes.c_int(6), _np_ptr(A), _np_ptr(B), _np_ptr(got), ctypes.c_long(32)) == 0
+    orc_check(orc.orc_fp_op(6, A, B, exp, 32))
+    assert (got[:32] == exp[:32]).all()
+
+
+def test_host_polynomial_eval_matches_horner():
+    lib = _lib()
+    rng = random.Random(13)
+    coefs = [rng.randrange(R_MOD) for _ in range(5)]
+    x = rng.randrange(R_MOD)
+    out = np.zeros(8, np.uint32)
+    C, X = fr_array(coefs), fr_array([x])
+    assert lib.zkp_poly_eval(_np_ptr(C), ctypes.c_int(5), _np_ptr(X), _np_ptr(out)) == 0
+    assert fr_ints(out) == [sum(c * pow(x, i, R_MOD) for i, c in enumerate(coefs)) % R_MOD]

@@ -1,0 +1,576 @@
+// FrTensor kernels for gfx950: elementwise, conversions, layout, sums, multilinear folds and
+// the inner-product sumcheck rounds.  Tensors hold standard-form residues, 32 B per element
+// (8 little-endian u32 limbs), exactly the reference's Fr_t layout (fr-tensor.cu:181-184).
+//
+// Differences from the reference's kernels that do not change any output byte:
+//  * broadcast operands and challenges are converted to Montgomery form once on the host, so a
+//    product with them costs one Montgomery multiplication instead of two;
+//  * sums of products are accumulated with the R^-1 factor still attached and corrected once;
+//  * folds run several levels per pass (registers) and finish in one workgroup (LDS).
+#include <cstring>
+#include "field.hpp"
+#include "rt.hpp"
+#include "../../include/zkllm_hip.h"
+
+using namespace zk;
+
+static constexpr int TPB = 256;
+
+// ------------------------------------------------------------------------------------------------
+// elementwise (fr-tensor.cu:71-153)
+// ------------------------------------------------------------------------------------------------
+enum { EW_ADD = 0, EW_SUB = 1, EW_MUL = 2, EW_MONTMUL = 3 };
+
+template <int OP> __global__ void __launch_bounds__(TPB) k_ew(Fr* __restrict__ out, const Fr* __restrict__ a, const Fr* __restrict__ b, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    const Fr x = a[i], y = b[i];
+    Fr r;
+    if (OP == EW_ADD) r = add(x, y);
+    else if (OP == EW_SUB) r = sub(x, y);
+    else if (OP == EW_MUL) r = fr_mul_std(x, y);
+    else r = mont_mul(x, y);
+    out[i] = r;
+}
+// s: for EW_MUL the scalar is already in Montgomery form (s*R), so one mont_mul yields a*s.
+template <int OP> __global__ void __launch_bounds__(TPB) k_ew_s(Fr* __restrict__ out, const Fr* __restrict__ a, const Fr s, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    const Fr x = a[i];
+    Fr r;
+    if (OP == EW_ADD) r = add(x, s);
+    else if (OP == EW_SUB) r = sub(x, s);
+    else r = mont_mul(x, s);
+    out[i] = r;
+}
+__global__ void __launch_bounds__(TPB) k_neg(Fr* __restrict__ out, const Fr* __restrict__ a, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) out[i] = neg(a[i]);
+}
+__global__ void __launch_bounds__(TPB) k_fill(Fr* __restrict__ out, const Fr s, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) out[i] = s;
+}
+// Z[i] += bias[i % cols] (zkfc.cu:36-41)
+__global__ void __launch_bounds__(TPB) k_bias(Fr* __restrict__ z, const Fr* __restrict__ bias, size_t n, uint32_t cols) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) z[i] = add(z[i], bias[i % cols]);
+}
+
+// ------------------------------------------------------------------------------------------------
+// conversions (fr-tensor.cu:186-208, 691-775, 922-945)
+// ------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(TPB) k_from_i32(Fr* __restrict__ out, const int32_t* __restrict__ in, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) out[i] = fr_from_i64((int64_t)in[i]);
+}
+__global__ void __launch_bounds__(TPB) k_from_i64(Fr* __restrict__ out, const int64_t* __restrict__ in, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) out[i] = fr_from_i64(in[i]);
+}
+__global__ void __launch_bounds__(TPB) k_from_u32(Fr* __restrict__ out, const uint32_t* __restrict__ in, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) out[i] = fr_from_u64((uint64_t)in[i]);
+}
+// round half away from zero after scaling (float_to_scalar / double_to_scalar)
+__global__ void __launch_bounds__(TPB) k_from_f32(Fr* __restrict__ out, const float* __restrict__ in, uint64_t sf, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    float x = in[i] * (float)sf;
+    const int64_t v = (x >= 0) ? (int64_t)((double)x + 0.5) : (int64_t)((double)x - 0.5);
+    out[i] = fr_from_i64(v);
+}
+__global__ void __launch_bounds__(TPB) k_from_f64(Fr* __restrict__ out, const double* __restrict__ in, uint64_t sf, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    double x = in[i] * (double)sf;
+    const int64_t v = (x >= 0) ? (int64_t)(x + 0.5) : (int64_t)(x - 0.5);
+    out[i] = fr_from_i64(v);
+}
+__global__ void __launch_bounds__(TPB) k_to_i32(int32_t* __restrict__ out, const Fr* __restrict__ in, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) out[i] = fr_to_i32(in[i]);
+}
+__global__ void __launch_bounds__(TPB) k_to_i64(int64_t* __restrict__ out, const Fr* __restrict__ in, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) out[i] = fr_to_i64(in[i]);
+}
+
+// ------------------------------------------------------------------------------------------------
+// layout (fr-tensor.cu:800-828 pad, :885-900 transpose; tlookup.cu:446-453 gather)
+// ------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(TPB) k_pad(Fr* __restrict__ out, const Fr* __restrict__ in, size_t n_out, uint32_t last_in, uint32_t last_out, const Fr pad) {
+    const size_t g = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (g >= n_out) return;
+    const size_t g0 = g / last_out;
+    const uint32_t g1 = (uint32_t)(g % last_out);
+    out[g] = (g1 >= last_in) ? pad : in[g0 * last_in + g1];
+}
+// 32x32 tile through LDS so both the read and the write are contiguous along the fast axis
+__global__ void __launch_bounds__(TPB) k_transpose(Fr* __restrict__ out, const Fr* __restrict__ in, uint32_t M, uint32_t N) {
+    __shared__ uint32_t tile[8][32][33];
+    const uint32_t bx = blockIdx.x * 32, by = blockIdx.y * 32;
+    const uint32_t tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 32 x 8
+    for (uint32_t r = ty; r < 32; r += 8) {
+        const uint32_t row = by + r, col = bx + tx;
+        if (row < M && col < N) {
+            const Fr v = in[(size_t)row * N + col];
+#pragma unroll
+            for (int l = 0; l < 8; ++l) tile[l][r][tx] = v.v[l];
+        }
+    }
+    __syncthreads();
+    for (uint32_t r = ty; r < 32; r += 8) {
+        const uint32_t col = bx + r, row = by + tx;     // output row = input col
+        if (row < M && col < N) {
+            Fr v;
+#pragma unroll
+            for (int l = 0; l < 8; ++l) v.v[l] = tile[l][tx][r];
+            out[(size_t)col * M + row] = v;
+        }
+    }
+}
+__global__ void __launch_bounds__(TPB) k_gather(Fr* __restrict__ out, const Fr* __restrict__ table, const uint32_t* __restrict__ idx, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) out[i] = table[idx[i]];
+}
+
+// ------------------------------------------------------------------------------------------------
+// block reduction of K running sums per thread; partials[k * gridDim.x + blockIdx.x]
+// ------------------------------------------------------------------------------------------------
+template <int K> __device__ __forceinline__ void block_reduce_store(Fr (&acc)[K], Fr* __restrict__ partials) {
+    __shared__ uint32_t red[8][TPB];
+    const uint32_t t = threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+#pragma unroll
+        for (int l = 0; l < 8; ++l) red[l][t] = acc[k].v[l];
+        __syncthreads();
+        for (uint32_t s = TPB / 2; s > 0; s >>= 1) {
+            if (t < s) {
+                Fr x, y;
+#pragma unroll
+                for (int l = 0; l < 8; ++l) { x.v[l] = red[l][t]; y.v[l] = red[l][t + s]; }
+                x = add(x, y);
+#pragma unroll
+                for (int l = 0; l < 8; ++l) red[l][t] = x.v[l];
+            }
+            __syncthreads();
+        }
+        if (t == 0) {
+            Fr x;
+#pragma unroll
+            for (int l = 0; l < 8; ++l) x.v[l] = red[l][0];
+            partials[(size_t)k * gridDim.x + blockIdx.x] = x;
+        }
+        __syncthreads();
+    }
+}
+// one block per k: out[k] = sum of partials[k*nb .. k*nb+nb)
+__global__ void __launch_bounds__(TPB) k_finish_sums(Fr* __restrict__ out, const Fr* __restrict__ partials, uint32_t nb) {
+    Fr acc[1] = {big_zero<8>()};
+    const Fr* p = partials + (size_t)blockIdx.x * nb;
+    for (uint32_t i = threadIdx.x; i < nb; i += TPB) acc[0] = add(acc[0], p[i]);
+    block_reduce_store<1>(acc, out);   // gridDim.x == K, so out[0*K + blockIdx.x] = out[k]
+}
+
+__global__ void __launch_bounds__(TPB) k_sum(Fr* __restrict__ partials, const Fr* __restrict__ a, size_t n) {
+    Fr acc[1] = {big_zero<8>()};
+    for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (size_t)gridDim.x * TPB) acc[0] = add(acc[0], a[i]);
+    block_reduce_store<1>(acc, partials);
+}
+// sum_i a_i*b_i*R^-1 (the caller applies the R^2 correction once)
+__global__ void __launch_bounds__(TPB) k_dot(Fr* __restrict__ partials, const Fr* __restrict__ a, const Fr* __restrict__ b, size_t n) {
+    Fr acc[1] = {big_zero<8>()};
+    for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (size_t)gridDim.x * TPB) acc[0] = add(acc[0], mont_mul(a[i], b[i]));
+    block_reduce_store<1>(acc, partials);
+}
+
+static inline unsigned reduce_grid(size_t n) {
+    size_t b = (n + TPB - 1) / TPB;
+    if (b > 2048) b = 2048;
+    if (b < 1) b = 1;
+    return (unsigned)b;
+}
+// finish K sums living in `partials` (K x nb) and bring them to the host (standard layout)
+template <int K> static int finish_to_host(Fr* partials, unsigned nb, Fr* host_out, hipStream_t st) {
+    void* stage = nullptr;
+    int rc = staging(&stage, sizeof(Fr) * K);
+    if (rc) return rc;
+    Scratch fin(sizeof(Fr) * K);
+    if (fin.rc) return fin.rc;
+    hipLaunchKernelGGL(k_finish_sums, dim3(K), dim3(TPB), 0, st, fin.as<Fr>(), partials, nb);
+    ZK_LAUNCH_CHECK();
+    ZK_HIP(hipMemcpyAsync(stage, fin.p, sizeof(Fr) * K, hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipStreamSynchronize(st));
+    memcpy(host_out, stage, sizeof(Fr) * K);
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// multilinear folds
+// ------------------------------------------------------------------------------------------------
+template <int L> struct FrPack { Fr x[L]; };
+
+// Folds L levels of the middle axis of in[other][cur][window] (adjacent pairs along `cur`, index
+// bit 0 first; positions past `cur` read as zero, which is the reference's odd-tail rule
+// a - x*a).  xs are in Montgomery form.  (fr-tensor.cu:518-560, 588-626)
+template <int L> __global__ void __launch_bounds__(TPB)
+k_fold_axis(Fr* __restrict__ out, const Fr* __restrict__ in, const FrPack<L> xs, size_t n_out, uint32_t cur, uint32_t cur_out, size_t window) {
+    const size_t g = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (g >= n_out) return;
+    const size_t i2 = g % window;
+    const size_t t = g / window;
+    const uint32_t i1 = (uint32_t)(t % cur_out);
+    const size_t i0 = t / cur_out;
+    const Fr* base = in + (i0 * cur) * window + i2;
+    const uint32_t first = i1 << L;
+    Fr v[1 << L];
+#pragma unroll
+    for (int j = 0; j < (1 << L); ++j) v[j] = (first + j < cur) ? base[(size_t)(first + j) * window] : big_zero<8>();
+#pragma unroll
+    for (int l = 0; l < L; ++l) {
+#pragma unroll
+        for (int j = 0; j < (1 << (L - 1 - l)); ++j) v[j] = add(v[2 * j], mont_mul(xs.x[l], sub(v[2 * j + 1], v[2 * j])));
+    }
+    out[g] = v[0];
+}
+
+// Finishes a multilinear evaluation inside one workgroup: n <= 1024 values, k levels.
+struct FrPack12 { Fr x[12]; };
+static constexpr uint32_t ME_SMALL_MAX = 1024;
+__global__ void __launch_bounds__(TPB) k_me_small(Fr* __restrict__ out, const Fr* __restrict__ in, const FrPack12 xs, uint32_t n, uint32_t k) {
+    __shared__ uint32_t buf[8][ME_SMALL_MAX];
+    const uint32_t t = threadIdx.x;
+    for (uint32_t i = t; i < ME_SMALL_MAX; i += TPB) {
+        Fr v = (i < n) ? in[i] : big_zero<8>();
+#pragma unroll
+        for (int l = 0; l < 8; ++l) buf[l][i] = v.v[l];
+    }
+    __syncthreads();
+    uint32_t cur = 1u << k;    // zero-extended length
+    for (uint32_t lvl = 0; lvl < k; ++lvl) {
+        const uint32_t half = cur >> 1;
+        Fr r[ME_SMALL_MAX / 2 / TPB];
+        int cnt = 0;
+        for (uint32_t j = t; j < half; j += TPB, ++cnt) {
+            Fr a, b;
+#pragma unroll
+            for (int l = 0; l < 8; ++l) { a.v[l] = buf[l][2 * j]; b.v[l] = buf[l][2 * j + 1]; }
+            r[cnt] = add(a, mont_mul(xs.x[lvl], sub(b, a)));
+        }
+        __syncthreads();
+        cnt = 0;
+        for (uint32_t j = t; j < half; j += TPB, ++cnt) {
+#pragma unroll
+            for (int l = 0; l < 8; ++l) buf[l][j] = r[cnt].v[l];
+        }
+        __syncthreads();
+        cur = half;
+    }
+    if (t == 0) {
+        Fr v;
+#pragma unroll
+        for (int l = 0; l < 8; ++l) v.v[l] = buf[l][0];
+        out[0] = v;
+    }
+}
+
+// MSB fold of the zero-extended vector: out[i] = a[i] + v*(a[i+n_out] - a[i])  (zkfc.cu:113-127,
+// tlookup.cu:94-103, proof.cu:180-188)
+__global__ void __launch_bounds__(TPB) k_fold_halves(Fr* __restrict__ out, const Fr* __restrict__ a, const Fr v_mont, size_t n_in, size_t n_out) {
+    const size_t g = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (g >= n_out) return;
+    const Fr a0 = (g < n_in) ? a[g] : big_zero<8>();
+    const Fr a1 = (g + n_out < n_in) ? a[g + n_out] : big_zero<8>();
+    out[g] = add(a0, mont_mul(v_mont, sub(a1, a0)));
+}
+// Stacked variant over [N][D] (zkfc.cu:169-185): same formula on whole rows
+// (covered by k_fold_halves with n_in = N*D, n_out = N_out*D).
+
+// ------------------------------------------------------------------------------------------------
+// inner-product sumcheck (zkfc.cu:94-151)
+// ------------------------------------------------------------------------------------------------
+// Three sums of one round, each still carrying R^-1:
+//   s0 = sum a0*b0, s1 = sum a0*(b1-b0) + b0*(a1-a0), s2 = sum (a1-a0)*(b1-b0)
+__global__ void __launch_bounds__(TPB) k_ip_round(Fr* __restrict__ partials, const Fr* __restrict__ a, const Fr* __restrict__ b, size_t n_in, size_t n_out) {
+    Fr acc[3] = {big_zero<8>(), big_zero<8>(), big_zero<8>()};
+    for (size_t g = (size_t)blockIdx.x * TPB + threadIdx.x; g < n_out; g += (size_t)gridDim.x * TPB) {
+        const Fr a0 = (g < n_in) ? a[g] : big_zero<8>();
+        const Fr b0 = (g < n_in) ? b[g] : big_zero<8>();
+        const Fr a1 = (g + n_out < n_in) ? a[g + n_out] : big_zero<8>();
+        const Fr b1 = (g + n_out < n_in) ? b[g + n_out] : big_zero<8>();
+        const Fr da = sub(a1, a0), db = sub(b1, b0);
+        acc[0] = add(acc[0], mont_mul(a0, b0));
+        acc[1] = add(acc[1], add(mont_mul(a0, db), mont_mul(b0, da)));
+        acc[2] = add(acc[2], mont_mul(da, db));
+    }
+    block_reduce_store<3>(acc, partials);
+}
+
+// Whole sumcheck in one workgroup for short vectors (n <= 8192): every round's three sums are
+// written to polys[round*3 + {0,1,2}] (standard form, R^2-corrected), the folded vectors
+// ping-pong through `work` (2 * 2 * n_pow2/2 elements) and the final a, b land in fin[0..1].
+// Challenges are consumed from the back of vs (Montgomery form), as the reference does.
+struct FrPack16 { Fr x[16]; };
+__global__ void __launch_bounds__(1024) k_ip_small(Fr* __restrict__ polys, Fr* __restrict__ fin, Fr* __restrict__ work,
+                                                   const Fr* __restrict__ a_in, const Fr* __restrict__ b_in, const FrPack16 vs, uint32_t n, uint32_t k) {
+    __shared__ uint32_t red[8][1024];
+    const uint32_t t = threadIdx.x;
+    const uint32_t half0 = (1u << k) >> 1;
+    const Fr* a = a_in;
+    const Fr* b = b_in;
+    uint32_t n_in = n;
+    const Fr r2 = big_r2<8>();
+    for (uint32_t round = 0; round < k; ++round) {
+        const uint32_t n_out = (1u << (k - round)) >> 1;
+        Fr* na = work + (size_t)(round & 1) * 2 * half0;
+        Fr* nb = na + half0;
+        const Fr v = vs.x[k - 1 - round];
+        Fr acc[3] = {big_zero<8>(), big_zero<8>(), big_zero<8>()};
+        for (uint32_t g = t; g < n_out; g += 1024) {
+            const Fr a0 = (g < n_in) ? a[g] : big_zero<8>();
+            const Fr b0 = (g < n_in) ? b[g] : big_zero<8>();
+            const Fr a1 = (g + n_out < n_in) ? a[g + n_out] : big_zero<8>();
+            const Fr b1 = (g + n_out < n_in) ? b[g + n_out] : big_zero<8>();
+            const Fr da = sub(a1, a0), db = sub(b1, b0);
+            acc[0] = add(acc[0], mont_mul(a0, b0));
+            acc[1] = add(acc[1], add(mont_mul(a0, db), mont_mul(b0, da)));
+            acc[2] = add(acc[2], mont_mul(da, db));
+            na[g] = add(a0, mont_mul(v, da));
+            nb[g] = add(b0, mont_mul(v, db));
+        }
+        for (int q = 0; q < 3; ++q) {
+#pragma unroll
+            for (int l = 0; l < 8; ++l) red[l][t] = acc[q].v[l];
+            __syncthreads();
+            for (uint32_t s = 512; s > 0; s >>= 1) {
+                if (t < s) {
+                    Fr x, y;
+#pragma unroll
+                    for (int l = 0; l < 8; ++l) { x.v[l] = red[l][t]; y.v[l] = red[l][t + s]; }
+                    x = add(x, y);
+#pragma unroll
+                    for (int l = 0; l < 8; ++l) red[l][t] = x.v[l];
+                }
+                __syncthreads();
+            }
+            if (t == 0) {
+                Fr x;
+#pragma unroll
+                for (int l = 0; l < 8; ++l) x.v[l] = red[l][0];
+                polys[round * 3 + q] = mont_mul(x, r2);
+            }
+            __syncthreads();
+        }
+        a = na; b = nb; n_in = n_out;
+    }
+    if (t == 0) { fin[0] = a[0]; fin[1] = b[0]; }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side of the C ABI
+// ------------------------------------------------------------------------------------------------
+static inline Fr load_fr(const uint32_t* p) { Fr r; memcpy(&r, p, 32); return r; }
+
+#define LAUNCH1D(kernel, n, st, ...)                                                         \
+    do {                                                                                     \
+        if ((n) > 0) {                                                                       \
+            hipLaunchKernelGGL(kernel, dim3(cdiv((n), TPB)), dim3(TPB), 0, (hipStream_t)(st), __VA_ARGS__); \
+            ZK_LAUNCH_CHECK();                                                               \
+        }                                                                                    \
+    } while (0)
+
+extern "C" {
+
+int zk_fr_add(void* out, const void* a, const void* b, size_t n, void* st) { LAUNCH1D(k_ew<EW_ADD>, n, st, (Fr*)out, (const Fr*)a, (const Fr*)b, n); return 0; }
+int zk_fr_sub(void* out, const void* a, const void* b, size_t n, void* st) { LAUNCH1D(k_ew<EW_SUB>, n, st, (Fr*)out, (const Fr*)a, (const Fr*)b, n); return 0; }
+int zk_fr_mul(void* out, const void* a, const void* b, size_t n, void* st) { LAUNCH1D(k_ew<EW_MUL>, n, st, (Fr*)out, (const Fr*)a, (const Fr*)b, n); return 0; }
+int zk_fr_montmul(void* out, const void* a, const void* b, size_t n, void* st) { LAUNCH1D(k_ew<EW_MONTMUL>, n, st, (Fr*)out, (const Fr*)a, (const Fr*)b, n); return 0; }
+int zk_fr_neg(void* out, const void* a, size_t n, void* st) { LAUNCH1D(k_neg, n, st, (Fr*)out, (const Fr*)a, n); return 0; }
+int zk_fr_add_s(void* out, const void* a, const uint32_t* s, size_t n, void* st) { LAUNCH1D(k_ew_s<EW_ADD>, n, st, (Fr*)out, (const Fr*)a, load_fr(s), n); return 0; }
+int zk_fr_sub_s(void* out, const void* a, const uint32_t* s, size_t n, void* st) { LAUNCH1D(k_ew_s<EW_SUB>, n, st, (Fr*)out, (const Fr*)a, load_fr(s), n); return 0; }
+int zk_fr_mul_s(void* out, const void* a, const uint32_t* s, size_t n, void* st) {
+    const Fr sm = to_mont(load_fr(s));
+    LAUNCH1D(k_ew_s<EW_MUL>, n, st, (Fr*)out, (const Fr*)a, sm, n);
+    return 0;
+}
+// a*R (Scalar_mont) is a Montgomery product with R^2; a*R^-1 (Scalar_unmont) one with 1.
+int zk_fr_mont(void* out, const void* a, size_t n, void* st) { LAUNCH1D(k_ew_s<EW_MUL>, n, st, (Fr*)out, (const Fr*)a, big_r2<8>(), n); return 0; }
+int zk_fr_unmont(void* out, const void* a, size_t n, void* st) {
+    Fr one = big_zero<8>(); one.v[0] = 1;
+    LAUNCH1D(k_ew_s<EW_MUL>, n, st, (Fr*)out, (const Fr*)a, one, n);
+    return 0;
+}
+int zk_fr_fill(void* out, const uint32_t* s, size_t n, void* st) { LAUNCH1D(k_fill, n, st, (Fr*)out, load_fr(s), n); return 0; }
+int zk_fr_bias_add(void* z, const void* bias, size_t rows, uint32_t cols, void* st) {
+    ZK_ARG(cols > 0, "zk_fr_bias_add: cols == 0");
+    LAUNCH1D(k_bias, rows * cols, st, (Fr*)z, (const Fr*)bias, rows * cols, cols);
+    return 0;
+}
+
+int zk_fr_from_i32(void* out, const void* in, size_t n, void* st) { LAUNCH1D(k_from_i32, n, st, (Fr*)out, (const int32_t*)in, n); return 0; }
+int zk_fr_from_i64(void* out, const void* in, size_t n, void* st) { LAUNCH1D(k_from_i64, n, st, (Fr*)out, (const int64_t*)in, n); return 0; }
+int zk_fr_from_u32(void* out, const void* in, size_t n, void* st) { LAUNCH1D(k_from_u32, n, st, (Fr*)out, (const uint32_t*)in, n); return 0; }
+int zk_fr_from_f32(void* out, const void* in, uint64_t sf, size_t n, void* st) { LAUNCH1D(k_from_f32, n, st, (Fr*)out, (const float*)in, sf, n); return 0; }
+int zk_fr_from_f64(void* out, const void* in, uint64_t sf, size_t n, void* st) { LAUNCH1D(k_from_f64, n, st, (Fr*)out, (const double*)in, sf, n); return 0; }
+int zk_fr_to_i32(void* out, const void* in, size_t n, void* st) { LAUNCH1D(k_to_i32, n, st, (int32_t*)out, (const Fr*)in, n); return 0; }
+int zk_fr_to_i64(void* out, const void* in, size_t n, void* st) { LAUNCH1D(k_to_i64, n, st, (int64_t*)out, (const Fr*)in, n); return 0; }
+
+int zk_fr_pad(void* out, const void* in, size_t rows, uint32_t last_in, uint32_t last_out, const uint32_t* pad, void* st) {
+    ZK_ARG(last_in > 0 && last_out >= last_in, "zk_fr_pad: need 0 < last_in <= last_out");
+    const size_t n_out = rows * last_out;
+    LAUNCH1D(k_pad, n_out, st, (Fr*)out, (const Fr*)in, n_out, last_in, last_out, load_fr(pad));
+    return 0;
+}
+int zk_fr_transpose(void* out, const void* in, uint32_t M, uint32_t N, void* st) {
+    if (M == 0 || N == 0) return 0;
+    ZK_ARG(out != in, "zk_fr_transpose: in-place transpose is not supported");
+    hipLaunchKernelGGL(k_transpose, dim3(cdiv(N, 32), cdiv(M, 32)), dim3(TPB), 0, (hipStream_t)st, (Fr*)out, (const Fr*)in, M, N);
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
+int zk_fr_gather(void* out, const void* table, const void* idx, size_t n, void* st) {
+    LAUNCH1D(k_gather, n, st, (Fr*)out, (const Fr*)table, (const uint32_t*)idx, n);
+    return 0;
+}
+
+int zk_fr_sum(uint32_t* out_host, const void* a, size_t n, void* st) {
+    if (n == 0) { memset(out_host, 0, 32); return 0; }
+    const unsigned nb = reduce_grid(n);
+    Scratch part(sizeof(Fr) * nb);
+    if (part.rc) return part.rc;
+    hipLaunchKernelGGL(k_sum, dim3(nb), dim3(TPB), 0, (hipStream_t)st, part.as<Fr>(), (const Fr*)a, n);
+    ZK_LAUNCH_CHECK();
+    return finish_to_host<1>(part.as<Fr>(), nb, (Fr*)out_host, (hipStream_t)st);
+}
+// sum_i a_i * b_i in standard form
+int zk_fr_dot(uint32_t* out_host, const void* a, const void* b, size_t n, void* st) {
+    if (n == 0) { memset(out_host, 0, 32); return 0; }
+    const unsigned nb = reduce_grid(n);
+    Scratch part(sizeof(Fr) * nb);
+    if (part.rc) return part.rc;
+    hipLaunchKernelGGL(k_dot, dim3(nb), dim3(TPB), 0, (hipStream_t)st, part.as<Fr>(), (const Fr*)a, (const Fr*)b, n);
+    ZK_LAUNCH_CHECK();
+    Fr s;
+    int rc = finish_to_host<1>(part.as<Fr>(), nb, &s, (hipStream_t)st);
+    if (rc) return rc;
+    s = to_mont(s);
+    memcpy(out_host, &s, 32);
+    return 0;
+}
+
+// One or more levels of the middle-axis fold; u[0..levels) are standard-form challenges.
+// out has other * ceil(cur / 2^levels) * window elements.  levels <= 3 per call.
+int zk_fr_fold_axis(void* out, const void* in, const uint32_t* u, int levels, size_t other, uint32_t cur, size_t window, void* st) {
+    ZK_ARG(levels >= 1 && levels <= 3, "zk_fr_fold_axis: levels must be 1..3");
+    ZK_ARG(cur >= 1 && window >= 1, "zk_fr_fold_axis: empty axis");
+    ZK_ARG(out != in, "zk_fr_fold_axis: out must differ from in");
+    const uint32_t cur_out = (uint32_t)(((uint64_t)cur + (1u << levels) - 1) >> levels);
+    const size_t n_out = other * cur_out * window;
+    if (n_out == 0) return 0;
+    if (levels == 1) {
+        FrPack<1> p; p.x[0] = to_mont(load_fr(u));
+        LAUNCH1D(k_fold_axis<1>, n_out, st, (Fr*)out, (const Fr*)in, p, n_out, cur, cur_out, window);
+    } else if (levels == 2) {
+        FrPack<2> p; for (int i = 0; i < 2; ++i) p.x[i] = to_mont(load_fr(u + 8 * i));
+        LAUNCH1D(k_fold_axis<2>, n_out, st, (Fr*)out, (const Fr*)in, p, n_out, cur, cur_out, window);
+    } else {
+        FrPack<3> p; for (int i = 0; i < 3; ++i) p.x[i] = to_mont(load_fr(u + 8 * i));
+        LAUNCH1D(k_fold_axis<3>, n_out, st, (Fr*)out, (const Fr*)in, p, n_out, cur, cur_out, window);
+    }
+    return 0;
+}
+
+// Multilinear extension of a (n elements, zero-extended to 2^k) at u[0..k): index bit j is bound
+// to u[j].  Requires 2^(k-1) < n <= 2^k (k = 0 allowed for n == 1).
+int zk_fr_me(uint32_t* out_host, const void* a, size_t n, const uint32_t* u, int k, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(n >= 1 && k >= 0 && k <= 32, "zk_fr_me: bad size");
+    ZK_ARG(n <= ((size_t)1 << k) && (k == 0 || n > ((size_t)1 << (k - 1))), "zk_fr_me: need 2^(k-1) < n <= 2^k");
+    const Fr* cur_ptr = (const Fr*)a;
+    size_t cur = n;
+    int done = 0;
+    void* bufs[2] = {nullptr, nullptr};
+    int which = 0, rc = 0;
+    while (cur > ME_SMALL_MAX && rc == 0) {
+        const int L = 3;
+        const size_t next = (cur + 7) >> 3;
+        if (!bufs[which]) rc = pool_alloc(&bufs[which], next * sizeof(Fr));
+        if (rc) break;
+        rc = zk_fr_fold_axis(bufs[which], cur_ptr, u + 8 * done, L, 1, (uint32_t)cur, 1, stv);
+        cur_ptr = (const Fr*)bufs[which];
+        which ^= 1;
+        cur = next;
+        done += L;
+    }
+    if (rc == 0) {
+        FrPack12 p;
+        const int rest = k - done;
+        for (int i = 0; i < 12; ++i) p.x[i] = (i < rest) ? to_mont(load_fr(u + 8 * (done + i))) : big_zero<8>();
+        Scratch fin(sizeof(Fr));
+        rc = fin.rc;
+        void* stage = nullptr;
+        if (!rc) rc = staging(&stage, sizeof(Fr));
+        if (!rc) {
+            hipLaunchKernelGGL(k_me_small, dim3(1), dim3(TPB), 0, st, fin.as<Fr>(), cur_ptr, p, (uint32_t)cur, (uint32_t)rest);
+            hipError_t e = hipGetLastError();
+            if (e == hipSuccess) e = hipMemcpyAsync(stage, fin.p, sizeof(Fr), hipMemcpyDeviceToHost, st);
+            if (e == hipSuccess) e = hipStreamSynchronize(st);
+            if (e != hipSuccess) rc = hip_fail(e, "zk_fr_me", __FILE__, __LINE__);
+            else memcpy(out_host, stage, 32);
+        }
+    }
+    for (int i = 0; i < 2; ++i) if (bufs[i]) pool_free(bufs[i]);
+    return rc;
+}
+
+int zk_fr_fold_halves(void* out, const void* a, const uint32_t* v, size_t n_in, size_t n_out, void* st) {
+    ZK_ARG(out != a, "zk_fr_fold_halves: out must differ from in");
+    LAUNCH1D(k_fold_halves, n_out, st, (Fr*)out, (const Fr*)a, to_mont(load_fr(v)), n_in, n_out);
+    return 0;
+}
+
+// One round of the inner-product sumcheck: poly3_host = [sum a0 b0, sum a0 db + b0 da, sum da db].
+int zk_ip_round(uint32_t* poly3_host, const void* a, const void* b, size_t n_in, size_t n_out, void* stv) {
+    ZK_ARG(n_out >= 1 && n_in >= 1 && n_in <= 2 * n_out, "zk_ip_round: need n_in <= 2*n_out");
+    const unsigned nb = reduce_grid(n_out);
+    Scratch part(sizeof(Fr) * 3 * nb);
+    if (part.rc) return part.rc;
+    hipLaunchKernelGGL(k_ip_round, dim3(nb), dim3(TPB), 0, (hipStream_t)stv, part.as<Fr>(), (const Fr*)a, (const Fr*)b, n_in, n_out);
+    ZK_LAUNCH_CHECK();
+    Fr s[3];
+    int rc = finish_to_host<3>(part.as<Fr>(), nb, s, (hipStream_t)stv);
+    if (rc) return rc;
+    for (int i = 0; i < 3; ++i) s[i] = to_mont(s[i]);
+    memcpy(poly3_host, s, 96);
+    return 0;
+}
+
+// Complete inner-product sumcheck for n <= 8192 in one launch.  u[0..k) standard form, consumed
+// from the back; polys_host gets 3*k coefficients, fin_host the folded a and b.
+int zk_ip_sumcheck_small(uint32_t* polys_host, uint32_t* fin_host, const void* a, const void* b, uint32_t n, const uint32_t* u, int k, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(k >= 1 && k <= 13, "zk_ip_sumcheck_small: k must be 1..13");
+    ZK_ARG(n >= 1 && n <= (1u << k) && n > ((1u << k) >> 1), "zk_ip_sumcheck_small: need 2^(k-1) < n <= 2^k");
+    FrPack16 p;
+    for (int i = 0; i < 16; ++i) p.x[i] = (i < k) ? to_mont(load_fr(u + 8 * i)) : big_zero<8>();
+    const size_t half0 = ((size_t)1 << k) >> 1;
+    Scratch work(sizeof(Fr) * (4 * half0 + 3 * (size_t)k + 2));
+    if (work.rc) return work.rc;
+    Fr* w = work.as<Fr>();
+    Fr* polys = w + 4 * half0;
+    Fr* fin = polys + 3 * k;
+    hipLaunchKernelGGL(k_ip_small, dim3(1), dim3(1024), 0, st, polys, fin, w, (const Fr*)a, (const Fr*)b, p, n, (uint32_t)k);
+    ZK_LAUNCH_CHECK();
+    void* stage = nullptr;
+    int rc = staging(&stage, sizeof(Fr) * (3 * k + 2));
+    if (rc) return rc;
+    ZK_HIP(hipMemcpyAsync(stage, polys, sizeof(Fr) * (3 * k + 2), hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipStreamSynchronize(st));
+    memcpy(polys_host, stage, sizeof(Fr) * 3 * k);
+    memcpy(fin_host, (char*)stage + sizeof(Fr) * 3 * k, sizeof(Fr) * 2);
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,257 @@
+// Fr matrix product C[M x P] = A[M x N] * B[N x P] for gfx950 (replaces matrixMultiplyOptimized,
+// fr-tensor.cu:831-881, used by zkFC::operator() zkfc.cu:44-58 and FrTensor::matmul).
+//
+// The work is VALU integer multiply-add (v_mad_u64_u32); MFMA cannot help a 255-bit modular
+// product.  Two paths, both bit-identical to the reference because results are canonical:
+//
+//  * generic: every MAC is a 255x255-bit product.  Eight products are accumulated limb-row by
+//    limb-row into one running value and share a single Montgomery reduction ("multi-term
+//    CIOS"): 64 multiply-adds per MAC for the products plus 64/8 for the reduction, against
+//    128 for a product reduced on its own.  The R^-1 factor is removed once per output.
+//  * small-integer: when both operands are embeddings of int32-range values and the whole dot
+//    product is bounded by 2^62, the same sum is computed in int64 and embedded at the end.
+//    The bound is established on the device from the operands (max |a|, max |b|, N); nothing is
+//    assumed.  This is the case for every matmul of the LLaMa pipeline except softmax(Y)*V.
+#include <cstring>
+#include "field.hpp"
+#include "rt.hpp"
+#include "../../include/zkllm_hip.h"
+
+using namespace zk;
+
+static constexpr int KT = 8;       // terms sharing one reduction
+static constexpr int TM = 16, TN = 16;
+
+// sum_q a[q]*b[q]*R^-1 mod r, canonical.  The running value stays below (KT+1)*r < 2^260.
+__device__ __forceinline__ Fr dot_mont(const Fr (&a)[KT], const Fr (&b)[KT]) {
+    uint32_t t[10];
+#pragma unroll
+    for (int i = 0; i < 10; ++i) t[i] = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#pragma unroll
+        for (int q = 0; q < KT; ++q) {
+            uint64_t c = 0;
+            const uint32_t bi = b[q].v[i];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                c += (uint64_t)a[q].v[j] * bi + t[j];
+                t[j] = (uint32_t)c;
+                c >>= 32;
+            }
+            c += t[8];
+            t[8] = (uint32_t)c;
+            t[9] += (uint32_t)(c >> 32);
+        }
+        const uint32_t m = 0u - t[0];                 // INV = -1 mod 2^32
+        uint64_t c = ((uint64_t)m * FrK::P(0) + t[0]) >> 32;
+#pragma unroll
+        for (int j = 1; j < 8; ++j) {
+            c += (uint64_t)m * FrK::P(j) + t[j];
+            t[j - 1] = (uint32_t)c;
+            c >>= 32;
+        }
+        c += t[8];
+        t[7] = (uint32_t)c;
+        c >>= 32;
+        c += t[9];
+        t[8] = (uint32_t)c;
+        t[9] = 0;
+    }
+    // t[0..8] < (KT+1) r : subtract 8r, 4r, 2r, r conditionally (constants built at compile time)
+#pragma unroll
+    for (int s = 3; s >= 0; --s) {
+        uint32_t d[9];
+        uint64_t br = 0;
+#pragma unroll
+        for (int i = 0; i < 9; ++i) {
+            // limb i of (r << s)
+            const uint32_t lo = (i < 8) ? FrK::P(i) : 0u;
+            const uint32_t prev = (i >= 1 && i <= 8) ? FrK::P(i - 1) : 0u;
+            const uint32_t ki = (s == 0) ? lo : (uint32_t)((lo << s) | (prev >> (32 - s)));
+            uint64_t x = (uint64_t)t[i] - ki - br;
+            d[i] = (uint32_t)x;
+            br = (x >> 32) & 1u;
+        }
+        const bool keep = br != 0;
+#pragma unroll
+        for (int i = 0; i < 9; ++i) t[i] = keep ? t[i] : d[i];
+    }
+    Fr r;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r.v[i] = t[i];
+    return r;
+}
+
+__global__ void __launch_bounds__(TM * TN) k_matmul(Fr* __restrict__ C, const Fr* __restrict__ A, const Fr* __restrict__ B, uint32_t M, uint32_t N, uint32_t P) {
+    __shared__ uint32_t As[8][TM][KT + 1];
+    __shared__ uint32_t Bs[8][KT][TN];
+    const uint32_t tx = threadIdx.x % TN, ty = threadIdx.x / TN;
+    const uint32_t row = blockIdx.y * TM + ty, col = blockIdx.x * TN + tx;
+    Fr acc = big_zero<8>();
+    for (uint32_t k0 = 0; k0 < N; k0 += KT) {
+        // 128 A elements + 128 B elements, one per thread
+        if (threadIdx.x < TM * KT) {
+            const uint32_t r = threadIdx.x / KT, q = threadIdx.x % KT;
+            const uint32_t gr = blockIdx.y * TM + r, gk = k0 + q;
+            Fr v = (gr < M && gk < N) ? A[(size_t)gr * N + gk] : big_zero<8>();
+#pragma unroll
+            for (int l = 0; l < 8; ++l) As[l][r][q] = v.v[l];
+        } else {
+            const uint32_t e = threadIdx.x - TM * KT;
+            const uint32_t q = e / TN, c = e % TN;
+            const uint32_t gk = k0 + q, gc = blockIdx.x * TN + c;
+            Fr v = (gk < N && gc < P) ? B[(size_t)gk * P + gc] : big_zero<8>();
+#pragma unroll
+            for (int l = 0; l < 8; ++l) Bs[l][q][c] = v.v[l];
+        }
+        __syncthreads();
+        Fr a[KT], b[KT];
+#pragma unroll
+        for (int q = 0; q < KT; ++q) {
+#pragma unroll
+            for (int l = 0; l < 8; ++l) { a[q].v[l] = As[l][ty][q]; b[q].v[l] = Bs[l][q][tx]; }
+        }
+        acc = add(acc, dot_mont(a, b));
+        __syncthreads();
+    }
+    if (row < M && col < P) C[(size_t)row * P + col] = to_mont(acc);
+}
+
+// ---- small-integer path ---------------------------------------------------------------------------
+// max |x| over a tensor of embedded integers; anything that is not an embedded int64 in
+// [-2^62, 2^62] poisons the result with UINT64_MAX.
+__global__ void __launch_bounds__(256) k_absmax(unsigned long long* __restrict__ out, const Fr* __restrict__ a, size_t n) {
+    unsigned long long m = 0;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        const Fr x = a[i];
+        unsigned long long v;
+        if (!(x.v[2] | x.v[3] | x.v[4] | x.v[5] | x.v[6] | x.v[7])) v = (unsigned long long)x.v[0] | ((unsigned long long)x.v[1] << 32);
+        else {
+            const Fr y = neg(x);
+            v = (y.v[2] | y.v[3] | y.v[4] | y.v[5] | y.v[6] | y.v[7]) ? ~0ull : ((unsigned long long)y.v[0] | ((unsigned long long)y.v[1] << 32));
+        }
+        if (v > (1ull << 62)) v = ~0ull;
+        m = v > m ? v : m;
+    }
+    __shared__ unsigned long long red[256];
+    red[threadIdx.x] = m;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if (threadIdx.x < s) red[threadIdx.x] = red[threadIdx.x] > red[threadIdx.x + s] ? red[threadIdx.x] : red[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) atomicMax(out, red[0]);
+}
+template <typename T> __global__ void __launch_bounds__(256) k_fr_to_int(T* __restrict__ out, const Fr* __restrict__ a, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = (T)fr_to_i64(a[i]);
+}
+// 64x64 output tile per workgroup, 4x4 per thread, K step 16, int64 accumulation.
+// T = int when both operands fit 31 bits (one v_mad_i64_i32 per MAC), long long otherwise.
+template <typename T> __global__ void __launch_bounds__(256) k_matmul_int(Fr* __restrict__ C, const T* __restrict__ A, const T* __restrict__ B, uint32_t M, uint32_t N, uint32_t P) {
+    __shared__ T As[16][64 + 1];
+    __shared__ T Bs[16][64 + 1];
+    const uint32_t tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    const uint32_t row0 = blockIdx.y * 64, col0 = blockIdx.x * 64;
+    long long acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0;
+    for (uint32_t k0 = 0; k0 < N; k0 += 16) {
+        for (uint32_t e = threadIdx.x; e < 64 * 16; e += 256) {
+            const uint32_t r = e / 16, q = e % 16;        // A: 64 rows x 16 k
+            As[q][r] = (row0 + r < M && k0 + q < N) ? A[(size_t)(row0 + r) * N + k0 + q] : (T)0;
+            const uint32_t q2 = e / 64, c = e % 64;       // B: 16 k x 64 cols
+            Bs[q2][c] = (k0 + q2 < N && col0 + c < P) ? B[(size_t)(k0 + q2) * P + col0 + c] : (T)0;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            T av[4], bv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { av[i] = As[q][ty * 4 + i]; bv[i] = Bs[q][tx * 4 + i]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] += (long long)av[i] * (long long)bv[j];
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t r = row0 + ty * 4 + i, c = col0 + tx * 4 + j;
+            if (r < M && c < P) C[(size_t)r * P + c] = fr_from_i64(acc[i][j]);
+        }
+}
+
+template <typename T> static int run_int_path(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, hipStream_t st) {
+    const size_t na = (size_t)M * N, nb = (size_t)N * P;
+    Scratch ai(na * sizeof(T)), bi(nb * sizeof(T));
+    if (ai.rc) return ai.rc;
+    if (bi.rc) return bi.rc;
+    hipLaunchKernelGGL(k_fr_to_int<T>, dim3(cdiv(na, 256)), dim3(256), 0, st, ai.as<T>(), (const Fr*)A, na);
+    hipLaunchKernelGGL(k_fr_to_int<T>, dim3(cdiv(nb, 256)), dim3(256), 0, st, bi.as<T>(), (const Fr*)B, nb);
+    hipLaunchKernelGGL(k_matmul_int<T>, dim3(cdiv(P, 64), cdiv(M, 64)), dim3(256), 0, st, (Fr*)C, ai.as<T>(), bi.as<T>(), M, N, P);
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
+
+static inline unsigned absmax_grid(size_t n) {
+    size_t b = n / (256 * 8) + 1;
+    return (unsigned)(b > 1024 ? 1024 : b);
+}
+
+extern "C" {
+
+int zk_fr_matmul_generic(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, void* st) {
+    if (M == 0 || P == 0) return 0;
+    ZK_ARG(N > 0, "zk_fr_matmul: inner dimension is 0");
+    hipLaunchKernelGGL(k_matmul, dim3(cdiv(P, TN), cdiv(M, TM)), dim3(TM * TN), 0, (hipStream_t)st, (Fr*)C, (const Fr*)A, (const Fr*)B, M, N, P);
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
+
+// mode: 0 = choose (small-integer path when the device-side bound check allows it),
+//       1 = always generic Montgomery, 2 = require the small-integer path (error if not applicable).
+// path_used (optional, host): 1 generic, 2 small-integer.
+int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    if (M == 0 || P == 0) return 0;
+    ZK_ARG(N > 0, "zk_fr_matmul: inner dimension is 0");
+    ZK_ARG(mode >= 0 && mode <= 2, "zk_fr_matmul: mode must be 0, 1 or 2");
+    bool small = false, fits32 = false;
+    if (mode != 1) {
+        Scratch mx(2 * sizeof(unsigned long long));
+        if (mx.rc) return mx.rc;
+        ZK_HIP(hipMemsetAsync(mx.p, 0, 2 * sizeof(unsigned long long), st));
+        const size_t na = (size_t)M * N, nb = (size_t)N * P;
+        hipLaunchKernelGGL(k_absmax, dim3(absmax_grid(na)), dim3(256), 0, st, mx.as<unsigned long long>(), (const Fr*)A, na);
+        hipLaunchKernelGGL(k_absmax, dim3(absmax_grid(nb)), dim3(256), 0, st, mx.as<unsigned long long>() + 1, (const Fr*)B, nb);
+        ZK_LAUNCH_CHECK();
+        void* stage = nullptr;
+        int rc = staging(&stage, 16);
+        if (rc) return rc;
+        ZK_HIP(hipMemcpyAsync(stage, mx.p, 16, hipMemcpyDeviceToHost, st));
+        ZK_HIP(hipStreamSynchronize(st));
+        const unsigned long long ma = ((unsigned long long*)stage)[0], mb = ((unsigned long long*)stage)[1];
+        if (ma != ~0ull && mb != ~0ull) {
+            // |sum| <= N * ma * mb must stay below 2^62
+            const unsigned __int128 bound = (unsigned __int128)ma * mb * N;
+            small = bound < ((unsigned __int128)1 << 62);
+            fits32 = ma < (1ull << 31) && mb < (1ull << 31);
+        }
+        if (mode == 2 && !small) { set_error(ZK_ERR_ARG, "zk_fr_matmul: operands do not satisfy the small-integer bound"); return ZK_ERR_ARG; }
+    }
+    if (!small) {
+        if (path_used) *path_used = 1;
+        return zk_fr_matmul_generic(C, A, B, M, N, P, stv);
+    }
+    if (path_used) *path_used = 2;
+    return fits32 ? run_int_path<int>(C, A, B, M, N, P, st) : run_int_path<long long>(C, A, B, M, N, P, st);
+}
+
+}  // extern "C"

@@ -1,0 +1,55 @@
+// Internal runtime helpers shared by the .hip translation units: error capture, the caching
+// device allocator behind zk_malloc/zk_free, and a pinned staging area for small results.
+#pragma once
+#include <cstddef>
+#include <cstdint>
+#include <string>
+#include <hip/hip_runtime.h>
+
+namespace zk {
+
+enum : int {
+    ZK_OK = 0,
+    ZK_ERR_ARG = 10001,      // bad argument (shape mismatch, null pointer, size over a stated limit)
+    ZK_ERR_NO_DEVICE = 10002
+};
+
+void set_error(int code, const std::string& msg);
+int hip_fail(hipError_t e, const char* what, const char* file, int line);
+
+#define ZK_HIP(call)                                                        \
+    do {                                                                    \
+        hipError_t e__ = (call);                                            \
+        if (e__ != hipSuccess) return zk::hip_fail(e__, #call, __FILE__, __LINE__); \
+    } while (0)
+
+#define ZK_ARG(cond, msg)                                                   \
+    do {                                                                    \
+        if (!(cond)) { zk::set_error(zk::ZK_ERR_ARG, msg); return zk::ZK_ERR_ARG; } \
+    } while (0)
+
+#define ZK_LAUNCH_CHECK() ZK_HIP(hipGetLastError())
+
+// Caching allocator: blocks are kept on per-size free lists and reused; all work is assumed to
+// run on one stream, so a block handed out again is ordered after its previous user.
+int pool_alloc(void** out, size_t bytes);
+int pool_free(void* p);
+int pool_trim();
+
+// RAII scratch from the pool for use inside one entry point.
+struct Scratch {
+    void* p = nullptr;
+    int rc = 0;
+    explicit Scratch(size_t bytes) { rc = pool_alloc(&p, bytes ? bytes : 1); }
+    ~Scratch() { if (p) pool_free(p); }
+    template <class T> T* as() const { return reinterpret_cast<T*>(p); }
+    Scratch(const Scratch&) = delete;
+    Scratch& operator=(const Scratch&) = delete;
+};
+
+// Pinned host buffer (64 KiB) for device->host results of reductions.
+int staging(void** host_ptr, size_t bytes);
+
+static inline unsigned cdiv(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
+
+}  // namespace zk

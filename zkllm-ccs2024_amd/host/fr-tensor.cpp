@@ -1,0 +1,378 @@
+#include "fr-tensor.hpp"
+
+#include <climits>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+
+#include "../../include/zkllm_hip.h"
+#include "../csrc/field.hpp"
+#include "ioutils.hpp"
+
+using namespace std;
+
+// ---- status / globals ---------------------------------------------------------------------------
+void zk_check(int rc, const char* where) {
+    if (rc != 0) throw std::runtime_error(string(where) + ": " + zk_last_error());
+}
+#define ZKC(call) zk_check((call), #call)
+
+namespace {
+struct Globals {
+    std::mt19937 mt;
+    bool seeded = false;
+    int matmul_mode = 0;
+    int last_matmul_path = 0;
+    bool recording = false;
+    std::vector<Fr_t> transcript;
+    Globals() {
+        if (const char* m = getenv("ZKLLM_MATMUL")) matmul_mode = (string(m) == "generic") ? 1 : 0;
+    }
+};
+Globals& G() { static Globals g; return g; }
+void ensure_seeded() {
+    Globals& g = G();
+    if (g.seeded) return;
+    if (const char* s = getenv("ZKLLM_SEED")) g.mt.seed((uint32_t)strtoul(s, nullptr, 10));
+    else { std::random_device rd; g.mt.seed(rd()); }
+    g.seeded = true;
+}
+}  // namespace
+
+void zk_seed_challenges(uint32_t seed) { G().mt.seed(seed); G().seeded = true; }
+void zk_set_matmul_mode(int mode) { G().matmul_mode = mode; }
+int zk_last_matmul_path() { return G().last_matmul_path; }
+void zk_transcript_begin() { G().transcript.clear(); G().recording = true; }
+const std::vector<Fr_t>& zk_transcript() { return G().transcript; }
+void zk_transcript_end() { G().recording = false; }
+void zk_record(const Fr_t& x) { if (G().recording) G().transcript.push_back(x); }
+void zk_record(const std::vector<Fr_t>& xs) { if (G().recording) G().transcript.insert(G().transcript.end(), xs.begin(), xs.end()); }
+
+ostream& operator<<(ostream& os, const Fr_t& x) {
+    os << "0x" << std::hex;
+    for (uint i = 8; i > 0; --i) os << std::setfill('0') << std::setw(8) << x.val[i - 1];
+    return os << std::dec << std::setw(0) << std::setfill(' ');
+}
+
+// 8 raw mt19937 outputs per element, the last reduced mod the top limb of r (fr-tensor.cu:16-24)
+vector<Fr_t> random_vec(uint len) {
+    ensure_seeded();
+    std::mt19937& mt = G().mt;
+    vector<Fr_t> out(len);
+    for (uint i = 0; i < len; ++i) {
+        for (int k = 0; k < 7; ++k) out[i].val[k] = (uint)mt();
+        out[i].val[7] = (uint)mt() % 1944954707u;
+    }
+    return out;
+}
+
+uint ceilLog2(uint num) {
+    if (num == 0) return 0;
+    num--;
+    uint result = 0;
+    while (num > 0) { num >>= 1; result++; }
+    return result;
+}
+
+// ---- raw device buffers / files -----------------------------------------------------------------------
+DevBuf::DevBuf(size_t bytes) { ZKC(zk_malloc(&p, bytes)); }
+DevBuf::~DevBuf() { if (p) zk_free(p); }
+
+void savebin(const string& filename, const void* gpudata, size_t size) {
+    std::vector<char> data(size);
+    ZKC(zk_memcpy_d2h(data.data(), gpudata, size, nullptr));
+    FILE* f = fopen(filename.c_str(), "wb");
+    if (!f) throw std::runtime_error("savebin: cannot open " + filename);
+    size_t w = fwrite(data.data(), 1, size, f);
+    fclose(f);
+    if (w != size) throw std::runtime_error("savebin: short write to " + filename);
+}
+size_t findsize(const string& filename) {
+    FILE* f = fopen(filename.c_str(), "rb");
+    if (!f) throw std::runtime_error("findsize: cannot open " + filename);
+    fseek(f, 0, SEEK_END);
+    long sz = ftell(f);
+    fclose(f);
+    return (size_t)sz;
+}
+void loadbin(const string& filename, void* gpudata, size_t size) {
+    std::vector<char> data(size);
+    FILE* f = fopen(filename.c_str(), "rb");
+    if (!f) throw std::runtime_error("loadbin: cannot open " + filename);
+    size_t r = fread(data.data(), 1, size, f);
+    fclose(f);
+    if (r != size) throw std::runtime_error("loadbin: short read from " + filename);
+    ZKC(zk_memcpy_h2d(gpudata, data.data(), size, nullptr));
+}
+
+// ---- FrTensor -------------------------------------------------------------------------------------------
+static Fr_t* fr_alloc(size_t n) {
+    void* p = nullptr;
+    ZKC(zk_malloc(&p, sizeof(Fr_t) * (n ? n : 1)));
+    return (Fr_t*)p;
+}
+
+FrTensor::FrTensor(uint size) : gpu_data(fr_alloc(size)), size(size) {}
+FrTensor::FrTensor(uint size, const Fr_t* cpu_data) : gpu_data(fr_alloc(size)), size(size) {
+    ZKC(zk_memcpy_h2d(gpu_data, cpu_data, sizeof(Fr_t) * size, nullptr));
+}
+FrTensor::FrTensor(uint size, const int* cpu_data) : gpu_data(fr_alloc(size)), size(size) {
+    DevBuf tmp(sizeof(int) * (size_t)size);
+    ZKC(zk_memcpy_h2d(tmp.p, cpu_data, sizeof(int) * (size_t)size, nullptr));
+    ZKC(zk_fr_from_i32(gpu_data, tmp.p, size, nullptr));
+    ZKC(zk_sync(nullptr));
+}
+FrTensor::FrTensor(uint size, const long* cpu_data) : gpu_data(fr_alloc(size)), size(size) {
+    DevBuf tmp(sizeof(long) * (size_t)size);
+    ZKC(zk_memcpy_h2d(tmp.p, cpu_data, sizeof(long) * (size_t)size, nullptr));
+    ZKC(zk_fr_from_i64(gpu_data, tmp.p, size, nullptr));
+    ZKC(zk_sync(nullptr));
+}
+FrTensor::FrTensor(uint size, const float* cpu_data, unsigned long sf) : gpu_data(fr_alloc(size)), size(size) {
+    DevBuf tmp(sizeof(float) * (size_t)size);
+    ZKC(zk_memcpy_h2d(tmp.p, cpu_data, sizeof(float) * (size_t)size, nullptr));
+    ZKC(zk_fr_from_f32(gpu_data, tmp.p, sf, size, nullptr));
+    ZKC(zk_sync(nullptr));
+}
+FrTensor::FrTensor(uint size, const double* cpu_data, unsigned long sf) : gpu_data(fr_alloc(size)), size(size) {
+    DevBuf tmp(sizeof(double) * (size_t)size);
+    ZKC(zk_memcpy_h2d(tmp.p, cpu_data, sizeof(double) * (size_t)size, nullptr));
+    ZKC(zk_fr_from_f64(gpu_data, tmp.p, sf, size, nullptr));
+    ZKC(zk_sync(nullptr));
+}
+FrTensor::FrTensor(const FrTensor& t) : gpu_data(fr_alloc(t.size)), size(t.size) {
+    ZKC(zk_memcpy_d2d(gpu_data, t.gpu_data, sizeof(Fr_t) * (size_t)size, nullptr));
+}
+FrTensor::FrTensor(FrTensor&& t) noexcept : gpu_data(t.gpu_data), size(t.size) { t.gpu_data = nullptr; }
+FrTensor::FrTensor(const string& filename) : gpu_data(nullptr), size((uint)(findsize(filename) / sizeof(Fr_t))) {
+    gpu_data = fr_alloc(size);
+    loadbin(filename, gpu_data, sizeof(Fr_t) * (size_t)size);
+}
+FrTensor::~FrTensor() {
+    if (gpu_data) zk_free(gpu_data);
+    gpu_data = nullptr;
+}
+
+FrTensor FrTensor::from_int_bin(const string& filename) {
+    size_t n = findsize(filename) / sizeof(int);
+    FrTensor out((uint)n);
+    DevBuf tmp(sizeof(int) * n);
+    loadbin(filename, tmp.p, sizeof(int) * n);
+    ZKC(zk_fr_from_i32(out.gpu_data, tmp.p, n, nullptr));
+    ZKC(zk_sync(nullptr));
+    return out;
+}
+// The reference loads only sizeof(int)*size bytes here (fr-tensor.cu:243-244); this reads all of them.
+FrTensor FrTensor::from_long_bin(const string& filename) {
+    size_t n = findsize(filename) / sizeof(long);
+    FrTensor out((uint)n);
+    DevBuf tmp(sizeof(long) * n);
+    loadbin(filename, tmp.p, sizeof(long) * n);
+    ZKC(zk_fr_from_i64(out.gpu_data, tmp.p, n, nullptr));
+    ZKC(zk_sync(nullptr));
+    return out;
+}
+void FrTensor::save(const string& filename) const { savebin(filename, gpu_data, sizeof(Fr_t) * (size_t)size); }
+void FrTensor::save_int(const string& filename) const {
+    DevBuf tmp(sizeof(int) * (size_t)size);
+    ZKC(zk_fr_to_i32(tmp.p, gpu_data, size, nullptr));
+    savebin(filename, tmp.p, sizeof(int) * (size_t)size);
+}
+void FrTensor::save_long(const string& filename) const {
+    DevBuf tmp(sizeof(long) * (size_t)size);
+    ZKC(zk_fr_to_i64(tmp.p, gpu_data, size, nullptr));
+    savebin(filename, tmp.p, sizeof(long) * (size_t)size);
+}
+
+Fr_t FrTensor::operator()(uint idx) const {
+    if (idx >= size) throw std::runtime_error("FrTensor::operator(): index out of range");
+    Fr_t out;
+    ZKC(zk_memcpy_d2h(&out, gpu_data + idx, sizeof(Fr_t), nullptr));
+    return out;
+}
+
+#define SAME_SIZE(t) if (size != (t).size) throw std::runtime_error("Incompatible dimensions")
+
+FrTensor FrTensor::operator+(const FrTensor& t) const { SAME_SIZE(t); FrTensor out(size); ZKC(zk_fr_add(out.gpu_data, gpu_data, t.gpu_data, size, nullptr)); return out; }
+FrTensor FrTensor::operator+(const Fr_t& x) const { FrTensor out(size); ZKC(zk_fr_add_s(out.gpu_data, gpu_data, x.val, size, nullptr)); return out; }
+FrTensor& FrTensor::operator+=(const FrTensor& t) { SAME_SIZE(t); ZKC(zk_fr_add(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator+=(const Fr_t& x) { ZKC(zk_fr_add_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
+FrTensor FrTensor::operator-() const { FrTensor out(size); ZKC(zk_fr_neg(out.gpu_data, gpu_data, size, nullptr)); return out; }
+FrTensor FrTensor::operator-(const FrTensor& t) const { SAME_SIZE(t); FrTensor out(size); ZKC(zk_fr_sub(out.gpu_data, gpu_data, t.gpu_data, size, nullptr)); return out; }
+FrTensor FrTensor::operator-(const Fr_t& x) const { FrTensor out(size); ZKC(zk_fr_sub_s(out.gpu_data, gpu_data, x.val, size, nullptr)); return out; }
+FrTensor& FrTensor::operator-=(const FrTensor& t) { SAME_SIZE(t); ZKC(zk_fr_sub(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator-=(const Fr_t& x) { ZKC(zk_fr_sub_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
+FrTensor& FrTensor::mont() { ZKC(zk_fr_mont(gpu_data, gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::unmont() { ZKC(zk_fr_unmont(gpu_data, gpu_data, size, nullptr)); return *this; }
+FrTensor FrTensor::operator*(const FrTensor& t) const { SAME_SIZE(t); FrTensor out(size); ZKC(zk_fr_mul(out.gpu_data, gpu_data, t.gpu_data, size, nullptr)); return out; }
+FrTensor FrTensor::operator*(const Fr_t& x) const { FrTensor out(size); ZKC(zk_fr_mul_s(out.gpu_data, gpu_data, x.val, size, nullptr)); return out; }
+FrTensor& FrTensor::operator*=(const FrTensor& t) { SAME_SIZE(t); ZKC(zk_fr_mul(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator*=(const Fr_t& x) { ZKC(zk_fr_mul_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator=(const FrTensor& t) {
+    if (size != t.size) throw std::runtime_error("operator=: Incompatible dimensions");
+    ZKC(zk_memcpy_d2d(gpu_data, t.gpu_data, sizeof(Fr_t) * (size_t)size, nullptr));
+    return *this;
+}
+
+Fr_t FrTensor::sum() const {
+    Fr_t out;
+    ZKC(zk_fr_sum(out.val, gpu_data, size, nullptr));
+    return out;
+}
+
+Fr_t FrTensor::operator()(const vector<Fr_t>& u) const {
+    uint log_dim = (uint)u.size();
+    if (size <= ((1u << log_dim) / 2) || size > (1u << log_dim)) throw std::runtime_error("Incompatible dimensions");
+    Fr_t out;
+    ZKC(zk_fr_me(out.val, gpu_data, size, u.empty() ? nullptr : u[0].val, (int)log_dim, nullptr));
+    return out;
+}
+
+// Folds `u.size()` levels of the middle axis, up to three levels per pass.
+static FrTensor fold_axis_all(const FrTensor& t, const vector<Fr_t>& u, uint cur_dim, size_t window) {
+    if (u.empty()) return t;
+    if ((size_t)t.size % ((size_t)cur_dim * window) != 0) throw std::runtime_error("t.size % (cur_dim * window_size) != 0");
+    const size_t other = (size_t)t.size / ((size_t)cur_dim * window);
+    const Fr_t* src = t.gpu_data;
+    std::vector<FrTensor> keep;   // intermediates stay alive until the last pass has been queued
+    size_t done = 0;
+    uint cur = cur_dim;
+    while (done < u.size()) {
+        const int L = (int)std::min<size_t>(3, u.size() - done);
+        const uint cur_out = (uint)(((uint64_t)cur + (1u << L) - 1) >> L);
+        keep.emplace_back((uint)(other * cur_out * window));
+        ZKC(zk_fr_fold_axis(keep.back().gpu_data, src, u[done].val, L, other, cur, window, nullptr));
+        src = keep.back().gpu_data;
+        cur = cur_out;
+        done += L;
+    }
+    FrTensor out(std::move(keep.back()));
+    return out;
+}
+
+// Deprecated window fold (fr-tensor.cu:512-516, :612-641): adjacent windows of the flat tensor,
+// zero-extended to a whole number of window pairs at every level.
+FrTensor FrTensor::partial_me(const vector<Fr_t>& u, uint window_size) const {
+    if (u.empty()) return *this;
+    if (size <= window_size * (1u << (u.size() - 1))) throw std::runtime_error("partial_me: Incompatible dimensions");
+    if (size % window_size == 0) return fold_axis_all(*this, u, size / window_size, window_size);
+    // ragged last window: the reference treats missing elements as zero, so pad the flat tensor first
+    const uint nwin = (size + window_size - 1) / window_size;
+    FrTensor padded = FrTensor::filled(nwin * window_size, Fr_t{{0, 0, 0, 0, 0, 0, 0, 0}});
+    ZKC(zk_memcpy_d2d(padded.gpu_data, gpu_data, sizeof(Fr_t) * (size_t)size, nullptr));
+    return fold_axis_all(padded, u, nwin, window_size);
+}
+
+FrTensor FrTensor::partial_me(const vector<Fr_t>& u, uint cur_dim, uint window_size) const {
+    if (cur_dim <= ((1u << u.size()) >> 1)) throw std::runtime_error("cur_dim <= ((1<<u.size()) >> 1)");
+    if (cur_dim > (1u << u.size())) throw std::runtime_error("cur_dim > (1<<u.size())");
+    return fold_axis_all(*this, u, cur_dim, window_size);
+}
+
+Fr_t FrTensor::multi_dim_me(const vector<vector<Fr_t>>& us, const vector<uint>& shape) const {
+    if (shape.size() != us.size()) throw std::runtime_error("Incompatible dimensions");
+    if (shape.size() == 0) return (*this)(0);
+    if (shape.size() == 1) return (*this)(us[0]);
+    FrTensor t_new = this->partial_me(us.back(), shape.back(), 1);
+    return t_new.multi_dim_me({us.begin(), us.end() - 1}, {shape.begin(), shape.end() - 1});
+}
+
+std::pair<FrTensor, FrTensor> FrTensor::split(uint window_size) const {
+    if (window_size < 1 || window_size >= size) throw std::runtime_error("Invalid window size.");
+    // even windows -> first, odd windows -> second (fr-tensor.cu:562-585); done with two strided gathers
+    uint num_window_in = (size + window_size - 1) / window_size;
+    uint num_window_out = (num_window_in + 1) / 2;
+    uint out_size = num_window_out * window_size;
+    std::vector<uint32_t> idx0(out_size), idx1(out_size);
+    FrTensor padded = FrTensor::filled(size + 1, Fr_t{{0, 0, 0, 0, 0, 0, 0, 0}});   // slot `size` reads as zero
+    ZKC(zk_memcpy_d2d(padded.gpu_data, gpu_data, sizeof(Fr_t) * (size_t)size, nullptr));
+    for (uint g = 0; g < out_size; ++g) {
+        uint w = g / window_size, j = g % window_size;
+        uint g0 = 2 * w * window_size + j, g1 = (2 * w + 1) * window_size + j;
+        idx0[g] = g0 < size ? g0 : size;
+        idx1[g] = g1 < size ? g1 : size;
+    }
+    DevBuf d0(sizeof(uint32_t) * (size_t)out_size), d1(sizeof(uint32_t) * (size_t)out_size);
+    ZKC(zk_memcpy_h2d(d0.p, idx0.data(), sizeof(uint32_t) * (size_t)out_size, nullptr));
+    ZKC(zk_memcpy_h2d(d1.p, idx1.data(), sizeof(uint32_t) * (size_t)out_size, nullptr));
+    std::pair<FrTensor, FrTensor> out{FrTensor(out_size), FrTensor(out_size)};
+    ZKC(zk_fr_gather(out.first.gpu_data, padded.gpu_data, d0.p, out_size, nullptr));
+    ZKC(zk_fr_gather(out.second.gpu_data, padded.gpu_data, d1.p, out_size, nullptr));
+    ZKC(zk_sync(nullptr));
+    return out;
+}
+
+FrTensor FrTensor::pad(const vector<uint>& shape, const Fr_t& pad_val) const {
+    size_t cum = 1;
+    for (auto& s : shape) cum *= s;
+    if (cum != size) throw std::runtime_error("pad: cum_shape != size");
+    uint last_dim = shape.back();
+    uint last_dim_padded = 1u << ceilLog2(last_dim);
+    FrTensor out((uint)((cum / last_dim) * last_dim_padded));
+    ZKC(zk_fr_pad(out.gpu_data, gpu_data, cum / last_dim, last_dim, last_dim_padded, pad_val.val, nullptr));
+    if (shape.size() == 1) return out;
+    vector<uint> shape_new(shape.begin(), shape.end() - 1);
+    shape_new.back() *= last_dim_padded;
+    return out.pad(shape_new, pad_val);
+}
+
+FrTensor FrTensor::transpose(uint M, uint N) const {
+    if (size != M * N) throw std::runtime_error("transpose: incompatible dimensions");
+    FrTensor out(N * M);
+    ZKC(zk_fr_transpose(out.gpu_data, gpu_data, M, N, nullptr));
+    return out;
+}
+
+FrTensor FrTensor::trunc(uint begin_idx, uint end_idx) const {
+    if (begin_idx >= end_idx || end_idx > size) throw std::runtime_error("trunc: invalid indices");
+    FrTensor out(end_idx - begin_idx);
+    ZKC(zk_memcpy_d2d(out.gpu_data, gpu_data + begin_idx, sizeof(Fr_t) * (size_t)out.size, nullptr));
+    return out;
+}
+
+FrTensor FrTensor::matmul(const FrTensor& x, const FrTensor& y, uint M, uint N, uint P) {
+    if (x.size != M * N || y.size != N * P) throw std::runtime_error("matmul: incompatible dimensions");
+    FrTensor out(M * P);
+    int path = 0;
+    ZKC(zk_fr_matmul(out.gpu_data, x.gpu_data, y.gpu_data, M, N, P, G().matmul_mode, &path, nullptr));
+    G().last_matmul_path = path;
+    return out;
+}
+
+// The reference draws these from cuRAND with a random_device seed (fr-tensor.cu:444-510); here they come
+// from the seedable host stream: same distributions, reproducible.
+FrTensor FrTensor::random_int(uint size, uint num_bits) {
+    ensure_seeded();
+    std::mt19937& mt = G().mt;
+    std::vector<long> v(size);
+    for (uint i = 0; i < size; ++i) v[i] = (long)((uint)mt() & ((1u << num_bits) - 1)) - (long)(1u << (num_bits - 1));
+    return FrTensor(size, v.data());
+}
+FrTensor FrTensor::random(uint size) {
+    vector<Fr_t> v = random_vec(size);
+    return FrTensor(size, v.data());
+}
+FrTensor FrTensor::filled(uint size, const Fr_t& x) {
+    FrTensor out(size);
+    ZKC(zk_fr_fill(out.gpu_data, x.val, size, nullptr));
+    return out;
+}
+
+ostream& operator<<(ostream& os, const FrTensor& A) {
+    os << '[';
+    for (uint i = 0; i + 1 < A.size; ++i) os << A(i) << '\n';
+    os << A(A.size - 1) << ']';
+    return os;
+}
+
+FrTensor catTensors(const vector<FrTensor>& vec) {
+    uint size = vec[0].size;
+    for (uint i = 1; i < vec.size(); i++)
+        if (vec[i].size != size) throw std::runtime_error("tensor size does not match!");
+    uint num = (uint)vec.size();
+    FrTensor out(num * size);
+    for (uint i = 0; i < num; i++)
+        ZKC(zk_memcpy_d2d(out.gpu_data + (size_t)i * size, vec[i].gpu_data, (size_t)size * sizeof(Fr_t), nullptr));
+    return out;
+}

@@ -1,0 +1,118 @@
+// FrTensor: owning device array of BLS12-381 scalars in standard form.  Public interface of the
+// reference class (fr-tensor.cuh:69-177) on top of the gfx950 C ABI (include/zkllm_hip.h).
+#pragma once
+#include <iomanip>
+#include <iostream>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+#include "bls12-381.hpp"
+
+using namespace std;
+
+ostream& operator<<(ostream& os, const Fr_t& x);
+
+// Challenge stream (fr-tensor.cu:16-24).  The reference seeds a fresh mt19937 from random_device on
+// every call; here one process-wide mt19937 serves all calls in order and can be seeded
+// (zk_seed_challenges, or ZKLLM_SEED in the environment) so that transcripts are reproducible.
+void zk_seed_challenges(uint32_t seed);
+vector<Fr_t> random_vec(uint len);
+uint ceilLog2(uint num);
+
+template <typename T>
+std::vector<T> concatenate(const std::vector<std::vector<T>>& vecs) {
+    std::vector<T> result;
+    size_t total = 0;
+    for (const auto& v : vecs) total += v.size();
+    result.reserve(total);
+    for (const auto& v : vecs) result.insert(result.end(), v.begin(), v.end());
+    return result;
+}
+
+// Matmul path selection: 0 = automatic (small-integer path when provably exact), 1 = generic
+// Montgomery only.  Also settable through ZKLLM_MATMUL=generic|auto.
+void zk_set_matmul_mode(int mode);
+int zk_last_matmul_path();
+
+// Optional transcript sink: when set, the protocol functions append every value a verifier would
+// receive (claims, round polynomials, openings).  Used for bit-exact parity checks.
+void zk_transcript_begin();
+const std::vector<Fr_t>& zk_transcript();
+void zk_transcript_end();
+void zk_record(const Fr_t& x);
+void zk_record(const std::vector<Fr_t>& xs);
+
+void zk_check(int rc, const char* where);   // throws std::runtime_error on a non-zero C-ABI status
+
+class FrTensor {
+   public:
+    Fr_t* gpu_data;
+    const uint size;
+
+    FrTensor(uint size);
+    FrTensor(uint size, const Fr_t* cpu_data);
+    FrTensor(uint size, const int* cpu_data);
+    FrTensor(uint size, const long* cpu_data);
+    FrTensor(uint size, const float* cpu_data, unsigned long scaling_factor);
+    FrTensor(uint size, const double* cpu_data, unsigned long scaling_factor);
+    FrTensor(const FrTensor& t);
+    FrTensor(FrTensor&& t) noexcept;
+    FrTensor(const string& filename);
+
+    static FrTensor from_int_bin(const string& filename);
+    static FrTensor from_long_bin(const string& filename);
+
+    ~FrTensor();
+
+    void save(const string& filename) const;
+    void save_int(const string& filename) const;
+    void save_long(const string& filename) const;
+
+    Fr_t operator()(uint idx) const;
+
+    FrTensor operator+(const FrTensor& t) const;
+    FrTensor operator+(const Fr_t& x) const;
+    FrTensor& operator+=(const FrTensor& t);
+    FrTensor& operator+=(const Fr_t& x);
+    FrTensor operator-() const;
+    FrTensor operator-(const FrTensor& t) const;
+    FrTensor operator-(const Fr_t& x) const;
+    FrTensor& operator-=(const FrTensor& t);
+    FrTensor& operator-=(const Fr_t& x);
+    FrTensor& mont();
+    FrTensor& unmont();
+    FrTensor operator*(const FrTensor& t) const;
+    FrTensor operator*(const Fr_t& x) const;
+    FrTensor& operator*=(const FrTensor& t);
+    FrTensor& operator*=(const Fr_t& x);
+    FrTensor& operator=(const FrTensor& x);
+
+    Fr_t sum() const;
+    Fr_t operator()(const vector<Fr_t>& u) const;
+    std::pair<FrTensor, FrTensor> split(uint window_size) const;
+    FrTensor partial_me(const vector<Fr_t>& u, uint window_size) const;
+    FrTensor partial_me(const vector<Fr_t>& u, uint cur_dim, uint window_size) const;
+    Fr_t multi_dim_me(const vector<vector<Fr_t>>& us, const vector<uint>& shape) const;
+    FrTensor pad(const vector<uint>& shape, const Fr_t& pad_val = {0, 0, 0, 0, 0, 0, 0, 0}) const;
+    FrTensor transpose(uint M, uint N) const;
+    FrTensor trunc(uint begin_idx, uint end_idx) const;
+
+    static FrTensor matmul(const FrTensor& x, const FrTensor& y, uint M, uint N, uint P);
+    static FrTensor random_int(uint size, uint num_bits);
+    static FrTensor random(uint size);
+    // all-`x` tensor (replaces the cudaMemset + `+= x` idiom of the reference's callers)
+    static FrTensor filled(uint size, const Fr_t& x);
+};
+
+ostream& operator<<(ostream& os, const FrTensor& A);
+FrTensor catTensors(const vector<FrTensor>& vec);
+
+// raw device buffer helper used by the lookup / rescaling code
+struct DevBuf {
+    void* p = nullptr;
+    explicit DevBuf(size_t bytes);
+    ~DevBuf();
+    DevBuf(const DevBuf&) = delete;
+    DevBuf& operator=(const DevBuf&) = delete;
+};

@@ -1,0 +1,180 @@
+// C entry points over the C++ class layer, for ctypes callers (the test-suite and bench.py):
+// tensors are opaque handles (FrTensor*), protocols run exactly as a C++ driver would run them, and
+// the recorded transcript can be read back for bit-exact comparison.
+#include <chrono>
+#include <cstring>
+#include <string>
+
+#include "../../include/zkllm_hip.h"
+#include "../csrc/field.hpp"
+#include "fr-tensor.hpp"
+#include "polynomial.hpp"
+#include "proof.hpp"
+#include "zkfc.hpp"
+
+typedef uint32_t u32;
+static thread_local std::string g_err;
+
+#define ZKP_TRY try {
+#define ZKP_END } catch (const std::exception& e) { g_err = e.what(); return 1; } return 0;
+#define ZKP_END_PTR } catch (const std::exception& e) { g_err = e.what(); return nullptr; }
+
+static FrTensor& FT(void* h) { return *reinterpret_cast<FrTensor*>(h); }
+static std::vector<Fr_t> frs(const u32* p, long n) { std::vector<Fr_t> v(n); if (n) memcpy(v.data(), p, (size_t)n * 32); return v; }
+
+extern "C" {
+
+const char* zkp_last_error() { return g_err.c_str(); }
+int zkp_init(int device) { ZKP_TRY zk_check(zk_init(device), "zk_init"); ZKP_END }
+void zkp_seed(u32 seed) { zk_seed_challenges(seed); }
+void zkp_set_matmul_mode(int mode) { zk_set_matmul_mode(mode); }
+int zkp_last_matmul_path() { return zk_last_matmul_path(); }
+void zkp_transcript_begin() { zk_transcript_begin(); }
+void zkp_transcript_end() { zk_transcript_end(); }
+long zkp_transcript_size() { return (long)zk_transcript().size(); }
+void zkp_transcript_get(u32* out) { if (!zk_transcript().empty()) memcpy(out, zk_transcript().data(), zk_transcript().size() * 32); }
+int zkp_sync() { ZKP_TRY zk_check(zk_sync(nullptr), "zk_sync"); ZKP_END }
+void zkp_random_vec(u32* out, u32 len) { auto v = random_vec(len); if (len) memcpy(out, v.data(), (size_t)len * 32); }
+
+// ---- host-side scalar arithmetic (the same field.hpp routines the kernels use, run on the CPU) ----
+// op: 0 add 1 sub 2 Montgomery product 3 double 4 to_mont 5 from_mont 6 inverse (Montgomery in/out)
+//     7 a*b standard 8 inverse standard 9 negate
+int zkp_host_fr_op(int op, const u32* a, const u32* b, u32* out, long n) {
+    ZKP_TRY
+    for (long i = 0; i < n; ++i) {
+        zk::Fr x, y, r;
+        memcpy(x.v, a + 8 * i, 32);
+        memcpy(y.v, b + 8 * i, 32);
+        switch (op) {
+            case 0: r = zk::add(x, y); break;
+            case 1: r = zk::sub(x, y); break;
+            case 2: r = zk::mont_mul(x, y); break;
+            case 3: r = zk::dbl(x); break;
+            case 4: r = zk::to_mont(x); break;
+            case 5: r = zk::from_mont(x); break;
+            case 6: r = zk::mont_inverse(x); break;
+            case 7: r = zk::fr_mul_std(x, y); break;
+            case 8: { Fr_t t; memcpy(t.val, x.v, 32); bool z = true; for (int k = 0; k < 8; ++k) z &= !t.val[k]; t = z ? t : inv(t); memcpy(r.v, t.val, 32); break; }
+            case 9: r = zk::neg(x); break;
+            default: throw std::runtime_error("bad op");
+        }
+        memcpy(out + 8 * i, r.v, 32);
+    }
+    ZKP_END
+}
+int zkp_host_fp_op(int op, const u32* a, const u32* b, u32* out, long n) {
+    ZKP_TRY
+    for (long i = 0; i < n; ++i) {
+        zk::Fp x, y, r;
+        memcpy(x.v, a + 12 * i, 48);
+        memcpy(y.v, b + 12 * i, 48);
+        switch (op) {
+            case 0: r = zk::add(x, y); break;
+            case 1: r = zk::sub(x, y); break;
+            case 2: r = zk::mont_mul(x, y); break;
+            case 3: r = zk::dbl(x); break;
+            case 4: r = zk::to_mont(x); break;
+            case 5: r = zk::from_mont(x); break;
+            case 6: r = zk::mont_inverse(x); break;
+            default: throw std::runtime_error("bad op");
+        }
+        memcpy(out + 12 * i, r.v, 48);
+    }
+    ZKP_END
+}
+int zkp_poly_eval(const u32* coefs, int ncoef, const u32* x, u32* out) {
+    ZKP_TRY
+    Polynomial p(frs(coefs, ncoef));
+    Fr_t xv; memcpy(xv.val, x, 32);
+    Fr_t r = p(xv);
+    memcpy(out, r.val, 32);
+    ZKP_END
+}
+
+// ---- tensor handles ------------------------------------------------------------------------------------
+void* zkp_fr_from_i32(const int32_t* p, u32 n) { ZKP_TRY return new FrTensor(n, (const int*)p); ZKP_END_PTR }
+void* zkp_fr_from_i64(const int64_t* p, u32 n) { ZKP_TRY return new FrTensor(n, (const long*)p); ZKP_END_PTR }
+void* zkp_fr_from_fr(const u32* p, u32 n) { ZKP_TRY return new FrTensor(n, (const Fr_t*)p); ZKP_END_PTR }
+void* zkp_fr_from_f32(const float* p, u32 n, uint64_t sf) { ZKP_TRY return new FrTensor(n, p, (unsigned long)sf); ZKP_END_PTR }
+void* zkp_fr_from_f64(const double* p, u32 n, uint64_t sf) { ZKP_TRY return new FrTensor(n, p, (unsigned long)sf); ZKP_END_PTR }
+void* zkp_fr_from_file(const char* path, int kind) {
+    ZKP_TRY
+    if (kind == 0) return new FrTensor(std::string(path));
+    if (kind == 1) return new FrTensor(FrTensor::from_int_bin(path));
+    return new FrTensor(FrTensor::from_long_bin(path));
+    ZKP_END_PTR
+}
+void zkp_fr_free(void* h) { delete reinterpret_cast<FrTensor*>(h); }
+u32 zkp_fr_size(void* h) { return FT(h).size; }
+void* zkp_fr_devptr(void* h) { return FT(h).gpu_data; }
+int zkp_fr_to_host(void* h, u32* out) { ZKP_TRY zk_check(zk_memcpy_d2h(out, FT(h).gpu_data, (size_t)FT(h).size * 32, nullptr), "d2h"); ZKP_END }
+int zkp_fr_save(void* h, const char* path, int kind) {
+    ZKP_TRY
+    if (kind == 0) FT(h).save(path); else if (kind == 1) FT(h).save_int(path); else FT(h).save_long(path);
+    ZKP_END
+}
+// binary op on tensors: 0 add 1 sub 2 mul; scalar variants take an 8-limb host scalar
+void* zkp_fr_binop(int op, void* a, void* b) {
+    ZKP_TRY
+    switch (op) {
+        case 0: return new FrTensor(FT(a) + FT(b));
+        case 1: return new FrTensor(FT(a) - FT(b));
+        case 2: return new FrTensor(FT(a) * FT(b));
+    }
+    throw std::runtime_error("bad op");
+    ZKP_END_PTR
+}
+void* zkp_fr_scalarop(int op, void* a, const u32* s) {
+    ZKP_TRY
+    Fr_t x; memcpy(x.val, s, 32);
+    switch (op) {
+        case 0: return new FrTensor(FT(a) + x);
+        case 1: return new FrTensor(FT(a) - x);
+        case 2: return new FrTensor(FT(a) * x);
+        case 3: return new FrTensor(-FT(a));
+        case 4: { auto* t = new FrTensor(FT(a)); t->mont(); return t; }
+        case 5: { auto* t = new FrTensor(FT(a)); t->unmont(); return t; }
+    }
+    throw std::runtime_error("bad op");
+    ZKP_END_PTR
+}
+int zkp_fr_sum(void* a, u32* out) { ZKP_TRY Fr_t s = FT(a).sum(); memcpy(out, s.val, 32); ZKP_END }
+int zkp_fr_me(void* a, const u32* u, int k, u32* out) { ZKP_TRY Fr_t s = FT(a)(frs(u, k)); memcpy(out, s.val, 32); ZKP_END }
+void* zkp_fr_partial_me(void* a, const u32* u, int k, u32 cur_dim, u32 window) { ZKP_TRY return new FrTensor(FT(a).partial_me(frs(u, k), cur_dim, window)); ZKP_END_PTR }
+void* zkp_fr_partial_me_window(void* a, const u32* u, int k, u32 window) { ZKP_TRY return new FrTensor(FT(a).partial_me(frs(u, k), window)); ZKP_END_PTR }
+int zkp_fr_multi_dim_me(void* a, const u32* us, const u32* lens, const u32* shape, int ndim, u32* out) {
+    ZKP_TRY
+    std::vector<std::vector<Fr_t>> uv; std::vector<uint> sh;
+    long off = 0;
+    for (int d = 0; d < ndim; ++d) { uv.push_back(frs(us + off * 8, lens[d])); off += lens[d]; sh.push_back(shape[d]); }
+    Fr_t s = FT(a).multi_dim_me(uv, sh);
+    memcpy(out, s.val, 32);
+    ZKP_END
+}
+void* zkp_fr_pad(void* a, const u32* shape, int ndim, const u32* pad_val) {
+    ZKP_TRY Fr_t pv; memcpy(pv.val, pad_val, 32); return new FrTensor(FT(a).pad(std::vector<uint>(shape, shape + ndim), pv)); ZKP_END_PTR
+}
+void* zkp_fr_transpose(void* a, u32 M, u32 N) { ZKP_TRY return new FrTensor(FT(a).transpose(M, N)); ZKP_END_PTR }
+void* zkp_fr_matmul(void* a, void* b, u32 M, u32 N, u32 P) { ZKP_TRY return new FrTensor(FrTensor::matmul(FT(a), FT(b), M, N, P)); ZKP_END_PTR }
+
+// ---- protocols ------------------------------------------------------------------------------------------
+// zkip with explicit challenges; proof_out: 3 coefficients per round
+int zkp_zkip(const u32* claim, void* a, void* b, const u32* u, int k, u32* proof_out, u32* final_claim) {
+    ZKP_TRY
+    Fr_t c; memcpy(c.val, claim, 32);
+    std::vector<Polynomial> proof;
+    Fr_t f = zkip(c, FT(a), FT(b), frs(u, k), proof);
+    for (size_t i = 0; i < proof.size(); ++i) memcpy(proof_out + i * 24, proof[i].coefficients().data(), 96);
+    memcpy(final_claim, f.val, 32);
+    ZKP_END
+}
+// zkFC::prove on existing tensors; challenges come from the seeded stream
+int zkp_zkfc_prove(void* X, void* W, void* Y, u32 in_dim, u32 out_dim, u32* claim_W) {
+    ZKP_TRY
+    zkFC fc(in_dim, out_dim, FT(W));
+    auto claims = fc.prove(FT(X), FT(Y));
+    if (claim_W) memcpy(claim_W, claims[0].claim.val, 32);
+    ZKP_END
+}
+
+}  // extern "C"

@@ -1,0 +1,117 @@
+#include "zkfc.hpp"
+
+#include "../../include/zkllm_hip.h"
+
+#define ZKC(call) zk_check((call), #call)
+
+static const Fr_t TEMP_ZERO{{0, 0, 0, 0, 0, 0, 0, 0}};
+static const Fr_t TEMP_ONE{{1, 0, 0, 0, 0, 0, 0, 0}};
+
+zkFC::zkFC(uint input_size, uint output_size, const FrTensor& weight)
+    : inputSize(input_size), outputSize(output_size), has_bias(false), weights(weight), bias(output_size) {
+    if (weight.size != input_size * output_size) throw std::runtime_error("weight size does not match");
+}
+zkFC::zkFC(uint input_size, uint output_size, const FrTensor& weight, const FrTensor& bias)
+    : inputSize(input_size), outputSize(output_size), has_bias(true), weights(weight), bias(bias) {
+    if (weight.size != input_size * output_size) throw std::runtime_error("weight size does not match");
+    if (bias.size != output_size) throw std::runtime_error("bias size does not match");
+}
+zkFC zkFC::from_float_gpu_ptr(uint in, uint out, unsigned long sf, float* weight_ptr, float* bias_ptr) {
+    FrTensor w(in * out), b(out);
+    ZKC(zk_fr_from_f32(w.gpu_data, weight_ptr, sf, (size_t)in * out, nullptr));
+    ZKC(zk_fr_from_f32(b.gpu_data, bias_ptr, sf * sf, out, nullptr));
+    return zkFC(in, out, w, b);
+}
+zkFC zkFC::from_float_gpu_ptr(uint in, uint out, unsigned long sf, float* weight_ptr) {
+    FrTensor w(in * out);
+    ZKC(zk_fr_from_f32(w.gpu_data, weight_ptr, sf, (size_t)in * out, nullptr));
+    return zkFC(in, out, w);
+}
+
+FrTensor zkFC::operator()(const FrTensor& X) const {
+    if (X.size % inputSize) throw std::runtime_error("input size does not match");
+    uint batchSize = X.size / inputSize;
+    FrTensor out = FrTensor::matmul(X, weights, batchSize, inputSize, outputSize);
+    if (has_bias) ZKC(zk_fr_bias_add(out.gpu_data, bias.gpu_data, batchSize, outputSize, nullptr));
+    return out;
+}
+
+// zkfc.cu:61-87.  Challenge order: u_batch, u_input, u_output.
+vector<Claim> zkFC::prove(const FrTensor& X, const FrTensor& Y) const {
+    if (has_bias) throw std::runtime_error("Cleaned-up version not implemented for zkFC with bias. Use zkFCStacked instead.");
+    uint batchSize = X.size / inputSize;
+    auto u_batch = random_vec(ceilLog2(batchSize));
+    auto u_input = random_vec(ceilLog2(inputSize));
+    auto u_output = random_vec(ceilLog2(outputSize));
+
+    auto claim = Y.multi_dim_me({u_batch, u_output}, {batchSize, outputSize});
+    zk_record(claim);
+    auto X_reduced = X.partial_me(u_batch, batchSize, inputSize);
+    auto W_reduced = weights.partial_me(u_output, outputSize, 1);
+    vector<Polynomial> proof;
+    auto final_claim = zkip(claim, X_reduced, W_reduced, u_input, proof);
+    // X(u_batch,u_input) and W(u_input,u_output) follow from the reduced vectors: folding X over the
+    // batch axis and then the input axis is the same multilinear evaluation as the reference's second
+    // pass over the full tensors (zkfc.cu:77-78), so the large tensors are not streamed again.
+    auto claim_X = X_reduced(u_input);
+    auto claim_W = W_reduced(u_input);
+    zk_record(final_claim);
+    zk_record(claim_X);
+    zk_record(claim_W);
+    if (claim_X * claim_W != final_claim) throw std::runtime_error("Claim does not match");
+    vector<Claim> claims;
+    claims.push_back({claim_W, vector<vector<Fr_t>>({u_input, u_output}), vector<uint>({inputSize, outputSize})});
+    return claims;
+}
+
+// zkfc.cu:129-151.  Rounds bind the most significant index bit first and consume u from the back.
+// The reference is only defined for u.size() <= ceilLog2(a.size); more challenges than index bits
+// would make it sum an empty tensor, so that case is rejected here.
+Fr_t zkip(const Fr_t& claim0, const FrTensor& a0, const FrTensor& b0, const vector<Fr_t>& u, vector<Polynomial>& proof) {
+    if (u.empty()) return claim0;
+    if (a0.size != b0.size) throw std::runtime_error("a.size != b.size");
+    if (u.size() > ceilLog2(a0.size)) throw std::runtime_error("zkip: more challenges than index bits");
+    Fr_t claim = claim0;
+    const FrTensor* a = &a0;
+    const FrTensor* b = &b0;
+    std::vector<FrTensor> keep;
+    keep.reserve(2 * u.size());
+    size_t k = u.size();
+    auto check_round = [&](Polynomial& p, const Fr_t& chal) {
+        proof.push_back(p);
+        zk_record(p.coefficients());
+        if (claim != p(TEMP_ZERO) + p(TEMP_ONE)) throw std::runtime_error("claim != p(0) + p(1)");
+        claim = p(chal);
+    };
+    while (k > 0) {
+        const uint n_in = a->size;
+        const uint bits = ceilLog2(n_in);
+        if (bits == k && bits <= 13) {
+            // the rest fits one workgroup: every remaining round in a single launch
+            std::vector<Fr_t> polys(3 * k);
+            Fr_t fin[2];
+            ZKC(zk_ip_sumcheck_small(polys[0].val, fin[0].val, a->gpu_data, b->gpu_data, n_in, u[0].val, (int)k, nullptr));
+            for (size_t r = 0; r < k; ++r) {
+                Polynomial p({polys[3 * r], polys[3 * r + 1], polys[3 * r + 2]});
+                check_round(p, u[k - 1 - r]);
+            }
+            return claim;
+        }
+        // long vectors: one launch for the three sums of the round, then the fold
+        const uint n_out = (1u << bits) >> 1;
+        Fr_t c[3];
+        ZKC(zk_ip_round(c[0].val, a->gpu_data, b->gpu_data, n_in, n_out, nullptr));
+        Polynomial p({c[0], c[1], c[2]});
+        check_round(p, u[k - 1]);
+        keep.emplace_back(n_out);
+        keep.emplace_back(n_out);
+        FrTensor& na = keep[keep.size() - 2];
+        FrTensor& nb = keep[keep.size() - 1];
+        ZKC(zk_fr_fold_halves(na.gpu_data, a->gpu_data, u[k - 1].val, n_in, n_out, nullptr));
+        ZKC(zk_fr_fold_halves(nb.gpu_data, b->gpu_data, u[k - 1].val, n_in, n_out, nullptr));
+        a = &na;
+        b = &nb;
+        --k;
+    }
+    return claim;
+}

@@ -1,0 +1,39 @@
+// Fully connected layer over Fr and its proof (zkfc.cuh:21-65).
+#pragma once
+#include "fr-tensor.hpp"
+#include "polynomial.hpp"
+#include "proof.hpp"
+
+class zkFC {
+   public:
+    const uint inputSize, outputSize;
+    bool has_bias;
+    FrTensor weights, bias;
+
+    zkFC(uint input_size, uint output_size, const FrTensor& weight);
+    zkFC(uint input_size, uint output_size, const FrTensor& weight, const FrTensor& bias);
+    FrTensor operator()(const FrTensor& X) const;
+    vector<Claim> prove(const FrTensor& X, const FrTensor& Y) const;
+
+    // weight_ptr / bias_ptr are device pointers to float data
+    static zkFC from_float_gpu_ptr(uint input_size, uint output_size, unsigned long scaling_factor, float* weight_ptr, float* bias_ptr);
+    static zkFC from_float_gpu_ptr(uint input_size, uint output_size, unsigned long scaling_factor, float* weight_ptr);
+};
+
+class zkFCStacked {
+   public:
+    bool has_bias;
+    const uint num;
+    const uint batchSize;
+    const uint inputSize;
+    const uint outputSize;
+
+    FrTensor X, W, b, Y;   // [num][batch][in], [num][in][out], [num][out], [num][batch][out]
+
+    zkFCStacked(bool has_bias, uint num, uint batch_size, uint input_size, uint output_size, const vector<zkFC>& layers, const vector<FrTensor>& Xs, const vector<FrTensor>& Ys);
+    void prove(vector<Polynomial>& proof) const;
+    void prove(const vector<Fr_t>& u_num, const vector<Fr_t>& v_num, const vector<Fr_t>& u_batch, const vector<Fr_t>& u_input, const vector<Fr_t>& u_output, vector<Polynomial>& proof) const;
+};
+
+Fr_t zkip(const Fr_t& claim, const FrTensor& a, const FrTensor& b, const vector<Fr_t>& u, vector<Polynomial>& proof);
+Fr_t zkip_stacked(const Fr_t& claim, const FrTensor& A, const FrTensor& B, const vector<Fr_t>& uN, const vector<Fr_t>& uD, const vector<Fr_t> vN, uint N, uint D, vector<Polynomial>& proof);
