@@ -100,6 +100,36 @@ int zk_ip_round(uint32_t* poly3_host, const void* a, const void* b, size_t n_in,
 /* all rounds of zkip (zkfc.cu:140-151) in one launch, n <= 8192 */
 int zk_ip_sumcheck_small(uint32_t* polys_host, uint32_t* fin_host, const void* a, const void* b, uint32_t n, const uint32_t* u, int k, void* stream);
 
+/* ---- G1 tensors (g1-tensor.cu) ------------------------------------------------------------------------ */
+int zk_g1_fill(void* out, const uint32_t* point36, size_t n, void* stream);               /* G1Jacobian_assign_broadcast :140 */
+int zk_g1_neg(void* out, const void* a, size_t n, void* stream);                          /* G1_jacobian_elementwise_minus :192 */
+int zk_g1_affine_neg(void* out, const void* a_affine, size_t n, void* stream);            /* G1_affine_elementwise_minus :105 */
+int zk_g1_affine_to_jacobian(void* out, const void* a_affine, size_t n, void* stream);    /* G1_affine_to_jacobian :154 */
+/* G1_jacobian_{elementwise,broadcast}_{add,sub} :207-320; b_count = n or 1 (b is a device pointer either way) */
+int zk_g1_add(void* out, const void* a, const void* b, size_t n, size_t b_count, int subtract, void* stream);
+/* G1_jacobian_{elementwise,broadcast}_{madd,msub}: b in affine form (96 B per point) */
+int zk_g1_madd(void* out, const void* a, const void* b_affine, size_t n, size_t b_count, int subtract, void* stream);
+/* out[i] = [s[i]] g[i % ng], s = Fr tensor read as 256-bit integers (G1_jacobian_elementwise_mul[_broadcast] :456-482) */
+int zk_g1_scalar_mul(void* out, const void* g, const void* s_fr, size_t ng, size_t n, void* stream);
+int zk_g1_sum(uint32_t* out_host36, const void* a, size_t n, void* stream);               /* G1TensorJacobian::sum :391-443 */
+int zk_g1_rowwise_sum(void* out, const void* in, size_t nrow, size_t ncol, void* stream); /* rowwise_sum :535-625 */
+int zk_g1_me(uint32_t* out_host36, const void* a, size_t n, const uint32_t* u, int k, void* stream);   /* G1_me :486-514 */
+/* (x/z^2, y/z^3, ONE); infinity -> all-zero limbs.  Not in the reference (it has no Fp inversion);
+ * used to compare and store points in a byte-stable form. */
+int zk_g1_normalize(void* out, const void* in, size_t n, void* stream);
+
+/* ---- Pedersen commitment (commitment.cu) ------------------------------------------------------------------ */
+/* Commitment::commit_int :31-58 -- out[row] = sum_j [t[row*ngen + j]] gens[j]; t holds embedded int32 values */
+int zk_g1_commit_int(void* out, const void* gens, const void* scalars_fr, size_t m, size_t ngen, void* stream);
+/* one round of Commitment::me_open (me_open_step :79-107 + the three G1 sums :125-127) */
+int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host108, const void* scalars, const void* gens, const uint32_t* u, size_t old_size, void* stream);
+
+/* ---- measurement helpers (no counterpart in the reference) ---------------------------------------- */
+/* v_mad_u64_u32 issue peak of the device: 16 independent chains per lane, no memory traffic */
+int zk_bench_mad_peak(uint32_t blocks, uint32_t iters, double* mad_per_s_host, void* stream);
+/* plain 16-byte-per-lane copy of known size, to scale profiler byte counters */
+int zk_bench_copy(void* dst, const void* src, size_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -126,16 +126,41 @@ class FrHandle:
             pass
 
 
+class G1Handle:
+    def __init__(self, pv, h):
+        if not h:
+            raise RuntimeError("prover error: " + pv.lib.zkp_last_error().decode())
+        self.pv, self.h = pv, h
+
+    @property
+    def size(self):
+        return self.pv.lib.zkp_g1_size(c_void_p(self.h))
+
+    def host(self):
+        out = np.zeros((self.size, 36), dtype=np.uint32)
+        self.pv.check(self.pv.lib.zkp_g1_to_host(c_void_p(self.h), _np_ptr(out)))
+        return out
+
+    def __del__(self):
+        try:
+            self.pv.lib.zkp_g1_free(c_void_p(self.h))
+        except Exception:
+            pass
+
+
 class Prover:
     def __init__(self, device=0):
         self.lib = pkg.load_prover()
         L = self.lib
         for name in ("zkp_fr_from_i32", "zkp_fr_from_i64", "zkp_fr_from_fr", "zkp_fr_from_f32", "zkp_fr_from_f64", "zkp_fr_from_file",
                      "zkp_fr_devptr", "zkp_fr_binop", "zkp_fr_scalarop", "zkp_fr_partial_me", "zkp_fr_partial_me_window",
-                     "zkp_fr_pad", "zkp_fr_transpose", "zkp_fr_matmul"):
+                     "zkp_fr_pad", "zkp_fr_transpose", "zkp_fr_matmul",
+                     "zkp_g1_from_host", "zkp_g1_from_file", "zkp_g1_devptr", "zkp_commitment_random", "zkp_g1_binop", "zkp_g1_pointop",
+                     "zkp_g1_scalar_mul", "zkp_g1_rowwise_sum", "zkp_commit_int", "zkp_commit"):
             getattr(L, name).restype = c_void_p
         L.zkp_transcript_size.restype = ctypes.c_long
         L.zkp_fr_size.restype = c_uint
+        L.zkp_g1_size.restype = c_uint
         self.check(L.zkp_init(c_int(device)))
 
     def check(self, rc):
@@ -210,6 +235,56 @@ class Prover:
 
     def matmul(self, a, b, M, N, P):
         return self.H(self.lib.zkp_fr_matmul(c_void_p(a.h), c_void_p(b.h), c_uint(M), c_uint(N), c_uint(P)))
+
+    # ---- G1 ----
+    def G(self, h):
+        return G1Handle(self, h)
+
+    def g1_from_host(self, pts):
+        pts = np.ascontiguousarray(pts, dtype=np.uint32).reshape(-1, 36)
+        return self.G(self.lib.zkp_g1_from_host(_np_ptr(pts), c_uint(pts.shape[0])))
+
+    def commitment_random(self, size):
+        return self.G(self.lib.zkp_commitment_random(c_uint(size)))
+
+    def g1_binop(self, op, a, b=None):
+        return self.G(self.lib.zkp_g1_binop(c_int(op), c_void_p(a.h), c_void_p(b.h if b is not None else a.h)))
+
+    def g1_pointop(self, op, a, p):
+        p = np.ascontiguousarray(p, dtype=np.uint32).reshape(36)
+        return self.G(self.lib.zkp_g1_pointop(c_int(op), c_void_p(a.h), _np_ptr(p)))
+
+    def g1_scalar_mul(self, g, s):
+        return self.G(self.lib.zkp_g1_scalar_mul(c_void_p(g.h), c_void_p(s.h)))
+
+    def g1_sum(self, a):
+        out = np.zeros(36, np.uint32)
+        self.check(self.lib.zkp_g1_sum(c_void_p(a.h), _np_ptr(out)))
+        return out
+
+    def g1_rowwise_sum(self, a, nrow, ncol):
+        return self.G(self.lib.zkp_g1_rowwise_sum(c_void_p(a.h), c_uint(nrow), c_uint(ncol)))
+
+    def g1_me(self, a, u):
+        u = np.ascontiguousarray(u, dtype=np.uint32).reshape(-1, 8)
+        out = np.zeros(36, np.uint32)
+        self.check(self.lib.zkp_g1_me(c_void_p(a.h), _np_ptr(u), c_int(u.shape[0]), _np_ptr(out)))
+        return out
+
+    def commit_int(self, gens, t):
+        return self.G(self.lib.zkp_commit_int(c_void_p(gens.h), c_void_p(t.h)))
+
+    def commit(self, gens, t):
+        return self.G(self.lib.zkp_commit(c_void_p(gens.h), c_void_p(t.h)))
+
+    def open(self, gens, t, com, u):
+        u = np.ascontiguousarray(u, dtype=np.uint32).reshape(-1, 8)
+        k = u.shape[0]
+        proof = np.zeros((3 * k + 1, 36), np.uint32)
+        npf = c_int(0)
+        val = np.zeros(8, np.uint32)
+        self.check(self.lib.zkp_open(c_void_p(gens.h), c_void_p(t.h), c_void_p(com.h), _np_ptr(u), c_int(k), _np_ptr(proof), ctypes.byref(npf), _np_ptr(val)))
+        return val, proof[:npf.value]
 
     # ---- transcript / challenges ----
     def seed(self, s):

@@ -1,0 +1,159 @@
+"""GPU parity: G1 tensor kernels, Pedersen commitment (fixed-base windowed MSM) and its opening, compared
+with the CPU oracle as group elements (both sides normalised to z = ONE, which makes them byte-equal)."""
+import random
+
+import numpy as np
+import pytest
+
+from zkhelp import (G1_X, G1_Y, P_MOD, R_MOD, affine_to_jac, ec_add, ec_mul, fr_array, fr_ints, jac_to_affine, load_oracle,
+                    mt_random_vec, orc_check)
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def pv():
+    from gpuhelp import Prover
+    return Prover()
+
+
+@pytest.fixture(scope="module")
+def orc():
+    return load_oracle()
+
+
+def norm(orc, pts):
+    pts = np.ascontiguousarray(pts, dtype=np.uint32).reshape(-1, 36)
+    out = np.zeros_like(pts)
+    orc_check(orc.orc_g1_op(3, pts, pts, out, pts.shape[0]))
+    return out
+
+
+def oracle_gens(orc, seed, n):
+    orc.orc_seed(seed)
+    g = np.zeros((n, 36), np.uint32)
+    orc_check(orc.orc_commitment_random(n, g))
+    return g
+
+
+def test_generators_match_oracle_stream(pv, orc):
+    pv.seed(321)
+    g = pv.commitment_random(8)
+    exp = oracle_gens(orc, 321, 8)
+    assert (norm(orc, g.host()) == norm(orc, exp)).all()
+    assert jac_to_affine(g.host()[0]) == ec_mul(fr_ints(mt_random_vec(np.random.RandomState(321), 1))[0], (G1_X, G1_Y))
+
+
+def test_elementwise_and_special_cases(pv, orc):
+    gens = oracle_gens(orc, 11, 16)
+    inf = np.zeros(36, np.uint32)
+    A = gens.copy()
+    B = gens[::-1].copy()
+    B[0] = A[0]                      # equal points -> doubling branch
+    neg = np.zeros_like(A[:1])
+    orc_check(orc.orc_g1_op(4, A[1:2].copy(), A[1:2].copy(), neg, 1))
+    B[1] = neg[0]                    # opposite points -> infinity
+    A[2] = inf                       # infinity + Q
+    B[3] = inf                       # P + infinity
+    hA, hB = pv.g1_from_host(A), pv.g1_from_host(B)
+    exp = np.zeros_like(A)
+    orc_check(orc.orc_g1_op(0, A, B, exp, 16))
+    got = pv.g1_binop(0, hA, hB).host()
+    assert (norm(orc, got) == norm(orc, exp)).all()
+    assert not norm(orc, got)[1].any()          # canonical infinity = all-zero limbs
+    # subtraction and negation
+    nb = np.zeros_like(B)
+    orc_check(orc.orc_g1_op(4, B, B, nb, 16))
+    orc_check(orc.orc_g1_op(0, A, nb, exp, 16))
+    assert (norm(orc, pv.g1_binop(1, hA, hB).host()) == norm(orc, exp)).all()
+    assert (norm(orc, pv.g1_binop(2, hB).host()) == norm(orc, nb)).all()
+    # device-side normalisation equals the oracle's
+    assert (pv.g1_binop(3, hA).host() == norm(orc, A)).all()
+    # broadcast add / mixed add of one point
+    P = gens[5]
+    Pb = np.tile(P, (16, 1))
+    orc_check(orc.orc_g1_op(0, A, Pb, exp, 16))
+    assert (norm(orc, pv.g1_pointop(0, hA, P).host()) == norm(orc, exp)).all()
+    Pn = norm(orc, P)[0]
+    assert (norm(orc, pv.g1_pointop(2, hA, Pn).host()) == norm(orc, exp)).all()
+
+
+def test_scalar_mul_sum_rowsum_me(pv, orc):
+    gens = oracle_gens(orc, 12, 8)
+    rng = random.Random(3)
+    ks = [0, 1, 2, R_MOD - 1, 2 ** 31 - 1] + [rng.randrange(R_MOD) for _ in range(19)]   # 24 = 3 x 8 scalars, broadcast over the generators
+    S = fr_array(ks)
+    exp = np.zeros((24, 36), np.uint32)
+    orc_check(orc.orc_g1_mul(gens, 8, S, exp, 24, 0))
+    hG, hS = pv.g1_from_host(gens), pv.from_fr(S)
+    got = pv.g1_scalar_mul(hG, hS)
+    assert (norm(orc, got.host()) == norm(orc, exp)).all()
+    tot = np.zeros(36, np.uint32)
+    orc_check(orc.orc_g1_sum(exp, 24, tot))
+    assert (norm(orc, pv.g1_sum(got)) == norm(orc, tot)).all()
+    rows = np.zeros((3, 36), np.uint32)
+    for r in range(3):
+        orc_check(orc.orc_g1_sum(exp[8 * r:8 * r + 8].copy(), 8, rows[r]))
+    assert (norm(orc, pv.g1_rowwise_sum(got, 3, 8).host()) == norm(orc, rows)).all()
+    u = mt_random_vec(np.random.RandomState(4), 3)
+    me = np.zeros(36, np.uint32)
+    orc_check(orc.orc_g1_me(gens, 8, u, 3, me))
+    assert (norm(orc, pv.g1_me(hG, u)) == norm(orc, me)).all()
+    # larger sum exercising the segmented reduction
+    big = np.tile(gens, (200, 1))[:1500]
+    orc_check(orc.orc_g1_sum(big, 1500, tot))
+    assert (norm(orc, pv.g1_sum(pv.g1_from_host(big))) == norm(orc, tot)).all()
+
+
+@pytest.mark.parametrize("m,n,lim", [(1, 1, 100), (3, 4, 2 ** 15), (16, 64, 2 ** 14), (5, 64, 2 ** 31 - 1), (300, 32, 2 ** 13)])
+def test_commit_int_matches_oracle(pv, orc, m, n, lim):
+    print("case", m, n, lim, flush=True)
+    gens = oracle_gens(orc, 13 + n, n)
+    rng = np.random.default_rng(m * n)
+    t = rng.integers(-lim, lim, m * n, endpoint=True).astype(np.int64)
+    t[0] = 0
+    if m * n > 2:
+        t[1], t[2] = lim, -lim
+    T = fr_array([int(x) % R_MOD for x in t])
+    exp = np.zeros((m, 36), np.uint32)
+    orc_check(orc.orc_commit_int(gens, n, T, m * n, exp))
+    got = pv.commit_int(pv.g1_from_host(gens), pv.from_fr(T)).host()
+    assert (norm(orc, got) == norm(orc, exp)).all()
+
+
+def test_commit_int_rejects_non_integer_scalars_and_is_linear(pv, orc):
+    gens = oracle_gens(orc, 14, 8)
+    hG = pv.g1_from_host(gens)
+    bad = fr_array([R_MOD >> 1] * 8)
+    with pytest.raises(RuntimeError, match="int32"):
+        pv.commit_int(hG, pv.from_fr(bad))
+    rng = np.random.default_rng(9)
+    a, b = rng.integers(-1000, 1000, 8), rng.integers(-1000, 1000, 8)
+    ca = jac_to_affine(pv.commit_int(hG, pv.from_i32(a)).host()[0])
+    cb = jac_to_affine(pv.commit_int(hG, pv.from_i32(b)).host()[0])
+    cab = jac_to_affine(pv.commit_int(hG, pv.from_i32(a + b)).host()[0])
+    assert ec_add(ca, cb) == cab
+    # the general-scalar commit agrees with commit_int on integers
+    assert jac_to_affine(pv.commit(hG, pv.from_i32(a)).host()[0]) == ca
+
+
+@pytest.mark.parametrize("n,m", [(4, 2), (8, 1), (16, 4), (5, 3)])
+def test_open_value_and_g1_transcript(pv, orc, n, m):
+    gens = oracle_gens(orc, 15 + n, n)
+    rng = np.random.default_rng(n * m)
+    t = rng.integers(-2 ** 15, 2 ** 15, m * n).astype(np.int64)
+    T = fr_array([int(x) % R_MOD for x in t])
+    k = (n - 1).bit_length() + (m - 1).bit_length()
+    u = mt_random_vec(np.random.RandomState(16), k)
+    exp_proof = np.zeros((3 * (n - 1).bit_length() + 1, 36), np.uint32)
+    exp_val = np.zeros(8, np.uint32)
+    # rows are padded to a power of two exactly as verifyWeightClaim pads the weight
+    mp = 1 << (m - 1).bit_length()
+    Tp = np.concatenate([T, np.zeros(((mp - m) * n, 8), np.uint32)])
+    orc_check(orc.orc_open(gens, n, Tp, mp * n, mp, u, k, exp_proof, exp_val))
+    hG, hT = pv.g1_from_host(gens), pv.from_fr(Tp)
+    com = pv.commit_int(hG, hT)
+    val, proof = pv.open(hG, hT, com, u)
+    assert (val == exp_val).all()
+    assert proof.shape == exp_proof.shape
+    assert (norm(orc, proof) == norm(orc, exp_proof)).all()

@@ -1,0 +1,98 @@
+#include "commitment.hpp"
+
+#include <cstdlib>
+
+#include "../../include/zkllm_hip.h"
+
+#define ZKC(call) zk_check((call), #call)
+
+static bool g_skip_g1 = [] { const char* e = getenv("ZKLLM_SKIP_G1_OPENING"); return e && e[0] == '1'; }();
+void zk_set_skip_g1_opening(bool skip) { g_skip_g1 = skip; }
+
+// generators [s_i]G with s_i from the (seedable) challenge stream; the reference draws s_i from cuRAND
+// (commitment.cu:3-8, fr-tensor.cu:479-510)
+Commitment Commitment::random(uint size) {
+    Commitment out(size, G1Jacobian_generator);
+    out *= FrTensor::random(size);
+    return out;
+}
+
+G1TensorJacobian Commitment::commit(const FrTensor& t) const {
+    if (t.size % size != 0) throw std::runtime_error("Commitment::commit - Incompatible dimensions");
+    uint m = t.size / size;
+    G1TensorJacobian temp = (*this) * t;
+    return temp.rowwise_sum(m, size);
+}
+
+G1TensorJacobian Commitment::commit_int(const FrTensor& t) const {
+    if (t.size % size != 0) throw std::runtime_error("Commitment::commit_int - Incompatible dimensions");
+    uint m = t.size / size;
+    G1TensorJacobian out(m);
+    ZKC(zk_g1_commit_int(out.gpu_data, gpu_data, t.gpu_data, m, size, nullptr));
+    return out;
+}
+
+G1TensorJacobian Commitment::commit_int_multi(const vector<FrTensor>& ts) const {
+    uint num_row = 0;
+    for (auto& t : ts) {
+        if (t.size % size != 0) throw std::runtime_error("Commitment::commit_int_multi - Incompatible dimensions");
+        num_row += t.size / size;
+    }
+    G1TensorJacobian out(num_row);
+    uint row = 0;
+    for (auto& t : ts) {
+        uint m = t.size / size;
+        ZKC(zk_g1_commit_int(out.gpu_data + row, gpu_data, t.gpu_data, m, size, nullptr));
+        row += m;
+    }
+    return out;
+}
+
+Fr_t Commitment::me_open(const FrTensor& t, const Commitment& generators, vector<Fr_t>::const_iterator begin, vector<Fr_t>::const_iterator end, vector<G1Jacobian_t>& proof) {
+    if (t.size != generators.size) throw std::runtime_error("Commitment::me_open - Incompatible dimensions " + std::to_string(t.size) + " " + std::to_string(generators.size));
+    const FrTensor* s = &t;
+    const G1TensorJacobian* g = &generators;
+    std::vector<FrTensor> ks;
+    std::vector<G1TensorJacobian> kg;
+    ks.reserve(end - begin);
+    kg.reserve(end - begin);
+    for (auto it = begin; it < end; ++it) {
+        const uint new_size = (s->size + 1) / 2;
+        ks.emplace_back(new_size);
+        kg.emplace_back(new_size);
+        G1Jacobian_t sums[3];
+        ZKC(zk_g1_open_round(ks.back().gpu_data, kg.back().gpu_data, sums[0].x.val, s->gpu_data, g->gpu_data, it->val, s->size, nullptr));
+        proof.push_back(sums[0]);
+        proof.push_back(sums[1]);
+        proof.push_back(sums[2]);
+        s = &ks.back();
+        g = &kg.back();
+    }
+    proof.push_back((*g)(0u));
+    return (*s)(0u);
+}
+
+Fr_t Commitment::open(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u, vector<G1Jacobian_t>& proof) const {
+    const uint k_out = ceilLog2(com.size);
+    if (u.size() < k_out) throw std::runtime_error("Commitment::open - too few challenges");
+    const vector<Fr_t> u_out(u.end() - k_out, u.end());
+    const vector<Fr_t> u_in(u.begin(), u.end() - k_out);
+    // The reference also evaluates com(u_out) here and never uses it (commitment.cu:137); omitted.
+    FrTensor folded = u_out.empty() ? FrTensor(t) : t.partial_me(u_out, t.size / com.size);
+    if (g_skip_g1) {
+        if (folded.size != size) throw std::runtime_error("Commitment::me_open - Incompatible dimensions");
+        return folded(u_in);
+    }
+    return me_open(folded, *this, u_in.begin(), u_in.end(), proof);
+}
+Fr_t Commitment::open(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u) const {
+    vector<G1Jacobian_t> proof;
+    return open(t, com, u, proof);
+}
+
+Weight create_weight(string generator_filename, string weight_filename, string com_filename, uint in_dim, uint out_dim) {
+    Commitment generator(generator_filename);
+    FrTensor weight = FrTensor::from_int_bin(weight_filename);
+    G1TensorJacobian com(com_filename);
+    return {generator, weight, com, in_dim, out_dim};
+}

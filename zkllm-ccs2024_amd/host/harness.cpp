@@ -11,6 +11,8 @@
 #include "polynomial.hpp"
 #include "proof.hpp"
 #include "zkfc.hpp"
+#include "g1-tensor.hpp"
+#include "commitment.hpp"
 
 typedef uint32_t u32;
 static thread_local std::string g_err;
@@ -19,6 +21,8 @@ static thread_local std::string g_err;
 #define ZKP_END } catch (const std::exception& e) { g_err = e.what(); return 1; } return 0;
 #define ZKP_END_PTR } catch (const std::exception& e) { g_err = e.what(); return nullptr; }
 
+// every G1 handle is a Commitment (it adds no members to G1TensorJacobian), so any tensor can act as generators
+static Commitment& GT(void* h) { return *reinterpret_cast<Commitment*>(h); }
 static FrTensor& FT(void* h) { return *reinterpret_cast<FrTensor*>(h); }
 static std::vector<Fr_t> frs(const u32* p, long n) { std::vector<Fr_t> v(n); if (n) memcpy(v.data(), p, (size_t)n * 32); return v; }
 
@@ -176,5 +180,66 @@ int zkp_zkfc_prove(void* X, void* W, void* Y, u32 in_dim, u32 out_dim, u32* clai
     if (claim_W) memcpy(claim_W, claims[0].claim.val, 32);
     ZKP_END
 }
+
+// ---- G1 tensors / commitment ---------------------------------------------------------------------------------
+void* zkp_g1_from_host(const u32* pts, u32 n) { ZKP_TRY return new Commitment(G1TensorJacobian(n, (const G1Jacobian_t*)pts)); ZKP_END_PTR }
+void* zkp_g1_from_file(const char* path) { ZKP_TRY return new Commitment(G1TensorJacobian(std::string(path))); ZKP_END_PTR }
+void zkp_g1_free(void* h) { delete reinterpret_cast<Commitment*>(h); }
+u32 zkp_g1_size(void* h) { return GT(h).size; }
+void* zkp_g1_devptr(void* h) { return GT(h).gpu_data; }
+int zkp_g1_to_host(void* h, u32* out) { ZKP_TRY zk_check(zk_memcpy_d2h(out, GT(h).gpu_data, (size_t)GT(h).size * 144, nullptr), "d2h"); ZKP_END }
+int zkp_g1_save(void* h, const char* path) { ZKP_TRY GT(h).save(path); ZKP_END }
+void* zkp_commitment_random(u32 size) { ZKP_TRY return new Commitment(Commitment::random(size)); ZKP_END_PTR }
+// op: 0 a+b, 1 a-b, 2 -a, 3 normalized(a)
+void* zkp_g1_binop(int op, void* a, void* b) {
+    ZKP_TRY
+    switch (op) {
+        case 0: return new Commitment(GT(a) + GT(b));
+        case 1: return new Commitment(GT(a) - GT(b));
+        case 2: return new Commitment(-GT(a));
+        case 3: return new Commitment(GT(a).normalized());
+    }
+    throw std::runtime_error("bad op");
+    ZKP_END_PTR
+}
+// broadcast: op 0 a + p, 1 a - p (p = one Jacobian point on the host); op 2/3 same with p affine (first 24 limbs)
+void* zkp_g1_pointop(int op, void* a, const u32* p) {
+    ZKP_TRY
+    G1Jacobian_t j; memcpy(&j, p, 144);
+    G1Affine_t af; memcpy(&af, p, 96);
+    switch (op) {
+        case 0: return new Commitment(GT(a) + j);
+        case 1: return new Commitment(GT(a) - j);
+        case 2: return new Commitment(GT(a) + af);
+        case 3: return new Commitment(GT(a) - af);
+    }
+    throw std::runtime_error("bad op");
+    ZKP_END_PTR
+}
+void* zkp_g1_scalar_mul(void* g, void* s) { ZKP_TRY return new Commitment(GT(g) * FT(s)); ZKP_END_PTR }
+int zkp_g1_sum(void* a, u32* out) { ZKP_TRY G1Jacobian_t s = GT(a).sum(); memcpy(out, &s, 144); ZKP_END }
+void* zkp_g1_rowwise_sum(void* a, u32 nrow, u32 ncol) { ZKP_TRY return new Commitment(GT(a).rowwise_sum(nrow, ncol)); ZKP_END_PTR }
+int zkp_g1_me(void* a, const u32* u, int k, u32* out) { ZKP_TRY G1Jacobian_t s = GT(a)(frs(u, k)); memcpy(out, &s, 144); ZKP_END }
+void* zkp_commit_int(void* gens, void* t) {
+    ZKP_TRY
+    return new Commitment(GT(gens).commit_int(FT(t)));
+    ZKP_END_PTR
+}
+void* zkp_commit(void* gens, void* t) {
+    ZKP_TRY
+    return new Commitment(GT(gens).commit(FT(t)));
+    ZKP_END_PTR
+}
+// Commitment::open; proof_out must hold 3*k+1 points; *nproof receives the count
+int zkp_open(void* gens, void* t, void* com, const u32* u, int k, u32* proof_out, int* nproof, u32* value) {
+    ZKP_TRY
+    std::vector<G1Jacobian_t> proof;
+    Fr_t v = GT(gens).open(FT(t), GT(com), frs(u, k), proof);
+    if (proof_out && !proof.empty()) memcpy(proof_out, proof.data(), proof.size() * 144);
+    if (nproof) *nproof = (int)proof.size();
+    memcpy(value, v.val, 32);
+    ZKP_END
+}
+void zkp_set_skip_g1_opening(int skip) { zk_set_skip_g1_opening(skip != 0); }
 
 }  // extern "C"
