@@ -97,6 +97,8 @@ int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, 
 
 /* ---- inner-product sumcheck (zkip_poly_kernel + 3 sums, zkfc.cu:94-138) ----------------------------- */
 int zk_ip_round(uint32_t* poly3_host, const void* a, const void* b, size_t n_in, size_t n_out, void* stream);
+/* zkip_stacked_step_poly (zkfc.cu:187-209): halves over the stacking axis of [N][D] tensors, rows weighted by the eq table E */
+int zk_ip_round_stacked(uint32_t* poly3_host, const void* a, const void* b, const void* E, size_t D, size_t rows_in, size_t rows_out, void* stream);
 /* all rounds of zkip (zkfc.cu:140-151) in one launch, n <= 8192 */
 int zk_ip_sumcheck_small(uint32_t* polys_host, uint32_t* fin_host, const void* a, const void* b, uint32_t n, const uint32_t* u, int k, void* stream);
 
@@ -123,6 +125,36 @@ int zk_g1_normalize(void* out, const void* in, size_t n, void* stream);
 int zk_g1_commit_int(void* out, const void* gens, const void* scalars_fr, size_t m, size_t ngen, void* stream);
 /* one round of Commitment::me_open (me_open_step :79-107 + the three G1 sums :125-127) */
 int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host108, const void* scalars, const void* gens, const uint32_t* u, size_t old_size, void* stream);
+
+/* ---- lookup argument (tlookup.cu) ------------------------------------------------------------------------ */
+/* idx = val - low as a table index (lookuprange_tensor_prep_kernel :414-421 / lookuprange_prep_kernel :393-400);
+ * unlike the reference, a value outside [low, low+table_size) is an error instead of an unchecked access */
+int zk_lookup_index_fr(void* idx_u32, const void* vals_fr, int32_t low, uint32_t table_size, size_t n, void* stream);
+int zk_lookup_index_i32(void* idx_u32, const void* vals_i32, int32_t low, uint32_t table_size, size_t n, void* stream);
+/* multiplicities (tlookup_kernel :10-15): counts[b] = #{i : idx[i] == b}; counts is cleared first */
+int zk_lookup_hist(void* counts_u32, const void* idx_u32, size_t n, uint32_t nbins, void* stream);
+int zk_range_table(void* table_fr, int32_t low, uint32_t len, uint32_t table_size, void* stream);   /* tlookuprange_init_kernel :372-380 */
+/* out[i] = 1/(in[i]+beta) (tlookup_inv_kernel :50-62), by batch inversion */
+int zk_fr_batch_inv(void* out, const void* in, const uint32_t* beta, size_t n, void* stream);
+/* eq(u, t) for t < 2^k in Montgomery form; zk_eq_halve drops the top variable */
+int zk_eq_table(void* out, const uint32_t* u, int k, void* stream);
+int zk_eq_halve(void* out, const void* in, size_t n_out, void* stream);
+/* one sumcheck round: every sum of tLookup_phase1_step_poly :184-200 / tLookup_phase2_step_poly :245-279 plus the
+ * folds of tLookup_phase1_reduce_kernel :94-103 / tLookup_phase2_reduce_kernel :161-175.
+ * sums_host (standard form): [E.(a0 s0), E.(da s0 + a0 ds), E.(da ds), sum a0, sum da] and, in phase 2,
+ * the same three for (B,T) followed by [sum m0 b0, sum (dm b0 + m0 db), sum dm db];  s0 = S + beta, E = eq table. */
+int zk_lookup_round(uint32_t* sums_host, void* new_A, void* new_S, void* new_B, void* new_T, void* new_m,
+                    const void* A, const void* S, const void* B, const void* T, const void* m, const void* E,
+                    const uint32_t* beta, const uint32_t* v, size_t n_out, int phase2, void* stream);
+/* one round of multi_hadamard_sumchecks (proof.cu:191-241) for K <= 4 tensors */
+int zk_hadamard_round(uint32_t* coefs_host, void* const* new_Xs, const void* const* Xs, int K, const void* E, const uint32_t* v, size_t n_out, void* stream);
+
+/* ---- rescaling / softmax ------------------------------------------------------------------------------------------ */
+int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* stream);       /* rescaling_kernel rescaling.cu:8-21 */
+/* zksoftmax_shift zksoftmax.cu:20-32 (scale = sf_in*sqrt(d)), zksoftmax_calculate_table :4-14, zksoftmax_decompose_kernel :95-109 */
+int zk_softmax_shift(void* shift, void* out_shifted, const void* X, uint32_t rows, uint32_t cols, double scale, void* stream);
+int zk_softmax_table(void* table, double log_theta, double step, uint32_t len, void* stream);
+int zk_softmax_decompose(void* planes, const void* X_shifted, const uint32_t* bs_host, int K, size_t n, void* stream);
 
 /* ---- measurement helpers (no counterpart in the reference) ---------------------------------------- */
 /* v_mad_u64_u32 issue peak of the device: 16 independent chains per lane, no memory traffic */

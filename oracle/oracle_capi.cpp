@@ -269,6 +269,9 @@ int orc_softmax(const u32* X, u32 m, u32 n, u32 d, const u32* bs, int K, u32 L, 
     ORC_END
 }
 
+// deterministic exp / log used by the softmax steps (kind 0 exp, 1 log)
+void orc_detmath(int kind, const double* x, double* out, long n) { for (long i = 0; i < n; ++i) out[i] = kind ? o_log(x[i]) : o_exp(x[i]); }
+
 // ---- commitment ----------------------------------------------------------------------------------------
 int orc_commitment_random(u32 size, u32* gens_out) { ORC_TRY g1_out(commitment_random(size), gens_out); ORC_END }
 int orc_commit_int(const u32* gens, long ngen, const u32* t, long n, u32* com_out) {

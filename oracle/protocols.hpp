@@ -11,11 +11,13 @@
 // G1 results are group elements: the reference's reduction trees fix a particular Jacobian
 // triple, which no other summation order reproduces, so sums here are sequential and callers
 // compare through g1_equal / g1_normalize.
-// Floating point (softmax shift and exp tables) is evaluated with the host libm in double;
-// parity for those two steps is unpinned against an NVIDIA run (device libm differs in the
-// last ulp) and pinned only between this file and the product's own host evaluation.
+// Floating point (softmax shift and exp tables): PARITY UNPINNED against the reference, whose CUDA
+// device libm cannot be reproduced; both steps follow the fixed recipe of detmath_ref.hpp instead,
+// and the row sum of exponentials is taken in a fixed order (64 strided partial sums combined by the
+// butterfly i ^ 32, 16, ..., 1), which is what the product's kernel does.
 #pragma once
 #include <cmath>
+#include "detmath_ref.hpp"
 #include "tensor.hpp"
 
 namespace orc {
@@ -244,7 +246,7 @@ struct ZkSoftmax {
             FrVec mv(bs[i]);
             const double theta_k = thetas[i - L], sfd = (double)sf_in, dd = (double)d, Bk = (double)Bs[i];
             for (uint x = 0; x < bs[i]; ++x) {
-                uint64_t r = (uint64_t)(std::exp(std::log(theta_k) - (Bk / (sfd * std::sqrt(dd))) * x) + 0.5);
+                uint64_t r = (uint64_t)(o_exp(o_log(theta_k) - (Bk / (sfd * std::sqrt(dd))) * (double)x) + 0.5);
                 mv[x] = fr_from_u64(r);
             }
             others.emplace_back(0, bs[i], mv);
@@ -260,9 +262,19 @@ struct ZkSoftmax {
         const double sfd = (double)sf_in, dd = (double)d;
         #pragma omp parallel for
         for (long r = 0; r < (long)m; ++r) {
-            double t = 0.0;
-            for (uint i = 0; i < n; ++i) t += std::exp((double)fr_to_i64(X[r * n + i]) / (sfd * std::sqrt(dd)));
-            shift[r] = fr_from_f64(sfd * std::sqrt(dd) * std::log(t), 1);
+            const double scale = sfd * std::sqrt(dd);
+            double part[64];
+            for (int l = 0; l < 64; ++l) {
+                double acc = 0.0;
+                for (uint i = l; i < n; i += 64) acc = acc + o_exp((double)fr_to_i64(X[r * n + i]) / scale);
+                part[l] = acc;
+            }
+            for (int off = 32; off >= 1; off >>= 1) {
+                double nxt[64];
+                for (int l = 0; l < 64; ++l) nxt[l] = part[l] + part[l ^ off];
+                for (int l = 0; l < 64; ++l) part[l] = nxt[l];
+            }
+            shift[r] = fr_from_f64(scale * o_log(part[0]), 1);
             for (uint i = 0; i < n; ++i) Xs[r * n + i] = sub(X[r * n + i], shift[r]);
         }
         const size_t N = X.size();

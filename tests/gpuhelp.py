@@ -156,7 +156,8 @@ class Prover:
                      "zkp_fr_devptr", "zkp_fr_binop", "zkp_fr_scalarop", "zkp_fr_partial_me", "zkp_fr_partial_me_window",
                      "zkp_fr_pad", "zkp_fr_transpose", "zkp_fr_matmul",
                      "zkp_g1_from_host", "zkp_g1_from_file", "zkp_g1_devptr", "zkp_commitment_random", "zkp_g1_binop", "zkp_g1_pointop",
-                     "zkp_g1_scalar_mul", "zkp_g1_rowwise_sum", "zkp_commit_int", "zkp_commit"):
+                     "zkp_g1_scalar_mul", "zkp_g1_rowwise_sum", "zkp_commit_int", "zkp_commit",
+                     "zkp_rescale", "zkp_rescale_prove", "zkp_range_prep", "zkp_batch_inv", "zkp_softmax"):
             getattr(L, name).restype = c_void_p
         L.zkp_transcript_size.restype = ctypes.c_long
         L.zkp_fr_size.restype = c_uint
@@ -285,6 +286,75 @@ class Prover:
         val = np.zeros(8, np.uint32)
         self.check(self.lib.zkp_open(c_void_p(gens.h), c_void_p(t.h), c_void_p(com.h), _np_ptr(u), c_int(k), _np_ptr(proof), ctypes.byref(npf), _np_ptr(val)))
         return val, proof[:npf.value]
+
+    # ---- lookup / rescaling / softmax ----
+    def rescale(self, X, sf):
+        rem = c_void_p()
+        out = self.H(self.lib.zkp_rescale(c_void_p(X.h), c_uint(sf), ctypes.byref(rem)))
+        return out, self.H(rem.value)
+
+    def rescale_prove(self, X, sf):
+        return self.H(self.lib.zkp_rescale_prove(c_void_p(X.h), c_uint(sf)))
+
+    def range_prep(self, vals, low, length):
+        return self.H(self.lib.zkp_range_prep(c_void_p(vals.h), c_int(low), c_uint(length)))
+
+    def batch_inv(self, a, beta):
+        beta = np.ascontiguousarray(beta, dtype=np.uint32)
+        return self.H(self.lib.zkp_batch_inv(c_void_p(a.h), _np_ptr(beta)))
+
+    def range_prove(self, S, low, length, alpha, beta, u, v):
+        fin = np.zeros(8, np.uint32)
+        args = [np.ascontiguousarray(x, dtype=np.uint32) for x in (alpha, beta, u, v)]
+        self.check(self.lib.zkp_range_prove(c_void_p(S.h), c_int(low), c_uint(length), *[_np_ptr(a) for a in args], _np_ptr(fin)))
+        return fin
+
+    def mapping(self, S_in, low, length, mvals, r=None, alpha=None, beta=None, u=None, v=None):
+        y, m = c_void_p(), c_void_p()
+        prove = r is not None
+        fin = np.zeros(8, np.uint32)
+        z = np.zeros(8, np.uint32)
+        args = [np.ascontiguousarray(x if x is not None else z, dtype=np.uint32) for x in (r, alpha, beta, u, v)]
+        self.check(self.lib.zkp_mapping(c_void_p(S_in.h), c_int(low), c_uint(length), c_void_p(mvals.h), *[_np_ptr(a) for a in args],
+                                        ctypes.byref(y), ctypes.byref(m), _np_ptr(fin) if prove else None))
+        return self.H(y.value), self.H(m.value), fin
+
+    def multi_hadamard(self, claim, Xs, u, v):
+        u = np.ascontiguousarray(u, dtype=np.uint32).reshape(-1, 8)
+        v = np.ascontiguousarray(v, dtype=np.uint32).reshape(-1, 8)
+        k = u.shape[0]
+        arr = (c_void_p * len(Xs))(*[x.h for x in Xs])
+        proof = np.zeros((k * (len(Xs) + 1), 8), np.uint32)
+        fin = np.zeros(8, np.uint32)
+        claim = np.ascontiguousarray(claim, dtype=np.uint32)
+        self.check(self.lib.zkp_multi_hadamard(_np_ptr(claim), arr, c_int(len(Xs)), _np_ptr(u), _np_ptr(v), c_int(k), _np_ptr(proof), _np_ptr(fin)))
+        return proof, fin
+
+    def hadamard_product_sumcheck(self, a, b, u, v):
+        u = np.ascontiguousarray(u, dtype=np.uint32).reshape(-1, 8)
+        v = np.ascontiguousarray(v, dtype=np.uint32).reshape(-1, 8)
+        k = u.shape[0]
+        proof = np.zeros((3 * k + 2, 8), np.uint32)
+        self.check(self.lib.zkp_hadamard_product_sumcheck(c_void_p(a.h), c_void_p(b.h), _np_ptr(u), _np_ptr(v), c_int(k), _np_ptr(proof)))
+        return proof
+
+    def softmax(self, X, m, n, d, bs, L, M, sf_in, thetas, prove):
+        bs = np.ascontiguousarray(bs, dtype=np.uint32)
+        thetas = np.ascontiguousarray(thetas, dtype=np.float64)
+        shift = c_void_p()
+        y = self.H(self.lib.zkp_softmax(c_void_p(X.h), c_uint(m), c_uint(n), c_uint(d), _np_ptr(bs), c_int(len(bs)), c_uint(L), c_uint(M), c_u64(sf_in),
+                                        _np_ptr(thetas), c_int(len(thetas)), ctypes.byref(shift), c_int(1 if prove else 0)))
+        return y, self.H(shift.value)
+
+    def zkip_stacked(self, claim, A, B, N, D, uN, vN, uD):
+        uN, vN, uD = (np.ascontiguousarray(x, dtype=np.uint32).reshape(-1, 8) for x in (uN, vN, uD))
+        kN, kD = uN.shape[0], uD.shape[0]
+        proof = np.zeros((kN + kD, 3, 8), np.uint32)
+        fin = np.zeros(8, np.uint32)
+        claim = np.ascontiguousarray(claim, dtype=np.uint32)
+        self.check(self.lib.zkp_zkip_stacked(_np_ptr(claim), c_void_p(A.h), c_void_p(B.h), c_uint(N), c_uint(D), _np_ptr(uN), _np_ptr(vN), c_int(kN),
+                                             _np_ptr(uD), c_int(kD), _np_ptr(proof), _np_ptr(fin)))
+        return proof, fin
 
     # ---- transcript / challenges ----
     def seed(self, s):

@@ -1,0 +1,193 @@
+"""GPU parity: multiplicities, batch inversion, the two-phase lookup sumcheck, range / mapping tables,
+rescaling, multi-Hadamard sumcheck, stacked inner-product sumcheck and zkSoftmax -- bit-exact against the oracle."""
+import numpy as np
+import pytest
+
+from zkhelp import R_MOD, fr_array, fr_ints, load_oracle, mt_random_vec, orc_check, orc_transcript
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def pv():
+    from gpuhelp import Prover
+    return Prover()
+
+
+@pytest.fixture(scope="module")
+def orc():
+    return load_oracle()
+
+
+def ch(seed, n):
+    return mt_random_vec(np.random.RandomState(seed), n)
+
+
+@pytest.mark.parametrize("n,sf", [(1, 16), (1000, 16), (4096, 1 << 16), (70000, 1 << 20)])
+def test_rescale(pv, orc, n, sf):
+    rng = np.random.default_rng(n)
+    x = rng.integers(-(1 << 40), 1 << 40, n)
+    x[: min(n, 6)] = [0, sf // 2, -(sf // 2), sf // 2 - 1, -(sf // 2) - 1, 3 * sf][: min(n, 6)]
+    X = fr_array([int(v) % R_MOD for v in x])
+    e_out, e_rem = np.zeros_like(X), np.zeros_like(X)
+    orc_check(orc.orc_rescale(X, n, sf, e_out, e_rem))
+    out, rem = pv.rescale(pv.from_fr(X), sf)
+    assert (out.host() == e_out).all() and (rem.host() == e_rem).all()
+
+
+@pytest.mark.parametrize("D,low,length", [(64, -5, 11), (5000, -8, 16), (1 << 16, -(1 << 15), 1 << 16), (300000, 0, 1 << 18), (100000, 0, 3)])
+def test_multiplicities(pv, D, low, length):
+    rng = np.random.default_rng(D)
+    vals = rng.integers(low, low + length, D)
+    vals[: D // 3] = low + length // 2               # a long run of equal values (wave aggregation path)
+    m = pv.range_prep(pv.from_i64(vals), low, length).host()
+    size = 1 << max(0, (length - 1).bit_length())
+    assert fr_ints(m) == [int(c) for c in np.bincount(vals - low, minlength=size)]
+
+
+def test_lookup_out_of_range_is_an_error(pv):
+    with pytest.raises(RuntimeError, match="outside the table"):
+        pv.range_prep(pv.from_i64(np.array([0, 1, 99])), 0, 8)
+
+
+@pytest.mark.parametrize("n", [1, 7, 4096, 4097, 50000])
+def test_batch_inverse(pv, orc, n):
+    S = ch(n, n)
+    beta = ch(5, 1)[0]
+    if n >= 7:
+        S[3] = fr_array([(-fr_ints(beta.reshape(1, 8))[0]) % R_MOD])[0]     # S + beta == 0 -> output 0
+    exp = np.zeros_like(S)
+    orc_check(orc.orc_lookup_inv(S, n, beta, exp))
+    got = pv.batch_inv(pv.from_fr(S), beta).host()
+    assert (got == exp).all()
+    if n >= 7:
+        assert not got[3].any()
+
+
+@pytest.mark.parametrize("D,low,length", [(16, 3, 4), (4, 0, 4), (256, -8, 16), (4096, -32, 64), (1 << 15, -(1 << 9), 1 << 10)])
+def test_range_lookup_proof_transcript(pv, orc, D, low, length):
+    rng = np.random.default_rng(D + length)
+    vals = rng.integers(low, low + length, D)
+    S = fr_array([int(v) % R_MOD for v in vals])
+    k = (D - 1).bit_length()
+    alpha, beta, u, v = ch(1, 1)[0], ch(2, 1)[0], ch(3, k), ch(4, k)
+    orc.orc_transcript_clear()
+    e_fin = np.zeros(8, np.uint32)
+    orc_check(orc.orc_range_prove(S, D, low, length, alpha, beta, u, v, e_fin))
+    e_t = orc_transcript(orc)
+    pv.transcript_begin()
+    fin = pv.range_prove(pv.from_fr(S), low, length, alpha, beta, u, v)
+    pv.lib.zkp_transcript_end()
+    assert (fin == e_fin).all()
+    t = pv.transcript()
+    assert t.shape == e_t.shape and (t == e_t).all()
+
+
+@pytest.mark.parametrize("D,low,length", [(6, -2, 4), (64, -8, 16), (1000, -16, 32)])
+def test_mapping_lookup(pv, orc, D, low, length):
+    rng = np.random.default_rng(D)
+    vals = rng.integers(low, low + length, D)
+    mv = ch(6, length)
+    S = fr_array([int(v) % R_MOD for v in vals])
+    k = (D - 1).bit_length()
+    r, alpha, beta, u, v = ch(7, 1)[0], ch(8, 1)[0], ch(9, 1)[0], ch(10, k), ch(11, k)
+    size = 1 << (length - 1).bit_length()
+    e_y, e_m, e_fin = np.zeros((D, 8), np.uint32), np.zeros((size, 8), np.uint32), np.zeros(8, np.uint32)
+    orc.orc_transcript_clear()
+    orc_check(orc.orc_mapping(S, D, low, length, mv, r, alpha, beta, u, v, e_y, e_m, e_fin))
+    e_t = orc_transcript(orc)
+    pv.transcript_begin()
+    y, m, fin = pv.mapping(pv.from_fr(S), low, length, pv.from_fr(mv), r, alpha, beta, u, v)
+    pv.lib.zkp_transcript_end()
+    assert (y.host() == e_y).all() and (m.host() == e_m).all() and (fin == e_fin).all()
+    t = pv.transcript()
+    assert t.shape == e_t.shape and (t == e_t).all()
+
+
+def test_rescaling_prove_seeded_transcript(pv, orc):
+    for n, sf in ((256, 16), (5000, 1 << 8)):
+        x = np.random.default_rng(n).integers(-(1 << 30), 1 << 30, n)
+        X = fr_array([int(v) % R_MOD for v in x])
+        orc.orc_seed(99)
+        orc.orc_transcript_clear()
+        e_out = np.zeros_like(X)
+        orc_check(orc.orc_rescale_prove(X, n, sf, e_out))
+        e_t = orc_transcript(orc)
+        pv.seed(99)
+        pv.transcript_begin()
+        out = pv.rescale_prove(pv.from_fr(X), sf)
+        pv.lib.zkp_transcript_end()
+        assert (out.host() == e_out).all()
+        t = pv.transcript()
+        assert t.shape == e_t.shape and (t == e_t).all()
+
+
+@pytest.mark.parametrize("nX,n", [(1, 8), (2, 16), (2, 4096), (3, 64), (4, 32)])
+def test_multi_hadamard(pv, orc, nX, n):
+    Xs = [ch(20 + i, n) for i in range(nX)]
+    k = (n - 1).bit_length()
+    u, v = ch(30, k), ch(31, k)
+    prod = Xs[0].copy()
+    tmp = np.zeros_like(prod)
+    for x in Xs[1:]:
+        orc_check(orc.orc_fr_op(7, prod, x, tmp, n))
+        prod = tmp.copy()
+    claim = np.zeros(8, np.uint32)
+    orc_check(orc.orc_fr_me(prod, n, u, k, claim))
+    e_proof, e_fin = np.zeros((k * (nX + 1), 8), np.uint32), np.zeros(8, np.uint32)
+    orc_check(orc.orc_multi_hadamard(claim, np.ascontiguousarray(np.concatenate(Xs)), nX, n, u, v, k, e_proof, e_fin))
+    proof, fin = pv.multi_hadamard(claim, [pv.from_fr(x) for x in Xs], u, v)
+    assert (proof == e_proof).all() and (fin == e_fin).all()
+
+
+@pytest.mark.parametrize("n", [2, 5, 64, 1000])
+def test_deprecated_hadamard_product_sumcheck(pv, orc, n):
+    a, b = ch(40, n), ch(41, n)
+    k = (n - 1).bit_length()
+    u, v = ch(42, k), ch(43, k)
+    exp = np.zeros((3 * k + 2, 8), np.uint32)
+    orc_check(orc.orc_hadamard_product_sumcheck(a, b, n, u, v, k, exp))
+    got = pv.hadamard_product_sumcheck(pv.from_fr(a), pv.from_fr(b), u, v)
+    assert (got == exp).all()
+
+
+@pytest.mark.parametrize("N,D", [(2, 4), (4, 16), (3, 8), (32, 128)])
+def test_zkip_stacked(pv, orc, N, D):
+    A, B = ch(50, N * D), ch(51, N * D)
+    kN, kD = (N - 1).bit_length(), (D - 1).bit_length()
+    uN, vN, uD = ch(52, kN), ch(53, kN), ch(54, kD)
+    # claim = sum_n eq(uN, n) <A_n, B_n>
+    per = np.zeros((N, 8), np.uint32)
+    tmp = np.zeros((D, 8), np.uint32)
+    for i in range(N):
+        orc_check(orc.orc_fr_op(7, A[i * D:(i + 1) * D].copy(), B[i * D:(i + 1) * D].copy(), tmp, D))
+        orc_check(orc.orc_fr_sum(tmp, D, per[i]))
+    claim = np.zeros(8, np.uint32)
+    orc_check(orc.orc_fr_me(per, N, uN, kN, claim))
+    e_proof, e_fin = np.zeros((kN + kD, 3, 8), np.uint32), np.zeros(8, np.uint32)
+    orc_check(orc.orc_zkip_stacked(claim, A, B, N, D, uN, vN, kN, uD, kD, e_proof, e_fin))
+    proof, fin = pv.zkip_stacked(claim, pv.from_fr(A), pv.from_fr(B), N, D, uN, vN, uD)
+    assert (proof == e_proof).all() and (fin == e_fin).all()
+
+
+@pytest.mark.parametrize("m,n,d,bs,sf,lim", [(16, 16, 16, [16, 16, 16], 256, 200), (64, 64, 32, [1 << 4, 1 << 6, 1 << 6], 1 << 10, 4000), (7, 64, 8, [1 << 3, 1 << 6, 1 << 6], 1 << 9, 1000)])
+def test_softmax_compute_and_prove(pv, orc, m, n, d, bs, sf, lim):
+    rng = np.random.default_rng(m * n)
+    X = rng.integers(-lim, lim, (m, n))
+    Xf = fr_array([int(x) % R_MOD for x in X.reshape(-1)])
+    thetas = np.array([float(1 << 10), float(1 << 12)])
+    bsa = np.array(bs, np.uint32)
+    prove = ((m * n) & (m * n - 1)) == 0
+    e_Y, e_shift = np.zeros((m * n, 8), np.uint32), np.zeros((m, 8), np.uint32)
+    orc.orc_seed(5)
+    orc.orc_transcript_clear()
+    orc_check(orc.orc_softmax(Xf, m, n, d, bsa, 3, 1, 0, sf, thetas, 2, e_Y, e_shift, 1 if prove else 0))
+    e_t = orc_transcript(orc)
+    pv.seed(5)
+    pv.transcript_begin()
+    Y, shift = pv.softmax(pv.from_fr(Xf), m, n, d, bsa, 1, 0, sf, thetas, prove)
+    pv.lib.zkp_transcript_end()
+    assert (shift.host() == e_shift).all()
+    assert (Y.host() == e_Y).all()
+    t = pv.transcript()
+    assert t.shape == e_t.shape and (t == e_t).all()

@@ -308,6 +308,26 @@ __global__ void __launch_bounds__(TPB) k_ip_round(Fr* __restrict__ partials, con
     block_reduce_store<3>(acc, partials);
 }
 
+// Stacked form (zkip_stacked_poly_kernel zkfc.cu:153-167 followed by the multilinear evaluation over the
+// stacking axis, zkfc.cu:187-209): tensors are [N][D], halves are taken over N, and row n of the three
+// term tensors is weighted by E[n] (eq table, Montgomery form) before everything is summed.
+__global__ void __launch_bounds__(TPB) k_ip_round_w(Fr* __restrict__ partials, const Fr* __restrict__ a, const Fr* __restrict__ b, const Fr* __restrict__ E,
+                                                    size_t D, size_t n_in, size_t n_out) {
+    Fr acc[3] = {big_zero<8>(), big_zero<8>(), big_zero<8>()};
+    for (size_t g = (size_t)blockIdx.x * TPB + threadIdx.x; g < n_out; g += (size_t)gridDim.x * TPB) {
+        const Fr a0 = (g < n_in) ? a[g] : big_zero<8>();
+        const Fr b0 = (g < n_in) ? b[g] : big_zero<8>();
+        const Fr a1 = (g + n_out < n_in) ? a[g + n_out] : big_zero<8>();
+        const Fr b1 = (g + n_out < n_in) ? b[g + n_out] : big_zero<8>();
+        const Fr da = sub(a1, a0), db = sub(b1, b0);
+        const Fr e = E[g / D];
+        acc[0] = add(acc[0], mont_mul(e, mont_mul(a0, b0)));
+        acc[1] = add(acc[1], mont_mul(e, add(mont_mul(a0, db), mont_mul(b0, da))));
+        acc[2] = add(acc[2], mont_mul(e, mont_mul(da, db)));
+    }
+    block_reduce_store<3>(acc, partials);
+}
+
 // Whole sumcheck in one workgroup for short vectors (n <= 8192): every round's three sums are
 // written to polys[round*3 + {0,1,2}] (standard form, R^2-corrected), the folded vectors
 // ping-pong through `work` (2 * 2 * n_pow2/2 elements) and the final a, b land in fin[0..1].
@@ -538,6 +558,24 @@ int zk_ip_round(uint32_t* poly3_host, const void* a, const void* b, size_t n_in,
     Scratch part(sizeof(Fr) * 3 * nb);
     if (part.rc) return part.rc;
     hipLaunchKernelGGL(k_ip_round, dim3(nb), dim3(TPB), 0, (hipStream_t)stv, part.as<Fr>(), (const Fr*)a, (const Fr*)b, n_in, n_out);
+    ZK_LAUNCH_CHECK();
+    Fr s[3];
+    int rc = finish_to_host<3>(part.as<Fr>(), nb, s, (hipStream_t)stv);
+    if (rc) return rc;
+    for (int i = 0; i < 3; ++i) s[i] = to_mont(s[i]);
+    memcpy(poly3_host, s, 96);
+    return 0;
+}
+
+// Stacked round over [N][D] tensors: rows_in = N, rows_out = 2^ceil(log2 N) / 2, E = eq table over the
+// remaining stacking challenges (rows_out entries, Montgomery form).
+int zk_ip_round_stacked(uint32_t* poly3_host, const void* a, const void* b, const void* E, size_t D, size_t rows_in, size_t rows_out, void* stv) {
+    ZK_ARG(D >= 1 && rows_out >= 1 && rows_in >= 1 && rows_in <= 2 * rows_out, "zk_ip_round_stacked: bad shape");
+    const size_t n_in = rows_in * D, n_out = rows_out * D;
+    const unsigned nb = reduce_grid(n_out);
+    Scratch part(sizeof(Fr) * 3 * nb);
+    if (part.rc) return part.rc;
+    hipLaunchKernelGGL(k_ip_round_w, dim3(nb), dim3(TPB), 0, (hipStream_t)stv, part.as<Fr>(), (const Fr*)a, (const Fr*)b, (const Fr*)E, D, n_in, n_out);
     ZK_LAUNCH_CHECK();
     Fr s[3];
     int rc = finish_to_host<3>(part.as<Fr>(), nb, s, (hipStream_t)stv);

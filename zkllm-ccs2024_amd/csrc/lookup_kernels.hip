@@ -1,0 +1,559 @@
+// Lookup argument, rescaling and softmax kernels for gfx950 (replaces the kernels of tlookup.cu,
+// rescaling.cu, zksoftmax.cu and the multi-Hadamard kernels of proof.cu:172-188).
+//
+//  * multiplicities: indices are histogrammed into LDS-private counters when the table fits
+//    (<= 16 Ki bins), otherwise with wave-aggregated global atomics, so a column of equal values
+//    costs one atomic per wave instead of 64 (tlookup.cu:10-48 uses one global atomic per query).
+//  * inverses: Montgomery's batch inversion across a whole 512-lane workgroup -- prefix and
+//    suffix products through LDS and a single Fermat exponentiation per 4096 elements -- instead of
+//    one 255-bit exponentiation per element (tlookup.cu:50-62).  Inverses are unique, so outputs
+//    are identical; zero inputs give zero as 0^(r-2) does.
+//  * sumcheck rounds: the multilinear evaluations of the per-round term tensors
+//    (tlookup.cu:184-279) are taken as inner products with the eq(u, .) table, so one pass over
+//    the operands yields every coefficient of the round polynomial and the folded operands; no
+//    term tensor is ever written.
+//  * softmax shift / exp tables use the deterministic exp/log of detmath.hpp.
+#include <cstring>
+#include "detmath.hpp"
+#include "field.hpp"
+#include "rt.hpp"
+#include "../../include/zkllm_hip.h"
+
+using namespace zk;
+
+static constexpr int TPB = 256;
+static inline Fr load_fr(const uint32_t* p) { Fr r; memcpy(&r, p, 32); return r; }
+
+// ---- block reduction helper (K sums per thread) -------------------------------------------------------
+template <int K> __device__ __forceinline__ void block_reduce_store(Fr (&acc)[K], Fr* __restrict__ partials) {
+    __shared__ uint32_t red[8][TPB];
+    const uint32_t t = threadIdx.x;
+#pragma unroll 1
+    for (int k = 0; k < K; ++k) {
+#pragma unroll
+        for (int l = 0; l < 8; ++l) red[l][t] = acc[k].v[l];
+        __syncthreads();
+        for (uint32_t s = TPB / 2; s > 0; s >>= 1) {
+            if (t < s) {
+                Fr x, y;
+#pragma unroll
+                for (int l = 0; l < 8; ++l) { x.v[l] = red[l][t]; y.v[l] = red[l][t + s]; }
+                x = add(x, y);
+#pragma unroll
+                for (int l = 0; l < 8; ++l) red[l][t] = x.v[l];
+            }
+            __syncthreads();
+        }
+        if (t == 0) {
+            Fr x;
+#pragma unroll
+            for (int l = 0; l < 8; ++l) x.v[l] = red[l][0];
+            partials[(size_t)k * gridDim.x + blockIdx.x] = x;
+        }
+        __syncthreads();
+    }
+}
+__global__ void __launch_bounds__(TPB) k_finish(Fr* __restrict__ out, const Fr* __restrict__ partials, uint32_t nb) {
+    Fr acc[1] = {big_zero<8>()};
+    const Fr* p = partials + (size_t)blockIdx.x * nb;
+    for (uint32_t i = threadIdx.x; i < nb; i += TPB) acc[0] = add(acc[0], p[i]);
+    block_reduce_store<1>(acc, out);
+}
+static inline unsigned reduce_grid(size_t n) {
+    size_t b = (n + TPB - 1) / TPB;
+    if (b > 1024) b = 1024;
+    if (b < 1) b = 1;
+    return (unsigned)b;
+}
+// finish K sums (K x nb partials) and copy them to the host, applying the R correction (to_mont)
+// to the first `n_mont` of them
+static int finish_sums(Fr* partials, unsigned nb, int K, int n_mont, Fr* host_out, hipStream_t st) {
+    void* stage = nullptr;
+    int rc = staging(&stage, sizeof(Fr) * K);
+    if (rc) return rc;
+    Scratch fin(sizeof(Fr) * K);
+    if (fin.rc) return fin.rc;
+    hipLaunchKernelGGL(k_finish, dim3(K), dim3(TPB), 0, st, fin.as<Fr>(), partials, nb);
+    ZK_LAUNCH_CHECK();
+    ZK_HIP(hipMemcpyAsync(stage, fin.p, sizeof(Fr) * K, hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipStreamSynchronize(st));
+    memcpy(host_out, stage, sizeof(Fr) * K);
+    for (int i = 0; i < n_mont; ++i) host_out[i] = to_mont(host_out[i]);
+    return 0;
+}
+
+// ---- table index / histogram ---------------------------------------------------------------------------------
+// idx = (val - low).val[0]  (lookuprange_tensor_prep_kernel tlookup.cu:414-421); an index outside the
+// table (which the reference would use unchecked) raises the flag instead.
+__global__ void __launch_bounds__(TPB) k_index_fr(uint32_t* __restrict__ idx, uint32_t* __restrict__ flag, const Fr* __restrict__ vals, const Fr low, uint32_t table_size, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    const Fr d = sub(vals[i], low);
+    const bool ok = !(d.v[1] | d.v[2] | d.v[3] | d.v[4] | d.v[5] | d.v[6] | d.v[7]) && d.v[0] < table_size;
+    idx[i] = ok ? d.v[0] : 0u;
+    if (!ok) atomicOr(flag, 1u);
+}
+__global__ void __launch_bounds__(TPB) k_index_i32(uint32_t* __restrict__ idx, uint32_t* __restrict__ flag, const int32_t* __restrict__ vals, int32_t low, uint32_t table_size, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    const int64_t d = (int64_t)vals[i] - (int64_t)low;
+    const bool ok = d >= 0 && d < (int64_t)table_size;
+    idx[i] = ok ? (uint32_t)d : 0u;
+    if (!ok) atomicOr(flag, 1u);
+}
+static constexpr uint32_t HIST_LDS_BINS = 16384;
+__global__ void __launch_bounds__(TPB) k_hist_lds(uint32_t* __restrict__ counts, const uint32_t* __restrict__ idx, size_t n, uint32_t nbins) {
+    __shared__ uint32_t h[HIST_LDS_BINS];
+    for (uint32_t b = threadIdx.x; b < nbins; b += TPB) h[b] = 0;
+    __syncthreads();
+    for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (size_t)gridDim.x * TPB) atomicAdd(&h[idx[i]], 1u);
+    __syncthreads();
+    for (uint32_t b = threadIdx.x; b < nbins; b += TPB) {
+        const uint32_t c = h[b];
+        if (c) atomicAdd(&counts[b], c);
+    }
+}
+// Large tables: lanes of a wave that hold the same index are merged (up to 4 distinct leaders per
+// step) before touching global memory.
+__global__ void __launch_bounds__(TPB) k_hist_global(uint32_t* __restrict__ counts, const uint32_t* __restrict__ idx, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    bool pending = i < n;
+    const uint32_t my = pending ? idx[i] : 0u;
+    const uint32_t lane = threadIdx.x & 63u;
+#pragma unroll 1
+    for (int it = 0; it < 4; ++it) {
+        const unsigned long long act = __ballot(pending);
+        if (!act) break;
+        const int leader = __ffsll((long long)act) - 1;
+        const uint32_t lead = __shfl(my, leader, 64);
+        const unsigned long long same = __ballot(pending && my == lead);
+        if (lane == (uint32_t)leader) atomicAdd(&counts[lead], (uint32_t)__popcll(same));
+        if (pending && my == lead) pending = false;
+    }
+    if (pending) atomicAdd(&counts[my], 1u);
+}
+// table[i] = low + min(i, len-1)  (tlookuprange_init_kernel tlookup.cu:372-380)
+__global__ void __launch_bounds__(TPB) k_range_table(Fr* __restrict__ table, int32_t low, uint32_t len, uint32_t table_size) {
+    const uint32_t t = blockIdx.x * TPB + threadIdx.x;
+    if (t >= table_size) return;
+    const int64_t v = (t < len) ? (int64_t)t + low : (int64_t)len + low - 1;
+    table[t] = fr_from_i64(v);
+}
+
+// ---- batch inversion -----------------------------------------------------------------------------------------------
+static constexpr int BI_T = 512, BI_CH = 8;
+__global__ void __launch_bounds__(BI_T) k_batch_inv(Fr* __restrict__ out, const Fr* __restrict__ in, const Fr beta, size_t n) {
+    __shared__ uint32_t sc[8][BI_T];
+    __shared__ uint32_t inv_tot[8];
+    const uint32_t t = threadIdx.x;
+    const size_t base = ((size_t)blockIdx.x * BI_T + t) * BI_CH;
+    const Fr one_m = big_one_mont<8>();
+    Fr xm[BI_CH], pre[BI_CH];
+    bool nz[BI_CH];
+    Fr tot = one_m;
+#pragma unroll
+    for (int c = 0; c < BI_CH; ++c) {
+        Fr x = big_zero<8>();
+        if (base + c < n) x = add(in[base + c], beta);
+        nz[c] = !is_zero(x);
+        xm[c] = nz[c] ? to_mont(x) : one_m;
+        pre[c] = tot;
+        tot = mont_mul(tot, xm[c]);
+    }
+    auto put = [&](const Fr& v, uint32_t i) {
+#pragma unroll
+        for (int l = 0; l < 8; ++l) sc[l][i] = v.v[l];
+    };
+    auto get = [&](uint32_t i) {
+        Fr v;
+#pragma unroll
+        for (int l = 0; l < 8; ++l) v.v[l] = sc[l][i];
+        return v;
+    };
+    // inclusive prefix products over the workgroup
+    Fr run = tot;
+    put(run, t);
+    __syncthreads();
+    for (uint32_t d = 1; d < BI_T; d <<= 1) {
+        Fr other = one_m;
+        if (t >= d) other = get(t - d);
+        __syncthreads();
+        if (t >= d) { run = mont_mul(run, other); put(run, t); }
+        __syncthreads();
+    }
+    const Fr prefix_excl = (t == 0) ? one_m : get(t - 1);
+    if (t < 64) {   // one wave inverts the workgroup's total
+        const Fr total = get(BI_T - 1);
+        const Fr it = mont_inverse(total);
+        if (t == 0) {
+#pragma unroll
+            for (int l = 0; l < 8; ++l) inv_tot[l] = it.v[l];
+        }
+    }
+    __syncthreads();
+    // inclusive suffix products
+    run = tot;
+    put(run, t);
+    __syncthreads();
+    for (uint32_t d = 1; d < BI_T; d <<= 1) {
+        Fr other = one_m;
+        if (t + d < BI_T) other = get(t + d);
+        __syncthreads();
+        if (t + d < BI_T) { run = mont_mul(run, other); put(run, t); }
+        __syncthreads();
+    }
+    const Fr suffix_excl = (t + 1 < BI_T) ? get(t + 1) : one_m;
+    Fr itot;
+#pragma unroll
+    for (int l = 0; l < 8; ++l) itot.v[l] = inv_tot[l];
+    // 1 / (this lane's product) = 1/total * (product of everything before) * (product of everything after)
+    Fr inv_run = mont_mul(mont_mul(itot, prefix_excl), suffix_excl);
+#pragma unroll
+    for (int c = BI_CH - 1; c >= 0; --c) {
+        const Fr inv_c = mont_mul(inv_run, pre[c]);      // Montgomery form of 1/x_c
+        inv_run = mont_mul(inv_run, xm[c]);
+        if (base + c < n) out[base + c] = nz[c] ? from_mont(inv_c) : big_zero<8>();
+    }
+}
+
+// ---- eq tables ----------------------------------------------------------------------------------------------------------
+// E[t] = prod_j (u_j if bit_j(t) else 1-u_j), Montgomery form.  Built by doubling: level j appends bit j.
+__global__ void __launch_bounds__(TPB) k_eq_double(Fr* __restrict__ e, const Fr u_mont, const Fr one_minus_u_mont, size_t half) {
+    const size_t t = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (t >= half) return;
+    const Fr x = e[t];
+    e[t + half] = mont_mul(x, u_mont);
+    e[t] = mont_mul(x, one_minus_u_mont);
+}
+// dropping the top variable: E'[t] = E[t] + E[t + n_out]
+__global__ void __launch_bounds__(TPB) k_eq_halve(Fr* __restrict__ out, const Fr* __restrict__ in, size_t n_out) {
+    const size_t t = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (t < n_out) out[t] = add(in[t], in[t + n_out]);
+}
+
+// ---- lookup sumcheck round --------------------------------------------------------------------------------------------------
+// Over halves (t, t + n_out):  a0 = A[t], da = A[t+n_out]-A[t], s0 = S[t]+beta, ds = S[t+n_out]-S[t]
+//   sums 0..2 : sum E[t] * {a0 s0, da s0 + a0 ds, da ds}          (R^-1 attached)
+//   sums 3..4 : sum a0, sum da
+// phase 2 adds the same three E-weighted sums for (B,T) as sums 5..7 and the plain products of (m,B)
+// as sums 8..10 (R^-1 attached), and folds all five tensors by v.
+template <bool PHASE2> __global__ void __launch_bounds__(TPB)
+k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ nS, Fr* __restrict__ nB, Fr* __restrict__ nT, Fr* __restrict__ nm,
+               const Fr* __restrict__ A, const Fr* __restrict__ S, const Fr* __restrict__ B, const Fr* __restrict__ T, const Fr* __restrict__ m,
+               const Fr* __restrict__ E, const Fr beta, const Fr v_mont, size_t n_out) {
+    constexpr int K = PHASE2 ? 11 : 5;
+    Fr acc[K];
+#pragma unroll
+    for (int i = 0; i < K; ++i) acc[i] = big_zero<8>();
+    for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
+        const Fr e = E[t];
+        {
+            const Fr a0 = A[t], a1 = A[t + n_out], s0r = S[t], s1 = S[t + n_out];
+            const Fr da = sub(a1, a0), ds = sub(s1, s0r), s0 = add(s0r, beta);
+            acc[0] = add(acc[0], mont_mul(e, mont_mul(a0, s0)));
+            acc[1] = add(acc[1], mont_mul(e, add(mont_mul(da, s0), mont_mul(a0, ds))));
+            acc[2] = add(acc[2], mont_mul(e, mont_mul(da, ds)));
+            acc[3] = add(acc[3], a0);
+            acc[4] = add(acc[4], da);
+            nA[t] = add(a0, mont_mul(v_mont, da));
+            nS[t] = add(s0r, mont_mul(v_mont, ds));
+        }
+        if (PHASE2) {
+            const Fr b0 = B[t], b1 = B[t + n_out], t0r = T[t], t1 = T[t + n_out], m0 = m[t], m1 = m[t + n_out];
+            const Fr db = sub(b1, b0), dt = sub(t1, t0r), t0 = add(t0r, beta), dm = sub(m1, m0);
+            acc[5] = add(acc[5], mont_mul(e, mont_mul(b0, t0)));
+            acc[6] = add(acc[6], mont_mul(e, add(mont_mul(db, t0), mont_mul(b0, dt))));
+            acc[7] = add(acc[7], mont_mul(e, mont_mul(db, dt)));
+            acc[8] = add(acc[8], mont_mul(m0, b0));
+            acc[9] = add(acc[9], add(mont_mul(dm, b0), mont_mul(m0, db)));
+            acc[10] = add(acc[10], mont_mul(dm, db));
+            nB[t] = add(b0, mont_mul(v_mont, db));
+            nT[t] = add(t0r, mont_mul(v_mont, dt));
+            nm[t] = add(m0, mont_mul(v_mont, dm));
+        }
+    }
+    block_reduce_store<K>(acc, partials);
+}
+
+// ---- multi-Hadamard sumcheck round (proof.cu:191-241) --------------------------------------------------------------------------
+// K tensors; coefficient j of prod_k (X0_k + t dX_k), weighted by E and summed (R^-K attached... see host);
+// also folds every tensor by v.
+template <int K> struct PtrPack { const Fr* in[K]; Fr* out[K]; };
+template <int K> __global__ void __launch_bounds__(TPB)
+k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __restrict__ E, const Fr v_mont, size_t n_out) {
+    Fr acc[K + 1];
+#pragma unroll
+    for (int i = 0; i <= K; ++i) acc[i] = big_zero<8>();
+    const Fr r2 = big_r2<8>();
+    for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
+        Fr c[K + 1];   // running product polynomial, standard form
+        {
+            const Fr x0 = p.in[0][t], x1 = p.in[0][t + n_out];
+            const Fr dx = sub(x1, x0);
+            c[0] = x0; c[1] = dx;
+            p.out[0][t] = add(x0, mont_mul(v_mont, dx));
+        }
+#pragma unroll
+        for (int k = 1; k < K; ++k) {
+            const Fr x0 = p.in[k][t], x1 = p.in[k][t + n_out];
+            const Fr dx = sub(x1, x0);
+            p.out[k][t] = add(x0, mont_mul(v_mont, dx));
+            const Fr x0m = mont_mul(x0, r2), dxm = mont_mul(dx, r2);    // Montgomery form so products stay standard
+            c[k + 1] = mont_mul(c[k], dxm);
+#pragma unroll
+            for (int j = k; j >= 1; --j) c[j] = add(mont_mul(c[j], x0m), mont_mul(c[j - 1], dxm));
+            c[0] = mont_mul(c[0], x0m);
+        }
+        const Fr e = E[t];   // Montgomery form: e*R
+#pragma unroll
+        for (int j = 0; j <= K; ++j) acc[j] = add(acc[j], mont_mul(e, c[j]));
+    }
+    block_reduce_store<K + 1>(acc, partials);
+}
+
+// ---- rescaling (rescaling.cu:8-21) ----------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(TPB) k_rescale(Fr* __restrict__ out, Fr* __restrict__ rem, const Fr* __restrict__ in, int64_t sf, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    const int64_t hsf = sf >> 1;
+    const int64_t x = fr_to_i64(in[i]);
+    const int64_t temp = (x + hsf) % sf;
+    const int64_t x_rem = (temp < 0 ? temp + sf : temp) - hsf;
+    const int64_t x_rescaled = (x - x_rem) / sf;
+    out[i] = fr_from_i64(x_rescaled);
+    rem[i] = fr_from_i64(x_rem);
+}
+
+// ---- softmax (zksoftmax.cu) ------------------------------------------------------------------------------------------------------
+// One wave per row.  Lane l sums exp(x_j / scale) over j = l, l+64, ... in index order, the 64 partial
+// sums are combined with the butterfly i ^ 32, 16, ..., 1 (every lane ends with the same total), and
+// shift = round_half_away(scale * log(total)).  out = x - shift.  scale = sf_in * sqrt(d).
+__global__ void __launch_bounds__(TPB) k_softmax_shift(Fr* __restrict__ shift, Fr* __restrict__ out, const Fr* __restrict__ X, uint32_t rows, uint32_t cols, double scale) {
+    const uint32_t row = blockIdx.x * (TPB / 64) + (threadIdx.x >> 6);
+    const uint32_t lane = threadIdx.x & 63u;
+    if (row >= rows) return;
+    const Fr* xr = X + (size_t)row * cols;
+    double part = 0.0;
+    for (uint32_t j = lane; j < cols; j += 64) part = part + zkd::exp_det((double)fr_to_i64(xr[j]) / scale);
+    for (int off = 32; off >= 1; off >>= 1) part = part + __shfl_xor(part, off, 64);
+    const double sv = scale * zkd::log_det(part);
+    const int64_t si = (sv >= 0) ? (int64_t)(sv + 0.5) : (int64_t)(sv - 0.5);
+    const Fr sh = fr_from_i64(si);
+    if (lane == 0) shift[row] = sh;
+    Fr* orow = out + (size_t)row * cols;
+    for (uint32_t j = lane; j < cols; j += 64) orow[j] = sub(xr[j], sh);
+}
+// table[x] = floor(exp(log_theta - step * x) + 0.5)  (zksoftmax.cu:4-14); step = B_k / (sf_in sqrt d)
+__global__ void __launch_bounds__(TPB) k_softmax_table(Fr* __restrict__ table, double log_theta, double step, uint32_t len) {
+    const uint32_t x = blockIdx.x * TPB + threadIdx.x;
+    if (x >= len) return;
+    const double v = zkd::exp_det(log_theta - step * (double)x) + 0.5;
+    table[x] = fr_from_u64((uint64_t)v);
+}
+// digits of -x in the mixed radix bs[0..K): plane k holds digit k (zksoftmax.cu:95-109).  Values whose
+// negation does not fit 64 bits raise the flag (the reference leaves their planes unwritten).
+struct U32Pack8 { uint32_t v[8]; };
+__global__ void __launch_bounds__(TPB) k_softmax_decompose(Fr* __restrict__ planes, uint32_t* __restrict__ flag, const Fr* __restrict__ X, const U32Pack8 bs, int K, size_t n) {
+    const size_t g = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (g >= n) return;
+    const Fr mx = neg(X[g]);
+    if (mx.v[2] | mx.v[3] | mx.v[4] | mx.v[5] | mx.v[6] | mx.v[7]) {
+        atomicOr(flag, 1u);
+        for (int k = 0; k < K; ++k) planes[(size_t)k * n + g] = big_zero<8>();
+        return;
+    }
+    unsigned long long tmp = ((unsigned long long)mx.v[1] << 32) | mx.v[0];
+    for (int k = 0; k < K; ++k) {
+        planes[(size_t)k * n + g] = fr_from_u64(tmp % bs.v[k]);
+        tmp /= bs.v[k];
+    }
+    if (tmp != 0) atomicOr(flag, 2u);   // more digits than the radices cover
+}
+
+// ---- host side ----------------------------------------------------------------------------------------------------------------------
+#define LAUNCH1D(kernel, n, st, ...)                                                         \
+    do {                                                                                     \
+        if ((n) > 0) {                                                                       \
+            hipLaunchKernelGGL(kernel, dim3(cdiv((n), TPB)), dim3(TPB), 0, (hipStream_t)(st), __VA_ARGS__); \
+            ZK_LAUNCH_CHECK();                                                               \
+        }                                                                                    \
+    } while (0)
+
+static int read_flag(uint32_t* dev_flag, uint32_t* host_val, hipStream_t st) {
+    void* stage = nullptr;
+    int rc = staging(&stage, 4);
+    if (rc) return rc;
+    ZK_HIP(hipMemcpyAsync(stage, dev_flag, 4, hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipStreamSynchronize(st));
+    *host_val = *(uint32_t*)stage;
+    return 0;
+}
+
+extern "C" {
+
+int zk_lookup_index_fr(void* idx_u32, const void* vals, int32_t low, uint32_t table_size, size_t n, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    if (n == 0) return 0;
+    Scratch flag(4);
+    if (flag.rc) return flag.rc;
+    ZK_HIP(hipMemsetAsync(flag.p, 0, 4, st));
+    LAUNCH1D(k_index_fr, n, st, (uint32_t*)idx_u32, flag.as<uint32_t>(), (const Fr*)vals, fr_from_i64((int64_t)low), table_size, n);
+    uint32_t f = 0;
+    int rc = read_flag(flag.as<uint32_t>(), &f, st);
+    if (rc) return rc;
+    ZK_ARG(f == 0, "lookup: a value lies outside the table range");
+    return 0;
+}
+int zk_lookup_index_i32(void* idx_u32, const void* vals_i32, int32_t low, uint32_t table_size, size_t n, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    if (n == 0) return 0;
+    Scratch flag(4);
+    if (flag.rc) return flag.rc;
+    ZK_HIP(hipMemsetAsync(flag.p, 0, 4, st));
+    LAUNCH1D(k_index_i32, n, st, (uint32_t*)idx_u32, flag.as<uint32_t>(), (const int32_t*)vals_i32, low, table_size, n);
+    uint32_t f = 0;
+    int rc = read_flag(flag.as<uint32_t>(), &f, st);
+    if (rc) return rc;
+    ZK_ARG(f == 0, "lookup: a value lies outside the table range");
+    return 0;
+}
+// counts[0..nbins) = number of occurrences of each index (zeroed here first)
+int zk_lookup_hist(void* counts_u32, const void* idx_u32, size_t n, uint32_t nbins, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(nbins >= 1, "zk_lookup_hist: no bins");
+    ZK_HIP(hipMemsetAsync(counts_u32, 0, sizeof(uint32_t) * (size_t)nbins, st));
+    if (n == 0) return 0;
+    if (nbins <= HIST_LDS_BINS) {
+        unsigned blocks = cdiv(n, (size_t)TPB * 16);
+        if (blocks > 2048) blocks = 2048;
+        hipLaunchKernelGGL(k_hist_lds, dim3(blocks), dim3(TPB), 0, st, (uint32_t*)counts_u32, (const uint32_t*)idx_u32, n, nbins);
+    } else {
+        hipLaunchKernelGGL(k_hist_global, dim3(cdiv(n, TPB)), dim3(TPB), 0, st, (uint32_t*)counts_u32, (const uint32_t*)idx_u32, n);
+    }
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
+int zk_range_table(void* table, int32_t low, uint32_t len, uint32_t table_size, void* st) {
+    ZK_ARG(len >= 1 && table_size >= len, "zk_range_table: need 1 <= len <= table_size");
+    LAUNCH1D(k_range_table, table_size, st, (Fr*)table, low, len, table_size);
+    return 0;
+}
+// out[i] = 1 / (in[i] + beta), standard form; 0 where in[i] + beta == 0 (tlookup_inv_kernel tlookup.cu:50-62)
+int zk_fr_batch_inv(void* out, const void* in, const uint32_t* beta, size_t n, void* st) {
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(k_batch_inv, dim3(cdiv(n, (size_t)BI_T * BI_CH)), dim3(BI_T), 0, (hipStream_t)st, (Fr*)out, (const Fr*)in, load_fr(beta), n);
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
+// E[t] for t < 2^k (Montgomery form) from k standard-form challenges; out holds 2^k elements
+int zk_eq_table(void* out, const uint32_t* u, int k, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(k >= 0 && k <= 30, "zk_eq_table: k out of range");
+    Fr one_m = big_one_mont<8>();
+    ZK_HIP(hipMemcpyAsync(out, &one_m, sizeof(Fr), hipMemcpyHostToDevice, st));
+    ZK_HIP(hipStreamSynchronize(st));
+    Fr one = big_zero<8>();
+    one.v[0] = 1;
+    for (int j = 0; j < k; ++j) {
+        const Fr uj = load_fr(u + 8 * j);
+        const size_t half = (size_t)1 << j;
+        LAUNCH1D(k_eq_double, half, st, (Fr*)out, to_mont(uj), to_mont(sub(one, uj)), half);
+    }
+    return 0;
+}
+int zk_eq_halve(void* out, const void* in, size_t n_out, void* st) {
+    LAUNCH1D(k_eq_halve, n_out, st, (Fr*)out, (const Fr*)in, n_out);
+    return 0;
+}
+// One round of the lookup sumcheck over tensors of 2*n_out elements.  sums_host receives 5 values
+// (phase 1) or 11 (phase 2), all in standard form; new_* receive the tensors folded by v.  B, T, m and
+// their outputs are ignored in phase 1.
+int zk_lookup_round(uint32_t* sums_host, void* nA, void* nS, void* nB, void* nT, void* nm, const void* A, const void* S, const void* B, const void* T,
+                    const void* m, const void* E, const uint32_t* beta, const uint32_t* v, size_t n_out, int phase2, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(n_out >= 1, "zk_lookup_round: empty round");
+    const unsigned nb = reduce_grid(n_out);
+    const int K = phase2 ? 11 : 5;
+    Scratch part(sizeof(Fr) * K * nb);
+    if (part.rc) return part.rc;
+    const Fr b = load_fr(beta), vm = to_mont(load_fr(v));
+    if (phase2)
+        hipLaunchKernelGGL(k_lookup_round<true>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), (Fr*)nA, (Fr*)nS, (Fr*)nB, (Fr*)nT, (Fr*)nm, (const Fr*)A, (const Fr*)S,
+                           (const Fr*)B, (const Fr*)T, (const Fr*)m, (const Fr*)E, b, vm, n_out);
+    else
+        hipLaunchKernelGGL(k_lookup_round<false>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), (Fr*)nA, (Fr*)nS, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, (const Fr*)A,
+                           (const Fr*)S, (const Fr*)nullptr, (const Fr*)nullptr, (const Fr*)nullptr, (const Fr*)E, b, vm, n_out);
+    ZK_LAUNCH_CHECK();
+    Fr s[11];
+    int rc = finish_sums(part.as<Fr>(), nb, K, 0, s, st);
+    if (rc) return rc;
+    // E carries R, each inner product one R^-1, the outer product with E another: sums 0..2, 5..7 and the
+    // plain products 8..10 need one multiplication by R; sums 3, 4 are already standard.
+    for (int i = 0; i < K; ++i)
+        if (i != 3 && i != 4) s[i] = to_mont(s[i]);
+    memcpy(sums_host, s, sizeof(Fr) * K);
+    return 0;
+}
+// One round of multi_hadamard_sumchecks for K tensors of 2*n_out elements (K = 1..4).
+// coefs_host: K+1 coefficients of sum_t E[t] prod_k (X0_k + x dX_k); new_Xs[k] receive the folds by v.
+int zk_hadamard_round(uint32_t* coefs_host, void* const* new_Xs, const void* const* Xs, int K, const void* E, const uint32_t* v, size_t n_out, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(K >= 1 && K <= 4, "zk_hadamard_round: K must be 1..4");
+    ZK_ARG(n_out >= 1, "zk_hadamard_round: empty round");
+    const unsigned nb = reduce_grid(n_out);
+    Scratch part(sizeof(Fr) * (K + 1) * nb);
+    if (part.rc) return part.rc;
+    const Fr vm = to_mont(load_fr(v));
+#define HAD_CASE(KK)                                                                                                           \
+    case KK: {                                                                                                                 \
+        PtrPack<KK> p;                                                                                                         \
+        for (int i = 0; i < KK; ++i) { p.in[i] = (const Fr*)Xs[i]; p.out[i] = (Fr*)new_Xs[i]; }                                 \
+        hipLaunchKernelGGL(k_hadamard_round<KK>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), p, (const Fr*)E, vm, n_out);        \
+        break;                                                                                                                 \
+    }
+    switch (K) { HAD_CASE(1) HAD_CASE(2) HAD_CASE(3) HAD_CASE(4) }
+#undef HAD_CASE
+    ZK_LAUNCH_CHECK();
+    Fr s[5];
+    // e (= E*R) times a standard-form coefficient leaves no Montgomery factor: nothing to correct
+    int rc = finish_sums(part.as<Fr>(), nb, K + 1, 0, s, st);
+    if (rc) return rc;
+    memcpy(coefs_host, s, sizeof(Fr) * (K + 1));
+    return 0;
+}
+int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* st) {
+    ZK_ARG(scaling_factor >= 1, "zk_rescale: scaling factor is 0");
+    LAUNCH1D(k_rescale, n, st, (Fr*)out, (Fr*)rem, (const Fr*)in, (int64_t)scaling_factor, n);
+    return 0;
+}
+int zk_softmax_shift(void* shift, void* out_shifted, const void* X, uint32_t rows, uint32_t cols, double scale, void* st) {
+    if (rows == 0) return 0;
+    ZK_ARG(cols >= 1 && scale > 0.0, "zk_softmax_shift: bad shape or scale");
+    hipLaunchKernelGGL(k_softmax_shift, dim3(cdiv(rows, TPB / 64)), dim3(TPB), 0, (hipStream_t)st, (Fr*)shift, (Fr*)out_shifted, (const Fr*)X, rows, cols, scale);
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
+int zk_softmax_table(void* table, double log_theta, double step, uint32_t len, void* st) {
+    LAUNCH1D(k_softmax_table, len, st, (Fr*)table, log_theta, step, len);
+    return 0;
+}
+// planes: K*n elements, plane k = digit k of -X in the mixed radix bs_host[0..K)
+int zk_softmax_decompose(void* planes, const void* X_shifted, const uint32_t* bs_host, int K, size_t n, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(K >= 1 && K <= 8, "zk_softmax_decompose: K must be 1..8");
+    if (n == 0) return 0;
+    U32Pack8 bs;
+    for (int i = 0; i < 8; ++i) bs.v[i] = i < K ? bs_host[i] : 1u;
+    for (int i = 0; i < K; ++i) ZK_ARG(bs.v[i] >= 1, "zk_softmax_decompose: zero radix");
+    Scratch flag(4);
+    if (flag.rc) return flag.rc;
+    ZK_HIP(hipMemsetAsync(flag.p, 0, 4, st));
+    LAUNCH1D(k_softmax_decompose, n, st, (Fr*)planes, flag.as<uint32_t>(), (const Fr*)X_shifted, bs, K, n);
+    uint32_t f = 0;
+    int rc = read_flag(flag.as<uint32_t>(), &f, st);
+    if (rc) return rc;
+    ZK_ARG(f == 0, "softmax: a shifted score is positive or exceeds the digit radices");
+    return 0;
+}
+
+}  // extern "C"

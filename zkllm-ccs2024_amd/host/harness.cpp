@@ -13,6 +13,9 @@
 #include "zkfc.hpp"
 #include "g1-tensor.hpp"
 #include "commitment.hpp"
+#include "tlookup.hpp"
+#include "rescaling.hpp"
+#include "zksoftmax.hpp"
 
 typedef uint32_t u32;
 static thread_local std::string g_err;
@@ -241,5 +244,102 @@ int zkp_open(void* gens, void* t, void* com, const u32* u, int k, u32* proof_out
     ZKP_END
 }
 void zkp_set_skip_g1_opening(int skip) { zk_set_skip_g1_opening(skip != 0); }
+
+// ---- lookup / rescaling / softmax -------------------------------------------------------------------------------
+static Fr_t fr1(const u32* p) { Fr_t x; memcpy(x.val, p, 32); return x; }
+
+// Rescaling::operator(): returns the rescaled tensor; *rem_out receives a copy of the remainder tensor
+void* zkp_rescale(void* X, u32 sf, void** rem_out) {
+    ZKP_TRY
+    Rescaling rs(sf);
+    FrTensor out = rs(FT(X));
+    if (rem_out) *rem_out = new FrTensor(*rs.rem_tensor_ptr);
+    return new FrTensor(std::move(out));
+    ZKP_END_PTR
+}
+// Rescaling::operator() + prove with challenges from the seeded stream
+void* zkp_rescale_prove(void* X, u32 sf) {
+    ZKP_TRY
+    Rescaling rs(sf);
+    FrTensor out = rs(FT(X));
+    rs.prove(FT(X), out);
+    return new FrTensor(std::move(out));
+    ZKP_END_PTR
+}
+void* zkp_range_prep(void* vals, int low, u32 len) { ZKP_TRY tLookupRange t(low, len); return new FrTensor(t.prep(FT(vals))); ZKP_END_PTR }
+void* zkp_batch_inv(void* in, const u32* beta) {
+    ZKP_TRY
+    FrTensor* out = new FrTensor(FT(in).size);
+    zk_check(zk_fr_batch_inv(out->gpu_data, FT(in).gpu_data, beta, FT(in).size, nullptr), "zk_fr_batch_inv");
+    return out;
+    ZKP_END_PTR
+}
+int zkp_range_prove(void* S, int low, u32 len, const u32* alpha, const u32* beta, const u32* u, const u32* v, u32* final_claim) {
+    ZKP_TRY
+    tLookupRange t(low, len);
+    FrTensor m = t.prep(FT(S));
+    const int k = (int)ceilLog2(FT(S).size);
+    std::vector<Polynomial> proof;
+    Fr_t f = t.prove(FT(S), m, fr1(alpha), fr1(beta), frs(u, k), frs(v, k), proof);
+    memcpy(final_claim, f.val, 32);
+    ZKP_END
+}
+// tLookupRangeMapping: y and m handles are returned through y_out / m_out; prove when final_claim != NULL
+int zkp_mapping(void* S_in, int low, u32 len, void* mvals, const u32* r, const u32* alpha, const u32* beta, const u32* u, const u32* v, void** y_out, void** m_out, u32* final_claim) {
+    ZKP_TRY
+    tLookupRangeMapping t(low, len, FT(mvals));
+    auto p = t(FT(S_in));
+    if (final_claim) {
+        const int k = (int)ceilLog2(FT(S_in).size);
+        std::vector<Polynomial> proof;
+        Fr_t f = t.prove(FT(S_in), p.first, p.second, fr1(r), fr1(alpha), fr1(beta), frs(u, k), frs(v, k), proof);
+        memcpy(final_claim, f.val, 32);
+    }
+    if (y_out) *y_out = new FrTensor(std::move(p.first));
+    if (m_out) *m_out = new FrTensor(std::move(p.second));
+    ZKP_END
+}
+// multi_hadamard_sumchecks with explicit challenges; proof_out: per round nX+1 coefficients
+int zkp_multi_hadamard(const u32* claim, void* const* Xs, int nX, const u32* u, const u32* v, int k, u32* proof_out, u32* final_claim) {
+    ZKP_TRY
+    std::vector<FrTensor> xs;
+    for (int i = 0; i < nX; ++i) xs.push_back(FT(Xs[i]));
+    std::vector<Polynomial> proof;
+    Fr_t f = multi_hadamard_sumchecks(fr1(claim), xs, frs(u, k), frs(v, k), proof);
+    size_t off = 0;
+    for (auto& p : proof) { memcpy(proof_out + off * 8, p.coefficients().data(), p.coefficients().size() * 32); off += p.coefficients().size(); }
+    memcpy(final_claim, f.val, 32);
+    ZKP_END
+}
+int zkp_hadamard_product_sumcheck(void* a, void* b, const u32* u, const u32* v, int k, u32* proof_out) {
+    ZKP_TRY
+    auto pr = hadamard_product_sumcheck(FT(a), FT(b), frs(u, k), frs(v, k));
+    memcpy(proof_out, pr.data(), pr.size() * 32);
+    ZKP_END
+}
+// zkSoftmax compute (+ prove with seeded challenges u_Y, v_Y, (r, alpha, beta)); returns Y, *shift_out the shift
+void* zkp_softmax(void* X, u32 m, u32 n, u32 d, const u32* bs, int K, u32 L, u32 M, uint64_t sf_in, const double* thetas, int nth, void** shift_out, int do_prove) {
+    ZKP_TRY
+    zkSoftmax sm(std::vector<uint>(bs, bs + K), L, M, (unsigned long)sf_in, std::vector<double>(thetas, thetas + nth), m, n, d, 1);
+    FrTensor shift(m), xs(m * n);
+    std::vector<FrTensor> xseg, yseg, mseg;
+    FrTensor y = sm.compute(FT(X), shift, xs, xseg, yseg, mseg);
+    if (do_prove) {
+        auto u_Y = random_vec(ceilLog2(y.size)), v_Y = random_vec(ceilLog2(y.size)), t3 = random_vec(3);
+        std::vector<Polynomial> proof;
+        sm.prove(y, FT(X), shift, xs, xseg, yseg, mseg, u_Y, v_Y, t3[0], t3[1], t3[2], proof);
+    }
+    if (shift_out) *shift_out = new FrTensor(std::move(shift));
+    return new FrTensor(std::move(y));
+    ZKP_END_PTR
+}
+int zkp_zkip_stacked(const u32* claim, void* A, void* B, u32 N, u32 D, const u32* uN, const u32* vN, int kN, const u32* uD, int kD, u32* proof_out, u32* final_claim) {
+    ZKP_TRY
+    std::vector<Polynomial> proof;
+    Fr_t f = zkip_stacked(fr1(claim), FT(A), FT(B), frs(uN, kN), frs(uD, kD), frs(vN, kN), N, D, proof);
+    for (size_t i = 0; i < proof.size(); ++i) memcpy(proof_out + i * 24, proof[i].coefficients().data(), 96);
+    memcpy(final_claim, f.val, 32);
+    ZKP_END
+}
 
 }  // extern "C"

@@ -14,3 +14,150 @@ void verifyWeightClaim(const Weight& w, const Claim& c) {
     if (opening != c.claim) throw std::runtime_error("verifyWeightClaim: opening != c.claim");
     cout << "Opening complete" << endl;
 }
+
+static const Fr_t kZero{{0, 0, 0, 0, 0, 0, 0, 0}};
+static const Fr_t kOne{{1, 0, 0, 0, 0, 0, 0, 0}};
+
+// proof.cu:191-241.  Each round is one pass over the tensors: the K+1 coefficient evaluations (inner
+// products with the eq table of u[:-1]) and the folds by v.back().
+Fr_t multi_hadamard_sumchecks(const Fr_t& claim0, const vector<FrTensor>& Xs, const vector<Fr_t>& u, const vector<Fr_t>& v, vector<Polynomial>& proof) {
+    uint N = Xs[0].size;
+    if (N == 1) return claim0;
+    if ((N & (N - 1)) != 0) throw std::runtime_error("N is not a power of 2");
+    const uint K = (uint)Xs.size();
+    if (K > 4) throw std::runtime_error("multi_hadamard_sumchecks: at most 4 factors are supported");
+    for (auto& X : Xs) if (X.size != N) throw std::runtime_error("Xs[i] size is not N");
+    const uint k = ceilLog2(N);
+    if (u.size() != k || v.size() != k) throw std::runtime_error("multi_hadamard_sumchecks: need ceilLog2(N) challenges");
+    Fr_t claim = claim0;
+    std::vector<FrTensor> keep, E;
+    keep.reserve((size_t)K * k);
+    E.emplace_back(1u << (k - 1));
+    ZKC(zk_eq_table(E.back().gpu_data, u[0].val, (int)k - 1, nullptr));
+    std::vector<const void*> cur(K);
+    for (uint i = 0; i < K; ++i) cur[i] = Xs[i].gpu_data;
+    for (uint r = 0; r < k; ++r) {
+        const uint half = N >> (r + 1);
+        std::vector<void*> nxt(K);
+        for (uint i = 0; i < K; ++i) { keep.emplace_back(half); nxt[i] = keep.back().gpu_data; }
+        std::vector<Fr_t> coefs(K + 1);
+        ZKC(zk_hadamard_round(coefs[0].val, nxt.data(), cur.data(), (int)K, E.back().gpu_data, v[k - 1 - r].val, half, nullptr));
+        proof.push_back(Polynomial(coefs));
+        zk_record(coefs);
+        Polynomial p = proof.back() * Polynomial::eq(u[k - 1 - r]);
+        if (claim != p(kZero) + p(kOne)) throw std::runtime_error("multi_hadamard_sumchecks: claim != p(0) + p(1)");
+        claim = proof.back()(v[k - 1 - r]);
+        for (uint i = 0; i < K; ++i) cur[i] = nxt[i];
+        if (r + 1 < k) {
+            const uint next = half >> 1;
+            E.emplace_back(next ? next : 1);
+            ZKC(zk_eq_halve(E.back().gpu_data, E[E.size() - 2].gpu_data, next, nullptr));
+        }
+    }
+    return claim;
+}
+
+// ---- deprecated sumchecks (proof.cu:12-157): adjacent-pair folding, first challenge first -------------------
+// even / odd entries of a (zero-extended) as tensors of (n+1)/2 elements: a fold by 0 keeps the even entry,
+// a fold by 1 the odd one.
+static FrTensor pick(const FrTensor& a, const Fr_t& which) {
+    FrTensor out((a.size + 1) / 2);
+    ZKC(zk_fr_fold_axis(out.gpu_data, a.gpu_data, which.val, 1, 1, a.size, 1, nullptr));
+    return out;
+}
+static FrTensor fold_first(const FrTensor& a, const Fr_t& x) { return pick(a, x); }
+static FrTensor raw_mul(const FrTensor& a, const FrTensor& b) {   // a*b*R^-1, as the deprecated step kernels compute
+    FrTensor out(a.size);
+    ZKC(zk_fr_montmul(out.gpu_data, a.gpu_data, b.gpu_data, a.size, nullptr));
+    return out;
+}
+// Fr_ip_sc_step (proof.cu:12-27): note the missing re-Montgomery, kept as is
+static void ip_sc_terms(const FrTensor& a, const FrTensor& b, FrTensor& o0, FrTensor& o1, FrTensor& o2) {
+    FrTensor a0 = pick(a, kZero), a1 = pick(a, kOne), b0 = pick(b, kZero), b1 = pick(b, kOne);
+    FrTensor da = a1 - a0, db = b1 - b0;
+    ZKC(zk_fr_montmul(o0.gpu_data, a0.gpu_data, b0.gpu_data, o0.size, nullptr));
+    FrTensor t1 = raw_mul(a0, db), t2 = raw_mul(b0, da);
+    ZKC(zk_fr_add(o1.gpu_data, t1.gpu_data, t2.gpu_data, o1.size, nullptr));
+    ZKC(zk_fr_montmul(o2.gpu_data, da.gpu_data, db.gpu_data, o2.size, nullptr));
+}
+
+vector<Fr_t> inner_product_sumcheck(const FrTensor& a0, const FrTensor& b0, vector<Fr_t> u) {
+    vector<Fr_t> proof;
+    uint log_size = (uint)u.size();
+    if (a0.size != b0.size) throw std::runtime_error("Incompatible dimensions");
+    if (a0.size <= (1u << log_size) / 2) throw std::runtime_error("Incompatible dimensions");
+    if (a0.size > (1u << log_size)) throw std::runtime_error("Incompatible dimensions");
+    FrTensor a(a0), b(b0);
+    std::vector<FrTensor> ka, kb;
+    const FrTensor *pa = &a0, *pb = &b0;
+    ka.reserve(u.size()); kb.reserve(u.size());
+    for (size_t i = 0; i < u.size(); ++i) {
+        uint out_size = (pa->size + 1) / 2;
+        FrTensor o0(out_size), o1(out_size), o2(out_size);
+        ip_sc_terms(*pa, *pb, o0, o1, o2);
+        proof.push_back(o0.sum());
+        proof.push_back(o1.sum());
+        proof.push_back(o2.sum());
+        ka.push_back(fold_first(*pa, u[i]));
+        kb.push_back(fold_first(*pb, u[i]));
+        pa = &ka.back(); pb = &kb.back();
+    }
+    proof.push_back((*pa)(0u));
+    proof.push_back((*pb)(0u));
+    return proof;
+}
+
+vector<Fr_t> hadamard_product_sumcheck(const FrTensor& a0, const FrTensor& b0, vector<Fr_t> u, vector<Fr_t> v) {
+    vector<Fr_t> proof;
+    if (u.size() != v.size()) throw std::runtime_error("Incompatible dimensions 1");
+    uint log_size = (uint)u.size();
+    if (a0.size != b0.size) throw std::runtime_error("Incompatible dimensions 2");
+    if (log_size == 0 || a0.size <= (1u << (log_size - 1))) throw std::runtime_error("Incompatible dimensions 3");
+    if (a0.size > (1u << log_size)) throw std::runtime_error("Incompatible dimensions 4");
+    std::vector<FrTensor> ka, kb;
+    const FrTensor *pa = &a0, *pb = &b0;
+    ka.reserve(u.size()); kb.reserve(u.size());
+    for (size_t i = 0; i < u.size(); ++i) {
+        uint out_size = (pa->size + 1) / 2;
+        FrTensor o0(out_size), o1(out_size), o2(out_size);
+        ip_sc_terms(*pa, *pb, o0, o1, o2);
+        vector<Fr_t> u_(u.begin() + i + 1, u.end());
+        proof.push_back(o0(u_));
+        proof.push_back(o1(u_));
+        proof.push_back(o2(u_));
+        ka.push_back(fold_first(*pa, v[i]));
+        kb.push_back(fold_first(*pb, v[i]));
+        pa = &ka.back(); pb = &kb.back();
+    }
+    proof.push_back((*pa)(0u));
+    proof.push_back((*pb)(0u));
+    zk_record(proof);
+    return proof;
+}
+
+// Fr_bin_sc_step (proof.cu:109-120)
+vector<Fr_t> binary_sumcheck(const FrTensor& a0, vector<Fr_t> u, vector<Fr_t> v) {
+    vector<Fr_t> proof;
+    if (u.size() != v.size()) throw std::runtime_error("Incompatible dimensions");
+    uint log_size = (uint)u.size();
+    if (a0.size <= (1u << log_size) / 2) throw std::runtime_error("Incompatible dimensions");
+    if (a0.size > (1u << log_size)) throw std::runtime_error("Incompatible dimensions");
+    std::vector<FrTensor> ka;
+    const FrTensor* pa = &a0;
+    ka.reserve(u.size());
+    for (size_t i = 0; i < u.size(); ++i) {
+        FrTensor x0 = pick(*pa, kZero), x1 = pick(*pa, kOne);
+        FrTensor diff = x1 - x0;
+        FrTensor o0 = raw_mul(x0, x0) - x0;
+        FrTensor o1 = raw_mul(x0 + x0, diff) - diff;
+        FrTensor o2 = raw_mul(diff, diff);
+        vector<Fr_t> u_(u.begin() + i + 1, u.end());
+        proof.push_back(o0(u_));
+        proof.push_back(o1(u_));
+        proof.push_back(o2(u_));
+        ka.push_back(fold_first(*pa, v[i]));
+        pa = &ka.back();
+    }
+    proof.push_back((*pa)(0u));
+    return proof;
+}

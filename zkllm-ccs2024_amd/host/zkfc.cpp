@@ -115,3 +115,91 @@ Fr_t zkip(const Fr_t& claim0, const FrTensor& a0, const FrTensor& b0, const vect
     }
     return claim;
 }
+
+// zkfc.cu:187-229.  Rounds over the stacking axis N of [N][D] tensors; then zkip over D.
+Fr_t zkip_stacked(const Fr_t& claim0, const FrTensor& A0, const FrTensor& B0, const vector<Fr_t>& uN, const vector<Fr_t>& uD, const vector<Fr_t> vN, uint N, uint D, vector<Polynomial>& proof) {
+    if (uN.empty()) return zkip(claim0, A0, B0, uD, proof);
+    if (vN.size() != uN.size()) throw std::runtime_error("zkip_stacked: uN and vN differ in length");
+    if (A0.size != N * D) throw std::runtime_error("a.size != N * D");
+    if (B0.size != N * D) throw std::runtime_error("b.size != N * D");
+    if (uN.size() != ceilLog2(N)) throw std::runtime_error("zkip_stacked: uN.size() != ceilLog2(N)");
+    Fr_t claim = claim0;
+    const FrTensor* a = &A0;
+    const FrTensor* b = &B0;
+    std::vector<FrTensor> keep, E;
+    keep.reserve(2 * uN.size());
+    const uint kN = (uint)uN.size();
+    E.emplace_back(1u << (kN - 1));
+    ZKC(zk_eq_table(E.back().gpu_data, uN[0].val, (int)kN - 1, nullptr));
+    uint n = N;
+    for (uint r = 0; r < kN; ++r) {
+        const uint n_out = (1u << ceilLog2(n)) >> 1;
+        Fr_t c[3];
+        ZKC(zk_ip_round_stacked(c[0].val, a->gpu_data, b->gpu_data, E.back().gpu_data, D, n, n_out, nullptr));
+        Polynomial p({c[0], c[1], c[2]});
+        proof.push_back(p);
+        zk_record(p.coefficients());
+        Polynomial q = Polynomial::eq(uN[kN - 1 - r]) * p;
+        if (claim != q(TEMP_ZERO) + q(TEMP_ONE)) throw std::runtime_error("claim != q(0) + q(1)");
+        claim = p(vN[kN - 1 - r]);
+        keep.emplace_back(n_out * D);
+        keep.emplace_back(n_out * D);
+        FrTensor& na = keep[keep.size() - 2];
+        FrTensor& nb = keep[keep.size() - 1];
+        ZKC(zk_fr_fold_halves(na.gpu_data, a->gpu_data, vN[kN - 1 - r].val, (size_t)n * D, (size_t)n_out * D, nullptr));
+        ZKC(zk_fr_fold_halves(nb.gpu_data, b->gpu_data, vN[kN - 1 - r].val, (size_t)n * D, (size_t)n_out * D, nullptr));
+        a = &na;
+        b = &nb;
+        n = n_out;
+        if (r + 1 < kN) {
+            const uint next = n_out >> 1;
+            E.emplace_back(next ? next : 1);
+            ZKC(zk_eq_halve(E.back().gpu_data, E[E.size() - 2].gpu_data, next, nullptr));
+        }
+    }
+    return zkip(claim, *a, *b, uD, proof);
+}
+
+static FrTensor catLayerWeights(const vector<zkFC>& layers) {
+    vector<FrTensor> ws;
+    for (auto& l : layers) ws.push_back(l.weights);
+    return catTensors(ws);
+}
+static FrTensor catLayerBiases(const vector<zkFC>& layers) {
+    vector<FrTensor> bs;
+    for (auto& l : layers) bs.push_back(l.bias);
+    return catTensors(bs);
+}
+
+zkFCStacked::zkFCStacked(bool has_bias, uint num, uint batch_size, uint input_size, uint output_size, const vector<zkFC>& layers, const vector<FrTensor>& Xs, const vector<FrTensor>& Ys)
+    : has_bias(has_bias), num(num), batchSize(batch_size), inputSize(input_size), outputSize(output_size),
+      X(catTensors(Xs)), W(catLayerWeights(layers)), b(catLayerBiases(layers)), Y(catTensors(Ys)) {
+    if (X.size != num * batchSize * inputSize) throw std::runtime_error("X size does not match");
+    if (Y.size != num * batchSize * outputSize) throw std::runtime_error("Y size does not match");
+    if (W.size != num * inputSize * outputSize) throw std::runtime_error("W size does not match");
+    if (has_bias && b.size != num * outputSize) throw std::runtime_error("b size does not match");
+}
+
+void zkFCStacked::prove(vector<Polynomial>& proof) const {
+    auto u_num = random_vec(ceilLog2(num));
+    auto v_num = random_vec(ceilLog2(num));
+    auto u_batch = random_vec(ceilLog2(batchSize));
+    auto u_input = random_vec(ceilLog2(inputSize));
+    auto u_output = random_vec(ceilLog2(outputSize));
+    prove(u_num, v_num, u_batch, u_input, u_output, proof);
+}
+
+void zkFCStacked::prove(const vector<Fr_t>& u_num, const vector<Fr_t>& v_num, const vector<Fr_t>& u_batch, const vector<Fr_t>& u_input, const vector<Fr_t>& u_output, vector<Polynomial>& proof) const {
+    auto claim = Y.multi_dim_me({u_num, u_batch, u_output}, {num, batchSize, outputSize});
+    if (has_bias) {
+        FrTensor ones = FrTensor::filled(batchSize, TEMP_ONE);
+        claim = claim - ones(u_batch) * b.multi_dim_me({u_num, u_output}, {num, outputSize});
+    }
+    zk_record(claim);
+    auto X_reduced = X.partial_me(u_batch, batchSize, inputSize);
+    auto W_reduced = W.partial_me(u_output, outputSize, 1);
+    auto final_claim = zkip_stacked(claim, X_reduced, W_reduced, u_num, u_input, v_num, num, inputSize, proof);
+    auto opening = X.multi_dim_me({v_num, u_batch, u_input}, {num, batchSize, inputSize}) * W.multi_dim_me({v_num, u_input, u_output}, {num, inputSize, outputSize});
+    zk_record(final_claim);
+    if (final_claim != opening) throw std::runtime_error("final claim != opening");
+}

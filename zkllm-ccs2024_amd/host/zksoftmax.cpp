@@ -1,0 +1,185 @@
+#include "zksoftmax.hpp"
+
+#include <cmath>
+
+#include "../../include/zkllm_hip.h"
+#include "../csrc/detmath.hpp"
+
+#define ZKC(call) zk_check((call), #call)
+
+// zksoftmax.cu:34-93.  Exp tables are evaluated with the deterministic exp/log of csrc/detmath.hpp (the
+// reference calls the CUDA device libm, which cannot be reproduced bit for bit anywhere else).
+zkSoftmax::zkSoftmax(const vector<uint>& bs, uint L, uint M, unsigned long scaling_factor_in, const vector<double>& thetas, uint m, uint n, uint d, uint E)
+    : bs(bs), K((uint)bs.size()), L(L), M(M), scaling_factor_in(scaling_factor_in), thetas(thetas), m(m), n(n), d(d), E(E) {
+    if (K - L - M != thetas.size()) throw std::invalid_argument("bs and thetas must have the same size");
+    if (K <= L + M) throw std::invalid_argument("K must be greater than L + M");
+    if (K > 8) throw std::invalid_argument("at most 8 segments are supported");
+
+    vector<unsigned long> Bs(K);
+    Bs[0] = 1UL;
+    for (uint i = 1; i < K; i++) Bs[i] = Bs[i - 1] * static_cast<unsigned long>(bs[i - 1]);
+
+    least_significant_segments.reserve(L);
+    other_segments.reserve(K - L);
+    for (uint i = 0; i < L; ++i) least_significant_segments.emplace_back(0, bs[i]);
+
+    const double sfd = static_cast<double>(scaling_factor_in), dd = static_cast<double>(d);
+    const double scale = sfd * std::sqrt(dd);
+    for (uint i = L; i < K - M; ++i) {
+        FrTensor mapped_values(bs[i]);
+        const double step = static_cast<double>(Bs[i]) / scale;
+        ZKC(zk_softmax_table(mapped_values.gpu_data, zkd::log_det(thetas[i - L]), step, bs[i], nullptr));
+        other_segments.emplace_back(0, bs[i], mapped_values);
+    }
+    for (uint i = K - M; i < K; ++i) {
+        // indicator of digit 0 (`int mvals[bs[i]] = {1}` in the reference)
+        std::vector<int> mvals(bs[i], 0);
+        mvals[0] = 1;
+        FrTensor mapped_values(bs[i], mvals.data());
+        other_segments.emplace_back(0, bs[i], mapped_values);
+    }
+}
+
+// zksoftmax.cu:112-173
+FrTensor zkSoftmax::compute(const FrTensor& X, FrTensor& shift, FrTensor& X_shifted, vector<FrTensor>& X_segments, vector<FrTensor>& Y_segments, vector<FrTensor>& m_segments) {
+    if (X.size != m * n) throw std::invalid_argument("X must be m * n");
+    if (shift.size != m) throw std::invalid_argument("shift must be m");
+    if (X_shifted.size != X.size) throw std::invalid_argument("X_shifted must be the same size as X");
+
+    const double scale = static_cast<double>(scaling_factor_in) * std::sqrt(static_cast<double>(d));
+    ZKC(zk_softmax_shift(shift.gpu_data, X_shifted.gpu_data, X.gpu_data, m, n, scale, nullptr));
+
+    const size_t N = (size_t)m * n;
+    FrTensor planes((uint)(N * K));
+    ZKC(zk_softmax_decompose(planes.gpu_data, X_shifted.gpu_data, bs.data(), (int)K, N, nullptr));
+
+    FrTensor out = FrTensor::filled((uint)N, Fr_t{{1, 0, 0, 0, 0, 0, 0, 0}});
+    X_segments.reserve(K);
+    for (uint i = 0; i < L; ++i) {
+        X_segments.push_back(planes.trunc((uint)(i * N), (uint)((i + 1) * N)));
+        m_segments.push_back(least_significant_segments[i].prep(X_segments[i]));
+    }
+    for (uint i = L; i < K; ++i) {
+        X_segments.push_back(planes.trunc((uint)(i * N), (uint)((i + 1) * N)));
+        auto p = other_segments[i - L](X_segments[i]);
+        out *= p.first;
+        Y_segments.push_back(std::move(p.first));
+        m_segments.push_back(std::move(p.second));
+    }
+    return out;
+}
+
+// zksoftmax.cu:175-220
+Fr_t zkSoftmax::prove(const FrTensor& Y, const FrTensor& X, const FrTensor& shift, const FrTensor& X_shifted, const vector<FrTensor>& X_segments,
+                      const vector<FrTensor>& Y_segments, const vector<FrTensor>& m_segments, const vector<Fr_t>& u_Y, const vector<Fr_t>& v_Y, const Fr_t& r_seg,
+                      const Fr_t& alpha_seg, const Fr_t& beta_seg, vector<Polynomial>& proof) {
+    uint N = Y.size;
+    if (X.size != N) throw std::invalid_argument("X and Y must have the same size " + to_string(X.size) + " " + to_string(Y.size));
+
+    auto claim_Y = Y(u_Y);
+    zk_record(claim_Y);
+    multi_hadamard_sumchecks(claim_Y, Y_segments, u_Y, v_Y, proof);
+
+    for (uint i = 0; i < L; ++i) least_significant_segments[i].prove(X_segments[i], m_segments[i], alpha_seg, beta_seg, u_Y, v_Y, proof);
+    for (uint i = L; i < K; ++i) other_segments[i - L].prove(X_segments[i], Y_segments[i - L], m_segments[i], r_seg, alpha_seg, beta_seg, u_Y, v_Y, proof);
+
+    vector<Fr_t> Y_seg_claims, X_seg_claims;
+    for (uint i = L; i < K; ++i) Y_seg_claims.push_back(Y_segments[i - L](v_Y));
+    for (uint i = 0; i < K; ++i) X_seg_claims.push_back(X_segments[i](v_Y));
+    zk_record(Y_seg_claims);
+    zk_record(X_seg_claims);
+
+    Fr_t minus_X_shifted_claim = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int i = (int)bs.size() - 1; i >= 0; --i) minus_X_shifted_claim = minus_X_shifted_claim * Fr_t({bs[i], 0, 0, 0, 0, 0, 0, 0}) + X_seg_claims[i];
+
+    vector<Fr_t> v_Y_(v_Y.begin() + ceilLog2(n), v_Y.end());
+    auto shift_const_opening = shift(v_Y_);
+    auto X_opening = X(v_Y);
+    zk_record(shift_const_opening);
+    zk_record(X_opening);
+    if (shift_const_opening - minus_X_shifted_claim != X_opening) throw std::runtime_error("X claim is not correct");
+    return X_opening;
+}
+
+// ---- attention wrappers (zksoftmax.cu:222-320) --------------------------------------------------------------
+zkAttn::zkAttn(unsigned long sf_Q, unsigned long sf_K, const vector<uint>& bs, uint L, uint M, const vector<double>& thetas, uint m, uint n, uint d, uint E)
+    : zkSoftmax(bs, L, M, sf_Q * sf_K, thetas, m, n, d, E) {}
+
+FrTensor zkAttn::compute(const FrTensor& Q, const FrTensor& K, const FrTensor& V, FrTensor& sm_in, FrTensor& sm_out, FrTensor& sm_shift, FrTensor& sm_in_shifted,
+                         vector<FrTensor>& sm_in_segments, vector<FrTensor>& sm_out_segments, vector<FrTensor>& sm_m_segments) {
+    if (Q.size != m * d) throw std::invalid_argument("Q must be m * d");
+    if (K.size != n * d) throw std::invalid_argument("K must be n * d");
+    if (V.size != n * d) throw std::invalid_argument("V must be n * d");
+    sm_in = FrTensor::matmul(Q, K.transpose(n, d), m, d, n);
+    sm_out = zkSoftmax::compute(sm_in, sm_shift, sm_in_shifted, sm_in_segments, sm_out_segments, sm_m_segments);
+    return FrTensor::matmul(sm_out, V, m, n, d);
+}
+
+vector<Claim> zkAttn::prove(const FrTensor& Q, const FrTensor& K, const FrTensor& V, const FrTensor& out, const FrTensor& sm_out, const FrTensor& sm_in,
+                            const FrTensor& sm_shift, const FrTensor& sm_in_shifted, const vector<FrTensor>& sm_in_segments, const vector<FrTensor>& sm_out_segments,
+                            const vector<FrTensor>& sm_m_segments) {
+    auto u_matmul_out = random_vec(ceilLog2(m));
+    auto v_matmul_out = random_vec(ceilLog2(n));
+    auto w_matmul_out = random_vec(ceilLog2(d));
+    auto v_sm = random_vec(ceilLog2(m) + ceilLog2(n));
+    auto temp_rand = random_vec(3);
+    auto v_matmul_in = random_vec(ceilLog2(d));
+    vector<Polynomial> proof;
+    this->prove(Q, K, V, out, sm_out, sm_in, sm_shift, sm_in_shifted, sm_in_segments, sm_out_segments, sm_m_segments, u_matmul_out, v_matmul_out, w_matmul_out, v_sm,
+                temp_rand[0], temp_rand[1], temp_rand[2], v_matmul_in, proof);
+    cout << "zkAttn proof complete." << endl;
+    return {};
+}
+
+Fr_t zkAttn::prove(const FrTensor& Q, const FrTensor& K, const FrTensor& V, const FrTensor& out, const FrTensor& sm_out, const FrTensor& sm_in, const FrTensor& sm_shift,
+                   const FrTensor& sm_in_shifted, const vector<FrTensor>& sm_in_segments, const vector<FrTensor>& sm_out_segments, const vector<FrTensor>& sm_m_segments,
+                   const vector<Fr_t>& u_matmul_out, const vector<Fr_t>& v_matmul_out, const vector<Fr_t>& w_matmul_out, const vector<Fr_t>& v_sm, const Fr_t& r_seg,
+                   const Fr_t& alpha_seg, const Fr_t& beta_seg, const vector<Fr_t>& v_matmul_in, vector<Polynomial>& proof) {
+    auto out_claim = out.multi_dim_me({u_matmul_out, w_matmul_out}, {m, d});
+    zk_record(out_claim);
+    auto out_vec0 = sm_out.partial_me(u_matmul_out, m, n);
+    auto out_vec1 = V.partial_me(w_matmul_out, d, 1);
+    auto out_matmul_claim = zkip(out_claim, out_vec0, out_vec1, v_matmul_out, proof);
+
+    auto V_claim = out_vec1(v_matmul_out);        // = V.multi_dim_me({v_matmul_out, w_matmul_out}, {n, d})
+    auto sm_out_claim = out_vec0(v_matmul_out);   // = sm_out.multi_dim_me({u_matmul_out, v_matmul_out}, {m, n})
+    if (out_matmul_claim != V_claim * sm_out_claim) throw std::runtime_error("out_matmul_claim is not correct");
+
+    auto sm_in_claim = zkSoftmax::prove(sm_out, sm_in, sm_shift, sm_in_shifted, sm_in_segments, sm_out_segments, sm_m_segments,
+                                        concatenate<Fr_t>({v_matmul_out, u_matmul_out}), v_sm, r_seg, alpha_seg, beta_seg, proof);
+
+    vector<Fr_t> u_matmul_in(v_sm.end() - ceilLog2(m), v_sm.end());
+    vector<Fr_t> w_matmul_in(v_sm.begin(), v_sm.end() - ceilLog2(m));
+    auto q = Q.partial_me(u_matmul_in, m, d);
+    auto k = K.partial_me(w_matmul_in, n, d);   // K is n x d: folding its rows gives the transposed operand
+    return zkip(sm_in_claim, q, k, v_matmul_in, proof);
+}
+
+zkAttnStacked::zkAttnStacked(uint num, unsigned long sf_Q, unsigned long sf_K, const vector<uint>& bs, uint L, uint M, const vector<double>& thetas, uint m, uint n, uint d, uint E)
+    : zkAttn(sf_Q, sf_K, bs, L, M, thetas, m, n, d, E), num(num) {}
+
+Fr_t zkAttnStacked::prove(const FrTensor& Q, const FrTensor& K, const FrTensor& V, const FrTensor& out, const FrTensor& sm_out, const FrTensor& sm_in,
+                          const FrTensor& sm_shift, const FrTensor& sm_in_shifted, const vector<FrTensor>& sm_in_segments, const vector<FrTensor>& sm_out_segments,
+                          const vector<FrTensor>& sm_m_segments, const vector<Fr_t>& u_matmul_out_num, const vector<Fr_t>& v_matmul_out_num,
+                          const vector<Fr_t>& u_matmul_out, const vector<Fr_t>& v_matmul_out, const vector<Fr_t>& w_matmul_out, const vector<Fr_t>& v_sm, const Fr_t& r_seg,
+                          const Fr_t& alpha_seg, const Fr_t& beta_seg, const vector<Fr_t>& v_matmul_in_num, const vector<Fr_t>& v_matmul_in, vector<Polynomial>& proof) {
+    auto out_claim = out.multi_dim_me({u_matmul_out_num, u_matmul_out, w_matmul_out}, {num, m, d});
+    zk_record(out_claim);
+    auto sm_out_reduced = sm_out.partial_me(u_matmul_out, m, n);
+    auto V_reduced = V.partial_me(w_matmul_out, d, 1);
+    auto out_matmul_claim = zkip_stacked(out_claim, sm_out_reduced, V_reduced, u_matmul_out_num, v_matmul_out, v_matmul_out_num, num, n, proof);
+
+    auto V_claim = V.multi_dim_me({v_matmul_out_num, v_matmul_out, w_matmul_out}, {num, n, d});
+    auto sm_out_claim = sm_out.multi_dim_me({v_matmul_out_num, u_matmul_out, v_matmul_out}, {num, m, n});
+    if (out_matmul_claim != V_claim * sm_out_claim) throw std::runtime_error("out_matmul_claim is not correct");
+
+    auto sm_in_claim = zkSoftmax::prove(sm_out, sm_in, sm_shift, sm_in_shifted, sm_in_segments, sm_out_segments, sm_m_segments,
+                                        concatenate<Fr_t>({v_matmul_out, u_matmul_out, v_matmul_out_num}), v_sm, r_seg, alpha_seg, beta_seg, proof);
+
+    vector<Fr_t> u_matmul_in_num(v_sm.end() - ceilLog2(num), v_sm.end());
+    vector<Fr_t> u_matmul_in(v_sm.end() - ceilLog2(num) - ceilLog2(m), v_sm.end() - ceilLog2(num));
+    vector<Fr_t> w_matmul_in(v_sm.begin(), v_sm.end() - ceilLog2(num) - ceilLog2(m));
+    auto Q_reduced = Q.partial_me(u_matmul_in, m, d);
+    auto K_reduced = K.partial_me(w_matmul_in, n, d);
+    return zkip_stacked(sm_in_claim, Q_reduced, K_reduced, u_matmul_in_num, v_matmul_in, v_matmul_in_num, num, d, proof);
+}
