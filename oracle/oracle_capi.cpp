@@ -6,7 +6,7 @@
 #include <cstring>
 #include <string>
 #include <omp.h>
-#include "protocols.hpp"
+#include "layer_ref.hpp"
 
 using namespace orc;
 typedef uint32_t u32;
@@ -294,6 +294,45 @@ int orc_open(const u32* gens, long ngen, const u32* t, long n, u32 com_size, con
     Fr v = commitment_open(g1_in(gens, ngen), vec_in(t, n), com_size, vec_in(u, k), proof);
     if (proof_out) g1_out(proof, proof_out);
     std::memcpy(value, &v, 32);
+    ORC_END
+}
+
+// ---- whole decoder layer (same argument packing as the product's harness) -------------------------------------------
+static OLayerConfig parse_cfg(const u32* cu, const double* cf) {
+    OLayerConfig c;
+    c.seq_len = cu[0]; c.embed_dim = cu[1]; c.num_heads = cu[2]; c.hidden_dim = cu[3];
+    c.sf_linear = cu[4]; c.sf_gate = cu[5]; c.sf_attn = cu[6]; c.softmax_L = cu[7]; c.softmax_M = cu[8];
+    c.swiglu_len = cu[9]; c.open_weights = cu[10] != 0;
+    const u32 K = cu[11];
+    c.softmax_bs.assign(cu + 12, cu + 12 + K);
+    c.softmax_sf_in = (uint64_t)cf[0]; c.swiglu_low = (int)cf[1]; c.swiglu_in_scale = cf[2]; c.swiglu_out_scale = cf[3]; c.rms_eps = cf[4]; c.value_scale = cf[5];
+    c.softmax_thetas.assign(cf + 6, cf + 6 + (K - c.softmax_L - c.softmax_M));
+    return c;
+}
+// generators are drawn from the seeded stream in the order norm1, q, k, v, o, norm2, up, gate, down; then the layer runs.
+// out: seq*embed elements.  com_out (optional): the nine commitments concatenated in that order.
+int orc_layer(const u32* cu, const double* cf, const int32_t* norm1, const int32_t* wq, const int32_t* wk, const int32_t* wv, const int32_t* wo,
+              const int32_t* norm2, const int32_t* wup, const int32_t* wgate, const int32_t* wdown, u32 lof, const int32_t* X, u32* out, u32* com_out) {
+    ORC_TRY
+    OLayerConfig c = parse_cfg(cu, cf);
+    const uint E = c.embed_dim, Hd = c.hidden_dim, S = c.seq_len;
+    OWeight n1 = o_make_weight(norm1, 1, E, E), q = o_make_weight(wq, E, E, E << lof), k = o_make_weight(wk, E, E, E << lof), v = o_make_weight(wv, E, E, E << lof),
+            o = o_make_weight(wo, E, E, E << lof), n2 = o_make_weight(norm2, 1, E, E), up = o_make_weight(wup, E, Hd, Hd << lof),
+            gate = o_make_weight(wgate, E, Hd, Hd << lof), down = o_make_weight(wdown, Hd, E, E << lof);
+    if (com_out) {
+        size_t off = 0;
+        for (const OWeight* w : {&n1, &q, &k, &v, &o, &n2, &up, &gate, &down}) { g1_out(w->com, com_out + off * 36); off += w->com.size(); }
+    }
+    FrVec table = o_swiglu_table(c.swiglu_low, c.swiglu_len, c.swiglu_in_scale, c.swiglu_out_scale);
+    FrVec x = t_from_i32(X, (size_t)S * E);
+    FrVec a = o_rmsnorm_block(c, n1, x, o_compute_rms_inv(x, S, E, c.rms_eps, c.value_scale));
+    FrVec Q_, K_, V_;
+    o_attn_linear_block(c, q, k, v, a, Q_, K_, V_);
+    FrVec att = o_attn_heads_block(c, Q_, K_, V_);
+    FrVec x2 = t_add(x, o_oproj_block(c, o, att));
+    FrVec b = o_rmsnorm_block(c, n2, x2, o_compute_rms_inv(x2, S, E, c.rms_eps, c.value_scale));
+    FrVec y = t_add(x2, o_ffn_block(c, up, gate, down, table, b));
+    vec_out(y, out);
     ORC_END
 }
 

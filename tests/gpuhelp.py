@@ -157,7 +157,8 @@ class Prover:
                      "zkp_fr_pad", "zkp_fr_transpose", "zkp_fr_matmul",
                      "zkp_g1_from_host", "zkp_g1_from_file", "zkp_g1_devptr", "zkp_commitment_random", "zkp_g1_binop", "zkp_g1_pointop",
                      "zkp_g1_scalar_mul", "zkp_g1_rowwise_sum", "zkp_commit_int", "zkp_commit",
-                     "zkp_rescale", "zkp_rescale_prove", "zkp_range_prep", "zkp_batch_inv", "zkp_softmax"):
+                     "zkp_rescale", "zkp_rescale_prove", "zkp_range_prep", "zkp_batch_inv", "zkp_softmax",
+                     "zkp_layer_create", "zkp_layer_create_random", "zkp_layer_run"):
             getattr(L, name).restype = c_void_p
         L.zkp_transcript_size.restype = ctypes.c_long
         L.zkp_fr_size.restype = c_uint
@@ -355,6 +356,28 @@ class Prover:
         self.check(self.lib.zkp_zkip_stacked(_np_ptr(claim), c_void_p(A.h), c_void_p(B.h), c_uint(N), c_uint(D), _np_ptr(uN), _np_ptr(vN), c_int(kN),
                                              _np_ptr(uD), c_int(kD), _np_ptr(proof), _np_ptr(fin)))
         return proof, fin
+
+    # ---- decoder layer ----
+    def layer_create(self, cu, cf, weights, log_off_factor):
+        ws = [np.ascontiguousarray(w, dtype=np.int32) for w in weights]
+        h = self.lib.zkp_layer_create(_np_ptr(cu), _np_ptr(cf), *[_np_ptr(w) for w in ws], c_uint(log_off_factor))
+        if not h:
+            raise RuntimeError("prover error: " + self.lib.zkp_last_error().decode())
+        return h
+
+    def layer_create_random(self, cu, cf, seed, log_off_factor):
+        h = self.lib.zkp_layer_create_random(_np_ptr(cu), _np_ptr(cf), c_uint(seed), c_uint(log_off_factor))
+        if not h:
+            raise RuntimeError("prover error: " + self.lib.zkp_last_error().decode())
+        return h
+
+    def layer_run(self, layer, X):
+        times = np.zeros(7, np.float64)
+        out = self.H(self.lib.zkp_layer_run(c_void_p(layer), c_void_p(X.h), _np_ptr(times)))
+        return out, times
+
+    def layer_free(self, layer):
+        self.lib.zkp_layer_free(c_void_p(layer))
 
     # ---- transcript / challenges ----
     def seed(self, s):

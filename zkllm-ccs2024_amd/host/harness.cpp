@@ -16,6 +16,7 @@
 #include "tlookup.hpp"
 #include "rescaling.hpp"
 #include "zksoftmax.hpp"
+#include "layer.hpp"
 
 typedef uint32_t u32;
 static thread_local std::string g_err;
@@ -340,6 +341,60 @@ int zkp_zkip_stacked(const u32* claim, void* A, void* B, u32 N, u32 D, const u32
     for (size_t i = 0; i < proof.size(); ++i) memcpy(proof_out + i * 24, proof[i].coefficients().data(), 96);
     memcpy(final_claim, f.val, 32);
     ZKP_END
+}
+
+// ---- whole decoder layer ------------------------------------------------------------------------------------------
+// cfg_u32: seq, embed, heads, hidden, sf_linear, sf_gate, sf_attn, softmax L, softmax M, swiglu_len, open_weights, K, bs[0..K)
+// cfg_f64: softmax_sf_in, swiglu_low, swiglu_in_scale, swiglu_out_scale, rms_eps, value_scale, thetas[0..K-L-M)
+static LayerConfig parse_cfg(const u32* cu, const double* cf) {
+    LayerConfig c;
+    c.seq_len = cu[0]; c.embed_dim = cu[1]; c.num_heads = cu[2]; c.hidden_dim = cu[3];
+    c.sf_linear = cu[4]; c.sf_gate = cu[5]; c.sf_attn = cu[6]; c.softmax_L = cu[7]; c.softmax_M = cu[8];
+    c.swiglu_len = cu[9]; c.open_weights = cu[10] != 0;
+    const u32 K = cu[11];
+    c.softmax_bs.assign(cu + 12, cu + 12 + K);
+    c.softmax_sf_in = (unsigned long)cf[0]; c.swiglu_low = (int)cf[1]; c.swiglu_in_scale = cf[2]; c.swiglu_out_scale = cf[3]; c.rms_eps = cf[4]; c.value_scale = cf[5];
+    c.softmax_thetas.assign(cf + 6, cf + 6 + (K - c.softmax_L - c.softmax_M));
+    return c;
+}
+struct LayerState { LayerConfig cfg; LayerWeights w; };
+// weights given as int32 arrays in the in x out layout of the *-int.bin files; generators from the seeded stream
+void* zkp_layer_create(const u32* cu, const double* cf, const int32_t* norm1, const int32_t* wq, const int32_t* wk, const int32_t* wv, const int32_t* wo,
+                       const int32_t* norm2, const int32_t* wup, const int32_t* wgate, const int32_t* wdown, u32 log_off_factor) {
+    ZKP_TRY
+    LayerConfig c = parse_cfg(cu, cf);
+    const uint E = c.embed_dim, Hd = c.hidden_dim;
+    auto mk = [&](const int32_t* p, uint in_dim, uint out_dim, uint pp) {
+        FrTensor weight(in_dim * out_dim, (const int*)p);
+        Commitment gen = Commitment::random(1u << ceilLog2(pp));
+        G1TensorJacobian com = gen.commit_int(weight.pad({in_dim, out_dim}));
+        return Weight{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim};
+    };
+    // same order of generator draws as the oracle: norm1, q, k, v, o, norm2, up, gate, down
+    Weight n1 = mk(norm1, 1, E, E), q = mk(wq, E, E, E << log_off_factor), k = mk(wk, E, E, E << log_off_factor), v = mk(wv, E, E, E << log_off_factor),
+           o = mk(wo, E, E, E << log_off_factor), n2 = mk(norm2, 1, E, E), up = mk(wup, E, Hd, Hd << log_off_factor), gate = mk(wgate, E, Hd, Hd << log_off_factor),
+           down = mk(wdown, Hd, E, E << log_off_factor);
+    return new LayerState{c, LayerWeights{std::move(n1), std::move(q), std::move(k), std::move(v), std::move(o), std::move(n2), std::move(up), std::move(gate),
+                                          std::move(down), make_swiglu_table(c.swiglu_low, c.swiglu_len, c.swiglu_in_scale, c.swiglu_out_scale)}};
+    ZKP_END_PTR
+}
+void* zkp_layer_create_random(const u32* cu, const double* cf, u32 seed, u32 log_off_factor) {
+    ZKP_TRY
+    LayerConfig c = parse_cfg(cu, cf);
+    return new LayerState{c, make_random_layer_weights(c, seed, log_off_factor)};
+    ZKP_END_PTR
+}
+void zkp_layer_free(void* h) { delete reinterpret_cast<LayerState*>(h); }
+void zkp_layer_set_open_weights(void* h, int on) { reinterpret_cast<LayerState*>(h)->cfg.open_weights = on != 0; }
+// runs the whole layer (compute + every proof); times_ms: rmsnorm1, qkv, attention, oproj, rmsnorm2, ffn, total
+void* zkp_layer_run(void* h, void* X, double* times_ms) {
+    ZKP_TRY
+    LayerState& s = *reinterpret_cast<LayerState*>(h);
+    LayerTimes t;
+    FrTensor out = llama_layer(s.cfg, s.w, FT(X), &t);
+    if (times_ms) { times_ms[0] = t.rmsnorm1; times_ms[1] = t.qkv; times_ms[2] = t.attention; times_ms[3] = t.oproj; times_ms[4] = t.rmsnorm2; times_ms[5] = t.ffn; times_ms[6] = t.total; }
+    return new FrTensor(std::move(out));
+    ZKP_END_PTR
 }
 
 }  // extern "C"

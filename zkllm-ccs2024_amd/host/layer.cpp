@@ -1,0 +1,241 @@
+#include "layer.hpp"
+
+#include <chrono>
+#include <cmath>
+#include <random>
+
+#include "../../include/zkllm_hip.h"
+
+#define ZKC(call) zk_check((call), #call)
+
+static double now_ms() {
+    ZKC(zk_sync(nullptr));
+    return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+FrTensor compute_rms_inv(const FrTensor& X, uint seq_len, uint embed_dim, double eps, double value_scale) {
+    if (X.size != seq_len * embed_dim) throw std::runtime_error("compute_rms_inv: X size does not match");
+    std::vector<long> xi((size_t)X.size);
+    {
+        DevBuf tmp(sizeof(long) * (size_t)X.size);
+        ZKC(zk_fr_to_i64(tmp.p, X.gpu_data, X.size, nullptr));
+        ZKC(zk_memcpy_d2h(xi.data(), tmp.p, sizeof(long) * (size_t)X.size, nullptr));
+    }
+    std::vector<long> out(seq_len);
+    for (uint r = 0; r < seq_len; ++r) {
+        double acc = 0.0;
+        for (uint j = 0; j < embed_dim; ++j) {
+            const double x = (double)xi[(size_t)r * embed_dim + j] / value_scale;
+            acc += x * x;
+        }
+        const double v = 1.0 / std::sqrt(acc / (double)embed_dim + eps);
+        out[r] = (long)std::nearbyint(v * value_scale);
+    }
+    return FrTensor(seq_len, out.data());
+}
+
+FrTensor make_swiglu_table(int low, uint len, double in_scale, double out_scale) {
+    std::vector<int> t(len);
+    for (uint i = 0; i < len; ++i) {
+        const double x = ((double)low + (double)i) / in_scale;
+        const double y = x / (1.0 + std::exp(-x));
+        t[i] = (int)std::nearbyint(y * out_scale);
+    }
+    return FrTensor(len, t.data());
+}
+
+// rmsnorm.cu:26-49
+FrTensor rmsnorm_block(const LayerConfig& c, const Weight& w, const FrTensor& X, const FrTensor& rms_inv) {
+    Rescaling rs1(c.sf_linear), rs2(c.sf_linear);
+    zkFC g(1, c.embed_dim, w.weight);
+    auto g_inv_rms = g(rms_inv);
+    auto g_inv_rms_ = rs1(g_inv_rms);
+    auto Y = g_inv_rms_ * X;
+    auto Y_ = rs2(Y);
+
+    rs2.prove(Y, Y_);
+    auto hu = random_vec(ceilLog2(Y.size));
+    auto hv = random_vec(ceilLog2(Y.size));
+    hadamard_product_sumcheck(g_inv_rms_, X, hu, hv);
+    rs1.prove(g_inv_rms, g_inv_rms_);
+    auto claims = g.prove(rms_inv, g_inv_rms);
+    if (c.open_weights) verifyWeightClaim(w, claims[0]);
+    return Y_;
+}
+
+// self-attn.cu:19-76 (linear mode)
+void attn_linear_block(const LayerConfig& c, const Weight& q, const Weight& k, const Weight& v, const FrTensor& input, FrTensor& Q_, FrTensor& K_, FrTensor& V_) {
+    zkFC q_layer(c.embed_dim, c.embed_dim, q.weight), k_layer(c.embed_dim, c.embed_dim, k.weight), v_layer(c.embed_dim, c.embed_dim, v.weight);
+    Rescaling q_rescale(c.sf_linear), k_rescale(c.sf_linear), v_rescale(c.sf_linear);
+    auto Q = q_layer(input);
+    Q_ = q_rescale(Q);
+    auto K = k_layer(input);
+    K_ = k_rescale(K);
+    auto V = v_layer(input);
+    V_ = v_rescale(V);
+    q_rescale.prove(Q, Q_);
+    k_rescale.prove(K, K_);
+    v_rescale.prove(V, V_);
+    auto ck = k_layer.prove(input, K);
+    if (c.open_weights) verifyWeightClaim(k, ck[0]);
+    auto cq = q_layer.prove(input, Q);
+    if (c.open_weights) verifyWeightClaim(q, cq[0]);
+    auto cv = v_layer.prove(input, V);
+    if (c.open_weights) verifyWeightClaim(v, cv[0]);
+}
+
+// columns [h*d, (h+1)*d) of a seq x embed tensor as a contiguous seq x d tensor
+static FrTensor head_slice(const FrTensor& t, uint seq, uint embed, uint h, uint d) {
+    // transpose -> rows [h*d, (h+1)*d) are contiguous -> transpose back
+    FrTensor tt = t.transpose(seq, embed);                       // embed x seq
+    FrTensor rows = tt.trunc(h * d * seq, (h + 1) * d * seq);    // d x seq
+    return rows.transpose(d, seq);                                // seq x d
+}
+
+// Per-head attention following self-attn.cu:78-121 (attn mode) with d = head width.
+FrTensor attn_heads_block(const LayerConfig& c, const FrTensor& Q_, const FrTensor& K_, const FrTensor& V_) {
+    const uint seq = c.seq_len, E = c.embed_dim, H = c.num_heads, d = E / H;
+    if (E % H) throw std::runtime_error("embed_dim must be a multiple of num_heads");
+    FrTensor QT = Q_.transpose(seq, E), KT = K_.transpose(seq, E), VT = V_.transpose(seq, E);   // embed x seq each
+    FrTensor outT(E * seq);                                                                   // embed x seq, head outputs stacked by rows
+    zkSoftmax softmax(c.softmax_bs, c.softmax_L, c.softmax_M, c.softmax_sf_in, c.softmax_thetas, seq, seq, d, 1);
+    for (uint h = 0; h < H; ++h) {
+        FrTensor Qh = QT.trunc(h * d * seq, (h + 1) * d * seq).transpose(d, seq);   // seq x d
+        FrTensor KhT = KT.trunc(h * d * seq, (h + 1) * d * seq);                      // d x seq  (= K_h^T)
+        FrTensor Kh = KhT.transpose(d, seq);                                          // seq x d
+        FrTensor Vh = VT.trunc(h * d * seq, (h + 1) * d * seq).transpose(d, seq);   // seq x d
+
+        auto X = FrTensor::matmul(Qh, KhT, seq, d, seq);
+        FrTensor shift(seq), X_shifted(seq * seq);
+        vector<FrTensor> X_segments, Y_segments, m_segments;
+        FrTensor Y = softmax.compute(X, shift, X_shifted, X_segments, Y_segments, m_segments);
+        auto out = FrTensor::matmul(Y, Vh, seq, seq, d);                              // seq x d
+        {
+            FrTensor oT = out.transpose(seq, d);                                      // d x seq
+            ZKC(zk_memcpy_d2d(outT.gpu_data + (size_t)h * d * seq, oT.gpu_data, sizeof(Fr_t) * (size_t)d * seq, nullptr));
+        }
+        // proofs for this head: out = Y V, softmax, X = Q K^T
+        auto temp_rand = random_vec(3);
+        vector<Polynomial> proof;
+        auto u1 = random_vec(ceilLog2(seq));
+        auto u2 = random_vec(ceilLog2(d));
+        auto ud = random_vec(ceilLog2(seq));
+        auto claim = out.multi_dim_me({u1, u2}, {seq, d});
+        zk_record(claim);
+        zkip(claim, Y.partial_me(u1, seq, seq), Vh.partial_me(u2, d, 1), ud, proof);
+        auto u_Y = random_vec(ceilLog2(Y.size));
+        auto v_Y = random_vec(ceilLog2(Y.size));
+        softmax.prove(Y, X, shift, X_shifted, X_segments, Y_segments, m_segments, u_Y, v_Y, temp_rand[0], temp_rand[1], temp_rand[2], proof);
+        auto u1_ = random_vec(ceilLog2(seq));
+        auto u2_ = random_vec(ceilLog2(seq));
+        auto ud_ = random_vec(ceilLog2(d));
+        auto claim_ = X.multi_dim_me({u1_, u2_}, {seq, seq});
+        zk_record(claim_);
+        zkip(claim_, Qh.partial_me(u1_, seq, d), Kh.partial_me(u2_, seq, d), ud_, proof);
+    }
+    FrTensor out_all = outT.transpose(E, seq);   // seq x embed
+    Rescaling rs1(c.sf_attn), rs2(c.sf_attn);
+    auto out_ = rs2(out_all);
+    auto out__ = rs1(out_);
+    rs1.prove(out_, out__);
+    rs2.prove(out_all, out_);
+    return out__;
+}
+
+FrTensor oproj_block(const LayerConfig& c, const Weight& o, const FrTensor& attn_out) {
+    zkFC o_layer(c.embed_dim, c.embed_dim, o.weight);
+    Rescaling o_rescale(c.sf_linear);
+    auto O = o_layer(attn_out);
+    auto O_ = o_rescale(O);
+    o_rescale.prove(O, O_);
+    auto co = o_layer.prove(attn_out, O);
+    if (c.open_weights) verifyWeightClaim(o, co[0]);
+    return O_;
+}
+
+// ffn.cu:44-93
+FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, const Weight& down, const FrTensor& swiglu_values, const FrTensor& input) {
+    zkFC up_layer(c.embed_dim, c.hidden_dim, up.weight), gate_layer(c.embed_dim, c.hidden_dim, gate.weight), down_layer(c.hidden_dim, c.embed_dim, down.weight);
+    Rescaling up_rescale(c.sf_linear), gate_rescale(c.sf_gate), hidden_rescale(c.sf_linear), down_rescale(c.sf_linear);
+    tLookupRangeMapping swiglu(c.swiglu_low, c.swiglu_len, swiglu_values);
+
+    auto up_out = up_layer(input);
+    auto up_out_ = up_rescale(up_out);
+    auto gate_out = gate_layer(input);
+    auto gate_out_ = gate_rescale(gate_out);
+    auto p = swiglu(gate_out_);
+    auto &swiglu_out = p.first, &swiglu_m = p.second;
+
+    auto temp_rand = random_vec(3);
+    auto swiglu_u = random_vec(ceilLog2(c.seq_len * c.hidden_dim));
+    auto swiglu_v = random_vec(ceilLog2(c.seq_len * c.hidden_dim));
+    vector<Polynomial> swiglu_proof;
+
+    auto down_in = swiglu_out * up_out_;
+    auto down_in_ = hidden_rescale(down_in);
+    auto down_out = down_layer(down_in_);
+    auto down_out_ = down_rescale(down_out);
+
+    down_rescale.prove(down_out, down_out_);
+    auto cd = down_layer.prove(down_in_, down_out);
+    if (c.open_weights) verifyWeightClaim(down, cd[0]);
+    hidden_rescale.prove(down_in, down_in_);
+    swiglu.prove(gate_out_, swiglu_out, swiglu_m, temp_rand[0], temp_rand[1], temp_rand[2], swiglu_u, swiglu_v, swiglu_proof);
+    gate_rescale.prove(gate_out, gate_out_);
+    auto cg = gate_layer.prove(input, gate_out);
+    if (c.open_weights) verifyWeightClaim(gate, cg[0]);
+    up_rescale.prove(up_out, up_out_);
+    auto cu = up_layer.prove(input, up_out);
+    if (c.open_weights) verifyWeightClaim(up, cu[0]);
+    // the reference saves the unrescaled down_out (ffn.cu:81); the rescaled tensor is what the next block consumes
+    return down_out_;
+}
+
+FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor& X, LayerTimes* times) {
+    LayerTimes t;
+    const double t0 = now_ms();
+    FrTensor rms1 = compute_rms_inv(X, c.seq_len, c.embed_dim, c.rms_eps, c.value_scale);
+    FrTensor n1 = rmsnorm_block(c, w.input_norm, X, rms1);
+    const double t1 = now_ms();
+    FrTensor Q_(X.size), K_(X.size), V_(X.size);
+    attn_linear_block(c, w.q, w.k, w.v, n1, Q_, K_, V_);
+    const double t2 = now_ms();
+    FrTensor attn = attn_heads_block(c, Q_, K_, V_);
+    const double t3 = now_ms();
+    FrTensor o = oproj_block(c, w.o, attn);
+    FrTensor x2 = X + o;                                   // skip-connection.cu:15-18
+    const double t4 = now_ms();
+    FrTensor rms2 = compute_rms_inv(x2, c.seq_len, c.embed_dim, c.rms_eps, c.value_scale);
+    FrTensor n2 = rmsnorm_block(c, w.post_norm, x2, rms2);
+    const double t5 = now_ms();
+    FrTensor f = ffn_block(c, w.up, w.gate, w.down, w.swiglu_table, n2);
+    FrTensor out = x2 + f;
+    const double t6 = now_ms();
+    t.rmsnorm1 = t1 - t0; t.qkv = t2 - t1; t.attention = t3 - t2; t.oproj = t4 - t3; t.rmsnorm2 = t5 - t4; t.ffn = t6 - t5; t.total = t6 - t0;
+    if (times) *times = t;
+    return out;
+}
+
+static Weight random_weight(std::mt19937_64& rng, uint in_dim, uint out_dim, uint pp_size, bool norm) {
+    std::normal_distribution<double> nd(0.0, 0.02);
+    std::vector<int> wi((size_t)in_dim * out_dim);
+    for (auto& x : wi) x = norm ? 65536 : (int)std::nearbyint(nd(rng) * 65536.0);   // scale 2^16 (llama-commit.py:34)
+    FrTensor weight((uint)wi.size(), wi.data());
+    Commitment gen = Commitment::random(1u << ceilLog2(pp_size));
+    FrTensor padded = weight.pad({in_dim, out_dim});
+    G1TensorJacobian com = gen.commit_int(padded);
+    return Weight{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim};
+}
+
+LayerWeights make_random_layer_weights(const LayerConfig& c, uint32_t seed, uint lof) {
+    std::mt19937_64 rng(seed);
+    const uint E = c.embed_dim, Hd = c.hidden_dim;
+    // llama-ppgen.py:21-31: 2-D parameters use (HF shape[0] = out_features) << log_off_factor, 1-D their length
+    return LayerWeights{
+        random_weight(rng, 1, E, E, true),
+        random_weight(rng, E, E, E << lof, false), random_weight(rng, E, E, E << lof, false), random_weight(rng, E, E, E << lof, false),
+        random_weight(rng, E, E, E << lof, false),
+        random_weight(rng, 1, E, E, true),
+        random_weight(rng, E, Hd, Hd << lof, false), random_weight(rng, E, Hd, Hd << lof, false), random_weight(rng, Hd, E, E << lof, false),
+        make_swiglu_table(c.swiglu_low, c.swiglu_len, c.swiglu_in_scale, c.swiglu_out_scale)};
+}

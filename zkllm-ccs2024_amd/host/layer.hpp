@@ -1,0 +1,67 @@
+// One LLaMa-2 decoder layer, computed and proved with the class API: the flows of the reference's
+// per-block executables (rmsnorm.cu, self-attn.cu, ffn.cu, skip-connection.cu) as functions, so the
+// executables and an in-memory whole-layer run share one implementation.
+//
+// Differences from the reference executables, all stated here because they define what "the layer
+// proof" contains:
+//  * attention is proved per head (the reference's `attn` mode treats the whole embedding as one head and
+//    never writes its output, so its pipeline cannot chain): for each head, X = Q_h K_h^T, zkSoftmax,
+//    out_h = Y V_h, the two inner-product sumchecks and the softmax proof; the heads' outputs are
+//    concatenated and rescaled twice as one tensor (a per-head 2^20 table would exceed the head's size);
+//  * an output projection (zkFC + rescaling + weight opening) follows, which the reference lacks;
+//  * challenges that the reference draws inside function-argument lists (unspecified order in C++) are
+//    drawn into named variables, first argument first;
+//  * RoPE, the causal mask and the RMS statistic are the reference's unproven float steps; RoPE and the
+//    mask are left out, the RMS statistic is computed on the host in double precision.
+#pragma once
+#include "commitment.hpp"
+#include "fr-tensor.hpp"
+#include "rescaling.hpp"
+#include "tlookup.hpp"
+#include "zkfc.hpp"
+#include "zksoftmax.hpp"
+
+struct LayerConfig {
+    uint seq_len = 2048, embed_dim = 4096, num_heads = 32, hidden_dim = 11008;
+    uint sf_linear = 1u << 16;    // rescaling after every projection and after the two Hadamard products
+    uint sf_gate = 1u << 20;      // gate projection (ffn.cu:47)
+    uint sf_attn = 1u << 20;      // applied twice to the attention output (self-attn.cu:88)
+    vector<uint> softmax_bs = {1u << 8, 1u << 20, 1u << 20};
+    uint softmax_L = 1, softmax_M = 0;
+    unsigned long softmax_sf_in = 1UL << 32;
+    vector<double> softmax_thetas = {double(1 << 18), double(1 << 22)};
+    int swiglu_low = -(1 << 21);
+    uint swiglu_len = 1u << 22;
+    double swiglu_in_scale = 4096.0, swiglu_out_scale = 16.0;   // llama-ffn.py:14-19 (x step 2^-12, outputs saved times 16)
+    double rms_eps = 1e-5;        // LLaMa-2's variance_epsilon
+    double value_scale = 65536.0; // fixed-point scale of activations (llama-rmsnorm.py:36-38 uses 1 << 16)
+    bool open_weights = true;     // run verifyWeightClaim for every weight claim
+};
+
+struct LayerWeights {
+    Weight input_norm, q, k, v, o, post_norm, up, gate, down;
+    FrTensor swiglu_table;        // swiglu_len mapped values
+};
+
+struct LayerTimes {               // milliseconds, wall clock with the device idle at both ends
+    double rmsnorm1 = 0, qkv = 0, attention = 0, oproj = 0, rmsnorm2 = 0, ffn = 0, total = 0;
+};
+
+// rms_inv = round(scale / sqrt(mean((x/scale)^2) + eps)) per row, scale = 2^16 in the reference (llama-rmsnorm.py:35-39), host double
+FrTensor compute_rms_inv(const FrTensor& X, uint seq_len, uint embed_dim, double eps, double value_scale = 65536.0);
+// SwiGLU table of llama-ffn.py:14-19 generalised to any range: entry i = round_half_even(x*sigmoid(x)*out_scale),
+// x = (low + i) / in_scale
+FrTensor make_swiglu_table(int low, uint len, double in_scale, double out_scale);
+
+FrTensor rmsnorm_block(const LayerConfig& c, const Weight& w, const FrTensor& X, const FrTensor& rms_inv);
+void attn_linear_block(const LayerConfig& c, const Weight& q, const Weight& k, const Weight& v, const FrTensor& input, FrTensor& Q_, FrTensor& K_, FrTensor& V_);
+FrTensor attn_heads_block(const LayerConfig& c, const FrTensor& Q_, const FrTensor& K_, const FrTensor& V_);
+FrTensor oproj_block(const LayerConfig& c, const Weight& o, const FrTensor& attn_out);
+FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, const Weight& down, const FrTensor& swiglu_table, const FrTensor& input);
+
+// whole layer: x -> x + attn(norm(x)) -> (+ ffn(norm(.)))
+FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor& X, LayerTimes* times);
+
+// random-init weights of the configured shape (round(N(0, 0.02) * 2^16), norm weights round(2^16)), generators from the
+// seeded stream sized as llama-ppgen.py does (out_features << log_off_factor, rounded up to a power of two) and commitments
+LayerWeights make_random_layer_weights(const LayerConfig& c, uint32_t seed, uint log_off_factor);
