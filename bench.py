@@ -1,0 +1,202 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X zkLLM prover core.
+
+One step = one LLaMa-2-7B-shape decoder layer at sequence length 2048, computed and proved end to end on one
+GPU with weights, generators, commitments and the input already resident in HBM: RMSNorm x2, Q/K/V/O
+projections, 32 attention heads (QK^T, zkSoftmax, YV), SwiGLU FFN, every rescaling / lookup / sumcheck and
+the opening of all nine weight commitments.  `value` is seconds per layer.
+
+The same JSON line also carries the two throughput figures of the headline metric (G1 MSM points/s on the
+4096 x 11008 commitment workload, Fr multiplications/s), a roofline entry for the dominant kernel timed
+live with HIP events, and a CPU baseline measured with the oracle on this host's cores.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+# VALU integer peak: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz lane-operations per second (v_mad_u64_u32 issues at
+# full rate on gfx950; bench measures it as well and reports the measured figure next to this one)
+VALU_PEAK_TOPS = 256 * 4 * 16 * 2.4e9 / 1e12
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--seq", type=int, default=2048)
+    ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--skip-extras", action="store_true", help="only the layer timing (used for profiling runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this prover runs on one GPU; every configuration of the benchmark fits a single MI355X, "
+              "so --gpus must be 1 (no multi-GPU path exists in this build)", file=sys.stderr)
+        sys.exit(2)
+
+    from gpuhelp import Hip, Prover, c_int, c_size_t, c_uint, c_void_p
+    import layercfg
+    from zkhelp import mt_random_vec
+
+    pv = Prover()
+    hip = Hip()
+    lib = hip.lib
+
+    def ev():
+        e = c_void_p()
+        hip.check(lib.zk_event_create(ctypes.byref(e)))
+        return e
+
+    def time_kernel(fn, reps, warm=1):
+        """average duration in ms of `fn` (one launch on the default stream), HIP events on that stream"""
+        for _ in range(warm):
+            fn()
+        e0, e1 = ev(), ev()
+        hip.check(lib.zk_event_record(e0, None))
+        for _ in range(reps):
+            fn()
+        hip.check(lib.zk_event_record(e1, None))
+        ms = ctypes.c_float()
+        hip.check(lib.zk_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+        return ms.value / reps
+
+    # ---- workload: the decoder layer ------------------------------------------------------------------------------
+    seq = args.seq
+    cu, cf = layercfg.llama7b(seq=seq, open_weights=True)
+    t0 = time.perf_counter()
+    pv.seed(2024)
+    layer = pv.layer_create_random(cu, cf, 7, 5)
+    pv.sync()
+    setup_s = time.perf_counter() - t0
+    X = np.round(np.random.default_rng(11).normal(0, 1, (seq, 4096)) * 65536).astype(np.int32)
+    hX = pv.from_i32(X)
+    devnull = os.open(os.devnull, os.O_WRONLY)
+    saved_stdout = os.dup(1)
+    os.dup2(devnull, 1)      # the class layer prints the reference's progress lines ("Opening complete", ...)
+    try:
+        parts = np.zeros(7)
+        for _ in range(args.warmup):
+            pv.layer_run(layer, hX)
+        pv.sync()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            _, times = pv.layer_run(layer, hX)
+            parts += times
+        pv.sync()
+        wall = time.perf_counter() - t0
+    finally:
+        os.dup2(saved_stdout, 1)
+    ms_per_step = wall * 1e3 / args.steps
+    parts /= args.steps
+    pv.layer_free(layer)
+    lib.zk_pool_trim()
+
+    out = {
+        "metric": "layer prove time (s), 7B shape seq 2048; G1 MSM points/s; Fr mul/s",
+        "value": ms_per_step / 1e3,
+        "unit": "s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u32",
+        "data": "synthetic",
+        "config": {"workload": f"C5: LLaMa-2-7B-shape decoder layer proof, seq {seq}, hidden 4096, 32 heads x 128, FFN 11008, "
+                               "random-init fixed-point weights (scale 2^16), generators of size out_features<<5, all nine weight openings included",
+                   "setup_s_untimed": round(setup_s, 3),
+                   "parts_ms": {k: round(float(v), 1) for k, v in zip(["rmsnorm1", "qkv", "attention", "oproj", "rmsnorm2", "ffn", "total"], parts)}},
+    }
+    if args.skip_extras:
+        print(json.dumps(out))
+        return
+
+    # ---- G1 MSM points/s: commitment of a 4096 x 11008 weight (stored 11008 rows x 4096 against 4096 generators) -------------
+    pv.seed(5)
+    gens = pv.commitment_random(4096)
+    Wm = np.round(np.random.default_rng(12).normal(0, 0.02, (11008, 4096)) * 65536).astype(np.int32)
+    hW = pv.from_i32(Wm)
+    pv.commit_int(gens, hW)
+    pv.sync()
+    t0 = time.perf_counter()
+    reps = 3
+    for _ in range(reps):
+        com = pv.commit_int(gens, hW)
+    pv.sync()
+    msm_s = (time.perf_counter() - t0) / reps
+    out["g1_msm_points_per_s"] = 11008 * 4096 / msm_s
+    out["g1_msm_ms"] = msm_s * 1e3
+    del com, hW, gens
+
+    # ---- Fr mul/s: n independent Montgomery products on resident operands ------------------------------------------------------
+    n = 1 << 26
+    seed_block = mt_random_vec(np.random.RandomState(1), 1 << 16)
+    src = hip.upload(seed_block)
+    dA, dB, dO = hip.malloc(32 * n), hip.malloc(32 * n), hip.malloc(32 * n)
+    for i in range(n >> 16):
+        lib.zk_memcpy_d2d(c_void_p(dA + i * (32 << 16)), c_void_p(src), c_size_t(32 << 16), None)
+        lib.zk_memcpy_d2d(c_void_p(dB + i * (32 << 16)), c_void_p(src + 32 * 5), c_size_t((32 << 16) - 32 * 5), None)
+    hip.sync()
+    mul_ms = time_kernel(lambda: hip.call("zk_fr_montmul", c_void_p(dO), c_void_p(dA), c_void_p(dB), c_size_t(n), None), reps=10)
+    add_ms = time_kernel(lambda: hip.call("zk_fr_add", c_void_p(dO), c_void_p(dA), c_void_p(dB), c_size_t(n), None), reps=10)
+    out["fr_mul_per_s"] = n / (mul_ms * 1e-3)
+    out["fr_mul_stream_gbs"] = 96 * n / (mul_ms * 1e-3) / 1e9
+    out["fr_add_stream_gbs"] = 96 * n / (add_ms * 1e-3) / 1e9
+
+    # measured VALU multiply-add peak
+    peak = ctypes.c_double()
+    hip.check(lib.zk_bench_mad_peak(c_uint(256 * 32), c_uint(10000), ctypes.byref(peak), None))
+    out["valu_mad32_peak_measured_tops"] = peak.value / 1e12
+
+    # ---- roofline of the kernels that dominate the layer ---------------------------------------------------------------------------
+    # (1) generic Fr matmul at the projection shape: M*N*P field multiplications, 136 MAD32 each (algorithmic)
+    M, N, P = 2048, 4096, 4096
+    mm_ms = time_kernel(lambda: hip.call("zk_fr_matmul_generic", c_void_p(dO), c_void_p(dA), c_void_p(dB), c_uint(M), c_uint(N), c_uint(P), None), reps=1)
+    mm_tops = M * N * P * 136 / (mm_ms * 1e-3) / 1e12
+    # (2) fused multilinear fold (3 levels per pass) over a 2048 x 4096 tensor: 32 B read per element
+    u = mt_random_vec(np.random.RandomState(2), 3)
+    fold_ms = time_kernel(lambda: hip.call("zk_fr_fold_axis", c_void_p(dO), c_void_p(dA), u, c_int(3), c_size_t(1), c_uint(2048), c_size_t(4096), None), reps=10)
+    fold_gbs = 32 * 2048 * 4096 / (fold_ms * 1e-3) / 1e9
+    out["roofline"] = {"kernel": "k_matmul (generic Montgomery Fr matmul, 2048x4096x4096)", "bound": "valu-int", "achieved": mm_tops, "peak": VALU_PEAK_TOPS,
+                       "unit": "T MAD32/s", "frac": mm_tops / VALU_PEAK_TOPS, "traffic": None,
+                       "note": "algorithmic 136 MAD32 per field multiplication; peak = 256 CU x 4 SIMD x 16 lanes x 2.4 GHz (v_mad_u64_u32 at full rate)",
+                       "avg_launch_ms": mm_ms, "gmac_per_s": M * N * P / (mm_ms * 1e-3) / 1e9}
+    out["roofline_hbm"] = {"kernel": "k_fold_axis<3> (fused 3-level multilinear fold, 2048x4096)", "bound": "hbm", "achieved": fold_gbs, "peak": HBM_PEAK_GBS,
+                           "unit": "GB/s", "frac": fold_gbs / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": fold_ms}
+    for p in (dA, dB, dO, src):
+        hip.free(p)
+
+    # ---- CPU baseline: the oracle's restatement of the reference's kernels on this host's cores ---------------------------------------
+    if not args.skip_cpu:
+        from zkhelp import load_oracle
+        orc = load_oracle()
+        cores = orc.dll.orc_num_threads()
+        rows = 2 * max(1, cores // 2)
+        A = mt_random_vec(np.random.RandomState(3), rows * 4096)
+        B = mt_random_vec(np.random.RandomState(4), 4096 * 1024)
+        C = np.zeros((rows * 1024, 8), np.uint32)
+        t0 = time.perf_counter()
+        orc.orc_fr_matmul_rows(A, B, rows, 4096, 1024, rows, C)
+        dt = time.perf_counter() - t0
+        mm_rate = rows * 4096 * 1024 / dt                      # field multiplications per second, all cores
+        layer_mm = 4.49e11                                     # field multiplications in the layer's matrix products (reference algorithm)
+        out["cpu_baseline"] = {"value": layer_mm / mm_rate, "unit": "s", "cores": int(cores), "kind": "port",
+                               "sample": f"oracle Fr matmul (reference algorithm, OpenMP) on {rows} rows x 4096 x 1024 = {rows * 4096 * 1024:.3g} multiplications in {dt:.2f} s; "
+                                         f"scaled to the 4.49e11 multiplications of the layer's matrix products alone (lower bound of the CPU layer time)",
+                               "fr_mul_per_s_all_cores": mm_rate}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,12 @@
+// ./skip-connection <block_input.bin> <block_output.bin> <output.bin>   z = x + y  (skip-connection.cu:9-21)
+#include <string>
+#include "fr-tensor.hpp"
+
+int main(int argc, char* argv[]) {
+    if (argc < 4) { std::cerr << "usage: skip-connection block_input.bin block_output.bin output.bin" << std::endl; return 2; }
+    FrTensor x = FrTensor::from_int_bin(argv[1]);
+    FrTensor y = FrTensor::from_int_bin(argv[2]);
+    FrTensor z = x + y;
+    z.save_int(argv[3]);
+    return 0;
+}
