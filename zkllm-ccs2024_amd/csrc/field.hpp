@@ -96,17 +96,23 @@ template <int N> ZK_HD bool equal(const Big<N>& a, const Big<N>& b) {
     return o == 0;
 }
 
+// 32-bit add/subtract with carry: the compiler's carry builtins map onto the hardware carry chain
+// (v_add_co / v_addc_co); a portable fallback serves other host compilers.
+#if defined(__clang__)
+ZK_HD uint32_t addc32(uint32_t a, uint32_t b, uint32_t& c) { unsigned co; const uint32_t r = __builtin_addc(a, b, c, &co); c = co; return r; }
+ZK_HD uint32_t subb32(uint32_t a, uint32_t b, uint32_t& c) { unsigned co; const uint32_t r = __builtin_subc(a, b, c, &co); c = co; return r; }
+#else
+ZK_HD uint32_t addc32(uint32_t a, uint32_t b, uint32_t& c) { const uint64_t t = (uint64_t)a + b + c; c = (uint32_t)(t >> 32); return (uint32_t)t; }
+ZK_HD uint32_t subb32(uint32_t a, uint32_t b, uint32_t& c) { const uint64_t t = (uint64_t)a - b - c; c = (uint32_t)(t >> 32) & 1u; return (uint32_t)t; }
+#endif
+
 // r = a - P if a >= P else a   (a < 2P, carry_in = bit 32N of a)
 template <int N> ZK_HD Big<N> reduce_once(const Big<N>& a, uint32_t carry_in = 0) {
     typedef typename KOf<N>::K K;
     Big<N> d;
-    uint64_t br = 0;
+    uint32_t br = 0;
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-        uint64_t t = (uint64_t)a.v[i] - K::P(i) - br;
-        d.v[i] = (uint32_t)t;
-        br = (t >> 32) & 1u;
-    }
+    for (int i = 0; i < N; ++i) d.v[i] = subb32(a.v[i], K::P(i), br);
     const bool keep = (br != 0) && (carry_in == 0);   // a < P
     Big<N> r;
 #pragma unroll
@@ -115,33 +121,21 @@ template <int N> ZK_HD Big<N> reduce_once(const Big<N>& a, uint32_t carry_in = 0
 }
 template <int N> ZK_HD Big<N> add(const Big<N>& a, const Big<N>& b) {
     Big<N> s;
-    uint64_t c = 0;
+    uint32_t c = 0;
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-        c += (uint64_t)a.v[i] + b.v[i];
-        s.v[i] = (uint32_t)c;
-        c >>= 32;
-    }
-    return reduce_once(s, (uint32_t)c);
+    for (int i = 0; i < N; ++i) s.v[i] = addc32(a.v[i], b.v[i], c);
+    return reduce_once(s, c);
 }
 template <int N> ZK_HD Big<N> sub(const Big<N>& a, const Big<N>& b) {
     typedef typename KOf<N>::K K;
     Big<N> d;
-    uint64_t br = 0;
+    uint32_t br = 0;
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-        uint64_t t = (uint64_t)a.v[i] - b.v[i] - br;
-        d.v[i] = (uint32_t)t;
-        br = (t >> 32) & 1u;
-    }
+    for (int i = 0; i < N; ++i) d.v[i] = subb32(a.v[i], b.v[i], br);
     const uint32_t mask = br ? 0xFFFFFFFFu : 0u;   // a < b: add P back
-    uint64_t c = 0;
+    uint32_t c = 0;
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-        c += (uint64_t)d.v[i] + (K::P(i) & mask);
-        d.v[i] = (uint32_t)c;
-        c >>= 32;
-    }
+    for (int i = 0; i < N; ++i) d.v[i] = addc32(d.v[i], K::P(i) & mask, c);
     return d;
 }
 template <int N> ZK_HD Big<N> neg(const Big<N>& a) { return sub(big_zero<N>(), a); }
@@ -153,8 +147,199 @@ template <int N> ZK_HD Big<N> dbl(const Big<N>& a) {
     return reduce_once(s, a.v[N - 1] >> 31);
 }
 
+#if defined(__HIP_DEVICE_COMPILE__)
+// 96-bit column accumulator (lo, hi) += sum of x_i * y_i.  Each limb product is one v_mad_u64_u32 whose
+// carry-out (a scalar register pair) feeds one add-with-carry into hi.  gfx950 needs two wait states between
+// a vector instruction that writes a scalar register and one that reads it, so inside a block every
+// add-with-carry sits at least two instructions behind its multiply-add (short blocks pad with s_nop) and
+// the carries rotate through three register pairs.  The "s" variants take the y factors from scalar
+// registers (modulus limbs).
+__device__ __forceinline__ void mac96v1(uint64_t& lo, uint32_t& hi, uint32_t x0, uint32_t y0) {
+    uint64_t c0;
+    asm("v_mad_u64_u32 %0, %2, %3, %4, %0\n\t"
+        "s_nop 1\n\t"
+        "v_addc_co_u32_e64 %1, %2, 0, %1, %2"
+        : "+v"(lo), "+v"(hi), "=&s"(c0)
+        : "v"(x0), "v"(y0));
+}
+__device__ __forceinline__ void mac96v2(uint64_t& lo, uint32_t& hi, uint32_t x0, uint32_t y0, uint32_t x1, uint32_t y1) {
+    uint64_t c0, c1;
+    asm("v_mad_u64_u32 %0, %2, %4, %5, %0\n\t"
+        "v_mad_u64_u32 %0, %3, %6, %7, %0\n\t"
+        "s_nop 0\n\t"
+        "v_addc_co_u32_e64 %1, %2, 0, %1, %2\n\t"
+        "v_addc_co_u32_e64 %1, %3, 0, %1, %3"
+        : "+v"(lo), "+v"(hi), "=&s"(c0), "=&s"(c1)
+        : "v"(x0), "v"(y0), "v"(x1), "v"(y1));
+}
+__device__ __forceinline__ void mac96v3(uint64_t& lo, uint32_t& hi, uint32_t x0, uint32_t y0, uint32_t x1, uint32_t y1, uint32_t x2, uint32_t y2) {
+    uint64_t c0, c1, c2;
+    asm("v_mad_u64_u32 %0, %2, %5, %6, %0\n\t"
+        "v_mad_u64_u32 %0, %3, %7, %8, %0\n\t"
+        "v_mad_u64_u32 %0, %4, %9, %10, %0\n\t"
+        "v_addc_co_u32_e64 %1, %2, 0, %1, %2\n\t"
+        "v_addc_co_u32_e64 %1, %3, 0, %1, %3\n\t"
+        "v_addc_co_u32_e64 %1, %4, 0, %1, %4"
+        : "+v"(lo), "+v"(hi), "=&s"(c0), "=&s"(c1), "=&s"(c2)
+        : "v"(x0), "v"(y0), "v"(x1), "v"(y1), "v"(x2), "v"(y2));
+}
+__device__ __forceinline__ void mac96v4(uint64_t& lo, uint32_t& hi, uint32_t x0, uint32_t y0, uint32_t x1, uint32_t y1, uint32_t x2, uint32_t y2, uint32_t x3, uint32_t y3) {
+    uint64_t c0, c1, c2;
+    asm("v_mad_u64_u32 %0, %2, %5, %6, %0\n\t"
+        "v_mad_u64_u32 %0, %3, %7, %8, %0\n\t"
+        "v_mad_u64_u32 %0, %4, %9, %10, %0\n\t"
+        "v_addc_co_u32_e64 %1, %2, 0, %1, %2\n\t"
+        "v_mad_u64_u32 %0, %2, %11, %12, %0\n\t"
+        "v_addc_co_u32_e64 %1, %3, 0, %1, %3\n\t"
+        "v_addc_co_u32_e64 %1, %4, 0, %1, %4\n\t"
+        "v_addc_co_u32_e64 %1, %2, 0, %1, %2"
+        : "+v"(lo), "+v"(hi), "=&s"(c0), "=&s"(c1), "=&s"(c2)
+        : "v"(x0), "v"(y0), "v"(x1), "v"(y1), "v"(x2), "v"(y2), "v"(x3), "v"(y3));
+}
+__device__ __forceinline__ void mac96s1(uint64_t& lo, uint32_t& hi, uint32_t x0, uint32_t y0) {
+    uint64_t c0;
+    asm("v_mad_u64_u32 %0, %2, %3, %4, %0\n\t"
+        "s_nop 1\n\t"
+        "v_addc_co_u32_e64 %1, %2, 0, %1, %2"
+        : "+v"(lo), "+v"(hi), "=&s"(c0)
+        : "v"(x0), "s"(y0));
+}
+__device__ __forceinline__ void mac96s2(uint64_t& lo, uint32_t& hi, uint32_t x0, uint32_t y0, uint32_t x1, uint32_t y1) {
+    uint64_t c0, c1;
+    asm("v_mad_u64_u32 %0, %2, %4, %5, %0\n\t"
+        "v_mad_u64_u32 %0, %3, %6, %7, %0\n\t"
+        "s_nop 0\n\t"
+        "v_addc_co_u32_e64 %1, %2, 0, %1, %2\n\t"
+        "v_addc_co_u32_e64 %1, %3, 0, %1, %3"
+        : "+v"(lo), "+v"(hi), "=&s"(c0), "=&s"(c1)
+        : "v"(x0), "s"(y0), "v"(x1), "s"(y1));
+}
+__device__ __forceinline__ void mac96s3(uint64_t& lo, uint32_t& hi, uint32_t x0, uint32_t y0, uint32_t x1, uint32_t y1, uint32_t x2, uint32_t y2) {
+    uint64_t c0, c1, c2;
+    asm("v_mad_u64_u32 %0, %2, %5, %6, %0\n\t"
+        "v_mad_u64_u32 %0, %3, %7, %8, %0\n\t"
+        "v_mad_u64_u32 %0, %4, %9, %10, %0\n\t"
+        "v_addc_co_u32_e64 %1, %2, 0, %1, %2\n\t"
+        "v_addc_co_u32_e64 %1, %3, 0, %1, %3\n\t"
+        "v_addc_co_u32_e64 %1, %4, 0, %1, %4"
+        : "+v"(lo), "+v"(hi), "=&s"(c0), "=&s"(c1), "=&s"(c2)
+        : "v"(x0), "s"(y0), "v"(x1), "s"(y1), "v"(x2), "s"(y2));
+}
+__device__ __forceinline__ void mac96s4(uint64_t& lo, uint32_t& hi, uint32_t x0, uint32_t y0, uint32_t x1, uint32_t y1, uint32_t x2, uint32_t y2, uint32_t x3, uint32_t y3) {
+    uint64_t c0, c1, c2;
+    asm("v_mad_u64_u32 %0, %2, %5, %6, %0\n\t"
+        "v_mad_u64_u32 %0, %3, %7, %8, %0\n\t"
+        "v_mad_u64_u32 %0, %4, %9, %10, %0\n\t"
+        "v_addc_co_u32_e64 %1, %2, 0, %1, %2\n\t"
+        "v_mad_u64_u32 %0, %2, %11, %12, %0\n\t"
+        "v_addc_co_u32_e64 %1, %3, 0, %1, %3\n\t"
+        "v_addc_co_u32_e64 %1, %4, 0, %1, %4\n\t"
+        "v_addc_co_u32_e64 %1, %2, 0, %1, %2"
+        : "+v"(lo), "+v"(hi), "=&s"(c0), "=&s"(c1), "=&s"(c2)
+        : "v"(x0), "s"(y0), "v"(x1), "s"(y1), "v"(x2), "s"(y2), "v"(x3), "s"(y3));
+}
+// (lo, hi) += sum_{i < CNT} x[i] * y[i]: blocks of four and three wherever possible (no padding needed)
+template <int CNT, bool SC> __device__ __forceinline__ void mac_chain(uint64_t& lo, uint32_t& hi, const uint32_t* x, const uint32_t* y) {
+    constexpr int TAKE = (CNT == 4 || CNT == 7 || CNT == 8 || CNT >= 10) ? 4 : (CNT >= 3 ? 3 : CNT);
+    if constexpr (TAKE == 4) {
+        if constexpr (SC) mac96s4(lo, hi, x[0], y[0], x[1], y[1], x[2], y[2], x[3], y[3]);
+        else mac96v4(lo, hi, x[0], y[0], x[1], y[1], x[2], y[2], x[3], y[3]);
+    } else if constexpr (TAKE == 3) {
+        if constexpr (SC) mac96s3(lo, hi, x[0], y[0], x[1], y[1], x[2], y[2]);
+        else mac96v3(lo, hi, x[0], y[0], x[1], y[1], x[2], y[2]);
+    } else if constexpr (TAKE == 2) {
+        if constexpr (SC) mac96s2(lo, hi, x[0], y[0], x[1], y[1]);
+        else mac96v2(lo, hi, x[0], y[0], x[1], y[1]);
+    } else if constexpr (TAKE == 1) {
+        if constexpr (SC) mac96s1(lo, hi, x[0], y[0]);
+        else mac96v1(lo, hi, x[0], y[0]);
+    }
+    if constexpr (CNT - TAKE > 0) mac_chain<CNT - TAKE, SC>(lo, hi, x + TAKE, y + TAKE);
+}
+// end of a reduction column: with m = -lo/p mod 2^32 the sum lo + m*p0 has a zero low word, so only its upper
+// part is needed: (lo >> 32) + hi*2^32 + mulhi(m, p0) + (low word of lo != 0).  No carry flag involved.
+template <uint32_t P0> __device__ __forceinline__ void col_shift_reduce(uint64_t& lo, uint32_t& hi, uint32_t m) {
+    const uint32_t l0 = (uint32_t)lo;
+    uint64_t nl = (lo >> 32) | ((uint64_t)hi << 32);
+    if (P0 != 1u) nl += __umulhi(m, P0);
+    nl += l0 ? 1u : 0u;
+    lo = nl;
+    hi = 0;
+}
+#elif defined(__HIPCC__)
+// host pass of a device source: same meaning, never on a hot path
+__host__ __device__ inline void mac96v4(uint64_t& lo, uint32_t& hi, uint32_t x0, uint32_t y0, uint32_t x1, uint32_t y1, uint32_t x2, uint32_t y2, uint32_t x3, uint32_t y3) {
+    const uint32_t x[4] = {x0, x1, x2, x3}, y[4] = {y0, y1, y2, y3};
+    for (int i = 0; i < 4; ++i) {
+        const uint64_t p = (uint64_t)x[i] * y[i], s = lo + p;
+        hi += (s < p) ? 1u : 0u;
+        lo = s;
+    }
+}
+template <uint32_t P0> __host__ __device__ inline void col_shift_reduce(uint64_t& lo, uint32_t& hi, uint32_t m) {
+    const uint32_t l0 = (uint32_t)lo;
+    lo = ((lo >> 32) | ((uint64_t)hi << 32)) + (uint32_t)(((uint64_t)m * P0) >> 32) + (l0 ? 1u : 0u);
+    hi = 0;
+}
+template <int CNT, bool SC> __host__ __device__ inline void mac_chain(uint64_t& lo, uint32_t& hi, const uint32_t* x, const uint32_t* y) {
+    for (int i = 0; i < CNT; ++i) {
+        const uint64_t p = (uint64_t)x[i] * y[i], s = lo + p;
+        hi += (s < p) ? 1u : 0u;
+        lo = s;
+    }
+}
+#endif
+#if defined(__HIP_DEVICE_COMPILE__)
+// Device Montgomery product: product scanning (column by column) with the reduction interleaved, so
+// every limb product is one mac96 and each column ends in one 32-bit shift of the accumulator.
+template <int N, int K> struct MontCol {
+    // column K < N: products a_i b_(K-i), i <= K, reduction terms m_i p_(K-i), i < K, then m_K
+    static __device__ __forceinline__ void low(uint64_t& lo, uint32_t& hi, const uint32_t* a, const uint32_t* b, uint32_t* m) {
+        typedef typename KOf<N>::K C;
+        uint32_t y[K + 1], pr[K + 1];
+#pragma unroll
+        for (int i = 0; i <= K; ++i) { y[i] = b[K - i]; pr[i] = C::P(K - i); }
+        mac_chain<K + 1, false>(lo, hi, a, y);
+        mac_chain<K, true>(lo, hi, m, pr);
+        m[K] = (uint32_t)lo * C::INV;
+        col_shift_reduce<C::P(0)>(lo, hi, m[K]);
+    }
+    // column K >= N: i runs from K-N+1 to N-1
+    static __device__ __forceinline__ void high(uint64_t& lo, uint32_t& hi, const uint32_t* a, const uint32_t* b, const uint32_t* m, uint32_t* t) {
+        typedef typename KOf<N>::K C;
+        constexpr int F = K - N + 1, CNT = N - F;
+        uint32_t y[CNT > 0 ? CNT : 1], pr[CNT > 0 ? CNT : 1];
+#pragma unroll
+        for (int i = 0; i < CNT; ++i) { y[i] = b[K - F - i]; pr[i] = C::P(K - F - i); }
+        mac_chain<CNT, false>(lo, hi, a + F, y);
+        mac_chain<CNT, true>(lo, hi, m + F, pr);
+        t[K - N] = (uint32_t)lo;
+        lo = (lo >> 32) | ((uint64_t)hi << 32);
+        hi = 0;
+    }
+};
+template <int N, int K> __device__ __forceinline__ void mont_cols(uint64_t& lo, uint32_t& hi, const uint32_t* a, const uint32_t* b, uint32_t* m, uint32_t* t) {
+    if constexpr (K < N) MontCol<N, K>::low(lo, hi, a, b, m);
+    else MontCol<N, K>::high(lo, hi, a, b, m, t);
+    if constexpr (K + 1 < 2 * N) mont_cols<N, K + 1>(lo, hi, a, b, m, t);
+}
+template <int N> __device__ __forceinline__ Big<N> mont_mul_columns(const Big<N>& a, const Big<N>& b) {
+    uint32_t m[N], t[N];
+    uint64_t lo = 0;
+    uint32_t hi = 0;
+    mont_cols<N, 0>(lo, hi, a.v, b.v, m, t);
+    Big<N> r;
+#pragma unroll
+    for (int i = 0; i < N; ++i) r.v[i] = t[i];
+    return reduce_once(r, (uint32_t)lo);
+}
+#endif
+
 // Montgomery product a*b*R^-1 mod p, canonical.  Inputs < p.
 template <int N> ZK_HD Big<N> mont_mul(const Big<N>& a, const Big<N>& b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return mont_mul_columns(a, b);
+#else
     typedef typename KOf<N>::K K;
     uint32_t t[N + 1];
 #pragma unroll
@@ -186,6 +371,7 @@ template <int N> ZK_HD Big<N> mont_mul(const Big<N>& a, const Big<N>& b) {
 #pragma unroll
     for (int i = 0; i < N; ++i) r.v[i] = t[i];
     return reduce_once(r, t[N]);
+#endif
 }
 template <int N> ZK_HD Big<N> mont_sqr(const Big<N>& a) { return mont_mul(a, a); }
 template <int N> ZK_HD Big<N> to_mont(const Big<N>& a) { return mont_mul(a, big_r2<N>()); }

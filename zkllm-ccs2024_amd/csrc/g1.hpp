@@ -14,8 +14,28 @@ namespace zk {
 #else
 #define ZK_NOINLINE_HD __attribute__((noinline))
 #endif
+#if defined(__HIP_DEVICE_COMPILE__)
+// On the device the operands travel in vector registers (six 4-dword vectors): aggregates beyond 16 dwords
+// would be passed through private memory, and every product would start with loads from it.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+static __device__ __attribute__((noinline)) Fp fp_mul_regs(u32x4 a0, u32x4 a1, u32x4 a2, u32x4 b0, u32x4 b1, u32x4 b2) {
+    Fp a, b;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        a.v[i] = a0[i]; a.v[4 + i] = a1[i]; a.v[8 + i] = a2[i];
+        b.v[i] = b0[i]; b.v[4 + i] = b1[i]; b.v[8 + i] = b2[i];
+    }
+    return mont_mul(a, b);
+}
+__device__ __forceinline__ Fp fp_mul(const Fp& a, const Fp& b) {
+    return fp_mul_regs(u32x4{a.v[0], a.v[1], a.v[2], a.v[3]}, u32x4{a.v[4], a.v[5], a.v[6], a.v[7]}, u32x4{a.v[8], a.v[9], a.v[10], a.v[11]},
+                       u32x4{b.v[0], b.v[1], b.v[2], b.v[3]}, u32x4{b.v[4], b.v[5], b.v[6], b.v[7]}, u32x4{b.v[8], b.v[9], b.v[10], b.v[11]});
+}
+__device__ __forceinline__ Fp fp_sqr(const Fp& a) { return fp_mul(a, a); }
+#else
 static ZK_NOINLINE_HD Fp fp_mul(const Fp& a, const Fp& b) { return mont_mul(a, b); }
 static ZK_NOINLINE_HD Fp fp_sqr(const Fp& a) { return mont_mul(a, a); }
+#endif
 
 struct G1Affine { Fp x, y; };
 struct G1Jac { Fp x, y, z; };

@@ -5,9 +5,9 @@
 // product.  Two paths, both bit-identical to the reference because results are canonical:
 //
 //  * generic: every MAC is a 255x255-bit product.  Eight products are accumulated limb-row by
-//    limb-row into one running value and share a single Montgomery reduction ("multi-term
-//    CIOS"): 64 multiply-adds per MAC for the products plus 64/8 for the reduction, against
-//    128 for a product reduced on its own.  The R^-1 factor is removed once per output.
+//    column by column into one running value and share a single Montgomery reduction: 64
+//    multiply-adds per MAC for the products plus 64/8 for the reduction, against 128 for a
+//    product reduced on its own.  The R^-1 factor is removed once per output.
 //  * small-integer: when both operands are embeddings of int32-range values and the whole dot
 //    product is bounded by 2^62, the same sum is computed in int64 and embedded at the end.
 //    The bound is established on the device from the operands (max |a|, max |b|, N); nothing is
@@ -22,42 +22,62 @@ using namespace zk;
 static constexpr int KT = 8;       // terms sharing one reduction
 static constexpr int TM = 16, TN = 16;
 
-// sum_q a[q]*b[q]*R^-1 mod r, canonical.  The running value stays below (KT+1)*r < 2^260.
+// sum_q a[q]*b[q]*R^-1 mod r, canonical.  Product scanning: column k gathers the limb products of all KT
+// terms and of the reduction in one 96-bit accumulator (at most 72 products of 64 bits per column), so a
+// limb product costs one multiply-add and one add-with-carry.  The value before the final subtractions is
+// below (KT*r/R + 1)*r < 5r.
 __device__ __forceinline__ Fr dot_mont(const Fr (&a)[KT], const Fr (&b)[KT]) {
-    uint32_t t[10];
+    uint32_t m[8], t[9];
+    uint64_t lo = 0;
+    uint32_t hi = 0;
 #pragma unroll
-    for (int i = 0; i < 10; ++i) t[i] = 0;
+    for (int k = 0; k < 8; ++k) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+        for (int q = 0; q < KT; q += 4) {
 #pragma unroll
-        for (int q = 0; q < KT; ++q) {
-            uint64_t c = 0;
-            const uint32_t bi = b[q].v[i];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                c += (uint64_t)a[q].v[j] * bi + t[j];
-                t[j] = (uint32_t)c;
-                c >>= 32;
-            }
-            c += t[8];
-            t[8] = (uint32_t)c;
-            t[9] += (uint32_t)(c >> 32);
+            for (int i = 0; i <= k; ++i)
+                mac96v4(lo, hi, a[q].v[i], b[q].v[k - i], a[q + 1].v[i], b[q + 1].v[k - i], a[q + 2].v[i], b[q + 2].v[k - i], a[q + 3].v[i], b[q + 3].v[k - i]);
         }
-        const uint32_t m = 0u - t[0];                 // INV = -1 mod 2^32
-        uint64_t c = ((uint64_t)m * FrK::P(0) + t[0]) >> 32;
+        {
+            uint32_t pr[8];
 #pragma unroll
-        for (int j = 1; j < 8; ++j) {
-            c += (uint64_t)m * FrK::P(j) + t[j];
-            t[j - 1] = (uint32_t)c;
-            c >>= 32;
+            for (int i = 0; i < 8; ++i) pr[i] = FrK::P((k - i) & 7);
+            if (k == 1) mac_chain<1, true>(lo, hi, m, pr);
+            if (k == 2) mac_chain<2, true>(lo, hi, m, pr);
+            if (k == 3) mac_chain<3, true>(lo, hi, m, pr);
+            if (k == 4) mac_chain<4, true>(lo, hi, m, pr);
+            if (k == 5) mac_chain<5, true>(lo, hi, m, pr);
+            if (k == 6) mac_chain<6, true>(lo, hi, m, pr);
+            if (k == 7) mac_chain<7, true>(lo, hi, m, pr);
         }
-        c += t[8];
-        t[7] = (uint32_t)c;
-        c >>= 32;
-        c += t[9];
-        t[8] = (uint32_t)c;
-        t[9] = 0;
+        m[k] = 0u - (uint32_t)lo;                     // INV = -1 mod 2^32
+        col_shift_reduce<FrK::P(0)>(lo, hi, m[k]);
     }
+#pragma unroll
+    for (int k = 8; k < 16; ++k) {
+#pragma unroll
+        for (int q = 0; q < KT; q += 4) {
+#pragma unroll
+            for (int i = k - 7; i < 8; ++i)
+                mac96v4(lo, hi, a[q].v[i], b[q].v[k - i], a[q + 1].v[i], b[q + 1].v[k - i], a[q + 2].v[i], b[q + 2].v[k - i], a[q + 3].v[i], b[q + 3].v[k - i]);
+        }
+        {
+            uint32_t pr[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pr[i] = FrK::P((7 - i) & 7);     // m[k-7+i] pairs with P(7-i)
+            if (k == 8) mac_chain<7, true>(lo, hi, m + 1, pr);
+            if (k == 9) mac_chain<6, true>(lo, hi, m + 2, pr);
+            if (k == 10) mac_chain<5, true>(lo, hi, m + 3, pr);
+            if (k == 11) mac_chain<4, true>(lo, hi, m + 4, pr);
+            if (k == 12) mac_chain<3, true>(lo, hi, m + 5, pr);
+            if (k == 13) mac_chain<2, true>(lo, hi, m + 6, pr);
+            if (k == 14) mac_chain<1, true>(lo, hi, m + 7, pr);
+        }
+        t[k - 8] = (uint32_t)lo;
+        lo = (lo >> 32) | ((uint64_t)hi << 32);
+        hi = 0;
+    }
+    t[8] = (uint32_t)lo;
     // t[0..8] < (KT+1) r : subtract 8r, 4r, 2r, r conditionally (constants built at compile time)
 #pragma unroll
     for (int s = 3; s >= 0; --s) {
