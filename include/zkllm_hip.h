@@ -125,6 +125,11 @@ int zk_g1_normalize(void* out, const void* in, size_t n, void* stream);
 int zk_g1_commit_int(void* out, const void* gens, const void* scalars_fr, size_t m, size_t ngen, void* stream);
 /* one round of Commitment::me_open (me_open_step :79-107 + the three G1 sums :125-127) */
 int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host108, const void* scalars, const void* gens, const uint32_t* u, size_t old_size, void* stream);
+/* the whole recursion of Commitment::me_open :109-129: `rounds` halvings of (scalars, gens) of length n with the
+ * challenges u[0..rounds) (8 limbs each, host).  proof_host: 3*rounds+1 points of 36 limbs -- T, T0, T1 per round,
+ * then the folded generator -- normalised to z = 1; final_scalar_host: the folded scalar (8 limbs).  The generators
+ * must lie in the order-r subgroup (Commitment::random, :9-20, only produces such points). */
+int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stream);
 
 /* ---- lookup argument (tlookup.cu) ------------------------------------------------------------------------ */
 /* idx = val - low as a table index (lookuprange_tensor_prep_kernel :414-421 / lookuprange_prep_kernel :393-400);

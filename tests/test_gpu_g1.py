@@ -137,7 +137,9 @@ def test_commit_int_rejects_non_integer_scalars_and_is_linear(pv, orc):
     assert jac_to_affine(pv.commit(hG, pv.from_i32(a)).host()[0]) == ca
 
 
-@pytest.mark.parametrize("n,m", [(4, 2), (8, 1), (16, 4), (5, 3)])
+# 300 x 1: raw small integers, whose negative embeddings share their high bytes (one bucket receives whole chunks);
+# 4500 x 2: more than one chunk of the bucket kernel and an odd tail in several rounds
+@pytest.mark.parametrize("n,m", [(4, 2), (8, 1), (16, 4), (5, 3), (1, 2), (300, 1), (4500, 2)])
 def test_open_value_and_g1_transcript(pv, orc, n, m):
     gens = oracle_gens(orc, 15 + n, n)
     rng = np.random.default_rng(n * m)

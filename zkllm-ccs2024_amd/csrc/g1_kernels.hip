@@ -12,6 +12,7 @@
 // All of it is VALU integer work on 12-limb Fp; results equal the reference's as group elements
 // (a Jacobian triple depends on the order of additions, so bytes are compared after normalising).
 #include <cstring>
+#include <memory>
 #include <vector>
 #include "g1.hpp"
 #include "rt.hpp"
@@ -213,44 +214,216 @@ __global__ void __launch_bounds__(256) k_fr_to_i32_checked(int32_t* __restrict__
     if (a) atomicMax(maxabs, a);
 }
 
-// ---- opening (me_open_step, commitment.cu:79-107) ------------------------------------------------------------------
-// Five scalar multiplications per pair, one lane each: which = 0: [u](g0-g1), 1: [s0]g0, 2: [s1]g1, 3: [s0]g1, 4: [s1]g0.
-// parts[which * new_size + pair].  Odd tail: 0: [u]g0, 1: [s0]g0, others infinity.
-__global__ void __launch_bounds__(GT) k_open_parts(G1Jac* __restrict__ parts, const Fr* __restrict__ scalars, const G1Jac* __restrict__ gens, const Fr u, size_t old_size, size_t new_size) {
-    const size_t t = (size_t)blockIdx.x * GT + threadIdx.x;
-    if (t >= 5 * new_size) return;
-    const uint32_t which = (uint32_t)(t / new_size);
-    const size_t g = t % new_size;
-    const size_t g0 = 2 * g, g1 = 2 * g + 1;
-    G1Jac r = g1_infinity();
-    if (g1 >= old_size) {
-        if (which == 0) r = g1_mul(gens[g0], u);
-        else if (which == 1) r = g1_mul(gens[g0], scalars[g0]);
-    } else {
-        switch (which) {
-            case 0: r = g1_mul(g1_add(gens[g0], g1_neg(gens[g1])), u); break;
-            case 1: r = g1_mul(gens[g0], scalars[g0]); break;
-            case 2: r = g1_mul(gens[g1], scalars[g1]); break;
-            case 3: r = g1_mul(gens[g1], scalars[g0]); break;
-            default: r = g1_mul(gens[g0], scalars[g1]); break;
+// ---- opening (Commitment::me_open, commitment.cu:79-129) -------------------------------------------------------------
+// A round of the opening halves the scalars s and the generators g with the challenge u,
+//   s'_i = s_2i + u (s_2i+1 - s_2i),   g'_i = g_2i+1 + [u](g_2i - g_2i+1),
+// and publishes T = sum [s_j] g_j, T0 = sum [s_2i] g_2i+1, T1 = sum [s_2i+1] g_2i.  The reference spends five
+// 255-bit scalar multiplications per pair on this.  Here
+//  * T0 and T1 (and T of the first round) are bucket multi-scalar multiplications over the affine-normalised
+//    generators: 8-bit signed windows, one workgroup per (sum, window, segment), one bucket per lane;
+//  * T of every later round follows from the previous round's three points, because <s', g'> expands to
+//    u(1-u) T + (1-u)^2 T0 + u^2 T1;
+//  * the one remaining scalar multiplication per pair, by the round's common challenge u, uses the curve
+//    endomorphism (x, y) -> (beta x, y) = [lambda](x, y): u = k1 + k2 lambda with k1, k2 < 2^128 (r = lambda^2 +
+//    lambda + 1, so this is one integer division on the host), then 128 doublings instead of 255.
+// The endomorphism and the expansion of T hold for points of the order-r subgroup, which is where the
+// generators live (Commitment::random draws multiples of the group generator, commitment.cu:9-20).
+// All rounds are queued without a host round trip; the proof points come back in one copy, normalised to z = 1.
+static constexpr int MW = 32;        // 8-bit signed windows over a 255-bit scalar
+static constexpr int MT = 128;       // lanes of a bucket workgroup = buckets (digit magnitudes 1..128)
+static constexpr int MSEG = 4096;    // elements per chunk (12-bit list entries)
+static constexpr int MCAP = 96;      // list slots per bucket and pass
+struct MsmDesc { uint32_t count, s_mul, s_off, b_mul, b_off; };   // element i: scalar S[i*s_mul+s_off], base A[i*b_mul+b_off]
+struct MsmDescs { MsmDesc d[3]; };
+struct GlvK { uint32_t k1[4], k2[4]; };
+
+__device__ __forceinline__ bool aff_is_inf(const G1Affine& p) { return is_zero(p.x) && is_zero(p.y); }   // normalised infinity: all-zero limbs
+__device__ __forceinline__ G1Jac aff_to_jac(const G1Affine& p) {
+    G1Jac r;
+    if (aff_is_inf(p)) return g1_infinity();
+    r.x = p.x; r.y = p.y; r.z = big_one_mont<12>();
+    return r;
+}
+// beta (Montgomery form): the cube root of unity in Fp with (beta x, y) = [lambda](x, y), lambda = 0xac45a4010001a40200000000ffffffff
+__device__ __forceinline__ Fp glv_beta() {
+    Fp b;
+    constexpr uint32_t t[12] = {2255614065u, 3439577572u, 533571026u, 1571496518u, 3548715925u, 1483752111u, 29019038u, 2394295998u, 2211467474u, 66682222u, 1415808833u, 418390117u};
+#pragma unroll
+    for (int i = 0; i < 12; ++i) b.v[i] = t[i];
+    return b;
+}
+// [k1]P + [k2]phi(P); every lane of a wave must carry the same k (the add pattern is uniform)
+static __device__ __attribute__((noinline)) G1Jac g1_mul_glv(const G1Jac& P, const GlvK& k) {
+    if (is_zero(P.z)) return P;
+    G1Jac Q = P;
+    Q.x = fp_mul(P.x, glv_beta());
+    const G1Jac PQ = g1_add(P, Q);
+    int top = -1;
+    for (int i = 3; i >= 0 && top < 0; --i) {
+        const uint32_t x = k.k1[i] | k.k2[i];
+        if (x) top = i * 32 + 31 - __builtin_clz(x);
+    }
+    G1Jac out = g1_infinity();
+    for (int i = top; i >= 0; --i) {
+        out = g1_double(out);
+        const uint32_t b = ((k.k1[i >> 5] >> (i & 31)) & 1u) | (((k.k2[i >> 5] >> (i & 31)) & 1u) << 1);
+        if (b == 1) out = g1_add(out, P);
+        else if (b == 2) out = g1_add(out, Q);
+        else if (b == 3) out = g1_add(out, PQ);
+    }
+    return out;
+}
+
+// signed 8-bit digit of window w: raw byte plus the carry of the lower windows (a lower digit above 128 is
+// replaced by digit - 256 and carries one).  The carry only depends on the first lower byte that is not 128.
+__device__ __forceinline__ int msm_digit(const uint32_t* __restrict__ sp, uint32_t w) {
+    int raw = (int)((sp[w >> 2] >> ((w & 3u) * 8u)) & 0xFFu);
+    for (int j = (int)w - 1; j >= 0; --j) {
+        const uint32_t b = (sp[j >> 2] >> ((j & 3) * 8)) & 0xFFu;
+        if (b != 128u) { raw += (b > 128u) ? 1 : 0; break; }
+    }
+    return raw > 128 ? raw - 256 : raw;
+}
+
+// partial[(sum * MW + w) * nseg + seg] = sum over the segment's elements of digit_w(s) * base.
+// Lane t owns the bucket of magnitude t+1.  Per chunk the elements are first sorted into per-bucket lists in LDS
+// (one atomic per element), then every lane walks its own list with mixed additions, so lanes stay busy in
+// lockstep whatever the digits are; elements that find their bucket's list full wait for the next pass over the chunk.
+__global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, const Fr* __restrict__ S, const G1Affine* __restrict__ A, const MsmDescs descs,
+                                                uint32_t nseg, uint32_t chunks_per_seg) {
+    __shared__ uint32_t cnt[MT];
+    __shared__ uint32_t pool[MCAP * MT / 2];       // u16 lists while accumulating, the 36 x MT point tree afterwards
+    static_assert(MCAP * MT / 2 >= 36 * MT, "pool too small for the point tree");
+    static_assert(MSEG / MT == 32, "one done-bit per element of a lane's chunk share");
+    uint16_t* list = reinterpret_cast<uint16_t*>(pool);
+    const MsmDesc d = descs.d[blockIdx.z];
+    const uint32_t w = blockIdx.y, seg = blockIdx.x, t = threadIdx.x;
+    G1Jac acc = g1_infinity();
+    for (uint32_t ch = 0; ch < chunks_per_seg; ++ch) {
+        const uint32_t e0 = (seg * chunks_per_seg + ch) * MSEG;
+        if (e0 >= d.count) break;
+        const uint32_t e1 = (e0 + MSEG < d.count) ? e0 + MSEG : d.count;
+        uint32_t done = 0;                      // bit i: this lane's i-th element of the chunk is in a list already (MSEG / MT = 32 per lane)
+        for (;;) {
+            cnt[t] = 0;
+            __syncthreads();
+            uint32_t left = 0;
+            for (uint32_t e = e0 + t, i = 0; e < e1; e += MT, ++i) {
+                if ((done >> i) & 1u) continue;
+                const int dg = msm_digit(reinterpret_cast<const uint32_t*>(S + ((size_t)e * d.s_mul + d.s_off)), w);
+                if (dg != 0) {
+                    const uint32_t mag = (uint32_t)(dg < 0 ? -dg : dg);
+                    const uint32_t pos = atomicAdd(&cnt[mag - 1], 1u);
+                    if (pos >= (uint32_t)MCAP) { left = 1; continue; }
+                    list[pos * MT + (mag - 1)] = (uint16_t)((e - e0) | (dg < 0 ? 0x8000u : 0u));
+                }
+                done |= 1u << i;
+            }
+            __syncthreads();
+            const uint32_t c = cnt[t];
+            const uint32_t mine = c < (uint32_t)MCAP ? c : (uint32_t)MCAP;
+            for (uint32_t k = 0; k < mine; ++k) {
+                const uint32_t en = list[k * MT + t];
+                G1Affine pt = A[(size_t)(e0 + (en & 0x7FFFu)) * d.b_mul + d.b_off];
+                if (aff_is_inf(pt)) continue;
+                if (en & 0x8000u) pt.y = neg(pt.y);
+                acc = g1_add_mixed(acc, pt);
+            }
+            if (!__syncthreads_or((int)left)) break;
         }
     }
-    parts[t] = r;
+    // bucket value t+1 times the bucket, then the sum over the lanes
+    G1Jac r = g1_infinity();
+    for (int bit = 7; bit >= 0; --bit) {
+        r = g1_double(r);
+        if (((t + 1) >> bit) & 1u) r = g1_add(r, acc);
+    }
+    __syncthreads();
+    {
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(&r);
+#pragma unroll
+        for (int l = 0; l < 36; ++l) pool[l * MT + t] = src[l];
+    }
+    __syncthreads();
+    for (uint32_t sd = MT / 2; sd > 0; sd >>= 1) {
+        if (t < sd) {
+            G1Jac x, y;
+            uint32_t* px = reinterpret_cast<uint32_t*>(&x);
+            uint32_t* py = reinterpret_cast<uint32_t*>(&y);
+#pragma unroll
+            for (int l = 0; l < 36; ++l) { px[l] = pool[l * MT + t]; py[l] = pool[l * MT + t + sd]; }
+            x = g1_add(x, y);
+#pragma unroll
+            for (int l = 0; l < 36; ++l) pool[l * MT + t] = px[l];
+        }
+        __syncthreads();
+    }
+    if (t == 0) {
+        G1Jac tot;
+        uint32_t* pr = reinterpret_cast<uint32_t*>(&tot);
+#pragma unroll
+        for (int l = 0; l < 36; ++l) pr[l] = pool[l * MT];
+        partial[((size_t)blockIdx.z * MW + w) * nseg + seg] = tot;
+    }
 }
-// new_gens = g1 + part0 (or part0 on the odd tail); T = part1 + part2 (in place in part1); new scalars
-__global__ void __launch_bounds__(GT) k_open_combine(Fr* __restrict__ new_scalars, G1Jac* __restrict__ new_gens, G1Jac* __restrict__ parts,
-                                                     const Fr* __restrict__ scalars, const G1Jac* __restrict__ gens, const Fr u_mont, size_t old_size, size_t new_size) {
+
+// The fold of one round plus the single-point work that rides along in spare workgroups:
+//  blocks [0, nb_main): pair g -> new scalar, new generator;
+//  next n_msm blocks: lane 0 assembles one sum from its window sums, sum_w 2^(8w) W[w] -> pts_round[3 - n_msm + i];
+//  next 3 blocks (rounds after the first): rec_round[j] = [c_j] (T, T0, T1 of the previous round)[j], whose sum is this round's T.
+struct OpenExtras {
+    const G1Jac* W;          // n_msm x MW window sums
+    G1Jac* pts_round;        // this round's T, T0, T1
+    const G1Jac* pts_prev;   // previous round's T, T0, T1 (T valid only for the first round)
+    const G1Jac* rec_prev;   // previous round's three parts of T (rounds >= 2)
+    G1Jac* rec_round;        // this round's three parts of T
+    uint32_t n_msm, round;
+    GlvK kc[3];
+};
+__global__ void __launch_bounds__(GT) k_open_fold(Fr* __restrict__ new_scalars, G1Jac* __restrict__ new_gens, const Fr* __restrict__ scalars, const G1Affine* __restrict__ A,
+                                                  const Fr u_mont, const GlvK ku, size_t old_size, size_t new_size, uint32_t nb_main, const OpenExtras ex) {
+    if (blockIdx.x >= nb_main) {
+        if (threadIdx.x != 0) return;
+        const uint32_t x = blockIdx.x - nb_main;
+        if (x < ex.n_msm) {
+            const G1Jac* W = ex.W + (size_t)x * MW;
+            G1Jac r = W[MW - 1];
+            for (int w = MW - 2; w >= 0; --w) {
+                for (int k = 0; k < 8; ++k) r = g1_double(r);
+                r = g1_add(r, W[w]);
+            }
+            ex.pts_round[3 - ex.n_msm + x] = r;
+        } else {
+            const uint32_t j = x - ex.n_msm;
+            G1Jac base;
+            if (j == 0) base = (ex.round == 1) ? ex.pts_prev[0] : g1_add(g1_add(ex.rec_prev[0], ex.rec_prev[1]), ex.rec_prev[2]);
+            else base = ex.pts_prev[j];
+            ex.rec_round[j] = g1_mul_glv(base, ex.kc[j]);
+        }
+        return;
+    }
     const size_t g = (size_t)blockIdx.x * GT + threadIdx.x;
     if (g >= new_size) return;
     const size_t g0 = 2 * g, g1 = 2 * g + 1;
+    const G1Affine a0 = A[g0];
     if (g1 >= old_size) {
         new_scalars[g] = sub(scalars[g0], mont_mul(u_mont, scalars[g0]));
-        new_gens[g] = parts[g];
+        new_gens[g] = g1_mul_glv(aff_to_jac(a0), ku);
         return;
     }
     new_scalars[g] = add(scalars[g0], mont_mul(u_mont, sub(scalars[g1], scalars[g0])));
-    new_gens[g] = g1_add(gens[g1], parts[g]);
-    parts[new_size + g] = g1_add(parts[new_size + g], parts[2 * new_size + g]);
+    const G1Affine a1 = A[g1];
+    G1Jac diff = aff_to_jac(a0);
+    if (!aff_is_inf(a1)) diff = g1_add_mixed(diff, g1_neg(a1));
+    G1Jac r = g1_mul_glv(diff, ku);
+    if (!aff_is_inf(a1)) r = g1_add_mixed(r, a1);
+    new_gens[g] = r;
+}
+// after the last round: T of rounds >= 1 from its three parts, and the folded generator as the last proof point
+__global__ void __launch_bounds__(GT) k_open_finish(G1Jac* __restrict__ pts, const G1Jac* __restrict__ rec, const G1Jac* __restrict__ last_gen, uint32_t rounds) {
+    const uint32_t r = blockIdx.x * GT + threadIdx.x;
+    if (r >= 1 && r < rounds) pts[3 * r] = g1_add(g1_add(rec[3 * r], rec[3 * r + 1]), rec[3 * r + 2]);
+    if (r == rounds) pts[3 * rounds] = last_gen[0];
 }
 
 // ---- host side ----------------------------------------------------------------------------------------------------------
@@ -284,6 +457,69 @@ static int g1_sum_device(G1Jac* out, const G1Jac* in, size_t n, hipStream_t st) 
     if (part.rc) return part.rc;
     hipLaunchKernelGGL(k_g1_rowsum, dim3(1, nseg), dim3(GT), 0, st, part.as<G1Jac>(), in, n, nseg);
     hipLaunchKernelGGL(k_g1_rowsum, dim3(1, 1), dim3(GT), 0, st, out, part.as<G1Jac>(), (size_t)nseg, 1u);
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
+
+// u = k1 + k2 * lambda with 0 <= k1 < lambda and k2 <= lambda + 1 (r = lambda^2 + lambda + 1): one long division
+static GlvK glv_split(const Fr& u) {
+    const unsigned __int128 lam = ((unsigned __int128)0xac45a4010001a402ull << 64) | 0x00000000ffffffffull;
+    unsigned __int128 rem = 0, q = 0;
+    for (int i = 255; i >= 0; --i) {
+        const bool top = (rem >> 127) != 0;
+        rem = (rem << 1) | ((u.v[i >> 5] >> (i & 31)) & 1u);
+        q <<= 1;
+        if (top || rem >= lam) { rem -= lam; q |= 1; }
+    }
+    GlvK k;
+    for (int i = 0; i < 4; ++i) { k.k1[i] = (uint32_t)(rem >> (32 * i)); k.k2[i] = (uint32_t)(q >> (32 * i)); }
+    return k;
+}
+// Queues one round.  round > 0 with prev_u: T comes from the previous round's points (pts_prev, rec[3*(round-1)..]);
+// otherwise T is a third bucket sum.  pts_round: this round's T, T0, T1 (T of later rounds is left to k_open_finish).
+static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars, const G1Jac* gens, const Fr& u, size_t old_size, int round, const Fr* prev_u,
+                             G1Jac* pts_round, const G1Jac* pts_prev, G1Jac* rec, hipStream_t st) {
+    ZK_ARG(old_size < (1ull << 31), "opening: more than 2^31 generators");
+    const size_t new_size = (old_size + 1) / 2;
+    const bool chained = round > 0 && prev_u != nullptr;
+    Scratch aff(sizeof(G1Affine) * old_size);
+    if (aff.rc) return aff.rc;
+    hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(old_size, CH), GT)), dim3(GT), 0, st, aff.p, gens, old_size);
+    MsmDescs descs;
+    const uint32_t half = (uint32_t)(old_size / 2);
+    const uint32_t n_msm = chained ? 2u : 3u;
+    uint32_t q = 0;
+    if (!chained) descs.d[q++] = MsmDesc{(uint32_t)old_size, 1u, 0u, 1u, 0u};
+    descs.d[q++] = MsmDesc{half, 2u, 0u, 2u, 1u};
+    descs.d[q++] = MsmDesc{half, 2u, 1u, 2u, 0u};
+    for (; q < 3; ++q) descs.d[q] = MsmDesc{0u, 1u, 0u, 1u, 0u};
+    const size_t count_max = chained ? half : old_size;
+    const uint32_t chunks = count_max ? cdiv(count_max, MSEG) : 1u;
+    const uint32_t nseg = chunks < 16u ? chunks : 16u;
+    const uint32_t cps = (chunks + nseg - 1) / nseg;
+    Scratch partial(sizeof(G1Jac) * n_msm * MW * nseg), wsum(sizeof(G1Jac) * n_msm * MW);
+    if (partial.rc) return partial.rc;
+    if (wsum.rc) return wsum.rc;
+    hipLaunchKernelGGL(k_msm_seg, dim3(nseg, MW, n_msm), dim3(MT), 0, st, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), scalars, aff.as<G1Affine>(), descs, nseg, cps);
+    if (nseg > 1) hipLaunchKernelGGL(k_g1_rowsum, dim3(n_msm * MW, 1), dim3(GT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), (size_t)nseg, 1u);
+    OpenExtras ex;
+    ex.W = wsum.as<G1Jac>();
+    ex.pts_round = pts_round;
+    ex.pts_prev = pts_prev;
+    ex.rec_prev = (chained && round >= 2) ? rec + 3 * (round - 1) : nullptr;
+    ex.rec_round = chained ? rec + 3 * round : nullptr;
+    ex.n_msm = n_msm;
+    ex.round = (uint32_t)round;
+    memset(ex.kc, 0, sizeof(ex.kc));
+    if (chained) {
+        const Fr one = fr_from_u64(1), pu = *prev_u, omu = sub(one, pu);
+        ex.kc[0] = glv_split(fr_mul_std(pu, omu));
+        ex.kc[1] = glv_split(fr_mul_std(omu, omu));
+        ex.kc[2] = glv_split(fr_mul_std(pu, pu));
+    }
+    const uint32_t nb_main = cdiv(new_size, GT);
+    hipLaunchKernelGGL(k_open_fold, dim3(nb_main + n_msm + (chained ? 3u : 0u)), dim3(GT), 0, st, new_scalars, new_gens, scalars, aff.as<G1Affine>(), to_mont(u), glv_split(u),
+                       old_size, new_size, nb_main, ex);
     ZK_LAUNCH_CHECK();
     return 0;
 }
@@ -433,31 +669,75 @@ int zk_g1_commit_int(void* out, const void* gens, const void* scalars_fr, size_t
     return 0;
 }
 
-// One round of Commitment::me_open (commitment.cu:79-129).  u: standard-form challenge (used both as the
-// field scalar of the fold and as the raw 256-bit integer of the scalar multiplications, as the reference does).
-// new_scalars / new_gens: (old_size+1)/2 elements.  sums_host: 3 points (sum T, sum T0, sum T1).
+// One round of Commitment::me_open (commitment.cu:79-129) with all three sums computed directly.  u: standard-form
+// challenge (the field scalar of the fold and the integer of the scalar multiplications, as in the reference).
+// new_scalars / new_gens: (old_size+1)/2 elements.  sums_host: 3 points (T, T0, T1), normalised to z = 1.
 int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host, const void* scalars, const void* gens, const uint32_t* u, size_t old_size, void* stv) {
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(old_size >= 1, "zk_g1_open_round: empty input");
-    const size_t new_size = (old_size + 1) / 2;
-    Scratch parts(sizeof(G1Jac) * 5 * new_size), sums(sizeof(G1Jac) * 3);
-    if (parts.rc) return parts.rc;
-    if (sums.rc) return sums.rc;
-    const Fr uu = load_fr(u);
-    hipLaunchKernelGGL(k_open_parts, dim3(cdiv(5 * new_size, GT)), dim3(GT), 0, st, parts.as<G1Jac>(), (const Fr*)scalars, (const G1Jac*)gens, uu, old_size, new_size);
-    hipLaunchKernelGGL(k_open_combine, dim3(cdiv(new_size, GT)), dim3(GT), 0, st, (Fr*)new_scalars, (G1Jac*)new_gens, parts.as<G1Jac>(), (const Fr*)scalars, (const G1Jac*)gens, to_mont(uu), old_size, new_size);
-    ZK_LAUNCH_CHECK();
-    G1Jac* P = parts.as<G1Jac>();
-    int rc = g1_sum_device(sums.as<G1Jac>() + 0, P + 1 * new_size, new_size, st);
-    if (!rc) rc = g1_sum_device(sums.as<G1Jac>() + 1, P + 3 * new_size, new_size, st);
-    if (!rc) rc = g1_sum_device(sums.as<G1Jac>() + 2, P + 4 * new_size, new_size, st);
+    Scratch pts(sizeof(G1Jac) * 3);
+    if (pts.rc) return pts.rc;
+    int rc = open_round_launch((Fr*)new_scalars, (G1Jac*)new_gens, (const Fr*)scalars, (const G1Jac*)gens, load_fr(u), old_size, 0, nullptr, pts.as<G1Jac>(), nullptr, nullptr, st);
     if (rc) return rc;
+    hipLaunchKernelGGL(k_g1_normalize<false>, dim3(1), dim3(GT), 0, st, pts.p, pts.as<G1Jac>(), (size_t)3);
+    ZK_LAUNCH_CHECK();
     void* stage = nullptr;
     rc = staging(&stage, sizeof(G1Jac) * 3);
     if (rc) return rc;
-    ZK_HIP(hipMemcpyAsync(stage, sums.p, sizeof(G1Jac) * 3, hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipMemcpyAsync(stage, pts.p, sizeof(G1Jac) * 3, hipMemcpyDeviceToHost, st));
     ZK_HIP(hipStreamSynchronize(st));
     memcpy(sums_host, stage, sizeof(G1Jac) * 3);
+    return 0;
+}
+
+// The whole recursion of Commitment::me_open (commitment.cu:109-129): `rounds` halvings of (scalars, gens) of length n
+// with the challenges u[0..rounds).  proof_host receives 3*rounds + 1 points: T, T0, T1 of every round, then the
+// folded generator; all normalised to z = 1 (infinity: all-zero limbs).  final_scalar_host: the folded scalar.
+int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(n >= 1, "zk_g1_open: empty input");
+    ZK_ARG(rounds >= 0 && rounds <= 64, "zk_g1_open: bad round count");
+    const size_t npts = 3 * (size_t)rounds + 1;
+    Scratch pts(sizeof(G1Jac) * npts), rec(sizeof(G1Jac) * 3 * (rounds ? rounds : 1));
+    if (pts.rc) return pts.rc;
+    if (rec.rc) return rec.rc;
+    std::vector<std::unique_ptr<Scratch>> keep;
+    const Fr* cs = (const Fr*)scalars;
+    const G1Jac* cg = (const G1Jac*)gens;
+    size_t size = n;
+    Fr prev_u = big_zero<8>();
+    for (int r = 0; r < rounds; ++r) {
+        const size_t ns = (size + 1) / 2;
+        keep.emplace_back(new Scratch(sizeof(Fr) * ns));
+        Scratch& s2 = *keep.back();
+        keep.emplace_back(new Scratch(sizeof(G1Jac) * ns));
+        Scratch& g2 = *keep.back();
+        if (s2.rc) return s2.rc;
+        if (g2.rc) return g2.rc;
+        const Fr ur = load_fr(u + 8 * r);
+        int rc = open_round_launch(s2.as<Fr>(), g2.as<G1Jac>(), cs, cg, ur, size, r, r ? &prev_u : nullptr, pts.as<G1Jac>() + 3 * r,
+                                   r ? pts.as<G1Jac>() + 3 * (r - 1) : nullptr, rec.as<G1Jac>(), st);
+        if (rc) return rc;
+        if (keep.size() > 4) { keep.erase(keep.begin(), keep.begin() + 2); }   // the round before the previous one is no longer read
+        cs = s2.as<Fr>();
+        cg = g2.as<G1Jac>();
+        size = ns;
+        prev_u = ur;
+    }
+    hipLaunchKernelGGL(k_open_finish, dim3(cdiv((size_t)rounds + 1, GT)), dim3(GT), 0, st, pts.as<G1Jac>(), rec.as<G1Jac>(), cg, (uint32_t)rounds);
+    hipLaunchKernelGGL(k_g1_normalize<false>, dim3(cdiv(cdiv(npts, CH), GT)), dim3(GT), 0, st, pts.p, pts.as<G1Jac>(), npts);
+    ZK_LAUNCH_CHECK();
+    std::vector<uint8_t> tmp;
+    void* stage = nullptr;
+    const size_t bytes = sizeof(G1Jac) * npts + sizeof(Fr);
+    ZK_ARG(bytes <= 65536, "zk_g1_open: proof larger than the staging buffer");
+    int rc = staging(&stage, bytes);
+    if (rc) return rc;
+    ZK_HIP(hipMemcpyAsync(stage, pts.p, sizeof(G1Jac) * npts, hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipMemcpyAsync((char*)stage + sizeof(G1Jac) * npts, cs, sizeof(Fr), hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipStreamSynchronize(st));
+    memcpy(proof_host, stage, sizeof(G1Jac) * npts);
+    memcpy(final_scalar_host, (char*)stage + sizeof(G1Jac) * npts, sizeof(Fr));
     return 0;
 }
 

@@ -1,3 +1,4 @@
+#include <cstring>
 #include "commitment.hpp"
 
 #include <cstdlib>
@@ -50,26 +51,14 @@ G1TensorJacobian Commitment::commit_int_multi(const vector<FrTensor>& ts) const 
 
 Fr_t Commitment::me_open(const FrTensor& t, const Commitment& generators, vector<Fr_t>::const_iterator begin, vector<Fr_t>::const_iterator end, vector<G1Jacobian_t>& proof) {
     if (t.size != generators.size) throw std::runtime_error("Commitment::me_open - Incompatible dimensions " + std::to_string(t.size) + " " + std::to_string(generators.size));
-    const FrTensor* s = &t;
-    const G1TensorJacobian* g = &generators;
-    std::vector<FrTensor> ks;
-    std::vector<G1TensorJacobian> kg;
-    ks.reserve(end - begin);
-    kg.reserve(end - begin);
-    for (auto it = begin; it < end; ++it) {
-        const uint new_size = (s->size + 1) / 2;
-        ks.emplace_back(new_size);
-        kg.emplace_back(new_size);
-        G1Jacobian_t sums[3];
-        ZKC(zk_g1_open_round(ks.back().gpu_data, kg.back().gpu_data, sums[0].x.val, s->gpu_data, g->gpu_data, it->val, s->size, nullptr));
-        proof.push_back(sums[0]);
-        proof.push_back(sums[1]);
-        proof.push_back(sums[2]);
-        s = &ks.back();
-        g = &kg.back();
-    }
-    proof.push_back((*g)(0u));
-    return (*s)(0u);
+    const int rounds = (int)(end - begin);
+    std::vector<uint32_t> uu((size_t)rounds * 8 + 8);
+    for (int r = 0; r < rounds; ++r) memcpy(&uu[(size_t)r * 8], (begin + r)->val, 32);
+    std::vector<G1Jacobian_t> pts(3 * (size_t)rounds + 1);
+    Fr_t out;
+    ZKC(zk_g1_open(pts[0].x.val, out.val, t.gpu_data, generators.gpu_data, t.size, uu.data(), rounds, nullptr));
+    proof.insert(proof.end(), pts.begin(), pts.end());
+    return out;
 }
 
 Fr_t Commitment::open(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u, vector<G1Jacobian_t>& proof) const {
