@@ -233,8 +233,12 @@ static constexpr int MW = 32;        // 8-bit signed windows over a 255-bit scal
 static constexpr int MT = 128;       // lanes of a bucket workgroup = buckets (digit magnitudes 1..128)
 static constexpr int MSEG = 4096;    // elements per chunk (12-bit list entries)
 static constexpr int MCAP = 96;      // list slots per bucket and pass
-struct MsmDesc { uint32_t count, s_mul, s_off, b_mul, b_off; };   // element i: scalar S[i*s_mul+s_off], base A[i*b_mul+b_off]
-struct MsmDescs { MsmDesc d[3]; };
+struct MsmDesc { const Fr* scalars; uint32_t count, s_mul, s_off, b_mul, b_off, slot; };   // element i: scalar scalars[i*s_mul+s_off], base A[i*b_mul+b_off]
+template <int NMAX> struct MsmDescs { MsmDesc d[NMAX]; };
+static constexpr int TAIL_N = 8192;        // generators at which the remaining rounds are computed in one batch
+static constexpr int TAIL_LEVELS = 20;     // most rounds the batch takes
+static constexpr int TAIL_SUMS = 3 * TAIL_LEVELS + 1;
+struct TailU { Fr u[TAIL_LEVELS]; };       // challenges of the batched rounds, Montgomery form
 struct GlvK { uint32_t k1[4], k2[4]; };
 
 __device__ __forceinline__ bool aff_is_inf(const G1Affine& p) { return is_zero(p.x) && is_zero(p.y); }   // normalised infinity: all-zero limbs
@@ -289,14 +293,15 @@ __device__ __forceinline__ int msm_digit(const uint32_t* __restrict__ sp, uint32
 // Lane t owns the bucket of magnitude t+1.  Per chunk the elements are first sorted into per-bucket lists in LDS
 // (one atomic per element), then every lane walks its own list with mixed additions, so lanes stay busy in
 // lockstep whatever the digits are; elements that find their bucket's list full wait for the next pass over the chunk.
-__global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, const Fr* __restrict__ S, const G1Affine* __restrict__ A, const MsmDescs descs,
-                                                uint32_t nseg, uint32_t chunks_per_seg) {
+template <int NMAX>
+__global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, const G1Affine* __restrict__ A, const MsmDescs<NMAX> descs, uint32_t nseg, uint32_t chunks_per_seg) {
     __shared__ uint32_t cnt[MT];
     __shared__ uint32_t pool[MCAP * MT / 2];       // u16 lists while accumulating, the 36 x MT point tree afterwards
     static_assert(MCAP * MT / 2 >= 36 * MT, "pool too small for the point tree");
     static_assert(MSEG / MT == 32, "one done-bit per element of a lane's chunk share");
     uint16_t* list = reinterpret_cast<uint16_t*>(pool);
     const MsmDesc d = descs.d[blockIdx.z];
+    const Fr* __restrict__ S = d.scalars;
     const uint32_t w = blockIdx.y, seg = blockIdx.x, t = threadIdx.x;
     G1Jac acc = g1_infinity();
     for (uint32_t ch = 0; ch < chunks_per_seg; ++ch) {
@@ -419,11 +424,71 @@ __global__ void __launch_bounds__(GT) k_open_fold(Fr* __restrict__ new_scalars, 
     if (!aff_is_inf(a1)) r = g1_add_mixed(r, a1);
     new_gens[g] = r;
 }
+// ---- the last rounds in one batch ---------------------------------------------------------------------------------------
+// Once n0 <= TAIL_N generators are left, every later round's generators are fixed linear combinations of these n0
+// points: g at level j, block i, is sum over k in block i of W_j(k) g_k with W_j(k) = prod_{b<j} (bit_b(k) ? 1-u_b : u_b).
+// So T, T0, T1 of all remaining rounds and the final generator are multi-scalar multiplications over the same n0
+// affine points with coefficients that are plain field arithmetic; they run as one launch instead of a chain of
+// rounds that each wait for a scalar multiplication.
+// Folded scalars of all levels: level 0 is S itself, level j >= 1 sits at SL + sum_{1<=i<j} n_i, n_i = ceil(n0 / 2^i).
+__global__ void __launch_bounds__(1024) k_tail_scalars(Fr* __restrict__ SL, const Fr* __restrict__ S, const TailU us, uint32_t n0, uint32_t levels) {
+    const Fr* cur = S;
+    Fr* nxt = SL;
+    uint32_t n = n0;
+    for (uint32_t j = 0; j < levels; ++j) {
+        const uint32_t ns = (n + 1) / 2;
+        for (uint32_t g = threadIdx.x; g < ns; g += 1024) {
+            const Fr s0 = cur[2 * g];
+            nxt[g] = (2 * g + 1 < n) ? add(s0, mont_mul(us.u[j], sub(cur[2 * g + 1], s0))) : sub(s0, mont_mul(us.u[j], s0));
+        }
+        __syncthreads();
+        cur = nxt;
+        nxt += ns;
+        n = ns;
+    }
+}
+// C[(3j+0)*n0 + k] = s_j[k>>j] W_j(k); C[(3j+1)*n0 + k] = s_j[(k>>j)-1] W_j(k) for odd k>>j; C[(3j+2)*n0 + k] = s_j[(k>>j)+1] W_j(k)
+// for even k>>j with a partner; zero elsewhere.  C[3*levels*n0 + k] = W_levels(k).
+__global__ void __launch_bounds__(256) k_tail_coeffs(Fr* __restrict__ C, const Fr* __restrict__ SL, const Fr* __restrict__ S, const TailU us, uint32_t n0, uint32_t levels) {
+    const uint32_t k = blockIdx.x * 256 + threadIdx.x;
+    if (k >= n0) return;
+    const Fr one_m = big_one_mont<8>();
+    Fr W = one_m;                 // Montgomery form
+    const Fr* sj = S;
+    const Fr* nxt = SL;
+    uint32_t n = n0;
+    const Fr zero = big_zero<8>();
+    for (uint32_t j = 0; j < levels; ++j) {
+        const uint32_t i = k >> j;
+        // mont_mul(Montgomery W, standard s) is the standard-form product
+        C[(size_t)(3 * j) * n0 + k] = mont_mul(W, sj[i]);
+        C[(size_t)(3 * j + 1) * n0 + k] = (i & 1u) ? mont_mul(W, sj[i - 1]) : zero;
+        C[(size_t)(3 * j + 2) * n0 + k] = (!(i & 1u) && i + 1 < n) ? mont_mul(W, sj[i + 1]) : zero;
+        W = mont_mul(W, (i & 1u) ? sub(one_m, us.u[j]) : us.u[j]);
+        const uint32_t ns = (n + 1) / 2;
+        sj = nxt;
+        nxt += ns;
+        n = ns;
+    }
+    C[(size_t)(3 * levels) * n0 + k] = from_mont(W);
+}
+// one workgroup per sum: lane 0 assembles sum_w 2^(8w) W[w] into pts[slot]
+__global__ void __launch_bounds__(GT) k_msm_horner(G1Jac* __restrict__ pts, const G1Jac* __restrict__ Wsum, const MsmDescs<TAIL_SUMS> descs) {
+    if (threadIdx.x != 0) return;
+    const G1Jac* W = Wsum + (size_t)blockIdx.x * MW;
+    G1Jac r = W[MW - 1];
+    for (int w = MW - 2; w >= 0; --w) {
+        for (int k = 0; k < 8; ++k) r = g1_double(r);
+        r = g1_add(r, W[w]);
+    }
+    pts[descs.d[blockIdx.x].slot] = r;
+}
+
 // after the last round: T of rounds >= 1 from its three parts, and the folded generator as the last proof point
-__global__ void __launch_bounds__(GT) k_open_finish(G1Jac* __restrict__ pts, const G1Jac* __restrict__ rec, const G1Jac* __restrict__ last_gen, uint32_t rounds) {
+__global__ void __launch_bounds__(GT) k_open_finish(G1Jac* __restrict__ pts, const G1Jac* __restrict__ rec, const G1Jac* __restrict__ last_gen, uint32_t chained_rounds, uint32_t rounds) {
     const uint32_t r = blockIdx.x * GT + threadIdx.x;
-    if (r >= 1 && r < rounds) pts[3 * r] = g1_add(g1_add(rec[3 * r], rec[3 * r + 1]), rec[3 * r + 2]);
-    if (r == rounds) pts[3 * rounds] = last_gen[0];
+    if (r >= 1 && r < chained_rounds) pts[3 * r] = g1_add(g1_add(rec[3 * r], rec[3 * r + 1]), rec[3 * r + 2]);
+    if (r == rounds && last_gen) pts[3 * rounds] = last_gen[0];
 }
 
 // ---- host side ----------------------------------------------------------------------------------------------------------
@@ -485,14 +550,14 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     Scratch aff(sizeof(G1Affine) * old_size);
     if (aff.rc) return aff.rc;
     hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(old_size, CH), GT)), dim3(GT), 0, st, aff.p, gens, old_size);
-    MsmDescs descs;
+    MsmDescs<3> descs;
     const uint32_t half = (uint32_t)(old_size / 2);
     const uint32_t n_msm = chained ? 2u : 3u;
     uint32_t q = 0;
-    if (!chained) descs.d[q++] = MsmDesc{(uint32_t)old_size, 1u, 0u, 1u, 0u};
-    descs.d[q++] = MsmDesc{half, 2u, 0u, 2u, 1u};
-    descs.d[q++] = MsmDesc{half, 2u, 1u, 2u, 0u};
-    for (; q < 3; ++q) descs.d[q] = MsmDesc{0u, 1u, 0u, 1u, 0u};
+    if (!chained) descs.d[q++] = MsmDesc{scalars, (uint32_t)old_size, 1u, 0u, 1u, 0u, 0u};
+    descs.d[q++] = MsmDesc{scalars, half, 2u, 0u, 2u, 1u, 1u};
+    descs.d[q++] = MsmDesc{scalars, half, 2u, 1u, 2u, 0u, 2u};
+    for (; q < 3; ++q) descs.d[q] = MsmDesc{scalars, 0u, 1u, 0u, 1u, 0u, 0u};
     const size_t count_max = chained ? half : old_size;
     const uint32_t chunks = count_max ? cdiv(count_max, MSEG) : 1u;
     const uint32_t nseg = chunks < 16u ? chunks : 16u;
@@ -500,7 +565,7 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     Scratch partial(sizeof(G1Jac) * n_msm * MW * nseg), wsum(sizeof(G1Jac) * n_msm * MW);
     if (partial.rc) return partial.rc;
     if (wsum.rc) return wsum.rc;
-    hipLaunchKernelGGL(k_msm_seg, dim3(nseg, MW, n_msm), dim3(MT), 0, st, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), scalars, aff.as<G1Affine>(), descs, nseg, cps);
+    hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MT), 0, st, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff.as<G1Affine>(), descs, nseg, cps);
     if (nseg > 1) hipLaunchKernelGGL(k_g1_rowsum, dim3(n_msm * MW, 1), dim3(GT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), (size_t)nseg, 1u);
     OpenExtras ex;
     ex.W = wsum.as<G1Jac>();
@@ -521,6 +586,43 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     hipLaunchKernelGGL(k_open_fold, dim3(nb_main + n_msm + (chained ? 3u : 0u)), dim3(GT), 0, st, new_scalars, new_gens, scalars, aff.as<G1Affine>(), to_mont(u), glv_split(u),
                        old_size, new_size, nb_main, ex);
     ZK_LAUNCH_CHECK();
+    return 0;
+}
+
+// Queues the batch for the last `levels` rounds (rounds r0 .. r0+levels-1 of `rounds`) over n0 <= TAIL_N generators.
+// Writes T, T0, T1 of those rounds and the final generator into pts; *final_scalar points at the folded scalar.
+static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, const uint32_t* u, int levels, int r0, int rounds, G1Jac* pts, const Fr** final_scalar,
+                            std::vector<std::unique_ptr<Scratch>>& keep, hipStream_t st) {
+    TailU us;
+    for (int j = 0; j < levels; ++j) us.u[j] = to_mont(load_fr(u + 8 * j));
+    for (int j = levels; j < TAIL_LEVELS; ++j) us.u[j] = big_zero<8>();
+    keep.emplace_back(new Scratch(sizeof(Fr) * (n0 + (size_t)levels + 1)));
+    Scratch& sl = *keep.back();
+    const int n_msm = 3 * levels + 1;
+    const uint32_t nseg = cdiv(n0, MSEG);
+    Scratch aff(sizeof(G1Affine) * n0), coef(sizeof(Fr) * (size_t)n_msm * n0), partial(sizeof(G1Jac) * n_msm * MW * nseg), wsum(sizeof(G1Jac) * n_msm * MW);
+    if (sl.rc) return sl.rc;
+    if (aff.rc) return aff.rc;
+    if (coef.rc) return coef.rc;
+    if (partial.rc) return partial.rc;
+    if (wsum.rc) return wsum.rc;
+    hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(n0, CH), GT)), dim3(GT), 0, st, aff.p, gens, n0);
+    hipLaunchKernelGGL(k_tail_scalars, dim3(1), dim3(1024), 0, st, sl.as<Fr>(), scalars, us, (uint32_t)n0, (uint32_t)levels);
+    hipLaunchKernelGGL(k_tail_coeffs, dim3(cdiv(n0, 256)), dim3(256), 0, st, coef.as<Fr>(), sl.as<Fr>(), scalars, us, (uint32_t)n0, (uint32_t)levels);
+    MsmDescs<TAIL_SUMS> descs;
+    for (int i = 0; i < TAIL_SUMS; ++i) {
+        const bool live = i < n_msm;
+        const uint32_t slot = !live ? 0u : (i == 3 * levels ? 3u * (uint32_t)rounds : 3u * (uint32_t)r0 + (uint32_t)i);
+        descs.d[i] = MsmDesc{coef.as<Fr>() + (live ? (size_t)i * n0 : 0), live ? (uint32_t)n0 : 0u, 1u, 0u, 1u, 0u, slot};
+    }
+    hipLaunchKernelGGL(k_msm_seg<TAIL_SUMS>, dim3(nseg, MW, n_msm), dim3(MT), 0, st, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff.as<G1Affine>(), descs, nseg, 1u);
+    if (nseg > 1) hipLaunchKernelGGL(k_g1_rowsum, dim3(n_msm * MW, 1), dim3(GT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), (size_t)nseg, 1u);
+    hipLaunchKernelGGL(k_msm_horner, dim3(n_msm), dim3(GT), 0, st, pts, wsum.as<G1Jac>(), descs);
+    ZK_LAUNCH_CHECK();
+    // the folded scalar is the single element of the last level
+    size_t off = 0, nn = n0;
+    for (int j = 1; j < levels; ++j) { nn = (nn + 1) / 2; off += nn; }
+    *final_scalar = sl.as<Fr>() + off;
     return 0;
 }
 
@@ -706,7 +808,16 @@ int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* sc
     const G1Jac* cg = (const G1Jac*)gens;
     size_t size = n;
     Fr prev_u = big_zero<8>();
+    int chained_rounds = rounds;
+    bool tail_done = false;
     for (int r = 0; r < rounds; ++r) {
+        if (size <= (size_t)TAIL_N && rounds - r <= TAIL_LEVELS) {
+            int rc = open_tail_launch(cs, cg, size, u + 8 * r, rounds - r, r, rounds, pts.as<G1Jac>(), &cs, keep, st);
+            if (rc) return rc;
+            chained_rounds = r;
+            tail_done = true;
+            break;
+        }
         const size_t ns = (size + 1) / 2;
         keep.emplace_back(new Scratch(sizeof(Fr) * ns));
         Scratch& s2 = *keep.back();
@@ -724,7 +835,8 @@ int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* sc
         size = ns;
         prev_u = ur;
     }
-    hipLaunchKernelGGL(k_open_finish, dim3(cdiv((size_t)rounds + 1, GT)), dim3(GT), 0, st, pts.as<G1Jac>(), rec.as<G1Jac>(), cg, (uint32_t)rounds);
+    hipLaunchKernelGGL(k_open_finish, dim3(cdiv((size_t)rounds + 1, GT)), dim3(GT), 0, st, pts.as<G1Jac>(), rec.as<G1Jac>(), tail_done ? (const G1Jac*)nullptr : cg,
+                       (uint32_t)chained_rounds, (uint32_t)rounds);
     hipLaunchKernelGGL(k_g1_normalize<false>, dim3(cdiv(cdiv(npts, CH), GT)), dim3(GT), 0, st, pts.p, pts.as<G1Jac>(), npts);
     ZK_LAUNCH_CHECK();
     std::vector<uint8_t> tmp;
