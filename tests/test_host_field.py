@@ -32,8 +32,13 @@ def test_host_fr_ops_match_bigint_and_oracle():
         assert fr_ints(got) == [f(x, y) for x, y in zip(a, b)], f"host fr op {op}"
         orc_check(orc.orc_fr_op(op, A, B, exp, len(a)))
         assert (got == exp).all(), f"host fr op {op} vs oracle"
-    assert lib.zkp_host_fr_op(ctypes.c_int(6), _np_ptr(A), _np_ptr(B), _np_ptr(got), ctypes.c_long(64)) == 0
-    orc_check(orc.orc_fr_op(6, A, B, exp, 64))
+    # Montgomery inverse (binary algorithm in the product, exponentiation in the oracle): x = aR -> a^-1 R = x^-1 R^2
+    inv_in = a + [1 << k for k in range(0, 255, 7)] + [R_MOD - (1 << k) for k in range(0, 254, 9)] + [(1 << 254) + 1, 3, R_MOD // 2, R_MOD // 2 + 1]
+    IA = fr_array(inv_in)
+    got, exp = np.zeros_like(IA), np.zeros_like(IA)
+    assert lib.zkp_host_fr_op(ctypes.c_int(6), _np_ptr(IA), _np_ptr(IA), _np_ptr(got), ctypes.c_long(len(inv_in))) == 0
+    assert fr_ints(got) == [pow(x, -1, R_MOD) * FR_R * FR_R % R_MOD if x else 0 for x in inv_in]
+    orc_check(orc.orc_fr_op(6, IA, IA, exp, 64))
     assert (got[:64] == exp[:64]).all()
 
 
@@ -52,8 +57,12 @@ def test_host_fp_ops_match_bigint_and_oracle():
         assert fp_ints(got) == [f(x, y) for x, y in zip(a, b)], f"host fp op {op}"
         orc_check(orc.orc_fp_op(op, A, B, exp, len(a)))
         assert (got == exp).all()
-    assert lib.zkp_host_fp_op(ctypes.c_int(6), _np_ptr(A), _np_ptr(B), _np_ptr(got), ctypes.c_long(32)) == 0
-    orc_check(orc.orc_fp_op(6, A, B, exp, 32))
+    inv_in = a + [1 << k for k in range(0, 381, 11)] + [P_MOD - (1 << k) for k in range(0, 380, 13)] + [3, P_MOD // 2, P_MOD // 2 + 1]
+    IA = fp_array(inv_in)
+    got, exp = np.zeros_like(IA), np.zeros_like(IA)
+    assert lib.zkp_host_fp_op(ctypes.c_int(6), _np_ptr(IA), _np_ptr(IA), _np_ptr(got), ctypes.c_long(len(inv_in))) == 0
+    assert fp_ints(got) == [pow(x, -1, P_MOD) * FP_R * FP_R % P_MOD if x else 0 for x in inv_in]
+    orc_check(orc.orc_fp_op(6, IA, IA, exp, 32))
     assert (got[:32] == exp[:32]).all()
 
 

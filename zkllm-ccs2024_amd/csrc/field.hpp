@@ -380,18 +380,14 @@ template <int N> ZK_HD Big<N> from_mont(const Big<N>& a) {
     one.v[0] = 1;
     return mont_mul(a, one);
 }
-// a^(p-2), Montgomery in / Montgomery out (0 -> 0).
-template <int N> ZK_HD Big<N> mont_inverse(Big<N> a) {
+// a^(p-2), Montgomery in / Montgomery out (0 -> 0): Fermat inversion, kept as the cross-check of mont_inverse.
+template <int N> ZK_HD Big<N> mont_inverse_fermat(Big<N> a) {
     typedef typename KOf<N>::K K;
     uint32_t e[N];
     {
-        uint64_t br = 2;
+        uint32_t br = 0;
 #pragma unroll
-        for (int i = 0; i < N; ++i) {
-            uint64_t t = (uint64_t)K::P(i) - br;
-            e[i] = (uint32_t)t;
-            br = (t >> 32) & 1u;
-        }
+        for (int i = 0; i < N; ++i) e[i] = subb32(K::P(i), i == 0 ? 2u : 0u, br);
     }
     Big<N> res = big_one_mont<N>();
     for (int i = 0; i < N; ++i)
@@ -400,6 +396,77 @@ template <int N> ZK_HD Big<N> mont_inverse(Big<N> a) {
             a = mont_sqr(a);
         }
     return res;
+}
+// Inverse, Montgomery in / Montgomery out (0 -> 0), by the binary "almost Montgomery inverse": shifts, additions and
+// subtractions on u, v, r, s (about 1.4 * bits steps) produce a^-1 * 2^k, and one or two Montgomery products remove
+// the power of two.  About twenty times less work than the exponentiation for one value; it is what bounds the
+// latency of every batched inversion (one inverse per batch, the other lanes wait for it).
+template <int N> ZK_HD Big<N> mont_inverse(const Big<N>& a) {
+    typedef typename KOf<N>::K K;
+    constexpr int BITS = (N == 8) ? 255 : 381;
+    if (is_zero(a)) return a;
+    uint32_t u[N], v[N], r[N], q[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) { u[i] = K::P(i); v[i] = a.v[i]; r[i] = 0; q[i] = 0; }
+    q[0] = 1;
+    int k = 0;
+    auto shr1 = [](uint32_t* x) {
+#pragma unroll
+        for (int i = 0; i < N - 1; ++i) x[i] = (x[i] >> 1) | (x[i + 1] << 31);
+        x[N - 1] >>= 1;
+    };
+    auto shl1 = [](uint32_t* x) {
+#pragma unroll
+        for (int i = N - 1; i > 0; --i) x[i] = (x[i] << 1) | (x[i - 1] >> 31);
+        x[0] <<= 1;
+    };
+    for (; k < 2 * BITS + 2; ++k) {
+        uint32_t nzv = 0;
+#pragma unroll
+        for (int i = 0; i < N; ++i) nzv |= v[i];
+        if (!nzv) break;
+        if (!(u[0] & 1u)) { shr1(u); shl1(q); }
+        else if (!(v[0] & 1u)) { shr1(v); shl1(r); }
+        else {
+            uint32_t d[N], br = 0;          // d = v - u, borrow: u > v
+#pragma unroll
+            for (int i = 0; i < N; ++i) d[i] = subb32(v[i], u[i], br);
+            if (br) {                        // u > v: u = (u - v) / 2, r += q, q *= 2
+                uint32_t b2 = 0, c = 0;
+#pragma unroll
+                for (int i = 0; i < N; ++i) u[i] = subb32(u[i], v[i], b2);
+                shr1(u);
+#pragma unroll
+                for (int i = 0; i < N; ++i) r[i] = addc32(r[i], q[i], c);
+                shl1(q);
+            } else {                         // v = (v - u) / 2, q += r, r *= 2
+                uint32_t c = 0;
+#pragma unroll
+                for (int i = 0; i < N; ++i) v[i] = d[i];
+                shr1(v);
+#pragma unroll
+                for (int i = 0; i < N; ++i) q[i] = addc32(q[i], r[i], c);
+                shl1(r);
+            }
+        }
+    }
+    // r < 2p holds a^-1 * 2^k up to sign: the inverse is p - (r mod p)
+    Big<N> rr;
+#pragma unroll
+    for (int i = 0; i < N; ++i) rr.v[i] = r[i];
+    rr = reduce_once(rr);
+    Big<N> y = sub(big_zero<N>(), rr);
+    // y = (aR)^-1 2^k; the Montgomery form of the inverse is y * 2^(64N - k)
+    int e = 64 * N - k;
+    while (e > 0) {
+        const int step = e < BITS - 1 ? e : BITS - 1;
+        Big<N> p2;
+#pragma unroll
+        for (int i = 0; i < N; ++i) p2.v[i] = ((step >> 5) == i) ? (1u << (step & 31)) : 0u;
+        y = mont_mul(mont_mul(y, big_r2<N>()), p2);
+        e -= step;
+    }
+    return y;
 }
 
 // ---- standard-form helpers (tensors hold standard-form residues) ---------------------------------

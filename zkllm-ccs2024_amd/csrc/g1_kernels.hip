@@ -278,15 +278,50 @@ static __device__ __attribute__((noinline)) G1Jac g1_mul_glv(const G1Jac& P, con
     return out;
 }
 
-// signed 8-bit digit of window w: raw byte plus the carry of the lower windows (a lower digit above 128 is
-// replaced by digit - 256 and carries one).  The carry only depends on the first lower byte that is not 128.
-__device__ __forceinline__ int msm_digit(const uint32_t* __restrict__ sp, uint32_t w) {
-    int raw = (int)((sp[w >> 2] >> ((w & 3u) * 8u)) & 0xFFu);
-    for (int j = (int)w - 1; j >= 0; --j) {
-        const uint32_t b = (sp[j >> 2] >> ((j & 3) * 8)) & 0xFFu;
-        if (b != 128u) { raw += (b > 128u) ? 1 : 0; break; }
+// signed 8-bit digit of window w of the scalar's balanced representative: s above r/2 is replaced by -(r - s), so
+// that small negative values (r - x, as weights are embedded) have as few non-zero windows as small positive ones
+// instead of sharing r's high bytes.  Within the magnitude, a digit above 128 is replaced by digit - 256 and carries
+// one; the carry into window w only depends on the first lower byte that is not 128.
+__device__ __forceinline__ int msm_digit(const Fr& sv, uint32_t w) {
+    // r - s, and whether it is the smaller of the two (s = 0 keeps s)
+    Fr n;
+    uint32_t br = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) n.v[i] = subb32(FrK::P(i), sv.v[i], br);
+    uint32_t lt = 0;    // borrow of n - s: n < s
+#pragma unroll
+    for (int i = 0; i < 8; ++i) (void)subb32(n.v[i], sv.v[i], lt);
+    const bool flip = lt != 0;
+    uint32_t m[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) m[i] = flip ? n.v[i] : sv.v[i];
+    uint32_t word = 0, lower = 0;      // the word holding byte w, and the bytes below it in that word
+#pragma unroll
+    for (int i = 0; i < 8; ++i) if ((w >> 2) == (uint32_t)i) word = m[i];
+    const uint32_t sh = (w & 3u) * 8u;
+    int raw = (int)((word >> sh) & 0xFFu);
+    // carry from below: scan bytes w-1 .. 0 for the first that is not 128
+    bool decided = false;
+    int carry = 0;
+    lower = sh ? (word << (32u - sh)) : 0u;            // bytes below w in this word, aligned to the top
+    for (uint32_t q = 0; q < sh && !decided; q += 8) {
+        const uint32_t b = (lower >> 24) & 0xFFu;
+        lower <<= 8;
+        if (b != 128u) { carry = b > 128u; decided = true; }
     }
-    return raw > 128 ? raw - 256 : raw;
+#pragma unroll
+    for (int i = 7; i >= 0; --i) {
+        if (decided || (uint32_t)i >= (w >> 2)) continue;
+        uint32_t x = m[i];
+        for (int q = 0; q < 4 && !decided; ++q) {
+            const uint32_t b = x >> 24;
+            x <<= 8;
+            if (b != 128u) { carry = b > 128u; decided = true; }
+        }
+    }
+    raw += carry;
+    const int dg = raw > 128 ? raw - 256 : raw;
+    return flip ? -dg : dg;
 }
 
 // partial[(sum * MW + w) * nseg + seg] = sum over the segment's elements of digit_w(s) * base.
@@ -315,7 +350,7 @@ __global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, con
             uint32_t left = 0;
             for (uint32_t e = e0 + t, i = 0; e < e1; e += MT, ++i) {
                 if ((done >> i) & 1u) continue;
-                const int dg = msm_digit(reinterpret_cast<const uint32_t*>(S + ((size_t)e * d.s_mul + d.s_off)), w);
+                const int dg = msm_digit(S[(size_t)e * d.s_mul + d.s_off], w);
                 if (dg != 0) {
                     const uint32_t mag = (uint32_t)(dg < 0 ? -dg : dg);
                     const uint32_t pos = atomicAdd(&cnt[mag - 1], 1u);
@@ -599,7 +634,7 @@ static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, con
     keep.emplace_back(new Scratch(sizeof(Fr) * (n0 + (size_t)levels + 1)));
     Scratch& sl = *keep.back();
     const int n_msm = 3 * levels + 1;
-    const uint32_t nseg = cdiv(n0, MSEG);
+    const uint32_t nseg = 1, cps = cdiv(n0, MSEG);       // one workgroup per (sum, window): buckets are reduced once
     Scratch aff(sizeof(G1Affine) * n0), coef(sizeof(Fr) * (size_t)n_msm * n0), partial(sizeof(G1Jac) * n_msm * MW * nseg), wsum(sizeof(G1Jac) * n_msm * MW);
     if (sl.rc) return sl.rc;
     if (aff.rc) return aff.rc;
@@ -615,7 +650,7 @@ static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, con
         const uint32_t slot = !live ? 0u : (i == 3 * levels ? 3u * (uint32_t)rounds : 3u * (uint32_t)r0 + (uint32_t)i);
         descs.d[i] = MsmDesc{coef.as<Fr>() + (live ? (size_t)i * n0 : 0), live ? (uint32_t)n0 : 0u, 1u, 0u, 1u, 0u, slot};
     }
-    hipLaunchKernelGGL(k_msm_seg<TAIL_SUMS>, dim3(nseg, MW, n_msm), dim3(MT), 0, st, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff.as<G1Affine>(), descs, nseg, 1u);
+    hipLaunchKernelGGL(k_msm_seg<TAIL_SUMS>, dim3(nseg, MW, n_msm), dim3(MT), 0, st, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff.as<G1Affine>(), descs, nseg, cps);
     if (nseg > 1) hipLaunchKernelGGL(k_g1_rowsum, dim3(n_msm * MW, 1), dim3(GT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), (size_t)nseg, 1u);
     hipLaunchKernelGGL(k_msm_horner, dim3(n_msm), dim3(GT), 0, st, pts, wsum.as<G1Jac>(), descs);
     ZK_LAUNCH_CHECK();

@@ -10,8 +10,8 @@
 //    product reduced on its own.  The R^-1 factor is removed once per output.
 //  * small-integer: when both operands are embeddings of int32-range values and the whole dot
 //    product is bounded by 2^62, the same sum is computed in int64 and embedded at the end.
-//    The bound is established on the device from the operands (max |a|, max |b|, N); nothing is
-//    assumed.  This is the case for every matmul of the LLaMa pipeline except softmax(Y)*V.
+//    The bound is established on the device from the operands (largest row sum of |a| times max |b|);
+//    nothing is assumed.  This is the case for every matmul of the LLaMa pipeline except softmax(Y)*V.
 #include <cstring>
 #include "field.hpp"
 #include "rt.hpp"
@@ -163,6 +163,34 @@ __global__ void __launch_bounds__(256) k_absmax(unsigned long long* __restrict__
     }
     if (threadIdx.x == 0) atomicMax(out, red[0]);
 }
+// max over rows of sum_j |a[row][j]| (saturating): with max |b| it bounds every dot product more tightly than
+// N * max|a| * max|b| does -- rows of a softmax output sum to its scale however long they are.
+__global__ void __launch_bounds__(256) k_rowabs(unsigned long long* __restrict__ out, const Fr* __restrict__ a, uint32_t ncol) {
+    const Fr* row = a + (size_t)blockIdx.x * ncol;
+    unsigned long long m = 0;
+    for (uint32_t j = threadIdx.x; j < ncol; j += 256) {
+        const Fr x = row[j];
+        unsigned long long v;
+        if (!(x.v[2] | x.v[3] | x.v[4] | x.v[5] | x.v[6] | x.v[7])) v = (unsigned long long)x.v[0] | ((unsigned long long)x.v[1] << 32);
+        else {
+            const Fr y = neg(x);
+            v = (y.v[2] | y.v[3] | y.v[4] | y.v[5] | y.v[6] | y.v[7]) ? ~0ull : ((unsigned long long)y.v[0] | ((unsigned long long)y.v[1] << 32));
+        }
+        if (v > (1ull << 62)) v = ~0ull;
+        m = (m == ~0ull || v == ~0ull || m + v > (1ull << 62)) ? ~0ull : m + v;
+    }
+    __shared__ unsigned long long red[256];
+    red[threadIdx.x] = m;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if (threadIdx.x < s) {
+            const unsigned long long x = red[threadIdx.x], y = red[threadIdx.x + s];
+            red[threadIdx.x] = (x == ~0ull || y == ~0ull || x + y > (1ull << 62)) ? ~0ull : x + y;
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) atomicMax(out, red[0]);
+}
 template <typename T> __global__ void __launch_bounds__(256) k_fr_to_int(T* __restrict__ out, const Fr* __restrict__ a, size_t n) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) out[i] = (T)fr_to_i64(a[i]);
@@ -245,22 +273,23 @@ int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, 
     ZK_ARG(mode >= 0 && mode <= 2, "zk_fr_matmul: mode must be 0, 1 or 2");
     bool small = false, fits32 = false;
     if (mode != 1) {
-        Scratch mx(2 * sizeof(unsigned long long));
+        Scratch mx(3 * sizeof(unsigned long long));
         if (mx.rc) return mx.rc;
-        ZK_HIP(hipMemsetAsync(mx.p, 0, 2 * sizeof(unsigned long long), st));
+        ZK_HIP(hipMemsetAsync(mx.p, 0, 3 * sizeof(unsigned long long), st));
         const size_t na = (size_t)M * N, nb = (size_t)N * P;
         hipLaunchKernelGGL(k_absmax, dim3(absmax_grid(na)), dim3(256), 0, st, mx.as<unsigned long long>(), (const Fr*)A, na);
         hipLaunchKernelGGL(k_absmax, dim3(absmax_grid(nb)), dim3(256), 0, st, mx.as<unsigned long long>() + 1, (const Fr*)B, nb);
+        hipLaunchKernelGGL(k_rowabs, dim3(M), dim3(256), 0, st, mx.as<unsigned long long>() + 2, (const Fr*)A, N);
         ZK_LAUNCH_CHECK();
         void* stage = nullptr;
-        int rc = staging(&stage, 16);
+        int rc = staging(&stage, 24);
         if (rc) return rc;
-        ZK_HIP(hipMemcpyAsync(stage, mx.p, 16, hipMemcpyDeviceToHost, st));
+        ZK_HIP(hipMemcpyAsync(stage, mx.p, 24, hipMemcpyDeviceToHost, st));
         ZK_HIP(hipStreamSynchronize(st));
-        const unsigned long long ma = ((unsigned long long*)stage)[0], mb = ((unsigned long long*)stage)[1];
-        if (ma != ~0ull && mb != ~0ull) {
-            // |sum| <= N * ma * mb must stay below 2^62
-            const unsigned __int128 bound = (unsigned __int128)ma * mb * N;
+        const unsigned long long ma = ((unsigned long long*)stage)[0], mb = ((unsigned long long*)stage)[1], ra = ((unsigned long long*)stage)[2];
+        if (ma != ~0ull && mb != ~0ull && ra != ~0ull) {
+            // |sum_j a_ij b_jk| <= (max_i sum_j |a_ij|) * max|b| must stay below 2^62
+            const unsigned __int128 bound = (unsigned __int128)ra * mb;
             small = bound < ((unsigned __int128)1 << 62);
             fits32 = ma < (1ull << 31) && mb < (1ull << 31);
         }
