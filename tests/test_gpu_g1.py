@@ -160,3 +160,21 @@ def test_open_value_and_g1_transcript(pv, orc, n, m):
     assert (val == exp_val).all()
     assert proof.shape == exp_proof.shape
     assert (norm(orc, proof) == norm(orc, exp_proof)).all()
+
+
+@pytest.mark.parametrize("n,val", [(300, 70000), (5000, -3), (5000, 0)])
+def test_open_with_equal_scalars(pv, orc, n, val):
+    """Every scalar in the same bucket of every window (norm weights share their high bytes; here all bytes): the
+    bucket sums must not depend on how the elements spread over the buckets."""
+    gens = oracle_gens(orc, 40 + n, n)
+    T = fr_array([val % R_MOD] * n)
+    k = (n - 1).bit_length()
+    u = mt_random_vec(np.random.RandomState(17), k)
+    exp_proof = np.zeros((3 * k + 1, 36), np.uint32)
+    exp_val = np.zeros(8, np.uint32)
+    orc_check(orc.orc_open(gens, n, T, n, 1, u, k, exp_proof, exp_val))
+    hG, hT = pv.g1_from_host(gens), pv.from_fr(T)
+    com = pv.commit_int(hG, hT)
+    val_got, proof = pv.open(hG, hT, com, u)
+    assert (val_got == exp_val).all()
+    assert (norm(orc, proof) == norm(orc, exp_proof)).all()

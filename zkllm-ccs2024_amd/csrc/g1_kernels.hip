@@ -233,7 +233,7 @@ static constexpr int MW = 32;        // 8-bit signed windows over a 255-bit scal
 static constexpr int MT = 128;       // lanes of a bucket workgroup = buckets (digit magnitudes 1..128)
 static constexpr int MSEG = 4096;    // elements per chunk (12-bit list entries)
 static constexpr int MCAP = 96;      // list slots per bucket and pass
-struct MsmDesc { const Fr* scalars; uint32_t count, s_mul, s_off, b_mul, b_off, slot; };   // element i: scalar scalars[i*s_mul+s_off], base A[i*b_mul+b_off]
+struct MsmDesc { const int8_t* digits; uint32_t dstride, count, s_mul, s_off, b_mul, b_off, slot; };   // element i: recoded scalar i*s_mul+s_off of dstride, base A[i*b_mul+b_off]
 template <int NMAX> struct MsmDescs { MsmDesc d[NMAX]; };
 static constexpr int TAIL_N = 8192;        // generators at which the remaining rounds are computed in one batch
 static constexpr int TAIL_LEVELS = 20;     // most rounds the batch takes
@@ -278,109 +278,42 @@ static __device__ __attribute__((noinline)) G1Jac g1_mul_glv(const G1Jac& P, con
     return out;
 }
 
-// signed 8-bit digit of window w of the scalar's balanced representative: s above r/2 is replaced by -(r - s), so
-// that small negative values (r - x, as weights are embedded) have as few non-zero windows as small positive ones
-// instead of sharing r's high bytes.  Within the magnitude, a digit above 128 is replaced by digit - 256 and carries
-// one; the carry into window w only depends on the first lower byte that is not 128.
-__device__ __forceinline__ int msm_digit(const Fr& sv, uint32_t w) {
-    // r - s, and whether it is the smaller of the two (s = 0 keeps s)
-    Fr n;
+// Signed 8-bit digits of the balanced representative of every scalar, written window-major: D[w*n + i] in [-128, 127]
+// for w < MW, and D[MW*n + i] = 1 when the scalar was replaced by r - s (its point is then subtracted).  Taking the
+// smaller of s and r - s gives small negative values (r - x, as weights are embedded) as few non-zero windows as
+// small positive ones, instead of r's high bytes in every one of them.  A window byte above 127 becomes byte - 256
+// and carries one into the next window; the top window of a value below 2^254 cannot overflow.
+__global__ void __launch_bounds__(256) k_msm_recode(int8_t* __restrict__ D, const Fr* __restrict__ S, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const Fr sv = S[i];
+    Fr ng;
     uint32_t br = 0;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) n.v[i] = subb32(FrK::P(i), sv.v[i], br);
-    uint32_t lt = 0;    // borrow of n - s: n < s
+    for (int l = 0; l < 8; ++l) ng.v[l] = subb32(FrK::P(l), sv.v[l], br);
+    uint32_t lt = 0;    // borrow of (r - s) - s: r - s is the smaller one
 #pragma unroll
-    for (int i = 0; i < 8; ++i) (void)subb32(n.v[i], sv.v[i], lt);
+    for (int l = 0; l < 8; ++l) (void)subb32(ng.v[l], sv.v[l], lt);
     const bool flip = lt != 0;
-    uint32_t m[8];
+    uint32_t carry = 0;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) m[i] = flip ? n.v[i] : sv.v[i];
-    uint32_t word = 0, lower = 0;      // the word holding byte w, and the bytes below it in that word
+    for (int l = 0; l < 8; ++l) {
+        const uint32_t word = flip ? ng.v[l] : sv.v[l];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) if ((w >> 2) == (uint32_t)i) word = m[i];
-    const uint32_t sh = (w & 3u) * 8u;
-    int raw = (int)((word >> sh) & 0xFFu);
-    // carry from below: scan bytes w-1 .. 0 for the first that is not 128
-    bool decided = false;
-    int carry = 0;
-    lower = sh ? (word << (32u - sh)) : 0u;            // bytes below w in this word, aligned to the top
-    for (uint32_t q = 0; q < sh && !decided; q += 8) {
-        const uint32_t b = (lower >> 24) & 0xFFu;
-        lower <<= 8;
-        if (b != 128u) { carry = b > 128u; decided = true; }
-    }
-#pragma unroll
-    for (int i = 7; i >= 0; --i) {
-        if (decided || (uint32_t)i >= (w >> 2)) continue;
-        uint32_t x = m[i];
-        for (int q = 0; q < 4 && !decided; ++q) {
-            const uint32_t b = x >> 24;
-            x <<= 8;
-            if (b != 128u) { carry = b > 128u; decided = true; }
+        for (int q = 0; q < 4; ++q) {
+            uint32_t raw = ((word >> (8 * q)) & 0xFFu) + carry;
+            carry = raw > 127u ? 1u : 0u;
+            D[(size_t)(4 * l + q) * n + i] = (int8_t)(raw > 127u ? (int)raw - 256 : (int)raw);
         }
     }
-    raw += carry;
-    const int dg = raw > 128 ? raw - 256 : raw;
-    return flip ? -dg : dg;
+    D[(size_t)MW * n + i] = flip ? 1 : 0;
 }
 
-// partial[(sum * MW + w) * nseg + seg] = sum over the segment's elements of digit_w(s) * base.
-// Lane t owns the bucket of magnitude t+1.  Per chunk the elements are first sorted into per-bucket lists in LDS
-// (one atomic per element), then every lane walks its own list with mixed additions, so lanes stay busy in
-// lockstep whatever the digits are; elements that find their bucket's list full wait for the next pass over the chunk.
-template <int NMAX>
-__global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, const G1Affine* __restrict__ A, const MsmDescs<NMAX> descs, uint32_t nseg, uint32_t chunks_per_seg) {
-    __shared__ uint32_t cnt[MT];
-    __shared__ uint32_t pool[MCAP * MT / 2];       // u16 lists while accumulating, the 36 x MT point tree afterwards
-    static_assert(MCAP * MT / 2 >= 36 * MT, "pool too small for the point tree");
-    static_assert(MSEG / MT == 32, "one done-bit per element of a lane's chunk share");
-    uint16_t* list = reinterpret_cast<uint16_t*>(pool);
-    const MsmDesc d = descs.d[blockIdx.z];
-    const Fr* __restrict__ S = d.scalars;
-    const uint32_t w = blockIdx.y, seg = blockIdx.x, t = threadIdx.x;
-    G1Jac acc = g1_infinity();
-    for (uint32_t ch = 0; ch < chunks_per_seg; ++ch) {
-        const uint32_t e0 = (seg * chunks_per_seg + ch) * MSEG;
-        if (e0 >= d.count) break;
-        const uint32_t e1 = (e0 + MSEG < d.count) ? e0 + MSEG : d.count;
-        uint32_t done = 0;                      // bit i: this lane's i-th element of the chunk is in a list already (MSEG / MT = 32 per lane)
-        for (;;) {
-            cnt[t] = 0;
-            __syncthreads();
-            uint32_t left = 0;
-            for (uint32_t e = e0 + t, i = 0; e < e1; e += MT, ++i) {
-                if ((done >> i) & 1u) continue;
-                const int dg = msm_digit(S[(size_t)e * d.s_mul + d.s_off], w);
-                if (dg != 0) {
-                    const uint32_t mag = (uint32_t)(dg < 0 ? -dg : dg);
-                    const uint32_t pos = atomicAdd(&cnt[mag - 1], 1u);
-                    if (pos >= (uint32_t)MCAP) { left = 1; continue; }
-                    list[pos * MT + (mag - 1)] = (uint16_t)((e - e0) | (dg < 0 ? 0x8000u : 0u));
-                }
-                done |= 1u << i;
-            }
-            __syncthreads();
-            const uint32_t c = cnt[t];
-            const uint32_t mine = c < (uint32_t)MCAP ? c : (uint32_t)MCAP;
-            for (uint32_t k = 0; k < mine; ++k) {
-                const uint32_t en = list[k * MT + t];
-                G1Affine pt = A[(size_t)(e0 + (en & 0x7FFFu)) * d.b_mul + d.b_off];
-                if (aff_is_inf(pt)) continue;
-                if (en & 0x8000u) pt.y = neg(pt.y);
-                acc = g1_add_mixed(acc, pt);
-            }
-            if (!__syncthreads_or((int)left)) break;
-        }
-    }
-    // bucket value t+1 times the bucket, then the sum over the lanes
-    G1Jac r = g1_infinity();
-    for (int bit = 7; bit >= 0; --bit) {
-        r = g1_double(r);
-        if (((t + 1) >> bit) & 1u) r = g1_add(r, acc);
-    }
+// sum over the MT lanes of a workgroup through the LDS pool (36 x MT words); every lane returns the total
+__device__ __forceinline__ G1Jac msm_block_sum(uint32_t* pool, const G1Jac& v, uint32_t t) {
     __syncthreads();
     {
-        const uint32_t* src = reinterpret_cast<const uint32_t*>(&r);
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(&v);
 #pragma unroll
         for (int l = 0; l < 36; ++l) pool[l * MT + t] = src[l];
     }
@@ -398,13 +331,87 @@ __global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, con
         }
         __syncthreads();
     }
-    if (t == 0) {
-        G1Jac tot;
-        uint32_t* pr = reinterpret_cast<uint32_t*>(&tot);
+    G1Jac tot;
+    uint32_t* pr = reinterpret_cast<uint32_t*>(&tot);
 #pragma unroll
-        for (int l = 0; l < 36; ++l) pr[l] = pool[l * MT];
-        partial[((size_t)blockIdx.z * MW + w) * nseg + seg] = tot;
+    for (int l = 0; l < 36; ++l) pr[l] = pool[l * MT];
+    __syncthreads();
+    return tot;
+}
+
+// partial[(sum * MW + w) * nseg + seg] = sum over the segment's elements of digit_w(s) * base.
+// Lane t owns the bucket of magnitude t+1.  Per chunk of MSEG elements:
+//  1. the bucket sizes are counted (one LDS atomic per element);
+//  2. a bucket with more than MCAP elements (scalars that share a digit: equal values, a common high byte) is summed by
+//     all lanes together, each over its own share of the chunk, and handed to its owner -- no lane ever walks a long list;
+//  3. the other elements are sorted into per-bucket lists in LDS and every lane walks its own list with mixed
+//     additions, in lockstep whatever the digits are.
+template <int NMAX>
+__global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, const G1Affine* __restrict__ A, const MsmDescs<NMAX> descs, uint32_t nseg, uint32_t chunks_per_seg) {
+    __shared__ uint32_t cnt[MT], cnt2[MT];
+    __shared__ uint32_t pool[MCAP * MT / 2];       // u16 lists, or the 36 x MT point tree
+    static_assert(MCAP * MT / 2 >= 36 * MT, "pool too small for the point tree");
+    uint16_t* list = reinterpret_cast<uint16_t*>(pool);
+    const MsmDesc d = descs.d[blockIdx.z];
+    const uint32_t w = blockIdx.y, seg = blockIdx.x, t = threadIdx.x;
+    const int8_t* __restrict__ Dw = d.digits + (size_t)w * d.dstride;
+    const int8_t* __restrict__ Df = d.digits + (size_t)MW * d.dstride;
+    G1Jac acc = g1_infinity();
+    for (uint32_t ch = 0; ch < chunks_per_seg; ++ch) {
+        const uint32_t e0 = (seg * chunks_per_seg + ch) * MSEG;
+        if (e0 >= d.count) break;
+        const uint32_t e1 = (e0 + MSEG < d.count) ? e0 + MSEG : d.count;
+        cnt[t] = 0;
+        cnt2[t] = 0;
+        __syncthreads();
+        for (uint32_t e = e0 + t; e < e1; e += MT) {
+            const int dg = Dw[(size_t)e * d.s_mul + d.s_off];
+            if (dg != 0) atomicAdd(&cnt[(dg < 0 ? -dg : dg) - 1], 1u);
+        }
+        __syncthreads();
+        for (uint32_t b = 0; b < (uint32_t)MT; ++b) {
+            if (cnt[b] <= (uint32_t)MCAP) continue;          // the same for every lane
+            G1Jac h = g1_infinity();
+            for (uint32_t e = e0 + t; e < e1; e += MT) {
+                const size_t si = (size_t)e * d.s_mul + d.s_off;
+                const int dg = Dw[si];
+                if ((uint32_t)(dg < 0 ? -dg : dg) != b + 1) continue;
+                G1Affine pt = A[(size_t)e * d.b_mul + d.b_off];
+                if (aff_is_inf(pt)) continue;
+                if ((dg < 0) != (Df[si] != 0)) pt.y = neg(pt.y);
+                h = g1_add_mixed(h, pt);
+            }
+            h = msm_block_sum(pool, h, t);
+            if (t == b) acc = g1_add(acc, h);
+        }
+        for (uint32_t e = e0 + t; e < e1; e += MT) {
+            const size_t si = (size_t)e * d.s_mul + d.s_off;
+            const int dg = Dw[si];
+            if (dg == 0) continue;
+            const uint32_t mag = (uint32_t)(dg < 0 ? -dg : dg);
+            if (cnt[mag - 1] > (uint32_t)MCAP) continue;
+            const uint32_t pos = atomicAdd(&cnt2[mag - 1], 1u);
+            list[pos * MT + (mag - 1)] = (uint16_t)((e - e0) | (((dg < 0) != (Df[si] != 0)) ? 0x8000u : 0u));
+        }
+        __syncthreads();
+        const uint32_t mine = cnt2[t];
+        for (uint32_t k = 0; k < mine; ++k) {
+            const uint32_t en = list[k * MT + t];
+            G1Affine pt = A[(size_t)(e0 + (en & 0x7FFFu)) * d.b_mul + d.b_off];
+            if (aff_is_inf(pt)) continue;
+            if (en & 0x8000u) pt.y = neg(pt.y);
+            acc = g1_add_mixed(acc, pt);
+        }
+        __syncthreads();
     }
+    // bucket value t+1 times the bucket, then the sum over the lanes
+    G1Jac r = g1_infinity();
+    for (int bit = 7; bit >= 0; --bit) {
+        r = g1_double(r);
+        if (((t + 1) >> bit) & 1u) r = g1_add(r, acc);
+    }
+    const G1Jac tot = msm_block_sum(pool, r, t);
+    if (t == 0) partial[((size_t)blockIdx.z * MW + w) * nseg + seg] = tot;
 }
 
 // The fold of one round plus the single-point work that rides along in spare workgroups:
@@ -589,10 +596,15 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     const uint32_t half = (uint32_t)(old_size / 2);
     const uint32_t n_msm = chained ? 2u : 3u;
     uint32_t q = 0;
-    if (!chained) descs.d[q++] = MsmDesc{scalars, (uint32_t)old_size, 1u, 0u, 1u, 0u, 0u};
-    descs.d[q++] = MsmDesc{scalars, half, 2u, 0u, 2u, 1u, 1u};
-    descs.d[q++] = MsmDesc{scalars, half, 2u, 1u, 2u, 0u, 2u};
-    for (; q < 3; ++q) descs.d[q] = MsmDesc{scalars, 0u, 1u, 0u, 1u, 0u, 0u};
+    Scratch dig((size_t)(MW + 1) * old_size);
+    if (dig.rc) return dig.rc;
+    hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(old_size, 256)), dim3(256), 0, st, dig.as<int8_t>(), scalars, old_size);
+    const int8_t* dg = dig.as<int8_t>();
+    const uint32_t ds = (uint32_t)old_size;
+    if (!chained) descs.d[q++] = MsmDesc{dg, ds, (uint32_t)old_size, 1u, 0u, 1u, 0u, 0u};
+    descs.d[q++] = MsmDesc{dg, ds, half, 2u, 0u, 2u, 1u, 1u};
+    descs.d[q++] = MsmDesc{dg, ds, half, 2u, 1u, 2u, 0u, 2u};
+    for (; q < 3; ++q) descs.d[q] = MsmDesc{dg, ds, 0u, 1u, 0u, 1u, 0u, 0u};
     const size_t count_max = chained ? half : old_size;
     const uint32_t chunks = count_max ? cdiv(count_max, MSEG) : 1u;
     const uint32_t nseg = chunks < 16u ? chunks : 16u;
@@ -644,11 +656,15 @@ static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, con
     hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(n0, CH), GT)), dim3(GT), 0, st, aff.p, gens, n0);
     hipLaunchKernelGGL(k_tail_scalars, dim3(1), dim3(1024), 0, st, sl.as<Fr>(), scalars, us, (uint32_t)n0, (uint32_t)levels);
     hipLaunchKernelGGL(k_tail_coeffs, dim3(cdiv(n0, 256)), dim3(256), 0, st, coef.as<Fr>(), sl.as<Fr>(), scalars, us, (uint32_t)n0, (uint32_t)levels);
+    const size_t ncoef = (size_t)n_msm * n0;
+    Scratch dig((size_t)(MW + 1) * ncoef);
+    if (dig.rc) return dig.rc;
+    hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(ncoef, 256)), dim3(256), 0, st, dig.as<int8_t>(), coef.as<Fr>(), ncoef);
     MsmDescs<TAIL_SUMS> descs;
     for (int i = 0; i < TAIL_SUMS; ++i) {
         const bool live = i < n_msm;
         const uint32_t slot = !live ? 0u : (i == 3 * levels ? 3u * (uint32_t)rounds : 3u * (uint32_t)r0 + (uint32_t)i);
-        descs.d[i] = MsmDesc{coef.as<Fr>() + (live ? (size_t)i * n0 : 0), live ? (uint32_t)n0 : 0u, 1u, 0u, 1u, 0u, slot};
+        descs.d[i] = MsmDesc{dig.as<int8_t>(), (uint32_t)ncoef, live ? (uint32_t)n0 : 0u, 1u, live ? (uint32_t)((size_t)i * n0) : 0u, 1u, 0u, slot};
     }
     hipLaunchKernelGGL(k_msm_seg<TAIL_SUMS>, dim3(nseg, MW, n_msm), dim3(MT), 0, st, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff.as<G1Affine>(), descs, nseg, cps);
     if (nseg > 1) hipLaunchKernelGGL(k_g1_rowsum, dim3(n_msm * MW, 1), dim3(GT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), (size_t)nseg, 1u);
