@@ -233,6 +233,7 @@ static constexpr int MW = 32;        // 8-bit signed windows over a 255-bit scal
 static constexpr int MT = 128;       // lanes of a bucket workgroup = buckets (digit magnitudes 1..128)
 static constexpr int MSEG = 4096;    // elements per chunk (12-bit list entries)
 static constexpr int MCAP = 96;      // list slots per bucket and pass
+static constexpr int MHEAVY = 256;   // a bucket above this many elements of a chunk is summed by the whole workgroup
 struct MsmDesc { const int8_t* digits; uint32_t dstride, count, s_mul, s_off, b_mul, b_off, slot; };   // element i: recoded scalar i*s_mul+s_off of dstride, base A[i*b_mul+b_off]
 template <int NMAX> struct MsmDescs { MsmDesc d[NMAX]; };
 static constexpr int TAIL_N = 8192;        // generators at which the remaining rounds are computed in one batch
@@ -342,15 +343,17 @@ __device__ __forceinline__ G1Jac msm_block_sum(uint32_t* pool, const G1Jac& v, u
 // partial[(sum * MW + w) * nseg + seg] = sum over the segment's elements of digit_w(s) * base.
 // Lane t owns the bucket of magnitude t+1.  Per chunk of MSEG elements:
 //  1. the bucket sizes are counted (one LDS atomic per element);
-//  2. a bucket with more than MCAP elements (scalars that share a digit: equal values, a common high byte) is summed by
-//     all lanes together, each over its own share of the chunk, and handed to its owner -- no lane ever walks a long list;
+//  2. a bucket with more than MHEAVY elements (scalars that share a digit: equal values, a common high byte) is summed by
+//     all lanes together, each over its own share of the chunk, and handed to its owner -- no lane walks a long list;
 //  3. the other elements are sorted into per-bucket lists in LDS and every lane walks its own list with mixed
-//     additions, in lockstep whatever the digits are.
+//     additions, in lockstep whatever the digits are; elements that find their bucket's list full (more than MCAP)
+//     wait for the next pass over the chunk.
 template <int NMAX>
 __global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, const G1Affine* __restrict__ A, const MsmDescs<NMAX> descs, uint32_t nseg, uint32_t chunks_per_seg) {
     __shared__ uint32_t cnt[MT], cnt2[MT];
     __shared__ uint32_t pool[MCAP * MT / 2];       // u16 lists, or the 36 x MT point tree
     static_assert(MCAP * MT / 2 >= 36 * MT, "pool too small for the point tree");
+    static_assert(MSEG / MT == 32, "one done-bit per element of a lane's share of a chunk");
     uint16_t* list = reinterpret_cast<uint16_t*>(pool);
     const MsmDesc d = descs.d[blockIdx.z];
     const uint32_t w = blockIdx.y, seg = blockIdx.x, t = threadIdx.x;
@@ -369,13 +372,15 @@ __global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, con
             if (dg != 0) atomicAdd(&cnt[(dg < 0 ? -dg : dg) - 1], 1u);
         }
         __syncthreads();
+        uint32_t done = 0;                       // bit i: this lane's i-th element of the chunk needs no more work (MSEG / MT = 32 per lane)
         for (uint32_t b = 0; b < (uint32_t)MT; ++b) {
-            if (cnt[b] <= (uint32_t)MCAP) continue;          // the same for every lane
+            if (cnt[b] <= (uint32_t)MHEAVY) continue;          // the same for every lane
             G1Jac h = g1_infinity();
-            for (uint32_t e = e0 + t; e < e1; e += MT) {
+            for (uint32_t e = e0 + t, i = 0; e < e1; e += MT, ++i) {
                 const size_t si = (size_t)e * d.s_mul + d.s_off;
                 const int dg = Dw[si];
                 if ((uint32_t)(dg < 0 ? -dg : dg) != b + 1) continue;
+                done |= 1u << i;
                 G1Affine pt = A[(size_t)e * d.b_mul + d.b_off];
                 if (aff_is_inf(pt)) continue;
                 if ((dg < 0) != (Df[si] != 0)) pt.y = neg(pt.y);
@@ -384,23 +389,33 @@ __global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, con
             h = msm_block_sum(pool, h, t);
             if (t == b) acc = g1_add(acc, h);
         }
-        for (uint32_t e = e0 + t; e < e1; e += MT) {
-            const size_t si = (size_t)e * d.s_mul + d.s_off;
-            const int dg = Dw[si];
-            if (dg == 0) continue;
-            const uint32_t mag = (uint32_t)(dg < 0 ? -dg : dg);
-            if (cnt[mag - 1] > (uint32_t)MCAP) continue;
-            const uint32_t pos = atomicAdd(&cnt2[mag - 1], 1u);
-            list[pos * MT + (mag - 1)] = (uint16_t)((e - e0) | (((dg < 0) != (Df[si] != 0)) ? 0x8000u : 0u));
-        }
-        __syncthreads();
-        const uint32_t mine = cnt2[t];
-        for (uint32_t k = 0; k < mine; ++k) {
-            const uint32_t en = list[k * MT + t];
-            G1Affine pt = A[(size_t)(e0 + (en & 0x7FFFu)) * d.b_mul + d.b_off];
-            if (aff_is_inf(pt)) continue;
-            if (en & 0x8000u) pt.y = neg(pt.y);
-            acc = g1_add_mixed(acc, pt);
+        for (;;) {
+            uint32_t left = 0;
+            for (uint32_t e = e0 + t, i = 0; e < e1; e += MT, ++i) {
+                if ((done >> i) & 1u) continue;
+                const size_t si = (size_t)e * d.s_mul + d.s_off;
+                const int dg = Dw[si];
+                if (dg != 0) {
+                    const uint32_t mag = (uint32_t)(dg < 0 ? -dg : dg);
+                    const uint32_t pos = atomicAdd(&cnt2[mag - 1], 1u);
+                    if (pos >= (uint32_t)MCAP) { left = 1; continue; }
+                    list[pos * MT + (mag - 1)] = (uint16_t)((e - e0) | (((dg < 0) != (Df[si] != 0)) ? 0x8000u : 0u));
+                }
+                done |= 1u << i;
+            }
+            __syncthreads();
+            const uint32_t c2 = cnt2[t];
+            const uint32_t mine = c2 < (uint32_t)MCAP ? c2 : (uint32_t)MCAP;
+            for (uint32_t k = 0; k < mine; ++k) {
+                const uint32_t en = list[k * MT + t];
+                G1Affine pt = A[(size_t)(e0 + (en & 0x7FFFu)) * d.b_mul + d.b_off];
+                if (aff_is_inf(pt)) continue;
+                if (en & 0x8000u) pt.y = neg(pt.y);
+                acc = g1_add_mixed(acc, pt);
+            }
+            if (!__syncthreads_or((int)left)) break;
+            cnt2[t] = 0;
+            __syncthreads();
         }
         __syncthreads();
     }
