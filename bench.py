@@ -7,8 +7,9 @@ projections, 32 attention heads (QK^T, zkSoftmax, YV), SwiGLU FFN, every rescali
 the opening of all nine weight commitments.  `value` is seconds per layer.
 
 The same JSON line also carries the two throughput figures of the headline metric (G1 MSM points/s on the
-4096 x 11008 commitment workload, Fr multiplications/s), a roofline entry for the dominant kernel timed
-live with HIP events, and a CPU baseline measured with the oracle on this host's cores.
+4096 x 11008 commitment workload, Fr multiplications/s), a roofline entry for the kernel with the largest share
+of the layer's GPU time (timed with HIP events around its launches inside the timed region), roofline entries of
+the generic Fr matmul and of an HBM-bound fold, and a CPU baseline measured with the oracle on this host's cores.
 """
 import argparse
 import ctypes
@@ -87,12 +88,15 @@ def main():
         for _ in range(args.warmup):
             pv.layer_run(layer, hX)
         pv.sync()
+        hip.check(lib.zk_prof_fold_begin())
         t0 = time.perf_counter()
         for _ in range(args.steps):
             _, times = pv.layer_run(layer, hX)
             parts += times
         pv.sync()
         wall = time.perf_counter() - t0
+        fold_ms, fold_launches, fold_mults, fold_pairs = ctypes.c_double(), ctypes.c_ulonglong(), ctypes.c_double(), ctypes.c_ulonglong()
+        hip.check(lib.zk_prof_fold_read(ctypes.byref(fold_ms), ctypes.byref(fold_launches), ctypes.byref(fold_mults), ctypes.byref(fold_pairs)))
     finally:
         os.dup2(saved_stdout, 1)
     ms_per_step = wall * 1e3 / args.steps
@@ -118,6 +122,18 @@ def main():
                    "setup_s_untimed": round(setup_s, 3),
                    "parts_ms": {k: round(float(v), 1) for k, v in zip(["rmsnorm1", "qkv", "attention", "oproj", "rmsnorm2", "ffn", "total"], parts)}},
     }
+    # roofline of the kernel with the largest share of the layer's GPU time: the generator fold of the openings
+    # (one endomorphism-split scalar multiplication per pair).  It is bound by 32-bit integer multiply-adds: an
+    # Fp multiplication is 2*12^2+12 = 300 of them.  Durations are HIP events around every launch inside the timed
+    # region above, on the launch stream.
+    MAD_PER_FP_MUL = 300
+    fold_tops = fold_mults.value * MAD_PER_FP_MUL / (fold_ms.value * 1e-3) / 1e12 if fold_ms.value > 0 else 0.0
+    out["roofline"] = {"kernel": "k_open_fold (opening: g' = g1 + [u](g0 - g1) per pair, 128-bit split scalars)", "bound": "valu-int",
+                       "achieved": fold_tops, "peak": VALU_PEAK_TOPS, "unit": "T MAD32/s", "frac": fold_tops / VALU_PEAK_TOPS, "traffic": None,
+                       "launches": int(fold_launches.value), "avg_launch_ms": fold_ms.value / max(1, fold_launches.value),
+                       "total_ms_in_timed_region": fold_ms.value, "pairs": int(fold_pairs.value), "fp_mul_per_s": fold_mults.value / (fold_ms.value * 1e-3) if fold_ms.value > 0 else 0.0,
+                       "note": "algorithmic work = Fp multiplications of the point formulas x 300 MAD32; peak = 256 CU x 4 SIMD x 16 lanes x 2.4 GHz; "
+                               "HBM traffic of this kernel is 336 B per pair, far below the bandwidth bound"}
     if args.skip_extras:
         print(json.dumps(out))
         return
@@ -163,37 +179,63 @@ def main():
     # (1) generic Fr matmul at the projection shape: M*N*P field multiplications, 136 MAD32 each (algorithmic)
     M, N, P = 2048, 4096, 4096
     mm_ms = time_kernel(lambda: hip.call("zk_fr_matmul_generic", c_void_p(dO), c_void_p(dA), c_void_p(dB), c_uint(M), c_uint(N), c_uint(P), None), reps=1)
-    mm_tops = M * N * P * 136 / (mm_ms * 1e-3) / 1e12
     # (2) fused multilinear fold (3 levels per pass) over a 2048 x 4096 tensor: 32 B read per element
     u = mt_random_vec(np.random.RandomState(2), 3)
     fold_ms = time_kernel(lambda: hip.call("zk_fr_fold_axis", c_void_p(dO), c_void_p(dA), u, c_int(3), c_size_t(1), c_uint(2048), c_size_t(4096), None), reps=10)
     fold_gbs = 32 * 2048 * 4096 / (fold_ms * 1e-3) / 1e9
-    out["roofline"] = {"kernel": "k_matmul (generic Montgomery Fr matmul, 2048x4096x4096)", "bound": "valu-int", "achieved": mm_tops, "peak": VALU_PEAK_TOPS,
-                       "unit": "T MAD32/s", "frac": mm_tops / VALU_PEAK_TOPS, "traffic": None,
-                       "note": "algorithmic 136 MAD32 per field multiplication; peak = 256 CU x 4 SIMD x 16 lanes x 2.4 GHz (v_mad_u64_u32 at full rate)",
-                       "avg_launch_ms": mm_ms, "gmac_per_s": M * N * P / (mm_ms * 1e-3) / 1e9}
+    mm_tops = M * N * P * 72 / (mm_ms * 1e-3) / 1e12
+    out["roofline_matmul"] = {"kernel": "k_matmul (generic Montgomery Fr matmul, 2048x4096x4096)", "bound": "valu-int", "achieved": mm_tops, "peak": VALU_PEAK_TOPS,
+                              "unit": "T MAD32/s", "frac": mm_tops / VALU_PEAK_TOPS, "traffic": None,
+                              "note": "algorithmic 72 MAD32 per field multiply-accumulate (64 limb products + 1/8 of a shared reduction); every MAD32 needs a second "
+                                      "VALU instruction for its carry, so 0.5 is the ceiling of this formulation",
+                              "avg_launch_ms": mm_ms, "gmac_per_s": M * N * P / (mm_ms * 1e-3) / 1e9}
     out["roofline_hbm"] = {"kernel": "k_fold_axis<3> (fused 3-level multilinear fold, 2048x4096)", "bound": "hbm", "achieved": fold_gbs, "peak": HBM_PEAK_GBS,
                            "unit": "GB/s", "frac": fold_gbs / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": fold_ms}
     for p in (dA, dB, dO, src):
         hip.free(p)
 
-    # ---- CPU baseline: the oracle's restatement of the reference's kernels on this host's cores ---------------------------------------
+    # ---- CPU baseline: the oracle's restatement of the reference's algorithm on this host's cores ---------------------------------------
+    # A bounded sample of the two costs that dominate the reference's layer: the field multiplications of the matrix products
+    # and the five 255-bit scalar multiplications per generator pair of the openings; both scaled to the layer's counts.
     if not args.skip_cpu:
         from zkhelp import load_oracle
         orc = load_oracle()
         cores = orc.dll.orc_num_threads()
-        rows = 2 * max(1, cores // 2)
-        A = mt_random_vec(np.random.RandomState(3), rows * 4096)
         B = mt_random_vec(np.random.RandomState(4), 4096 * 1024)
-        C = np.zeros((rows * 1024, 8), np.uint32)
-        t0 = time.perf_counter()
-        orc.orc_fr_matmul_rows(A, B, rows, 4096, 1024, rows, C)
-        dt = time.perf_counter() - t0
+
+        def mm_sample(rows):
+            A = mt_random_vec(np.random.RandomState(3), rows * 4096)
+            C = np.zeros((rows * 1024, 8), np.uint32)
+            t0 = time.perf_counter()
+            orc.orc_fr_matmul_rows(A, B, rows, 4096, 1024, rows, C)
+            return time.perf_counter() - t0
+        probe_rows = 2 * max(1, cores // 2)
+        dt = mm_sample(probe_rows)
+        rows = int(max(probe_rows, min(4096, probe_rows * 20.0 / max(dt, 1e-3)))) // max(1, cores) * max(1, cores)
+        rows = max(rows, probe_rows)
+        dt = mm_sample(rows)
         mm_rate = rows * 4096 * 1024 / dt                      # field multiplications per second, all cores
+        # opening sample: n generators, one row
+        n_open = 4096
+        gens = np.zeros((n_open, 36), np.uint32)
+        orc.orc_seed(99)
+        gens = np.zeros((n_open, 36), np.uint32)
+        orc.orc_commitment_random(n_open, gens)
+        T = mt_random_vec(np.random.RandomState(6), n_open)
+        k = 12
+        u = mt_random_vec(np.random.RandomState(7), k)
+        proof = np.zeros((3 * k + 1, 36), np.uint32)
+        val = np.zeros(8, np.uint32)
+        t0 = time.perf_counter()
+        orc.orc_open(gens, n_open, T, n_open, 1, u, k, proof, val)
+        open_s = time.perf_counter() - t0
         layer_mm = 4.49e11                                     # field multiplications in the layer's matrix products (reference algorithm)
-        out["cpu_baseline"] = {"value": layer_mm / mm_rate, "unit": "s", "cores": int(cores), "kind": "port",
-                               "sample": f"oracle Fr matmul (reference algorithm, OpenMP) on {rows} rows x 4096 x 1024 = {rows * 4096 * 1024:.3g} multiplications in {dt:.2f} s; "
-                                         f"scaled to the 4.49e11 multiplications of the layer's matrix products alone (lower bound of the CPU layer time)",
+        layer_gens = 5 * (4096 << 5) + 2 * (11008 << 5) + 2 * 4096   # generators of the nine openings; pairs over all rounds ~ the same number
+        cpu_s = layer_mm / mm_rate + open_s * layer_gens / n_open
+        out["cpu_baseline"] = {"value": cpu_s, "unit": "s", "cores": int(cores), "kind": "port",
+                               "sample": f"oracle (reference algorithm, OpenMP): Fr matmul {rows} x 4096 x 1024 = {rows * 4096 * 1024:.3g} multiplications in {dt:.1f} s, "
+                                         f"scaled to the layer's 4.49e11; opening of {n_open} generators in {open_s:.1f} s, scaled to the layer's "
+                                         f"{layer_gens} generators; sumchecks and lookups not included (lower bound of the CPU layer time)",
                                "fr_mul_per_s_all_cores": mm_rate}
     print(json.dumps(out))
 

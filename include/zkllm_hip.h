@@ -166,6 +166,11 @@ int zk_softmax_decompose(void* planes, const void* X_shifted, const uint32_t* bs
 int zk_bench_mad_peak(uint32_t blocks, uint32_t iters, double* mad_per_s_host, void* stream);
 /* plain 16-byte-per-lane copy of known size, to scale profiler byte counters */
 int zk_bench_copy(void* dst, const void* src, size_t bytes, void* stream);
+/* time the launches of the opening's fold kernel (the generator halving of me_open_step, commitment.cu:79-107) with
+ * events on their stream: everything between begin and read.  fp_mults: base-field multiplications those launches
+ * perform by the point formulas' count; pairs: generator pairs folded */
+int zk_prof_fold_begin(void);
+int zk_prof_fold_read(double* total_ms, unsigned long long* launches, double* fp_mults, unsigned long long* pairs);
 
 #ifdef __cplusplus
 }

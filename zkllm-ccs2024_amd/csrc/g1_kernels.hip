@@ -13,6 +13,7 @@
 // (a Jacobian triple depends on the order of additions, so bytes are compared after normalising).
 #include <cstring>
 #include <memory>
+#include <utility>
 #include <vector>
 #include "g1.hpp"
 #include "rt.hpp"
@@ -583,6 +584,26 @@ static int g1_sum_device(G1Jac* out, const G1Jac* in, size_t n, hipStream_t st) 
     return 0;
 }
 
+// Optional timing of the fold kernel's launches with events on its own stream (measurement only).
+struct FoldTimer {
+    bool on = false;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> ev;
+    double fp_mults = 0;      // Fp multiplications the timed launches perform by the formulas' count
+    unsigned long long pairs = 0;
+};
+static FoldTimer g_fold_timer;
+// Fp multiplications of one pair of the fold: difference (11), endomorphism (1), P+Q (16), the double-and-add walk
+// (7 per doubling from the top set bit, 16 per non-zero bit pair), final mixed addition (11), two 8-limb products aside
+static double fold_fp_mults_per_pair(const GlvK& k) {
+    int top = -1, adds = 0;
+    for (int i = 127; i >= 0; --i) {
+        const uint32_t b = ((k.k1[i >> 5] >> (i & 31)) & 1u) | ((k.k2[i >> 5] >> (i & 31)) & 1u);
+        if (b && top < 0) top = i;
+        adds += (int)b;
+    }
+    return 11.0 + 1.0 + 16.0 + 7.0 * (top + 1) + 16.0 * adds + 11.0;
+}
+
 // u = k1 + k2 * lambda with 0 <= k1 < lambda and k2 <= lambda + 1 (r = lambda^2 + lambda + 1): one long division
 static GlvK glv_split(const Fr& u) {
     const unsigned __int128 lam = ((unsigned __int128)0xac45a4010001a402ull << 64) | 0x00000000ffffffffull;
@@ -645,8 +666,21 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
         ex.kc[2] = glv_split(fr_mul_std(pu, pu));
     }
     const uint32_t nb_main = cdiv(new_size, GT);
-    hipLaunchKernelGGL(k_open_fold, dim3(nb_main + n_msm + (chained ? 3u : 0u)), dim3(GT), 0, st, new_scalars, new_gens, scalars, aff.as<G1Affine>(), to_mont(u), glv_split(u),
+    const GlvK ku = glv_split(u);
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    if (g_fold_timer.on) {
+        ZK_HIP(hipEventCreate(&t0));
+        ZK_HIP(hipEventCreate(&t1));
+        ZK_HIP(hipEventRecord(t0, st));
+    }
+    hipLaunchKernelGGL(k_open_fold, dim3(nb_main + n_msm + (chained ? 3u : 0u)), dim3(GT), 0, st, new_scalars, new_gens, scalars, aff.as<G1Affine>(), to_mont(u), ku,
                        old_size, new_size, nb_main, ex);
+    if (g_fold_timer.on) {
+        ZK_HIP(hipEventRecord(t1, st));
+        g_fold_timer.ev.emplace_back(t0, t1);
+        g_fold_timer.fp_mults += fold_fp_mults_per_pair(ku) * (double)new_size;
+        g_fold_timer.pairs += new_size;
+    }
     ZK_LAUNCH_CHECK();
     return 0;
 }
@@ -916,6 +950,34 @@ int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* sc
     ZK_HIP(hipStreamSynchronize(st));
     memcpy(proof_host, stage, sizeof(G1Jac) * npts);
     memcpy(final_scalar_host, (char*)stage + sizeof(G1Jac) * npts, sizeof(Fr));
+    return 0;
+}
+
+// Measurement: time every launch of the opening's fold kernel between begin and read with events on the launch stream.
+int zk_prof_fold_begin(void) {
+    for (auto& e : g_fold_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
+    g_fold_timer.ev.clear();
+    g_fold_timer.fp_mults = 0;
+    g_fold_timer.pairs = 0;
+    g_fold_timer.on = true;
+    return 0;
+}
+// total_ms / launches: summed durations and number of timed launches; fp_mults: Fp multiplications they performed; pairs: pairs folded
+int zk_prof_fold_read(double* total_ms, unsigned long long* launches, double* fp_mults, unsigned long long* pairs) {
+    g_fold_timer.on = false;
+    double tot = 0;
+    for (auto& e : g_fold_timer.ev) {
+        ZK_HIP(hipEventSynchronize(e.second));
+        float ms = 0;
+        ZK_HIP(hipEventElapsedTime(&ms, e.first, e.second));
+        tot += ms;
+    }
+    *total_ms = tot;
+    *launches = g_fold_timer.ev.size();
+    *fp_mults = g_fold_timer.fp_mults;
+    *pairs = g_fold_timer.pairs;
+    for (auto& e : g_fold_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
+    g_fold_timer.ev.clear();
     return 0;
 }
 
