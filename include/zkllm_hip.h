@@ -130,6 +130,13 @@ int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host108, 
  * then the folded generator -- normalised to z = 1; final_scalar_host: the folded scalar (8 limbs).  The generators
  * must lie in the order-r subgroup (Commitment::random, :9-20, only produces such points). */
 int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stream);
+/* zk_g1_open in two halves, for callers that prove on while a weight is being opened (the reference opens each weight
+ * in place, verifyWeightClaim proof.cu:9-15; the opening depends on nothing the prover does afterwards).  begin
+ * queues the recursion on a stream of the library's own, ordered after the work queued on `stream` so far, and
+ * returns; scalars and gens must stay alive and unmodified until end.  end waits, delivers what zk_g1_open
+ * delivers, and releases the opening's buffers; every handle must be ended exactly once. */
+int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stream);
+int zk_g1_open_end(void* handle, uint32_t* proof_host, uint32_t* final_scalar_host);
 
 /* ---- lookup argument (tlookup.cu) ------------------------------------------------------------------------ */
 /* idx = val - low as a table index (lookuprange_tensor_prep_kernel :414-421 / lookuprange_prep_kernel :393-400);

@@ -584,6 +584,13 @@ static int g1_sum_device(G1Jac* out, const G1Jac* in, size_t n, hipStream_t st) 
     return 0;
 }
 
+// Device buffers of one opening, all released together once its stream has drained: an opening may run on a
+// stream of its own, so none of its buffers may return to the allocator while its kernels are pending.
+struct Arena {
+    std::vector<std::unique_ptr<Scratch>> v;
+    Scratch& add(size_t bytes) { v.emplace_back(new Scratch(bytes)); return *v.back(); }
+};
+
 // Optional timing of the fold kernel's launches with events on its own stream (measurement only).
 struct FoldTimer {
     bool on = false;
@@ -621,18 +628,18 @@ static GlvK glv_split(const Fr& u) {
 // Queues one round.  round > 0 with prev_u: T comes from the previous round's points (pts_prev, rec[3*(round-1)..]);
 // otherwise T is a third bucket sum.  pts_round: this round's T, T0, T1 (T of later rounds is left to k_open_finish).
 static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars, const G1Jac* gens, const Fr& u, size_t old_size, int round, const Fr* prev_u,
-                             G1Jac* pts_round, const G1Jac* pts_prev, G1Jac* rec, hipStream_t st) {
+                             G1Jac* pts_round, const G1Jac* pts_prev, G1Jac* rec, Arena& arena, hipStream_t st) {
     ZK_ARG(old_size < (1ull << 31), "opening: more than 2^31 generators");
     const size_t new_size = (old_size + 1) / 2;
     const bool chained = round > 0 && prev_u != nullptr;
-    Scratch aff(sizeof(G1Affine) * old_size);
+    Scratch& aff = arena.add(sizeof(G1Affine) * old_size);
     if (aff.rc) return aff.rc;
     hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(old_size, CH), GT)), dim3(GT), 0, st, aff.p, gens, old_size);
     MsmDescs<3> descs;
     const uint32_t half = (uint32_t)(old_size / 2);
     const uint32_t n_msm = chained ? 2u : 3u;
     uint32_t q = 0;
-    Scratch dig((size_t)(MW + 1) * old_size);
+    Scratch& dig = arena.add((size_t)(MW + 1) * old_size);
     if (dig.rc) return dig.rc;
     hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(old_size, 256)), dim3(256), 0, st, dig.as<int8_t>(), scalars, old_size);
     const int8_t* dg = dig.as<int8_t>();
@@ -645,7 +652,8 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     const uint32_t chunks = count_max ? cdiv(count_max, MSEG) : 1u;
     const uint32_t nseg = chunks < 16u ? chunks : 16u;
     const uint32_t cps = (chunks + nseg - 1) / nseg;
-    Scratch partial(sizeof(G1Jac) * n_msm * MW * nseg), wsum(sizeof(G1Jac) * n_msm * MW);
+    Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * nseg);
+    Scratch& wsum = arena.add(sizeof(G1Jac) * n_msm * MW);
     if (partial.rc) return partial.rc;
     if (wsum.rc) return wsum.rc;
     hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MT), 0, st, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff.as<G1Affine>(), descs, nseg, cps);
@@ -688,15 +696,17 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
 // Queues the batch for the last `levels` rounds (rounds r0 .. r0+levels-1 of `rounds`) over n0 <= TAIL_N generators.
 // Writes T, T0, T1 of those rounds and the final generator into pts; *final_scalar points at the folded scalar.
 static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, const uint32_t* u, int levels, int r0, int rounds, G1Jac* pts, const Fr** final_scalar,
-                            std::vector<std::unique_ptr<Scratch>>& keep, hipStream_t st) {
+                            Arena& arena, hipStream_t st) {
     TailU us;
     for (int j = 0; j < levels; ++j) us.u[j] = to_mont(load_fr(u + 8 * j));
     for (int j = levels; j < TAIL_LEVELS; ++j) us.u[j] = big_zero<8>();
-    keep.emplace_back(new Scratch(sizeof(Fr) * (n0 + (size_t)levels + 1)));
-    Scratch& sl = *keep.back();
+    Scratch& sl = arena.add(sizeof(Fr) * (n0 + (size_t)levels + 1));
     const int n_msm = 3 * levels + 1;
     const uint32_t nseg = 1, cps = cdiv(n0, MSEG);       // one workgroup per (sum, window): buckets are reduced once
-    Scratch aff(sizeof(G1Affine) * n0), coef(sizeof(Fr) * (size_t)n_msm * n0), partial(sizeof(G1Jac) * n_msm * MW * nseg), wsum(sizeof(G1Jac) * n_msm * MW);
+    Scratch& aff = arena.add(sizeof(G1Affine) * n0);
+    Scratch& coef = arena.add(sizeof(Fr) * (size_t)n_msm * n0);
+    Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * nseg);
+    Scratch& wsum = arena.add(sizeof(G1Jac) * n_msm * MW);
     if (sl.rc) return sl.rc;
     if (aff.rc) return aff.rc;
     if (coef.rc) return coef.rc;
@@ -706,7 +716,7 @@ static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, con
     hipLaunchKernelGGL(k_tail_scalars, dim3(1), dim3(1024), 0, st, sl.as<Fr>(), scalars, us, (uint32_t)n0, (uint32_t)levels);
     hipLaunchKernelGGL(k_tail_coeffs, dim3(cdiv(n0, 256)), dim3(256), 0, st, coef.as<Fr>(), sl.as<Fr>(), scalars, us, (uint32_t)n0, (uint32_t)levels);
     const size_t ncoef = (size_t)n_msm * n0;
-    Scratch dig((size_t)(MW + 1) * ncoef);
+    Scratch& dig = arena.add((size_t)(MW + 1) * ncoef);
     if (dig.rc) return dig.rc;
     hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(ncoef, 256)), dim3(256), 0, st, dig.as<int8_t>(), coef.as<Fr>(), ncoef);
     MsmDescs<TAIL_SUMS> descs;
@@ -879,7 +889,8 @@ int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host, con
     ZK_ARG(old_size >= 1, "zk_g1_open_round: empty input");
     Scratch pts(sizeof(G1Jac) * 3);
     if (pts.rc) return pts.rc;
-    int rc = open_round_launch((Fr*)new_scalars, (G1Jac*)new_gens, (const Fr*)scalars, (const G1Jac*)gens, load_fr(u), old_size, 0, nullptr, pts.as<G1Jac>(), nullptr, nullptr, st);
+    Arena arena;
+    int rc = open_round_launch((Fr*)new_scalars, (G1Jac*)new_gens, (const Fr*)scalars, (const G1Jac*)gens, load_fr(u), old_size, 0, nullptr, pts.as<G1Jac>(), nullptr, nullptr, arena, st);
     if (rc) return rc;
     hipLaunchKernelGGL(k_g1_normalize<false>, dim3(1), dim3(GT), 0, st, pts.p, pts.as<G1Jac>(), (size_t)3);
     ZK_LAUNCH_CHECK();
@@ -893,17 +904,28 @@ int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host, con
 }
 
 // The whole recursion of Commitment::me_open (commitment.cu:109-129): `rounds` halvings of (scalars, gens) of length n
-// with the challenges u[0..rounds).  proof_host receives 3*rounds + 1 points: T, T0, T1 of every round, then the
-// folded generator; all normalised to z = 1 (infinity: all-zero limbs).  final_scalar_host: the folded scalar.
-int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stv) {
-    hipStream_t st = (hipStream_t)stv;
+// with the challenges u[0..rounds).  An OpenJob queues all of it on one stream and keeps every buffer until the
+// result has been fetched.
+struct OpenJob {
+    Arena arena;
+    hipStream_t st = nullptr;
+    int rounds = 0;
+    G1Jac* pts = nullptr;
+    const Fr* final_scalar = nullptr;
+    hipEvent_t ready = nullptr;    // only for jobs on a side stream
+};
+static int open_queue(OpenJob& job, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, hipStream_t st) {
     ZK_ARG(n >= 1, "zk_g1_open: empty input");
     ZK_ARG(rounds >= 0 && rounds <= 64, "zk_g1_open: bad round count");
+    ZK_ARG(sizeof(G1Jac) * (3 * (size_t)rounds + 1) + sizeof(Fr) <= 65536, "zk_g1_open: proof larger than the staging buffer");
+    job.st = st;
+    job.rounds = rounds;
     const size_t npts = 3 * (size_t)rounds + 1;
-    Scratch pts(sizeof(G1Jac) * npts), rec(sizeof(G1Jac) * 3 * (rounds ? rounds : 1));
+    Scratch& pts = job.arena.add(sizeof(G1Jac) * npts);
+    Scratch& rec = job.arena.add(sizeof(G1Jac) * 3 * (rounds ? rounds : 1));
     if (pts.rc) return pts.rc;
     if (rec.rc) return rec.rc;
-    std::vector<std::unique_ptr<Scratch>> keep;
+    job.pts = pts.as<G1Jac>();
     const Fr* cs = (const Fr*)scalars;
     const G1Jac* cg = (const G1Jac*)gens;
     size_t size = n;
@@ -912,24 +934,21 @@ int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* sc
     bool tail_done = false;
     for (int r = 0; r < rounds; ++r) {
         if (size <= (size_t)TAIL_N && rounds - r <= TAIL_LEVELS) {
-            int rc = open_tail_launch(cs, cg, size, u + 8 * r, rounds - r, r, rounds, pts.as<G1Jac>(), &cs, keep, st);
+            int rc = open_tail_launch(cs, cg, size, u + 8 * r, rounds - r, r, rounds, pts.as<G1Jac>(), &cs, job.arena, st);
             if (rc) return rc;
             chained_rounds = r;
             tail_done = true;
             break;
         }
         const size_t ns = (size + 1) / 2;
-        keep.emplace_back(new Scratch(sizeof(Fr) * ns));
-        Scratch& s2 = *keep.back();
-        keep.emplace_back(new Scratch(sizeof(G1Jac) * ns));
-        Scratch& g2 = *keep.back();
+        Scratch& s2 = job.arena.add(sizeof(Fr) * ns);
+        Scratch& g2 = job.arena.add(sizeof(G1Jac) * ns);
         if (s2.rc) return s2.rc;
         if (g2.rc) return g2.rc;
         const Fr ur = load_fr(u + 8 * r);
         int rc = open_round_launch(s2.as<Fr>(), g2.as<G1Jac>(), cs, cg, ur, size, r, r ? &prev_u : nullptr, pts.as<G1Jac>() + 3 * r,
-                                   r ? pts.as<G1Jac>() + 3 * (r - 1) : nullptr, rec.as<G1Jac>(), st);
+                                   r ? pts.as<G1Jac>() + 3 * (r - 1) : nullptr, rec.as<G1Jac>(), job.arena, st);
         if (rc) return rc;
-        if (keep.size() > 4) { keep.erase(keep.begin(), keep.begin() + 2); }   // the round before the previous one is no longer read
         cs = s2.as<Fr>();
         cg = g2.as<G1Jac>();
         size = ns;
@@ -939,18 +958,66 @@ int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* sc
                        (uint32_t)chained_rounds, (uint32_t)rounds);
     hipLaunchKernelGGL(k_g1_normalize<false>, dim3(cdiv(cdiv(npts, CH), GT)), dim3(GT), 0, st, pts.p, pts.as<G1Jac>(), npts);
     ZK_LAUNCH_CHECK();
-    std::vector<uint8_t> tmp;
+    job.final_scalar = cs;
+    return 0;
+}
+// waits for the job's stream and copies the proof points and the folded scalar out
+static int open_collect(OpenJob& job, uint32_t* proof_host, uint32_t* final_scalar_host) {
+    const size_t npts = 3 * (size_t)job.rounds + 1;
     void* stage = nullptr;
-    const size_t bytes = sizeof(G1Jac) * npts + sizeof(Fr);
-    ZK_ARG(bytes <= 65536, "zk_g1_open: proof larger than the staging buffer");
-    int rc = staging(&stage, bytes);
+    int rc = staging(&stage, sizeof(G1Jac) * npts + sizeof(Fr));
     if (rc) return rc;
-    ZK_HIP(hipMemcpyAsync(stage, pts.p, sizeof(G1Jac) * npts, hipMemcpyDeviceToHost, st));
-    ZK_HIP(hipMemcpyAsync((char*)stage + sizeof(G1Jac) * npts, cs, sizeof(Fr), hipMemcpyDeviceToHost, st));
-    ZK_HIP(hipStreamSynchronize(st));
+    ZK_HIP(hipMemcpyAsync(stage, job.pts, sizeof(G1Jac) * npts, hipMemcpyDeviceToHost, job.st));
+    ZK_HIP(hipMemcpyAsync((char*)stage + sizeof(G1Jac) * npts, job.final_scalar, sizeof(Fr), hipMemcpyDeviceToHost, job.st));
+    ZK_HIP(hipStreamSynchronize(job.st));
     memcpy(proof_host, stage, sizeof(G1Jac) * npts);
     memcpy(final_scalar_host, (char*)stage + sizeof(G1Jac) * npts, sizeof(Fr));
     return 0;
+}
+// streams for openings that run beside the caller's stream (default priority, not synchronising with the null stream)
+static hipStream_t side_stream() {
+    static hipStream_t streams[4] = {nullptr, nullptr, nullptr, nullptr};
+    static unsigned next = 0;
+    const unsigned i = next++ % 4;
+    if (!streams[i] && hipStreamCreateWithFlags(&streams[i], hipStreamNonBlocking) != hipSuccess) return nullptr;
+    return streams[i];
+}
+
+// proof_host receives 3*rounds + 1 points: T, T0, T1 of every round, then the folded generator; all normalised to
+// z = 1 (infinity: all-zero limbs).  final_scalar_host: the folded scalar.
+int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stv) {
+    OpenJob job;
+    int rc = open_queue(job, scalars, gens, n, u, rounds, (hipStream_t)stv);
+    if (rc) { (void)hipStreamSynchronize((hipStream_t)stv); return rc; }
+    return open_collect(job, proof_host, final_scalar_host);
+}
+// The same in two halves.  begin queues the recursion on a stream of the library's own, ordered after everything queued
+// on `stream` so far, and returns at once; the caller goes on using `stream`, and both run side by side.  scalars and gens
+// must stay alive and unmodified until end, which waits for the opening, delivers its results and releases its buffers.
+int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stv) {
+    ZK_ARG(handle != nullptr, "zk_g1_open_begin: null handle");
+    hipStream_t side = side_stream();
+    ZK_ARG(side != nullptr, "zk_g1_open_begin: could not create a stream");
+    std::unique_ptr<OpenJob> job(new OpenJob);
+    ZK_HIP(hipEventCreateWithFlags(&job->ready, hipEventDisableTiming));
+    ZK_HIP(hipEventRecord(job->ready, (hipStream_t)stv));
+    ZK_HIP(hipStreamWaitEvent(side, job->ready, 0));
+    int rc = open_queue(*job, scalars, gens, n, u, rounds, side);
+    if (rc) {
+        (void)hipStreamSynchronize(side);
+        (void)hipEventDestroy(job->ready);
+        return rc;
+    }
+    *handle = job.release();
+    return 0;
+}
+int zk_g1_open_end(void* handle, uint32_t* proof_host, uint32_t* final_scalar_host) {
+    ZK_ARG(handle != nullptr, "zk_g1_open_end: null handle");
+    std::unique_ptr<OpenJob> job((OpenJob*)handle);
+    int rc = open_collect(*job, proof_host, final_scalar_host);
+    if (rc) (void)hipStreamSynchronize(job->st);
+    (void)hipEventDestroy(job->ready);
+    return rc;
 }
 
 // Measurement: time every launch of the opening's fold kernel between begin and read with events on the launch stream.

@@ -74,6 +74,35 @@ Fr_t Commitment::open(const FrTensor& t, const G1TensorJacobian& com, const vect
     }
     return me_open(folded, *this, u_in.begin(), u_in.end(), proof);
 }
+Commitment::Pending Commitment::open_begin(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u) const {
+    const uint k_out = ceilLog2(com.size);
+    if (u.size() < k_out) throw std::runtime_error("Commitment::open - too few challenges");
+    const vector<Fr_t> u_out(u.end() - k_out, u.end());
+    const vector<Fr_t> u_in(u.begin(), u.end() - k_out);
+    Pending p;
+    p.folded.reset(new FrTensor(u_out.empty() ? FrTensor(t) : t.partial_me(u_out, t.size / com.size)));
+    if (p.folded->size != size) throw std::runtime_error("Commitment::me_open - Incompatible dimensions " + std::to_string(p.folded->size) + " " + std::to_string(size));
+    if (g_skip_g1) {
+        p.value = (*p.folded)(u_in);
+        return p;
+    }
+    p.rounds = (int)u_in.size();
+    std::vector<uint32_t> uu((size_t)p.rounds * 8 + 8);
+    for (int r = 0; r < p.rounds; ++r) memcpy(&uu[(size_t)r * 8], u_in[r].val, 32);
+    ZKC(zk_g1_open_begin(&p.handle, p.folded->gpu_data, gpu_data, size, uu.data(), p.rounds, nullptr));
+    return p;
+}
+Fr_t Commitment::open_end(Pending& p, vector<G1Jacobian_t>& proof) {
+    if (!p.handle) return p.value;
+    std::vector<G1Jacobian_t> pts(3 * (size_t)p.rounds + 1);
+    void* h = p.handle;
+    p.handle = nullptr;
+    ZKC(zk_g1_open_end(h, pts[0].x.val, p.value.val));
+    proof.insert(proof.end(), pts.begin(), pts.end());
+    p.folded.reset();
+    return p.value;
+}
+
 Fr_t Commitment::open(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u) const {
     vector<G1Jacobian_t> proof;
     return open(t, com, u, proof);

@@ -1,5 +1,6 @@
 // Pedersen vector commitment over G1 (commitment.cuh:8-36).
 #pragma once
+#include <memory>
 #include "fr-tensor.hpp"
 #include "g1-tensor.hpp"
 #include "proof.hpp"
@@ -21,6 +22,17 @@ class Commitment : public G1TensorJacobian {
     Fr_t open(const FrTensor& t, const G1TensorJacobian& c, const vector<Fr_t>& u) const;
     // same evaluation, and keeps the G1 transcript of the opening (3 points per round + the last generator)
     Fr_t open(const FrTensor& t, const G1TensorJacobian& c, const vector<Fr_t>& u, vector<G1Jacobian_t>& proof) const;
+
+    // The opening in two halves: open_begin folds the rows and queues the G1 recursion beside the caller's work,
+    // open_end waits for it and returns what open returns.  The generators must outlive the pending opening.
+    struct Pending {
+        void* handle = nullptr;             // null: the value is already known (G1 part skipped)
+        std::unique_ptr<FrTensor> folded;   // the scalars the queued kernels read
+        int rounds = 0;
+        Fr_t value{{0, 0, 0, 0, 0, 0, 0, 0}};
+    };
+    Pending open_begin(const FrTensor& t, const G1TensorJacobian& c, const vector<Fr_t>& u) const;
+    static Fr_t open_end(Pending& p, vector<G1Jacobian_t>& proof);
 
     static Commitment random(uint size);
     static Fr_t me_open(const FrTensor& t, const Commitment& generators, vector<Fr_t>::const_iterator begin, vector<Fr_t>::const_iterator end, vector<G1Jacobian_t>& proof);

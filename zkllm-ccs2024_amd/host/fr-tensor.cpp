@@ -47,6 +47,12 @@ void zk_transcript_begin() { G().transcript.clear(); G().recording = true; }
 const std::vector<Fr_t>& zk_transcript() { return G().transcript; }
 void zk_transcript_end() { G().recording = false; }
 void zk_record(const Fr_t& x) { if (G().recording) G().transcript.push_back(x); }
+size_t zk_record_reserve() {
+    if (!G().recording) return (size_t)-1;
+    G().transcript.push_back(Fr_t{{0, 0, 0, 0, 0, 0, 0, 0}});
+    return G().transcript.size() - 1;
+}
+void zk_record_fill(size_t slot, const Fr_t& x) { if (slot != (size_t)-1 && slot < G().transcript.size()) G().transcript[slot] = x; }
 void zk_record(const std::vector<Fr_t>& xs) { if (G().recording) G().transcript.insert(G().transcript.end(), xs.begin(), xs.end()); }
 
 ostream& operator<<(ostream& os, const Fr_t& x) {

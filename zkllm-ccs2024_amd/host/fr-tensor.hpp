@@ -42,6 +42,9 @@ const std::vector<Fr_t>& zk_transcript();
 void zk_transcript_end();
 void zk_record(const Fr_t& x);
 void zk_record(const std::vector<Fr_t>& xs);
+// a transcript position whose value arrives later (an opening that runs beside the prover): reserve keeps the order
+size_t zk_record_reserve();
+void zk_record_fill(size_t slot, const Fr_t& x);
 
 void zk_check(int rc, const char* where);   // throws std::runtime_error on a non-zero C-ABI status
 

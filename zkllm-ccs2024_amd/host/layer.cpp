@@ -193,6 +193,7 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
 
 FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor& X, LayerTimes* times) {
     LayerTimes t;
+    DeferredOpenings openings;       // the nine weight openings run on the device beside the sumchecks
     const double t0 = now_ms();
     FrTensor rms1 = compute_rms_inv(X, c.seq_len, c.embed_dim, c.rms_eps, c.value_scale);
     FrTensor n1 = rmsnorm_block(c, w.input_norm, X, rms1);
@@ -210,6 +211,7 @@ FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor
     const double t5 = now_ms();
     FrTensor f = ffn_block(c, w.up, w.gate, w.down, w.swiglu_table, n2);
     FrTensor out = x2 + f;
+    openings.finish();
     const double t6 = now_ms();
     t.rmsnorm1 = t1 - t0; t.qkv = t2 - t1; t.attention = t3 - t2; t.oproj = t4 - t3; t.rmsnorm2 = t5 - t4; t.ffn = t6 - t5; t.total = t6 - t0;
     if (times) *times = t;

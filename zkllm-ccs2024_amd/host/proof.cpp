@@ -5,10 +5,48 @@
 
 #define ZKC(call) zk_check((call), #call)
 
+struct DeferredOpenings::Item {
+    Commitment::Pending op;
+    Fr_t claim;
+    size_t slot;
+};
+static thread_local DeferredOpenings* g_deferred = nullptr;
+DeferredOpenings::DeferredOpenings() : prev(g_deferred) { g_deferred = this; }
+DeferredOpenings::~DeferredOpenings() {
+    g_deferred = prev;
+    for (Item* it : items) {          // only reached with pending items when an exception unwinds: release them
+        try { vector<G1Jacobian_t> drop; Commitment::open_end(it->op, drop); } catch (...) {}
+        delete it;
+    }
+}
+void DeferredOpenings::finish() {
+    std::vector<Item*> todo;
+    todo.swap(items);
+    std::string failure;
+    for (Item* it : todo) {
+        try {
+            vector<G1Jacobian_t> g1_proof;
+            const Fr_t opening = Commitment::open_end(it->op, g1_proof);
+            zk_record_fill(it->slot, opening);
+            if (opening != it->claim && failure.empty()) failure = "verifyWeightClaim: opening != c.claim";
+            else cout << "Opening complete" << endl;
+        } catch (const std::exception& e) {
+            if (failure.empty()) failure = e.what();
+        }
+        delete it;
+    }
+    if (!failure.empty()) throw std::runtime_error(failure);
+}
+
 // proof.cu:3-10
 void verifyWeightClaim(const Weight& w, const Claim& c) {
     vector<Fr_t> u_cat = concatenate(vector<vector<Fr_t>>({c.u[1], c.u[0]}));
     auto w_padded = w.weight.pad({w.in_dim, w.out_dim});
+    if (g_deferred) {
+        DeferredOpenings::Item* it = new DeferredOpenings::Item{w.generator.open_begin(w_padded, w.com, u_cat), c.claim, zk_record_reserve()};
+        g_deferred->items.push_back(it);
+        return;
+    }
     auto opening = w.generator.open(w_padded, w.com, u_cat);
     zk_record(opening);
     if (opening != c.claim) throw std::runtime_error("verifyWeightClaim: opening != c.claim");

@@ -13,6 +13,23 @@ struct Claim {
 
 struct Weight;
 void verifyWeightClaim(const Weight& w, const Claim& c);
+// While a DeferredOpenings object is alive, verifyWeightClaim only starts each opening (it runs on the device beside
+// the rest of the proof) and finish() waits for all of them, checks every claim and throws as verifyWeightClaim does.
+// The transcript keeps the position of each opened value.
+class DeferredOpenings {
+   public:
+    DeferredOpenings();
+    ~DeferredOpenings();
+    void finish();
+    DeferredOpenings(const DeferredOpenings&) = delete;
+    DeferredOpenings& operator=(const DeferredOpenings&) = delete;
+
+   private:
+    struct Item;
+    std::vector<Item*> items;
+    DeferredOpenings* prev;
+    friend void verifyWeightClaim(const Weight& w, const Claim& c);
+};
 
 vector<Fr_t> inner_product_sumcheck(const FrTensor& a, const FrTensor& b, vector<Fr_t> u);
 vector<Fr_t> hadamard_product_sumcheck(const FrTensor& a, const FrTensor& b, vector<Fr_t> u, vector<Fr_t> v);
