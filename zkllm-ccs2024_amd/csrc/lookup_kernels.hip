@@ -311,6 +311,156 @@ k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __rest
     block_reduce_store<K + 1>(acc, partials);
 }
 
+// ---- the last rounds of a sumcheck in one launch ---------------------------------------------------------------------------------
+// Once the tensors are short, a round is a few microseconds of arithmetic between two host round trips.  The
+// challenges of these sumchecks are fixed before the first round (tLookup::prove and multi_hadamard_sumchecks take u and
+// v as arguments, tlookup.cu:150-176, proof.cu:191-241), so one workgroup can run every remaining round back to back --
+// sums, fold by v, halving of the eq table, workgroup barrier -- and hand all rounds' sums back in one copy.
+static constexpr int TAIL_T = 1024;          // lanes of the single workgroup
+static constexpr int TAIL_HALF = 512;        // largest n_out of the first fused round: one compute unit does all of it
+static constexpr int TAIL_ROUNDS = 16;
+struct TailV { Fr v[TAIL_ROUNDS]; };         // Montgomery form, in round order
+
+__device__ __forceinline__ Fr wave_sum(Fr x) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        Fr y;
+#pragma unroll
+        for (int l = 0; l < 8; ++l) y.v[l] = __shfl_down(x.v[l], off, 64);
+        x = add(x, y);
+    }
+    return x;
+}
+// sums of K values over the TAIL_T lanes into out[0..K) (lane 0 writes); red: K x 16 x 8 words of LDS
+template <int K> __device__ __forceinline__ void tail_block_sum(Fr (&acc)[K], Fr* __restrict__ out, uint32_t* red) {
+    const uint32_t t = threadIdx.x, wv = t >> 6, ln = t & 63u;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const Fr w = wave_sum(acc[k]);
+        if (ln == 0) {
+#pragma unroll
+            for (int l = 0; l < 8; ++l) red[(k * 16 + wv) * 8 + l] = w.v[l];
+        }
+    }
+    __syncthreads();
+    if (wv == 0) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            Fr x = big_zero<8>();
+            if (ln < 16) {
+#pragma unroll
+                for (int l = 0; l < 8; ++l) x.v[l] = red[(k * 16 + ln) * 8 + l];
+            }
+            x = wave_sum(x);
+            if (ln == 0) out[k] = x;
+        }
+    }
+    __syncthreads();
+}
+
+// All remaining rounds of the lookup sumcheck.  Round 0 reads the caller's tensors (2*n_out elements; E: n_out) and
+// writes the work buffers; later rounds fold the work buffers in place (lane t reads t and t + half and writes t,
+// which no other lane reads).  sums[r*11 + i] as k_lookup_round orders them (5 used in phase 1).  Rounds from
+// `phase2_from` on are phase-2 rounds.
+__global__ void __launch_bounds__(TAIL_T)
+k_lookup_tail(Fr* __restrict__ sums, Fr* wA, Fr* wS, Fr* wB, Fr* wT, Fr* wm, Fr* wE, const Fr* A, const Fr* S, const Fr* B, const Fr* T, const Fr* m, const Fr* E,
+              const Fr beta, const TailV vs, uint32_t n_out0, uint32_t rounds, uint32_t phase2_from) {
+    __shared__ uint32_t red[11 * 16 * 8];
+    const Fr *cA = A, *cS = S, *cB = B, *cT = T, *cm = m, *cE = E;
+    uint32_t n_out = n_out0;
+    for (uint32_t r = 0; r < rounds; ++r) {
+        const bool phase2 = r >= phase2_from;
+        const Fr v_mont = vs.v[r];
+        Fr acc[11];
+#pragma unroll
+        for (int i = 0; i < 11; ++i) acc[i] = big_zero<8>();
+        for (uint32_t t = threadIdx.x; t < n_out; t += TAIL_T) {
+            const Fr e = cE[t];
+            {
+                const Fr a0 = cA[t], a1 = cA[t + n_out], s0r = cS[t], s1 = cS[t + n_out];
+                const Fr da = sub(a1, a0), ds = sub(s1, s0r), s0 = add(s0r, beta);
+                acc[0] = add(acc[0], mont_mul(e, mont_mul(a0, s0)));
+                acc[1] = add(acc[1], mont_mul(e, add(mont_mul(da, s0), mont_mul(a0, ds))));
+                acc[2] = add(acc[2], mont_mul(e, mont_mul(da, ds)));
+                acc[3] = add(acc[3], a0);
+                acc[4] = add(acc[4], da);
+                wA[t] = add(a0, mont_mul(v_mont, da));
+                wS[t] = add(s0r, mont_mul(v_mont, ds));
+            }
+            if (phase2) {
+                const Fr b0 = cB[t], b1 = cB[t + n_out], t0r = cT[t], t1 = cT[t + n_out], m0 = cm[t], m1 = cm[t + n_out];
+                const Fr db = sub(b1, b0), dt = sub(t1, t0r), t0 = add(t0r, beta), dm = sub(m1, m0);
+                acc[5] = add(acc[5], mont_mul(e, mont_mul(b0, t0)));
+                acc[6] = add(acc[6], mont_mul(e, add(mont_mul(db, t0), mont_mul(b0, dt))));
+                acc[7] = add(acc[7], mont_mul(e, mont_mul(db, dt)));
+                acc[8] = add(acc[8], mont_mul(m0, b0));
+                acc[9] = add(acc[9], add(mont_mul(dm, b0), mont_mul(m0, db)));
+                acc[10] = add(acc[10], mont_mul(dm, db));
+                wB[t] = add(b0, mont_mul(v_mont, db));
+                wT[t] = add(t0r, mont_mul(v_mont, dt));
+                wm[t] = add(m0, mont_mul(v_mont, dm));
+            }
+        }
+        tail_block_sum<11>(acc, sums + (size_t)r * 11, red);      // ends with a barrier: every read of this round's E is done
+        cA = wA; cS = wS;
+        if (phase2) { cB = wB; cT = wT; cm = wm; }
+        const uint32_t nh = n_out >> 1;
+        for (uint32_t t = threadIdx.x; t < nh; t += TAIL_T) wE[t] = add(cE[t], cE[t + nh]);
+        cE = wE;
+        n_out = nh;
+        __syncthreads();
+    }
+}
+
+// All remaining rounds of the multi-Hadamard sumcheck for K tensors; sums[r*(K+1) + j].
+template <int K> __global__ void __launch_bounds__(TAIL_T)
+k_hadamard_tail(Fr* __restrict__ sums, const PtrPack<K> p, Fr* wE, const Fr* E, const TailV vs, uint32_t n_out0, uint32_t rounds) {
+    __shared__ uint32_t red[(K + 1) * 16 * 8];
+    const Fr* cur[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) cur[k] = p.in[k];
+    const Fr* cE = E;
+    const Fr r2 = big_r2<8>();
+    uint32_t n_out = n_out0;
+    for (uint32_t r = 0; r < rounds; ++r) {
+        const Fr v_mont = vs.v[r];
+        Fr acc[K + 1];
+#pragma unroll
+        for (int i = 0; i <= K; ++i) acc[i] = big_zero<8>();
+        for (uint32_t t = threadIdx.x; t < n_out; t += TAIL_T) {
+            Fr c[K + 1];
+            {
+                const Fr x0 = cur[0][t], x1 = cur[0][t + n_out];
+                const Fr dx = sub(x1, x0);
+                c[0] = x0; c[1] = dx;
+                p.out[0][t] = add(x0, mont_mul(v_mont, dx));
+            }
+#pragma unroll
+            for (int k = 1; k < K; ++k) {
+                const Fr x0 = cur[k][t], x1 = cur[k][t + n_out];
+                const Fr dx = sub(x1, x0);
+                p.out[k][t] = add(x0, mont_mul(v_mont, dx));
+                const Fr x0m = mont_mul(x0, r2), dxm = mont_mul(dx, r2);
+                c[k + 1] = mont_mul(c[k], dxm);
+#pragma unroll
+                for (int j = k; j >= 1; --j) c[j] = add(mont_mul(c[j], x0m), mont_mul(c[j - 1], dxm));
+                c[0] = mont_mul(c[0], x0m);
+            }
+            const Fr e = cE[t];
+#pragma unroll
+            for (int j = 0; j <= K; ++j) acc[j] = add(acc[j], mont_mul(e, c[j]));
+        }
+        tail_block_sum<K + 1>(acc, sums + (size_t)r * (K + 1), red);
+#pragma unroll
+        for (int k = 0; k < K; ++k) cur[k] = p.out[k];
+        const uint32_t nh = n_out >> 1;
+        for (uint32_t t = threadIdx.x; t < nh; t += TAIL_T) wE[t] = add(cE[t], cE[t + nh]);
+        cE = wE;
+        n_out = nh;
+        __syncthreads();
+    }
+}
+
 // ---- rescaling (rescaling.cu:8-21) ----------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(TPB) k_rescale(Fr* __restrict__ out, Fr* __restrict__ rem, const Fr* __restrict__ in, int64_t sf, size_t n) {
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
@@ -519,6 +669,75 @@ int zk_hadamard_round(uint32_t* coefs_host, void* const* new_Xs, const void* con
     int rc = finish_sums(part.as<Fr>(), nb, K + 1, 0, s, st);
     if (rc) return rc;
     memcpy(coefs_host, s, sizeof(Fr) * (K + 1));
+    return 0;
+}
+// The last `rounds` rounds of the lookup sumcheck in one launch (n_out of the first of them at most 512, at most 16
+// rounds).  A, S (and B, T, m from round phase2_from on) hold 2*n_out elements, E n_out; none of them is modified.
+// v: the rounds' fold challenges in round order (standard form, host).  sums_host: rounds x 11 values ordered as
+// zk_lookup_round orders them (entries 5..10 of a phase-1 round are zero).
+int zk_lookup_rounds_tail(uint32_t* sums_host, const void* A, const void* S, const void* B, const void* T, const void* m, const void* E, const uint32_t* beta,
+                          const uint32_t* v, size_t n_out, int rounds, int phase2_from, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(n_out >= 1 && n_out <= (size_t)TAIL_HALF, "zk_lookup_rounds_tail: n_out must be 1..512");
+    ZK_ARG(rounds >= 1 && rounds <= TAIL_ROUNDS, "zk_lookup_rounds_tail: 1..16 rounds");
+    ZK_ARG(((size_t)1 << (rounds - 1)) <= n_out, "zk_lookup_rounds_tail: more rounds than the tensors have variables");
+    ZK_ARG(phase2_from >= 0, "zk_lookup_rounds_tail: bad phase-2 start");
+    Scratch work(sizeof(Fr) * 6 * n_out), sums(sizeof(Fr) * 11 * rounds);
+    if (work.rc) return work.rc;
+    if (sums.rc) return sums.rc;
+    TailV vs;
+    for (int r = 0; r < TAIL_ROUNDS; ++r) vs.v[r] = r < rounds ? to_mont(load_fr(v + 8 * r)) : big_zero<8>();
+    Fr* w = work.as<Fr>();
+    hipLaunchKernelGGL(k_lookup_tail, dim3(1), dim3(TAIL_T), 0, st, sums.as<Fr>(), w, w + n_out, w + 2 * n_out, w + 3 * n_out, w + 4 * n_out, w + 5 * n_out, (const Fr*)A,
+                       (const Fr*)S, (const Fr*)B, (const Fr*)T, (const Fr*)m, (const Fr*)E, load_fr(beta), vs, (uint32_t)n_out, (uint32_t)rounds, (uint32_t)phase2_from);
+    ZK_LAUNCH_CHECK();
+    void* stage = nullptr;
+    int rc = staging(&stage, sizeof(Fr) * 11 * rounds);
+    if (rc) return rc;
+    ZK_HIP(hipMemcpyAsync(stage, sums.p, sizeof(Fr) * 11 * rounds, hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipStreamSynchronize(st));
+    Fr* out = (Fr*)sums_host;
+    const Fr* in = (const Fr*)stage;
+    for (int r = 0; r < rounds; ++r)
+        for (int i = 0; i < 11; ++i) {
+            Fr x = in[r * 11 + i];
+            if (i != 3 && i != 4) x = to_mont(x);        // same R correction as zk_lookup_round
+            if (r < phase2_from && i >= 5) x = big_zero<8>();
+            memcpy(&out[r * 11 + i], &x, sizeof(Fr));
+        }
+    return 0;
+}
+// The last `rounds` rounds of multi_hadamard_sumchecks in one launch (same limits).  Xs hold 2*n_out elements and are
+// not modified; coefs_host: rounds x (K+1) coefficients; v in round order.
+int zk_hadamard_rounds_tail(uint32_t* coefs_host, const void* const* Xs, int K, const void* E, const uint32_t* v, size_t n_out, int rounds, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(K >= 1 && K <= 4, "zk_hadamard_rounds_tail: K must be 1..4");
+    ZK_ARG(n_out >= 1 && n_out <= (size_t)TAIL_HALF, "zk_hadamard_rounds_tail: n_out must be 1..512");
+    ZK_ARG(rounds >= 1 && rounds <= TAIL_ROUNDS, "zk_hadamard_rounds_tail: 1..16 rounds");
+    ZK_ARG(((size_t)1 << (rounds - 1)) <= n_out, "zk_hadamard_rounds_tail: more rounds than the tensors have variables");
+    Scratch work(sizeof(Fr) * (K + 1) * n_out), sums(sizeof(Fr) * (K + 1) * rounds);
+    if (work.rc) return work.rc;
+    if (sums.rc) return sums.rc;
+    TailV vs;
+    for (int r = 0; r < TAIL_ROUNDS; ++r) vs.v[r] = r < rounds ? to_mont(load_fr(v + 8 * r)) : big_zero<8>();
+    Fr* w = work.as<Fr>();
+#define HADT_CASE(KK)                                                                                                                  \
+    case KK: {                                                                                                                         \
+        PtrPack<KK> p;                                                                                                                 \
+        for (int i = 0; i < KK; ++i) { p.in[i] = (const Fr*)Xs[i]; p.out[i] = w + (size_t)i * n_out; }                                  \
+        hipLaunchKernelGGL(k_hadamard_tail<KK>, dim3(1), dim3(TAIL_T), 0, st, sums.as<Fr>(), p, w + (size_t)KK * n_out, (const Fr*)E, vs, \
+                           (uint32_t)n_out, (uint32_t)rounds);                                                                         \
+        break;                                                                                                                         \
+    }
+    switch (K) { HADT_CASE(1) HADT_CASE(2) HADT_CASE(3) HADT_CASE(4) }
+#undef HADT_CASE
+    ZK_LAUNCH_CHECK();
+    void* stage = nullptr;
+    int rc = staging(&stage, sizeof(Fr) * (K + 1) * rounds);
+    if (rc) return rc;
+    ZK_HIP(hipMemcpyAsync(stage, sums.p, sizeof(Fr) * (K + 1) * rounds, hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipStreamSynchronize(st));
+    memcpy(coefs_host, stage, sizeof(Fr) * (K + 1) * rounds);
     return 0;
 }
 int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* st) {

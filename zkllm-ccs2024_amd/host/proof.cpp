@@ -74,17 +74,30 @@ Fr_t multi_hadamard_sumchecks(const Fr_t& claim0, const vector<FrTensor>& Xs, co
     ZKC(zk_eq_table(E.back().gpu_data, u[0].val, (int)k - 1, nullptr));
     std::vector<const void*> cur(K);
     for (uint i = 0; i < K; ++i) cur[i] = Xs[i].gpu_data;
-    for (uint r = 0; r < k; ++r) {
-        const uint half = N >> (r + 1);
-        std::vector<void*> nxt(K);
-        for (uint i = 0; i < K; ++i) { keep.emplace_back(half); nxt[i] = keep.back().gpu_data; }
-        std::vector<Fr_t> coefs(K + 1);
-        ZKC(zk_hadamard_round(coefs[0].val, nxt.data(), cur.data(), (int)K, E.back().gpu_data, v[k - 1 - r].val, half, nullptr));
+    auto absorb = [&](uint r, const Fr_t* c) {
+        std::vector<Fr_t> coefs(c, c + K + 1);
         proof.push_back(Polynomial(coefs));
         zk_record(coefs);
         Polynomial p = proof.back() * Polynomial::eq(u[k - 1 - r]);
         if (claim != p(kZero) + p(kOne)) throw std::runtime_error("multi_hadamard_sumchecks: claim != p(0) + p(1)");
         claim = proof.back()(v[k - 1 - r]);
+    };
+    for (uint r = 0; r < k; ++r) {
+        const uint half = N >> (r + 1);
+        if (half <= 512 && k - r <= 16) {
+            // short tensors: every remaining round in one launch (the challenges are all known), the host work afterwards
+            const uint rest = k - r;
+            std::vector<Fr_t> vs(rest), sums((size_t)rest * (K + 1));
+            for (uint i = 0; i < rest; ++i) vs[i] = v[k - 1 - (r + i)];
+            ZKC(zk_hadamard_rounds_tail(sums[0].val, cur.data(), (int)K, E.back().gpu_data, vs[0].val, half, (int)rest, nullptr));
+            for (uint i = 0; i < rest; ++i) absorb(r + i, &sums[(size_t)i * (K + 1)]);
+            break;
+        }
+        std::vector<void*> nxt(K);
+        for (uint i = 0; i < K; ++i) { keep.emplace_back(half); nxt[i] = keep.back().gpu_data; }
+        std::vector<Fr_t> coefs(K + 1);
+        ZKC(zk_hadamard_round(coefs[0].val, nxt.data(), cur.data(), (int)K, E.back().gpu_data, v[k - 1 - r].val, half, nullptr));
+        absorb(r, coefs.data());
         for (uint i = 0; i < K; ++i) cur[i] = nxt[i];
         if (r + 1 < k) {
             const uint next = half >> 1;

@@ -102,24 +102,15 @@ Fr_t tLookup_sumcheck(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0
     std::vector<FrTensor> keep;
     keep.reserve(5 * k + 8);
     const FrTensor *cA = &A, *cS = &S0, *cB = &B, *cT = &T0, *cm = &m0;
-    for (uint r = 0; r < k; ++r) {
-        const bool phase2 = r >= n1;
-        const uint cur = cA->size, half = cur >> 1;
-        const Fr_t& ub = u[k - 1 - r];
+    auto challenge_of = [&](uint r) -> const Fr_t& {
         // v1 = v[0..n1) consumed from its back, then v2 = v[n1..k) from its back
-        const Fr_t& vr = phase2 ? v[k - 1 - (r - n1)] : v[n1 - 1 - r];
-        keep.emplace_back(half); FrTensor* nA = &keep.back();
-        keep.emplace_back(half); FrTensor* nS = &keep.back();
-        FrTensor *nB = nullptr, *nT = nullptr, *nm = nullptr;
-        if (phase2) {
-            keep.emplace_back(half); nB = &keep.back();
-            keep.emplace_back(half); nT = &keep.back();
-            keep.emplace_back(half); nm = &keep.back();
-        }
-        Fr_t s[11];
-        ZKC(zk_lookup_round(s[0].val, nA->gpu_data, nS->gpu_data, phase2 ? nB->gpu_data : nullptr, phase2 ? nT->gpu_data : nullptr, phase2 ? nm->gpu_data : nullptr,
-                            cA->gpu_data, cS->gpu_data, phase2 ? cB->gpu_data : nullptr, phase2 ? cT->gpu_data : nullptr, phase2 ? cm->gpu_data : nullptr,
-                            E.back().gpu_data, beta.val, vr.val, half, phase2 ? 1 : 0, nullptr));
+        return r >= n1 ? v[k - 1 - (r - n1)] : v[n1 - 1 - r];
+    };
+    // host side of a round: the round polynomial from the device's sums, the check, the next claim
+    auto absorb = [&](uint r, const Fr_t* s) {
+        const bool phase2 = r >= n1;
+        const Fr_t& ub = u[k - 1 - r];
+        const Fr_t& vr = challenge_of(r);
         Polynomial p;
         if (!phase2) {
             Polynomial p0({alpha * s[0], alpha * s[1], alpha * s[2]});
@@ -140,6 +131,34 @@ Fr_t tLookup_sumcheck(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0
         alpha = alpha * e;
         if (phase2) alpha_sq = alpha_sq * e;
         else C = C * TWO_INV;
+    };
+    for (uint r = 0; r < k; ++r) {
+        const bool phase2 = r >= n1;
+        const uint cur = cA->size, half = cur >> 1;
+        if (half <= 512 && k - r <= 16) {
+            // short tensors: every remaining round in one launch, the host work afterwards
+            const uint rest = k - r;
+            std::vector<Fr_t> vs(rest), sums((size_t)rest * 11);
+            for (uint i = 0; i < rest; ++i) vs[i] = challenge_of(r + i);
+            ZKC(zk_lookup_rounds_tail(sums[0].val, cA->gpu_data, cS->gpu_data, cB->gpu_data, cT->gpu_data, cm->gpu_data, E.back().gpu_data, beta.val, vs[0].val, half,
+                                      (int)rest, phase2 ? 0 : (int)(n1 - r), nullptr));
+            for (uint i = 0; i < rest; ++i) absorb(r + i, &sums[(size_t)i * 11]);
+            break;
+        }
+        const Fr_t& vr = challenge_of(r);
+        keep.emplace_back(half); FrTensor* nA = &keep.back();
+        keep.emplace_back(half); FrTensor* nS = &keep.back();
+        FrTensor *nB = nullptr, *nT = nullptr, *nm = nullptr;
+        if (phase2) {
+            keep.emplace_back(half); nB = &keep.back();
+            keep.emplace_back(half); nT = &keep.back();
+            keep.emplace_back(half); nm = &keep.back();
+        }
+        Fr_t s[11];
+        ZKC(zk_lookup_round(s[0].val, nA->gpu_data, nS->gpu_data, phase2 ? nB->gpu_data : nullptr, phase2 ? nT->gpu_data : nullptr, phase2 ? nm->gpu_data : nullptr,
+                            cA->gpu_data, cS->gpu_data, phase2 ? cB->gpu_data : nullptr, phase2 ? cT->gpu_data : nullptr, phase2 ? cm->gpu_data : nullptr,
+                            E.back().gpu_data, beta.val, vr.val, half, phase2 ? 1 : 0, nullptr));
+        absorb(r, s);
         cA = nA; cS = nS;
         if (phase2) { cB = nB; cT = nT; cm = nm; }
         if (r + 1 < k) {
