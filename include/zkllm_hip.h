@@ -167,6 +167,12 @@ int zk_hadamard_round(uint32_t* coefs_host, void* const* new_Xs, const void* con
 int zk_lookup_rounds_tail(uint32_t* sums_host, const void* A, const void* S, const void* B, const void* T, const void* m, const void* E, const uint32_t* beta,
                           const uint32_t* v, size_t n_out, int rounds, int phase2_from, void* stream);
 int zk_hadamard_rounds_tail(uint32_t* coefs_host, const void* const* Xs, int K, const void* E, const uint32_t* v, size_t n_out, int rounds, void* stream);
+/* both sumchecks whole, queued without a host round trip (all rounds' sums come back in one copy).  Lookup: A, S of
+ * D elements, B, T, m of N (D/N a power of two), E of D/2; v: rounds x 8 limbs in round order; sums_host: rounds x 11.
+ * Hadamard: K tensors of N elements (a power of two), E of N/2; coefs_host: log2(N) x (K+1).  Inputs are not modified. */
+int zk_lookup_sumcheck(uint32_t* sums_host, const void* A, const void* S, const void* B, const void* T, const void* m, const void* E, const uint32_t* beta,
+                       const uint32_t* v, size_t D, size_t N, int rounds, void* stream);
+int zk_hadamard_sumcheck(uint32_t* coefs_host, const void* const* Xs, int K, const void* E, const uint32_t* v, size_t N, void* stream);
 
 /* ---- rescaling / softmax ------------------------------------------------------------------------------------------ */
 int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* stream);       /* rescaling_kernel rescaling.cu:8-21 */

@@ -14,6 +14,8 @@
 //    term tensor is ever written.
 //  * softmax shift / exp tables use the deterministic exp/log of detmath.hpp.
 #include <cstring>
+#include <memory>
+#include <vector>
 #include "detmath.hpp"
 #include "field.hpp"
 #include "rt.hpp"
@@ -733,6 +735,167 @@ int zk_hadamard_rounds_tail(uint32_t* coefs_host, const void* const* Xs, int K, 
     switch (K) { HADT_CASE(1) HADT_CASE(2) HADT_CASE(3) HADT_CASE(4) }
 #undef HADT_CASE
     ZK_LAUNCH_CHECK();
+    void* stage = nullptr;
+    int rc = staging(&stage, sizeof(Fr) * (K + 1) * rounds);
+    if (rc) return rc;
+    ZK_HIP(hipMemcpyAsync(stage, sums.p, sizeof(Fr) * (K + 1) * rounds, hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipStreamSynchronize(st));
+    memcpy(coefs_host, stage, sizeof(Fr) * (K + 1) * rounds);
+    return 0;
+}
+// The whole lookup sumcheck (tLookup_phase1 + tLookup_phase2, tlookup.cu:150-330) queued without a host round trip: the
+// fold challenges v (rounds x 8 limbs, in round order) are known up front.  A, S hold D elements, B, T, m hold N
+// (D/N a power of two: log2(D/N) phase-1 rounds, then phase-2 rounds), E holds D/2 (Montgomery form).  No input is
+// modified.  sums_host: rounds x 11 values ordered as zk_lookup_round orders them.
+int zk_lookup_sumcheck(uint32_t* sums_host, const void* A, const void* S, const void* B, const void* T, const void* m, const void* E, const uint32_t* beta,
+                       const uint32_t* v, size_t D, size_t N, int rounds, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(D >= 2 && N >= 1 && D % N == 0 && ((D / N) & (D / N - 1)) == 0, "zk_lookup_sumcheck: D must be N times a power of two");
+    ZK_ARG((D & (D - 1)) == 0, "zk_lookup_sumcheck: D must be a power of two");
+    ZK_ARG(rounds >= 1 && ((size_t)1 << rounds) <= D && rounds <= 40, "zk_lookup_sumcheck: bad round count");
+    ZK_ARG(sizeof(Fr) * 11 * (size_t)rounds <= 65536, "zk_lookup_sumcheck: too many rounds for the staging buffer");
+    int n1 = 0;
+    while (((size_t)N << n1) < D) ++n1;
+    Scratch sums(sizeof(Fr) * 11 * rounds), part(sizeof(Fr) * 11 * reduce_grid(D / 2));
+    if (sums.rc) return sums.rc;
+    if (part.rc) return part.rc;
+    ZK_HIP(hipMemsetAsync(sums.p, 0, sizeof(Fr) * 11 * rounds, st));
+    std::vector<std::unique_ptr<Scratch>> keep;
+    const Fr b = load_fr(beta);
+    const Fr *cA = (const Fr*)A, *cS = (const Fr*)S, *cB = (const Fr*)B, *cT = (const Fr*)T, *cm = (const Fr*)m, *cE = (const Fr*)E;
+    Fr* ownE = nullptr;
+    size_t cur = D;
+    for (int r = 0; r < rounds; ++r) {
+        const size_t half = cur >> 1;
+        const bool phase2 = r >= n1;
+        if (half <= (size_t)TAIL_HALF && rounds - r <= TAIL_ROUNDS) {
+            const int rest = rounds - r;
+            keep.emplace_back(new Scratch(sizeof(Fr) * 6 * half));
+            Scratch& work = *keep.back();
+            if (work.rc) return work.rc;
+            TailV vs;
+            for (int i = 0; i < TAIL_ROUNDS; ++i) vs.v[i] = i < rest ? to_mont(load_fr(v + 8 * (r + i))) : big_zero<8>();
+            Fr* w = work.as<Fr>();
+            hipLaunchKernelGGL(k_lookup_tail, dim3(1), dim3(TAIL_T), 0, st, sums.as<Fr>() + (size_t)r * 11, w, w + half, w + 2 * half, w + 3 * half, w + 4 * half, w + 5 * half,
+                               cA, cS, cB, cT, cm, cE, b, vs, (uint32_t)half, (uint32_t)rest, (uint32_t)(phase2 ? 0 : n1 - r));
+            ZK_LAUNCH_CHECK();
+            break;
+        }
+        keep.emplace_back(new Scratch(sizeof(Fr) * half * (phase2 ? 5 : 2)));
+        Scratch& nx = *keep.back();
+        if (nx.rc) return nx.rc;
+        Fr* w = nx.as<Fr>();
+        const unsigned nb = reduce_grid(half);
+        const Fr vm = to_mont(load_fr(v + 8 * r));
+        if (phase2)
+            hipLaunchKernelGGL(k_lookup_round<true>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, w + 2 * half, w + 3 * half, w + 4 * half, cA, cS, cB, cT, cm, cE, b, vm, half);
+        else
+            hipLaunchKernelGGL(k_lookup_round<false>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, cA, cS, (const Fr*)nullptr,
+                               (const Fr*)nullptr, (const Fr*)nullptr, cE, b, vm, half);
+        hipLaunchKernelGGL(k_finish, dim3(phase2 ? 11 : 5), dim3(TPB), 0, st, sums.as<Fr>() + (size_t)r * 11, part.as<Fr>(), nb);
+        ZK_LAUNCH_CHECK();
+        cA = w; cS = w + half;
+        if (phase2) { cB = w + 2 * half; cT = w + 3 * half; cm = w + 4 * half; }
+        cur = half;
+        if (r + 1 < rounds) {
+            const size_t nh = half >> 1;
+            if (!ownE) {
+                keep.emplace_back(new Scratch(sizeof(Fr) * (nh ? nh : 1)));
+                if (keep.back()->rc) return keep.back()->rc;
+                ownE = keep.back()->as<Fr>();
+            }
+            LAUNCH1D(k_eq_halve, nh, st, ownE, cE, nh);       // in place after the first halving: lane t reads t and t + nh, writes t
+            cE = ownE;
+        }
+    }
+    void* stage = nullptr;
+    int rc = staging(&stage, sizeof(Fr) * 11 * rounds);
+    if (rc) return rc;
+    ZK_HIP(hipMemcpyAsync(stage, sums.p, sizeof(Fr) * 11 * rounds, hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipStreamSynchronize(st));
+    Fr* out = (Fr*)sums_host;
+    const Fr* in = (const Fr*)stage;
+    for (int r = 0; r < rounds; ++r)
+        for (int i = 0; i < 11; ++i) {
+            Fr x = in[r * 11 + i];
+            if (i != 3 && i != 4) x = to_mont(x);        // E carries R, each product one R^-1: the same correction as zk_lookup_round
+            if (r < n1 && i >= 5) x = big_zero<8>();
+            memcpy(&out[r * 11 + i], &x, sizeof(Fr));
+        }
+    return 0;
+}
+// The whole multi-Hadamard sumcheck (proof.cu:191-241) queued without a host round trip.  Xs: K tensors of N elements
+// (N a power of two), E: N/2 elements (Montgomery form), v: log2(N) fold challenges in round order.  coefs_host:
+// log2(N) x (K+1) coefficients.  No input is modified.
+int zk_hadamard_sumcheck(uint32_t* coefs_host, const void* const* Xs, int K, const void* E, const uint32_t* v, size_t N, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(K >= 1 && K <= 4, "zk_hadamard_sumcheck: K must be 1..4");
+    ZK_ARG(N >= 2 && (N & (N - 1)) == 0, "zk_hadamard_sumcheck: N must be a power of two >= 2");
+    int rounds = 0;
+    while (((size_t)1 << rounds) < N) ++rounds;
+    ZK_ARG(sizeof(Fr) * (K + 1) * (size_t)rounds <= 65536, "zk_hadamard_sumcheck: too many rounds for the staging buffer");
+    Scratch sums(sizeof(Fr) * (K + 1) * rounds), part(sizeof(Fr) * (K + 1) * reduce_grid(N / 2));
+    if (sums.rc) return sums.rc;
+    if (part.rc) return part.rc;
+    std::vector<std::unique_ptr<Scratch>> keep;
+    const Fr* cur[4];
+    for (int i = 0; i < K; ++i) cur[i] = (const Fr*)Xs[i];
+    const Fr* cE = (const Fr*)E;
+    Fr* ownE = nullptr;
+    size_t n = N;
+    for (int r = 0; r < rounds; ++r) {
+        const size_t half = n >> 1;
+        if (half <= (size_t)TAIL_HALF && rounds - r <= TAIL_ROUNDS) {
+            const int rest = rounds - r;
+            keep.emplace_back(new Scratch(sizeof(Fr) * (K + 1) * half));
+            Scratch& work = *keep.back();
+            if (work.rc) return work.rc;
+            TailV vs;
+            for (int i = 0; i < TAIL_ROUNDS; ++i) vs.v[i] = i < rest ? to_mont(load_fr(v + 8 * (r + i))) : big_zero<8>();
+            Fr* w = work.as<Fr>();
+            Fr* so = sums.as<Fr>() + (size_t)r * (K + 1);
+#define HADS_TAIL(KK)                                                                                                                       \
+    case KK: {                                                                                                                              \
+        PtrPack<KK> p;                                                                                                                      \
+        for (int i = 0; i < KK; ++i) { p.in[i] = cur[i]; p.out[i] = w + (size_t)i * half; }                                                  \
+        hipLaunchKernelGGL(k_hadamard_tail<KK>, dim3(1), dim3(TAIL_T), 0, st, so, p, w + (size_t)KK * half, cE, vs, (uint32_t)half, (uint32_t)rest); \
+        break;                                                                                                                              \
+    }
+            switch (K) { HADS_TAIL(1) HADS_TAIL(2) HADS_TAIL(3) HADS_TAIL(4) }
+#undef HADS_TAIL
+            ZK_LAUNCH_CHECK();
+            break;
+        }
+        keep.emplace_back(new Scratch(sizeof(Fr) * half * K));
+        Scratch& nx = *keep.back();
+        if (nx.rc) return nx.rc;
+        Fr* w = nx.as<Fr>();
+        const unsigned nb = reduce_grid(half);
+        const Fr vm = to_mont(load_fr(v + 8 * r));
+#define HADS_ROUND(KK)                                                                                                            \
+    case KK: {                                                                                                                    \
+        PtrPack<KK> p;                                                                                                            \
+        for (int i = 0; i < KK; ++i) { p.in[i] = cur[i]; p.out[i] = w + (size_t)i * half; }                                        \
+        hipLaunchKernelGGL(k_hadamard_round<KK>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), p, cE, vm, half);                      \
+        break;                                                                                                                    \
+    }
+        switch (K) { HADS_ROUND(1) HADS_ROUND(2) HADS_ROUND(3) HADS_ROUND(4) }
+#undef HADS_ROUND
+        hipLaunchKernelGGL(k_finish, dim3(K + 1), dim3(TPB), 0, st, sums.as<Fr>() + (size_t)r * (K + 1), part.as<Fr>(), nb);
+        ZK_LAUNCH_CHECK();
+        for (int i = 0; i < K; ++i) cur[i] = w + (size_t)i * half;
+        n = half;
+        if (r + 1 < rounds) {
+            const size_t nh = half >> 1;
+            if (!ownE) {
+                keep.emplace_back(new Scratch(sizeof(Fr) * (nh ? nh : 1)));
+                if (keep.back()->rc) return keep.back()->rc;
+                ownE = keep.back()->as<Fr>();
+            }
+            LAUNCH1D(k_eq_halve, nh, st, ownE, cE, nh);
+            cE = ownE;
+        }
+    }
     void* stage = nullptr;
     int rc = staging(&stage, sizeof(Fr) * (K + 1) * rounds);
     if (rc) return rc;

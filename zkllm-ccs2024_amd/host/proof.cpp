@@ -68,8 +68,7 @@ Fr_t multi_hadamard_sumchecks(const Fr_t& claim0, const vector<FrTensor>& Xs, co
     const uint k = ceilLog2(N);
     if (u.size() != k || v.size() != k) throw std::runtime_error("multi_hadamard_sumchecks: need ceilLog2(N) challenges");
     Fr_t claim = claim0;
-    std::vector<FrTensor> keep, E;
-    keep.reserve((size_t)K * k);
+    std::vector<FrTensor> E;
     E.emplace_back(1u << (k - 1));
     ZKC(zk_eq_table(E.back().gpu_data, u[0].val, (int)k - 1, nullptr));
     std::vector<const void*> cur(K);
@@ -82,28 +81,12 @@ Fr_t multi_hadamard_sumchecks(const Fr_t& claim0, const vector<FrTensor>& Xs, co
         if (claim != p(kZero) + p(kOne)) throw std::runtime_error("multi_hadamard_sumchecks: claim != p(0) + p(1)");
         claim = proof.back()(v[k - 1 - r]);
     };
-    for (uint r = 0; r < k; ++r) {
-        const uint half = N >> (r + 1);
-        if (half <= 512 && k - r <= 16) {
-            // short tensors: every remaining round in one launch (the challenges are all known), the host work afterwards
-            const uint rest = k - r;
-            std::vector<Fr_t> vs(rest), sums((size_t)rest * (K + 1));
-            for (uint i = 0; i < rest; ++i) vs[i] = v[k - 1 - (r + i)];
-            ZKC(zk_hadamard_rounds_tail(sums[0].val, cur.data(), (int)K, E.back().gpu_data, vs[0].val, half, (int)rest, nullptr));
-            for (uint i = 0; i < rest; ++i) absorb(r + i, &sums[(size_t)i * (K + 1)]);
-            break;
-        }
-        std::vector<void*> nxt(K);
-        for (uint i = 0; i < K; ++i) { keep.emplace_back(half); nxt[i] = keep.back().gpu_data; }
-        std::vector<Fr_t> coefs(K + 1);
-        ZKC(zk_hadamard_round(coefs[0].val, nxt.data(), cur.data(), (int)K, E.back().gpu_data, v[k - 1 - r].val, half, nullptr));
-        absorb(r, coefs.data());
-        for (uint i = 0; i < K; ++i) cur[i] = nxt[i];
-        if (r + 1 < k) {
-            const uint next = half >> 1;
-            E.emplace_back(next ? next : 1);
-            ZKC(zk_eq_halve(E.back().gpu_data, E[E.size() - 2].gpu_data, next, nullptr));
-        }
+    // every round on the device back to back (the challenges are all known), then the host side of each round
+    {
+        std::vector<Fr_t> vs(k), sums((size_t)k * (K + 1));
+        for (uint r = 0; r < k; ++r) vs[r] = v[k - 1 - r];
+        ZKC(zk_hadamard_sumcheck(sums[0].val, cur.data(), (int)K, E.back().gpu_data, vs[0].val, N, nullptr));
+        for (uint r = 0; r < k; ++r) absorb(r, &sums[(size_t)r * (K + 1)]);
     }
     return claim;
 }

@@ -98,9 +98,6 @@ Fr_t tLookup_sumcheck(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0
     E.emplace_back(1u << (k - 1));
     ZKC(zk_eq_table(E.back().gpu_data, u[0].val, (int)k - 1, nullptr));
 
-    // working copies (ping-pong): cur -> next
-    std::vector<FrTensor> keep;
-    keep.reserve(5 * k + 8);
     const FrTensor *cA = &A, *cS = &S0, *cB = &B, *cT = &T0, *cm = &m0;
     auto challenge_of = [&](uint r) -> const Fr_t& {
         // v1 = v[0..n1) consumed from its back, then v2 = v[n1..k) from its back
@@ -132,41 +129,12 @@ Fr_t tLookup_sumcheck(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0
         if (phase2) alpha_sq = alpha_sq * e;
         else C = C * TWO_INV;
     };
-    for (uint r = 0; r < k; ++r) {
-        const bool phase2 = r >= n1;
-        const uint cur = cA->size, half = cur >> 1;
-        if (half <= 512 && k - r <= 16) {
-            // short tensors: every remaining round in one launch, the host work afterwards
-            const uint rest = k - r;
-            std::vector<Fr_t> vs(rest), sums((size_t)rest * 11);
-            for (uint i = 0; i < rest; ++i) vs[i] = challenge_of(r + i);
-            ZKC(zk_lookup_rounds_tail(sums[0].val, cA->gpu_data, cS->gpu_data, cB->gpu_data, cT->gpu_data, cm->gpu_data, E.back().gpu_data, beta.val, vs[0].val, half,
-                                      (int)rest, phase2 ? 0 : (int)(n1 - r), nullptr));
-            for (uint i = 0; i < rest; ++i) absorb(r + i, &sums[(size_t)i * 11]);
-            break;
-        }
-        const Fr_t& vr = challenge_of(r);
-        keep.emplace_back(half); FrTensor* nA = &keep.back();
-        keep.emplace_back(half); FrTensor* nS = &keep.back();
-        FrTensor *nB = nullptr, *nT = nullptr, *nm = nullptr;
-        if (phase2) {
-            keep.emplace_back(half); nB = &keep.back();
-            keep.emplace_back(half); nT = &keep.back();
-            keep.emplace_back(half); nm = &keep.back();
-        }
-        Fr_t s[11];
-        ZKC(zk_lookup_round(s[0].val, nA->gpu_data, nS->gpu_data, phase2 ? nB->gpu_data : nullptr, phase2 ? nT->gpu_data : nullptr, phase2 ? nm->gpu_data : nullptr,
-                            cA->gpu_data, cS->gpu_data, phase2 ? cB->gpu_data : nullptr, phase2 ? cT->gpu_data : nullptr, phase2 ? cm->gpu_data : nullptr,
-                            E.back().gpu_data, beta.val, vr.val, half, phase2 ? 1 : 0, nullptr));
-        absorb(r, s);
-        cA = nA; cS = nS;
-        if (phase2) { cB = nB; cT = nT; cm = nm; }
-        if (r + 1 < k) {
-            const uint next_half = half >> 1;   // next round pairs (t, t + next_half)
-            E.emplace_back(next_half ? next_half : 1);
-            FrTensor& prev = E[E.size() - 2];
-            ZKC(zk_eq_halve(E.back().gpu_data, prev.gpu_data, next_half, nullptr));
-        }
+    // every round on the device back to back (the fold challenges are all known), then the host side of each round
+    {
+        std::vector<Fr_t> vs(k), sums((size_t)k * 11);
+        for (uint r = 0; r < k; ++r) vs[r] = challenge_of(r);
+        ZKC(zk_lookup_sumcheck(sums[0].val, cA->gpu_data, cS->gpu_data, cB->gpu_data, cT->gpu_data, cm->gpu_data, E.back().gpu_data, beta.val, vs[0].val, D, N, (int)k, nullptr));
+        for (uint r = 0; r < k; ++r) absorb(r, &sums[(size_t)r * 11]);
     }
     zk_record(claim);
     return claim;
