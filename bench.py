@@ -84,7 +84,7 @@ def main():
     saved_stdout = os.dup(1)
     os.dup2(devnull, 1)      # the class layer prints the reference's progress lines ("Opening complete", ...)
     try:
-        parts = np.zeros(7)
+        parts = np.zeros(8)
         for _ in range(args.warmup):
             pv.layer_run(layer, hX)
         pv.sync()
@@ -120,7 +120,7 @@ def main():
         "config": {"workload": f"C5: LLaMa-2-7B-shape decoder layer proof, seq {seq}, hidden 4096, 32 heads x 128, FFN 11008, "
                                "random-init fixed-point weights (scale 2^16), generators of size out_features<<5, all nine weight openings included",
                    "setup_s_untimed": round(setup_s, 3),
-                   "parts_ms": {k: round(float(v), 1) for k, v in zip(["rmsnorm1", "qkv", "attention", "oproj", "rmsnorm2", "ffn", "total"], parts)}},
+                   "parts_ms": {k: round(float(v), 1) for k, v in zip(["rmsnorm1", "qkv", "attention", "oproj", "rmsnorm2", "ffn", "total", "open_wait"], parts)}},
     }
     # roofline of the kernel with the largest share of the layer's GPU time: the generator fold of the openings
     # (one endomorphism-split scalar multiplication per pair).  It is bound by 32-bit integer multiply-adds: an

@@ -173,6 +173,15 @@ int zk_hadamard_rounds_tail(uint32_t* coefs_host, const void* const* Xs, int K, 
 int zk_lookup_sumcheck(uint32_t* sums_host, const void* A, const void* S, const void* B, const void* T, const void* m, const void* E, const uint32_t* beta,
                        const uint32_t* v, size_t D, size_t N, int rounds, void* stream);
 int zk_hadamard_sumcheck(uint32_t* coefs_host, const void* const* Xs, int K, const void* E, const uint32_t* v, size_t N, void* stream);
+/* the device side of a lookup proof / a multi-Hadamard proof as a job on a stream of the library's own, beside the
+ * caller's stream (ordered after what `stream` holds at begin).  The lookup job also computes A = 1/(S+beta),
+ * B = 1/(T+beta) (tlookup_inv_kernel tlookup.cu:337-352), <B, m> and the eq table of u_eq (rounds-1 challenges).
+ * Inputs must stay alive and unmodified until end; every handle must be ended exactly once.  bm_host: <B, m>, 8 limbs. */
+int zk_lookup_prove_begin(void** handle, const void* S, const void* T, const void* m, const uint32_t* beta, const uint32_t* u_eq, const uint32_t* v, size_t D, size_t N,
+                          int rounds, void* stream);
+int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host);
+int zk_hadamard_prove_begin(void** handle, const void* const* Xs, int K, const uint32_t* u_eq, const uint32_t* v, size_t N, void* stream);
+int zk_hadamard_prove_end(void* handle, uint32_t* coefs_host);
 
 /* ---- rescaling / softmax ------------------------------------------------------------------------------------------ */
 int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* stream);       /* rescaling_kernel rescaling.cu:8-21 */

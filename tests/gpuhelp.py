@@ -372,7 +372,7 @@ class Prover:
         return h
 
     def layer_run(self, layer, X):
-        times = np.zeros(7, np.float64)
+        times = np.zeros(8, np.float64)
         out = self.H(self.lib.zkp_layer_run(c_void_p(layer), c_void_p(X.h), _np_ptr(times)))
         return out, times
 

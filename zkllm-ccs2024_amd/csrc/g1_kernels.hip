@@ -11,6 +11,7 @@
 // per-pair doublings and no materialised m*n temporary (the reference writes 144 B per pair).
 // All of it is VALU integer work on 12-limb Fp; results equal the reference's as group elements
 // (a Jacobian triple depends on the order of additions, so bytes are compared after normalising).
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <utility>
@@ -584,13 +585,6 @@ static int g1_sum_device(G1Jac* out, const G1Jac* in, size_t n, hipStream_t st) 
     return 0;
 }
 
-// Device buffers of one opening, all released together once its stream has drained: an opening may run on a
-// stream of its own, so none of its buffers may return to the allocator while its kernels are pending.
-struct Arena {
-    std::vector<std::unique_ptr<Scratch>> v;
-    Scratch& add(size_t bytes) { v.emplace_back(new Scratch(bytes)); return *v.back(); }
-};
-
 // Optional timing of the fold kernel's launches with events on its own stream (measurement only).
 struct FoldTimer {
     bool on = false;
@@ -974,15 +968,6 @@ static int open_collect(OpenJob& job, uint32_t* proof_host, uint32_t* final_scal
     memcpy(final_scalar_host, (char*)stage + sizeof(G1Jac) * npts, sizeof(Fr));
     return 0;
 }
-// streams for openings that run beside the caller's stream (default priority, not synchronising with the null stream)
-static hipStream_t side_stream() {
-    static hipStream_t streams[4] = {nullptr, nullptr, nullptr, nullptr};
-    static unsigned next = 0;
-    const unsigned i = next++ % 4;
-    if (!streams[i] && hipStreamCreateWithFlags(&streams[i], hipStreamNonBlocking) != hipSuccess) return nullptr;
-    return streams[i];
-}
-
 // proof_host receives 3*rounds + 1 points: T, T0, T1 of every round, then the folded generator; all normalised to
 // z = 1 (infinity: all-zero limbs).  final_scalar_host: the folded scalar.
 int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stv) {
@@ -996,7 +981,7 @@ int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* sc
 // must stay alive and unmodified until end, which waits for the opening, delivers its results and releases its buffers.
 int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stv) {
     ZK_ARG(handle != nullptr, "zk_g1_open_begin: null handle");
-    hipStream_t side = side_stream();
+    hipStream_t side = side_stream(0);
     ZK_ARG(side != nullptr, "zk_g1_open_begin: could not create a stream");
     std::unique_ptr<OpenJob> job(new OpenJob);
     ZK_HIP(hipEventCreateWithFlags(&job->ready, hipEventDisableTiming));

@@ -743,26 +743,49 @@ int zk_hadamard_rounds_tail(uint32_t* coefs_host, const void* const* Xs, int K, 
     memcpy(coefs_host, stage, sizeof(Fr) * (K + 1) * rounds);
     return 0;
 }
-// The whole lookup sumcheck (tLookup_phase1 + tLookup_phase2, tlookup.cu:150-330) queued without a host round trip: the
-// fold challenges v (rounds x 8 limbs, in round order) are known up front.  A, S hold D elements, B, T, m hold N
-// (D/N a power of two: log2(D/N) phase-1 rounds, then phase-2 rounds), E holds D/2 (Montgomery form).  No input is
-// modified.  sums_host: rounds x 11 values ordered as zk_lookup_round orders them.
-int zk_lookup_sumcheck(uint32_t* sums_host, const void* A, const void* S, const void* B, const void* T, const void* m, const void* E, const uint32_t* beta,
-                       const uint32_t* v, size_t D, size_t N, int rounds, void* stv) {
-    hipStream_t st = (hipStream_t)stv;
-    ZK_ARG(D >= 2 && N >= 1 && D % N == 0 && ((D / N) & (D / N - 1)) == 0, "zk_lookup_sumcheck: D must be N times a power of two");
-    ZK_ARG((D & (D - 1)) == 0, "zk_lookup_sumcheck: D must be a power of two");
-    ZK_ARG(rounds >= 1 && ((size_t)1 << rounds) <= D && rounds <= 40, "zk_lookup_sumcheck: bad round count");
-    ZK_ARG(sizeof(Fr) * 11 * (size_t)rounds <= 65536, "zk_lookup_sumcheck: too many rounds for the staging buffer");
+// ---- whole sumchecks as jobs ---------------------------------------------------------------------------------------------------
+// A job queues every kernel of a sumcheck on one stream without a host round trip (the challenges are known up front),
+// keeps its buffers until the results have been fetched, and can run on a stream of the library's own beside the caller.
+struct SumJob {
+    Arena arena;
+    hipStream_t st = nullptr;
+    Fr* sums = nullptr;          // rounds x per_round values
+    Fr* extra = nullptr;         // one more value fetched with the sums (lookup: <B, m> with R^-1 attached), or null
+    int rounds = 0, per_round = 0, n1 = 0;
+    hipEvent_t ready = nullptr;
+};
+__global__ void __launch_bounds__(TPB) k_dot_part(Fr* __restrict__ partials, const Fr* __restrict__ a, const Fr* __restrict__ b, size_t n) {
+    Fr acc[1] = {big_zero<8>()};
+    for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (size_t)gridDim.x * TPB) acc[0] = add(acc[0], mont_mul(a[i], b[i]));
+    block_reduce_store<1>(acc, partials);
+}
+__global__ void k_set_one_mont(Fr* __restrict__ e) { if (threadIdx.x == 0 && blockIdx.x == 0) e[0] = big_one_mont<8>(); }
+// eq table of k challenges into out (2^k elements, Montgomery form), all on the stream
+static void eq_table_queue(Fr* out, const uint32_t* u, int k, hipStream_t st) {
+    hipLaunchKernelGGL(k_set_one_mont, dim3(1), dim3(64), 0, st, out);
+    Fr one = big_zero<8>();
+    one.v[0] = 1;
+    for (int j = 0; j < k; ++j) {
+        const Fr uj = load_fr(u + 8 * j);
+        const size_t half = (size_t)1 << j;
+        hipLaunchKernelGGL(k_eq_double, dim3(cdiv(half, TPB)), dim3(TPB), 0, st, out, to_mont(uj), to_mont(sub(one, uj)), half);
+    }
+}
+// all rounds of the lookup sumcheck; sums land in job.sums
+static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, const Fr* T, const Fr* m, const Fr* E, const Fr& b, const uint32_t* v, size_t D, size_t N, int rounds) {
+    hipStream_t st = job.st;
     int n1 = 0;
     while (((size_t)N << n1) < D) ++n1;
-    Scratch sums(sizeof(Fr) * 11 * rounds), part(sizeof(Fr) * 11 * reduce_grid(D / 2));
+    job.rounds = rounds;
+    job.per_round = 11;
+    job.n1 = n1;
+    Scratch& sums = job.arena.add(sizeof(Fr) * 11 * rounds);
+    Scratch& part = job.arena.add(sizeof(Fr) * 11 * reduce_grid(D / 2));
     if (sums.rc) return sums.rc;
     if (part.rc) return part.rc;
+    job.sums = sums.as<Fr>();
     ZK_HIP(hipMemsetAsync(sums.p, 0, sizeof(Fr) * 11 * rounds, st));
-    std::vector<std::unique_ptr<Scratch>> keep;
-    const Fr b = load_fr(beta);
-    const Fr *cA = (const Fr*)A, *cS = (const Fr*)S, *cB = (const Fr*)B, *cT = (const Fr*)T, *cm = (const Fr*)m, *cE = (const Fr*)E;
+    const Fr *cA = A, *cS = S, *cB = B, *cT = T, *cm = m, *cE = E;
     Fr* ownE = nullptr;
     size_t cur = D;
     for (int r = 0; r < rounds; ++r) {
@@ -770,8 +793,7 @@ int zk_lookup_sumcheck(uint32_t* sums_host, const void* A, const void* S, const 
         const bool phase2 = r >= n1;
         if (half <= (size_t)TAIL_HALF && rounds - r <= TAIL_ROUNDS) {
             const int rest = rounds - r;
-            keep.emplace_back(new Scratch(sizeof(Fr) * 6 * half));
-            Scratch& work = *keep.back();
+            Scratch& work = job.arena.add(sizeof(Fr) * 6 * half);
             if (work.rc) return work.rc;
             TailV vs;
             for (int i = 0; i < TAIL_ROUNDS; ++i) vs.v[i] = i < rest ? to_mont(load_fr(v + 8 * (r + i))) : big_zero<8>();
@@ -781,8 +803,7 @@ int zk_lookup_sumcheck(uint32_t* sums_host, const void* A, const void* S, const 
             ZK_LAUNCH_CHECK();
             break;
         }
-        keep.emplace_back(new Scratch(sizeof(Fr) * half * (phase2 ? 5 : 2)));
-        Scratch& nx = *keep.back();
+        Scratch& nx = job.arena.add(sizeof(Fr) * half * (phase2 ? 5 : 2));
         if (nx.rc) return nx.rc;
         Fr* w = nx.as<Fr>();
         const unsigned nb = reduce_grid(half);
@@ -800,55 +821,37 @@ int zk_lookup_sumcheck(uint32_t* sums_host, const void* A, const void* S, const 
         if (r + 1 < rounds) {
             const size_t nh = half >> 1;
             if (!ownE) {
-                keep.emplace_back(new Scratch(sizeof(Fr) * (nh ? nh : 1)));
-                if (keep.back()->rc) return keep.back()->rc;
-                ownE = keep.back()->as<Fr>();
+                Scratch& e = job.arena.add(sizeof(Fr) * (nh ? nh : 1));
+                if (e.rc) return e.rc;
+                ownE = e.as<Fr>();
             }
             LAUNCH1D(k_eq_halve, nh, st, ownE, cE, nh);       // in place after the first halving: lane t reads t and t + nh, writes t
             cE = ownE;
         }
     }
-    void* stage = nullptr;
-    int rc = staging(&stage, sizeof(Fr) * 11 * rounds);
-    if (rc) return rc;
-    ZK_HIP(hipMemcpyAsync(stage, sums.p, sizeof(Fr) * 11 * rounds, hipMemcpyDeviceToHost, st));
-    ZK_HIP(hipStreamSynchronize(st));
-    Fr* out = (Fr*)sums_host;
-    const Fr* in = (const Fr*)stage;
-    for (int r = 0; r < rounds; ++r)
-        for (int i = 0; i < 11; ++i) {
-            Fr x = in[r * 11 + i];
-            if (i != 3 && i != 4) x = to_mont(x);        // E carries R, each product one R^-1: the same correction as zk_lookup_round
-            if (r < n1 && i >= 5) x = big_zero<8>();
-            memcpy(&out[r * 11 + i], &x, sizeof(Fr));
-        }
     return 0;
 }
-// The whole multi-Hadamard sumcheck (proof.cu:191-241) queued without a host round trip.  Xs: K tensors of N elements
-// (N a power of two), E: N/2 elements (Montgomery form), v: log2(N) fold challenges in round order.  coefs_host:
-// log2(N) x (K+1) coefficients.  No input is modified.
-int zk_hadamard_sumcheck(uint32_t* coefs_host, const void* const* Xs, int K, const void* E, const uint32_t* v, size_t N, void* stv) {
-    hipStream_t st = (hipStream_t)stv;
-    ZK_ARG(K >= 1 && K <= 4, "zk_hadamard_sumcheck: K must be 1..4");
-    ZK_ARG(N >= 2 && (N & (N - 1)) == 0, "zk_hadamard_sumcheck: N must be a power of two >= 2");
+static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, const uint32_t* v, size_t N) {
+    hipStream_t st = job.st;
     int rounds = 0;
     while (((size_t)1 << rounds) < N) ++rounds;
-    ZK_ARG(sizeof(Fr) * (K + 1) * (size_t)rounds <= 65536, "zk_hadamard_sumcheck: too many rounds for the staging buffer");
-    Scratch sums(sizeof(Fr) * (K + 1) * rounds), part(sizeof(Fr) * (K + 1) * reduce_grid(N / 2));
+    job.rounds = rounds;
+    job.per_round = K + 1;
+    Scratch& sums = job.arena.add(sizeof(Fr) * (K + 1) * rounds);
+    Scratch& part = job.arena.add(sizeof(Fr) * (K + 1) * reduce_grid(N / 2));
     if (sums.rc) return sums.rc;
     if (part.rc) return part.rc;
-    std::vector<std::unique_ptr<Scratch>> keep;
+    job.sums = sums.as<Fr>();
     const Fr* cur[4];
-    for (int i = 0; i < K; ++i) cur[i] = (const Fr*)Xs[i];
-    const Fr* cE = (const Fr*)E;
+    for (int i = 0; i < K; ++i) cur[i] = Xs[i];
+    const Fr* cE = E;
     Fr* ownE = nullptr;
     size_t n = N;
     for (int r = 0; r < rounds; ++r) {
         const size_t half = n >> 1;
         if (half <= (size_t)TAIL_HALF && rounds - r <= TAIL_ROUNDS) {
             const int rest = rounds - r;
-            keep.emplace_back(new Scratch(sizeof(Fr) * (K + 1) * half));
-            Scratch& work = *keep.back();
+            Scratch& work = job.arena.add(sizeof(Fr) * (K + 1) * half);
             if (work.rc) return work.rc;
             TailV vs;
             for (int i = 0; i < TAIL_ROUNDS; ++i) vs.v[i] = i < rest ? to_mont(load_fr(v + 8 * (r + i))) : big_zero<8>();
@@ -866,8 +869,7 @@ int zk_hadamard_sumcheck(uint32_t* coefs_host, const void* const* Xs, int K, con
             ZK_LAUNCH_CHECK();
             break;
         }
-        keep.emplace_back(new Scratch(sizeof(Fr) * half * K));
-        Scratch& nx = *keep.back();
+        Scratch& nx = job.arena.add(sizeof(Fr) * half * K);
         if (nx.rc) return nx.rc;
         Fr* w = nx.as<Fr>();
         const unsigned nb = reduce_grid(half);
@@ -888,21 +890,158 @@ int zk_hadamard_sumcheck(uint32_t* coefs_host, const void* const* Xs, int K, con
         if (r + 1 < rounds) {
             const size_t nh = half >> 1;
             if (!ownE) {
-                keep.emplace_back(new Scratch(sizeof(Fr) * (nh ? nh : 1)));
-                if (keep.back()->rc) return keep.back()->rc;
-                ownE = keep.back()->as<Fr>();
+                Scratch& e = job.arena.add(sizeof(Fr) * (nh ? nh : 1));
+                if (e.rc) return e.rc;
+                ownE = e.as<Fr>();
             }
             LAUNCH1D(k_eq_halve, nh, st, ownE, cE, nh);
             cE = ownE;
         }
     }
-    void* stage = nullptr;
-    int rc = staging(&stage, sizeof(Fr) * (K + 1) * rounds);
-    if (rc) return rc;
-    ZK_HIP(hipMemcpyAsync(stage, sums.p, sizeof(Fr) * (K + 1) * rounds, hipMemcpyDeviceToHost, st));
-    ZK_HIP(hipStreamSynchronize(st));
-    memcpy(coefs_host, stage, sizeof(Fr) * (K + 1) * rounds);
     return 0;
+}
+// waits for the job's stream and copies its sums (and the extra value) to the host
+static int sumjob_collect(SumJob& job, Fr* sums_host, Fr* extra_host) {
+    const size_t nsum = (size_t)job.rounds * job.per_round;
+    void* stage = nullptr;
+    int rc = staging(&stage, sizeof(Fr) * (nsum + 1));
+    if (rc) return rc;
+    ZK_HIP(hipMemcpyAsync(stage, job.sums, sizeof(Fr) * nsum, hipMemcpyDeviceToHost, job.st));
+    if (job.extra) ZK_HIP(hipMemcpyAsync((Fr*)stage + nsum, job.extra, sizeof(Fr), hipMemcpyDeviceToHost, job.st));
+    ZK_HIP(hipStreamSynchronize(job.st));
+    memcpy(sums_host, stage, sizeof(Fr) * nsum);
+    if (job.extra && extra_host) memcpy(extra_host, (Fr*)stage + nsum, sizeof(Fr));
+    return 0;
+}
+// the R corrections of the lookup sums: E carries R, each product one R^-1 (same as zk_lookup_round)
+static void lookup_fix_sums(Fr* s, int rounds, int n1) {
+    for (int r = 0; r < rounds; ++r)
+        for (int i = 0; i < 11; ++i) {
+            Fr& x = s[r * 11 + i];
+            if (i != 3 && i != 4) x = to_mont(x);
+            if (r < n1 && i >= 5) x = big_zero<8>();
+        }
+}
+static int lookup_args_ok(size_t D, size_t N, int rounds) {
+    ZK_ARG(D >= 2 && N >= 1 && D % N == 0 && ((D / N) & (D / N - 1)) == 0, "lookup sumcheck: D must be N times a power of two");
+    ZK_ARG((D & (D - 1)) == 0, "lookup sumcheck: D must be a power of two");
+    ZK_ARG(rounds >= 1 && ((size_t)1 << rounds) <= D && rounds <= 40, "lookup sumcheck: bad round count");
+    ZK_ARG(sizeof(Fr) * (11 * (size_t)rounds + 1) <= 65536, "lookup sumcheck: too many rounds for the staging buffer");
+    return 0;
+}
+// puts a new job on one of the library's streams, ordered after everything queued on `caller` so far
+static int sumjob_on_side_stream(SumJob& job, hipStream_t caller) {
+    job.st = side_stream(1);
+    ZK_ARG(job.st != nullptr, "could not create a stream");
+    ZK_HIP(hipEventCreateWithFlags(&job.ready, hipEventDisableTiming));
+    ZK_HIP(hipEventRecord(job.ready, caller));
+    ZK_HIP(hipStreamWaitEvent(job.st, job.ready, 0));
+    return 0;
+}
+static void sumjob_abort(SumJob* job) {
+    if (job->st) (void)hipStreamSynchronize(job->st);
+    if (job->ready) (void)hipEventDestroy(job->ready);
+    delete job;
+}
+
+// The whole lookup sumcheck (tLookup_phase1 + tLookup_phase2, tlookup.cu:150-330) queued without a host round trip: the
+// fold challenges v (rounds x 8 limbs, in round order) are known up front.  A, S hold D elements, B, T, m hold N
+// (D/N a power of two: log2(D/N) phase-1 rounds, then phase-2 rounds), E holds D/2 (Montgomery form).  No input is
+// modified.  sums_host: rounds x 11 values ordered as zk_lookup_round orders them.
+int zk_lookup_sumcheck(uint32_t* sums_host, const void* A, const void* S, const void* B, const void* T, const void* m, const void* E, const uint32_t* beta,
+                       const uint32_t* v, size_t D, size_t N, int rounds, void* stv) {
+    int rc = lookup_args_ok(D, N, rounds);
+    if (rc) return rc;
+    SumJob job;
+    job.st = (hipStream_t)stv;
+    rc = lookup_queue(job, (const Fr*)A, (const Fr*)S, (const Fr*)B, (const Fr*)T, (const Fr*)m, (const Fr*)E, load_fr(beta), v, D, N, rounds);
+    if (rc) { (void)hipStreamSynchronize(job.st); return rc; }
+    rc = sumjob_collect(job, (Fr*)sums_host, nullptr);
+    if (rc) return rc;
+    lookup_fix_sums((Fr*)sums_host, rounds, job.n1);
+    return 0;
+}
+// The device side of tLookup's proof (tlookup.cu:150-330) as one job beside the caller's stream: A = 1/(S + beta),
+// B = 1/(T + beta), <B, m>, the eq table of u_eq (rounds - 1 challenges), then every round.  S: D elements; T, m: N.
+// begin returns at once; S, T, m must stay alive and unmodified until end, which waits and delivers <B, m>
+// (standard form) and the rounds x 11 sums.  Every handle must be ended exactly once.
+int zk_lookup_prove_begin(void** handle, const void* S, const void* T, const void* m, const uint32_t* beta, const uint32_t* u_eq, const uint32_t* v, size_t D, size_t N,
+                          int rounds, void* stv) {
+    ZK_ARG(handle != nullptr, "zk_lookup_prove_begin: null handle");
+    int rc = lookup_args_ok(D, N, rounds);
+    if (rc) return rc;
+    SumJob* job = new SumJob;
+    rc = sumjob_on_side_stream(*job, (hipStream_t)stv);
+    if (rc) { sumjob_abort(job); return rc; }
+    hipStream_t st = job->st;
+    Scratch& A = job->arena.add(sizeof(Fr) * D);
+    Scratch& B = job->arena.add(sizeof(Fr) * N);
+    Scratch& E = job->arena.add(sizeof(Fr) * (D / 2));
+    Scratch& dp = job->arena.add(sizeof(Fr) * (reduce_grid(N) + 1));
+    if (A.rc || B.rc || E.rc || dp.rc) { rc = A.rc ? A.rc : (B.rc ? B.rc : (E.rc ? E.rc : dp.rc)); sumjob_abort(job); return rc; }
+    const Fr b = load_fr(beta);
+    hipLaunchKernelGGL(k_batch_inv, dim3(cdiv(D, (size_t)BI_T * BI_CH)), dim3(BI_T), 0, st, A.as<Fr>(), (const Fr*)S, b, D);
+    hipLaunchKernelGGL(k_batch_inv, dim3(cdiv(N, (size_t)BI_T * BI_CH)), dim3(BI_T), 0, st, B.as<Fr>(), (const Fr*)T, b, N);
+    const unsigned nb = reduce_grid(N);
+    hipLaunchKernelGGL(k_dot_part, dim3(nb), dim3(TPB), 0, st, dp.as<Fr>() + 1, B.as<Fr>(), (const Fr*)m, N);
+    hipLaunchKernelGGL(k_finish, dim3(1), dim3(TPB), 0, st, dp.as<Fr>(), dp.as<Fr>() + 1, nb);
+    job->extra = dp.as<Fr>();
+    eq_table_queue(E.as<Fr>(), u_eq, rounds - 1, st);
+    rc = lookup_queue(*job, A.as<Fr>(), (const Fr*)S, B.as<Fr>(), (const Fr*)T, (const Fr*)m, E.as<Fr>(), b, v, D, N, rounds);
+    if (rc) { sumjob_abort(job); return rc; }
+    *handle = job;
+    return 0;
+}
+int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host) {
+    ZK_ARG(handle != nullptr, "zk_lookup_prove_end: null handle");
+    SumJob* job = (SumJob*)handle;
+    Fr bm = big_zero<8>();
+    int rc = sumjob_collect(*job, (Fr*)sums_host, &bm);
+    if (!rc) {
+        lookup_fix_sums((Fr*)sums_host, job->rounds, job->n1);
+        bm = to_mont(bm);          // the products carried R^-1
+        memcpy(bm_host, &bm, sizeof(Fr));
+    }
+    sumjob_abort(job);
+    return rc;
+}
+// The whole multi-Hadamard sumcheck (proof.cu:191-241) queued without a host round trip.  Xs: K tensors of N elements
+// (N a power of two), E: N/2 elements (Montgomery form), v: log2(N) fold challenges in round order.  coefs_host:
+// log2(N) x (K+1) coefficients.  No input is modified.
+int zk_hadamard_sumcheck(uint32_t* coefs_host, const void* const* Xs, int K, const void* E, const uint32_t* v, size_t N, void* stv) {
+    ZK_ARG(K >= 1 && K <= 4, "zk_hadamard_sumcheck: K must be 1..4");
+    ZK_ARG(N >= 2 && (N & (N - 1)) == 0, "zk_hadamard_sumcheck: N must be a power of two >= 2");
+    SumJob job;
+    job.st = (hipStream_t)stv;
+    int rc = hadamard_queue(job, (const Fr* const*)Xs, K, (const Fr*)E, v, N);
+    if (rc) { (void)hipStreamSynchronize(job.st); return rc; }
+    return sumjob_collect(job, (Fr*)coefs_host, nullptr);
+}
+// The same beside the caller's stream, eq table of u_eq (log2(N) - 1 challenges) included.  Xs must stay alive and
+// unmodified until end; every handle must be ended exactly once.
+int zk_hadamard_prove_begin(void** handle, const void* const* Xs, int K, const uint32_t* u_eq, const uint32_t* v, size_t N, void* stv) {
+    ZK_ARG(handle != nullptr, "zk_hadamard_prove_begin: null handle");
+    ZK_ARG(K >= 1 && K <= 4, "zk_hadamard_prove_begin: K must be 1..4");
+    ZK_ARG(N >= 2 && (N & (N - 1)) == 0, "zk_hadamard_prove_begin: N must be a power of two >= 2");
+    SumJob* job = new SumJob;
+    int rc = sumjob_on_side_stream(*job, (hipStream_t)stv);
+    if (rc) { sumjob_abort(job); return rc; }
+    Scratch& E = job->arena.add(sizeof(Fr) * (N / 2));
+    if (E.rc) { rc = E.rc; sumjob_abort(job); return rc; }
+    int k = 0;
+    while (((size_t)1 << k) < N) ++k;
+    eq_table_queue(E.as<Fr>(), u_eq, k - 1, job->st);
+    rc = hadamard_queue(*job, (const Fr* const*)Xs, K, E.as<Fr>(), v, N);
+    if (rc) { sumjob_abort(job); return rc; }
+    *handle = job;
+    return 0;
+}
+int zk_hadamard_prove_end(void* handle, uint32_t* coefs_host) {
+    ZK_ARG(handle != nullptr, "zk_hadamard_prove_end: null handle");
+    SumJob* job = (SumJob*)handle;
+    int rc = sumjob_collect(*job, (Fr*)coefs_host, nullptr);
+    sumjob_abort(job);
+    return rc;
 }
 int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* st) {
     ZK_ARG(scaling_factor >= 1, "zk_rescale: scaling factor is 0");

@@ -1,4 +1,5 @@
 // Runtime pieces of the C ABI: device selection, the caching allocator, copies, error text.
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <unordered_map>
@@ -93,6 +94,23 @@ int pool_trim() {
     if (!victims.empty()) (void)hipDeviceSynchronize();
     for (void* p : victims) (void)hipFree(p);
     return 0;
+}
+
+hipStream_t side_stream(int pool) {
+    static hipStream_t streams[2][8] = {};
+    static unsigned next[2] = {0, 0};
+    static int count[2] = {0, 0}, shared = 0;
+    if (!count[0]) {
+        count[0] = 2; count[1] = 2;       // measured on the 7B layer: more streams only move time between the blocks and the final wait
+        if (const char* e = getenv("ZKLLM_SIDE_STREAMS")) {          // "openings,sumchecks[,shared]" (experiments)
+            int a = 0, b2 = 0, c = 0;
+            if (sscanf(e, "%d,%d,%d", &a, &b2, &c) >= 2 && a >= 1 && a <= 8 && b2 >= 1 && b2 <= 8) { count[0] = a; count[1] = b2; shared = c; }
+        }
+    }
+    const int q = (pool && !shared) ? 1 : 0;
+    const unsigned i = next[q]++ % (unsigned)count[q];
+    if (!streams[q][i] && hipStreamCreateWithFlags(&streams[q][i], hipStreamNonBlocking) != hipSuccess) { (void)hipGetLastError(); streams[q][i] = nullptr; return nullptr; }
+    return streams[q][i];
 }
 
 int staging(void** host_ptr, size_t bytes) {

@@ -1,6 +1,8 @@
 // Internal runtime helpers shared by the .hip translation units: error capture, the caching
 // device allocator behind zk_malloc/zk_free, and a pinned staging area for small results.
 #pragma once
+#include <memory>
+#include <vector>
 #include <cstddef>
 #include <cstdint>
 #include <string>
@@ -46,6 +48,16 @@ struct Scratch {
     Scratch(const Scratch&) = delete;
     Scratch& operator=(const Scratch&) = delete;
 };
+
+// Device buffers of one job that may run on a stream of its own: all released together once that stream has drained,
+// so none of them returns to the allocator while the job's kernels are pending.
+struct Arena {
+    std::vector<std::unique_ptr<Scratch>> v;
+    Scratch& add(size_t bytes) { v.emplace_back(new Scratch(bytes)); return *v.back(); }
+};
+// One of the library's own streams (non-blocking, default priority), handed out round-robin; null on failure.
+// Two pools, so that a short job (pool 1: sumchecks) never queues behind a long one (pool 0: openings).
+hipStream_t side_stream(int pool);
 
 // Pinned host buffer (64 KiB) for device->host results of reductions.
 int staging(void** host_ptr, size_t bytes);

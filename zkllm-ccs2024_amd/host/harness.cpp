@@ -386,13 +386,13 @@ void* zkp_layer_create_random(const u32* cu, const double* cf, u32 seed, u32 log
 }
 void zkp_layer_free(void* h) { delete reinterpret_cast<LayerState*>(h); }
 void zkp_layer_set_open_weights(void* h, int on) { reinterpret_cast<LayerState*>(h)->cfg.open_weights = on != 0; }
-// runs the whole layer (compute + every proof); times_ms: rmsnorm1, qkv, attention, oproj, rmsnorm2, ffn, total
+// runs the whole layer (compute + every proof); times_ms (8 values): rmsnorm1, qkv, attention, oproj, rmsnorm2, ffn, total, open_wait
 void* zkp_layer_run(void* h, void* X, double* times_ms) {
     ZKP_TRY
     LayerState& s = *reinterpret_cast<LayerState*>(h);
     LayerTimes t;
     FrTensor out = llama_layer(s.cfg, s.w, FT(X), &t);
-    if (times_ms) { times_ms[0] = t.rmsnorm1; times_ms[1] = t.qkv; times_ms[2] = t.attention; times_ms[3] = t.oproj; times_ms[4] = t.rmsnorm2; times_ms[5] = t.ffn; times_ms[6] = t.total; }
+    if (times_ms) { times_ms[0] = t.rmsnorm1; times_ms[1] = t.qkv; times_ms[2] = t.attention; times_ms[3] = t.oproj; times_ms[4] = t.rmsnorm2; times_ms[5] = t.ffn; times_ms[6] = t.total; times_ms[7] = t.open_wait; }
     return new FrTensor(std::move(out));
     ZKP_END_PTR
 }

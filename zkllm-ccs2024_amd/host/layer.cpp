@@ -211,9 +211,10 @@ FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor
     const double t5 = now_ms();
     FrTensor f = ffn_block(c, w.up, w.gate, w.down, w.swiglu_table, n2);
     FrTensor out = x2 + f;
-    openings.finish();
     const double t6 = now_ms();
-    t.rmsnorm1 = t1 - t0; t.qkv = t2 - t1; t.attention = t3 - t2; t.oproj = t4 - t3; t.rmsnorm2 = t5 - t4; t.ffn = t6 - t5; t.total = t6 - t0;
+    openings.finish();
+    const double t7 = now_ms();
+    t.rmsnorm1 = t1 - t0; t.qkv = t2 - t1; t.attention = t3 - t2; t.oproj = t4 - t3; t.rmsnorm2 = t5 - t4; t.ffn = t6 - t5; t.open_wait = t7 - t6; t.total = t7 - t0;
     if (times) *times = t;
     return out;
 }

@@ -43,8 +43,9 @@ struct LayerWeights {
     FrTensor swiglu_table;        // swiglu_len mapped values
 };
 
-struct LayerTimes {               // milliseconds, wall clock with the device idle at both ends
-    double rmsnorm1 = 0, qkv = 0, attention = 0, oproj = 0, rmsnorm2 = 0, ffn = 0, total = 0;
+struct LayerTimes {               // milliseconds, wall clock with the caller's stream idle at both ends; weight openings run beside the blocks,
+                                  // open_wait is what is left of them after the last block
+    double rmsnorm1 = 0, qkv = 0, attention = 0, oproj = 0, rmsnorm2 = 0, ffn = 0, total = 0, open_wait = 0;
 };
 
 // rms_inv = round(scale / sqrt(mean((x/scale)^2) + eps)) per row, scale = 2^16 in the reference (llama-rmsnorm.py:35-39), host double

@@ -56,39 +56,53 @@ void verifyWeightClaim(const Weight& w, const Claim& c) {
 static const Fr_t kZero{{0, 0, 0, 0, 0, 0, 0, 0}};
 static const Fr_t kOne{{1, 0, 0, 0, 0, 0, 0, 0}};
 
-// proof.cu:191-241.  Each round is one pass over the tensors: the K+1 coefficient evaluations (inner
-// products with the eq table of u[:-1]) and the folds by v.back().
-Fr_t multi_hadamard_sumchecks(const Fr_t& claim0, const vector<FrTensor>& Xs, const vector<Fr_t>& u, const vector<Fr_t>& v, vector<Polynomial>& proof) {
-    uint N = Xs[0].size;
-    if (N == 1) return claim0;
+// proof.cu:191-241.  Each round is one pass over the tensors: the K+1 coefficient evaluations (inner products with
+// the eq table of u[:-1]) and the folds by v.back().  The device side is one job that runs beside the caller.
+HadamardPending::~HadamardPending() {
+    if (!handle) return;
+    std::vector<Fr_t> sums((size_t)(K + 1) * 40 + 1);
+    (void)zk_hadamard_prove_end(handle, sums[0].val);
+}
+HadamardPending multi_hadamard_begin(const Fr_t& claim0, const vector<FrTensor>& Xs, const vector<Fr_t>& u, const vector<Fr_t>& v) {
+    HadamardPending p;
+    p.claim = claim0; p.u = u; p.v = v;
+    const uint N = Xs[0].size;
+    p.N = N;
+    p.K = (uint)Xs.size();
+    if (N == 1) return p;
     if ((N & (N - 1)) != 0) throw std::runtime_error("N is not a power of 2");
-    const uint K = (uint)Xs.size();
-    if (K > 4) throw std::runtime_error("multi_hadamard_sumchecks: at most 4 factors are supported");
+    if (p.K > 4) throw std::runtime_error("multi_hadamard_sumchecks: at most 4 factors are supported");
     for (auto& X : Xs) if (X.size != N) throw std::runtime_error("Xs[i] size is not N");
     const uint k = ceilLog2(N);
     if (u.size() != k || v.size() != k) throw std::runtime_error("multi_hadamard_sumchecks: need ceilLog2(N) challenges");
-    Fr_t claim = claim0;
-    std::vector<FrTensor> E;
-    E.emplace_back(1u << (k - 1));
-    ZKC(zk_eq_table(E.back().gpu_data, u[0].val, (int)k - 1, nullptr));
-    std::vector<const void*> cur(K);
-    for (uint i = 0; i < K; ++i) cur[i] = Xs[i].gpu_data;
-    auto absorb = [&](uint r, const Fr_t* c) {
-        std::vector<Fr_t> coefs(c, c + K + 1);
+    std::vector<const void*> cur(p.K);
+    for (uint i = 0; i < p.K; ++i) cur[i] = Xs[i].gpu_data;
+    std::vector<Fr_t> vs(k);
+    for (uint r = 0; r < k; ++r) vs[r] = v[k - 1 - r];
+    ZKC(zk_hadamard_prove_begin(&p.handle, cur.data(), (int)p.K, u[0].val, vs[0].val, N, nullptr));
+    return p;
+}
+Fr_t multi_hadamard_end(HadamardPending& pd, vector<Polynomial>& proof) {
+    if (pd.N == 1) return pd.claim;
+    const uint K = pd.K, k = ceilLog2(pd.N);
+    std::vector<Fr_t> sums((size_t)k * (K + 1));
+    void* h = pd.handle;
+    pd.handle = nullptr;
+    ZKC(zk_hadamard_prove_end(h, sums[0].val));
+    Fr_t claim = pd.claim;
+    for (uint r = 0; r < k; ++r) {
+        std::vector<Fr_t> coefs(sums.begin() + (size_t)r * (K + 1), sums.begin() + (size_t)(r + 1) * (K + 1));
         proof.push_back(Polynomial(coefs));
         zk_record(coefs);
-        Polynomial p = proof.back() * Polynomial::eq(u[k - 1 - r]);
+        Polynomial p = proof.back() * Polynomial::eq(pd.u[k - 1 - r]);
         if (claim != p(kZero) + p(kOne)) throw std::runtime_error("multi_hadamard_sumchecks: claim != p(0) + p(1)");
-        claim = proof.back()(v[k - 1 - r]);
-    };
-    // every round on the device back to back (the challenges are all known), then the host side of each round
-    {
-        std::vector<Fr_t> vs(k), sums((size_t)k * (K + 1));
-        for (uint r = 0; r < k; ++r) vs[r] = v[k - 1 - r];
-        ZKC(zk_hadamard_sumcheck(sums[0].val, cur.data(), (int)K, E.back().gpu_data, vs[0].val, N, nullptr));
-        for (uint r = 0; r < k; ++r) absorb(r, &sums[(size_t)r * (K + 1)]);
+        claim = proof.back()(pd.v[k - 1 - r]);
     }
     return claim;
+}
+Fr_t multi_hadamard_sumchecks(const Fr_t& claim0, const vector<FrTensor>& Xs, const vector<Fr_t>& u, const vector<Fr_t>& v, vector<Polynomial>& proof) {
+    HadamardPending p = multi_hadamard_begin(claim0, Xs, u, v);
+    return multi_hadamard_end(p, proof);
 }
 
 // ---- deprecated sumchecks (proof.cu:12-157): adjacent-pair folding, first challenge first -------------------

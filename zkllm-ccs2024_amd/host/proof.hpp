@@ -36,3 +36,17 @@ vector<Fr_t> hadamard_product_sumcheck(const FrTensor& a, const FrTensor& b, vec
 vector<Fr_t> binary_sumcheck(const FrTensor& a, vector<Fr_t> u, vector<Fr_t> v);
 
 Fr_t multi_hadamard_sumchecks(const Fr_t& claim, const vector<FrTensor>& Xs, const vector<Fr_t>& u, const vector<Fr_t>& v, vector<Polynomial>& proof);
+// the same in two halves: begin queues the device side beside the caller (Xs must stay alive until end), end does the host side
+struct HadamardPending {
+    HadamardPending() = default;
+    HadamardPending(HadamardPending&& o) noexcept : handle(o.handle), claim(o.claim), u(std::move(o.u)), v(std::move(o.v)), K(o.K), N(o.N) { o.handle = nullptr; }
+    HadamardPending(const HadamardPending&) = delete;
+    HadamardPending& operator=(const HadamardPending&) = delete;
+    ~HadamardPending();               // a job that was never ended is waited for and dropped
+    void* handle = nullptr;
+    Fr_t claim;
+    vector<Fr_t> u, v;
+    uint K = 0, N = 0;
+};
+HadamardPending multi_hadamard_begin(const Fr_t& claim, const vector<FrTensor>& Xs, const vector<Fr_t>& u, const vector<Fr_t>& v);
+Fr_t multi_hadamard_end(HadamardPending& p, vector<Polynomial>& proof);

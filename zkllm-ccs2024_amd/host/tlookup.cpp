@@ -69,45 +69,68 @@ pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const FrTensor& vals) {
     return {std::move(y), std::move(m)};
 }
 
-// tLookup_phase1 / tLookup_phase2 (tlookup.cu:184-320) as one loop.  Each round is a single pass over the
-// current tensors that yields all sums of the round polynomial and the folded tensors.
-Fr_t tLookup_sumcheck(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0, const Fr_t& alpha0, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v) {
+static void drop_lookup_job(void* h, size_t rounds) {
+    if (!h) return;
+    std::vector<Fr_t> sums(rounds * 11 + 1);
+    Fr_t bm;
+    (void)zk_lookup_prove_end(h, bm.val, sums[0].val);
+}
+LookupPending::~LookupPending() { drop_lookup_job(handle, u.size()); }
+LookupPending& LookupPending::operator=(LookupPending&& o) noexcept {
+    if (this != &o) {
+        drop_lookup_job(handle, u.size());
+        handle = o.handle; o.handle = nullptr;
+        keep = std::move(o.keep);
+        alpha = o.alpha; beta = o.beta;
+        u = std::move(o.u); v = std::move(o.v);
+        D = o.D; N = o.N;
+    }
+    return *this;
+}
+
+// tLookup_phase1 / tLookup_phase2 (tlookup.cu:184-320).  The device side -- inverses, <B, m>, eq table and every round --
+// is one job that runs beside the caller; the host side turns each round's sums into its polynomial, checks it and
+// derives the next claim.
+LookupPending tLookup_sumcheck_begin(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0, const Fr_t& alpha0, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v) {
     const uint D = S0.size, N = m0.size;
     if (m0.size != T0.size) throw std::runtime_error("m.size != table.size");
     if (D != (1u << ceilLog2(D)) || N != (1u << ceilLog2(N)) || D % N != 0) throw std::runtime_error("D or N is not power of 2, or D is not divisible by N");
     if (u.size() != ceilLog2(D)) throw std::runtime_error("u.size() != ceilLog2(D)");
     if (v.size() != ceilLog2(D)) throw std::runtime_error("v.size() != ceilLog2(D)");
+    LookupPending p;
+    p.alpha = alpha0; p.beta = beta; p.u = u; p.v = v; p.D = D; p.N = N;
+    const uint k = (uint)u.size();
+    if (k == 0) return p;
+    const uint n1 = ceilLog2(D / N);
+    // fold challenges in round order: v1 = v[0..n1) consumed from its back, then v2 = v[n1..k) from its back
+    std::vector<Fr_t> vs(k);
+    for (uint r = 0; r < k; ++r) vs[r] = r >= n1 ? v[k - 1 - (r - n1)] : v[n1 - 1 - r];
+    ZKC(zk_lookup_prove_begin(&p.handle, S0.gpu_data, T0.gpu_data, m0.gpu_data, beta.val, u[0].val, vs[0].val, D, N, (int)k, nullptr));
+    return p;
+}
 
-    FrTensor A(D), B(N);
-    ZKC(zk_fr_batch_inv(A.gpu_data, S0.gpu_data, beta.val, D, nullptr));
-    ZKC(zk_fr_batch_inv(B.gpu_data, T0.gpu_data, beta.val, N, nullptr));
-
+Fr_t tLookup_sumcheck_end(LookupPending& pd) {
+    const uint D = pd.D, N = pd.N;
+    const vector<Fr_t>&u = pd.u, &v = pd.v;
     const uint n1 = ceilLog2(D / N);               // phase-1 rounds
     const uint k = (uint)u.size();
-    Fr_t bm;
-    ZKC(zk_fr_dot(bm.val, B.gpu_data, m0.gpu_data, N, nullptr));
-    Fr_t alpha = alpha0;
-    Fr_t alpha_sq = alpha0 * alpha0;
-    Fr_t C = alpha_sq - bm;
-    Fr_t claim = alpha0 + alpha_sq;
-    const Fr_t inv_ratio = Fr_t{{N, 0, 0, 0, 0, 0, 0, 0}} / Fr_t{{D, 0, 0, 0, 0, 0, 0, 0}};
+    Fr_t alpha = pd.alpha;
+    Fr_t alpha_sq = pd.alpha * pd.alpha;
+    Fr_t claim = pd.alpha + alpha_sq;
     if (k == 0) { zk_record(claim); return claim; }
-
-    // eq table over u[0 .. k-2], halved after every round
-    std::vector<FrTensor> E;
-    E.emplace_back(1u << (k - 1));
-    ZKC(zk_eq_table(E.back().gpu_data, u[0].val, (int)k - 1, nullptr));
-
-    const FrTensor *cA = &A, *cS = &S0, *cB = &B, *cT = &T0, *cm = &m0;
-    auto challenge_of = [&](uint r) -> const Fr_t& {
-        // v1 = v[0..n1) consumed from its back, then v2 = v[n1..k) from its back
-        return r >= n1 ? v[k - 1 - (r - n1)] : v[n1 - 1 - r];
-    };
-    // host side of a round: the round polynomial from the device's sums, the check, the next claim
-    auto absorb = [&](uint r, const Fr_t* s) {
+    Fr_t bm;
+    std::vector<Fr_t> sums((size_t)k * 11);
+    void* h = pd.handle;
+    pd.handle = nullptr;
+    ZKC(zk_lookup_prove_end(h, bm.val, sums[0].val));
+    pd.keep.clear();
+    Fr_t C = alpha_sq - bm;
+    const Fr_t inv_ratio = Fr_t{{N, 0, 0, 0, 0, 0, 0, 0}} / Fr_t{{D, 0, 0, 0, 0, 0, 0, 0}};
+    for (uint r = 0; r < k; ++r) {
+        const Fr_t* s = &sums[(size_t)r * 11];
         const bool phase2 = r >= n1;
         const Fr_t& ub = u[k - 1 - r];
-        const Fr_t& vr = challenge_of(r);
+        const Fr_t& vr = phase2 ? v[k - 1 - (r - n1)] : v[n1 - 1 - r];
         Polynomial p;
         if (!phase2) {
             Polynomial p0({alpha * s[0], alpha * s[1], alpha * s[2]});
@@ -128,16 +151,48 @@ Fr_t tLookup_sumcheck(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0
         alpha = alpha * e;
         if (phase2) alpha_sq = alpha_sq * e;
         else C = C * TWO_INV;
-    };
-    // every round on the device back to back (the fold challenges are all known), then the host side of each round
-    {
-        std::vector<Fr_t> vs(k), sums((size_t)k * 11);
-        for (uint r = 0; r < k; ++r) vs[r] = challenge_of(r);
-        ZKC(zk_lookup_sumcheck(sums[0].val, cA->gpu_data, cS->gpu_data, cB->gpu_data, cT->gpu_data, cm->gpu_data, E.back().gpu_data, beta.val, vs[0].val, D, N, (int)k, nullptr));
-        for (uint r = 0; r < k; ++r) absorb(r, &sums[(size_t)r * 11]);
     }
     zk_record(claim);
     return claim;
+}
+
+Fr_t tLookup_sumcheck(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0, const Fr_t& alpha0, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v) {
+    LookupPending p = tLookup_sumcheck_begin(S0, T0, m0, alpha0, beta, u, v);
+    return tLookup_sumcheck_end(p);
+}
+
+LookupPending tLookup::prove_begin(const FrTensor& S, const FrTensor& m, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v) {
+    if (m.size != table.size) throw std::runtime_error("m.size != table.size");
+    return tLookup_sumcheck_begin(S, table, m, alpha, beta, u, v);
+}
+
+LookupPending tLookupRangeMapping::prove_begin(const FrTensor& S_in, const FrTensor& S_out, const FrTensor& m, const Fr_t& r, const Fr_t& alpha, const Fr_t& beta,
+                                               const vector<Fr_t>& u, const vector<Fr_t>& v) {
+    const uint D = S_in.size;
+    if (m.size != table.size) throw std::runtime_error("m.size != table.size");
+    std::vector<std::unique_ptr<FrTensor>> keep;
+    const FrTensor *si = &S_in, *so = &S_out, *mm = &m;
+    if (D != (1u << ceilLog2(D))) {
+        // pad the queries with the first table entry and account for them in m[0] (tlookup.cu:502-510)
+        keep.emplace_back(new FrTensor(S_in.pad({D}, table(0))));
+        si = keep.back().get();
+        keep.emplace_back(new FrTensor(S_out.pad({D}, mapped_vals(0))));
+        so = keep.back().get();
+        keep.emplace_back(new FrTensor(m));
+        FrTensor* m_ = keep.back().get();
+        Fr_t m0 = (*m_)(0) + Fr_t{{(1u << ceilLog2(D)) - D, 0, 0, 0, 0, 0, 0, 0}};
+        ZKC(zk_memcpy_h2d(m_->gpu_data, &m0, sizeof(Fr_t), nullptr));
+        mm = m_;
+    }
+    const uint N = mm->size;
+    if (N != (1u << ceilLog2(N)) || si->size % N != 0) throw std::runtime_error("N is not power of 2, or D is not divisible by N");
+    keep.emplace_back(new FrTensor(*si + *so * r));
+    const FrTensor* S_com = keep.back().get();
+    keep.emplace_back(new FrTensor(table + mapped_vals * r));
+    const FrTensor* T_com = keep.back().get();
+    LookupPending p = tLookup_sumcheck_begin(*S_com, *T_com, *mm, alpha, beta, u, v);
+    p.keep = std::move(keep);
+    return p;
 }
 
 Fr_t tLookup::prove(const FrTensor& S, const FrTensor& m, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v, vector<Polynomial>& proof) {
@@ -147,20 +202,6 @@ Fr_t tLookup::prove(const FrTensor& S, const FrTensor& m, const Fr_t& alpha, con
 
 Fr_t tLookupRangeMapping::prove(const FrTensor& S_in, const FrTensor& S_out, const FrTensor& m, const Fr_t& r, const Fr_t& alpha, const Fr_t& beta,
                                 const vector<Fr_t>& u, const vector<Fr_t>& v, vector<Polynomial>& proof) {
-    const uint D = S_in.size;
-    if (m.size != table.size) throw std::runtime_error("m.size != table.size");
-    if (D != (1u << ceilLog2(D))) {
-        // pad the queries with the first table entry and account for them in m[0] (tlookup.cu:502-510)
-        auto S_in_ = S_in.pad({D}, table(0));
-        auto S_out_ = S_out.pad({D}, mapped_vals(0));
-        FrTensor m_(m);
-        Fr_t m0 = m_(0) + Fr_t{{(1u << ceilLog2(D)) - D, 0, 0, 0, 0, 0, 0, 0}};
-        ZKC(zk_memcpy_h2d(m_.gpu_data, &m0, sizeof(Fr_t), nullptr));
-        return prove(S_in_, S_out_, m_, r, alpha, beta, u, v, proof);
-    }
-    const uint N = m.size;
-    if (N != (1u << ceilLog2(N)) || D % N != 0) throw std::runtime_error("N is not power of 2, or D is not divisible by N");
-    auto S_com = S_in + S_out * r;
-    auto T_com = table + mapped_vals * r;
-    return tLookup_sumcheck(S_com, T_com, m, alpha, beta, u, v);
+    LookupPending p = prove_begin(S_in, S_out, m, r, alpha, beta, u, v);
+    return tLookup_sumcheck_end(p);
 }

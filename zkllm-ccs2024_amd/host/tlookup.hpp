@@ -1,9 +1,28 @@
 // LogUp-style lookup argument (tlookup.cuh:11-52): generic table, integer range table, and range table
 // with mapped values.
 #pragma once
+#include <memory>
 #include "fr-tensor.hpp"
 #include "polynomial.hpp"
 #include "proof.hpp"
+
+// A lookup proof whose device side is running beside the caller (tLookup*::prove_begin); prove_end waits for it and does
+// the host side.  The tensors passed to prove_begin must stay alive until prove_end; temporaries made on the way live here.
+struct LookupPending {
+    LookupPending() = default;
+    LookupPending(LookupPending&& o) noexcept { *this = std::move(o); }
+    LookupPending& operator=(LookupPending&& o) noexcept;
+    LookupPending(const LookupPending&) = delete;
+    LookupPending& operator=(const LookupPending&) = delete;
+    ~LookupPending();                 // a job that was never ended (an exception on the way) is waited for and dropped
+    void* handle = nullptr;
+    std::vector<std::unique_ptr<FrTensor>> keep;
+    Fr_t alpha, beta;
+    vector<Fr_t> u, v;
+    uint D = 0, N = 0;
+};
+LookupPending tLookup_sumcheck_begin(const FrTensor& S, const FrTensor& T, const FrTensor& m, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v);
+Fr_t tLookup_sumcheck_end(LookupPending& p);
 
 class tLookup {
    public:
@@ -15,6 +34,9 @@ class tLookup {
     FrTensor prep(const uint* indices, const uint D);
 
     Fr_t prove(const FrTensor& S, const FrTensor& m, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v, vector<Polynomial>& proof);
+    // prove in two halves (same transcript): begin queues the device work beside the caller, end finishes the proof
+    LookupPending prove_begin(const FrTensor& S, const FrTensor& m, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v);
+    static Fr_t prove_end(LookupPending& p) { return tLookup_sumcheck_end(p); }
 };
 
 class tLookupRange : public tLookup {
@@ -26,6 +48,7 @@ class tLookupRange : public tLookup {
     FrTensor prep(const FrTensor& vals);
 
     using tLookup::prove;
+    using tLookup::prove_begin;
 };
 
 class tLookupRangeMapping : public tLookupRange {
@@ -40,6 +63,8 @@ class tLookupRangeMapping : public tLookupRange {
 
     Fr_t prove(const FrTensor& S_in, const FrTensor& S_out, const FrTensor& m, const Fr_t& r, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u,
                const vector<Fr_t>& v, vector<Polynomial>& proof);
+    LookupPending prove_begin(const FrTensor& S_in, const FrTensor& S_out, const FrTensor& m, const Fr_t& r, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u,
+                              const vector<Fr_t>& v);
 };
 
 // the sumcheck behind both prove() functions: T is the (possibly combined) table

@@ -78,10 +78,19 @@ Fr_t zkSoftmax::prove(const FrTensor& Y, const FrTensor& X, const FrTensor& shif
 
     auto claim_Y = Y(u_Y);
     zk_record(claim_Y);
-    multi_hadamard_sumchecks(claim_Y, Y_segments, u_Y, v_Y, proof);
-
-    for (uint i = 0; i < L; ++i) least_significant_segments[i].prove(X_segments[i], m_segments[i], alpha_seg, beta_seg, u_Y, v_Y, proof);
-    for (uint i = L; i < K; ++i) other_segments[i - L].prove(X_segments[i], Y_segments[i - L], m_segments[i], r_seg, alpha_seg, beta_seg, u_Y, v_Y, proof);
+    // The Hadamard sumcheck and the K segment lookups share nothing but their challenges: their device sides are queued
+    // together and run side by side; the host sides follow in the reference's order (zksoftmax.cu:177-187).
+    HadamardPending had = multi_hadamard_begin(claim_Y, Y_segments, u_Y, v_Y);
+    std::vector<LookupPending> looks;
+    looks.reserve(K);
+    for (uint i = 0; i < L; ++i) looks.push_back(least_significant_segments[i].prove_begin(X_segments[i], m_segments[i], alpha_seg, beta_seg, u_Y, v_Y));
+    for (uint i = L; i < K; ++i) looks.push_back(other_segments[i - L].prove_begin(X_segments[i], Y_segments[i - L], m_segments[i], r_seg, alpha_seg, beta_seg, u_Y, v_Y));
+    std::string failure;
+    try { multi_hadamard_end(had, proof); } catch (const std::exception& e) { failure = e.what(); }
+    for (auto& lp : looks) {
+        try { tLookup::prove_end(lp); } catch (const std::exception& e) { if (failure.empty()) failure = e.what(); }
+    }
+    if (!failure.empty()) throw std::runtime_error(failure);
 
     vector<Fr_t> Y_seg_claims, X_seg_claims;
     for (uint i = L; i < K; ++i) Y_seg_claims.push_back(Y_segments[i - L](v_Y));
