@@ -259,6 +259,66 @@ __device__ __forceinline__ Fp glv_beta() {
     for (int i = 0; i < 12; ++i) b.v[i] = t[i];
     return b;
 }
+__device__ __forceinline__ Fp glv_beta2() {   // beta^2 = -1 - beta
+    Fp b;
+    constexpr uint32_t t[12] = {2039112936u, 821114395u, 2127452714u, 4088978859u, 3323295735u, 380160570u, 1962738331u, 3261739000u, 1617960046u, 909555558u, 605774176u, 85697707u};
+#pragma unroll
+    for (int i = 0; i < 12; ++i) b.v[i] = t[i];
+    return b;
+}
+__device__ __forceinline__ Fp glv_minus2_over_beta_minus_1() {   // -2 / (beta - 1), Montgomery form
+    Fp b;
+    constexpr uint32_t t[12] = {72385493u, 4027593027u, 4077721914u, 4036542869u, 1636888181u, 235204061u, 17598343u, 35324347u, 360752738u, 1434563812u, 3508079257u, 43087383u};
+#pragma unroll
+    for (int i = 0; i < 12; ++i) b.v[i] = t[i];
+    return b;
+}
+// joint sparse form of (k1, k2): position i holds (d1 + 1) | (d2 + 1) << 2 in 4 bits, d in {-1, 0, 1}; len <= 129
+struct JsfK { uint32_t dig[17]; uint32_t len; };
+// 1 / v for every lane of a 64-lane workgroup with one field inversion: product tree up, inverse down (a child's
+// inverse is the parent's inverse times its sibling).  v must be non-zero (lanes with nothing to invert pass one).
+// lds: 12 x 128 words.
+__device__ __forceinline__ Fp block_inv64(const Fp& v, uint32_t (*lds)[2 * GT]) {
+    const uint32_t t = threadIdx.x;
+    auto put = [&](const Fp& x, uint32_t i) {
+#pragma unroll
+        for (int l = 0; l < 12; ++l) lds[l][i] = x.v[l];
+    };
+    auto get = [&](uint32_t i) {
+        Fp x;
+#pragma unroll
+        for (int l = 0; l < 12; ++l) x.v[l] = lds[l][i];
+        return x;
+    };
+    __syncthreads();
+    put(v, t);
+    __syncthreads();
+    uint32_t off = 0;
+    for (uint32_t cnt = GT / 2; cnt >= 1; cnt >>= 1) {
+        const uint32_t noff = off + 2 * cnt;
+        if (t < cnt) put(fp_mul(get(off + 2 * t), get(off + 2 * t + 1)), noff + t);
+        __syncthreads();
+        off = noff;
+    }
+    {
+        const Fp root_inv = mont_inverse(get(off));      // every lane the same value: no divergence
+        __syncthreads();
+        if (t == 0) put(root_inv, off);
+        __syncthreads();
+    }
+    for (uint32_t cnt = 1; cnt < (uint32_t)GT; cnt <<= 1) {
+        const uint32_t coff = off - 2 * cnt;
+        Fp c = big_one_mont<12>();
+        if (t < 2 * cnt) c = fp_mul(get(off + (t >> 1)), get(coff + (t ^ 1u)));
+        __syncthreads();
+        if (t < 2 * cnt) put(c, coff + t);
+        __syncthreads();
+        off = coff;
+    }
+    const Fp r = get(t);
+    __syncthreads();
+    return r;
+}
 // [k1]P + [k2]phi(P); every lane of a wave must carry the same k (the add pattern is uniform)
 static __device__ __attribute__((noinline)) G1Jac g1_mul_glv(const G1Jac& P, const GlvK& k) {
     if (is_zero(P.z)) return P;
@@ -445,7 +505,7 @@ struct OpenExtras {
     GlvK kc[3];
 };
 __global__ void __launch_bounds__(GT) k_open_fold(Fr* __restrict__ new_scalars, G1Jac* __restrict__ new_gens, const Fr* __restrict__ scalars, const G1Affine* __restrict__ A,
-                                                  const Fr u_mont, const GlvK ku, size_t old_size, size_t new_size, uint32_t nb_main, const OpenExtras ex) {
+                                                  const Fr u_mont, const GlvK ku, const JsfK jsf, size_t old_size, size_t new_size, uint32_t nb_main, const OpenExtras ex) {
     if (blockIdx.x >= nb_main) {
         if (threadIdx.x != 0) return;
         const uint32_t x = blockIdx.x - nb_main;
@@ -466,22 +526,75 @@ __global__ void __launch_bounds__(GT) k_open_fold(Fr* __restrict__ new_scalars, 
         }
         return;
     }
+    // ---- pair g: s' and g' = a1 + [u](a0 - a1) -------------------------------------------------------------------------------
+    // The scalar multiplication works on affine points throughout its table: D = a0 - a1 (one inversion, batched over
+    // the 64 lanes), phi(D) = (beta x, y), D + phi(D) = (beta^2 x, -y) (the three images of the endomorphism sum to zero) and
+    // D - phi(D) (a second batched inversion).  With the joint sparse form of (k1, k2) -- digits in {-1, 0, 1}, a non-zero
+    // pair in about half of the 129 positions -- the walk is one doubling per position and one mixed addition per
+    // non-zero pair.  Lanes whose inputs are special (infinity, equal abscissae, x = 0) take the general Jacobian route.
+    __shared__ uint32_t inv_lds[12][2 * GT];
     const size_t g = (size_t)blockIdx.x * GT + threadIdx.x;
-    if (g >= new_size) return;
+    const bool live = g < new_size;
     const size_t g0 = 2 * g, g1 = 2 * g + 1;
-    const G1Affine a0 = A[g0];
-    if (g1 >= old_size) {
-        new_scalars[g] = sub(scalars[g0], mont_mul(u_mont, scalars[g0]));
-        new_gens[g] = g1_mul_glv(aff_to_jac(a0), ku);
-        return;
+    const bool has1 = live && g1 < old_size;
+    G1Affine a0, a1;
+    a0.x = a0.y = a1.x = a1.y = big_zero<12>();
+    if (live) a0 = A[g0];
+    if (has1) a1 = A[g1];
+    if (live) {
+        if (has1) new_scalars[g] = add(scalars[g0], mont_mul(u_mont, sub(scalars[g1], scalars[g0])));
+        else new_scalars[g] = sub(scalars[g0], mont_mul(u_mont, scalars[g0]));
     }
-    new_scalars[g] = add(scalars[g0], mont_mul(u_mont, sub(scalars[g1], scalars[g0])));
-    const G1Affine a1 = A[g1];
-    G1Jac diff = aff_to_jac(a0);
-    if (!aff_is_inf(a1)) diff = g1_add_mixed(diff, g1_neg(a1));
-    G1Jac r = g1_mul_glv(diff, ku);
-    if (!aff_is_inf(a1)) r = g1_add_mixed(r, a1);
-    new_gens[g] = r;
+    const bool inf0 = aff_is_inf(a0), inf1 = !has1 || aff_is_inf(a1);
+    const Fp one_m = big_one_mont<12>();
+    // general = the old route; fast = everything regular
+    bool general = live && (inf0 || (!inf1 && equal(a0.x, a1.x)));
+    const bool need_sub = live && !general && !inf1;          // D = a0 - a1 needs 1 / (x0 - x1)
+    Fp den = need_sub ? sub(a0.x, a1.x) : one_m;
+    Fp inv = block_inv64(den, inv_lds);
+    G1Affine D = a0;
+    if (need_sub) {
+        const Fp lam = fp_mul(add(a0.y, a1.y), inv);          // -a1 = (x1, -y1)
+        D.x = sub(sub(fp_sqr(lam), a0.x), a1.x);
+        D.y = sub(fp_mul(lam, sub(a0.x, D.x)), a0.y);
+    }
+    if (live && !general && is_zero(D.x)) general = true;       // x = 0: not in the subgroup; the table below would divide by it
+    const bool fast = live && !general;
+    den = fast ? D.x : one_m;
+    inv = block_inv64(den, inv_lds);
+    G1Jac r = g1_infinity();
+    if (fast) {
+        const Fp beta = glv_beta(), beta2 = glv_beta2();
+        G1Affine Q, PQ, PmQ;
+        Q.x = fp_mul(D.x, beta); Q.y = D.y;
+        PQ.x = fp_mul(D.x, beta2); PQ.y = neg(D.y);
+        {
+            const Fp lam = fp_mul(fp_mul(glv_minus2_over_beta_minus_1(), D.y), inv);   // slope of D + (beta x, -y)
+            PmQ.x = add(fp_sqr(lam), PQ.x);
+            PmQ.y = sub(fp_mul(lam, sub(D.x, PmQ.x)), D.y);
+        }
+        for (int i = (int)jsf.len - 1; i >= 0; --i) {
+            r = g1_double(r);
+            const uint32_t dg = (jsf.dig[i >> 3] >> ((i & 7) * 4)) & 0xFu;    // (d1 + 1) | (d2 + 1) << 2, the same for every lane
+            const int d1 = (int)(dg & 3u) - 1, d2 = (int)(dg >> 2) - 1;
+            if (d1 == 0 && d2 == 0) continue;
+            G1Affine t;
+            bool ng;
+            if (d2 == 0) { t = D; ng = d1 < 0; }
+            else if (d1 == 0) { t = Q; ng = d2 < 0; }
+            else if (d1 == d2) { t = PQ; ng = d1 < 0; }
+            else { t = PmQ; ng = d1 < 0; }
+            if (ng) t.y = neg(t.y);
+            r = g1_add_mixed(r, t);
+        }
+        if (!inf1) r = g1_add_mixed(r, a1);
+    } else if (general) {
+        G1Jac diff = aff_to_jac(a0);
+        if (!inf1) diff = g1_add_mixed(diff, g1_neg(a1));
+        r = g1_mul_glv(diff, ku);
+        if (!inf1) r = g1_add_mixed(r, a1);
+    }
+    if (live) new_gens[g] = r;
 }
 // ---- the last rounds in one batch ---------------------------------------------------------------------------------------
 // Once n0 <= TAIL_N generators are left, every later round's generators are fixed linear combinations of these n0
@@ -593,16 +706,12 @@ struct FoldTimer {
     unsigned long long pairs = 0;
 };
 static FoldTimer g_fold_timer;
-// Fp multiplications of one pair of the fold: difference (11), endomorphism (1), P+Q (16), the double-and-add walk
-// (7 per doubling from the top set bit, 16 per non-zero bit pair), final mixed addition (11), two 8-limb products aside
-static double fold_fp_mults_per_pair(const GlvK& k) {
-    int top = -1, adds = 0;
-    for (int i = 127; i >= 0; --i) {
-        const uint32_t b = ((k.k1[i >> 5] >> (i & 31)) & 1u) | ((k.k2[i >> 5] >> (i & 31)) & 1u);
-        if (b && top < 0) top = i;
-        adds += (int)b;
-    }
-    return 11.0 + 1.0 + 16.0 + 7.0 * (top + 1) + 16.0 * adds + 11.0;
+// Fp multiplications of one pair of the fold by the formulas' count (two 8-limb products aside)
+static double fold_fp_mults_per_pair(const JsfK& j) {
+    int adds = 0;
+    for (uint32_t i = 0; i < j.len; ++i) adds += (((j.dig[i >> 3] >> ((i & 7) * 4)) & 0xFu) != 5u) ? 1 : 0;    // 5 = both digits zero
+    // difference (4), its share of two batched inversions (6), table (7), doublings (7 each), mixed additions (11 each), final addition (11)
+    return 4.0 + 6.0 + 7.0 + 7.0 * j.len + 11.0 * adds + 11.0;
 }
 
 // u = k1 + k2 * lambda with 0 <= k1 < lambda and k2 <= lambda + 1 (r = lambda^2 + lambda + 1): one long division
@@ -619,6 +728,29 @@ static GlvK glv_split(const Fr& u) {
     for (int i = 0; i < 4; ++i) { k.k1[i] = (uint32_t)(rem >> (32 * i)); k.k2[i] = (uint32_t)(q >> (32 * i)); }
     return k;
 }
+// joint sparse form of the two halves of a split scalar (Solinas): the fewest non-zero digit pairs among signed binary forms
+static JsfK jsf_of(const GlvK& k) {
+    unsigned __int128 a = 0, b = 0;
+    for (int i = 3; i >= 0; --i) { a = (a << 32) | k.k1[i]; b = (b << 32) | k.k2[i]; }
+    JsfK out;
+    memset(&out, 0, sizeof(out));
+    unsigned d1 = 0, d2 = 0, len = 0;
+    while (a + d1 > 0 || b + d2 > 0) {
+        const unsigned l1 = (unsigned)((a & 7) + d1) & 7u, l2 = (unsigned)((b & 7) + d2) & 7u;
+        int u1 = 0, u2 = 0;
+        if (l1 & 1u) { u1 = 2 - (int)(l1 & 3u); if ((l1 == 3 || l1 == 5) && (l2 & 3u) == 2) u1 = -u1; }
+        if (l2 & 1u) { u2 = 2 - (int)(l2 & 3u); if ((l2 == 3 || l2 == 5) && (l1 & 3u) == 2) u2 = -u2; }
+        if (2 * (int)d1 == 1 + u1) d1 = 1 - d1;
+        if (2 * (int)d2 == 1 + u2) d2 = 1 - d2;
+        a >>= 1;
+        b >>= 1;
+        out.dig[len >> 3] |= (uint32_t)((u1 + 1) | ((u2 + 1) << 2)) << ((len & 7) * 4);
+        ++len;
+    }
+    out.len = len;
+    return out;
+}
+
 // Queues one round.  round > 0 with prev_u: T comes from the previous round's points (pts_prev, rec[3*(round-1)..]);
 // otherwise T is a third bucket sum.  pts_round: this round's T, T0, T1 (T of later rounds is left to k_open_finish).
 static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars, const G1Jac* gens, const Fr& u, size_t old_size, int round, const Fr* prev_u,
@@ -675,12 +807,12 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
         ZK_HIP(hipEventCreate(&t1));
         ZK_HIP(hipEventRecord(t0, st));
     }
-    hipLaunchKernelGGL(k_open_fold, dim3(nb_main + n_msm + (chained ? 3u : 0u)), dim3(GT), 0, st, new_scalars, new_gens, scalars, aff.as<G1Affine>(), to_mont(u), ku,
+    hipLaunchKernelGGL(k_open_fold, dim3(nb_main + n_msm + (chained ? 3u : 0u)), dim3(GT), 0, st, new_scalars, new_gens, scalars, aff.as<G1Affine>(), to_mont(u), ku, jsf_of(ku),
                        old_size, new_size, nb_main, ex);
     if (g_fold_timer.on) {
         ZK_HIP(hipEventRecord(t1, st));
         g_fold_timer.ev.emplace_back(t0, t1);
-        g_fold_timer.fp_mults += fold_fp_mults_per_pair(ku) * (double)new_size;
+        g_fold_timer.fp_mults += fold_fp_mults_per_pair(jsf_of(ku)) * (double)new_size;
         g_fold_timer.pairs += new_size;
     }
     ZK_LAUNCH_CHECK();
