@@ -160,14 +160,9 @@ int zk_lookup_round(uint32_t* sums_host, void* new_A, void* new_S, void* new_B, 
                     const uint32_t* beta, const uint32_t* v, size_t n_out, int phase2, void* stream);
 /* one round of multi_hadamard_sumchecks (proof.cu:191-241) for K <= 4 tensors */
 int zk_hadamard_round(uint32_t* coefs_host, void* const* new_Xs, const void* const* Xs, int K, const void* E, const uint32_t* v, size_t n_out, void* stream);
-/* the last rounds of the two sumchecks above in one launch each: their challenges are fixed before the first round
- * (tLookup::prove tlookup.cu:150-176 and multi_hadamard_sumchecks proof.cu:191-241 take u and v as arguments), so short
- * tensors need no host round trip per round.  n_out (of the first fused round) <= 512, rounds <= 16; v in round
- * order; the input tensors are not modified.  sums_host: rounds x 11 (lookup) or rounds x (K+1) (Hadamard) */
-int zk_lookup_rounds_tail(uint32_t* sums_host, const void* A, const void* S, const void* B, const void* T, const void* m, const void* E, const uint32_t* beta,
-                          const uint32_t* v, size_t n_out, int rounds, int phase2_from, void* stream);
-int zk_hadamard_rounds_tail(uint32_t* coefs_host, const void* const* Xs, int K, const void* E, const uint32_t* v, size_t n_out, int rounds, void* stream);
-/* both sumchecks whole, queued without a host round trip (all rounds' sums come back in one copy).  Lookup: A, S of
+/* both sumchecks whole, queued without a host round trip (all rounds' sums come back in one copy): their challenges
+ * are fixed before the first round (tLookup::prove tlookup.cu:150-176 and multi_hadamard_sumchecks proof.cu:191-241 take
+ * u and v as arguments).  Rounds on short tensors (<= 512 pairs) run inside one launch.  Lookup: A, S of
  * D elements, B, T, m of N (D/N a power of two), E of D/2; v: rounds x 8 limbs in round order; sums_host: rounds x 11.
  * Hadamard: K tensors of N elements (a power of two), E of N/2; coefs_host: log2(N) x (K+1).  Inputs are not modified. */
 int zk_lookup_sumcheck(uint32_t* sums_host, const void* A, const void* S, const void* B, const void* T, const void* m, const void* E, const uint32_t* beta,

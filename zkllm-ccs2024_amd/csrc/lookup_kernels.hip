@@ -674,75 +674,6 @@ int zk_hadamard_round(uint32_t* coefs_host, void* const* new_Xs, const void* con
     memcpy(coefs_host, s, sizeof(Fr) * (K + 1));
     return 0;
 }
-// The last `rounds` rounds of the lookup sumcheck in one launch (n_out of the first of them at most 512, at most 16
-// rounds).  A, S (and B, T, m from round phase2_from on) hold 2*n_out elements, E n_out; none of them is modified.
-// v: the rounds' fold challenges in round order (standard form, host).  sums_host: rounds x 11 values ordered as
-// zk_lookup_round orders them (entries 5..10 of a phase-1 round are zero).
-int zk_lookup_rounds_tail(uint32_t* sums_host, const void* A, const void* S, const void* B, const void* T, const void* m, const void* E, const uint32_t* beta,
-                          const uint32_t* v, size_t n_out, int rounds, int phase2_from, void* stv) {
-    hipStream_t st = (hipStream_t)stv;
-    ZK_ARG(n_out >= 1 && n_out <= (size_t)TAIL_HALF, "zk_lookup_rounds_tail: n_out must be 1..512");
-    ZK_ARG(rounds >= 1 && rounds <= TAIL_ROUNDS, "zk_lookup_rounds_tail: 1..16 rounds");
-    ZK_ARG(((size_t)1 << (rounds - 1)) <= n_out, "zk_lookup_rounds_tail: more rounds than the tensors have variables");
-    ZK_ARG(phase2_from >= 0, "zk_lookup_rounds_tail: bad phase-2 start");
-    Scratch work(sizeof(Fr) * 6 * n_out), sums(sizeof(Fr) * 11 * rounds);
-    if (work.rc) return work.rc;
-    if (sums.rc) return sums.rc;
-    TailV vs;
-    for (int r = 0; r < TAIL_ROUNDS; ++r) vs.v[r] = r < rounds ? to_mont(load_fr(v + 8 * r)) : big_zero<8>();
-    Fr* w = work.as<Fr>();
-    hipLaunchKernelGGL(k_lookup_tail, dim3(1), dim3(TAIL_T), 0, st, sums.as<Fr>(), w, w + n_out, w + 2 * n_out, w + 3 * n_out, w + 4 * n_out, w + 5 * n_out, (const Fr*)A,
-                       (const Fr*)S, (const Fr*)B, (const Fr*)T, (const Fr*)m, (const Fr*)E, load_fr(beta), vs, (uint32_t)n_out, (uint32_t)rounds, (uint32_t)phase2_from);
-    ZK_LAUNCH_CHECK();
-    void* stage = nullptr;
-    int rc = staging(&stage, sizeof(Fr) * 11 * rounds);
-    if (rc) return rc;
-    ZK_HIP(hipMemcpyAsync(stage, sums.p, sizeof(Fr) * 11 * rounds, hipMemcpyDeviceToHost, st));
-    ZK_HIP(hipStreamSynchronize(st));
-    Fr* out = (Fr*)sums_host;
-    const Fr* in = (const Fr*)stage;
-    for (int r = 0; r < rounds; ++r)
-        for (int i = 0; i < 11; ++i) {
-            Fr x = in[r * 11 + i];
-            if (i != 3 && i != 4) x = to_mont(x);        // same R correction as zk_lookup_round
-            if (r < phase2_from && i >= 5) x = big_zero<8>();
-            memcpy(&out[r * 11 + i], &x, sizeof(Fr));
-        }
-    return 0;
-}
-// The last `rounds` rounds of multi_hadamard_sumchecks in one launch (same limits).  Xs hold 2*n_out elements and are
-// not modified; coefs_host: rounds x (K+1) coefficients; v in round order.
-int zk_hadamard_rounds_tail(uint32_t* coefs_host, const void* const* Xs, int K, const void* E, const uint32_t* v, size_t n_out, int rounds, void* stv) {
-    hipStream_t st = (hipStream_t)stv;
-    ZK_ARG(K >= 1 && K <= 4, "zk_hadamard_rounds_tail: K must be 1..4");
-    ZK_ARG(n_out >= 1 && n_out <= (size_t)TAIL_HALF, "zk_hadamard_rounds_tail: n_out must be 1..512");
-    ZK_ARG(rounds >= 1 && rounds <= TAIL_ROUNDS, "zk_hadamard_rounds_tail: 1..16 rounds");
-    ZK_ARG(((size_t)1 << (rounds - 1)) <= n_out, "zk_hadamard_rounds_tail: more rounds than the tensors have variables");
-    Scratch work(sizeof(Fr) * (K + 1) * n_out), sums(sizeof(Fr) * (K + 1) * rounds);
-    if (work.rc) return work.rc;
-    if (sums.rc) return sums.rc;
-    TailV vs;
-    for (int r = 0; r < TAIL_ROUNDS; ++r) vs.v[r] = r < rounds ? to_mont(load_fr(v + 8 * r)) : big_zero<8>();
-    Fr* w = work.as<Fr>();
-#define HADT_CASE(KK)                                                                                                                  \
-    case KK: {                                                                                                                         \
-        PtrPack<KK> p;                                                                                                                 \
-        for (int i = 0; i < KK; ++i) { p.in[i] = (const Fr*)Xs[i]; p.out[i] = w + (size_t)i * n_out; }                                  \
-        hipLaunchKernelGGL(k_hadamard_tail<KK>, dim3(1), dim3(TAIL_T), 0, st, sums.as<Fr>(), p, w + (size_t)KK * n_out, (const Fr*)E, vs, \
-                           (uint32_t)n_out, (uint32_t)rounds);                                                                         \
-        break;                                                                                                                         \
-    }
-    switch (K) { HADT_CASE(1) HADT_CASE(2) HADT_CASE(3) HADT_CASE(4) }
-#undef HADT_CASE
-    ZK_LAUNCH_CHECK();
-    void* stage = nullptr;
-    int rc = staging(&stage, sizeof(Fr) * (K + 1) * rounds);
-    if (rc) return rc;
-    ZK_HIP(hipMemcpyAsync(stage, sums.p, sizeof(Fr) * (K + 1) * rounds, hipMemcpyDeviceToHost, st));
-    ZK_HIP(hipStreamSynchronize(st));
-    memcpy(coefs_host, stage, sizeof(Fr) * (K + 1) * rounds);
-    return 0;
-}
 // ---- whole sumchecks as jobs ---------------------------------------------------------------------------------------------------
 // A job queues every kernel of a sumcheck on one stream without a host round trip (the challenges are known up front),
 // keeps its buffers until the results have been fetched, and can run on a stream of the library's own beside the caller.
