@@ -320,9 +320,10 @@ k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __rest
 // v as arguments, tlookup.cu:150-176, proof.cu:191-241), so one workgroup can run every remaining round back to back --
 // sums, fold by v, halving of the eq table, workgroup barrier -- and hand all rounds' sums back in one copy.
 static constexpr int TAIL_T = 1024;          // lanes of the single workgroup
-static constexpr int TAIL_HALF = 512;        // largest n_out of the first fused round: one compute unit does all of it
+static constexpr int TAIL_HALF = 256;        // largest n_out of the first fused round: one compute unit does all of it
 static constexpr int TAIL_ROUNDS = 16;
 struct TailV { Fr v[TAIL_ROUNDS]; };         // Montgomery form, in round order
+static constexpr int SPLIT_HALF = 32768;     // rounds of at most this many pairs spread each pair over several lanes
 
 __device__ __forceinline__ Fr wave_sum(Fr x) {
 #pragma unroll
@@ -361,55 +362,128 @@ template <int K> __device__ __forceinline__ void tail_block_sum(Fr (&acc)[K], Fr
     __syncthreads();
 }
 
-// All remaining rounds of the lookup sumcheck.  Round 0 reads the caller's tensors (2*n_out elements; E: n_out) and
-// writes the work buffers; later rounds fold the work buffers in place (lane t reads t and t + half and writes t,
-// which no other lane reads).  sums[r*11 + i] as k_lookup_round orders them (5 used in phase 1).  Rounds from
-// `phase2_from` on are phase-2 rounds.
+// A lookup round splits into four independent tasks per pair, so that short rounds -- where lanes are plentiful and the
+// chain of ~20 dependent field multiplications per pair is what takes the time -- can spread a pair over four lanes:
+//   task 0: sums 0..2 (E-weighted products of A and S + beta)        task 1: sums 5..7 (the same for B and T + beta)
+//   task 2: sums 8..10 (products of m and B), folds of m, A and S     task 3: sums 3..4 (a0, da), folds of B and T
+// Phase 1 has tasks 0 and 3' only (3' = sums 3..4 and the folds of A and S).  acc receives the task's sums (up to 3).
+struct LookupPtrs {
+    const Fr *A, *S, *B, *T, *m, *E;
+    Fr *nA, *nS, *nB, *nT, *nm;
+};
+__device__ __forceinline__ void lookup_task(Fr (&acc)[3], int task, bool phase2, const LookupPtrs& p, const Fr& beta, const Fr& v_mont, size_t t, size_t n_out) {
+    if (task == 0) {
+        const Fr e = p.E[t];
+        const Fr a0 = p.A[t], a1 = p.A[t + n_out], s0r = p.S[t], s1 = p.S[t + n_out];
+        const Fr da = sub(a1, a0), ds = sub(s1, s0r), s0 = add(s0r, beta);
+        acc[0] = add(acc[0], mont_mul(e, mont_mul(a0, s0)));
+        acc[1] = add(acc[1], mont_mul(e, add(mont_mul(da, s0), mont_mul(a0, ds))));
+        acc[2] = add(acc[2], mont_mul(e, mont_mul(da, ds)));
+    } else if (task == 1) {
+        const Fr e = p.E[t];
+        const Fr b0 = p.B[t], b1 = p.B[t + n_out], t0r = p.T[t], t1 = p.T[t + n_out];
+        const Fr db = sub(b1, b0), dt = sub(t1, t0r), t0 = add(t0r, beta);
+        acc[0] = add(acc[0], mont_mul(e, mont_mul(b0, t0)));
+        acc[1] = add(acc[1], mont_mul(e, add(mont_mul(db, t0), mont_mul(b0, dt))));
+        acc[2] = add(acc[2], mont_mul(e, mont_mul(db, dt)));
+    } else if (task == 2) {
+        const Fr b0 = p.B[t], b1 = p.B[t + n_out], m0 = p.m[t], m1 = p.m[t + n_out];
+        const Fr db = sub(b1, b0), dm = sub(m1, m0);
+        acc[0] = add(acc[0], mont_mul(m0, b0));
+        acc[1] = add(acc[1], add(mont_mul(dm, b0), mont_mul(m0, db)));
+        acc[2] = add(acc[2], mont_mul(dm, db));
+        p.nm[t] = add(m0, mont_mul(v_mont, dm));
+        const Fr a0 = p.A[t], s0 = p.S[t];
+        p.nA[t] = add(a0, mont_mul(v_mont, sub(p.A[t + n_out], a0)));
+        p.nS[t] = add(s0, mont_mul(v_mont, sub(p.S[t + n_out], s0)));
+    } else {
+        const Fr a0 = p.A[t];
+        const Fr da = sub(p.A[t + n_out], a0);
+        acc[0] = add(acc[0], a0);
+        acc[1] = add(acc[1], da);
+        if (phase2) {
+            const Fr b0 = p.B[t], t0 = p.T[t];
+            p.nB[t] = add(b0, mont_mul(v_mont, sub(p.B[t + n_out], b0)));
+            p.nT[t] = add(t0, mont_mul(v_mont, sub(p.T[t + n_out], t0)));
+        } else {
+            const Fr s0 = p.S[t];
+            p.nA[t] = add(a0, mont_mul(v_mont, da));
+            p.nS[t] = add(s0, mont_mul(v_mont, sub(p.S[t + n_out], s0)));
+        }
+    }
+}
+// where a task's sums go in the 11-value layout of a round, and how many it has
+__device__ __forceinline__ int lookup_task_base(int task) { return task == 0 ? 0 : (task == 1 ? 5 : (task == 2 ? 8 : 3)); }
+__device__ __forceinline__ int lookup_task_count(int task) { return task == 3 ? 2 : 3; }
+
+// One round, one task per blockIdx.y (phase 1: y = 0 -> task 0, y = 1 -> task 3; phase 2: y = task).
+// partials[k * gridDim.x + blockIdx.x] for the sums k the task owns.
+template <bool PHASE2> __global__ void __launch_bounds__(TPB)
+k_lookup_round_split(Fr* __restrict__ partials, const LookupPtrs p, const Fr beta, const Fr v_mont, size_t n_out) {
+    const int task = PHASE2 ? (int)blockIdx.y : (blockIdx.y == 0 ? 0 : 3);
+    Fr acc[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) acc[i] = big_zero<8>();
+    for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) lookup_task(acc, task, PHASE2, p, beta, v_mont, t, n_out);
+    if (task == 3) {                      // two sums only: row 5 belongs to task 1
+        Fr a2[2] = {acc[0], acc[1]};
+        block_reduce_store<2>(a2, partials + (size_t)3 * gridDim.x);
+    } else {
+        block_reduce_store<3>(acc, partials + (size_t)lookup_task_base(task) * gridDim.x);
+    }
+}
+
+// All remaining rounds of the lookup sumcheck in one workgroup of four 256-lane groups, one per task.  Round r reads
+// buffer set r & 1 and writes the other (round 0 reads the caller's tensors).  sums[r*11 + i] as k_lookup_round orders
+// them (5 used in phase 1).  Rounds from `phase2_from` on are phase-2 rounds.  w: 2 x 6 x n_out0 elements of work space.
 __global__ void __launch_bounds__(TAIL_T)
-k_lookup_tail(Fr* __restrict__ sums, Fr* wA, Fr* wS, Fr* wB, Fr* wT, Fr* wm, Fr* wE, const Fr* A, const Fr* S, const Fr* B, const Fr* T, const Fr* m, const Fr* E,
+k_lookup_tail(Fr* __restrict__ sums, Fr* w, const Fr* A, const Fr* S, const Fr* B, const Fr* T, const Fr* m, const Fr* E,
               const Fr beta, const TailV vs, uint32_t n_out0, uint32_t rounds, uint32_t phase2_from) {
-    __shared__ uint32_t red[11 * 16 * 8];
-    const Fr *cA = A, *cS = S, *cB = B, *cT = T, *cm = m, *cE = E;
+    __shared__ uint32_t red[4 * 3 * 4 * 8];       // task x sum x wave x limb
+    const uint32_t grp = threadIdx.x >> 8, lt = threadIdx.x & 255u, wv = lt >> 6, ln = lt & 63u;
+    LookupPtrs p;
+    p.A = A; p.S = S; p.B = B; p.T = T; p.m = m; p.E = E;
+    const Fr* cE = E;
     uint32_t n_out = n_out0;
     for (uint32_t r = 0; r < rounds; ++r) {
         const bool phase2 = r >= phase2_from;
-        const Fr v_mont = vs.v[r];
-        Fr acc[11];
+        Fr* ws = w + (size_t)(r & 1u) * 6 * n_out0;
+        p.nA = ws; p.nS = ws + n_out0; p.nB = ws + 2 * (size_t)n_out0; p.nT = ws + 3 * (size_t)n_out0; p.nm = ws + 4 * (size_t)n_out0;
+        Fr* nE = ws + 5 * (size_t)n_out0;
+        p.E = cE;
+        const int task = (int)grp;
+        const bool works = phase2 || task == 0 || task == 3;
+        Fr acc[3];
 #pragma unroll
-        for (int i = 0; i < 11; ++i) acc[i] = big_zero<8>();
-        for (uint32_t t = threadIdx.x; t < n_out; t += TAIL_T) {
-            const Fr e = cE[t];
-            {
-                const Fr a0 = cA[t], a1 = cA[t + n_out], s0r = cS[t], s1 = cS[t + n_out];
-                const Fr da = sub(a1, a0), ds = sub(s1, s0r), s0 = add(s0r, beta);
-                acc[0] = add(acc[0], mont_mul(e, mont_mul(a0, s0)));
-                acc[1] = add(acc[1], mont_mul(e, add(mont_mul(da, s0), mont_mul(a0, ds))));
-                acc[2] = add(acc[2], mont_mul(e, mont_mul(da, ds)));
-                acc[3] = add(acc[3], a0);
-                acc[4] = add(acc[4], da);
-                wA[t] = add(a0, mont_mul(v_mont, da));
-                wS[t] = add(s0r, mont_mul(v_mont, ds));
-            }
-            if (phase2) {
-                const Fr b0 = cB[t], b1 = cB[t + n_out], t0r = cT[t], t1 = cT[t + n_out], m0 = cm[t], m1 = cm[t + n_out];
-                const Fr db = sub(b1, b0), dt = sub(t1, t0r), t0 = add(t0r, beta), dm = sub(m1, m0);
-                acc[5] = add(acc[5], mont_mul(e, mont_mul(b0, t0)));
-                acc[6] = add(acc[6], mont_mul(e, add(mont_mul(db, t0), mont_mul(b0, dt))));
-                acc[7] = add(acc[7], mont_mul(e, mont_mul(db, dt)));
-                acc[8] = add(acc[8], mont_mul(m0, b0));
-                acc[9] = add(acc[9], add(mont_mul(dm, b0), mont_mul(m0, db)));
-                acc[10] = add(acc[10], mont_mul(dm, db));
-                wB[t] = add(b0, mont_mul(v_mont, db));
-                wT[t] = add(t0r, mont_mul(v_mont, dt));
-                wm[t] = add(m0, mont_mul(v_mont, dm));
+        for (int i = 0; i < 3; ++i) acc[i] = big_zero<8>();
+        if (works)
+            for (uint32_t t = lt; t < n_out; t += 256) lookup_task(acc, task, phase2, p, beta, vs.v[r], t, n_out);
+        // the halved eq table for the next round, by the lanes that idle in phase 1 (task 1) or finish early (any)
+        const uint32_t nh = n_out >> 1;
+        if (task == 1)
+            for (uint32_t t = lt; t < nh; t += 256) nE[t] = add(cE[t], cE[t + nh]);
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const Fr s = wave_sum(acc[k]);
+            if (ln == 0) {
+#pragma unroll
+                for (int l = 0; l < 8; ++l) red[((grp * 3 + k) * 4 + wv) * 8 + l] = s.v[l];
             }
         }
-        tail_block_sum<11>(acc, sums + (size_t)r * 11, red);      // ends with a barrier: every read of this round's E is done
-        cA = wA; cS = wS;
-        if (phase2) { cB = wB; cT = wT; cm = wm; }
-        const uint32_t nh = n_out >> 1;
-        for (uint32_t t = threadIdx.x; t < nh; t += TAIL_T) wE[t] = add(cE[t], cE[t + nh]);
-        cE = wE;
+        __syncthreads();
+        if (wv == 0 && ln < 3 && (int)ln < lookup_task_count(task) && works) {
+            Fr x = big_zero<8>();
+            for (int q = 0; q < 4; ++q) {
+                Fr y;
+#pragma unroll
+                for (int l = 0; l < 8; ++l) y.v[l] = red[((grp * 3 + ln) * 4 + q) * 8 + l];
+                x = add(x, y);
+            }
+            sums[(size_t)r * 11 + lookup_task_base(task) + ln] = x;
+        }
+        p.A = p.nA; p.S = p.nS;
+        if (phase2) { p.B = p.nB; p.T = p.nT; p.m = p.nm; }
+        cE = nE;
         n_out = nh;
         __syncthreads();
     }
@@ -724,13 +798,12 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
         const bool phase2 = r >= n1;
         if (half <= (size_t)TAIL_HALF && rounds - r <= TAIL_ROUNDS) {
             const int rest = rounds - r;
-            Scratch& work = job.arena.add(sizeof(Fr) * 6 * half);
+            Scratch& work = job.arena.add(sizeof(Fr) * 12 * half);
             if (work.rc) return work.rc;
             TailV vs;
             for (int i = 0; i < TAIL_ROUNDS; ++i) vs.v[i] = i < rest ? to_mont(load_fr(v + 8 * (r + i))) : big_zero<8>();
-            Fr* w = work.as<Fr>();
-            hipLaunchKernelGGL(k_lookup_tail, dim3(1), dim3(TAIL_T), 0, st, sums.as<Fr>() + (size_t)r * 11, w, w + half, w + 2 * half, w + 3 * half, w + 4 * half, w + 5 * half,
-                               cA, cS, cB, cT, cm, cE, b, vs, (uint32_t)half, (uint32_t)rest, (uint32_t)(phase2 ? 0 : n1 - r));
+            hipLaunchKernelGGL(k_lookup_tail, dim3(1), dim3(TAIL_T), 0, st, sums.as<Fr>() + (size_t)r * 11, work.as<Fr>(), cA, cS, cB, cT, cm, cE, b, vs, (uint32_t)half,
+                               (uint32_t)rest, (uint32_t)(phase2 ? 0 : n1 - r));
             ZK_LAUNCH_CHECK();
             break;
         }
@@ -739,7 +812,14 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
         Fr* w = nx.as<Fr>();
         const unsigned nb = reduce_grid(half);
         const Fr vm = to_mont(load_fr(v + 8 * r));
-        if (phase2)
+        if (half <= (size_t)SPLIT_HALF) {
+            // short round: four lanes per pair (two in phase 1), one task per grid row
+            LookupPtrs lp;
+            lp.A = cA; lp.S = cS; lp.B = cB; lp.T = cT; lp.m = cm; lp.E = cE;
+            lp.nA = w; lp.nS = w + half; lp.nB = w + 2 * half; lp.nT = w + 3 * half; lp.nm = w + 4 * half;
+            if (phase2) hipLaunchKernelGGL(k_lookup_round_split<true>, dim3(nb, 4), dim3(TPB), 0, st, part.as<Fr>(), lp, b, vm, half);
+            else hipLaunchKernelGGL(k_lookup_round_split<false>, dim3(nb, 2), dim3(TPB), 0, st, part.as<Fr>(), lp, b, vm, half);
+        } else if (phase2)
             hipLaunchKernelGGL(k_lookup_round<true>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, w + 2 * half, w + 3 * half, w + 4 * half, cA, cS, cB, cT, cm, cE, b, vm, half);
         else
             hipLaunchKernelGGL(k_lookup_round<false>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, cA, cS, (const Fr*)nullptr,
