@@ -234,6 +234,25 @@ __global__ void __launch_bounds__(TPB) k_eq_halve(Fr* __restrict__ out, const Fr
     if (t < n_out) out[t] = add(in[t], in[t + n_out]);
 }
 
+// The table in two launches instead of one per variable: small tables over the low and the high half of the variables
+// (every entry is a product of at most 15 factors), then their outer product.
+struct EqChallenges { Fr u[30], omu[30]; };     // u_j and 1 - u_j, Montgomery form
+__global__ void __launch_bounds__(TPB) k_eq_halves(Fr* __restrict__ lo, Fr* __restrict__ hi, const EqChallenges c, int kl, int kh) {
+    const uint32_t g = blockIdx.x * TPB + threadIdx.x;
+    const uint32_t nlo = 1u << kl, nhi = 1u << kh;
+    if (g >= nlo + nhi) return;
+    const bool is_hi = g >= nlo;
+    const uint32_t t = is_hi ? g - nlo : g;
+    const int first = is_hi ? kl : 0, cnt = is_hi ? kh : kl;
+    Fr e = big_one_mont<8>();
+    for (int j = 0; j < cnt; ++j) e = mont_mul(e, ((t >> j) & 1u) ? c.u[first + j] : c.omu[first + j]);
+    (is_hi ? hi : lo)[t] = e;
+}
+__global__ void __launch_bounds__(TPB) k_eq_outer(Fr* __restrict__ e, const Fr* __restrict__ lo, const Fr* __restrict__ hi, int kl, size_t n) {
+    const size_t t = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (t < n) e[t] = mont_mul(lo[t & ((1u << kl) - 1u)], hi[t >> kl]);
+}
+
 // ---- lookup sumcheck round --------------------------------------------------------------------------------------------------
 // Over halves (t, t + n_out):  a0 = A[t], da = A[t+n_out]-A[t], s0 = S[t]+beta, ds = S[t+n_out]-S[t]
 //   sums 0..2 : sum E[t] * {a0 s0, da s0 + a0 ds, da ds}          (R^-1 attached)
@@ -243,13 +262,14 @@ __global__ void __launch_bounds__(TPB) k_eq_halve(Fr* __restrict__ out, const Fr
 template <bool PHASE2> __global__ void __launch_bounds__(TPB)
 k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ nS, Fr* __restrict__ nB, Fr* __restrict__ nT, Fr* __restrict__ nm,
                const Fr* __restrict__ A, const Fr* __restrict__ S, const Fr* __restrict__ B, const Fr* __restrict__ T, const Fr* __restrict__ m,
-               const Fr* __restrict__ E, const Fr beta, const Fr v_mont, size_t n_out) {
+               const Fr* __restrict__ E, const Fr beta, const Fr v_mont, size_t n_out, Fr* __restrict__ nE) {
     constexpr int K = PHASE2 ? 11 : 5;
     Fr acc[K];
 #pragma unroll
     for (int i = 0; i < K; ++i) acc[i] = big_zero<8>();
     for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
         const Fr e = E[t];
+        if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table: the top variable summed out
         {
             const Fr a0 = A[t], a1 = A[t + n_out], s0r = S[t], s1 = S[t + n_out];
             const Fr da = sub(a1, a0), ds = sub(s1, s0r), s0 = add(s0r, beta);
@@ -283,7 +303,7 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
 // also folds every tensor by v.
 template <int K> struct PtrPack { const Fr* in[K]; Fr* out[K]; };
 template <int K> __global__ void __launch_bounds__(TPB)
-k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __restrict__ E, const Fr v_mont, size_t n_out) {
+k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __restrict__ E, const Fr v_mont, size_t n_out, Fr* __restrict__ nE) {
     Fr acc[K + 1];
 #pragma unroll
     for (int i = 0; i <= K; ++i) acc[i] = big_zero<8>();
@@ -308,6 +328,7 @@ k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __rest
             c[0] = mont_mul(c[0], x0m);
         }
         const Fr e = E[t];   // Montgomery form: e*R
+        if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table
 #pragma unroll
         for (int j = 0; j <= K; ++j) acc[j] = add(acc[j], mont_mul(e, c[j]));
     }
@@ -370,6 +391,7 @@ template <int K> __device__ __forceinline__ void tail_block_sum(Fr (&acc)[K], Fr
 struct LookupPtrs {
     const Fr *A, *S, *B, *T, *m, *E;
     Fr *nA, *nS, *nB, *nT, *nm;
+    Fr* nE;      // the next round's eq table (the top variable summed out), written by task 3; may be null
 };
 __device__ __forceinline__ void lookup_task(Fr (&acc)[3], int task, bool phase2, const LookupPtrs& p, const Fr& beta, const Fr& v_mont, size_t t, size_t n_out) {
     if (task == 0) {
@@ -397,6 +419,7 @@ __device__ __forceinline__ void lookup_task(Fr (&acc)[3], int task, bool phase2,
         p.nA[t] = add(a0, mont_mul(v_mont, sub(p.A[t + n_out], a0)));
         p.nS[t] = add(s0, mont_mul(v_mont, sub(p.S[t + n_out], s0)));
     } else {
+        if (p.nE && t < n_out / 2) p.nE[t] = add(p.E[t], p.E[t + n_out / 2]);
         const Fr a0 = p.A[t];
         const Fr da = sub(p.A[t + n_out], a0);
         acc[0] = add(acc[0], a0);
@@ -442,7 +465,7 @@ k_lookup_tail(Fr* __restrict__ sums, Fr* w, const Fr* A, const Fr* S, const Fr* 
     __shared__ uint32_t red[4 * 3 * 4 * 8];       // task x sum x wave x limb
     const uint32_t grp = threadIdx.x >> 8, lt = threadIdx.x & 255u, wv = lt >> 6, ln = lt & 63u;
     LookupPtrs p;
-    p.A = A; p.S = S; p.B = B; p.T = T; p.m = m; p.E = E;
+    p.A = A; p.S = S; p.B = B; p.T = T; p.m = m; p.E = E; p.nE = nullptr;
     const Fr* cE = E;
     uint32_t n_out = n_out0;
     for (uint32_t r = 0; r < rounds; ++r) {
@@ -616,6 +639,28 @@ static int read_flag(uint32_t* dev_flag, uint32_t* host_val, hipStream_t st) {
     return 0;
 }
 
+// eq table of k challenges into out (2^k elements, Montgomery form), queued on the stream; the two half tables live in the arena
+static int eq_table_queue(Fr* out, const uint32_t* u, int k, Arena& arena, hipStream_t st) {
+    EqChallenges c;
+    Fr one = big_zero<8>();
+    one.v[0] = 1;
+    for (int j = 0; j < 30; ++j) {
+        const Fr uj = j < k ? load_fr(u + 8 * j) : big_zero<8>();
+        c.u[j] = to_mont(uj);
+        c.omu[j] = to_mont(sub(one, uj));
+    }
+    const int kl = (k + 1) / 2, kh = k - kl;
+    Scratch& half = arena.add(sizeof(Fr) * (((size_t)1 << kl) + ((size_t)1 << kh)));
+    if (half.rc) return half.rc;
+    Fr* lo = half.as<Fr>();
+    Fr* hi = lo + ((size_t)1 << kl);
+    const size_t n = (size_t)1 << k;
+    hipLaunchKernelGGL(k_eq_halves, dim3(cdiv(((size_t)1 << kl) + ((size_t)1 << kh), TPB)), dim3(TPB), 0, st, lo, hi, c, kl, kh);
+    hipLaunchKernelGGL(k_eq_outer, dim3(cdiv(n, TPB)), dim3(TPB), 0, st, out, lo, hi, kl, n);
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
+
 extern "C" {
 
 int zk_lookup_index_fr(void* idx_u32, const void* vals, int32_t low, uint32_t table_size, size_t n, void* stv) {
@@ -674,19 +719,9 @@ int zk_fr_batch_inv(void* out, const void* in, const uint32_t* beta, size_t n, v
 }
 // E[t] for t < 2^k (Montgomery form) from k standard-form challenges; out holds 2^k elements
 int zk_eq_table(void* out, const uint32_t* u, int k, void* stv) {
-    hipStream_t st = (hipStream_t)stv;
     ZK_ARG(k >= 0 && k <= 30, "zk_eq_table: k out of range");
-    Fr one_m = big_one_mont<8>();
-    ZK_HIP(hipMemcpyAsync(out, &one_m, sizeof(Fr), hipMemcpyHostToDevice, st));
-    ZK_HIP(hipStreamSynchronize(st));
-    Fr one = big_zero<8>();
-    one.v[0] = 1;
-    for (int j = 0; j < k; ++j) {
-        const Fr uj = load_fr(u + 8 * j);
-        const size_t half = (size_t)1 << j;
-        LAUNCH1D(k_eq_double, half, st, (Fr*)out, to_mont(uj), to_mont(sub(one, uj)), half);
-    }
-    return 0;
+    Arena tmp;        // the half tables return to the allocator at once: later users are ordered behind these launches on the same stream
+    return eq_table_queue((Fr*)out, u, k, tmp, (hipStream_t)stv);
 }
 int zk_eq_halve(void* out, const void* in, size_t n_out, void* st) {
     LAUNCH1D(k_eq_halve, n_out, st, (Fr*)out, (const Fr*)in, n_out);
@@ -706,10 +741,10 @@ int zk_lookup_round(uint32_t* sums_host, void* nA, void* nS, void* nB, void* nT,
     const Fr b = load_fr(beta), vm = to_mont(load_fr(v));
     if (phase2)
         hipLaunchKernelGGL(k_lookup_round<true>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), (Fr*)nA, (Fr*)nS, (Fr*)nB, (Fr*)nT, (Fr*)nm, (const Fr*)A, (const Fr*)S,
-                           (const Fr*)B, (const Fr*)T, (const Fr*)m, (const Fr*)E, b, vm, n_out);
+                           (const Fr*)B, (const Fr*)T, (const Fr*)m, (const Fr*)E, b, vm, n_out, (Fr*)nullptr);
     else
         hipLaunchKernelGGL(k_lookup_round<false>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), (Fr*)nA, (Fr*)nS, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, (const Fr*)A,
-                           (const Fr*)S, (const Fr*)nullptr, (const Fr*)nullptr, (const Fr*)nullptr, (const Fr*)E, b, vm, n_out);
+                           (const Fr*)S, (const Fr*)nullptr, (const Fr*)nullptr, (const Fr*)nullptr, (const Fr*)E, b, vm, n_out, (Fr*)nullptr);
     ZK_LAUNCH_CHECK();
     Fr s[11];
     int rc = finish_sums(part.as<Fr>(), nb, K, 0, s, st);
@@ -735,7 +770,7 @@ int zk_hadamard_round(uint32_t* coefs_host, void* const* new_Xs, const void* con
     case KK: {                                                                                                                 \
         PtrPack<KK> p;                                                                                                         \
         for (int i = 0; i < KK; ++i) { p.in[i] = (const Fr*)Xs[i]; p.out[i] = (Fr*)new_Xs[i]; }                                 \
-        hipLaunchKernelGGL(k_hadamard_round<KK>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), p, (const Fr*)E, vm, n_out);        \
+        hipLaunchKernelGGL(k_hadamard_round<KK>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), p, (const Fr*)E, vm, n_out, (Fr*)nullptr); \
         break;                                                                                                                 \
     }
     switch (K) { HAD_CASE(1) HAD_CASE(2) HAD_CASE(3) HAD_CASE(4) }
@@ -764,18 +799,6 @@ __global__ void __launch_bounds__(TPB) k_dot_part(Fr* __restrict__ partials, con
     for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (size_t)gridDim.x * TPB) acc[0] = add(acc[0], mont_mul(a[i], b[i]));
     block_reduce_store<1>(acc, partials);
 }
-__global__ void k_set_one_mont(Fr* __restrict__ e) { if (threadIdx.x == 0 && blockIdx.x == 0) e[0] = big_one_mont<8>(); }
-// eq table of k challenges into out (2^k elements, Montgomery form), all on the stream
-static void eq_table_queue(Fr* out, const uint32_t* u, int k, hipStream_t st) {
-    hipLaunchKernelGGL(k_set_one_mont, dim3(1), dim3(64), 0, st, out);
-    Fr one = big_zero<8>();
-    one.v[0] = 1;
-    for (int j = 0; j < k; ++j) {
-        const Fr uj = load_fr(u + 8 * j);
-        const size_t half = (size_t)1 << j;
-        hipLaunchKernelGGL(k_eq_double, dim3(cdiv(half, TPB)), dim3(TPB), 0, st, out, to_mont(uj), to_mont(sub(one, uj)), half);
-    }
-}
 // all rounds of the lookup sumcheck; sums land in job.sums
 static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, const Fr* T, const Fr* m, const Fr* E, const Fr& b, const uint32_t* v, size_t D, size_t N, int rounds) {
     hipStream_t st = job.st;
@@ -791,7 +814,7 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
     job.sums = sums.as<Fr>();
     ZK_HIP(hipMemsetAsync(sums.p, 0, sizeof(Fr) * 11 * rounds, st));
     const Fr *cA = A, *cS = S, *cB = B, *cT = T, *cm = m, *cE = E;
-    Fr* ownE = nullptr;
+    Fr* eqbuf[2] = {nullptr, nullptr};
     size_t cur = D;
     for (int r = 0; r < rounds; ++r) {
         const size_t half = cur >> 1;
@@ -812,33 +835,36 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
         Fr* w = nx.as<Fr>();
         const unsigned nb = reduce_grid(half);
         const Fr vm = to_mont(load_fr(v + 8 * r));
+        // the next round's eq table is written by this round's kernel (ping-pong between two buffers of the job)
+        Fr* nE = nullptr;
+        if (r + 1 < rounds) {
+            const size_t nh = half >> 1;
+            if (!eqbuf[0]) {
+                Scratch& e = job.arena.add(sizeof(Fr) * 2 * (nh ? nh : 1));
+                if (e.rc) return e.rc;
+                eqbuf[0] = e.as<Fr>();
+                eqbuf[1] = eqbuf[0] + (nh ? nh : 1);
+            }
+            nE = eqbuf[r & 1];
+        }
         if (half <= (size_t)SPLIT_HALF) {
             // short round: four lanes per pair (two in phase 1), one task per grid row
             LookupPtrs lp;
-            lp.A = cA; lp.S = cS; lp.B = cB; lp.T = cT; lp.m = cm; lp.E = cE;
+            lp.A = cA; lp.S = cS; lp.B = cB; lp.T = cT; lp.m = cm; lp.E = cE; lp.nE = nE;
             lp.nA = w; lp.nS = w + half; lp.nB = w + 2 * half; lp.nT = w + 3 * half; lp.nm = w + 4 * half;
             if (phase2) hipLaunchKernelGGL(k_lookup_round_split<true>, dim3(nb, 4), dim3(TPB), 0, st, part.as<Fr>(), lp, b, vm, half);
             else hipLaunchKernelGGL(k_lookup_round_split<false>, dim3(nb, 2), dim3(TPB), 0, st, part.as<Fr>(), lp, b, vm, half);
         } else if (phase2)
-            hipLaunchKernelGGL(k_lookup_round<true>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, w + 2 * half, w + 3 * half, w + 4 * half, cA, cS, cB, cT, cm, cE, b, vm, half);
+            hipLaunchKernelGGL(k_lookup_round<true>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, w + 2 * half, w + 3 * half, w + 4 * half, cA, cS, cB, cT, cm, cE, b, vm, half, nE);
         else
             hipLaunchKernelGGL(k_lookup_round<false>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, cA, cS, (const Fr*)nullptr,
-                               (const Fr*)nullptr, (const Fr*)nullptr, cE, b, vm, half);
+                               (const Fr*)nullptr, (const Fr*)nullptr, cE, b, vm, half, nE);
         hipLaunchKernelGGL(k_finish, dim3(phase2 ? 11 : 5), dim3(TPB), 0, st, sums.as<Fr>() + (size_t)r * 11, part.as<Fr>(), nb);
         ZK_LAUNCH_CHECK();
         cA = w; cS = w + half;
         if (phase2) { cB = w + 2 * half; cT = w + 3 * half; cm = w + 4 * half; }
         cur = half;
-        if (r + 1 < rounds) {
-            const size_t nh = half >> 1;
-            if (!ownE) {
-                Scratch& e = job.arena.add(sizeof(Fr) * (nh ? nh : 1));
-                if (e.rc) return e.rc;
-                ownE = e.as<Fr>();
-            }
-            LAUNCH1D(k_eq_halve, nh, st, ownE, cE, nh);       // in place after the first halving: lane t reads t and t + nh, writes t
-            cE = ownE;
-        }
+        if (nE) cE = nE;
     }
     return 0;
 }
@@ -856,7 +882,7 @@ static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, 
     const Fr* cur[4];
     for (int i = 0; i < K; ++i) cur[i] = Xs[i];
     const Fr* cE = E;
-    Fr* ownE = nullptr;
+    Fr* eqbuf[2] = {nullptr, nullptr};
     size_t n = N;
     for (int r = 0; r < rounds; ++r) {
         const size_t half = n >> 1;
@@ -885,11 +911,22 @@ static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, 
         Fr* w = nx.as<Fr>();
         const unsigned nb = reduce_grid(half);
         const Fr vm = to_mont(load_fr(v + 8 * r));
+        Fr* nE = nullptr;
+        if (r + 1 < rounds) {
+            const size_t nh = half >> 1;
+            if (!eqbuf[0]) {
+                Scratch& e = job.arena.add(sizeof(Fr) * 2 * (nh ? nh : 1));
+                if (e.rc) return e.rc;
+                eqbuf[0] = e.as<Fr>();
+                eqbuf[1] = eqbuf[0] + (nh ? nh : 1);
+            }
+            nE = eqbuf[r & 1];
+        }
 #define HADS_ROUND(KK)                                                                                                            \
     case KK: {                                                                                                                    \
         PtrPack<KK> p;                                                                                                            \
         for (int i = 0; i < KK; ++i) { p.in[i] = cur[i]; p.out[i] = w + (size_t)i * half; }                                        \
-        hipLaunchKernelGGL(k_hadamard_round<KK>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), p, cE, vm, half);                      \
+        hipLaunchKernelGGL(k_hadamard_round<KK>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), p, cE, vm, half, nE);                  \
         break;                                                                                                                    \
     }
         switch (K) { HADS_ROUND(1) HADS_ROUND(2) HADS_ROUND(3) HADS_ROUND(4) }
@@ -898,16 +935,7 @@ static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, 
         ZK_LAUNCH_CHECK();
         for (int i = 0; i < K; ++i) cur[i] = w + (size_t)i * half;
         n = half;
-        if (r + 1 < rounds) {
-            const size_t nh = half >> 1;
-            if (!ownE) {
-                Scratch& e = job.arena.add(sizeof(Fr) * (nh ? nh : 1));
-                if (e.rc) return e.rc;
-                ownE = e.as<Fr>();
-            }
-            LAUNCH1D(k_eq_halve, nh, st, ownE, cE, nh);
-            cE = ownE;
-        }
+        if (nE) cE = nE;
     }
     return 0;
 }
@@ -997,7 +1025,8 @@ int zk_lookup_prove_begin(void** handle, const void* S, const void* T, const voi
     hipLaunchKernelGGL(k_dot_part, dim3(nb), dim3(TPB), 0, st, dp.as<Fr>() + 1, B.as<Fr>(), (const Fr*)m, N);
     hipLaunchKernelGGL(k_finish, dim3(1), dim3(TPB), 0, st, dp.as<Fr>(), dp.as<Fr>() + 1, nb);
     job->extra = dp.as<Fr>();
-    eq_table_queue(E.as<Fr>(), u_eq, rounds - 1, st);
+    rc = eq_table_queue(E.as<Fr>(), u_eq, rounds - 1, job->arena, st);
+    if (rc) { sumjob_abort(job); return rc; }
     rc = lookup_queue(*job, A.as<Fr>(), (const Fr*)S, B.as<Fr>(), (const Fr*)T, (const Fr*)m, E.as<Fr>(), b, v, D, N, rounds);
     if (rc) { sumjob_abort(job); return rc; }
     *handle = job;
@@ -1041,7 +1070,8 @@ int zk_hadamard_prove_begin(void** handle, const void* const* Xs, int K, const u
     if (E.rc) { rc = E.rc; sumjob_abort(job); return rc; }
     int k = 0;
     while (((size_t)1 << k) < N) ++k;
-    eq_table_queue(E.as<Fr>(), u_eq, k - 1, job->st);
+    rc = eq_table_queue(E.as<Fr>(), u_eq, k - 1, job->arena, job->st);
+    if (rc) { sumjob_abort(job); return rc; }
     rc = hadamard_queue(*job, (const Fr* const*)Xs, K, E.as<Fr>(), v, N);
     if (rc) { sumjob_abort(job); return rc; }
     *handle = job;
