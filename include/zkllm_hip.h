@@ -151,6 +151,9 @@ int zk_fr_batch_inv(void* out, const void* in, const uint32_t* beta, size_t n, v
 /* eq(u, t) for t < 2^k in Montgomery form; zk_eq_halve drops the top variable */
 int zk_eq_table(void* out, const uint32_t* u, int k, void* stream);
 int zk_eq_halve(void* out, const void* in, size_t n_out, void* stream);
+/* FrTensor::operator()(u) (Fr_me fr-tensor.cu:602-609) for up to 8 tensors of n elements at the same point in one pass:
+ * out_host[i] = multilinear extension of Xs[i] at u (k challenges, 2^(k-1) < n <= 2^k) */
+int zk_fr_me_multi(uint32_t* out_host, const void* const* Xs, int K, size_t n, const uint32_t* u, int k, void* stream);
 /* one sumcheck round: every sum of tLookup_phase1_step_poly :184-200 / tLookup_phase2_step_poly :245-279 plus the
  * folds of tLookup_phase1_reduce_kernel :94-103 / tLookup_phase2_reduce_kernel :161-175.
  * sums_host (standard form): [E.(a0 s0), E.(da s0 + a0 ds), E.(da ds), sum a0, sum da] and, in phase 2,

@@ -253,6 +253,22 @@ __global__ void __launch_bounds__(TPB) k_eq_outer(Fr* __restrict__ e, const Fr* 
     if (t < n) e[t] = mont_mul(lo[t & ((1u << kl) - 1u)], hi[t >> kl]);
 }
 
+// Multilinear evaluations of up to 8 tensors at one point: a single pass that reads the point's eq table once and
+// every tensor once (Fr_me, fr-tensor.cu:602-609, run once per tensor in the reference).  E carries R, each product
+// one R^-1: the sums come out in standard form.
+struct MePtrs { const Fr* x[8]; };
+template <int K> __global__ void __launch_bounds__(TPB) k_me_multi(Fr* __restrict__ partials, const MePtrs p, const Fr* __restrict__ E, size_t n) {
+    Fr acc[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) acc[k] = big_zero<8>();
+    for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n; t += (size_t)gridDim.x * TPB) {
+        const Fr e = E[t];
+#pragma unroll
+        for (int k = 0; k < K; ++k) acc[k] = add(acc[k], mont_mul(e, p.x[k][t]));
+    }
+    block_reduce_store<K>(acc, partials);
+}
+
 // ---- lookup sumcheck round --------------------------------------------------------------------------------------------------
 // Over halves (t, t + n_out):  a0 = A[t], da = A[t+n_out]-A[t], s0 = S[t]+beta, ds = S[t+n_out]-S[t]
 //   sums 0..2 : sum E[t] * {a0 s0, da s0 + a0 ds, da ds}          (R^-1 attached)
@@ -722,6 +738,31 @@ int zk_eq_table(void* out, const uint32_t* u, int k, void* stv) {
     ZK_ARG(k >= 0 && k <= 30, "zk_eq_table: k out of range");
     Arena tmp;        // the half tables return to the allocator at once: later users are ordered behind these launches on the same stream
     return eq_table_queue((Fr*)out, u, k, tmp, (hipStream_t)stv);
+}
+// out_host[i] = multilinear extension of Xs[i] (n elements each, zero beyond) at u (k challenges, 2^(k-1) < n <= 2^k)
+int zk_fr_me_multi(uint32_t* out_host, const void* const* Xs, int K, size_t n, const uint32_t* u, int k, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(K >= 1 && K <= 8, "zk_fr_me_multi: 1..8 tensors");
+    ZK_ARG(k >= 0 && k <= 30 && n >= 1 && n <= ((size_t)1 << k) && (k == 0 || n > ((size_t)1 << (k - 1))), "zk_fr_me_multi: n does not match the number of challenges");
+    Arena tmp;
+    Scratch& E = tmp.add(sizeof(Fr) * ((size_t)1 << k));
+    if (E.rc) return E.rc;
+    int rc = eq_table_queue(E.as<Fr>(), u, k, tmp, st);
+    if (rc) return rc;
+    const unsigned nb = reduce_grid(n);
+    Scratch& part = tmp.add(sizeof(Fr) * K * nb);
+    if (part.rc) return part.rc;
+    MePtrs p;
+    for (int i = 0; i < 8; ++i) p.x[i] = (const Fr*)Xs[i < K ? i : 0];
+#define ME_CASE(KK) case KK: hipLaunchKernelGGL(k_me_multi<KK>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), p, E.as<Fr>(), n); break;
+    switch (K) { ME_CASE(1) ME_CASE(2) ME_CASE(3) ME_CASE(4) ME_CASE(5) ME_CASE(6) ME_CASE(7) ME_CASE(8) }
+#undef ME_CASE
+    ZK_LAUNCH_CHECK();
+    Fr s8[8];
+    rc = finish_sums(part.as<Fr>(), nb, K, 0, s8, st);
+    if (rc) return rc;
+    memcpy(out_host, s8, sizeof(Fr) * K);
+    return 0;
 }
 int zk_eq_halve(void* out, const void* in, size_t n_out, void* st) {
     LAUNCH1D(k_eq_halve, n_out, st, (Fr*)out, (const Fr*)in, n_out);

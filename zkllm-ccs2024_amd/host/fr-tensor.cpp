@@ -235,6 +235,22 @@ Fr_t FrTensor::operator()(const vector<Fr_t>& u) const {
     return out;
 }
 
+vector<Fr_t> FrTensor::me_batch(const vector<const FrTensor*>& ts, const vector<Fr_t>& u) {
+    vector<Fr_t> out(ts.size());
+    if (ts.empty()) return out;
+    const uint log_dim = (uint)u.size();
+    const uint n = ts[0]->size;
+    if (n <= ((1u << log_dim) / 2) || n > (1u << log_dim)) throw std::runtime_error("Incompatible dimensions");
+    for (auto* t : ts) if (t->size != n) throw std::runtime_error("me_batch: tensors of different sizes");
+    for (size_t i0 = 0; i0 < ts.size(); i0 += 8) {
+        const int K = (int)std::min<size_t>(8, ts.size() - i0);
+        const void* ptrs[8];
+        for (int i = 0; i < K; ++i) ptrs[i] = ts[i0 + i]->gpu_data;
+        ZKC(zk_fr_me_multi(out[i0].val, ptrs, K, n, u.empty() ? nullptr : u[0].val, (int)log_dim, nullptr));
+    }
+    return out;
+}
+
 // Folds `u.size()` levels of the middle axis, up to three levels per pass.
 static FrTensor fold_axis_all(const FrTensor& t, const vector<Fr_t>& u, uint cur_dim, size_t window) {
     if (u.empty()) return t;

@@ -93,6 +93,8 @@ class FrTensor {
 
     Fr_t sum() const;
     Fr_t operator()(const vector<Fr_t>& u) const;
+    // the same evaluation for several tensors of one size at one point, in a single pass over all of them
+    static vector<Fr_t> me_batch(const vector<const FrTensor*>& ts, const vector<Fr_t>& u);
     std::pair<FrTensor, FrTensor> split(uint window_size) const;
     FrTensor partial_me(const vector<Fr_t>& u, uint window_size) const;
     FrTensor partial_me(const vector<Fr_t>& u, uint cur_dim, uint window_size) const;

@@ -92,9 +92,13 @@ Fr_t zkSoftmax::prove(const FrTensor& Y, const FrTensor& X, const FrTensor& shif
     }
     if (!failure.empty()) throw std::runtime_error(failure);
 
-    vector<Fr_t> Y_seg_claims, X_seg_claims;
-    for (uint i = L; i < K; ++i) Y_seg_claims.push_back(Y_segments[i - L](v_Y));
-    for (uint i = 0; i < K; ++i) X_seg_claims.push_back(X_segments[i](v_Y));
+    // all evaluations at v_Y in one pass over the tensors (zksoftmax.cu:189-196 evaluates them one by one)
+    vector<const FrTensor*> at_v;
+    for (uint i = L; i < K; ++i) at_v.push_back(&Y_segments[i - L]);
+    for (uint i = 0; i < K; ++i) at_v.push_back(&X_segments[i]);
+    at_v.push_back(&X);
+    const vector<Fr_t> evals = FrTensor::me_batch(at_v, v_Y);
+    vector<Fr_t> Y_seg_claims(evals.begin(), evals.begin() + (K - L)), X_seg_claims(evals.begin() + (K - L), evals.begin() + (K - L) + K);
     zk_record(Y_seg_claims);
     zk_record(X_seg_claims);
 
@@ -103,7 +107,7 @@ Fr_t zkSoftmax::prove(const FrTensor& Y, const FrTensor& X, const FrTensor& shif
 
     vector<Fr_t> v_Y_(v_Y.begin() + ceilLog2(n), v_Y.end());
     auto shift_const_opening = shift(v_Y_);
-    auto X_opening = X(v_Y);
+    auto X_opening = evals.back();
     zk_record(shift_const_opening);
     zk_record(X_opening);
     if (shift_const_opening - minus_X_shifted_claim != X_opening) throw std::runtime_error("X claim is not correct");
