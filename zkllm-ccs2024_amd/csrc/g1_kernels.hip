@@ -491,10 +491,10 @@ __global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, con
     if (t == 0) partial[((size_t)blockIdx.z * MW + w) * nseg + seg] = tot;
 }
 
-// The fold of one round plus the single-point work that rides along in spare workgroups:
-//  blocks [0, nb_main): pair g -> new scalar, new generator;
-//  next n_msm blocks: lane 0 assembles one sum from its window sums, sum_w 2^(8w) W[w] -> pts_round[3 - n_msm + i];
-//  next 3 blocks (rounds after the first): rec_round[j] = [c_j] (T, T0, T1 of the previous round)[j], whose sum is this round's T.
+// The single-point work of a round, one lane per workgroup:
+//  first n_msm workgroups: assemble one sum from its window sums, sum_w 2^(8w) W[w] -> pts_round[3 - n_msm + i];
+//  next 3 (rounds after the first): rec_round[j] = [c_j] (T, T0, T1 of the previous round)[j], whose sum is this round's T.
+// None of it feeds the next round's fold, so it runs with the bucket sums on the opening's second stream.
 struct OpenExtras {
     const G1Jac* W;          // n_msm x MW window sums
     G1Jac* pts_round;        // this round's T, T0, T1
@@ -504,11 +504,10 @@ struct OpenExtras {
     uint32_t n_msm, round;
     GlvK kc[3];
 };
-__global__ void __launch_bounds__(GT) k_open_fold(Fr* __restrict__ new_scalars, G1Jac* __restrict__ new_gens, const Fr* __restrict__ scalars, const G1Affine* __restrict__ A,
-                                                  const Fr u_mont, const GlvK ku, const JsfK jsf, size_t old_size, size_t new_size, uint32_t nb_main, const OpenExtras ex) {
-    if (blockIdx.x >= nb_main) {
+__global__ void __launch_bounds__(GT) k_open_extras(const OpenExtras ex) {
+    {
         if (threadIdx.x != 0) return;
-        const uint32_t x = blockIdx.x - nb_main;
+        const uint32_t x = blockIdx.x;
         if (x < ex.n_msm) {
             const G1Jac* W = ex.W + (size_t)x * MW;
             G1Jac r = W[MW - 1];
@@ -524,8 +523,11 @@ __global__ void __launch_bounds__(GT) k_open_fold(Fr* __restrict__ new_scalars, 
             else base = ex.pts_prev[j];
             ex.rec_round[j] = g1_mul_glv(base, ex.kc[j]);
         }
-        return;
     }
+}
+// The fold itself: pair g -> new scalar and new generator.
+__global__ void __launch_bounds__(GT) k_open_fold(Fr* __restrict__ new_scalars, G1Jac* __restrict__ new_gens, const Fr* __restrict__ scalars, const G1Affine* __restrict__ A,
+                                                  const Fr u_mont, const GlvK ku, const JsfK jsf, size_t old_size, size_t new_size) {
     // ---- pair g: s' and g' = a1 + [u](a0 - a1) -------------------------------------------------------------------------------
     // The scalar multiplication works on affine points throughout its table: D = a0 - a1 (one inversion, batched over
     // the 64 lanes), phi(D) = (beta x, y), D + phi(D) = (beta^2 x, -y) (the three images of the endomorphism sum to zero) and
@@ -754,20 +756,30 @@ static JsfK jsf_of(const GlvK& k) {
 // Queues one round.  round > 0 with prev_u: T comes from the previous round's points (pts_prev, rec[3*(round-1)..]);
 // otherwise T is a third bucket sum.  pts_round: this round's T, T0, T1 (T of later rounds is left to k_open_finish).
 static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars, const G1Jac* gens, const Fr& u, size_t old_size, int round, const Fr* prev_u,
-                             G1Jac* pts_round, const G1Jac* pts_prev, G1Jac* rec, Arena& arena, hipStream_t st) {
+                             G1Jac* pts_round, const G1Jac* pts_prev, G1Jac* rec, Arena& arena, hipStream_t st, hipStream_t aux, std::vector<hipEvent_t>& events) {
     ZK_ARG(old_size < (1ull << 31), "opening: more than 2^31 generators");
     const size_t new_size = (old_size + 1) / 2;
     const bool chained = round > 0 && prev_u != nullptr;
+    // ---- both chains start from the affine generators and the recoded scalars ----
     Scratch& aff = arena.add(sizeof(G1Affine) * old_size);
     if (aff.rc) return aff.rc;
     hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(old_size, CH), GT)), dim3(GT), 0, st, aff.p, gens, old_size);
+    Scratch& dig = arena.add((size_t)(MW + 1) * old_size);
+    if (dig.rc) return dig.rc;
+    hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(old_size, 256)), dim3(256), 0, st, dig.as<int8_t>(), scalars, old_size);
+    ZK_LAUNCH_CHECK();
+    if (aux != st) {
+        hipEvent_t ready;
+        ZK_HIP(hipEventCreateWithFlags(&ready, hipEventDisableTiming));
+        events.push_back(ready);
+        ZK_HIP(hipEventRecord(ready, st));
+        ZK_HIP(hipStreamWaitEvent(aux, ready, 0));
+    }
+    // ---- side chain (aux): bucket sums, window sums, the round's single points; nothing here feeds the next fold ----
     MsmDescs<3> descs;
     const uint32_t half = (uint32_t)(old_size / 2);
     const uint32_t n_msm = chained ? 2u : 3u;
     uint32_t q = 0;
-    Scratch& dig = arena.add((size_t)(MW + 1) * old_size);
-    if (dig.rc) return dig.rc;
-    hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(old_size, 256)), dim3(256), 0, st, dig.as<int8_t>(), scalars, old_size);
     const int8_t* dg = dig.as<int8_t>();
     const uint32_t ds = (uint32_t)old_size;
     if (!chained) descs.d[q++] = MsmDesc{dg, ds, (uint32_t)old_size, 1u, 0u, 1u, 0u, 0u};
@@ -782,8 +794,8 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     Scratch& wsum = arena.add(sizeof(G1Jac) * n_msm * MW);
     if (partial.rc) return partial.rc;
     if (wsum.rc) return wsum.rc;
-    hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MT), 0, st, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff.as<G1Affine>(), descs, nseg, cps);
-    if (nseg > 1) hipLaunchKernelGGL(k_g1_rowsum, dim3(n_msm * MW, 1), dim3(GT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), (size_t)nseg, 1u);
+    hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MT), 0, aux, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff.as<G1Affine>(), descs, nseg, cps);
+    if (nseg > 1) hipLaunchKernelGGL(k_g1_rowsum, dim3(n_msm * MW, 1), dim3(GT), 0, aux, wsum.as<G1Jac>(), partial.as<G1Jac>(), (size_t)nseg, 1u);
     OpenExtras ex;
     ex.W = wsum.as<G1Jac>();
     ex.pts_round = pts_round;
@@ -799,20 +811,22 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
         ex.kc[1] = glv_split(fr_mul_std(omu, omu));
         ex.kc[2] = glv_split(fr_mul_std(pu, pu));
     }
-    const uint32_t nb_main = cdiv(new_size, GT);
+    hipLaunchKernelGGL(k_open_extras, dim3(n_msm + (chained ? 3u : 0u)), dim3(GT), 0, aux, ex);
+    ZK_LAUNCH_CHECK();
+    // ---- critical chain (st): the fold ----
     const GlvK ku = glv_split(u);
+    const JsfK jsf = jsf_of(ku);
     hipEvent_t t0 = nullptr, t1 = nullptr;
     if (g_fold_timer.on) {
         ZK_HIP(hipEventCreate(&t0));
         ZK_HIP(hipEventCreate(&t1));
         ZK_HIP(hipEventRecord(t0, st));
     }
-    hipLaunchKernelGGL(k_open_fold, dim3(nb_main + n_msm + (chained ? 3u : 0u)), dim3(GT), 0, st, new_scalars, new_gens, scalars, aff.as<G1Affine>(), to_mont(u), ku, jsf_of(ku),
-                       old_size, new_size, nb_main, ex);
+    hipLaunchKernelGGL(k_open_fold, dim3(cdiv(new_size, GT)), dim3(GT), 0, st, new_scalars, new_gens, scalars, aff.as<G1Affine>(), to_mont(u), ku, jsf, old_size, new_size);
     if (g_fold_timer.on) {
         ZK_HIP(hipEventRecord(t1, st));
         g_fold_timer.ev.emplace_back(t0, t1);
-        g_fold_timer.fp_mults += fold_fp_mults_per_pair(jsf_of(ku)) * (double)new_size;
+        g_fold_timer.fp_mults += fold_fp_mults_per_pair(jsf) * (double)new_size;
         g_fold_timer.pairs += new_size;
     }
     ZK_LAUNCH_CHECK();
@@ -1016,7 +1030,9 @@ int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host, con
     Scratch pts(sizeof(G1Jac) * 3);
     if (pts.rc) return pts.rc;
     Arena arena;
-    int rc = open_round_launch((Fr*)new_scalars, (G1Jac*)new_gens, (const Fr*)scalars, (const G1Jac*)gens, load_fr(u), old_size, 0, nullptr, pts.as<G1Jac>(), nullptr, nullptr, arena, st);
+    std::vector<hipEvent_t> evs;
+    int rc = open_round_launch((Fr*)new_scalars, (G1Jac*)new_gens, (const Fr*)scalars, (const G1Jac*)gens, load_fr(u), old_size, 0, nullptr, pts.as<G1Jac>(), nullptr, nullptr, arena, st, st, evs);
+    (void)evs;
     if (rc) return rc;
     hipLaunchKernelGGL(k_g1_normalize<false>, dim3(1), dim3(GT), 0, st, pts.p, pts.as<G1Jac>(), (size_t)3);
     ZK_LAUNCH_CHECK();
@@ -1039,12 +1055,15 @@ struct OpenJob {
     G1Jac* pts = nullptr;
     const Fr* final_scalar = nullptr;
     hipEvent_t ready = nullptr;    // only for jobs on a side stream
+    hipStream_t aux = nullptr;     // second stream of the job (bucket sums beside the folds); equals st when the job has one stream
+    std::vector<hipEvent_t> events;
 };
-static int open_queue(OpenJob& job, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, hipStream_t st) {
+static int open_queue(OpenJob& job, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, hipStream_t st, hipStream_t aux) {
     ZK_ARG(n >= 1, "zk_g1_open: empty input");
     ZK_ARG(rounds >= 0 && rounds <= 64, "zk_g1_open: bad round count");
     ZK_ARG(sizeof(G1Jac) * (3 * (size_t)rounds + 1) + sizeof(Fr) <= 65536, "zk_g1_open: proof larger than the staging buffer");
     job.st = st;
+    job.aux = aux;
     job.rounds = rounds;
     const size_t npts = 3 * (size_t)rounds + 1;
     Scratch& pts = job.arena.add(sizeof(G1Jac) * npts);
@@ -1073,12 +1092,19 @@ static int open_queue(OpenJob& job, const void* scalars, const void* gens, size_
         if (g2.rc) return g2.rc;
         const Fr ur = load_fr(u + 8 * r);
         int rc = open_round_launch(s2.as<Fr>(), g2.as<G1Jac>(), cs, cg, ur, size, r, r ? &prev_u : nullptr, pts.as<G1Jac>() + 3 * r,
-                                   r ? pts.as<G1Jac>() + 3 * (r - 1) : nullptr, rec.as<G1Jac>(), job.arena, st);
+                                   r ? pts.as<G1Jac>() + 3 * (r - 1) : nullptr, rec.as<G1Jac>(), job.arena, st, aux, job.events);
         if (rc) return rc;
         cs = s2.as<Fr>();
         cg = g2.as<G1Jac>();
         size = ns;
         prev_u = ur;
+    }
+    if (aux != st) {          // the points of the halving rounds come from the second stream
+        hipEvent_t done;
+        ZK_HIP(hipEventCreateWithFlags(&done, hipEventDisableTiming));
+        job.events.push_back(done);
+        ZK_HIP(hipEventRecord(done, aux));
+        ZK_HIP(hipStreamWaitEvent(st, done, 0));
     }
     hipLaunchKernelGGL(k_open_finish, dim3(cdiv((size_t)rounds + 1, GT)), dim3(GT), 0, st, pts.as<G1Jac>(), rec.as<G1Jac>(), tail_done ? (const G1Jac*)nullptr : cg,
                        (uint32_t)chained_rounds, (uint32_t)rounds);
@@ -1104,7 +1130,7 @@ static int open_collect(OpenJob& job, uint32_t* proof_host, uint32_t* final_scal
 // z = 1 (infinity: all-zero limbs).  final_scalar_host: the folded scalar.
 int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stv) {
     OpenJob job;
-    int rc = open_queue(job, scalars, gens, n, u, rounds, (hipStream_t)stv);
+    int rc = open_queue(job, scalars, gens, n, u, rounds, (hipStream_t)stv, (hipStream_t)stv);
     if (rc) { (void)hipStreamSynchronize((hipStream_t)stv); return rc; }
     return open_collect(job, proof_host, final_scalar_host);
 }
@@ -1113,15 +1139,17 @@ int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* sc
 // must stay alive and unmodified until end, which waits for the opening, delivers its results and releases its buffers.
 int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stv) {
     ZK_ARG(handle != nullptr, "zk_g1_open_begin: null handle");
-    hipStream_t side = side_stream(0);
-    ZK_ARG(side != nullptr, "zk_g1_open_begin: could not create a stream");
+    hipStream_t side = side_stream(0), aux = side_stream(0);      // consecutive streams of the pool: the folds on one, the bucket sums on the other
+    ZK_ARG(side != nullptr && aux != nullptr, "zk_g1_open_begin: could not create a stream");
     std::unique_ptr<OpenJob> job(new OpenJob);
     ZK_HIP(hipEventCreateWithFlags(&job->ready, hipEventDisableTiming));
     ZK_HIP(hipEventRecord(job->ready, (hipStream_t)stv));
     ZK_HIP(hipStreamWaitEvent(side, job->ready, 0));
-    int rc = open_queue(*job, scalars, gens, n, u, rounds, side);
+    int rc = open_queue(*job, scalars, gens, n, u, rounds, side, aux);
     if (rc) {
         (void)hipStreamSynchronize(side);
+        (void)hipStreamSynchronize(aux);
+        for (hipEvent_t e : job->events) (void)hipEventDestroy(e);
         (void)hipEventDestroy(job->ready);
         return rc;
     }
@@ -1132,8 +1160,9 @@ int zk_g1_open_end(void* handle, uint32_t* proof_host, uint32_t* final_scalar_ho
     ZK_ARG(handle != nullptr, "zk_g1_open_end: null handle");
     std::unique_ptr<OpenJob> job((OpenJob*)handle);
     int rc = open_collect(*job, proof_host, final_scalar_host);
-    if (rc) (void)hipStreamSynchronize(job->st);
+    if (rc) { (void)hipStreamSynchronize(job->st); (void)hipStreamSynchronize(job->aux); }
     (void)hipEventDestroy(job->ready);
+    for (hipEvent_t e : job->events) (void)hipEventDestroy(e);
     return rc;
 }
 
