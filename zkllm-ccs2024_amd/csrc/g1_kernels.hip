@@ -402,7 +402,8 @@ __device__ __forceinline__ G1Jac msm_block_sum(uint32_t* pool, const G1Jac& v, u
     return tot;
 }
 
-// partial[(sum * MW + w) * nseg + seg] = sum over the segment's elements of digit_w(s) * base.
+// One segment's share of sum over elements of digit_w(s) * base: with nseg == 1 the finished window sum partial[sum * MW + w],
+// otherwise the segment's MT raw buckets partial[((sum * MW + w) * nseg + seg) * MT + t] for k_msm_buckets.
 // Lane t owns the bucket of magnitude t+1.  Per chunk of MSEG elements:
 //  1. the bucket sizes are counted (one LDS atomic per element);
 //  2. a bucket with more than MHEAVY elements (scalars that share a digit: equal values, a common high byte) is summed by
@@ -481,6 +482,11 @@ __global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, con
         }
         __syncthreads();
     }
+    if (nseg > 1) {
+        // several segments share this (sum, window): leave the buckets as they are, k_msm_buckets reduces them once for all segments
+        partial[(((size_t)blockIdx.z * MW + w) * nseg + seg) * MT + t] = acc;
+        return;
+    }
     // bucket value t+1 times the bucket, then the sum over the lanes
     G1Jac r = g1_infinity();
     for (int bit = 7; bit >= 0; --bit) {
@@ -488,7 +494,32 @@ __global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, con
         if (((t + 1) >> bit) & 1u) r = g1_add(r, acc);
     }
     const G1Jac tot = msm_block_sum(pool, r, t);
-    if (t == 0) partial[((size_t)blockIdx.z * MW + w) * nseg + seg] = tot;
+    if (t == 0) partial[(size_t)blockIdx.z * MW + w] = tot;
+}
+// raw buckets of up to 8 consecutive segments summed: out[(row * gridDim.y + group) * MT + t], row = sum * MW + w
+__global__ void __launch_bounds__(MT) k_msm_bucket_fold(G1Jac* __restrict__ out, const G1Jac* __restrict__ buckets, uint32_t nseg) {
+    const uint32_t t = threadIdx.x, row = blockIdx.x, grp = blockIdx.y;
+    const uint32_t s0 = grp * 8, s1 = (s0 + 8 < nseg) ? s0 + 8 : nseg;
+    const G1Jac* b = buckets + (size_t)row * nseg * MT;
+    G1Jac acc = b[(size_t)s0 * MT + t];
+    for (uint32_t sg = s0 + 1; sg < s1; ++sg) acc = g1_add(acc, b[(size_t)sg * MT + t]);
+    out[((size_t)row * gridDim.y + grp) * MT + t] = acc;
+}
+// wsum[(sum * MW + w)] from the raw buckets of nseg segments: lane t adds up bucket t+1 over the segments, weights it,
+// and the lanes are summed.  One workgroup per (sum, window).
+__global__ void __launch_bounds__(MT) k_msm_buckets(G1Jac* __restrict__ wsum, const G1Jac* __restrict__ buckets, uint32_t nseg) {
+    __shared__ uint32_t pool[36 * MT];
+    const uint32_t t = threadIdx.x;
+    const G1Jac* b = buckets + (size_t)blockIdx.x * nseg * MT;
+    G1Jac acc = b[t];
+    for (uint32_t sg = 1; sg < nseg; ++sg) acc = g1_add(acc, b[(size_t)sg * MT + t]);
+    G1Jac r = g1_infinity();
+    for (int bit = 7; bit >= 0; --bit) {
+        r = g1_double(r);
+        if (((t + 1) >> bit) & 1u) r = g1_add(r, acc);
+    }
+    const G1Jac tot = msm_block_sum(pool, r, t);
+    if (t == 0) wsum[blockIdx.x] = tot;
 }
 
 // The single-point work of a round, one lane per workgroup:
@@ -786,16 +817,32 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     descs.d[q++] = MsmDesc{dg, ds, half, 2u, 0u, 2u, 1u, 1u};
     descs.d[q++] = MsmDesc{dg, ds, half, 2u, 1u, 2u, 0u, 2u};
     for (; q < 3; ++q) descs.d[q] = MsmDesc{dg, ds, 0u, 1u, 0u, 1u, 0u, 0u};
+    // One chunk per workgroup: many short workgroups keep every compute unit busy to the end of the launch (with few
+    // long ones, all equally long, whatever does not fit the first turn waits a whole turn); the raw buckets of the
+    // segments are summed afterwards.  Very large inputs take more chunks per workgroup to bound the bucket storage.
     const size_t count_max = chained ? half : old_size;
     const uint32_t chunks = count_max ? cdiv(count_max, MSEG) : 1u;
-    const uint32_t nseg = chunks < 16u ? chunks : 16u;
-    const uint32_t cps = (chunks + nseg - 1) / nseg;
-    Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * nseg);
+    const uint32_t cps = (chunks + 255u) / 256u;
+    const uint32_t nseg = (chunks + cps - 1) / cps;
+    Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (nseg > 1 ? (size_t)nseg * MT : 1));
     Scratch& wsum = arena.add(sizeof(G1Jac) * n_msm * MW);
     if (partial.rc) return partial.rc;
     if (wsum.rc) return wsum.rc;
     hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MT), 0, aux, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff.as<G1Affine>(), descs, nseg, cps);
-    if (nseg > 1) hipLaunchKernelGGL(k_g1_rowsum, dim3(n_msm * MW, 1), dim3(GT), 0, aux, wsum.as<G1Jac>(), partial.as<G1Jac>(), (size_t)nseg, 1u);
+    if (nseg > 1) {
+        // sum the segments' raw buckets eight at a time, then weight and total
+        const G1Jac* cur = partial.as<G1Jac>();
+        uint32_t ns = nseg;
+        while (ns > 8) {
+            const uint32_t ng = (ns + 7) / 8;
+            Scratch& nxt = arena.add(sizeof(G1Jac) * n_msm * MW * (size_t)ng * MT);
+            if (nxt.rc) return nxt.rc;
+            hipLaunchKernelGGL(k_msm_bucket_fold, dim3(n_msm * MW, ng), dim3(MT), 0, aux, nxt.as<G1Jac>(), cur, ns);
+            cur = nxt.as<G1Jac>();
+            ns = ng;
+        }
+        hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, aux, wsum.as<G1Jac>(), cur, ns);
+    }
     OpenExtras ex;
     ex.W = wsum.as<G1Jac>();
     ex.pts_round = pts_round;
@@ -842,10 +889,10 @@ static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, con
     for (int j = levels; j < TAIL_LEVELS; ++j) us.u[j] = big_zero<8>();
     Scratch& sl = arena.add(sizeof(Fr) * (n0 + (size_t)levels + 1));
     const int n_msm = 3 * levels + 1;
-    const uint32_t nseg = 1, cps = cdiv(n0, MSEG);       // one workgroup per (sum, window): buckets are reduced once
+    const uint32_t nseg = cdiv(n0, MSEG), cps = 1;       // one chunk per workgroup, as in the halving rounds
     Scratch& aff = arena.add(sizeof(G1Affine) * n0);
     Scratch& coef = arena.add(sizeof(Fr) * (size_t)n_msm * n0);
-    Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * nseg);
+    Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (nseg > 1 ? (size_t)nseg * MT : 1));
     Scratch& wsum = arena.add(sizeof(G1Jac) * n_msm * MW);
     if (sl.rc) return sl.rc;
     if (aff.rc) return aff.rc;
@@ -866,7 +913,7 @@ static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, con
         descs.d[i] = MsmDesc{dig.as<int8_t>(), (uint32_t)ncoef, live ? (uint32_t)n0 : 0u, 1u, live ? (uint32_t)((size_t)i * n0) : 0u, 1u, 0u, slot};
     }
     hipLaunchKernelGGL(k_msm_seg<TAIL_SUMS>, dim3(nseg, MW, n_msm), dim3(MT), 0, st, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff.as<G1Affine>(), descs, nseg, cps);
-    if (nseg > 1) hipLaunchKernelGGL(k_g1_rowsum, dim3(n_msm * MW, 1), dim3(GT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), (size_t)nseg, 1u);
+    if (nseg > 1) hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), nseg);
     hipLaunchKernelGGL(k_msm_horner, dim3(n_msm), dim3(GT), 0, st, pts, wsum.as<G1Jac>(), descs);
     ZK_LAUNCH_CHECK();
     // the folded scalar is the single element of the last level
