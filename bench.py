@@ -133,10 +133,35 @@ def main():
                        "launches": int(fold_launches.value), "avg_launch_ms": fold_ms.value / max(1, fold_launches.value),
                        "total_ms_in_timed_region": fold_ms.value, "pairs": int(fold_pairs.value), "fp_mul_per_s": fold_mults.value / (fold_ms.value * 1e-3) if fold_ms.value > 0 else 0.0,
                        "note": "algorithmic work = Fp multiplications of the point formulas x 300 MAD32; peak = 256 CU x 4 SIMD x 16 lanes x 2.4 GHz; "
-                               "HBM traffic of this kernel is 336 B per pair, far below the bandwidth bound"}
+                               "HBM traffic of this kernel is 336 B per pair, far below the bandwidth bound.  The average covers every launch of the timed "
+                               "region: most are short rounds (a few thousand pairs, one wave per SIMD or less) that run beside the rest of the proof"}
     if args.skip_extras:
         print(json.dumps(out))
         return
+
+    # ---- the same fold kernel alone at its largest shape in the layer: one halving of 352256 generators (the FFN weights' opening) ----
+    pv.seed(6)
+    n_big = 11008 << 5
+    gens_big = pv.commitment_random(n_big)
+    pv.lib.zkp_g1_devptr.restype = ctypes.c_void_p
+    gp = pv.lib.zkp_g1_devptr(c_void_p(gens_big.h))
+    sc = hip.upload(mt_random_vec(np.random.RandomState(8), n_big))
+    ns, ng = hip.malloc(32 * (n_big // 2)), hip.malloc(144 * (n_big // 2))
+    u1 = mt_random_vec(np.random.RandomState(9), 1)
+    sums3 = np.zeros((3, 36), np.uint32)
+    hip.call("zk_g1_open_round", c_void_p(ns), c_void_p(ng), sums3, c_void_p(sc), c_void_p(gp), u1, c_size_t(n_big), None)
+    hip.check(lib.zk_prof_fold_begin())
+    for _ in range(3):
+        hip.call("zk_g1_open_round", c_void_p(ns), c_void_p(ng), sums3, c_void_p(sc), c_void_p(gp), u1, c_size_t(n_big), None)
+    hip.check(lib.zk_prof_fold_read(ctypes.byref(fold_ms), ctypes.byref(fold_launches), ctypes.byref(fold_mults), ctypes.byref(fold_pairs)))
+    iso_tops = fold_mults.value * MAD_PER_FP_MUL / (fold_ms.value * 1e-3) / 1e12
+    out["roofline_fold_alone"] = {"kernel": "k_open_fold, 176128 pairs, nothing else on the device", "bound": "valu-int", "achieved": iso_tops, "peak": VALU_PEAK_TOPS,
+                                  "unit": "T MAD32/s", "frac": iso_tops / VALU_PEAK_TOPS, "traffic": None, "avg_launch_ms": fold_ms.value / max(1, fold_launches.value),
+                                  "fp_mul_per_s": fold_mults.value / (fold_ms.value * 1e-3),
+                                  "note": "2752 waves on 2048 wave slots (two per SIMD at 248 VGPRs): the launch takes two full turns"}
+    for p_ in (sc, ns, ng):
+        hip.free(p_)
+    del gens_big
 
     # ---- G1 MSM points/s: commitment of a 4096 x 11008 weight (stored 11008 rows x 4096 against 4096 generators) -------------
     pv.seed(5)
