@@ -16,7 +16,7 @@
 #include <memory>
 #include <utility>
 #include <vector>
-#include "g1.hpp"
+#include "fq29.hpp"
 #include "rt.hpp"
 #include "../../include/zkllm_hip.h"
 
@@ -156,6 +156,12 @@ template <bool AFFINE_OUT> __global__ void __launch_bounds__(GT) k_g1_normalize(
             out[base + c].x = ox; out[base + c].y = oy; out[base + c].z = oz;
         }
     }
+}
+
+// the normalised points once more in the 29-bit-limb form that the bucket kernels add in (infinity stays all-zero)
+__global__ void __launch_bounds__(256) k_g1aff_to_a29(A29* __restrict__ out, const G1Affine* __restrict__ in, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = a29_from_affine(in[i]);
 }
 
 // ---- fixed-base table for commit_int -------------------------------------------------------------------------
@@ -412,7 +418,7 @@ __device__ __forceinline__ G1Jac msm_block_sum(uint32_t* pool, const G1Jac& v, u
 //     additions, in lockstep whatever the digits are; elements that find their bucket's list full (more than MCAP)
 //     wait for the next pass over the chunk.
 template <int NMAX>
-__global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, const G1Affine* __restrict__ A, const MsmDescs<NMAX> descs, uint32_t nseg, uint32_t chunks_per_seg) {
+__global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, const A29* __restrict__ A, const MsmDescs<NMAX> descs, uint32_t nseg, uint32_t chunks_per_seg) {
     __shared__ uint32_t cnt[MT], cnt2[MT];
     __shared__ uint32_t pool[MCAP * MT / 2];       // u16 lists, or the 36 x MT point tree
     static_assert(MCAP * MT / 2 >= 36 * MT, "pool too small for the point tree");
@@ -422,7 +428,9 @@ __global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, con
     const uint32_t w = blockIdx.y, seg = blockIdx.x, t = threadIdx.x;
     const int8_t* __restrict__ Dw = d.digits + (size_t)w * d.dstride;
     const int8_t* __restrict__ Df = d.digits + (size_t)MW * d.dstride;
-    G1Jac acc = g1_infinity();
+    J29 acc29 = j29_infinity();          // the lane's bucket, in 29-bit limbs while points are added to it
+    G1Jac heavy = g1_infinity();         // what the cooperative path hands to this lane
+    bool any_heavy = false;
     for (uint32_t ch = 0; ch < chunks_per_seg; ++ch) {
         const uint32_t e0 = (seg * chunks_per_seg + ch) * MSEG;
         if (e0 >= d.count) break;
@@ -438,19 +446,20 @@ __global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, con
         uint32_t done = 0;                       // bit i: this lane's i-th element of the chunk needs no more work (MSEG / MT = 32 per lane)
         for (uint32_t b = 0; b < (uint32_t)MT; ++b) {
             if (cnt[b] <= (uint32_t)MHEAVY) continue;          // the same for every lane
-            G1Jac h = g1_infinity();
+            J29 h29 = j29_infinity();
             for (uint32_t e = e0 + t, i = 0; e < e1; e += MT, ++i) {
                 const size_t si = (size_t)e * d.s_mul + d.s_off;
                 const int dg = Dw[si];
                 if ((uint32_t)(dg < 0 ? -dg : dg) != b + 1) continue;
                 done |= 1u << i;
-                G1Affine pt = A[(size_t)e * d.b_mul + d.b_off];
-                if (aff_is_inf(pt)) continue;
-                if ((dg < 0) != (Df[si] != 0)) pt.y = neg(pt.y);
-                h = g1_add_mixed(h, pt);
+                A29 pt = A[(size_t)e * d.b_mul + d.b_off];
+                if (a29_is_inf(pt)) continue;
+                if ((dg < 0) != (Df[si] != 0)) pt.y = fq29_neg(pt.y);
+                h29 = j29_add_mixed(h29, pt);
             }
-            h = msm_block_sum(pool, h, t);
-            if (t == b) acc = g1_add(acc, h);
+            const G1Jac h = msm_block_sum(pool, j29_to_jac(h29), t);
+            if (t == b) heavy = g1_add(heavy, h);
+            any_heavy = true;
         }
         for (;;) {
             uint32_t left = 0;
@@ -471,10 +480,10 @@ __global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, con
             const uint32_t mine = c2 < (uint32_t)MCAP ? c2 : (uint32_t)MCAP;
             for (uint32_t k = 0; k < mine; ++k) {
                 const uint32_t en = list[k * MT + t];
-                G1Affine pt = A[(size_t)(e0 + (en & 0x7FFFu)) * d.b_mul + d.b_off];
-                if (aff_is_inf(pt)) continue;
-                if (en & 0x8000u) pt.y = neg(pt.y);
-                acc = g1_add_mixed(acc, pt);
+                A29 pt = A[(size_t)(e0 + (en & 0x7FFFu)) * d.b_mul + d.b_off];
+                if (a29_is_inf(pt)) continue;
+                if (en & 0x8000u) pt.y = fq29_neg(pt.y);
+                acc29 = j29_add_mixed(acc29, pt);
             }
             if (!__syncthreads_or((int)left)) break;
             cnt2[t] = 0;
@@ -482,6 +491,8 @@ __global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, con
         }
         __syncthreads();
     }
+    G1Jac acc = j29_to_jac(acc29);
+    if (any_heavy) acc = g1_add(acc, heavy);           // the same branch for every lane
     if (nseg > 1) {
         // several segments share this (sum, window): leave the buckets as they are, k_msm_buckets reduces them once for all segments
         partial[(((size_t)blockIdx.z * MW + w) * nseg + seg) * MT + t] = acc;
@@ -606,21 +617,25 @@ __global__ void __launch_bounds__(GT) k_open_fold(Fr* __restrict__ new_scalars, 
             PmQ.x = add(fp_sqr(lam), PQ.x);
             PmQ.y = sub(fp_mul(lam, sub(D.x, PmQ.x)), D.y);
         }
+        // the walk itself in 29-bit limbs: the four table points differ in four abscissae and two ordinates
+        const Fq29 xD = fq29_from_fp(D.x), xQ = fq29_from_fp(Q.x), xPQ = fq29_from_fp(PQ.x), xPmQ = fq29_from_fp(PmQ.x);
+        const Fq29 yD = fq29_from_fp(D.y), yPmQ = fq29_from_fp(PmQ.y);
+        const Fq29 yDn = fq29_neg(yD), yPmQn = fq29_neg(yPmQ);
+        J29 w = j29_infinity();
         for (int i = (int)jsf.len - 1; i >= 0; --i) {
-            r = g1_double(r);
+            w = j29_double(w);
             const uint32_t dg = (jsf.dig[i >> 3] >> ((i & 7) * 4)) & 0xFu;    // (d1 + 1) | (d2 + 1) << 2, the same for every lane
             const int d1 = (int)(dg & 3u) - 1, d2 = (int)(dg >> 2) - 1;
             if (d1 == 0 && d2 == 0) continue;
-            G1Affine t;
-            bool ng;
-            if (d2 == 0) { t = D; ng = d1 < 0; }
-            else if (d1 == 0) { t = Q; ng = d2 < 0; }
-            else if (d1 == d2) { t = PQ; ng = d1 < 0; }
-            else { t = PmQ; ng = d1 < 0; }
-            if (ng) t.y = neg(t.y);
-            r = g1_add_mixed(r, t);
+            A29 t;
+            if (d2 == 0) { t.x = xD; t.y = d1 < 0 ? yDn : yD; }
+            else if (d1 == 0) { t.x = xQ; t.y = d2 < 0 ? yDn : yD; }
+            else if (d1 == d2) { t.x = xPQ; t.y = d1 < 0 ? yD : yDn; }          // D + phi(D) = (beta^2 x, -y)
+            else { t.x = xPmQ; t.y = d1 < 0 ? yPmQn : yPmQ; }
+            w = j29_add_mixed(w, t);
         }
-        if (!inf1) r = g1_add_mixed(r, a1);
+        if (!inf1) w = j29_add_mixed(w, a29_from_affine(a1));
+        r = j29_to_jac(w);
     } else if (general) {
         G1Jac diff = aff_to_jac(a0);
         if (!inf1) diff = g1_add_mixed(diff, g1_neg(a1));
@@ -828,7 +843,10 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     Scratch& wsum = arena.add(sizeof(G1Jac) * n_msm * MW);
     if (partial.rc) return partial.rc;
     if (wsum.rc) return wsum.rc;
-    hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MT), 0, aux, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff.as<G1Affine>(), descs, nseg, cps);
+    Scratch& aff29 = arena.add(sizeof(A29) * old_size);
+    if (aff29.rc) return aff29.rc;
+    hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(old_size, 256)), dim3(256), 0, aux, aff29.as<A29>(), aff.as<G1Affine>(), old_size);
+    hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MT), 0, aux, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff29.as<A29>(), descs, nseg, cps);
     if (nseg > 1) {
         // sum the segments' raw buckets eight at a time, then weight and total
         const G1Jac* cur = partial.as<G1Jac>();
@@ -891,11 +909,13 @@ static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, con
     const int n_msm = 3 * levels + 1;
     const uint32_t nseg = cdiv(n0, MSEG), cps = 1;       // one chunk per workgroup, as in the halving rounds
     Scratch& aff = arena.add(sizeof(G1Affine) * n0);
+    Scratch& aff29 = arena.add(sizeof(A29) * n0);
     Scratch& coef = arena.add(sizeof(Fr) * (size_t)n_msm * n0);
     Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (nseg > 1 ? (size_t)nseg * MT : 1));
     Scratch& wsum = arena.add(sizeof(G1Jac) * n_msm * MW);
     if (sl.rc) return sl.rc;
     if (aff.rc) return aff.rc;
+    if (aff29.rc) return aff29.rc;
     if (coef.rc) return coef.rc;
     if (partial.rc) return partial.rc;
     if (wsum.rc) return wsum.rc;
@@ -912,7 +932,8 @@ static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, con
         const uint32_t slot = !live ? 0u : (i == 3 * levels ? 3u * (uint32_t)rounds : 3u * (uint32_t)r0 + (uint32_t)i);
         descs.d[i] = MsmDesc{dig.as<int8_t>(), (uint32_t)ncoef, live ? (uint32_t)n0 : 0u, 1u, live ? (uint32_t)((size_t)i * n0) : 0u, 1u, 0u, slot};
     }
-    hipLaunchKernelGGL(k_msm_seg<TAIL_SUMS>, dim3(nseg, MW, n_msm), dim3(MT), 0, st, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff.as<G1Affine>(), descs, nseg, cps);
+    hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(n0, 256)), dim3(256), 0, st, aff29.as<A29>(), aff.as<G1Affine>(), n0);
+    hipLaunchKernelGGL(k_msm_seg<TAIL_SUMS>, dim3(nseg, MW, n_msm), dim3(MT), 0, st, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff29.as<A29>(), descs, nseg, cps);
     if (nseg > 1) hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), nseg);
     hipLaunchKernelGGL(k_msm_horner, dim3(n_msm), dim3(GT), 0, st, pts, wsum.as<G1Jac>(), descs);
     ZK_LAUNCH_CHECK();
