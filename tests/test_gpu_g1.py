@@ -139,8 +139,9 @@ def test_commit_int_rejects_non_integer_scalars_and_is_linear(pv, orc):
 
 # 300 x 1: raw small integers, whose negative embeddings share their high bytes (one bucket receives whole chunks);
 # 4500 x 2: more than one chunk of the bucket kernel and odd sizes in several rounds; 20000 x 2: two halving rounds
-# (the second takes T from the first round's points) before the batched rest
-@pytest.mark.parametrize("n,m", [(4, 2), (8, 1), (16, 4), (5, 3), (1, 2), (300, 1), (4500, 2), (20000, 2)])
+# (the second takes T from the first round's points) before the batched rest; 70000 x 1: four halving rounds, so T of
+# rounds 1..3 are combinations of up to seven earlier points, with an odd size (4375 pairs + 1) on the way
+@pytest.mark.parametrize("n,m", [(4, 2), (8, 1), (16, 4), (5, 3), (1, 2), (300, 1), (4500, 2), (20000, 2), (70000, 1)])
 def test_open_value_and_g1_transcript(pv, orc, n, m):
     gens = oracle_gens(orc, 15 + n, n)
     rng = np.random.default_rng(n * m)

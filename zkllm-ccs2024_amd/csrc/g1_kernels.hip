@@ -533,38 +533,112 @@ __global__ void __launch_bounds__(MT) k_msm_buckets(G1Jac* __restrict__ wsum, co
     if (t == 0) wsum[blockIdx.x] = tot;
 }
 
-// The single-point work of a round, one lane per workgroup:
-//  first n_msm workgroups: assemble one sum from its window sums, sum_w 2^(8w) W[w] -> pts_round[3 - n_msm + i];
-//  next 3 (rounds after the first): rec_round[j] = [c_j] (T, T0, T1 of the previous round)[j], whose sum is this round's T.
-// None of it feeds the next round's fold, so it runs with the bucket sums on the opening's second stream.
-struct OpenExtras {
-    const G1Jac* W;          // n_msm x MW window sums
-    G1Jac* pts_round;        // this round's T, T0, T1
-    const G1Jac* pts_prev;   // previous round's T, T0, T1 (T valid only for the first round)
-    const G1Jac* rec_prev;   // previous round's three parts of T (rounds >= 2)
-    G1Jac* rec_round;        // this round's three parts of T
-    uint32_t n_msm, round;
-    GlvK kc[3];
-};
-__global__ void __launch_bounds__(GT) k_open_extras(const OpenExtras ex) {
-    {
-        if (threadIdx.x != 0) return;
-        const uint32_t x = blockIdx.x;
-        if (x < ex.n_msm) {
-            const G1Jac* W = ex.W + (size_t)x * MW;
-            G1Jac r = W[MW - 1];
-            for (int w = MW - 2; w >= 0; --w) {
-                for (int k = 0; k < 8; ++k) r = g1_double(r);
-                r = g1_add(r, W[w]);
-            }
-            ex.pts_round[3 - ex.n_msm + x] = r;
-        } else {
-            const uint32_t j = x - ex.n_msm;
-            G1Jac base;
-            if (j == 0) base = (ex.round == 1) ? ex.pts_prev[0] : g1_add(g1_add(ex.rec_prev[0], ex.rec_prev[1]), ex.rec_prev[2]);
-            else base = ex.pts_prev[j];
-            ex.rec_round[j] = g1_mul_glv(base, ex.kc[j]);
+// ---- the single points of the halving rounds, once per opening ---------------------------------------------------------
+// None of this feeds a fold, so nothing of it sits between two rounds: the rounds only leave their window sums behind
+// (W[(3 * round + j) * MW + w], j = 0, 1, 2 for T, T0, T1), and after the last round
+//  k_open_horner assembles every sum from its windows, sum_w 2^(8w) W[w], one lane per sum, all sums side by side;
+//  k_open_chain  computes T of every round r >= 1 (the reference sums s_i g_i over the folded vectors, commitment.cu:103): unrolling
+//                T_r = u(1-u) T_(r-1) + (1-u)^2 T0_(r-1) + u^2 T1_(r-1)   (u = the challenge of round r-1)
+//                down to round 0 makes T_r a combination of T_0 and the T0, T1 of the rounds before r with coefficients
+//                that are products of the challenges -- all rounds at once, one lane per term.
+struct OpenUs { Fr u[64]; };      // challenges of the halving rounds, Montgomery form
+__global__ void __launch_bounds__(GT) k_open_horner(G1Jac* __restrict__ pts, const G1Jac* __restrict__ Wall, uint32_t halving_rounds) {
+    if (threadIdx.x != 0) return;
+    const uint32_t x = blockIdx.x, round = x / 3, j = x % 3;
+    if (round >= halving_rounds || (round > 0 && j == 0)) return;
+    const G1Jac* W = Wall + (size_t)x * MW;
+    G1Jac r = W[MW - 1];
+    for (int w = MW - 2; w >= 0; --w) {
+        for (int k = 0; k < 8; ++k) r = g1_double(r);
+        r = g1_add(r, W[w]);
+    }
+    pts[x] = r;
+}
+// k = k1 + k2 * lambda, 0 <= k1 < lambda (r = lambda^2 + lambda + 1, so k2 <= lambda + 1): one long division, as glv_split on the host
+__device__ __forceinline__ GlvK glv_split_device(const Fr& k) {
+    const uint64_t lam_hi = 0xac45a4010001a402ull, lam_lo = 0x00000000ffffffffull;
+    uint64_t rh = 0, rl = 0, qh = 0, ql = 0;
+    for (int i = 255; i >= 0; --i) {
+        const bool top = (rh >> 63) != 0;
+        rh = (rh << 1) | (rl >> 63);
+        rl = (rl << 1) | ((k.v[i >> 5] >> (i & 31)) & 1u);
+        qh = (qh << 1) | (ql >> 63);
+        ql <<= 1;
+        if (top || rh > lam_hi || (rh == lam_hi && rl >= lam_lo)) {
+            const uint64_t nl = rl - lam_lo;
+            rh = rh - lam_hi - (rl < lam_lo ? 1u : 0u);
+            rl = nl;
+            ql |= 1u;
         }
+    }
+    GlvK o;
+    o.k1[0] = (uint32_t)rl; o.k1[1] = (uint32_t)(rl >> 32); o.k1[2] = (uint32_t)rh; o.k1[3] = (uint32_t)(rh >> 32);
+    o.k2[0] = (uint32_t)ql; o.k2[1] = (uint32_t)(ql >> 32); o.k2[2] = (uint32_t)qh; o.k2[3] = (uint32_t)(qh >> 32);
+    return o;
+}
+// [k1]P + [k2]phi(P) with a k of the lane's own: one doubling and at most one addition per bit, whatever the other lanes hold
+static __device__ __attribute__((noinline)) G1Jac g1_mul_glv_lane(const G1Jac& P, const GlvK& k) {
+    G1Jac Q = P;
+    Q.x = fp_mul(P.x, glv_beta());
+    const G1Jac PQ = g1_add(P, Q);
+    G1Jac out = g1_infinity();
+    for (int i = 127; i >= 0; --i) {
+        out = g1_double(out);
+        const uint32_t b = ((k.k1[i >> 5] >> (i & 31)) & 1u) | (((k.k2[i >> 5] >> (i & 31)) & 1u) << 1);
+        if (b) {
+            const G1Jac t = b == 1 ? P : (b == 2 ? Q : PQ);
+            out = g1_add(out, t);
+        }
+    }
+    return out;
+}
+// grid: halving_rounds - 1 workgroups; workgroup x computes T of round x + 1 into pts[3 * (x + 1)].  Needs T_0 and all T0, T1.
+__global__ void __launch_bounds__(GT) k_open_chain(G1Jac* __restrict__ pts, const OpenUs us, uint32_t halving_rounds) {
+    __shared__ uint32_t pool[36 * GT];
+    const uint32_t r = blockIdx.x + 1, t = threadIdx.x;
+    const Fr one = big_one_mont<8>();
+    G1Jac acc = g1_infinity();
+    if (r < halving_rounds) {
+        for (uint32_t i = t; i < 2 * r + 1; i += GT) {
+            // term i: i == 0 -> T_0 with prod_{j<r} a_j;  i = 1 + 2k + s -> (s ? T1_k : T0_k) with (s ? u_k^2 : (1-u_k)^2) prod_{k<j<r} a_j,  a_j = u_j (1 - u_j)
+            const uint32_t k = i == 0 ? 0u : (i - 1) / 2, s1 = i == 0 ? 0u : (i - 1) & 1u;
+            Fr c = one;
+            for (uint32_t j = (i == 0 ? 0u : k + 1); j < r; ++j) c = mont_mul(c, mont_mul(us.u[j], sub(one, us.u[j])));
+            if (i != 0) {
+                const Fr f = s1 ? us.u[k] : sub(one, us.u[k]);
+                c = mont_mul(c, mont_mul(f, f));
+            }
+            const G1Jac P = pts[i == 0 ? 0u : 3 * k + 1 + s1];
+            if (!is_zero(P.z)) acc = g1_add(acc, g1_mul_glv_lane(P, glv_split_device(from_mont(c))));
+        }
+    }
+    // sum over the lanes
+    __syncthreads();
+    {
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(&acc);
+#pragma unroll
+        for (int l = 0; l < 36; ++l) pool[l * GT + t] = src[l];
+    }
+    __syncthreads();
+    for (uint32_t sd = GT / 2; sd > 0; sd >>= 1) {
+        if (t < sd) {
+            G1Jac x, y;
+            uint32_t* px = reinterpret_cast<uint32_t*>(&x);
+            uint32_t* py = reinterpret_cast<uint32_t*>(&y);
+#pragma unroll
+            for (int l = 0; l < 36; ++l) { px[l] = pool[l * GT + t]; py[l] = pool[l * GT + t + sd]; }
+            x = g1_add(x, y);
+#pragma unroll
+            for (int l = 0; l < 36; ++l) pool[l * GT + t] = px[l];
+        }
+        __syncthreads();
+    }
+    if (t == 0 && r < halving_rounds) {
+        G1Jac tot;
+        uint32_t* pr = reinterpret_cast<uint32_t*>(&tot);
+#pragma unroll
+        for (int l = 0; l < 36; ++l) pr[l] = pool[l * GT];
+        pts[3 * r] = tot;
     }
 }
 // The fold itself: pair g -> new scalar and new generator.
@@ -704,11 +778,9 @@ __global__ void __launch_bounds__(GT) k_msm_horner(G1Jac* __restrict__ pts, cons
     pts[descs.d[blockIdx.x].slot] = r;
 }
 
-// after the last round: T of rounds >= 1 from its three parts, and the folded generator as the last proof point
-__global__ void __launch_bounds__(GT) k_open_finish(G1Jac* __restrict__ pts, const G1Jac* __restrict__ rec, const G1Jac* __restrict__ last_gen, uint32_t chained_rounds, uint32_t rounds) {
-    const uint32_t r = blockIdx.x * GT + threadIdx.x;
-    if (r >= 1 && r < chained_rounds) pts[3 * r] = g1_add(g1_add(rec[3 * r], rec[3 * r + 1]), rec[3 * r + 2]);
-    if (r == rounds && last_gen) pts[3 * rounds] = last_gen[0];
+// after the last round of an opening without a batched tail: the folded generator is the last proof point
+__global__ void __launch_bounds__(GT) k_open_finish(G1Jac* __restrict__ pts, const G1Jac* __restrict__ last_gen, uint32_t rounds) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) pts[3 * rounds] = last_gen[0];
 }
 
 // ---- host side ----------------------------------------------------------------------------------------------------------
@@ -799,13 +871,13 @@ static JsfK jsf_of(const GlvK& k) {
     return out;
 }
 
-// Queues one round.  round > 0 with prev_u: T comes from the previous round's points (pts_prev, rec[3*(round-1)..]);
-// otherwise T is a third bucket sum.  pts_round: this round's T, T0, T1 (T of later rounds is left to k_open_finish).
-static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars, const G1Jac* gens, const Fr& u, size_t old_size, int round, const Fr* prev_u,
-                             G1Jac* pts_round, const G1Jac* pts_prev, G1Jac* rec, Arena& arena, hipStream_t st, hipStream_t aux, std::vector<hipEvent_t>& events) {
+// Queues one round: the fold on st, the bucket sums on aux.  wsum_round: the round's 3 x MW window sums (T, T0, T1); with_T
+// false leaves the first MW alone (T of that round then comes from k_open_chain).
+static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars, const G1Jac* gens, const Fr& u, size_t old_size, bool with_T,
+                             G1Jac* wsum_round, Arena& arena, hipStream_t st, hipStream_t aux, std::vector<hipEvent_t>& events) {
     ZK_ARG(old_size < (1ull << 31), "opening: more than 2^31 generators");
     const size_t new_size = (old_size + 1) / 2;
-    const bool chained = round > 0 && prev_u != nullptr;
+    const bool chained = !with_T;
     // ---- both chains start from the affine generators and the recoded scalars ----
     Scratch& aff = arena.add(sizeof(G1Affine) * old_size);
     if (aff.rc) return aff.rc;
@@ -840,13 +912,12 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     const uint32_t cps = (chunks + 255u) / 256u;
     const uint32_t nseg = (chunks + cps - 1) / cps;
     Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (nseg > 1 ? (size_t)nseg * MT : 1));
-    Scratch& wsum = arena.add(sizeof(G1Jac) * n_msm * MW);
     if (partial.rc) return partial.rc;
-    if (wsum.rc) return wsum.rc;
+    G1Jac* wsum = wsum_round + (size_t)(3 - n_msm) * MW;
     Scratch& aff29 = arena.add(sizeof(A29) * old_size);
     if (aff29.rc) return aff29.rc;
     hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(old_size, 256)), dim3(256), 0, aux, aff29.as<A29>(), aff.as<G1Affine>(), old_size);
-    hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MT), 0, aux, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff29.as<A29>(), descs, nseg, cps);
+    hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MT), 0, aux, nseg > 1 ? partial.as<G1Jac>() : wsum, aff29.as<A29>(), descs, nseg, cps);
     if (nseg > 1) {
         // sum the segments' raw buckets eight at a time, then weight and total
         const G1Jac* cur = partial.as<G1Jac>();
@@ -859,24 +930,8 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
             cur = nxt.as<G1Jac>();
             ns = ng;
         }
-        hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, aux, wsum.as<G1Jac>(), cur, ns);
+        hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, aux, wsum, cur, ns);
     }
-    OpenExtras ex;
-    ex.W = wsum.as<G1Jac>();
-    ex.pts_round = pts_round;
-    ex.pts_prev = pts_prev;
-    ex.rec_prev = (chained && round >= 2) ? rec + 3 * (round - 1) : nullptr;
-    ex.rec_round = chained ? rec + 3 * round : nullptr;
-    ex.n_msm = n_msm;
-    ex.round = (uint32_t)round;
-    memset(ex.kc, 0, sizeof(ex.kc));
-    if (chained) {
-        const Fr one = fr_from_u64(1), pu = *prev_u, omu = sub(one, pu);
-        ex.kc[0] = glv_split(fr_mul_std(pu, omu));
-        ex.kc[1] = glv_split(fr_mul_std(omu, omu));
-        ex.kc[2] = glv_split(fr_mul_std(pu, pu));
-    }
-    hipLaunchKernelGGL(k_open_extras, dim3(n_msm + (chained ? 3u : 0u)), dim3(GT), 0, aux, ex);
     ZK_LAUNCH_CHECK();
     // ---- critical chain (st): the fold ----
     const GlvK ku = glv_split(u);
@@ -1097,11 +1152,14 @@ int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host, con
     ZK_ARG(old_size >= 1, "zk_g1_open_round: empty input");
     Scratch pts(sizeof(G1Jac) * 3);
     if (pts.rc) return pts.rc;
+    Scratch wsum(sizeof(G1Jac) * 3 * MW);
+    if (wsum.rc) return wsum.rc;
     Arena arena;
     std::vector<hipEvent_t> evs;
-    int rc = open_round_launch((Fr*)new_scalars, (G1Jac*)new_gens, (const Fr*)scalars, (const G1Jac*)gens, load_fr(u), old_size, 0, nullptr, pts.as<G1Jac>(), nullptr, nullptr, arena, st, st, evs);
+    int rc = open_round_launch((Fr*)new_scalars, (G1Jac*)new_gens, (const Fr*)scalars, (const G1Jac*)gens, load_fr(u), old_size, true, wsum.as<G1Jac>(), arena, st, st, evs);
     (void)evs;
     if (rc) return rc;
+    hipLaunchKernelGGL(k_open_horner, dim3(3), dim3(GT), 0, st, pts.as<G1Jac>(), wsum.as<G1Jac>(), 1u);
     hipLaunchKernelGGL(k_g1_normalize<false>, dim3(1), dim3(GT), 0, st, pts.p, pts.as<G1Jac>(), (size_t)3);
     ZK_LAUNCH_CHECK();
     void* stage = nullptr;
@@ -1135,21 +1193,22 @@ static int open_queue(OpenJob& job, const void* scalars, const void* gens, size_
     job.rounds = rounds;
     const size_t npts = 3 * (size_t)rounds + 1;
     Scratch& pts = job.arena.add(sizeof(G1Jac) * npts);
-    Scratch& rec = job.arena.add(sizeof(G1Jac) * 3 * (rounds ? rounds : 1));
+    Scratch& wsum = job.arena.add(sizeof(G1Jac) * 3 * MW * (rounds ? rounds : 1));      // window sums of the halving rounds
     if (pts.rc) return pts.rc;
-    if (rec.rc) return rec.rc;
+    if (wsum.rc) return wsum.rc;
     job.pts = pts.as<G1Jac>();
     const Fr* cs = (const Fr*)scalars;
     const G1Jac* cg = (const G1Jac*)gens;
     size_t size = n;
-    Fr prev_u = big_zero<8>();
-    int chained_rounds = rounds;
+    int halving_rounds = rounds;
     bool tail_done = false;
+    OpenUs us;
+    memset(&us, 0, sizeof(us));
     for (int r = 0; r < rounds; ++r) {
         if (size <= (size_t)TAIL_N && rounds - r <= TAIL_LEVELS) {
             int rc = open_tail_launch(cs, cg, size, u + 8 * r, rounds - r, r, rounds, pts.as<G1Jac>(), &cs, job.arena, st);
             if (rc) return rc;
-            chained_rounds = r;
+            halving_rounds = r;
             tail_done = true;
             break;
         }
@@ -1159,23 +1218,27 @@ static int open_queue(OpenJob& job, const void* scalars, const void* gens, size_
         if (s2.rc) return s2.rc;
         if (g2.rc) return g2.rc;
         const Fr ur = load_fr(u + 8 * r);
-        int rc = open_round_launch(s2.as<Fr>(), g2.as<G1Jac>(), cs, cg, ur, size, r, r ? &prev_u : nullptr, pts.as<G1Jac>() + 3 * r,
-                                   r ? pts.as<G1Jac>() + 3 * (r - 1) : nullptr, rec.as<G1Jac>(), job.arena, st, aux, job.events);
+        us.u[r] = to_mont(ur);
+        int rc = open_round_launch(s2.as<Fr>(), g2.as<G1Jac>(), cs, cg, ur, size, r == 0, wsum.as<G1Jac>() + (size_t)3 * MW * r, job.arena, st, aux, job.events);
         if (rc) return rc;
         cs = s2.as<Fr>();
         cg = g2.as<G1Jac>();
         size = ns;
-        prev_u = ur;
     }
-    if (aux != st) {          // the points of the halving rounds come from the second stream
+    // the single points of the halving rounds, behind the last bucket sums
+    if (halving_rounds > 0) {
+        hipLaunchKernelGGL(k_open_horner, dim3(3 * halving_rounds), dim3(GT), 0, aux, pts.as<G1Jac>(), wsum.as<G1Jac>(), (uint32_t)halving_rounds);
+        if (halving_rounds > 1) hipLaunchKernelGGL(k_open_chain, dim3(halving_rounds - 1), dim3(GT), 0, aux, pts.as<G1Jac>(), us, (uint32_t)halving_rounds);
+        ZK_LAUNCH_CHECK();
+    }
+    if (aux != st) {
         hipEvent_t done;
         ZK_HIP(hipEventCreateWithFlags(&done, hipEventDisableTiming));
         job.events.push_back(done);
         ZK_HIP(hipEventRecord(done, aux));
         ZK_HIP(hipStreamWaitEvent(st, done, 0));
     }
-    hipLaunchKernelGGL(k_open_finish, dim3(cdiv((size_t)rounds + 1, GT)), dim3(GT), 0, st, pts.as<G1Jac>(), rec.as<G1Jac>(), tail_done ? (const G1Jac*)nullptr : cg,
-                       (uint32_t)chained_rounds, (uint32_t)rounds);
+    if (!tail_done) hipLaunchKernelGGL(k_open_finish, dim3(1), dim3(GT), 0, st, pts.as<G1Jac>(), cg, (uint32_t)rounds);
     hipLaunchKernelGGL(k_g1_normalize<false>, dim3(cdiv(cdiv(npts, CH), GT)), dim3(GT), 0, st, pts.p, pts.as<G1Jac>(), npts);
     ZK_LAUNCH_CHECK();
     job.final_scalar = cs;
