@@ -64,6 +64,25 @@ def test_batch_inverse(pv, orc, n):
         assert not got[3].any()
 
 
+def test_batch_inverse_at_full_size_inverts(pv):
+    """2^24 + 5 values: the products of the workgroups are themselves too many for one step, so the scheme nests twice.
+    Checked by what an inverse is: out * (in + beta) == 1 everywhere (0 where in + beta == 0)."""
+    n = (1 << 24) + 5
+    rng = np.random.default_rng(24)
+    S = np.zeros((n, 8), np.uint32)
+    S[:, :7] = rng.integers(0, 1 << 32, (n, 7), dtype=np.uint64).astype(np.uint32)     # below 2^224: standard-form residues
+    beta = ch(6, 1)[0]
+    hole = n - 3
+    S[hole] = fr_array([(-fr_ints(beta.reshape(1, 8))[0]) % R_MOD])[0]
+    hS = pv.from_fr(S)
+    inv = pv.batch_inv(hS, beta)
+    prod = pv.binop(2, inv, pv.scalarop(0, hS, beta)).host()
+    expect = np.zeros((n, 8), np.uint32)
+    expect[:, 0] = 1
+    expect[hole, 0] = 0
+    assert (prod == expect).all()
+
+
 @pytest.mark.parametrize("D,low,length", [(16, 3, 4), (4, 0, 4), (256, -8, 16), (4096, -32, 64), (1 << 15, -(1 << 9), 1 << 10)])
 def test_range_lookup_proof_transcript(pv, orc, D, low, length):
     rng = np.random.default_rng(D + length)

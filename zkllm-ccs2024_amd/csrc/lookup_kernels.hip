@@ -143,18 +143,27 @@ __global__ void __launch_bounds__(TPB) k_range_table(Fr* __restrict__ table, int
 }
 
 // ---- batch inversion -----------------------------------------------------------------------------------------------
-// out[i] = 1 / (in[i] + beta), 0 where the sum is 0.  A workgroup inverts 4096 values with one field inversion:
-// every lane multiplies its 8 values up, the 512 lane products go up a product tree in LDS, the root is inverted, and
+// out[i] = 1 / (in[i] + beta), 0 where the sum is 0.  A workgroup inverts T * 8 values with one field inversion:
+// every lane multiplies its 8 values up, the T lane products go up a product tree in LDS, the root is inverted, and
 // the inverse comes down the tree (a child's inverse is the parent's inverse times the sibling) and through each
 // lane's values backwards.  About 3.4 multiplications per value.
 // The standard-form inputs are used as they are: x is the Montgomery representation of x/R, every product of the
 // scheme is then a Montgomery representation too, and the two stray factors of R in each result are removed once per
 // workgroup by multiplying the root's inverse by R^-1 (a Montgomery product with R^-1 multiplies by R^-2).
-static constexpr int BI_T = 512, BI_CH = 8, BI_NODES = 2 * BI_T - 1;
-__global__ void __launch_bounds__(BI_T) k_batch_inv(Fr* __restrict__ out, const Fr* __restrict__ in, const Fr beta, size_t n) {
-    __shared__ uint32_t node[8][BI_NODES + 1];      // level 0 (lane products) at [0, 512), level 1 at [512, 768), ... root at 1022
+//
+// One field inversion is a serial computation of about 140 us on one lane, during which the rest of its workgroup
+// waits with its registers held.  Large inputs therefore run in three steps (MODE): BI_UP only multiplies up to the
+// workgroup's root and writes it to roots[workgroup]; the roots -- a few thousand numbers -- are inverted by this same
+// scheme (the corrected inverse of a root is exactly the plain inverse of the number written); BI_DOWN repeats the
+// way up, takes its root's inverse from roots_inv[workgroup] and comes down.  The two large steps then have no serial part.
+enum { BI_FULL = 0, BI_UP = 1, BI_DOWN = 2 };
+static constexpr int BI_T = 512, BI_CH = 8;        // single-step form (small inputs)
+static constexpr int BI_T3 = 256;                  // three-step form
+template <int T, int MODE>
+__global__ void __launch_bounds__(T) k_batch_inv(Fr* __restrict__ out, const Fr* __restrict__ in, const Fr beta, size_t n, Fr* __restrict__ roots, const Fr* __restrict__ roots_inv) {
+    __shared__ uint32_t node[8][2 * T];      // level 0 (lane products) at [0, T), level 1 at [T, T + T/2), ... root at 2T - 2
     const uint32_t t = threadIdx.x;
-    const size_t base = ((size_t)blockIdx.x * BI_T + t) * BI_CH;
+    const size_t base = ((size_t)blockIdx.x * T + t) * BI_CH;
     const Fr one_m = big_one_mont<8>();
     Fr x[BI_CH], pre[BI_CH];
     uint32_t nz = 0;
@@ -181,16 +190,22 @@ __global__ void __launch_bounds__(BI_T) k_batch_inv(Fr* __restrict__ out, const 
     };
     put(tot, t);
     __syncthreads();
-    // up: level L has BI_T >> L nodes starting at off(L) = 2*BI_T - (2*BI_T >> L)
+    // up: level L has T >> L nodes starting at off(L) = 2*T - (2*T >> L)
     uint32_t off = 0;
-    for (uint32_t cnt = BI_T / 2; cnt >= 1; cnt >>= 1) {
+    for (uint32_t cnt = T / 2; cnt >= 1; cnt >>= 1) {
         const uint32_t noff = off + 2 * cnt;
         if (t < cnt) put(mont_mul(get(off + 2 * t), get(off + 2 * t + 1)), noff + t);
         __syncthreads();
         off = noff;
     }
     // off is now the root's index
-    if (t < 64) {
+    if (MODE == BI_UP) {
+        if (t == 0) roots[blockIdx.x] = get(off);
+        return;
+    }
+    if (MODE == BI_DOWN) {
+        if (t == 0) put(roots_inv[blockIdx.x], off);
+    } else if (t < 64) {
         Fr inv = mont_inverse(get(off));
         constexpr uint32_t RINV[8] = {4269129792u, 334977897u, 165441631u, 2876230287u, 1333208682u, 1912866698u, 805346647u, 465471123u};   // R^-1 mod r
         Fr k;
@@ -201,7 +216,7 @@ __global__ void __launch_bounds__(BI_T) k_batch_inv(Fr* __restrict__ out, const 
     }
     __syncthreads();
     // down: the inverse of a node replaces its value; a child reads the parent's inverse and its sibling's value first
-    for (uint32_t cnt = 1; cnt < (uint32_t)BI_T; cnt <<= 1) {
+    for (uint32_t cnt = 1; cnt < (uint32_t)T; cnt <<= 1) {
         const uint32_t coff = off - 2 * cnt;          // children level: 2*cnt nodes
         Fr inv_c = one_m;
         if (t < 2 * cnt) inv_c = mont_mul(get(off + (t >> 1)), get(coff + (t ^ 1u)));
@@ -217,6 +232,26 @@ __global__ void __launch_bounds__(BI_T) k_batch_inv(Fr* __restrict__ out, const 
         inv_run = mont_mul(inv_run, x[c]);
         if (base + c < n) out[base + c] = ((nz >> c) & 1u) ? inv_c : big_zero<8>();
     }
+}
+// queues out = 1 / (in + beta) on st; scratch comes from the arena, which must outlive the launches
+static int batch_inv_queue(Fr* out, const Fr* in, const Fr& beta, size_t n, Arena& arena, hipStream_t st) {
+    if (n == 0) return 0;
+    if (n <= (size_t)2 * BI_T * BI_CH) {
+        hipLaunchKernelGGL((k_batch_inv<BI_T, BI_FULL>), dim3(cdiv(n, (size_t)BI_T * BI_CH)), dim3(BI_T), 0, st, out, in, beta, n, (Fr*)nullptr, (const Fr*)nullptr);
+        ZK_LAUNCH_CHECK();
+        return 0;
+    }
+    const size_t m = cdiv(n, (size_t)BI_T3 * BI_CH);
+    Scratch& roots = arena.add(sizeof(Fr) * 2 * m);
+    if (roots.rc) return roots.rc;
+    Fr* r = roots.as<Fr>();
+    hipLaunchKernelGGL((k_batch_inv<BI_T3, BI_UP>), dim3(m), dim3(BI_T3), 0, st, (Fr*)nullptr, in, beta, n, r, (const Fr*)nullptr);
+    ZK_LAUNCH_CHECK();
+    int rc = batch_inv_queue(r + m, r, big_zero<8>(), m, arena, st);
+    if (rc) return rc;
+    hipLaunchKernelGGL((k_batch_inv<BI_T3, BI_DOWN>), dim3(m), dim3(BI_T3), 0, st, out, in, beta, n, (Fr*)nullptr, (const Fr*)(r + m));
+    ZK_LAUNCH_CHECK();
+    return 0;
 }
 
 // ---- eq tables ----------------------------------------------------------------------------------------------------------
@@ -729,9 +764,11 @@ int zk_range_table(void* table, int32_t low, uint32_t len, uint32_t table_size, 
 // out[i] = 1 / (in[i] + beta), standard form; 0 where in[i] + beta == 0 (tlookup_inv_kernel tlookup.cu:50-62)
 int zk_fr_batch_inv(void* out, const void* in, const uint32_t* beta, size_t n, void* st) {
     if (n == 0) return 0;
-    hipLaunchKernelGGL(k_batch_inv, dim3(cdiv(n, (size_t)BI_T * BI_CH)), dim3(BI_T), 0, (hipStream_t)st, (Fr*)out, (const Fr*)in, load_fr(beta), n);
-    ZK_LAUNCH_CHECK();
-    return 0;
+    Arena tmp;
+    int rc = batch_inv_queue((Fr*)out, (const Fr*)in, load_fr(beta), n, tmp, (hipStream_t)st);
+    // large inputs use scratch memory that goes back to the allocator when this returns: wait for its last use
+    if (!tmp.v.empty()) { hipError_t e = hipStreamSynchronize((hipStream_t)st); if (rc == 0 && e != hipSuccess) return hip_fail(e, "hipStreamSynchronize", __FILE__, __LINE__); }
+    return rc;
 }
 // E[t] for t < 2^k (Montgomery form) from k standard-form challenges; out holds 2^k elements
 int zk_eq_table(void* out, const uint32_t* u, int k, void* stv) {
@@ -1060,8 +1097,9 @@ int zk_lookup_prove_begin(void** handle, const void* S, const void* T, const voi
     Scratch& dp = job->arena.add(sizeof(Fr) * (reduce_grid(N) + 1));
     if (A.rc || B.rc || E.rc || dp.rc) { rc = A.rc ? A.rc : (B.rc ? B.rc : (E.rc ? E.rc : dp.rc)); sumjob_abort(job); return rc; }
     const Fr b = load_fr(beta);
-    hipLaunchKernelGGL(k_batch_inv, dim3(cdiv(D, (size_t)BI_T * BI_CH)), dim3(BI_T), 0, st, A.as<Fr>(), (const Fr*)S, b, D);
-    hipLaunchKernelGGL(k_batch_inv, dim3(cdiv(N, (size_t)BI_T * BI_CH)), dim3(BI_T), 0, st, B.as<Fr>(), (const Fr*)T, b, N);
+    rc = batch_inv_queue(A.as<Fr>(), (const Fr*)S, b, D, job->arena, st);
+    if (rc == 0) rc = batch_inv_queue(B.as<Fr>(), (const Fr*)T, b, N, job->arena, st);
+    if (rc) { sumjob_abort(job); return rc; }
     const unsigned nb = reduce_grid(N);
     hipLaunchKernelGGL(k_dot_part, dim3(nb), dim3(TPB), 0, st, dp.as<Fr>() + 1, B.as<Fr>(), (const Fr*)m, N);
     hipLaunchKernelGGL(k_finish, dim3(1), dim3(TPB), 0, st, dp.as<Fr>(), dp.as<Fr>() + 1, nb);
