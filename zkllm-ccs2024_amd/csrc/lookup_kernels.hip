@@ -115,24 +115,37 @@ __global__ void __launch_bounds__(TPB) k_hist_lds(uint32_t* __restrict__ counts,
         if (c) atomicAdd(&counts[b], c);
     }
 }
-// Large tables: lanes of a wave that hold the same index are merged (up to 4 distinct leaders per
-// step) before touching global memory.
+// Large tables: a workgroup first counts its 4096 indices in a small hash table in LDS (key = bin, up to four probes)
+// and touches global memory once per distinct bin it has seen; an index that finds its four slots taken by other
+// bins goes to global memory directly.  Skewed inputs (digits of a narrow distribution: most indices in a few dozen
+// bins) then cost a few dozen global atomics per workgroup instead of thousands on the same addresses; spread-out
+// inputs fill the table and pay one global atomic per index, as they must.
+static constexpr uint32_t HH_SLOTS = 1024, HH_PER_LANE = 16, HH_EMPTY = 0xFFFFFFFFu;
 __global__ void __launch_bounds__(TPB) k_hist_global(uint32_t* __restrict__ counts, const uint32_t* __restrict__ idx, size_t n) {
-    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
-    bool pending = i < n;
-    const uint32_t my = pending ? idx[i] : 0u;
-    const uint32_t lane = threadIdx.x & 63u;
-#pragma unroll 1
-    for (int it = 0; it < 4; ++it) {
-        const unsigned long long act = __ballot(pending);
-        if (!act) break;
-        const int leader = __ffsll((long long)act) - 1;
-        const uint32_t lead = __shfl(my, leader, 64);
-        const unsigned long long same = __ballot(pending && my == lead);
-        if (lane == (uint32_t)leader) atomicAdd(&counts[lead], (uint32_t)__popcll(same));
-        if (pending && my == lead) pending = false;
+    __shared__ uint32_t keys[HH_SLOTS], cnts[HH_SLOTS];
+    for (uint32_t s = threadIdx.x; s < HH_SLOTS; s += TPB) { keys[s] = HH_EMPTY; cnts[s] = 0; }
+    __syncthreads();
+    const size_t base = (size_t)blockIdx.x * TPB * HH_PER_LANE;
+#pragma unroll 4
+    for (uint32_t k = 0; k < HH_PER_LANE; ++k) {
+        const size_t i = base + (size_t)k * TPB + threadIdx.x;
+        if (i >= n) break;
+        const uint32_t key = idx[i];
+        const uint32_t h = (key * 2654435761u) >> 22;          // 10 bits
+        bool placed = false;
+#pragma unroll
+        for (uint32_t p = 0; p < 4 && !placed; ++p) {
+            const uint32_t slot = (h + p) & (HH_SLOTS - 1);
+            const uint32_t prev = atomicCAS(&keys[slot], HH_EMPTY, key);
+            if (prev == HH_EMPTY || prev == key) { atomicAdd(&cnts[slot], 1u); placed = true; }
+        }
+        if (!placed) atomicAdd(&counts[key], 1u);
     }
-    if (pending) atomicAdd(&counts[my], 1u);
+    __syncthreads();
+    for (uint32_t s = threadIdx.x; s < HH_SLOTS; s += TPB) {
+        const uint32_t key = keys[s];
+        if (key != HH_EMPTY) atomicAdd(&counts[key], cnts[s]);
+    }
 }
 // table[i] = low + min(i, len-1)  (tlookuprange_init_kernel tlookup.cu:372-380)
 __global__ void __launch_bounds__(TPB) k_range_table(Fr* __restrict__ table, int32_t low, uint32_t len, uint32_t table_size) {
@@ -751,7 +764,7 @@ int zk_lookup_hist(void* counts_u32, const void* idx_u32, size_t n, uint32_t nbi
         if (blocks > 2048) blocks = 2048;
         hipLaunchKernelGGL(k_hist_lds, dim3(blocks), dim3(TPB), 0, st, (uint32_t*)counts_u32, (const uint32_t*)idx_u32, n, nbins);
     } else {
-        hipLaunchKernelGGL(k_hist_global, dim3(cdiv(n, TPB)), dim3(TPB), 0, st, (uint32_t*)counts_u32, (const uint32_t*)idx_u32, n);
+        hipLaunchKernelGGL(k_hist_global, dim3(cdiv(n, (size_t)TPB * HH_PER_LANE)), dim3(TPB), 0, st, (uint32_t*)counts_u32, (const uint32_t*)idx_u32, n);
     }
     ZK_LAUNCH_CHECK();
     return 0;
