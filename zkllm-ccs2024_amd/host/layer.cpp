@@ -99,12 +99,21 @@ FrTensor attn_heads_block(const LayerConfig& c, const FrTensor& Q_, const FrTens
     FrTensor QT = Q_.transpose(seq, E), KT = K_.transpose(seq, E), VT = V_.transpose(seq, E);   // embed x seq each
     FrTensor outT(E * seq);                                                                   // embed x seq, head outputs stacked by rows
     zkSoftmax softmax(c.softmax_bs, c.softmax_L, c.softmax_M, c.softmax_sf_in, c.softmax_thetas, seq, seq, d, 1);
-    for (uint h = 0; h < H; ++h) {
+    // A head's forward pass draws no challenges and records nothing, and the device side of its softmax proof runs on
+    // the library's side streams: the next head's forward pass is queued while that proof is in flight, and the proof
+    // is collected afterwards.  Challenges and transcript entries keep the order of a plain loop over the heads.
+    struct Head {
+        FrTensor Qh, Kh, Vh, X, shift, X_shifted, Y, out;
+        vector<FrTensor> X_segments, Y_segments, m_segments;
+        vector<Fr_t> v_Y;
+        vector<Polynomial> proof;
+        zkSoftmax::Pending pending;
+    };
+    auto forward = [&](uint h) {
         FrTensor Qh = QT.trunc(h * d * seq, (h + 1) * d * seq).transpose(d, seq);   // seq x d
         FrTensor KhT = KT.trunc(h * d * seq, (h + 1) * d * seq);                      // d x seq  (= K_h^T)
         FrTensor Kh = KhT.transpose(d, seq);                                          // seq x d
         FrTensor Vh = VT.trunc(h * d * seq, (h + 1) * d * seq).transpose(d, seq);   // seq x d
-
         auto X = FrTensor::matmul(Qh, KhT, seq, d, seq);
         FrTensor shift(seq), X_shifted(seq * seq);
         vector<FrTensor> X_segments, Y_segments, m_segments;
@@ -114,25 +123,40 @@ FrTensor attn_heads_block(const LayerConfig& c, const FrTensor& Q_, const FrTens
             FrTensor oT = out.transpose(seq, d);                                      // d x seq
             ZKC(zk_memcpy_d2d(outT.gpu_data + (size_t)h * d * seq, oT.gpu_data, sizeof(Fr_t) * (size_t)d * seq, nullptr));
         }
-        // proofs for this head: out = Y V, softmax, X = Q K^T
+        return std::unique_ptr<Head>(new Head{std::move(Qh), std::move(Kh), std::move(Vh), std::move(X), std::move(shift), std::move(X_shifted), std::move(Y), std::move(out),
+                                              std::move(X_segments), std::move(Y_segments), std::move(m_segments), {}, {}, {}});
+    };
+    // proofs for a head: out = Y V, softmax (begun here, finished in prove_finish), X = Q K^T
+    auto prove_start = [&](Head& hd) {
         auto temp_rand = random_vec(3);
-        vector<Polynomial> proof;
         auto u1 = random_vec(ceilLog2(seq));
         auto u2 = random_vec(ceilLog2(d));
         auto ud = random_vec(ceilLog2(seq));
-        auto claim = out.multi_dim_me({u1, u2}, {seq, d});
+        auto claim = hd.out.multi_dim_me({u1, u2}, {seq, d});
         zk_record(claim);
-        zkip(claim, Y.partial_me(u1, seq, seq), Vh.partial_me(u2, d, 1), ud, proof);
-        auto u_Y = random_vec(ceilLog2(Y.size));
-        auto v_Y = random_vec(ceilLog2(Y.size));
-        softmax.prove(Y, X, shift, X_shifted, X_segments, Y_segments, m_segments, u_Y, v_Y, temp_rand[0], temp_rand[1], temp_rand[2], proof);
+        zkip(claim, hd.Y.partial_me(u1, seq, seq), hd.Vh.partial_me(u2, d, 1), ud, hd.proof);
+        auto u_Y = random_vec(ceilLog2(hd.Y.size));
+        hd.v_Y = random_vec(ceilLog2(hd.Y.size));
+        hd.pending = softmax.prove_begin(hd.Y, hd.X_segments, hd.Y_segments, hd.m_segments, u_Y, hd.v_Y, temp_rand[0], temp_rand[1], temp_rand[2]);
+    };
+    auto prove_finish = [&](Head& hd) {
+        softmax.prove_end(hd.pending, hd.X, hd.shift, hd.X_segments, hd.Y_segments, hd.v_Y, hd.proof);
         auto u1_ = random_vec(ceilLog2(seq));
         auto u2_ = random_vec(ceilLog2(seq));
         auto ud_ = random_vec(ceilLog2(d));
-        auto claim_ = X.multi_dim_me({u1_, u2_}, {seq, seq});
+        auto claim_ = hd.X.multi_dim_me({u1_, u2_}, {seq, seq});
         zk_record(claim_);
-        zkip(claim_, Qh.partial_me(u1_, seq, d), Kh.partial_me(u2_, seq, d), ud_, proof);
+        zkip(claim_, hd.Qh.partial_me(u1_, seq, d), hd.Kh.partial_me(u2_, seq, d), ud_, hd.proof);
+    };
+    std::unique_ptr<Head> prev;
+    for (uint h = 0; h < H; ++h) {
+        std::unique_ptr<Head> cur = forward(h);
+        if (prev) prove_finish(*prev);
+        prove_start(*cur);
+        prev = std::move(cur);
     }
+    if (prev) prove_finish(*prev);
+    prev.reset();
     FrTensor out_all = outT.transpose(E, seq);   // seq x embed
     Rescaling rs1(c.sf_attn), rs2(c.sf_attn);
     auto out_ = rs2(out_all);

@@ -58,10 +58,20 @@ static const Fr_t kOne{{1, 0, 0, 0, 0, 0, 0, 0}};
 
 // proof.cu:191-241.  Each round is one pass over the tensors: the K+1 coefficient evaluations (inner products with
 // the eq table of u[:-1]) and the folds by v.back().  The device side is one job that runs beside the caller.
-HadamardPending::~HadamardPending() {
+static void hadamard_drop(void*& handle, uint K) {       // a job that was never ended is waited for and dropped
     if (!handle) return;
     std::vector<Fr_t> sums((size_t)(K + 1) * 40 + 1);
     (void)zk_hadamard_prove_end(handle, sums[0].val);
+    handle = nullptr;
+}
+HadamardPending::~HadamardPending() { hadamard_drop(handle, K); }
+HadamardPending& HadamardPending::operator=(HadamardPending&& o) noexcept {
+    if (this != &o) {
+        hadamard_drop(handle, K);
+        handle = o.handle; claim = o.claim; u = std::move(o.u); v = std::move(o.v); K = o.K; N = o.N;
+        o.handle = nullptr;
+    }
+    return *this;
 }
 HadamardPending multi_hadamard_begin(const Fr_t& claim0, const vector<FrTensor>& Xs, const vector<Fr_t>& u, const vector<Fr_t>& v) {
     HadamardPending p;

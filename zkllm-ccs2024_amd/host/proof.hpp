@@ -42,6 +42,7 @@ struct HadamardPending {
     HadamardPending(HadamardPending&& o) noexcept : handle(o.handle), claim(o.claim), u(std::move(o.u)), v(std::move(o.v)), K(o.K), N(o.N) { o.handle = nullptr; }
     HadamardPending(const HadamardPending&) = delete;
     HadamardPending& operator=(const HadamardPending&) = delete;
+    HadamardPending& operator=(HadamardPending&& o) noexcept;
     ~HadamardPending();               // a job that was never ended is waited for and dropped
     void* handle = nullptr;
     Fr_t claim;

@@ -73,21 +73,30 @@ FrTensor zkSoftmax::compute(const FrTensor& X, FrTensor& shift, FrTensor& X_shif
 Fr_t zkSoftmax::prove(const FrTensor& Y, const FrTensor& X, const FrTensor& shift, const FrTensor& X_shifted, const vector<FrTensor>& X_segments,
                       const vector<FrTensor>& Y_segments, const vector<FrTensor>& m_segments, const vector<Fr_t>& u_Y, const vector<Fr_t>& v_Y, const Fr_t& r_seg,
                       const Fr_t& alpha_seg, const Fr_t& beta_seg, vector<Polynomial>& proof) {
-    uint N = Y.size;
-    if (X.size != N) throw std::invalid_argument("X and Y must have the same size " + to_string(X.size) + " " + to_string(Y.size));
+    if (X.size != Y.size) throw std::invalid_argument("X and Y must have the same size " + to_string(X.size) + " " + to_string(Y.size));
+    Pending p = prove_begin(Y, X_segments, Y_segments, m_segments, u_Y, v_Y, r_seg, alpha_seg, beta_seg);
+    return prove_end(p, X, shift, X_segments, Y_segments, v_Y, proof);
+}
 
+zkSoftmax::Pending zkSoftmax::prove_begin(const FrTensor& Y, const vector<FrTensor>& X_segments, const vector<FrTensor>& Y_segments, const vector<FrTensor>& m_segments,
+                                          const vector<Fr_t>& u_Y, const vector<Fr_t>& v_Y, const Fr_t& r_seg, const Fr_t& alpha_seg, const Fr_t& beta_seg) {
     auto claim_Y = Y(u_Y);
     zk_record(claim_Y);
     // The Hadamard sumcheck and the K segment lookups share nothing but their challenges: their device sides are queued
     // together and run side by side; the host sides follow in the reference's order (zksoftmax.cu:177-187).
-    HadamardPending had = multi_hadamard_begin(claim_Y, Y_segments, u_Y, v_Y);
-    std::vector<LookupPending> looks;
-    looks.reserve(K);
-    for (uint i = 0; i < L; ++i) looks.push_back(least_significant_segments[i].prove_begin(X_segments[i], m_segments[i], alpha_seg, beta_seg, u_Y, v_Y));
-    for (uint i = L; i < K; ++i) looks.push_back(other_segments[i - L].prove_begin(X_segments[i], Y_segments[i - L], m_segments[i], r_seg, alpha_seg, beta_seg, u_Y, v_Y));
+    Pending p;
+    p.had = multi_hadamard_begin(claim_Y, Y_segments, u_Y, v_Y);
+    p.looks.reserve(K);
+    for (uint i = 0; i < L; ++i) p.looks.push_back(least_significant_segments[i].prove_begin(X_segments[i], m_segments[i], alpha_seg, beta_seg, u_Y, v_Y));
+    for (uint i = L; i < K; ++i) p.looks.push_back(other_segments[i - L].prove_begin(X_segments[i], Y_segments[i - L], m_segments[i], r_seg, alpha_seg, beta_seg, u_Y, v_Y));
+    return p;
+}
+
+Fr_t zkSoftmax::prove_end(Pending& pending, const FrTensor& X, const FrTensor& shift, const vector<FrTensor>& X_segments, const vector<FrTensor>& Y_segments,
+                          const vector<Fr_t>& v_Y, vector<Polynomial>& proof) {
     std::string failure;
-    try { multi_hadamard_end(had, proof); } catch (const std::exception& e) { failure = e.what(); }
-    for (auto& lp : looks) {
+    try { multi_hadamard_end(pending.had, proof); } catch (const std::exception& e) { failure = e.what(); }
+    for (auto& lp : pending.looks) {
         try { tLookup::prove_end(lp); } catch (const std::exception& e) { if (failure.empty()) failure = e.what(); }
     }
     if (!failure.empty()) throw std::runtime_error(failure);

@@ -13,6 +13,18 @@ class zkSoftmax {
                const vector<FrTensor>& Y_segments, const vector<FrTensor>& m_segments, const vector<Fr_t>& u_Y, const vector<Fr_t>& v_Y, const Fr_t& r_seg,
                const Fr_t& alpha_seg, const Fr_t& beta_seg, vector<Polynomial>& proof);
 
+    // prove in two halves: begin evaluates Y at u_Y and queues the Hadamard sumcheck and the K segment lookups on the
+    // library's side streams; end collects them in the reference's order and finishes the claims.  The caller may queue
+    // other work in between (the next head's forward pass); every tensor passed to begin must stay alive until end.
+    struct Pending {
+        HadamardPending had;
+        std::vector<LookupPending> looks;
+    };
+    Pending prove_begin(const FrTensor& Y, const vector<FrTensor>& X_segments, const vector<FrTensor>& Y_segments, const vector<FrTensor>& m_segments,
+                        const vector<Fr_t>& u_Y, const vector<Fr_t>& v_Y, const Fr_t& r_seg, const Fr_t& alpha_seg, const Fr_t& beta_seg);
+    Fr_t prove_end(Pending& pending, const FrTensor& X, const FrTensor& shift, const vector<FrTensor>& X_segments, const vector<FrTensor>& Y_segments,
+                   const vector<Fr_t>& v_Y, vector<Polynomial>& proof);
+
    protected:
     const vector<uint> bs;
     const uint K, L, M;
