@@ -223,6 +223,19 @@ def test_matmul_small_integer_path_equals_generic(pv):
     pv.lib.zkp_set_matmul_mode(ctypes.c_int(0))
     got = pv.matmul(pv.from_i64(A64), pv.from_i64(B64), 8, 16, 8).host()
     assert pv.lib.zkp_last_matmul_path() == 2 and fr_ints(got) == exp
+    # several tiles of the wide-by-narrow kernel (left operand split at 31 bits), ragged edges, negative values on both sides
+    Aw = rng.integers(-2 ** 40, 2 ** 40, (130, 300)).astype(np.int64)
+    Bn = rng.integers(-2 ** 12, 2 ** 12, (300, 70)).astype(np.int64)
+    Aw[0, :4] = [2 ** 31, -(2 ** 31), 2 ** 31 - 1, -(2 ** 31) - 1]
+    expw = [int(v) % R_MOD for v in (Aw.astype(object) @ Bn.astype(object)).reshape(-1)]
+    got = pv.matmul(pv.from_i64(Aw), pv.from_i64(Bn), 130, 300, 70).host()
+    assert pv.lib.zkp_last_matmul_path() == 2 and fr_ints(got) == expw
+    # narrow left, wide right: the 64-bit kernel
+    An = rng.integers(-2 ** 20, 2 ** 20, (8, 16)).astype(np.int64)
+    Bw = rng.integers(-2 ** 33, 2 ** 33, (16, 8)).astype(np.int64)
+    expn = [int(v) % R_MOD for v in (An.astype(object) @ Bw.astype(object)).reshape(-1)]
+    got = pv.matmul(pv.from_i64(An), pv.from_i64(Bw), 8, 16, 8).host()
+    assert pv.lib.zkp_last_matmul_path() == 2 and fr_ints(got) == expn
     A64 = rng.integers(-2 ** 50, 2 ** 50, (8, 16)).astype(np.int64)
     exp = [int(v) % R_MOD for v in (A64.astype(object) @ B64.astype(object)).reshape(-1)]
     got = pv.matmul(pv.from_i64(A64), pv.from_i64(B64), 8, 16, 8).host()

@@ -236,6 +236,66 @@ template <typename T> __global__ void __launch_bounds__(256) k_matmul_int(Fr* __
         }
 }
 
+// The same tiling for a wide left operand (|a| < 2^62) and a right operand that fits 31 bits: a = hi * 2^31 + lo with
+// 0 <= lo < 2^31, and each half takes one v_mad_i64_i32 per product; the two sums are recombined modulo 2^64, which is exact
+// because the true result is below 2^62 in magnitude.  Two multiply-adds per product instead of a 64 x 64-bit product.
+__global__ void __launch_bounds__(256) k_matmul_wide_narrow(Fr* __restrict__ C, const long long* __restrict__ A, const int* __restrict__ B, uint32_t M, uint32_t N, uint32_t P) {
+    __shared__ int Alo[16][64 + 1];
+    __shared__ int Ahi[16][64 + 1];
+    __shared__ int Bs[16][64 + 1];
+    const uint32_t tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    const uint32_t row0 = blockIdx.y * 64, col0 = blockIdx.x * 64;
+    long long lo[4][4], hi[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { lo[i][j] = 0; hi[i][j] = 0; }
+    for (uint32_t k0 = 0; k0 < N; k0 += 16) {
+        for (uint32_t e = threadIdx.x; e < 64 * 16; e += 256) {
+            const uint32_t r = e / 16, q = e % 16;        // A: 64 rows x 16 k
+            const long long a = (row0 + r < M && k0 + q < N) ? A[(size_t)(row0 + r) * N + k0 + q] : 0ll;
+            Alo[q][r] = (int)(a & 0x7FFFFFFFll);
+            Ahi[q][r] = (int)(a >> 31);
+            const uint32_t q2 = e / 64, c = e % 64;       // B: 16 k x 64 cols
+            Bs[q2][c] = (k0 + q2 < N && col0 + c < P) ? B[(size_t)(k0 + q2) * P + col0 + c] : 0;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            int al[4], ah[4], bv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { al[i] = Alo[q][ty * 4 + i]; ah[i] = Ahi[q][ty * 4 + i]; bv[i] = Bs[q][tx * 4 + i]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    lo[i][j] += (long long)al[i] * (long long)bv[j];
+                    hi[i][j] += (long long)ah[i] * (long long)bv[j];
+                }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t r = row0 + ty * 4 + i, c = col0 + tx * 4 + j;
+            const long long v = (long long)(((unsigned long long)hi[i][j] << 31) + (unsigned long long)lo[i][j]);
+            if (r < M && c < P) C[(size_t)r * P + c] = fr_from_i64(v);
+        }
+}
+static int run_wide_narrow_path(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, hipStream_t st) {
+    const size_t na = (size_t)M * N, nb = (size_t)N * P;
+    Scratch ai(na * sizeof(long long)), bi(nb * sizeof(int));
+    if (ai.rc) return ai.rc;
+    if (bi.rc) return bi.rc;
+    hipLaunchKernelGGL(k_fr_to_int<long long>, dim3(cdiv(na, 256)), dim3(256), 0, st, ai.as<long long>(), (const Fr*)A, na);
+    hipLaunchKernelGGL(k_fr_to_int<int>, dim3(cdiv(nb, 256)), dim3(256), 0, st, bi.as<int>(), (const Fr*)B, nb);
+    hipLaunchKernelGGL(k_matmul_wide_narrow, dim3(cdiv(P, 64), cdiv(M, 64)), dim3(256), 0, st, (Fr*)C, ai.as<long long>(), bi.as<int>(), M, N, P);
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
+
 template <typename T> static int run_int_path(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, hipStream_t st) {
     const size_t na = (size_t)M * N, nb = (size_t)N * P;
     Scratch ai(na * sizeof(T)), bi(nb * sizeof(T));
@@ -271,7 +331,7 @@ int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, 
     if (M == 0 || P == 0) return 0;
     ZK_ARG(N > 0, "zk_fr_matmul: inner dimension is 0");
     ZK_ARG(mode >= 0 && mode <= 2, "zk_fr_matmul: mode must be 0, 1 or 2");
-    bool small = false, fits32 = false;
+    bool small = false, fits32 = false, b_fits32 = false;
     if (mode != 1) {
         Scratch mx(3 * sizeof(unsigned long long));
         if (mx.rc) return mx.rc;
@@ -292,6 +352,7 @@ int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, 
             const unsigned __int128 bound = (unsigned __int128)ra * mb;
             small = bound < ((unsigned __int128)1 << 62);
             fits32 = ma < (1ull << 31) && mb < (1ull << 31);
+            b_fits32 = mb < (1ull << 31) && ma < (1ull << 62);
         }
         if (mode == 2 && !small) { set_error(ZK_ERR_ARG, "zk_fr_matmul: operands do not satisfy the small-integer bound"); return ZK_ERR_ARG; }
     }
@@ -300,7 +361,9 @@ int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, 
         return zk_fr_matmul_generic(C, A, B, M, N, P, stv);
     }
     if (path_used) *path_used = 2;
-    return fits32 ? run_int_path<int>(C, A, B, M, N, P, st) : run_int_path<long long>(C, A, B, M, N, P, st);
+    if (fits32) return run_int_path<int>(C, A, B, M, N, P, st);
+    if (b_fits32) return run_wide_narrow_path(C, A, B, M, N, P, st);
+    return run_int_path<long long>(C, A, B, M, N, P, st);
 }
 
 }  // extern "C"
