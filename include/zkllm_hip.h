@@ -177,6 +177,12 @@ int zk_hadamard_sumcheck(uint32_t* coefs_host, const void* const* Xs, int K, con
  * Inputs must stay alive and unmodified until end; every handle must be ended exactly once.  bm_host: <B, m>, 8 limbs. */
 int zk_lookup_prove_begin(void** handle, const void* S, const void* T, const void* m, const uint32_t* beta, const uint32_t* u_eq, const uint32_t* v, size_t D, size_t N,
                           int rounds, void* stream);
+/* the same job when the queries are expected to be table entries (tLookupRange::prep / tLookupRangeMapping, tlookup.cu:393-421,
+ * build S from the table): query i should equal T[hint[i] - low], hint being D field elements (for a range table the
+ * looked-up values themselves).  Results are identical to zk_lookup_prove_begin's for every input; where the hint
+ * holds, 1/(S[i]+beta) is read from B instead of being computed, and a query that does not match is inverted on its own. */
+int zk_lookup_prove_begin_hinted(void** handle, const void* S, const void* T, const void* m, const void* hint_fr, int32_t low, const uint32_t* beta, const uint32_t* u_eq,
+                                 const uint32_t* v, size_t D, size_t N, int rounds, void* stream);
 int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host);
 int zk_hadamard_prove_begin(void** handle, const void* const* Xs, int K, const uint32_t* u_eq, const uint32_t* v, size_t N, void* stream);
 int zk_hadamard_prove_end(void* handle, uint32_t* coefs_host);

@@ -210,3 +210,43 @@ def test_softmax_compute_and_prove(pv, orc, m, n, d, bs, sf, lim):
     assert (Y.host() == e_Y).all()
     t = pv.transcript()
     assert t.shape == e_t.shape and (t == e_t).all()
+
+
+def test_hinted_lookup_job_equals_the_plain_one_whatever_the_hints():
+    """zk_lookup_prove_begin_hinted reads 1/(S+beta) from the table's inverses where the hinted entry matches and must
+    deliver what zk_lookup_prove_begin delivers for every input: right hints, wrong hints, hints outside the table,
+    queries that are no table entry at all, and a query with S + beta == 0."""
+    import ctypes
+    from gpuhelp import Hip, c_void_p, c_size_t, c_int
+    hip = Hip()
+    D, N, low = 1 << 13, 64, -7
+    k = 13
+    rng = np.random.default_rng(99)
+    T = ch(41, N)                                   # arbitrary table entries
+    pos = rng.integers(0, N, D)
+    S = T[pos].copy()
+    hint_int = (pos + low).astype(np.int64)         # right hints: hint - low == position
+    wrong = rng.choice(D, 300, replace=False)
+    hint_int[wrong[:100]] = (pos[wrong[:100]] + 1) % N + low          # another entry of the table
+    hint_int[wrong[100:200]] = low + N + 5                            # outside the table
+    S[wrong[200:]] = ch(42, 100)                                      # queries that are no table entries
+    beta = ch(43, 1)[0]
+    S[wrong[7]] = fr_array([(-fr_ints(beta.reshape(1, 8))[0]) % R_MOD])[0]
+    hint = fr_array([int(x) % R_MOD for x in hint_int])
+    m = fr_array([int(c) for c in np.bincount(pos, minlength=N)])
+    u, v = ch(44, k - 1), ch(45, k)
+    dS, dT, dm, dh = hip.upload(S), hip.upload(T), hip.upload(m), hip.upload(hint)
+    res = []
+    for hinted in (False, True):
+        h = c_void_p()
+        if hinted:
+            hip.call("zk_lookup_prove_begin_hinted", ctypes.byref(h), c_void_p(dS), c_void_p(dT), c_void_p(dm), c_void_p(dh), c_int(low), beta, u, v, c_size_t(D), c_size_t(N), c_int(k), None)
+        else:
+            hip.call("zk_lookup_prove_begin", ctypes.byref(h), c_void_p(dS), c_void_p(dT), c_void_p(dm), beta, u, v, c_size_t(D), c_size_t(N), c_int(k), None)
+        bm, sums = np.zeros(8, np.uint32), np.zeros((k * 11, 8), np.uint32)
+        hip.call("zk_lookup_prove_end", h, bm, sums)
+        res.append((bm, sums))
+    assert (res[0][0] == res[1][0]).all() and (res[0][1] == res[1][1]).all()
+    assert res[0][1].any()
+    for p in (dS, dT, dm, dh):
+        hip.free(p)

@@ -267,6 +267,35 @@ static int batch_inv_queue(Fr* out, const Fr* in, const Fr& beta, size_t n, Aren
     return 0;
 }
 
+// A[i] = 1 / (S[i] + beta) when every S[i] is expected to be a table entry: if S[i] equals T[j] for the hinted position
+// j = hint[i] - low, the inverse is B[j] = 1 / (T[j] + beta), already computed for the table -- one gather instead of a
+// share of a batch inversion over all D queries.  Whatever the hint, the result is the inverse itself: a query that
+// does not match its hinted entry (a hint outside the table, inconsistent inputs) is inverted on its own.
+__global__ void __launch_bounds__(TPB) k_inv_by_hint(Fr* __restrict__ A, const Fr* __restrict__ S, const Fr* __restrict__ T, const Fr* __restrict__ B, const Fr* __restrict__ hint,
+                                                     const Fr low, const Fr beta, size_t D, uint32_t N) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= D) return;
+    const Fr sv = S[i];
+    const Fr d = sub(hint[i], low);
+    const bool in_table = !(d.v[1] | d.v[2] | d.v[3] | d.v[4] | d.v[5] | d.v[6] | d.v[7]) && d.v[0] < N;
+    const uint32_t j = in_table ? d.v[0] : 0u;
+    if (equal(sv, T[j])) {
+        A[i] = B[j];
+        return;
+    }
+    const Fr v = add(sv, beta);
+    Fr out = big_zero<8>();
+    if (!is_zero(v)) {
+        // v is the Montgomery form of v/R: its Montgomery inverse is R^2/v, and a Montgomery product with R^-1 leaves 1/v
+        constexpr uint32_t RINV[8] = {4269129792u, 334977897u, 165441631u, 2876230287u, 1333208682u, 1912866698u, 805346647u, 465471123u};
+        Fr k;
+#pragma unroll
+        for (int l = 0; l < 8; ++l) k.v[l] = RINV[l];
+        out = mont_mul(mont_inverse(v), k);
+    }
+    A[i] = out;
+}
+
 // ---- eq tables ----------------------------------------------------------------------------------------------------------
 // E[t] = prod_j (u_j if bit_j(t) else 1-u_j), Montgomery form.  Built by doubling: level j appends bit j.
 __global__ void __launch_bounds__(TPB) k_eq_double(Fr* __restrict__ e, const Fr u_mont, const Fr one_minus_u_mont, size_t half) {
@@ -1095,8 +1124,8 @@ int zk_lookup_sumcheck(uint32_t* sums_host, const void* A, const void* S, const 
 // B = 1/(T + beta), <B, m>, the eq table of u_eq (rounds - 1 challenges), then every round.  S: D elements; T, m: N.
 // begin returns at once; S, T, m must stay alive and unmodified until end, which waits and delivers <B, m>
 // (standard form) and the rounds x 11 sums.  Every handle must be ended exactly once.
-int zk_lookup_prove_begin(void** handle, const void* S, const void* T, const void* m, const uint32_t* beta, const uint32_t* u_eq, const uint32_t* v, size_t D, size_t N,
-                          int rounds, void* stv) {
+static int lookup_prove_begin(void** handle, const void* S, const void* T, const void* m, const void* hint, int32_t low, const uint32_t* beta, const uint32_t* u_eq,
+                              const uint32_t* v, size_t D, size_t N, int rounds, void* stv) {
     ZK_ARG(handle != nullptr, "zk_lookup_prove_begin: null handle");
     int rc = lookup_args_ok(D, N, rounds);
     if (rc) return rc;
@@ -1110,8 +1139,17 @@ int zk_lookup_prove_begin(void** handle, const void* S, const void* T, const voi
     Scratch& dp = job->arena.add(sizeof(Fr) * (reduce_grid(N) + 1));
     if (A.rc || B.rc || E.rc || dp.rc) { rc = A.rc ? A.rc : (B.rc ? B.rc : (E.rc ? E.rc : dp.rc)); sumjob_abort(job); return rc; }
     const Fr b = load_fr(beta);
-    rc = batch_inv_queue(A.as<Fr>(), (const Fr*)S, b, D, job->arena, st);
-    if (rc == 0) rc = batch_inv_queue(B.as<Fr>(), (const Fr*)T, b, N, job->arena, st);
+    rc = batch_inv_queue(B.as<Fr>(), (const Fr*)T, b, N, job->arena, st);
+    if (rc == 0) {
+        if (hint) {
+            hipLaunchKernelGGL(k_inv_by_hint, dim3(cdiv(D, TPB)), dim3(TPB), 0, st, A.as<Fr>(), (const Fr*)S, (const Fr*)T, B.as<Fr>(), (const Fr*)hint, fr_from_i64((int64_t)low), b, D,
+                               (uint32_t)N);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) rc = hip_fail(e, "k_inv_by_hint", __FILE__, __LINE__);
+        } else {
+            rc = batch_inv_queue(A.as<Fr>(), (const Fr*)S, b, D, job->arena, st);
+        }
+    }
     if (rc) { sumjob_abort(job); return rc; }
     const unsigned nb = reduce_grid(N);
     hipLaunchKernelGGL(k_dot_part, dim3(nb), dim3(TPB), 0, st, dp.as<Fr>() + 1, B.as<Fr>(), (const Fr*)m, N);
@@ -1123,6 +1161,18 @@ int zk_lookup_prove_begin(void** handle, const void* S, const void* T, const voi
     if (rc) { sumjob_abort(job); return rc; }
     *handle = job;
     return 0;
+}
+int zk_lookup_prove_begin(void** handle, const void* S, const void* T, const void* m, const uint32_t* beta, const uint32_t* u_eq, const uint32_t* v, size_t D, size_t N,
+                          int rounds, void* stv) {
+    return lookup_prove_begin(handle, S, T, m, nullptr, 0, beta, u_eq, v, D, N, rounds, stv);
+}
+// The same for queries that are expected to be table entries, with a hint where: query i should equal T[hint[i] - low]
+// (hint: D field elements -- for a range table, the looked-up values themselves).  The results are those of
+// zk_lookup_prove_begin for every input; where the hint holds, 1/(S[i] + beta) is read from the table's inverses.
+int zk_lookup_prove_begin_hinted(void** handle, const void* S, const void* T, const void* m, const void* hint, int32_t low, const uint32_t* beta, const uint32_t* u_eq,
+                                 const uint32_t* v, size_t D, size_t N, int rounds, void* stv) {
+    ZK_ARG(hint != nullptr, "zk_lookup_prove_begin_hinted: null hint");
+    return lookup_prove_begin(handle, S, T, m, hint, low, beta, u_eq, v, D, N, rounds, stv);
 }
 int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host) {
     ZK_ARG(handle != nullptr, "zk_lookup_prove_end: null handle");

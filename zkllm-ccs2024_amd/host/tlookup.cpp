@@ -91,7 +91,8 @@ LookupPending& LookupPending::operator=(LookupPending&& o) noexcept {
 // tLookup_phase1 / tLookup_phase2 (tlookup.cu:184-320).  The device side -- inverses, <B, m>, eq table and every round --
 // is one job that runs beside the caller; the host side turns each round's sums into its polynomial, checks it and
 // derives the next claim.
-LookupPending tLookup_sumcheck_begin(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0, const Fr_t& alpha0, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v) {
+LookupPending tLookup_sumcheck_begin(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0, const Fr_t& alpha0, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v,
+                                     const FrTensor* hint, int low) {
     const uint D = S0.size, N = m0.size;
     if (m0.size != T0.size) throw std::runtime_error("m.size != table.size");
     if (D != (1u << ceilLog2(D)) || N != (1u << ceilLog2(N)) || D % N != 0) throw std::runtime_error("D or N is not power of 2, or D is not divisible by N");
@@ -105,7 +106,9 @@ LookupPending tLookup_sumcheck_begin(const FrTensor& S0, const FrTensor& T0, con
     // fold challenges in round order: v1 = v[0..n1) consumed from its back, then v2 = v[n1..k) from its back
     std::vector<Fr_t> vs(k);
     for (uint r = 0; r < k; ++r) vs[r] = r >= n1 ? v[k - 1 - (r - n1)] : v[n1 - 1 - r];
-    ZKC(zk_lookup_prove_begin(&p.handle, S0.gpu_data, T0.gpu_data, m0.gpu_data, beta.val, u[0].val, vs[0].val, D, N, (int)k, nullptr));
+    if (hint && hint->size != D) throw std::runtime_error("lookup hint must have one entry per query");
+    if (hint) ZKC(zk_lookup_prove_begin_hinted(&p.handle, S0.gpu_data, T0.gpu_data, m0.gpu_data, hint->gpu_data, low, beta.val, u[0].val, vs[0].val, D, N, (int)k, nullptr));
+    else ZKC(zk_lookup_prove_begin(&p.handle, S0.gpu_data, T0.gpu_data, m0.gpu_data, beta.val, u[0].val, vs[0].val, D, N, (int)k, nullptr));
     return p;
 }
 
@@ -166,6 +169,15 @@ LookupPending tLookup::prove_begin(const FrTensor& S, const FrTensor& m, const F
     return tLookup_sumcheck_begin(S, table, m, alpha, beta, u, v);
 }
 
+LookupPending tLookupRange::prove_begin(const FrTensor& S, const FrTensor& m, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v) {
+    if (m.size != table.size) throw std::runtime_error("m.size != table.size");
+    return tLookup_sumcheck_begin(S, table, m, alpha, beta, u, v, &S, low);
+}
+Fr_t tLookupRange::prove(const FrTensor& S, const FrTensor& m, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v, vector<Polynomial>& proof) {
+    LookupPending p = prove_begin(S, m, alpha, beta, u, v);
+    return tLookup_sumcheck_end(p);
+}
+
 LookupPending tLookupRangeMapping::prove_begin(const FrTensor& S_in, const FrTensor& S_out, const FrTensor& m, const Fr_t& r, const Fr_t& alpha, const Fr_t& beta,
                                                const vector<Fr_t>& u, const vector<Fr_t>& v) {
     const uint D = S_in.size;
@@ -190,7 +202,7 @@ LookupPending tLookupRangeMapping::prove_begin(const FrTensor& S_in, const FrTen
     const FrTensor* S_com = keep.back().get();
     keep.emplace_back(new FrTensor(table + mapped_vals * r));
     const FrTensor* T_com = keep.back().get();
-    LookupPending p = tLookup_sumcheck_begin(*S_com, *T_com, *mm, alpha, beta, u, v);
+    LookupPending p = tLookup_sumcheck_begin(*S_com, *T_com, *mm, alpha, beta, u, v, si, low);
     p.keep = std::move(keep);
     return p;
 }

@@ -21,7 +21,9 @@ struct LookupPending {
     vector<Fr_t> u, v;
     uint D = 0, N = 0;
 };
-LookupPending tLookup_sumcheck_begin(const FrTensor& S, const FrTensor& T, const FrTensor& m, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v);
+// hint / low: optionally, where each query is expected in the table (query i == T[hint[i] - low]); never changes a result
+LookupPending tLookup_sumcheck_begin(const FrTensor& S, const FrTensor& T, const FrTensor& m, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v,
+                                     const FrTensor* hint = nullptr, int low = 0);
 Fr_t tLookup_sumcheck_end(LookupPending& p);
 
 class tLookup {
@@ -47,8 +49,9 @@ class tLookupRange : public tLookup {
     FrTensor prep(const int* vals, const uint D);   // vals: device pointer
     FrTensor prep(const FrTensor& vals);
 
-    using tLookup::prove;
-    using tLookup::prove_begin;
+    // the queries of a range lookup are their own hints for the table position (value - low)
+    Fr_t prove(const FrTensor& S, const FrTensor& m, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v, vector<Polynomial>& proof);
+    LookupPending prove_begin(const FrTensor& S, const FrTensor& m, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v);
 };
 
 class tLookupRangeMapping : public tLookupRange {
