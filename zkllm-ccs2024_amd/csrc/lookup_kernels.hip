@@ -913,6 +913,8 @@ struct SumJob {
     Fr* extra = nullptr;         // one more value fetched with the sums (lookup: <B, m> with R^-1 attached), or null
     int rounds = 0, per_round = 0, n1 = 0;
     hipEvent_t ready = nullptr;
+    void* host = nullptr;        // jobs on a side stream: pinned buffer the results are copied to behind the last kernel ...
+    hipEvent_t done = nullptr;   // ... and the event behind that copy
 };
 __global__ void __launch_bounds__(TPB) k_dot_part(Fr* __restrict__ partials, const Fr* __restrict__ a, const Fr* __restrict__ b, size_t n) {
     Fr acc[1] = {big_zero<8>()};
@@ -1060,8 +1062,25 @@ static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, 
     return 0;
 }
 // waits for the job's stream and copies its sums (and the extra value) to the host
+// a job on a side stream: the copy of its results is queued with it, and collecting waits for that copy only
+static int sumjob_queue_results(SumJob& job) {
+    const size_t nsum = (size_t)job.rounds * job.per_round;
+    int rc = pinned_acquire(&job.host);
+    if (rc) return rc;
+    ZK_HIP(hipMemcpyAsync(job.host, job.sums, sizeof(Fr) * nsum, hipMemcpyDeviceToHost, job.st));
+    if (job.extra) ZK_HIP(hipMemcpyAsync((Fr*)job.host + nsum, job.extra, sizeof(Fr), hipMemcpyDeviceToHost, job.st));
+    ZK_HIP(hipEventCreateWithFlags(&job.done, hipEventDisableTiming));
+    ZK_HIP(hipEventRecord(job.done, job.st));
+    return 0;
+}
 static int sumjob_collect(SumJob& job, Fr* sums_host, Fr* extra_host) {
     const size_t nsum = (size_t)job.rounds * job.per_round;
+    if (job.done) {
+        ZK_HIP(hipEventSynchronize(job.done));
+        memcpy(sums_host, job.host, sizeof(Fr) * nsum);
+        if (job.extra && extra_host) memcpy(extra_host, (Fr*)job.host + nsum, sizeof(Fr));
+        return 0;
+    }
     void* stage = nullptr;
     int rc = staging(&stage, sizeof(Fr) * (nsum + 1));
     if (rc) return rc;
@@ -1098,7 +1117,11 @@ static int sumjob_on_side_stream(SumJob& job, hipStream_t caller) {
     return 0;
 }
 static void sumjob_abort(SumJob* job) {
-    if (job->st) (void)hipStreamSynchronize(job->st);
+    // the job's buffers go back to the allocator: wait for its last use (the whole stream when the job never got as far as its event)
+    if (job->done) (void)hipEventSynchronize(job->done);
+    else if (job->st) (void)hipStreamSynchronize(job->st);
+    if (job->done) (void)hipEventDestroy(job->done);
+    pinned_release(job->host);
     if (job->ready) (void)hipEventDestroy(job->ready);
     delete job;
 }
@@ -1158,6 +1181,7 @@ static int lookup_prove_begin(void** handle, const void* S, const void* T, const
     rc = eq_table_queue(E.as<Fr>(), u_eq, rounds - 1, job->arena, st);
     if (rc) { sumjob_abort(job); return rc; }
     rc = lookup_queue(*job, A.as<Fr>(), (const Fr*)S, B.as<Fr>(), (const Fr*)T, (const Fr*)m, E.as<Fr>(), b, v, D, N, rounds);
+    if (rc == 0) rc = sumjob_queue_results(*job);
     if (rc) { sumjob_abort(job); return rc; }
     *handle = job;
     return 0;
@@ -1215,6 +1239,7 @@ int zk_hadamard_prove_begin(void** handle, const void* const* Xs, int K, const u
     rc = eq_table_queue(E.as<Fr>(), u_eq, k - 1, job->arena, job->st);
     if (rc) { sumjob_abort(job); return rc; }
     rc = hadamard_queue(*job, (const Fr* const*)Xs, K, E.as<Fr>(), v, N);
+    if (rc == 0) rc = sumjob_queue_results(*job);
     if (rc) { sumjob_abort(job); return rc; }
     *handle = job;
     return 0;

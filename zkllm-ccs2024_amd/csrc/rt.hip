@@ -113,6 +113,24 @@ hipStream_t side_stream(int pool) {
     return streams[q][i];
 }
 
+static std::mutex g_pinned_mu;
+static std::vector<void*> g_pinned_free;
+int pinned_acquire(void** host_ptr) {
+    {
+        std::lock_guard<std::mutex> lk(g_pinned_mu);
+        if (!g_pinned_free.empty()) { *host_ptr = g_pinned_free.back(); g_pinned_free.pop_back(); return 0; }
+    }
+    void* p = nullptr;
+    ZK_HIP(hipHostMalloc(&p, 64 << 10, hipHostMallocDefault));
+    *host_ptr = p;
+    return 0;
+}
+void pinned_release(void* host_ptr) {
+    if (!host_ptr) return;
+    std::lock_guard<std::mutex> lk(g_pinned_mu);
+    g_pinned_free.push_back(host_ptr);
+}
+
 int staging(void** host_ptr, size_t bytes) {
     static void* buf = nullptr;
     static const size_t cap = 64 << 10;

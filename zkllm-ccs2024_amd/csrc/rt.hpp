@@ -59,6 +59,11 @@ struct Arena {
 // Two pools, so that a short job (pool 1: sumchecks) never queues behind a long one (pool 0: openings).
 hipStream_t side_stream(int pool);
 
+// Pinned host buffers of 64 KiB for results that a job on a side stream copies out behind its last kernel, so that
+// fetching them waits for that job alone (an event) and not for whatever was queued on the stream after it.
+int pinned_acquire(void** host_ptr);
+void pinned_release(void* host_ptr);
+
 // Pinned host buffer (64 KiB) for device->host results of reductions.
 int staging(void** host_ptr, size_t bytes);
 

@@ -99,13 +99,16 @@ FrTensor attn_heads_block(const LayerConfig& c, const FrTensor& Q_, const FrTens
     FrTensor QT = Q_.transpose(seq, E), KT = K_.transpose(seq, E), VT = V_.transpose(seq, E);   // embed x seq each
     FrTensor outT(E * seq);                                                                   // embed x seq, head outputs stacked by rows
     zkSoftmax softmax(c.softmax_bs, c.softmax_L, c.softmax_M, c.softmax_sf_in, c.softmax_thetas, seq, seq, d, 1);
-    // A head's forward pass draws no challenges and records nothing, and the device side of its softmax proof runs on
-    // the library's side streams: the next head's forward pass is queued while that proof is in flight, and the proof
-    // is collected afterwards.  Challenges and transcript entries keep the order of a plain loop over the heads.
+    // A head's forward pass draws no challenges and records nothing, and the device side of its softmax proof (the
+    // Hadamard and lookup sumcheck jobs) needs only challenges and the forward pass's tensors.  So the loop runs one head
+    // ahead: head h's forward pass and its proof jobs are queued first, then the host finishes head h-1 (collects its
+    // jobs, writes its transcript entries) and writes the entries of head h that precede its jobs' results.  The jobs run
+    // on the library's side streams beside all of that.  Challenges are drawn and transcript entries written in the order
+    // of a plain loop over the heads.
     struct Head {
         FrTensor Qh, Kh, Vh, X, shift, X_shifted, Y, out;
         vector<FrTensor> X_segments, Y_segments, m_segments;
-        vector<Fr_t> v_Y;
+        vector<Fr_t> temp_rand, u1, u2, ud, u_Y, v_Y, u1_, u2_, ud_;
         vector<Polynomial> proof;
         zkSoftmax::Pending pending;
     };
@@ -123,39 +126,51 @@ FrTensor attn_heads_block(const LayerConfig& c, const FrTensor& Q_, const FrTens
             FrTensor oT = out.transpose(seq, d);                                      // d x seq
             ZKC(zk_memcpy_d2d(outT.gpu_data + (size_t)h * d * seq, oT.gpu_data, sizeof(Fr_t) * (size_t)d * seq, nullptr));
         }
-        return std::unique_ptr<Head>(new Head{std::move(Qh), std::move(Kh), std::move(Vh), std::move(X), std::move(shift), std::move(X_shifted), std::move(Y), std::move(out),
-                                              std::move(X_segments), std::move(Y_segments), std::move(m_segments), {}, {}, {}});
+        std::unique_ptr<Head> hd(new Head{std::move(Qh), std::move(Kh), std::move(Vh), std::move(X), std::move(shift), std::move(X_shifted), std::move(Y), std::move(out),
+                                          std::move(X_segments), std::move(Y_segments), std::move(m_segments), {}, {}, {}, {}, {}, {}, {}, {}, {}, {}, {}});
+        return hd;
     };
-    // proofs for a head: out = Y V, softmax (begun here, finished in prove_finish), X = Q K^T
-    auto prove_start = [&](Head& hd) {
-        auto temp_rand = random_vec(3);
-        auto u1 = random_vec(ceilLog2(seq));
-        auto u2 = random_vec(ceilLog2(d));
-        auto ud = random_vec(ceilLog2(seq));
-        auto claim = hd.out.multi_dim_me({u1, u2}, {seq, d});
-        zk_record(claim);
-        zkip(claim, hd.Y.partial_me(u1, seq, seq), hd.Vh.partial_me(u2, d, 1), ud, hd.proof);
-        auto u_Y = random_vec(ceilLog2(hd.Y.size));
+    // challenges of a head in the order self-attn.cu:97-119 draws them: first part before the proofs, second before X = Q K^T
+    auto draw_first = [&](Head& hd) {
+        hd.temp_rand = random_vec(3);
+        hd.u1 = random_vec(ceilLog2(seq));
+        hd.u2 = random_vec(ceilLog2(d));
+        hd.ud = random_vec(ceilLog2(seq));
+        hd.u_Y = random_vec(ceilLog2(hd.Y.size));
         hd.v_Y = random_vec(ceilLog2(hd.Y.size));
-        hd.pending = softmax.prove_begin(hd.Y, hd.X_segments, hd.Y_segments, hd.m_segments, u_Y, hd.v_Y, temp_rand[0], temp_rand[1], temp_rand[2]);
     };
-    auto prove_finish = [&](Head& hd) {
+    auto draw_second = [&](Head& hd) {
+        hd.u1_ = random_vec(ceilLog2(seq));
+        hd.u2_ = random_vec(ceilLog2(seq));
+        hd.ud_ = random_vec(ceilLog2(d));
+    };
+    // proofs for a head: out = Y V, softmax, X = Q K^T
+    auto records_first = [&](Head& hd) {
+        auto claim = hd.out.multi_dim_me({hd.u1, hd.u2}, {seq, d});
+        zk_record(claim);
+        zkip(claim, hd.Y.partial_me(hd.u1, seq, seq), hd.Vh.partial_me(hd.u2, d, 1), hd.ud, hd.proof);
+        softmax.claim_record(hd.pending, hd.Y, hd.u_Y);
+    };
+    auto records_second = [&](Head& hd) {
         softmax.prove_end(hd.pending, hd.X, hd.shift, hd.X_segments, hd.Y_segments, hd.v_Y, hd.proof);
-        auto u1_ = random_vec(ceilLog2(seq));
-        auto u2_ = random_vec(ceilLog2(seq));
-        auto ud_ = random_vec(ceilLog2(d));
-        auto claim_ = hd.X.multi_dim_me({u1_, u2_}, {seq, seq});
+        auto claim_ = hd.X.multi_dim_me({hd.u1_, hd.u2_}, {seq, seq});
         zk_record(claim_);
-        zkip(claim_, hd.Qh.partial_me(u1_, seq, d), hd.Kh.partial_me(u2_, seq, d), ud_, hd.proof);
+        zkip(claim_, hd.Qh.partial_me(hd.u1_, seq, d), hd.Kh.partial_me(hd.u2_, seq, d), hd.ud_, hd.proof);
     };
     std::unique_ptr<Head> prev;
     for (uint h = 0; h < H; ++h) {
         std::unique_ptr<Head> cur = forward(h);
-        if (prev) prove_finish(*prev);
-        prove_start(*cur);
+        if (prev) draw_second(*prev);
+        draw_first(*cur);
+        cur->pending = softmax.jobs_begin(cur->X_segments, cur->Y_segments, cur->m_segments, cur->u_Y, cur->v_Y, cur->temp_rand[0], cur->temp_rand[1], cur->temp_rand[2]);
+        if (prev) records_second(*prev);
+        records_first(*cur);
         prev = std::move(cur);
     }
-    if (prev) prove_finish(*prev);
+    if (prev) {
+        draw_second(*prev);
+        records_second(*prev);
+    }
     prev.reset();
     FrTensor out_all = outT.transpose(E, seq);   // seq x embed
     Rescaling rs1(c.sf_attn), rs2(c.sf_attn);

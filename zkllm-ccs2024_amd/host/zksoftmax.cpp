@@ -82,14 +82,27 @@ zkSoftmax::Pending zkSoftmax::prove_begin(const FrTensor& Y, const vector<FrTens
                                           const vector<Fr_t>& u_Y, const vector<Fr_t>& v_Y, const Fr_t& r_seg, const Fr_t& alpha_seg, const Fr_t& beta_seg) {
     auto claim_Y = Y(u_Y);
     zk_record(claim_Y);
+    Pending p = jobs_begin(X_segments, Y_segments, m_segments, u_Y, v_Y, r_seg, alpha_seg, beta_seg);
+    p.had.claim = claim_Y;
+    return p;
+}
+
+zkSoftmax::Pending zkSoftmax::jobs_begin(const vector<FrTensor>& X_segments, const vector<FrTensor>& Y_segments, const vector<FrTensor>& m_segments, const vector<Fr_t>& u_Y,
+                                         const vector<Fr_t>& v_Y, const Fr_t& r_seg, const Fr_t& alpha_seg, const Fr_t& beta_seg) {
     // The Hadamard sumcheck and the K segment lookups share nothing but their challenges: their device sides are queued
     // together and run side by side; the host sides follow in the reference's order (zksoftmax.cu:177-187).
     Pending p;
-    p.had = multi_hadamard_begin(claim_Y, Y_segments, u_Y, v_Y);
+    p.had = multi_hadamard_begin(Fr_t{{0, 0, 0, 0, 0, 0, 0, 0}}, Y_segments, u_Y, v_Y);     // the claim is only looked at by multi_hadamard_end
     p.looks.reserve(K);
     for (uint i = 0; i < L; ++i) p.looks.push_back(least_significant_segments[i].prove_begin(X_segments[i], m_segments[i], alpha_seg, beta_seg, u_Y, v_Y));
     for (uint i = L; i < K; ++i) p.looks.push_back(other_segments[i - L].prove_begin(X_segments[i], Y_segments[i - L], m_segments[i], r_seg, alpha_seg, beta_seg, u_Y, v_Y));
     return p;
+}
+
+void zkSoftmax::claim_record(Pending& pending, const FrTensor& Y, const vector<Fr_t>& u_Y) {
+    auto claim_Y = Y(u_Y);
+    zk_record(claim_Y);
+    pending.had.claim = claim_Y;
 }
 
 Fr_t zkSoftmax::prove_end(Pending& pending, const FrTensor& X, const FrTensor& shift, const vector<FrTensor>& X_segments, const vector<FrTensor>& Y_segments,

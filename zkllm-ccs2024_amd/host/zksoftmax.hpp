@@ -22,6 +22,11 @@ class zkSoftmax {
     };
     Pending prove_begin(const FrTensor& Y, const vector<FrTensor>& X_segments, const vector<FrTensor>& Y_segments, const vector<FrTensor>& m_segments,
                         const vector<Fr_t>& u_Y, const vector<Fr_t>& v_Y, const Fr_t& r_seg, const Fr_t& alpha_seg, const Fr_t& beta_seg);
+    // prove_begin in two steps, for a caller that has transcript entries of its own to write between them: jobs_begin only
+    // queues the device side (it records nothing), claim_record evaluates Y at u_Y and records it -- call it before prove_end.
+    Pending jobs_begin(const vector<FrTensor>& X_segments, const vector<FrTensor>& Y_segments, const vector<FrTensor>& m_segments, const vector<Fr_t>& u_Y,
+                       const vector<Fr_t>& v_Y, const Fr_t& r_seg, const Fr_t& alpha_seg, const Fr_t& beta_seg);
+    void claim_record(Pending& pending, const FrTensor& Y, const vector<Fr_t>& u_Y);
     Fr_t prove_end(Pending& pending, const FrTensor& X, const FrTensor& shift, const vector<FrTensor>& X_segments, const vector<FrTensor>& Y_segments,
                    const vector<Fr_t>& v_Y, vector<Polynomial>& proof);
 
