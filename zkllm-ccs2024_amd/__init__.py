@@ -26,8 +26,25 @@ def _load(path):
     return _libs[path]
 
 
+def _want_hw_queues():
+    """The library keeps up to seven streams busy (the caller's, four for openings, two for sumcheck jobs).  HIP maps
+    streams onto GPU_MAX_HW_QUEUES hardware queues (4 unless set) and streams that share a queue run one after the
+    other, so ask for at least eight.  The HIP runtime reads the variable when it is loaded: this must run before that.
+    ZKLLM_HW_QUEUES=0 leaves the variable alone, ZKLLM_HW_QUEUES=N sets it to N."""
+    want = os.environ.get("ZKLLM_HW_QUEUES", "")
+    if want == "0":
+        return
+    try:
+        cur = int(os.environ.get("GPU_MAX_HW_QUEUES", "0"))
+    except ValueError:
+        cur = 0
+    n = int(want) if want.isdigit() else max(cur, 8)
+    os.environ["GPU_MAX_HW_QUEUES"] = str(min(n, 32))
+
+
 def load_hip():
     """ctypes handle of the C-ABI kernel library."""
+    _want_hw_queues()
     lib = _load(HIP_LIB)
     lib.zk_last_error.restype = ctypes.c_char_p
     return lib
