@@ -192,7 +192,8 @@ int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, si
 /* zksoftmax_shift zksoftmax.cu:20-32 (scale = sf_in*sqrt(d)), zksoftmax_calculate_table :4-14, zksoftmax_decompose_kernel :95-109 */
 int zk_softmax_shift(void* shift, void* out_shifted, const void* X, uint32_t rows, uint32_t cols, double scale, void* stream);
 int zk_softmax_table(void* table, double log_theta, double step, uint32_t len, void* stream);
-int zk_softmax_decompose(void* planes, const void* X_shifted, const uint32_t* bs_host, int K, size_t n, void* stream);
+/* planes: K device tensors of n elements each (host array of K pointers); plane k receives digit k */
+int zk_softmax_decompose(void* const* planes, const void* X_shifted, const uint32_t* bs_host, int K, size_t n, void* stream);
 
 /* ---- measurement helpers (no counterpart in the reference) ---------------------------------------- */
 /* v_mad_u64_u32 issue peak of the device: 16 independent chains per lane, no memory traffic */

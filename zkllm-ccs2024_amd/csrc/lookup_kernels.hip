@@ -696,18 +696,19 @@ __global__ void __launch_bounds__(TPB) k_softmax_table(Fr* __restrict__ table, d
 // digits of -x in the mixed radix bs[0..K): plane k holds digit k (zksoftmax.cu:95-109).  Values whose
 // negation does not fit 64 bits raise the flag (the reference leaves their planes unwritten).
 struct U32Pack8 { uint32_t v[8]; };
-__global__ void __launch_bounds__(TPB) k_softmax_decompose(Fr* __restrict__ planes, uint32_t* __restrict__ flag, const Fr* __restrict__ X, const U32Pack8 bs, int K, size_t n) {
+struct PlanePtrs { Fr* p[8]; };
+__global__ void __launch_bounds__(TPB) k_softmax_decompose(const PlanePtrs planes, uint32_t* __restrict__ flag, const Fr* __restrict__ X, const U32Pack8 bs, int K, size_t n) {
     const size_t g = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (g >= n) return;
     const Fr mx = neg(X[g]);
     if (mx.v[2] | mx.v[3] | mx.v[4] | mx.v[5] | mx.v[6] | mx.v[7]) {
         atomicOr(flag, 1u);
-        for (int k = 0; k < K; ++k) planes[(size_t)k * n + g] = big_zero<8>();
+        for (int k = 0; k < K; ++k) planes.p[k][g] = big_zero<8>();
         return;
     }
     unsigned long long tmp = ((unsigned long long)mx.v[1] << 32) | mx.v[0];
     for (int k = 0; k < K; ++k) {
-        planes[(size_t)k * n + g] = fr_from_u64(tmp % bs.v[k]);
+        planes.p[k][g] = fr_from_u64(tmp % bs.v[k]);
         tmp /= bs.v[k];
     }
     if (tmp != 0) atomicOr(flag, 2u);   // more digits than the radices cover
@@ -1267,8 +1268,8 @@ int zk_softmax_table(void* table, double log_theta, double step, uint32_t len, v
     LAUNCH1D(k_softmax_table, len, st, (Fr*)table, log_theta, step, len);
     return 0;
 }
-// planes: K*n elements, plane k = digit k of -X in the mixed radix bs_host[0..K)
-int zk_softmax_decompose(void* planes, const void* X_shifted, const uint32_t* bs_host, int K, size_t n, void* stv) {
+// planes: K device tensors of n elements, plane k = digit k of -X in the mixed radix bs_host[0..K)
+int zk_softmax_decompose(void* const* planes, const void* X_shifted, const uint32_t* bs_host, int K, size_t n, void* stv) {
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(K >= 1 && K <= 8, "zk_softmax_decompose: K must be 1..8");
     if (n == 0) return 0;
@@ -1278,7 +1279,10 @@ int zk_softmax_decompose(void* planes, const void* X_shifted, const uint32_t* bs
     Scratch flag(4);
     if (flag.rc) return flag.rc;
     ZK_HIP(hipMemsetAsync(flag.p, 0, 4, st));
-    LAUNCH1D(k_softmax_decompose, n, st, (Fr*)planes, flag.as<uint32_t>(), (const Fr*)X_shifted, bs, K, n);
+    PlanePtrs pp;
+    for (int i = 0; i < 8; ++i) pp.p[i] = i < K ? (Fr*)planes[i] : nullptr;
+    for (int i = 0; i < K; ++i) ZK_ARG(pp.p[i] != nullptr, "zk_softmax_decompose: null plane");
+    LAUNCH1D(k_softmax_decompose, n, st, pp, flag.as<uint32_t>(), (const Fr*)X_shifted, bs, K, n);
     uint32_t f = 0;
     int rc = read_flag(flag.as<uint32_t>(), &f, st);
     if (rc) return rc;

@@ -50,22 +50,24 @@ FrTensor zkSoftmax::compute(const FrTensor& X, FrTensor& shift, FrTensor& X_shif
     ZKC(zk_softmax_shift(shift.gpu_data, X_shifted.gpu_data, X.gpu_data, m, n, scale, nullptr));
 
     const size_t N = (size_t)m * n;
-    FrTensor planes((uint)(N * K));
-    ZKC(zk_softmax_decompose(planes.gpu_data, X_shifted.gpu_data, bs.data(), (int)K, N, nullptr));
-
-    FrTensor out = FrTensor::filled((uint)N, Fr_t{{1, 0, 0, 0, 0, 0, 0, 0}});
     X_segments.reserve(K);
-    for (uint i = 0; i < L; ++i) {
-        X_segments.push_back(planes.trunc((uint)(i * N), (uint)((i + 1) * N)));
-        m_segments.push_back(least_significant_segments[i].prep(X_segments[i]));
+    std::vector<void*> planes(K);
+    for (uint i = 0; i < K; ++i) {
+        X_segments.emplace_back((uint)N);
+        planes[i] = X_segments[i].gpu_data;
     }
+    ZKC(zk_softmax_decompose(planes.data(), X_shifted.gpu_data, bs.data(), (int)K, N, nullptr));
+
+    for (uint i = 0; i < L; ++i) m_segments.push_back(least_significant_segments[i].prep(X_segments[i]));
     for (uint i = L; i < K; ++i) {
-        X_segments.push_back(planes.trunc((uint)(i * N), (uint)((i + 1) * N)));
         auto p = other_segments[i - L](X_segments[i]);
-        out *= p.first;
         Y_segments.push_back(std::move(p.first));
         m_segments.push_back(std::move(p.second));
     }
+    // the product of the segments' table values (the reference multiplies them one by one into a tensor of ones)
+    if (Y_segments.size() == 1) return FrTensor(Y_segments[0]);
+    FrTensor out = Y_segments[0] * Y_segments[1];
+    for (size_t i = 2; i < Y_segments.size(); ++i) out *= Y_segments[i];
     return out;
 }
 
