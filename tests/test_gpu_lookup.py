@@ -212,15 +212,16 @@ def test_softmax_compute_and_prove(pv, orc, m, n, d, bs, sf, lim):
     assert t.shape == e_t.shape and (t == e_t).all()
 
 
-def test_hinted_lookup_job_equals_the_plain_one_whatever_the_hints():
+@pytest.mark.parametrize("k", [13, 17])
+def test_hinted_lookup_job_equals_the_plain_one_whatever_the_hints(k):
     """zk_lookup_prove_begin_hinted reads 1/(S+beta) from the table's inverses where the hinted entry matches and must
     deliver what zk_lookup_prove_begin delivers for every input: right hints, wrong hints, hints outside the table,
-    queries that are no table entry at all, and a query with S + beta == 0."""
+    queries that are no table entry at all, and a query with S + beta == 0.  2^13 queries: the inverses are written out
+    before the first round; 2^17: the first round computes them on the fly."""
     import ctypes
     from gpuhelp import Hip, c_void_p, c_size_t, c_int
     hip = Hip()
-    D, N, low = 1 << 13, 64, -7
-    k = 13
+    D, N, low = 1 << k, 64, -7
     rng = np.random.default_rng(99)
     T = ch(41, N)                                   # arbitrary table entries
     pos = rng.integers(0, N, D)

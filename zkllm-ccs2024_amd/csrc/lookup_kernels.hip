@@ -267,35 +267,6 @@ static int batch_inv_queue(Fr* out, const Fr* in, const Fr& beta, size_t n, Aren
     return 0;
 }
 
-// A[i] = 1 / (S[i] + beta) when every S[i] is expected to be a table entry: if S[i] equals T[j] for the hinted position
-// j = hint[i] - low, the inverse is B[j] = 1 / (T[j] + beta), already computed for the table -- one gather instead of a
-// share of a batch inversion over all D queries.  Whatever the hint, the result is the inverse itself: a query that
-// does not match its hinted entry (a hint outside the table, inconsistent inputs) is inverted on its own.
-__global__ void __launch_bounds__(TPB) k_inv_by_hint(Fr* __restrict__ A, const Fr* __restrict__ S, const Fr* __restrict__ T, const Fr* __restrict__ B, const Fr* __restrict__ hint,
-                                                     const Fr low, const Fr beta, size_t D, uint32_t N) {
-    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
-    if (i >= D) return;
-    const Fr sv = S[i];
-    const Fr d = sub(hint[i], low);
-    const bool in_table = !(d.v[1] | d.v[2] | d.v[3] | d.v[4] | d.v[5] | d.v[6] | d.v[7]) && d.v[0] < N;
-    const uint32_t j = in_table ? d.v[0] : 0u;
-    if (equal(sv, T[j])) {
-        A[i] = B[j];
-        return;
-    }
-    const Fr v = add(sv, beta);
-    Fr out = big_zero<8>();
-    if (!is_zero(v)) {
-        // v is the Montgomery form of v/R: its Montgomery inverse is R^2/v, and a Montgomery product with R^-1 leaves 1/v
-        constexpr uint32_t RINV[8] = {4269129792u, 334977897u, 165441631u, 2876230287u, 1333208682u, 1912866698u, 805346647u, 465471123u};
-        Fr k;
-#pragma unroll
-        for (int l = 0; l < 8; ++l) k.v[l] = RINV[l];
-        out = mont_mul(mont_inverse(v), k);
-    }
-    A[i] = out;
-}
-
 // ---- eq tables ----------------------------------------------------------------------------------------------------------
 // E[t] = prod_j (u_j if bit_j(t) else 1-u_j), Montgomery form.  Built by doubling: level j appends bit j.
 __global__ void __launch_bounds__(TPB) k_eq_double(Fr* __restrict__ e, const Fr u_mont, const Fr one_minus_u_mont, size_t half) {
@@ -346,16 +317,44 @@ template <int K> __global__ void __launch_bounds__(TPB) k_me_multi(Fr* __restric
     block_reduce_store<K>(acc, partials);
 }
 
+// 1 / (S[i] + beta) when every S[i] is expected to be a table entry: if S[i] equals T[j] for the hinted position
+// j = hint[i] - low, the inverse is B[j] = 1 / (T[j] + beta), already computed for the table -- one gather instead of a
+// share of a batch inversion over all D queries.  Whatever the hint, the result is the inverse itself: a query that
+// does not match its hinted entry (a hint outside the table, inconsistent inputs) is inverted on its own.
+struct HintSrc { const Fr* T; const Fr* B; const Fr* hint; Fr low; Fr beta; uint32_t N; };
+static __device__ __attribute__((noinline)) Fr inv_plus_beta_alone(const Fr& sv, const Fr& beta) {
+    const Fr v = add(sv, beta);
+    if (is_zero(v)) return big_zero<8>();
+    // v is the Montgomery form of v/R: its Montgomery inverse is R^2/v, and a Montgomery product with R^-1 leaves 1/v
+    constexpr uint32_t RINV[8] = {4269129792u, 334977897u, 165441631u, 2876230287u, 1333208682u, 1912866698u, 805346647u, 465471123u};
+    Fr k;
+#pragma unroll
+    for (int l = 0; l < 8; ++l) k.v[l] = RINV[l];
+    return mont_mul(mont_inverse(v), k);
+}
+__device__ __forceinline__ Fr inv_by_hint(const Fr& sv, size_t i, const HintSrc& h) {
+    const Fr d = sub(h.hint[i], h.low);
+    const bool in_table = !(d.v[1] | d.v[2] | d.v[3] | d.v[4] | d.v[5] | d.v[6] | d.v[7]) && d.v[0] < h.N;
+    const uint32_t j = in_table ? d.v[0] : 0u;
+    if (equal(sv, h.T[j])) return h.B[j];
+    return inv_plus_beta_alone(sv, h.beta);
+}
+__global__ void __launch_bounds__(TPB) k_inv_by_hint(Fr* __restrict__ A, const Fr* __restrict__ S, const HintSrc h, size_t D) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < D) A[i] = inv_by_hint(S[i], i, h);
+}
+
 // ---- lookup sumcheck round --------------------------------------------------------------------------------------------------
 // Over halves (t, t + n_out):  a0 = A[t], da = A[t+n_out]-A[t], s0 = S[t]+beta, ds = S[t+n_out]-S[t]
 //   sums 0..2 : sum E[t] * {a0 s0, da s0 + a0 ds, da ds}          (R^-1 attached)
 //   sums 3..4 : sum a0, sum da
 // phase 2 adds the same three E-weighted sums for (B,T) as sums 5..7 and the plain products of (m,B)
 // as sums 8..10 (R^-1 attached), and folds all five tensors by v.
-template <bool PHASE2> __global__ void __launch_bounds__(TPB)
+// HINTED (first round of a job whose A was never written): a0, a1 come from inv_by_hint instead of A.
+template <bool PHASE2, bool HINTED = false> __global__ void __launch_bounds__(TPB)
 k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ nS, Fr* __restrict__ nB, Fr* __restrict__ nT, Fr* __restrict__ nm,
                const Fr* __restrict__ A, const Fr* __restrict__ S, const Fr* __restrict__ B, const Fr* __restrict__ T, const Fr* __restrict__ m,
-               const Fr* __restrict__ E, const Fr beta, const Fr v_mont, size_t n_out, Fr* __restrict__ nE) {
+               const Fr* __restrict__ E, const Fr beta, const Fr v_mont, size_t n_out, Fr* __restrict__ nE, const HintSrc hs = HintSrc()) {
     constexpr int K = PHASE2 ? 11 : 5;
     Fr acc[K];
 #pragma unroll
@@ -364,7 +363,8 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
         const Fr e = E[t];
         if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table: the top variable summed out
         {
-            const Fr a0 = A[t], a1 = A[t + n_out], s0r = S[t], s1 = S[t + n_out];
+            const Fr s0r = S[t], s1 = S[t + n_out];
+            const Fr a0 = HINTED ? inv_by_hint(s0r, t, hs) : A[t], a1 = HINTED ? inv_by_hint(s1, t + n_out, hs) : A[t + n_out];
             const Fr da = sub(a1, a0), ds = sub(s1, s0r), s0 = add(s0r, beta);
             acc[0] = add(acc[0], mont_mul(e, mont_mul(a0, s0)));
             acc[1] = add(acc[1], mont_mul(e, add(mont_mul(da, s0), mont_mul(a0, ds))));
@@ -923,8 +923,23 @@ __global__ void __launch_bounds__(TPB) k_dot_part(Fr* __restrict__ partials, con
     block_reduce_store<1>(acc, partials);
 }
 // all rounds of the lookup sumcheck; sums land in job.sums
-static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, const Fr* T, const Fr* m, const Fr* E, const Fr& b, const uint32_t* v, size_t D, size_t N, int rounds) {
+// A == nullptr with a hint source: 1 / (S + beta) has not been written anywhere; a large first round computes it on
+// the fly, anything else writes it out first.
+static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, const Fr* T, const Fr* m, const Fr* E, const Fr& b, const uint32_t* v, size_t D, size_t N, int rounds,
+                        const HintSrc* hs = nullptr) {
     hipStream_t st = job.st;
+    bool fuse_first = false;
+    if (!A) {
+        ZK_ARG(hs != nullptr, "lookup sumcheck: neither A nor a hint");
+        fuse_first = D > N && (D >> 1) > (size_t)SPLIT_HALF;       // a phase-1 round that the full-size kernel takes
+        if (!fuse_first) {
+            Scratch& Abuf = job.arena.add(sizeof(Fr) * D);
+            if (Abuf.rc) return Abuf.rc;
+            hipLaunchKernelGGL(k_inv_by_hint, dim3(cdiv(D, TPB)), dim3(TPB), 0, st, Abuf.as<Fr>(), S, *hs, D);
+            ZK_LAUNCH_CHECK();
+            A = Abuf.as<Fr>();
+        }
+    }
     int n1 = 0;
     while (((size_t)N << n1) < D) ++n1;
     job.rounds = rounds;
@@ -978,10 +993,14 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
             if (phase2) hipLaunchKernelGGL(k_lookup_round_split<true>, dim3(nb, 4), dim3(TPB), 0, st, part.as<Fr>(), lp, b, vm, half);
             else hipLaunchKernelGGL(k_lookup_round_split<false>, dim3(nb, 2), dim3(TPB), 0, st, part.as<Fr>(), lp, b, vm, half);
         } else if (phase2)
-            hipLaunchKernelGGL(k_lookup_round<true>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, w + 2 * half, w + 3 * half, w + 4 * half, cA, cS, cB, cT, cm, cE, b, vm, half, nE);
+            hipLaunchKernelGGL((k_lookup_round<true, false>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, w + 2 * half, w + 3 * half, w + 4 * half, cA, cS, cB, cT, cm, cE, b, vm, half, nE,
+                               HintSrc());
+        else if (r == 0 && fuse_first)
+            hipLaunchKernelGGL((k_lookup_round<false, true>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, (const Fr*)nullptr, cS,
+                               (const Fr*)nullptr, (const Fr*)nullptr, (const Fr*)nullptr, cE, b, vm, half, nE, *hs);
         else
-            hipLaunchKernelGGL(k_lookup_round<false>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, cA, cS, (const Fr*)nullptr,
-                               (const Fr*)nullptr, (const Fr*)nullptr, cE, b, vm, half, nE);
+            hipLaunchKernelGGL((k_lookup_round<false, false>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, cA, cS, (const Fr*)nullptr,
+                               (const Fr*)nullptr, (const Fr*)nullptr, cE, b, vm, half, nE, HintSrc());
         hipLaunchKernelGGL(k_finish, dim3(phase2 ? 11 : 5), dim3(TPB), 0, st, sums.as<Fr>() + (size_t)r * 11, part.as<Fr>(), nb);
         ZK_LAUNCH_CHECK();
         cA = w; cS = w + half;
@@ -1157,22 +1176,21 @@ static int lookup_prove_begin(void** handle, const void* S, const void* T, const
     rc = sumjob_on_side_stream(*job, (hipStream_t)stv);
     if (rc) { sumjob_abort(job); return rc; }
     hipStream_t st = job->st;
-    Scratch& A = job->arena.add(sizeof(Fr) * D);
     Scratch& B = job->arena.add(sizeof(Fr) * N);
     Scratch& E = job->arena.add(sizeof(Fr) * (D / 2));
     Scratch& dp = job->arena.add(sizeof(Fr) * (reduce_grid(N) + 1));
-    if (A.rc || B.rc || E.rc || dp.rc) { rc = A.rc ? A.rc : (B.rc ? B.rc : (E.rc ? E.rc : dp.rc)); sumjob_abort(job); return rc; }
+    if (B.rc || E.rc || dp.rc) { rc = B.rc ? B.rc : (E.rc ? E.rc : dp.rc); sumjob_abort(job); return rc; }
     const Fr b = load_fr(beta);
     rc = batch_inv_queue(B.as<Fr>(), (const Fr*)T, b, N, job->arena, st);
-    if (rc == 0) {
-        if (hint) {
-            hipLaunchKernelGGL(k_inv_by_hint, dim3(cdiv(D, TPB)), dim3(TPB), 0, st, A.as<Fr>(), (const Fr*)S, (const Fr*)T, B.as<Fr>(), (const Fr*)hint, fr_from_i64((int64_t)low), b, D,
-                               (uint32_t)N);
-            hipError_t e = hipGetLastError();
-            if (e != hipSuccess) rc = hip_fail(e, "k_inv_by_hint", __FILE__, __LINE__);
-        } else {
-            rc = batch_inv_queue(A.as<Fr>(), (const Fr*)S, b, D, job->arena, st);
-        }
+    const Fr* Aptr = nullptr;
+    HintSrc hs;
+    if (rc == 0 && hint) {
+        hs.T = (const Fr*)T; hs.B = B.as<Fr>(); hs.hint = (const Fr*)hint; hs.low = fr_from_i64((int64_t)low); hs.beta = b; hs.N = (uint32_t)N;
+    } else if (rc == 0) {
+        Scratch& A = job->arena.add(sizeof(Fr) * D);
+        rc = A.rc;
+        if (rc == 0) rc = batch_inv_queue(A.as<Fr>(), (const Fr*)S, b, D, job->arena, st);
+        Aptr = A.as<Fr>();
     }
     if (rc) { sumjob_abort(job); return rc; }
     const unsigned nb = reduce_grid(N);
@@ -1181,7 +1199,7 @@ static int lookup_prove_begin(void** handle, const void* S, const void* T, const
     job->extra = dp.as<Fr>();
     rc = eq_table_queue(E.as<Fr>(), u_eq, rounds - 1, job->arena, st);
     if (rc) { sumjob_abort(job); return rc; }
-    rc = lookup_queue(*job, A.as<Fr>(), (const Fr*)S, B.as<Fr>(), (const Fr*)T, (const Fr*)m, E.as<Fr>(), b, v, D, N, rounds);
+    rc = lookup_queue(*job, Aptr, (const Fr*)S, B.as<Fr>(), (const Fr*)T, (const Fr*)m, E.as<Fr>(), b, v, D, N, rounds, hint ? &hs : nullptr);
     if (rc == 0) rc = sumjob_queue_results(*job);
     if (rc) { sumjob_abort(job); return rc; }
     *handle = job;
