@@ -73,9 +73,12 @@ void attn_linear_block(const LayerConfig& c, const Weight& q, const Weight& k, c
     K_ = k_rescale(K);
     auto V = v_layer(input);
     V_ = v_rescale(V);
-    q_rescale.prove(Q, Q_);
-    k_rescale.prove(K, K_);
-    v_rescale.prove(V, V_);
+    auto pq = q_rescale.prove_begin(Q, Q_);      // three range proofs side by side
+    auto pk = k_rescale.prove_begin(K, K_);
+    auto pv = v_rescale.prove_begin(V, V_);
+    q_rescale.prove_end(pq);
+    k_rescale.prove_end(pk);
+    v_rescale.prove_end(pv);
     auto ck = k_layer.prove(input, K);
     if (c.open_weights) verifyWeightClaim(k, ck[0]);
     auto cq = q_layer.prove(input, Q);
@@ -176,8 +179,10 @@ FrTensor attn_heads_block(const LayerConfig& c, const FrTensor& Q_, const FrTens
     Rescaling rs1(c.sf_attn), rs2(c.sf_attn);
     auto out_ = rs2(out_all);
     auto out__ = rs1(out_);
-    rs1.prove(out_, out__);
-    rs2.prove(out_all, out_);
+    auto p1 = rs1.prove_begin(out_, out__);
+    auto p2 = rs2.prove_begin(out_all, out_);
+    rs1.prove_end(p1);
+    rs2.prove_end(p2);
     return out__;
 }
 
@@ -218,9 +223,13 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
     down_rescale.prove(down_out, down_out_);
     auto cd = down_layer.prove(down_in_, down_out);
     if (c.open_weights) verifyWeightClaim(down, cd[0]);
-    hidden_rescale.prove(down_in, down_in_);
-    swiglu.prove(gate_out_, swiglu_out, swiglu_m, temp_rand[0], temp_rand[1], temp_rand[2], swiglu_u, swiglu_v, swiglu_proof);
-    gate_rescale.prove(gate_out, gate_out_);
+    // three lookup proofs in a row with nothing between them: all begun, then collected in order
+    auto ph = hidden_rescale.prove_begin(down_in, down_in_);
+    auto ps = swiglu.prove_begin(gate_out_, swiglu_out, swiglu_m, temp_rand[0], temp_rand[1], temp_rand[2], swiglu_u, swiglu_v);
+    auto pg = gate_rescale.prove_begin(gate_out, gate_out_);
+    hidden_rescale.prove_end(ph);
+    tLookup::prove_end(ps);
+    gate_rescale.prove_end(pg);
     auto cg = gate_layer.prove(input, gate_out);
     if (c.open_weights) verifyWeightClaim(gate, cg[0]);
     up_rescale.prove(up_out, up_out_);

@@ -17,19 +17,31 @@ Rescaling::~Rescaling() { if (rem_tensor_ptr) delete rem_tensor_ptr; }
 
 // rescaling.cu:41-79.  Challenge order: u, v, (alpha, beta).
 vector<Claim> Rescaling::prove(const FrTensor& X, const FrTensor& X_) {
+    Pending p = prove_begin(X, X_);
+    prove_end(p);
+    return {};
+}
+Rescaling::Pending Rescaling::prove_begin(const FrTensor& X, const FrTensor& X_) {
     if (X.size != X_.size) throw std::runtime_error("Error: the size of X and X_ should be the same.");
     if (!rem_tensor_ptr) throw std::runtime_error("Rescaling::prove called before operator()");
     auto u = random_vec(ceilLog2(X.size));
     auto v = random_vec(ceilLog2(X.size));
     auto rand_temp = random_vec(2);
-    vector<Polynomial> proof;
 
-    auto rem = rem_tensor_ptr->pad({rem_tensor_ptr->size});
-    auto m = tl_rem.prep(rem);
-    const Fr_t lhs = X(u);
-    zk_record(lhs);
-    if (lhs != X_(u) * Fr_t({scaling_factor, 0, 0, 0, 0, 0, 0, 0}) + rem(u)) throw std::runtime_error("Error: the rem is not correct.");
-    tl_rem.prove(rem, m, rand_temp[0], rand_temp[1], u, v, proof);
+    Pending p;
+    p.rem.reset(new FrTensor(rem_tensor_ptr->pad({rem_tensor_ptr->size})));
+    p.m.reset(new FrTensor(tl_rem.prep(*p.rem)));
+    // X(u), X_(u), rem(u): one pass over the tensors that have the same length (the remainder is padded to a power of two)
+    vector<Fr_t> ev;
+    if (p.rem->size == X.size) ev = FrTensor::me_batch({&X, &X_, p.rem.get()}, u);
+    else { ev = FrTensor::me_batch({&X, &X_}, u); ev.push_back((*p.rem)(u)); }
+    p.lhs = ev[0];
+    if (p.lhs != ev[1] * Fr_t({scaling_factor, 0, 0, 0, 0, 0, 0, 0}) + ev[2]) throw std::runtime_error("Error: the rem is not correct.");
+    p.look = tl_rem.prove_begin(*p.rem, *p.m, rand_temp[0], rand_temp[1], u, v);
+    return p;
+}
+void Rescaling::prove_end(Pending& p) {
+    zk_record(p.lhs);
+    tLookup::prove_end(p.look);
     cout << "Rescaling proof complete." << endl;
-    return {};
 }

@@ -1,5 +1,6 @@
 // Fixed-point rescaling with a range-proved remainder (rescaling.cuh:11-22).
 #pragma once
+#include <memory>
 #include "fr-tensor.hpp"
 #include "proof.hpp"
 #include "tlookup.hpp"
@@ -13,6 +14,16 @@ class Rescaling {
     Rescaling(uint scaling_factor);
     FrTensor operator()(const FrTensor& X);
     vector<Claim> prove(const FrTensor& X, const FrTensor& X_);
+    // prove in two halves: begin draws the challenges, checks X = sf * X_ + rem at u and queues the range proof of the
+    // remainder on a side stream; end writes the transcript entries.  Proofs that follow each other without anything
+    // in between may all be begun before the first is ended: challenges and entries keep their order.
+    struct Pending {
+        Fr_t lhs;
+        std::unique_ptr<FrTensor> rem, m;
+        LookupPending look;
+    };
+    Pending prove_begin(const FrTensor& X, const FrTensor& X_);
+    void prove_end(Pending& p);
     ~Rescaling();
     Rescaling(const Rescaling&) = delete;
     Rescaling& operator=(const Rescaling&) = delete;
