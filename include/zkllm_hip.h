@@ -184,6 +184,10 @@ int zk_lookup_prove_begin(void** handle, const void* S, const void* T, const voi
 int zk_lookup_prove_begin_hinted(void** handle, const void* S, const void* T, const void* m, const void* hint_fr, int32_t low, const uint32_t* beta, const uint32_t* u_eq,
                                  const uint32_t* v, size_t D, size_t N, int rounds, void* stream);
 int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host);
+/* hadamard_product_sumcheck (Fr_hp_sc, proof.cu:66-109): adjacent-pair folding, first challenge first.  a, b: n elements,
+ * 2^(k-1) < n <= 2^k; u, v: k challenges each.  proof_host: 3k + 2 values (per round the three terms evaluated at the
+ * remaining u, then the folded a and b).  The three term tensors of the reference's step kernel are never materialised. */
+int zk_hadamard_product_sumcheck(uint32_t* proof_host, const void* a, const void* b, const uint32_t* u, const uint32_t* v, size_t n, int k, void* stream);
 int zk_hadamard_prove_begin(void** handle, const void* const* Xs, int K, const uint32_t* u_eq, const uint32_t* v, size_t N, void* stream);
 int zk_hadamard_prove_end(void* handle, uint32_t* coefs_host);
 

@@ -159,7 +159,8 @@ def test_multi_hadamard(pv, orc, nX, n):
     assert (proof == e_proof).all() and (fin == e_fin).all()
 
 
-@pytest.mark.parametrize("n", [2, 5, 64, 1000])
+# 70001: several workgroups per round and odd lengths on the way down (70001, 35001, 17501, 8751, 4376, ...)
+@pytest.mark.parametrize("n", [2, 3, 5, 64, 1000, 70001])
 def test_deprecated_hadamard_product_sumcheck(pv, orc, n):
     a, b = ch(40, n), ch(41, n)
     k = (n - 1).bit_length()

@@ -391,6 +391,33 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
     block_reduce_store<K>(acc, partials);
 }
 
+// ---- Hadamard-product sumcheck with adjacent-pair folding (Fr_hp_sc, proof.cu:66-98) -------------------------------------
+// One round over pairs (2g, 2g+1), zero beyond in_size: the three term tensors of the reference's step kernel
+//   o0 = a0 b0,  o1 = a0 db + b0 da,  o2 = da db      (each product carries R^-1: the reference multiplies standard-form
+//                                                      values with the Montgomery routine and does not convert back)
+// are never written: their multilinear evaluations at the remaining challenges, sum_g eq[g] o_k[g], are accumulated
+// directly (E in Montgomery form, so E * o is a plain product), a and b are folded by v, and the eq table of the next
+// round (this round's lowest variable summed out) is written on the way.
+__global__ void __launch_bounds__(TPB) k_hp_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ nB, Fr* __restrict__ nE, const Fr* __restrict__ A,
+                                                  const Fr* __restrict__ B, const Fr* __restrict__ E, const Fr v_mont, size_t in_size, size_t out_size, size_t ne_count) {
+    Fr acc[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) acc[i] = big_zero<8>();
+    for (size_t g = (size_t)blockIdx.x * TPB + threadIdx.x; g < out_size; g += (size_t)gridDim.x * TPB) {
+        const Fr a0 = A[2 * g], b0 = B[2 * g];
+        const Fr a1 = (2 * g + 1 < in_size) ? A[2 * g + 1] : big_zero<8>(), b1 = (2 * g + 1 < in_size) ? B[2 * g + 1] : big_zero<8>();
+        const Fr da = sub(a1, a0), db = sub(b1, b0);
+        const Fr e = E[g];
+        acc[0] = add(acc[0], mont_mul(e, mont_mul(a0, b0)));
+        acc[1] = add(acc[1], mont_mul(e, add(mont_mul(a0, db), mont_mul(b0, da))));
+        acc[2] = add(acc[2], mont_mul(e, mont_mul(da, db)));
+        nA[g] = add(a0, mont_mul(v_mont, da));
+        nB[g] = add(b0, mont_mul(v_mont, db));
+        if (g < ne_count) nE[g] = add(E[2 * g], E[2 * g + 1]);
+    }
+    block_reduce_store<3>(acc, partials);
+}
+
 // ---- multi-Hadamard sumcheck round (proof.cu:191-241) --------------------------------------------------------------------------
 // K tensors; coefficient j of prod_k (X0_k + t dX_k), weighted by E and summed (R^-K attached... see host);
 // also folds every tensor by v.
@@ -1269,6 +1296,48 @@ int zk_hadamard_prove_end(void* handle, uint32_t* coefs_host) {
     int rc = sumjob_collect(*job, (Fr*)coefs_host, nullptr);
     sumjob_abort(job);
     return rc;
+}
+// hadamard_product_sumcheck (proof.cu:66-109): k rounds over a, b of n elements (2^(k-1) < n <= 2^k), evaluation
+// challenges u and fold challenges v, both in the order the reference consumes them (first challenge first).
+// proof_host: 3k + 2 values -- per round the three evaluated terms, then the fully folded a and b.  Neither input is modified.
+int zk_hadamard_product_sumcheck(uint32_t* proof_host, const void* a, const void* b, const uint32_t* u, const uint32_t* v, size_t n, int k, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(k >= 1 && k <= 30 && n <= ((size_t)1 << k) && n > ((size_t)1 << (k - 1)), "zk_hadamard_product_sumcheck: n does not match the number of challenges");
+    ZK_ARG(sizeof(Fr) * (3 * (size_t)k + 2) <= 65536, "zk_hadamard_product_sumcheck: too many rounds for the staging buffer");
+    Arena arena;
+    const size_t half = (n + 1) / 2, etab = (size_t)1 << (k - 1);
+    Scratch& E = arena.add(sizeof(Fr) * (etab + etab / 2 + 1));          // eq tables, ping-pong
+    Scratch& W = arena.add(sizeof(Fr) * 2 * (half + (half + 1) / 2 + 1));   // folded a, b, ping-pong
+    Scratch& part = arena.add(sizeof(Fr) * 3 * reduce_grid(half));
+    Scratch& sums = arena.add(sizeof(Fr) * (3 * (size_t)k + 2));
+    if (E.rc || W.rc || part.rc || sums.rc) return E.rc ? E.rc : (W.rc ? W.rc : (part.rc ? part.rc : sums.rc));
+    int rc = eq_table_queue(E.as<Fr>(), u + 8, k - 1, arena, st);
+    if (rc) { (void)hipStreamSynchronize(st); return rc; }
+    Fr* ebuf[2] = {E.as<Fr>(), E.as<Fr>() + etab};
+    Fr* wa[2] = {W.as<Fr>(), W.as<Fr>() + half};
+    Fr* wb[2] = {wa[1] + (half + 1) / 2 + 1, nullptr};
+    wb[1] = wb[0] + half;
+    const Fr *ca = (const Fr*)a, *cb = (const Fr*)b, *ce = ebuf[0];
+    size_t cur = n, ecur = etab;
+    for (int r = 0; r < k; ++r) {
+        const size_t out = (cur + 1) / 2;
+        const unsigned nb = reduce_grid(out);
+        hipLaunchKernelGGL(k_hp_round, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), wa[r & 1], wb[r & 1], ebuf[(r + 1) & 1], ca, cb, ce, to_mont(load_fr(v + 8 * r)), cur, out, ecur / 2);
+        hipLaunchKernelGGL(k_finish, dim3(3), dim3(TPB), 0, st, sums.as<Fr>() + 3 * (size_t)r, part.as<Fr>(), nb);
+        ZK_LAUNCH_CHECK();
+        ca = wa[r & 1]; cb = wb[r & 1]; ce = ebuf[(r + 1) & 1];
+        cur = out;
+        ecur /= 2;
+    }
+    ZK_HIP(hipMemcpyAsync(sums.as<Fr>() + 3 * (size_t)k, ca, sizeof(Fr), hipMemcpyDeviceToDevice, st));
+    ZK_HIP(hipMemcpyAsync(sums.as<Fr>() + 3 * (size_t)k + 1, cb, sizeof(Fr), hipMemcpyDeviceToDevice, st));
+    void* stage = nullptr;
+    rc = staging(&stage, sizeof(Fr) * (3 * (size_t)k + 2));
+    if (rc) { (void)hipStreamSynchronize(st); return rc; }
+    ZK_HIP(hipMemcpyAsync(stage, sums.p, sizeof(Fr) * (3 * (size_t)k + 2), hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipStreamSynchronize(st));
+    memcpy(proof_host, stage, sizeof(Fr) * (3 * (size_t)k + 2));
+    return 0;
 }
 int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* st) {
     ZK_ARG(scaling_factor >= 1, "zk_rescale: scaling factor is 0");

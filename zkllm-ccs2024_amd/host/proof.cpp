@@ -165,30 +165,15 @@ vector<Fr_t> inner_product_sumcheck(const FrTensor& a0, const FrTensor& b0, vect
     return proof;
 }
 
+// proof.cu:66-109: every round of the device side in one queue of launches (the challenges are all known), one copy back
 vector<Fr_t> hadamard_product_sumcheck(const FrTensor& a0, const FrTensor& b0, vector<Fr_t> u, vector<Fr_t> v) {
-    vector<Fr_t> proof;
     if (u.size() != v.size()) throw std::runtime_error("Incompatible dimensions 1");
     uint log_size = (uint)u.size();
     if (a0.size != b0.size) throw std::runtime_error("Incompatible dimensions 2");
     if (log_size == 0 || a0.size <= (1u << (log_size - 1))) throw std::runtime_error("Incompatible dimensions 3");
     if (a0.size > (1u << log_size)) throw std::runtime_error("Incompatible dimensions 4");
-    std::vector<FrTensor> ka, kb;
-    const FrTensor *pa = &a0, *pb = &b0;
-    ka.reserve(u.size()); kb.reserve(u.size());
-    for (size_t i = 0; i < u.size(); ++i) {
-        uint out_size = (pa->size + 1) / 2;
-        FrTensor o0(out_size), o1(out_size), o2(out_size);
-        ip_sc_terms(*pa, *pb, o0, o1, o2);
-        vector<Fr_t> u_(u.begin() + i + 1, u.end());
-        proof.push_back(o0(u_));
-        proof.push_back(o1(u_));
-        proof.push_back(o2(u_));
-        ka.push_back(fold_first(*pa, v[i]));
-        kb.push_back(fold_first(*pb, v[i]));
-        pa = &ka.back(); pb = &kb.back();
-    }
-    proof.push_back((*pa)(0u));
-    proof.push_back((*pb)(0u));
+    vector<Fr_t> proof(3 * (size_t)log_size + 2);
+    ZKC(zk_hadamard_product_sumcheck(proof[0].val, a0.gpu_data, b0.gpu_data, u[0].val, v[0].val, a0.size, (int)log_size, nullptr));
     zk_record(proof);
     return proof;
 }
