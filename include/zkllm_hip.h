@@ -70,6 +70,9 @@ int zk_fr_from_f32(void* out, const void* in_f32, uint64_t scaling_factor, size_
 int zk_fr_from_f64(void* out, const void* in_f64, uint64_t scaling_factor, size_t n, void* stream);
 int zk_fr_to_i32(void* out_i32, const void* in, size_t n, void* stream);
 int zk_fr_to_i64(void* out_i64, const void* in, size_t n, void* stream);
+/* out_f64[r] = sum_j (X[r][j] / scale)^2 in double precision, terms added in index order (the mean square that
+ * llama-rmsnorm.py:38-39 computes with torch before calling the prover).  out_f64: rows doubles on the device. */
+int zk_row_sumsq_f64(void* out_f64, const void* X, uint32_t rows, uint32_t cols, double scale, void* stream);
 
 /* ---- layout (pad fr-tensor.cu:800-828, transpose :885-900, gather tlookup.cu:446-453) ----------- */
 int zk_fr_pad(void* out, const void* in, size_t rows, uint32_t last_in, uint32_t last_out, const uint32_t* pad, void* stream);

@@ -281,3 +281,29 @@ def test_zkfc_forward_and_proof_transcript(pv, orc, B, I, O, mode):
     assert (got_Y == exp_Y).all()
     assert got_t.shape == exp_t.shape and (got_t == exp_t).all()
     pv.lib.zkp_set_matmul_mode(ctypes.c_int(0))
+
+
+def test_row_sums_of_squares_in_double_follow_a_plain_loop():
+    """zk_row_sumsq_f64 must round exactly as `for j: acc += (x[j] / scale) ** 2` does: Python floats are IEEE doubles and
+    every operation involved is exactly rounded, so the device result is compared bit for bit."""
+    from gpuhelp import Hip, c_void_p
+    hip = Hip()
+    rng = np.random.default_rng(77)
+    rows, cols, scale = 7, 333, 65536.0
+    x = rng.integers(-(1 << 22), 1 << 22, (rows, cols))
+    x[0, :3] = [0, -1, (1 << 40) + 12345]
+    X = fr_array([int(v) % R_MOD for v in x.reshape(-1)])
+    dX = hip.upload(X)
+    dout = hip.malloc(8 * rows)
+    hip.call("zk_row_sumsq_f64", c_void_p(dout), c_void_p(dX), ctypes.c_uint32(rows), ctypes.c_uint32(cols), ctypes.c_double(scale), None)
+    got = hip.download(dout, (rows,), np.float64)
+    exp = np.zeros(rows, np.float64)
+    for r in range(rows):
+        acc = 0.0
+        for j in range(cols):
+            t = float(int(x[r, j])) / scale
+            acc += t * t
+        exp[r] = acc
+    assert (got.view(np.uint64) == exp.view(np.uint64)).all()
+    hip.free(dX)
+    hip.free(dout)

@@ -401,6 +401,32 @@ static inline Fr load_fr(const uint32_t* p) { Fr r; memcpy(&r, p, 32); return r;
         }                                                                                    \
     } while (0)
 
+// out[r] = sum_j (x_rj / scale)^2 in double precision, the terms added one after the other from j = 0 (the order a plain
+// host loop uses, so the rounding is the same).  One wave per row: the lanes form 64 terms at a time -- conversion,
+// division and square are exactly rounded operations -- and lane 0 adds them in order.
+__global__ void __launch_bounds__(64) k_row_sumsq_f64(double* __restrict__ out, const Fr* __restrict__ X, uint32_t cols, double scale) {
+    __shared__ double term[64];
+    const uint32_t r = blockIdx.x, t = threadIdx.x;
+    const Fr* row = X + (size_t)r * cols;
+    double acc = 0.0;
+    for (uint32_t j0 = 0; j0 < cols; j0 += 64) {
+        const uint32_t j = j0 + t;
+        double v = 0.0;
+        if (j < cols) {
+            const double x = (double)fr_to_i64(row[j]) / scale;
+            v = x * x;
+        }
+        term[t] = v;
+        __syncthreads();
+        if (t == 0) {
+            const uint32_t cnt = cols - j0 < 64u ? cols - j0 : 64u;
+            for (uint32_t q = 0; q < cnt; ++q) acc += term[q];
+        }
+        __syncthreads();
+    }
+    if (t == 0) out[r] = acc;
+}
+
 extern "C" {
 
 int zk_fr_add(void* out, const void* a, const void* b, size_t n, void* st) { LAUNCH1D(k_ew<EW_ADD>, n, st, (Fr*)out, (const Fr*)a, (const Fr*)b, n); return 0; }
@@ -435,6 +461,16 @@ int zk_fr_from_u32(void* out, const void* in, size_t n, void* st) { LAUNCH1D(k_f
 int zk_fr_from_f32(void* out, const void* in, uint64_t sf, size_t n, void* st) { LAUNCH1D(k_from_f32, n, st, (Fr*)out, (const float*)in, sf, n); return 0; }
 int zk_fr_from_f64(void* out, const void* in, uint64_t sf, size_t n, void* st) { LAUNCH1D(k_from_f64, n, st, (Fr*)out, (const double*)in, sf, n); return 0; }
 int zk_fr_to_i32(void* out, const void* in, size_t n, void* st) { LAUNCH1D(k_to_i32, n, st, (int32_t*)out, (const Fr*)in, n); return 0; }
+// sums of squares of the rows of a rows x cols tensor of small signed integers, each divided by `scale` first, in double
+// precision with the terms added in index order (the mean square of RMSNorm as a host loop would compute it;
+// llama-rmsnorm.py:38-39 computes it with torch before the prover runs).  out_f64: rows doubles on the device.
+int zk_row_sumsq_f64(void* out_f64, const void* X, uint32_t rows, uint32_t cols, double scale, void* st) {
+    if (rows == 0) return 0;
+    ZK_ARG(cols >= 1 && scale != 0.0, "zk_row_sumsq_f64: empty rows or zero scale");
+    hipLaunchKernelGGL(k_row_sumsq_f64, dim3(rows), dim3(64), 0, (hipStream_t)st, (double*)out_f64, (const Fr*)X, cols, scale);
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
 int zk_fr_to_i64(void* out, const void* in, size_t n, void* st) { LAUNCH1D(k_to_i64, n, st, (int64_t*)out, (const Fr*)in, n); return 0; }
 
 int zk_fr_pad(void* out, const void* in, size_t rows, uint32_t last_in, uint32_t last_out, const uint32_t* pad, void* st) {

@@ -15,20 +15,16 @@ static double now_ms() {
 
 FrTensor compute_rms_inv(const FrTensor& X, uint seq_len, uint embed_dim, double eps, double value_scale) {
     if (X.size != seq_len * embed_dim) throw std::runtime_error("compute_rms_inv: X size does not match");
-    std::vector<long> xi((size_t)X.size);
+    // the sums of squares on the device, in the order and precision of a plain loop over each row; the rest on the host
+    std::vector<double> sq(seq_len);
     {
-        DevBuf tmp(sizeof(long) * (size_t)X.size);
-        ZKC(zk_fr_to_i64(tmp.p, X.gpu_data, X.size, nullptr));
-        ZKC(zk_memcpy_d2h(xi.data(), tmp.p, sizeof(long) * (size_t)X.size, nullptr));
+        DevBuf tmp(sizeof(double) * (size_t)seq_len);
+        ZKC(zk_row_sumsq_f64(tmp.p, X.gpu_data, seq_len, embed_dim, value_scale, nullptr));
+        ZKC(zk_memcpy_d2h(sq.data(), tmp.p, sizeof(double) * (size_t)seq_len, nullptr));
     }
     std::vector<long> out(seq_len);
     for (uint r = 0; r < seq_len; ++r) {
-        double acc = 0.0;
-        for (uint j = 0; j < embed_dim; ++j) {
-            const double x = (double)xi[(size_t)r * embed_dim + j] / value_scale;
-            acc += x * x;
-        }
-        const double v = 1.0 / std::sqrt(acc / (double)embed_dim + eps);
+        const double v = 1.0 / std::sqrt(sq[r] / (double)embed_dim + eps);
         out[r] = (long)std::nearbyint(v * value_scale);
     }
     return FrTensor(seq_len, out.data());
