@@ -38,6 +38,9 @@ def main():
     ap.add_argument("--seq", type=int, default=2048)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extras", action="store_true", help="only the layer timing (used for profiling runs)")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="for rocprofv3 --pmc runs: only three launches of the opening's fold kernel at 176128 pairs and one "
+                         "zk_fr_add over 2^24 elements (1 GiB read, 512 MiB written) to scale the counters by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this prover runs on one GPU; every configuration of the benchmark fits a single MI355X, "
@@ -51,6 +54,26 @@ def main():
     pv = Prover()
     hip = Hip()
     lib = hip.lib
+
+    if args.pmc_probe:
+        n_big = 11008 << 5
+        pv.seed(6)
+        gens_big = pv.commitment_random(n_big)
+        pv.lib.zkp_g1_devptr.restype = ctypes.c_void_p
+        gp = pv.lib.zkp_g1_devptr(c_void_p(gens_big.h))
+        sc = hip.upload(mt_random_vec(np.random.RandomState(8), n_big))
+        ns, ng = hip.malloc(32 * (n_big // 2)), hip.malloc(144 * (n_big // 2))
+        u1 = mt_random_vec(np.random.RandomState(9), 1)
+        sums3 = np.zeros((3, 36), np.uint32)
+        for _ in range(3):
+            hip.call("zk_g1_open_round", c_void_p(ns), c_void_p(ng), sums3, c_void_p(sc), c_void_p(gp), u1, c_size_t(n_big), None)
+        n = 1 << 24
+        dA, dB, dO = hip.malloc(32 * n), hip.malloc(32 * n), hip.malloc(32 * n)
+        hip.call("zk_fr_add", c_void_p(dO), c_void_p(dA), c_void_p(dB), c_size_t(n), None)
+        hip.sync()
+        print(json.dumps({"pmc_probe": {"fold_pairs_per_launch": n_big // 2, "fold_launches": 3, "copy_kernel": "k_ew<0> (zk_fr_add)",
+                                        "copy_read_bytes": 64 * n, "copy_write_bytes": 32 * n}}))
+        return
 
     def ev():
         e = c_void_p()

@@ -231,6 +231,14 @@ ZK_HD Fp fq29_to_fp(const Fq29& a) {
 }
 
 // ---- points -----------------------------------------------------------------------------------------------------------
+// The point formulas are inlined into the kernels' loops on the device (the field products inside them stay calls with
+// their operands in registers): as functions of their own they take and return points through private memory, and that
+// traffic -- half a kilobyte per lane and point operation -- cost more than the arithmetic.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define FQ29_POINT_FN ZK_HD
+#else
+#define FQ29_POINT_FN static ZK_NOINLINE_HD
+#endif
 struct A29 { Fq29 x, y; };                 // affine; all-zero limbs = infinity (as the normalised 32-bit tables mark it)
 struct J29 { Fq29 x, y, z; uint32_t inf; };
 ZK_HD bool a29_is_inf(const A29& p) {
@@ -252,7 +260,7 @@ ZK_HD G1Jac j29_to_jac(const J29& p) {
     r.x = fq29_to_fp(p.x); r.y = fq29_to_fp(p.y); r.z = fq29_to_fp(p.z);
     return r;
 }
-static ZK_NOINLINE_HD J29 j29_double(const J29& p) {
+FQ29_POINT_FN J29 j29_double(const J29& p) {
     if (p.inf) return p;
     const Fq29 a = fq29_sqr(p.x);
     const Fq29 b = fq29_sqr(p.y);
@@ -269,7 +277,7 @@ static ZK_NOINLINE_HD J29 j29_double(const J29& p) {
     r.y = fq29_sub(fq29_mul(fq29_sub(d, r.x), e), c);
     return r;
 }
-static ZK_NOINLINE_HD J29 j29_add_mixed(const J29& a, const A29& b) {
+FQ29_POINT_FN J29 j29_add_mixed(const J29& a, const A29& b) {
     if (a.inf) { J29 r; r.x = b.x; r.y = b.y; r.z = fq29_one(); r.inf = 0u; return r; }
     const Fq29 z1z1 = fq29_sqr(a.z);
     const Fq29 u2 = fq29_mul(b.x, z1z1);
