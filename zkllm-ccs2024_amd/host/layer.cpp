@@ -199,6 +199,27 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
     Rescaling up_rescale(c.sf_linear), gate_rescale(c.sf_gate), hidden_rescale(c.sf_linear), down_rescale(c.sf_linear);
     tLookupRangeMapping swiglu(c.swiglu_low, c.swiglu_len, swiglu_values);
 
+    // Every challenge of this block, drawn first and in the order ffn.cu draws them (:67-69 the three of the activation
+    // lookup, then inside the proofs of :83-93): the forward pass draws none.  The three weight openings need nothing but
+    // their points, so they start here and run beside the forward pass and the whole proof instead of behind them.
+    const uint seq = input.size / c.embed_dim;
+    auto temp_rand = random_vec(3);
+    auto swiglu_u = random_vec(ceilLog2(c.seq_len * c.hidden_dim));
+    auto swiglu_v = random_vec(ceilLog2(c.seq_len * c.hidden_dim));
+    const auto ch_dr = Rescaling::draw(seq * c.embed_dim);       // down_out
+    const auto ch_d = down_layer.draw(seq);
+    const auto ch_hr = Rescaling::draw(seq * c.hidden_dim);      // down_in
+    const auto ch_gr = Rescaling::draw(seq * c.hidden_dim);      // gate_out
+    const auto ch_g = gate_layer.draw(seq);
+    const auto ch_ur = Rescaling::draw(seq * c.hidden_dim);      // up_out
+    const auto ch_u = up_layer.draw(seq);
+    WeightOpeningAhead od, og, ou;
+    if (c.open_weights) {
+        ou = openWeightAhead(up, ch_u.u_input, ch_u.u_output);      // the two large ones first
+        og = openWeightAhead(gate, ch_g.u_input, ch_g.u_output);
+        od = openWeightAhead(down, ch_d.u_input, ch_d.u_output);
+    }
+
     auto up_out = up_layer(input);
     auto up_out_ = up_rescale(up_out);
     auto gate_out = gate_layer(input);
@@ -206,31 +227,32 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
     auto p = swiglu(gate_out_);
     auto &swiglu_out = p.first, &swiglu_m = p.second;
 
-    auto temp_rand = random_vec(3);
-    auto swiglu_u = random_vec(ceilLog2(c.seq_len * c.hidden_dim));
-    auto swiglu_v = random_vec(ceilLog2(c.seq_len * c.hidden_dim));
-    vector<Polynomial> swiglu_proof;
-
     auto down_in = swiglu_out * up_out_;
     auto down_in_ = hidden_rescale(down_in);
     auto down_out = down_layer(down_in_);
     auto down_out_ = down_rescale(down_out);
 
-    down_rescale.prove(down_out, down_out_);
-    auto cd = down_layer.prove(down_in_, down_out);
-    if (c.open_weights) verifyWeightClaim(down, cd[0]);
+    {
+        auto pd = down_rescale.prove_begin(down_out, down_out_, ch_dr);
+        down_rescale.prove_end(pd);
+    }
+    auto cd = down_layer.prove(down_in_, down_out, ch_d);
+    if (c.open_weights) verifyWeightClaim(down, cd[0], od);
     // three lookup proofs in a row with nothing between them: all begun, then collected in order
-    auto ph = hidden_rescale.prove_begin(down_in, down_in_);
+    auto ph = hidden_rescale.prove_begin(down_in, down_in_, ch_hr);
     auto ps = swiglu.prove_begin(gate_out_, swiglu_out, swiglu_m, temp_rand[0], temp_rand[1], temp_rand[2], swiglu_u, swiglu_v);
-    auto pg = gate_rescale.prove_begin(gate_out, gate_out_);
+    auto pg = gate_rescale.prove_begin(gate_out, gate_out_, ch_gr);
     hidden_rescale.prove_end(ph);
     tLookup::prove_end(ps);
     gate_rescale.prove_end(pg);
-    auto cg = gate_layer.prove(input, gate_out);
-    if (c.open_weights) verifyWeightClaim(gate, cg[0]);
-    up_rescale.prove(up_out, up_out_);
-    auto cu = up_layer.prove(input, up_out);
-    if (c.open_weights) verifyWeightClaim(up, cu[0]);
+    auto cg = gate_layer.prove(input, gate_out, ch_g);
+    if (c.open_weights) verifyWeightClaim(gate, cg[0], og);
+    {
+        auto pu = up_rescale.prove_begin(up_out, up_out_, ch_ur);
+        up_rescale.prove_end(pu);
+    }
+    auto cu = up_layer.prove(input, up_out, ch_u);
+    if (c.open_weights) verifyWeightClaim(up, cu[0], ou);
     // the reference saves the unrescaled down_out (ffn.cu:81); the rescaled tensor is what the next block consumes
     return down_out_;
 }

@@ -53,6 +53,36 @@ void verifyWeightClaim(const Weight& w, const Claim& c) {
     cout << "Opening complete" << endl;
 }
 
+struct WeightOpeningAhead::Impl {
+    Commitment::Pending op;
+    vector<Fr_t> u_cat;
+};
+WeightOpeningAhead::WeightOpeningAhead() : impl(nullptr) {}
+WeightOpeningAhead::WeightOpeningAhead(WeightOpeningAhead&& o) noexcept : impl(o.impl) { o.impl = nullptr; }
+WeightOpeningAhead& WeightOpeningAhead::operator=(WeightOpeningAhead&& o) noexcept { std::swap(impl, o.impl); return *this; }
+WeightOpeningAhead::~WeightOpeningAhead() {
+    if (!impl) return;
+    try { vector<G1Jacobian_t> drop; Commitment::open_end(impl->op, drop); } catch (...) {}      // started and never handed over: wait and release
+    delete impl;
+}
+WeightOpeningAhead openWeightAhead(const Weight& w, const vector<Fr_t>& u_input, const vector<Fr_t>& u_output) {
+    WeightOpeningAhead a;
+    if (!g_deferred) return a;            // nothing runs ahead outside a deferred scope
+    a.impl = new WeightOpeningAhead::Impl;
+    a.impl->u_cat = concatenate(vector<vector<Fr_t>>({u_output, u_input}));
+    auto w_padded = w.weight.pad({w.in_dim, w.out_dim});
+    a.impl->op = w.generator.open_begin(w_padded, w.com, a.impl->u_cat);
+    return a;
+}
+void verifyWeightClaim(const Weight& w, const Claim& c, WeightOpeningAhead& ahead) {
+    if (!ahead.impl || !g_deferred) { verifyWeightClaim(w, c); return; }
+    if (ahead.impl->u_cat != concatenate(vector<vector<Fr_t>>({c.u[1], c.u[0]}))) throw std::runtime_error("verifyWeightClaim: the opening started ahead is at another point");
+    DeferredOpenings::Item* it = new DeferredOpenings::Item{std::move(ahead.impl->op), c.claim, zk_record_reserve()};
+    g_deferred->items.push_back(it);
+    delete ahead.impl;
+    ahead.impl = nullptr;
+}
+
 static const Fr_t kZero{{0, 0, 0, 0, 0, 0, 0, 0}};
 static const Fr_t kOne{{1, 0, 0, 0, 0, 0, 0, 0}};
 

@@ -13,6 +13,21 @@ struct Claim {
 
 struct Weight;
 void verifyWeightClaim(const Weight& w, const Claim& c);
+// The opening of a weight depends on the weight, its commitment and the point -- challenges that the prover draws, not on
+// anything it computes.  A caller that has drawn the challenges of a fully connected layer's proof ahead of time (in the
+// order the proof would draw them) may start the opening there and hand it to verifyWeightClaim when the proof reaches
+// that point: the opened value keeps its place in the transcript, the device work starts earlier.  Only inside a
+// DeferredOpenings scope; u_input / u_output are the layer's challenges of those names (Claim::u of its weight claim).
+struct WeightOpeningAhead {
+    WeightOpeningAhead();
+    ~WeightOpeningAhead();
+    WeightOpeningAhead(WeightOpeningAhead&&) noexcept;
+    WeightOpeningAhead& operator=(WeightOpeningAhead&&) noexcept;
+    struct Impl;
+    Impl* impl;
+};
+WeightOpeningAhead openWeightAhead(const Weight& w, const std::vector<Fr_t>& u_input, const std::vector<Fr_t>& u_output);
+void verifyWeightClaim(const Weight& w, const Claim& c, WeightOpeningAhead& ahead);
 // While a DeferredOpenings object is alive, verifyWeightClaim only starts each opening (it runs on the device beside
 // the rest of the proof) and finish() waits for all of them, checks every claim and throws as verifyWeightClaim does.
 // The transcript keeps the position of each opened value.
@@ -29,6 +44,7 @@ class DeferredOpenings {
     std::vector<Item*> items;
     DeferredOpenings* prev;
     friend void verifyWeightClaim(const Weight& w, const Claim& c);
+    friend void verifyWeightClaim(const Weight& w, const Claim& c, WeightOpeningAhead& ahead);
 };
 
 vector<Fr_t> inner_product_sumcheck(const FrTensor& a, const FrTensor& b, vector<Fr_t> u);

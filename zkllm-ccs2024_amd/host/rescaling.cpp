@@ -21,12 +21,23 @@ vector<Claim> Rescaling::prove(const FrTensor& X, const FrTensor& X_) {
     prove_end(p);
     return {};
 }
+Rescaling::Challenges Rescaling::draw(uint size) {
+    Challenges ch;
+    ch.u = random_vec(ceilLog2(size));
+    ch.v = random_vec(ceilLog2(size));
+    ch.rand_temp = random_vec(2);
+    return ch;
+}
 Rescaling::Pending Rescaling::prove_begin(const FrTensor& X, const FrTensor& X_) {
     if (X.size != X_.size) throw std::runtime_error("Error: the size of X and X_ should be the same.");
     if (!rem_tensor_ptr) throw std::runtime_error("Rescaling::prove called before operator()");
-    auto u = random_vec(ceilLog2(X.size));
-    auto v = random_vec(ceilLog2(X.size));
-    auto rand_temp = random_vec(2);
+    return prove_begin(X, X_, draw(X.size));
+}
+Rescaling::Pending Rescaling::prove_begin(const FrTensor& X, const FrTensor& X_, const Challenges& ch) {
+    if (X.size != X_.size) throw std::runtime_error("Error: the size of X and X_ should be the same.");
+    if (!rem_tensor_ptr) throw std::runtime_error("Rescaling::prove called before operator()");
+    const vector<Fr_t>&u = ch.u, &v = ch.v, &rand_temp = ch.rand_temp;
+    if (u.size() != ceilLog2(X.size) || v.size() != u.size() || rand_temp.size() != 2) throw std::runtime_error("Rescaling::prove: challenges do not match the shape");
 
     Pending p;
     p.rem.reset(new FrTensor(rem_tensor_ptr->pad({rem_tensor_ptr->size})));

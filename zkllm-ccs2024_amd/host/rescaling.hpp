@@ -23,6 +23,10 @@ class Rescaling {
         LookupPending look;
     };
     Pending prove_begin(const FrTensor& X, const FrTensor& X_);
+    // challenges drawn apart from the proof (same order: u, v, then the lookup's two)
+    struct Challenges { vector<Fr_t> u, v, rand_temp; };
+    static Challenges draw(uint size);
+    Pending prove_begin(const FrTensor& X, const FrTensor& X_, const Challenges& ch);
     void prove_end(Pending& p);
     ~Rescaling();
     Rescaling(const Rescaling&) = delete;

@@ -37,12 +37,23 @@ FrTensor zkFC::operator()(const FrTensor& X) const {
 }
 
 // zkfc.cu:61-87.  Challenge order: u_batch, u_input, u_output.
+zkFC::Challenges zkFC::draw(uint batchSize) const {
+    Challenges ch;
+    ch.u_batch = random_vec(ceilLog2(batchSize));
+    ch.u_input = random_vec(ceilLog2(inputSize));
+    ch.u_output = random_vec(ceilLog2(outputSize));
+    return ch;
+}
 vector<Claim> zkFC::prove(const FrTensor& X, const FrTensor& Y) const {
     if (has_bias) throw std::runtime_error("Cleaned-up version not implemented for zkFC with bias. Use zkFCStacked instead.");
+    return prove(X, Y, draw(X.size / inputSize));
+}
+vector<Claim> zkFC::prove(const FrTensor& X, const FrTensor& Y, const Challenges& ch) const {
+    if (has_bias) throw std::runtime_error("Cleaned-up version not implemented for zkFC with bias. Use zkFCStacked instead.");
     uint batchSize = X.size / inputSize;
-    auto u_batch = random_vec(ceilLog2(batchSize));
-    auto u_input = random_vec(ceilLog2(inputSize));
-    auto u_output = random_vec(ceilLog2(outputSize));
+    const vector<Fr_t>&u_batch = ch.u_batch, &u_input = ch.u_input, &u_output = ch.u_output;
+    if (u_batch.size() != ceilLog2(batchSize) || u_input.size() != ceilLog2(inputSize) || u_output.size() != ceilLog2(outputSize))
+        throw std::runtime_error("zkFC::prove: challenges do not match the shapes");
 
     auto claim = Y.multi_dim_me({u_batch, u_output}, {batchSize, outputSize});
     zk_record(claim);

@@ -14,6 +14,11 @@ class zkFC {
     zkFC(uint input_size, uint output_size, const FrTensor& weight, const FrTensor& bias);
     FrTensor operator()(const FrTensor& X) const;
     vector<Claim> prove(const FrTensor& X, const FrTensor& Y) const;
+    // the proof's challenges drawn apart from its execution (same order: u_batch, u_input, u_output), for callers that draw
+    // the challenges of several proofs first and then run them
+    struct Challenges { vector<Fr_t> u_batch, u_input, u_output; };
+    Challenges draw(uint batchSize) const;
+    vector<Claim> prove(const FrTensor& X, const FrTensor& Y, const Challenges& ch) const;
 
     // weight_ptr / bias_ptr are device pointers to float data
     static zkFC from_float_gpu_ptr(uint input_size, uint output_size, unsigned long scaling_factor, float* weight_ptr, float* bias_ptr);
