@@ -28,6 +28,10 @@ HBM_PEAK_GBS = 8000.0
 # VALU integer peak: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz lane-operations per second (v_mad_u64_u32 issues at
 # full rate on gfx950; bench measures it as well and reports the measured figure next to this one)
 VALU_PEAK_TOPS = 256 * 4 * 16 * 2.4e9 / 1e12
+# HBM traffic of k_open_fold per generator pair, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the kernel alone
+# (python3 bench.py --pmc-probe; summary in profiles/k_open_fold_pmc_traffic.txt), each counter scaled by what it reads for
+# zk_fr_add over 2^24 elements (1 GiB read, 512 MiB written)
+FOLD_TRAFFIC_BYTES_PER_PAIR = 6090.0
 
 
 def main():
@@ -39,7 +43,7 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extras", action="store_true", help="only the layer timing (used for profiling runs)")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="for rocprofv3 --pmc runs: only three launches of the opening's fold kernel at 176128 pairs and one "
+                    help="for rocprofv3 --pmc runs: only three launches of the opening's fold kernel at 262144 pairs and one "
                          "zk_fr_add over 2^24 elements (1 GiB read, 512 MiB written) to scale the counters by")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -56,7 +60,7 @@ def main():
     lib = hip.lib
 
     if args.pmc_probe:
-        n_big = 11008 << 5
+        n_big = 1 << 19
         pv.seed(6)
         gens_big = pv.commitment_random(n_big)
         pv.lib.zkp_g1_devptr.restype = ctypes.c_void_p
@@ -152,19 +156,22 @@ def main():
     MAD_PER_FP_MUL = 300
     fold_tops = fold_mults.value * MAD_PER_FP_MUL / (fold_ms.value * 1e-3) / 1e12 if fold_ms.value > 0 else 0.0
     out["roofline"] = {"kernel": "k_open_fold (opening: g' = g1 + [u](g0 - g1) per pair, 128-bit split scalars)", "bound": "valu-int",
-                       "achieved": fold_tops, "peak": VALU_PEAK_TOPS, "unit": "T MAD32/s", "frac": fold_tops / VALU_PEAK_TOPS, "traffic": None,
+                       "achieved": fold_tops, "peak": VALU_PEAK_TOPS, "unit": "T MAD32/s", "frac": fold_tops / VALU_PEAK_TOPS,
+                       "traffic": FOLD_TRAFFIC_BYTES_PER_PAIR * fold_pairs.value / max(1, fold_launches.value),
                        "launches": int(fold_launches.value), "avg_launch_ms": fold_ms.value / max(1, fold_launches.value),
                        "total_ms_in_timed_region": fold_ms.value, "pairs": int(fold_pairs.value), "fp_mul_per_s": fold_mults.value / (fold_ms.value * 1e-3) if fold_ms.value > 0 else 0.0,
-                       "note": "algorithmic work = Fp multiplications of the point formulas x 300 MAD32; peak = 256 CU x 4 SIMD x 16 lanes x 2.4 GHz; "
-                               "HBM traffic of this kernel is 336 B per pair, far below the bandwidth bound.  The average covers every launch of the timed "
-                               "region: most are short rounds (a few thousand pairs, one wave per SIMD or less) that run beside the rest of the proof"}
+                       "note": "algorithmic work = Fp multiplications of the point formulas x 300 MAD32 (12-limb schoolbook product and reduction; the kernel "
+                               "itself works on 14 limbs of 29 bits: 392 multiply-adds and ~110 other instructions per product, 301 per square); "
+                               "peak = 256 CU x 4 SIMD x 16 lanes x 2.4 GHz.  traffic = measured bytes per pair (rocprofv3 FETCH_SIZE + WRITE_SIZE of the kernel alone, "
+                               "profiles/k_open_fold_pmc_traffic.txt) x the average pairs per launch; algorithmic traffic is 336 B per pair.  The average covers every "
+                               "launch of the timed region: most are short rounds (one wave per SIMD or less) that run beside the rest of the proof"}
     if args.skip_extras:
         print(json.dumps(out))
         return
 
-    # ---- the same fold kernel alone at its largest shape in the layer: one halving of 352256 generators (the FFN weights' opening) ----
+    # ---- the same fold kernel alone at its largest shape in the layer: one halving of 2^19 generators (the FFN weights' opening) ----
     pv.seed(6)
-    n_big = 11008 << 5
+    n_big = 1 << 19
     gens_big = pv.commitment_random(n_big)
     pv.lib.zkp_g1_devptr.restype = ctypes.c_void_p
     gp = pv.lib.zkp_g1_devptr(c_void_p(gens_big.h))
@@ -178,10 +185,12 @@ def main():
         hip.call("zk_g1_open_round", c_void_p(ns), c_void_p(ng), sums3, c_void_p(sc), c_void_p(gp), u1, c_size_t(n_big), None)
     hip.check(lib.zk_prof_fold_read(ctypes.byref(fold_ms), ctypes.byref(fold_launches), ctypes.byref(fold_mults), ctypes.byref(fold_pairs)))
     iso_tops = fold_mults.value * MAD_PER_FP_MUL / (fold_ms.value * 1e-3) / 1e12
-    out["roofline_fold_alone"] = {"kernel": "k_open_fold, 176128 pairs, nothing else on the device", "bound": "valu-int", "achieved": iso_tops, "peak": VALU_PEAK_TOPS,
-                                  "unit": "T MAD32/s", "frac": iso_tops / VALU_PEAK_TOPS, "traffic": None, "avg_launch_ms": fold_ms.value / max(1, fold_launches.value),
+    out["roofline_fold_alone"] = {"kernel": "k_open_fold, 262144 pairs, nothing else on the device", "bound": "valu-int", "achieved": iso_tops, "peak": VALU_PEAK_TOPS,
+                                  "unit": "T MAD32/s", "frac": iso_tops / VALU_PEAK_TOPS, "traffic": FOLD_TRAFFIC_BYTES_PER_PAIR * (n_big // 2),
+                                  "avg_launch_ms": fold_ms.value / max(1, fold_launches.value),
                                   "fp_mul_per_s": fold_mults.value / (fold_ms.value * 1e-3),
-                                  "note": "2752 waves on 2048 wave slots (two per SIMD at 248 VGPRs): the launch takes two full turns"}
+                                  "note": "4096 waves on 2048 wave slots (two per SIMD at 256 VGPRs): two full turns.  traffic: FETCH_SIZE + WRITE_SIZE of this "
+                                          "launch from profiles/k_open_fold_pmc_traffic.txt, against 336 B per pair of algorithmic traffic (the rest is register spill)"}
     for p_ in (sc, ns, ng):
         hip.free(p_)
     del gens_big
@@ -278,7 +287,7 @@ def main():
         orc.orc_open(gens, n_open, T, n_open, 1, u, k, proof, val)
         open_s = time.perf_counter() - t0
         layer_mm = 4.49e11                                     # field multiplications in the layer's matrix products (reference algorithm)
-        layer_gens = 5 * (4096 << 5) + 2 * (11008 << 5) + 2 * 4096   # generators of the nine openings; pairs over all rounds ~ the same number
+        layer_gens = 5 * (4096 << 5) + 2 * (1 << 19) + 2 * 4096      # generators of the nine openings (11008 << 5 rounds up to 2^19); pairs over all rounds ~ the same number
         cpu_s = layer_mm / mm_rate + open_s * layer_gens / n_open
         out["cpu_baseline"] = {"value": cpu_s, "unit": "s", "cores": int(cores), "kind": "port",
                                "sample": f"oracle (reference algorithm, OpenMP): Fr matmul {rows} x 4096 x 1024 = {rows * 4096 * 1024:.3g} multiplications in {dt:.1f} s, "
