@@ -307,3 +307,30 @@ def test_row_sums_of_squares_in_double_follow_a_plain_loop():
     assert (got.view(np.uint64) == exp.view(np.uint64)).all()
     hip.free(dX)
     hip.free(dout)
+
+
+def test_matmul_int8_plane_path_equals_generic_at_projection_size(pv):
+    """1024 x 4096 x 1024 (2^32 multiply-accumulates): the small-integer product goes to the matrix cores as balanced
+    base-256 digit planes.  Checked against the generic Montgomery kernel on the whole output and against big-int dot
+    products on sampled entries; the operands hold the values around every digit carry."""
+    rng = np.random.default_rng(5)
+    M, N, P = 1024, 4096, 1024
+    A = rng.integers(-(1 << 19), 1 << 19, (M, N)).astype(np.int64)
+    B = rng.integers(-(1 << 13), 1 << 13, (N, P)).astype(np.int64)
+    edge = np.array([0, 1, -1, 127, 128, -128, -129, 255, 256, -255, -256, 32767, 32768, -32768, -32769, 65535, 65536, -65536, -65537, (1 << 19) - 1, -(1 << 19)])
+    A[0, :edge.size] = edge
+    A[1:1 + edge.size, 0] = edge
+    B[:12, 0] = edge[:12]
+    B[0, :15] = edge[:15] // 8
+    hA, hB = pv.from_i64(A), pv.from_i64(B)
+    pv.lib.zkp_set_matmul_mode(ctypes.c_int(0))
+    got = pv.matmul(hA, hB, M, N, P).host()
+    assert pv.lib.zkp_last_matmul_path() == 2
+    pv.lib.zkp_set_matmul_mode(ctypes.c_int(1))
+    ref = pv.matmul(hA, hB, M, N, P).host()
+    pv.lib.zkp_set_matmul_mode(ctypes.c_int(0))
+    assert (got == ref).all()
+    Ao, Bo = A.astype(object), B.astype(object)
+    for (i, j) in [(0, 0), (1, 0), (5, 0), (0, 3)] + [(int(rng.integers(M)), int(rng.integers(P))) for _ in range(40)]:
+        want = int(sum(Ao[i, :] * Bo[:, j])) % R_MOD
+        assert fr_ints(got[i * P + j].reshape(1, 8))[0] == want

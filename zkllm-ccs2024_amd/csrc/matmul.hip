@@ -12,7 +12,15 @@
 //    product is bounded by 2^62, the same sum is computed in int64 and embedded at the end.
 //    The bound is established on the device from the operands (largest row sum of |a| times max |b|);
 //    nothing is assumed.  This is the case for every matmul of the LLaMa pipeline except softmax(Y)*V.
+//    Large products of this kind (the seven projections of a layer) are plain integer GEMMs and go to the matrix
+//    cores: both operands are split into balanced base-256 digits (int8 planes), every pair of planes is an int8 GEMM
+//    with int32 accumulation (rocBLAS, MFMA), planes of equal weight 2^(8s) accumulate into the same output, and one
+//    pass recombines the outputs in int64.  Exact: a dot product of digits stays below 2^31 (checked), the
+//    recombined value is the true integer result, below 2^62 by the bound above.
+#include <cstdlib>
 #include <cstring>
+#include <mutex>
+#include <rocblas/rocblas.h>
 #include "field.hpp"
 #include "rt.hpp"
 #include "../../include/zkllm_hip.h"
@@ -308,6 +316,92 @@ template <typename T> static int run_int_path(void* C, const void* A, const void
     return 0;
 }
 
+// ---- int8-plane path -----------------------------------------------------------------------------------------------
+// balanced base-256 digits of a small signed integer: x = sum_j d_j 256^j, d_j in [-128, 127]; planes[j * n + i] = d_j of element i
+__global__ void __launch_bounds__(256) k_split_planes(int8_t* __restrict__ planes, const Fr* __restrict__ a, size_t n, int np) {
+    const size_t i0 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i0 >= n) return;
+    long long x[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[e] = (i0 + e < n) ? fr_to_i64(a[i0 + e]) : 0ll;
+    for (int j = 0; j < np; ++j) {
+        uint32_t packed = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const long long d = (long long)(int8_t)(x[e] & 0xFF);
+            x[e] = (x[e] - d) >> 8;
+            packed |= (uint32_t)(uint8_t)d << (8 * e);
+        }
+        int8_t* dst = planes + (size_t)j * n + i0;
+        if (i0 + 3 < n && (((size_t)j * n + i0) & 3) == 0) *reinterpret_cast<uint32_t*>(dst) = packed;
+        else
+            for (int e = 0; e < 4 && i0 + e < n; ++e) dst[e] = (int8_t)(packed >> (8 * e));
+    }
+}
+// C[i] = sum_s Cs[s * n + i] * 2^(8s), embedded
+__global__ void __launch_bounds__(256) k_combine_planes(Fr* __restrict__ C, const int32_t* __restrict__ Cs, size_t n, int ns) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    unsigned long long v = 0;
+    for (int s2 = 0; s2 < ns; ++s2) v += (unsigned long long)(long long)Cs[(size_t)s2 * n + i] << (8 * s2);
+    C[i] = fr_from_i64((long long)v);
+}
+static int digits_for(unsigned long long absmax) {      // planes needed for |x| <= absmax: p digits reach 127 (256^p - 1) / 255
+    int p = 1;
+    unsigned __int128 reach = 127;
+    while (reach < absmax && p < 8) { reach = reach * 256 + 127; ++p; }
+    return reach >= absmax ? p : 0;
+}
+static rocblas_handle blas_handle() {
+    static rocblas_handle h = nullptr;
+    static std::mutex mu;
+    std::lock_guard<std::mutex> lk(mu);
+    if (!h && rocblas_create_handle(&h) != rocblas_status_success) h = nullptr;
+    return h;
+}
+// returns ZK status; *done = false when the path does not apply (the caller then takes a VALU kernel)
+static int run_int8_plane_path(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, unsigned long long ma, unsigned long long mb, hipStream_t st,
+                               bool* done) {
+    *done = false;
+    const int pa = digits_for(ma), pb = digits_for(mb);
+    if (!pa || !pb) return 0;
+    const int ns = pa + pb - 1;
+    const int most_pairs = pa < pb ? pa : pb;                       // planes pairs that share a weight
+    if ((unsigned long long)most_pairs * N >= (1ull << 17)) return 0;   // |sum of digit products| must stay below 2^31
+    if (M > (1u << 30) || N > (1u << 30) || P > (1u << 30)) return 0;
+    rocblas_handle h = blas_handle();
+    if (!h) return 0;
+    const size_t na = (size_t)M * N, nb = (size_t)N * P, nc = (size_t)M * P;
+    Scratch pla(na * pa), plb(nb * pb), cs(nc * ns * sizeof(int32_t));
+    if (pla.rc) return pla.rc;
+    if (plb.rc) return plb.rc;
+    if (cs.rc) return cs.rc;
+    hipLaunchKernelGGL(k_split_planes, dim3(cdiv(cdiv(na, 4), 256)), dim3(256), 0, st, pla.as<int8_t>(), (const Fr*)A, na, pa);
+    hipLaunchKernelGGL(k_split_planes, dim3(cdiv(cdiv(nb, 4), 256)), dim3(256), 0, st, plb.as<int8_t>(), (const Fr*)B, nb, pb);
+    ZK_LAUNCH_CHECK();
+    if (rocblas_set_stream(h, st) != rocblas_status_success) { set_error(ZK_ERR_BLAS, "rocblas_set_stream failed"); return ZK_ERR_BLAS; }
+    const int32_t one = 1, zero = 0;
+    for (int s2 = 0; s2 < ns; ++s2) {
+        int32_t* out = cs.as<int32_t>() + (size_t)s2 * nc;
+        bool first = true;
+        for (int i = 0; i < pa; ++i) {
+            const int j = s2 - i;
+            if (j < 0 || j >= pb) continue;
+            // row-major C = A_i B_j is column-major C^T = B_j^T A_i^T: the row-major arrays are those transposes as they lie
+            const rocblas_status rs = rocblas_gemm_ex(h, rocblas_operation_none, rocblas_operation_none, (rocblas_int)P, (rocblas_int)M, (rocblas_int)N, &one,
+                                                      plb.as<int8_t>() + (size_t)j * nb, rocblas_datatype_i8_r, (rocblas_int)P, pla.as<int8_t>() + (size_t)i * na,
+                                                      rocblas_datatype_i8_r, (rocblas_int)N, first ? &zero : &one, out, rocblas_datatype_i32_r, (rocblas_int)P, out,
+                                                      rocblas_datatype_i32_r, (rocblas_int)P, rocblas_datatype_i32_r, rocblas_gemm_algo_standard, 0, 0);
+            if (rs != rocblas_status_success) { (void)hipStreamSynchronize(st); set_error(ZK_ERR_BLAS, "rocblas_gemm_ex (int8) failed"); return ZK_ERR_BLAS; }
+            first = false;
+        }
+    }
+    hipLaunchKernelGGL(k_combine_planes, dim3(cdiv(nc, 256)), dim3(256), 0, st, (Fr*)C, cs.as<int32_t>(), nc, ns);
+    ZK_LAUNCH_CHECK();
+    *done = true;
+    return 0;
+}
+
 static inline unsigned absmax_grid(size_t n) {
     size_t b = n / (256 * 8) + 1;
     return (unsigned)(b > 1024 ? 1024 : b);
@@ -332,6 +426,7 @@ int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, 
     ZK_ARG(N > 0, "zk_fr_matmul: inner dimension is 0");
     ZK_ARG(mode >= 0 && mode <= 2, "zk_fr_matmul: mode must be 0, 1 or 2");
     bool small = false, fits32 = false, b_fits32 = false;
+    unsigned long long ma_ = 0, mb_ = 0;
     if (mode != 1) {
         Scratch mx(3 * sizeof(unsigned long long));
         if (mx.rc) return mx.rc;
@@ -353,6 +448,7 @@ int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, 
             small = bound < ((unsigned __int128)1 << 62);
             fits32 = ma < (1ull << 31) && mb < (1ull << 31);
             b_fits32 = mb < (1ull << 31) && ma < (1ull << 62);
+            ma_ = ma; mb_ = mb;
         }
         if (mode == 2 && !small) { set_error(ZK_ERR_ARG, "zk_fr_matmul: operands do not satisfy the small-integer bound"); return ZK_ERR_ARG; }
     }
@@ -361,6 +457,14 @@ int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, 
         return zk_fr_matmul_generic(C, A, B, M, N, P, stv);
     }
     if (path_used) *path_used = 2;
+    // large products go to the matrix cores as int8 digit planes; below ~4 G multiply-accumulates the conversions outweigh the gain
+    // (ZKLLM_MATMUL_PLANES: log2 of that threshold, 0 = never)
+    static const int planes_log2 = getenv("ZKLLM_MATMUL_PLANES") ? atoi(getenv("ZKLLM_MATMUL_PLANES")) : 32;
+    if (planes_log2 > 0 && (unsigned long long)M * N * P >= (1ull << planes_log2)) {
+        bool done = false;
+        const int rc = run_int8_plane_path(C, A, B, M, N, P, ma_, mb_, st, &done);
+        if (rc || done) return rc;
+    }
     if (fits32) return run_int_path<int>(C, A, B, M, N, P, st);
     if (b_fits32) return run_wide_narrow_path(C, A, B, M, N, P, st);
     return run_int_path<long long>(C, A, B, M, N, P, st);
