@@ -196,6 +196,8 @@ int zk_hadamard_prove_end(void* handle, uint32_t* coefs_host);
 
 /* ---- rescaling / softmax ------------------------------------------------------------------------------------------ */
 int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* stream);       /* rescaling_kernel rescaling.cu:8-21 */
+/* zkrelu_decomp_kernel zkrelu.cu:8-29: the same rescaling, then sign (1 when the rescaled value is >= 0), magnitude and max(., 0) */
+int zk_relu_decomp(void* res, void* sign, void* mag, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* stream);
 /* zksoftmax_shift zksoftmax.cu:20-32 (scale = sf_in*sqrt(d)), zksoftmax_calculate_table :4-14, zksoftmax_decompose_kernel :95-109 */
 int zk_softmax_shift(void* shift, void* out_shifted, const void* X, uint32_t rows, uint32_t cols, double scale, void* stream);
 int zk_softmax_table(void* table, double log_theta, double step, uint32_t len, void* stream);

@@ -206,6 +206,10 @@ int orc_zkfc(const int32_t* X, const int32_t* W, u32 B, u32 I, u32 O, u32* Y_out
 int orc_rescale(const u32* X, long n, u32 sf, u32* out, u32* rem) {
     ORC_TRY Rescaling rs(sf); vec_out(rs.apply(vec_in(X, n)), out); vec_out(rs.rem, rem); ORC_END
 }
+// zkReLU::operator(): res, sign, abs, rem (n each) and the multiplicities m (table size, sf rounded up to a power of two)
+int orc_relu(const u32* X, long n, u32 sf, u32* res, u32* sign, u32* mag, u32* rem, u32* m) {
+    ORC_TRY ZkReLU z(sf); vec_out(z.apply(vec_in(X, n)), res); vec_out(z.sign, sign); vec_out(z.mag, mag); vec_out(z.rem, rem); vec_out(z.m, m); ORC_END
+}
 // full Rescaling::operator() + prove with seeded challenges; transcript records the round polys
 int orc_rescale_prove(const u32* X, long n, u32 sf, u32* out) {
     ORC_TRY

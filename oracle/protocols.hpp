@@ -3,6 +3,7 @@
 //   tlookup.cu     prep :10-48, inverse :50-62, phase 1 :74-103,184-200,300-320,
 //                  phase 2 :161-175,202-298, prove :324-370, range :372-433, mapping :435-551
 //   rescaling.cu   :8-79
+//   zkrelu.cu      :8-50
 //   zksoftmax.cu   tables :4-14, shift :20-32, ctor :34-93, decompose :95-109, compute :112-173,
 //                  prove :175-220
 //   g1-tensor.cu   sum :391-443, scalar mul :445-482, G1_me :486-514, rowwise_sum :535-625
@@ -227,6 +228,35 @@ struct Rescaling {
         rec(lhs);
         if (lhs != rhs) throw std::runtime_error("Error: the rem is not correct.");
         tl_rem.prove(remp, m, rt[0], rt[1], u, v);
+    }
+};
+
+// =============================== zkReLU (zkrelu.cu:8-50) ==========================================
+// Rescaling's quotient and remainder, then the quotient split into sign (1 when >= 0), magnitude and max(., 0);
+// operator() also keeps the multiplicities of the remainders in the remainder table.  prove() is empty in the reference.
+struct ZkReLU {
+    uint sf;
+    TLookupRange tl_rem;
+    FrVec sign, mag, rem, m;
+    explicit ZkReLU(uint sf_) : sf(sf_), tl_rem(-(int)(sf_ >> 1), sf_) {}
+    FrVec apply(const FrVec& X) {
+        const long n = (long)X.size();
+        FrVec res(n);
+        sign.assign(n, fr_from_u32(0)); mag.resize(n); rem.resize(n);
+        const int64_t s = (int64_t)sf, h = s >> 1;
+        for (long i = 0; i < n; ++i) {
+            int64_t x = fr_to_i64(X[i]);
+            int64_t t = (x + h) % s;
+            int64_t xr = (t < 0 ? t + s : t) - h;
+            int64_t q = (x - xr) / s;
+            bool pos = q >= 0;
+            sign[i] = fr_from_u32(pos ? 1u : 0u);
+            mag[i] = fr_from_i64(pos ? q : -q);
+            rem[i] = fr_from_i64(xr);
+            res[i] = pos ? fr_from_i64(q) : fr_from_u32(0);
+        }
+        m = tl_rem.prep(rem);
+        return res;
     }
 };
 

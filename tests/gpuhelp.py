@@ -157,7 +157,7 @@ class Prover:
                      "zkp_fr_pad", "zkp_fr_transpose", "zkp_fr_matmul",
                      "zkp_g1_from_host", "zkp_g1_from_file", "zkp_g1_devptr", "zkp_commitment_random", "zkp_g1_binop", "zkp_g1_pointop",
                      "zkp_g1_scalar_mul", "zkp_g1_rowwise_sum", "zkp_commit_int", "zkp_commit",
-                     "zkp_rescale", "zkp_rescale_prove", "zkp_range_prep", "zkp_batch_inv", "zkp_softmax",
+                     "zkp_rescale", "zkp_rescale_prove", "zkp_relu", "zkp_range_prep", "zkp_batch_inv", "zkp_softmax",
                      "zkp_layer_create", "zkp_layer_create_random", "zkp_layer_run"):
             getattr(L, name).restype = c_void_p
         L.zkp_transcript_size.restype = ctypes.c_long
@@ -293,6 +293,11 @@ class Prover:
         rem = c_void_p()
         out = self.H(self.lib.zkp_rescale(c_void_p(X.h), c_uint(sf), ctypes.byref(rem)))
         return out, self.H(rem.value)
+
+    def relu(self, X, sf):
+        parts = (c_void_p * 4)()
+        out = self.H(self.lib.zkp_relu(c_void_p(X.h), c_uint(sf), parts))
+        return out, [self.H(p) for p in parts]
 
     def rescale_prove(self, X, sf):
         return self.H(self.lib.zkp_rescale_prove(c_void_p(X.h), c_uint(sf)))

@@ -19,3 +19,14 @@ def test_reference_driver_compiles_against_compat_headers(name, tmp_path):
     # the source is fed on stdin so that its quoted includes resolve to the forwarding headers, not to the reference's own
     r = subprocess.run(["g++", "-std=c++17", "-x", "c++", "-fsyntax-only", "-w", "-I" + inc, "-"], input=src, text=True, capture_output=True, cwd=tmp_path)
     assert r.returncode == 0, r.stderr[:2000]
+
+
+def test_every_reference_header_name_has_a_forwarding_header(tmp_path):
+    """A source that includes each class header by the reference's file name and touches one member of each compiles."""
+    names = ["bls12-381", "fr-tensor", "g1-tensor", "ioutils", "commitment", "polynomial", "proof", "zkfc", "tlookup",
+             "rescaling", "zksoftmax", "zkrelu"]
+    src = "".join(f'#include "{n}.cuh"\n' for n in names)
+    src += "void use(const FrTensor& X) { zkReLU r(16); FrTensor y = r(X); r.prove(X, y); Rescaling s(16); FrTensor z = s(X); }\n"
+    inc = os.path.join(ROOT, "zkllm-ccs2024_amd", "host", "compat")
+    r = subprocess.run(["g++", "-std=c++17", "-x", "c++", "-fsyntax-only", "-w", "-I" + inc, "-"], input=src, text=True, capture_output=True, cwd=tmp_path)
+    assert r.returncode == 0, r.stderr[:2000]

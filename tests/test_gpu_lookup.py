@@ -35,6 +35,21 @@ def test_rescale(pv, orc, n, sf):
     assert (out.host() == e_out).all() and (rem.host() == e_rem).all()
 
 
+@pytest.mark.parametrize("n,sf", [(1, 16), (1000, 16), (70000, 1 << 16)])
+def test_relu_decomposition(pv, orc, n, sf):
+    rng = np.random.default_rng(n + 1)
+    x = rng.integers(-(1 << 40), 1 << 40, n)
+    x[: min(n, 7)] = [0, sf // 2, -(sf // 2), sf // 2 - 1, -(sf // 2) - 1, 3 * sf, -3 * sf][: min(n, 7)]
+    X = fr_array([int(v) % R_MOD for v in x])
+    e = [np.zeros_like(X) for _ in range(4)]
+    e_m = np.zeros((sf, 8), np.uint32)
+    orc_check(orc.orc_relu(X, n, sf, *e, e_m))
+    out, parts = pv.relu(pv.from_fr(X), sf)
+    assert (out.host() == e[0]).all()
+    for got, want in zip(parts, e[1:] + [e_m]):
+        assert (got.host() == want).all()
+
+
 @pytest.mark.parametrize("D,low,length", [(64, -5, 11), (5000, -8, 16), (1 << 16, -(1 << 15), 1 << 16), (300000, 0, 1 << 18), (100000, 0, 3)])
 def test_multiplicities(pv, D, low, length):
     rng = np.random.default_rng(D)

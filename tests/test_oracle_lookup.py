@@ -26,6 +26,28 @@ def test_rescaling_exhaustive_small_range():
             assert ri == ((x + h) % sf) - h          # python's floor-mod is the kernel's adjusted C remainder
 
 
+def test_relu_decomposition_exhaustive_small_range():
+    """zkReLU's parts from python's floor division: x = q sf + rem with rem in [-h, sf - h); sign = [q >= 0], abs = |q|,
+    result = max(q, 0); multiplicities of the remainders = bincount.  sign * abs - (1 - sign) * abs = q ties them."""
+    orc = load_oracle()
+    for sf in (16, 8):
+        h = sf >> 1
+        xs = list(range(-3 * sf - 3, 3 * sf + 4)) + [2 ** 40 + 5, -(2 ** 40) - 5]
+        n = len(xs)
+        X = fr_array([x % R_MOD for x in xs])
+        res, sign, mag, rem = (np.zeros_like(X) for _ in range(4))
+        m = np.zeros((sf, 8), np.uint32)
+        orc_check(orc.orc_relu(X, n, sf, res, sign, mag, rem, m))
+        signed = lambda a: [v if v < R_MOD // 2 else v - R_MOD for v in fr_ints(a)]
+        q = [(x + h) // sf for x in xs]
+        assert signed(rem) == [x - qi * sf for x, qi in zip(xs, q)]
+        assert fr_ints(sign) == [int(qi >= 0) for qi in q]
+        assert fr_ints(mag) == [abs(qi) for qi in q]
+        assert fr_ints(res) == [max(qi, 0) for qi in q]
+        assert fr_ints(m) == list(np.bincount(np.array(signed(rem)) + h, minlength=sf))
+        assert all(s * a - (1 - s) * a == qi for s, a, qi in zip(fr_ints(sign), fr_ints(mag), q))
+
+
 def test_range_prep_is_bincount_and_inverse_identity():
     orc = load_oracle()
     rng = random.Random(51)

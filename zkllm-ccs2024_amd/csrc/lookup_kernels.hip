@@ -694,6 +694,24 @@ __global__ void __launch_bounds__(TPB) k_rescale(Fr* __restrict__ out, Fr* __res
     rem[i] = fr_from_i64(x_rem);
 }
 
+// ---- ReLU decomposition (zkrelu.cu:8-29) -----------------------------------------------------------------------------------------
+// The rescaling above, then the rescaled value split into sign (1 when >= 0), magnitude and max(., 0).
+__global__ void __launch_bounds__(TPB) k_relu_decomp(Fr* __restrict__ res, Fr* __restrict__ sign, Fr* __restrict__ mag, Fr* __restrict__ rem,
+                                                     const Fr* __restrict__ in, int64_t sf, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    const int64_t hsf = sf >> 1;
+    const int64_t x = fr_to_i64(in[i]);
+    const int64_t temp = (x + hsf) % sf;
+    const int64_t x_rem = (temp < 0 ? temp + sf : temp) - hsf;
+    const int64_t x_rescaled = (x - x_rem) / sf;
+    const bool pos = x_rescaled >= 0;
+    sign[i] = fr_from_u64(pos ? 1u : 0u);
+    mag[i] = fr_from_i64(pos ? x_rescaled : -x_rescaled);
+    rem[i] = fr_from_i64(x_rem);
+    res[i] = pos ? fr_from_i64(x_rescaled) : big_zero<8>();
+}
+
 // ---- softmax (zksoftmax.cu) ------------------------------------------------------------------------------------------------------
 // One wave per row.  Lane l sums exp(x_j / scale) over j = l, l+64, ... in index order, the 64 partial
 // sums are combined with the butterfly i ^ 32, 16, ..., 1 (every lane ends with the same total), and
@@ -1342,6 +1360,11 @@ int zk_hadamard_product_sumcheck(uint32_t* proof_host, const void* a, const void
 int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* st) {
     ZK_ARG(scaling_factor >= 1, "zk_rescale: scaling factor is 0");
     LAUNCH1D(k_rescale, n, st, (Fr*)out, (Fr*)rem, (const Fr*)in, (int64_t)scaling_factor, n);
+    return 0;
+}
+int zk_relu_decomp(void* res, void* sign, void* mag, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* st) {
+    ZK_ARG(scaling_factor >= 1, "zk_relu_decomp: scaling factor is 0");
+    LAUNCH1D(k_relu_decomp, n, st, (Fr*)res, (Fr*)sign, (Fr*)mag, (Fr*)rem, (const Fr*)in, (int64_t)scaling_factor, n);
     return 0;
 }
 int zk_softmax_shift(void* shift, void* out_shifted, const void* X, uint32_t rows, uint32_t cols, double scale, void* st) {

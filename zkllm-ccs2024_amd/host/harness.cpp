@@ -15,6 +15,7 @@
 #include "commitment.hpp"
 #include "tlookup.hpp"
 #include "rescaling.hpp"
+#include "zkrelu.hpp"
 #include "zksoftmax.hpp"
 #include "layer.hpp"
 
@@ -264,6 +265,19 @@ void* zkp_rescale_prove(void* X, u32 sf) {
     Rescaling rs(sf);
     FrTensor out = rs(FT(X));
     rs.prove(FT(X), out);
+    return new FrTensor(std::move(out));
+    ZKP_END_PTR
+}
+// zkReLU::operator(): returns max(rescaled, 0); parts[0..3] receive copies of sign, abs, rem and the multiplicities
+void* zkp_relu(void* X, u32 sf, void** parts) {
+    ZKP_TRY
+    zkReLU z(sf);
+    FrTensor out = z(FT(X));
+    z.prove(FT(X), out);
+    parts[0] = new FrTensor(*z.sign_tensor_ptr);
+    parts[1] = new FrTensor(*z.abs_tensor_ptr);
+    parts[2] = new FrTensor(*z.rem_tensor_ptr);
+    parts[3] = new FrTensor(*z.m_tensor_ptr);
     return new FrTensor(std::move(out));
     ZKP_END_PTR
 }
