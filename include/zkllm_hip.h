@@ -77,6 +77,8 @@ int zk_row_sumsq_f64(void* out_f64, const void* X, uint32_t rows, uint32_t cols,
 /* ---- layout (pad fr-tensor.cu:800-828, transpose :885-900, gather tlookup.cu:446-453) ----------- */
 int zk_fr_pad(void* out, const void* in, size_t rows, uint32_t last_in, uint32_t last_out, const uint32_t* pad, void* stream);
 int zk_fr_transpose(void* out, const void* in, uint32_t M, uint32_t N, void* stream);
+/* the same for a stack of `batch` M x N matrices stored one after the other (per-head K^T of zkAttn::compute, zksoftmax.cu:234) */
+int zk_fr_transpose_batched(void* out, const void* in, uint32_t batch, uint32_t M, uint32_t N, void* stream);
 int zk_fr_gather(void* out, const void* table, const void* idx_u32, size_t n, void* stream);
 
 /* ---- reductions and folds ------------------------------------------------------------------------ */

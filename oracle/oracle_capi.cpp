@@ -273,6 +273,44 @@ int orc_softmax(const u32* X, u32 m, u32 n, u32 d, const u32* bs, int K, u32 L, 
     ORC_END
 }
 
+// zkFCStacked: forward of num layers (bias optional: b == nullptr means none), then prove with seeded challenges
+int orc_zkfc_stacked(const u32* X, const u32* W, const u32* b, u32 num, u32 batch, u32 in, u32 out, u32* Y_out) {
+    ORC_TRY
+    FrVec x = vec_in(X, (long)num * batch * in), w = vec_in(W, (long)num * in * out), bias = b ? vec_in(b, (long)num * out) : FrVec();
+    FrVec y = zkfc_stacked_forward(x, w, bias, num, batch, in, out);
+    if (Y_out) vec_out(y, Y_out);
+    std::vector<Poly> proof;
+    zkfc_stacked_prove(x, w, bias, y, num, batch, in, out, proof);
+    ORC_END
+}
+// zkAttn (stacked = 0: one head, zkAttn::compute + zkAttn::prove) or zkAttnStacked over num heads; challenges are
+// drawn from the seeded stream in the order of the prove function's parameters; final_claim receives the returned claim
+int orc_attn(const u32* Q, const u32* K, const u32* V, u32 num, u32 m, u32 n, u32 d, int stacked, const u32* bs, int nb, u32 L, u32 M, uint64_t sf_Q, uint64_t sf_K,
+             const double* thetas, int nth, u32* out_host, u32* final_claim) {
+    ORC_TRY
+    ZkSoftmax sm(std::vector<uint>(bs, bs + nb), L, M, sf_Q * sf_K, std::vector<double>(thetas, thetas + nth), num * m, n, d);
+    FrVec q = vec_in(Q, (long)num * m * d), k = vec_in(K, (long)num * n * d), v = vec_in(V, (long)num * n * d);
+    ZkAttnTensors t;
+    FrVec out = zkattn_compute(sm, num, m, n, d, q, k, v, t);
+    if (out_host) vec_out(out, out_host);
+    std::vector<Poly> proof;
+    Fr fin;
+    if (!stacked) {
+        need(num == 1, "zkAttn proves one head");
+        FrVec u_mo = random_vec(ceilLog2(m)), v_mo = random_vec(ceilLog2(n)), w_mo = random_vec(ceilLog2(d));
+        FrVec v_sm = random_vec(ceilLog2(m) + ceilLog2(n)), t3 = random_vec(3), v_mi = random_vec(ceilLog2(d));
+        fin = zkattn_prove(sm, m, n, d, q, k, v, out, t, u_mo, v_mo, w_mo, v_sm, t3[0], t3[1], t3[2], v_mi, proof);
+    } else {
+        FrVec u_mo_num = random_vec(ceilLog2(num)), v_mo_num = random_vec(ceilLog2(num));
+        FrVec u_mo = random_vec(ceilLog2(m)), v_mo = random_vec(ceilLog2(n)), w_mo = random_vec(ceilLog2(d));
+        FrVec v_sm = random_vec(ceilLog2(num) + ceilLog2(m) + ceilLog2(n)), t3 = random_vec(3);
+        FrVec v_mi_num = random_vec(ceilLog2(num)), v_mi = random_vec(ceilLog2(d));
+        fin = zkattn_stacked_prove(sm, num, m, n, d, q, k, v, out, t, u_mo_num, v_mo_num, u_mo, v_mo, w_mo, v_sm, t3[0], t3[1], t3[2], v_mi_num, v_mi, proof);
+    }
+    if (final_claim) std::memcpy(final_claim, &fin, 32);
+    ORC_END
+}
+
 // deterministic exp / log used by the softmax steps (kind 0 exp, 1 log)
 void orc_detmath(int kind, const double* x, double* out, long n) { for (long i = 0; i < n; ++i) out[i] = kind ? o_log(x[i]) : o_exp(x[i]); }
 

@@ -5,7 +5,7 @@
 //   rescaling.cu   :8-79
 //   zkrelu.cu      :8-50
 //   zksoftmax.cu   tables :4-14, shift :20-32, ctor :34-93, decompose :95-109, compute :112-173,
-//                  prove :175-220
+//                  prove :175-220, zkAttn :222-287, zkAttnStacked :289-320
 //   g1-tensor.cu   sum :391-443, scalar mul :445-482, G1_me :486-514, rowwise_sum :535-625
 //   commitment.cu  random :3-8, commit :22-29, commit_int :31-58, me_open :79-129, open :133-141
 //   proof.cu       verifyWeightClaim :3-10
@@ -351,6 +351,64 @@ struct ZkSoftmax {
         return Xo;
     }
 };
+
+// =============================== zkAttn / zkAttnStacked (zksoftmax.cu:222-320) =====================
+// Tensors of `num` heads are stacked head-major: Q [num][m][d], K and V [num][n][d], scores [num][m][n], out [num][m][d].
+// `sm` is built for num * m rows: softmax rows are independent and prove() only uses its n.
+struct ZkAttnTensors { FrVec sm_in, sm_out, shift, shifted; std::vector<FrVec> in_seg, out_seg, m_seg; };
+
+// zkAttn::compute (:225-239) on every head's slice; the row softmax once over all heads (the reference has the forward
+// pass of one head only)
+static inline FrVec zkattn_compute(ZkSoftmax& sm, uint num, uint m, uint n, uint d, const FrVec& Q, const FrVec& K, const FrVec& V, ZkAttnTensors& t) {
+    need(Q.size() == (size_t)num * m * d, "Q must be m * d");
+    need(K.size() == (size_t)num * n * d, "K must be n * d");
+    need(V.size() == (size_t)num * n * d, "V must be n * d");
+    t.sm_in.assign((size_t)num * m * n, FR_ZERO);
+    for (uint h = 0; h < num; ++h) {
+        FrVec Qh(Q.begin() + (size_t)h * m * d, Q.begin() + (size_t)(h + 1) * m * d), Kh(K.begin() + (size_t)h * n * d, K.begin() + (size_t)(h + 1) * n * d);
+        FrVec X = t_matmul(Qh, t_transpose(Kh, n, d), m, d, n);
+        std::copy(X.begin(), X.end(), t.sm_in.begin() + (size_t)h * m * n);
+    }
+    t.sm_out = sm.compute(t.sm_in, t.shift, t.shifted, t.in_seg, t.out_seg, t.m_seg);
+    FrVec out((size_t)num * m * d);
+    for (uint h = 0; h < num; ++h) {
+        FrVec Yh(t.sm_out.begin() + (size_t)h * m * n, t.sm_out.begin() + (size_t)(h + 1) * m * n), Vh(V.begin() + (size_t)h * n * d, V.begin() + (size_t)(h + 1) * n * d);
+        FrVec o = t_matmul(Yh, Vh, m, n, d);
+        std::copy(o.begin(), o.end(), out.begin() + (size_t)h * m * d);
+    }
+    return out;
+}
+// zkAttn::prove with given challenges (:258-287)
+static inline Fr zkattn_prove(ZkSoftmax& sm, uint m, uint n, uint d, const FrVec& Q, const FrVec& K, const FrVec& V, const FrVec& out, const ZkAttnTensors& t,
+                              const FrVec& u_mo, const FrVec& v_mo, const FrVec& w_mo, const FrVec& v_sm, const Fr& r_seg, const Fr& alpha_seg, const Fr& beta_seg,
+                              const FrVec& v_mi, std::vector<Poly>& proof) {
+    Fr out_claim = t_multi_dim_me(out, {u_mo, w_mo}, {m, d});
+    rec(out_claim);
+    FrVec vec0 = t_partial_me(t.sm_out, u_mo, m, n), vec1 = t_partial_me(V, w_mo, d, 1);
+    Fr mm = zkip(out_claim, vec0, vec1, v_mo, proof);
+    Fr V_claim = t_multi_dim_me(V, {v_mo, w_mo}, {n, d}), sm_out_claim = t_multi_dim_me(t.sm_out, {u_mo, v_mo}, {m, n});
+    if (mm != V_claim * sm_out_claim) throw std::runtime_error("out_matmul_claim is not correct");
+    FrVec u_Y = v_mo; u_Y.insert(u_Y.end(), u_mo.begin(), u_mo.end());
+    Fr sm_in_claim = sm.prove(t.sm_out, t.sm_in, t.shift, t.in_seg, t.out_seg, t.m_seg, u_Y, v_sm, r_seg, alpha_seg, beta_seg, proof);
+    FrVec u_mi(v_sm.end() - ceilLog2(m), v_sm.end()), w_mi(v_sm.begin(), v_sm.end() - ceilLog2(m));
+    return zkip(sm_in_claim, t_partial_me(Q, u_mi, m, d), t_partial_me(K, w_mi, n, d), v_mi, proof);
+}
+// zkAttnStacked::prove (:292-320)
+static inline Fr zkattn_stacked_prove(ZkSoftmax& sm, uint num, uint m, uint n, uint d, const FrVec& Q, const FrVec& K, const FrVec& V, const FrVec& out, const ZkAttnTensors& t,
+                                      const FrVec& u_mo_num, const FrVec& v_mo_num, const FrVec& u_mo, const FrVec& v_mo, const FrVec& w_mo, const FrVec& v_sm,
+                                      const Fr& r_seg, const Fr& alpha_seg, const Fr& beta_seg, const FrVec& v_mi_num, const FrVec& v_mi, std::vector<Poly>& proof) {
+    Fr out_claim = t_multi_dim_me(out, {u_mo_num, u_mo, w_mo}, {num, m, d});
+    rec(out_claim);
+    FrVec sm_out_reduced = t_partial_me(t.sm_out, u_mo, m, n), V_reduced = t_partial_me(V, w_mo, d, 1);
+    Fr mm = zkip_stacked(out_claim, sm_out_reduced, V_reduced, u_mo_num, v_mo, v_mo_num, num, n, proof);
+    Fr V_claim = t_multi_dim_me(V, {v_mo_num, v_mo, w_mo}, {num, n, d}), sm_out_claim = t_multi_dim_me(t.sm_out, {v_mo_num, u_mo, v_mo}, {num, m, n});
+    if (mm != V_claim * sm_out_claim) throw std::runtime_error("out_matmul_claim is not correct");
+    FrVec u_Y = v_mo; u_Y.insert(u_Y.end(), u_mo.begin(), u_mo.end()); u_Y.insert(u_Y.end(), v_mo_num.begin(), v_mo_num.end());
+    Fr sm_in_claim = sm.prove(t.sm_out, t.sm_in, t.shift, t.in_seg, t.out_seg, t.m_seg, u_Y, v_sm, r_seg, alpha_seg, beta_seg, proof);
+    const uint ln = ceilLog2(num), lm = ceilLog2(m);
+    FrVec u_mi_num(v_sm.end() - ln, v_sm.end()), u_mi(v_sm.end() - ln - lm, v_sm.end() - ln), w_mi(v_sm.begin(), v_sm.end() - ln - lm);
+    return zkip_stacked(sm_in_claim, t_partial_me(Q, u_mi, m, d), t_partial_me(K, w_mi, n, d), u_mi_num, v_mi, v_mi_num, num, d, proof);
+}
 
 // =============================== G1 tensors / commitment ==========================================
 typedef std::vector<G1Jac> G1Vec;

@@ -5,7 +5,7 @@
 //                  multi-dim fold :518-560, multi_dim_me :643-652, pad :800-828, matmul :831-881,
 //                  transpose :885-900, random_vec :16-24, ceilLog2 :26-43
 //   polynomial.cu  host Fr operators :4-150, Polynomial :152-329, eq :342-372
-//   zkfc.cu        zkip :94-151, zkip_stacked :153-229, zkFC::prove :61-87
+//   zkfc.cu        zkip :94-151, zkip_stacked :153-229, zkFC::prove :61-87, zkFCStacked :261-307
 //   proof.cu       hadamard_product_sumcheck :67-107, multi_hadamard_sumchecks :172-241
 // Every value is the canonical residue in [0, r), so summation order is free.
 // OpenMP parallel loops are used where the reference launches one thread per element; this
@@ -425,6 +425,34 @@ static inline Claim zkfc_prove(const FrVec& X, const FrVec& W, const FrVec& Y, u
     rec(final_claim); rec(claim_X); rec(claim_W);
     if (claim_X * claim_W != final_claim) throw std::runtime_error("Claim does not match");
     return Claim{claim_W, {u_input, u_output}, {in, out}};
+}
+
+// ---- zkFCStacked (zkfc.cu:44-58 forward with bias per layer, prove :261-307) ------------------------------------
+// X [num][batch][in], W [num][in][out], b [num][out] (empty = no bias), Y [num][batch][out]
+static inline FrVec zkfc_stacked_forward(const FrVec& X, const FrVec& W, const FrVec& b, uint num, uint batch, uint in, uint out) {
+    FrVec Y((size_t)num * batch * out);
+    for (uint l = 0; l < num; ++l) {
+        FrVec Xl(X.begin() + (size_t)l * batch * in, X.begin() + (size_t)(l + 1) * batch * in), Wl(W.begin() + (size_t)l * in * out, W.begin() + (size_t)(l + 1) * in * out);
+        FrVec y = t_matmul(Xl, Wl, batch, in, out);
+        if (!b.empty()) for (size_t i = 0; i < y.size(); ++i) y[i] = add(y[i], b[(size_t)l * out + i % out]);
+        std::copy(y.begin(), y.end(), Y.begin() + (size_t)l * batch * out);
+    }
+    return Y;
+}
+static inline void zkfc_stacked_prove(const FrVec& X, const FrVec& W, const FrVec& b, const FrVec& Y, uint num, uint batch, uint in, uint out, std::vector<Poly>& proof) {
+    FrVec u_num = random_vec(ceilLog2(num)), v_num = random_vec(ceilLog2(num));
+    FrVec u_batch = random_vec(ceilLog2(batch)), u_input = random_vec(ceilLog2(in)), u_output = random_vec(ceilLog2(out));
+    Fr claim = t_multi_dim_me(Y, {u_num, u_batch, u_output}, {num, batch, out});
+    if (!b.empty()) {
+        FrVec ones(batch, F_ONE);
+        claim = claim - t_me(ones, u_batch) * t_multi_dim_me(b, {u_num, u_output}, {num, out});
+    }
+    rec(claim);
+    FrVec Xr = t_partial_me(X, u_batch, batch, in), Wr = t_partial_me(W, u_output, out, 1);
+    Fr final_claim = zkip_stacked(claim, Xr, Wr, u_num, u_input, v_num, num, in, proof);
+    Fr opening = t_multi_dim_me(X, {v_num, u_batch, u_input}, {num, batch, in}) * t_multi_dim_me(W, {v_num, u_input, u_output}, {num, in, out});
+    rec(final_claim);
+    if (final_claim != opening) throw std::runtime_error("final claim != opening");
 }
 
 // ---- deprecated Hadamard sumcheck still used by the rmsnorm driver (proof.cu:12-27, 67-107) ----------------

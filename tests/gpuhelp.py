@@ -157,7 +157,7 @@ class Prover:
                      "zkp_fr_pad", "zkp_fr_transpose", "zkp_fr_matmul",
                      "zkp_g1_from_host", "zkp_g1_from_file", "zkp_g1_devptr", "zkp_commitment_random", "zkp_g1_binop", "zkp_g1_pointop",
                      "zkp_g1_scalar_mul", "zkp_g1_rowwise_sum", "zkp_commit_int", "zkp_commit",
-                     "zkp_rescale", "zkp_rescale_prove", "zkp_relu", "zkp_range_prep", "zkp_batch_inv", "zkp_softmax",
+                     "zkp_rescale", "zkp_rescale_prove", "zkp_relu", "zkp_attn", "zkp_zkfc_stacked", "zkp_range_prep", "zkp_batch_inv", "zkp_softmax",
                      "zkp_layer_create", "zkp_layer_create_random", "zkp_layer_run"):
             getattr(L, name).restype = c_void_p
         L.zkp_transcript_size.restype = ctypes.c_long
@@ -351,6 +351,19 @@ class Prover:
         y = self.H(self.lib.zkp_softmax(c_void_p(X.h), c_uint(m), c_uint(n), c_uint(d), _np_ptr(bs), c_int(len(bs)), c_uint(L), c_uint(M), c_u64(sf_in),
                                         _np_ptr(thetas), c_int(len(thetas)), ctypes.byref(shift), c_int(1 if prove else 0)))
         return y, self.H(shift.value)
+
+    def attn(self, Q, K, V, num, m, n, d, stacked, bs, L, M, sf_Q, sf_K, thetas):
+        bs = np.ascontiguousarray(bs, dtype=np.uint32)
+        th = np.ascontiguousarray(thetas, dtype=np.float64)
+        fin = np.zeros(8, np.uint32)
+        out = self.H(self.lib.zkp_attn(c_void_p(Q.h), c_void_p(K.h), c_void_p(V.h), c_uint(num), c_uint(m), c_uint(n), c_uint(d), c_int(int(stacked)),
+                                       _np_ptr(bs), c_int(len(bs)), c_uint(L), c_uint(M), ctypes.c_uint64(sf_Q), ctypes.c_uint64(sf_K),
+                                       th.ctypes.data_as(c_void_p), c_int(len(th)), _np_ptr(fin)))
+        return out, fin
+
+    def zkfc_stacked(self, X, W, b, num, batch, n_in, n_out):
+        return self.H(self.lib.zkp_zkfc_stacked(c_void_p(X.h), c_void_p(W.h), c_void_p(b.h) if b is not None else None, c_uint(num), c_uint(batch),
+                                                c_uint(n_in), c_uint(n_out)))
 
     def zkip_stacked(self, claim, A, B, N, D, uN, vN, uD):
         uN, vN, uD = (np.ascontiguousarray(x, dtype=np.uint32).reshape(-1, 8) for x in (uN, vN, uD))

@@ -2,6 +2,7 @@
 rescaling, multi-Hadamard sumcheck, stacked inner-product sumcheck and zkSoftmax -- bit-exact against the oracle."""
 import numpy as np
 import pytest
+from ctypes import c_uint64 as c_u64
 
 from zkhelp import R_MOD, fr_array, fr_ints, load_oracle, mt_random_vec, orc_check, orc_transcript
 
@@ -223,6 +224,48 @@ def test_softmax_compute_and_prove(pv, orc, m, n, d, bs, sf, lim):
     Y, shift = pv.softmax(pv.from_fr(Xf), m, n, d, bsa, 1, 0, sf, thetas, prove)
     pv.lib.zkp_transcript_end()
     assert (shift.host() == e_shift).all()
+    assert (Y.host() == e_Y).all()
+    t = pv.transcript()
+    assert t.shape == e_t.shape and (t == e_t).all()
+
+
+@pytest.mark.parametrize("num,stacked,m,n,d", [(1, 0, 16, 16, 16), (1, 1, 16, 16, 16), (4, 1, 16, 16, 16), (2, 1, 8, 32, 4)])
+def test_attention_forward_and_proof(pv, orc, num, stacked, m, n, d):
+    """zkAttn (one head) and zkAttnStacked (head-major stacks): forward pass, transcript and returned claim."""
+    rng = np.random.default_rng(num * 1000 + m + n + d)
+    qmax = 3 if d == 16 else 6
+    Q, K, V = (fr_array([int(x) % R_MOD for x in rng.integers(-qmax, qmax + 1, num * r * d)]) for r in (m, n, n))
+    bs = np.array([16, 16, 16], np.uint32)
+    thetas = np.array([float(1 << 10), float(1 << 12)])
+    e_out, e_fin = np.zeros((num * m * d, 8), np.uint32), np.zeros(8, np.uint32)
+    orc.orc_seed(11)
+    orc.orc_transcript_clear()
+    orc_check(orc.orc_attn(Q, K, V, num, m, n, d, stacked, bs, 3, 1, 0, c_u64(16), c_u64(16), thetas, 2, e_out, e_fin))
+    e_t = orc_transcript(orc)
+    pv.seed(11)
+    pv.transcript_begin()
+    out, fin = pv.attn(pv.from_fr(Q), pv.from_fr(K), pv.from_fr(V), num, m, n, d, stacked, bs, 1, 0, 16, 16, thetas)
+    pv.lib.zkp_transcript_end()
+    assert (out.host() == e_out).all() and (fin == e_fin).all()
+    t = pv.transcript()
+    assert t.shape == e_t.shape and (t == e_t).all()
+
+
+@pytest.mark.parametrize("num,batch,n_in,n_out,bias", [(1, 4, 8, 8, False), (4, 8, 16, 4, False), (4, 8, 16, 4, True), (3, 5, 6, 7, True)])
+def test_stacked_fully_connected_proof(pv, orc, num, batch, n_in, n_out, bias):
+    rng = np.random.default_rng(num + batch + n_in + n_out)
+    X = fr_array([int(x) % R_MOD for x in rng.integers(-1000, 1000, num * batch * n_in)])
+    W = fr_array([int(x) % R_MOD for x in rng.integers(-1000, 1000, num * n_in * n_out)])
+    b = fr_array([int(x) % R_MOD for x in rng.integers(-10 ** 6, 10 ** 6, num * n_out)]) if bias else None
+    e_Y = np.zeros((num * batch * n_out, 8), np.uint32)
+    orc.orc_seed(12)
+    orc.orc_transcript_clear()
+    orc_check(orc.orc_zkfc_stacked(X, W, b, num, batch, n_in, n_out, e_Y))
+    e_t = orc_transcript(orc)
+    pv.seed(12)
+    pv.transcript_begin()
+    Y = pv.zkfc_stacked(pv.from_fr(X), pv.from_fr(W), pv.from_fr(b) if bias else None, num, batch, n_in, n_out)
+    pv.lib.zkp_transcript_end()
     assert (Y.host() == e_Y).all()
     t = pv.transcript()
     assert t.shape == e_t.shape and (t == e_t).all()

@@ -222,3 +222,35 @@ def test_softmax_integer_structure():
     orc.orc_transcript_clear()
     orc_check(orc.orc_softmax(Xf, m, n, d, bs, 3, 1, 0, sf, thetas, 2, Y, shift, 1))
     assert len(orc_transcript(orc)) > 20
+
+
+def _fr_signed(a):
+    return [v if v < R_MOD // 2 else v - R_MOD for v in fr_ints(a)]
+
+
+def test_attention_forward_is_per_head_softmax_attention_and_both_proofs_run():
+    """zkattn_compute against numpy integer matrix products around the (separately pinned) row softmax: scores = Q_h K_h^T
+    per head of the head-major stacks, out = Y_h V_h; then zkAttn::prove (one head) and zkAttnStacked::prove run through
+    all their in-prover identities (inner-product rounds, out = Y V at the drawn point, scores = Q K^T at the softmax's
+    point): a transposed operand or a wrong split of the challenge vectors fails one of them."""
+    orc = load_oracle()
+    bs = np.array([16, 16, 16], np.uint32)
+    thetas = np.array([float(1 << 10), float(1 << 12)])
+    for num, stacked, m, n, d in [(1, 0, 16, 16, 16), (4, 1, 8, 16, 16), (2, 1, 4, 8, 4)]:
+        rng = np.random.default_rng(num * 100 + m)
+        qmax = 3 if d == 16 else 6
+        Qi, Ki, Vi = (rng.integers(-qmax, qmax + 1, (num, r, d)) for r in (m, n, n))
+        Q, K, V = (fr_array([int(x) % R_MOD for x in a.reshape(-1)]) for a in (Qi, Ki, Vi))
+        out, fin = np.zeros((num * m * d, 8), np.uint32), np.zeros(8, np.uint32)
+        orc.orc_seed(3)
+        orc.orc_transcript_clear()
+        orc_check(orc.orc_attn(Q, K, V, num, m, n, d, stacked, bs, 3, 1, 0, 16, 16, thetas, 2, out, fin))
+        assert len(orc_transcript(orc)) > 30
+        # the softmax of the stacked scores through the entry point that test_softmax_integer_structure pins
+        X = np.einsum("hik,hjk->hij", Qi, Ki)
+        Xf = fr_array([int(x) % R_MOD for x in X.reshape(-1)])
+        Y, shift = np.zeros((num * m * n, 8), np.uint32), np.zeros((num * m, 8), np.uint32)
+        orc_check(orc.orc_softmax(Xf, num * m, n, d, bs, 3, 1, 0, 256, thetas, 2, Y, shift, 0))
+        Yi = np.array(fr_ints(Y), dtype=object).reshape(num, m, n)
+        want = [[[sum(int(Yi[h][i][j]) * int(Vi[h][j][k]) for j in range(n)) for k in range(d)] for i in range(m)] for h in range(num)]
+        assert _fr_signed(out) == [v for h in want for row in h for v in row]

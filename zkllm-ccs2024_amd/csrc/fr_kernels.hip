@@ -107,8 +107,11 @@ __global__ void __launch_bounds__(TPB) k_pad(Fr* __restrict__ out, const Fr* __r
     out[g] = (g1 >= last_in) ? pad : in[g0 * last_in + g1];
 }
 // 32x32 tile through LDS so both the read and the write are contiguous along the fast axis
+// blockIdx.z selects one of a stack of M x N matrices
 __global__ void __launch_bounds__(TPB) k_transpose(Fr* __restrict__ out, const Fr* __restrict__ in, uint32_t M, uint32_t N) {
     __shared__ uint32_t tile[8][32][33];
+    in += (size_t)blockIdx.z * M * N;
+    out += (size_t)blockIdx.z * M * N;
     const uint32_t bx = blockIdx.x * 32, by = blockIdx.y * 32;
     const uint32_t tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 32 x 8
     for (uint32_t r = ty; r < 32; r += 8) {
@@ -479,13 +482,15 @@ int zk_fr_pad(void* out, const void* in, size_t rows, uint32_t last_in, uint32_t
     LAUNCH1D(k_pad, n_out, st, (Fr*)out, (const Fr*)in, n_out, last_in, last_out, load_fr(pad));
     return 0;
 }
-int zk_fr_transpose(void* out, const void* in, uint32_t M, uint32_t N, void* st) {
-    if (M == 0 || N == 0) return 0;
+int zk_fr_transpose_batched(void* out, const void* in, uint32_t batch, uint32_t M, uint32_t N, void* st) {
+    if (batch == 0 || M == 0 || N == 0) return 0;
     ZK_ARG(out != in, "zk_fr_transpose: in-place transpose is not supported");
-    hipLaunchKernelGGL(k_transpose, dim3(cdiv(N, 32), cdiv(M, 32)), dim3(TPB), 0, (hipStream_t)st, (Fr*)out, (const Fr*)in, M, N);
+    ZK_ARG(batch <= 65535 && cdiv(M, 32) <= 65535, "zk_fr_transpose: too many matrices or rows for one launch");
+    hipLaunchKernelGGL(k_transpose, dim3(cdiv(N, 32), cdiv(M, 32), batch), dim3(TPB), 0, (hipStream_t)st, (Fr*)out, (const Fr*)in, M, N);
     ZK_LAUNCH_CHECK();
     return 0;
 }
+int zk_fr_transpose(void* out, const void* in, uint32_t M, uint32_t N, void* st) { return zk_fr_transpose_batched(out, in, 1, M, N, st); }
 int zk_fr_gather(void* out, const void* table, const void* idx, size_t n, void* st) {
     LAUNCH1D(k_gather, n, st, (Fr*)out, (const Fr*)table, (const uint32_t*)idx, n);
     return 0;

@@ -362,6 +362,26 @@ FrTensor FrTensor::matmul(const FrTensor& x, const FrTensor& y, uint M, uint N, 
     return out;
 }
 
+FrTensor FrTensor::transpose_stack(uint num, uint M, uint N) const {
+    if ((size_t)size != (size_t)num * M * N) throw std::runtime_error("transpose: incompatible dimensions");
+    FrTensor out(size);
+    ZKC(zk_fr_transpose_batched(out.gpu_data, gpu_data, num, M, N, nullptr));
+    return out;
+}
+FrTensor FrTensor::matmul_stack(const FrTensor& x, const FrTensor& y, uint num, uint M, uint N, uint P) {
+    FrTensor out(num * M * P);
+    matmul_stack_into(out, x, y, num, M, N, P);
+    return out;
+}
+void FrTensor::matmul_stack_into(FrTensor& out, const FrTensor& x, const FrTensor& y, uint num, uint M, uint N, uint P) {
+    if ((size_t)x.size != (size_t)num * M * N || (size_t)y.size != (size_t)num * N * P || (size_t)out.size != (size_t)num * M * P)
+        throw std::runtime_error("matmul: incompatible dimensions");
+    int path = 0;
+    for (uint i = 0; i < num; ++i)
+        ZKC(zk_fr_matmul(out.gpu_data + (size_t)i * M * P, x.gpu_data + (size_t)i * M * N, y.gpu_data + (size_t)i * N * P, M, N, P, G().matmul_mode, &path, nullptr));
+    G().last_matmul_path = path;
+}
+
 // The reference draws these from cuRAND with a random_device seed (fr-tensor.cu:444-510); here they come
 // from the seedable host stream: same distributions, reproducible.
 FrTensor FrTensor::random_int(uint size, uint num_bits) {

@@ -104,6 +104,11 @@ class FrTensor {
     FrTensor trunc(uint begin_idx, uint end_idx) const;
 
     static FrTensor matmul(const FrTensor& x, const FrTensor& y, uint M, uint N, uint P);
+    // additions for stacks of `num` equally shaped matrices stored one after the other: every M x N matrix transposed,
+    // and the num products x_i (M x N) * y_i (N x P)
+    FrTensor transpose_stack(uint num, uint M, uint N) const;
+    static FrTensor matmul_stack(const FrTensor& x, const FrTensor& y, uint num, uint M, uint N, uint P);
+    static void matmul_stack_into(FrTensor& out, const FrTensor& x, const FrTensor& y, uint num, uint M, uint N, uint P);
     static FrTensor random_int(uint size, uint num_bits);
     static FrTensor random(uint size);
     // all-`x` tensor (replaces the cudaMemset + `+= x` idiom of the reference's callers)

@@ -348,6 +348,55 @@ void* zkp_softmax(void* X, u32 m, u32 n, u32 d, const u32* bs, int K, u32 L, u32
     return new FrTensor(std::move(y));
     ZKP_END_PTR
 }
+// zkAttn (stacked = 0: one head, zkAttn::compute + zkAttn::prove) or zkAttnStacked over num heads (its compute + prove);
+// challenges from the seeded stream in the order of the prove function's parameters; returns out, final_claim the returned claim
+void* zkp_attn(void* Q, void* K, void* V, u32 num, u32 m, u32 n, u32 d, int stacked, const u32* bs, int nb, u32 L, u32 M, uint64_t sf_Q, uint64_t sf_K,
+               const double* thetas, int nth, u32* final_claim) {
+    ZKP_TRY
+    const std::vector<uint> bsv(bs, bs + nb);
+    const std::vector<double> th(thetas, thetas + nth);
+    std::vector<FrTensor> xseg, yseg, mseg;
+    std::vector<Polynomial> proof;
+    Fr_t fin;
+    if (!stacked) {
+        if (num != 1) throw std::runtime_error("zkAttn proves one head");
+        zkAttn at((unsigned long)sf_Q, (unsigned long)sf_K, bsv, L, M, th, m, n, d, 1);
+        FrTensor sm_in(m * n), sm_out(m * n), shift(m), xs(m * n);
+        FrTensor out = at.compute(FT(Q), FT(K), FT(V), sm_in, sm_out, shift, xs, xseg, yseg, mseg);
+        auto u_mo = random_vec(ceilLog2(m)), v_mo = random_vec(ceilLog2(n)), w_mo = random_vec(ceilLog2(d));
+        auto v_sm = random_vec(ceilLog2(m) + ceilLog2(n)), t3 = random_vec(3), v_mi = random_vec(ceilLog2(d));
+        fin = at.prove(FT(Q), FT(K), FT(V), out, sm_out, sm_in, shift, xs, xseg, yseg, mseg, u_mo, v_mo, w_mo, v_sm, t3[0], t3[1], t3[2], v_mi, proof);
+        if (final_claim) memcpy(final_claim, fin.val, 32);
+        return new FrTensor(std::move(out));
+    }
+    zkAttnStacked at(num, (unsigned long)sf_Q, (unsigned long)sf_K, bsv, L, M, th, m, n, d, 1);
+    FrTensor sm_in(num * m * n), sm_out(num * m * n), shift(num * m), xs(num * m * n);
+    FrTensor out = at.compute(FT(Q), FT(K), FT(V), sm_in, sm_out, shift, xs, xseg, yseg, mseg);
+    auto c = at.draw();
+    fin = at.prove(FT(Q), FT(K), FT(V), out, sm_out, sm_in, shift, xs, xseg, yseg, mseg, c.u_matmul_out_num, c.v_matmul_out_num, c.u_matmul_out, c.v_matmul_out,
+                   c.w_matmul_out, c.v_sm, c.temp_rand[0], c.temp_rand[1], c.temp_rand[2], c.v_matmul_in_num, c.v_matmul_in, proof);
+    if (final_claim) memcpy(final_claim, fin.val, 32);
+    return new FrTensor(std::move(out));
+    ZKP_END_PTR
+}
+// zkFCStacked over num layers: X [num][batch][in], W [num][in][out], b [num][out] or null; forward per layer, then prove
+void* zkp_zkfc_stacked(void* X, void* W, void* b, u32 num, u32 batch, u32 in, u32 out) {
+    ZKP_TRY
+    std::vector<zkFC> layers;
+    std::vector<FrTensor> Xs, Ys;
+    for (u32 l = 0; l < num; ++l) {
+        FrTensor w = FT(W).trunc(l * in * out, (l + 1) * in * out);
+        if (b) layers.emplace_back(in, out, w, FT(b).trunc(l * out, (l + 1) * out));
+        else layers.emplace_back(in, out, w);
+        Xs.push_back(FT(X).trunc(l * batch * in, (l + 1) * batch * in));
+        Ys.push_back(layers.back()(Xs.back()));
+    }
+    zkFCStacked st(b != nullptr, num, batch, in, out, layers, Xs, Ys);
+    std::vector<Polynomial> proof;
+    st.prove(proof);
+    return new FrTensor(catTensors(Ys));
+    ZKP_END_PTR
+}
 int zkp_zkip_stacked(const u32* claim, void* A, void* B, u32 N, u32 D, const u32* uN, const u32* vN, int kN, const u32* uD, int kD, u32* proof_out, u32* final_claim) {
     ZKP_TRY
     std::vector<Polynomial> proof;

@@ -42,7 +42,11 @@ zkSoftmax::zkSoftmax(const vector<uint>& bs, uint L, uint M, unsigned long scali
 
 // zksoftmax.cu:112-173
 FrTensor zkSoftmax::compute(const FrTensor& X, FrTensor& shift, FrTensor& X_shifted, vector<FrTensor>& X_segments, vector<FrTensor>& Y_segments, vector<FrTensor>& m_segments) {
-    if (X.size != m * n) throw std::invalid_argument("X must be m * n");
+    return compute_rows(m, X, shift, X_shifted, X_segments, Y_segments, m_segments);
+}
+FrTensor zkSoftmax::compute_rows(uint m, const FrTensor& X, FrTensor& shift, FrTensor& X_shifted, vector<FrTensor>& X_segments, vector<FrTensor>& Y_segments,
+                                 vector<FrTensor>& m_segments, FrTensor* into) {
+    if ((size_t)X.size != (size_t)m * n) throw std::invalid_argument("X must be m * n");
     if (shift.size != m) throw std::invalid_argument("shift must be m");
     if (X_shifted.size != X.size) throw std::invalid_argument("X_shifted must be the same size as X");
 
@@ -65,6 +69,13 @@ FrTensor zkSoftmax::compute(const FrTensor& X, FrTensor& shift, FrTensor& X_shif
         m_segments.push_back(std::move(p.second));
     }
     // the product of the segments' table values (the reference multiplies them one by one into a tensor of ones)
+    if (into) {
+        if (into->size != X.size) throw std::invalid_argument("the result must be the same size as X");
+        if (Y_segments.size() == 1) { *into = Y_segments[0]; return FrTensor(0); }
+        ZKC(zk_fr_mul(into->gpu_data, Y_segments[0].gpu_data, Y_segments[1].gpu_data, N, nullptr));
+        for (size_t i = 2; i < Y_segments.size(); ++i) *into *= Y_segments[i];
+        return FrTensor(0);
+    }
     if (Y_segments.size() == 1) return FrTensor(Y_segments[0]);
     FrTensor out = Y_segments[0] * Y_segments[1];
     for (size_t i = 2; i < Y_segments.size(); ++i) out *= Y_segments[i];
@@ -194,6 +205,32 @@ Fr_t zkAttn::prove(const FrTensor& Q, const FrTensor& K, const FrTensor& V, cons
 
 zkAttnStacked::zkAttnStacked(uint num, unsigned long sf_Q, unsigned long sf_K, const vector<uint>& bs, uint L, uint M, const vector<double>& thetas, uint m, uint n, uint d, uint E)
     : zkAttn(sf_Q, sf_K, bs, L, M, thetas, m, n, d, E), num(num) {}
+
+FrTensor zkAttnStacked::compute(const FrTensor& Q, const FrTensor& K, const FrTensor& V, FrTensor& sm_in, FrTensor& sm_out, FrTensor& sm_shift, FrTensor& sm_in_shifted,
+                                vector<FrTensor>& sm_in_segments, vector<FrTensor>& sm_out_segments, vector<FrTensor>& sm_m_segments) {
+    if ((size_t)Q.size != (size_t)num * m * d) throw std::invalid_argument("Q must be m * d");
+    if ((size_t)K.size != (size_t)num * n * d) throw std::invalid_argument("K must be n * d");
+    if ((size_t)V.size != (size_t)num * n * d) throw std::invalid_argument("V must be n * d");
+    if ((size_t)sm_in.size != (size_t)num * m * n || sm_out.size != sm_in.size || sm_in_shifted.size != sm_in.size || sm_shift.size != num * m)
+        throw std::invalid_argument("softmax tensors must be num * m * n (shift: num * m)");
+    FrTensor::matmul_stack_into(sm_in, Q, K.transpose_stack(num, n, d), num, m, d, n);
+    compute_rows(num * m, sm_in, sm_shift, sm_in_shifted, sm_in_segments, sm_out_segments, sm_m_segments, &sm_out);
+    return FrTensor::matmul_stack(sm_out, V, num, m, n, d);
+}
+
+zkAttnStacked::Challenges zkAttnStacked::draw() const {
+    Challenges c;
+    c.u_matmul_out_num = random_vec(ceilLog2(num));
+    c.v_matmul_out_num = random_vec(ceilLog2(num));
+    c.u_matmul_out = random_vec(ceilLog2(m));
+    c.v_matmul_out = random_vec(ceilLog2(n));
+    c.w_matmul_out = random_vec(ceilLog2(d));
+    c.v_sm = random_vec(ceilLog2(num) + ceilLog2(m) + ceilLog2(n));
+    c.temp_rand = random_vec(3);
+    c.v_matmul_in_num = random_vec(ceilLog2(num));
+    c.v_matmul_in = random_vec(ceilLog2(d));
+    return c;
+}
 
 Fr_t zkAttnStacked::prove(const FrTensor& Q, const FrTensor& K, const FrTensor& V, const FrTensor& out, const FrTensor& sm_out, const FrTensor& sm_in,
                           const FrTensor& sm_shift, const FrTensor& sm_in_shifted, const vector<FrTensor>& sm_in_segments, const vector<FrTensor>& sm_out_segments,

@@ -31,6 +31,10 @@ class zkSoftmax {
                    const vector<Fr_t>& v_Y, vector<Polynomial>& proof);
 
    protected:
+    // compute() for `rows` rows of n scores (rows = m for one head, num * m for a stack of heads: rows are independent)
+    // the result goes to *into when given (no copy of a large tensor), else it is returned
+    FrTensor compute_rows(uint rows, const FrTensor& X, FrTensor& shift, FrTensor& X_shifted, vector<FrTensor>& X_segments, vector<FrTensor>& Y_segments,
+                          vector<FrTensor>& m_segments, FrTensor* into = nullptr);
     const vector<uint> bs;
     const uint K, L, M;
     const unsigned long scaling_factor_in;
@@ -62,6 +66,16 @@ class zkAttn : public zkSoftmax {
 class zkAttnStacked : public zkAttn {
    public:
     zkAttnStacked(uint num, unsigned long sf_Q, unsigned long sf_K, const vector<uint>& bs, uint L, uint M, const vector<double>& thetas, uint m, uint n, uint d, uint E);
+
+    // Addition (the reference has the forward pass of one head only): zkAttn::compute on every head of the head-major stacks
+    // Q [num][m][d], K and V [num][n][d]; scores and softmax tensors come back as [num][m][n], the result as [num][m][d].
+    FrTensor compute(const FrTensor& Q, const FrTensor& K, const FrTensor& V, FrTensor& sm_in, FrTensor& sm_out, FrTensor& sm_shift, FrTensor& sm_in_shifted,
+                     vector<FrTensor>& sm_in_segments, vector<FrTensor>& sm_out_segments, vector<FrTensor>& sm_m_segments);
+    // Addition: the challenges of prove() drawn from the challenge stream in the order of its parameters
+    struct Challenges {
+        vector<Fr_t> u_matmul_out_num, v_matmul_out_num, u_matmul_out, v_matmul_out, w_matmul_out, v_sm, temp_rand, v_matmul_in_num, v_matmul_in;
+    };
+    Challenges draw() const;
 
     Fr_t prove(const FrTensor& Q, const FrTensor& K, const FrTensor& V, const FrTensor& out, const FrTensor& sm_out, const FrTensor& sm_in, const FrTensor& sm_shift,
                const FrTensor& sm_in_shifted, const vector<FrTensor>& sm_in_segments, const vector<FrTensor>& sm_out_segments, const vector<FrTensor>& sm_m_segments,
