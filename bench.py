@@ -40,6 +40,8 @@ def main():
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--seq", type=int, default=2048)
+    ap.add_argument("--head-group", type=int, default=0,
+                    help="attention proved this many heads at a time with zkAttnStacked (a divisor of 32); 0 = head by head")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extras", action="store_true", help="only the layer timing (used for profiling runs)")
     ap.add_argument("--pmc-probe", action="store_true",
@@ -99,7 +101,7 @@ def main():
 
     # ---- workload: the decoder layer ------------------------------------------------------------------------------
     seq = args.seq
-    cu, cf = layercfg.llama7b(seq=seq, open_weights=True)
+    cu, cf = layercfg.llama7b(seq=seq, open_weights=True, head_group=args.head_group)
     t0 = time.perf_counter()
     pv.seed(2024)
     layer = pv.layer_create_random(cu, cf, 7, 5)

@@ -99,6 +99,9 @@ int zk_fr_matmul_generic(void* C, const void* A, const void* B, uint32_t M, uint
 /* mode 0: pick the small-integer path when a device-side bound check proves it exact; 1: generic
  * Montgomery only; 2: small-integer only (error if the bound fails).  path_used: 1 generic, 2 small-int. */
 int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used_host, void* stream);
+/* the same for a stack of `batch` products, A [batch][M][N], B [batch][N][P], C [batch][M][P] (the per-head products of
+ * zkAttn::compute, zksoftmax.cu:234-238, for all heads at once); the bound check covers the whole stacks, so one path serves all */
+int zk_fr_matmul_batched(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used_host, void* stream);
 
 /* ---- inner-product sumcheck (zkip_poly_kernel + 3 sums, zkfc.cu:94-138) ----------------------------- */
 int zk_ip_round(uint32_t* poly3_host, const void* a, const void* b, size_t n_in, size_t n_out, void* stream);

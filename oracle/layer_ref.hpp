@@ -3,7 +3,8 @@
 // Composes the oracle's primitives in the order of the reference's per-block executables:
 //   rmsnorm.cu:26-49, self-attn.cu:19-76 (linear) and :78-121 (attn), ffn.cu:44-93, skip-connection.cu:15-18.
 // Where the reference cannot be followed literally the same choices as the product's layer are made and
-// recorded: attention is proved per head with d = head width and the concatenated output rescaled twice;
+// recorded: attention is proved per head with d = head width (or, with attn_head_group = g, g heads at a time
+// through zkAttnStacked) and the concatenated output rescaled twice;
 // an output projection follows; challenges drawn inside argument lists in the reference (rmsnorm.cu:47,
 // self-attn.cu:112-113) are drawn first-argument-first; the RMS statistic is host double arithmetic
 // (llama-rmsnorm.py:35-39) and RoPE / causal mask (unproven float steps of llama-self-attn.py) are left out.
@@ -17,6 +18,7 @@ struct OLayerConfig {
     uint sf_linear, sf_gate, sf_attn;
     std::vector<uint> softmax_bs; uint softmax_L, softmax_M; uint64_t softmax_sf_in; std::vector<double> softmax_thetas;
     int swiglu_low; uint swiglu_len; double swiglu_in_scale, swiglu_out_scale; double rms_eps, value_scale; bool open_weights;
+    uint attn_head_group = 0;   // 0: head by head; g: g heads at a time through zkAttnStacked
 };
 struct OWeight { G1Vec gens; FrVec weight; G1Vec com; uint in_dim, out_dim; };
 
@@ -81,8 +83,42 @@ static inline FrVec o_head(const FrVec& t, uint S, uint E, uint h, uint d) {
     for (uint r = 0; r < S; ++r) for (uint j = 0; j < d; ++j) out[(size_t)r * d + j] = t[(size_t)r * E + h * d + j];
     return out;
 }
+// g heads at a time as head-major stacks with zkAttnStacked (zksoftmax.cu:289-320); challenges in the order of its parameters
+static inline FrVec o_attn_stacked_heads(const OLayerConfig& c, const FrVec& Q_, const FrVec& K_, const FrVec& V_) {
+    const uint S = c.seq_len, E = c.embed_dim, H = c.num_heads, d = E / H, g = c.attn_head_group;
+    need(H % g == 0, "attn_head_group must divide num_heads");
+    FrVec out_all((size_t)S * E);
+    for (uint h0 = 0; h0 < H; h0 += g) {
+        FrVec Q, K, V;
+        for (uint h = h0; h < h0 + g; ++h) {
+            FrVec q = o_head(Q_, S, E, h, d), k = o_head(K_, S, E, h, d), v = o_head(V_, S, E, h, d);
+            Q.insert(Q.end(), q.begin(), q.end()); K.insert(K.end(), k.begin(), k.end()); V.insert(V.end(), v.begin(), v.end());
+        }
+        ZkSoftmax sm(c.softmax_bs, c.softmax_L, c.softmax_M, c.softmax_sf_in, c.softmax_thetas, g * S, S, d);
+        ZkAttnTensors t;
+        FrVec out = zkattn_compute(sm, g, S, S, d, Q, K, V, t);
+        for (uint h = h0; h < h0 + g; ++h)
+            for (uint r = 0; r < S; ++r) for (uint j = 0; j < d; ++j) out_all[(size_t)r * E + h * d + j] = out[((size_t)(h - h0) * S + r) * d + j];
+        FrVec u_mo_num = random_vec(ceilLog2(g)), v_mo_num = random_vec(ceilLog2(g));
+        FrVec u_mo = random_vec(ceilLog2(S)), v_mo = random_vec(ceilLog2(S)), w_mo = random_vec(ceilLog2(d));
+        FrVec v_sm = random_vec(ceilLog2(g) + 2 * ceilLog2(S)), t3 = random_vec(3);
+        FrVec v_mi_num = random_vec(ceilLog2(g)), v_mi = random_vec(ceilLog2(d));
+        std::vector<Poly> proof;
+        zkattn_stacked_prove(sm, g, S, S, d, Q, K, V, out, t, u_mo_num, v_mo_num, u_mo, v_mo, w_mo, v_sm, t3[0], t3[1], t3[2], v_mi_num, v_mi, proof);
+    }
+    return out_all;
+}
 static inline FrVec o_attn_heads_block(const OLayerConfig& c, const FrVec& Q_, const FrVec& K_, const FrVec& V_) {
     const uint S = c.seq_len, E = c.embed_dim, H = c.num_heads, d = E / H;
+    if (c.attn_head_group) {
+        FrVec out_all = o_attn_stacked_heads(c, Q_, K_, V_);
+        Rescaling rs1(c.sf_attn), rs2(c.sf_attn);
+        FrVec o_ = rs2.apply(out_all);
+        FrVec o__ = rs1.apply(o_);
+        rs1.prove(o_, o__);
+        rs2.prove(out_all, o_);
+        return o__;
+    }
     FrVec out_all((size_t)S * E);
     ZkSoftmax sm(c.softmax_bs, c.softmax_L, c.softmax_M, c.softmax_sf_in, c.softmax_thetas, S, S, d);
     for (uint h = 0; h < H; ++h) {

@@ -347,6 +347,7 @@ static OLayerConfig parse_cfg(const u32* cu, const double* cf) {
     c.swiglu_len = cu[9]; c.open_weights = cu[10] != 0;
     const u32 K = cu[11];
     c.softmax_bs.assign(cu + 12, cu + 12 + K);
+    c.attn_head_group = cu[12 + K];
     c.softmax_sf_in = (uint64_t)cf[0]; c.swiglu_low = (int)cf[1]; c.swiglu_in_scale = cf[2]; c.swiglu_out_scale = cf[3]; c.rms_eps = cf[4]; c.value_scale = cf[5];
     c.softmax_thetas.assign(cf + 6, cf + 6 + (K - c.softmax_L - c.softmax_M));
     return c;

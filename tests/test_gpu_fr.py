@@ -334,3 +334,28 @@ def test_matmul_int8_plane_path_equals_generic_at_projection_size(pv):
     for (i, j) in [(0, 0), (1, 0), (5, 0), (0, 3)] + [(int(rng.integers(M)), int(rng.integers(P))) for _ in range(40)]:
         want = int(sum(Ao[i, :] * Bo[:, j])) % R_MOD
         assert fr_ints(got[i * P + j].reshape(1, 8))[0] == want
+
+
+def test_stacks_of_matrices_transpose_and_multiply_like_their_members(pv):
+    """zk_fr_matmul_batched / zk_fr_transpose_batched on every path of the dispatcher (both operands in 31 bits, wide left
+    operand, wide right operand, full-width residues): each product of the stack against big-int arithmetic."""
+    rng = np.random.default_rng(77)
+    num, M, N, P = 3, 70, 130, 50
+    cases = [((-2 ** 17, 2 ** 17), (-2 ** 10, 2 ** 10), 2), ((-2 ** 40, 2 ** 40), (-2 ** 12, 2 ** 12), 2), ((-2 ** 20, 2 ** 20), (-2 ** 33, 2 ** 33), 2)]
+    pv.lib.zkp_set_matmul_mode(ctypes.c_int(0))
+    for (alo, ahi), (blo, bhi), path in cases:
+        A = rng.integers(alo, ahi, (num, M, N)).astype(np.int64)
+        B = rng.integers(blo, bhi, (num, N, P)).astype(np.int64)
+        got = pv.matmul_stack(pv.from_i64(A), pv.from_i64(B), num, M, N, P).host()
+        assert pv.lib.zkp_last_matmul_path() == path
+        want = [int(v) % R_MOD for i in range(num) for v in (A[i].astype(object) @ B[i].astype(object)).reshape(-1)]
+        assert fr_ints(got) == want
+    Af = mt_random_vec(np.random.RandomState(1), num * 9 * 20)
+    Bf = mt_random_vec(np.random.RandomState(2), num * 20 * 7)
+    got = pv.matmul_stack(pv.from_fr(Af), pv.from_fr(Bf), num, 9, 20, 7).host()
+    assert pv.lib.zkp_last_matmul_path() == 1
+    Ai, Bi = np.array(fr_ints(Af), dtype=object).reshape(num, 9, 20), np.array(fr_ints(Bf), dtype=object).reshape(num, 20, 7)
+    assert fr_ints(got) == [int(v) % R_MOD for i in range(num) for v in (Ai[i] @ Bi[i]).reshape(-1)]
+    T = rng.integers(-2 ** 40, 2 ** 40, (5, 37, 70)).astype(np.int64)
+    got = pv.transpose_stack(pv.from_i64(T), 5, 37, 70).host()
+    assert fr_ints(got) == [int(v) % R_MOD for v in T.transpose(0, 2, 1).reshape(-1)]

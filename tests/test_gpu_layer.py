@@ -16,10 +16,10 @@ def pv():
     return Prover()
 
 
-@pytest.mark.parametrize("open_weights,seed", [(True, 3), (False, 4)])
-def test_tiny_layer_transcript(pv, open_weights, seed):
+@pytest.mark.parametrize("open_weights,seed,head_group", [(True, 3, 0), (False, 4, 0), (False, 5, 2), (True, 6, 1)])
+def test_tiny_layer_transcript(pv, open_weights, seed, head_group):
     orc = load_oracle()
-    cu, cf = layercfg.tiny(open_weights=open_weights)
+    cu, cf = layercfg.tiny(open_weights=open_weights, head_group=head_group)
     ws = layercfg.tiny_weights(seed, cu)
     S, E = int(cu[0]), int(cu[1])
     X = np.round(np.random.default_rng(seed + 10).normal(0, 1, (S, E)) * 256).astype(np.int32)

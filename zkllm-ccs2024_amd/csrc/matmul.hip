@@ -114,6 +114,7 @@ __device__ __forceinline__ Fr dot_mont(const Fr (&a)[KT], const Fr (&b)[KT]) {
 __global__ void __launch_bounds__(TM * TN) k_matmul(Fr* __restrict__ C, const Fr* __restrict__ A, const Fr* __restrict__ B, uint32_t M, uint32_t N, uint32_t P) {
     __shared__ uint32_t As[8][TM][KT + 1];
     __shared__ uint32_t Bs[8][KT][TN];
+    A += (size_t)blockIdx.z * M * N; B += (size_t)blockIdx.z * N * P; C += (size_t)blockIdx.z * M * P;   // one product of a stack per grid plane
     const uint32_t tx = threadIdx.x % TN, ty = threadIdx.x / TN;
     const uint32_t row = blockIdx.y * TM + ty, col = blockIdx.x * TN + tx;
     Fr acc = big_zero<8>();
@@ -208,6 +209,7 @@ template <typename T> __global__ void __launch_bounds__(256) k_fr_to_int(T* __re
 template <typename T> __global__ void __launch_bounds__(256) k_matmul_int(Fr* __restrict__ C, const T* __restrict__ A, const T* __restrict__ B, uint32_t M, uint32_t N, uint32_t P) {
     __shared__ T As[16][64 + 1];
     __shared__ T Bs[16][64 + 1];
+    A += (size_t)blockIdx.z * M * N; B += (size_t)blockIdx.z * N * P; C += (size_t)blockIdx.z * M * P;   // one product of a stack per grid plane
     const uint32_t tx = threadIdx.x % 16, ty = threadIdx.x / 16;
     const uint32_t row0 = blockIdx.y * 64, col0 = blockIdx.x * 64;
     long long acc[4][4];
@@ -251,6 +253,7 @@ __global__ void __launch_bounds__(256) k_matmul_wide_narrow(Fr* __restrict__ C, 
     __shared__ int Alo[16][64 + 1];
     __shared__ int Ahi[16][64 + 1];
     __shared__ int Bs[16][64 + 1];
+    A += (size_t)blockIdx.z * M * N; B += (size_t)blockIdx.z * N * P; C += (size_t)blockIdx.z * M * P;
     const uint32_t tx = threadIdx.x % 16, ty = threadIdx.x / 16;
     const uint32_t row0 = blockIdx.y * 64, col0 = blockIdx.x * 64;
     long long lo[4][4], hi[4][4];
@@ -292,26 +295,26 @@ __global__ void __launch_bounds__(256) k_matmul_wide_narrow(Fr* __restrict__ C, 
             if (r < M && c < P) C[(size_t)r * P + c] = fr_from_i64(v);
         }
 }
-static int run_wide_narrow_path(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, hipStream_t st) {
-    const size_t na = (size_t)M * N, nb = (size_t)N * P;
+static int run_wide_narrow_path(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, hipStream_t st) {
+    const size_t na = (size_t)batch * M * N, nb = (size_t)batch * N * P;
     Scratch ai(na * sizeof(long long)), bi(nb * sizeof(int));
     if (ai.rc) return ai.rc;
     if (bi.rc) return bi.rc;
     hipLaunchKernelGGL(k_fr_to_int<long long>, dim3(cdiv(na, 256)), dim3(256), 0, st, ai.as<long long>(), (const Fr*)A, na);
     hipLaunchKernelGGL(k_fr_to_int<int>, dim3(cdiv(nb, 256)), dim3(256), 0, st, bi.as<int>(), (const Fr*)B, nb);
-    hipLaunchKernelGGL(k_matmul_wide_narrow, dim3(cdiv(P, 64), cdiv(M, 64)), dim3(256), 0, st, (Fr*)C, ai.as<long long>(), bi.as<int>(), M, N, P);
+    hipLaunchKernelGGL(k_matmul_wide_narrow, dim3(cdiv(P, 64), cdiv(M, 64), batch), dim3(256), 0, st, (Fr*)C, ai.as<long long>(), bi.as<int>(), M, N, P);
     ZK_LAUNCH_CHECK();
     return 0;
 }
 
-template <typename T> static int run_int_path(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, hipStream_t st) {
-    const size_t na = (size_t)M * N, nb = (size_t)N * P;
+template <typename T> static int run_int_path(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, hipStream_t st) {
+    const size_t na = (size_t)batch * M * N, nb = (size_t)batch * N * P;
     Scratch ai(na * sizeof(T)), bi(nb * sizeof(T));
     if (ai.rc) return ai.rc;
     if (bi.rc) return bi.rc;
     hipLaunchKernelGGL(k_fr_to_int<T>, dim3(cdiv(na, 256)), dim3(256), 0, st, ai.as<T>(), (const Fr*)A, na);
     hipLaunchKernelGGL(k_fr_to_int<T>, dim3(cdiv(nb, 256)), dim3(256), 0, st, bi.as<T>(), (const Fr*)B, nb);
-    hipLaunchKernelGGL(k_matmul_int<T>, dim3(cdiv(P, 64), cdiv(M, 64)), dim3(256), 0, st, (Fr*)C, ai.as<T>(), bi.as<T>(), M, N, P);
+    hipLaunchKernelGGL(k_matmul_int<T>, dim3(cdiv(P, 64), cdiv(M, 64), batch), dim3(256), 0, st, (Fr*)C, ai.as<T>(), bi.as<T>(), M, N, P);
     ZK_LAUNCH_CHECK();
     return 0;
 }
@@ -420,21 +423,25 @@ int zk_fr_matmul_generic(void* C, const void* A, const void* B, uint32_t M, uint
 // mode: 0 = choose (small-integer path when the device-side bound check allows it),
 //       1 = always generic Montgomery, 2 = require the small-integer path (error if not applicable).
 // path_used (optional, host): 1 generic, 2 small-integer.
-int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv) {
+// `batch` products of equally shaped matrices stored one after the other; the bound is taken over the whole stacks, so
+// one path serves every product of the call
+static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv) {
     hipStream_t st = (hipStream_t)stv;
-    if (M == 0 || P == 0) return 0;
+    if (batch == 0 || M == 0 || P == 0) return 0;
     ZK_ARG(N > 0, "zk_fr_matmul: inner dimension is 0");
     ZK_ARG(mode >= 0 && mode <= 2, "zk_fr_matmul: mode must be 0, 1 or 2");
+    ZK_ARG(batch <= 65535, "zk_fr_matmul: at most 65535 products per call");
+    ZK_ARG((size_t)batch * M < ((size_t)1 << 31), "zk_fr_matmul: too many rows in one call");
     bool small = false, fits32 = false, b_fits32 = false;
     unsigned long long ma_ = 0, mb_ = 0;
     if (mode != 1) {
         Scratch mx(3 * sizeof(unsigned long long));
         if (mx.rc) return mx.rc;
         ZK_HIP(hipMemsetAsync(mx.p, 0, 3 * sizeof(unsigned long long), st));
-        const size_t na = (size_t)M * N, nb = (size_t)N * P;
+        const size_t na = (size_t)batch * M * N, nb = (size_t)batch * N * P;
         hipLaunchKernelGGL(k_absmax, dim3(absmax_grid(na)), dim3(256), 0, st, mx.as<unsigned long long>(), (const Fr*)A, na);
         hipLaunchKernelGGL(k_absmax, dim3(absmax_grid(nb)), dim3(256), 0, st, mx.as<unsigned long long>() + 1, (const Fr*)B, nb);
-        hipLaunchKernelGGL(k_rowabs, dim3(M), dim3(256), 0, st, mx.as<unsigned long long>() + 2, (const Fr*)A, N);
+        hipLaunchKernelGGL(k_rowabs, dim3(batch * M), dim3(256), 0, st, mx.as<unsigned long long>() + 2, (const Fr*)A, N);
         ZK_LAUNCH_CHECK();
         void* stage = nullptr;
         int rc = staging(&stage, 24);
@@ -454,20 +461,36 @@ int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, 
     }
     if (!small) {
         if (path_used) *path_used = 1;
-        return zk_fr_matmul_generic(C, A, B, M, N, P, stv);
+        hipLaunchKernelGGL(k_matmul, dim3(cdiv(P, TN), cdiv(M, TM), batch), dim3(TM * TN), 0, st, (Fr*)C, (const Fr*)A, (const Fr*)B, M, N, P);
+        ZK_LAUNCH_CHECK();
+        return 0;
     }
     if (path_used) *path_used = 2;
     // large products go to the matrix cores as int8 digit planes; below ~4 G multiply-accumulates the conversions outweigh the gain
     // (ZKLLM_MATMUL_PLANES: log2 of that threshold, 0 = never)
     static const int planes_log2 = getenv("ZKLLM_MATMUL_PLANES") ? atoi(getenv("ZKLLM_MATMUL_PLANES")) : 32;
     if (planes_log2 > 0 && (unsigned long long)M * N * P >= (1ull << planes_log2)) {
-        bool done = false;
-        const int rc = run_int8_plane_path(C, A, B, M, N, P, ma_, mb_, st, &done);
-        if (rc || done) return rc;
+        bool all_done = true;
+        for (uint32_t i = 0; i < batch && all_done; ++i) {
+            bool done = false;
+            const int rc = run_int8_plane_path((Fr*)C + (size_t)i * M * P, (const Fr*)A + (size_t)i * M * N, (const Fr*)B + (size_t)i * N * P, M, N, P, ma_, mb_, st, &done);
+            if (rc) return rc;
+            if (!done) {
+                if (i) { set_error(ZK_ERR_ARG, "zk_fr_matmul: the int8-plane path applied to part of a stack only"); return ZK_ERR_ARG; }
+                all_done = false;
+            }
+        }
+        if (all_done) return 0;
     }
-    if (fits32) return run_int_path<int>(C, A, B, M, N, P, st);
-    if (b_fits32) return run_wide_narrow_path(C, A, B, M, N, P, st);
-    return run_int_path<long long>(C, A, B, M, N, P, st);
+    if (fits32) return run_int_path<int>(C, A, B, batch, M, N, P, st);
+    if (b_fits32) return run_wide_narrow_path(C, A, B, batch, M, N, P, st);
+    return run_int_path<long long>(C, A, B, batch, M, N, P, st);
+}
+int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv) {
+    return matmul_dispatch(C, A, B, 1, M, N, P, mode, path_used, stv);
+}
+int zk_fr_matmul_batched(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv) {
+    return matmul_dispatch(C, A, B, batch, M, N, P, mode, path_used, stv);
 }
 
 }  // extern "C"

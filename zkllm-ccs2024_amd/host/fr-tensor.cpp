@@ -377,8 +377,7 @@ void FrTensor::matmul_stack_into(FrTensor& out, const FrTensor& x, const FrTenso
     if ((size_t)x.size != (size_t)num * M * N || (size_t)y.size != (size_t)num * N * P || (size_t)out.size != (size_t)num * M * P)
         throw std::runtime_error("matmul: incompatible dimensions");
     int path = 0;
-    for (uint i = 0; i < num; ++i)
-        ZKC(zk_fr_matmul(out.gpu_data + (size_t)i * M * P, x.gpu_data + (size_t)i * M * N, y.gpu_data + (size_t)i * N * P, M, N, P, G().matmul_mode, &path, nullptr));
+    ZKC(zk_fr_matmul_batched(out.gpu_data, x.gpu_data, y.gpu_data, num, M, N, P, G().matmul_mode, &path, nullptr));
     G().last_matmul_path = path;
 }
 

@@ -164,6 +164,8 @@ void* zkp_fr_pad(void* a, const u32* shape, int ndim, const u32* pad_val) {
     ZKP_TRY Fr_t pv; memcpy(pv.val, pad_val, 32); return new FrTensor(FT(a).pad(std::vector<uint>(shape, shape + ndim), pv)); ZKP_END_PTR
 }
 void* zkp_fr_transpose(void* a, u32 M, u32 N) { ZKP_TRY return new FrTensor(FT(a).transpose(M, N)); ZKP_END_PTR }
+void* zkp_fr_matmul_stack(void* a, void* b, u32 num, u32 M, u32 N, u32 P) { ZKP_TRY return new FrTensor(FrTensor::matmul_stack(FT(a), FT(b), num, M, N, P)); ZKP_END_PTR }
+void* zkp_fr_transpose_stack(void* a, u32 num, u32 M, u32 N) { ZKP_TRY return new FrTensor(FT(a).transpose_stack(num, M, N)); ZKP_END_PTR }
 void* zkp_fr_matmul(void* a, void* b, u32 M, u32 N, u32 P) { ZKP_TRY return new FrTensor(FrTensor::matmul(FT(a), FT(b), M, N, P)); ZKP_END_PTR }
 
 // ---- protocols ------------------------------------------------------------------------------------------
@@ -407,7 +409,7 @@ int zkp_zkip_stacked(const u32* claim, void* A, void* B, u32 N, u32 D, const u32
 }
 
 // ---- whole decoder layer ------------------------------------------------------------------------------------------
-// cfg_u32: seq, embed, heads, hidden, sf_linear, sf_gate, sf_attn, softmax L, softmax M, swiglu_len, open_weights, K, bs[0..K)
+// cfg_u32: seq, embed, heads, hidden, sf_linear, sf_gate, sf_attn, softmax L, softmax M, swiglu_len, open_weights, K, bs[0..K), attn_head_group
 // cfg_f64: softmax_sf_in, swiglu_low, swiglu_in_scale, swiglu_out_scale, rms_eps, value_scale, thetas[0..K-L-M)
 static LayerConfig parse_cfg(const u32* cu, const double* cf) {
     LayerConfig c;
@@ -416,6 +418,7 @@ static LayerConfig parse_cfg(const u32* cu, const double* cf) {
     c.swiglu_len = cu[9]; c.open_weights = cu[10] != 0;
     const u32 K = cu[11];
     c.softmax_bs.assign(cu + 12, cu + 12 + K);
+    c.attn_head_group = cu[12 + K];
     c.softmax_sf_in = (unsigned long)cf[0]; c.swiglu_low = (int)cf[1]; c.swiglu_in_scale = cf[2]; c.swiglu_out_scale = cf[3]; c.rms_eps = cf[4]; c.value_scale = cf[5];
     c.softmax_thetas.assign(cf + 6, cf + 6 + (K - c.softmax_L - c.softmax_M));
     return c;

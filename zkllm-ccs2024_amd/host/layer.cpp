@@ -91,10 +91,48 @@ static FrTensor head_slice(const FrTensor& t, uint seq, uint embed, uint h, uint
     return rows.transpose(d, seq);                                // seq x d
 }
 
+// Attention proved g heads at a time with zkAttnStacked (zksoftmax.cu:289-320) on head-major stacks [head][seq][d].
+static FrTensor attn_stacked_heads(const LayerConfig& c, const FrTensor& Q_, const FrTensor& K_, const FrTensor& V_) {
+    const uint seq = c.seq_len, E = c.embed_dim, H = c.num_heads, d = E / H, g = c.attn_head_group;
+    if (H % g) throw std::runtime_error("attn_head_group must divide num_heads");
+    // seq x embed -> embed x seq = [head][d][seq] -> [head][seq][d]
+    auto to_stack = [&](const FrTensor& t) { return t.transpose(seq, E).transpose_stack(H, d, seq); };
+    FrTensor Qs = to_stack(Q_), Ks = to_stack(K_), Vs = to_stack(V_);
+    FrTensor outs(H * seq * d);
+    zkAttnStacked attn(g, c.softmax_sf_in, 1UL, c.softmax_bs, c.softmax_L, c.softmax_M, c.softmax_thetas, seq, seq, d, 1);
+    const uint per = g * seq * d;
+    for (uint h0 = 0; h0 < H; h0 += g) {
+        const uint b = (h0 / g) * per;
+        std::unique_ptr<FrTensor> Qg, Kg, Vg;
+        if (g != H) { Qg.reset(new FrTensor(Qs.trunc(b, b + per))); Kg.reset(new FrTensor(Ks.trunc(b, b + per))); Vg.reset(new FrTensor(Vs.trunc(b, b + per))); }
+        const FrTensor &Q = g != H ? *Qg : Qs, &K = g != H ? *Kg : Ks, &V = g != H ? *Vg : Vs;
+        FrTensor sm_in(g * seq * seq), sm_out(g * seq * seq), shift(g * seq), shifted(g * seq * seq);
+        vector<FrTensor> in_seg, out_seg, m_seg;
+        FrTensor out = attn.compute(Q, K, V, sm_in, sm_out, shift, shifted, in_seg, out_seg, m_seg);
+        ZKC(zk_memcpy_d2d(outs.gpu_data + b, out.gpu_data, sizeof(Fr_t) * (size_t)per, nullptr));
+        auto ch = attn.draw();
+        vector<Polynomial> proof;
+        attn.prove(Q, K, V, out, sm_out, sm_in, shift, shifted, in_seg, out_seg, m_seg, ch.u_matmul_out_num, ch.v_matmul_out_num, ch.u_matmul_out, ch.v_matmul_out,
+                   ch.w_matmul_out, ch.v_sm, ch.temp_rand[0], ch.temp_rand[1], ch.temp_rand[2], ch.v_matmul_in_num, ch.v_matmul_in, proof);
+    }
+    return outs.transpose_stack(H, seq, d).transpose(E, seq);   // [head][d][seq] = embed x seq -> seq x embed
+}
+
 // Per-head attention following self-attn.cu:78-121 (attn mode) with d = head width.
 FrTensor attn_heads_block(const LayerConfig& c, const FrTensor& Q_, const FrTensor& K_, const FrTensor& V_) {
     const uint seq = c.seq_len, E = c.embed_dim, H = c.num_heads, d = E / H;
     if (E % H) throw std::runtime_error("embed_dim must be a multiple of num_heads");
+    if (c.attn_head_group) {
+        FrTensor out_all = attn_stacked_heads(c, Q_, K_, V_);
+        Rescaling rs1(c.sf_attn), rs2(c.sf_attn);
+        auto out_ = rs2(out_all);
+        auto out__ = rs1(out_);
+        auto p1 = rs1.prove_begin(out_, out__);
+        auto p2 = rs2.prove_begin(out_all, out_);
+        rs1.prove_end(p1);
+        rs2.prove_end(p2);
+        return out__;
+    }
     FrTensor QT = Q_.transpose(seq, E), KT = K_.transpose(seq, E), VT = V_.transpose(seq, E);   // embed x seq each
     FrTensor outT(E * seq);                                                                   // embed x seq, head outputs stacked by rows
     zkSoftmax softmax(c.softmax_bs, c.softmax_L, c.softmax_M, c.softmax_sf_in, c.softmax_thetas, seq, seq, d, 1);

@@ -7,7 +7,9 @@
 //  * attention is proved per head (the reference's `attn` mode treats the whole embedding as one head and
 //    never writes its output, so its pipeline cannot chain): for each head, X = Q_h K_h^T, zkSoftmax,
 //    out_h = Y V_h, the two inner-product sumchecks and the softmax proof; the heads' outputs are
-//    concatenated and rescaled twice as one tensor (a per-head 2^20 table would exceed the head's size);
+//    concatenated and rescaled twice as one tensor (a per-head 2^20 table would exceed the head's size).
+//    With attn_head_group = g the same statement is proved g heads at a time with the reference's
+//    zkAttnStacked (one softmax proof over g * seq rows, two stacked inner-product sumchecks);
 //  * an output projection (zkFC + rescaling + weight opening) follows, which the reference lacks;
 //  * challenges that the reference draws inside function-argument lists (unspecified order in C++) are
 //    drawn into named variables, first argument first;
@@ -36,6 +38,8 @@ struct LayerConfig {
     double rms_eps = 1e-5;        // LLaMa-2's variance_epsilon
     double value_scale = 65536.0; // fixed-point scale of activations (llama-rmsnorm.py:36-38 uses 1 << 16)
     bool open_weights = true;     // run verifyWeightClaim for every weight claim
+    uint attn_head_group = 0;     // 0: every head proved on its own (the flow of self-attn.cu:78-121 per head); g > 0 (a divisor of
+                                  // num_heads): heads proved g at a time as head-major stacks with zkAttnStacked (zksoftmax.cu:289-320)
 };
 
 struct LayerWeights {

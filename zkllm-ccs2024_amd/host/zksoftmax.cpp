@@ -237,23 +237,32 @@ Fr_t zkAttnStacked::prove(const FrTensor& Q, const FrTensor& K, const FrTensor& 
                           const vector<FrTensor>& sm_m_segments, const vector<Fr_t>& u_matmul_out_num, const vector<Fr_t>& v_matmul_out_num,
                           const vector<Fr_t>& u_matmul_out, const vector<Fr_t>& v_matmul_out, const vector<Fr_t>& w_matmul_out, const vector<Fr_t>& v_sm, const Fr_t& r_seg,
                           const Fr_t& alpha_seg, const Fr_t& beta_seg, const vector<Fr_t>& v_matmul_in_num, const vector<Fr_t>& v_matmul_in, vector<Polynomial>& proof) {
+    if (sm_in.size != sm_out.size) throw std::invalid_argument("X and Y must have the same size " + to_string(sm_in.size) + " " + to_string(sm_out.size));
+    // The softmax proof's sumcheck jobs need only tensors of the forward pass and challenges, so they are queued first and
+    // run on the library's side streams beside the proof of out = Y V; values are recorded in the reference's order.  (Jobs left
+    // unfinished by an exception are waited for and dropped by the pending object.)
+    const auto u_Y = concatenate<Fr_t>({v_matmul_out, u_matmul_out, v_matmul_out_num});
+    Pending pending = jobs_begin(sm_in_segments, sm_out_segments, sm_m_segments, u_Y, v_sm, r_seg, alpha_seg, beta_seg);
     auto out_claim = out.multi_dim_me({u_matmul_out_num, u_matmul_out, w_matmul_out}, {num, m, d});
     zk_record(out_claim);
     auto sm_out_reduced = sm_out.partial_me(u_matmul_out, m, n);
     auto V_reduced = V.partial_me(w_matmul_out, d, 1);
     auto out_matmul_claim = zkip_stacked(out_claim, sm_out_reduced, V_reduced, u_matmul_out_num, v_matmul_out, v_matmul_out_num, num, n, proof);
 
-    auto V_claim = V.multi_dim_me({v_matmul_out_num, v_matmul_out, w_matmul_out}, {num, n, d});
-    auto sm_out_claim = sm_out.multi_dim_me({v_matmul_out_num, u_matmul_out, v_matmul_out}, {num, m, n});
+    // V and sm_out at (v_num, ., v_matmul_out, .) follow from the reduced tensors [num][n]: fold n, then num
+    auto V_claim = V_reduced.multi_dim_me({v_matmul_out_num, v_matmul_out}, {num, n});
+    auto sm_out_claim = sm_out_reduced.multi_dim_me({v_matmul_out_num, v_matmul_out}, {num, n});
     if (out_matmul_claim != V_claim * sm_out_claim) throw std::runtime_error("out_matmul_claim is not correct");
 
-    auto sm_in_claim = zkSoftmax::prove(sm_out, sm_in, sm_shift, sm_in_shifted, sm_in_segments, sm_out_segments, sm_m_segments,
-                                        concatenate<Fr_t>({v_matmul_out, u_matmul_out, v_matmul_out_num}), v_sm, r_seg, alpha_seg, beta_seg, proof);
+    // zkSoftmax::prove opens with sm_out(u_Y) (zksoftmax.cu:187); u_Y is (v_matmul_out, u_matmul_out, v_matmul_out_num), so that is sm_out_claim
+    zk_record(sm_out_claim);
+    pending.had.claim = sm_out_claim;
 
     vector<Fr_t> u_matmul_in_num(v_sm.end() - ceilLog2(num), v_sm.end());
     vector<Fr_t> u_matmul_in(v_sm.end() - ceilLog2(num) - ceilLog2(m), v_sm.end() - ceilLog2(num));
     vector<Fr_t> w_matmul_in(v_sm.begin(), v_sm.end() - ceilLog2(num) - ceilLog2(m));
     auto Q_reduced = Q.partial_me(u_matmul_in, m, d);
     auto K_reduced = K.partial_me(w_matmul_in, n, d);
+    auto sm_in_claim = prove_end(pending, sm_in, sm_shift, sm_in_segments, sm_out_segments, v_sm, proof);
     return zkip_stacked(sm_in_claim, Q_reduced, K_reduced, u_matmul_in_num, v_matmul_in, v_matmul_in_num, num, d, proof);
 }
