@@ -191,6 +191,10 @@ int zk_lookup_prove_begin(void** handle, const void* S, const void* T, const voi
  * holds, 1/(S[i]+beta) is read from B instead of being computed, and a query that does not match is inverted on its own. */
 int zk_lookup_prove_begin_hinted(void** handle, const void* S, const void* T, const void* m, const void* hint_fr, int32_t low, const uint32_t* beta, const uint32_t* u_eq,
                                  const uint32_t* v, size_t D, size_t N, int rounds, void* stream);
+/* the combined lookup of a mapping table (tLookupRangeMapping::prove, tlookup.cu:517-551): query i = S_in[i] + r * S_out[i], expected at
+ * T[S_in[i] - low], T = table + r * mapped values; the combined queries are formed inside the first round instead of being written out */
+int zk_lookup_prove_begin_mapped(void** handle, const void* S_in, const void* S_out, const uint32_t* r, const void* T, const void* m, int32_t low, const uint32_t* beta,
+                                 const uint32_t* u_eq, const uint32_t* v, size_t D, size_t N, int rounds, void* stream);
 int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host);
 /* hadamard_product_sumcheck (Fr_hp_sc, proof.cu:66-109): adjacent-pair folding, first challenge first.  a, b: n elements,
  * 2^(k-1) < n <= 2^k; u, v: k challenges each.  proof_host: 3k + 2 values (per round the three terms evaluated at the

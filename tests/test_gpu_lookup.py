@@ -118,7 +118,7 @@ def test_range_lookup_proof_transcript(pv, orc, D, low, length):
     assert t.shape == e_t.shape and (t == e_t).all()
 
 
-@pytest.mark.parametrize("D,low,length", [(6, -2, 4), (64, -8, 16), (1000, -16, 32)])
+@pytest.mark.parametrize("D,low,length", [(6, -2, 4), (64, -8, 16), (1000, -16, 32), (1 << 17, -16, 32)])
 def test_mapping_lookup(pv, orc, D, low, length):
     rng = np.random.default_rng(D)
     vals = rng.integers(low, low + length, D)
@@ -309,4 +309,49 @@ def test_hinted_lookup_job_equals_the_plain_one_whatever_the_hints(k):
     assert (res[0][0] == res[1][0]).all() and (res[0][1] == res[1][1]).all()
     assert res[0][1].any()
     for p in (dS, dT, dm, dh):
+        hip.free(p)
+
+
+@pytest.mark.parametrize("k", [13, 17])
+def test_mapped_lookup_job_equals_the_plain_one_on_the_combined_queries(k):
+    """zk_lookup_prove_begin_mapped forms S_in + r * S_out itself (2^13 queries: written out first; 2^17: inside the first
+    round) and must deliver what zk_lookup_prove_begin delivers on the combined queries computed here with big integers,
+    also where an input is outside the table, an output is not the mapped value, or a combined query is -beta."""
+    import ctypes
+    from gpuhelp import Hip, c_void_p, c_size_t, c_int
+    hip = Hip()
+    D, N, low = 1 << k, 64, -9
+    rng = np.random.default_rng(k)
+    mapped = fr_ints(ch(51, N))
+    r_fr, beta = ch(52, 1)[0], ch(53, 1)[0]
+    r, b = fr_ints(r_fr.reshape(1, 8))[0], fr_ints(beta.reshape(1, 8))[0]
+    pos = rng.integers(0, N, D)
+    s_in = [(int(p) + low) % R_MOD for p in pos]
+    s_out = [mapped[int(p)] for p in pos]
+    odd = rng.choice(D, 200, replace=False)
+    for i in odd[:100]:
+        s_out[i] = (s_out[i] + 1 + int(i)) % R_MOD           # not the mapped value
+    for i in odd[100:199]:
+        s_in[i] = (low + N + 3 + int(i)) % R_MOD             # outside the table
+    i0 = int(odd[199])
+    s_out[i0] = ((-b - s_in[i0]) * pow(r, -1, R_MOD)) % R_MOD    # combined query + beta == 0
+    T = fr_array([((low + j) + r * mapped[j]) % R_MOD for j in range(N)])
+    S_com = fr_array([(a + r * o) % R_MOD for a, o in zip(s_in, s_out)])
+    m = fr_array([int(c) for c in np.bincount(pos, minlength=N)])
+    u, v = ch(54, k - 1), ch(55, k)
+    dS, dT, dm, dSi, dSo = hip.upload(S_com), hip.upload(T), hip.upload(m), hip.upload(fr_array(s_in)), hip.upload(fr_array(s_out))
+    res = []
+    for mapped_job in (False, True):
+        h = c_void_p()
+        if mapped_job:
+            hip.call("zk_lookup_prove_begin_mapped", ctypes.byref(h), c_void_p(dSi), c_void_p(dSo), r_fr, c_void_p(dT), c_void_p(dm), c_int(low), beta, u, v,
+                     c_size_t(D), c_size_t(N), c_int(k), None)
+        else:
+            hip.call("zk_lookup_prove_begin", ctypes.byref(h), c_void_p(dS), c_void_p(dT), c_void_p(dm), beta, u, v, c_size_t(D), c_size_t(N), c_int(k), None)
+        bm, sums = np.zeros(8, np.uint32), np.zeros((k * 11, 8), np.uint32)
+        hip.call("zk_lookup_prove_end", h, bm, sums)
+        res.append((bm, sums))
+    assert (res[0][0] == res[1][0]).all() and (res[0][1] == res[1][1]).all()
+    assert res[0][1].any()
+    for p in (dS, dT, dm, dSi, dSo):
         hip.free(p)

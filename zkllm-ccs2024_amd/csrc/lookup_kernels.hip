@@ -321,7 +321,12 @@ template <int K> __global__ void __launch_bounds__(TPB) k_me_multi(Fr* __restric
 // j = hint[i] - low, the inverse is B[j] = 1 / (T[j] + beta), already computed for the table -- one gather instead of a
 // share of a batch inversion over all D queries.  Whatever the hint, the result is the inverse itself: a query that
 // does not match its hinted entry (a hint outside the table, inconsistent inputs) is inverted on its own.
-struct HintSrc { const Fr* T; const Fr* B; const Fr* hint; Fr low; Fr beta; uint32_t N; };
+// S_out != nullptr: the queries themselves are not stored; query i is hint[i] + r * S_out[i] (a mapping table's combined
+// query, r_mont = r in Montgomery form) and is formed where it is needed.
+struct HintSrc { const Fr* T; const Fr* B; const Fr* hint; Fr low; Fr beta; uint32_t N; const Fr* S_out = nullptr; Fr r_mont; };
+__device__ __forceinline__ Fr hinted_query(const Fr* __restrict__ S, size_t i, const HintSrc& h) {
+    return h.S_out ? add(h.hint[i], mont_mul(h.r_mont, h.S_out[i])) : S[i];
+}
 static __device__ __attribute__((noinline)) Fr inv_plus_beta_alone(const Fr& sv, const Fr& beta) {
     const Fr v = add(sv, beta);
     if (is_zero(v)) return big_zero<8>();
@@ -343,6 +348,11 @@ __global__ void __launch_bounds__(TPB) k_inv_by_hint(Fr* __restrict__ A, const F
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (i < D) A[i] = inv_by_hint(S[i], i, h);
 }
+// out = a + r * b (the combined queries of a mapping table written out, for jobs too small for the fused first round)
+__global__ void __launch_bounds__(TPB) k_combine_queries(Fr* __restrict__ out, const Fr* __restrict__ a, const Fr* __restrict__ b, const Fr r_mont, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) out[i] = add(a[i], mont_mul(r_mont, b[i]));
+}
 
 // ---- lookup sumcheck round --------------------------------------------------------------------------------------------------
 // Over halves (t, t + n_out):  a0 = A[t], da = A[t+n_out]-A[t], s0 = S[t]+beta, ds = S[t+n_out]-S[t]
@@ -363,7 +373,7 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
         const Fr e = E[t];
         if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table: the top variable summed out
         {
-            const Fr s0r = S[t], s1 = S[t + n_out];
+            const Fr s0r = HINTED ? hinted_query(S, t, hs) : S[t], s1 = HINTED ? hinted_query(S, t + n_out, hs) : S[t + n_out];
             const Fr a0 = HINTED ? inv_by_hint(s0r, t, hs) : A[t], a1 = HINTED ? inv_by_hint(s1, t + n_out, hs) : A[t + n_out];
             const Fr da = sub(a1, a0), ds = sub(s1, s0r), s0 = add(s0r, beta);
             acc[0] = add(acc[0], mont_mul(e, mont_mul(a0, s0)));
@@ -977,6 +987,13 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
     if (!A) {
         ZK_ARG(hs != nullptr, "lookup sumcheck: neither A nor a hint");
         fuse_first = D > N && (D >> 1) > (size_t)SPLIT_HALF;       // a phase-1 round that the full-size kernel takes
+        if (!fuse_first && hs->S_out) {
+            Scratch& Sbuf = job.arena.add(sizeof(Fr) * D);
+            if (Sbuf.rc) return Sbuf.rc;
+            hipLaunchKernelGGL(k_combine_queries, dim3(cdiv(D, TPB)), dim3(TPB), 0, st, Sbuf.as<Fr>(), hs->hint, hs->S_out, hs->r_mont, D);
+            ZK_LAUNCH_CHECK();
+            S = Sbuf.as<Fr>();
+        }
         if (!fuse_first) {
             Scratch& Abuf = job.arena.add(sizeof(Fr) * D);
             if (Abuf.rc) return Abuf.rc;
@@ -1213,7 +1230,7 @@ int zk_lookup_sumcheck(uint32_t* sums_host, const void* A, const void* S, const 
 // begin returns at once; S, T, m must stay alive and unmodified until end, which waits and delivers <B, m>
 // (standard form) and the rounds x 11 sums.  Every handle must be ended exactly once.
 static int lookup_prove_begin(void** handle, const void* S, const void* T, const void* m, const void* hint, int32_t low, const uint32_t* beta, const uint32_t* u_eq,
-                              const uint32_t* v, size_t D, size_t N, int rounds, void* stv) {
+                              const uint32_t* v, size_t D, size_t N, int rounds, void* stv, const void* S_out = nullptr, const uint32_t* r = nullptr) {
     ZK_ARG(handle != nullptr, "zk_lookup_prove_begin: null handle");
     int rc = lookup_args_ok(D, N, rounds);
     if (rc) return rc;
@@ -1231,6 +1248,7 @@ static int lookup_prove_begin(void** handle, const void* S, const void* T, const
     HintSrc hs;
     if (rc == 0 && hint) {
         hs.T = (const Fr*)T; hs.B = B.as<Fr>(); hs.hint = (const Fr*)hint; hs.low = fr_from_i64((int64_t)low); hs.beta = b; hs.N = (uint32_t)N;
+        if (S_out) { hs.S_out = (const Fr*)S_out; hs.r_mont = to_mont(load_fr(r)); }
     } else if (rc == 0) {
         Scratch& A = job->arena.add(sizeof(Fr) * D);
         rc = A.rc;
@@ -1261,6 +1279,14 @@ int zk_lookup_prove_begin_hinted(void** handle, const void* S, const void* T, co
                                  const uint32_t* v, size_t D, size_t N, int rounds, void* stv) {
     ZK_ARG(hint != nullptr, "zk_lookup_prove_begin_hinted: null hint");
     return lookup_prove_begin(handle, S, T, m, hint, low, beta, u_eq, v, D, N, rounds, stv);
+}
+// The same for a mapping table's combined lookup (tlookup.cu:517-518): query i is S_in[i] + r * S_out[i], expected at
+// T[S_in[i] - low] with T the combined table.  The combined queries are never written out when the job is large enough for
+// its first round to form them on the fly.
+int zk_lookup_prove_begin_mapped(void** handle, const void* S_in, const void* S_out, const uint32_t* r, const void* T, const void* m, int32_t low, const uint32_t* beta,
+                                 const uint32_t* u_eq, const uint32_t* v, size_t D, size_t N, int rounds, void* stv) {
+    ZK_ARG(S_in != nullptr && S_out != nullptr && r != nullptr, "zk_lookup_prove_begin_mapped: null queries or challenge");
+    return lookup_prove_begin(handle, nullptr, T, m, S_in, low, beta, u_eq, v, D, N, rounds, stv, S_out, r);
 }
 int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host) {
     ZK_ARG(handle != nullptr, "zk_lookup_prove_end: null handle");

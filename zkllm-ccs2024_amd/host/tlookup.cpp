@@ -91,9 +91,17 @@ LookupPending& LookupPending::operator=(LookupPending&& o) noexcept {
 // tLookup_phase1 / tLookup_phase2 (tlookup.cu:184-320).  The device side -- inverses, <B, m>, eq table and every round --
 // is one job that runs beside the caller; the host side turns each round's sums into its polynomial, checks it and
 // derives the next claim.
+// S_out / r given: S0 holds the input queries of a mapping table, the combined query S0 + r * S_out is formed on the device
+static LookupPending sumcheck_begin(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0, const Fr_t& alpha0, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v,
+                                    const FrTensor* hint, int low, const FrTensor* S_out, const Fr_t* r);
 LookupPending tLookup_sumcheck_begin(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0, const Fr_t& alpha0, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v,
                                      const FrTensor* hint, int low) {
+    return sumcheck_begin(S0, T0, m0, alpha0, beta, u, v, hint, low, nullptr, nullptr);
+}
+static LookupPending sumcheck_begin(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0, const Fr_t& alpha0, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v,
+                                    const FrTensor* hint, int low, const FrTensor* S_out, const Fr_t* r) {
     const uint D = S0.size, N = m0.size;
+    if (S_out && S_out->size != D) throw std::runtime_error("lookup: input and output queries differ in size");
     if (m0.size != T0.size) throw std::runtime_error("m.size != table.size");
     if (D != (1u << ceilLog2(D)) || N != (1u << ceilLog2(N)) || D % N != 0) throw std::runtime_error("D or N is not power of 2, or D is not divisible by N");
     if (u.size() != ceilLog2(D)) throw std::runtime_error("u.size() != ceilLog2(D)");
@@ -107,7 +115,8 @@ LookupPending tLookup_sumcheck_begin(const FrTensor& S0, const FrTensor& T0, con
     std::vector<Fr_t> vs(k);
     for (uint r = 0; r < k; ++r) vs[r] = r >= n1 ? v[k - 1 - (r - n1)] : v[n1 - 1 - r];
     if (hint && hint->size != D) throw std::runtime_error("lookup hint must have one entry per query");
-    if (hint) ZKC(zk_lookup_prove_begin_hinted(&p.handle, S0.gpu_data, T0.gpu_data, m0.gpu_data, hint->gpu_data, low, beta.val, u[0].val, vs[0].val, D, N, (int)k, nullptr));
+    if (S_out) ZKC(zk_lookup_prove_begin_mapped(&p.handle, S0.gpu_data, S_out->gpu_data, r->val, T0.gpu_data, m0.gpu_data, low, beta.val, u[0].val, vs[0].val, D, N, (int)k, nullptr));
+    else if (hint) ZKC(zk_lookup_prove_begin_hinted(&p.handle, S0.gpu_data, T0.gpu_data, m0.gpu_data, hint->gpu_data, low, beta.val, u[0].val, vs[0].val, D, N, (int)k, nullptr));
     else ZKC(zk_lookup_prove_begin(&p.handle, S0.gpu_data, T0.gpu_data, m0.gpu_data, beta.val, u[0].val, vs[0].val, D, N, (int)k, nullptr));
     return p;
 }
@@ -198,11 +207,10 @@ LookupPending tLookupRangeMapping::prove_begin(const FrTensor& S_in, const FrTen
     }
     const uint N = mm->size;
     if (N != (1u << ceilLog2(N)) || si->size % N != 0) throw std::runtime_error("N is not power of 2, or D is not divisible by N");
-    keep.emplace_back(new FrTensor(*si + *so * r));
-    const FrTensor* S_com = keep.back().get();
+    // S_com = S_in + r * S_out (tlookup.cu:517) is formed by the job itself; T_com is small
     keep.emplace_back(new FrTensor(table + mapped_vals * r));
     const FrTensor* T_com = keep.back().get();
-    LookupPending p = tLookup_sumcheck_begin(*S_com, *T_com, *mm, alpha, beta, u, v, si, low);
+    LookupPending p = sumcheck_begin(*si, *T_com, *mm, alpha, beta, u, v, si, low, so, &r);
     p.keep = std::move(keep);
     return p;
 }
