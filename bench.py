@@ -40,8 +40,9 @@ def main():
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--seq", type=int, default=2048)
-    ap.add_argument("--head-group", type=int, default=0,
-                    help="attention proved this many heads at a time with zkAttnStacked (a divisor of 32); 0 = head by head")
+    ap.add_argument("--head-group", type=int, default=32,
+                    help="attention proved this many heads at a time with zkAttnStacked (a divisor of 32; default: all 32 as one stack); "
+                         "0 = head by head, the flow of self-attn.cu per head")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extras", action="store_true", help="only the layer timing (used for profiling runs)")
     ap.add_argument("--pmc-probe", action="store_true",
@@ -130,6 +131,9 @@ def main():
         os.dup2(saved_stdout, 1)
     ms_per_step = wall * 1e3 / args.steps
     parts /= args.steps
+    live_b, cached_b = ctypes.c_size_t(), ctypes.c_size_t()
+    hip.check(lib.zk_pool_stats(ctypes.byref(live_b), ctypes.byref(cached_b)))
+    pool_gib = (live_b.value + cached_b.value) / 2 ** 30      # the allocator keeps what it once needed: live + cached = the layer's peak
     pv.layer_free(layer)
     lib.zk_pool_trim()
 
@@ -147,7 +151,9 @@ def main():
         "dtype": "u32",
         "data": "synthetic",
         "config": {"workload": f"C5: LLaMa-2-7B-shape decoder layer proof, seq {seq}, hidden 4096, 32 heads x 128, FFN 11008, "
-                               "random-init fixed-point weights (scale 2^16), generators of size out_features<<5, all nine weight openings included",
+                               "random-init fixed-point weights (scale 2^16), generators of size out_features<<5, all nine weight openings included; attention proved "
+                               + (f"{args.head_group} heads at a time as head-major stacks (zkAttnStacked)" if args.head_group else "head by head"),
+                   "device_pool_gib": round(pool_gib, 1),
                    "setup_s_untimed": round(setup_s, 3),
                    "parts_ms": {k: round(float(v), 1) for k, v in zip(["rmsnorm1", "qkv", "attention", "oproj", "rmsnorm2", "ffn", "total", "open_wait"], parts)}},
     }
