@@ -400,6 +400,12 @@ class Prover:
         out = self.H(self.lib.zkp_layer_run(c_void_p(layer), c_void_p(X.h), _np_ptr(times)))
         return out, times
 
+    def layer_set(self, layer, head_group=None, open_weights=None):
+        if head_group is not None:
+            self.lib.zkp_layer_set_head_group(c_void_p(layer), c_uint(head_group))
+        if open_weights is not None:
+            self.lib.zkp_layer_set_open_weights(c_void_p(layer), c_int(1 if open_weights else 0))
+
     def layer_free(self, layer):
         self.lib.zkp_layer_free(c_void_p(layer))
 

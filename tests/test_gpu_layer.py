@@ -38,3 +38,27 @@ def test_tiny_layer_transcript(pv, open_weights, seed, head_group):
     assert (out.host() == exp).all()
     assert got_t.shape == exp_t.shape and (got_t == exp_t).all()
     assert times[6] > 0
+
+
+def test_full_shape_layer_gives_one_output_head_by_head_and_stacked(pv):
+    """LLaMa-2-7B shape, seq 2048 (tensors of up to 2^27 elements in the stacked proof, beyond what the oracle can follow):
+    every proof of the layer runs through its in-prover identities in both attention variants (a failed identity throws),
+    the two variants and a group size in between give the same layer output, and the transcripts differ only in length."""
+    cu, cf = layercfg.llama7b(seq=2048, open_weights=False)
+    pv.seed(2024)
+    layer = pv.layer_create_random(cu, cf, 7, 5)
+    X = pv.from_i32(np.round(np.random.default_rng(11).normal(0, 1, (2048, 4096)) * 65536).astype(np.int32))
+    outs, sizes = [], []
+    for g in (0, 32, 8):
+        pv.layer_set(layer, head_group=g)
+        pv.seed(5)
+        pv.transcript_begin()
+        out, _ = pv.layer_run(layer, X)
+        pv.lib.zkp_transcript_end()
+        sizes.append(pv.transcript().shape[0])
+        outs.append(out.host())
+        del out
+    pv.layer_free(layer)
+    assert (outs[0] == outs[1]).all() and (outs[0] == outs[2]).all()
+    assert np.unique(outs[0], axis=0).shape[0] > 1000
+    assert sizes[1] < sizes[2] < sizes[0]

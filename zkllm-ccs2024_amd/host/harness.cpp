@@ -451,6 +451,7 @@ void* zkp_layer_create_random(const u32* cu, const double* cf, u32 seed, u32 log
     ZKP_END_PTR
 }
 void zkp_layer_free(void* h) { delete reinterpret_cast<LayerState*>(h); }
+void zkp_layer_set_head_group(void* h, u32 g) { reinterpret_cast<LayerState*>(h)->cfg.attn_head_group = g; }
 void zkp_layer_set_open_weights(void* h, int on) { reinterpret_cast<LayerState*>(h)->cfg.open_weights = on != 0; }
 // runs the whole layer (compute + every proof); times_ms (8 values): rmsnorm1, qkv, attention, oproj, rmsnorm2, ffn, total, open_wait
 void* zkp_layer_run(void* h, void* X, double* times_ms) {
