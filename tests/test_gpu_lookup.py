@@ -275,7 +275,8 @@ def test_stacked_fully_connected_proof(pv, orc, num, batch, n_in, n_out, bias):
 def test_hinted_lookup_job_equals_the_plain_one_whatever_the_hints(k):
     """zk_lookup_prove_begin_hinted reads 1/(S+beta) from the table's inverses where the hinted entry matches and must
     deliver what zk_lookup_prove_begin delivers for every input: right hints, wrong hints, hints outside the table,
-    queries that are no table entry at all, and a query with S + beta == 0.  2^13 queries: the inverses are written out
+    queries that are no table entry at all, a query with S + beta == 0 and a table entry with T + beta == 0 (pairs of
+    matched invertible entries take a shortcut through (a0 + a1)(s0 + s1); every other pair must not).  2^13 queries: the inverses are written out
     before the first round; 2^17: the first round computes them on the fly."""
     import ctypes
     from gpuhelp import Hip, c_void_p, c_size_t, c_int
@@ -283,6 +284,8 @@ def test_hinted_lookup_job_equals_the_plain_one_whatever_the_hints(k):
     D, N, low = 1 << k, 64, -7
     rng = np.random.default_rng(99)
     T = ch(41, N)                                   # arbitrary table entries
+    beta = ch(43, 1)[0]
+    T[3] = fr_array([(-fr_ints(beta.reshape(1, 8))[0]) % R_MOD])[0]     # a table entry with T + beta == 0: its "inverse" is 0, not a unit
     pos = rng.integers(0, N, D)
     S = T[pos].copy()
     hint_int = (pos + low).astype(np.int64)         # right hints: hint - low == position
@@ -290,7 +293,6 @@ def test_hinted_lookup_job_equals_the_plain_one_whatever_the_hints(k):
     hint_int[wrong[:100]] = (pos[wrong[:100]] + 1) % N + low          # another entry of the table
     hint_int[wrong[100:200]] = low + N + 5                            # outside the table
     S[wrong[200:]] = ch(42, 100)                                      # queries that are no table entries
-    beta = ch(43, 1)[0]
     S[wrong[7]] = fr_array([(-fr_ints(beta.reshape(1, 8))[0]) % R_MOD])[0]
     hint = fr_array([int(x) % R_MOD for x in hint_int])
     m = fr_array([int(c) for c in np.bincount(pos, minlength=N)])

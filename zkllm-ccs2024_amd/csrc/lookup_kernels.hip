@@ -337,11 +337,17 @@ static __device__ __attribute__((noinline)) Fr inv_plus_beta_alone(const Fr& sv,
     for (int l = 0; l < 8; ++l) k.v[l] = RINV[l];
     return mont_mul(mont_inverse(v), k);
 }
-__device__ __forceinline__ Fr inv_by_hint(const Fr& sv, size_t i, const HintSrc& h) {
+// *unit (optional): the returned a satisfies a * (sv + beta) == 1 by construction (the hinted entry matched and is invertible)
+__device__ __forceinline__ Fr inv_by_hint(const Fr& sv, size_t i, const HintSrc& h, bool* unit = nullptr) {
     const Fr d = sub(h.hint[i], h.low);
     const bool in_table = !(d.v[1] | d.v[2] | d.v[3] | d.v[4] | d.v[5] | d.v[6] | d.v[7]) && d.v[0] < h.N;
     const uint32_t j = in_table ? d.v[0] : 0u;
-    if (equal(sv, h.T[j])) return h.B[j];
+    if (equal(sv, h.T[j])) {
+        const Fr b = h.B[j];
+        if (unit) *unit = !is_zero(b);
+        return b;
+    }
+    if (unit) *unit = false;
     return inv_plus_beta_alone(sv, h.beta);
 }
 __global__ void __launch_bounds__(TPB) k_inv_by_hint(Fr* __restrict__ A, const Fr* __restrict__ S, const HintSrc h, size_t D) {
@@ -360,7 +366,9 @@ __global__ void __launch_bounds__(TPB) k_combine_queries(Fr* __restrict__ out, c
 //   sums 3..4 : sum a0, sum da
 // phase 2 adds the same three E-weighted sums for (B,T) as sums 5..7 and the plain products of (m,B)
 // as sums 8..10 (R^-1 attached), and folds all five tensors by v.
-// HINTED (first round of a job whose A was never written): a0, a1 come from inv_by_hint instead of A.
+// HINTED (first round of a job whose A was never written): a0, a1 come from inv_by_hint instead of A.  Where both are
+// inverses by construction (a0 s0 = a1 s1' = 1, s1' = S[t+n_out]+beta), the three E-weighted terms are 1, M - 4 and 4 - M
+// with M = (a0 + a1)(s0 + s1'): one product instead of five, and the constants go through the sum of E.
 template <bool PHASE2, bool HINTED = false> __global__ void __launch_bounds__(TPB)
 k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ nS, Fr* __restrict__ nB, Fr* __restrict__ nT, Fr* __restrict__ nm,
                const Fr* __restrict__ A, const Fr* __restrict__ S, const Fr* __restrict__ B, const Fr* __restrict__ T, const Fr* __restrict__ m,
@@ -369,16 +377,24 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
     Fr acc[K];
 #pragma unroll
     for (int i = 0; i < K; ++i) acc[i] = big_zero<8>();
+    Fr acc_e = big_zero<8>(), acc_em = big_zero<8>();       // HINTED: sum of E and of E * M over the pairs of unit inverses
     for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
         const Fr e = E[t];
         if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table: the top variable summed out
         {
             const Fr s0r = HINTED ? hinted_query(S, t, hs) : S[t], s1 = HINTED ? hinted_query(S, t + n_out, hs) : S[t + n_out];
-            const Fr a0 = HINTED ? inv_by_hint(s0r, t, hs) : A[t], a1 = HINTED ? inv_by_hint(s1, t + n_out, hs) : A[t + n_out];
+            bool unit0 = false, unit1 = false;
+            const Fr a0 = HINTED ? inv_by_hint(s0r, t, hs, &unit0) : A[t], a1 = HINTED ? inv_by_hint(s1, t + n_out, hs, &unit1) : A[t + n_out];
             const Fr da = sub(a1, a0), ds = sub(s1, s0r), s0 = add(s0r, beta);
-            acc[0] = add(acc[0], mont_mul(e, mont_mul(a0, s0)));
-            acc[1] = add(acc[1], mont_mul(e, add(mont_mul(da, s0), mont_mul(a0, ds))));
-            acc[2] = add(acc[2], mont_mul(e, mont_mul(da, ds)));
+            if (HINTED && unit0 && unit1) {
+                const Fr M = mont_mul(add(a0, a1), add(s0, add(s1, beta)));
+                acc_em = add(acc_em, mont_mul(e, M));
+                acc_e = add(acc_e, e);
+            } else {
+                acc[0] = add(acc[0], mont_mul(e, mont_mul(a0, s0)));
+                acc[1] = add(acc[1], mont_mul(e, add(mont_mul(da, s0), mont_mul(a0, ds))));
+                acc[2] = add(acc[2], mont_mul(e, mont_mul(da, ds)));
+            }
             acc[3] = add(acc[3], a0);
             acc[4] = add(acc[4], da);
             nA[t] = add(a0, mont_mul(v_mont, da));
@@ -397,6 +413,17 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
             nT[t] = add(t0r, mont_mul(v_mont, dt));
             nm[t] = add(m0, mont_mul(v_mont, dm));
         }
+    }
+    if (HINTED) {
+        // E is in Montgomery form and the sums carry R^-1: sum(E) * R^-2 through one product with R^-1
+        constexpr uint32_t RINV[8] = {4269129792u, 334977897u, 165441631u, 2876230287u, 1333208682u, 1912866698u, 805346647u, 465471123u};
+        Fr k;
+#pragma unroll
+        for (int l = 0; l < 8; ++l) k.v[l] = RINV[l];
+        const Fr one = mont_mul(acc_e, k), two = add(one, one), four = add(two, two);
+        acc[0] = add(acc[0], one);
+        acc[1] = add(acc[1], sub(acc_em, four));
+        acc[2] = add(acc[2], sub(four, acc_em));
     }
     block_reduce_store<K>(acc, partials);
 }
