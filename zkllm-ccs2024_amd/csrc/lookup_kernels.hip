@@ -464,30 +464,48 @@ k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __rest
     Fr acc[K + 1];
 #pragma unroll
     for (int i = 0; i <= K; ++i) acc[i] = big_zero<8>();
-    const Fr r2 = big_r2<8>();
     for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
-        Fr c[K + 1];   // running product polynomial, standard form
-        {
-            const Fr x0 = p.in[0][t], x1 = p.in[0][t + n_out];
-            const Fr dx = sub(x1, x0);
-            c[0] = x0; c[1] = dx;
+        // Coefficients of the running product from standard-form values: every coefficient is a sum of products of the same
+        // number of factors, so each Montgomery product leaves one more R^-1 on all of them alike (K - 1 in the end), which
+        // the lane's sums shed once after the loop instead of every value being converted before it is multiplied.
+        Fr c[K + 1];
+        if constexpr (K == 2) {
+            const Fr x0 = p.in[0][t], x1 = p.in[0][t + n_out], y0 = p.in[1][t], y1 = p.in[1][t + n_out];
+            const Fr dx = sub(x1, x0), dy = sub(y1, y0);
             p.out[0][t] = add(x0, mont_mul(v_mont, dx));
-        }
+            p.out[1][t] = add(y0, mont_mul(v_mont, dy));
+            c[0] = mont_mul(x0, y0);
+            c[2] = mont_mul(dx, dy);
+            c[1] = sub(sub(mont_mul(x1, y1), c[0]), c[2]);      // x0 dy + y0 dx = x1 y1 - x0 y0 - dx dy
+        } else {
+            {
+                const Fr x0 = p.in[0][t], x1 = p.in[0][t + n_out];
+                const Fr dx = sub(x1, x0);
+                c[0] = x0; c[1] = dx;
+                p.out[0][t] = add(x0, mont_mul(v_mont, dx));
+            }
 #pragma unroll
-        for (int k = 1; k < K; ++k) {
-            const Fr x0 = p.in[k][t], x1 = p.in[k][t + n_out];
-            const Fr dx = sub(x1, x0);
-            p.out[k][t] = add(x0, mont_mul(v_mont, dx));
-            const Fr x0m = mont_mul(x0, r2), dxm = mont_mul(dx, r2);    // Montgomery form so products stay standard
-            c[k + 1] = mont_mul(c[k], dxm);
+            for (int k = 1; k < K; ++k) {
+                const Fr x0 = p.in[k][t], x1 = p.in[k][t + n_out];
+                const Fr dx = sub(x1, x0);
+                p.out[k][t] = add(x0, mont_mul(v_mont, dx));
+                c[k + 1] = mont_mul(c[k], dx);
 #pragma unroll
-            for (int j = k; j >= 1; --j) c[j] = add(mont_mul(c[j], x0m), mont_mul(c[j - 1], dxm));
-            c[0] = mont_mul(c[0], x0m);
+                for (int j = k; j >= 1; --j) c[j] = add(mont_mul(c[j], x0), mont_mul(c[j - 1], dx));
+                c[0] = mont_mul(c[0], x0);
+            }
         }
         const Fr e = E[t];   // Montgomery form: e*R
         if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table
 #pragma unroll
         for (int j = 0; j <= K; ++j) acc[j] = add(acc[j], mont_mul(e, c[j]));
+    }
+    if (K > 1) {
+        const Fr r2 = big_r2<8>();
+#pragma unroll
+        for (int j = 0; j <= K; ++j)
+#pragma unroll
+            for (int f = 1; f < K; ++f) acc[j] = mont_mul(acc[j], r2);
     }
     block_reduce_store<K + 1>(acc, partials);
 }
