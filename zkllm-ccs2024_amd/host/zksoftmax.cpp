@@ -119,20 +119,34 @@ void zkSoftmax::claim_record(Pending& pending, const FrTensor& Y, const vector<F
 }
 
 Fr_t zkSoftmax::prove_end(Pending& pending, const FrTensor& X, const FrTensor& shift, const vector<FrTensor>& X_segments, const vector<FrTensor>& Y_segments,
-                          const vector<Fr_t>& v_Y, vector<Polynomial>& proof) {
-    std::string failure;
-    try { multi_hadamard_end(pending.had, proof); } catch (const std::exception& e) { failure = e.what(); }
-    for (auto& lp : pending.looks) {
-        try { tLookup::prove_end(lp); } catch (const std::exception& e) { if (failure.empty()) failure = e.what(); }
-    }
-    if (!failure.empty()) throw std::runtime_error(failure);
-
-    // all evaluations at v_Y in one pass over the tensors (zksoftmax.cu:189-196 evaluates them one by one)
+                          const vector<Fr_t>& v_Y, vector<Polynomial>& proof, bool evaluate_first) {
+    // all evaluations at v_Y in one pass over the tensors (zksoftmax.cu:189-196 evaluates them one by one).  They need
+    // nothing from the sumcheck jobs: with evaluate_first they run on the caller's stream while the jobs finish on theirs
+    // (worth it when the jobs are long, as for a stack of heads; beside short jobs the contention costs more than the
+    // wait); their values are recorded after the jobs' entries, where the reference computes them.
     vector<const FrTensor*> at_v;
     for (uint i = L; i < K; ++i) at_v.push_back(&Y_segments[i - L]);
     for (uint i = 0; i < K; ++i) at_v.push_back(&X_segments[i]);
     at_v.push_back(&X);
-    const vector<Fr_t> evals = FrTensor::me_batch(at_v, v_Y);
+    vector<Fr_t> evals;
+    Fr_t shift_const_opening;
+    std::string failure;
+    auto evaluate = [&]() {
+        try {
+            evals = FrTensor::me_batch(at_v, v_Y);
+            vector<Fr_t> v_Y_(v_Y.begin() + ceilLog2(n), v_Y.end());
+            shift_const_opening = shift(v_Y_);
+        } catch (const std::exception& e) { if (failure.empty()) failure = e.what(); }
+    };
+    if (evaluate_first) evaluate();
+
+    try { multi_hadamard_end(pending.had, proof); } catch (const std::exception& e) { if (failure.empty()) failure = e.what(); }
+    for (auto& lp : pending.looks) {
+        try { tLookup::prove_end(lp); } catch (const std::exception& e) { if (failure.empty()) failure = e.what(); }
+    }
+    if (!evaluate_first) evaluate();
+    if (!failure.empty()) throw std::runtime_error(failure);
+
     vector<Fr_t> Y_seg_claims(evals.begin(), evals.begin() + (K - L)), X_seg_claims(evals.begin() + (K - L), evals.begin() + (K - L) + K);
     zk_record(Y_seg_claims);
     zk_record(X_seg_claims);
@@ -140,8 +154,6 @@ Fr_t zkSoftmax::prove_end(Pending& pending, const FrTensor& X, const FrTensor& s
     Fr_t minus_X_shifted_claim = {0, 0, 0, 0, 0, 0, 0, 0};
     for (int i = (int)bs.size() - 1; i >= 0; --i) minus_X_shifted_claim = minus_X_shifted_claim * Fr_t({bs[i], 0, 0, 0, 0, 0, 0, 0}) + X_seg_claims[i];
 
-    vector<Fr_t> v_Y_(v_Y.begin() + ceilLog2(n), v_Y.end());
-    auto shift_const_opening = shift(v_Y_);
     auto X_opening = evals.back();
     zk_record(shift_const_opening);
     zk_record(X_opening);
@@ -263,6 +275,6 @@ Fr_t zkAttnStacked::prove(const FrTensor& Q, const FrTensor& K, const FrTensor& 
     vector<Fr_t> w_matmul_in(v_sm.begin(), v_sm.end() - ceilLog2(num) - ceilLog2(m));
     auto Q_reduced = Q.partial_me(u_matmul_in, m, d);
     auto K_reduced = K.partial_me(w_matmul_in, n, d);
-    auto sm_in_claim = prove_end(pending, sm_in, sm_shift, sm_in_segments, sm_out_segments, v_sm, proof);
+    auto sm_in_claim = prove_end(pending, sm_in, sm_shift, sm_in_segments, sm_out_segments, v_sm, proof, true);
     return zkip_stacked(sm_in_claim, Q_reduced, K_reduced, u_matmul_in_num, v_matmul_in, v_matmul_in_num, num, d, proof);
 }

@@ -28,7 +28,7 @@ class zkSoftmax {
                        const vector<Fr_t>& v_Y, const Fr_t& r_seg, const Fr_t& alpha_seg, const Fr_t& beta_seg);
     void claim_record(Pending& pending, const FrTensor& Y, const vector<Fr_t>& u_Y);
     Fr_t prove_end(Pending& pending, const FrTensor& X, const FrTensor& shift, const vector<FrTensor>& X_segments, const vector<FrTensor>& Y_segments,
-                   const vector<Fr_t>& v_Y, vector<Polynomial>& proof);
+                   const vector<Fr_t>& v_Y, vector<Polynomial>& proof, bool evaluate_first = false);
 
    protected:
     // compute() for `rows` rows of n scores (rows = m for one head, num * m for a stack of heads: rows are independent)
