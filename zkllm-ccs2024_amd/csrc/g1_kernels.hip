@@ -240,7 +240,7 @@ __global__ void __launch_bounds__(256) k_fr_to_i32_checked(int32_t* __restrict__
 static constexpr int MW = 32;        // 8-bit signed windows over a 255-bit scalar
 static constexpr int MT = 128;       // lanes of a bucket workgroup = buckets (digit magnitudes 1..128)
 static constexpr int MSEG = 4096;    // elements per chunk (12-bit list entries)
-static constexpr int MCAP = 96;      // list slots per bucket and pass
+static constexpr int MSL = 64;       // lanes of a bucket-accumulation workgroup (one wave): each takes two buckets of its chunk
 static constexpr int MHEAVY = 256;   // a bucket above this many elements of a chunk is summed by the whole workgroup
 struct MsmDesc { const int8_t* digits; uint32_t dstride, count, s_mul, s_off, b_mul, b_off, slot; };   // element i: recoded scalar i*s_mul+s_off of dstride, base A[i*b_mul+b_off]
 template <int NMAX> struct MsmDescs { MsmDesc d[NMAX]; };
@@ -378,134 +378,151 @@ __global__ void __launch_bounds__(256) k_msm_recode(int8_t* __restrict__ D, cons
     D[(size_t)MW * n + i] = flip ? 1 : 0;
 }
 
-// sum over the MT lanes of a workgroup through the LDS pool (36 x MT words); every lane returns the total
-__device__ __forceinline__ G1Jac msm_block_sum(uint32_t* pool, const G1Jac& v, uint32_t t) {
+// sum over the NT lanes of a workgroup through the LDS pool (36 x NT words); every lane returns the total
+template <int NT = MT> __device__ __forceinline__ G1Jac msm_block_sum(uint32_t* pool, const G1Jac& v, uint32_t t) {
     __syncthreads();
     {
         const uint32_t* src = reinterpret_cast<const uint32_t*>(&v);
 #pragma unroll
-        for (int l = 0; l < 36; ++l) pool[l * MT + t] = src[l];
+        for (int l = 0; l < 36; ++l) pool[l * NT + t] = src[l];
     }
     __syncthreads();
-    for (uint32_t sd = MT / 2; sd > 0; sd >>= 1) {
+    for (uint32_t sd = NT / 2; sd > 0; sd >>= 1) {
         if (t < sd) {
             G1Jac x, y;
             uint32_t* px = reinterpret_cast<uint32_t*>(&x);
             uint32_t* py = reinterpret_cast<uint32_t*>(&y);
 #pragma unroll
-            for (int l = 0; l < 36; ++l) { px[l] = pool[l * MT + t]; py[l] = pool[l * MT + t + sd]; }
+            for (int l = 0; l < 36; ++l) { px[l] = pool[l * NT + t]; py[l] = pool[l * NT + t + sd]; }
             x = g1_add(x, y);
 #pragma unroll
-            for (int l = 0; l < 36; ++l) pool[l * MT + t] = px[l];
+            for (int l = 0; l < 36; ++l) pool[l * NT + t] = px[l];
         }
         __syncthreads();
     }
     G1Jac tot;
     uint32_t* pr = reinterpret_cast<uint32_t*>(&tot);
 #pragma unroll
-    for (int l = 0; l < 36; ++l) pr[l] = pool[l * MT];
+    for (int l = 0; l < 36; ++l) pr[l] = pool[l * NT];
     __syncthreads();
     return tot;
 }
 
-// One segment's share of sum over elements of digit_w(s) * base: with nseg == 1 the finished window sum partial[sum * MW + w],
-// otherwise the segment's MT raw buckets partial[((sum * MW + w) * nseg + seg) * MT + t] for k_msm_buckets.
-// Lane t owns the bucket of magnitude t+1.  Per chunk of MSEG elements:
-//  1. the bucket sizes are counted (one LDS atomic per element);
-//  2. a bucket with more than MHEAVY elements (scalars that share a digit: equal values, a common high byte) is summed by
-//     all lanes together, each over its own share of the chunk, and handed to its owner -- no lane walks a long list;
-//  3. the other elements are sorted into per-bucket lists in LDS and every lane walks its own list with mixed
-//     additions, in lockstep whatever the digits are; elements that find their bucket's list full (more than MCAP)
-//     wait for the next pass over the chunk.
+// One segment's share of sum over elements of digit_w(s) * base: the segment's MT raw buckets,
+// partial[((sum * MW + w) * nseg + seg) * MT + b] for bucket magnitude b + 1 (k_msm_bucket_fold / k_msm_buckets reduce them).
+// One wave per workgroup.  Per chunk of MSEG elements:
+//  1. the bucket sizes are counted (one LDS atomic per element) and the elements are sorted by bucket into one list in
+//     LDS (counting sort: 12-bit position in the chunk + sign);
+//  2. the buckets are ranked by size and lane j takes the j-th largest and the j-th smallest: list lengths of uniform
+//     digits are Poisson(32), the largest of 64 is ~47, while the 64 pair sums all lie within a few elements of 64 -- the
+//     lanes walk their two lists as one sequence of mixed additions, in lockstep, and 96 % of the lane-steps add a point
+//     (67 % with one bucket per lane);
+//  3. a bucket with more than MHEAVY elements (scalars that share a digit: equal values, a common high byte) is left out
+//     of the lists and summed by all lanes together, each over its own share of the chunk.
 template <int NMAX>
-__global__ void __launch_bounds__(MT) k_msm_seg(G1Jac* __restrict__ partial, const A29* __restrict__ A, const MsmDescs<NMAX> descs, uint32_t nseg, uint32_t chunks_per_seg) {
-    __shared__ uint32_t cnt[MT], cnt2[MT];
-    __shared__ uint32_t pool[MCAP * MT / 2];       // u16 lists, or the 36 x MT point tree
-    static_assert(MCAP * MT / 2 >= 36 * MT, "pool too small for the point tree");
-    static_assert(MSEG / MT == 32, "one done-bit per element of a lane's share of a chunk");
+__global__ void __launch_bounds__(MSL) __attribute__((amdgpu_waves_per_eu(2, 2))) k_msm_seg(G1Jac* __restrict__ partial, const A29* __restrict__ A, const MsmDescs<NMAX> descs, uint32_t nseg, uint32_t chunks_per_seg) {
+    __shared__ uint32_t cnt[MT], off[MT], cursor[MT];
+    __shared__ uint8_t order[MT];
+    __shared__ uint32_t pool[36 * MSL];            // the sorted list (u16 x MSEG), then the 36 x MSL point tree of the heavy buckets
+    static_assert(36 * MSL * 4 >= MSEG * 2, "pool too small for the list");
+    static_assert(MSEG <= 4096, "12-bit list entries");
     uint16_t* list = reinterpret_cast<uint16_t*>(pool);
     const MsmDesc d = descs.d[blockIdx.z];
     const uint32_t w = blockIdx.y, seg = blockIdx.x, t = threadIdx.x;
     const int8_t* __restrict__ Dw = d.digits + (size_t)w * d.dstride;
     const int8_t* __restrict__ Df = d.digits + (size_t)MW * d.dstride;
-    J29 acc29 = j29_infinity();          // the lane's bucket, in 29-bit limbs while points are added to it
-    G1Jac heavy = g1_infinity();         // what the cooperative path hands to this lane
-    bool any_heavy = false;
+    G1Jac* __restrict__ out = partial + (((size_t)blockIdx.z * MW + w) * nseg + seg) * MT;
+    bool first = true;                                  // nothing written to `out` yet (the same for every lane)
     for (uint32_t ch = 0; ch < chunks_per_seg; ++ch) {
         const uint32_t e0 = (seg * chunks_per_seg + ch) * MSEG;
         if (e0 >= d.count) break;
         const uint32_t e1 = (e0 + MSEG < d.count) ? e0 + MSEG : d.count;
-        cnt[t] = 0;
-        cnt2[t] = 0;
+        cnt[t] = 0; cnt[t + MSL] = 0;
         __syncthreads();
-        for (uint32_t e = e0 + t; e < e1; e += MT) {
+        for (uint32_t e = e0 + t; e < e1; e += MSL) {
             const int dg = Dw[(size_t)e * d.s_mul + d.s_off];
             if (dg != 0) atomicAdd(&cnt[(dg < 0 ? -dg : dg) - 1], 1u);
         }
         __syncthreads();
-        uint32_t done = 0;                       // bit i: this lane's i-th element of the chunk needs no more work (MSEG / MT = 32 per lane)
-        for (uint32_t b = 0; b < (uint32_t)MT; ++b) {
-            if (cnt[b] <= (uint32_t)MHEAVY) continue;          // the same for every lane
-            J29 h29 = j29_infinity();
-            for (uint32_t e = e0 + t, i = 0; e < e1; e += MT, ++i) {
-                const size_t si = (size_t)e * d.s_mul + d.s_off;
-                const int dg = Dw[si];
-                if ((uint32_t)(dg < 0 ? -dg : dg) != b + 1) continue;
-                done |= 1u << i;
-                A29 pt = A[(size_t)e * d.b_mul + d.b_off];
-                if (a29_is_inf(pt)) continue;
-                if ((dg < 0) != (Df[si] != 0)) pt.y = fq29_neg(pt.y);
-                h29 = j29_add_mixed(h29, pt);
+        if (t == 0) {
+            uint32_t run = 0;
+            for (uint32_t b = 0; b < (uint32_t)MT; ++b) {
+                off[b] = run; cursor[b] = run;
+                run += cnt[b] > (uint32_t)MHEAVY ? 0u : cnt[b];
             }
-            const G1Jac h = msm_block_sum(pool, j29_to_jac(h29), t);
-            if (t == b) heavy = g1_add(heavy, h);
-            any_heavy = true;
         }
-        for (;;) {
-            uint32_t left = 0;
-            for (uint32_t e = e0 + t, i = 0; e < e1; e += MT, ++i) {
-                if ((done >> i) & 1u) continue;
-                const size_t si = (size_t)e * d.s_mul + d.s_off;
-                const int dg = Dw[si];
-                if (dg != 0) {
-                    const uint32_t mag = (uint32_t)(dg < 0 ? -dg : dg);
-                    const uint32_t pos = atomicAdd(&cnt2[mag - 1], 1u);
-                    if (pos >= (uint32_t)MCAP) { left = 1; continue; }
-                    list[pos * MT + (mag - 1)] = (uint16_t)((e - e0) | (((dg < 0) != (Df[si] != 0)) ? 0x8000u : 0u));
-                }
-                done |= 1u << i;
+        // rank of a bucket by list length (heavy buckets have none), ties by index: a permutation
+        for (uint32_t b = t; b < (uint32_t)MT; b += MSL) {
+            const uint32_t cb = cnt[b] > (uint32_t)MHEAVY ? 0u : cnt[b];
+            uint32_t r = 0;
+            for (uint32_t o = 0; o < (uint32_t)MT; ++o) {
+                const uint32_t co = cnt[o] > (uint32_t)MHEAVY ? 0u : cnt[o];
+                r += (co > cb || (co == cb && o < b)) ? 1u : 0u;
             }
-            __syncthreads();
-            const uint32_t c2 = cnt2[t];
-            const uint32_t mine = c2 < (uint32_t)MCAP ? c2 : (uint32_t)MCAP;
-            for (uint32_t k = 0; k < mine; ++k) {
-                const uint32_t en = list[k * MT + t];
+            order[r] = (uint8_t)b;
+        }
+        __syncthreads();
+        for (uint32_t e = e0 + t; e < e1; e += MSL) {
+            const size_t si = (size_t)e * d.s_mul + d.s_off;
+            const int dg = Dw[si];
+            if (dg == 0) continue;
+            const uint32_t mag = (uint32_t)(dg < 0 ? -dg : dg);
+            if (cnt[mag - 1] > (uint32_t)MHEAVY) continue;
+            const uint32_t pos = atomicAdd(&cursor[mag - 1], 1u);
+            list[pos] = (uint16_t)((e - e0) | (((dg < 0) != (Df[si] != 0)) ? 0x8000u : 0u));
+        }
+        __syncthreads();
+        {
+            const uint32_t bA = order[t], bB = order[MT - 1 - t];
+            const uint32_t lenA = cnt[bA] > (uint32_t)MHEAVY ? 0u : cnt[bA], lenB = cnt[bB] > (uint32_t)MHEAVY ? 0u : cnt[bB];
+            const uint32_t total = lenA + lenB;
+            uint32_t pos = off[bA];
+            J29 acc29 = j29_infinity();
+            for (uint32_t i = 0;; ++i) {
+                if (i == lenA) {
+                    // the end of the first list: its bucket goes out (added to what earlier chunks of this segment left there)
+                    G1Jac v = j29_to_jac(acc29);
+                    if (!first) v = g1_add(out[bA], v);
+                    out[bA] = v;
+                    acc29 = j29_infinity();
+                    pos = off[bB];
+                }
+                if (i >= total) break;
+                const uint32_t en = list[pos++];
                 A29 pt = A[(size_t)(e0 + (en & 0x7FFFu)) * d.b_mul + d.b_off];
                 if (a29_is_inf(pt)) continue;
                 if (en & 0x8000u) pt.y = fq29_neg(pt.y);
                 acc29 = j29_add_mixed(acc29, pt);
             }
-            if (!__syncthreads_or((int)left)) break;
-            cnt2[t] = 0;
-            __syncthreads();
+            G1Jac v = j29_to_jac(acc29);
+            if (!first) v = g1_add(out[bB], v);
+            out[bB] = v;
         }
+        __threadfence_block();
         __syncthreads();
+        for (uint32_t b = 0; b < (uint32_t)MT; ++b) {
+            if (cnt[b] <= (uint32_t)MHEAVY) continue;          // the same for every lane
+            J29 h29 = j29_infinity();
+            for (uint32_t e = e0 + t; e < e1; e += MSL) {
+                const size_t si = (size_t)e * d.s_mul + d.s_off;
+                const int dg = Dw[si];
+                if ((uint32_t)(dg < 0 ? -dg : dg) != b + 1) continue;
+                A29 pt = A[(size_t)e * d.b_mul + d.b_off];
+                if (a29_is_inf(pt)) continue;
+                if ((dg < 0) != (Df[si] != 0)) pt.y = fq29_neg(pt.y);
+                h29 = j29_add_mixed(h29, pt);
+            }
+            const G1Jac h = msm_block_sum<MSL>(pool, j29_to_jac(h29), t);
+            if (t == 0) out[b] = g1_add(out[b], h);            // its list was empty: the slot holds what earlier chunks left (or infinity)
+        }
+        __threadfence_block();
+        __syncthreads();
+        first = false;
     }
-    G1Jac acc = j29_to_jac(acc29);
-    if (any_heavy) acc = g1_add(acc, heavy);           // the same branch for every lane
-    if (nseg > 1) {
-        // several segments share this (sum, window): leave the buckets as they are, k_msm_buckets reduces them once for all segments
-        partial[(((size_t)blockIdx.z * MW + w) * nseg + seg) * MT + t] = acc;
-        return;
+    if (first) {                                       // a segment past the end of this sum: empty buckets
+        out[t] = g1_infinity();
+        out[t + MSL] = g1_infinity();
     }
-    // bucket value t+1 times the bucket, then the sum over the lanes
-    G1Jac r = g1_infinity();
-    for (int bit = 7; bit >= 0; --bit) {
-        r = g1_double(r);
-        if (((t + 1) >> bit) & 1u) r = g1_add(r, acc);
-    }
-    const G1Jac tot = msm_block_sum(pool, r, t);
-    if (t == 0) partial[(size_t)blockIdx.z * MW + w] = tot;
 }
 // raw buckets of up to 8 consecutive segments summed: out[(row * gridDim.y + group) * MT + t], row = sum * MW + w
 __global__ void __launch_bounds__(MT) k_msm_bucket_fold(G1Jac* __restrict__ out, const G1Jac* __restrict__ buckets, uint32_t nseg) {
@@ -642,7 +659,7 @@ __global__ void __launch_bounds__(GT) k_open_chain(G1Jac* __restrict__ pts, cons
     }
 }
 // The fold itself: pair g -> new scalar and new generator.
-__global__ void __launch_bounds__(GT) k_open_fold(Fr* __restrict__ new_scalars, G1Jac* __restrict__ new_gens, const Fr* __restrict__ scalars, const G1Affine* __restrict__ A,
+__global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2))) k_open_fold(Fr* __restrict__ new_scalars, G1Jac* __restrict__ new_gens, const Fr* __restrict__ scalars, const G1Affine* __restrict__ A,
                                                   const Fr u_mont, const GlvK ku, const JsfK jsf, size_t old_size, size_t new_size) {
     // ---- pair g: s' and g' = a1 + [u](a0 - a1) -------------------------------------------------------------------------------
     // The scalar multiplication works on affine points throughout its table: D = a0 - a1 (one inversion, batched over
@@ -911,14 +928,14 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     const uint32_t chunks = count_max ? cdiv(count_max, MSEG) : 1u;
     const uint32_t cps = (chunks + 255u) / 256u;
     const uint32_t nseg = (chunks + cps - 1) / cps;
-    Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (nseg > 1 ? (size_t)nseg * MT : 1));
+    Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (size_t)nseg * MT);
     if (partial.rc) return partial.rc;
     G1Jac* wsum = wsum_round + (size_t)(3 - n_msm) * MW;
     Scratch& aff29 = arena.add(sizeof(A29) * old_size);
     if (aff29.rc) return aff29.rc;
     hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(old_size, 256)), dim3(256), 0, aux, aff29.as<A29>(), aff.as<G1Affine>(), old_size);
-    hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MT), 0, aux, nseg > 1 ? partial.as<G1Jac>() : wsum, aff29.as<A29>(), descs, nseg, cps);
-    if (nseg > 1) {
+    hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MSL), 0, aux, partial.as<G1Jac>(), aff29.as<A29>(), descs, nseg, cps);
+    {
         // sum the segments' raw buckets eight at a time, then weight and total
         const G1Jac* cur = partial.as<G1Jac>();
         uint32_t ns = nseg;
@@ -966,7 +983,7 @@ static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, con
     Scratch& aff = arena.add(sizeof(G1Affine) * n0);
     Scratch& aff29 = arena.add(sizeof(A29) * n0);
     Scratch& coef = arena.add(sizeof(Fr) * (size_t)n_msm * n0);
-    Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (nseg > 1 ? (size_t)nseg * MT : 1));
+    Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (size_t)nseg * MT);
     Scratch& wsum = arena.add(sizeof(G1Jac) * n_msm * MW);
     if (sl.rc) return sl.rc;
     if (aff.rc) return aff.rc;
@@ -988,8 +1005,8 @@ static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, con
         descs.d[i] = MsmDesc{dig.as<int8_t>(), (uint32_t)ncoef, live ? (uint32_t)n0 : 0u, 1u, live ? (uint32_t)((size_t)i * n0) : 0u, 1u, 0u, slot};
     }
     hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(n0, 256)), dim3(256), 0, st, aff29.as<A29>(), aff.as<G1Affine>(), n0);
-    hipLaunchKernelGGL(k_msm_seg<TAIL_SUMS>, dim3(nseg, MW, n_msm), dim3(MT), 0, st, nseg > 1 ? partial.as<G1Jac>() : wsum.as<G1Jac>(), aff29.as<A29>(), descs, nseg, cps);
-    if (nseg > 1) hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), nseg);
+    hipLaunchKernelGGL(k_msm_seg<TAIL_SUMS>, dim3(nseg, MW, n_msm), dim3(MSL), 0, st, partial.as<G1Jac>(), aff29.as<A29>(), descs, nseg, cps);
+    hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), nseg);
     hipLaunchKernelGGL(k_msm_horner, dim3(n_msm), dim3(GT), 0, st, pts, wsum.as<G1Jac>(), descs);
     ZK_LAUNCH_CHECK();
     // the folded scalar is the single element of the last level
