@@ -667,7 +667,11 @@ __global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2)))
     // D - phi(D) (a second batched inversion).  With the joint sparse form of (k1, k2) -- digits in {-1, 0, 1}, a non-zero
     // pair in about half of the 129 positions -- the walk is one doubling per position and one mixed addition per
     // non-zero pair.  Lanes whose inputs are special (infinity, equal abscissae, x = 0) take the general Jacobian route.
-    __shared__ uint32_t inv_lds[12][2 * GT];
+    // one wave per workgroup: the batched inversions are over before the table is written, and LDS serves a wave in order
+    __shared__ int32_t fold_lds[4 * 14 * GT];
+    static_assert(4 * 14 * GT >= 12 * 2 * GT, "the inversion buffer shares the table's space");
+    uint32_t (*inv_lds)[2 * GT] = reinterpret_cast<uint32_t (*)[2 * GT]>(fold_lds);
+    int32_t (*tab)[14][GT] = reinterpret_cast<int32_t (*)[14][GT]>(fold_lds);
     const size_t g = (size_t)blockIdx.x * GT + threadIdx.x;
     const bool live = g < new_size;
     const size_t g0 = 2 * g, g1 = 2 * g + 1;
@@ -708,10 +712,20 @@ __global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2)))
             PmQ.x = add(fp_sqr(lam), PQ.x);
             PmQ.y = sub(fp_mul(lam, sub(D.x, PmQ.x)), D.y);
         }
-        // the walk itself in 29-bit limbs: the four table points differ in four abscissae and two ordinates
-        const Fq29 xD = fq29_from_fp(D.x), xQ = fq29_from_fp(Q.x), xPQ = fq29_from_fp(PQ.x), xPmQ = fq29_from_fp(PmQ.x);
-        const Fq29 yD = fq29_from_fp(D.y), yPmQ = fq29_from_fp(PmQ.y);
-        const Fq29 yDn = fq29_neg(yD), yPmQn = fq29_neg(yPmQ);
+        // the walk itself in 29-bit limbs: the four table points differ in four abscissae and two ordinates.  D stays in
+        // registers; the other three abscissae and the second ordinate wait in LDS (word-interleaved over the lanes) and
+        // negations are formed when a point is taken: the walk then fits 256 registers without spilling.
+        const Fq29 xD = fq29_from_fp(D.x), yD = fq29_from_fp(D.y);
+        {
+            const Fq29 xQ = fq29_from_fp(Q.x), xPQ = fq29_from_fp(PQ.x), xPmQ = fq29_from_fp(PmQ.x), yPmQ = fq29_from_fp(PmQ.y);
+#pragma unroll
+            for (int l = 0; l < 14; ++l) {
+                tab[0][l][threadIdx.x] = xQ.l[l];
+                tab[1][l][threadIdx.x] = xPQ.l[l];
+                tab[2][l][threadIdx.x] = xPmQ.l[l];
+                tab[3][l][threadIdx.x] = yPmQ.l[l];
+            }
+        }
         J29 w = j29_infinity();
         for (int i = (int)jsf.len - 1; i >= 0; --i) {
             w = j29_double(w);
@@ -719,10 +733,22 @@ __global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2)))
             const int d1 = (int)(dg & 3u) - 1, d2 = (int)(dg >> 2) - 1;
             if (d1 == 0 && d2 == 0) continue;
             A29 t;
-            if (d2 == 0) { t.x = xD; t.y = d1 < 0 ? yDn : yD; }
-            else if (d1 == 0) { t.x = xQ; t.y = d2 < 0 ? yDn : yD; }
-            else if (d1 == d2) { t.x = xPQ; t.y = d1 < 0 ? yD : yDn; }          // D + phi(D) = (beta^2 x, -y)
-            else { t.x = xPmQ; t.y = d1 < 0 ? yPmQn : yPmQ; }
+            bool negate;
+            if (d2 == 0) { t.x = xD; t.y = yD; negate = d1 < 0; }
+            else {
+                const int xi = d1 == 0 ? 0 : (d1 == d2 ? 1 : 2);
+#pragma unroll
+                for (int l = 0; l < 14; ++l) t.x.l[l] = tab[xi][l][threadIdx.x];
+                if (xi == 2) {
+#pragma unroll
+                    for (int l = 0; l < 14; ++l) t.y.l[l] = tab[3][l][threadIdx.x];
+                    negate = d1 < 0;
+                } else {
+                    t.y = yD;
+                    negate = xi == 0 ? d2 < 0 : d1 > 0;                          // D + phi(D) = (beta^2 x, -y)
+                }
+            }
+            if (negate) t.y = fq29_neg(t.y);
             w = j29_add_mixed(w, t);
         }
         if (!inf1) w = j29_add_mixed(w, a29_from_affine(a1));
