@@ -31,7 +31,7 @@ VALU_PEAK_TOPS = 256 * 4 * 16 * 2.4e9 / 1e12
 # HBM traffic of k_open_fold per generator pair, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the kernel alone
 # (python3 bench.py --pmc-probe; summary in profiles/k_open_fold_pmc_traffic.txt), each counter scaled by what it reads for
 # zk_fr_add over 2^24 elements (1 GiB read, 512 MiB written)
-FOLD_TRAFFIC_BYTES_PER_PAIR = 6090.0
+FOLD_TRAFFIC_BYTES_PER_PAIR = 2477.0
 
 
 def main():
@@ -197,8 +197,9 @@ def main():
                                   "unit": "T MAD32/s", "frac": iso_tops / VALU_PEAK_TOPS, "traffic": FOLD_TRAFFIC_BYTES_PER_PAIR * (n_big // 2),
                                   "avg_launch_ms": fold_ms.value / max(1, fold_launches.value),
                                   "fp_mul_per_s": fold_mults.value / (fold_ms.value * 1e-3),
-                                  "note": "4096 waves on 2048 wave slots (two per SIMD at 256 VGPRs): two full turns.  traffic: FETCH_SIZE + WRITE_SIZE of this "
-                                          "launch from profiles/k_open_fold_pmc_traffic.txt, against 336 B per pair of algorithmic traffic (the rest is register spill)"}
+                                  "note": "4096 waves on 2048 wave slots (two per SIMD: 250 registers, most of the walk's table in LDS): two full turns.  traffic: FETCH_SIZE + "
+                                          "WRITE_SIZE of this launch from profiles/k_open_fold_pmc_traffic.txt, against 336 B per pair of algorithmic traffic (the rest is "
+                                          "private memory of the out-of-line special cases)"}
     for p_ in (sc, ns, ng):
         hip.free(p_)
     del gens_big

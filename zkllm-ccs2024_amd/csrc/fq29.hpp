@@ -182,7 +182,23 @@ ZK_HD Fq29 fq29_kp(int k) {
     r.l[13] = (int32_t)((int64_t)k * fq29_p(13) + c);
     return r;
 }
+// out of line, and on the device with the value in registers: a reference parameter would make every caller keep the
+// value in private memory for a call that almost never happens
+#if defined(__HIP_DEVICE_COMPILE__)
+static __device__ __attribute__((noinline)) bool fq29_is_kp_regs(i32x4 a0, i32x4 a1, i32x4 a2, i32x2 a3, int k) {
+    Fq29 a;
+    a.l[0] = a0[0]; a.l[1] = a0[1]; a.l[2] = a0[2]; a.l[3] = a0[3];
+    a.l[4] = a1[0]; a.l[5] = a1[1]; a.l[6] = a1[2]; a.l[7] = a1[3];
+    a.l[8] = a2[0]; a.l[9] = a2[1]; a.l[10] = a2[2]; a.l[11] = a2[3];
+    a.l[12] = a3[0]; a.l[13] = a3[1];
+    return fq29_same(a, fq29_kp(k));
+}
+__device__ __forceinline__ bool fq29_is_kp(const Fq29& a, int k) {
+    return fq29_is_kp_regs(i32x4{a.l[0], a.l[1], a.l[2], a.l[3]}, i32x4{a.l[4], a.l[5], a.l[6], a.l[7]}, i32x4{a.l[8], a.l[9], a.l[10], a.l[11]}, i32x2{a.l[12], a.l[13]}, k);
+}
+#else
 static ZK_NOINLINE_HD bool fq29_is_kp(const Fq29& a, int k) { return fq29_same(a, fq29_kp(k)); }
+#endif
 // a == 0 mod p, for |a| < 40 p.  A multiple k*p has top limb 13k (k >= 0) or 13k - 1 (k < 0): the top limb names the
 // only candidate k, the low limb then rules it out except with probability 2^-29, and the full comparison
 // runs out of line in the rare remaining case.
