@@ -141,7 +141,8 @@ def test_commit_int_rejects_non_integer_scalars_and_is_linear(pv, orc):
 # 4500 x 2: more than one chunk of the bucket kernel and odd sizes in several rounds; 20000 x 2: two halving rounds
 # (the second takes T from the first round's points) before the batched rest; 70000 x 1: four halving rounds, so T of
 # rounds 1..3 are combinations of up to seven earlier points, with an odd size (4375 pairs + 1) on the way
-@pytest.mark.parametrize("n,m", [(4, 2), (8, 1), (16, 4), (5, 3), (1, 2), (300, 1), (4500, 2), (20000, 2), (70000, 1)])
+# 9001 x 1: an odd size in the first halving round, whose T is the sum over pairs with one element left alone
+@pytest.mark.parametrize("n,m", [(4, 2), (8, 1), (16, 4), (5, 3), (1, 2), (300, 1), (4500, 2), (9001, 1), (20000, 2), (70000, 1)])
 def test_open_value_and_g1_transcript(pv, orc, n, m):
     gens = oracle_gens(orc, 15 + n, n)
     rng = np.random.default_rng(n * m)
@@ -176,6 +177,33 @@ def test_open_with_equal_scalars(pv, orc, n, val):
     orc_check(orc.orc_open(gens, n, T, n, 1, u, k, exp_proof, exp_val))
     hG, hT = pv.g1_from_host(gens), pv.from_fr(T)
     com = pv.commit_int(hG, hT)
+    val_got, proof = pv.open(hG, hT, com, u)
+    assert (val_got == exp_val).all()
+    assert (norm(orc, proof) == norm(orc, exp_proof)).all()
+
+
+def test_open_with_equal_opposite_and_infinite_generators_in_the_first_round(pv, orc):
+    """More generators than the batched rest takes, so the first round halves them on the device: pairs of equal
+    generators (their sum is a doubling), of opposite ones (their sum is infinity), with an infinite member, and an
+    infinite pair, in the pair sums that give T, in the fold and in the bucket sums."""
+    n = 8200
+    gens = oracle_gens(orc, 77, n)
+    neg = np.zeros((1, 36), np.uint32)
+    gens[1] = gens[0]
+    orc_check(orc.orc_g1_op(4, gens[2:3].copy(), gens[2:3].copy(), neg, 1))
+    gens[3] = neg[0]
+    gens[5] = 0
+    gens[6] = 0
+    gens[7] = 0
+    gens[8] = 0
+    T = mt_random_vec(np.random.RandomState(3), n)
+    k = (n - 1).bit_length()
+    u = mt_random_vec(np.random.RandomState(18), k)
+    exp_proof = np.zeros((3 * k + 1, 36), np.uint32)
+    exp_val = np.zeros(8, np.uint32)
+    orc_check(orc.orc_open(gens, n, T, n, 1, u, k, exp_proof, exp_val))
+    hG, hT = pv.g1_from_host(gens), pv.from_fr(T)
+    com = pv.g1_from_host(np.zeros((1, 36), np.uint32))
     val_got, proof = pv.open(hG, hT, com, u)
     assert (val_got == exp_val).all()
     assert (norm(orc, proof) == norm(orc, exp_proof)).all()

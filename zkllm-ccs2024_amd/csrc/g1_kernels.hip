@@ -916,6 +916,30 @@ static JsfK jsf_of(const GlvK& k) {
 
 // Queues one round: the fold on st, the bucket sums on aux.  wsum_round: the round's 3 x MW window sums (T, T0, T1); with_T
 // false leaves the first MW alone (T of that round then comes from k_open_chain).
+// Round 0 needs T = sum_j s_j g_j over all generators besides T0 and T1.  With the pairs' sums,
+//   sum_i (s_2i + s_2i+1)(g_2i + g_2i+1) = T + T0 + T1,
+// so T costs a bucket sum over half as many points: pair i gets the scalar s_2i + s_2i+1 (mod r: the generators have
+// order r) and the point g_2i + g_2i+1; an odd last element stands alone.  k_open_t_fix takes T0 and T1 off again,
+// window by window.
+__global__ void __launch_bounds__(GT) k_open_pairs(Fr* __restrict__ ps, G1Jac* __restrict__ pj, const Fr* __restrict__ scalars, const G1Affine* __restrict__ A,
+                                                   size_t old_size, size_t half_up) {
+    const size_t i = (size_t)blockIdx.x * GT + threadIdx.x;
+    if (i >= half_up) return;
+    const bool has1 = 2 * i + 1 < old_size;
+    ps[i] = has1 ? add(scalars[2 * i], scalars[2 * i + 1]) : scalars[2 * i];
+    G1Jac p = aff_to_jac(A[2 * i]);
+    if (has1) {
+        const G1Affine b = A[2 * i + 1];
+        if (!aff_is_inf(b)) p = g1_add_mixed(p, b);
+    }
+    pj[i] = p;
+}
+__global__ void __launch_bounds__(64) k_open_t_fix(G1Jac* __restrict__ wsum) {
+    const uint32_t w = threadIdx.x;
+    if (w >= (uint32_t)MW) return;
+    wsum[w] = g1_add(g1_add(wsum[w], g1_neg(wsum[MW + w])), g1_neg(wsum[2 * MW + w]));
+}
+
 static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars, const G1Jac* gens, const Fr& u, size_t old_size, bool with_T,
                              G1Jac* wsum_round, Arena& arena, hipStream_t st, hipStream_t aux, std::vector<hipEvent_t>& events) {
     ZK_ARG(old_size < (1ull << 31), "opening: more than 2^31 generators");
@@ -939,27 +963,40 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     // ---- side chain (aux): bucket sums, window sums, the round's single points; nothing here feeds the next fold ----
     MsmDescs<3> descs;
     const uint32_t half = (uint32_t)(old_size / 2);
+    const uint32_t half_up = (uint32_t)new_size;
     const uint32_t n_msm = chained ? 2u : 3u;
     uint32_t q = 0;
     const int8_t* dg = dig.as<int8_t>();
     const uint32_t ds = (uint32_t)old_size;
-    if (!chained) descs.d[q++] = MsmDesc{dg, ds, (uint32_t)old_size, 1u, 0u, 1u, 0u, 0u};
+    Scratch& aff29 = arena.add(sizeof(A29) * (old_size + (chained ? 0 : half_up)));
+    if (aff29.rc) return aff29.rc;
+    hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(old_size, 256)), dim3(256), 0, aux, aff29.as<A29>(), aff.as<G1Affine>(), old_size);
+    if (!chained) {
+        // T of round 0 through the pairs' sums: half_up points appended to the table, their scalars recoded apart
+        Scratch& ps = arena.add(sizeof(Fr) * half_up);
+        Scratch& pj = arena.add(sizeof(G1Jac) * half_up);
+        Scratch& paff = arena.add(sizeof(G1Affine) * half_up);
+        Scratch& dig2 = arena.add((size_t)(MW + 1) * half_up);
+        if (ps.rc || pj.rc || paff.rc || dig2.rc) return ps.rc ? ps.rc : (pj.rc ? pj.rc : (paff.rc ? paff.rc : dig2.rc));
+        hipLaunchKernelGGL(k_open_pairs, dim3(cdiv(half_up, GT)), dim3(GT), 0, aux, ps.as<Fr>(), pj.as<G1Jac>(), scalars, aff.as<G1Affine>(), old_size, (size_t)half_up);
+        hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(half_up, CH), GT)), dim3(GT), 0, aux, paff.p, pj.as<G1Jac>(), (size_t)half_up);
+        hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(half_up, 256)), dim3(256), 0, aux, dig2.as<int8_t>(), ps.as<Fr>(), (size_t)half_up);
+        hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(half_up, 256)), dim3(256), 0, aux, aff29.as<A29>() + old_size, paff.as<G1Affine>(), (size_t)half_up);
+        descs.d[q++] = MsmDesc{dig2.as<int8_t>(), half_up, half_up, 1u, 0u, 1u, (uint32_t)old_size, 0u};
+    }
     descs.d[q++] = MsmDesc{dg, ds, half, 2u, 0u, 2u, 1u, 1u};
     descs.d[q++] = MsmDesc{dg, ds, half, 2u, 1u, 2u, 0u, 2u};
     for (; q < 3; ++q) descs.d[q] = MsmDesc{dg, ds, 0u, 1u, 0u, 1u, 0u, 0u};
     // One chunk per workgroup: many short workgroups keep every compute unit busy to the end of the launch (with few
     // long ones, all equally long, whatever does not fit the first turn waits a whole turn); the raw buckets of the
     // segments are summed afterwards.  Very large inputs take more chunks per workgroup to bound the bucket storage.
-    const size_t count_max = chained ? half : old_size;
+    const size_t count_max = chained ? half : half_up;
     const uint32_t chunks = count_max ? cdiv(count_max, MSEG) : 1u;
     const uint32_t cps = (chunks + 255u) / 256u;
     const uint32_t nseg = (chunks + cps - 1) / cps;
     Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (size_t)nseg * MT);
     if (partial.rc) return partial.rc;
     G1Jac* wsum = wsum_round + (size_t)(3 - n_msm) * MW;
-    Scratch& aff29 = arena.add(sizeof(A29) * old_size);
-    if (aff29.rc) return aff29.rc;
-    hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(old_size, 256)), dim3(256), 0, aux, aff29.as<A29>(), aff.as<G1Affine>(), old_size);
     hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MSL), 0, aux, partial.as<G1Jac>(), aff29.as<A29>(), descs, nseg, cps);
     {
         // sum the segments' raw buckets eight at a time, then weight and total
@@ -975,6 +1012,7 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
         }
         hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, aux, wsum, cur, ns);
     }
+    if (!chained) hipLaunchKernelGGL(k_open_t_fix, dim3(1), dim3(64), 0, aux, wsum);
     ZK_LAUNCH_CHECK();
     // ---- critical chain (st): the fold ----
     const GlvK ku = glv_split(u);
