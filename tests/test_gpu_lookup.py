@@ -61,6 +61,21 @@ def test_multiplicities(pv, D, low, length):
     assert fr_ints(m) == [int(c) for c in np.bincount(vals - low, minlength=size)]
 
 
+@pytest.mark.parametrize("D,low,length,skew", [((1 << 21) + 12345, -5, (1 << 18) + 777, 3), (1500000, 0, 1 << 20, 1), ((1 << 20) + 1, -9, 1 << 22, 0)])
+def test_multiplicities_of_many_queries_into_a_large_table(pv, D, low, length, skew):
+    """Above 2^20 queries and 16384 bins the counts come from the partitioned path (scatter by high bits, LDS counts per
+    partition): ragged sizes, a table that is no power of two, a third of the queries equal, all queries equal."""
+    rng = np.random.default_rng(D)
+    vals = rng.integers(low, low + length, D)
+    if skew == 3:
+        vals[: D // 3] = low + length // 2
+    elif skew == 1:
+        vals[:] = low + 4097
+    m = pv.range_prep(pv.from_i64(vals), low, length).host()
+    want = np.bincount(vals - low, minlength=m.shape[0]).astype(np.uint32)
+    assert (m[:, 0] == want).all() and not m[:, 1:].any()
+
+
 def test_lookup_out_of_range_is_an_error(pv):
     with pytest.raises(RuntimeError, match="outside the table"):
         pv.range_prep(pv.from_i64(np.array([0, 1, 99])), 0, 8)

@@ -147,6 +147,108 @@ __global__ void __launch_bounds__(TPB) k_hist_global(uint32_t* __restrict__ coun
         if (key != HH_EMPTY) atomicAdd(&counts[key], cnts[s]);
     }
 }
+// Large tables and many queries: global atomics are the cost of k_hist_global when the queries spread over the table
+// (13 G/s).  Here the queries are first partitioned by their high bits -- per-tile sizes, one exclusive scan, a scatter of
+// the low 12 bits as u16 -- and every partition is then counted in LDS, 4096 bins at a time, by as many workgroups as its
+// size asks for; global memory sees one atomic per non-empty bin and slice.  Skewed inputs (one partition holding nearly
+// everything) only make that partition's slices hit the same LDS counters, which an LDS serves far faster than L2 does.
+static constexpr uint32_t HP_BITS = 12, HP_BINS = 1u << HP_BITS;   // bins per partition
+static constexpr uint32_t HP_TILE = 65536;                           // queries per workgroup of the partition passes
+static constexpr uint32_t HP_SLICE = 32768;                          // queries per workgroup of the counting pass
+static constexpr uint32_t HP_MAXP = 1024;                            // partitions: tables up to 2^22 bins
+static constexpr size_t HP_MIN_QUERIES = (size_t)1 << 20;
+__global__ void __launch_bounds__(TPB) k_hp_sizes(uint32_t* __restrict__ sizes, const uint32_t* __restrict__ idx, size_t n, uint32_t P, uint32_t ntiles) {
+    __shared__ uint32_t c[HP_MAXP];
+    for (uint32_t q = threadIdx.x; q < P; q += TPB) c[q] = 0;
+    __syncthreads();
+    const size_t base = (size_t)blockIdx.x * HP_TILE, end = base + HP_TILE < n ? base + HP_TILE : n;
+    for (size_t i = base + threadIdx.x; i < end; i += TPB) atomicAdd(&c[idx[i] >> HP_BITS], 1u);
+    __syncthreads();
+    for (uint32_t q = threadIdx.x; q < P; q += TPB) sizes[(size_t)q * ntiles + blockIdx.x] = c[q];
+}
+// one workgroup: a[0..M) -> its exclusive prefix sums (partition-major), part_off[q] = where partition q starts, part_off[P] = n
+__global__ void __launch_bounds__(1024) k_hp_scan(uint32_t* __restrict__ a, uint32_t* __restrict__ part_off, uint32_t M, uint32_t P, uint32_t ntiles, uint32_t n) {
+    __shared__ uint32_t part[1024];
+    const uint32_t t = threadIdx.x, L = (M + 1023u) / 1024u;
+    const uint32_t b0 = t * L < M ? t * L : M, b1 = b0 + L < M ? b0 + L : M;
+    uint32_t s = 0;
+    for (uint32_t i = b0; i < b1; ++i) s += a[i];
+    part[t] = s;
+    __syncthreads();
+    for (uint32_t off = 1; off < 1024u; off <<= 1) {
+        const uint32_t v = t >= off ? part[t - off] : 0u;
+        __syncthreads();
+        part[t] += v;
+        __syncthreads();
+    }
+    uint32_t run = part[t] - s;
+    for (uint32_t i = b0; i < b1; ++i) {
+        const uint32_t v = a[i];
+        a[i] = run;
+        if (i % ntiles == 0) part_off[i / ntiles] = run;
+        run += v;
+    }
+    if (t == 0) part_off[P] = n;
+}
+// one workgroup: the list of (partition, slice) pairs the counting pass works through, slice_tab[k] = partition << 22 | slice
+__global__ void __launch_bounds__(1024) k_hp_slices(uint32_t* __restrict__ slice_tab, uint32_t* __restrict__ nslices, const uint32_t* __restrict__ part_off, uint32_t P) {
+    __shared__ uint32_t part[1024];
+    const uint32_t t = threadIdx.x;
+    const uint32_t ns = t < P ? (part_off[t + 1] - part_off[t] + HP_SLICE - 1) / HP_SLICE : 0u;
+    part[t] = ns;
+    __syncthreads();
+    for (uint32_t off = 1; off < 1024u; off <<= 1) {
+        const uint32_t v = t >= off ? part[t - off] : 0u;
+        __syncthreads();
+        part[t] += v;
+        __syncthreads();
+    }
+    const uint32_t o = part[t] - ns;
+    for (uint32_t q = 0; q < ns; ++q) slice_tab[o + q] = (t << 22) | q;
+    if (t == 1023u) *nslices = part[1023];
+}
+__global__ void __launch_bounds__(TPB) k_hp_scatter(uint16_t* __restrict__ parted, const uint32_t* __restrict__ offs, const uint32_t* __restrict__ idx, size_t n, uint32_t P,
+                                                    uint32_t ntiles) {
+    __shared__ uint32_t cur[HP_MAXP];
+    for (uint32_t q = threadIdx.x; q < P; q += TPB) cur[q] = offs[(size_t)q * ntiles + blockIdx.x];
+    __syncthreads();
+    const size_t base = (size_t)blockIdx.x * HP_TILE, end = base + HP_TILE < n ? base + HP_TILE : n;
+    for (size_t i = base + threadIdx.x; i < end; i += TPB) {
+        const uint32_t key = idx[i];
+        const uint32_t pos = atomicAdd(&cur[key >> HP_BITS], 1u);
+        parted[pos] = (uint16_t)(key & (HP_BINS - 1u));
+    }
+}
+__global__ void __launch_bounds__(TPB) k_hp_count(uint32_t* __restrict__ counts, const uint16_t* __restrict__ parted, const uint32_t* __restrict__ part_off,
+                                                  const uint32_t* __restrict__ slice_tab, const uint32_t* __restrict__ nslices, uint32_t nbins) {
+    if (blockIdx.x >= *nslices) return;
+    __shared__ uint32_t h[HP_BINS];
+    const uint32_t e = slice_tab[blockIdx.x], q = e >> 22, sl = e & ((1u << 22) - 1u);
+    for (uint32_t b = threadIdx.x; b < HP_BINS; b += TPB) h[b] = 0;
+    __syncthreads();
+    const uint32_t start = part_off[q] + sl * HP_SLICE, stop = part_off[q + 1];
+    const uint32_t end = stop - start > HP_SLICE ? start + HP_SLICE : stop;
+    for (uint32_t i = start + threadIdx.x; i < end; i += TPB) atomicAdd(&h[parted[i]], 1u);
+    __syncthreads();
+    for (uint32_t b = threadIdx.x; b < HP_BINS; b += TPB) {
+        const uint32_t c = h[b], bin = q * HP_BINS + b;
+        if (c && bin < nbins) atomicAdd(&counts[bin], c);
+    }
+}
+static int hist_partitioned(uint32_t* counts, const uint32_t* idx, size_t n, uint32_t nbins, hipStream_t st) {
+    const uint32_t P = (nbins + HP_BINS - 1) / HP_BINS, ntiles = cdiv(n, HP_TILE), M = P * ntiles;
+    const uint32_t max_slices = (uint32_t)(n / HP_SLICE) + P + 1;
+    Scratch sizes(sizeof(uint32_t) * (size_t)M), part_off(sizeof(uint32_t) * (P + 1)), slice_tab(sizeof(uint32_t) * max_slices), nsl(sizeof(uint32_t)),
+        parted(sizeof(uint16_t) * n);
+    if (sizes.rc || part_off.rc || slice_tab.rc || nsl.rc || parted.rc) return sizes.rc ? sizes.rc : (part_off.rc ? part_off.rc : (slice_tab.rc ? slice_tab.rc : (nsl.rc ? nsl.rc : parted.rc)));
+    hipLaunchKernelGGL(k_hp_sizes, dim3(ntiles), dim3(TPB), 0, st, sizes.as<uint32_t>(), idx, n, P, ntiles);
+    hipLaunchKernelGGL(k_hp_scan, dim3(1), dim3(1024), 0, st, sizes.as<uint32_t>(), part_off.as<uint32_t>(), M, P, ntiles, (uint32_t)n);
+    hipLaunchKernelGGL(k_hp_slices, dim3(1), dim3(1024), 0, st, slice_tab.as<uint32_t>(), nsl.as<uint32_t>(), part_off.as<uint32_t>(), P);
+    hipLaunchKernelGGL(k_hp_scatter, dim3(ntiles), dim3(TPB), 0, st, parted.as<uint16_t>(), sizes.as<uint32_t>(), idx, n, P, ntiles);
+    hipLaunchKernelGGL(k_hp_count, dim3(max_slices), dim3(TPB), 0, st, counts, parted.as<uint16_t>(), part_off.as<uint32_t>(), slice_tab.as<uint32_t>(), nsl.as<uint32_t>(), nbins);
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
 // table[i] = low + min(i, len-1)  (tlookuprange_init_kernel tlookup.cu:372-380)
 __global__ void __launch_bounds__(TPB) k_range_table(Fr* __restrict__ table, int32_t low, uint32_t len, uint32_t table_size) {
     const uint32_t t = blockIdx.x * TPB + threadIdx.x;
@@ -893,6 +995,8 @@ int zk_lookup_hist(void* counts_u32, const void* idx_u32, size_t n, uint32_t nbi
         unsigned blocks = cdiv(n, (size_t)TPB * 16);
         if (blocks > 2048) blocks = 2048;
         hipLaunchKernelGGL(k_hist_lds, dim3(blocks), dim3(TPB), 0, st, (uint32_t*)counts_u32, (const uint32_t*)idx_u32, n, nbins);
+    } else if (n >= HP_MIN_QUERIES && n < ((size_t)1 << 32) && nbins <= HP_MAXP * HP_BINS) {
+        return hist_partitioned((uint32_t*)counts_u32, (const uint32_t*)idx_u32, n, nbins, st);
     } else {
         hipLaunchKernelGGL(k_hist_global, dim3(cdiv(n, (size_t)TPB * HH_PER_LANE)), dim3(TPB), 0, st, (uint32_t*)counts_u32, (const uint32_t*)idx_u32, n);
     }
