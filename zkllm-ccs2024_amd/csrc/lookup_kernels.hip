@@ -166,14 +166,36 @@ __global__ void __launch_bounds__(TPB) k_hp_sizes(uint32_t* __restrict__ sizes, 
     __syncthreads();
     for (uint32_t q = threadIdx.x; q < P; q += TPB) sizes[(size_t)q * ntiles + blockIdx.x] = c[q];
 }
-// one workgroup: a[0..M) -> its exclusive prefix sums (partition-major), part_off[q] = where partition q starts, part_off[P] = n
-__global__ void __launch_bounds__(1024) k_hp_scan(uint32_t* __restrict__ a, uint32_t* __restrict__ part_off, uint32_t M, uint32_t P, uint32_t ntiles, uint32_t n) {
+// workgroup q: row q of the sizes (one entry per tile) -> its exclusive prefix sums; totals[q] = the row's sum
+__global__ void __launch_bounds__(TPB) k_hp_rowscan(uint32_t* __restrict__ a, uint32_t* __restrict__ totals, uint32_t ntiles) {
+    __shared__ uint32_t part[TPB];
+    uint32_t* row = a + (size_t)blockIdx.x * ntiles;
+    const uint32_t t = threadIdx.x;
+    uint32_t carry = 0;
+    for (uint32_t base = 0; base < ntiles; base += TPB) {
+        const uint32_t i = base + t, v = i < ntiles ? row[i] : 0u;
+        part[t] = v;
+        __syncthreads();
+        for (uint32_t off = 1; off < (uint32_t)TPB; off <<= 1) {
+            const uint32_t x = t >= off ? part[t - off] : 0u;
+            __syncthreads();
+            part[t] += x;
+            __syncthreads();
+        }
+        if (i < ntiles) row[i] = carry + part[t] - v;
+        carry += part[TPB - 1];
+        __syncthreads();
+    }
+    if (t == 0) totals[blockIdx.x] = carry;
+}
+// one workgroup: part_off[q] = where partition q starts (part_off[P] = n), and the list of (partition, slice) pairs the
+// counting pass works through, slice_tab[k] = partition << 22 | slice
+__global__ void __launch_bounds__(1024) k_hp_slices(uint32_t* __restrict__ slice_tab, uint32_t* __restrict__ nslices, uint32_t* __restrict__ part_off,
+                                                    const uint32_t* __restrict__ totals, uint32_t P) {
     __shared__ uint32_t part[1024];
-    const uint32_t t = threadIdx.x, L = (M + 1023u) / 1024u;
-    const uint32_t b0 = t * L < M ? t * L : M, b1 = b0 + L < M ? b0 + L : M;
-    uint32_t s = 0;
-    for (uint32_t i = b0; i < b1; ++i) s += a[i];
-    part[t] = s;
+    const uint32_t t = threadIdx.x;
+    const uint32_t size = t < P ? totals[t] : 0u;
+    part[t] = size;
     __syncthreads();
     for (uint32_t off = 1; off < 1024u; off <<= 1) {
         const uint32_t v = t >= off ? part[t - off] : 0u;
@@ -181,20 +203,10 @@ __global__ void __launch_bounds__(1024) k_hp_scan(uint32_t* __restrict__ a, uint
         part[t] += v;
         __syncthreads();
     }
-    uint32_t run = part[t] - s;
-    for (uint32_t i = b0; i < b1; ++i) {
-        const uint32_t v = a[i];
-        a[i] = run;
-        if (i % ntiles == 0) part_off[i / ntiles] = run;
-        run += v;
-    }
-    if (t == 0) part_off[P] = n;
-}
-// one workgroup: the list of (partition, slice) pairs the counting pass works through, slice_tab[k] = partition << 22 | slice
-__global__ void __launch_bounds__(1024) k_hp_slices(uint32_t* __restrict__ slice_tab, uint32_t* __restrict__ nslices, const uint32_t* __restrict__ part_off, uint32_t P) {
-    __shared__ uint32_t part[1024];
-    const uint32_t t = threadIdx.x;
-    const uint32_t ns = t < P ? (part_off[t + 1] - part_off[t] + HP_SLICE - 1) / HP_SLICE : 0u;
+    if (t < P) part_off[t] = part[t] - size;
+    if (t == 1023u) part_off[P] = part[1023];
+    __syncthreads();
+    const uint32_t ns = (size + HP_SLICE - 1) / HP_SLICE;
     part[t] = ns;
     __syncthreads();
     for (uint32_t off = 1; off < 1024u; off <<= 1) {
@@ -207,10 +219,10 @@ __global__ void __launch_bounds__(1024) k_hp_slices(uint32_t* __restrict__ slice
     for (uint32_t q = 0; q < ns; ++q) slice_tab[o + q] = (t << 22) | q;
     if (t == 1023u) *nslices = part[1023];
 }
-__global__ void __launch_bounds__(TPB) k_hp_scatter(uint16_t* __restrict__ parted, const uint32_t* __restrict__ offs, const uint32_t* __restrict__ idx, size_t n, uint32_t P,
-                                                    uint32_t ntiles) {
+__global__ void __launch_bounds__(TPB) k_hp_scatter(uint16_t* __restrict__ parted, const uint32_t* __restrict__ offs, const uint32_t* __restrict__ part_off,
+                                                    const uint32_t* __restrict__ idx, size_t n, uint32_t P, uint32_t ntiles) {
     __shared__ uint32_t cur[HP_MAXP];
-    for (uint32_t q = threadIdx.x; q < P; q += TPB) cur[q] = offs[(size_t)q * ntiles + blockIdx.x];
+    for (uint32_t q = threadIdx.x; q < P; q += TPB) cur[q] = part_off[q] + offs[(size_t)q * ntiles + blockIdx.x];
     __syncthreads();
     const size_t base = (size_t)blockIdx.x * HP_TILE, end = base + HP_TILE < n ? base + HP_TILE : n;
     for (size_t i = base + threadIdx.x; i < end; i += TPB) {
@@ -238,13 +250,14 @@ __global__ void __launch_bounds__(TPB) k_hp_count(uint32_t* __restrict__ counts,
 static int hist_partitioned(uint32_t* counts, const uint32_t* idx, size_t n, uint32_t nbins, hipStream_t st) {
     const uint32_t P = (nbins + HP_BINS - 1) / HP_BINS, ntiles = cdiv(n, HP_TILE), M = P * ntiles;
     const uint32_t max_slices = (uint32_t)(n / HP_SLICE) + P + 1;
-    Scratch sizes(sizeof(uint32_t) * (size_t)M), part_off(sizeof(uint32_t) * (P + 1)), slice_tab(sizeof(uint32_t) * max_slices), nsl(sizeof(uint32_t)),
-        parted(sizeof(uint16_t) * n);
-    if (sizes.rc || part_off.rc || slice_tab.rc || nsl.rc || parted.rc) return sizes.rc ? sizes.rc : (part_off.rc ? part_off.rc : (slice_tab.rc ? slice_tab.rc : (nsl.rc ? nsl.rc : parted.rc)));
+    Scratch sizes(sizeof(uint32_t) * (size_t)M), part_off(sizeof(uint32_t) * (P + 1)), totals(sizeof(uint32_t) * P), slice_tab(sizeof(uint32_t) * max_slices),
+        nsl(sizeof(uint32_t)), parted(sizeof(uint16_t) * n);
+    for (const Scratch* b : {&sizes, &part_off, &totals, &slice_tab, &nsl, &parted})
+        if (b->rc) return b->rc;
     hipLaunchKernelGGL(k_hp_sizes, dim3(ntiles), dim3(TPB), 0, st, sizes.as<uint32_t>(), idx, n, P, ntiles);
-    hipLaunchKernelGGL(k_hp_scan, dim3(1), dim3(1024), 0, st, sizes.as<uint32_t>(), part_off.as<uint32_t>(), M, P, ntiles, (uint32_t)n);
-    hipLaunchKernelGGL(k_hp_slices, dim3(1), dim3(1024), 0, st, slice_tab.as<uint32_t>(), nsl.as<uint32_t>(), part_off.as<uint32_t>(), P);
-    hipLaunchKernelGGL(k_hp_scatter, dim3(ntiles), dim3(TPB), 0, st, parted.as<uint16_t>(), sizes.as<uint32_t>(), idx, n, P, ntiles);
+    hipLaunchKernelGGL(k_hp_rowscan, dim3(P), dim3(TPB), 0, st, sizes.as<uint32_t>(), totals.as<uint32_t>(), ntiles);
+    hipLaunchKernelGGL(k_hp_slices, dim3(1), dim3(1024), 0, st, slice_tab.as<uint32_t>(), nsl.as<uint32_t>(), part_off.as<uint32_t>(), totals.as<uint32_t>(), P);
+    hipLaunchKernelGGL(k_hp_scatter, dim3(ntiles), dim3(TPB), 0, st, parted.as<uint16_t>(), sizes.as<uint32_t>(), part_off.as<uint32_t>(), idx, n, P, ntiles);
     hipLaunchKernelGGL(k_hp_count, dim3(max_slices), dim3(TPB), 0, st, counts, parted.as<uint16_t>(), part_off.as<uint32_t>(), slice_tab.as<uint32_t>(), nsl.as<uint32_t>(), nbins);
     ZK_LAUNCH_CHECK();
     return 0;
