@@ -1,5 +1,7 @@
 #include "layer.hpp"
 
+#include <cstdlib>
+
 #include <chrono>
 #include <cmath>
 #include <random>
@@ -239,7 +241,7 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
 
     // Every challenge of this block, drawn first and in the order ffn.cu draws them (:67-69 the three of the activation
     // lookup, then inside the proofs of :83-93): the forward pass draws none.  The three weight openings need nothing but
-    // their points, so they start here and run beside the forward pass and the whole proof instead of behind them.
+    // their points, so they start as soon as the forward pass is queued and run beside the whole proof instead of behind it.
     const uint seq = input.size / c.embed_dim;
     auto temp_rand = random_vec(3);
     auto swiglu_u = random_vec(ceilLog2(c.seq_len * c.hidden_dim));
@@ -252,11 +254,6 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
     const auto ch_ur = Rescaling::draw(seq * c.hidden_dim);      // up_out
     const auto ch_u = up_layer.draw(seq);
     WeightOpeningAhead od, og, ou;
-    if (c.open_weights) {
-        ou = openWeightAhead(up, ch_u.u_input, ch_u.u_output);      // the two large ones first
-        og = openWeightAhead(gate, ch_g.u_input, ch_g.u_output);
-        od = openWeightAhead(down, ch_d.u_input, ch_d.u_output);
-    }
 
     auto up_out = up_layer(input);
     auto up_out_ = up_rescale(up_out);
@@ -269,6 +266,13 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
     auto down_in_ = hidden_rescale(down_in);
     auto down_out = down_layer(down_in_);
     auto down_out_ = down_rescale(down_out);
+    if (c.open_weights) {
+        // behind the forward pass (the openings are ordered after what is queued here): started before it, their kernels keep
+        // the forward pass's matrix products waiting for most of their own duration
+        ou = openWeightAhead(up, ch_u.u_input, ch_u.u_output);      // the two large ones first
+        og = openWeightAhead(gate, ch_g.u_input, ch_g.u_output);
+        od = openWeightAhead(down, ch_d.u_input, ch_d.u_output);
+    }
 
     {
         auto pd = down_rescale.prove_begin(down_out, down_out_, ch_dr);
