@@ -165,30 +165,39 @@ __global__ void __launch_bounds__(256) k_g1aff_to_a29(A29* __restrict__ out, con
 }
 
 // ---- fixed-base table for commit_int -------------------------------------------------------------------------
-// table (Jacobian, before normalisation): tab[(w * ngen + j) * half + (d-1)] = d * 2^(c*w) * G_j, d = 1..half
+// table (Jacobian, before normalisation): tab[(w * ngen + j) * half + (d-1)] = d * 2^(c*w) * G_j, d = 1..half.
+// One wave per (generator, window): the base by c*w doublings, then the multiples by doubling the filled part of the row,
+// row[k + l] = row[l] + row[k - 1] for l < k, k = 1, 2, 4, ... -- log2(half) additions deep instead of half of them in a row.
 __global__ void __launch_bounds__(GT) k_msm_table(G1Jac* __restrict__ tab, const G1Jac* __restrict__ gens, size_t ngen, uint32_t c, uint32_t nwin) {
-    const size_t j = (size_t)blockIdx.x * GT + threadIdx.x;
-    if (j >= ngen) return;
+    const size_t j = blockIdx.x;
+    const uint32_t w = blockIdx.y, l = threadIdx.x;
     const uint32_t half = 1u << (c - 1);
-    G1Jac base = gens[j];
-    for (uint32_t w = 0; w < nwin; ++w) {
-        G1Jac* row = tab + ((size_t)w * ngen + j) * half;
-        G1Jac acc = base;
-        row[0] = acc;
-        for (uint32_t d = 1; d < half; ++d) { acc = g1_add(acc, base); row[d] = acc; }
-        if (w + 1 < nwin) for (uint32_t k = 0; k < c; ++k) base = g1_double(base);
+    G1Jac* row = tab + ((size_t)w * ngen + j) * half;
+    if (l == 0) {
+        G1Jac base = gens[j];
+        for (uint32_t k = 0; k < c * w; ++k) base = g1_double(base);
+        row[0] = base;
+    }
+    __threadfence_block();
+    __syncthreads();
+    for (uint32_t k = 1; k < half; k <<= 1) {
+        const G1Jac top = row[k - 1];
+        for (uint32_t i = l; i < k && k + i < half; i += GT) row[k + i] = g1_add(row[i], top);
+        __threadfence_block();
+        __syncthreads();
     }
 }
 // One workgroup per (row, segment): sum_j [s_j] G_j over the segment as mixed additions out of the
-// affine table.  Scalars are embedded int32 values (commit_int_dev_func, commitment.cu:31-42).
-__global__ void __launch_bounds__(GT) k_msm_rows(G1Jac* __restrict__ out, const G1Affine* __restrict__ tab, const int32_t* __restrict__ scalars,
-                                                 size_t ngen, uint32_t c, uint32_t nwin, uint32_t nseg) {
+// affine table, in 29-bit limbs (the table is converted once per call).  Scalars are embedded int32 values
+// (commit_int_dev_func, commitment.cu:31-42).
+__global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+k_msm_rows(G1Jac* __restrict__ out, const A29* __restrict__ tab, const int32_t* __restrict__ scalars, size_t ngen, uint32_t c, uint32_t nwin, uint32_t nseg) {
     const size_t row = blockIdx.x;
     const uint32_t seg = blockIdx.y;
     const uint32_t half = 1u << (c - 1);
     const size_t per = (ngen + nseg - 1) / nseg;
     const size_t j0 = seg * per, j1 = (j0 + per < ngen) ? j0 + per : ngen;
-    G1Jac acc = g1_infinity();
+    J29 acc29 = j29_infinity();
     for (size_t j = j0 + threadIdx.x; j < j1; j += GT) {
         const int32_t s = scalars[row * ngen + j];
         if (s == 0) continue;
@@ -201,25 +210,37 @@ __global__ void __launch_bounds__(GT) k_msm_rows(G1Jac* __restrict__ out, const 
             if (d == 0) continue;
             const bool nd = (d < 0) != negs;
             const uint32_t mag = (uint32_t)(d < 0 ? -d : d);
-            G1Affine p = tab[((size_t)w * ngen + j) * half + (mag - 1)];
-            if (nd) p.y = neg(p.y);
-            acc = g1_add_mixed(acc, p);
+            A29 p = tab[((size_t)w * ngen + j) * half + (mag - 1)];
+            if (a29_is_inf(p)) continue;
+            if (nd) p.y = fq29_neg(p.y);
+            acc29 = j29_add_mixed(acc29, p);
         }
     }
-    acc = block_sum_g1(acc);
+    const G1Jac acc = block_sum_g1(j29_to_jac(acc29));
     if (threadIdx.x == 0) out[row * nseg + seg] = acc;
 }
 __global__ void __launch_bounds__(256) k_fr_to_i32_checked(int32_t* __restrict__ out, uint32_t* __restrict__ bad, uint32_t* __restrict__ maxabs, const Fr* __restrict__ in, size_t n) {
+    __shared__ uint32_t wmax[4];
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    const Fr x = in[i];
-    // scalar_to_int semantics: values outside the int32 embedding collapse to what the reference reads
-    const int32_t v = fr_to_i32(x);
-    out[i] = v;
-    const Fr back = fr_from_i64((int64_t)v);
-    if (!equal(back, x)) atomicOr(bad, 1u);
-    const uint32_t a = v < 0 ? (uint32_t)(-(int64_t)v) : (uint32_t)v;
-    if (a) atomicMax(maxabs, a);
+    uint32_t a = 0;
+    if (i < n) {
+        const Fr x = in[i];
+        // scalar_to_int semantics: values outside the int32 embedding collapse to what the reference reads
+        const int32_t v = fr_to_i32(x);
+        out[i] = v;
+        const Fr back = fr_from_i64((int64_t)v);
+        if (!equal(back, x)) atomicOr(bad, 1u);
+        a = v < 0 ? (uint32_t)(-(int64_t)v) : (uint32_t)v;
+    }
+    // one atomic per workgroup: the largest magnitude of its 256 values
+    for (int off = 32; off >= 1; off >>= 1) { const uint32_t o = (uint32_t)__shfl_xor((int)a, off, 64); a = o > a ? o : a; }
+    if ((threadIdx.x & 63u) == 0) wmax[threadIdx.x >> 6] = a;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t m = wmax[0];
+        for (int k = 1; k < 4; ++k) m = wmax[k] > m ? wmax[k] : m;
+        if (m) atomicMax(maxabs, m);
+    }
 }
 
 // ---- opening (Commitment::me_open, commitment.cu:79-129) -------------------------------------------------------------
@@ -1207,19 +1228,22 @@ int zk_g1_commit_int(void* out, const void* gens, const void* scalars_fr, size_t
     Scratch tabj(sizeof(G1Jac) * tab_n), taba(sizeof(G1Affine) * tab_n);
     if (tabj.rc) return tabj.rc;
     if (taba.rc) return taba.rc;
-    hipLaunchKernelGGL(k_msm_table, dim3(cdiv(ngen, GT)), dim3(GT), 0, st, tabj.as<G1Jac>(), (const G1Jac*)gens, ngen, c, nwin);
+    hipLaunchKernelGGL(k_msm_table, dim3((unsigned)ngen, nwin), dim3(GT), 0, st, tabj.as<G1Jac>(), (const G1Jac*)gens, ngen, c, nwin);
     hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(tab_n, CH), GT)), dim3(GT), 0, st, taba.p, tabj.as<G1Jac>(), tab_n);
+    Scratch tab29(sizeof(A29) * tab_n);
+    if (tab29.rc) return tab29.rc;
+    hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(tab_n, 256)), dim3(256), 0, st, tab29.as<A29>(), taba.as<G1Affine>(), tab_n);
     ZK_LAUNCH_CHECK();
     uint32_t nseg = 1;
     if (m < 2048) { nseg = (uint32_t)(2048 / m); const uint32_t cap = (uint32_t)((ngen + GT - 1) / GT); if (nseg > cap) nseg = cap; if (nseg < 1) nseg = 1; }
     if (nseg == 1) {
-        hipLaunchKernelGGL(k_msm_rows, dim3((unsigned)m, 1), dim3(GT), 0, st, (G1Jac*)out, taba.as<G1Affine>(), ints.as<int32_t>(), ngen, c, nwin, 1u);
+        hipLaunchKernelGGL(k_msm_rows, dim3((unsigned)m, 1), dim3(GT), 0, st, (G1Jac*)out, tab29.as<A29>(), ints.as<int32_t>(), ngen, c, nwin, 1u);
         ZK_LAUNCH_CHECK();
         return 0;
     }
     Scratch part(sizeof(G1Jac) * m * nseg);
     if (part.rc) return part.rc;
-    hipLaunchKernelGGL(k_msm_rows, dim3((unsigned)m, nseg), dim3(GT), 0, st, part.as<G1Jac>(), taba.as<G1Affine>(), ints.as<int32_t>(), ngen, c, nwin, nseg);
+    hipLaunchKernelGGL(k_msm_rows, dim3((unsigned)m, nseg), dim3(GT), 0, st, part.as<G1Jac>(), tab29.as<A29>(), ints.as<int32_t>(), ngen, c, nwin, nseg);
     hipLaunchKernelGGL(k_g1_rowsum, dim3((unsigned)m, 1), dim3(GT), 0, st, (G1Jac*)out, part.as<G1Jac>(), (size_t)nseg, 1u);
     ZK_LAUNCH_CHECK();
     return 0;
