@@ -176,6 +176,17 @@ int orc_poly_eval(const u32* coefs, int ncoef, const u32* x, u32* out) {
 int orc_hadamard_product_sumcheck(const u32* a, const u32* b, long n, const u32* u, const u32* v, long k, u32* proof_out) {
     ORC_TRY vec_out(hadamard_product_sumcheck(vec_in(a, n), vec_in(b, n), vec_in(u, k), vec_in(v, k)), proof_out); ORC_END
 }
+// proof_out: 3k+2 (inner product) or 3k+1 (binary) elements
+int orc_inner_product_sumcheck(const u32* a, const u32* b, long n, const u32* u, long k, u32* proof_out) {
+    ORC_TRY vec_out(inner_product_sumcheck(vec_in(a, n), vec_in(b, n), vec_in(u, k)), proof_out); ORC_END
+}
+int orc_binary_sumcheck(const u32* a, long n, const u32* u, const u32* v, long k, u32* proof_out) {
+    ORC_TRY vec_out(binary_sumcheck(vec_in(a, n), vec_in(u, k), vec_in(v, k)), proof_out); ORC_END
+}
+// even/odd: ceil(ceil(n/window)/2)*window elements each
+int orc_fr_split(const u32* t, long n, u32 window, u32* even, u32* odd) {
+    ORC_TRY auto pr = t_split(vec_in(t, n), window); vec_out(pr.first, even); vec_out(pr.second, odd); ORC_END
+}
 // Xs: nX tensors of n elements, concatenated. proof_out: per round (nX+1) coefficients. returns final claim.
 int orc_multi_hadamard(const u32* claim, const u32* Xs, int nX, long n, const u32* u, const u32* v, long k, u32* proof_out, u32* final_claim) {
     ORC_TRY

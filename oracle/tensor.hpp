@@ -489,6 +489,76 @@ static inline FrVec hadamard_product_sumcheck(const FrVec& a0, const FrVec& b0, 
     return proof;
 }
 
+// ---- deprecated inner-product and binary sumchecks (proof.cu:12-65, 109-155); the same raw products -------------
+// Adjacent pairs (2g, 2g+1), zero beyond the end; every round pushes the three sums (inner product) or the three
+// evaluations at the remaining u (binary), then folds by the round's challenge.
+static inline FrVec inner_product_sumcheck(const FrVec& a0, const FrVec& b0, const FrVec& u) {
+    uint ls = (uint)u.size();
+    need(a0.size() == b0.size(), "Incompatible dimensions");
+    need(!(a0.size() <= (1u << ls) / 2), "Incompatible dimensions");
+    need(!(a0.size() > (1u << ls)), "Incompatible dimensions");
+    FrVec proof, a = a0, b = b0;
+    for (size_t k = 0; k < u.size(); ++k) {
+        const long in_size = (long)a.size(), out_size = (in_size + 1) / 2;
+        Fr s0 = FR_ZERO, s1 = FR_ZERO, s2 = FR_ZERO;
+        for (long g = 0; g < out_size; ++g) {
+            long g0 = 2 * g, g1 = 2 * g + 1;
+            Fr x0 = g0 < in_size ? a[g0] : FR_ZERO, y0 = g0 < in_size ? b[g0] : FR_ZERO;
+            Fr x1 = g1 < in_size ? a[g1] : FR_ZERO, y1 = g1 < in_size ? b[g1] : FR_ZERO;
+            s0 = add(s0, mul(x0, y0));
+            s1 = add(s1, add(mul(x0, sub(y1, y0)), mul(y0, sub(x1, x0))));
+            s2 = add(s2, mul(sub(x1, x0), sub(y1, y0)));
+        }
+        proof.push_back(s0); proof.push_back(s1); proof.push_back(s2);
+        a = me_step(a, u[k]);
+        b = me_step(b, u[k]);
+    }
+    proof.push_back(a[0]);
+    proof.push_back(b[0]);
+    return proof;
+}
+static inline FrVec binary_sumcheck(const FrVec& a0, const FrVec& u, const FrVec& v) {
+    need(u.size() == v.size(), "Incompatible dimensions");
+    uint ls = (uint)u.size();
+    need(!(a0.size() <= (1u << ls) / 2), "Incompatible dimensions");
+    need(!(a0.size() > (1u << ls)), "Incompatible dimensions");
+    FrVec proof, a = a0;
+    for (size_t k = 0; k < u.size(); ++k) {
+        const long in_size = (long)a.size(), out_size = (in_size + 1) / 2;
+        FrVec o0(out_size), o1(out_size), o2(out_size);
+        for (long g = 0; g < out_size; ++g) {
+            long g0 = 2 * g, g1 = 2 * g + 1;
+            Fr x0 = g0 < in_size ? a[g0] : FR_ZERO, x1 = g1 < in_size ? a[g1] : FR_ZERO;
+            Fr diff = sub(x1, x0);
+            o0[g] = sub(mul(x0, x0), x0);
+            o1[g] = sub(mul(add(x0, x0), diff), diff);
+            o2[g] = mul(diff, diff);
+        }
+        // FrTensor::operator()(u_) checks the size range (fr-tensor.cu:437-442)
+        FrVec u_(u.begin() + k + 1, u.end());
+        proof.push_back(t_me(o0, u_));
+        proof.push_back(t_me(o1, u_));
+        proof.push_back(t_me(o2, u_));
+        a = me_step(a, v[k]);
+    }
+    proof.push_back(a[0]);
+    return proof;
+}
+
+// ---- FrTensor::split (fr-tensor.cu:562-585): even windows to the first tensor, odd windows to the second, zero beyond --
+static inline std::pair<FrVec, FrVec> t_split(const FrVec& t, uint window) {
+    need(!(window < 1 || window >= t.size()), "Invalid window size.");
+    uint nin = ((uint)t.size() + window - 1) / window, nout = (nin + 1) / 2, out_size = nout * window;
+    FrVec e(out_size, FR_ZERO), o(out_size, FR_ZERO);
+    for (uint g = 0; g < out_size; ++g) {
+        uint w = g / window, j = g % window;
+        size_t g0 = (size_t)2 * w * window + j, g1 = (size_t)(2 * w + 1) * window + j;
+        if (g0 < t.size()) e[g] = t[g0];
+        if (g1 < t.size()) o[g] = t[g1];
+    }
+    return {e, o};
+}
+
 // ---- multi_hadamard_sumchecks (proof.cu:172-241) ------------------------------------------------------------------
 static inline Fr multi_hadamard_sumchecks(const Fr& claim, const std::vector<FrVec>& Xs, const FrVec& u, const FrVec& v, std::vector<Poly>& proof) {
     const size_t N = Xs[0].size();

@@ -154,7 +154,7 @@ class Prover:
         L = self.lib
         for name in ("zkp_fr_from_i32", "zkp_fr_from_i64", "zkp_fr_from_fr", "zkp_fr_from_f32", "zkp_fr_from_f64", "zkp_fr_from_file",
                      "zkp_fr_devptr", "zkp_fr_binop", "zkp_fr_scalarop", "zkp_fr_partial_me", "zkp_fr_partial_me_window",
-                     "zkp_fr_pad", "zkp_fr_transpose", "zkp_fr_matmul", "zkp_fr_matmul_stack", "zkp_fr_transpose_stack",
+                     "zkp_fr_pad", "zkp_fr_split", "zkp_fr_transpose", "zkp_fr_matmul", "zkp_fr_matmul_stack", "zkp_fr_transpose_stack",
                      "zkp_g1_from_host", "zkp_g1_from_file", "zkp_g1_devptr", "zkp_commitment_random", "zkp_g1_binop", "zkp_g1_pointop",
                      "zkp_g1_scalar_mul", "zkp_g1_rowwise_sum", "zkp_commit_int", "zkp_commit",
                      "zkp_rescale", "zkp_rescale_prove", "zkp_relu", "zkp_attn", "zkp_zkfc_stacked", "zkp_range_prep", "zkp_batch_inv", "zkp_softmax",
@@ -349,6 +349,26 @@ class Prover:
         proof = np.zeros((3 * k + 2, 8), np.uint32)
         self.check(self.lib.zkp_hadamard_product_sumcheck(c_void_p(a.h), c_void_p(b.h), _np_ptr(u), _np_ptr(v), c_int(k), _np_ptr(proof)))
         return proof
+
+    def inner_product_sumcheck(self, a, b, u):
+        u = np.ascontiguousarray(u, dtype=np.uint32).reshape(-1, 8)
+        k = u.shape[0]
+        proof = np.zeros((3 * k + 2, 8), np.uint32)
+        self.check(self.lib.zkp_inner_product_sumcheck(c_void_p(a.h), c_void_p(b.h), _np_ptr(u), c_int(k), _np_ptr(proof)))
+        return proof
+
+    def binary_sumcheck(self, a, u, v):
+        u = np.ascontiguousarray(u, dtype=np.uint32).reshape(-1, 8)
+        v = np.ascontiguousarray(v, dtype=np.uint32).reshape(-1, 8)
+        k = u.shape[0]
+        proof = np.zeros((3 * k + 1, 8), np.uint32)
+        self.check(self.lib.zkp_binary_sumcheck(c_void_p(a.h), _np_ptr(u), _np_ptr(v), c_int(k), _np_ptr(proof)))
+        return proof
+
+    def split(self, t, window):
+        odd = c_void_p()
+        even = self.H(self.lib.zkp_fr_split(c_void_p(t.h), c_uint(window), ctypes.byref(odd)))
+        return even, self.H(odd.value)
 
     def softmax(self, X, m, n, d, bs, L, M, sf_in, thetas, prove):
         bs = np.ascontiguousarray(bs, dtype=np.uint32)

@@ -189,6 +189,23 @@ def test_pad_and_transpose(pv, orc):
         assert (pv.transpose(pv.from_fr(A), M, N).host() == exp).all(), (M, N)
 
 
+@pytest.mark.parametrize("n,w", [(8, 2), (8, 1), (13, 4), (10, 3), (7, 6), (4096 * 9 + 5, 4096), (100003, 7)])
+def test_split_into_even_and_odd_windows(pv, orc, n, w):
+    A = mt_random_vec(np.random.RandomState(n % 997), n)
+    out_n = ((-(-n // w) + 1) // 2) * w
+    e_exp, o_exp = np.zeros((out_n, 8), np.uint32), np.zeros((out_n, 8), np.uint32)
+    orc_check(orc.orc_fr_split(A, n, w, e_exp, o_exp))
+    even, odd = pv.split(pv.from_fr(A), w)
+    assert (even.host() == e_exp).all() and (odd.host() == o_exp).all()
+
+
+def test_split_rejects_bad_windows(pv):
+    t = pv.from_fr(mt_random_vec(np.random.RandomState(1), 4))
+    for w in (0, 4, 9):
+        with pytest.raises(RuntimeError, match="Invalid window size"):
+            pv.split(t, w)
+
+
 @pytest.mark.parametrize("M,N,P", [(1, 1, 1), (3, 4, 5), (16, 64, 64), (17, 9, 33), (40, 100, 24)])
 def test_matmul_generic_matches_oracle(pv, orc, M, N, P):
     print("case", M, N, P, flush=True)

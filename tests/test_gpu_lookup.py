@@ -202,6 +202,38 @@ def test_deprecated_hadamard_product_sumcheck(pv, orc, n):
     assert (got == exp).all()
 
 
+@pytest.mark.parametrize("n", [2, 3, 5, 64, 1000, 70001])
+def test_deprecated_inner_product_sumcheck(pv, orc, n):
+    a, b = ch(44, n), ch(45, n)
+    k = (n - 1).bit_length()
+    u = ch(46, k)
+    exp = np.zeros((3 * k + 2, 8), np.uint32)
+    orc_check(orc.orc_inner_product_sumcheck(a, b, n, u, k, exp))
+    got = pv.inner_product_sumcheck(pv.from_fr(a), pv.from_fr(b), u)
+    assert (got == exp).all()
+
+
+@pytest.mark.parametrize("n", [2, 3, 5, 64, 1000, 70001])
+def test_deprecated_binary_sumcheck(pv, orc, n):
+    a = ch(47, n)
+    k = (n - 1).bit_length()
+    u, v = ch(48, k), ch(49, k)
+    exp = np.zeros((3 * k + 1, 8), np.uint32)
+    orc_check(orc.orc_binary_sumcheck(a, n, u, v, k, exp))
+    got = pv.binary_sumcheck(pv.from_fr(a), u, v)
+    assert (got == exp).all()
+
+
+def test_deprecated_sumchecks_reject_sizes_out_of_range(pv):
+    a = pv.from_fr(ch(47, 4))
+    with pytest.raises(RuntimeError, match="Incompatible dimensions"):
+        pv.inner_product_sumcheck(a, a, ch(46, 3))
+    with pytest.raises(RuntimeError, match="Incompatible dimensions"):
+        pv.inner_product_sumcheck(a, pv.from_fr(ch(47, 3)), ch(46, 2))
+    with pytest.raises(RuntimeError, match="Incompatible dimensions"):
+        pv.binary_sumcheck(a, ch(46, 1), ch(48, 1))
+
+
 @pytest.mark.parametrize("N,D", [(2, 4), (4, 16), (3, 8), (32, 128)])
 def test_zkip_stacked(pv, orc, N, D):
     A, B = ch(50, N * D), ch(51, N * D)

@@ -334,6 +334,26 @@ int zkp_hadamard_product_sumcheck(void* a, void* b, const u32* u, const u32* v, 
     memcpy(proof_out, pr.data(), pr.size() * 32);
     ZKP_END
 }
+int zkp_inner_product_sumcheck(void* a, void* b, const u32* u, int k, u32* proof_out) {
+    ZKP_TRY
+    auto pr = inner_product_sumcheck(FT(a), FT(b), frs(u, k));
+    memcpy(proof_out, pr.data(), pr.size() * 32);
+    ZKP_END
+}
+int zkp_binary_sumcheck(void* a, const u32* u, const u32* v, int k, u32* proof_out) {
+    ZKP_TRY
+    auto pr = binary_sumcheck(FT(a), frs(u, k), frs(v, k));
+    memcpy(proof_out, pr.data(), pr.size() * 32);
+    ZKP_END
+}
+// FrTensor::split: returns the tensor of the even windows, *odd_out the odd ones
+void* zkp_fr_split(void* t, u32 window, void** odd_out) {
+    ZKP_TRY
+    auto pr = FT(t).split(window);
+    *odd_out = new FrTensor(std::move(pr.second));
+    return new FrTensor(std::move(pr.first));
+    ZKP_END_PTR
+}
 // zkSoftmax compute (+ prove with seeded challenges u_Y, v_Y, (r, alpha, beta)); returns Y, *shift_out the shift
 void* zkp_softmax(void* X, u32 m, u32 n, u32 d, const u32* bs, int K, u32 L, u32 M, uint64_t sf_in, const double* thetas, int nth, void** shift_out, int do_prove) {
     ZKP_TRY

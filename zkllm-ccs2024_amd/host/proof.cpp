@@ -175,7 +175,6 @@ vector<Fr_t> inner_product_sumcheck(const FrTensor& a0, const FrTensor& b0, vect
     if (a0.size != b0.size) throw std::runtime_error("Incompatible dimensions");
     if (a0.size <= (1u << log_size) / 2) throw std::runtime_error("Incompatible dimensions");
     if (a0.size > (1u << log_size)) throw std::runtime_error("Incompatible dimensions");
-    FrTensor a(a0), b(b0);
     std::vector<FrTensor> ka, kb;
     const FrTensor *pa = &a0, *pb = &b0;
     ka.reserve(u.size()); kb.reserve(u.size());
