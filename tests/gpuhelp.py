@@ -155,7 +155,7 @@ class Prover:
         for name in ("zkp_fr_from_i32", "zkp_fr_from_i64", "zkp_fr_from_fr", "zkp_fr_from_f32", "zkp_fr_from_f64", "zkp_fr_from_file",
                      "zkp_fr_devptr", "zkp_fr_binop", "zkp_fr_scalarop", "zkp_fr_partial_me", "zkp_fr_partial_me_window",
                      "zkp_fr_pad", "zkp_fr_split", "zkp_fr_transpose", "zkp_fr_matmul", "zkp_fr_matmul_stack", "zkp_fr_transpose_stack",
-                     "zkp_g1_from_host", "zkp_g1_from_file", "zkp_g1_devptr", "zkp_commitment_random", "zkp_g1_binop", "zkp_g1_pointop",
+                     "zkp_g1_from_host", "zkp_g1_from_file", "zkp_g1_devptr", "zkp_commitment_random", "zkp_g1_binop", "zkp_g1_pointop", "zkp_g1_affineop",
                      "zkp_g1_scalar_mul", "zkp_g1_rowwise_sum", "zkp_commit_int", "zkp_commit",
                      "zkp_rescale", "zkp_rescale_prove", "zkp_relu", "zkp_attn", "zkp_zkfc_stacked", "zkp_range_prep", "zkp_batch_inv", "zkp_softmax",
                      "zkp_layer_create", "zkp_layer_create_random", "zkp_layer_run"):
@@ -261,6 +261,11 @@ class Prover:
     def g1_pointop(self, op, a, p):
         p = np.ascontiguousarray(p, dtype=np.uint32).reshape(36)
         return self.G(self.lib.zkp_g1_pointop(c_int(op), c_void_p(a.h), _np_ptr(p)))
+
+    def g1_affineop(self, op, a, aff, path=None):
+        aff = np.ascontiguousarray(aff, dtype=np.uint32).reshape(-1, 24)
+        return self.G(self.lib.zkp_g1_affineop(c_int(op), c_void_p(a.h), _np_ptr(aff), c_uint(aff.shape[0]),
+                                               ctypes.c_char_p(path.encode() if path else None)))
 
     def g1_scalar_mul(self, g, s):
         return self.G(self.lib.zkp_g1_scalar_mul(c_void_p(g.h), c_void_p(s.h)))

@@ -78,6 +78,39 @@ def test_elementwise_and_special_cases(pv, orc):
     assert (norm(orc, pv.g1_pointop(2, hA, Pn).host()) == norm(orc, exp)).all()
 
 
+def test_affine_tensor_ops(pv, orc, tmp_path):
+    """G1TensorAffine against the Jacobian arithmetic of the oracle: mixed additions and subtractions (also in place,
+    with an equal point -> doubling, an opposite point -> infinity and an infinite left operand), negation, the
+    conversion, the file round trip and the element read."""
+    n = 70                                         # more than one workgroup
+    gens = oracle_gens(orc, 12, n)
+    A = gens.copy()
+    B = norm(orc, gens[::-1].copy())
+    B[0] = norm(orc, A[:1])[0]                     # equal
+    neg = np.zeros_like(A[:1])
+    orc_check(orc.orc_g1_op(4, A[1:2].copy(), A[1:2].copy(), neg, 1))
+    B[1] = norm(orc, neg)[0]                       # opposite
+    A[2] = np.zeros(36, np.uint32)                 # infinity + Q
+    aff = np.ascontiguousarray(B[:, :24])
+    hA = pv.g1_from_host(A)
+    exp, nb = np.zeros_like(A), np.zeros_like(B)
+    orc_check(orc.orc_g1_op(2, A, B, exp, n))
+    for op in (0, 2):
+        got = norm(orc, pv.g1_affineop(op, hA, aff).host())
+        assert (got == norm(orc, exp)).all() and not got[1].any()
+    orc_check(orc.orc_g1_op(4, B, B, nb, n))
+    orc_check(orc.orc_g1_op(2, A, nb, exp, n))
+    for op in (1, 3):
+        assert (norm(orc, pv.g1_affineop(op, hA, aff).host()) == norm(orc, exp)).all()
+    assert (pv.g1_affineop(4, hA, aff).host() == B).all()                          # z = one in Montgomery form
+    assert (pv.g1_affineop(5, hA, aff).host() == norm(orc, nb)).all()
+    assert (pv.g1_affineop(6, hA, aff, str(tmp_path / "aff.bin")).host() == B).all()
+    assert (tmp_path / "aff.bin").stat().st_size == n * 96
+    assert (pv.g1_affineop(7, hA, aff).host() == B[-1:]).all()
+    with pytest.raises(RuntimeError):
+        pv.g1_affineop(0, hA, aff[:5])
+
+
 def test_scalar_mul_sum_rowsum_me(pv, orc):
     gens = oracle_gens(orc, 12, 8)
     rng = random.Random(3)

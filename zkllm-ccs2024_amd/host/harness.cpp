@@ -223,6 +223,25 @@ void* zkp_g1_pointop(int op, void* a, const u32* p) {
     throw std::runtime_error("bad op");
     ZKP_END_PTR
 }
+// G1TensorAffine T of n points (24 limbs each, Montgomery x then y) from the host. op: 0 a + T, 1 a - T, 2 a += T,
+// 3 a -= T, 4 G1TensorJacobian(T), 5 G1TensorJacobian(-T), 6 G1TensorJacobian(T saved to path and loaded back),
+// 7 the one point T(n - 1) as a tensor of size 1
+void* zkp_g1_affineop(int op, void* a, const u32* aff, u32 n, const char* path) {
+    ZKP_TRY
+    G1TensorAffine T(n, (const G1Affine_t*)aff);
+    switch (op) {
+        case 0: return new Commitment(GT(a) + T);
+        case 1: return new Commitment(GT(a) - T);
+        case 2: { G1TensorJacobian c(GT(a)); c += T; return new Commitment(std::move(c)); }
+        case 3: { G1TensorJacobian c(GT(a)); c -= T; return new Commitment(std::move(c)); }
+        case 4: return new Commitment(G1TensorJacobian(T));
+        case 5: return new Commitment(G1TensorJacobian(-T));
+        case 6: { T.save(path); G1TensorAffine back{std::string(path)}; return new Commitment(G1TensorJacobian(back)); }
+        case 7: { G1Affine_t p = T(n - 1); return new Commitment(G1TensorJacobian(G1TensorAffine(1, p))); }
+    }
+    throw std::runtime_error("bad op");
+    ZKP_END_PTR
+}
 void* zkp_g1_scalar_mul(void* g, void* s) { ZKP_TRY return new Commitment(GT(g) * FT(s)); ZKP_END_PTR }
 int zkp_g1_sum(void* a, u32* out) { ZKP_TRY G1Jacobian_t s = GT(a).sum(); memcpy(out, &s, 144); ZKP_END }
 void* zkp_g1_rowwise_sum(void* a, u32 nrow, u32 ncol) { ZKP_TRY return new Commitment(GT(a).rowwise_sum(nrow, ncol)); ZKP_END_PTR }
