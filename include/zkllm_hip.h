@@ -121,6 +121,11 @@ int zk_g1_add(void* out, const void* a, const void* b, size_t n, size_t b_count,
 int zk_g1_madd(void* out, const void* a, const void* b_affine, size_t n, size_t b_count, int subtract, void* stream);
 /* out[i] = [s[i]] g[i % ng], s = Fr tensor read as 256-bit integers (G1_jacobian_elementwise_mul[_broadcast] :456-482) */
 int zk_g1_scalar_mul(void* out, const void* g, const void* s_fr, size_t ng, size_t n, void* stream);
+/* out[i] = [s_i] B for ONE base point B (host pointer: 36 limbs, Jacobian, Montgomery form) and n scalars in standard
+ * form on the device: the broadcast G1Jacobian_mul of Commitment::random (commitment.cu:3-8, the generator times random
+ * scalars; g1-tensor.cu:469-482).  Fixed-base windows: 33 mixed additions per scalar out of a table of B's multiples that
+ * stays on the device between calls with the same base.  Results equal zk_g1_scalar_mul's as group elements. */
+int zk_g1_fixed_base_mul(void* out, const uint32_t* base_host, const void* s_fr, size_t n, void* stream);
 int zk_g1_sum(uint32_t* out_host36, const void* a, size_t n, void* stream);               /* G1TensorJacobian::sum :391-443 */
 int zk_g1_rowwise_sum(void* out, const void* in, size_t nrow, size_t ncol, void* stream); /* rowwise_sum :535-625 */
 int zk_g1_me(uint32_t* out_host36, const void* a, size_t n, const uint32_t* u, int k, void* stream);   /* G1_me :486-514 */

@@ -273,3 +273,31 @@ def test_open_begin_end_matches_open_through_the_c_abi(orc):
     for _, _, _, dG, dS, _, _ in cases:
         hip.free(dG)
         hip.free(dS)
+
+
+def test_fixed_base_multiplication_equals_the_generic_one_and_big_integer_arithmetic(orc):
+    """zk_g1_fixed_base_mul (what Commitment::random runs on) against zk_g1_scalar_mul on the same base and, for the
+    small cases, against affine big-integer arithmetic: digits at the signed-window boundaries (127, 128, 129, bytes of
+    0x80 and 0xff that carry all the way up), zero, r - 1 and integers above r up to 2^256 - 1; a second base replaces the
+    table kept on the device and the first base builds it again."""
+    from gpuhelp import Hip, c_void_p, c_size_t
+    hip = Hip()
+    edge = [0, 1, 2, 127, 128, 129, 255, 256, 0x8080, 0x80 << 248, (1 << 255) - 1, R_MOD - 1, R_MOD, R_MOD + 5,
+            (1 << 256) - 1, int("80" * 32, 16), int("7f" * 32, 16), int("81" * 32, 16), 1 << 255]
+    S = np.concatenate([fr_array(edge), mt_random_vec(np.random.RandomState(77), 300)])
+    n = S.shape[0]
+    G = affine_to_jac((G1_X, G1_Y))
+    other = oracle_gens(orc, 91, 1)[0]
+    dS, dF, dM, dB = hip.upload(S), hip.malloc(144 * n), hip.malloc(144 * n), hip.malloc(144)
+    for base in (G, other, G):
+        base = np.ascontiguousarray(base, dtype=np.uint32)
+        hip.call("zk_memcpy_h2d", c_void_p(dB), base, c_size_t(144), None)
+        hip.call("zk_g1_fixed_base_mul", c_void_p(dF), base, c_void_p(dS), c_size_t(n), None)
+        hip.call("zk_g1_scalar_mul", c_void_p(dM), c_void_p(dB), c_void_p(dS), c_size_t(1), c_size_t(n), None)
+        fixed, generic = hip.download(dF, (n, 36), np.uint32), hip.download(dM, (n, 36), np.uint32)
+        assert (norm(orc, fixed) == norm(orc, generic)).all()
+        assert not norm(orc, fixed)[0].any()                     # [0] B is the point at infinity
+    for i in (1, 3, 4, 5, 11, 14):
+        assert jac_to_affine(fixed[i]) == ec_mul(edge[i] % R_MOD, (G1_X, G1_Y)), i
+    for p in (dS, dF, dM, dB):
+        hip.free(p)

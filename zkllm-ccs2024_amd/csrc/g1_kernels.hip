@@ -14,6 +14,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <utility>
 #include <vector>
 #include "fq29.hpp"
@@ -166,26 +167,26 @@ __global__ void __launch_bounds__(256) k_g1aff_to_a29(A29* __restrict__ out, con
 
 // ---- fixed-base table for commit_int -------------------------------------------------------------------------
 // table (Jacobian, before normalisation): tab[(w * ngen + j) * half + (d-1)] = d * 2^(c*w) * G_j, d = 1..half.
-// One wave per (generator, window): the base by c*w doublings, then the multiples by doubling the filled part of the row,
-// row[k + l] = row[l] + row[k - 1] for l < k, k = 1, 2, 4, ... -- log2(half) additions deep instead of half of them in a row.
-__global__ void __launch_bounds__(GT) k_msm_table(G1Jac* __restrict__ tab, const G1Jac* __restrict__ gens, size_t ngen, uint32_t c, uint32_t nwin) {
-    const size_t j = blockIdx.x;
-    const uint32_t w = blockIdx.y, l = threadIdx.x;
+// Bases first, one lane per generator walking up the windows by c doublings each; then the multiples by doubling the
+// filled part of every row, row[k + i] = row[i] + row[k - 1] for i < k, k = 1, 2, 4, ...: one launch per k with one lane
+// per new entry, so every launch is dense whatever the row length (rows are as short as 4 entries when few tensor rows
+// share the generators) and the chain of additions is log2(half) deep.
+__global__ void __launch_bounds__(GT) k_msm_table_bases(G1Jac* __restrict__ tab, const G1Jac* __restrict__ gens, size_t ngen, uint32_t c, uint32_t nwin) {
+    const size_t j = (size_t)blockIdx.x * GT + threadIdx.x;
+    if (j >= ngen) return;
     const uint32_t half = 1u << (c - 1);
-    G1Jac* row = tab + ((size_t)w * ngen + j) * half;
-    if (l == 0) {
-        G1Jac base = gens[j];
-        for (uint32_t k = 0; k < c * w; ++k) base = g1_double(base);
-        row[0] = base;
+    G1Jac base = gens[j];
+    for (uint32_t w = 0; w < nwin; ++w) {
+        tab[((size_t)w * ngen + j) * half] = base;
+        if (w + 1 < nwin) for (uint32_t k = 0; k < c; ++k) base = g1_double(base);
     }
-    __threadfence_block();
-    __syncthreads();
-    for (uint32_t k = 1; k < half; k <<= 1) {
-        const G1Jac top = row[k - 1];
-        for (uint32_t i = l; i < k && k + i < half; i += GT) row[k + i] = g1_add(row[i], top);
-        __threadfence_block();
-        __syncthreads();
-    }
+}
+__global__ void __launch_bounds__(GT) k_msm_table_fill(G1Jac* __restrict__ tab, size_t nrows, uint32_t logh, uint32_t logk) {
+    const size_t t = (size_t)blockIdx.x * GT + threadIdx.x;
+    if ((t >> logk) >= nrows) return;
+    const uint32_t k = 1u << logk, i = (uint32_t)(t & (k - 1));
+    G1Jac* row = tab + ((t >> logk) << logh);
+    row[k + i] = g1_add(row[i], row[k - 1]);
 }
 // One workgroup per (row, segment): sum_j [s_j] G_j over the segment as mixed additions out of the
 // affine table, in 29-bit limbs (the table is converted once per call).  Scalars are embedded int32 values
@@ -218,6 +219,29 @@ k_msm_rows(G1Jac* __restrict__ out, const A29* __restrict__ tab, const int32_t* 
     }
     const G1Jac acc = block_sum_g1(j29_to_jac(acc29));
     if (threadIdx.x == 0) out[row * nseg + seg] = acc;
+}
+// out[i] = [s_i] B for one base point B: additions out of the table of B's multiples d * 2^(8w) B, d = 1..128, w = 0..32
+// (signed 8-bit digits of the 256-bit integer s_i; window 32 only ever holds the last carry).  33 mixed additions at
+// most instead of 255 doublings and ~128 additions.
+static constexpr uint32_t FB_WIN = 33;
+__global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+k_g1_fixed_base_mul(G1Jac* __restrict__ out, const A29* __restrict__ tab, const Fr* __restrict__ scalars, size_t n) {
+    const size_t i = (size_t)blockIdx.x * GT + threadIdx.x;
+    if (i >= n) return;
+    const Fr x = scalars[i];
+    J29 acc29 = j29_infinity();
+    uint32_t carry = 0;
+    for (uint32_t w = 0; w < FB_WIN; ++w) {
+        const uint32_t b = (w < 32 ? ((x.v[w >> 2] >> (8 * (w & 3))) & 255u) : 0u) + carry;
+        carry = b > 128u ? 1u : 0u;
+        const uint32_t mag = carry ? 256u - b : b;
+        if (mag == 0) continue;
+        A29 p = tab[w * 128u + (mag - 1)];
+        if (a29_is_inf(p)) continue;
+        if (carry) p.y = fq29_neg(p.y);
+        acc29 = j29_add_mixed(acc29, p);
+    }
+    out[i] = j29_to_jac(acc29);
 }
 __global__ void __launch_bounds__(256) k_fr_to_i32_checked(int32_t* __restrict__ out, uint32_t* __restrict__ bad, uint32_t* __restrict__ maxabs, const Fr* __restrict__ in, size_t n) {
     __shared__ uint32_t wmax[4];
@@ -1228,7 +1252,9 @@ int zk_g1_commit_int(void* out, const void* gens, const void* scalars_fr, size_t
     Scratch tabj(sizeof(G1Jac) * tab_n), taba(sizeof(G1Affine) * tab_n);
     if (tabj.rc) return tabj.rc;
     if (taba.rc) return taba.rc;
-    hipLaunchKernelGGL(k_msm_table, dim3((unsigned)ngen, nwin), dim3(GT), 0, st, tabj.as<G1Jac>(), (const G1Jac*)gens, ngen, c, nwin);
+    hipLaunchKernelGGL(k_msm_table_bases, dim3(cdiv(ngen, GT)), dim3(GT), 0, st, tabj.as<G1Jac>(), (const G1Jac*)gens, ngen, c, nwin);
+    for (uint32_t logk = 0; logk + 1 < c; ++logk)
+        hipLaunchKernelGGL(k_msm_table_fill, dim3(cdiv(((size_t)nwin * ngen) << logk, GT)), dim3(GT), 0, st, tabj.as<G1Jac>(), (size_t)nwin * ngen, c - 1, logk);
     hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(tab_n, CH), GT)), dim3(GT), 0, st, taba.p, tabj.as<G1Jac>(), tab_n);
     Scratch tab29(sizeof(A29) * tab_n);
     if (tab29.rc) return tab29.rc;
@@ -1245,6 +1271,44 @@ int zk_g1_commit_int(void* out, const void* gens, const void* scalars_fr, size_t
     if (part.rc) return part.rc;
     hipLaunchKernelGGL(k_msm_rows, dim3((unsigned)m, nseg), dim3(GT), 0, st, part.as<G1Jac>(), tab29.as<A29>(), ints.as<int32_t>(), ngen, c, nwin, nseg);
     hipLaunchKernelGGL(k_g1_rowsum, dim3((unsigned)m, 1), dim3(GT), 0, st, (G1Jac*)out, part.as<G1Jac>(), (size_t)nseg, 1u);
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
+
+// out[i] = [s_i] B for a base point B given on the host (Jacobian, Montgomery form) and n scalars in standard form: what
+// Commitment::random does with the group generator (commitment.cu:3-8, a broadcast G1Jacobian_mul).  The table of B's
+// multiples is kept on the device from one call to the next with the same base (one table per process, 4224 points).
+int zk_g1_fixed_base_mul(void* out, const uint32_t* base_host, const void* scalars_fr, size_t n, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    if (n == 0) return 0;
+    static std::mutex mu;
+    static void* tab = nullptr;
+    static int tab_dev = -1;
+    static uint32_t tab_base[36];
+    std::lock_guard<std::mutex> lk(mu);
+    int dev = 0;
+    ZK_HIP(hipGetDevice(&dev));
+    if (!tab || tab_dev != dev || std::memcmp(tab_base, base_host, sizeof(tab_base)) != 0) {
+        const size_t tab_n = (size_t)FB_WIN * 128;
+        if (tab && tab_dev != dev) { int cur = dev; ZK_HIP(hipSetDevice(tab_dev)); ZK_HIP(hipFree(tab)); ZK_HIP(hipSetDevice(cur)); tab = nullptr; }
+        if (!tab) ZK_HIP(hipMalloc(&tab, sizeof(A29) * tab_n));
+        tab_dev = -1;                                   // not valid until the build below has finished
+        Scratch b(sizeof(G1Jac)), tabj(sizeof(G1Jac) * tab_n), taba(sizeof(G1Affine) * tab_n);
+        if (b.rc) return b.rc;
+        if (tabj.rc) return tabj.rc;
+        if (taba.rc) return taba.rc;
+        ZK_HIP(hipMemcpyAsync(b.p, base_host, sizeof(G1Jac), hipMemcpyHostToDevice, st));
+        hipLaunchKernelGGL(k_msm_table_bases, dim3(1), dim3(GT), 0, st, tabj.as<G1Jac>(), b.as<G1Jac>(), (size_t)1, 8u, FB_WIN);
+        for (uint32_t logk = 0; logk < 7; ++logk)
+            hipLaunchKernelGGL(k_msm_table_fill, dim3(cdiv((size_t)FB_WIN << logk, GT)), dim3(GT), 0, st, tabj.as<G1Jac>(), (size_t)FB_WIN, 7u, logk);
+        hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(tab_n, CH), GT)), dim3(GT), 0, st, taba.p, tabj.as<G1Jac>(), tab_n);
+        hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(tab_n, 256)), dim3(256), 0, st, (A29*)tab, taba.as<G1Affine>(), tab_n);
+        ZK_LAUNCH_CHECK();
+        ZK_HIP(hipStreamSynchronize(st));               // later calls may come on other streams
+        std::memcpy(tab_base, base_host, sizeof(tab_base));
+        tab_dev = dev;
+    }
+    hipLaunchKernelGGL(k_g1_fixed_base_mul, dim3(cdiv(n, GT)), dim3(GT), 0, st, (G1Jac*)out, (const A29*)tab, (const Fr*)scalars_fr, n);
     ZK_LAUNCH_CHECK();
     return 0;
 }

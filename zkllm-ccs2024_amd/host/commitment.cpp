@@ -13,8 +13,10 @@ void zk_set_skip_g1_opening(bool skip) { g_skip_g1 = skip; }
 // generators [s_i]G with s_i from the (seedable) challenge stream; the reference draws s_i from cuRAND
 // (commitment.cu:3-8, fr-tensor.cu:479-510)
 Commitment Commitment::random(uint size) {
-    Commitment out(size, G1Jacobian_generator);
-    out *= FrTensor::random(size);
+    // the generator times random scalars, as a fixed-base multiplication
+    Commitment out(size);
+    FrTensor s = FrTensor::random(size);
+    ZKC(zk_g1_fixed_base_mul(out.gpu_data, (const uint32_t*)&G1Jacobian_generator, s.gpu_data, size, nullptr));
     return out;
 }
 
