@@ -114,5 +114,7 @@ Weight create_weight(string generator_filename, string weight_filename, string c
     Commitment generator(generator_filename);
     FrTensor weight = FrTensor::from_int_bin(weight_filename);
     G1TensorJacobian com(com_filename);
-    return {generator, weight, com, in_dim, out_dim};
+    Weight w{generator, weight, com, in_dim, out_dim, nullptr};
+    if (in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim))) w.padded = std::make_shared<const FrTensor>(w.weight.pad({in_dim, out_dim}));
+    return w;
 }

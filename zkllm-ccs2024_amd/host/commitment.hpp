@@ -44,6 +44,10 @@ struct Weight {
     G1TensorJacobian com;
     uint in_dim;
     uint out_dim;
+    // addition: the weight padded to powers of two in both dimensions, the form that is committed and opened
+    // (proof.cu:3-10 pads at every opening).  Set where the weight is loaded or made when a dimension is not a power of
+    // two; verifyWeightClaim pads on the spot when it is needed and absent.
+    std::shared_ptr<const FrTensor> padded;
 };
 
 Weight create_weight(string generator_filename, string weight_filename, string com_filename, uint in_dim, uint out_dim);

@@ -1,3 +1,4 @@
+#include <memory>
 #include "fr-tensor.hpp"
 
 #include <climits>
@@ -329,14 +330,25 @@ FrTensor FrTensor::pad(const vector<uint>& shape, const Fr_t& pad_val) const {
     size_t cum = 1;
     for (auto& s : shape) cum *= s;
     if (cum != size) throw std::runtime_error("pad: cum_shape != size");
-    uint last_dim = shape.back();
-    uint last_dim_padded = 1u << ceilLog2(last_dim);
-    FrTensor out((uint)((cum / last_dim) * last_dim_padded));
-    ZKC(zk_fr_pad(out.gpu_data, gpu_data, cum / last_dim, last_dim, last_dim_padded, pad_val.val, nullptr));
-    if (shape.size() == 1) return out;
-    vector<uint> shape_new(shape.begin(), shape.end() - 1);
-    shape_new.back() *= last_dim_padded;
-    return out.pad(shape_new, pad_val);
+    // fr-tensor.cu:800-828 pads the last dimension, merges it into the one before and repeats; a level whose length already
+    // is a power of two changes nothing and takes no pass here
+    vector<uint> sh(shape);
+    std::unique_ptr<FrTensor> cur;
+    for (;;) {
+        const FrTensor& src = cur ? *cur : *this;
+        const uint last_dim = sh.back(), last_dim_padded = 1u << ceilLog2(last_dim);
+        if (last_dim != last_dim_padded) {
+            const size_t rows = src.size / last_dim;
+            std::unique_ptr<FrTensor> out(new FrTensor((uint)(rows * last_dim_padded)));
+            ZKC(zk_fr_pad(out->gpu_data, src.gpu_data, rows, last_dim, last_dim_padded, pad_val.val, nullptr));
+            cur = std::move(out);
+        }
+        if (sh.size() == 1) break;
+        sh.pop_back();
+        sh.back() *= last_dim_padded;
+    }
+    if (!cur) return FrTensor(*this);
+    return FrTensor(std::move(*cur));
 }
 
 FrTensor FrTensor::transpose(uint M, uint N) const {

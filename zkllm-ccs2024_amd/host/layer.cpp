@@ -333,9 +333,10 @@ static Weight random_weight(std::mt19937_64& rng, uint in_dim, uint out_dim, uin
     for (auto& x : wi) x = norm ? 65536 : (int)std::nearbyint(nd(rng) * 65536.0);   // scale 2^16 (llama-commit.py:34)
     FrTensor weight((uint)wi.size(), wi.data());
     Commitment gen = Commitment::random(1u << ceilLog2(pp_size));
-    FrTensor padded = weight.pad({in_dim, out_dim});
-    G1TensorJacobian com = gen.commit_int(padded);
-    return Weight{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim};
+    const bool ragged = in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim));
+    std::shared_ptr<const FrTensor> padded = ragged ? std::make_shared<const FrTensor>(weight.pad({in_dim, out_dim})) : nullptr;
+    G1TensorJacobian com = gen.commit_int(ragged ? *padded : weight);
+    return Weight{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim, std::move(padded)};
 }
 
 LayerWeights make_random_layer_weights(const LayerConfig& c, uint32_t seed, uint lof) {

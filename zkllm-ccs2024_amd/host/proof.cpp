@@ -1,3 +1,4 @@
+#include <memory>
 #include "proof.hpp"
 
 #include "../../include/zkllm_hip.h"
@@ -39,9 +40,18 @@ void DeferredOpenings::finish() {
 }
 
 // proof.cu:3-10
+// the weight in its committed form: itself when both dimensions are powers of two, else the padded tensor kept with it,
+// else padded here into `local`
+static const FrTensor& padded_form(const Weight& w, std::unique_ptr<FrTensor>& local) {
+    if (w.in_dim == (1u << ceilLog2(w.in_dim)) && w.out_dim == (1u << ceilLog2(w.out_dim))) return w.weight;
+    if (w.padded) return *w.padded;
+    local.reset(new FrTensor(w.weight.pad({w.in_dim, w.out_dim})));
+    return *local;
+}
 void verifyWeightClaim(const Weight& w, const Claim& c) {
     vector<Fr_t> u_cat = concatenate(vector<vector<Fr_t>>({c.u[1], c.u[0]}));
-    auto w_padded = w.weight.pad({w.in_dim, w.out_dim});
+    std::unique_ptr<FrTensor> local;
+    const FrTensor& w_padded = padded_form(w, local);
     if (g_deferred) {
         DeferredOpenings::Item* it = new DeferredOpenings::Item{w.generator.open_begin(w_padded, w.com, u_cat), c.claim, zk_record_reserve()};
         g_deferred->items.push_back(it);
@@ -70,8 +80,8 @@ WeightOpeningAhead openWeightAhead(const Weight& w, const vector<Fr_t>& u_input,
     if (!g_deferred) return a;            // nothing runs ahead outside a deferred scope
     a.impl = new WeightOpeningAhead::Impl;
     a.impl->u_cat = concatenate(vector<vector<Fr_t>>({u_output, u_input}));
-    auto w_padded = w.weight.pad({w.in_dim, w.out_dim});
-    a.impl->op = w.generator.open_begin(w_padded, w.com, a.impl->u_cat);
+    std::unique_ptr<FrTensor> local;
+    a.impl->op = w.generator.open_begin(padded_form(w, local), w.com, a.impl->u_cat);
     return a;
 }
 void verifyWeightClaim(const Weight& w, const Claim& c, WeightOpeningAhead& ahead) {

@@ -7,13 +7,13 @@
 Rescaling::Rescaling(uint scaling_factor) : scaling_factor(scaling_factor), tl_rem(-static_cast<int>(scaling_factor >> 1), scaling_factor), rem_tensor_ptr(nullptr) {}
 
 FrTensor Rescaling::operator()(const FrTensor& X) {
-    if (rem_tensor_ptr) delete rem_tensor_ptr;
-    rem_tensor_ptr = new FrTensor(X.size);
+    rem_hold = std::make_shared<FrTensor>(X.size);
+    rem_tensor_ptr = rem_hold.get();
     FrTensor out(X.size);
     ZKC(zk_rescale(out.gpu_data, rem_tensor_ptr->gpu_data, X.gpu_data, scaling_factor, X.size, nullptr));
     return out;
 }
-Rescaling::~Rescaling() { if (rem_tensor_ptr) delete rem_tensor_ptr; }
+Rescaling::~Rescaling() {}
 
 // rescaling.cu:41-79.  Challenge order: u, v, (alpha, beta).
 vector<Claim> Rescaling::prove(const FrTensor& X, const FrTensor& X_) {
@@ -40,7 +40,8 @@ Rescaling::Pending Rescaling::prove_begin(const FrTensor& X, const FrTensor& X_,
     if (u.size() != ceilLog2(X.size) || v.size() != u.size() || rand_temp.size() != 2) throw std::runtime_error("Rescaling::prove: challenges do not match the shape");
 
     Pending p;
-    p.rem.reset(new FrTensor(rem_tensor_ptr->pad({rem_tensor_ptr->size})));
+    if (rem_tensor_ptr->size == (1u << ceilLog2(rem_tensor_ptr->size))) p.rem = rem_hold;
+    else p.rem = std::make_shared<FrTensor>(rem_tensor_ptr->pad({rem_tensor_ptr->size}));
     p.m.reset(new FrTensor(tl_rem.prep(*p.rem)));
     // X(u), X_(u), rem(u): one pass over the tensors that have the same length (the remainder is padded to a power of two)
     vector<Fr_t> ev;

@@ -9,7 +9,7 @@ class Rescaling {
    public:
     uint scaling_factor;
     tLookupRange tl_rem;   // table for the remainder
-    FrTensor* rem_tensor_ptr;
+    FrTensor* rem_tensor_ptr;   // the remainders of the last operator() call (owned through rem_hold)
 
     Rescaling(uint scaling_factor);
     FrTensor operator()(const FrTensor& X);
@@ -19,7 +19,8 @@ class Rescaling {
     // in between may all be begun before the first is ended: challenges and entries keep their order.
     struct Pending {
         Fr_t lhs;
-        std::unique_ptr<FrTensor> rem, m;
+        std::shared_ptr<FrTensor> rem;   // the remainder tensor itself when its length is a power of two, else a padded copy
+        std::unique_ptr<FrTensor> m;
         LookupPending look;
     };
     Pending prove_begin(const FrTensor& X, const FrTensor& X_);
@@ -31,4 +32,7 @@ class Rescaling {
     ~Rescaling();
     Rescaling(const Rescaling&) = delete;
     Rescaling& operator=(const Rescaling&) = delete;
+
+   private:
+    std::shared_ptr<FrTensor> rem_hold;   // shared with the proofs begun on it, which may outlive the next operator() call
 };
