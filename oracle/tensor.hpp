@@ -2,11 +2,12 @@
 //
 // Restates, as plain loops over std::vector<Fr>, the reference's kernels and host recursions:
 //   fr-tensor.cu   elementwise ops :71-153, sum :382-434, Fr_me :588-609, window fold :612-641,
-//                  multi-dim fold :518-560, multi_dim_me :643-652, pad :800-828, matmul :831-881,
+//                  multi-dim fold :518-560, split :562-585, multi_dim_me :643-652, pad :800-828, matmul :831-881,
 //                  transpose :885-900, random_vec :16-24, ceilLog2 :26-43
 //   polynomial.cu  host Fr operators :4-150, Polynomial :152-329, eq :342-372
 //   zkfc.cu        zkip :94-151, zkip_stacked :153-229, zkFC::prove :61-87, zkFCStacked :261-307
-//   proof.cu       hadamard_product_sumcheck :67-107, multi_hadamard_sumchecks :172-241
+//   proof.cu       inner_product_sumcheck :12-65, hadamard_product_sumcheck :67-107, binary_sumcheck :109-155,
+//                  multi_hadamard_sumchecks :172-241
 // Every value is the canonical residue in [0, r), so summation order is free.
 // OpenMP parallel loops are used where the reference launches one thread per element; this
 // file is also the CPU baseline timed by the benchmark.
