@@ -376,3 +376,43 @@ def test_stacks_of_matrices_transpose_and_multiply_like_their_members(pv):
     T = rng.integers(-2 ** 40, 2 ** 40, (5, 37, 70)).astype(np.int64)
     got = pv.transpose_stack(pv.from_i64(T), 5, 37, 70).host()
     assert fr_ints(got) == [int(v) % R_MOD for v in T.transpose(0, 2, 1).reshape(-1)]
+
+
+def test_config2_full_size_fully_connected_proof_passes_the_verifier(pv):
+    """X 2048 x 4096 times W 4096 x 4096 (fixed point, scale 2^16, N(0, 0.02)), beyond what the oracle can follow: rows
+    of the product are compared with int64 arithmetic, and the proof transcript under a seeded stream is checked as a
+    verifier would in big integers: the claim is Y at (u_batch, u_output), each of the 12 rounds satisfies p(0) + p(1) =
+    claim and hands on p(v), and the last claim is X(u_batch, u_input) * W(u_input, u_output), both recomputed from the
+    full tensors apart from the proof."""
+    B, I, O = 2048, 4096, 4096
+    rng = np.random.default_rng(20242)
+    X = np.round(rng.normal(0, 0.02, (B, I)) * 65536).astype(np.int32)
+    W = np.round(rng.normal(0, 0.02, (I, O)) * 65536).astype(np.int32)
+    hX, hW = pv.from_i32(X), pv.from_i32(W)
+    hY = pv.matmul(hX, hW, B, I, O)
+    Y = hY.host()
+    for r in (0, 777, 2047):
+        exp = X[r].astype(np.int64) @ W.astype(np.int64)
+        assert fr_ints(Y[r * O:(r + 1) * O]) == [int(v) % R_MOD for v in exp], r
+    del Y
+    seed = 909
+    pv.seed(seed)
+    pv.transcript_begin()
+    pv.zkfc_prove(hX, hW, hY, I, O)
+    pv.lib.zkp_transcript_end()
+    t = fr_ints(pv.transcript())
+    rs = np.random.RandomState(seed)
+    u_b, u_i, u_o = mt_random_vec(rs, 11), mt_random_vec(rs, 12), mt_random_vec(rs, 12)
+    assert len(t) == 1 + 3 * 12 + 3
+    claim = t[0]
+    assert [claim] == fr_ints(pv.multi_dim_me(hY, [u_b, u_o], (B, O)))
+    vi = fr_ints(u_i)
+    for r in range(12):
+        c0, c1, c2 = t[1 + 3 * r:4 + 3 * r]
+        assert (2 * c0 + c1 + c2) % R_MOD == claim, r
+        v = vi[11 - r]                                   # the rounds consume u_input from the back
+        claim = (c0 + c1 * v + c2 * v * v) % R_MOD
+    final, cX, cW = t[37:40]
+    assert final == claim and cX * cW % R_MOD == final
+    assert [cX] == fr_ints(pv.multi_dim_me(hX, [u_b, u_i], (B, I)))
+    assert [cW] == fr_ints(pv.multi_dim_me(hW, [u_i, u_o], (I, O)))

@@ -301,3 +301,45 @@ def test_fixed_base_multiplication_equals_the_generic_one_and_big_integer_arithm
         assert jac_to_affine(fixed[i]) == ec_mul(edge[i] % R_MOD, (G1_X, G1_Y)), i
     for p in (dS, dF, dM, dB):
         hip.free(p)
+
+
+def test_config3_full_size_commitment_and_opening_pass_the_verifier(pv, orc):
+    """A 11008 x 4096 fixed-point weight (scale 2^16, N(0, 0.02)) over 4096 generators, far beyond what the oracle can
+    follow: the 11008 commitments and the opening at a random point are checked the way a verifier would, in big-integer
+    affine arithmetic.  The first T of the opening is the commitments' own multilinear extension at the row challenges
+    (this ties commit_int to the opening), every round satisfies T' = u(1-u) T + (1-u)^2 T0 + u^2 T1, the last one
+    against [value] g_final, and the value is the tensor's multilinear extension computed apart from the opening."""
+    m, n = 11008, 4096
+    rng = np.random.default_rng(2024)
+    W = np.round(rng.normal(0, 0.02, m * n) * 65536).astype(np.int32)
+    pv.seed(33)
+    hG = pv.commitment_random(n)
+    hW = pv.from_i32(W)
+    com = pv.commit_int(hG, hW)
+    assert com.size == m
+    k_in, k_out = 12, 14
+    u = mt_random_vec(np.random.RandomState(34), k_in + k_out)
+    val, proof = pv.open(hG, hW, com, u)
+    assert proof.shape[0] == 3 * k_in + 1
+    ui = fr_ints(u)
+    # value = W(u_out, u_in), rows by the last 14 challenges
+    assert (pv.multi_dim_me(hW, [u[k_in:], u[:k_in]], (m, n)) == val).all()
+    # T of the first round = sum_rows eq(u_out, row) com_row; G1TensorJacobian::operator()(u) reads its challenges as u / R
+    u_me = fr_array([x * (1 << 256) % R_MOD for x in ui[k_in:]])
+    pts = [jac_to_affine(p) for p in proof]
+    assert pts[0] == jac_to_affine(pv.g1_me(com, u_me))
+    for r in range(k_in):
+        x = ui[r]
+        T, T0, T1 = pts[3 * r:3 * r + 3]
+        nxt = ec_add(ec_add(ec_mul(x * (1 - x) % R_MOD, T), ec_mul((1 - x) * (1 - x) % R_MOD, T0)), ec_mul(x * x % R_MOD, T1))
+        expect = pts[3 * r + 3] if r + 1 < k_in else ec_mul(fr_ints(val)[0], pts[3 * k_in])
+        assert nxt == expect, r
+    # linearity of the commitment on a few rows: com(a) + com(b) = com(a + b)
+    rows = [0, 1, 5503, 11007]
+    A = np.concatenate([W[r * n:(r + 1) * n] for r in rows])
+    B = np.concatenate([W[((r + 7) % m) * n:((r + 7) % m + 1) * n] for r in rows])
+    ca, cb, cab = (pv.commit_int(hG, pv.from_i32(x)).host() for x in (A, B, A + B))
+    exp = np.zeros_like(ca)
+    orc_check(orc.orc_g1_op(0, ca, cb, exp, len(rows)))
+    assert (norm(orc, cab) == norm(orc, exp)).all()
+    assert (norm(orc, ca) == norm(orc, com.host()[rows])).all()

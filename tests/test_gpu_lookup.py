@@ -404,3 +404,66 @@ def test_mapped_lookup_job_equals_the_plain_one_on_the_combined_queries(k):
     assert res[0][1].any()
     for p in (dS, dT, dm, dSi, dSo):
         hip.free(p)
+
+
+def test_config4_full_size_range_lookup_and_softmax_of_one_head(pv):
+    """One attention head at sequence length 2048: 2^22 scores uniform in [-2^15, 2^15), a range table of 2^16 entries.
+    Beyond what the oracle can follow, so checked through what the protocol fixes: the multiplicities are numpy's
+    bincount, the inverses satisfy the LogUp identity sum_i 1/(S_i + beta) = sum_k m_k/(T_k + beta), the 22 round
+    polynomials of the lookup sumcheck chain from alpha + alpha^2 to the returned claim (p(0) + p(1) = claim, claim <- p(v)),
+    and zkSoftmax with the attention driver's parameters (self-attn.cu:87) proves these scores (every identity inside the
+    prover holds) and returns, at scale 2^40, the softmax of the scores to 1e-6, rows summing to one."""
+    n_rows = n_cols = 2048
+    D, low, length = n_rows * n_cols, -(1 << 15), 1 << 16
+    rng = np.random.default_rng(44)
+    vals = rng.integers(low, low + length, D).astype(np.int32)
+    hS = pv.from_i32(vals)
+    m = pv.range_prep(hS, low, length)
+    counts = np.bincount(vals.astype(np.int64) - low, minlength=length)
+    mh = m.host()
+    assert (mh[:, 0] == counts).all() and not mh[:, 1:].any()
+    beta = ch(61, 1)[0]
+    hT = pv.from_i32(np.arange(low, low + length, dtype=np.int32))
+    A, B = pv.batch_inv(hS, beta), pv.batch_inv(hT, beta)
+    assert (pv.sum(A) == pv.sum(pv.binop(2, m, B))).all()
+    del A, B
+    k, n1 = 22, 6
+    alpha, u, v = ch(62, 1)[0], ch(63, k), ch(64, k)
+    pv.transcript_begin()
+    fin = pv.range_prove(hS, low, length, alpha, beta, u, v)
+    pv.lib.zkp_transcript_end()
+    t = fr_ints(pv.transcript())
+    assert len(t) == 4 * k + 1 and t[-1] == fr_ints(fin)[0]
+    a, vi = fr_ints(alpha)[0], fr_ints(v)
+    claim = (a + a * a) % R_MOD
+    for r in range(k):
+        c = t[4 * r:4 * r + 4]
+        assert (2 * c[0] + c[1] + c[2] + c[3]) % R_MOD == claim, r
+        x = vi[n1 - 1 - r] if r < n1 else vi[k - 1 - (r - n1)]
+        claim = (c[0] + c[1] * x + c[2] * x * x + c[3] * x * x * x) % R_MOD
+    assert claim == t[-1]
+    # zkSoftmax on the same scores
+    sf_in, d = 1 << 32, 128
+    pv.seed(65)
+    Y, shift = pv.softmax(hS, n_rows, n_cols, d, np.array([1 << 8, 1 << 20, 1 << 20], np.uint32), 1, 0, sf_in, np.array([float(1 << 18), float(1 << 22)]), True)
+    y = Y.host()
+    assert not y[:, 2:].any()
+    yf = (y[:, 0].astype(np.float64) + y[:, 1].astype(np.float64) * 2.0 ** 32).reshape(n_rows, n_cols) / 2.0 ** 40
+    z = vals.reshape(n_rows, n_cols).astype(np.float64) / sf_in / np.sqrt(d)
+    e = np.exp(z - z.max(axis=1, keepdims=True))
+    ref = e / e.sum(axis=1, keepdims=True)
+    assert np.abs(yf - ref).max() < 1e-6
+    assert np.abs(yf.sum(axis=1) - 1.0).max() < 1e-3
+    # the same head with scores spread over +-2^36 (+-1.4 after the division by sqrt(d)): the rows are far from uniform
+    wide = rng.integers(-(1 << 36), 1 << 36, D)
+    pv.seed(66)
+    Y, shift = pv.softmax(pv.from_i64(wide), n_rows, n_cols, d, np.array([1 << 8, 1 << 20, 1 << 20], np.uint32), 1, 0, sf_in,
+                          np.array([float(1 << 18), float(1 << 22)]), True)
+    y = Y.host()
+    yf = (y[:, 0].astype(np.float64) + y[:, 1].astype(np.float64) * 2.0 ** 32).reshape(n_rows, n_cols) / 2.0 ** 40
+    z = wide.reshape(n_rows, n_cols).astype(np.float64) / sf_in / np.sqrt(d)
+    e = np.exp(z - z.max(axis=1, keepdims=True))
+    ref = e / e.sum(axis=1, keepdims=True)
+    assert ref.max() / ref.min() > 10
+    # the exponential tables are rounded at scales 2^18 and 2^22: a few 1e-4 relative on the small entries
+    assert np.abs(yf - ref).max() < 5e-7 and ref.max() > 1e-3
