@@ -59,6 +59,20 @@ def test_full_shape_layer_gives_one_output_head_by_head_and_stacked(pv):
         outs.append(out.host())
         del out
     pv.layer_free(layer)
+    # the same layer with its nine weight openings (the benchmark's workload): each opened value must equal the claim the
+    # fully connected layer's or the norm's proof left on the weight, or the prover throws; the output does not change
+    cu_o, cf_o = layercfg.llama7b(seq=2048, open_weights=True)
+    pv.seed(2024)
+    layer = pv.layer_create_random(cu_o, cf_o, 7, 5)
+    pv.layer_set(layer, head_group=32)
+    pv.seed(5)
+    pv.transcript_begin()
+    out, _ = pv.layer_run(layer, X)
+    pv.lib.zkp_transcript_end()
+    assert pv.transcript().shape[0] == sizes[1] + 9
+    assert (out.host() == outs[0]).all()
+    del out
+    pv.layer_free(layer)
     assert (outs[0] == outs[1]).all() and (outs[0] == outs[2]).all()
     assert np.unique(outs[0], axis=0).shape[0] > 1000
     assert sizes[1] < sizes[2] < sizes[0]
