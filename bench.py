@@ -31,7 +31,7 @@ VALU_PEAK_TOPS = 256 * 4 * 16 * 2.4e9 / 1e12
 # HBM traffic of k_open_fold per generator pair, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the kernel alone
 # (python3 bench.py --pmc-probe; summary in profiles/k_open_fold_pmc_traffic.txt), each counter scaled by what it reads for
 # zk_fr_add over 2^24 elements (1 GiB read, 512 MiB written)
-FOLD_TRAFFIC_BYTES_PER_PAIR = 2477.0
+FOLD_TRAFFIC_BYTES_PER_PAIR = 2551.0
 
 
 def main():
@@ -77,9 +77,24 @@ def main():
         n = 1 << 24
         dA, dB, dO = hip.malloc(32 * n), hip.malloc(32 * n), hip.malloc(32 * n)
         hip.call("zk_fr_add", c_void_p(dO), c_void_p(dA), c_void_p(dB), c_size_t(n), None)
+        # the kernels behind the other reported rates, once each on operands of known size: the Montgomery product
+        # (Fr mul/s), the fused three-level fold (HBM GB/s) and the commitment of the 11008 x 4096 weight (MSM points/s)
+        seed_block = mt_random_vec(np.random.RandomState(1), 1 << 16)
+        src = hip.upload(seed_block)
+        for i in range(n >> 16):
+            lib.zk_memcpy_d2d(c_void_p(dA + i * (32 << 16)), c_void_p(src), c_size_t(32 << 16), None)
+            lib.zk_memcpy_d2d(c_void_p(dB + i * (32 << 16)), c_void_p(src + 32 * 5), c_size_t((32 << 16) - 32 * 5), None)
+        hip.call("zk_fr_montmul", c_void_p(dO), c_void_p(dA), c_void_p(dB), c_size_t(n), None)
+        u3 = mt_random_vec(np.random.RandomState(2), 3)
+        hip.call("zk_fr_fold_axis", c_void_p(dO), c_void_p(dA), u3, c_int(3), c_size_t(1), c_uint(2048), c_size_t(4096), None)
+        pv.seed(5)
+        gens = pv.commitment_random(4096)
+        Wm = np.round(np.random.default_rng(12).normal(0, 0.02, (11008, 4096)) * 65536).astype(np.int32)
+        com = pv.commit_int(gens, pv.from_i32(Wm))
         hip.sync()
         print(json.dumps({"pmc_probe": {"fold_pairs_per_launch": n_big // 2, "fold_launches": 3, "copy_kernel": "k_ew<0> (zk_fr_add)",
-                                        "copy_read_bytes": 64 * n, "copy_write_bytes": 32 * n}}))
+                                        "copy_read_bytes": 64 * n, "copy_write_bytes": 32 * n, "montmul_elements": n,
+                                        "fold_axis_elements_in": 2048 * 4096, "msm_pairs": 11008 * 4096}}))
         return
 
     def ev():
