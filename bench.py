@@ -270,7 +270,7 @@ def main():
                               "note": "algorithmic 72 MAD32 per field multiply-accumulate (64 limb products + 1/8 of a shared reduction); every MAD32 needs a second "
                                       "VALU instruction for its carry, so 0.5 is the ceiling of this formulation",
                               "avg_launch_ms": mm_ms, "gmac_per_s": M * N * P / (mm_ms * 1e-3) / 1e9}
-    out["roofline_hbm"] = {"kernel": "k_fold_axis<3> (fused 3-level multilinear fold, 2048x4096)", "bound": "hbm", "achieved": fold_gbs, "peak": HBM_PEAK_GBS,
+    out["roofline_hbm"] = {"kernel": "k_fold_axis_dot<3> (fused 3-level multilinear fold, 2048x4096)", "bound": "hbm", "achieved": fold_gbs, "peak": HBM_PEAK_GBS,
                            "unit": "GB/s", "frac": fold_gbs / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": fold_ms}
     for p in (dA, dB, dO, src):
         hip.free(p)
