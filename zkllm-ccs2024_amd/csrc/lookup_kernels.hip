@@ -424,10 +424,19 @@ template <int K> __global__ void __launch_bounds__(TPB) k_me_multi(Fr* __restric
     Fr acc[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) acc[k] = big_zero<8>();
-    for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n; t += (size_t)gridDim.x * TPB) {
-        const Fr e = E[t];
+    // four positions per step: their products with the eq entries share one Montgomery reduction (mont_dot)
+    const size_t stride = (size_t)gridDim.x * TPB;
+    for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n; t += 4 * stride) {
+        Fr e[4];
 #pragma unroll
-        for (int k = 0; k < K; ++k) acc[k] = add(acc[k], mont_mul(e, p.x[k][t]));
+        for (int j = 0; j < 4; ++j) e[j] = (t + j * stride < n) ? E[t + j * stride] : big_zero<8>();
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            Fr x[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) x[j] = (t + j * stride < n) ? p.x[k][t + j * stride] : big_zero<8>();
+            acc[k] = add(acc[k], mont_dot<8, 4>(e, x));
+        }
     }
     block_reduce_store<K>(acc, partials);
 }
