@@ -515,9 +515,13 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
                 acc_em = add(acc_em, mont_mul(e, M));
                 acc_e = add(acc_e, e);
             } else {
-                acc[0] = add(acc[0], mont_mul(e, mont_mul(a0, s0)));
-                acc[1] = add(acc[1], mont_mul(e, add(mont_mul(da, s0), mont_mul(a0, ds))));
-                acc[2] = add(acc[2], mont_mul(e, mont_mul(da, ds)));
+                // E goes onto a0 and da first, and the middle term comes from (a0 + da)(s0 + ds): five products for the
+                // three weighted terms instead of seven
+                const Fr ea0 = mont_mul(e, a0), eda = mont_mul(e, da);
+                const Fr c0 = mont_mul(ea0, s0), c2 = mont_mul(eda, ds);
+                acc[0] = add(acc[0], c0);
+                acc[1] = add(acc[1], sub(sub(mont_mul(add(ea0, eda), add(s0, ds)), c0), c2));
+                acc[2] = add(acc[2], c2);
             }
             acc[3] = add(acc[3], a0);
             acc[4] = add(acc[4], da);
@@ -527,12 +531,15 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
         if (PHASE2) {
             const Fr b0 = B[t], b1 = B[t + n_out], t0r = T[t], t1 = T[t + n_out], m0 = m[t], m1 = m[t + n_out];
             const Fr db = sub(b1, b0), dt = sub(t1, t0r), t0 = add(t0r, beta), dm = sub(m1, m0);
-            acc[5] = add(acc[5], mont_mul(e, mont_mul(b0, t0)));
-            acc[6] = add(acc[6], mont_mul(e, add(mont_mul(db, t0), mont_mul(b0, dt))));
-            acc[7] = add(acc[7], mont_mul(e, mont_mul(db, dt)));
-            acc[8] = add(acc[8], mont_mul(m0, b0));
-            acc[9] = add(acc[9], add(mont_mul(dm, b0), mont_mul(m0, db)));
-            acc[10] = add(acc[10], mont_mul(dm, db));
+            const Fr eb0 = mont_mul(e, b0), edb = mont_mul(e, db);
+            const Fr c5 = mont_mul(eb0, t0), c7 = mont_mul(edb, dt);
+            acc[5] = add(acc[5], c5);
+            acc[6] = add(acc[6], sub(sub(mont_mul(add(eb0, edb), add(t0, dt)), c5), c7));
+            acc[7] = add(acc[7], c7);
+            const Fr k0 = mont_mul(m0, b0), k2 = mont_mul(dm, db);
+            acc[8] = add(acc[8], k0);
+            acc[9] = add(acc[9], sub(sub(mont_mul(m1, b1), k0), k2));          // dm b0 + m0 db = m1 b1 - m0 b0 - dm db
+            acc[10] = add(acc[10], k2);
             nB[t] = add(b0, mont_mul(v_mont, db));
             nT[t] = add(t0r, mont_mul(v_mont, dt));
             nm[t] = add(m0, mont_mul(v_mont, dm));
@@ -598,9 +605,13 @@ k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __rest
             const Fr dx = sub(x1, x0), dy = sub(y1, y0);
             p.out[0][t] = add(x0, mont_mul(v_mont, dx));
             p.out[1][t] = add(y0, mont_mul(v_mont, dy));
-            c[0] = mont_mul(x0, y0);
-            c[2] = mont_mul(dx, dy);
-            c[1] = sub(sub(mont_mul(x1, y1), c[0]), c[2]);      // x0 dy + y0 dx = x1 y1 - x0 y0 - dx dy
+            // E goes onto x0 and dx first (e is loaded below for the other K): the three weighted coefficients cost five
+            // products instead of six.  x0 dy + y0 dx = x1 y1 - x0 y0 - dx dy.
+            const Fr e2 = E[t];
+            const Fr ex0 = mont_mul(e2, x0), edx = mont_mul(e2, dx);
+            c[0] = mont_mul(ex0, y0);
+            c[2] = mont_mul(edx, dy);
+            c[1] = sub(sub(mont_mul(add(ex0, edx), y1), c[0]), c[2]);
         } else {
             {
                 const Fr x0 = p.in[0][t], x1 = p.in[0][t + n_out];
@@ -622,7 +633,7 @@ k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __rest
         const Fr e = E[t];   // Montgomery form: e*R
         if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table
 #pragma unroll
-        for (int j = 0; j <= K; ++j) acc[j] = add(acc[j], mont_mul(e, c[j]));
+        for (int j = 0; j <= K; ++j) acc[j] = add(acc[j], K == 2 ? c[j] : mont_mul(e, c[j]));
     }
     if (K > 1) {
         const Fr r2 = big_r2<8>();
