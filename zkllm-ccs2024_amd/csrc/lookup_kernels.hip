@@ -616,7 +616,8 @@ k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __rest
             {
                 const Fr x0 = p.in[0][t], x1 = p.in[0][t + n_out];
                 const Fr dx = sub(x1, x0);
-                c[0] = x0; c[1] = dx;
+                const Fr e1 = E[t];
+                c[0] = mont_mul(e1, x0); c[1] = mont_mul(e1, dx);       // the weight first: no product with E per coefficient later
                 p.out[0][t] = add(x0, mont_mul(v_mont, dx));
             }
 #pragma unroll
@@ -633,7 +634,7 @@ k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __rest
         const Fr e = E[t];   // Montgomery form: e*R
         if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table
 #pragma unroll
-        for (int j = 0; j <= K; ++j) acc[j] = add(acc[j], K == 2 ? c[j] : mont_mul(e, c[j]));
+        for (int j = 0; j <= K; ++j) acc[j] = add(acc[j], c[j]);
     }
     if (K > 1) {
         const Fr r2 = big_r2<8>();
