@@ -84,6 +84,15 @@ int zk_fr_gather(void* out, const void* table, const void* idx_u32, size_t n, vo
 /* ---- reductions and folds ------------------------------------------------------------------------ */
 /* FrTensor::sum (fr-tensor.cu:382-434) */
 int zk_fr_sum(uint32_t* out_host, const void* a, size_t n, void* stream);
+/* zk_fr_sum for callers that cannot allocate.  No counterpart in the reference: it is for code under HIP stream capture,
+ * tight serving loops and harnesses that forbid hipMalloc.  Calls no hipMalloc/hipFree or any other allocating routine
+ * and does not synchronise: the block partials that zk_fr_sum keeps in a pool block live in a 64 KiB device array inside
+ * the library (one per GPU, held until the process ends), and the sum is written to out_dev, ONE Fr element on the
+ * device (standard form), behind the work already queued on `stream`.  n <= ZK_FR_SUM_STATIC_MAX_N, else an error.
+ * Every call on a GPU uses that GPU's one array: calls that overlap on the same GPU (two streams or two host threads)
+ * race.  zk_init looks the array's address up for its device; otherwise the first call on a device does. */
+#define ZK_FR_SUM_STATIC_MAX_N ((size_t)0xFFFFFFFFu)       /* the reference's tensor sizes are `uint` */
+int zk_fr_sum_static(void* out_dev, const void* a, size_t n, void* stream);
 /* sum_i a_i*b_i; replaces (a*b).sum() at tlookup.cu:360 */
 int zk_fr_dot(uint32_t* out_host, const void* a, const void* b, size_t n, void* stream);
 /* 1..3 levels of Fr_multi_dim_partial_me_step / Fr_me_step / Fr_partial_me_step in one pass over

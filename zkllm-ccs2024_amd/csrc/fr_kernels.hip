@@ -8,6 +8,7 @@
 //  * sums of products are accumulated with the R^-1 factor still attached and corrected once;
 //  * folds run several levels per pass (registers) and finish in one workgroup (LDS).
 #include <cstring>
+#include <mutex>
 #include "field.hpp"
 #include "rt.hpp"
 #include "../../include/zkllm_hip.h"
@@ -455,6 +456,39 @@ __global__ void __launch_bounds__(64) k_row_sumsq_f64(double* __restrict__ out, 
     if (t == 0) out[r] = acc;
 }
 
+// ------------------------------------------------------------------------------------------------
+// FrTensor::sum for callers that cannot allocate (code under stream capture, serving loops, harnesses that forbid
+// hipMalloc).  The block partials of k_sum live in a file-scope device array instead of a pool block; the result goes
+// to a device element of the caller's.  The array is one per GPU and is shared by every call on that GPU: calls that
+// overlap on one GPU (two streams, two threads) race on it.  k_sum writes every partial that k_finish_sums reads, so
+// nothing has to be cleared between calls.
+// ------------------------------------------------------------------------------------------------
+static constexpr unsigned SUM_STATIC_MAX_BLOCKS = 2048;                 // reduce_grid's cap
+static constexpr int SUM_STATIC_MAX_DEVICES = 64;
+static __device__ __align__(256) uint32_t scratch[SUM_STATIC_MAX_BLOCKS * 8];   // 64 KiB of block partials
+
+static std::mutex g_scratch_mu;
+static Fr* g_scratch_ptr[SUM_STATIC_MAX_DEVICES] = {};
+
+// Address of this device's copy of `scratch` (the array's name is only a host-side handle), resolved once per device.
+static int scratch_address(Fr** out) {
+    int dev = -1;
+    ZK_HIP(hipGetDevice(&dev));
+    ZK_ARG(dev >= 0 && dev < SUM_STATIC_MAX_DEVICES, "zk_fr_sum_static: device index over 63");
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        ZK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        ZK_ARG(p != nullptr, "zk_fr_sum_static: the scratch array has no device address");
+        g_scratch_ptr[dev] = (Fr*)p;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+namespace zk {
+int fr_static_scratch_setup() { Fr* p = nullptr; return scratch_address(&p); }
+}
+
 extern "C" {
 
 int zk_fr_add(void* out, const void* a, const void* b, size_t n, void* st) { LAUNCH1D(k_ew<EW_ADD>, n, st, (Fr*)out, (const Fr*)a, (const Fr*)b, n); return 0; }
@@ -685,6 +719,21 @@ int zk_ip_sumcheck_small(uint32_t* polys_host, uint32_t* fin_host, const void* a
     ZK_HIP(hipStreamSynchronize(st));
     memcpy(polys_host, stage, sizeof(Fr) * 3 * k);
     memcpy(fin_host, (char*)stage + sizeof(Fr) * 3 * k, sizeof(Fr) * 2);
+    return 0;
+}
+
+int zk_fr_sum_static(void* out_dev, const void* a, size_t n, void* st) {
+    ZK_ARG(out_dev != nullptr, "zk_fr_sum_static: null output");
+    ZK_ARG(n <= ZK_FR_SUM_STATIC_MAX_N, "zk_fr_sum_static: more than 2^32 - 1 elements (ZK_FR_SUM_STATIC_MAX_N)");
+    ZK_ARG(n == 0 || a != nullptr, "zk_fr_sum_static: null input");
+    Fr* part = nullptr;
+    int rc = scratch_address(&part);
+    if (rc) return rc;
+    const unsigned nb = n ? reduce_grid(n) : 1;       // n == 0: one block that writes a zero partial
+    hipLaunchKernelGGL(k_sum, dim3(nb), dim3(TPB), 0, (hipStream_t)st, part, (const Fr*)a, n);
+    ZK_LAUNCH_CHECK();
+    hipLaunchKernelGGL(k_finish_sums, dim3(1), dim3(TPB), 0, (hipStream_t)st, (Fr*)out_dev, (const Fr*)part, nb);
+    ZK_LAUNCH_CHECK();
     return 0;
 }
 

@@ -158,7 +158,7 @@ int zk_init(int device) {
     }
     ZK_ARG(device >= 0 && device < n, "zk_init: device index out of range");
     ZK_HIP(hipSetDevice(device));
-    return 0;
+    return fr_static_scratch_setup();     // zk_fr_sum_static's array: its address on this device, looked up once
 }
 int zk_device_info(char* name, int name_len, int* compute_units, int* clock_khz, size_t* total_mem) {
     hipDeviceProp_t prop;

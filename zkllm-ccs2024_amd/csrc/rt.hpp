@@ -68,6 +68,10 @@ void pinned_release(void* host_ptr);
 // Pinned host buffer (64 KiB) for device->host results of reductions.
 int staging(void** host_ptr, size_t bytes);
 
+// Looks up, for the current device, the address of the device array behind zk_fr_sum_static (fr_kernels.hip); called
+// by zk_init so that the entry point itself has nothing left to set up.
+int fr_static_scratch_setup();
+
 static inline unsigned cdiv(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
 
 }  // namespace zk
