@@ -2,12 +2,18 @@
 //
 // Composes the oracle's primitives in the order of the reference's per-block executables:
 //   rmsnorm.cu:26-49, self-attn.cu:19-76 (linear) and :78-121 (attn), ffn.cu:44-93, skip-connection.cu:15-18.
+// o_attn_reference_block is the attn mode exactly as the executable runs it (one head as wide as Q); the per-head and
+// stacked variants below are what a whole layer needs.
 // Where the reference cannot be followed literally the same choices as the product's layer are made and
 // recorded: attention is proved per head with d = head width (or, with attn_head_group = g, g heads at a time
 // through zkAttnStacked) and the concatenated output rescaled twice;
 // an output projection follows; challenges drawn inside argument lists in the reference (rmsnorm.cu:47,
 // self-attn.cu:112-113) are drawn first-argument-first; the RMS statistic is host double arithmetic
 // (llama-rmsnorm.py:35-39) and RoPE / causal mask (unproven float steps of llama-self-attn.py) are left out.
+// Pinned by tests/test_oracle_layer.py: the activation table and the RMS statistic against their closed forms in numpy,
+// every block against an exact integer model in numpy (numpy matrix products, rescaling as floor((x + sf/2) / sf), the
+// table softmax rebuilt from its definition), the reference attn mode against the one-head model, and the whole layer
+// against a float64 decoder block within a tolerance derived from the fixed-point scales, with negative controls.
 #pragma once
 #include "protocols.hpp"
 
@@ -47,10 +53,14 @@ static inline OWeight o_make_weight(const int32_t* p, uint in_dim, uint out_dim,
     w.in_dim = in_dim; w.out_dim = out_dim;
     return w;
 }
+// the points of every weight opening in the order the openings happen: per opening T, T0, T1 of each round and the last
+// generator (commitment.cu:125-127), as the recursion leaves them (not normalised)
+static G1Vec g_g1_transcript;
 static inline void o_open(const OLayerConfig& c, const OWeight& w, const Claim& cl) {
     if (!c.open_weights) return;
     G1Vec proof;
     verify_weight_claim(w.gens, w.weight, (uint)w.com.size(), w.in_dim, w.out_dim, cl, proof);
+    g_g1_transcript.insert(g_g1_transcript.end(), proof.begin(), proof.end());
 }
 
 static inline FrVec o_rmsnorm_block(const OLayerConfig& c, const OWeight& w, const FrVec& X, const FrVec& rms_inv) {
@@ -149,6 +159,40 @@ static inline FrVec o_attn_heads_block(const OLayerConfig& c, const FrVec& Q_, c
     rs2.prove(out_all, o_);
     return o__;
 }
+// `self-attn attn` as the reference executable runs it (self-attn.cu:78-121), statement by statement: the whole width of
+// Q is ONE head (d = Q.size / seq_len), the output is rescaled twice and those two range proofs come first, then the
+// proof of out = Y V, the softmax proof and the proof of X = Q K^T.  Y_out receives the softmax output (what the
+// executable saves as temp_head_Y.bin); the return value is what it saves as temp_head_out.bin.
+static inline FrVec o_attn_reference_block(const OLayerConfig& c, const FrVec& Q, const FrVec& K, const FrVec& V, FrVec* Y_out) {
+    const uint S = c.seq_len;
+    need(S > 0 && Q.size() % S == 0 && K.size() == Q.size() && V.size() == Q.size(), "attn: Q, K, V must be seq_len x d");
+    const uint d = (uint)(Q.size() / S);
+    FrVec X = t_matmul(Q, t_transpose(K, S, d), S, d, S);
+    ZkSoftmax sm(c.softmax_bs, c.softmax_L, c.softmax_M, c.softmax_sf_in, c.softmax_thetas, S, S, d);
+    Rescaling rs1(c.sf_attn), rs2(c.sf_attn);
+    FrVec shift, Xs;
+    std::vector<FrVec> xseg, yseg, mseg;
+    FrVec Y = sm.compute(X, shift, Xs, xseg, yseg, mseg);
+    if (Y_out) *Y_out = Y;
+    FrVec out = t_matmul(Y, V, S, S, d);
+    FrVec out_ = rs2.apply(out);
+    FrVec out__ = rs1.apply(out_);
+    rs1.prove(out_, out__);
+    rs2.prove(out, out_);
+    FrVec t3 = random_vec(3);
+    std::vector<Poly> proof;
+    FrVec u1 = random_vec(ceilLog2(S)), u2 = random_vec(ceilLog2(d)), ud = random_vec(ceilLog2(S));
+    Fr claim = t_multi_dim_me(out, {u1, u2}, {S, d});
+    rec(claim);
+    zkip(claim, t_partial_me(Y, u1, S, S), t_partial_me(V, u2, d, 1), ud, proof);
+    FrVec u_Y = random_vec(ceilLog2((uint)Y.size())), v_Y = random_vec(ceilLog2((uint)Y.size()));
+    sm.prove(Y, X, shift, xseg, yseg, mseg, u_Y, v_Y, t3[0], t3[1], t3[2], proof);
+    FrVec u1_ = random_vec(ceilLog2(S)), u2_ = random_vec(ceilLog2(S)), ud_ = random_vec(ceilLog2(d));
+    Fr claim_ = t_multi_dim_me(X, {u1_, u2_}, {S, S});
+    rec(claim_);
+    zkip(claim_, t_partial_me(Q, u1_, S, d), t_partial_me(K, u2_, S, d), ud_, proof);
+    return out__;
+}
 static inline FrVec o_oproj_block(const OLayerConfig& c, const OWeight& o, const FrVec& a) {
     const uint E = c.embed_dim, S = c.seq_len;
     Rescaling r(c.sf_linear);
@@ -158,7 +202,7 @@ static inline FrVec o_oproj_block(const OLayerConfig& c, const OWeight& o, const
     o_open(c, o, zkfc_prove(a, o.weight, O, E, E));
     return O_;
 }
-static inline FrVec o_ffn_block(const OLayerConfig& c, const OWeight& up, const OWeight& gate, const OWeight& down, const FrVec& table, const FrVec& in) {
+static inline FrVec o_ffn_block(const OLayerConfig& c, const OWeight& up, const OWeight& gate, const OWeight& down, const FrVec& table, const FrVec& in, FrVec* down_out_unrescaled = nullptr) {
     const uint E = c.embed_dim, Hd = c.hidden_dim, S = c.seq_len;
     Rescaling upr(c.sf_linear), gr(c.sf_gate), hr(c.sf_linear), dr(c.sf_linear);
     TLookupRangeMapping swiglu(c.swiglu_low, c.swiglu_len, table);
@@ -168,6 +212,7 @@ static inline FrVec o_ffn_block(const OLayerConfig& c, const OWeight& up, const 
     FrVec t3 = random_vec(3), su = random_vec(ceilLog2(S * Hd)), sv = random_vec(ceilLog2(S * Hd));
     FrVec down_in = t_mul(p.first, up_), down_in_ = hr.apply(down_in);
     FrVec down_out = t_matmul(down_in_, down.weight, S, Hd, E), down_out_ = dr.apply(down_out);
+    if (down_out_unrescaled) *down_out_unrescaled = down_out;
     dr.prove(down_out, down_out_);
     o_open(c, down, zkfc_prove(down_in_, down.weight, down_out, Hd, E));
     hr.prove(down_in, down_in_);

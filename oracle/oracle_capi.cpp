@@ -29,7 +29,7 @@ void orc_seed(u32 seed) { g_chal = Challenger(seed); }
 void orc_random_vec(u32* out, u32 len) { vec_out(random_vec(len), out); }
 long orc_transcript_size() { return (long)g_transcript.size(); }
 void orc_transcript_get(u32* out) { vec_out(g_transcript, out); }
-void orc_transcript_clear() { g_transcript.clear(); }
+void orc_transcript_clear() { g_transcript.clear(); g_g1_transcript.clear(); }
 u32 orc_ceil_log2(u32 n) { return ceilLog2(n); }
 
 // ---- field / curve, vectorised over n -----------------------------------------------------------
@@ -387,6 +387,81 @@ int orc_layer(const u32* cu, const double* cf, const int32_t* norm1, const int32
     FrVec b = o_rmsnorm_block(c, n2, x2, o_compute_rms_inv(x2, S, E, c.rms_eps, c.value_scale));
     FrVec y = t_add(x2, o_ffn_block(c, up, gate, down, table, b));
     vec_out(y, out);
+    ORC_END
+}
+
+
+// ---- the layer's blocks one at a time (what the per-block executables compute), on weights kept as handles -------------
+// A weight handle owns the int32 matrix as field elements and, when it is to be opened, its generators and commitment.
+// gens == nullptr with ngen > 0: draw ngen generators from the seeded stream (Commitment::random) and commit;
+// ngen == 0: no generators (only for configurations with open_weights off).
+void* orc_weight_new(const int32_t* w, u32 in_dim, u32 out_dim, const u32* gens, long ngen, const u32* com, long ncom) {
+    try {
+        OWeight* h = new OWeight;
+        h->weight = t_from_i32(w, (size_t)in_dim * out_dim);
+        h->in_dim = in_dim; h->out_dim = out_dim;
+        if (ngen > 0) {
+            h->gens = gens ? g1_in(gens, ngen) : commitment_random((uint)ngen);
+            h->com = com ? g1_in(com, ncom) : commit_int(h->gens, t_pad(h->weight, {in_dim, out_dim}));
+        }
+        return h;
+    } catch (const std::exception& e) { g_err = e.what(); return nullptr; }
+}
+void orc_weight_free(void* h) { delete (OWeight*)h; }
+long orc_weight_sizes(void* h, long* ncom) { *ncom = (long)((OWeight*)h)->com.size(); return (long)((OWeight*)h)->gens.size(); }
+void orc_weight_get(void* h, u32* gens_out, u32* com_out) { if (gens_out) g1_out(((OWeight*)h)->gens, gens_out); if (com_out) g1_out(((OWeight*)h)->com, com_out); }
+long orc_g1_transcript_size() { return (long)g_g1_transcript.size(); }
+void orc_g1_transcript_get(u32* out) { g1_out(g_g1_transcript, out); }
+void orc_g1_transcript_clear() { g_g1_transcript.clear(); }
+
+int orc_rms_inv(const u32* X, u32 seq, u32 embed, double eps, double scale, u32* out) {
+    ORC_TRY vec_out(o_compute_rms_inv(vec_in(X, (long)seq * embed), seq, embed, eps, scale), out); ORC_END
+}
+int orc_swiglu_table(int low, u32 len, double in_scale, double out_scale, u32* out) {
+    ORC_TRY vec_out(o_swiglu_table(low, len, in_scale, out_scale), out); ORC_END
+}
+int orc_rmsnorm_block(const u32* cu, const double* cf, void* w, const u32* X, const u32* rms_inv, u32* out) {
+    ORC_TRY
+    OLayerConfig c = parse_cfg(cu, cf);
+    vec_out(o_rmsnorm_block(c, *(OWeight*)w, vec_in(X, (long)c.seq_len * c.embed_dim), vec_in(rms_inv, c.seq_len)), out);
+    ORC_END
+}
+int orc_attn_linear_block(const u32* cu, const double* cf, void* q, void* k, void* v, const u32* in, u32* Q_, u32* K_, u32* V_) {
+    ORC_TRY
+    OLayerConfig c = parse_cfg(cu, cf);
+    FrVec Q, K, V;
+    o_attn_linear_block(c, *(OWeight*)q, *(OWeight*)k, *(OWeight*)v, vec_in(in, (long)c.seq_len * c.embed_dim), Q, K, V);
+    vec_out(Q, Q_); vec_out(K, K_); vec_out(V, V_);
+    ORC_END
+}
+// reference == 1: the attn mode of the executable (one head as wide as the tensors, self-attn.cu:78-121; Y_out = softmax output);
+// reference == 0: per head / stacked by the configuration's num_heads and attn_head_group (Y_out unused)
+int orc_attn_block(const u32* cu, const double* cf, int reference, const u32* Q_, const u32* K_, const u32* V_, u32* out, u32* Y_out) {
+    ORC_TRY
+    OLayerConfig c = parse_cfg(cu, cf);
+    const long n = (long)c.seq_len * c.embed_dim;
+    if (reference) {
+        FrVec Y;
+        vec_out(o_attn_reference_block(c, vec_in(Q_, n), vec_in(K_, n), vec_in(V_, n), &Y), out);
+        if (Y_out) vec_out(Y, Y_out);
+    } else vec_out(o_attn_heads_block(c, vec_in(Q_, n), vec_in(K_, n), vec_in(V_, n)), out);
+    ORC_END
+}
+int orc_oproj_block(const u32* cu, const double* cf, void* o, const u32* a, u32* out) {
+    ORC_TRY
+    OLayerConfig c = parse_cfg(cu, cf);
+    vec_out(o_oproj_block(c, *(OWeight*)o, vec_in(a, (long)c.seq_len * c.embed_dim)), out);
+    ORC_END
+}
+// table: swiglu_len mapped values (nullptr: built from the configuration).  down_out (optional): the product before its
+// rescaling, which is what the reference executable saves (ffn.cu:81)
+int orc_ffn_block(const u32* cu, const double* cf, void* up, void* gate, void* down, const u32* table, const u32* in, u32* out, u32* down_out) {
+    ORC_TRY
+    OLayerConfig c = parse_cfg(cu, cf);
+    FrVec tb = table ? vec_in(table, c.swiglu_len) : o_swiglu_table(c.swiglu_low, c.swiglu_len, c.swiglu_in_scale, c.swiglu_out_scale);
+    FrVec unrescaled;
+    vec_out(o_ffn_block(c, *(OWeight*)up, *(OWeight*)gate, *(OWeight*)down, tb, vec_in(in, (long)c.seq_len * c.embed_dim), down_out ? &unrescaled : nullptr), out);
+    if (down_out) vec_out(unrescaled, down_out);
     ORC_END
 }
 

@@ -13,9 +13,9 @@
 // triple, which no other summation order reproduces, so sums here are sequential and callers
 // compare through g1_equal / g1_normalize.
 // Floating point (softmax shift and exp tables): PARITY UNPINNED against the reference, whose CUDA
-// device libm cannot be reproduced; both steps follow the fixed recipe of detmath_ref.hpp instead,
-// and the row sum of exponentials is taken in a fixed order (64 strided partial sums combined by the
-// butterfly i ^ 32, 16, ..., 1), which is what the product's kernel does.
+// device libm cannot be reproduced; both steps follow the fixed recipe of detmath_ref.hpp instead.
+// The row sum of exponentials is one running sum in index order, as in zksoftmax.cu:24-26, so the only
+// difference left against the reference is the last ulp of exp and log.
 #pragma once
 #include <cmath>
 #include "detmath_ref.hpp"
@@ -293,18 +293,9 @@ struct ZkSoftmax {
         #pragma omp parallel for
         for (long r = 0; r < (long)m; ++r) {
             const double scale = sfd * std::sqrt(dd);
-            double part[64];
-            for (int l = 0; l < 64; ++l) {
-                double acc = 0.0;
-                for (uint i = l; i < n; i += 64) acc = acc + o_exp((double)fr_to_i64(X[r * n + i]) / scale);
-                part[l] = acc;
-            }
-            for (int off = 32; off >= 1; off >>= 1) {
-                double nxt[64];
-                for (int l = 0; l < 64; ++l) nxt[l] = part[l] + part[l ^ off];
-                for (int l = 0; l < 64; ++l) part[l] = nxt[l];
-            }
-            shift[r] = fr_from_f64(scale * o_log(part[0]), 1);
+            double temp = 0.0;                                   // zksoftmax.cu:24-26: one running sum in index order
+            for (uint i = 0; i < n; ++i) temp = temp + o_exp((double)fr_to_i64(X[r * n + i]) / scale);
+            shift[r] = fr_from_f64(scale * o_log(temp), 1);
             for (uint i = 0; i < n; ++i) Xs[r * n + i] = sub(X[r * n + i], shift[r]);
         }
         const size_t N = X.size();

@@ -904,18 +904,32 @@ __global__ void __launch_bounds__(TPB) k_relu_decomp(Fr* __restrict__ res, Fr* _
 }
 
 // ---- softmax (zksoftmax.cu) ------------------------------------------------------------------------------------------------------
-// One wave per row.  Lane l sums exp(x_j / scale) over j = l, l+64, ... in index order, the 64 partial
-// sums are combined with the butterfly i ^ 32, 16, ..., 1 (every lane ends with the same total), and
+// One wave per row.  The row's exponentials are added into ONE running sum in index order, as the one-thread-per-row
+// loop of zksoftmax.cu:24-26 does: the 64 lanes evaluate 64 consecutive terms side by side, park them in LDS, and every
+// lane then adds them in order (the additions are the same in all lanes, so all end with the same total).
 // shift = round_half_away(scale * log(total)).  out = x - shift.  scale = sf_in * sqrt(d).
 __global__ void __launch_bounds__(TPB) k_softmax_shift(Fr* __restrict__ shift, Fr* __restrict__ out, const Fr* __restrict__ X, uint32_t rows, uint32_t cols, double scale) {
-    const uint32_t row = blockIdx.x * (TPB / 64) + (threadIdx.x >> 6);
-    const uint32_t lane = threadIdx.x & 63u;
-    if (row >= rows) return;
-    const Fr* xr = X + (size_t)row * cols;
-    double part = 0.0;
-    for (uint32_t j = lane; j < cols; j += 64) part = part + zkd::exp_det((double)fr_to_i64(xr[j]) / scale);
-    for (int off = 32; off >= 1; off >>= 1) part = part + __shfl_xor(part, off, 64);
-    const double sv = scale * zkd::log_det(part);
+    __shared__ double term[TPB / 64][64];
+    const uint32_t w = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    const uint32_t row = blockIdx.x * (TPB / 64) + w;
+    const bool live = row < rows;                         // a whole wave is live or idle; idle waves still reach every barrier
+    const Fr* xr = X + (size_t)(live ? row : 0) * cols;
+    double total = 0.0;
+    for (uint32_t j0 = 0; j0 < cols; j0 += 64) {
+        const uint32_t j = j0 + lane;
+        term[w][lane] = (live && j < cols) ? zkd::exp_det((double)fr_to_i64(xr[j]) / scale) : 0.0;
+        __syncthreads();
+        const uint32_t cnt = cols - j0 < 64u ? cols - j0 : 64u;
+        if (cnt == 64u) {
+#pragma unroll
+            for (int q = 0; q < 64; ++q) total = total + term[w][q];
+        } else {
+            for (uint32_t q = 0; q < cnt; ++q) total = total + term[w][q];
+        }
+        __syncthreads();
+    }
+    if (!live) return;
+    const double sv = scale * zkd::log_det(total);
     const int64_t si = (sv >= 0) ? (int64_t)(sv + 0.5) : (int64_t)(sv - 0.5);
     const Fr sh = fr_from_i64(si);
     if (lane == 0) shift[row] = sh;
