@@ -193,6 +193,14 @@ class Prover:
         a = np.ascontiguousarray(a, dtype=np.float64)
         return self.H(self.lib.zkp_fr_from_f64(_np_ptr(a), c_uint(a.size), c_u64(sf)))
 
+    def from_file(self, path, kind):
+        """kind 0: raw field elements (FrTensor(filename)), 1: int32 (from_int_bin), 2: int64 (from_long_bin)"""
+        return self.H(self.lib.zkp_fr_from_file(str(path).encode(), c_int(kind)))
+
+    def save(self, t, path, kind):
+        """kind 0: save, 1: save_int, 2: save_long"""
+        self.check(self.lib.zkp_fr_save(c_void_p(t.h), str(path).encode(), c_int(kind)))
+
     def binop(self, op, a, b):
         return self.H(self.lib.zkp_fr_binop(c_int(op), c_void_p(a.h), c_void_p(b.h)))
 

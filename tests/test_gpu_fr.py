@@ -419,3 +419,52 @@ def test_config2_full_size_fully_connected_proof_passes_the_verifier(pv):
     assert final == claim and cX * cW % R_MOD == final
     assert [cX] == fr_ints(pv.multi_dim_me(hX, [u_b, u_i], (B, I)))
     assert [cW] == fr_ints(pv.multi_dim_me(hW, [u_i, u_o], (I, O)))
+
+
+# ---- .bin files (fr-tensor.cu:181-248, ioutils.cu:3-45) ---------------------------------------------------------------------
+def ref_scalar_to_int(x, bits):
+    """scalar_to_int / scalar_to_long (fr-tensor.cu:922-945): the value when it is a non-negative number below 2^(bits-1),
+    else minus the low word of r - x, which scalar_to_uint / scalar_to_ulong read as 0 when r - x does not fit the word"""
+    top = 1 << bits
+    if x < (top >> 1):
+        return x
+    n = (R_MOD - x) % R_MOD
+    u = n if n < top else 0
+    v = (-u) % top
+    return v - top if v >= (top >> 1) else v
+
+
+def test_fr_bin_files_round_trip_and_conversions(pv, tmp_path):
+    rng = np.random.default_rng(3)
+    # int32 files: from_int_bin embeds negatives as r - |x|; save_int gives the same bytes back
+    a32 = np.concatenate([np.array([0, 1, -1, 2**31 - 1, -2**31, 65536, -65536], dtype=np.int32), rng.integers(-2**31, 2**31, 1000).astype(np.int32)])
+    a32.tofile(tmp_path / "a32.bin")
+    t = pv.from_file(tmp_path / "a32.bin", 1)
+    assert fr_ints(t.host()) == [int(v) % R_MOD for v in a32]
+    pv.save(t, tmp_path / "a32_back.bin", 1)
+    assert (tmp_path / "a32_back.bin").read_bytes() == (tmp_path / "a32.bin").read_bytes()
+    # int64 files: every byte of the file is read (the reference's from_long_bin copies only the first half of the buffer to
+    # the device, fr-tensor.cu:243-244, and converts whatever the second half of its allocation holds)
+    a64 = np.concatenate([np.array([0, 1, -1, 2**63 - 1, -2**63 + 1, 2**40, -2**40], dtype=np.int64), rng.integers(-2**62, 2**62, 1000)])
+    a64.tofile(tmp_path / "a64.bin")
+    t64 = pv.from_file(tmp_path / "a64.bin", 2)
+    assert t64.size == a64.size and fr_ints(t64.host()) == [int(v) % R_MOD for v in a64]
+    pv.save(t64, tmp_path / "a64_back.bin", 2)
+    assert (tmp_path / "a64_back.bin").read_bytes() == (tmp_path / "a64.bin").read_bytes()
+    # raw field elements: 32 bytes each, standard form, as they lie in device memory
+    raw = seeded(500, 9)
+    h = pv.from_fr(raw)
+    pv.save(h, tmp_path / "raw.bin", 0)
+    assert (tmp_path / "raw.bin").read_bytes() == raw.tobytes()
+    assert (pv.from_file(tmp_path / "raw.bin", 0).host() == raw).all()
+    # values outside the integer types: what scalar_to_int / scalar_to_long give
+    odd = [2**31, 2**31 + 5, 2**32 + 7, R_MOD - 2**31, R_MOD - 2**31 - 5, R_MOD - 2**32 - 9, R_MOD - 1, 2**63, 2**64 + 3, R_MOD - 2**63, R_MOD - 2**64 - 1, R_MOD >> 1]
+    ho = pv.from_fr(fr_array(odd))
+    pv.save(ho, tmp_path / "odd32.bin", 1)
+    pv.save(ho, tmp_path / "odd64.bin", 2)
+    assert list(np.fromfile(tmp_path / "odd32.bin", dtype=np.int32)) == [ref_scalar_to_int(x, 32) for x in odd]
+    assert list(np.fromfile(tmp_path / "odd64.bin", dtype=np.int64)) == [ref_scalar_to_int(x, 64) for x in odd]
+    # an int32 file read as int64 halves the element count (sizes come from the file length alone)
+    assert pv.from_file(tmp_path / "a32.bin", 2).size == a32.size // 2
+    with pytest.raises(RuntimeError):
+        pv.from_file(tmp_path / "missing.bin", 1)

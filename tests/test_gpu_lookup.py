@@ -81,6 +81,24 @@ def test_lookup_out_of_range_is_an_error(pv):
         pv.range_prep(pv.from_i64(np.array([0, 1, 99])), 0, 8)
 
 
+def test_range_lookup_rejects_values_in_the_padding_gap(pv):
+    """A range of 6 values is kept in a table of 8 whose last two entries repeat low + 5: a query of low + 6 or low + 7 has
+    room in the padded table but is outside the range, and must be refused like any other stray value."""
+    low, length = -3, 6
+    good = [-3, 2, 0, 1, -1, 2, 2, -3]
+    mv = pv.from_fr(ch(31, length))
+    pv.range_prep(pv.from_fr(fr_array([v % R_MOD for v in good])), low, length)
+    pv.mapping(pv.from_fr(fr_array([v % R_MOD for v in good])), low, length, mv)
+    for bad in (3, 4, 5, -4):
+        vals = list(good)
+        vals[5] = bad
+        S = pv.from_fr(fr_array([v % R_MOD for v in vals]))
+        with pytest.raises(RuntimeError, match="outside the table"):
+            pv.range_prep(S, low, length)
+        with pytest.raises(RuntimeError, match="outside the table"):
+            pv.mapping(S, low, length, mv)
+
+
 @pytest.mark.parametrize("n", [1, 7, 4096, 4097, 50000])
 def test_batch_inverse(pv, orc, n):
     S = ch(n, n)

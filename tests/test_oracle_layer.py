@@ -14,7 +14,7 @@ import numpy as np
 import pytest
 
 import layercfg
-from zkhelp import R_MOD, fr_array, fr_ints, load_oracle, orc_check
+from zkhelp import R_MOD, fr_array, fr_signed as signed, load_oracle, orc_check
 
 VS_BITS = 10            # fixed-point scale of activations and weights in the mid-size configuration
 
@@ -24,19 +24,6 @@ def mid_cfg(swiglu_out_scale=1024.0, heads=2, head_group=0, seq=64, embed=64, hi
     softmax digit tables (2^10) and an activation table over [-4, 4) in steps of 2^-8 fit their tensors"""
     return layercfg.pack(seq, embed, heads, hidden, 1 << 10, 1 << 12, 1 << 9, [1 << 8, 1 << 10, 1 << 10], 1, 0, 1 << 20, [1 << 8, 1 << 10],
                          -1024, 2048, 256.0, swiglu_out_scale=swiglu_out_scale, value_scale=1024.0, open_weights=False, head_group=head_group)
-
-
-def signed(fr):
-    """(n, 8) uint32 field elements of magnitude below 2^63 -> list of python ints in (-r/2, r/2)"""
-    fr = np.asarray(fr, dtype=np.uint32).reshape(-1, 8)
-    lo = fr[:, 0].astype(np.uint64) | (fr[:, 1].astype(np.uint64) << np.uint64(32))
-    neg = fr[:, 7] != 0
-    r_lo = np.uint64(R_MOD & ((1 << 64) - 1))
-    mag = np.where(neg, r_lo - lo, lo)                       # wraps mod 2^64, which is the low half of r - x
-    small = np.where(neg, (fr[:, 2:] == fr_array([R_MOD - 1])[0, 2:]).all(axis=1), (fr[:, 2:] == 0).all(axis=1))
-    if not small.all():
-        return [x - R_MOD if x > R_MOD // 2 else x for x in fr_ints(fr)]
-    return [int(v) for v in np.where(neg, -mag.astype(np.int64), mag.astype(np.int64))]
 
 
 def as_fr(a):

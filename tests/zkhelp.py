@@ -36,6 +36,19 @@ def fr_ints(arr):
     return [from_limbs(row) for row in arr]
 
 
+def fr_signed(fr):
+    """(n, 8) uint32 field elements of magnitude below 2^63 -> list of python ints in (-r/2, r/2)"""
+    fr = np.asarray(fr, dtype=np.uint32).reshape(-1, 8)
+    lo = fr[:, 0].astype(np.uint64) | (fr[:, 1].astype(np.uint64) << np.uint64(32))
+    neg = fr[:, 7] != 0
+    r_lo = np.uint64(R_MOD & ((1 << 64) - 1))
+    mag = np.where(neg, r_lo - lo, lo)                       # wraps mod 2^64, which is the low half of r - x
+    small = np.where(neg, (fr[:, 2:] == fr_array([R_MOD - 1])[0, 2:]).all(axis=1), (fr[:, 2:] == 0).all(axis=1))
+    if not small.all():
+        return [x - R_MOD if x > R_MOD // 2 else x for x in fr_ints(fr)]
+    return [int(v) for v in np.where(neg, -mag.astype(np.int64), mag.astype(np.int64))]
+
+
 def fp_array(vals):
     return np.array([to_limbs(v, 12) for v in vals], dtype=np.uint32).reshape(-1, 12)
 

@@ -118,3 +118,17 @@ Weight create_weight(string generator_filename, string weight_filename, string c
     if (in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim))) w.padded = std::make_shared<const FrTensor>(w.weight.pad({in_dim, out_dim}));
     return w;
 }
+
+// commit-param.cu:4-29 as a function: the parameter file (int32, in_dim x out_dim) is padded to powers of two in both
+// dimensions and each padded row block of generator length is committed.  The points are written with z = ONE, so the
+// file does not depend on the order in which the sums were formed (readers accept any Jacobian form).
+uint commit_param_file(const string& generator_filename, const string& param_filename, const string& output_filename, uint in_dim, uint out_dim) {
+    Commitment generator(generator_filename);
+    if (generator.size != (1u << ceilLog2(generator.size))) throw std::runtime_error("Generator size has to be a power of 2");
+    FrTensor param = FrTensor::from_int_bin(param_filename);
+    if (param.size != in_dim * out_dim) throw std::runtime_error("commit-param: the parameter file does not hold in_dim x out_dim values");
+    const bool ragged = in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim));
+    G1TensorJacobian com = ragged ? generator.commit_int(param.pad({in_dim, out_dim})) : generator.commit_int(param);
+    com.normalized().save(output_filename);
+    return com.size;
+}

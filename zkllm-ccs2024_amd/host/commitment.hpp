@@ -52,6 +52,10 @@ struct Weight {
 
 Weight create_weight(string generator_filename, string weight_filename, string com_filename, uint in_dim, uint out_dim);
 
+// The flow of the commit-param executable (commit-param.cu:4-29): loads the generators and the int32 parameter file, pads,
+// commits with commit_int and saves the commitment with z = ONE; returns the number of points written.
+uint commit_param_file(const string& generator_filename, const string& param_filename, const string& output_filename, uint in_dim, uint out_dim);
+
 // When set, Commitment::open skips the G1 part of the opening (whose result the reference computes and
 // then drops) and returns the evaluation alone.  Default off.  ZKLLM_SKIP_G1_OPENING=1 sets it.
 void zk_set_skip_g1_opening(bool skip);

@@ -27,8 +27,14 @@ struct Globals {
     int last_matmul_path = 0;
     bool recording = false;
     std::vector<Fr_t> transcript;
+    std::vector<G1Jacobian_t> transcript_g1;
+    std::string proof_file;
     Globals() {
         if (const char* m = getenv("ZKLLM_MATMUL")) matmul_mode = (string(m) == "generic") ? 1 : 0;
+        if (const char* f = getenv("ZKLLM_PROOF_FILE")) { proof_file = f; recording = !proof_file.empty(); }
+    }
+    ~Globals() {
+        if (!proof_file.empty()) try { zk_write_proof_file(proof_file); } catch (...) {}
     }
 };
 Globals& G() { static Globals g; return g; }
@@ -44,7 +50,20 @@ void ensure_seeded() {
 void zk_seed_challenges(uint32_t seed) { G().mt.seed(seed); G().seeded = true; }
 void zk_set_matmul_mode(int mode) { G().matmul_mode = mode; }
 int zk_last_matmul_path() { return G().last_matmul_path; }
-void zk_transcript_begin() { G().transcript.clear(); G().recording = true; }
+void zk_transcript_begin() { G().transcript.clear(); G().transcript_g1.clear(); G().recording = true; }
+void zk_record_g1(const std::vector<G1Jacobian_t>& points) { if (G().recording) G().transcript_g1.insert(G().transcript_g1.end(), points.begin(), points.end()); }
+const std::vector<G1Jacobian_t>& zk_transcript_g1() { return G().transcript_g1; }
+void zk_write_proof_file(const std::string& path) {
+    FILE* f = fopen(path.c_str(), "wb");
+    if (!f) throw std::runtime_error("zk_write_proof_file: cannot open " + path);
+    const Globals& g = G();
+    const uint64_t counts[2] = {(uint64_t)g.transcript.size(), (uint64_t)g.transcript_g1.size()};
+    bool ok = fwrite("ZKLLMPF1", 1, 8, f) == 8 && fwrite(counts, 8, 2, f) == 2;
+    if (ok && counts[0]) ok = fwrite(g.transcript.data(), sizeof(Fr_t), counts[0], f) == counts[0];
+    if (ok && counts[1]) ok = fwrite(g.transcript_g1.data(), sizeof(G1Jacobian_t), counts[1], f) == counts[1];
+    fclose(f);
+    if (!ok) throw std::runtime_error("zk_write_proof_file: short write to " + path);
+}
 const std::vector<Fr_t>& zk_transcript() { return G().transcript; }
 void zk_transcript_end() { G().recording = false; }
 void zk_record(const Fr_t& x) { if (G().recording) G().transcript.push_back(x); }

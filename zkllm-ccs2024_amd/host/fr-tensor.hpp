@@ -46,6 +46,15 @@ void zk_record(const std::vector<Fr_t>& xs);
 size_t zk_record_reserve();
 void zk_record_fill(size_t slot, const Fr_t& x);
 
+// the points of a weight opening (T, T0, T1 per round, then the last generator; z = ONE), kept beside the transcript
+void zk_record_g1(const std::vector<G1Jacobian_t>& points);
+const std::vector<G1Jacobian_t>& zk_transcript_g1();
+// Proof artifact.  With ZKLLM_PROOF_FILE=<path> in the environment a process records from its start and writes, when it
+// exits normally: the 8 bytes "ZKLLMPF1", two little-endian u64 counts n_fr and n_g1, then n_fr field elements (32 bytes each,
+// standard form: claims, round polynomial coefficients and opened values in proving order) and n_g1 points (144 bytes each,
+// Jacobian with z = ONE in Montgomery form, infinity as zero bytes: the weight openings' points in opening order).
+void zk_write_proof_file(const std::string& path);
+
 void zk_check(int rc, const char* where);   // throws std::runtime_error on a non-zero C-ABI status
 
 class FrTensor {

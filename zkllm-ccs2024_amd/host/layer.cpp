@@ -42,6 +42,46 @@ FrTensor make_swiglu_table(int low, uint len, double in_scale, double out_scale)
     return FrTensor(len, t.data());
 }
 
+// "key=value,key=value": numbers; lists separated by ':'
+void layer_config_from_env(LayerConfig& c) {
+    const char* e = getenv("ZKLLM_LAYER_CONFIG");
+    if (!e) return;
+    std::string s(e);
+    size_t pos = 0;
+    while (pos < s.size()) {
+        size_t end = s.find(',', pos);
+        if (end == std::string::npos) end = s.size();
+        const std::string item = s.substr(pos, end - pos);
+        pos = end + 1;
+        if (item.empty()) continue;
+        const size_t eq = item.find('=');
+        if (eq == std::string::npos) throw std::runtime_error("ZKLLM_LAYER_CONFIG: expected key=value, got " + item);
+        const std::string key = item.substr(0, eq), val = item.substr(eq + 1);
+        auto list = [&] {
+            std::vector<double> out;
+            size_t p0 = 0;
+            while (p0 <= val.size()) {
+                size_t p1 = val.find(':', p0);
+                if (p1 == std::string::npos) p1 = val.size();
+                out.push_back(std::stod(val.substr(p0, p1 - p0)));
+                p0 = p1 + 1;
+            }
+            return out;
+        };
+        if (key == "sf_linear") c.sf_linear = (uint)std::stoul(val);
+        else if (key == "sf_gate") c.sf_gate = (uint)std::stoul(val);
+        else if (key == "sf_attn") c.sf_attn = (uint)std::stoul(val);
+        else if (key == "softmax_L") c.softmax_L = (uint)std::stoul(val);
+        else if (key == "softmax_M") c.softmax_M = (uint)std::stoul(val);
+        else if (key == "softmax_sf_in") c.softmax_sf_in = std::stoul(val);
+        else if (key == "softmax_bs") { c.softmax_bs.clear(); for (double x : list()) c.softmax_bs.push_back((uint)x); }
+        else if (key == "softmax_thetas") c.softmax_thetas = list();
+        else if (key == "value_scale") c.value_scale = std::stod(val);
+        else if (key == "rms_eps") c.rms_eps = std::stod(val);
+        else throw std::runtime_error("ZKLLM_LAYER_CONFIG: unknown key " + key);
+    }
+}
+
 // rmsnorm.cu:26-49
 FrTensor rmsnorm_block(const LayerConfig& c, const Weight& w, const FrTensor& X, const FrTensor& rms_inv) {
     Rescaling rs1(c.sf_linear), rs2(c.sf_linear);
@@ -222,6 +262,44 @@ FrTensor attn_heads_block(const LayerConfig& c, const FrTensor& Q_, const FrTens
     return out__;
 }
 
+// self-attn.cu:78-121 statement by statement: one head as wide as Q; the two rescalings are proved first, then
+// out = Y V, the softmax, X = Q K^T.  Challenges that the reference draws inside an argument list are drawn first argument first.
+FrTensor attn_reference_block(const LayerConfig& c, const FrTensor& Q, const FrTensor& K, const FrTensor& V, std::unique_ptr<FrTensor>* softmax_out) {
+    const uint seq_len = c.seq_len;
+    if (seq_len == 0 || Q.size % seq_len || K.size != Q.size || V.size != Q.size) throw std::runtime_error("attn: Q, K, V must be seq_len x d");
+    const uint d = Q.size / seq_len;
+    auto X = FrTensor::matmul(Q, K.transpose(seq_len, d), seq_len, d, seq_len);
+    zkSoftmax softmax(c.softmax_bs, c.softmax_L, c.softmax_M, c.softmax_sf_in, c.softmax_thetas, seq_len, seq_len, d, 1);
+    Rescaling rs1(c.sf_attn), rs2(c.sf_attn);
+    FrTensor shift(seq_len), X_shifted(seq_len * seq_len);
+    vector<FrTensor> X_segments, Y_segments, m_segments;
+    FrTensor Y = softmax.compute(X, shift, X_shifted, X_segments, Y_segments, m_segments);
+    auto out = FrTensor::matmul(Y, V, seq_len, seq_len, d);
+    auto out_ = rs2(out);
+    auto out__ = rs1(out_);
+    rs1.prove(out_, out__);
+    rs2.prove(out, out_);
+    auto temp_rand = random_vec(3);
+    vector<Polynomial> proof;
+    auto u1 = random_vec(ceilLog2(seq_len));
+    auto u2 = random_vec(ceilLog2(d));
+    auto ud = random_vec(ceilLog2(seq_len));
+    auto claim = out.multi_dim_me({u1, u2}, {seq_len, d});
+    zk_record(claim);
+    zkip(claim, Y.partial_me(u1, seq_len, seq_len), V.partial_me(u2, d, 1), ud, proof);
+    auto u_Y = random_vec(ceilLog2(Y.size));
+    auto v_Y = random_vec(ceilLog2(Y.size));
+    softmax.prove(Y, X, shift, X_shifted, X_segments, Y_segments, m_segments, u_Y, v_Y, temp_rand[0], temp_rand[1], temp_rand[2], proof);
+    auto u1_ = random_vec(ceilLog2(seq_len));
+    auto u2_ = random_vec(ceilLog2(seq_len));
+    auto ud_ = random_vec(ceilLog2(d));
+    auto claim_ = X.multi_dim_me({u1_, u2_}, {seq_len, seq_len});
+    zk_record(claim_);
+    zkip(claim_, Q.partial_me(u1_, seq_len, d), K.partial_me(u2_, seq_len, d), ud_, proof);
+    if (softmax_out) softmax_out->reset(new FrTensor(std::move(Y)));
+    return out__;
+}
+
 FrTensor oproj_block(const LayerConfig& c, const Weight& o, const FrTensor& attn_out) {
     zkFC o_layer(c.embed_dim, c.embed_dim, o.weight);
     Rescaling o_rescale(c.sf_linear);
@@ -234,7 +312,8 @@ FrTensor oproj_block(const LayerConfig& c, const Weight& o, const FrTensor& attn
 }
 
 // ffn.cu:44-93
-FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, const Weight& down, const FrTensor& swiglu_values, const FrTensor& input) {
+FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, const Weight& down, const FrTensor& swiglu_values, const FrTensor& input,
+                   std::unique_ptr<FrTensor>* down_out_unrescaled) {
     zkFC up_layer(c.embed_dim, c.hidden_dim, up.weight), gate_layer(c.embed_dim, c.hidden_dim, gate.weight), down_layer(c.hidden_dim, c.embed_dim, down.weight);
     Rescaling up_rescale(c.sf_linear), gate_rescale(c.sf_gate), hidden_rescale(c.sf_linear), down_rescale(c.sf_linear);
     tLookupRangeMapping swiglu(c.swiglu_low, c.swiglu_len, swiglu_values);
@@ -295,7 +374,8 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
     }
     auto cu = up_layer.prove(input, up_out, ch_u);
     if (c.open_weights) verifyWeightClaim(up, cu[0], ou);
-    // the reference saves the unrescaled down_out (ffn.cu:81); the rescaled tensor is what the next block consumes
+    // the reference's executable saves the unrescaled down_out (ffn.cu:81); the rescaled tensor is what the next block consumes
+    if (down_out_unrescaled) down_out_unrescaled->reset(new FrTensor(std::move(down_out)));
     return down_out_;
 }
 

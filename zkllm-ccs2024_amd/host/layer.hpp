@@ -16,6 +16,7 @@
 //  * RoPE, the causal mask and the RMS statistic are the reference's unproven float steps; RoPE and the
 //    mask are left out, the RMS statistic is computed on the host in double precision.
 #pragma once
+#include <memory>
 #include "commitment.hpp"
 #include "fr-tensor.hpp"
 #include "rescaling.hpp"
@@ -42,6 +43,11 @@ struct LayerConfig {
                                   // num_heads): heads proved g at a time as head-major stacks with zkAttnStacked (zksoftmax.cu:289-320)
 };
 
+// The executables use the reference's constants (the defaults above).  ZKLLM_LAYER_CONFIG in the environment replaces any
+// of them, e.g. "sf_linear=256,sf_gate=1024,sf_attn=128,softmax_bs=256:256:256,softmax_sf_in=65536,softmax_thetas=64:256":
+// a lookup table cannot be larger than the tensor it serves, so shapes far below the 7B layer need smaller tables.
+void layer_config_from_env(LayerConfig& c);
+
 struct LayerWeights {
     Weight input_norm, q, k, v, o, post_norm, up, gate, down;
     FrTensor swiglu_table;        // swiglu_len mapped values
@@ -62,7 +68,14 @@ FrTensor rmsnorm_block(const LayerConfig& c, const Weight& w, const FrTensor& X,
 void attn_linear_block(const LayerConfig& c, const Weight& q, const Weight& k, const Weight& v, const FrTensor& input, FrTensor& Q_, FrTensor& K_, FrTensor& V_);
 FrTensor attn_heads_block(const LayerConfig& c, const FrTensor& Q_, const FrTensor& K_, const FrTensor& V_);
 FrTensor oproj_block(const LayerConfig& c, const Weight& o, const FrTensor& attn_out);
-FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, const Weight& down, const FrTensor& swiglu_table, const FrTensor& input);
+// down_out_unrescaled (optional) receives the down projection before its rescaling: what the reference's executable
+// writes to its output file (ffn.cu:81), while the return value (rescaled) is what a following block consumes
+FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, const Weight& down, const FrTensor& swiglu_table, const FrTensor& input,
+                   std::unique_ptr<FrTensor>* down_out_unrescaled = nullptr);
+// the attn mode exactly as the reference's executable runs it (self-attn.cu:78-121): ONE head of width Q.size / seq_len,
+// proofs in the executable's order; softmax_out (optional) receives the softmax output, which the executable saves as
+// temp_head_Y.bin; the return value is what it saves as temp_head_out.bin
+FrTensor attn_reference_block(const LayerConfig& c, const FrTensor& Q, const FrTensor& K, const FrTensor& V, std::unique_ptr<FrTensor>* softmax_out = nullptr);
 
 // whole layer: x -> x + attn(norm(x)) -> (+ ffn(norm(.)))
 FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor& X, LayerTimes* times);

@@ -29,8 +29,9 @@ void DeferredOpenings::finish() {
             vector<G1Jacobian_t> g1_proof;
             const Fr_t opening = Commitment::open_end(it->op, g1_proof);
             zk_record_fill(it->slot, opening);
-            if (opening != it->claim && failure.empty()) failure = "verifyWeightClaim: opening != c.claim";
-            else cout << "Opening complete" << endl;
+            zk_record_g1(g1_proof);
+            if (opening == it->claim) cout << "Opening complete" << endl;
+            else if (failure.empty()) failure = "verifyWeightClaim: opening != c.claim";
         } catch (const std::exception& e) {
             if (failure.empty()) failure = e.what();
         }
@@ -57,8 +58,10 @@ void verifyWeightClaim(const Weight& w, const Claim& c) {
         g_deferred->items.push_back(it);
         return;
     }
-    auto opening = w.generator.open(w_padded, w.com, u_cat);
+    vector<G1Jacobian_t> g1_proof;
+    auto opening = w.generator.open(w_padded, w.com, u_cat, g1_proof);
     zk_record(opening);
+    zk_record_g1(g1_proof);
     if (opening != c.claim) throw std::runtime_error("verifyWeightClaim: opening != c.claim");
     cout << "Opening complete" << endl;
 }

@@ -28,16 +28,16 @@ static FrTensor make_range_table(int low, uint len) {
     ZKC(zk_range_table(t.gpu_data, low, len, t.size, nullptr));
     return t;
 }
-tLookupRange::tLookupRange(int low, uint len) : tLookup(make_range_table(low, len)), low(low) {}
+tLookupRange::tLookupRange(int low, uint len) : tLookup(make_range_table(low, len)), low(low), len(len) {}
 
 FrTensor tLookupRange::prep(const int* vals, const uint D) {
     DevBuf idx(sizeof(uint) * (size_t)D);
-    ZKC(zk_lookup_index_i32(idx.p, vals, low, table.size, D, nullptr));
+    ZKC(zk_lookup_index_i32(idx.p, vals, low, len, D, nullptr));
     return counts_to_m(idx.p, D, table.size);
 }
 FrTensor tLookupRange::prep(const FrTensor& vals) {
     DevBuf idx(sizeof(uint) * (size_t)vals.size);
-    ZKC(zk_lookup_index_fr(idx.p, vals.gpu_data, low, table.size, vals.size, nullptr));
+    ZKC(zk_lookup_index_fr(idx.p, vals.gpu_data, low, len, vals.size, nullptr));
     return counts_to_m(idx.p, vals.size, table.size);
 }
 
@@ -52,7 +52,7 @@ tLookupRangeMapping::tLookupRangeMapping(int low, uint len, const FrTensor& mval
 
 pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const int* vals, const uint D) {
     DevBuf idx(sizeof(uint) * (size_t)D);
-    ZKC(zk_lookup_index_i32(idx.p, vals, low, table.size, D, nullptr));
+    ZKC(zk_lookup_index_i32(idx.p, vals, low, len, D, nullptr));
     FrTensor m = counts_to_m(idx.p, D, table.size);
     FrTensor y(D);
     ZKC(zk_fr_gather(y.gpu_data, mapped_vals.gpu_data, idx.p, D, nullptr));
@@ -61,7 +61,7 @@ pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const int* vals, const 
 }
 pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const FrTensor& vals) {
     DevBuf idx(sizeof(uint) * (size_t)vals.size);
-    ZKC(zk_lookup_index_fr(idx.p, vals.gpu_data, low, table.size, vals.size, nullptr));
+    ZKC(zk_lookup_index_fr(idx.p, vals.gpu_data, low, len, vals.size, nullptr));
     FrTensor m = counts_to_m(idx.p, vals.size, table.size);
     FrTensor y(vals.size);
     ZKC(zk_fr_gather(y.gpu_data, mapped_vals.gpu_data, idx.p, vals.size, nullptr));

@@ -44,6 +44,8 @@ class tLookup {
 class tLookupRange : public tLookup {
    public:
     const int low;
+    const uint len;        // addition: the range's own length (the table is padded to a power of two by repeating its last value);
+                           // a query outside [low, low + len) is an error even when the padded table has room for it
     tLookupRange(int low, uint len);
 
     FrTensor prep(const int* vals, const uint D);   // vals: device pointer
