@@ -15,8 +15,11 @@
  *     Any z == 0 is the point at infinity.
  *   - `stream` is a hipStream_t passed as void* (NULL = default stream).  Launches are
  *     asynchronous; functions that return host values synchronise that stream.
- *   - Scratch memory comes from the library's caching allocator (zk_malloc/zk_free); all work
- *     is expected on one stream at a time.
+ *   - Scratch memory comes from the library's caching allocator (zk_malloc/zk_free).  The allocator
+ *     remembers for every freed block the stream of its last user and makes a new user on another
+ *     stream wait for it, so entry points may be called on different streams.  zk_free assumes the
+ *     default stream; name another with zk_free_async.  Host threads may call concurrently (errors
+ *     and staging buffers are per thread); a *_begin / *_end pair belongs to one thread.
  */
 #ifndef ZKLLM_HIP_H
 #define ZKLLM_HIP_H
@@ -34,7 +37,8 @@ int zk_init(int device);                                   /* hipSetDevice; fail
 int zk_device_info(char* name, int name_len, int* compute_units, int* clock_khz, size_t* total_mem);
 /* replaces the cudaMalloc/cudaFree pair of every FrTensor/G1Tensor ctor/dtor (fr-tensor.cu:158-179) */
 int zk_malloc(void** out, size_t bytes);
-int zk_free(void* p);
+int zk_free(void* p);                                      /* last user: the default stream */
+int zk_free_async(void* p, void* stream);                  /* last user: kernels already queued on `stream` */
 int zk_pool_trim(void);                                    /* return cached blocks to the driver */
 int zk_pool_stats(size_t* live_bytes, size_t* cached_bytes);
 /* replace cudaMemcpy in ctors, operator()(idx), savebin/loadbin (ioutils.cu:3-45) */

@@ -468,3 +468,77 @@ def test_fr_bin_files_round_trip_and_conversions(pv, tmp_path):
     assert pv.from_file(tmp_path / "a32.bin", 2).size == a32.size // 2
     with pytest.raises(RuntimeError):
         pv.from_file(tmp_path / "missing.bin", 1)
+
+
+# ---- the allocator across streams and host threads ---------------------------------------------------------------------------------
+def _hip_streams(n):
+    rt = ctypes.CDLL("libamdhip64.so")
+    out = []
+    for _ in range(n):
+        s = ctypes.c_void_p()
+        assert rt.hipStreamCreateWithFlags(ctypes.byref(s), ctypes.c_uint(1)) == 0      # non-blocking, default priority
+        out.append(s)
+    return rt, out
+
+
+def test_scratch_blocks_reused_on_another_stream_wait_for_their_last_user(hip):
+    """Two matrix products of one shape on two streams back to back: the second call gets the scratch blocks that the first
+    call has just given back while its kernels are still queued, and must not overwrite them early."""
+    rt, (sA, sB) = _hip_streams(2)
+    M, N, P = 2048, 1024, 2048
+    rng = np.random.default_rng(12)
+    mats = [rng.integers(-2000, 2000, size=(M, N)), rng.integers(-2000, 2000, size=(N, P)), rng.integers(-2000, 2000, size=(M, N)), rng.integers(-2000, 2000, size=(N, P))]
+    dev = []
+    for m in mats:
+        d_i = hip.upload(m.astype(np.int64))
+        d_f = hip.malloc(32 * m.size)
+        hip.call("zk_fr_from_i64", ctypes.c_void_p(d_f), ctypes.c_void_p(d_i), ctypes.c_size_t(m.size), None)
+        hip.free(d_i)
+        dev.append(d_f)
+    hip.sync()
+    C = [hip.malloc(32 * M * P) for _ in range(2)]
+    path = ctypes.c_int(0)
+    # entries below 2000 and 1024 terms: every sum stays below 2^53, so the float64 product is exact
+    want = [(mats[0].astype(np.float64) @ mats[1].astype(np.float64)).astype(np.int64).reshape(-1), (mats[2].astype(np.float64) @ mats[3].astype(np.float64)).astype(np.int64).reshape(-1)]
+    for rep in range(3):
+        print("case two streams rep", rep, flush=True)
+        hip.call("zk_fr_matmul", ctypes.c_void_p(C[0]), ctypes.c_void_p(dev[0]), ctypes.c_void_p(dev[1]), ctypes.c_uint32(M), ctypes.c_uint32(N), ctypes.c_uint32(P), ctypes.c_int(2), ctypes.byref(path), sA)
+        hip.call("zk_fr_matmul", ctypes.c_void_p(C[1]), ctypes.c_void_p(dev[2]), ctypes.c_void_p(dev[3]), ctypes.c_uint32(M), ctypes.c_uint32(N), ctypes.c_uint32(P), ctypes.c_int(2), ctypes.byref(path), sB)
+        assert rt.hipStreamSynchronize(sA) == 0 and rt.hipStreamSynchronize(sB) == 0
+        for c, exp in zip(C, want):
+            got = hip.download(c, (M * P, 8), np.uint32)
+            lo = got[:, 0].astype(np.uint64) | (got[:, 1].astype(np.uint64) << np.uint64(32))
+            neg = got[:, 7] != 0
+            val = np.where(neg, -((np.uint64(R_MOD & (2**64 - 1)) - lo).astype(np.int64)), lo.astype(np.int64))
+            assert (val == exp).all()
+    for p in dev + C:
+        hip.free(p)
+    assert rt.hipStreamDestroy(sA) == 0 and rt.hipStreamDestroy(sB) == 0
+
+
+def test_two_host_threads_reduce_on_two_streams(hip):
+    """results come back through a pinned buffer per host thread"""
+    import threading
+    rt, streams = _hip_streams(2)
+    data = [seeded(1 << 18, 50 + i) for i in range(2)]
+    want = [sum(fr_ints(d)) % R_MOD for d in data]
+    dev = [hip.upload(d) for d in data]
+    bad = []
+
+    def work(i):
+        out = np.zeros(8, np.uint32)
+        for _ in range(200):
+            rc = hip.lib.zk_fr_sum(ctypes.c_void_p(out.ctypes.data), ctypes.c_void_p(dev[i]), ctypes.c_size_t(data[i].shape[0]), streams[i])
+            if rc != 0 or fr_ints(out.reshape(1, 8))[0] != want[i]:
+                bad.append((i, rc))
+                return
+    th = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in th:
+        t.start()
+    for t in th:
+        t.join()
+    assert not bad
+    for p in dev:
+        hip.free(p)
+    for s in streams:
+        assert rt.hipStreamDestroy(s) == 0

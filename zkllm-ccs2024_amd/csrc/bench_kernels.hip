@@ -37,7 +37,7 @@ extern "C" {
 int zk_bench_mad_peak(uint32_t blocks, uint32_t iters, double* mad_per_s_host, void* stv) {
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(blocks >= 1 && iters >= 1, "zk_bench_mad_peak: empty launch");
-    Scratch out((size_t)blocks * 256 * 8);
+    Scratch out((size_t)blocks * 256 * 8, st);
     if (out.rc) return out.rc;
     hipEvent_t e0, e1;
     ZK_HIP(hipEventCreate(&e0));

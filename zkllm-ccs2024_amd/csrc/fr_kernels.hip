@@ -201,7 +201,7 @@ template <int K> static int finish_to_host(Fr* partials, unsigned nb, Fr* host_o
     void* stage = nullptr;
     int rc = staging(&stage, sizeof(Fr) * K);
     if (rc) return rc;
-    Scratch fin(sizeof(Fr) * K);
+    Scratch fin(sizeof(Fr) * K, st);
     if (fin.rc) return fin.rc;
     hipLaunchKernelGGL(k_finish_sums, dim3(K), dim3(TPB), 0, st, fin.as<Fr>(), partials, nb);
     ZK_LAUNCH_CHECK();
@@ -558,7 +558,7 @@ int zk_fr_gather(void* out, const void* table, const void* idx, size_t n, void* 
 int zk_fr_sum(uint32_t* out_host, const void* a, size_t n, void* st) {
     if (n == 0) { memset(out_host, 0, 32); return 0; }
     const unsigned nb = reduce_grid(n);
-    Scratch part(sizeof(Fr) * nb);
+    Scratch part(sizeof(Fr) * nb, (hipStream_t)st);
     if (part.rc) return part.rc;
     hipLaunchKernelGGL(k_sum, dim3(nb), dim3(TPB), 0, (hipStream_t)st, part.as<Fr>(), (const Fr*)a, n);
     ZK_LAUNCH_CHECK();
@@ -568,7 +568,7 @@ int zk_fr_sum(uint32_t* out_host, const void* a, size_t n, void* st) {
 int zk_fr_dot(uint32_t* out_host, const void* a, const void* b, size_t n, void* st) {
     if (n == 0) { memset(out_host, 0, 32); return 0; }
     const unsigned nb = reduce_grid(n);
-    Scratch part(sizeof(Fr) * nb);
+    Scratch part(sizeof(Fr) * nb, (hipStream_t)st);
     if (part.rc) return part.rc;
     hipLaunchKernelGGL(k_dot, dim3(nb), dim3(TPB), 0, (hipStream_t)st, part.as<Fr>(), (const Fr*)a, (const Fr*)b, n);
     ZK_LAUNCH_CHECK();
@@ -627,7 +627,7 @@ int zk_fr_me(uint32_t* out_host, const void* a, size_t n, const uint32_t* u, int
     while (cur > ME_SMALL_MAX && rc == 0) {
         const int L = 3;
         const size_t next = (cur + 7) >> 3;
-        if (!bufs[which]) rc = pool_alloc(&bufs[which], next * sizeof(Fr));
+        if (!bufs[which]) rc = pool_alloc(&bufs[which], next * sizeof(Fr), st);
         if (rc) break;
         rc = zk_fr_fold_axis(bufs[which], cur_ptr, u + 8 * done, L, 1, (uint32_t)cur, 1, stv);
         cur_ptr = (const Fr*)bufs[which];
@@ -639,7 +639,7 @@ int zk_fr_me(uint32_t* out_host, const void* a, size_t n, const uint32_t* u, int
         FrPack12 p;
         const int rest = k - done;
         for (int i = 0; i < 12; ++i) p.x[i] = (i < rest) ? to_mont(load_fr(u + 8 * (done + i))) : big_zero<8>();
-        Scratch fin(sizeof(Fr));
+        Scratch fin(sizeof(Fr), st);
         rc = fin.rc;
         void* stage = nullptr;
         if (!rc) rc = staging(&stage, sizeof(Fr));
@@ -652,7 +652,7 @@ int zk_fr_me(uint32_t* out_host, const void* a, size_t n, const uint32_t* u, int
             else memcpy(out_host, stage, 32);
         }
     }
-    for (int i = 0; i < 2; ++i) if (bufs[i]) pool_free(bufs[i]);
+    for (int i = 0; i < 2; ++i) if (bufs[i]) pool_free(bufs[i], st);
     return rc;
 }
 
@@ -666,7 +666,7 @@ int zk_fr_fold_halves(void* out, const void* a, const uint32_t* v, size_t n_in, 
 int zk_ip_round(uint32_t* poly3_host, const void* a, const void* b, size_t n_in, size_t n_out, void* stv) {
     ZK_ARG(n_out >= 1 && n_in >= 1 && n_in <= 2 * n_out, "zk_ip_round: need n_in <= 2*n_out");
     const unsigned nb = reduce_grid(n_out);
-    Scratch part(sizeof(Fr) * 3 * nb);
+    Scratch part(sizeof(Fr) * 3 * nb, (hipStream_t)stv);
     if (part.rc) return part.rc;
     hipLaunchKernelGGL(k_ip_round, dim3(nb), dim3(TPB), 0, (hipStream_t)stv, part.as<Fr>(), (const Fr*)a, (const Fr*)b, n_in, n_out);
     ZK_LAUNCH_CHECK();
@@ -684,7 +684,7 @@ int zk_ip_round_stacked(uint32_t* poly3_host, const void* a, const void* b, cons
     ZK_ARG(D >= 1 && rows_out >= 1 && rows_in >= 1 && rows_in <= 2 * rows_out, "zk_ip_round_stacked: bad shape");
     const size_t n_in = rows_in * D, n_out = rows_out * D;
     const unsigned nb = reduce_grid(n_out);
-    Scratch part(sizeof(Fr) * 3 * nb);
+    Scratch part(sizeof(Fr) * 3 * nb, (hipStream_t)stv);
     if (part.rc) return part.rc;
     hipLaunchKernelGGL(k_ip_round_w, dim3(nb), dim3(TPB), 0, (hipStream_t)stv, part.as<Fr>(), (const Fr*)a, (const Fr*)b, (const Fr*)E, D, n_in, n_out);
     ZK_LAUNCH_CHECK();
@@ -705,7 +705,7 @@ int zk_ip_sumcheck_small(uint32_t* polys_host, uint32_t* fin_host, const void* a
     FrPack16 p;
     for (int i = 0; i < 16; ++i) p.x[i] = (i < k) ? to_mont(load_fr(u + 8 * i)) : big_zero<8>();
     const size_t half0 = ((size_t)1 << k) >> 1;
-    Scratch work(sizeof(Fr) * (4 * half0 + 3 * (size_t)k + 2));
+    Scratch work(sizeof(Fr) * (4 * half0 + 3 * (size_t)k + 2), st);
     if (work.rc) return work.rc;
     Fr* w = work.as<Fr>();
     Fr* polys = w + 4 * half0;

@@ -898,7 +898,7 @@ static int g1_sum_device(G1Jac* out, const G1Jac* in, size_t n, hipStream_t st) 
         ZK_LAUNCH_CHECK();
         return 0;
     }
-    Scratch part(sizeof(G1Jac) * nseg);
+    Scratch part(sizeof(G1Jac) * nseg, st);
     if (part.rc) return part.rc;
     hipLaunchKernelGGL(k_g1_rowsum, dim3(1, nseg), dim3(GT), 0, st, part.as<G1Jac>(), in, n, nseg);
     hipLaunchKernelGGL(k_g1_rowsum, dim3(1, 1), dim3(GT), 0, st, out, part.as<G1Jac>(), (size_t)nseg, 1u);
@@ -1149,7 +1149,7 @@ int zk_g1_scalar_mul(void* out, const void* g, const void* s, size_t ng, size_t 
 }
 int zk_g1_sum(uint32_t* out_host, const void* a, size_t n, void* stv) {
     hipStream_t st = (hipStream_t)stv;
-    Scratch res(sizeof(G1Jac));
+    Scratch res(sizeof(G1Jac), st);
     if (res.rc) return res.rc;
     int rc = g1_sum_device(res.as<G1Jac>(), (const G1Jac*)a, n, st);
     if (rc) return rc;
@@ -1173,7 +1173,7 @@ int zk_g1_rowwise_sum(void* out, const void* in, size_t nrow, size_t ncol, void*
         ZK_LAUNCH_CHECK();
         return 0;
     }
-    Scratch part(sizeof(G1Jac) * nrow * nseg);
+    Scratch part(sizeof(G1Jac) * nrow * nseg, st);
     if (part.rc) return part.rc;
     hipLaunchKernelGGL(k_g1_rowsum, dim3((unsigned)nrow, nseg), dim3(GT), 0, st, part.as<G1Jac>(), (const G1Jac*)in, ncol, nseg);
     hipLaunchKernelGGL(k_g1_rowsum, dim3((unsigned)nrow, 1), dim3(GT), 0, st, (G1Jac*)out, part.as<G1Jac>(), (size_t)nseg, 1u);
@@ -1190,7 +1190,7 @@ int zk_g1_me(uint32_t* out_host, const void* a, size_t n, const uint32_t* u, int
     int which = 0, rc = 0;
     for (int lvl = 0; lvl < k && rc == 0; ++lvl) {
         const size_t out_n = (cur_n + 1) / 2;
-        if (!bufs[which]) rc = pool_alloc(&bufs[which], sizeof(G1Jac) * out_n);
+        if (!bufs[which]) rc = pool_alloc(&bufs[which], sizeof(G1Jac) * out_n, st);
         if (rc) break;
         const Fr x = from_mont(load_fr(u + 8 * lvl));   // the reference passes unmont(u) to the scalar multiplication
         hipLaunchKernelGGL(k_g1_me_step, dim3(cdiv(out_n, GT)), dim3(GT), 0, st, (G1Jac*)bufs[which], cur, x, cur_n, out_n);
@@ -1209,7 +1209,7 @@ int zk_g1_me(uint32_t* out_host, const void* a, size_t n, const uint32_t* u, int
             else memcpy(out_host, stage, sizeof(G1Jac));
         }
     }
-    for (int i = 0; i < 2; ++i) if (bufs[i]) pool_free(bufs[i]);
+    for (int i = 0; i < 2; ++i) if (bufs[i]) pool_free(bufs[i], st);
     return rc;
 }
 // canonical form: z = ONE (Montgomery), infinity = all-zero limbs.  out may alias in.
@@ -1228,7 +1228,7 @@ int zk_g1_commit_int(void* out, const void* gens, const void* scalars_fr, size_t
     ZK_ARG(ngen >= 1, "zk_g1_commit_int: no generators");
     ZK_ARG(m <= 0x7fffffffu, "zk_g1_commit_int: too many rows");
     const size_t total = m * ngen;
-    Scratch ints(sizeof(int32_t) * total), flags(8);
+    Scratch ints(sizeof(int32_t) * total, st), flags(8, st);
     if (ints.rc) return ints.rc;
     if (flags.rc) return flags.rc;
     ZK_HIP(hipMemsetAsync(flags.p, 0, 8, st));
@@ -1249,14 +1249,14 @@ int zk_g1_commit_int(void* out, const void* gens, const void* scalars_fr, size_t
     if (nwin == 0) nwin = 1;
     const uint32_t half = 1u << (c - 1);
     const size_t tab_n = (size_t)nwin * ngen * half;
-    Scratch tabj(sizeof(G1Jac) * tab_n), taba(sizeof(G1Affine) * tab_n);
+    Scratch tabj(sizeof(G1Jac) * tab_n, st), taba(sizeof(G1Affine) * tab_n, st);
     if (tabj.rc) return tabj.rc;
     if (taba.rc) return taba.rc;
     hipLaunchKernelGGL(k_msm_table_bases, dim3(cdiv(ngen, GT)), dim3(GT), 0, st, tabj.as<G1Jac>(), (const G1Jac*)gens, ngen, c, nwin);
     for (uint32_t logk = 0; logk + 1 < c; ++logk)
         hipLaunchKernelGGL(k_msm_table_fill, dim3(cdiv(((size_t)nwin * ngen) << logk, GT)), dim3(GT), 0, st, tabj.as<G1Jac>(), (size_t)nwin * ngen, c - 1, logk);
     hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(tab_n, CH), GT)), dim3(GT), 0, st, taba.p, tabj.as<G1Jac>(), tab_n);
-    Scratch tab29(sizeof(A29) * tab_n);
+    Scratch tab29(sizeof(A29) * tab_n, st);
     if (tab29.rc) return tab29.rc;
     hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(tab_n, 256)), dim3(256), 0, st, tab29.as<A29>(), taba.as<G1Affine>(), tab_n);
     ZK_LAUNCH_CHECK();
@@ -1267,7 +1267,7 @@ int zk_g1_commit_int(void* out, const void* gens, const void* scalars_fr, size_t
         ZK_LAUNCH_CHECK();
         return 0;
     }
-    Scratch part(sizeof(G1Jac) * m * nseg);
+    Scratch part(sizeof(G1Jac) * m * nseg, st);
     if (part.rc) return part.rc;
     hipLaunchKernelGGL(k_msm_rows, dim3((unsigned)m, nseg), dim3(GT), 0, st, part.as<G1Jac>(), tab29.as<A29>(), ints.as<int32_t>(), ngen, c, nwin, nseg);
     hipLaunchKernelGGL(k_g1_rowsum, dim3((unsigned)m, 1), dim3(GT), 0, st, (G1Jac*)out, part.as<G1Jac>(), (size_t)nseg, 1u);
@@ -1293,7 +1293,7 @@ int zk_g1_fixed_base_mul(void* out, const uint32_t* base_host, const void* scala
         if (tab && tab_dev != dev) { int cur = dev; ZK_HIP(hipSetDevice(tab_dev)); ZK_HIP(hipFree(tab)); ZK_HIP(hipSetDevice(cur)); tab = nullptr; }
         if (!tab) ZK_HIP(hipMalloc(&tab, sizeof(A29) * tab_n));
         tab_dev = -1;                                   // not valid until the build below has finished
-        Scratch b(sizeof(G1Jac)), tabj(sizeof(G1Jac) * tab_n), taba(sizeof(G1Affine) * tab_n);
+        Scratch b(sizeof(G1Jac), st), tabj(sizeof(G1Jac) * tab_n, st), taba(sizeof(G1Affine) * tab_n, st);
         if (b.rc) return b.rc;
         if (tabj.rc) return tabj.rc;
         if (taba.rc) return taba.rc;
@@ -1319,11 +1319,11 @@ int zk_g1_fixed_base_mul(void* out, const uint32_t* base_host, const void* scala
 int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host, const void* scalars, const void* gens, const uint32_t* u, size_t old_size, void* stv) {
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(old_size >= 1, "zk_g1_open_round: empty input");
-    Scratch pts(sizeof(G1Jac) * 3);
+    Scratch pts(sizeof(G1Jac) * 3, st);
     if (pts.rc) return pts.rc;
-    Scratch wsum(sizeof(G1Jac) * 3 * MW);
+    Scratch wsum(sizeof(G1Jac) * 3 * MW, st);
     if (wsum.rc) return wsum.rc;
-    Arena arena;
+    Arena arena(st);
     std::vector<hipEvent_t> evs;
     int rc = open_round_launch((Fr*)new_scalars, (G1Jac*)new_gens, (const Fr*)scalars, (const G1Jac*)gens, load_fr(u), old_size, true, wsum.as<G1Jac>(), arena, st, st, evs);
     (void)evs;
@@ -1359,6 +1359,7 @@ static int open_queue(OpenJob& job, const void* scalars, const void* gens, size_
     ZK_ARG(sizeof(G1Jac) * (3 * (size_t)rounds + 1) + sizeof(Fr) <= 65536, "zk_g1_open: proof larger than the staging buffer");
     job.st = st;
     job.aux = aux;
+    job.arena.streams(st, aux);      // blocks serve kernels of both streams; aux joins st before the job ends
     job.rounds = rounds;
     const size_t npts = 3 * (size_t)rounds + 1;
     Scratch& pts = job.arena.add(sizeof(G1Jac) * npts);
@@ -1461,6 +1462,7 @@ int zk_g1_open_end(void* handle, uint32_t* proof_host, uint32_t* final_scalar_ho
     std::unique_ptr<OpenJob> job((OpenJob*)handle);
     int rc = open_collect(*job, proof_host, final_scalar_host);
     if (rc) { (void)hipStreamSynchronize(job->st); (void)hipStreamSynchronize(job->aux); }
+    job->arena.mark_idle();          // both streams have drained behind the job's last kernel
     (void)hipEventDestroy(job->ready);
     for (hipEvent_t e : job->events) (void)hipEventDestroy(e);
     return rc;

@@ -73,7 +73,7 @@ static int finish_sums(Fr* partials, unsigned nb, int K, int n_mont, Fr* host_ou
     void* stage = nullptr;
     int rc = staging(&stage, sizeof(Fr) * K);
     if (rc) return rc;
-    Scratch fin(sizeof(Fr) * K);
+    Scratch fin(sizeof(Fr) * K, st);
     if (fin.rc) return fin.rc;
     hipLaunchKernelGGL(k_finish, dim3(K), dim3(TPB), 0, st, fin.as<Fr>(), partials, nb);
     ZK_LAUNCH_CHECK();
@@ -250,8 +250,8 @@ __global__ void __launch_bounds__(TPB) k_hp_count(uint32_t* __restrict__ counts,
 static int hist_partitioned(uint32_t* counts, const uint32_t* idx, size_t n, uint32_t nbins, hipStream_t st) {
     const uint32_t P = (nbins + HP_BINS - 1) / HP_BINS, ntiles = cdiv(n, HP_TILE), M = P * ntiles;
     const uint32_t max_slices = (uint32_t)(n / HP_SLICE) + P + 1;
-    Scratch sizes(sizeof(uint32_t) * (size_t)M), part_off(sizeof(uint32_t) * (P + 1)), totals(sizeof(uint32_t) * P), slice_tab(sizeof(uint32_t) * max_slices),
-        nsl(sizeof(uint32_t)), parted(sizeof(uint16_t) * n);
+    Scratch sizes(sizeof(uint32_t) * (size_t)M, st), part_off(sizeof(uint32_t) * (P + 1), st), totals(sizeof(uint32_t) * P, st), slice_tab(sizeof(uint32_t) * max_slices, st),
+        nsl(sizeof(uint32_t), st), parted(sizeof(uint16_t) * n, st);
     for (const Scratch* b : {&sizes, &part_off, &totals, &slice_tab, &nsl, &parted})
         if (b->rc) return b->rc;
     hipLaunchKernelGGL(k_hp_sizes, dim3(ntiles), dim3(TPB), 0, st, sizes.as<uint32_t>(), idx, n, P, ntiles);
@@ -1010,7 +1010,7 @@ extern "C" {
 int zk_lookup_index_fr(void* idx_u32, const void* vals, int32_t low, uint32_t table_size, size_t n, void* stv) {
     hipStream_t st = (hipStream_t)stv;
     if (n == 0) return 0;
-    Scratch flag(4);
+    Scratch flag(4, st);
     if (flag.rc) return flag.rc;
     ZK_HIP(hipMemsetAsync(flag.p, 0, 4, st));
     LAUNCH1D(k_index_fr, n, st, (uint32_t*)idx_u32, flag.as<uint32_t>(), (const Fr*)vals, fr_from_i64((int64_t)low), table_size, n);
@@ -1023,7 +1023,7 @@ int zk_lookup_index_fr(void* idx_u32, const void* vals, int32_t low, uint32_t ta
 int zk_lookup_index_i32(void* idx_u32, const void* vals_i32, int32_t low, uint32_t table_size, size_t n, void* stv) {
     hipStream_t st = (hipStream_t)stv;
     if (n == 0) return 0;
-    Scratch flag(4);
+    Scratch flag(4, st);
     if (flag.rc) return flag.rc;
     ZK_HIP(hipMemsetAsync(flag.p, 0, 4, st));
     LAUNCH1D(k_index_i32, n, st, (uint32_t*)idx_u32, flag.as<uint32_t>(), (const int32_t*)vals_i32, low, table_size, n);
@@ -1059,16 +1059,14 @@ int zk_range_table(void* table, int32_t low, uint32_t len, uint32_t table_size, 
 // out[i] = 1 / (in[i] + beta), standard form; 0 where in[i] + beta == 0 (tlookup_inv_kernel tlookup.cu:50-62)
 int zk_fr_batch_inv(void* out, const void* in, const uint32_t* beta, size_t n, void* st) {
     if (n == 0) return 0;
-    Arena tmp;
-    int rc = batch_inv_queue((Fr*)out, (const Fr*)in, load_fr(beta), n, tmp, (hipStream_t)st);
-    // large inputs use scratch memory that goes back to the allocator when this returns: wait for its last use
-    if (!tmp.v.empty()) { hipError_t e = hipStreamSynchronize((hipStream_t)st); if (rc == 0 && e != hipSuccess) return hip_fail(e, "hipStreamSynchronize", __FILE__, __LINE__); }
-    return rc;
+    Arena tmp((hipStream_t)st);
+    // large inputs use scratch memory that goes back to the allocator when this returns, remembered as last used on `st`
+    return batch_inv_queue((Fr*)out, (const Fr*)in, load_fr(beta), n, tmp, (hipStream_t)st);
 }
 // E[t] for t < 2^k (Montgomery form) from k standard-form challenges; out holds 2^k elements
 int zk_eq_table(void* out, const uint32_t* u, int k, void* stv) {
     ZK_ARG(k >= 0 && k <= 30, "zk_eq_table: k out of range");
-    Arena tmp;        // the half tables return to the allocator at once: later users are ordered behind these launches on the same stream
+    Arena tmp((hipStream_t)stv);        // the half tables return to the allocator at once: later users are ordered behind these launches on the same stream
     return eq_table_queue((Fr*)out, u, k, tmp, (hipStream_t)stv);
 }
 // out_host[i] = multilinear extension of Xs[i] (n elements each, zero beyond) at u (k challenges, 2^(k-1) < n <= 2^k)
@@ -1076,7 +1074,7 @@ int zk_fr_me_multi(uint32_t* out_host, const void* const* Xs, int K, size_t n, c
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(K >= 1 && K <= 8, "zk_fr_me_multi: 1..8 tensors");
     ZK_ARG(k >= 0 && k <= 30 && n >= 1 && n <= ((size_t)1 << k) && (k == 0 || n > ((size_t)1 << (k - 1))), "zk_fr_me_multi: n does not match the number of challenges");
-    Arena tmp;
+    Arena tmp(st);
     Scratch& E = tmp.add(sizeof(Fr) * ((size_t)1 << k));
     if (E.rc) return E.rc;
     int rc = eq_table_queue(E.as<Fr>(), u, k, tmp, st);
@@ -1109,7 +1107,7 @@ int zk_lookup_round(uint32_t* sums_host, void* nA, void* nS, void* nB, void* nT,
     ZK_ARG(n_out >= 1, "zk_lookup_round: empty round");
     const unsigned nb = reduce_grid(n_out);
     const int K = phase2 ? 11 : 5;
-    Scratch part(sizeof(Fr) * K * nb);
+    Scratch part(sizeof(Fr) * K * nb, st);
     if (part.rc) return part.rc;
     const Fr b = load_fr(beta), vm = to_mont(load_fr(v));
     if (phase2)
@@ -1136,7 +1134,7 @@ int zk_hadamard_round(uint32_t* coefs_host, void* const* new_Xs, const void* con
     ZK_ARG(K >= 1 && K <= 4, "zk_hadamard_round: K must be 1..4");
     ZK_ARG(n_out >= 1, "zk_hadamard_round: empty round");
     const unsigned nb = reduce_grid(n_out);
-    Scratch part(sizeof(Fr) * (K + 1) * nb);
+    Scratch part(sizeof(Fr) * (K + 1) * nb, st);
     if (part.rc) return part.rc;
     const Fr vm = to_mont(load_fr(v));
 #define HAD_CASE(KK)                                                                                                           \
@@ -1389,6 +1387,7 @@ static int lookup_args_ok(size_t D, size_t N, int rounds) {
 // puts a new job on one of the library's streams, ordered after everything queued on `caller` so far
 static int sumjob_on_side_stream(SumJob& job, hipStream_t caller) {
     job.st = side_stream(1);
+    job.arena.st = job.st;
     ZK_ARG(job.st != nullptr, "could not create a stream");
     ZK_HIP(hipEventCreateWithFlags(&job.ready, hipEventDisableTiming));
     ZK_HIP(hipEventRecord(job.ready, caller));
@@ -1399,6 +1398,7 @@ static void sumjob_abort(SumJob* job) {
     // the job's buffers go back to the allocator: wait for its last use (the whole stream when the job never got as far as its event)
     if (job->done) (void)hipEventSynchronize(job->done);
     else if (job->st) (void)hipStreamSynchronize(job->st);
+    job->arena.mark_idle();          // the job's kernels have all finished
     if (job->done) (void)hipEventDestroy(job->done);
     pinned_release(job->host);
     if (job->ready) (void)hipEventDestroy(job->ready);
@@ -1415,6 +1415,7 @@ int zk_lookup_sumcheck(uint32_t* sums_host, const void* A, const void* S, const 
     if (rc) return rc;
     SumJob job;
     job.st = (hipStream_t)stv;
+    job.arena.st = job.st;
     rc = lookup_queue(job, (const Fr*)A, (const Fr*)S, (const Fr*)B, (const Fr*)T, (const Fr*)m, (const Fr*)E, load_fr(beta), v, D, N, rounds);
     if (rc) { (void)hipStreamSynchronize(job.st); return rc; }
     rc = sumjob_collect(job, (Fr*)sums_host, nullptr);
@@ -1506,6 +1507,7 @@ int zk_hadamard_sumcheck(uint32_t* coefs_host, const void* const* Xs, int K, con
     ZK_ARG(N >= 2 && (N & (N - 1)) == 0, "zk_hadamard_sumcheck: N must be a power of two >= 2");
     SumJob job;
     job.st = (hipStream_t)stv;
+    job.arena.st = job.st;
     int rc = hadamard_queue(job, (const Fr* const*)Xs, K, (const Fr*)E, v, N);
     if (rc) { (void)hipStreamSynchronize(job.st); return rc; }
     return sumjob_collect(job, (Fr*)coefs_host, nullptr);
@@ -1545,7 +1547,7 @@ int zk_hadamard_product_sumcheck(uint32_t* proof_host, const void* a, const void
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(k >= 1 && k <= 30 && n <= ((size_t)1 << k) && n > ((size_t)1 << (k - 1)), "zk_hadamard_product_sumcheck: n does not match the number of challenges");
     ZK_ARG(sizeof(Fr) * (3 * (size_t)k + 2) <= 65536, "zk_hadamard_product_sumcheck: too many rounds for the staging buffer");
-    Arena arena;
+    Arena arena(st);
     const size_t half = (n + 1) / 2, etab = (size_t)1 << (k - 1);
     Scratch& E = arena.add(sizeof(Fr) * (etab + etab / 2 + 1));          // eq tables, ping-pong
     Scratch& W = arena.add(sizeof(Fr) * 2 * (half + (half + 1) / 2 + 1));   // folded a, b, ping-pong
@@ -1609,7 +1611,7 @@ int zk_softmax_decompose(void* const* planes, const void* X_shifted, const uint3
     U32Pack8 bs;
     for (int i = 0; i < 8; ++i) bs.v[i] = i < K ? bs_host[i] : 1u;
     for (int i = 0; i < K; ++i) ZK_ARG(bs.v[i] >= 1, "zk_softmax_decompose: zero radix");
-    Scratch flag(4);
+    Scratch flag(4, st);
     if (flag.rc) return flag.rc;
     ZK_HIP(hipMemsetAsync(flag.p, 0, 4, st));
     PlanePtrs pp;

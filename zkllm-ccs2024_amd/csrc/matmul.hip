@@ -297,7 +297,7 @@ __global__ void __launch_bounds__(256) k_matmul_wide_narrow(Fr* __restrict__ C, 
 }
 static int run_wide_narrow_path(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, hipStream_t st) {
     const size_t na = (size_t)batch * M * N, nb = (size_t)batch * N * P;
-    Scratch ai(na * sizeof(long long)), bi(nb * sizeof(int));
+    Scratch ai(na * sizeof(long long), st), bi(nb * sizeof(int), st);
     if (ai.rc) return ai.rc;
     if (bi.rc) return bi.rc;
     hipLaunchKernelGGL(k_fr_to_int<long long>, dim3(cdiv(na, 256)), dim3(256), 0, st, ai.as<long long>(), (const Fr*)A, na);
@@ -309,7 +309,7 @@ static int run_wide_narrow_path(void* C, const void* A, const void* B, uint32_t 
 
 template <typename T> static int run_int_path(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, hipStream_t st) {
     const size_t na = (size_t)batch * M * N, nb = (size_t)batch * N * P;
-    Scratch ai(na * sizeof(T)), bi(nb * sizeof(T));
+    Scratch ai(na * sizeof(T), st), bi(nb * sizeof(T), st);
     if (ai.rc) return ai.rc;
     if (bi.rc) return bi.rc;
     hipLaunchKernelGGL(k_fr_to_int<T>, dim3(cdiv(na, 256)), dim3(256), 0, st, ai.as<T>(), (const Fr*)A, na);
@@ -375,7 +375,7 @@ static int run_int8_plane_path(void* C, const void* A, const void* B, uint32_t M
     rocblas_handle h = blas_handle();
     if (!h) return 0;
     const size_t na = (size_t)M * N, nb = (size_t)N * P, nc = (size_t)M * P;
-    Scratch pla(na * pa), plb(nb * pb), cs(nc * ns * sizeof(int32_t));
+    Scratch pla(na * pa, st), plb(nb * pb, st), cs(nc * ns * sizeof(int32_t), st);
     if (pla.rc) return pla.rc;
     if (plb.rc) return plb.rc;
     if (cs.rc) return cs.rc;
@@ -435,7 +435,7 @@ static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch
     bool small = false, fits32 = false, b_fits32 = false;
     unsigned long long ma_ = 0, mb_ = 0;
     if (mode != 1) {
-        Scratch mx(3 * sizeof(unsigned long long));
+        Scratch mx(3 * sizeof(unsigned long long), st);
         if (mx.rc) return mx.rc;
         ZK_HIP(hipMemsetAsync(mx.p, 0, 3 * sizeof(unsigned long long), st));
         const size_t na = (size_t)batch * M * N, nb = (size_t)batch * N * P;

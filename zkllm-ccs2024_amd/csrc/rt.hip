@@ -3,6 +3,7 @@
 #include <map>
 #include <mutex>
 #include <unordered_map>
+#include <utility>
 #include <vector>
 #include <cstdio>
 #include <cstring>
@@ -22,11 +23,16 @@ int hip_fail(hipError_t e, const char* what, const char* file, int line) {
     return (int)e;
 }
 
+struct Block { size_t size; hipStream_t last; bool idle; uint64_t freed_tick; hipEvent_t ev; bool ev_set; };
 struct Pool {
     std::mutex mu;
     std::map<size_t, std::vector<void*>> free_lists;
-    std::unordered_map<void*, size_t> live;     // every block we own -> rounded size
+    std::unordered_map<void*, Block> live;      // every block we own -> rounded size and last user
     size_t cached_bytes = 0, live_bytes = 0;
+    hipEvent_t events[32] = {};
+    unsigned next_event = 0;
+    uint64_t tick = 0;                                                     // counts frees
+    std::map<std::pair<hipStream_t, hipStream_t>, uint64_t> synced;        // (from, to) -> frees on `from` up to this tick are already waited for by `to`
 };
 static Pool& pool() { static Pool p; return p; }
 
@@ -41,17 +47,59 @@ static size_t round_size(size_t b) {
     return (b + g - 1) / g * g;
 }
 
-int pool_alloc(void** out, size_t bytes) {
+// The library's own streams and the default stream live as long as the process.  A caller's stream may be destroyed while
+// blocks it used last still sit in the free lists, and a destroyed stream must never be passed to the runtime again: for
+// such streams the event is recorded when the block is freed (the stream is certainly alive then) and kept with the block.
+static std::mutex g_side_mu;
+static hipStream_t g_side_streams[2][8] = {};
+static bool is_persistent_stream(hipStream_t s) {
+    if (s == nullptr) return true;
+    std::lock_guard<std::mutex> lk(g_side_mu);
+    for (auto& row : g_side_streams) for (hipStream_t t : row) if (t == s) return true;
+    return false;
+}
+
+// Makes `stream` wait for what `blk`'s last user had queued when it let the block go.  Called with the pool locked.
+static void order_behind_last_user(Pool& P, const Block& blk, hipStream_t stream) {
+    if (blk.idle || blk.last == stream) return;
+    if (blk.ev_set) {                                             // recorded at free time on a caller's stream
+        if (hipStreamWaitEvent(stream, blk.ev, 0) != hipSuccess) { (void)hipGetLastError(); (void)hipDeviceSynchronize(); }
+        return;
+    }
+    uint64_t& covered = P.synced[std::make_pair(blk.last, stream)];
+    if (blk.freed_tick <= covered && covered != 0) return;      // an earlier wait of this stream on that one was placed after this block's free
+    const uint64_t now = P.tick;
+    hipEvent_t& ev = P.events[P.next_event++ % 32];
+    if (!ev && hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) { (void)hipGetLastError(); ev = nullptr; }
+    // a wait takes the event's state at this call, so the event can be recorded again for the next block at once
+    if (ev && hipEventRecord(ev, blk.last) == hipSuccess && hipStreamWaitEvent(stream, ev, 0) == hipSuccess) { covered = now; return; }
+    (void)hipGetLastError();
+    (void)hipDeviceSynchronize();        // no event: wait for everything
+    covered = now;
+}
+
+int pool_alloc(void** out, size_t bytes, hipStream_t stream, const hipStream_t* also) {
     Pool& P = pool();
     const size_t sz = round_size(bytes);
     {
         std::lock_guard<std::mutex> lk(P.mu);
         auto it = P.free_lists.find(sz);
         if (it != P.free_lists.end() && !it->second.empty()) {
-            *out = it->second.back();
-            it->second.pop_back();
+            std::vector<void*>& fl = it->second;
+            // prefer a block that needs no wait (same stream or idle) among the most recently freed
+            size_t pick = fl.size() - 1;
+            for (size_t k = 0; k < 8 && k < fl.size(); ++k) {
+                const Block& b = P.live[fl[fl.size() - 1 - k]];
+                if (b.idle || b.last == stream) { pick = fl.size() - 1 - k; break; }
+            }
+            void* p = fl[pick];
+            fl[pick] = fl.back();
+            fl.pop_back();
+            order_behind_last_user(P, P.live[p], stream);
+            if (also) order_behind_last_user(P, P.live[p], *also);
             P.cached_bytes -= sz;
             P.live_bytes += sz;
+            *out = p;
             return 0;
         }
     }
@@ -64,20 +112,31 @@ int pool_alloc(void** out, size_t bytes) {
         if (e != hipSuccess) return hip_fail(e, "hipMalloc", __FILE__, __LINE__);
     }
     std::lock_guard<std::mutex> lk(P.mu);
-    P.live[p] = sz;
+    P.live[p] = Block{sz, stream, true, 0, nullptr, false};
     P.live_bytes += sz;
     *out = p;
     return 0;
 }
-int pool_free(void* p) {
+int pool_free(void* p, hipStream_t stream, bool idle) {
     if (!p) return 0;
+    const bool persistent = idle || is_persistent_stream(stream);
     Pool& P = pool();
     std::lock_guard<std::mutex> lk(P.mu);
     auto it = P.live.find(p);
     if (it == P.live.end()) { set_error(ZK_ERR_ARG, "zk_free: pointer was not allocated by zk_malloc"); return ZK_ERR_ARG; }
-    P.free_lists[it->second].push_back(p);
-    P.cached_bytes += it->second;
-    P.live_bytes -= it->second;
+    Block& b = it->second;
+    b.last = stream;
+    b.idle = idle;
+    b.freed_tick = ++P.tick;
+    b.ev_set = false;
+    if (!idle && !persistent) {
+        if (!b.ev && hipEventCreateWithFlags(&b.ev, hipEventDisableTiming) != hipSuccess) { (void)hipGetLastError(); b.ev = nullptr; }
+        if (b.ev && hipEventRecord(b.ev, stream) == hipSuccess) b.ev_set = true;
+        else { (void)hipGetLastError(); (void)hipStreamSynchronize(stream); b.idle = true; }
+    }
+    P.free_lists[it->second.size].push_back(p);
+    P.cached_bytes += it->second.size;
+    P.live_bytes -= it->second.size;
     return 0;
 }
 int pool_trim() {
@@ -86,7 +145,11 @@ int pool_trim() {
     {
         std::lock_guard<std::mutex> lk(P.mu);
         for (auto& kv : P.free_lists) {
-            for (void* p : kv.second) { victims.push_back(p); P.live.erase(p); }
+            for (void* p : kv.second) {
+                victims.push_back(p);
+                auto it = P.live.find(p);
+                if (it != P.live.end()) { if (it->second.ev) (void)hipEventDestroy(it->second.ev); P.live.erase(it); }
+            }
             kv.second.clear();
         }
         P.cached_bytes = 0;
@@ -97,7 +160,7 @@ int pool_trim() {
 }
 
 hipStream_t side_stream(int pool) {
-    static hipStream_t streams[2][8] = {};
+    std::lock_guard<std::mutex> lk(g_side_mu);
     static unsigned next[2] = {0, 0};
     static int count[2] = {0, 0}, shared = 0;
     if (!count[0]) {
@@ -109,8 +172,9 @@ hipStream_t side_stream(int pool) {
     }
     const int q = (pool && !shared) ? 1 : 0;
     const unsigned i = next[q]++ % (unsigned)count[q];
-    if (!streams[q][i] && hipStreamCreateWithFlags(&streams[q][i], hipStreamNonBlocking) != hipSuccess) { (void)hipGetLastError(); streams[q][i] = nullptr; return nullptr; }
-    return streams[q][i];
+    hipStream_t& s = g_side_streams[q][i];
+    if (!s && hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) { (void)hipGetLastError(); s = nullptr; return nullptr; }
+    return s;
 }
 
 static std::mutex g_pinned_mu;
@@ -132,7 +196,7 @@ void pinned_release(void* host_ptr) {
 }
 
 int staging(void** host_ptr, size_t bytes) {
-    static void* buf = nullptr;
+    static thread_local void* buf = nullptr;     // one per host thread, kept until the process ends
     static const size_t cap = 64 << 10;
     ZK_ARG(bytes <= cap, "staging request over 64 KiB");
     if (!buf) ZK_HIP(hipHostMalloc(&buf, cap, hipHostMallocDefault));
@@ -171,8 +235,9 @@ int zk_device_info(char* name, int name_len, int* compute_units, int* clock_khz,
     if (total_mem) *total_mem = prop.totalGlobalMem;
     return 0;
 }
-int zk_malloc(void** out, size_t bytes) { ZK_ARG(out != nullptr, "zk_malloc: null out"); return pool_alloc(out, bytes ? bytes : 1); }
-int zk_free(void* p) { return pool_free(p); }
+int zk_malloc(void** out, size_t bytes) { ZK_ARG(out != nullptr, "zk_malloc: null out"); return pool_alloc(out, bytes ? bytes : 1, nullptr); }
+int zk_free(void* p) { return pool_free(p, nullptr); }
+int zk_free_async(void* p, void* stream) { return pool_free(p, (hipStream_t)stream); }
 int zk_pool_trim(void) { return pool_trim(); }
 int zk_pool_stats(size_t* live_bytes, size_t* cached_bytes) {
     Pool& P = pool();

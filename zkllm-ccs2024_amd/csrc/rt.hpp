@@ -33,28 +33,40 @@ int hip_fail(hipError_t e, const char* what, const char* file, int line);
 
 #define ZK_LAUNCH_CHECK() ZK_HIP(hipGetLastError())
 
-// Caching allocator: blocks are kept on per-size free lists and reused; all work is assumed to
-// run on one stream, so a block handed out again is ordered after its previous user.
-int pool_alloc(void** out, size_t bytes);
-int pool_free(void* p);
+// Caching allocator: blocks are kept on per-size free lists and reused.  Every block remembers the stream its last user
+// named when it was freed.  A block handed out for another stream makes that stream wait (an event recorded on the old
+// stream at that moment covers everything queued there before the free) -- so reuse is ordered behind the previous user
+// whatever streams the two run on.  Blocks freed as `idle` (their stream is known to have drained) need no wait.
+// `also`: a second stream whose kernels will touch the block too (a job that runs on two streams); it is ordered as well.
+int pool_alloc(void** out, size_t bytes, hipStream_t stream, const hipStream_t* also = nullptr);
+int pool_free(void* p, hipStream_t stream, bool idle = false);
 int pool_trim();
 
-// RAII scratch from the pool for use inside one entry point.
+// RAII scratch from the pool for use inside one entry point; `stream` is the stream the entry point's kernels run on.
 struct Scratch {
     void* p = nullptr;
     int rc = 0;
-    explicit Scratch(size_t bytes) { rc = pool_alloc(&p, bytes ? bytes : 1); }
-    ~Scratch() { if (p) pool_free(p); }
+    hipStream_t st = nullptr;
+    bool idle_on_free = false;      // set when the owner has synchronised the stream before releasing
+    Scratch(size_t bytes, hipStream_t stream, const hipStream_t* also = nullptr) : st(stream) { rc = pool_alloc(&p, bytes ? bytes : 1, stream, also); }
+    ~Scratch() { if (p) pool_free(p, st, idle_on_free); }
     template <class T> T* as() const { return reinterpret_cast<T*>(p); }
     Scratch(const Scratch&) = delete;
     Scratch& operator=(const Scratch&) = delete;
 };
 
-// Device buffers of one job that may run on a stream of its own: all released together once that stream has drained,
-// so none of them returns to the allocator while the job's kernels are pending.
+// Device buffers of one job that may run on a stream of its own: all released together, tagged with the job's stream (or
+// as idle once the owner has waited for that stream), so none of them reaches another stream's kernels early.
 struct Arena {
+    hipStream_t st = nullptr;       // set before the first add(); blocks are released as last used on this stream
+    hipStream_t st2 = nullptr;      // a job's second stream, when it has one: its work must have joined `st` before release
+    bool two = false;
     std::vector<std::unique_ptr<Scratch>> v;
-    Scratch& add(size_t bytes) { v.emplace_back(new Scratch(bytes)); return *v.back(); }
+    Arena() = default;
+    explicit Arena(hipStream_t stream) : st(stream) {}
+    void streams(hipStream_t a, hipStream_t b) { st = a; st2 = b; two = (a != b); }
+    Scratch& add(size_t bytes) { v.emplace_back(new Scratch(bytes, st, two ? &st2 : nullptr)); return *v.back(); }
+    void mark_idle() { for (auto& s : v) s->idle_on_free = true; }
 };
 // One of the library's own streams (non-blocking, default priority), handed out round-robin; null on failure.
 // Two pools, so that a short job (pool 1: sumchecks) never queues behind a long one (pool 0: openings).
@@ -65,7 +77,7 @@ hipStream_t side_stream(int pool);
 int pinned_acquire(void** host_ptr);
 void pinned_release(void* host_ptr);
 
-// Pinned host buffer (64 KiB) for device->host results of reductions.
+// Pinned host buffer (64 KiB, one per host thread) for device->host results of reductions.
 int staging(void** host_ptr, size_t bytes);
 
 // Looks up, for the current device, the address of the device array behind zk_fr_sum_static (fr_kernels.hip); called
