@@ -30,7 +30,7 @@ static inline Fr load_fr(const uint32_t* p) { Fr r; memcpy(&r, p, 32); return r;
 template <int K> __device__ __forceinline__ void block_reduce_store(Fr (&acc)[K], Fr* __restrict__ partials) {
     __shared__ uint32_t red[8][TPB];
     const uint32_t t = threadIdx.x;
-#pragma unroll 1
+#pragma unroll
     for (int k = 0; k < K; ++k) {
 #pragma unroll
         for (int l = 0; l < 8; ++l) red[l][t] = acc[k].v[l];
@@ -447,7 +447,9 @@ template <int K> __global__ void __launch_bounds__(TPB) k_me_multi(Fr* __restric
 // does not match its hinted entry (a hint outside the table, inconsistent inputs) is inverted on its own.
 // S_out != nullptr: the queries themselves are not stored; query i is hint[i] + r * S_out[i] (a mapping table's combined
 // query, r_mont = r in Montgomery form) and is formed where it is needed.
-struct HintSrc { const Fr* T; const Fr* B; const Fr* hint; Fr low; Fr beta; uint32_t N; const Fr* S_out = nullptr; Fr r_mont; };
+// TB: table entry j and its inverse side by side, TB[2j] = T[j], TB[2j+1] = 1 / (T[j] + beta): the comparison and the
+// inverse of one query come out of one 64-byte line (two gathers into separate arrays fetched two).
+struct HintSrc { const Fr* TB; const Fr* hint; Fr low; Fr beta; uint32_t N; const Fr* S_out = nullptr; Fr r_mont; };
 __device__ __forceinline__ Fr hinted_query(const Fr* __restrict__ S, size_t i, const HintSrc& h) {
     return h.S_out ? add(h.hint[i], mont_mul(h.r_mont, h.S_out[i])) : S[i];
 }
@@ -466,13 +468,17 @@ __device__ __forceinline__ Fr inv_by_hint(const Fr& sv, size_t i, const HintSrc&
     const Fr d = sub(h.hint[i], h.low);
     const bool in_table = !(d.v[1] | d.v[2] | d.v[3] | d.v[4] | d.v[5] | d.v[6] | d.v[7]) && d.v[0] < h.N;
     const uint32_t j = in_table ? d.v[0] : 0u;
-    if (equal(sv, h.T[j])) {
-        const Fr b = h.B[j];
+    if (equal(sv, h.TB[2 * (size_t)j])) {
+        const Fr b = h.TB[2 * (size_t)j + 1];
         if (unit) *unit = !is_zero(b);
         return b;
     }
     if (unit) *unit = false;
     return inv_plus_beta_alone(sv, h.beta);
+}
+__global__ void __launch_bounds__(TPB) k_interleave(Fr* __restrict__ out, const Fr* __restrict__ a, const Fr* __restrict__ b, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) { out[2 * i] = a[i]; out[2 * i + 1] = b[i]; }
 }
 __global__ void __launch_bounds__(TPB) k_inv_by_hint(Fr* __restrict__ A, const Fr* __restrict__ S, const HintSrc h, size_t D) {
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
@@ -1445,7 +1451,10 @@ static int lookup_prove_begin(void** handle, const void* S, const void* T, const
     const Fr* Aptr = nullptr;
     HintSrc hs;
     if (rc == 0 && hint) {
-        hs.T = (const Fr*)T; hs.B = B.as<Fr>(); hs.hint = (const Fr*)hint; hs.low = fr_from_i64((int64_t)low); hs.beta = b; hs.N = (uint32_t)N;
+        Scratch& TB = job->arena.add(sizeof(Fr) * 2 * N);
+        if (TB.rc) { rc = TB.rc; sumjob_abort(job); return rc; }
+        hipLaunchKernelGGL(k_interleave, dim3(cdiv(N, TPB)), dim3(TPB), 0, st, TB.as<Fr>(), (const Fr*)T, B.as<Fr>(), N);
+        hs.TB = TB.as<Fr>(); hs.hint = (const Fr*)hint; hs.low = fr_from_i64((int64_t)low); hs.beta = b; hs.N = (uint32_t)N;
         if (S_out) { hs.S_out = (const Fr*)S_out; hs.r_mont = to_mont(load_fr(r)); }
     } else if (rc == 0) {
         Scratch& A = job->arena.add(sizeof(Fr) * D);
