@@ -163,6 +163,14 @@ int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* sc
  * delivers, and releases the opening's buffers; every handle must be ended exactly once. */
 int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stream);
 int zk_g1_open_end(void* handle, uint32_t* proof_host, uint32_t* final_scalar_host);
+/* The generators of me_open (commitment.cu:109-129 takes the Commitment itself) in the form the rounds work on, made once
+ * for any number of openings against them: affine points in 29-bit limbs and the first round's pair sums (1.5 n points
+ * of 112 bytes; nothing in it depends on the opened tensor).  zk_g1_open_begin_prepared is zk_g1_open_begin with
+ * such generators; the handle must outlive every opening started with it and is released with
+ * zk_g1_open_prepared_free. */
+int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stream);
+int zk_g1_open_prepared_free(void* prepared);
+int zk_g1_open_begin_prepared(void** handle, const void* scalars, const void* prepared, const uint32_t* u, int rounds, void* stream);
 
 /* ---- lookup argument (tlookup.cu) ------------------------------------------------------------------------ */
 /* idx = val - low as a table index (lookuprange_tensor_prep_kernel :414-421 / lookuprange_prep_kernel :393-400);

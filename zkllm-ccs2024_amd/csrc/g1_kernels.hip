@@ -290,6 +290,7 @@ static constexpr int MHEAVY = 256;   // a bucket above this many elements of a c
 struct MsmDesc { const int8_t* digits; uint32_t dstride, count, s_mul, s_off, b_mul, b_off, slot; };   // element i: recoded scalar i*s_mul+s_off of dstride, base A[i*b_mul+b_off]
 template <int NMAX> struct MsmDescs { MsmDesc d[NMAX]; };
 static constexpr int TAIL_N = 8192;        // generators at which the remaining rounds are computed in one batch
+static int tail_n_env() { static int v = [] { const char* e = getenv("ZKLLM_TAIL_N"); return e ? atoi(e) : TAIL_N; }(); return v; }
 static constexpr int TAIL_LEVELS = 20;     // most rounds the batch takes
 static constexpr int TAIL_SUMS = 3 * TAIL_LEVELS + 1;
 struct TailU { Fr u[TAIL_LEVELS]; };       // challenges of the batched rounds, Montgomery form
@@ -326,50 +327,6 @@ __device__ __forceinline__ Fp glv_minus2_over_beta_minus_1() {   // -2 / (beta -
 }
 // joint sparse form of (k1, k2): position i holds (d1 + 1) | (d2 + 1) << 2 in 4 bits, d in {-1, 0, 1}; len <= 129
 struct JsfK { uint32_t dig[17]; uint32_t len; };
-// 1 / v for every lane of a 64-lane workgroup with one field inversion: product tree up, inverse down (a child's
-// inverse is the parent's inverse times its sibling).  v must be non-zero (lanes with nothing to invert pass one).
-// lds: 12 x 128 words.
-__device__ __forceinline__ Fp block_inv64(const Fp& v, uint32_t (*lds)[2 * GT]) {
-    const uint32_t t = threadIdx.x;
-    auto put = [&](const Fp& x, uint32_t i) {
-#pragma unroll
-        for (int l = 0; l < 12; ++l) lds[l][i] = x.v[l];
-    };
-    auto get = [&](uint32_t i) {
-        Fp x;
-#pragma unroll
-        for (int l = 0; l < 12; ++l) x.v[l] = lds[l][i];
-        return x;
-    };
-    __syncthreads();
-    put(v, t);
-    __syncthreads();
-    uint32_t off = 0;
-    for (uint32_t cnt = GT / 2; cnt >= 1; cnt >>= 1) {
-        const uint32_t noff = off + 2 * cnt;
-        if (t < cnt) put(fp_mul(get(off + 2 * t), get(off + 2 * t + 1)), noff + t);
-        __syncthreads();
-        off = noff;
-    }
-    {
-        const Fp root_inv = mont_inverse(get(off));      // every lane the same value: no divergence
-        __syncthreads();
-        if (t == 0) put(root_inv, off);
-        __syncthreads();
-    }
-    for (uint32_t cnt = 1; cnt < (uint32_t)GT; cnt <<= 1) {
-        const uint32_t coff = off - 2 * cnt;
-        Fp c = big_one_mont<12>();
-        if (t < 2 * cnt) c = fp_mul(get(off + (t >> 1)), get(coff + (t ^ 1u)));
-        __syncthreads();
-        if (t < 2 * cnt) put(c, coff + t);
-        __syncthreads();
-        off = coff;
-    }
-    const Fp r = get(t);
-    __syncthreads();
-    return r;
-}
 // [k1]P + [k2]phi(P); every lane of a wave must carry the same k (the add pattern is uniform)
 static __device__ __attribute__((noinline)) G1Jac g1_mul_glv(const G1Jac& P, const GlvK& k) {
     if (is_zero(P.z)) return P;
@@ -703,66 +660,107 @@ __global__ void __launch_bounds__(GT) k_open_chain(G1Jac* __restrict__ pts, cons
         pts[3 * r] = tot;
     }
 }
-// The fold itself: pair g -> new scalar and new generator.
-__global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2))) k_open_fold(Fr* __restrict__ new_scalars, G1Jac* __restrict__ new_gens, const Fr* __restrict__ scalars, const G1Affine* __restrict__ A,
-                                                  const Fr u_mont, const GlvK ku, const JsfK jsf, size_t old_size, size_t new_size) {
-    // ---- pair g: s' and g' = a1 + [u](a0 - a1) -------------------------------------------------------------------------------
-    // The scalar multiplication works on affine points throughout its table: D = a0 - a1 (one inversion, batched over
-    // the 64 lanes), phi(D) = (beta x, y), D + phi(D) = (beta^2 x, -y) (the three images of the endomorphism sum to zero) and
-    // D - phi(D) (a second batched inversion).  With the joint sparse form of (k1, k2) -- digits in {-1, 0, 1}, a non-zero
-    // pair in about half of the 129 positions -- the walk is one doubling per position and one mixed addition per
-    // non-zero pair.  Lanes whose inputs are special (infinity, equal abscissae, x = 0) take the general Jacobian route.
-    // one wave per workgroup: the batched inversions are over before the table is written, and LDS serves a wave in order
+// ---- the fold on 29-bit-limb affine points ----------------------------------------------------------------------------------
+// The rounds of an opening keep the generators in ONE form: affine, 29-bit limbs (A29; all-zero limbs = infinity), canonical
+// limbs.  The bucket sums add out of it, the fold reads it and writes the next round's generators in it -- no
+// normalisation or conversion pass between two rounds.
+// 1 / v for every lane of a 64-lane workgroup with one field inversion (product tree in LDS; the root goes through the
+// 32-bit form, where the binary inverse lives).  v must not be 0 mod p (lanes with nothing to invert pass one).
+// lds: 14 x 128 words.
+__device__ __forceinline__ Fq29 block_inv64_29(const Fq29& v, int32_t (*lds)[2 * GT]) {
+    const uint32_t t = threadIdx.x;
+    auto put = [&](const Fq29& x, uint32_t i) {
+#pragma unroll
+        for (int l = 0; l < 14; ++l) lds[l][i] = x.l[l];
+    };
+    auto get = [&](uint32_t i) {
+        Fq29 x;
+#pragma unroll
+        for (int l = 0; l < 14; ++l) x.l[l] = lds[l][i];
+        return x;
+    };
+    __syncthreads();
+    put(v, t);
+    __syncthreads();
+    uint32_t off = 0;
+    for (uint32_t cnt = GT / 2; cnt >= 1; cnt >>= 1) {
+        const uint32_t noff = off + 2 * cnt;
+        if (t < cnt) put(fq29_mul(get(off + 2 * t), get(off + 2 * t + 1)), noff + t);
+        __syncthreads();
+        off = noff;
+    }
+    {
+        const Fq29 root_inv = fq29_from_fp(mont_inverse(fq29_to_fp(get(off))));      // every lane the same value: no divergence
+        __syncthreads();
+        if (t == 0) put(root_inv, off);
+        __syncthreads();
+    }
+    for (uint32_t cnt = 1; cnt < (uint32_t)GT; cnt <<= 1) {
+        const uint32_t coff = off - 2 * cnt;
+        Fq29 c = fq29_one();
+        if (t < 2 * cnt) c = fq29_mul(get(off + (t >> 1)), get(coff + (t ^ 1u)));
+        __syncthreads();
+        if (t < 2 * cnt) put(c, coff + t);
+        __syncthreads();
+        off = coff;
+    }
+    const Fq29 r = get(t);
+    __syncthreads();
+    return r;
+}
+// Pair g of the round: s' and g' = a1 + [u](a0 - a1), all in 29-bit limbs.  The scalar multiplication walks the joint
+// sparse form of the split challenge over the all-affine table {D, phi(D), D + phi(D), D - phi(D)}, D = a0 - a1, and the
+// result is brought back to affine form in the kernel (a third inversion batched over the 64 lanes).  Pairs whose inputs
+// are special (a0 at infinity, equal abscissae, an abscissa of zero) are not computed here: their indices go to
+// `special` ([0] = count, then the indices) and k_open_fold_special takes them.
+__global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+k_open_fold29(Fr* __restrict__ new_scalars, A29* __restrict__ new_gens, const Fr* __restrict__ scalars, const A29* __restrict__ A, const Fr u_mont, const JsfK jsf,
+              size_t old_size, size_t new_size, uint32_t* __restrict__ special) {
     __shared__ int32_t fold_lds[4 * 14 * GT];
-    static_assert(4 * 14 * GT >= 12 * 2 * GT, "the inversion buffer shares the table's space");
-    uint32_t (*inv_lds)[2 * GT] = reinterpret_cast<uint32_t (*)[2 * GT]>(fold_lds);
+    static_assert(4 * 14 * GT >= 14 * 2 * GT, "the inversion buffer shares the table's space");
+    int32_t (*inv_lds)[2 * GT] = reinterpret_cast<int32_t (*)[2 * GT]>(fold_lds);
     int32_t (*tab)[14][GT] = reinterpret_cast<int32_t (*)[14][GT]>(fold_lds);
     const size_t g = (size_t)blockIdx.x * GT + threadIdx.x;
     const bool live = g < new_size;
     const size_t g0 = 2 * g, g1 = 2 * g + 1;
     const bool has1 = live && g1 < old_size;
-    G1Affine a0, a1;
-    a0.x = a0.y = a1.x = a1.y = big_zero<12>();
+    A29 a0, a1;
+    a0.x = a0.y = a1.x = a1.y = fq29_zero();
     if (live) a0 = A[g0];
     if (has1) a1 = A[g1];
     if (live) {
         if (has1) new_scalars[g] = add(scalars[g0], mont_mul(u_mont, sub(scalars[g1], scalars[g0])));
         else new_scalars[g] = sub(scalars[g0], mont_mul(u_mont, scalars[g0]));
     }
-    const bool inf0 = aff_is_inf(a0), inf1 = !has1 || aff_is_inf(a1);
-    const Fp one_m = big_one_mont<12>();
-    // general = the old route; fast = everything regular
-    bool general = live && (inf0 || (!inf1 && equal(a0.x, a1.x)));
-    const bool need_sub = live && !general && !inf1;          // D = a0 - a1 needs 1 / (x0 - x1)
-    Fp den = need_sub ? sub(a0.x, a1.x) : one_m;
-    Fp inv = block_inv64(den, inv_lds);
-    G1Affine D = a0;
-    if (need_sub) {
-        const Fp lam = fp_mul(add(a0.y, a1.y), inv);          // -a1 = (x1, -y1)
-        D.x = sub(sub(fp_sqr(lam), a0.x), a1.x);
-        D.y = sub(fp_mul(lam, sub(a0.x, D.x)), a0.y);
+    const bool inf0 = a29_is_inf(a0), inf1 = !has1 || a29_is_inf(a1);
+    const Fq29 one29 = fq29_one();
+    bool general = live && inf0;
+    Fq29 den = one29;
+    if (live && !general && !inf1) {
+        den = fq29_sub(a0.x, a1.x);
+        if (fq29_is_zero_mod_p(den)) { general = true; den = one29; }
     }
-    if (live && !general && is_zero(D.x)) general = true;       // x = 0: not in the subgroup; the table below would divide by it
+    const bool need_sub = live && !general && !inf1;          // D = a0 - a1 needs 1 / (x0 - x1)
+    Fq29 inv = block_inv64_29(den, inv_lds);
+    Fq29 xD = a0.x, yD = a0.y;
+    if (need_sub) {
+        const Fq29 lam = fq29_mul(fq29_add(a0.y, a1.y), inv);          // -a1 = (x1, -y1)
+        const Fq29 x3 = fq29_sub(fq29_sub(fq29_sqr(lam), a0.x), a1.x);
+        yD = fq29_mul(fq29_sub(fq29_mul(lam, fq29_sub(a0.x, x3)), a0.y), one29);      // the products by one bring the sums back into (-eps, p + eps)
+        xD = fq29_mul(x3, one29);
+    }
+    if (live && !general && fq29_is_zero_mod_p(xD)) general = true;       // x = 0: not in the subgroup; the table below would divide by it
     const bool fast = live && !general;
-    den = fast ? D.x : one_m;
-    inv = block_inv64(den, inv_lds);
-    G1Jac r = g1_infinity();
+    inv = block_inv64_29(fast ? xD : one29, inv_lds);
+    J29 w = j29_infinity();
     if (fast) {
-        const Fp beta = glv_beta(), beta2 = glv_beta2();
-        G1Affine Q, PQ, PmQ;
-        Q.x = fp_mul(D.x, beta); Q.y = D.y;
-        PQ.x = fp_mul(D.x, beta2); PQ.y = neg(D.y);
         {
-            const Fp lam = fp_mul(fp_mul(glv_minus2_over_beta_minus_1(), D.y), inv);   // slope of D + (beta x, -y)
-            PmQ.x = add(fp_sqr(lam), PQ.x);
-            PmQ.y = sub(fp_mul(lam, sub(D.x, PmQ.x)), D.y);
-        }
-        // the walk itself in 29-bit limbs: the four table points differ in four abscissae and two ordinates.  D stays in
-        // registers; the other three abscissae and the second ordinate wait in LDS (word-interleaved over the lanes) and
-        // negations are formed when a point is taken: the walk then fits 256 registers without spilling.
-        const Fq29 xD = fq29_from_fp(D.x), yD = fq29_from_fp(D.y);
-        {
-            const Fq29 xQ = fq29_from_fp(Q.x), xPQ = fq29_from_fp(PQ.x), xPmQ = fq29_from_fp(PmQ.x), yPmQ = fq29_from_fp(PmQ.y);
+            const Fq29 xQ = fq29_mul(xD, fq29_from_fp(glv_beta())), xPQ = fq29_mul(xD, fq29_from_fp(glv_beta2()));
+            const Fq29 lam = fq29_mul(fq29_mul(fq29_from_fp(glv_minus2_over_beta_minus_1()), yD), inv);   // slope of D + (beta x, -y)
+            const Fq29 xPmQ = fq29_mul(fq29_add(fq29_sqr(lam), xPQ), one29);
+            const Fq29 yPmQ = fq29_mul(fq29_sub(fq29_mul(lam, fq29_sub(xD, xPmQ)), yD), one29);
+            // D stays in registers; the other three abscissae and the second ordinate wait in LDS (word-interleaved over the
+            // lanes) and negations are formed when a point is taken: the walk then fits 256 registers without spilling.
 #pragma unroll
             for (int l = 0; l < 14; ++l) {
                 tab[0][l][threadIdx.x] = xQ.l[l];
@@ -771,7 +769,6 @@ __global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 tab[3][l][threadIdx.x] = yPmQ.l[l];
             }
         }
-        J29 w = j29_infinity();
         for (int i = (int)jsf.len - 1; i >= 0; --i) {
             w = j29_double(w);
             const uint32_t dg = (jsf.dig[i >> 3] >> ((i & 7) * 4)) & 0xFu;    // (d1 + 1) | (d2 + 1) << 2, the same for every lane
@@ -796,15 +793,85 @@ __global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2)))
             if (negate) t.y = fq29_neg(t.y);
             w = j29_add_mixed(w, t);
         }
-        if (!inf1) w = j29_add_mixed(w, a29_from_affine(a1));
-        r = j29_to_jac(w);
+        if (!inf1) w = j29_add_mixed(w, a1);
+    }
+    // back to affine: 1 / z batched over the lanes (the table in LDS is no longer needed)
+    const bool has_z = fast && !w.inf;
+    const Fq29 zi = block_inv64_29(has_z ? w.z : one29, inv_lds);
+    if (fast) {
+        A29 o;
+        o.x = o.y = fq29_zero();
+        if (has_z) {
+            const Fq29 zi2 = fq29_sqr(zi);
+            o.x = fq29_canon(fq29_mul(w.x, zi2));
+            o.y = fq29_canon(fq29_mul(fq29_mul(w.y, zi2), zi));
+        }
+        new_gens[g] = o;
     } else if (general) {
+        const uint32_t slot = atomicAdd(&special[0], 1u);
+        special[1 + slot] = (uint32_t)g;
+    }
+}
+// the pairs k_open_fold29 left out, by the general Jacobian route in 32-bit limbs (one lane per pair, an inversion each)
+__device__ __forceinline__ G1Affine a29_to_affine(const A29& p) {
+    G1Affine r;
+    r.x = fq29_to_fp(p.x); r.y = fq29_to_fp(p.y);
+    return r;
+}
+__global__ void __launch_bounds__(GT) k_open_fold_special(A29* __restrict__ new_gens, const A29* __restrict__ A, const GlvK ku, size_t old_size, const uint32_t* __restrict__ special) {
+    const uint32_t count = special[0];
+    for (uint32_t i = blockIdx.x * GT + threadIdx.x; i < count; i += gridDim.x * GT) {
+        const size_t g = special[1 + i];
+        const G1Affine a0 = a29_to_affine(A[2 * g]);
+        const bool has1 = 2 * g + 1 < old_size;
+        G1Affine a1;
+        a1.x = a1.y = big_zero<12>();
+        if (has1) a1 = a29_to_affine(A[2 * g + 1]);
+        const bool inf1 = !has1 || aff_is_inf(a1);
         G1Jac diff = aff_to_jac(a0);
         if (!inf1) diff = g1_add_mixed(diff, g1_neg(a1));
-        r = g1_mul_glv(diff, ku);
+        G1Jac r = g1_mul_glv(diff, ku);
         if (!inf1) r = g1_add_mixed(r, a1);
+        A29 o;
+        o.x = o.y = fq29_zero();
+        if (!is_zero(r.z)) {
+            const Fp zi = mont_inverse(r.z), zi2 = fp_sqr(zi);
+            G1Affine af;
+            af.x = fp_mul(r.x, zi2);
+            af.y = fp_mul(fp_mul(r.y, zi2), zi);
+            o = a29_from_affine(af);
+            o.x = fq29_canon(o.x); o.y = fq29_canon(o.y);
+        }
+        new_gens[g] = o;
     }
-    if (live) new_gens[g] = r;
+}
+// generator pairs' sums g_2i + g_2i+1 (an odd last element alone) for T of the first round; and the pairs' scalar sums
+__global__ void __launch_bounds__(GT) k_open_pair_points(G1Jac* __restrict__ pj, const G1Affine* __restrict__ A, size_t old_size, size_t half_up) {
+    const size_t i = (size_t)blockIdx.x * GT + threadIdx.x;
+    if (i >= half_up) return;
+    G1Jac p = aff_to_jac(A[2 * i]);
+    if (2 * i + 1 < old_size) {
+        const G1Affine b = A[2 * i + 1];
+        if (!aff_is_inf(b)) p = g1_add_mixed(p, b);
+    }
+    pj[i] = p;
+}
+__global__ void __launch_bounds__(256) k_open_pair_scalars(Fr* __restrict__ ps, const Fr* __restrict__ scalars, size_t old_size, size_t half_up) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= half_up) return;
+    ps[i] = (2 * i + 1 < old_size) ? add(scalars[2 * i], scalars[2 * i + 1]) : scalars[2 * i];
+}
+__global__ void __launch_bounds__(GT) k_a29_to_jac(G1Jac* __restrict__ out, const A29* __restrict__ in, size_t n) {
+    const size_t i = (size_t)blockIdx.x * GT + threadIdx.x;
+    if (i >= n) return;
+    out[i] = a29_is_inf(in[i]) ? g1_infinity() : aff_to_jac(a29_to_affine(in[i]));
+}
+__global__ void __launch_bounds__(256) k_a29_canon(A29* __restrict__ a, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    A29 v = a[i];
+    v.x = fq29_canon(v.x); v.y = fq29_canon(v.y);
+    a[i] = v;
 }
 // ---- the last rounds in one batch ---------------------------------------------------------------------------------------
 // Once n0 <= TAIL_N generators are left, every later round's generators are fixed linear combinations of these n0
@@ -866,9 +933,12 @@ __global__ void __launch_bounds__(GT) k_msm_horner(G1Jac* __restrict__ pts, cons
     pts[descs.d[blockIdx.x].slot] = r;
 }
 
+__global__ void __launch_bounds__(64) k_u32_zero(uint32_t* __restrict__ p, uint32_t n) {
+    for (uint32_t i = threadIdx.x; i < n; i += 64) p[i] = 0u;
+}
 // after the last round of an opening without a batched tail: the folded generator is the last proof point
-__global__ void __launch_bounds__(GT) k_open_finish(G1Jac* __restrict__ pts, const G1Jac* __restrict__ last_gen, uint32_t rounds) {
-    if (blockIdx.x == 0 && threadIdx.x == 0) pts[3 * rounds] = last_gen[0];
+__global__ void __launch_bounds__(GT) k_open_finish(G1Jac* __restrict__ pts, const A29* __restrict__ last_gen, uint32_t rounds) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) pts[3 * rounds] = a29_is_inf(last_gen[0]) ? g1_infinity() : aff_to_jac(a29_to_affine(last_gen[0]));
 }
 
 // ---- host side ----------------------------------------------------------------------------------------------------------
@@ -959,41 +1029,42 @@ static JsfK jsf_of(const GlvK& k) {
     return out;
 }
 
-// Queues one round: the fold on st, the bucket sums on aux.  wsum_round: the round's 3 x MW window sums (T, T0, T1); with_T
-// false leaves the first MW alone (T of that round then comes from k_open_chain).
+// The generators of an opening in the form its rounds work on: A29 points, and behind them the pair sums
+// g_2i + g_2i+1 that T of the first round is summed over (n + ceil(n/2) points in one array).  Nothing in it depends on
+// what is opened, so a caller that opens against the same generators again keeps it (zk_g1_open_prepare).
+static int open_prep_build(A29* out, const G1Jac* gens, size_t n, Arena& arena, hipStream_t st) {
+    const size_t half_up = (n + 1) / 2;
+    Scratch& aff = arena.add(sizeof(G1Affine) * n);
+    Scratch& pj = arena.add(sizeof(G1Jac) * half_up);
+    Scratch& paff = arena.add(sizeof(G1Affine) * half_up);
+    if (aff.rc || pj.rc || paff.rc) return aff.rc ? aff.rc : (pj.rc ? pj.rc : paff.rc);
+    hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(n, CH), GT)), dim3(GT), 0, st, aff.p, gens, n);
+    hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(n, 256)), dim3(256), 0, st, out, aff.as<G1Affine>(), n);
+    hipLaunchKernelGGL(k_open_pair_points, dim3(cdiv(half_up, GT)), dim3(GT), 0, st, pj.as<G1Jac>(), aff.as<G1Affine>(), n, half_up);
+    hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(half_up, CH), GT)), dim3(GT), 0, st, paff.p, pj.as<G1Jac>(), half_up);
+    hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(half_up, 256)), dim3(256), 0, st, out + n, paff.as<G1Affine>(), half_up);
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
+
+// Queues one round: the scalars' digits and the fold on st, the bucket sums on aux.  gens: the round's generators (A29);
+// with_T (the first round): the pair sums follow them at gens + old_size.  wsum_round: the round's 3 x MW window sums
+// (T, T0, T1); without with_T the first MW are left alone (T of that round then comes from k_open_chain).
 // Round 0 needs T = sum_j s_j g_j over all generators besides T0 and T1.  With the pairs' sums,
 //   sum_i (s_2i + s_2i+1)(g_2i + g_2i+1) = T + T0 + T1,
 // so T costs a bucket sum over half as many points: pair i gets the scalar s_2i + s_2i+1 (mod r: the generators have
 // order r) and the point g_2i + g_2i+1; an odd last element stands alone.  k_open_t_fix takes T0 and T1 off again,
 // window by window.
-__global__ void __launch_bounds__(GT) k_open_pairs(Fr* __restrict__ ps, G1Jac* __restrict__ pj, const Fr* __restrict__ scalars, const G1Affine* __restrict__ A,
-                                                   size_t old_size, size_t half_up) {
-    const size_t i = (size_t)blockIdx.x * GT + threadIdx.x;
-    if (i >= half_up) return;
-    const bool has1 = 2 * i + 1 < old_size;
-    ps[i] = has1 ? add(scalars[2 * i], scalars[2 * i + 1]) : scalars[2 * i];
-    G1Jac p = aff_to_jac(A[2 * i]);
-    if (has1) {
-        const G1Affine b = A[2 * i + 1];
-        if (!aff_is_inf(b)) p = g1_add_mixed(p, b);
-    }
-    pj[i] = p;
-}
 __global__ void __launch_bounds__(64) k_open_t_fix(G1Jac* __restrict__ wsum) {
     const uint32_t w = threadIdx.x;
     if (w >= (uint32_t)MW) return;
     wsum[w] = g1_add(g1_add(wsum[w], g1_neg(wsum[MW + w])), g1_neg(wsum[2 * MW + w]));
 }
-
-static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars, const G1Jac* gens, const Fr& u, size_t old_size, bool with_T,
+static int open_round_launch(Fr* new_scalars, A29* new_gens, const Fr* scalars, const A29* gens, const Fr& u, size_t old_size, bool with_T,
                              G1Jac* wsum_round, Arena& arena, hipStream_t st, hipStream_t aux, std::vector<hipEvent_t>& events) {
     ZK_ARG(old_size < (1ull << 31), "opening: more than 2^31 generators");
     const size_t new_size = (old_size + 1) / 2;
     const bool chained = !with_T;
-    // ---- both chains start from the affine generators and the recoded scalars ----
-    Scratch& aff = arena.add(sizeof(G1Affine) * old_size);
-    if (aff.rc) return aff.rc;
-    hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(old_size, CH), GT)), dim3(GT), 0, st, aff.p, gens, old_size);
     Scratch& dig = arena.add((size_t)(MW + 1) * old_size);
     if (dig.rc) return dig.rc;
     hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(old_size, 256)), dim3(256), 0, st, dig.as<int8_t>(), scalars, old_size);
@@ -1005,7 +1076,7 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
         ZK_HIP(hipEventRecord(ready, st));
         ZK_HIP(hipStreamWaitEvent(aux, ready, 0));
     }
-    // ---- side chain (aux): bucket sums, window sums, the round's single points; nothing here feeds the next fold ----
+    // ---- side chain (aux): bucket sums, window sums; nothing here feeds the next fold ----
     MsmDescs<3> descs;
     const uint32_t half = (uint32_t)(old_size / 2);
     const uint32_t half_up = (uint32_t)new_size;
@@ -1013,20 +1084,12 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     uint32_t q = 0;
     const int8_t* dg = dig.as<int8_t>();
     const uint32_t ds = (uint32_t)old_size;
-    Scratch& aff29 = arena.add(sizeof(A29) * (old_size + (chained ? 0 : half_up)));
-    if (aff29.rc) return aff29.rc;
-    hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(old_size, 256)), dim3(256), 0, aux, aff29.as<A29>(), aff.as<G1Affine>(), old_size);
     if (!chained) {
-        // T of round 0 through the pairs' sums: half_up points appended to the table, their scalars recoded apart
         Scratch& ps = arena.add(sizeof(Fr) * half_up);
-        Scratch& pj = arena.add(sizeof(G1Jac) * half_up);
-        Scratch& paff = arena.add(sizeof(G1Affine) * half_up);
         Scratch& dig2 = arena.add((size_t)(MW + 1) * half_up);
-        if (ps.rc || pj.rc || paff.rc || dig2.rc) return ps.rc ? ps.rc : (pj.rc ? pj.rc : (paff.rc ? paff.rc : dig2.rc));
-        hipLaunchKernelGGL(k_open_pairs, dim3(cdiv(half_up, GT)), dim3(GT), 0, aux, ps.as<Fr>(), pj.as<G1Jac>(), scalars, aff.as<G1Affine>(), old_size, (size_t)half_up);
-        hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(half_up, CH), GT)), dim3(GT), 0, aux, paff.p, pj.as<G1Jac>(), (size_t)half_up);
+        if (ps.rc || dig2.rc) return ps.rc ? ps.rc : dig2.rc;
+        hipLaunchKernelGGL(k_open_pair_scalars, dim3(cdiv(half_up, 256)), dim3(256), 0, aux, ps.as<Fr>(), scalars, old_size, (size_t)half_up);
         hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(half_up, 256)), dim3(256), 0, aux, dig2.as<int8_t>(), ps.as<Fr>(), (size_t)half_up);
-        hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(half_up, 256)), dim3(256), 0, aux, aff29.as<A29>() + old_size, paff.as<G1Affine>(), (size_t)half_up);
         descs.d[q++] = MsmDesc{dig2.as<int8_t>(), half_up, half_up, 1u, 0u, 1u, (uint32_t)old_size, 0u};
     }
     descs.d[q++] = MsmDesc{dg, ds, half, 2u, 0u, 2u, 1u, 1u};
@@ -1042,7 +1105,7 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (size_t)nseg * MT);
     if (partial.rc) return partial.rc;
     G1Jac* wsum = wsum_round + (size_t)(3 - n_msm) * MW;
-    hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MSL), 0, aux, partial.as<G1Jac>(), aff29.as<A29>(), descs, nseg, cps);
+    hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MSL), 0, aux, partial.as<G1Jac>(), gens, descs, nseg, cps);
     {
         // sum the segments' raw buckets eight at a time, then weight and total
         const G1Jac* cur = partial.as<G1Jac>();
@@ -1062,26 +1125,30 @@ static int open_round_launch(Fr* new_scalars, G1Jac* new_gens, const Fr* scalars
     // ---- critical chain (st): the fold ----
     const GlvK ku = glv_split(u);
     const JsfK jsf = jsf_of(ku);
+    Scratch& special = arena.add(sizeof(uint32_t) * (1 + new_size));
+    if (special.rc) return special.rc;
+    hipLaunchKernelGGL(k_u32_zero, dim3(1), dim3(64), 0, st, special.as<uint32_t>(), 1u);
     hipEvent_t t0 = nullptr, t1 = nullptr;
     if (g_fold_timer.on) {
         ZK_HIP(hipEventCreate(&t0));
         ZK_HIP(hipEventCreate(&t1));
         ZK_HIP(hipEventRecord(t0, st));
     }
-    hipLaunchKernelGGL(k_open_fold, dim3(cdiv(new_size, GT)), dim3(GT), 0, st, new_scalars, new_gens, scalars, aff.as<G1Affine>(), to_mont(u), ku, jsf, old_size, new_size);
+    hipLaunchKernelGGL(k_open_fold29, dim3(cdiv(new_size, GT)), dim3(GT), 0, st, new_scalars, new_gens, scalars, gens, to_mont(u), jsf, old_size, new_size, special.as<uint32_t>());
     if (g_fold_timer.on) {
         ZK_HIP(hipEventRecord(t1, st));
         g_fold_timer.ev.emplace_back(t0, t1);
         g_fold_timer.fp_mults += fold_fp_mults_per_pair(jsf) * (double)new_size;
         g_fold_timer.pairs += new_size;
     }
+    hipLaunchKernelGGL(k_open_fold_special, dim3(16), dim3(GT), 0, st, new_gens, gens, ku, old_size, special.as<uint32_t>());
     ZK_LAUNCH_CHECK();
     return 0;
 }
 
 // Queues the batch for the last `levels` rounds (rounds r0 .. r0+levels-1 of `rounds`) over n0 <= TAIL_N generators.
 // Writes T, T0, T1 of those rounds and the final generator into pts; *final_scalar points at the folded scalar.
-static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, const uint32_t* u, int levels, int r0, int rounds, G1Jac* pts, const Fr** final_scalar,
+static int open_tail_launch(const Fr* scalars, const A29* gens, size_t n0, const uint32_t* u, int levels, int r0, int rounds, G1Jac* pts, const Fr** final_scalar,
                             Arena& arena, hipStream_t st) {
     TailU us;
     for (int j = 0; j < levels; ++j) us.u[j] = to_mont(load_fr(u + 8 * j));
@@ -1089,18 +1156,13 @@ static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, con
     Scratch& sl = arena.add(sizeof(Fr) * (n0 + (size_t)levels + 1));
     const int n_msm = 3 * levels + 1;
     const uint32_t nseg = cdiv(n0, MSEG), cps = 1;       // one chunk per workgroup, as in the halving rounds
-    Scratch& aff = arena.add(sizeof(G1Affine) * n0);
-    Scratch& aff29 = arena.add(sizeof(A29) * n0);
     Scratch& coef = arena.add(sizeof(Fr) * (size_t)n_msm * n0);
     Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (size_t)nseg * MT);
     Scratch& wsum = arena.add(sizeof(G1Jac) * n_msm * MW);
     if (sl.rc) return sl.rc;
-    if (aff.rc) return aff.rc;
-    if (aff29.rc) return aff29.rc;
     if (coef.rc) return coef.rc;
     if (partial.rc) return partial.rc;
     if (wsum.rc) return wsum.rc;
-    hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(n0, CH), GT)), dim3(GT), 0, st, aff.p, gens, n0);
     hipLaunchKernelGGL(k_tail_scalars, dim3(1), dim3(1024), 0, st, sl.as<Fr>(), scalars, us, (uint32_t)n0, (uint32_t)levels);
     hipLaunchKernelGGL(k_tail_coeffs, dim3(cdiv(n0, 256)), dim3(256), 0, st, coef.as<Fr>(), sl.as<Fr>(), scalars, us, (uint32_t)n0, (uint32_t)levels);
     const size_t ncoef = (size_t)n_msm * n0;
@@ -1113,8 +1175,7 @@ static int open_tail_launch(const Fr* scalars, const G1Jac* gens, size_t n0, con
         const uint32_t slot = !live ? 0u : (i == 3 * levels ? 3u * (uint32_t)rounds : 3u * (uint32_t)r0 + (uint32_t)i);
         descs.d[i] = MsmDesc{dig.as<int8_t>(), (uint32_t)ncoef, live ? (uint32_t)n0 : 0u, 1u, live ? (uint32_t)((size_t)i * n0) : 0u, 1u, 0u, slot};
     }
-    hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(n0, 256)), dim3(256), 0, st, aff29.as<A29>(), aff.as<G1Affine>(), n0);
-    hipLaunchKernelGGL(k_msm_seg<TAIL_SUMS>, dim3(nseg, MW, n_msm), dim3(MSL), 0, st, partial.as<G1Jac>(), aff29.as<A29>(), descs, nseg, cps);
+    hipLaunchKernelGGL(k_msm_seg<TAIL_SUMS>, dim3(nseg, MW, n_msm), dim3(MSL), 0, st, partial.as<G1Jac>(), gens, descs, nseg, cps);
     hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), nseg);
     hipLaunchKernelGGL(k_msm_horner, dim3(n_msm), dim3(GT), 0, st, pts, wsum.as<G1Jac>(), descs);
     ZK_LAUNCH_CHECK();
@@ -1319,15 +1380,22 @@ int zk_g1_fixed_base_mul(void* out, const uint32_t* base_host, const void* scala
 int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host, const void* scalars, const void* gens, const uint32_t* u, size_t old_size, void* stv) {
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(old_size >= 1, "zk_g1_open_round: empty input");
+    const size_t new_size = (old_size + 1) / 2;
     Scratch pts(sizeof(G1Jac) * 3, st);
     if (pts.rc) return pts.rc;
     Scratch wsum(sizeof(G1Jac) * 3 * MW, st);
     if (wsum.rc) return wsum.rc;
     Arena arena(st);
+    Scratch& g29 = arena.add(sizeof(A29) * (old_size + new_size));
+    Scratch& n29 = arena.add(sizeof(A29) * new_size);
+    if (g29.rc || n29.rc) return g29.rc ? g29.rc : n29.rc;
+    int rc = open_prep_build(g29.as<A29>(), (const G1Jac*)gens, old_size, arena, st);
+    if (rc) return rc;
     std::vector<hipEvent_t> evs;
-    int rc = open_round_launch((Fr*)new_scalars, (G1Jac*)new_gens, (const Fr*)scalars, (const G1Jac*)gens, load_fr(u), old_size, true, wsum.as<G1Jac>(), arena, st, st, evs);
+    rc = open_round_launch((Fr*)new_scalars, n29.as<A29>(), (const Fr*)scalars, g29.as<A29>(), load_fr(u), old_size, true, wsum.as<G1Jac>(), arena, st, st, evs);
     (void)evs;
     if (rc) return rc;
+    hipLaunchKernelGGL(k_a29_to_jac, dim3(cdiv(new_size, GT)), dim3(GT), 0, st, (G1Jac*)new_gens, n29.as<A29>(), new_size);
     hipLaunchKernelGGL(k_open_horner, dim3(3), dim3(GT), 0, st, pts.as<G1Jac>(), wsum.as<G1Jac>(), 1u);
     hipLaunchKernelGGL(k_g1_normalize<false>, dim3(1), dim3(GT), 0, st, pts.p, pts.as<G1Jac>(), (size_t)3);
     ZK_LAUNCH_CHECK();
@@ -1353,7 +1421,8 @@ struct OpenJob {
     hipStream_t aux = nullptr;     // second stream of the job (bucket sums beside the folds); equals st when the job has one stream
     std::vector<hipEvent_t> events;
 };
-static int open_queue(OpenJob& job, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, hipStream_t st, hipStream_t aux) {
+// gens: Jacobian generators, or null when `prep` (their prepared form, open_prep_build) is given
+static int open_queue(OpenJob& job, const void* scalars, const void* gens, const A29* prep, size_t n, const uint32_t* u, int rounds, hipStream_t st, hipStream_t aux) {
     ZK_ARG(n >= 1, "zk_g1_open: empty input");
     ZK_ARG(rounds >= 0 && rounds <= 64, "zk_g1_open: bad round count");
     ZK_ARG(sizeof(G1Jac) * (3 * (size_t)rounds + 1) + sizeof(Fr) <= 65536, "zk_g1_open: proof larger than the staging buffer");
@@ -1368,14 +1437,21 @@ static int open_queue(OpenJob& job, const void* scalars, const void* gens, size_
     if (wsum.rc) return wsum.rc;
     job.pts = pts.as<G1Jac>();
     const Fr* cs = (const Fr*)scalars;
-    const G1Jac* cg = (const G1Jac*)gens;
+    const A29* cg = prep;
+    if (!cg) {
+        Scratch& g29 = job.arena.add(sizeof(A29) * (n + (n + 1) / 2));
+        if (g29.rc) return g29.rc;
+        int rc = open_prep_build(g29.as<A29>(), (const G1Jac*)gens, n, job.arena, st);
+        if (rc) return rc;
+        cg = g29.as<A29>();
+    }
     size_t size = n;
     int halving_rounds = rounds;
     bool tail_done = false;
     OpenUs us;
     memset(&us, 0, sizeof(us));
     for (int r = 0; r < rounds; ++r) {
-        if (size <= (size_t)TAIL_N && rounds - r <= TAIL_LEVELS) {
+        if (size <= (size_t)tail_n_env() && rounds - r <= TAIL_LEVELS) {
             int rc = open_tail_launch(cs, cg, size, u + 8 * r, rounds - r, r, rounds, pts.as<G1Jac>(), &cs, job.arena, st);
             if (rc) return rc;
             halving_rounds = r;
@@ -1384,15 +1460,15 @@ static int open_queue(OpenJob& job, const void* scalars, const void* gens, size_
         }
         const size_t ns = (size + 1) / 2;
         Scratch& s2 = job.arena.add(sizeof(Fr) * ns);
-        Scratch& g2 = job.arena.add(sizeof(G1Jac) * ns);
+        Scratch& g2 = job.arena.add(sizeof(A29) * ns);
         if (s2.rc) return s2.rc;
         if (g2.rc) return g2.rc;
         const Fr ur = load_fr(u + 8 * r);
         us.u[r] = to_mont(ur);
-        int rc = open_round_launch(s2.as<Fr>(), g2.as<G1Jac>(), cs, cg, ur, size, r == 0, wsum.as<G1Jac>() + (size_t)3 * MW * r, job.arena, st, aux, job.events);
+        int rc = open_round_launch(s2.as<Fr>(), g2.as<A29>(), cs, cg, ur, size, r == 0, wsum.as<G1Jac>() + (size_t)3 * MW * r, job.arena, st, aux, job.events);
         if (rc) return rc;
         cs = s2.as<Fr>();
-        cg = g2.as<G1Jac>();
+        cg = g2.as<A29>();
         size = ns;
     }
     // the single points of the halving rounds, behind the last bucket sums
@@ -1431,14 +1507,14 @@ static int open_collect(OpenJob& job, uint32_t* proof_host, uint32_t* final_scal
 // z = 1 (infinity: all-zero limbs).  final_scalar_host: the folded scalar.
 int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stv) {
     OpenJob job;
-    int rc = open_queue(job, scalars, gens, n, u, rounds, (hipStream_t)stv, (hipStream_t)stv);
+    int rc = open_queue(job, scalars, gens, nullptr, n, u, rounds, (hipStream_t)stv, (hipStream_t)stv);
     if (rc) { (void)hipStreamSynchronize((hipStream_t)stv); return rc; }
     return open_collect(job, proof_host, final_scalar_host);
 }
 // The same in two halves.  begin queues the recursion on a stream of the library's own, ordered after everything queued
 // on `stream` so far, and returns at once; the caller goes on using `stream`, and both run side by side.  scalars and gens
 // must stay alive and unmodified until end, which waits for the opening, delivers its results and releases its buffers.
-int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stv) {
+static int open_begin_impl(void** handle, const void* scalars, const void* gens, const A29* prep, size_t n, const uint32_t* u, int rounds, void* stv) {
     ZK_ARG(handle != nullptr, "zk_g1_open_begin: null handle");
     hipStream_t side = side_stream(0), aux = side_stream(0);      // consecutive streams of the pool: the folds on one, the bucket sums on the other
     ZK_ARG(side != nullptr && aux != nullptr, "zk_g1_open_begin: could not create a stream");
@@ -1446,7 +1522,7 @@ int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_
     ZK_HIP(hipEventCreateWithFlags(&job->ready, hipEventDisableTiming));
     ZK_HIP(hipEventRecord(job->ready, (hipStream_t)stv));
     ZK_HIP(hipStreamWaitEvent(side, job->ready, 0));
-    int rc = open_queue(*job, scalars, gens, n, u, rounds, side, aux);
+    int rc = open_queue(*job, scalars, gens, prep, n, u, rounds, side, aux);
     if (rc) {
         (void)hipStreamSynchronize(side);
         (void)hipStreamSynchronize(aux);
@@ -1456,6 +1532,42 @@ int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_
     }
     *handle = job.release();
     return 0;
+}
+int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stv) {
+    return open_begin_impl(handle, scalars, gens, nullptr, n, u, rounds, stv);
+}
+// Generators prepared once for any number of openings against them: their affine 29-bit-limb form and the pair sums of
+// the first round (weight-independent; 1.5 n points of 112 bytes).  The handle is freed with zk_g1_open_prepared_free
+// once no opening that uses it is pending.
+struct OpenPrepared { void* a29 = nullptr; size_t n = 0; };
+int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(prepared != nullptr && n >= 1, "zk_g1_open_prepare: null handle or no generators");
+    std::unique_ptr<OpenPrepared> pr(new OpenPrepared);
+    int rc = pool_alloc(&pr->a29, sizeof(A29) * (n + (n + 1) / 2), st);
+    if (rc) return rc;
+    pr->n = n;
+    {
+        Arena arena(st);
+        rc = open_prep_build((A29*)pr->a29, (const G1Jac*)gens, n, arena, st);
+    }
+    // openings read it on the library's own streams: it must be complete before the handle is used
+    if (rc == 0 && hipStreamSynchronize(st) != hipSuccess) rc = hip_fail(hipGetLastError(), "zk_g1_open_prepare sync", __FILE__, __LINE__);
+    if (rc) { (void)hipStreamSynchronize(st); pool_free(pr->a29, st, true); return rc; }
+    *prepared = pr.release();
+    return 0;
+}
+int zk_g1_open_prepared_free(void* prepared) {
+    if (!prepared) return 0;
+    OpenPrepared* pr = (OpenPrepared*)prepared;
+    int rc = pool_free(pr->a29, nullptr);
+    delete pr;
+    return rc;
+}
+int zk_g1_open_begin_prepared(void** handle, const void* scalars, const void* prepared, const uint32_t* u, int rounds, void* stv) {
+    ZK_ARG(prepared != nullptr, "zk_g1_open_begin_prepared: null generators");
+    const OpenPrepared* pr = (const OpenPrepared*)prepared;
+    return open_begin_impl(handle, scalars, nullptr, (const A29*)pr->a29, pr->n, u, rounds, stv);
 }
 int zk_g1_open_end(void* handle, uint32_t* proof_host, uint32_t* final_scalar_host) {
     ZK_ARG(handle != nullptr, "zk_g1_open_end: null handle");

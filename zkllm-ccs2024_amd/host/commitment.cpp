@@ -76,22 +76,36 @@ Fr_t Commitment::open(const FrTensor& t, const G1TensorJacobian& com, const vect
     }
     return me_open(folded, *this, u_in.begin(), u_in.end(), proof);
 }
-Commitment::Pending Commitment::open_begin(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u) const {
+Commitment::Pending Commitment::open_fold(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u) const {
     const uint k_out = ceilLog2(com.size);
     if (u.size() < k_out) throw std::runtime_error("Commitment::open - too few challenges");
     const vector<Fr_t> u_out(u.end() - k_out, u.end());
-    const vector<Fr_t> u_in(u.begin(), u.end() - k_out);
     Pending p;
+    p.u_in.assign(u.begin(), u.end() - k_out);
     p.folded.reset(new FrTensor(u_out.empty() ? FrTensor(t) : t.partial_me(u_out, t.size / com.size)));
     if (p.folded->size != size) throw std::runtime_error("Commitment::me_open - Incompatible dimensions " + std::to_string(p.folded->size) + " " + std::to_string(size));
+    return p;
+}
+void Commitment::open_start(Pending& p) const {
     if (g_skip_g1) {
-        p.value = (*p.folded)(u_in);
-        return p;
+        p.value = (*p.folded)(p.u_in);
+        return;
     }
-    p.rounds = (int)u_in.size();
+    p.rounds = (int)p.u_in.size();
     std::vector<uint32_t> uu((size_t)p.rounds * 8 + 8);
-    for (int r = 0; r < p.rounds; ++r) memcpy(&uu[(size_t)r * 8], u_in[r].val, 32);
-    ZKC(zk_g1_open_begin(&p.handle, p.folded->gpu_data, gpu_data, size, uu.data(), p.rounds, nullptr));
+    for (int r = 0; r < p.rounds; ++r) memcpy(&uu[(size_t)r * 8], p.u_in[r].val, 32);
+    if (prepared) ZKC(zk_g1_open_begin_prepared(&p.handle, p.folded->gpu_data, prepared.get(), uu.data(), p.rounds, nullptr));
+    else ZKC(zk_g1_open_begin(&p.handle, p.folded->gpu_data, gpu_data, size, uu.data(), p.rounds, nullptr));
+}
+void Commitment::prepare_openings() const {
+    if (prepared || size == 0) return;
+    void* h = nullptr;
+    ZKC(zk_g1_open_prepare(&h, gpu_data, size, nullptr));
+    prepared = std::shared_ptr<void>(h, [](void* q) { (void)zk_g1_open_prepared_free(q); });
+}
+Commitment::Pending Commitment::open_begin(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u) const {
+    Pending p = open_fold(t, com, u);
+    open_start(p);
     return p;
 }
 Fr_t Commitment::open_end(Pending& p, vector<G1Jacobian_t>& proof) {
@@ -114,6 +128,7 @@ Weight create_weight(string generator_filename, string weight_filename, string c
     Commitment generator(generator_filename);
     FrTensor weight = FrTensor::from_int_bin(weight_filename);
     G1TensorJacobian com(com_filename);
+    generator.prepare_openings();
     Weight w{generator, weight, com, in_dim, out_dim, nullptr};
     if (in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim))) w.padded = std::make_shared<const FrTensor>(w.weight.pad({in_dim, out_dim}));
     return w;

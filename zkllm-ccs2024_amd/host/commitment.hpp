@@ -15,6 +15,11 @@ class Commitment : public G1TensorJacobian {
     using G1TensorJacobian::operator*;
     using G1TensorJacobian::operator*=;
 
+   private:
+    mutable std::shared_ptr<void> prepared;      // zk_g1_open_prepare handle
+
+   public:
+
     G1TensorJacobian commit(const FrTensor& t) const;
     G1TensorJacobian commit_int(const FrTensor& t) const;
     G1TensorJacobian commit_int_multi(const vector<FrTensor>& t) const;
@@ -30,14 +35,27 @@ class Commitment : public G1TensorJacobian {
         std::unique_ptr<FrTensor> folded;   // the scalars the queued kernels read
         int rounds = 0;
         Fr_t value{{0, 0, 0, 0, 0, 0, 0, 0}};
+        vector<Fr_t> u_in;                  // between open_fold and open_start: the challenges of the G1 recursion
     };
     Pending open_begin(const FrTensor& t, const G1TensorJacobian& c, const vector<Fr_t>& u) const;
+    // open_begin in its two steps: open_fold reduces the rows to the vector that is opened (a pass over the whole tensor
+    // on the caller's stream), open_start queues the G1 recursion.  Several openings started together fold first and
+    // start afterwards: a fold queued behind another opening's G1 kernels waits for the registers they hold.
+    Pending open_fold(const FrTensor& t, const G1TensorJacobian& c, const vector<Fr_t>& u) const;
+    void open_start(Pending& p) const;
     static Fr_t open_end(Pending& p, vector<G1Jacobian_t>& proof);
+
+    // The generators' form for openings (zk_g1_open_prepare), made once and kept with this object: openings started
+    // afterwards skip the normalisation and conversion of the generators.  Anything that changes the points must not
+    // be applied afterwards (the prepared form would no longer match); copies share it.
+    void prepare_openings() const;
+    bool openings_prepared() const { return (bool)prepared; }
 
     static Commitment random(uint size);
     static Fr_t me_open(const FrTensor& t, const Commitment& generators, vector<Fr_t>::const_iterator begin, vector<Fr_t>::const_iterator end, vector<G1Jacobian_t>& proof);
 };
 
+// (Commitment's prepared form is a shared handle: see prepare_openings)
 struct Weight {
     Commitment generator;
     FrTensor weight;

@@ -348,9 +348,8 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
     if (c.open_weights) {
         // behind the forward pass (the openings are ordered after what is queued here): started before it, their kernels keep
         // the forward pass's matrix products waiting for most of their own duration
-        ou = openWeightAhead(up, ch_u.u_input, ch_u.u_output);      // the two large ones first
-        og = openWeightAhead(gate, ch_g.u_input, ch_g.u_output);
-        od = openWeightAhead(down, ch_d.u_input, ch_d.u_output);
+        auto ahead = openWeightsAhead({&up, &gate, &down}, {&ch_u.u_input, &ch_g.u_input, &ch_d.u_input}, {&ch_u.u_output, &ch_g.u_output, &ch_d.u_output});   // the two large ones first
+        ou = std::move(ahead[0]); og = std::move(ahead[1]); od = std::move(ahead[2]);
     }
 
     {
@@ -416,6 +415,7 @@ static Weight random_weight(std::mt19937_64& rng, uint in_dim, uint out_dim, uin
     const bool ragged = in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim));
     std::shared_ptr<const FrTensor> padded = ragged ? std::make_shared<const FrTensor>(weight.pad({in_dim, out_dim})) : nullptr;
     G1TensorJacobian com = gen.commit_int(ragged ? *padded : weight);
+    gen.prepare_openings();
     return Weight{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim, std::move(padded)};
 }
 

@@ -87,6 +87,19 @@ WeightOpeningAhead openWeightAhead(const Weight& w, const vector<Fr_t>& u_input,
     a.impl->op = w.generator.open_begin(padded_form(w, local), w.com, a.impl->u_cat);
     return a;
 }
+std::vector<WeightOpeningAhead> openWeightsAhead(const std::vector<const Weight*>& ws, const std::vector<const std::vector<Fr_t>*>& u_inputs,
+                                                 const std::vector<const std::vector<Fr_t>*>& u_outputs) {
+    std::vector<WeightOpeningAhead> out(ws.size());
+    if (!g_deferred) return out;
+    for (size_t i = 0; i < ws.size(); ++i) {
+        out[i].impl = new WeightOpeningAhead::Impl;
+        out[i].impl->u_cat = concatenate(vector<vector<Fr_t>>({*u_outputs[i], *u_inputs[i]}));
+        std::unique_ptr<FrTensor> local;
+        out[i].impl->op = ws[i]->generator.open_fold(padded_form(*ws[i], local), ws[i]->com, out[i].impl->u_cat);
+    }
+    for (size_t i = 0; i < ws.size(); ++i) ws[i]->generator.open_start(out[i].impl->op);
+    return out;
+}
 void verifyWeightClaim(const Weight& w, const Claim& c, WeightOpeningAhead& ahead) {
     if (!ahead.impl || !g_deferred) { verifyWeightClaim(w, c); return; }
     if (ahead.impl->u_cat != concatenate(vector<vector<Fr_t>>({c.u[1], c.u[0]}))) throw std::runtime_error("verifyWeightClaim: the opening started ahead is at another point");

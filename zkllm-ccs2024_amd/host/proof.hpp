@@ -27,6 +27,9 @@ struct WeightOpeningAhead {
     Impl* impl;
 };
 WeightOpeningAhead openWeightAhead(const Weight& w, const std::vector<Fr_t>& u_input, const std::vector<Fr_t>& u_output);
+// several at once: every weight's rows are folded first, then the G1 recursions are queued (Commitment::open_fold / open_start)
+std::vector<WeightOpeningAhead> openWeightsAhead(const std::vector<const Weight*>& ws, const std::vector<const std::vector<Fr_t>*>& u_inputs,
+                                                 const std::vector<const std::vector<Fr_t>*>& u_outputs);
 void verifyWeightClaim(const Weight& w, const Claim& c, WeightOpeningAhead& ahead);
 // While a DeferredOpenings object is alive, verifyWeightClaim only starts each opening (it runs on the device beside
 // the rest of the proof) and finish() waits for all of them, checks every claim and throws as verifyWeightClaim does.
