@@ -171,6 +171,12 @@ int zk_g1_open_end(void* handle, uint32_t* proof_host, uint32_t* final_scalar_ho
 int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stream);
 int zk_g1_open_prepared_free(void* prepared);
 int zk_g1_open_begin_prepared(void** handle, const void* scalars, const void* prepared, const uint32_t* u, int rounds, void* stream);
+/* `count` (1..8) openings against prepared generator sets of ONE size with ONE round count as a single job: every kernel
+ * of a halving round is launched once for all of them (the reference opens weight after weight, proof.cu:9-15; openings
+ * are independent of each other).  scalars[i] / prepared[i]: opening i; u: its challenges at u + i * rounds * 8.  end
+ * delivers opening i's points at proof_host + i * (3 rounds + 1) * 36 and its folded scalar at final_scalar_host + i * 8. */
+int zk_g1_open_begin_batch(void** handle, int count, const void* const* scalars, const void* const* prepared, const uint32_t* u, int rounds, void* stream);
+int zk_g1_open_end_batch(void* handle, uint32_t* proof_host, uint32_t* final_scalar_host);
 
 /* ---- lookup argument (tlookup.cu) ------------------------------------------------------------------------ */
 /* idx = val - low as a table index (lookuprange_tensor_prep_kernel :414-421 / lookuprange_prep_kernel :393-400);

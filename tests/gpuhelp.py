@@ -456,6 +456,14 @@ class Prover:
             self.lib.zkp_transcript_get(_np_ptr(out))
         return out
 
+    def transcript_g1(self):
+        self.lib.zkp_transcript_g1_size.restype = ctypes.c_long
+        n = self.lib.zkp_transcript_g1_size()
+        out = np.zeros((n, 36), dtype=np.uint32)
+        if n:
+            self.lib.zkp_transcript_g1_get(_np_ptr(out))
+        return out
+
     def sync(self):
         self.check(self.lib.zkp_sync())
 

@@ -275,6 +275,61 @@ def test_open_begin_end_matches_open_through_the_c_abi(orc):
         hip.free(dS)
 
 
+def test_open_batch_over_prepared_generators_matches_single_openings(orc):
+    """zk_g1_open_begin_batch (openings of one size as ONE job: every round's kernels launched once for all of them) over
+    generators prepared with zk_g1_open_prepare delivers, opening by opening, the bytes of zk_g1_open.  Sizes on both
+    sides of the batched last rounds, a ragged one (odd halves), special generators (equal, opposite, infinite) in one
+    member of the batch, and zk_g1_open_begin_prepared alone."""
+    import ctypes
+    from gpuhelp import Hip, c_void_p, c_size_t, c_int
+    hip = Hip()
+    for n, count in ((9001, 3), (600, 2), (4096, 8)):
+        k = (n - 1).bit_length()
+        npts = 3 * k + 1
+        gens, dG, dS, us, preps = [], [], [], [], []
+        exp_p = np.zeros((count, npts, 36), np.uint32)
+        exp_v = np.zeros((count, 8), np.uint32)
+        for i in range(count):
+            g = oracle_gens(orc, 300 + 7 * i + n, n)
+            if i == 1 and n > 20:
+                neg = np.zeros((1, 36), np.uint32)
+                g[1] = g[0]
+                orc_check(orc.orc_g1_op(4, g[2:3].copy(), g[2:3].copy(), neg, 1))
+                g[3] = neg[0]
+                g[6] = 0
+                g[7] = 0
+                g[9] = 0
+            S = mt_random_vec(np.random.RandomState(50 + i), n)
+            u = mt_random_vec(np.random.RandomState(70 + i), k)
+            gens.append(g); us.append(u)
+            dG.append(hip.upload(g)); dS.append(hip.upload(S))
+            hip.call("zk_g1_open", exp_p[i], exp_v[i], c_void_p(dS[i]), c_void_p(dG[i]), c_size_t(n), u, c_int(k), None)
+            pr = c_void_p()
+            hip.call("zk_g1_open_prepare", ctypes.byref(pr), c_void_p(dG[i]), c_size_t(n), None)
+            preps.append(pr)
+        h = c_void_p()
+        sc = (c_void_p * count)(*[c_void_p(x) for x in dS])
+        pp = (c_void_p * count)(*preps)
+        uall = np.ascontiguousarray(np.concatenate(us), dtype=np.uint32)
+        hip.call("zk_g1_open_begin_batch", ctypes.byref(h), c_int(count), sc, pp, uall, c_int(k), None)
+        got_p = np.zeros_like(exp_p)
+        got_v = np.zeros_like(exp_v)
+        hip.call("zk_g1_open_end_batch", h, got_p, got_v)
+        assert (got_v == exp_v).all(), n
+        assert (got_p == exp_p).all(), n
+        # one prepared opening on its own
+        h1 = c_void_p()
+        hip.call("zk_g1_open_begin_prepared", ctypes.byref(h1), c_void_p(dS[0]), preps[0], us[0], c_int(k), None)
+        p1 = np.zeros((npts, 36), np.uint32)
+        v1 = np.zeros(8, np.uint32)
+        hip.call("zk_g1_open_end", h1, p1, v1)
+        assert (v1 == exp_v[0]).all() and (p1 == exp_p[0]).all(), n
+        for pr in preps:
+            hip.call("zk_g1_open_prepared_free", pr)
+        for x in dG + dS:
+            hip.free(x)
+
+
 def test_fixed_base_multiplication_equals_the_generic_one_and_big_integer_arithmetic(orc):
     """zk_g1_fixed_base_mul (what Commitment::random runs on) against zk_g1_scalar_mul on the same base and, for the
     small cases, against affine big-integer arithmetic: digits at the signed-window boundaries (127, 128, 129, bytes of

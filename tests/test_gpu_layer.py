@@ -1,6 +1,8 @@
 """GPU parity for a whole decoder layer (RMSNorm, QKV, per-head attention with zkSoftmax, output projection,
 skip, RMSNorm, SwiGLU FFN, skip; every rescaling, lookup, sumcheck and weight opening): outputs and the full proof
 transcript under a seeded challenge stream are bit-exact against the CPU oracle at small shapes."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -38,6 +40,51 @@ def test_tiny_layer_transcript(pv, open_weights, seed, head_group):
     assert (out.host() == exp).all()
     assert got_t.shape == exp_t.shape and (got_t == exp_t).all()
     assert times[6] > 0
+
+
+def test_layer_run_again_starts_its_openings_ahead_and_proves_the_same(pv):
+    """The first run over a set of weights learns where the nine opening points sit in the challenge stream; a second run
+    starts every opening when the layer starts (batched by generator size) and must deliver the transcript of the first,
+    field elements and G1 points alike, which is the oracle's.  A run under another seed (other challenges at the same
+    positions) and one with the weight openings switched off and on again go through the same plan."""
+    orc = load_oracle()
+    cu, cf = layercfg.tiny(open_weights=True, head_group=2)
+    ws = layercfg.tiny_weights(21, cu)
+    S, E = int(cu[0]), int(cu[1])
+    X = np.round(np.random.default_rng(31).normal(0, 1, (S, E)) * 256).astype(np.int32)
+    layer = None
+    for run, seed in enumerate((8, 8, 9, 8)):
+        exp = np.zeros((S * E, 8), np.uint32)
+        orc.orc_seed(seed)
+        orc.orc_transcript_clear()
+        orc_check(orc.orc_layer(cu, cf, *ws, 1, X, exp, None))
+        exp_t = orc_transcript(orc)
+        pv.seed(seed)
+        if layer is None:
+            layer = pv.layer_create(cu, cf, ws, 1)      # draws the generators from the stream seeded just above, as the oracle does
+        else:
+            # the generators were made at the first creation; skip the same draws
+            pv.lib.zkp_challenge_skip.argtypes = [ctypes.c_ulonglong]
+            pv.lib.zkp_challenge_skip(ctypes.c_ulonglong(layer_draws))
+        if run == 0:
+            pv.lib.zkp_challenge_position.restype = ctypes.c_ulonglong
+            layer_draws = pv.lib.zkp_challenge_position()
+        assert pv.lib.zkp_layer_planned_openings(ctypes.c_void_p(layer)) == (0 if run == 0 else 9)
+        pv.transcript_begin()
+        out, _ = pv.layer_run(layer, pv.from_i32(X))
+        pv.lib.zkp_transcript_end()
+        got_t = pv.transcript()
+        if seed == 8:
+            assert (out.host() == exp).all(), run
+            assert got_t.shape == exp_t.shape and (got_t == exp_t).all(), run
+            g1 = pv.transcript_g1()
+            if run == 0:
+                first_g1 = g1
+            else:
+                assert g1.shape == first_g1.shape and (g1 == first_g1).all(), run
+        else:
+            assert got_t.shape == exp_t.shape, run
+    pv.layer_free(layer)
 
 
 def test_full_shape_layer_gives_one_output_head_by_head_and_stacked(pv):

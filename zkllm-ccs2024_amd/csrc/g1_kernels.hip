@@ -287,13 +287,13 @@ static constexpr int MT = 128;       // lanes of a bucket workgroup = buckets (d
 static constexpr int MSEG = 4096;    // elements per chunk (12-bit list entries)
 static constexpr int MSL = 64;       // lanes of a bucket-accumulation workgroup (one wave): each takes two buckets of its chunk
 static constexpr int MHEAVY = 256;   // a bucket above this many elements of a chunk is summed by the whole workgroup
-struct MsmDesc { const int8_t* digits; uint32_t dstride, count, s_mul, s_off, b_mul, b_off, slot; };   // element i: recoded scalar i*s_mul+s_off of dstride, base A[i*b_mul+b_off]
+struct MsmDesc { const int8_t* digits; const A29* base; uint32_t dstride, count, s_mul, s_off, b_mul, b_off, slot; };   // element i: recoded scalar i*s_mul+s_off of dstride, point base[i*b_mul+b_off]
+static constexpr int OB_MAX = 8;           // openings of equal size that share their rounds' launches
+static constexpr int OB_SUMS = 3 * OB_MAX;
 template <int NMAX> struct MsmDescs { MsmDesc d[NMAX]; };
-static constexpr int TAIL_N = 8192;        // generators at which the remaining rounds are computed in one batch
-static int tail_n_env() { static int v = [] { const char* e = getenv("ZKLLM_TAIL_N"); return e ? atoi(e) : TAIL_N; }(); return v; }
+static constexpr int TAIL_N = 2048;        // generators at which the remaining rounds are computed in one batch (work grows with it, latency shrinks)
 static constexpr int TAIL_LEVELS = 20;     // most rounds the batch takes
 static constexpr int TAIL_SUMS = 3 * TAIL_LEVELS + 1;
-struct TailU { Fr u[TAIL_LEVELS]; };       // challenges of the batched rounds, Montgomery form
 struct GlvK { uint32_t k1[4], k2[4]; };
 
 __device__ __forceinline__ bool aff_is_inf(const G1Affine& p) { return is_zero(p.x) && is_zero(p.y); }   // normalised infinity: all-zero limbs
@@ -354,9 +354,12 @@ static __device__ __attribute__((noinline)) G1Jac g1_mul_glv(const G1Jac& P, con
 // smaller of s and r - s gives small negative values (r - x, as weights are embedded) as few non-zero windows as
 // small positive ones, instead of r's high bytes in every one of them.  A window byte above 127 becomes byte - 256
 // and carries one into the next window; the top window of a value below 2^254 cannot overflow.
-__global__ void __launch_bounds__(256) k_msm_recode(int8_t* __restrict__ D, const Fr* __restrict__ S, size_t n) {
+struct RecodeBatch { int8_t* D[OB_MAX]; const Fr* S[OB_MAX]; };      // blockIdx.y names the pair
+__global__ void __launch_bounds__(256) k_msm_recode(const RecodeBatch rb, size_t n) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
+    int8_t* __restrict__ D = rb.D[blockIdx.y];
+    const Fr* __restrict__ S = rb.S[blockIdx.y];
     const Fr sv = S[i];
     Fr ng;
     uint32_t br = 0;
@@ -422,18 +425,19 @@ template <int NT = MT> __device__ __forceinline__ G1Jac msm_block_sum(uint32_t* 
 //  3. a bucket with more than MHEAVY elements (scalars that share a digit: equal values, a common high byte) is left out
 //     of the lists and summed by all lanes together, each over its own share of the chunk.
 template <int NMAX>
-__global__ void __launch_bounds__(MSL) __attribute__((amdgpu_waves_per_eu(2, 2))) k_msm_seg(G1Jac* __restrict__ partial, const A29* __restrict__ A, const MsmDescs<NMAX> descs, uint32_t nseg, uint32_t chunks_per_seg) {
+__global__ void __launch_bounds__(MSL) __attribute__((amdgpu_waves_per_eu(2, 2))) k_msm_seg(G1Jac* __restrict__ partial, const MsmDescs<NMAX> descs, const MsmDesc* __restrict__ ddescs, uint32_t nseg, uint32_t chunks_per_seg) {
     __shared__ uint32_t cnt[MT], off[MT], cursor[MT];
     __shared__ uint8_t order[MT];
     __shared__ uint32_t pool[36 * MSL];            // the sorted list (u16 x MSEG), then the 36 x MSL point tree of the heavy buckets
     static_assert(36 * MSL * 4 >= MSEG * 2, "pool too small for the list");
     static_assert(MSEG <= 4096, "12-bit list entries");
     uint16_t* list = reinterpret_cast<uint16_t*>(pool);
-    const MsmDesc d = descs.d[blockIdx.z];
-    const uint32_t w = blockIdx.y, seg = blockIdx.x, t = threadIdx.x;
+    const MsmDesc d = ddescs ? ddescs[blockIdx.z] : descs.d[blockIdx.z];      // many sums: the descriptors lie in device memory
+    const A29* __restrict__ A = d.base;
+    const uint32_t w = blockIdx.y, seg = blockIdx.x, t = threadIdx.x, zz = blockIdx.z;
     const int8_t* __restrict__ Dw = d.digits + (size_t)w * d.dstride;
     const int8_t* __restrict__ Df = d.digits + (size_t)MW * d.dstride;
-    G1Jac* __restrict__ out = partial + (((size_t)blockIdx.z * MW + w) * nseg + seg) * MT;
+    G1Jac* __restrict__ out = partial + (((size_t)zz * MW + w) * nseg + seg) * MT;
     bool first = true;                                  // nothing written to `out` yet (the same for every lane)
     for (uint32_t ch = 0; ch < chunks_per_seg; ++ch) {
         const uint32_t e0 = (seg * chunks_per_seg + ch) * MSEG;
@@ -537,7 +541,9 @@ __global__ void __launch_bounds__(MT) k_msm_bucket_fold(G1Jac* __restrict__ out,
 }
 // wsum[(sum * MW + w)] from the raw buckets of nseg segments: lane t adds up bucket t+1 over the segments, weights it,
 // and the lanes are summed.  One workgroup per (sum, window).
-__global__ void __launch_bounds__(MT) k_msm_buckets(G1Jac* __restrict__ wsum, const G1Jac* __restrict__ buckets, uint32_t nseg) {
+// Row z * MW + w (sum z, window w) goes to wsum[(z / n_per) * item_stride + (z % n_per) * MW + w]: the sums of one opening lie
+// together, the openings of a batch item_stride apart (one opening: n_per = all sums, stride 0).
+__global__ void __launch_bounds__(MT) k_msm_buckets(G1Jac* __restrict__ wsum, const G1Jac* __restrict__ buckets, uint32_t nseg, uint32_t n_per, uint32_t item_stride) {
     __shared__ uint32_t pool[36 * MT];
     const uint32_t t = threadIdx.x;
     const G1Jac* b = buckets + (size_t)blockIdx.x * nseg * MT;
@@ -549,7 +555,10 @@ __global__ void __launch_bounds__(MT) k_msm_buckets(G1Jac* __restrict__ wsum, co
         if (((t + 1) >> bit) & 1u) r = g1_add(r, acc);
     }
     const G1Jac tot = msm_block_sum(pool, r, t);
-    if (t == 0) wsum[blockIdx.x] = tot;
+    if (t == 0) {
+        const uint32_t z = blockIdx.x / MW, w = blockIdx.x % MW;
+        wsum[(size_t)(z / n_per) * item_stride + (size_t)(z % n_per) * MW + w] = tot;
+    }
 }
 
 // ---- the single points of the halving rounds, once per opening ---------------------------------------------------------
@@ -560,9 +569,11 @@ __global__ void __launch_bounds__(MT) k_msm_buckets(G1Jac* __restrict__ wsum, co
 //                T_r = u(1-u) T_(r-1) + (1-u)^2 T0_(r-1) + u^2 T1_(r-1)   (u = the challenge of round r-1)
 //                down to round 0 makes T_r a combination of T_0 and the T0, T1 of the rounds before r with coefficients
 //                that are products of the challenges -- all rounds at once, one lane per term.
-struct OpenUs { Fr u[64]; };      // challenges of the halving rounds, Montgomery form
-__global__ void __launch_bounds__(GT) k_open_horner(G1Jac* __restrict__ pts, const G1Jac* __restrict__ Wall, uint32_t halving_rounds) {
+// blockIdx.y: the opening of a batch (its points npts apart, its window sums wstride apart)
+__global__ void __launch_bounds__(GT) k_open_horner(G1Jac* __restrict__ pts0, const G1Jac* __restrict__ Wall0, uint32_t halving_rounds, uint32_t npts, uint32_t wstride) {
     if (threadIdx.x != 0) return;
+    G1Jac* __restrict__ pts = pts0 + (size_t)blockIdx.y * npts;
+    const G1Jac* __restrict__ Wall = Wall0 + (size_t)blockIdx.y * wstride;
     const uint32_t x = blockIdx.x, round = x / 3, j = x % 3;
     if (round >= halving_rounds || (round > 0 && j == 0)) return;
     const G1Jac* W = Wall + (size_t)x * MW;
@@ -612,8 +623,11 @@ static __device__ __attribute__((noinline)) G1Jac g1_mul_glv_lane(const G1Jac& P
     return out;
 }
 // grid: halving_rounds - 1 workgroups; workgroup x computes T of round x + 1 into pts[3 * (x + 1)].  Needs T_0 and all T0, T1.
-__global__ void __launch_bounds__(GT) k_open_chain(G1Jac* __restrict__ pts, const OpenUs us, uint32_t halving_rounds) {
+// U: the openings' challenges in Montgomery form, opening y's at U + y * ustride
+__global__ void __launch_bounds__(GT) k_open_chain(G1Jac* __restrict__ pts0, const Fr* __restrict__ U, uint32_t halving_rounds, uint32_t npts, uint32_t ustride) {
     __shared__ uint32_t pool[36 * GT];
+    G1Jac* __restrict__ pts = pts0 + (size_t)blockIdx.y * npts;
+    const Fr* __restrict__ usu = U + (size_t)blockIdx.y * ustride;
     const uint32_t r = blockIdx.x + 1, t = threadIdx.x;
     const Fr one = big_one_mont<8>();
     G1Jac acc = g1_infinity();
@@ -622,9 +636,9 @@ __global__ void __launch_bounds__(GT) k_open_chain(G1Jac* __restrict__ pts, cons
             // term i: i == 0 -> T_0 with prod_{j<r} a_j;  i = 1 + 2k + s -> (s ? T1_k : T0_k) with (s ? u_k^2 : (1-u_k)^2) prod_{k<j<r} a_j,  a_j = u_j (1 - u_j)
             const uint32_t k = i == 0 ? 0u : (i - 1) / 2, s1 = i == 0 ? 0u : (i - 1) & 1u;
             Fr c = one;
-            for (uint32_t j = (i == 0 ? 0u : k + 1); j < r; ++j) c = mont_mul(c, mont_mul(us.u[j], sub(one, us.u[j])));
+            for (uint32_t j = (i == 0 ? 0u : k + 1); j < r; ++j) c = mont_mul(c, mont_mul(usu[j], sub(one, usu[j])));
             if (i != 0) {
-                const Fr f = s1 ? us.u[k] : sub(one, us.u[k]);
+                const Fr f = s1 ? usu[k] : sub(one, usu[k]);
                 c = mont_mul(c, mont_mul(f, f));
             }
             const G1Jac P = pts[i == 0 ? 0u : 3 * k + 1 + s1];
@@ -708,14 +722,22 @@ __device__ __forceinline__ Fq29 block_inv64_29(const Fq29& v, int32_t (*lds)[2 *
     __syncthreads();
     return r;
 }
+struct FoldItem { Fr* ns; A29* ng; const Fr* s; const A29* g; uint32_t* special; Fr u_mont; JsfK jsf; };
+struct FoldBatch { FoldItem it[OB_MAX]; };          // blockIdx.y names the opening; all of one size
 // Pair g of the round: s' and g' = a1 + [u](a0 - a1), all in 29-bit limbs.  The scalar multiplication walks the joint
 // sparse form of the split challenge over the all-affine table {D, phi(D), D + phi(D), D - phi(D)}, D = a0 - a1, and the
 // result is brought back to affine form in the kernel (a third inversion batched over the 64 lanes).  Pairs whose inputs
 // are special (a0 at infinity, equal abscissae, an abscissa of zero) are not computed here: their indices go to
 // `special` ([0] = count, then the indices) and k_open_fold_special takes them.
 __global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-k_open_fold29(Fr* __restrict__ new_scalars, A29* __restrict__ new_gens, const Fr* __restrict__ scalars, const A29* __restrict__ A, const Fr u_mont, const JsfK jsf,
-              size_t old_size, size_t new_size, uint32_t* __restrict__ special) {
+k_open_fold29(const FoldBatch fb, size_t old_size, size_t new_size) {
+    Fr* __restrict__ new_scalars = fb.it[blockIdx.y].ns;
+    A29* __restrict__ new_gens = fb.it[blockIdx.y].ng;
+    const Fr* __restrict__ scalars = fb.it[blockIdx.y].s;
+    const A29* __restrict__ A = fb.it[blockIdx.y].g;
+    uint32_t* __restrict__ special = fb.it[blockIdx.y].special;
+    const Fr u_mont = fb.it[blockIdx.y].u_mont;
+    const JsfK& jsf = fb.it[blockIdx.y].jsf;
     __shared__ int32_t fold_lds[4 * 14 * GT];
     static_assert(4 * 14 * GT >= 14 * 2 * GT, "the inversion buffer shares the table's space");
     int32_t (*inv_lds)[2 * GT] = reinterpret_cast<int32_t (*)[2 * GT]>(fold_lds);
@@ -818,7 +840,12 @@ __device__ __forceinline__ G1Affine a29_to_affine(const A29& p) {
     r.x = fq29_to_fp(p.x); r.y = fq29_to_fp(p.y);
     return r;
 }
-__global__ void __launch_bounds__(GT) k_open_fold_special(A29* __restrict__ new_gens, const A29* __restrict__ A, const GlvK ku, size_t old_size, const uint32_t* __restrict__ special) {
+struct SpecialBatch { A29* ng[OB_MAX]; const A29* g[OB_MAX]; const uint32_t* special[OB_MAX]; GlvK ku[OB_MAX]; };
+__global__ void __launch_bounds__(GT) k_open_fold_special(const SpecialBatch sb, size_t old_size) {
+    A29* __restrict__ new_gens = sb.ng[blockIdx.y];
+    const A29* __restrict__ A = sb.g[blockIdx.y];
+    const uint32_t* __restrict__ special = sb.special[blockIdx.y];
+    const GlvK ku = sb.ku[blockIdx.y];
     const uint32_t count = special[0];
     for (uint32_t i = blockIdx.x * GT + threadIdx.x; i < count; i += gridDim.x * GT) {
         const size_t g = special[1 + i];
@@ -856,9 +883,12 @@ __global__ void __launch_bounds__(GT) k_open_pair_points(G1Jac* __restrict__ pj,
     }
     pj[i] = p;
 }
-__global__ void __launch_bounds__(256) k_open_pair_scalars(Fr* __restrict__ ps, const Fr* __restrict__ scalars, size_t old_size, size_t half_up) {
+struct PairBatch { Fr* ps[OB_MAX]; const Fr* s[OB_MAX]; };
+__global__ void __launch_bounds__(256) k_open_pair_scalars(const PairBatch pb, size_t old_size, size_t half_up) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= half_up) return;
+    Fr* __restrict__ ps = pb.ps[blockIdx.y];
+    const Fr* __restrict__ scalars = pb.s[blockIdx.y];
     ps[i] = (2 * i + 1 < old_size) ? add(scalars[2 * i], scalars[2 * i + 1]) : scalars[2 * i];
 }
 __global__ void __launch_bounds__(GT) k_a29_to_jac(G1Jac* __restrict__ out, const A29* __restrict__ in, size_t n) {
@@ -880,15 +910,18 @@ __global__ void __launch_bounds__(256) k_a29_canon(A29* __restrict__ a, size_t n
 // affine points with coefficients that are plain field arithmetic; they run as one launch instead of a chain of
 // rounds that each wait for a scalar multiplication.
 // Folded scalars of all levels: level 0 is S itself, level j >= 1 sits at SL + sum_{1<=i<j} n_i, n_i = ceil(n0 / 2^i).
-__global__ void __launch_bounds__(1024) k_tail_scalars(Fr* __restrict__ SL, const Fr* __restrict__ S, const TailU us, uint32_t n0, uint32_t levels) {
-    const Fr* cur = S;
-    Fr* nxt = SL;
+struct TailPtrs { Fr* SL[OB_MAX]; const Fr* S[OB_MAX]; };      // per opening of a batch (blockIdx.x of k_tail_scalars, blockIdx.y of k_tail_coeffs)
+// U: the tail's challenges (Montgomery form), opening y's at U + y * ustride
+__global__ void __launch_bounds__(1024) k_tail_scalars(const TailPtrs tp, const Fr* __restrict__ U, uint32_t ustride, uint32_t n0, uint32_t levels) {
+    const Fr* __restrict__ usu = U + (size_t)blockIdx.x * ustride;
+    const Fr* cur = tp.S[blockIdx.x];
+    Fr* nxt = tp.SL[blockIdx.x];
     uint32_t n = n0;
     for (uint32_t j = 0; j < levels; ++j) {
         const uint32_t ns = (n + 1) / 2;
         for (uint32_t g = threadIdx.x; g < ns; g += 1024) {
             const Fr s0 = cur[2 * g];
-            nxt[g] = (2 * g + 1 < n) ? add(s0, mont_mul(us.u[j], sub(cur[2 * g + 1], s0))) : sub(s0, mont_mul(us.u[j], s0));
+            nxt[g] = (2 * g + 1 < n) ? add(s0, mont_mul(usu[j], sub(cur[2 * g + 1], s0))) : sub(s0, mont_mul(usu[j], s0));
         }
         __syncthreads();
         cur = nxt;
@@ -898,9 +931,13 @@ __global__ void __launch_bounds__(1024) k_tail_scalars(Fr* __restrict__ SL, cons
 }
 // C[(3j+0)*n0 + k] = s_j[k>>j] W_j(k); C[(3j+1)*n0 + k] = s_j[(k>>j)-1] W_j(k) for odd k>>j; C[(3j+2)*n0 + k] = s_j[(k>>j)+1] W_j(k)
 // for even k>>j with a partner; zero elsewhere.  C[3*levels*n0 + k] = W_levels(k).
-__global__ void __launch_bounds__(256) k_tail_coeffs(Fr* __restrict__ C, const Fr* __restrict__ SL, const Fr* __restrict__ S, const TailU us, uint32_t n0, uint32_t levels) {
+__global__ void __launch_bounds__(256) k_tail_coeffs(Fr* __restrict__ C0, const TailPtrs tp, const Fr* __restrict__ U, uint32_t ustride, uint32_t n0, uint32_t levels) {
     const uint32_t k = blockIdx.x * 256 + threadIdx.x;
     if (k >= n0) return;
+    const Fr* __restrict__ usu = U + (size_t)blockIdx.y * ustride;
+    Fr* __restrict__ C = C0 + (size_t)blockIdx.y * (3 * levels + 1) * n0;
+    const Fr* __restrict__ SL = tp.SL[blockIdx.y];
+    const Fr* __restrict__ S = tp.S[blockIdx.y];
     const Fr one_m = big_one_mont<8>();
     Fr W = one_m;                 // Montgomery form
     const Fr* sj = S;
@@ -913,7 +950,7 @@ __global__ void __launch_bounds__(256) k_tail_coeffs(Fr* __restrict__ C, const F
         C[(size_t)(3 * j) * n0 + k] = mont_mul(W, sj[i]);
         C[(size_t)(3 * j + 1) * n0 + k] = (i & 1u) ? mont_mul(W, sj[i - 1]) : zero;
         C[(size_t)(3 * j + 2) * n0 + k] = (!(i & 1u) && i + 1 < n) ? mont_mul(W, sj[i + 1]) : zero;
-        W = mont_mul(W, (i & 1u) ? sub(one_m, us.u[j]) : us.u[j]);
+        W = mont_mul(W, (i & 1u) ? sub(one_m, usu[j]) : usu[j]);
         const uint32_t ns = (n + 1) / 2;
         sj = nxt;
         nxt += ns;
@@ -922,7 +959,7 @@ __global__ void __launch_bounds__(256) k_tail_coeffs(Fr* __restrict__ C, const F
     C[(size_t)(3 * levels) * n0 + k] = from_mont(W);
 }
 // one workgroup per sum: lane 0 assembles sum_w 2^(8w) W[w] into pts[slot]
-__global__ void __launch_bounds__(GT) k_msm_horner(G1Jac* __restrict__ pts, const G1Jac* __restrict__ Wsum, const MsmDescs<TAIL_SUMS> descs) {
+__global__ void __launch_bounds__(GT) k_msm_horner(G1Jac* __restrict__ pts, const G1Jac* __restrict__ Wsum, const MsmDesc* __restrict__ descs) {
     if (threadIdx.x != 0) return;
     const G1Jac* W = Wsum + (size_t)blockIdx.x * MW;
     G1Jac r = W[MW - 1];
@@ -930,11 +967,11 @@ __global__ void __launch_bounds__(GT) k_msm_horner(G1Jac* __restrict__ pts, cons
         for (int k = 0; k < 8; ++k) r = g1_double(r);
         r = g1_add(r, W[w]);
     }
-    pts[descs.d[blockIdx.x].slot] = r;
+    pts[descs[blockIdx.x].slot] = r;
 }
 
-__global__ void __launch_bounds__(64) k_u32_zero(uint32_t* __restrict__ p, uint32_t n) {
-    for (uint32_t i = threadIdx.x; i < n; i += 64) p[i] = 0u;
+__global__ void __launch_bounds__(64) k_u32_zero(uint32_t* __restrict__ p, uint32_t n, size_t stride) {      // p[i * stride] = 0, i < n
+    for (uint32_t i = threadIdx.x; i < n; i += 64) p[(size_t)i * stride] = 0u;
 }
 // after the last round of an opening without a batched tail: the folded generator is the last proof point
 __global__ void __launch_bounds__(GT) k_open_finish(G1Jac* __restrict__ pts, const A29* __restrict__ last_gen, uint32_t rounds) {
@@ -978,6 +1015,7 @@ static int g1_sum_device(G1Jac* out, const G1Jac* in, size_t n, hipStream_t st) 
 
 // Optional timing of the fold kernel's launches with events on its own stream (measurement only).
 struct FoldTimer {
+    std::mutex mu;
     bool on = false;
     std::vector<std::pair<hipEvent_t, hipEvent_t>> ev;
     double fp_mults = 0;      // Fp multiplications the timed launches perform by the formulas' count
@@ -1055,20 +1093,29 @@ static int open_prep_build(A29* out, const G1Jac* gens, size_t n, Arena& arena, 
 // so T costs a bucket sum over half as many points: pair i gets the scalar s_2i + s_2i+1 (mod r: the generators have
 // order r) and the point g_2i + g_2i+1; an odd last element stands alone.  k_open_t_fix takes T0 and T1 off again,
 // window by window.
-__global__ void __launch_bounds__(64) k_open_t_fix(G1Jac* __restrict__ wsum) {
+__global__ void __launch_bounds__(64) k_open_t_fix(G1Jac* __restrict__ wsum0, uint32_t item_stride) {
     const uint32_t w = threadIdx.x;
     if (w >= (uint32_t)MW) return;
+    G1Jac* __restrict__ wsum = wsum0 + (size_t)blockIdx.x * item_stride;
     wsum[w] = g1_add(g1_add(wsum[w], g1_neg(wsum[MW + w])), g1_neg(wsum[2 * MW + w]));
 }
-static int open_round_launch(Fr* new_scalars, A29* new_gens, const Fr* scalars, const A29* gens, const Fr& u, size_t old_size, bool with_T,
-                             G1Jac* wsum_round, Arena& arena, hipStream_t st, hipStream_t aux, std::vector<hipEvent_t>& events) {
+// One round of `count` openings of equal size (count <= OB_MAX): one launch of each kernel covers all of them.
+struct RoundItem { Fr* new_scalars; A29* new_gens; const Fr* scalars; const A29* gens; Fr u; };
+static int open_round_launch(const RoundItem* items, int count, size_t old_size, bool with_T, G1Jac* wsum_round, uint32_t wsum_item_stride, Arena& arena, hipStream_t st,
+                             hipStream_t aux, std::vector<hipEvent_t>& events) {
     ZK_ARG(old_size < (1ull << 31), "opening: more than 2^31 generators");
+    ZK_ARG(count >= 1 && count <= OB_MAX, "opening: bad batch size");
     const size_t new_size = (old_size + 1) / 2;
     const bool chained = !with_T;
-    Scratch& dig = arena.add((size_t)(MW + 1) * old_size);
+    const size_t dig_bytes = (size_t)(MW + 1) * old_size;
+    Scratch& dig = arena.add(dig_bytes * count);
     if (dig.rc) return dig.rc;
-    hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(old_size, 256)), dim3(256), 0, st, dig.as<int8_t>(), scalars, old_size);
-    ZK_LAUNCH_CHECK();
+    {
+        RecodeBatch rb;
+        for (int i = 0; i < OB_MAX; ++i) { rb.D[i] = dig.as<int8_t>() + dig_bytes * (i < count ? i : 0); rb.S[i] = items[i < count ? i : 0].scalars; }
+        hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(old_size, 256), count), dim3(256), 0, st, rb, old_size);
+        ZK_LAUNCH_CHECK();
+    }
     if (aux != st) {
         hipEvent_t ready;
         ZK_HIP(hipEventCreateWithFlags(&ready, hipEventDisableTiming));
@@ -1077,24 +1124,36 @@ static int open_round_launch(Fr* new_scalars, A29* new_gens, const Fr* scalars, 
         ZK_HIP(hipStreamWaitEvent(aux, ready, 0));
     }
     // ---- side chain (aux): bucket sums, window sums; nothing here feeds the next fold ----
-    MsmDescs<3> descs;
+    MsmDescs<OB_SUMS> descs;
     const uint32_t half = (uint32_t)(old_size / 2);
     const uint32_t half_up = (uint32_t)new_size;
-    const uint32_t n_msm = chained ? 2u : 3u;
-    uint32_t q = 0;
-    const int8_t* dg = dig.as<int8_t>();
+    const uint32_t n_per = chained ? 2u : 3u, n_msm = n_per * (uint32_t)count;
     const uint32_t ds = (uint32_t)old_size;
+    const int8_t* dig2p = nullptr;
+    const size_t dig2_bytes = (size_t)(MW + 1) * half_up;
     if (!chained) {
-        Scratch& ps = arena.add(sizeof(Fr) * half_up);
-        Scratch& dig2 = arena.add((size_t)(MW + 1) * half_up);
+        Scratch& ps = arena.add(sizeof(Fr) * half_up * count);
+        Scratch& dig2 = arena.add(dig2_bytes * count);
         if (ps.rc || dig2.rc) return ps.rc ? ps.rc : dig2.rc;
-        hipLaunchKernelGGL(k_open_pair_scalars, dim3(cdiv(half_up, 256)), dim3(256), 0, aux, ps.as<Fr>(), scalars, old_size, (size_t)half_up);
-        hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(half_up, 256)), dim3(256), 0, aux, dig2.as<int8_t>(), ps.as<Fr>(), (size_t)half_up);
-        descs.d[q++] = MsmDesc{dig2.as<int8_t>(), half_up, half_up, 1u, 0u, 1u, (uint32_t)old_size, 0u};
+        PairBatch pb;
+        RecodeBatch rb;
+        for (int i = 0; i < OB_MAX; ++i) {
+            const int k = i < count ? i : 0;
+            pb.ps[i] = ps.as<Fr>() + (size_t)half_up * k; pb.s[i] = items[k].scalars;
+            rb.D[i] = dig2.as<int8_t>() + dig2_bytes * k; rb.S[i] = pb.ps[i];
+        }
+        hipLaunchKernelGGL(k_open_pair_scalars, dim3(cdiv(half_up, 256), count), dim3(256), 0, aux, pb, old_size, (size_t)half_up);
+        hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(half_up, 256), count), dim3(256), 0, aux, rb, (size_t)half_up);
+        dig2p = dig2.as<int8_t>();
     }
-    descs.d[q++] = MsmDesc{dg, ds, half, 2u, 0u, 2u, 1u, 1u};
-    descs.d[q++] = MsmDesc{dg, ds, half, 2u, 1u, 2u, 0u, 2u};
-    for (; q < 3; ++q) descs.d[q] = MsmDesc{dg, ds, 0u, 1u, 0u, 1u, 0u, 0u};
+    uint32_t q = 0;
+    for (int i = 0; i < count; ++i) {
+        const int8_t* dg = dig.as<int8_t>() + dig_bytes * i;
+        if (!chained) descs.d[q++] = MsmDesc{dig2p + dig2_bytes * i, items[i].gens, half_up, half_up, 1u, 0u, 1u, (uint32_t)old_size, 0u};
+        descs.d[q++] = MsmDesc{dg, items[i].gens, ds, half, 2u, 0u, 2u, 1u, 1u};
+        descs.d[q++] = MsmDesc{dg, items[i].gens, ds, half, 2u, 1u, 2u, 0u, 2u};
+    }
+    for (; q < (uint32_t)OB_SUMS; ++q) descs.d[q] = MsmDesc{dig.as<int8_t>(), items[0].gens, ds, 0u, 1u, 0u, 1u, 0u, 0u};
     // One chunk per workgroup: many short workgroups keep every compute unit busy to the end of the launch (with few
     // long ones, all equally long, whatever does not fit the first turn waits a whole turn); the raw buckets of the
     // segments are summed afterwards.  Very large inputs take more chunks per workgroup to bound the bucket storage.
@@ -1104,8 +1163,8 @@ static int open_round_launch(Fr* new_scalars, A29* new_gens, const Fr* scalars, 
     const uint32_t nseg = (chunks + cps - 1) / cps;
     Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (size_t)nseg * MT);
     if (partial.rc) return partial.rc;
-    G1Jac* wsum = wsum_round + (size_t)(3 - n_msm) * MW;
-    hipLaunchKernelGGL(k_msm_seg<3>, dim3(nseg, MW, n_msm), dim3(MSL), 0, aux, partial.as<G1Jac>(), gens, descs, nseg, cps);
+    G1Jac* wsum = wsum_round + (size_t)(3 - n_per) * MW;
+    hipLaunchKernelGGL(k_msm_seg<OB_SUMS>, dim3(nseg, MW, n_msm), dim3(MSL), 0, aux, partial.as<G1Jac>(), descs, (const MsmDesc*)nullptr, nseg, cps);
     {
         // sum the segments' raw buckets eight at a time, then weight and total
         const G1Jac* cur = partial.as<G1Jac>();
@@ -1118,71 +1177,99 @@ static int open_round_launch(Fr* new_scalars, A29* new_gens, const Fr* scalars, 
             cur = nxt.as<G1Jac>();
             ns = ng;
         }
-        hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, aux, wsum, cur, ns);
+        hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, aux, wsum, cur, ns, n_per, wsum_item_stride);
     }
-    if (!chained) hipLaunchKernelGGL(k_open_t_fix, dim3(1), dim3(64), 0, aux, wsum);
+    if (!chained) hipLaunchKernelGGL(k_open_t_fix, dim3(count), dim3(64), 0, aux, wsum, wsum_item_stride);
     ZK_LAUNCH_CHECK();
     // ---- critical chain (st): the fold ----
-    const GlvK ku = glv_split(u);
-    const JsfK jsf = jsf_of(ku);
-    Scratch& special = arena.add(sizeof(uint32_t) * (1 + new_size));
+    const size_t sp_stride = 1 + new_size;
+    Scratch& special = arena.add(sizeof(uint32_t) * sp_stride * count);
     if (special.rc) return special.rc;
-    hipLaunchKernelGGL(k_u32_zero, dim3(1), dim3(64), 0, st, special.as<uint32_t>(), 1u);
+    FoldBatch fb;
+    SpecialBatch sb;
+    double fp_mults = 0;
+    for (int i = 0; i < OB_MAX; ++i) {
+        const int k = i < count ? i : 0;
+        const GlvK ku = glv_split(items[k].u);
+        FoldItem& f = fb.it[i];
+        f.ns = items[k].new_scalars; f.ng = items[k].new_gens; f.s = items[k].scalars; f.g = items[k].gens;
+        f.special = special.as<uint32_t>() + sp_stride * k;
+        f.u_mont = to_mont(items[k].u);
+        f.jsf = jsf_of(ku);
+        sb.ng[i] = f.ng; sb.g[i] = f.g; sb.special[i] = f.special; sb.ku[i] = ku;
+        if (i < count) fp_mults += fold_fp_mults_per_pair(f.jsf) * (double)new_size;
+    }
+    hipLaunchKernelGGL(k_u32_zero, dim3(1), dim3(64), 0, st, special.as<uint32_t>(), (uint32_t)count, sp_stride);
     hipEvent_t t0 = nullptr, t1 = nullptr;
     if (g_fold_timer.on) {
         ZK_HIP(hipEventCreate(&t0));
         ZK_HIP(hipEventCreate(&t1));
         ZK_HIP(hipEventRecord(t0, st));
     }
-    hipLaunchKernelGGL(k_open_fold29, dim3(cdiv(new_size, GT)), dim3(GT), 0, st, new_scalars, new_gens, scalars, gens, to_mont(u), jsf, old_size, new_size, special.as<uint32_t>());
+    hipLaunchKernelGGL(k_open_fold29, dim3(cdiv(new_size, GT), count), dim3(GT), 0, st, fb, old_size, new_size);
     if (g_fold_timer.on) {
         ZK_HIP(hipEventRecord(t1, st));
+        std::lock_guard<std::mutex> lk(g_fold_timer.mu);
         g_fold_timer.ev.emplace_back(t0, t1);
-        g_fold_timer.fp_mults += fold_fp_mults_per_pair(jsf) * (double)new_size;
-        g_fold_timer.pairs += new_size;
+        g_fold_timer.fp_mults += fp_mults;
+        g_fold_timer.pairs += new_size * (size_t)count;
     }
-    hipLaunchKernelGGL(k_open_fold_special, dim3(16), dim3(GT), 0, st, new_gens, gens, ku, old_size, special.as<uint32_t>());
+    hipLaunchKernelGGL(k_open_fold_special, dim3(16, count), dim3(GT), 0, st, sb, old_size);
     ZK_LAUNCH_CHECK();
     return 0;
 }
 
 // Queues the batch for the last `levels` rounds (rounds r0 .. r0+levels-1 of `rounds`) over n0 <= TAIL_N generators.
 // Writes T, T0, T1 of those rounds and the final generator into pts; *final_scalar points at the folded scalar.
-static int open_tail_launch(const Fr* scalars, const A29* gens, size_t n0, const uint32_t* u, int levels, int r0, int rounds, G1Jac* pts, const Fr** final_scalar,
-                            Arena& arena, hipStream_t st) {
-    TailU us;
-    for (int j = 0; j < levels; ++j) us.u[j] = to_mont(load_fr(u + 8 * j));
-    for (int j = levels; j < TAIL_LEVELS; ++j) us.u[j] = big_zero<8>();
-    Scratch& sl = arena.add(sizeof(Fr) * (n0 + (size_t)levels + 1));
+// Challenges and bucket-sum descriptors of a job travel through one pinned host buffer of 64 KiB (held until the job
+// ends) into one device block: the challenges of all openings (Montgomery form, `rounds` per opening) in its first half, the
+// descriptors of the batched last rounds in its second.
+static constexpr size_t JOB_U_BYTES = 32768, JOB_DESC_BYTES = 32768;
+static int open_tail_launch(const Fr** scalars, const A29* const* gens, int count, size_t n0, int levels, int r0, int rounds, G1Jac* pts, const Fr* U_dev, void* pin_host,
+                            void* desc_dev, Arena& arena, hipStream_t st) {
     const int n_msm = 3 * levels + 1;
+    const int total = n_msm * count;
+    ZK_ARG(sizeof(MsmDesc) * (size_t)total <= JOB_DESC_BYTES, "opening: too many sums in the batched last rounds");
+    const size_t npts = 3 * (size_t)rounds + 1;
+    const size_t sl_n = n0 + (size_t)levels + 1;
+    Scratch& sl = arena.add(sizeof(Fr) * sl_n * count);
     const uint32_t nseg = cdiv(n0, MSEG), cps = 1;       // one chunk per workgroup, as in the halving rounds
-    Scratch& coef = arena.add(sizeof(Fr) * (size_t)n_msm * n0);
-    Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (size_t)nseg * MT);
-    Scratch& wsum = arena.add(sizeof(G1Jac) * n_msm * MW);
+    const size_t ncoef = (size_t)n_msm * n0 * count;
+    Scratch& coef = arena.add(sizeof(Fr) * ncoef);
+    Scratch& partial = arena.add(sizeof(G1Jac) * total * MW * (size_t)nseg * MT);
+    Scratch& wsum = arena.add(sizeof(G1Jac) * (size_t)total * MW);
+    Scratch& dig = arena.add((size_t)(MW + 1) * ncoef);
     if (sl.rc) return sl.rc;
     if (coef.rc) return coef.rc;
     if (partial.rc) return partial.rc;
     if (wsum.rc) return wsum.rc;
-    hipLaunchKernelGGL(k_tail_scalars, dim3(1), dim3(1024), 0, st, sl.as<Fr>(), scalars, us, (uint32_t)n0, (uint32_t)levels);
-    hipLaunchKernelGGL(k_tail_coeffs, dim3(cdiv(n0, 256)), dim3(256), 0, st, coef.as<Fr>(), sl.as<Fr>(), scalars, us, (uint32_t)n0, (uint32_t)levels);
-    const size_t ncoef = (size_t)n_msm * n0;
-    Scratch& dig = arena.add((size_t)(MW + 1) * ncoef);
     if (dig.rc) return dig.rc;
-    hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(ncoef, 256)), dim3(256), 0, st, dig.as<int8_t>(), coef.as<Fr>(), ncoef);
-    MsmDescs<TAIL_SUMS> descs;
-    for (int i = 0; i < TAIL_SUMS; ++i) {
-        const bool live = i < n_msm;
-        const uint32_t slot = !live ? 0u : (i == 3 * levels ? 3u * (uint32_t)rounds : 3u * (uint32_t)r0 + (uint32_t)i);
-        descs.d[i] = MsmDesc{dig.as<int8_t>(), (uint32_t)ncoef, live ? (uint32_t)n0 : 0u, 1u, live ? (uint32_t)((size_t)i * n0) : 0u, 1u, 0u, slot};
+    ZK_ARG(ncoef < (1ull << 32), "opening: batched last rounds too large");
+    TailPtrs tp;
+    for (int i = 0; i < OB_MAX; ++i) { const int k = i < count ? i : 0; tp.SL[i] = sl.as<Fr>() + sl_n * k; tp.S[i] = scalars[k]; }
+    hipLaunchKernelGGL(k_tail_scalars, dim3(count), dim3(1024), 0, st, tp, U_dev + r0, (uint32_t)rounds, (uint32_t)n0, (uint32_t)levels);
+    hipLaunchKernelGGL(k_tail_coeffs, dim3(cdiv(n0, 256), count), dim3(256), 0, st, coef.as<Fr>(), tp, U_dev + r0, (uint32_t)rounds, (uint32_t)n0, (uint32_t)levels);
+    {
+        RecodeBatch rb;
+        for (int i = 0; i < OB_MAX; ++i) { rb.D[i] = dig.as<int8_t>(); rb.S[i] = coef.as<Fr>(); }
+        hipLaunchKernelGGL(k_msm_recode, dim3(cdiv(ncoef, 256), 1), dim3(256), 0, st, rb, ncoef);
     }
-    hipLaunchKernelGGL(k_msm_seg<TAIL_SUMS>, dim3(nseg, MW, n_msm), dim3(MSL), 0, st, partial.as<G1Jac>(), gens, descs, nseg, cps);
-    hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), nseg);
-    hipLaunchKernelGGL(k_msm_horner, dim3(n_msm), dim3(GT), 0, st, pts, wsum.as<G1Jac>(), descs);
+    MsmDesc* hd = reinterpret_cast<MsmDesc*>((char*)pin_host + JOB_U_BYTES);
+    for (int it = 0; it < count; ++it)
+        for (int i = 0; i < n_msm; ++i) {
+            const uint32_t slot = (uint32_t)(npts * it) + (i == 3 * levels ? 3u * (uint32_t)rounds : 3u * (uint32_t)r0 + (uint32_t)i);
+            hd[it * n_msm + i] = MsmDesc{dig.as<int8_t>(), gens[it], (uint32_t)ncoef, (uint32_t)n0, 1u, (uint32_t)(((size_t)it * n_msm + i) * n0), 1u, 0u, slot};
+        }
+    ZK_HIP(hipMemcpyAsync(desc_dev, hd, sizeof(MsmDesc) * (size_t)total, hipMemcpyHostToDevice, st));
+    const MsmDesc* dd = (const MsmDesc*)desc_dev;
+    hipLaunchKernelGGL(k_msm_seg<1>, dim3(nseg, MW, total), dim3(MSL), 0, st, partial.as<G1Jac>(), MsmDescs<1>(), dd, nseg, cps);
+    hipLaunchKernelGGL(k_msm_buckets, dim3(total * MW), dim3(MT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), nseg, (uint32_t)total, 0u);
+    hipLaunchKernelGGL(k_msm_horner, dim3(total), dim3(GT), 0, st, pts, wsum.as<G1Jac>(), dd);
     ZK_LAUNCH_CHECK();
     // the folded scalar is the single element of the last level
     size_t off = 0, nn = n0;
     for (int j = 1; j < levels; ++j) { nn = (nn + 1) / 2; off += nn; }
-    *final_scalar = sl.as<Fr>() + off;
+    for (int it = 0; it < count; ++it) scalars[it] = sl.as<Fr>() + sl_n * it + off;
     return 0;
 }
 
@@ -1392,11 +1479,12 @@ int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host, con
     int rc = open_prep_build(g29.as<A29>(), (const G1Jac*)gens, old_size, arena, st);
     if (rc) return rc;
     std::vector<hipEvent_t> evs;
-    rc = open_round_launch((Fr*)new_scalars, n29.as<A29>(), (const Fr*)scalars, g29.as<A29>(), load_fr(u), old_size, true, wsum.as<G1Jac>(), arena, st, st, evs);
+    const RoundItem item{(Fr*)new_scalars, n29.as<A29>(), (const Fr*)scalars, g29.as<A29>(), load_fr(u)};
+    rc = open_round_launch(&item, 1, old_size, true, wsum.as<G1Jac>(), 0u, arena, st, st, evs);
     (void)evs;
     if (rc) return rc;
     hipLaunchKernelGGL(k_a29_to_jac, dim3(cdiv(new_size, GT)), dim3(GT), 0, st, (G1Jac*)new_gens, n29.as<A29>(), new_size);
-    hipLaunchKernelGGL(k_open_horner, dim3(3), dim3(GT), 0, st, pts.as<G1Jac>(), wsum.as<G1Jac>(), 1u);
+    hipLaunchKernelGGL(k_open_horner, dim3(3, 1), dim3(GT), 0, st, pts.as<G1Jac>(), wsum.as<G1Jac>(), 1u, 3u, 0u);
     hipLaunchKernelGGL(k_g1_normalize<false>, dim3(1), dim3(GT), 0, st, pts.p, pts.as<G1Jac>(), (size_t)3);
     ZK_LAUNCH_CHECK();
     void* stage = nullptr;
@@ -1414,67 +1502,88 @@ int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host, con
 struct OpenJob {
     Arena arena;
     hipStream_t st = nullptr;
-    int rounds = 0;
-    G1Jac* pts = nullptr;
-    const Fr* final_scalar = nullptr;
+    int rounds = 0, count = 0;
+    G1Jac* pts = nullptr;                      // count x (3 rounds + 1) points
+    const Fr* final_scalar[OB_MAX] = {};
     hipEvent_t ready = nullptr;    // only for jobs on a side stream
     hipStream_t aux = nullptr;     // second stream of the job (bucket sums beside the folds); equals st when the job has one stream
     std::vector<hipEvent_t> events;
+    void* pin = nullptr;           // pinned host buffer behind the job's challenges and descriptors
+    ~OpenJob() { pinned_release(pin); }
 };
-// gens: Jacobian generators, or null when `prep` (their prepared form, open_prep_build) is given
-static int open_queue(OpenJob& job, const void* scalars, const void* gens, const A29* prep, size_t n, const uint32_t* u, int rounds, hipStream_t st, hipStream_t aux) {
+// One opening of the batch: its scalars, its challenges (rounds x 8 limbs) and its generators -- Jacobian, or null when
+// `prep` (their prepared form, open_prep_build) is given
+struct OpenItem { const void* scalars; const void* gens; const A29* prep; const uint32_t* u; };
+static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, int rounds, hipStream_t st, hipStream_t aux) {
     ZK_ARG(n >= 1, "zk_g1_open: empty input");
+    ZK_ARG(count >= 1 && count <= OB_MAX, "zk_g1_open: a batch holds 1 to 8 openings");
     ZK_ARG(rounds >= 0 && rounds <= 64, "zk_g1_open: bad round count");
     ZK_ARG(sizeof(G1Jac) * (3 * (size_t)rounds + 1) + sizeof(Fr) <= 65536, "zk_g1_open: proof larger than the staging buffer");
     job.st = st;
     job.aux = aux;
     job.arena.streams(st, aux);      // blocks serve kernels of both streams; aux joins st before the job ends
     job.rounds = rounds;
+    job.count = count;
     const size_t npts = 3 * (size_t)rounds + 1;
-    Scratch& pts = job.arena.add(sizeof(G1Jac) * npts);
-    Scratch& wsum = job.arena.add(sizeof(G1Jac) * 3 * MW * (rounds ? rounds : 1));      // window sums of the halving rounds
+    const uint32_t wstride = 3u * MW * (uint32_t)(rounds ? rounds : 1);      // window sums of one opening's halving rounds
+    Scratch& pts = job.arena.add(sizeof(G1Jac) * npts * count);
+    Scratch& wsum = job.arena.add(sizeof(G1Jac) * (size_t)wstride * count);
     if (pts.rc) return pts.rc;
     if (wsum.rc) return wsum.rc;
     job.pts = pts.as<G1Jac>();
-    const Fr* cs = (const Fr*)scalars;
-    const A29* cg = prep;
-    if (!cg) {
-        Scratch& g29 = job.arena.add(sizeof(A29) * (n + (n + 1) / 2));
-        if (g29.rc) return g29.rc;
-        int rc = open_prep_build(g29.as<A29>(), (const G1Jac*)gens, n, job.arena, st);
-        if (rc) return rc;
-        cg = g29.as<A29>();
+    ZK_ARG(sizeof(Fr) * (size_t)rounds * count <= JOB_U_BYTES, "zk_g1_open: too many rounds for the batch");
+    Scratch& jdev = job.arena.add(JOB_U_BYTES + JOB_DESC_BYTES);
+    if (jdev.rc) return jdev.rc;
+    {
+        int prc = pinned_acquire(&job.pin);
+        if (prc) return prc;
+        Fr* hu = (Fr*)job.pin;
+        for (int i = 0; i < count; ++i)
+            for (int r = 0; r < rounds; ++r) hu[(size_t)i * rounds + r] = to_mont(load_fr(items[i].u + 8 * r));
+        if (rounds) ZK_HIP(hipMemcpyAsync(jdev.p, job.pin, sizeof(Fr) * (size_t)rounds * count, hipMemcpyHostToDevice, st));
+    }
+    const Fr* U_dev = jdev.as<Fr>();
+    const Fr* cs[OB_MAX];
+    const A29* cg[OB_MAX];
+    for (int i = 0; i < count; ++i) {
+        cs[i] = (const Fr*)items[i].scalars;
+        cg[i] = items[i].prep;
+        if (!cg[i]) {
+            Scratch& g29 = job.arena.add(sizeof(A29) * (n + (n + 1) / 2));
+            if (g29.rc) return g29.rc;
+            int rc = open_prep_build(g29.as<A29>(), (const G1Jac*)items[i].gens, n, job.arena, st);
+            if (rc) return rc;
+            cg[i] = g29.as<A29>();
+        }
     }
     size_t size = n;
     int halving_rounds = rounds;
     bool tail_done = false;
-    OpenUs us;
-    memset(&us, 0, sizeof(us));
     for (int r = 0; r < rounds; ++r) {
-        if (size <= (size_t)tail_n_env() && rounds - r <= TAIL_LEVELS) {
-            int rc = open_tail_launch(cs, cg, size, u + 8 * r, rounds - r, r, rounds, pts.as<G1Jac>(), &cs, job.arena, st);
+        if (size <= (size_t)TAIL_N && rounds - r <= TAIL_LEVELS) {
+            int rc = open_tail_launch(cs, cg, count, size, rounds - r, r, rounds, pts.as<G1Jac>(), U_dev, job.pin, (char*)jdev.p + JOB_U_BYTES, job.arena, st);
             if (rc) return rc;
             halving_rounds = r;
             tail_done = true;
             break;
         }
         const size_t ns = (size + 1) / 2;
-        Scratch& s2 = job.arena.add(sizeof(Fr) * ns);
-        Scratch& g2 = job.arena.add(sizeof(A29) * ns);
+        Scratch& s2 = job.arena.add(sizeof(Fr) * ns * count);
+        Scratch& g2 = job.arena.add(sizeof(A29) * ns * count);
         if (s2.rc) return s2.rc;
         if (g2.rc) return g2.rc;
-        const Fr ur = load_fr(u + 8 * r);
-        us.u[r] = to_mont(ur);
-        int rc = open_round_launch(s2.as<Fr>(), g2.as<A29>(), cs, cg, ur, size, r == 0, wsum.as<G1Jac>() + (size_t)3 * MW * r, job.arena, st, aux, job.events);
+        RoundItem ri[OB_MAX];
+        for (int i = 0; i < count; ++i) ri[i] = RoundItem{s2.as<Fr>() + ns * i, g2.as<A29>() + ns * i, cs[i], cg[i], load_fr(items[i].u + 8 * r)};
+        int rc = open_round_launch(ri, count, size, r == 0, wsum.as<G1Jac>() + (size_t)3 * MW * r, wstride, job.arena, st, aux, job.events);
         if (rc) return rc;
-        cs = s2.as<Fr>();
-        cg = g2.as<A29>();
+        for (int i = 0; i < count; ++i) { cs[i] = ri[i].new_scalars; cg[i] = ri[i].new_gens; }
         size = ns;
     }
     // the single points of the halving rounds, behind the last bucket sums
     if (halving_rounds > 0) {
-        hipLaunchKernelGGL(k_open_horner, dim3(3 * halving_rounds), dim3(GT), 0, aux, pts.as<G1Jac>(), wsum.as<G1Jac>(), (uint32_t)halving_rounds);
-        if (halving_rounds > 1) hipLaunchKernelGGL(k_open_chain, dim3(halving_rounds - 1), dim3(GT), 0, aux, pts.as<G1Jac>(), us, (uint32_t)halving_rounds);
+        hipLaunchKernelGGL(k_open_horner, dim3(3 * halving_rounds, count), dim3(GT), 0, aux, pts.as<G1Jac>(), wsum.as<G1Jac>(), (uint32_t)halving_rounds, (uint32_t)npts, wstride);
+        if (halving_rounds > 1)
+            hipLaunchKernelGGL(k_open_chain, dim3(halving_rounds - 1, count), dim3(GT), 0, aux, pts.as<G1Jac>(), U_dev, (uint32_t)halving_rounds, (uint32_t)npts, (uint32_t)rounds);
         ZK_LAUNCH_CHECK();
     }
     if (aux != st) {
@@ -1484,37 +1593,42 @@ static int open_queue(OpenJob& job, const void* scalars, const void* gens, const
         ZK_HIP(hipEventRecord(done, aux));
         ZK_HIP(hipStreamWaitEvent(st, done, 0));
     }
-    if (!tail_done) hipLaunchKernelGGL(k_open_finish, dim3(1), dim3(GT), 0, st, pts.as<G1Jac>(), cg, (uint32_t)rounds);
-    hipLaunchKernelGGL(k_g1_normalize<false>, dim3(cdiv(cdiv(npts, CH), GT)), dim3(GT), 0, st, pts.p, pts.as<G1Jac>(), npts);
+    if (!tail_done)
+        for (int i = 0; i < count; ++i) hipLaunchKernelGGL(k_open_finish, dim3(1), dim3(GT), 0, st, pts.as<G1Jac>() + npts * i, cg[i], (uint32_t)rounds);
+    hipLaunchKernelGGL(k_g1_normalize<false>, dim3(cdiv(cdiv(npts * count, CH), GT)), dim3(GT), 0, st, pts.p, pts.as<G1Jac>(), npts * count);
     ZK_LAUNCH_CHECK();
-    job.final_scalar = cs;
+    for (int i = 0; i < count; ++i) job.final_scalar[i] = cs[i];
     return 0;
 }
-// waits for the job's stream and copies the proof points and the folded scalar out
+// waits for the job's stream and copies the proof points and the folded scalars out: opening i's points at
+// proof_host + i * (3 rounds + 1) * 36, its scalar at final_scalar_host + i * 8
 static int open_collect(OpenJob& job, uint32_t* proof_host, uint32_t* final_scalar_host) {
     const size_t npts = 3 * (size_t)job.rounds + 1;
     void* stage = nullptr;
     int rc = staging(&stage, sizeof(G1Jac) * npts + sizeof(Fr));
     if (rc) return rc;
-    ZK_HIP(hipMemcpyAsync(stage, job.pts, sizeof(G1Jac) * npts, hipMemcpyDeviceToHost, job.st));
-    ZK_HIP(hipMemcpyAsync((char*)stage + sizeof(G1Jac) * npts, job.final_scalar, sizeof(Fr), hipMemcpyDeviceToHost, job.st));
-    ZK_HIP(hipStreamSynchronize(job.st));
-    memcpy(proof_host, stage, sizeof(G1Jac) * npts);
-    memcpy(final_scalar_host, (char*)stage + sizeof(G1Jac) * npts, sizeof(Fr));
+    for (int i = 0; i < job.count; ++i) {
+        ZK_HIP(hipMemcpyAsync(stage, job.pts + npts * i, sizeof(G1Jac) * npts, hipMemcpyDeviceToHost, job.st));
+        ZK_HIP(hipMemcpyAsync((char*)stage + sizeof(G1Jac) * npts, job.final_scalar[i], sizeof(Fr), hipMemcpyDeviceToHost, job.st));
+        ZK_HIP(hipStreamSynchronize(job.st));
+        memcpy(proof_host + 36 * npts * i, stage, sizeof(G1Jac) * npts);
+        memcpy(final_scalar_host + 8 * (size_t)i, (char*)stage + sizeof(G1Jac) * npts, sizeof(Fr));
+    }
     return 0;
 }
 // proof_host receives 3*rounds + 1 points: T, T0, T1 of every round, then the folded generator; all normalised to
 // z = 1 (infinity: all-zero limbs).  final_scalar_host: the folded scalar.
 int zk_g1_open(uint32_t* proof_host, uint32_t* final_scalar_host, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stv) {
     OpenJob job;
-    int rc = open_queue(job, scalars, gens, nullptr, n, u, rounds, (hipStream_t)stv, (hipStream_t)stv);
+    const OpenItem item{scalars, gens, nullptr, u};
+    int rc = open_queue(job, &item, 1, n, rounds, (hipStream_t)stv, (hipStream_t)stv);
     if (rc) { (void)hipStreamSynchronize((hipStream_t)stv); return rc; }
     return open_collect(job, proof_host, final_scalar_host);
 }
 // The same in two halves.  begin queues the recursion on a stream of the library's own, ordered after everything queued
 // on `stream` so far, and returns at once; the caller goes on using `stream`, and both run side by side.  scalars and gens
 // must stay alive and unmodified until end, which waits for the opening, delivers its results and releases its buffers.
-static int open_begin_impl(void** handle, const void* scalars, const void* gens, const A29* prep, size_t n, const uint32_t* u, int rounds, void* stv) {
+static int open_begin_impl(void** handle, const OpenItem* items, int count, size_t n, int rounds, void* stv) {
     ZK_ARG(handle != nullptr, "zk_g1_open_begin: null handle");
     hipStream_t side = side_stream(0), aux = side_stream(0);      // consecutive streams of the pool: the folds on one, the bucket sums on the other
     ZK_ARG(side != nullptr && aux != nullptr, "zk_g1_open_begin: could not create a stream");
@@ -1522,7 +1636,7 @@ static int open_begin_impl(void** handle, const void* scalars, const void* gens,
     ZK_HIP(hipEventCreateWithFlags(&job->ready, hipEventDisableTiming));
     ZK_HIP(hipEventRecord(job->ready, (hipStream_t)stv));
     ZK_HIP(hipStreamWaitEvent(side, job->ready, 0));
-    int rc = open_queue(*job, scalars, gens, prep, n, u, rounds, side, aux);
+    int rc = open_queue(*job, items, count, n, rounds, side, aux);
     if (rc) {
         (void)hipStreamSynchronize(side);
         (void)hipStreamSynchronize(aux);
@@ -1534,7 +1648,8 @@ static int open_begin_impl(void** handle, const void* scalars, const void* gens,
     return 0;
 }
 int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_t n, const uint32_t* u, int rounds, void* stv) {
-    return open_begin_impl(handle, scalars, gens, nullptr, n, u, rounds, stv);
+    const OpenItem item{scalars, gens, nullptr, u};
+    return open_begin_impl(handle, &item, 1, n, rounds, stv);
 }
 // Generators prepared once for any number of openings against them: their affine 29-bit-limb form and the pair sums of
 // the first round (weight-independent; 1.5 n points of 112 bytes).  The handle is freed with zk_g1_open_prepared_free
@@ -1567,8 +1682,28 @@ int zk_g1_open_prepared_free(void* prepared) {
 int zk_g1_open_begin_prepared(void** handle, const void* scalars, const void* prepared, const uint32_t* u, int rounds, void* stv) {
     ZK_ARG(prepared != nullptr, "zk_g1_open_begin_prepared: null generators");
     const OpenPrepared* pr = (const OpenPrepared*)prepared;
-    return open_begin_impl(handle, scalars, nullptr, (const A29*)pr->a29, pr->n, u, rounds, stv);
+    const OpenItem item{scalars, nullptr, (const A29*)pr->a29, u};
+    return open_begin_impl(handle, &item, 1, pr->n, rounds, stv);
 }
+// `count` (1 to 8) openings against prepared generator sets of one size and with one round count, as ONE job: every
+// kernel of a round is launched once for all of them, so the late rounds have count times the waves.  u: opening i's
+// challenges at u + i * rounds * 8.  zk_g1_open_end_batch delivers opening i's points at proof_host + i * (3 rounds + 1) * 36
+// and its folded scalar at final_scalar_host + i * 8.
+int zk_g1_open_begin_batch(void** handle, int count, const void* const* scalars, const void* const* prepared, const uint32_t* u, int rounds, void* stv) {
+    ZK_ARG(count >= 1 && count <= OB_MAX, "zk_g1_open_begin_batch: 1 to 8 openings");
+    ZK_ARG(scalars != nullptr && prepared != nullptr && u != nullptr, "zk_g1_open_begin_batch: null argument");
+    OpenItem items[OB_MAX];
+    size_t n = 0;
+    for (int i = 0; i < count; ++i) {
+        ZK_ARG(prepared[i] != nullptr && scalars[i] != nullptr, "zk_g1_open_begin_batch: null opening");
+        const OpenPrepared* pr = (const OpenPrepared*)prepared[i];
+        if (i == 0) n = pr->n;
+        ZK_ARG(pr->n == n, "zk_g1_open_begin_batch: the generator sets differ in size");
+        items[i] = OpenItem{scalars[i], nullptr, (const A29*)pr->a29, u + (size_t)i * rounds * 8};
+    }
+    return open_begin_impl(handle, items, count, n, rounds, stv);
+}
+int zk_g1_open_end_batch(void* handle, uint32_t* proof_host, uint32_t* final_scalar_host) { return zk_g1_open_end(handle, proof_host, final_scalar_host); }
 int zk_g1_open_end(void* handle, uint32_t* proof_host, uint32_t* final_scalar_host) {
     ZK_ARG(handle != nullptr, "zk_g1_open_end: null handle");
     std::unique_ptr<OpenJob> job((OpenJob*)handle);

@@ -51,7 +51,7 @@ static size_t round_size(size_t b) {
 // blocks it used last still sit in the free lists, and a destroyed stream must never be passed to the runtime again: for
 // such streams the event is recorded when the block is freed (the stream is certainly alive then) and kept with the block.
 static std::mutex g_side_mu;
-static hipStream_t g_side_streams[2][8] = {};
+static hipStream_t g_side_streams[2][24] = {};
 static bool is_persistent_stream(hipStream_t s) {
     if (s == nullptr) return true;
     std::lock_guard<std::mutex> lk(g_side_mu);
@@ -167,7 +167,7 @@ hipStream_t side_stream(int pool) {
         count[0] = 6; count[1] = 2;       // an opening takes two consecutive streams of pool 0 (folds / bucket sums); three openings in flight
         if (const char* e = getenv("ZKLLM_SIDE_STREAMS")) {          // "openings,sumchecks[,shared]" (experiments)
             int a = 0, b2 = 0, c = 0;
-            if (sscanf(e, "%d,%d,%d", &a, &b2, &c) >= 2 && a >= 1 && a <= 8 && b2 >= 1 && b2 <= 8) { count[0] = a; count[1] = b2; shared = c; }
+            if (sscanf(e, "%d,%d,%d", &a, &b2, &c) >= 2 && a >= 1 && a <= 24 && b2 >= 1 && b2 <= 24) { count[0] = a; count[1] = b2; shared = c; }
         }
     }
     const int q = (pool && !shared) ? 1 : 0;

@@ -97,6 +97,54 @@ void Commitment::open_start(Pending& p) const {
     if (prepared) ZKC(zk_g1_open_begin_prepared(&p.handle, p.folded->gpu_data, prepared.get(), uu.data(), p.rounds, nullptr));
     else ZKC(zk_g1_open_begin(&p.handle, p.folded->gpu_data, gpu_data, size, uu.data(), p.rounds, nullptr));
 }
+struct Commitment::Pending::Batch {
+    void* handle = nullptr;
+    int count = 0, rounds = 0;
+    bool collected = false;
+    std::vector<G1Jacobian_t> pts;
+    std::vector<Fr_t> finals;
+    std::vector<std::unique_ptr<FrTensor>> folded;      // what the queued kernels read, kept until the job has been collected
+    ~Batch() {
+        if (handle && !collected) {
+            pts.resize((size_t)count * (3 * (size_t)rounds + 1));
+            finals.resize(count);
+            (void)zk_g1_open_end_batch(handle, pts[0].x.val, finals[0].val);
+        }
+    }
+};
+void Commitment::open_start_batch(const std::vector<std::pair<const Commitment*, Pending*>>& ops) {
+    std::vector<bool> done(ops.size(), false);
+    for (size_t i = 0; i < ops.size(); ++i) {
+        if (done[i]) continue;
+        const Commitment* c = ops[i].first;
+        Pending* p = ops[i].second;
+        std::vector<size_t> group{i};
+        if (!g_skip_g1 && c->prepared)
+            for (size_t j = i + 1; j < ops.size() && group.size() < 8; ++j)
+                if (!done[j] && ops[j].first->prepared && ops[j].first->size == c->size && ops[j].second->u_in.size() == p->u_in.size()) group.push_back(j);
+        if (group.size() == 1) { c->open_start(*p); done[i] = true; continue; }
+        auto b = std::make_shared<Pending::Batch>();
+        b->count = (int)group.size();
+        b->rounds = (int)p->u_in.size();
+        std::vector<const void*> sc, pr;
+        std::vector<uint32_t> uu((size_t)b->count * b->rounds * 8 + 8);
+        for (size_t k = 0; k < group.size(); ++k) {
+            Pending* q = ops[group[k]].second;
+            sc.push_back(q->folded->gpu_data);
+            pr.push_back(ops[group[k]].first->prepared.get());
+            for (int r = 0; r < b->rounds; ++r) memcpy(&uu[((size_t)k * b->rounds + r) * 8], q->u_in[r].val, 32);
+        }
+        ZKC(zk_g1_open_begin_batch(&b->handle, b->count, sc.data(), pr.data(), uu.data(), b->rounds, nullptr));
+        for (size_t k = 0; k < group.size(); ++k) {
+            Pending* q = ops[group[k]].second;
+            q->rounds = b->rounds;
+            q->batch = b;
+            q->batch_index = (int)k;
+            b->folded.push_back(std::move(q->folded));
+            done[group[k]] = true;
+        }
+    }
+}
 void Commitment::prepare_openings() const {
     if (prepared || size == 0) return;
     void* h = nullptr;
@@ -109,6 +157,23 @@ Commitment::Pending Commitment::open_begin(const FrTensor& t, const G1TensorJaco
     return p;
 }
 Fr_t Commitment::open_end(Pending& p, vector<G1Jacobian_t>& proof) {
+    if (p.batch) {
+        Pending::Batch& b = *p.batch;
+        const size_t npts = 3 * (size_t)b.rounds + 1;
+        if (!b.collected) {
+            b.pts.resize((size_t)b.count * npts);
+            b.finals.resize(b.count);
+            void* h = b.handle;
+            b.handle = nullptr;
+            b.collected = true;
+            ZKC(zk_g1_open_end_batch(h, b.pts[0].x.val, b.finals[0].val));
+            b.folded.clear();
+        }
+        proof.insert(proof.end(), b.pts.begin() + npts * p.batch_index, b.pts.begin() + npts * (p.batch_index + 1));
+        p.value = b.finals[p.batch_index];
+        p.batch.reset();
+        return p.value;
+    }
     if (!p.handle) return p.value;
     std::vector<G1Jacobian_t> pts(3 * (size_t)p.rounds + 1);
     void* h = p.handle;

@@ -36,6 +36,9 @@ class Commitment : public G1TensorJacobian {
         int rounds = 0;
         Fr_t value{{0, 0, 0, 0, 0, 0, 0, 0}};
         vector<Fr_t> u_in;                  // between open_fold and open_start: the challenges of the G1 recursion
+        struct Batch;                       // openings started as one job (open_start_batch) share its handle and results
+        std::shared_ptr<Batch> batch;
+        int batch_index = 0;
     };
     Pending open_begin(const FrTensor& t, const G1TensorJacobian& c, const vector<Fr_t>& u) const;
     // open_begin in its two steps: open_fold reduces the rows to the vector that is opened (a pass over the whole tensor
@@ -43,6 +46,9 @@ class Commitment : public G1TensorJacobian {
     // start afterwards: a fold queued behind another opening's G1 kernels waits for the registers they hold.
     Pending open_fold(const FrTensor& t, const G1TensorJacobian& c, const vector<Fr_t>& u) const;
     void open_start(Pending& p) const;
+    // open_start for several folded openings at once: those whose generators are prepared and agree in size and round
+    // count run as one device job each group (zk_g1_open_begin_batch), the rest one by one
+    static void open_start_batch(const std::vector<std::pair<const Commitment*, Pending*>>& ops);
     static Fr_t open_end(Pending& p, vector<G1Jacobian_t>& proof);
 
     // The generators' form for openings (zk_g1_open_prepare), made once and kept with this object: openings started

@@ -5,6 +5,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <deque>
 #include <random>
 
 #include "../../include/zkllm_hip.h"
@@ -29,6 +30,8 @@ struct Globals {
     std::vector<Fr_t> transcript;
     std::vector<G1Jacobian_t> transcript_g1;
     std::string proof_file;
+    unsigned long long drawn = 0;                                             // challenge elements drawn so far
+    std::deque<std::pair<unsigned long long, std::vector<Fr_t>>> draw_log;    // recent short draws with their positions
     Globals() {
         if (const char* m = getenv("ZKLLM_MATMUL")) matmul_mode = (string(m) == "generic") ? 1 : 0;
         if (const char* f = getenv("ZKLLM_PROOF_FILE")) { proof_file = f; recording = !proof_file.empty(); }
@@ -47,7 +50,7 @@ void ensure_seeded() {
 }
 }  // namespace
 
-void zk_seed_challenges(uint32_t seed) { G().mt.seed(seed); G().seeded = true; }
+void zk_seed_challenges(uint32_t seed) { G().mt.seed(seed); G().seeded = true; G().drawn = 0; G().draw_log.clear(); }
 void zk_set_matmul_mode(int mode) { G().matmul_mode = mode; }
 int zk_last_matmul_path() { return G().last_matmul_path; }
 void zk_transcript_begin() { G().transcript.clear(); G().transcript_g1.clear(); G().recording = true; }
@@ -82,15 +85,39 @@ ostream& operator<<(ostream& os, const Fr_t& x) {
 }
 
 // 8 raw mt19937 outputs per element, the last reduced mod the top limb of r (fr-tensor.cu:16-24)
-vector<Fr_t> random_vec(uint len) {
-    ensure_seeded();
-    std::mt19937& mt = G().mt;
-    vector<Fr_t> out(len);
-    for (uint i = 0; i < len; ++i) {
+static void draw_elements(std::mt19937& mt, vector<Fr_t>& out) {
+    for (size_t i = 0; i < out.size(); ++i) {
         for (int k = 0; k < 7; ++k) out[i].val[k] = (uint)mt();
         out[i].val[7] = (uint)mt() % 1944954707u;
     }
+}
+vector<Fr_t> random_vec(uint len) {
+    ensure_seeded();
+    Globals& g = G();
+    vector<Fr_t> out(len);
+    draw_elements(g.mt, out);
+    if (len >= 1 && len <= 64) {
+        g.draw_log.emplace_back(g.drawn, out);
+        if (g.draw_log.size() > 4096) g.draw_log.pop_front();
+    }
+    g.drawn += len;
     return out;
+}
+unsigned long long zk_challenge_position() { return G().drawn; }
+vector<Fr_t> zk_challenge_peek(unsigned long long ahead, uint len) {
+    ensure_seeded();
+    std::mt19937 mt = G().mt;          // a copy: the stream itself does not move
+    mt.discard(8ull * ahead);
+    vector<Fr_t> out(len);
+    draw_elements(mt, out);
+    return out;
+}
+bool zk_challenge_find(const vector<Fr_t>& v, unsigned long long* position) {
+    if (v.empty()) { *position = G().drawn; return true; }          // an empty draw sits anywhere
+    const auto& log = G().draw_log;
+    for (auto it = log.rbegin(); it != log.rend(); ++it)
+        if (it->second.size() == v.size() && std::memcmp(it->second.data(), v.data(), v.size() * sizeof(Fr_t)) == 0) { *position = it->first; return true; }
+    return false;
 }
 
 uint ceilLog2(uint num) {

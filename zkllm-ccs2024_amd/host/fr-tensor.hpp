@@ -18,6 +18,13 @@ ostream& operator<<(ostream& os, const Fr_t& x);
 // (zk_seed_challenges, or ZKLLM_SEED in the environment) so that transcripts are reproducible.
 void zk_seed_challenges(uint32_t seed);
 vector<Fr_t> random_vec(uint len);
+// The stream is position-addressable (eight raw generator outputs per element, whatever their values):
+// zk_challenge_position counts the elements drawn so far, zk_challenge_peek returns the `len` elements that start
+// `ahead` elements from here without drawing them, zk_challenge_find tells at which position a vector drawn
+// recently (at most 64 elements long, among the last few thousand draws) began.
+unsigned long long zk_challenge_position();
+vector<Fr_t> zk_challenge_peek(unsigned long long ahead, uint len);
+bool zk_challenge_find(const vector<Fr_t>& v, unsigned long long* position);
 uint ceilLog2(uint num);
 
 template <typename T>

@@ -42,6 +42,11 @@ void zkp_transcript_begin() { zk_transcript_begin(); }
 void zkp_transcript_end() { zk_transcript_end(); }
 long zkp_transcript_size() { return (long)zk_transcript().size(); }
 void zkp_transcript_get(u32* out) { if (!zk_transcript().empty()) memcpy(out, zk_transcript().data(), zk_transcript().size() * 32); }
+long zkp_transcript_g1_size() { return (long)zk_transcript_g1().size(); }
+void zkp_transcript_g1_get(u32* out) { if (!zk_transcript_g1().empty()) memcpy(out, zk_transcript_g1().data(), zk_transcript_g1().size() * sizeof(G1Jacobian_t)); }
+// position of the challenge stream (elements drawn since it was seeded) and a way to move it on without using the draws
+unsigned long long zkp_challenge_position() { return zk_challenge_position(); }
+void zkp_challenge_skip(unsigned long long n) { while (n) { const uint c = n > 65536 ? 65536u : (uint)n; (void)random_vec(c); n -= c; } }
 int zkp_sync() { ZKP_TRY zk_check(zk_sync(nullptr), "zk_sync"); ZKP_END }
 void zkp_random_vec(u32* out, u32 len) { auto v = random_vec(len); if (len) memcpy(out, v.data(), (size_t)len * 32); }
 
@@ -473,6 +478,7 @@ void* zkp_layer_create(const u32* cu, const double* cf, const int32_t* norm1, co
         FrTensor weight(in_dim * out_dim, (const int*)p);
         Commitment gen = Commitment::random(1u << ceilLog2(pp));
         G1TensorJacobian com = gen.commit_int(weight.pad({in_dim, out_dim}));
+        gen.prepare_openings();
         return Weight{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim};
     };
     // same order of generator draws as the oracle: norm1, q, k, v, o, norm2, up, gate, down
@@ -492,6 +498,8 @@ void* zkp_layer_create_random(const u32* cu, const double* cf, u32 seed, u32 log
 void zkp_layer_free(void* h) { delete reinterpret_cast<LayerState*>(h); }
 void zkp_layer_set_head_group(void* h, u32 g) { reinterpret_cast<LayerState*>(h)->cfg.attn_head_group = g; }
 void zkp_layer_set_open_weights(void* h, int on) { reinterpret_cast<LayerState*>(h)->cfg.open_weights = on != 0; }
+// openings of the layer whose points are known ahead (0 until the first run with weight openings has finished)
+int zkp_layer_planned_openings(void* h) { const LayerState& s = *reinterpret_cast<LayerState*>(h); return s.w.plan && s.w.plan->learned ? (int)s.w.plan->entries.size() : 0; }
 // runs the whole layer (compute + every proof); times_ms (8 values): rmsnorm1, qkv, attention, oproj, rmsnorm2, ffn, total, open_wait
 void* zkp_layer_run(void* h, void* X, double* times_ms) {
     ZKP_TRY

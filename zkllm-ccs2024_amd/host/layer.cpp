@@ -380,7 +380,8 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
 
 FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor& X, LayerTimes* times) {
     LayerTimes t;
-    DeferredOpenings openings;       // the nine weight openings run on the device beside the sumchecks
+    static const bool ahead_off = [] { const char* e = getenv("ZKLLM_OPEN_AHEAD"); return e && e[0] == '0'; }();
+    DeferredOpenings openings(c.open_weights && !ahead_off ? w.plan.get() : nullptr);       // the nine weight openings run on the device beside the sumchecks
     const double t0 = now_ms();
     FrTensor rms1 = compute_rms_inv(X, c.seq_len, c.embed_dim, c.rms_eps, c.value_scale);
     FrTensor n1 = rmsnorm_block(c, w.input_norm, X, rms1);

@@ -51,6 +51,9 @@ void layer_config_from_env(LayerConfig& c);
 struct LayerWeights {
     Weight input_norm, q, k, v, o, post_norm, up, gate, down;
     FrTensor swiglu_table;        // swiglu_len mapped values
+    // where the nine opening points sit in the challenge stream, learned by the first llama_layer over these weights;
+    // later runs start every opening when the layer starts (OpeningPlan in proof.hpp).  ZKLLM_OPEN_AHEAD=0 turns it off.
+    std::shared_ptr<OpeningPlan> plan = std::make_shared<OpeningPlan>();
 };
 
 struct LayerTimes {               // milliseconds, wall clock with the caller's stream idle at both ends; weight openings run beside the blocks,

@@ -1,3 +1,5 @@
+#include <chrono>
+#include <algorithm>
 #include <memory>
 #include "proof.hpp"
 
@@ -11,16 +13,55 @@ struct DeferredOpenings::Item {
     Fr_t claim;
     size_t slot;
 };
+struct DeferredOpenings::Ahead {
+    Commitment::Pending op;
+    const Weight* w;
+    vector<Fr_t> u_cat;
+};
 static thread_local DeferredOpenings* g_deferred = nullptr;
+static const FrTensor& padded_form(const Weight& w, std::unique_ptr<FrTensor>& local);
 DeferredOpenings::DeferredOpenings() : prev(g_deferred) { g_deferred = this; }
+DeferredOpenings::DeferredOpenings(OpeningPlan* pl) : prev(g_deferred), plan(pl) {
+    g_deferred = this;
+    if (!plan) return;
+    base = zk_challenge_position();
+    if (!plan->learned) { learning = true; plan->entries.clear(); return; }
+    // every opening of the plan: rows folded first (the folds are passes over whole weights on the caller's stream), then
+    // the G1 recursions queued
+    try {
+        for (const OpeningPlan::Entry& e : plan->entries) {
+            Ahead* a = new Ahead;
+            ahead.push_back(a);
+            a->w = e.w;
+            a->u_cat = concatenate(vector<vector<Fr_t>>({zk_challenge_peek(e.pos[1], e.len[1]), zk_challenge_peek(e.pos[0], e.len[0])}));
+            std::unique_ptr<FrTensor> local;
+            a->op = e.w->generator.open_fold(padded_form(*e.w, local), e.w->com, a->u_cat);
+        }
+        // the longest recursions first; openings of one size run as one job
+        std::vector<Ahead*> order(ahead);
+        std::stable_sort(order.begin(), order.end(), [](const Ahead* x, const Ahead* y) { return x->w->generator.size > y->w->generator.size; });
+        std::vector<std::pair<const Commitment*, Commitment::Pending*>> ops;
+        for (Ahead* a : order) ops.emplace_back(&a->w->generator, &a->op);
+        Commitment::open_start_batch(ops);
+    } catch (...) {
+        for (Ahead* a : ahead) { try { vector<G1Jacobian_t> drop; Commitment::open_end(a->op, drop); } catch (...) {} delete a; }
+        ahead.clear();
+        g_deferred = prev;
+        throw;
+    }
+}
 DeferredOpenings::~DeferredOpenings() {
     g_deferred = prev;
+    for (Ahead* a : ahead) {          // started from the plan and never claimed
+        if (a) { try { vector<G1Jacobian_t> drop; Commitment::open_end(a->op, drop); } catch (...) {} delete a; }
+    }
     for (Item* it : items) {          // only reached with pending items when an exception unwinds: release them
         try { vector<G1Jacobian_t> drop; Commitment::open_end(it->op, drop); } catch (...) {}
         delete it;
     }
 }
 void DeferredOpenings::finish() {
+    if (learning && plan) { plan->learned = true; learning = false; }
     std::vector<Item*> todo;
     todo.swap(items);
     std::string failure;
@@ -49,13 +90,39 @@ static const FrTensor& padded_form(const Weight& w, std::unique_ptr<FrTensor>& l
     local.reset(new FrTensor(w.weight.pad({w.in_dim, w.out_dim})));
     return *local;
 }
+// while a plan is being learned: where this opening's point was drawn; a point that is not two recent draws ends the
+// learning (nothing runs ahead then)
+void DeferredOpenings::learn(const Weight& w, const Claim& c) {
+    if (!learning) return;
+    OpeningPlan::Entry e{&w, {0, 0}, {0, 0}};
+    if (c.u.size() == 2 && zk_challenge_find(c.u[0], &e.pos[0]) && zk_challenge_find(c.u[1], &e.pos[1]) && e.pos[0] >= base && e.pos[1] >= base) {
+        e.len[0] = (uint)c.u[0].size(); e.len[1] = (uint)c.u[1].size();
+        e.pos[0] -= base; e.pos[1] -= base;
+        plan->entries.push_back(e);
+    } else { learning = false; plan->entries.clear(); }
+}
 void verifyWeightClaim(const Weight& w, const Claim& c) {
     vector<Fr_t> u_cat = concatenate(vector<vector<Fr_t>>({c.u[1], c.u[0]}));
     std::unique_ptr<FrTensor> local;
     const FrTensor& w_padded = padded_form(w, local);
     if (g_deferred) {
+        DeferredOpenings& d = *g_deferred;
+        const size_t k = d.next++;
+        d.learn(w, c);
+        if (k < d.ahead.size() && d.ahead[k]) {
+            DeferredOpenings::Ahead* a = d.ahead[k];
+            d.ahead[k] = nullptr;
+            if (a->w == &w && a->u_cat == u_cat) {
+                d.items.push_back(new DeferredOpenings::Item{std::move(a->op), c.claim, zk_record_reserve()});
+                delete a;
+                return;
+            }
+            try { vector<G1Jacobian_t> drop; Commitment::open_end(a->op, drop); } catch (...) {}      // not the planned opening: dropped
+            delete a;
+            d.plan->learned = false;          // the plan does not describe this sequence: learn it again next time
+        }
         DeferredOpenings::Item* it = new DeferredOpenings::Item{w.generator.open_begin(w_padded, w.com, u_cat), c.claim, zk_record_reserve()};
-        g_deferred->items.push_back(it);
+        d.items.push_back(it);
         return;
     }
     vector<G1Jacobian_t> g1_proof;
@@ -80,7 +147,7 @@ WeightOpeningAhead::~WeightOpeningAhead() {
 }
 WeightOpeningAhead openWeightAhead(const Weight& w, const vector<Fr_t>& u_input, const vector<Fr_t>& u_output) {
     WeightOpeningAhead a;
-    if (!g_deferred) return a;            // nothing runs ahead outside a deferred scope
+    if (!g_deferred || !g_deferred->ahead.empty()) return a;            // nothing runs ahead outside a deferred scope
     a.impl = new WeightOpeningAhead::Impl;
     a.impl->u_cat = concatenate(vector<vector<Fr_t>>({u_output, u_input}));
     std::unique_ptr<FrTensor> local;
@@ -90,19 +157,23 @@ WeightOpeningAhead openWeightAhead(const Weight& w, const vector<Fr_t>& u_input,
 std::vector<WeightOpeningAhead> openWeightsAhead(const std::vector<const Weight*>& ws, const std::vector<const std::vector<Fr_t>*>& u_inputs,
                                                  const std::vector<const std::vector<Fr_t>*>& u_outputs) {
     std::vector<WeightOpeningAhead> out(ws.size());
-    if (!g_deferred) return out;
+    if (!g_deferred || !g_deferred->ahead.empty()) return out;      // a scope that runs from a plan has started them already
     for (size_t i = 0; i < ws.size(); ++i) {
         out[i].impl = new WeightOpeningAhead::Impl;
         out[i].impl->u_cat = concatenate(vector<vector<Fr_t>>({*u_outputs[i], *u_inputs[i]}));
         std::unique_ptr<FrTensor> local;
         out[i].impl->op = ws[i]->generator.open_fold(padded_form(*ws[i], local), ws[i]->com, out[i].impl->u_cat);
     }
-    for (size_t i = 0; i < ws.size(); ++i) ws[i]->generator.open_start(out[i].impl->op);
+    std::vector<std::pair<const Commitment*, Commitment::Pending*>> ops;
+    for (size_t i = 0; i < ws.size(); ++i) ops.emplace_back(&ws[i]->generator, &out[i].impl->op);
+    Commitment::open_start_batch(ops);
     return out;
 }
 void verifyWeightClaim(const Weight& w, const Claim& c, WeightOpeningAhead& ahead) {
     if (!ahead.impl || !g_deferred) { verifyWeightClaim(w, c); return; }
     if (ahead.impl->u_cat != concatenate(vector<vector<Fr_t>>({c.u[1], c.u[0]}))) throw std::runtime_error("verifyWeightClaim: the opening started ahead is at another point");
+    g_deferred->next++;
+    g_deferred->learn(w, c);
     DeferredOpenings::Item* it = new DeferredOpenings::Item{std::move(ahead.impl->op), c.claim, zk_record_reserve()};
     g_deferred->items.push_back(it);
     delete ahead.impl;

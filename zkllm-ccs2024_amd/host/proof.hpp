@@ -34,9 +34,21 @@ void verifyWeightClaim(const Weight& w, const Claim& c, WeightOpeningAhead& ahea
 // While a DeferredOpenings object is alive, verifyWeightClaim only starts each opening (it runs on the device beside
 // the rest of the proof) and finish() waits for all of them, checks every claim and throws as verifyWeightClaim does.
 // The transcript keeps the position of each opened value.
+// Where in the challenge stream the opening points of a fixed sequence of weight openings are drawn, relative to the
+// start of that sequence (a decoder layer: nine openings).  The challenges come from a seeded generator and not from the
+// transcript, as in the reference (fr-tensor.cu:16-24), so a point that will be drawn later is already determined: a
+// DeferredOpenings scope with a learned plan starts every opening at once, beside everything the prover does before
+// it reaches that weight, and verifyWeightClaim finds it running.  The first scope with an empty plan fills it in.  An
+// opening whose point or weight turns out different from the plan's is dropped and opened where the reference opens it.
+struct OpeningPlan {
+    struct Entry { const Weight* w; unsigned long long pos[2]; uint len[2]; };      // Claim::u[0], u[1]: offsets from the scope's start
+    std::vector<Entry> entries;
+    bool learned = false;
+};
 class DeferredOpenings {
    public:
     DeferredOpenings();
+    explicit DeferredOpenings(OpeningPlan* plan);
     ~DeferredOpenings();
     void finish();
     DeferredOpenings(const DeferredOpenings&) = delete;
@@ -46,6 +58,15 @@ class DeferredOpenings {
     struct Item;
     std::vector<Item*> items;
     DeferredOpenings* prev;
+    OpeningPlan* plan = nullptr;
+    bool learning = false;
+    unsigned long long base = 0;          // stream position at the start of the scope
+    struct Ahead;
+    std::vector<Ahead*> ahead;            // openings started from the plan, in the plan's order
+    size_t next = 0;                      // index of the next verifyWeightClaim within the scope
+    void learn(const Weight& w, const Claim& c);
+    friend WeightOpeningAhead openWeightAhead(const Weight& w, const std::vector<Fr_t>& u_input, const std::vector<Fr_t>& u_output);
+    friend std::vector<WeightOpeningAhead> openWeightsAhead(const std::vector<const Weight*>&, const std::vector<const std::vector<Fr_t>*>&, const std::vector<const std::vector<Fr_t>*>&);
     friend void verifyWeightClaim(const Weight& w, const Claim& c);
     friend void verifyWeightClaim(const Weight& w, const Claim& c, WeightOpeningAhead& ahead);
 };
