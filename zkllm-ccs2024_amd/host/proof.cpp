@@ -40,6 +40,18 @@ DeferredOpenings::DeferredOpenings(OpeningPlan* pl) : prev(g_deferred), plan(pl)
         // the longest recursions first; openings of one size run as one job
         std::vector<Ahead*> order(ahead);
         std::stable_sort(order.begin(), order.end(), [](const Ahead* x, const Ahead* y) { return x->w->generator.size > y->w->generator.size; });
+        // The library runs the jobs on two pairs of streams in turn.  The group of the shortest recursions (all latency, hardly any
+        // work) goes second: it runs beside the first long job, and the second long job follows the first on its pair of streams.
+        if (order.size() > 2) {
+            const uint smallest = order.back()->w->generator.size, largest = order.front()->w->generator.size;
+            if (smallest != largest) {
+                std::vector<Ahead*> big, mid, small;
+                for (Ahead* a : order) (a->w->generator.size == largest ? big : (a->w->generator.size == smallest ? small : mid)).push_back(a);
+                order = big;
+                order.insert(order.end(), small.begin(), small.end());
+                order.insert(order.end(), mid.begin(), mid.end());
+            }
+        }
         std::vector<std::pair<const Commitment*, Commitment::Pending*>> ops;
         for (Ahead* a : order) ops.emplace_back(&a->w->generator, &a->op);
         Commitment::open_start_batch(ops);
