@@ -6,10 +6,12 @@ GPU with weights, generators, commitments and the input already resident in HBM:
 projections, 32 attention heads (QK^T, zkSoftmax, YV), SwiGLU FFN, every rescaling / lookup / sumcheck and
 the opening of all nine weight commitments.  `value` is seconds per layer.
 
-The same JSON line also carries the two throughput figures of the headline metric (G1 MSM points/s on the
-4096 x 11008 commitment workload, Fr multiplications/s), a roofline entry for the kernel with the largest share
-of the layer's GPU time (timed with HIP events around its launches inside the timed region), roofline entries of
-the generic Fr matmul and of an HBM-bound fold, and a CPU baseline measured with the oracle on this host's cores.
+The same JSON line also carries the layer time without the openings and with the nine commitments included, the
+two throughput figures of the headline metric (G1 MSM points/s on the 4096 x 11008 commitment workload, Fr
+multiplications/s) with their roofline fractions, a roofline entry for the kernel with the largest share of the
+layer's GPU time (timed with HIP events around its launches inside the timed region), roofline entries of the first
+lookup-sumcheck round, the generic Fr matmul and an HBM-bound fold, and a CPU baseline measured with the oracle on
+this host's cores.
 """
 import argparse
 import ctypes
@@ -28,10 +30,14 @@ HBM_PEAK_GBS = 8000.0
 # VALU integer peak: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz lane-operations per second (v_mad_u64_u32 issues at
 # full rate on gfx950; bench measures it as well and reports the measured figure next to this one)
 VALU_PEAK_TOPS = 256 * 4 * 16 * 2.4e9 / 1e12
-# HBM traffic of k_open_fold per generator pair, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the kernel alone
-# (python3 bench.py --pmc-probe; summary in profiles/k_open_fold_pmc_traffic.txt), each counter scaled by what it reads for
-# zk_fr_add over 2^24 elements (1 GiB read, 512 MiB written)
-FOLD_TRAFFIC_BYTES_PER_PAIR = 2551.0
+# HBM traffic of k_open_fold29 per generator pair in a launch of 262144 pairs, measured with rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE on the kernel alone (python3 bench.py --pmc-probe; summary in profiles/k_open_fold29_pmc_traffic.txt), each
+# counter scaled by what it reads for zk_fr_add over 2^24 elements (1 GiB read, 512 MiB written).  It holds for launches of
+# that size; `traffic` of the in-layer entry, whose launches are of every size, is left null and the algorithmic figure given.
+FOLD_TRAFFIC_BYTES_PER_PAIR_AT_262144 = 618.0
+FOLD_ALGO_BYTES_PER_PAIR = 2 * 112 + 112 + 3 * 32      # two points in, one out (affine, 29-bit limbs: 112 B), two scalars in, one out
+MAD_PER_FP_MUL = 300                                   # 2 * 12^2 + 12 limb products of a 381-bit Montgomery product
+MAD_PER_FR_MUL = 136                                   # 2 * 8^2 + 8
 
 
 def main():
@@ -46,7 +52,8 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extras", action="store_true", help="only the layer timing (used for profiling runs)")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="for rocprofv3 --pmc runs: only three launches of the opening's fold kernel at 262144 pairs and one "
+                    help="for rocprofv3 --pmc runs: three launches of the opening's fold kernel at 262144 pairs, one hinted lookup "
+                         "sumcheck over 2^27 queries, the Montgomery product, the three-level fold, the commitment of config 3 and one "
                          "zk_fr_add over 2^24 elements (1 GiB read, 512 MiB written) to scale the counters by")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -62,7 +69,7 @@ def main():
     hip = Hip()
     lib = hip.lib
 
-    if args.pmc_probe:
+    def fold_probe_setup():
         n_big = 1 << 19
         pv.seed(6)
         gens_big = pv.commitment_random(n_big)
@@ -72,13 +79,31 @@ def main():
         ns, ng = hip.malloc(32 * (n_big // 2)), hip.malloc(144 * (n_big // 2))
         u1 = mt_random_vec(np.random.RandomState(9), 1)
         sums3 = np.zeros((3, 36), np.uint32)
+        run = lambda: hip.call("zk_g1_open_round", c_void_p(ns), c_void_p(ng), sums3, c_void_p(sc), c_void_p(gp), u1, c_size_t(n_big), None)
+        return n_big, gens_big, (sc, ns, ng), run
+
+    def lookup_probe(logD=27, logN=20):
+        """one mapping-table lookup proof (tLookupRangeMapping::prove) over 2^logD uniformly spread queries into 2^logN entries"""
+        D, N = 1 << logD, 1 << logN
+        rng = np.random.default_rng(1)
+        low = -(N // 2)
+        S = pv.from_i32((rng.integers(0, N, D, dtype=np.int64) + low).astype(np.int32))
+        mv = pv.from_i32(rng.integers(0, 1 << 22, N, dtype=np.int64).astype(np.int32))
+        rs = np.random.RandomState(3)
+        r, al, be = mt_random_vec(rs, 1), mt_random_vec(rs, 1), mt_random_vec(rs, 1)
+        u, v = mt_random_vec(rs, logD), mt_random_vec(rs, logD)
+        return (lambda: pv.mapping(S, low, N, mv, r, al, be, u, v)), (S, mv)
+
+    if args.pmc_probe:
+        n_big, gens_big, bufs, fold_round = fold_probe_setup()
         for _ in range(3):
-            hip.call("zk_g1_open_round", c_void_p(ns), c_void_p(ng), sums3, c_void_p(sc), c_void_p(gp), u1, c_size_t(n_big), None)
+            fold_round()
         n = 1 << 24
         dA, dB, dO = hip.malloc(32 * n), hip.malloc(32 * n), hip.malloc(32 * n)
         hip.call("zk_fr_add", c_void_p(dO), c_void_p(dA), c_void_p(dB), c_size_t(n), None)
         # the kernels behind the other reported rates, once each on operands of known size: the Montgomery product
-        # (Fr mul/s), the fused three-level fold (HBM GB/s) and the commitment of the 11008 x 4096 weight (MSM points/s)
+        # (Fr mul/s), the fused three-level fold (HBM GB/s), the commitment of the 11008 x 4096 weight (MSM points/s)
+        # and the hinted first round of a lookup sumcheck
         seed_block = mt_random_vec(np.random.RandomState(1), 1 << 16)
         src = hip.upload(seed_block)
         for i in range(n >> 16):
@@ -91,10 +116,13 @@ def main():
         gens = pv.commitment_random(4096)
         Wm = np.round(np.random.default_rng(12).normal(0, 0.02, (11008, 4096)) * 65536).astype(np.int32)
         com = pv.commit_int(gens, pv.from_i32(Wm))
+        look, keep = lookup_probe()
+        y, m, fin = look()
         hip.sync()
         print(json.dumps({"pmc_probe": {"fold_pairs_per_launch": n_big // 2, "fold_launches": 3, "copy_kernel": "k_ew<0> (zk_fr_add)",
                                         "copy_read_bytes": 64 * n, "copy_write_bytes": 32 * n, "montmul_elements": n,
-                                        "fold_axis_elements_in": 2048 * 4096, "msm_pairs": 11008 * 4096}}))
+                                        "fold_axis_elements_in": 2048 * 4096, "msm_pairs": 11008 * 4096,
+                                        "lookup_first_round_pairs": 1 << 26, "lookup_first_round_algorithmic_bytes": (1 << 26) * 240}}))
         return
 
     def ev():
@@ -115,6 +143,16 @@ def main():
         hip.check(lib.zk_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
         return ms.value / reps
 
+    def read_fold_timer():
+        fold_ms, fold_launches, fold_mults, fold_pairs = ctypes.c_double(), ctypes.c_ulonglong(), ctypes.c_double(), ctypes.c_ulonglong()
+        hip.check(lib.zk_prof_fold_read(ctypes.byref(fold_ms), ctypes.byref(fold_launches), ctypes.byref(fold_mults), ctypes.byref(fold_pairs)))
+        return fold_ms.value, fold_launches.value, fold_mults.value, fold_pairs.value
+
+    def read_lookup_timer():
+        ms, launches, pairs, nbytes = ctypes.c_double(), ctypes.c_ulonglong(), ctypes.c_ulonglong(), ctypes.c_double()
+        hip.check(lib.zk_prof_lookup_read(ctypes.byref(ms), ctypes.byref(launches), ctypes.byref(pairs), ctypes.byref(nbytes)))
+        return ms.value, launches.value, pairs.value, nbytes.value
+
     # ---- workload: the decoder layer ------------------------------------------------------------------------------
     seq = args.seq
     cu, cf = layercfg.llama7b(seq=seq, open_weights=True, head_group=args.head_group)
@@ -123,6 +161,8 @@ def main():
     layer = pv.layer_create_random(cu, cf, 7, 5)
     pv.sync()
     setup_s = time.perf_counter() - t0
+    setup4 = np.zeros(4)
+    pv.lib.zkp_layer_setup_times(setup4.ctypes.data_as(ctypes.POINTER(ctypes.c_double)))
     X = np.round(np.random.default_rng(11).normal(0, 1, (seq, 4096)) * 65536).astype(np.int32)
     hX = pv.from_i32(X)
     devnull = os.open(os.devnull, os.O_WRONLY)
@@ -134,14 +174,30 @@ def main():
             pv.layer_run(layer, hX)
         pv.sync()
         hip.check(lib.zk_prof_fold_begin())
+        hip.check(lib.zk_prof_lookup_begin())
         t0 = time.perf_counter()
         for _ in range(args.steps):
             _, times = pv.layer_run(layer, hX)
             parts += times
         pv.sync()
         wall = time.perf_counter() - t0
-        fold_ms, fold_launches, fold_mults, fold_pairs = ctypes.c_double(), ctypes.c_ulonglong(), ctypes.c_double(), ctypes.c_ulonglong()
-        hip.check(lib.zk_prof_fold_read(ctypes.byref(fold_ms), ctypes.byref(fold_launches), ctypes.byref(fold_mults), ctypes.byref(fold_pairs)))
+        fold_ms, fold_launches, fold_mults, fold_pairs = read_fold_timer()
+        lk_ms, lk_launches, lk_pairs, lk_bytes = read_lookup_timer()
+        # the same layer without its nine openings (the G1 part of verifyWeightClaim switched off), and the nine commitments alone
+        noopen_s = commit_ms = None
+        if not args.skip_extras:
+            pv.layer_set(layer, open_weights=False)
+            pv.layer_run(layer, hX)
+            pv.sync()
+            t1 = time.perf_counter()
+            for _ in range(2):
+                pv.layer_run(layer, hX)
+            pv.sync()
+            noopen_s = (time.perf_counter() - t1) / 2
+            pv.layer_set(layer, open_weights=True)
+            pv.lib.zkp_layer_recommit_ms.restype = ctypes.c_double
+            commit_ms = pv.lib.zkp_layer_recommit_ms(c_void_p(layer))
+            commit_ms = pv.lib.zkp_layer_recommit_ms(c_void_p(layer))      # second call: the tables' buffers are cached blocks now
     finally:
         os.dup2(saved_stdout, 1)
     ms_per_step = wall * 1e3 / args.steps
@@ -166,56 +222,63 @@ def main():
         "dtype": "u32",
         "data": "synthetic",
         "config": {"workload": f"C5: LLaMa-2-7B-shape decoder layer proof, seq {seq}, hidden 4096, 32 heads x 128, FFN 11008, "
-                               "random-init fixed-point weights (scale 2^16), generators of size out_features<<5, all nine weight openings included; attention proved "
+                               "random-init fixed-point weights (scale 2^16), generators of size out_features<<5, all nine weight openings included "
+                               "(their points are read ahead from the seeded challenge stream, so all nine run from the start of the layer, batched by "
+                               "generator size); attention proved "
                                + (f"{args.head_group} heads at a time as head-major stacks (zkAttnStacked)" if args.head_group else "head by head"),
                    "device_pool_gib": round(pool_gib, 1),
                    "setup_s_untimed": round(setup_s, 3),
-                   "parts_ms": {k: round(float(v), 1) for k, v in zip(["rmsnorm1", "qkv", "attention", "oproj", "rmsnorm2", "ffn", "total", "open_wait"], parts)}},
+                   "setup_parts_s": {"random_weights_host_and_upload": round(setup4[0] / 1e3, 3), "generators": round(setup4[1] / 1e3, 3),
+                                     "commitments": round(setup4[2] / 1e3, 3), "generators_prepared_for_openings": round(setup4[3] / 1e3, 3)},
+                   "parts_ms": {k: round(float(v), 1) for k, v in zip(["rmsnorm1", "qkv", "attention", "oproj", "rmsnorm2", "ffn", "total", "open_wait"], parts)},
+                   "parts_note": "host-side block times; the openings run on the library's streams from the start of the layer, so the first blocks' "
+                                 "figures include the time their kernels share the device with them"},
     }
+    if noopen_s is not None:
+        out["layer_without_openings_s"] = noopen_s
+        out["commitments_s"] = commit_ms / 1e3
+        out["layer_with_commitments_s"] = ms_per_step / 1e3 + commit_ms / 1e3
     # roofline of the kernel with the largest share of the layer's GPU time: the generator fold of the openings
     # (one endomorphism-split scalar multiplication per pair).  It is bound by 32-bit integer multiply-adds: an
     # Fp multiplication is 2*12^2+12 = 300 of them.  Durations are HIP events around every launch inside the timed
     # region above, on the launch stream.
-    MAD_PER_FP_MUL = 300
-    fold_tops = fold_mults.value * MAD_PER_FP_MUL / (fold_ms.value * 1e-3) / 1e12 if fold_ms.value > 0 else 0.0
-    out["roofline"] = {"kernel": "k_open_fold (opening: g' = g1 + [u](g0 - g1) per pair, 128-bit split scalars)", "bound": "valu-int",
-                       "achieved": fold_tops, "peak": VALU_PEAK_TOPS, "unit": "T MAD32/s", "frac": fold_tops / VALU_PEAK_TOPS,
-                       "traffic": FOLD_TRAFFIC_BYTES_PER_PAIR * fold_pairs.value / max(1, fold_launches.value),
-                       "launches": int(fold_launches.value), "avg_launch_ms": fold_ms.value / max(1, fold_launches.value),
-                       "total_ms_in_timed_region": fold_ms.value, "pairs": int(fold_pairs.value), "fp_mul_per_s": fold_mults.value / (fold_ms.value * 1e-3) if fold_ms.value > 0 else 0.0,
+    fold_tops = fold_mults * MAD_PER_FP_MUL / (fold_ms * 1e-3) / 1e12 if fold_ms > 0 else 0.0
+    out["roofline"] = {"kernel": "k_open_fold29 (opening: g' = g1 + [u](g0 - g1) per pair, 128-bit split scalars; one launch per round for all openings of a size)",
+                       "bound": "valu-int", "achieved": fold_tops, "peak": VALU_PEAK_TOPS, "unit": "T MAD32/s", "frac": fold_tops / VALU_PEAK_TOPS,
+                       "traffic": None, "algorithmic_bytes_per_launch": FOLD_ALGO_BYTES_PER_PAIR * fold_pairs / max(1, fold_launches),
+                       "launches": int(fold_launches), "avg_launch_ms": fold_ms / max(1, fold_launches),
+                       "total_ms_in_timed_region": fold_ms, "pairs": int(fold_pairs), "fp_mul_per_s": fold_mults / (fold_ms * 1e-3) if fold_ms > 0 else 0.0,
                        "note": "algorithmic work = Fp multiplications of the point formulas x 300 MAD32 (12-limb schoolbook product and reduction; the kernel "
                                "itself works on 14 limbs of 29 bits: 392 multiply-adds and ~110 other instructions per product, 301 per square); "
-                               "peak = 256 CU x 4 SIMD x 16 lanes x 2.4 GHz.  traffic = measured bytes per pair (rocprofv3 FETCH_SIZE + WRITE_SIZE of the kernel alone, "
-                               "profiles/k_open_fold_pmc_traffic.txt) x the average pairs per launch; algorithmic traffic is 336 B per pair.  The average covers every "
-                               "launch of the timed region: most are short rounds (one wave per SIMD or less) that run beside the rest of the proof"}
+                               "peak = 256 CU x 4 SIMD x 16 lanes x 2.4 GHz.  The launches are of every size (524288 pairs in the first round of the "
+                               "two 2^19 openings down to 2048 in the last halving round) and run beside the bucket sums of their own job and beside "
+                               "the rest of the proof; traffic was measured for the kernel alone at 262144 pairs (roofline_fold_alone)"}
+    if lk_launches:
+        out["roofline_lookup_round_in_layer"] = {
+            "kernel": "k_lookup_round<false,true> (first round of the hinted lookup sumchecks, every launch of the timed layers)", "bound": "hbm",
+            "achieved": lk_bytes / (lk_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": lk_bytes / (lk_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "traffic": None, "launches": int(lk_launches), "pairs": int(lk_pairs), "total_ms_in_timed_region": lk_ms,
+            "note": "algorithmic bytes (per pair: the two queries, 32 B each or 64 B for a mapping table's two tensors; the eq weight 32 B; two folded "
+                    "values out 64 B; the next round's eq table 16 B) over the summed launch durations; the launches share the device with each other"}
     if args.skip_extras:
         print(json.dumps(out))
         return
 
-    # ---- the same fold kernel alone at its largest shape in the layer: one halving of 2^19 generators (the FFN weights' opening) ----
-    pv.seed(6)
-    n_big = 1 << 19
-    gens_big = pv.commitment_random(n_big)
-    pv.lib.zkp_g1_devptr.restype = ctypes.c_void_p
-    gp = pv.lib.zkp_g1_devptr(c_void_p(gens_big.h))
-    sc = hip.upload(mt_random_vec(np.random.RandomState(8), n_big))
-    ns, ng = hip.malloc(32 * (n_big // 2)), hip.malloc(144 * (n_big // 2))
-    u1 = mt_random_vec(np.random.RandomState(9), 1)
-    sums3 = np.zeros((3, 36), np.uint32)
-    hip.call("zk_g1_open_round", c_void_p(ns), c_void_p(ng), sums3, c_void_p(sc), c_void_p(gp), u1, c_size_t(n_big), None)
+    # ---- the same fold kernel alone at its largest per-opening shape in the layer: one halving of 2^19 generators ----
+    n_big, gens_big, bufs, fold_round = fold_probe_setup()
+    fold_round()
     hip.check(lib.zk_prof_fold_begin())
     for _ in range(3):
-        hip.call("zk_g1_open_round", c_void_p(ns), c_void_p(ng), sums3, c_void_p(sc), c_void_p(gp), u1, c_size_t(n_big), None)
-    hip.check(lib.zk_prof_fold_read(ctypes.byref(fold_ms), ctypes.byref(fold_launches), ctypes.byref(fold_mults), ctypes.byref(fold_pairs)))
-    iso_tops = fold_mults.value * MAD_PER_FP_MUL / (fold_ms.value * 1e-3) / 1e12
-    out["roofline_fold_alone"] = {"kernel": "k_open_fold, 262144 pairs, nothing else on the device", "bound": "valu-int", "achieved": iso_tops, "peak": VALU_PEAK_TOPS,
-                                  "unit": "T MAD32/s", "frac": iso_tops / VALU_PEAK_TOPS, "traffic": FOLD_TRAFFIC_BYTES_PER_PAIR * (n_big // 2),
-                                  "avg_launch_ms": fold_ms.value / max(1, fold_launches.value),
-                                  "fp_mul_per_s": fold_mults.value / (fold_ms.value * 1e-3),
-                                  "note": "4096 waves on 2048 wave slots (two per SIMD: 250 registers, most of the walk's table in LDS): two full turns.  traffic: FETCH_SIZE + "
-                                          "WRITE_SIZE of this launch from profiles/k_open_fold_pmc_traffic.txt, against 336 B per pair of algorithmic traffic (the rest is "
-                                          "private memory of the out-of-line special cases)"}
-    for p_ in (sc, ns, ng):
+        fold_round()
+    f_ms, f_launches, f_mults, f_pairs = read_fold_timer()
+    iso_tops = f_mults * MAD_PER_FP_MUL / (f_ms * 1e-3) / 1e12
+    out["roofline_fold_alone"] = {"kernel": "k_open_fold29, 262144 pairs, nothing else on the device", "bound": "valu-int", "achieved": iso_tops,
+                                  "peak": VALU_PEAK_TOPS, "unit": "T MAD32/s", "frac": iso_tops / VALU_PEAK_TOPS,
+                                  "traffic": FOLD_TRAFFIC_BYTES_PER_PAIR_AT_262144 * (n_big // 2), "algorithmic_bytes_per_launch": FOLD_ALGO_BYTES_PER_PAIR * (n_big // 2),
+                                  "avg_launch_ms": f_ms / max(1, f_launches), "fp_mul_per_s": f_mults / (f_ms * 1e-3),
+                                  "note": "4096 waves on 2048 wave slots (two per SIMD: 256 registers, most of the walk's table in LDS): two full turns.  traffic: "
+                                          "FETCH_SIZE + WRITE_SIZE of this launch from profiles/k_open_fold29_pmc_traffic.txt"}
+    for p_ in bufs:
         hip.free(p_)
     del gens_big
 
@@ -234,6 +297,17 @@ def main():
     msm_s = (time.perf_counter() - t0) / reps
     out["g1_msm_points_per_s"] = 11008 * 4096 / msm_s
     out["g1_msm_ms"] = msm_s * 1e3
+    # algorithmic work of the commitment: one mixed addition (11 Fp multiplications) per c-bit window of the bits the data covers
+    msm_c = 8
+    msm_bits = int(np.abs(Wm).max()).bit_length()
+    msm_windows = (msm_bits + 1 + msm_c - 1) // msm_c      # one spare bit for the signed digits' carry, as zk_g1_commit_int counts them
+    msm_tops = 11008 * 4096 * msm_windows * 11 * MAD_PER_FP_MUL / msm_s / 1e12
+    out["roofline_msm"] = {"kernel": "zk_g1_commit_int (k_msm_rows and the table build, conversion and row sums around it), 11008 x 4096 scalars over 4096 generators",
+                           "bound": "valu-int", "achieved": msm_tops, "peak": VALU_PEAK_TOPS, "unit": "T MAD32/s", "frac": msm_tops / VALU_PEAK_TOPS, "traffic": None,
+                           "window_bits_c": msm_c, "scalar_bits_b": msm_bits, "windows": msm_windows,
+                           "note": "algorithmic work = ceil((b + 1) / c) windows x 11 Fp multiplications (one mixed addition) x 300 MAD32 per (scalar, generator) pair, "
+                                   "b = bits of the largest |scalar| in the data, c = 8; the time is the whole commit_int call (fixed-base table of the "
+                                   "generators' multiples built and normalised, scalars range-checked, row sums) -- what g1_msm_points_per_s is quoted on"}
     del com, hW, gens
 
     # ---- Fr mul/s: n independent Montgomery products on resident operands ------------------------------------------------------
@@ -250,6 +324,15 @@ def main():
     out["fr_mul_per_s"] = n / (mul_ms * 1e-3)
     out["fr_mul_stream_gbs"] = 96 * n / (mul_ms * 1e-3) / 1e9
     out["fr_add_stream_gbs"] = 96 * n / (add_ms * 1e-3) / 1e9
+    mul_gbs = 96 * n / (mul_ms * 1e-3) / 1e9
+    mul_tops = n * MAD_PER_FR_MUL / (mul_ms * 1e-3) / 1e12
+    out["roofline_fr_mul"] = {"kernel": "k_ew<MONTMUL> (2^26 independent Montgomery products, operands streamed from HBM)", "bound": "hbm",
+                              "achieved": mul_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": mul_gbs / HBM_PEAK_GBS, "traffic": None,
+                              "valu_bound": {"achieved": mul_tops, "peak": VALU_PEAK_TOPS, "unit": "T MAD32/s", "frac": mul_tops / VALU_PEAK_TOPS},
+                              "binds": "hbm", "avg_launch_ms": mul_ms,
+                              "note": "96 B per product (two operands in, one out) against 136 MAD32 per product: at these rates the memory side is at "
+                                      f"{mul_gbs / HBM_PEAK_GBS:.2f} of its peak and the multiply-add side at {mul_tops / VALU_PEAK_TOPS:.2f}, so HBM binds; the plain addition "
+                                      f"kernel streams the same bytes at {96 * n / (add_ms * 1e-3) / 1e9:.0f} GB/s"}
 
     # measured VALU multiply-add peak
     peak = ctypes.c_double()
@@ -262,8 +345,8 @@ def main():
     mm_ms = time_kernel(lambda: hip.call("zk_fr_matmul_generic", c_void_p(dO), c_void_p(dA), c_void_p(dB), c_uint(M), c_uint(N), c_uint(P), None), reps=1)
     # (2) fused multilinear fold (3 levels per pass) over a 2048 x 4096 tensor: 32 B read per element
     u = mt_random_vec(np.random.RandomState(2), 3)
-    fold_ms = time_kernel(lambda: hip.call("zk_fr_fold_axis", c_void_p(dO), c_void_p(dA), u, c_int(3), c_size_t(1), c_uint(2048), c_size_t(4096), None), reps=10)
-    fold_gbs = 32 * 2048 * 4096 / (fold_ms * 1e-3) / 1e9
+    fold_ax_ms = time_kernel(lambda: hip.call("zk_fr_fold_axis", c_void_p(dO), c_void_p(dA), u, c_int(3), c_size_t(1), c_uint(2048), c_size_t(4096), None), reps=10)
+    fold_gbs = 32 * 2048 * 4096 / (fold_ax_ms * 1e-3) / 1e9
     mm_tops = M * N * P * 72 / (mm_ms * 1e-3) / 1e12
     out["roofline_matmul"] = {"kernel": "k_matmul (generic Montgomery Fr matmul, 2048x4096x4096)", "bound": "valu-int", "achieved": mm_tops, "peak": VALU_PEAK_TOPS,
                               "unit": "T MAD32/s", "frac": mm_tops / VALU_PEAK_TOPS, "traffic": None,
@@ -271,17 +354,44 @@ def main():
                                       "VALU instruction for its carry, so 0.5 is the ceiling of this formulation",
                               "avg_launch_ms": mm_ms, "gmac_per_s": M * N * P / (mm_ms * 1e-3) / 1e9}
     out["roofline_hbm"] = {"kernel": "k_fold_axis_dot<3> (fused 3-level multilinear fold, 2048x4096)", "bound": "hbm", "achieved": fold_gbs, "peak": HBM_PEAK_GBS,
-                           "unit": "GB/s", "frac": fold_gbs / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": fold_ms}
+                           "unit": "GB/s", "frac": fold_gbs / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": fold_ax_ms}
     for p in (dA, dB, dO, src):
         hip.free(p)
 
+    # (3) the first round of a hinted lookup sumcheck alone: 2^26 pairs of a mapping table's 2^27 queries (the size of the stacked attention's)
+    look, keep = lookup_probe()
+    look()
+    hip.check(lib.zk_prof_lookup_begin())
+    t0 = time.perf_counter()
+    look()
+    pv.sync()
+    look_total_ms = (time.perf_counter() - t0) * 1e3
+    l_ms, l_launches, l_pairs, l_bytes = read_lookup_timer()
+    if l_launches:
+        out["roofline_lookup_round"] = {"kernel": "k_lookup_round<false,true> alone: first round of tLookupRangeMapping::prove, 2^27 queries uniformly spread over 2^20 entries",
+                                        "bound": "hbm", "achieved": l_bytes / (l_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                        "frac": l_bytes / (l_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": l_ms / l_launches, "pairs": int(l_pairs),
+                                        "whole_proof_ms": look_total_ms,
+                                        "note": "algorithmic 240 B per pair (two queries of two tensors, eq weight, two folded values out, next eq table); the kernel also gathers "
+                                                "a 64-byte record (table entry and its inverse) per query from a 64 MiB table, and does six field products per pair"}
+    del keep, look
+
     # ---- CPU baseline: the oracle's restatement of the reference's algorithm on this host's cores ---------------------------------------
-    # A bounded sample of the two costs that dominate the reference's layer: the field multiplications of the matrix products
-    # and the five 255-bit scalar multiplications per generator pair of the openings; both scaled to the layer's counts.
+    # Measured parts, each scaled to its count in the layer: the field multiplications of the matrix products (a row sample),
+    # the openings (five 255-bit scalar multiplications per generator pair; a 4096-generator opening), and the lookup arguments
+    # (configuration 4 in full: multiplicities, 2^22 + 2^16 Fermat inversions, the 22-round sumcheck).  Configuration 1 runs in full.
     if not args.skip_cpu:
-        from zkhelp import load_oracle
+        from zkhelp import load_oracle, orc_check
         orc = load_oracle()
         cores = orc.dll.orc_num_threads()
+        # C1: zkFC toy, forward + 6-round sumcheck
+        rng1 = np.random.default_rng(7)
+        X1 = np.round(rng1.normal(0, 0.02, (16, 64)) * 65536).astype(np.int32)
+        W1 = np.round(rng1.normal(0, 0.02, (64, 64)) * 65536).astype(np.int32)
+        orc.orc_seed(1234)
+        t0 = time.perf_counter()
+        orc_check(orc.orc_zkfc(X1, W1, 16, 64, 64, np.zeros((16 * 64, 8), np.uint32), np.zeros(8, np.uint32)))
+        c1_s = time.perf_counter() - t0
         B = mt_random_vec(np.random.RandomState(4), 4096 * 1024)
 
         def mm_sample(rows):
@@ -292,13 +402,12 @@ def main():
             return time.perf_counter() - t0
         probe_rows = 2 * max(1, cores // 2)
         dt = mm_sample(probe_rows)
-        rows = int(max(probe_rows, min(4096, probe_rows * 20.0 / max(dt, 1e-3)))) // max(1, cores) * max(1, cores)
+        rows = int(max(probe_rows, min(4096, probe_rows * 10.0 / max(dt, 1e-3)))) // max(1, cores) * max(1, cores)
         rows = max(rows, probe_rows)
         dt = mm_sample(rows)
         mm_rate = rows * 4096 * 1024 / dt                      # field multiplications per second, all cores
         # opening sample: n generators, one row
         n_open = 4096
-        gens = np.zeros((n_open, 36), np.uint32)
         orc.orc_seed(99)
         gens = np.zeros((n_open, 36), np.uint32)
         orc.orc_commitment_random(n_open, gens)
@@ -310,13 +419,35 @@ def main():
         t0 = time.perf_counter()
         orc.orc_open(gens, n_open, T, n_open, 1, u, k, proof, val)
         open_s = time.perf_counter() - t0
+        # C4: range lookup of 2^22 queries into 2^16 entries, in full
+        D4, N4 = 1 << 22, 1 << 16
+        S4 = np.zeros((D4, 8), np.uint32)
+        v4 = np.random.default_rng(4).integers(-(1 << 15), 1 << 15, D4)
+        orc.orc_fr_from_i64(np.ascontiguousarray(v4, dtype=np.int64), S4, D4)
+        rs4 = np.random.RandomState(14)
+        al4, be4 = mt_random_vec(rs4, 1), mt_random_vec(rs4, 1)
+        u4, w4 = mt_random_vec(rs4, 22), mt_random_vec(rs4, 22)
+        m4 = np.zeros((N4, 8), np.uint32)
+        fin4 = np.zeros(8, np.uint32)
+        t0 = time.perf_counter()
+        orc_check(orc.orc_range_prep(S4, D4, -(1 << 15), N4, m4))
+        orc_check(orc.orc_range_prove(S4, D4, -(1 << 15), N4, al4, be4, u4, w4, fin4))
+        c4_s = time.perf_counter() - t0
         layer_mm = 4.49e11                                     # field multiplications in the layer's matrix products (reference algorithm)
         layer_gens = 5 * (4096 << 5) + 2 * (1 << 19) + 2 * 4096      # generators of the nine openings (11008 << 5 rounds up to 2^19); pairs over all rounds ~ the same number
-        cpu_s = layer_mm / mm_rate + open_s * layer_gens / n_open
+        # queries of the layer's lookup arguments: three softmax segments over 32 x 2048 x 2048, the activation table and four rescalings over the
+        # padded 2048 x 11008 tensors, nine rescalings over 2048 x 4096, two over 4096
+        layer_queries = 3 * (1 << 27) + 4 * (1 << 25) + 9 * (1 << 23) + 2 * 4096
+        parts_cpu = {"matrix_products_s": layer_mm / mm_rate, "openings_s": open_s * layer_gens / n_open, "lookup_arguments_s": c4_s * layer_queries / D4}
+        cpu_s = sum(parts_cpu.values())
         out["cpu_baseline"] = {"value": cpu_s, "unit": "s", "cores": int(cores), "kind": "port",
-                               "sample": f"oracle (reference algorithm, OpenMP): Fr matmul {rows} x 4096 x 1024 = {rows * 4096 * 1024:.3g} multiplications in {dt:.1f} s, "
+                               "sample": f"oracle (reference algorithm, OpenMP, {int(cores)} threads): Fr matmul {rows} x 4096 x 1024 = {rows * 4096 * 1024:.3g} multiplications in {dt:.1f} s, "
                                          f"scaled to the layer's 4.49e11; opening of {n_open} generators in {open_s:.1f} s, scaled to the layer's "
-                                         f"{layer_gens} generators; sumchecks and lookups not included (lower bound of the CPU layer time)",
+                                         f"{layer_gens} generators; configuration 4 in full (2^22 queries into 2^16 entries: multiplicities, Fermat inversions, 22 rounds) in "
+                                         f"{c4_s:.1f} s, scaled to the layer's {layer_queries:.3g} queries; the sumchecks of the matrix products and the softmax's "
+                                         "Hadamard argument are not included",
+                               "parts_s": {k_: round(v_, 1) for k_, v_ in parts_cpu.items()},
+                               "config1_zkfc_toy_s": c1_s, "config4_lookup_s": c4_s,
                                "fr_mul_per_s_all_cores": mm_rate}
     print(json.dumps(out))
 

@@ -18,6 +18,9 @@
 #include <vector>
 #include "detmath.hpp"
 #include "field.hpp"
+#include <mutex>
+#include <utility>
+#include <vector>
 #include "rt.hpp"
 #include "../../include/zkllm_hip.h"
 
@@ -1178,6 +1181,15 @@ __global__ void __launch_bounds__(TPB) k_dot_part(Fr* __restrict__ partials, con
     for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (size_t)gridDim.x * TPB) acc[0] = add(acc[0], mont_mul(a[i], b[i]));
     block_reduce_store<1>(acc, partials);
 }
+// Optional timing of the hinted first round's launches with events on their own stream (measurement only).
+struct RoundTimer {
+    std::mutex mu;
+    bool on = false;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> ev;
+    unsigned long long pairs = 0;
+    double bytes = 0;          // algorithmic traffic of the timed launches
+};
+static RoundTimer g_round_timer;
 // all rounds of the lookup sumcheck; sums land in job.sums
 // A == nullptr with a hint source: 1 / (S + beta) has not been written anywhere; a large first round computes it on
 // the fly, anything else writes it out first.
@@ -1258,9 +1270,25 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
         } else if (phase2)
             hipLaunchKernelGGL((k_lookup_round<true, false>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, w + 2 * half, w + 3 * half, w + 4 * half, cA, cS, cB, cT, cm, cE, b, vm, half, nE,
                                HintSrc());
-        else if (r == 0 && fuse_first)
+        else if (r == 0 && fuse_first) {
+            hipEvent_t t0 = nullptr, t1 = nullptr;
+            if (g_round_timer.on) {
+                ZK_HIP(hipEventCreate(&t0));
+                ZK_HIP(hipEventCreate(&t1));
+                ZK_HIP(hipEventRecord(t0, st));
+            }
             hipLaunchKernelGGL((k_lookup_round<false, true>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, (const Fr*)nullptr, cS,
                                (const Fr*)nullptr, (const Fr*)nullptr, (const Fr*)nullptr, cE, b, vm, half, nE, *hs);
+            if (g_round_timer.on) {
+                ZK_HIP(hipEventRecord(t1, st));
+                std::lock_guard<std::mutex> lk(g_round_timer.mu);
+                g_round_timer.ev.emplace_back(t0, t1);
+                g_round_timer.pairs += half;
+                // per pair: two queries (32 B each; a mapping table's query is two tensors), the eq weight (32 B), two folded values
+                // written (64 B), the next round's eq table (16 B)
+                g_round_timer.bytes += (double)half * ((hs->S_out ? 128.0 : 64.0) + 32.0 + 64.0 + (nE ? 16.0 : 0.0));
+            }
+        }
         else
             hipLaunchKernelGGL((k_lookup_round<false, false>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, cA, cS, (const Fr*)nullptr,
                                (const Fr*)nullptr, (const Fr*)nullptr, cE, b, vm, half, nE, HintSrc());
@@ -1507,6 +1535,35 @@ int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host) {
     }
     sumjob_abort(job);
     return rc;
+}
+// Measurement: time every launch of the hinted first round (k_lookup_round<false, true>) between begin and read, with events
+// on the launch stream.  bytes: the algorithmic traffic of those launches.
+int zk_prof_lookup_begin(void) {
+    std::lock_guard<std::mutex> lk(g_round_timer.mu);
+    for (auto& e : g_round_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
+    g_round_timer.ev.clear();
+    g_round_timer.pairs = 0;
+    g_round_timer.bytes = 0;
+    g_round_timer.on = true;
+    return 0;
+}
+int zk_prof_lookup_read(double* total_ms, unsigned long long* launches, unsigned long long* pairs, double* bytes) {
+    std::lock_guard<std::mutex> lk(g_round_timer.mu);
+    g_round_timer.on = false;
+    double tot = 0;
+    for (auto& e : g_round_timer.ev) {
+        ZK_HIP(hipEventSynchronize(e.second));
+        float ms = 0;
+        ZK_HIP(hipEventElapsedTime(&ms, e.first, e.second));
+        tot += ms;
+    }
+    *total_ms = tot;
+    *launches = g_round_timer.ev.size();
+    *pairs = g_round_timer.pairs;
+    *bytes = g_round_timer.bytes;
+    for (auto& e : g_round_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
+    g_round_timer.ev.clear();
+    return 0;
 }
 // The whole multi-Hadamard sumcheck (proof.cu:191-241) queued without a host round trip.  Xs: K tensors of N elements
 // (N a power of two), E: N/2 elements (Montgomery form), v: log2(N) fold challenges in round order.  coefs_host:

@@ -498,6 +498,12 @@ void* zkp_layer_create_random(const u32* cu, const double* cf, u32 seed, u32 log
 void zkp_layer_free(void* h) { delete reinterpret_cast<LayerState*>(h); }
 void zkp_layer_set_head_group(void* h, u32 g) { reinterpret_cast<LayerState*>(h)->cfg.attn_head_group = g; }
 void zkp_layer_set_open_weights(void* h, int on) { reinterpret_cast<LayerState*>(h)->cfg.open_weights = on != 0; }
+// setup times of the last zkp_layer_create_random (ms): weights, generators, commitments, prepared generators
+void zkp_layer_setup_times(double* out4) { const LayerSetupTimes& t = layer_setup_times(); out4[0] = t.weights; out4[1] = t.generators; out4[2] = t.commitments; out4[3] = t.prepare; }
+// the nine commitments of the layer computed once more (ms); negative on error
+double zkp_layer_recommit_ms(void* h) {
+    try { return layer_recommit_ms(reinterpret_cast<LayerState*>(h)->w); } catch (const std::exception& e) { g_err = e.what(); return -1.0; }
+}
 // openings of the layer whose points are known ahead (0 until the first run with weight openings has finished)
 int zkp_layer_planned_openings(void* h) { const LayerState& s = *reinterpret_cast<LayerState*>(h); return s.w.plan && s.w.plan->learned ? (int)s.w.plan->entries.size() : 0; }
 // runs the whole layer (compute + every proof); times_ms (8 values): rmsnorm1, qkv, attention, oproj, rmsnorm2, ffn, total, open_wait

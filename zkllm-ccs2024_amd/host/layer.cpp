@@ -407,20 +407,38 @@ FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor
     return out;
 }
 
+static LayerSetupTimes g_setup_times;
+const LayerSetupTimes& layer_setup_times() { return g_setup_times; }
 static Weight random_weight(std::mt19937_64& rng, uint in_dim, uint out_dim, uint pp_size, bool norm) {
+    const double t0 = now_ms();
     std::normal_distribution<double> nd(0.0, 0.02);
     std::vector<int> wi((size_t)in_dim * out_dim);
     for (auto& x : wi) x = norm ? 65536 : (int)std::nearbyint(nd(rng) * 65536.0);   // scale 2^16 (llama-commit.py:34)
     FrTensor weight((uint)wi.size(), wi.data());
-    Commitment gen = Commitment::random(1u << ceilLog2(pp_size));
     const bool ragged = in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim));
     std::shared_ptr<const FrTensor> padded = ragged ? std::make_shared<const FrTensor>(weight.pad({in_dim, out_dim})) : nullptr;
+    const double t1 = now_ms();
+    Commitment gen = Commitment::random(1u << ceilLog2(pp_size));
+    const double t2 = now_ms();
     G1TensorJacobian com = gen.commit_int(ragged ? *padded : weight);
+    const double t3 = now_ms();
     gen.prepare_openings();
+    const double t4 = now_ms();
+    g_setup_times.weights += t1 - t0; g_setup_times.generators += t2 - t1; g_setup_times.commitments += t3 - t2; g_setup_times.prepare += t4 - t3;
     return Weight{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim, std::move(padded)};
+}
+double layer_recommit_ms(const LayerWeights& w) {
+    const Weight* all[9] = {&w.input_norm, &w.q, &w.k, &w.v, &w.o, &w.post_norm, &w.up, &w.gate, &w.down};
+    const double t0 = now_ms();
+    for (const Weight* x : all) {
+        G1TensorJacobian com = x->generator.commit_int(x->padded ? *x->padded : x->weight);
+        (void)com;
+    }
+    return now_ms() - t0;
 }
 
 LayerWeights make_random_layer_weights(const LayerConfig& c, uint32_t seed, uint lof) {
+    g_setup_times = LayerSetupTimes();
     std::mt19937_64 rng(seed);
     const uint E = c.embed_dim, Hd = c.hidden_dim;
     // llama-ppgen.py:21-31: 2-D parameters use (HF shape[0] = out_features) << log_off_factor, 1-D their length

@@ -83,6 +83,13 @@ FrTensor attn_reference_block(const LayerConfig& c, const FrTensor& Q, const FrT
 // whole layer: x -> x + attn(norm(x)) -> (+ ffn(norm(.)))
 FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor& X, LayerTimes* times);
 
+// how long make_random_layer_weights last spent on each part of the setup (ms, device idle at both ends of every part):
+// the random fixed-point weights (host generator + upload + padding), the generator sets, the nine commitments, the
+// generators' prepared form for openings
+struct LayerSetupTimes { double weights = 0, generators = 0, commitments = 0, prepare = 0; };
+const LayerSetupTimes& layer_setup_times();
+// commits the nine weights again (the results are dropped): the commitment cost of a layer, in ms
+double layer_recommit_ms(const LayerWeights& w);
 // random-init weights of the configured shape (round(N(0, 0.02) * 2^16), norm weights round(2^16)), generators from the
 // seeded stream sized as llama-ppgen.py does (out_features << log_off_factor, rounded up to a power of two) and commitments
 LayerWeights make_random_layer_weights(const LayerConfig& c, uint32_t seed, uint log_off_factor);
