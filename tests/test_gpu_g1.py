@@ -303,14 +303,17 @@ def test_open_batch_over_prepared_generators_matches_single_openings(orc):
             u = mt_random_vec(np.random.RandomState(70 + i), k)
             gens.append(g); us.append(u)
             dG.append(hip.upload(g)); dS.append(hip.upload(S))
+            print(f"open n={n} item={i}: zk_g1_open", flush=True)
             hip.call("zk_g1_open", exp_p[i], exp_v[i], c_void_p(dS[i]), c_void_p(dG[i]), c_size_t(n), u, c_int(k), None)
             pr = c_void_p()
+            print(f"open n={n} item={i}: zk_g1_open_prepare", flush=True)
             hip.call("zk_g1_open_prepare", ctypes.byref(pr), c_void_p(dG[i]), c_size_t(n), None)
             preps.append(pr)
         h = c_void_p()
         sc = (c_void_p * count)(*[c_void_p(x) for x in dS])
         pp = (c_void_p * count)(*preps)
         uall = np.ascontiguousarray(np.concatenate(us), dtype=np.uint32)
+        print(f"open n={n}: zk_g1_open_begin_batch of {count}", flush=True)
         hip.call("zk_g1_open_begin_batch", ctypes.byref(h), c_int(count), sc, pp, uall, c_int(k), None)
         got_p = np.zeros_like(exp_p)
         got_v = np.zeros_like(exp_v)
@@ -319,6 +322,7 @@ def test_open_batch_over_prepared_generators_matches_single_openings(orc):
         assert (got_p == exp_p).all(), n
         # one prepared opening on its own
         h1 = c_void_p()
+        print(f"open n={n}: zk_g1_open_begin_prepared", flush=True)
         hip.call("zk_g1_open_begin_prepared", ctypes.byref(h1), c_void_p(dS[0]), preps[0], us[0], c_int(k), None)
         p1 = np.zeros((npts, 36), np.uint32)
         v1 = np.zeros(8, np.uint32)

@@ -834,6 +834,79 @@ k_open_fold29(const FoldBatch fb, size_t old_size, size_t new_size) {
         special[1 + slot] = (uint32_t)g;
     }
 }
+// ---- the first round over prepared generators: a fixed-base comb per pair ----------------------------------------------------------
+// The generators of an opening are public and fixed, so D_i = g_2i - g_2i+1 is known before any challenge is.  For each
+// pair the prepared form holds the COMB_N = 2^COMB_A - 1 sums  E[m] = sum_{j : bit j of m} 2^(j COMB_W) D_i  as affine
+// points.  With u = k1 + k2 lambda (k1, k2 < 2^128 <= 2^(COMB_A COMB_W)), position b of the comb takes bit j COMB_W + b
+// of k1 for every tooth j as the index m1(b), likewise m2(b) from k2, and
+//     [u] D = sum_b 2^b ( E[m1(b)] + phi(E[m2(b)]) ),   phi(x, y) = (beta x, y):
+// COMB_W doublings and at most 2 COMB_W mixed additions instead of 129 doublings and ~65 additions, and no inversion for a
+// table.  Every lane of the launch uses the same indices, so the table is laid out entry-major ([m][pair]): the lanes of a
+// wave read consecutive points.
+static constexpr int COMB_A = 6, COMB_W = 22, COMB_N = (1 << COMB_A) - 1;
+static_assert(COMB_A * COMB_W >= 128, "the comb must cover 128-bit half scalars");
+struct CombK { uint8_t m1[COMB_W + 2], m2[COMB_W + 2]; };
+// No pair is special here: the table holds multiples of D whatever D is (infinity when the two generators are equal, a
+// doubling when they are opposite), an entry at infinity is skipped, and the mixed addition itself handles a sum that
+// meets its own operand.
+struct CombItem { Fr* ns; A29* ng; const Fr* s; const A29* g; const A29* tab; Fr u_mont; CombK ck; };
+struct CombBatch { CombItem it[OB_MAX]; };
+__global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+k_open_fold_comb(const CombBatch cb, size_t old_size, size_t new_size) {
+    __shared__ int32_t inv_lds[14][2 * GT];
+    Fr* __restrict__ new_scalars = cb.it[blockIdx.y].ns;
+    A29* __restrict__ new_gens = cb.it[blockIdx.y].ng;
+    const Fr* __restrict__ scalars = cb.it[blockIdx.y].s;
+    const A29* __restrict__ A = cb.it[blockIdx.y].g;
+    const A29* __restrict__ tab = cb.it[blockIdx.y].tab;
+    const Fr u_mont = cb.it[blockIdx.y].u_mont;
+    const CombK& ck = cb.it[blockIdx.y].ck;
+    const size_t g = (size_t)blockIdx.x * GT + threadIdx.x;
+    const bool live = g < new_size;
+    const size_t g0 = 2 * g, g1 = 2 * g + 1;
+    const bool has1 = live && g1 < old_size;
+    A29 a1;
+    a1.x = a1.y = fq29_zero();
+    if (has1) a1 = A[g1];
+    if (live) {
+        if (has1) new_scalars[g] = add(scalars[g0], mont_mul(u_mont, sub(scalars[g1], scalars[g0])));
+        else new_scalars[g] = sub(scalars[g0], mont_mul(u_mont, scalars[g0]));
+    }
+    const bool inf1 = !has1 || a29_is_inf(a1);
+    const bool fast = live;
+    J29 w = j29_infinity();
+    if (fast) {
+        const Fq29 beta = fq29_from_fp(glv_beta());
+        for (int b = COMB_W - 1; b >= 0; --b) {
+            w = j29_double(w);
+            const uint32_t m1 = ck.m1[b], m2 = ck.m2[b];          // the same for every lane
+            if (m1) {
+                const A29 t = tab[(size_t)(m1 - 1) * new_size + g];
+                if (!a29_is_inf(t)) w = j29_add_mixed(w, t);
+            }
+            if (m2) {
+                A29 t = tab[(size_t)(m2 - 1) * new_size + g];
+                if (!a29_is_inf(t)) {
+                    t.x = fq29_mul(t.x, beta);
+                    w = j29_add_mixed(w, t);
+                }
+            }
+        }
+        if (!inf1) w = j29_add_mixed(w, a1);
+    }
+    const bool has_z = fast && !w.inf;
+    const Fq29 zi = block_inv64_29(has_z ? w.z : fq29_one(), inv_lds);
+    if (fast) {
+        A29 o;
+        o.x = o.y = fq29_zero();
+        if (has_z) {
+            const Fq29 zi2 = fq29_sqr(zi);
+            o.x = fq29_canon(fq29_mul(w.x, zi2));
+            o.y = fq29_canon(fq29_mul(fq29_mul(w.y, zi2), zi));
+        }
+        new_gens[g] = o;
+    }
+}
 // the pairs k_open_fold29 left out, by the general Jacobian route in 32-bit limbs (one lane per pair, an inversion each)
 __device__ __forceinline__ G1Affine a29_to_affine(const A29& p) {
     G1Affine r;
@@ -873,12 +946,14 @@ __global__ void __launch_bounds__(GT) k_open_fold_special(const SpecialBatch sb,
     }
 }
 // generator pairs' sums g_2i + g_2i+1 (an odd last element alone) for T of the first round; and the pairs' scalar sums
-__global__ void __launch_bounds__(GT) k_open_pair_points(G1Jac* __restrict__ pj, const G1Affine* __restrict__ A, size_t old_size, size_t half_up) {
+// negate: the differences g_2i - g_2i+1 instead (what the first round's comb is built on)
+__global__ void __launch_bounds__(GT) k_open_pair_points(G1Jac* __restrict__ pj, const G1Affine* __restrict__ A, size_t old_size, size_t half_up, int negate) {
     const size_t i = (size_t)blockIdx.x * GT + threadIdx.x;
     if (i >= half_up) return;
     G1Jac p = aff_to_jac(A[2 * i]);
     if (2 * i + 1 < old_size) {
-        const G1Affine b = A[2 * i + 1];
+        G1Affine b = A[2 * i + 1];
+        if (negate) b = g1_neg(b);
         if (!aff_is_inf(b)) p = g1_add_mixed(p, b);
     }
     pj[i] = p;
@@ -1078,7 +1153,7 @@ static int open_prep_build(A29* out, const G1Jac* gens, size_t n, Arena& arena, 
     if (aff.rc || pj.rc || paff.rc) return aff.rc ? aff.rc : (pj.rc ? pj.rc : paff.rc);
     hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(n, CH), GT)), dim3(GT), 0, st, aff.p, gens, n);
     hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(n, 256)), dim3(256), 0, st, out, aff.as<G1Affine>(), n);
-    hipLaunchKernelGGL(k_open_pair_points, dim3(cdiv(half_up, GT)), dim3(GT), 0, st, pj.as<G1Jac>(), aff.as<G1Affine>(), n, half_up);
+    hipLaunchKernelGGL(k_open_pair_points, dim3(cdiv(half_up, GT)), dim3(GT), 0, st, pj.as<G1Jac>(), aff.as<G1Affine>(), n, half_up, 0);
     hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(half_up, CH), GT)), dim3(GT), 0, st, paff.p, pj.as<G1Jac>(), half_up);
     hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(half_up, 256)), dim3(256), 0, st, out + n, paff.as<G1Affine>(), half_up);
     ZK_LAUNCH_CHECK();
@@ -1100,7 +1175,26 @@ __global__ void __launch_bounds__(64) k_open_t_fix(G1Jac* __restrict__ wsum0, ui
     wsum[w] = g1_add(g1_add(wsum[w], g1_neg(wsum[MW + w])), g1_neg(wsum[2 * MW + w]));
 }
 // One round of `count` openings of equal size (count <= OB_MAX): one launch of each kernel covers all of them.
-struct RoundItem { Fr* new_scalars; A29* new_gens; const Fr* scalars; const A29* gens; Fr u; };
+struct RoundItem { Fr* new_scalars; A29* new_gens; const Fr* scalars; const A29* gens; Fr u; const A29* comb = nullptr; };
+// Fp multiplications of one pair of the comb fold by the formulas' count
+static double comb_fp_mults_per_pair(const CombK& ck) {
+    int adds = 0, phis = 0;
+    for (int b = 0; b < COMB_W; ++b) { adds += (ck.m1[b] ? 1 : 0) + (ck.m2[b] ? 1 : 0); phis += ck.m2[b] ? 1 : 0; }
+    // doublings (7 each), mixed additions (11 each), the endomorphism's product, final addition (11), its share of one batched inversion (3) and the way back to affine (5)
+    return 7.0 * COMB_W + 11.0 * adds + phis + 11.0 + 3.0 + 5.0;
+}
+static CombK comb_of(const GlvK& k) {
+    CombK ck;
+    memset(&ck, 0, sizeof(ck));
+    for (int b = 0; b < COMB_W; ++b)
+        for (int j = 0; j < COMB_A; ++j) {
+            const int bit = j * COMB_W + b;
+            if (bit >= 128) continue;
+            ck.m1[b] |= (uint8_t)(((k.k1[bit >> 5] >> (bit & 31)) & 1u) << j);
+            ck.m2[b] |= (uint8_t)(((k.k2[bit >> 5] >> (bit & 31)) & 1u) << j);
+        }
+    return ck;
+}
 static int open_round_launch(const RoundItem* items, int count, size_t old_size, bool with_T, G1Jac* wsum_round, uint32_t wsum_item_stride, Arena& arena, hipStream_t st,
                              hipStream_t aux, std::vector<hipEvent_t>& events) {
     ZK_ARG(old_size < (1ull << 31), "opening: more than 2^31 generators");
@@ -1185,19 +1279,31 @@ static int open_round_launch(const RoundItem* items, int count, size_t old_size,
     const size_t sp_stride = 1 + new_size;
     Scratch& special = arena.add(sizeof(uint32_t) * sp_stride * count);
     if (special.rc) return special.rc;
+    bool use_comb = with_T;
+    for (int i = 0; i < count; ++i) use_comb = use_comb && items[i].comb != nullptr;
     FoldBatch fb;
+    CombBatch cbt;
     SpecialBatch sb;
     double fp_mults = 0;
     for (int i = 0; i < OB_MAX; ++i) {
         const int k = i < count ? i : 0;
         const GlvK ku = glv_split(items[k].u);
-        FoldItem& f = fb.it[i];
-        f.ns = items[k].new_scalars; f.ng = items[k].new_gens; f.s = items[k].scalars; f.g = items[k].gens;
-        f.special = special.as<uint32_t>() + sp_stride * k;
-        f.u_mont = to_mont(items[k].u);
-        f.jsf = jsf_of(ku);
-        sb.ng[i] = f.ng; sb.g[i] = f.g; sb.special[i] = f.special; sb.ku[i] = ku;
-        if (i < count) fp_mults += fold_fp_mults_per_pair(f.jsf) * (double)new_size;
+        uint32_t* sp = special.as<uint32_t>() + sp_stride * k;
+        if (use_comb) {
+            CombItem& f = cbt.it[i];
+            f.ns = items[k].new_scalars; f.ng = items[k].new_gens; f.s = items[k].scalars; f.g = items[k].gens;
+            f.tab = items[k].comb;
+            f.u_mont = to_mont(items[k].u);
+            f.ck = comb_of(ku);
+            if (i < count) fp_mults += comb_fp_mults_per_pair(f.ck) * (double)new_size;
+        } else {
+            FoldItem& f = fb.it[i];
+            f.ns = items[k].new_scalars; f.ng = items[k].new_gens; f.s = items[k].scalars; f.g = items[k].gens; f.special = sp;
+            f.u_mont = to_mont(items[k].u);
+            f.jsf = jsf_of(ku);
+            if (i < count) fp_mults += fold_fp_mults_per_pair(f.jsf) * (double)new_size;
+        }
+        sb.ng[i] = items[k].new_gens; sb.g[i] = items[k].gens; sb.special[i] = sp; sb.ku[i] = ku;
     }
     hipLaunchKernelGGL(k_u32_zero, dim3(1), dim3(64), 0, st, special.as<uint32_t>(), (uint32_t)count, sp_stride);
     hipEvent_t t0 = nullptr, t1 = nullptr;
@@ -1206,7 +1312,8 @@ static int open_round_launch(const RoundItem* items, int count, size_t old_size,
         ZK_HIP(hipEventCreate(&t1));
         ZK_HIP(hipEventRecord(t0, st));
     }
-    hipLaunchKernelGGL(k_open_fold29, dim3(cdiv(new_size, GT), count), dim3(GT), 0, st, fb, old_size, new_size);
+    if (use_comb) hipLaunchKernelGGL(k_open_fold_comb, dim3(cdiv(new_size, GT), count), dim3(GT), 0, st, cbt, old_size, new_size);
+    else hipLaunchKernelGGL(k_open_fold29, dim3(cdiv(new_size, GT), count), dim3(GT), 0, st, fb, old_size, new_size);
     if (g_fold_timer.on) {
         ZK_HIP(hipEventRecord(t1, st));
         std::lock_guard<std::mutex> lk(g_fold_timer.mu);
@@ -1479,7 +1586,7 @@ int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host, con
     int rc = open_prep_build(g29.as<A29>(), (const G1Jac*)gens, old_size, arena, st);
     if (rc) return rc;
     std::vector<hipEvent_t> evs;
-    const RoundItem item{(Fr*)new_scalars, n29.as<A29>(), (const Fr*)scalars, g29.as<A29>(), load_fr(u)};
+    const RoundItem item{(Fr*)new_scalars, n29.as<A29>(), (const Fr*)scalars, g29.as<A29>(), load_fr(u), nullptr};
     rc = open_round_launch(&item, 1, old_size, true, wsum.as<G1Jac>(), 0u, arena, st, st, evs);
     (void)evs;
     if (rc) return rc;
@@ -1513,7 +1620,7 @@ struct OpenJob {
 };
 // One opening of the batch: its scalars, its challenges (rounds x 8 limbs) and its generators -- Jacobian, or null when
 // `prep` (their prepared form, open_prep_build) is given
-struct OpenItem { const void* scalars; const void* gens; const A29* prep; const uint32_t* u; };
+struct OpenItem { const void* scalars; const void* gens; const A29* prep; const uint32_t* u; const A29* comb = nullptr; };
 static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, int rounds, hipStream_t st, hipStream_t aux) {
     ZK_ARG(n >= 1, "zk_g1_open: empty input");
     ZK_ARG(count >= 1 && count <= OB_MAX, "zk_g1_open: a batch holds 1 to 8 openings");
@@ -1573,7 +1680,10 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
         if (s2.rc) return s2.rc;
         if (g2.rc) return g2.rc;
         RoundItem ri[OB_MAX];
-        for (int i = 0; i < count; ++i) ri[i] = RoundItem{s2.as<Fr>() + ns * i, g2.as<A29>() + ns * i, cs[i], cg[i], load_fr(items[i].u + 8 * r)};
+        for (int i = 0; i < count; ++i) {
+            ri[i] = RoundItem{s2.as<Fr>() + ns * i, g2.as<A29>() + ns * i, cs[i], cg[i], load_fr(items[i].u + 8 * r)};
+            if (r == 0) ri[i].comb = items[i].comb;
+        }
         int rc = open_round_launch(ri, count, size, r == 0, wsum.as<G1Jac>() + (size_t)3 * MW * r, wstride, job.arena, st, aux, job.events);
         if (rc) return rc;
         for (int i = 0; i < count; ++i) { cs[i] = ri[i].new_scalars; cg[i] = ri[i].new_gens; }
@@ -1654,7 +1764,7 @@ int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_
 // Generators prepared once for any number of openings against them: their affine 29-bit-limb form and the pair sums of
 // the first round (weight-independent; 1.5 n points of 112 bytes).  The handle is freed with zk_g1_open_prepared_free
 // once no opening that uses it is pending.
-struct OpenPrepared { void* a29 = nullptr; size_t n = 0; };
+struct OpenPrepared { void* a29 = nullptr; size_t n = 0; void* comb = nullptr; };
 int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stv) {
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(prepared != nullptr && n >= 1, "zk_g1_open_prepare: null handle or no generators");
@@ -1665,10 +1775,52 @@ int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stv) {
     {
         Arena arena(st);
         rc = open_prep_build((A29*)pr->a29, (const G1Jac*)gens, n, arena, st);
+        // The first round's comb, when that round is a fold (more generators than the batched last rounds take): entry-major
+        // table of the subset sums of 2^(j COMB_W) D, built from elementwise point kernels -- the teeth by repeated doubling
+        // (an addition of an array to itself), entry m = entry (m without its lowest bit) + entry (that bit).
+        if (rc == 0 && n > (size_t)TAIL_N) {
+            const size_t np = (n + 1) / 2, ne = np * COMB_N;
+            rc = pool_alloc(&pr->comb, sizeof(A29) * ne, st);
+            Scratch& aff = arena.add(sizeof(G1Affine) * n);
+            Scratch& tj = arena.add(sizeof(G1Jac) * ne);
+            Scratch& ta = arena.add(sizeof(G1Affine) * ne);
+            Scratch& tmp = arena.add(sizeof(G1Jac) * np);
+            if (rc == 0) rc = aff.rc ? aff.rc : (tj.rc ? tj.rc : (ta.rc ? ta.rc : tmp.rc));
+            if (rc == 0) {
+                G1Jac* T = tj.as<G1Jac>();
+                auto entry = [&](int m) { return T + (size_t)(m - 1) * np; };
+                hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(n, CH), GT)), dim3(GT), 0, st, aff.p, (const G1Jac*)gens, n);
+                hipLaunchKernelGGL(k_open_pair_points, dim3(cdiv(np, GT)), dim3(GT), 0, st, entry(1), aff.as<G1Affine>(), n, np, 1);
+                static_assert(COMB_W % 2 == 0, "the doublings alternate between two buffers and must end in the table");
+                for (int j = 1; j < COMB_A; ++j) {
+                    const G1Jac* src = entry(1 << (j - 1));
+                    for (int k = 0; k < COMB_W; ++k) {          // no launch writes what it reads
+                        G1Jac* dst = (k & 1) ? entry(1 << j) : tmp.as<G1Jac>();
+                        hipLaunchKernelGGL(k_g1_add, dim3(cdiv(np, GT)), dim3(GT), 0, st, dst, src, src, np, np, 0);
+                        src = dst;
+                    }
+                }
+                for (int m = 3; m <= COMB_N; ++m) {
+                    const int prev = m & (m - 1);
+                    if (!prev) continue;
+                    hipLaunchKernelGGL(k_g1_add, dim3(cdiv(np, GT)), dim3(GT), 0, st, entry(m), entry(prev), entry(m ^ prev), np, np, 0);
+                }
+                hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(ne, CH), GT)), dim3(GT), 0, st, ta.p, tj.as<G1Jac>(), ne);
+                hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(ne, 256)), dim3(256), 0, st, (A29*)pr->comb, ta.as<G1Affine>(), ne);
+                if (rc == 0 && hipGetLastError() != hipSuccess) rc = hip_fail(hipErrorLaunchFailure, "comb build", __FILE__, __LINE__);
+            }
+        }
+        // the temporaries go back to the allocator only when the stream has drained
+        if (hipStreamSynchronize(st) != hipSuccess && rc == 0) rc = hip_fail(hipGetLastError(), "zk_g1_open_prepare sync", __FILE__, __LINE__);
+        arena.mark_idle();
     }
-    // openings read it on the library's own streams: it must be complete before the handle is used
-    if (rc == 0 && hipStreamSynchronize(st) != hipSuccess) rc = hip_fail(hipGetLastError(), "zk_g1_open_prepare sync", __FILE__, __LINE__);
-    if (rc) { (void)hipStreamSynchronize(st); pool_free(pr->a29, st, true); return rc; }
+    // (openings read the prepared form on the library's own streams: it is complete before the handle is handed out)
+    if (rc) {
+        (void)hipStreamSynchronize(st);
+        pool_free(pr->a29, st, true);
+        if (pr->comb) pool_free(pr->comb, st, true);
+        return rc;
+    }
     *prepared = pr.release();
     return 0;
 }
@@ -1676,13 +1828,14 @@ int zk_g1_open_prepared_free(void* prepared) {
     if (!prepared) return 0;
     OpenPrepared* pr = (OpenPrepared*)prepared;
     int rc = pool_free(pr->a29, nullptr);
+    if (pr->comb) (void)pool_free(pr->comb, nullptr);
     delete pr;
     return rc;
 }
 int zk_g1_open_begin_prepared(void** handle, const void* scalars, const void* prepared, const uint32_t* u, int rounds, void* stv) {
     ZK_ARG(prepared != nullptr, "zk_g1_open_begin_prepared: null generators");
     const OpenPrepared* pr = (const OpenPrepared*)prepared;
-    const OpenItem item{scalars, nullptr, (const A29*)pr->a29, u};
+    const OpenItem item{scalars, nullptr, (const A29*)pr->a29, u, (const A29*)pr->comb};
     return open_begin_impl(handle, &item, 1, pr->n, rounds, stv);
 }
 // `count` (1 to 8) openings against prepared generator sets of one size and with one round count, as ONE job: every
@@ -1699,7 +1852,7 @@ int zk_g1_open_begin_batch(void** handle, int count, const void* const* scalars,
         const OpenPrepared* pr = (const OpenPrepared*)prepared[i];
         if (i == 0) n = pr->n;
         ZK_ARG(pr->n == n, "zk_g1_open_begin_batch: the generator sets differ in size");
-        items[i] = OpenItem{scalars[i], nullptr, (const A29*)pr->a29, u + (size_t)i * rounds * 8};
+        items[i] = OpenItem{scalars[i], nullptr, (const A29*)pr->a29, u + (size_t)i * rounds * 8, (const A29*)pr->comb};
     }
     return open_begin_impl(handle, items, count, n, rounds, stv);
 }
