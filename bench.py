@@ -82,6 +82,21 @@ def main():
         run = lambda: hip.call("zk_g1_open_round", c_void_p(ns), c_void_p(ng), sums3, c_void_p(sc), c_void_p(gp), u1, c_size_t(n_big), None)
         return n_big, gens_big, (sc, ns, ng), run
 
+    def prepared_opening(n_big, gens_big, scalars):
+        """one opening (zk_g1_open_begin_prepared / zk_g1_open_end) of `scalars` against generators prepared once"""
+        gp = pv.lib.zkp_g1_devptr(c_void_p(gens_big.h))
+        prep = c_void_p()
+        hip.call("zk_g1_open_prepare", ctypes.byref(prep), c_void_p(gp), c_size_t(n_big), None)
+        k = (n_big - 1).bit_length()
+        uk = mt_random_vec(np.random.RandomState(10), k)
+        pts, fin = np.zeros((3 * k + 1, 36), np.uint32), np.zeros(8, np.uint32)
+
+        def run():
+            h = c_void_p()
+            hip.call("zk_g1_open_begin_prepared", ctypes.byref(h), c_void_p(scalars), prep, uk, c_int(k), None)
+            hip.call("zk_g1_open_end", h, pts, fin)
+        return run
+
     def lookup_probe(logD=27, logN=20):
         """one mapping-table lookup proof (tLookupRangeMapping::prove) over 2^logD uniformly spread queries into 2^logN entries"""
         D, N = 1 << logD, 1 << logN
@@ -98,6 +113,10 @@ def main():
         n_big, gens_big, bufs, fold_round = fold_probe_setup()
         for _ in range(3):
             fold_round()
+        # a whole opening over the same generators in their prepared form: the first round's comb fold on 262144 pairs,
+        # then k_open_fold29 on 131072, 65536, ... pairs
+        prep_open = prepared_opening(n_big, gens_big, bufs[0])
+        prep_open()
         n = 1 << 24
         dA, dB, dO = hip.malloc(32 * n), hip.malloc(32 * n), hip.malloc(32 * n)
         hip.call("zk_fr_add", c_void_p(dO), c_void_p(dA), c_void_p(dB), c_size_t(n), None)
@@ -243,7 +262,8 @@ def main():
     # Fp multiplication is 2*12^2+12 = 300 of them.  Durations are HIP events around every launch inside the timed
     # region above, on the launch stream.
     fold_tops = fold_mults * MAD_PER_FP_MUL / (fold_ms * 1e-3) / 1e12 if fold_ms > 0 else 0.0
-    out["roofline"] = {"kernel": "k_open_fold29 (opening: g' = g1 + [u](g0 - g1) per pair, 128-bit split scalars; one launch per round for all openings of a size)",
+    out["roofline"] = {"kernel": "k_open_fold29 and, in an opening's first round, k_open_fold_comb (g' = g1 + [u](g0 - g1) per generator pair, 128-bit split scalars; "
+                                 "one launch per round for all openings of a size)",
                        "bound": "valu-int", "achieved": fold_tops, "peak": VALU_PEAK_TOPS, "unit": "T MAD32/s", "frac": fold_tops / VALU_PEAK_TOPS,
                        "traffic": None, "algorithmic_bytes_per_launch": FOLD_ALGO_BYTES_PER_PAIR * fold_pairs / max(1, fold_launches),
                        "launches": int(fold_launches), "avg_launch_ms": fold_ms / max(1, fold_launches),
@@ -278,6 +298,20 @@ def main():
                                   "avg_launch_ms": f_ms / max(1, f_launches), "fp_mul_per_s": f_mults / (f_ms * 1e-3),
                                   "note": "4096 waves on 2048 wave slots (two per SIMD: 256 registers, most of the walk's table in LDS): two full turns.  traffic: "
                                           "FETCH_SIZE + WRITE_SIZE of this launch from profiles/k_open_fold29_pmc_traffic.txt"}
+    # the fold kernels of one whole opening over the same generators prepared: the comb fold of the first round
+    # (262144 pairs) and k_open_fold29 on the later rounds down to the batched last rounds
+    prep_open = prepared_opening(n_big, gens_big, bufs[0])
+    prep_open()
+    hip.check(lib.zk_prof_fold_begin())
+    t0 = time.perf_counter()
+    prep_open()
+    open_alone_s = time.perf_counter() - t0
+    o_ms, o_launches, o_mults, o_pairs = read_fold_timer()
+    o_tops = o_mults * MAD_PER_FP_MUL / (o_ms * 1e-3) / 1e12
+    out["roofline_fold_opening_alone"] = {"kernel": "k_open_fold_comb (first round, 262144 pairs) + k_open_fold29 (later rounds) of one opening over 2^19 prepared generators, "
+                                                    "beside that opening's own bucket sums only", "bound": "valu-int", "achieved": o_tops, "peak": VALU_PEAK_TOPS,
+                                          "unit": "T MAD32/s", "frac": o_tops / VALU_PEAK_TOPS, "traffic": None, "launches": int(o_launches), "pairs": int(o_pairs),
+                                          "total_ms": o_ms, "fp_mul_per_pair": o_mults / max(1, o_pairs), "opening_wall_s": open_alone_s}
     for p_ in bufs:
         hip.free(p_)
     del gens_big

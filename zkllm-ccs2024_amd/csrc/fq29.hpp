@@ -276,8 +276,9 @@ ZK_HD G1Jac j29_to_jac(const J29& p) {
     r.x = fq29_to_fp(p.x); r.y = fq29_to_fp(p.y); r.z = fq29_to_fp(p.z);
     return r;
 }
+// The flag alone says infinity: the formulas run on whatever the coordinates hold (no branch, so the result of a walk
+// step is one set of registers whatever the lanes' cases are).
 FQ29_POINT_FN J29 j29_double(const J29& p) {
-    if (p.inf) return p;
     const Fq29 a = fq29_sqr(p.x);
     const Fq29 b = fq29_sqr(p.y);
     Fq29 c = fq29_sqr(b);
@@ -286,7 +287,7 @@ FQ29_POINT_FN J29 j29_double(const J29& p) {
     const Fq29 e = fq29_add(fq29_dbl(a), a);
     const Fq29 f = fq29_sqr(e);
     J29 r;
-    r.inf = 0u;
+    r.inf = p.inf;
     r.z = fq29_dbl(fq29_mul(p.y, p.z));
     r.x = fq29_sub(fq29_sub(f, d), d);
     c = fq29_dbl(fq29_dbl(fq29_dbl(c)));
@@ -294,16 +295,11 @@ FQ29_POINT_FN J29 j29_double(const J29& p) {
     return r;
 }
 FQ29_POINT_FN J29 j29_add_mixed(const J29& a, const A29& b) {
-    if (a.inf) { J29 r; r.x = b.x; r.y = b.y; r.z = fq29_one(); r.inf = 0u; return r; }
     const Fq29 z1z1 = fq29_sqr(a.z);
     const Fq29 u2 = fq29_mul(b.x, z1z1);
     const Fq29 s2 = fq29_mul(fq29_mul(b.y, a.z), z1z1);
     const Fq29 h = fq29_sub(u2, a.x);
     const Fq29 rr0 = fq29_sub(s2, a.y);
-    if (fq29_is_zero_mod_p(h)) {                       // same abscissa: the same point (double it) or its opposite
-        if (fq29_is_zero_mod_p(rr0)) return j29_double(a);
-        return j29_infinity();
-    }
     const Fq29 hh = fq29_sqr(h);
     const Fq29 i = fq29_dbl(fq29_dbl(hh));
     Fq29 j = fq29_mul(h, i);
@@ -315,6 +311,12 @@ FQ29_POINT_FN J29 j29_add_mixed(const J29& a, const A29& b) {
     j = fq29_dbl(fq29_mul(a.y, j));
     r.y = fq29_sub(fq29_mul(fq29_sub(v, r.x), rr), j);
     r.z = fq29_sub(fq29_sub(fq29_sqr(fq29_add(a.z, h)), z1z1), hh);
+    if (a.inf) {                                       // infinity + b = b
+        r.x = b.x; r.y = b.y; r.z = fq29_one();
+    } else if (fq29_is_zero_mod_p(h)) {                // same abscissa: the same point (double it) or its opposite
+        if (fq29_is_zero_mod_p(rr0)) r = j29_double(a);
+        else r = j29_infinity();
+    }
     return r;
 }
 

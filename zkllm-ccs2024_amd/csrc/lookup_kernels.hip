@@ -456,7 +456,9 @@ struct HintSrc { const Fr* TB; const Fr* hint; Fr low; Fr beta; uint32_t N; cons
 __device__ __forceinline__ Fr hinted_query(const Fr* __restrict__ S, size_t i, const HintSrc& h) {
     return h.S_out ? add(h.hint[i], mont_mul(h.r_mont, h.S_out[i])) : S[i];
 }
-static __device__ __attribute__((noinline)) Fr inv_plus_beta_alone(const Fr& sv, const Fr& beta) {
+// Operands by value: a reference would have the caller keep every query in private memory ahead of the rarely taken call
+// (64 bytes of private-memory stores per pair of the round kernel).
+static __device__ __attribute__((noinline)) Fr inv_plus_beta_alone(const Fr sv, const Fr beta) {
     const Fr v = add(sv, beta);
     if (is_zero(v)) return big_zero<8>();
     // v is the Montgomery form of v/R: its Montgomery inverse is R^2/v, and a Montgomery product with R^-1 leaves 1/v
