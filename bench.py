@@ -387,6 +387,29 @@ def main():
                               "note": "algorithmic 72 MAD32 per field multiply-accumulate (64 limb products + 1/8 of a shared reduction); every MAD32 needs a second "
                                       "VALU instruction for its carry, so 0.5 is the ceiling of this formulation",
                               "avg_launch_ms": mm_ms, "gmac_per_s": M * N * P / (mm_ms * 1e-3) / 1e9}
+    # (1b) the same shape as the layer computes it: fixed-point operands (activations to 2^20, weights N(0, 0.02) at scale 2^16) through
+    # zk_fr_matmul -> digit planes -> k_gemm_i8_planes on the matrix cores
+    rngm = np.random.default_rng(3)
+    hXa = pv.from_i32(np.clip(np.round(rngm.normal(0, 1, (M, N)) * 65536), -(1 << 20), 1 << 20).astype(np.int32))
+    hWa = pv.from_i32(np.round(rngm.normal(0, 0.02, (N, P)) * 65536).astype(np.int32))
+    pv.matmul(hXa, hWa, M, N, P)
+    hip.check(lib.zk_prof_gemm_begin())
+    t0 = time.perf_counter()
+    for _ in range(3):
+        pv.matmul(hXa, hWa, M, N, P)
+    pv.sync()
+    mm_call_ms = (time.perf_counter() - t0) * 1e3 / 3
+    g_ms, g_launches, g_macs = ctypes.c_double(), ctypes.c_ulonglong(), ctypes.c_double()
+    hip.check(lib.zk_prof_gemm_read(ctypes.byref(g_ms), ctypes.byref(g_launches), ctypes.byref(g_macs)))
+    if g_launches.value:
+        g_tops = 2 * g_macs.value / (g_ms.value * 1e-3) / 1e12
+        out["roofline_matmul_mfma"] = {"kernel": "k_gemm_i8_planes_all<3,2> (v_mfma_i32_32x32x32_i8 over base-256 digit planes: three of the activations, two of the weights; 2048x4096x4096, exact)", "bound": "mfma",
+                                       "achieved": g_tops, "peak": 5000.0, "unit": "TOP/s", "frac": g_tops / 5000.0, "traffic": None,
+                                       "avg_launch_ms": g_ms.value / g_launches.value, "plane_pairs": g_macs.value / g_launches.value / (M * N * P),
+                                       "whole_product_ms": mm_call_ms,
+                                       "note": "int8 multiply-accumulates x 2 over the kernel's launch time; whole_product_ms is zk_fr_matmul end to end (bound check on the "
+                                               "device, both digit splits, the GEMM with the recombination to field elements in its epilogue)"}
+    del hXa, hWa
     out["roofline_hbm"] = {"kernel": "k_fold_axis_dot<3> (fused 3-level multilinear fold, 2048x4096)", "bound": "hbm", "achieved": fold_gbs, "peak": HBM_PEAK_GBS,
                            "unit": "GB/s", "frac": fold_gbs / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": fold_ax_ms}
     for p in (dA, dB, dO, src):

@@ -255,6 +255,10 @@ int zk_bench_copy(void* dst, const void* src, size_t bytes, void* stream);
  * perform by the point formulas' count; pairs: generator pairs folded */
 int zk_prof_fold_begin(void);
 int zk_prof_fold_read(double* total_ms, unsigned long long* launches, double* fp_mults, unsigned long long* pairs);
+/* the same for the int8-plane GEMM of the small-integer matrix products (k_gemm_i8_planes, behind zk_fr_matmul);
+ * macs: int8 multiply-accumulates of those launches (rows x contraction x columns x plane pairs) */
+int zk_prof_gemm_begin(void);
+int zk_prof_gemm_read(double* total_ms, unsigned long long* launches, double* macs);
 /* the same for the first round of the hinted lookup sumchecks (k_lookup_round<false, true>); bytes: their algorithmic traffic */
 int zk_prof_lookup_begin(void);
 int zk_prof_lookup_read(double* total_ms, unsigned long long* launches, unsigned long long* pairs, double* bytes);

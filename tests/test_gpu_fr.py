@@ -356,6 +356,38 @@ def test_matmul_int8_plane_path_equals_generic_at_projection_size(pv):
         assert fr_ints(got[i * P + j].reshape(1, 8))[0] == want
 
 
+def test_matmul_int8_plane_path_on_ragged_stacks_and_wide_operands(pv):
+    """The matrix-core path (digit planes, k_gemm_i8_planes) forced onto small stacks whose sizes are no multiples of its
+    tiles (rows, columns and the contraction all ragged; a single row; a contraction shorter than one tile), with a left
+    operand of up to 2^38 (five planes) and a right operand of up to 2^33 (five planes), which go pair by pair, and with one to three
+    planes a side, which take every pair in one pass: every entry against big integers."""
+    import os
+    rng = np.random.default_rng(91)
+    pv.lib.zkp_set_matmul_mode(ctypes.c_int(0))
+    old = os.environ.get("ZKLLM_MATMUL_PLANES")
+    os.environ["ZKLLM_MATMUL_PLANES"] = "1"
+    try:
+        for num, M, N, P, (alo, ahi), (blo, bhi) in [(3, 70, 130, 50, (-2 ** 17, 2 ** 17), (-2 ** 10, 2 ** 10)),
+                                                     (2, 200, 1000, 150, (-2 ** 38, 2 ** 38), (-2 ** 12, 2 ** 12)),
+                                                     (1, 33, 5, 257, (-2 ** 20, 2 ** 20), (-2 ** 33, 2 ** 33)),
+                                                     (4, 129, 257, 32, (-128, 128), (-129, 129)),
+                                                     (2, 64, 128, 64, (-127, 128), (-127, 128)),
+                                                     (1, 100, 300, 90, (-2 ** 22, 2 ** 22), (-2 ** 22, 2 ** 22))]:
+            A = rng.integers(alo, ahi, (num, M, N)).astype(np.int64)
+            B = rng.integers(blo, bhi, (num, N, P)).astype(np.int64)
+            A[0, 0, :3] = [alo, ahi - 1, 0]
+            B[0, :3, 0] = [bhi - 1, blo, 0]
+            got = pv.matmul_stack(pv.from_i64(A), pv.from_i64(B), num, M, N, P).host()
+            assert pv.lib.zkp_last_matmul_path() == 2
+            want = [int(v) % R_MOD for i in range(num) for v in (A[i].astype(object) @ B[i].astype(object)).reshape(-1)]
+            assert fr_ints(got) == want, (num, M, N, P)
+    finally:
+        if old is None:
+            del os.environ["ZKLLM_MATMUL_PLANES"]
+        else:
+            os.environ["ZKLLM_MATMUL_PLANES"] = old
+
+
 def test_stacks_of_matrices_transpose_and_multiply_like_their_members(pv):
     """zk_fr_matmul_batched / zk_fr_transpose_batched on every path of the dispatcher (both operands in 31 bits, wide left
     operand, wide right operand, full-width residues): each product of the stack against big-int arithmetic."""

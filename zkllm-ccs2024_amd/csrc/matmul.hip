@@ -20,7 +20,8 @@
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
-#include <rocblas/rocblas.h>
+#include <utility>
+#include <vector>
 #include "field.hpp"
 #include "rt.hpp"
 #include "../../include/zkllm_hip.h"
@@ -319,14 +320,27 @@ template <typename T> static int run_int_path(void* C, const void* A, const void
     return 0;
 }
 
-// ---- int8-plane path -----------------------------------------------------------------------------------------------
-// balanced base-256 digits of a small signed integer: x = sum_j d_j 256^j, d_j in [-128, 127]; planes[j * n + i] = d_j of element i
-__global__ void __launch_bounds__(256) k_split_planes(int8_t* __restrict__ planes, const Fr* __restrict__ a, size_t n, int np) {
-    const size_t i0 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i0 >= n) return;
+// ---- int8-plane path: digit planes and a GEMM on the matrix cores ------------------------------------------------------
+// Balanced base-256 digits of a small signed integer: x = sum_j d_j 256^j, d_j in [-128, 127].  Both operands are laid
+// out with the contraction index fastest and padded with zeros to a multiple of the GEMM's K tile:
+//   planes of A[b][m][k]:  PA[((b * pa + i) * M + m) * Kp + k]
+//   planes of B[b][k][p]:  PB[((b * pb + j) * P + p) * Kp + k]      (transposed on the way)
+// so that every operand fragment of the matrix instruction is 16 consecutive bytes.
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+static constexpr int GBM = 128, GBN = 128, GBK = 128;      // block tile of the GEMM: 4 waves, 64 x 64 outputs each
+static constexpr int GLD = GBK + 16;                       // LDS row stride in bytes: 16-byte aligned rows whose 16-byte reads spread over all banks
+
+__global__ void __launch_bounds__(256) k_split_rows(int8_t* __restrict__ planes, const Fr* __restrict__ a, size_t rows, uint32_t M, uint32_t N, uint32_t Kp, int np) {
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const uint32_t groups = Kp / 4;
+    const size_t row = gid / groups;
+    if (row >= rows) return;
+    const uint32_t k = 4 * (uint32_t)(gid % groups);
+    const size_t b = row / M, m = row % M;
     long long x[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) x[e] = (i0 + e < n) ? fr_to_i64(a[i0 + e]) : 0ll;
+    for (int e = 0; e < 4; ++e) x[e] = (k + e < N) ? fr_to_i64(a[row * N + k + e]) : 0ll;
     for (int j = 0; j < np; ++j) {
         uint32_t packed = 0;
 #pragma unroll
@@ -335,76 +349,243 @@ __global__ void __launch_bounds__(256) k_split_planes(int8_t* __restrict__ plane
             x[e] = (x[e] - d) >> 8;
             packed |= (uint32_t)(uint8_t)d << (8 * e);
         }
-        int8_t* dst = planes + (size_t)j * n + i0;
-        if (i0 + 3 < n && (((size_t)j * n + i0) & 3) == 0) *reinterpret_cast<uint32_t*>(dst) = packed;
-        else
-            for (int e = 0; e < 4 && i0 + e < n; ++e) dst[e] = (int8_t)(packed >> (8 * e));
+        *reinterpret_cast<uint32_t*>(planes + ((b * np + j) * M + m) * Kp + k) = packed;
     }
 }
-// C[i] = sum_s Cs[s * n + i] * 2^(8s), embedded
-__global__ void __launch_bounds__(256) k_combine_planes(Fr* __restrict__ C, const int32_t* __restrict__ Cs, size_t n, int ns) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    unsigned long long v = 0;
-    for (int s2 = 0; s2 < ns; ++s2) v += (unsigned long long)(long long)Cs[(size_t)s2 * n + i] << (8 * s2);
-    C[i] = fr_from_i64((long long)v);
+// grid (P tiles of 64, K tiles of 64, batch): a 64 x 64 tile of B goes through LDS so that reads run along p and writes along k
+__global__ void __launch_bounds__(256) k_split_cols(int8_t* __restrict__ planes, const Fr* __restrict__ B, uint32_t N, uint32_t P, uint32_t Kp, int np) {
+    __shared__ __attribute__((aligned(16))) int8_t tile[8][64][80];
+    const uint32_t t = threadIdx.x, p = t & 63, kq = t >> 6;
+    const uint32_t p0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
+    const size_t b = blockIdx.z;
+    for (int r = 0; r < 16; ++r) {
+        const uint32_t k = k0 + kq * 16 + r;
+        long long x = (k < N && p0 + p < P) ? fr_to_i64(B[(b * N + k) * P + p0 + p]) : 0ll;
+        for (int j = 0; j < np; ++j) {
+            const long long d = (long long)(int8_t)(x & 0xFF);
+            x = (x - d) >> 8;
+            tile[j][p][kq * 16 + r] = (int8_t)d;
+        }
+    }
+    __syncthreads();
+    const uint32_t row = t >> 2, ch = t & 3;
+    if (p0 + row < P)
+        for (int j = 0; j < np; ++j)
+            *reinterpret_cast<v4i*>(planes + ((b * np + j) * P + p0 + row) * Kp + k0 + ch * 16) = *reinterpret_cast<const v4i*>(&tile[j][row][ch * 16]);
 }
+
+// C[b][m][p] = sum_{i,j} 256^(i+j) sum_k PA_i[b][m][k] PB_j[b][p][k], embedded in Fr.
+// One block computes a 128 x 128 tile of C; each of its four waves a 64 x 64 quarter as 2 x 2 tiles of
+// v_mfma_i32_32x32x32_i8.  Plane pairs are taken one after the other: int32 accumulators over the whole contraction
+// (|sum| <= K * 2^14, the caller keeps K below 2^17), then shifted into the int64 totals, which are exact modulo 2^64 and
+// therefore exact, the true result being below 2^62.  Operand tiles of 128 rows x 128 bytes pass through LDS; the next
+// tile is fetched into registers while the current one is multiplied.
+// Fragments: lane l supplies row (or column) l % 32 and the 16 contraction bytes 16 (l / 32) + 0..15 of a 32-byte step for
+// both operands alike, so whatever order the instruction takes the bytes in, every product pairs equal k.  Outputs:
+// register r of lane l is row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of the 32 x 32 tile.
+struct PlaneGemm { const int8_t* A; const int8_t* B; Fr* C; uint32_t M, P, Kp; int pa, pb; };
+__global__ void __launch_bounds__(256) k_gemm_i8_planes(const PlaneGemm g) {
+    __shared__ __attribute__((aligned(16))) int8_t sA[GBM * GLD];
+    __shared__ __attribute__((aligned(16))) int8_t sB[GBN * GLD];
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1;
+    const uint32_t m0 = blockIdx.y * GBM, n0 = blockIdx.x * GBN;
+    const size_t b = blockIdx.z;
+    long long tot[4][16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) tot[q][r] = 0;
+    for (int i = 0; i < g.pa; ++i)
+        for (int j = 0; j < g.pb; ++j) {
+            const int8_t* __restrict__ Ai = g.A + ((b * g.pa + i) * g.M) * (size_t)g.Kp;
+            const int8_t* __restrict__ Bj = g.B + ((b * g.pb + j) * g.P) * (size_t)g.Kp;
+            v16i acc[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[q][r] = 0;
+            v4i ra[4], rb[4];
+            auto fetch = [&](uint32_t k0) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t c = t + 256 * q, row = c >> 3, kc = c & 7;
+                    const v4i zero = {0, 0, 0, 0};
+                    ra[q] = (m0 + row < g.M) ? *reinterpret_cast<const v4i*>(Ai + (size_t)(m0 + row) * g.Kp + k0 + kc * 16) : zero;
+                    rb[q] = (n0 + row < g.P) ? *reinterpret_cast<const v4i*>(Bj + (size_t)(n0 + row) * g.Kp + k0 + kc * 16) : zero;
+                }
+            };
+            fetch(0);
+            for (uint32_t k0 = 0; k0 < g.Kp; k0 += GBK) {
+                __syncthreads();                    // every wave is done with the previous tile
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t c = t + 256 * q, row = c >> 3, kc = c & 7;
+                    *reinterpret_cast<v4i*>(sA + row * GLD + kc * 16) = ra[q];
+                    *reinterpret_cast<v4i*>(sB + row * GLD + kc * 16) = rb[q];
+                }
+                __syncthreads();
+                if (k0 + GBK < g.Kp) fetch(k0 + GBK);
+#pragma unroll
+                for (int ks = 0; ks < GBK / 32; ++ks) {
+                    const uint32_t ko = ks * 32 + 16 * (lane >> 5);
+                    const v4i a0 = *reinterpret_cast<const v4i*>(sA + (wm * 64 + (lane & 31)) * GLD + ko);
+                    const v4i a1 = *reinterpret_cast<const v4i*>(sA + (wm * 64 + 32 + (lane & 31)) * GLD + ko);
+                    const v4i b0 = *reinterpret_cast<const v4i*>(sB + (wn * 64 + (lane & 31)) * GLD + ko);
+                    const v4i b1 = *reinterpret_cast<const v4i*>(sB + (wn * 64 + 32 + (lane & 31)) * GLD + ko);
+                    acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b0, acc[0], 0, 0, 0);
+                    acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b1, acc[1], 0, 0, 0);
+                    acc[2] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b0, acc[2], 0, 0, 0);
+                    acc[3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b1, acc[3], 0, 0, 0);
+                }
+            }
+            const int shift = 8 * (i + j);
+            if (shift < 64) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) tot[q][r] = (long long)((unsigned long long)tot[q][r] + ((unsigned long long)(long long)acc[q][r] << shift));
+            }
+        }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const uint32_t row = m0 + wm * 64 + (q >> 1) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            const uint32_t col = n0 + wn * 64 + (q & 1) * 32 + (lane & 31);
+            if (row < g.M && col < g.P) g.C[(b * g.M + row) * (size_t)g.P + col] = fr_from_i64(tot[q][r]);
+        }
+}
+// The same product for up to three planes a side (every projection and attention product of the LLaMa layer): all plane pairs
+// are multiplied while a K tile lies in LDS, pairs of equal weight 256^(i+j) into one int32 accumulator (at most three pairs
+// of at most K * 2^14 each; the caller keeps 3 K below 2^17), and the int64 recombination happens once, in the epilogue.
+// Against the pair-by-pair kernel: one pass over the operands instead of PA * PB, PA * PB times the matrix instructions per
+// barrier, no int64 totals held through the loop.  Block tile 64 x 64, one 32 x 32 tile per wave, two blocks per CU.
+template <int PA, int PB> __global__ void __launch_bounds__(256, 2) k_gemm_i8_planes_all(const PlaneGemm g) {
+    constexpr int NS = PA + PB - 1, TB = 64;
+    __shared__ __attribute__((aligned(16))) int8_t sA[PA][TB * GLD];
+    __shared__ __attribute__((aligned(16))) int8_t sB[PB][TB * GLD];
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1;
+    const uint32_t m0 = blockIdx.y * TB, n0 = blockIdx.x * TB;
+    const size_t b = blockIdx.z;
+    const int8_t* __restrict__ A0 = g.A + (b * PA * g.M) * (size_t)g.Kp;
+    const int8_t* __restrict__ B0 = g.B + (b * PB * g.P) * (size_t)g.Kp;
+    const size_t a_plane = (size_t)g.M * g.Kp, b_plane = (size_t)g.P * g.Kp;
+    v16i acc[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[s][r] = 0;
+    v4i ra[PA][2], rb[PB][2];
+    auto fetch = [&](uint32_t k0) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t c = t + 256 * q, row = c >> 3, kc = c & 7;
+            const v4i zero = {0, 0, 0, 0};
+            const bool in_a = m0 + row < g.M, in_b = n0 + row < g.P;
+            const size_t oa = (size_t)(m0 + row) * g.Kp + k0 + kc * 16, ob = (size_t)(n0 + row) * g.Kp + k0 + kc * 16;
+#pragma unroll
+            for (int i = 0; i < PA; ++i) ra[i][q] = in_a ? *reinterpret_cast<const v4i*>(A0 + i * a_plane + oa) : zero;
+#pragma unroll
+            for (int j = 0; j < PB; ++j) rb[j][q] = in_b ? *reinterpret_cast<const v4i*>(B0 + j * b_plane + ob) : zero;
+        }
+    };
+    fetch(0);
+    for (uint32_t k0 = 0; k0 < g.Kp; k0 += GBK) {
+        __syncthreads();                    // every wave is done with the previous tile
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t c = t + 256 * q, row = c >> 3, kc = c & 7;
+#pragma unroll
+            for (int i = 0; i < PA; ++i) *reinterpret_cast<v4i*>(&sA[i][row * GLD + kc * 16]) = ra[i][q];
+#pragma unroll
+            for (int j = 0; j < PB; ++j) *reinterpret_cast<v4i*>(&sB[j][row * GLD + kc * 16]) = rb[j][q];
+        }
+        __syncthreads();
+        if (k0 + GBK < g.Kp) fetch(k0 + GBK);
+#pragma unroll
+        for (int ks = 0; ks < GBK / 32; ++ks) {
+            const uint32_t ko = ks * 32 + 16 * (lane >> 5);
+            v4i fa[PA], fb[PB];
+#pragma unroll
+            for (int i = 0; i < PA; ++i) fa[i] = *reinterpret_cast<const v4i*>(&sA[i][(wm * 32 + (lane & 31)) * GLD + ko]);
+#pragma unroll
+            for (int j = 0; j < PB; ++j) fb[j] = *reinterpret_cast<const v4i*>(&sB[j][(wn * 32 + (lane & 31)) * GLD + ko]);
+#pragma unroll
+            for (int i = 0; i < PA; ++i)
+#pragma unroll
+                for (int j = 0; j < PB; ++j) acc[i + j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i + j], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        unsigned long long v = 0;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) v += (unsigned long long)(long long)acc[s][r] << (8 * s);
+        const uint32_t row = m0 + wm * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const uint32_t col = n0 + wn * 32 + (lane & 31);
+        if (row < g.M && col < g.P) g.C[(b * g.M + row) * (size_t)g.P + col] = fr_from_i64((long long)v);
+    }
+}
+template <int PA> static bool launch_gemm_all_b(int pb, dim3 grid, hipStream_t st, const PlaneGemm& g) {
+    switch (pb) {
+        case 1: hipLaunchKernelGGL((k_gemm_i8_planes_all<PA, 1>), grid, dim3(256), 0, st, g); return true;
+        case 2: hipLaunchKernelGGL((k_gemm_i8_planes_all<PA, 2>), grid, dim3(256), 0, st, g); return true;
+        case 3: hipLaunchKernelGGL((k_gemm_i8_planes_all<PA, 3>), grid, dim3(256), 0, st, g); return true;
+        default: return false;
+    }
+}
+static bool launch_gemm_all(int pa, int pb, dim3 grid, hipStream_t st, const PlaneGemm& g) {
+    switch (pa) {
+        case 1: return launch_gemm_all_b<1>(pb, grid, st, g);
+        case 2: return launch_gemm_all_b<2>(pb, grid, st, g);
+        case 3: return launch_gemm_all_b<3>(pb, grid, st, g);
+        default: return false;
+    }
+}
+// Measurement: every launch of k_gemm_i8_planes between zk_prof_gemm_begin and zk_prof_gemm_read is timed with events on its stream.
+struct GemmTimer { bool on = false; std::mutex mu; std::vector<std::pair<hipEvent_t, hipEvent_t>> ev; double macs = 0; };
+static GemmTimer g_gemm_timer;
 static int digits_for(unsigned long long absmax) {      // planes needed for |x| <= absmax: p digits reach 127 (256^p - 1) / 255
     int p = 1;
     unsigned __int128 reach = 127;
     while (reach < absmax && p < 8) { reach = reach * 256 + 127; ++p; }
     return reach >= absmax ? p : 0;
 }
-static rocblas_handle blas_handle() {
-    static rocblas_handle h = nullptr;
-    static std::mutex mu;
-    std::lock_guard<std::mutex> lk(mu);
-    if (!h && rocblas_create_handle(&h) != rocblas_status_success) h = nullptr;
-    return h;
-}
 // returns ZK status; *done = false when the path does not apply (the caller then takes a VALU kernel)
-static int run_int8_plane_path(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, unsigned long long ma, unsigned long long mb, hipStream_t st,
-                               bool* done) {
+static int run_int8_plane_path(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, unsigned long long ma, unsigned long long mb,
+                               hipStream_t st, bool* done) {
     *done = false;
     const int pa = digits_for(ma), pb = digits_for(mb);
     if (!pa || !pb) return 0;
-    const int ns = pa + pb - 1;
-    const int most_pairs = pa < pb ? pa : pb;                       // planes pairs that share a weight
-    if ((unsigned long long)most_pairs * N >= (1ull << 17)) return 0;   // |sum of digit products| must stay below 2^31
-    if (M > (1u << 30) || N > (1u << 30) || P > (1u << 30)) return 0;
-    rocblas_handle h = blas_handle();
-    if (!h) return 0;
-    const size_t na = (size_t)M * N, nb = (size_t)N * P, nc = (size_t)M * P;
-    Scratch pla(na * pa, st), plb(nb * pb, st), cs(nc * ns * sizeof(int32_t), st);
+    if (N >= (1u << 17)) return 0;                                   // |sum_k of digit products| must stay below 2^31
+    if (M > (1u << 30) || P > (1u << 30)) return 0;
+    const uint32_t Kp = (N + GBK - 1) / GBK * GBK;
+    const size_t rows_a = (size_t)batch * M;
+    Scratch pla(rows_a * pa * Kp, st), plb((size_t)batch * pb * P * Kp, st);
     if (pla.rc) return pla.rc;
     if (plb.rc) return plb.rc;
-    if (cs.rc) return cs.rc;
-    hipLaunchKernelGGL(k_split_planes, dim3(cdiv(cdiv(na, 4), 256)), dim3(256), 0, st, pla.as<int8_t>(), (const Fr*)A, na, pa);
-    hipLaunchKernelGGL(k_split_planes, dim3(cdiv(cdiv(nb, 4), 256)), dim3(256), 0, st, plb.as<int8_t>(), (const Fr*)B, nb, pb);
-    ZK_LAUNCH_CHECK();
-    if (rocblas_set_stream(h, st) != rocblas_status_success) { set_error(ZK_ERR_BLAS, "rocblas_set_stream failed"); return ZK_ERR_BLAS; }
-    const int32_t one = 1, zero = 0;
-    for (int s2 = 0; s2 < ns; ++s2) {
-        int32_t* out = cs.as<int32_t>() + (size_t)s2 * nc;
-        bool first = true;
-        for (int i = 0; i < pa; ++i) {
-            const int j = s2 - i;
-            if (j < 0 || j >= pb) continue;
-            // row-major C = A_i B_j is column-major C^T = B_j^T A_i^T: the row-major arrays are those transposes as they lie
-            const rocblas_status rs = rocblas_gemm_ex(h, rocblas_operation_none, rocblas_operation_none, (rocblas_int)P, (rocblas_int)M, (rocblas_int)N, &one,
-                                                      plb.as<int8_t>() + (size_t)j * nb, rocblas_datatype_i8_r, (rocblas_int)P, pla.as<int8_t>() + (size_t)i * na,
-                                                      rocblas_datatype_i8_r, (rocblas_int)N, first ? &zero : &one, out, rocblas_datatype_i32_r, (rocblas_int)P, out,
-                                                      rocblas_datatype_i32_r, (rocblas_int)P, rocblas_datatype_i32_r, rocblas_gemm_algo_standard, 0, 0);
-            if (rs != rocblas_status_success) { (void)hipStreamSynchronize(st); set_error(ZK_ERR_BLAS, "rocblas_gemm_ex (int8) failed"); return ZK_ERR_BLAS; }
-            first = false;
-        }
+    hipLaunchKernelGGL(k_split_rows, dim3(cdiv(rows_a * (Kp / 4), 256)), dim3(256), 0, st, pla.as<int8_t>(), (const Fr*)A, rows_a, M, N, Kp, pa);
+    hipLaunchKernelGGL(k_split_cols, dim3(cdiv(P, 64), Kp / 64, batch), dim3(256), 0, st, plb.as<int8_t>(), (const Fr*)B, N, P, Kp, pb);
+    const PlaneGemm g{pla.as<int8_t>(), plb.as<int8_t>(), (Fr*)C, M, P, Kp, pa, pb};
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    if (g_gemm_timer.on) {
+        ZK_HIP(hipEventCreate(&t0));
+        ZK_HIP(hipEventCreate(&t1));
+        ZK_HIP(hipEventRecord(t0, st));
     }
-    hipLaunchKernelGGL(k_combine_planes, dim3(cdiv(nc, 256)), dim3(256), 0, st, (Fr*)C, cs.as<int32_t>(), nc, ns);
+    // up to three planes a side and three pairs' sums within int32: every pair in one pass; else pair by pair
+    const bool all_pairs = pa <= 3 && pb <= 3 && 3ull * N < (1ull << 17) && launch_gemm_all(pa, pb, dim3(cdiv(P, 64), cdiv(M, 64), batch), st, g);
+    if (!all_pairs) hipLaunchKernelGGL(k_gemm_i8_planes, dim3(cdiv(P, GBN), cdiv(M, GBM), batch), dim3(256), 0, st, g);
+    if (g_gemm_timer.on) {
+        ZK_HIP(hipEventRecord(t1, st));
+        std::lock_guard<std::mutex> lk(g_gemm_timer.mu);
+        g_gemm_timer.ev.emplace_back(t0, t1);
+        g_gemm_timer.macs += (double)batch * M * N * P * pa * pb;
+    }
     ZK_LAUNCH_CHECK();
     *done = true;
     return 0;
 }
-
 static inline unsigned absmax_grid(size_t n) {
     size_t b = n / (256 * 8) + 1;
     return (unsigned)(b > 1024 ? 1024 : b);
@@ -466,25 +647,44 @@ static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch
         return 0;
     }
     if (path_used) *path_used = 2;
-    // large products go to the matrix cores as int8 digit planes; below ~4 G multiply-accumulates the conversions outweigh the gain
-    // (ZKLLM_MATMUL_PLANES: log2 of that threshold, 0 = never)
-    static const int planes_log2 = getenv("ZKLLM_MATMUL_PLANES") ? atoi(getenv("ZKLLM_MATMUL_PLANES")) : 32;
-    if (planes_log2 > 0 && (unsigned long long)M * N * P >= (1ull << planes_log2)) {
-        bool all_done = true;
-        for (uint32_t i = 0; i < batch && all_done; ++i) {
-            bool done = false;
-            const int rc = run_int8_plane_path((Fr*)C + (size_t)i * M * P, (const Fr*)A + (size_t)i * M * N, (const Fr*)B + (size_t)i * N * P, M, N, P, ma_, mb_, st, &done);
-            if (rc) return rc;
-            if (!done) {
-                if (i) { set_error(ZK_ERR_ARG, "zk_fr_matmul: the int8-plane path applied to part of a stack only"); return ZK_ERR_ARG; }
-                all_done = false;
-            }
-        }
-        if (all_done) return 0;
+    // large products go to the matrix cores as int8 digit planes; below ~1 G multiply-accumulates (over the whole stack)
+    // the conversions outweigh the gain (ZKLLM_MATMUL_PLANES: log2 of that threshold, 0 = never)
+    const char* planes_env = getenv("ZKLLM_MATMUL_PLANES");           // read at every call: tests lower it around single products
+    const int planes_log2 = planes_env ? atoi(planes_env) : 30;
+    if (planes_log2 > 0 && (unsigned __int128)batch * M * N * P >= ((unsigned __int128)1 << planes_log2) && M >= 32 && P >= 32) {
+        bool done = false;
+        const int rc = run_int8_plane_path(C, A, B, batch, M, N, P, ma_, mb_, st, &done);
+        if (rc) return rc;
+        if (done) return 0;
     }
     if (fits32) return run_int_path<int>(C, A, B, batch, M, N, P, st);
     if (b_fits32) return run_wide_narrow_path(C, A, B, batch, M, N, P, st);
     return run_int_path<long long>(C, A, B, batch, M, N, P, st);
+}
+int zk_prof_gemm_begin(void) {
+    std::lock_guard<std::mutex> lk(g_gemm_timer.mu);
+    for (auto& e : g_gemm_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
+    g_gemm_timer.ev.clear();
+    g_gemm_timer.macs = 0;
+    g_gemm_timer.on = true;
+    return 0;
+}
+// total_ms / launches: summed durations and number of the timed launches; macs: int8 multiply-accumulates they performed
+// (rows x contraction x columns x plane pairs, without the padding)
+int zk_prof_gemm_read(double* total_ms, unsigned long long* launches, double* macs) {
+    std::lock_guard<std::mutex> lk(g_gemm_timer.mu);
+    g_gemm_timer.on = false;
+    double tot = 0;
+    for (auto& e : g_gemm_timer.ev) {
+        ZK_HIP(hipEventSynchronize(e.second));
+        float ms = 0;
+        ZK_HIP(hipEventElapsedTime(&ms, e.first, e.second));
+        tot += ms;
+    }
+    *total_ms = tot;
+    *launches = g_gemm_timer.ev.size();
+    *macs = g_gemm_timer.macs;
+    return 0;
 }
 int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv) {
     return matmul_dispatch(C, A, B, 1, M, N, P, mode, path_used, stv);
