@@ -393,6 +393,61 @@ template <int N, int T> __device__ __forceinline__ Big<N> mont_dot(const Big<N>*
 }
 #endif
 
+// ---- sums of products with ONE reduction for the whole sum -------------------------------------------------------------------
+// WideAcc holds an unreduced integer sum of 512-bit products in 17 limbs.  wide_mac adds a*b (any a, b < 2^256) by product
+// scanning: 64 limb products, each column taking the accumulator's limb along -- no reduction, no modular addition.  wide_redc
+// gives sum * R^-1 mod r as the canonical residue, the value that adding up mont_mul(a, b) would have given.  Room: a
+// product is below 2^512, so 2^32 of them fit.
+struct WideAcc { uint32_t v[17]; };
+ZK_HD WideAcc wide_zero() {
+    WideAcc w;
+#pragma unroll
+    for (int i = 0; i < 17; ++i) w.v[i] = 0;
+    return w;
+}
+#if defined(__HIPCC__)
+template <int K> __host__ __device__ __forceinline__ void wide_cols(uint64_t& lo, uint32_t& hi, const uint32_t* a, const uint32_t* b, WideAcc& w) {
+    constexpr int F = K < 8 ? 0 : K - 7, CNT = K < 8 ? K + 1 : 15 - K;
+    uint32_t y[CNT];
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) y[i] = b[K - F - i];
+    mac_chain<CNT, false>(lo, hi, a + F, y);
+    const uint64_t s = lo + w.v[K];
+    hi += (s < lo) ? 1u : 0u;
+    w.v[K] = (uint32_t)s;
+    lo = (s >> 32) | ((uint64_t)hi << 32);
+    hi = 0;
+    if constexpr (K < 14) wide_cols<K + 1>(lo, hi, a, b, w);
+}
+__host__ __device__ __forceinline__ void wide_mac(WideAcc& w, const Big<8>& a, const Big<8>& b) {
+    uint64_t lo = 0;
+    uint32_t hi = 0;
+    wide_cols<0>(lo, hi, a.v, b.v, w);
+    const uint64_t s = lo + w.v[15];          // lo: what is left above column 14, below 2^33
+    w.v[15] = (uint32_t)s;
+    w.v[16] += (uint32_t)(s >> 32);
+}
+#else
+static inline void wide_mac(WideAcc& w, const Big<8>& a, const Big<8>& b) {
+    uint32_t t[17];
+    for (int i = 0; i < 17; ++i) t[i] = 0;
+    for (int i = 0; i < 8; ++i) {
+        uint64_t c = 0;
+        for (int j = 0; j < 8; ++j) {
+            c += (uint64_t)a.v[i] * b.v[j] + t[i + j];
+            t[i + j] = (uint32_t)c;
+            c >>= 32;
+        }
+        t[i + 8] = (uint32_t)c;
+    }
+    uint64_t c = 0;
+    for (int i = 0; i < 17; ++i) {
+        c += (uint64_t)w.v[i] + t[i];
+        w.v[i] = (uint32_t)c;
+        c >>= 32;
+    }
+}
+#endif
 // Montgomery product a*b*R^-1 mod p, canonical.  Inputs < p.
 template <int N> ZK_HD Big<N> mont_mul(const Big<N>& a, const Big<N>& b) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -445,6 +500,17 @@ template <int N> ZK_HD Big<N> from_mont(const Big<N>& a) {
     Big<N> one = big_zero<N>();
     one.v[0] = 1;
     return mont_mul(a, one);
+}
+// sum = H 2^256 + L + T 2^512 (H, L of eight limbs, T the top limb):  sum R^-1 = H + L R^-1 + T R  (mod r)
+ZK_HD Big<8> wide_redc(const WideAcc& w) {
+    Big<8> L, H, T = big_zero<8>(), one = big_zero<8>();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { L.v[i] = w.v[i]; H.v[i] = w.v[8 + i]; }
+    T.v[0] = w.v[16];
+    one.v[0] = 1u;
+    H = reduce_once(reduce_once(H));                 // below 2^256 < 2.21 r
+    L = reduce_once(reduce_once(L));
+    return add(add(H, mont_mul(L, one)), mont_mul(T, big_r2<8>()));
 }
 // a^(p-2), Montgomery in / Montgomery out (0 -> 0): Fermat inversion, kept as the cross-check of mont_inverse.
 template <int N> ZK_HD Big<N> mont_inverse_fermat(Big<N> a) {

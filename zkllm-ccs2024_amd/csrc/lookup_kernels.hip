@@ -509,10 +509,12 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
                const Fr* __restrict__ A, const Fr* __restrict__ S, const Fr* __restrict__ B, const Fr* __restrict__ T, const Fr* __restrict__ m,
                const Fr* __restrict__ E, const Fr beta, const Fr v_mont, size_t n_out, Fr* __restrict__ nE, const HintSrc hs = HintSrc()) {
     constexpr int K = PHASE2 ? 11 : 5;
+    constexpr bool WIDE = !PHASE2;      // phase 1: the E-weighted products are summed unreduced, one reduction per lane (wide_redc)
     Fr acc[K];
 #pragma unroll
     for (int i = 0; i < K; ++i) acc[i] = big_zero<8>();
     Fr acc_e = big_zero<8>(), acc_em = big_zero<8>();       // HINTED: sum of E and of E * M over the pairs of unit inverses
+    WideAcc w0 = wide_zero(), w2 = wide_zero(), wx = wide_zero();      // sums of c0, c2 and of the cross products (a0 + da)(s0 + ds) E; HINTED: wx also takes E * M
     for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
         const Fr e = E[t];
         if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table: the top variable summed out
@@ -523,16 +525,29 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
             const Fr da = sub(a1, a0), ds = sub(s1, s0r), s0 = add(s0r, beta);
             if (HINTED && unit0 && unit1) {
                 const Fr M = mont_mul(add(a0, a1), add(s0, add(s1, beta)));
-                acc_em = add(acc_em, mont_mul(e, M));
+                if constexpr (WIDE) wide_mac(wx, e, M);
+                else acc_em = add(acc_em, mont_mul(e, M));
                 acc_e = add(acc_e, e);
             } else {
                 // E goes onto a0 and da first, and the middle term comes from (a0 + da)(s0 + ds): five products for the
                 // three weighted terms instead of seven
                 const Fr ea0 = mont_mul(e, a0), eda = mont_mul(e, da);
-                const Fr c0 = mont_mul(ea0, s0), c2 = mont_mul(eda, ds);
-                acc[0] = add(acc[0], c0);
-                acc[1] = add(acc[1], sub(sub(mont_mul(add(ea0, eda), add(s0, ds)), c0), c2));
-                acc[2] = add(acc[2], c2);
+                if constexpr (WIDE) {
+                    wide_mac(w0, ea0, s0);
+                    wide_mac(w2, eda, ds);
+                    if constexpr (HINTED) {
+                        // rare here (a pair whose inverses did not come from the table): its middle term goes in reduced
+                        const Fr c0 = mont_mul(ea0, s0), c2 = mont_mul(eda, ds);
+                        acc[1] = add(acc[1], sub(sub(mont_mul(add(ea0, eda), add(s0, ds)), c0), c2));
+                    } else {
+                        wide_mac(wx, add(ea0, eda), add(s0, ds));
+                    }
+                } else {
+                    const Fr c0 = mont_mul(ea0, s0), c2 = mont_mul(eda, ds);
+                    acc[0] = add(acc[0], c0);
+                    acc[1] = add(acc[1], sub(sub(mont_mul(add(ea0, eda), add(s0, ds)), c0), c2));
+                    acc[2] = add(acc[2], c2);
+                }
             }
             acc[3] = add(acc[3], a0);
             acc[4] = add(acc[4], da);
@@ -555,6 +570,12 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
             nT[t] = add(t0r, mont_mul(v_mont, dt));
             nm[t] = add(m0, mont_mul(v_mont, dm));
         }
+    }
+    if constexpr (WIDE) {
+        acc[0] = add(acc[0], wide_redc(w0));
+        acc[2] = add(acc[2], wide_redc(w2));
+        if constexpr (HINTED) acc_em = wide_redc(wx);
+        else acc[1] = add(acc[1], sub(sub(wide_redc(wx), acc[0]), acc[2]));
     }
     if (HINTED) {
         // E is in Montgomery form and the sums carry R^-1: sum(E) * R^-2 through one product with R^-1
@@ -606,6 +627,7 @@ k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __rest
     Fr acc[K + 1];
 #pragma unroll
     for (int i = 0; i <= K; ++i) acc[i] = big_zero<8>();
+    WideAcc w0 = wide_zero(), w2 = wide_zero(), wx = wide_zero();      // K == 2: sums of E x0 y0, E dx dy and E x1 y1
     for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
         // Coefficients of the running product from standard-form values: every coefficient is a sum of products of the same
         // number of factors, so each Montgomery product leaves one more R^-1 on all of them alike (K - 1 in the end), which
@@ -620,9 +642,11 @@ k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __rest
             // products instead of six.  x0 dy + y0 dx = x1 y1 - x0 y0 - dx dy.
             const Fr e2 = E[t];
             const Fr ex0 = mont_mul(e2, x0), edx = mont_mul(e2, dx);
-            c[0] = mont_mul(ex0, y0);
-            c[2] = mont_mul(edx, dy);
-            c[1] = sub(sub(mont_mul(add(ex0, edx), y1), c[0]), c[2]);
+            // the three products are summed unreduced (one reduction per lane after the loop); c stays zero
+            wide_mac(w0, ex0, y0);
+            wide_mac(w2, edx, dy);
+            wide_mac(wx, add(ex0, edx), y1);
+            c[0] = c[1] = c[2] = big_zero<8>();
         } else {
             {
                 const Fr x0 = p.in[0][t], x1 = p.in[0][t + n_out];
@@ -644,8 +668,15 @@ k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __rest
         }
         const Fr e = E[t];   // Montgomery form: e*R
         if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table
+        if constexpr (K != 2) {
 #pragma unroll
-        for (int j = 0; j <= K; ++j) acc[j] = add(acc[j], c[j]);
+            for (int j = 0; j <= K; ++j) acc[j] = add(acc[j], c[j]);
+        }
+    }
+    if constexpr (K == 2) {
+        acc[0] = wide_redc(w0);
+        acc[2] = wide_redc(w2);
+        acc[1] = sub(sub(wide_redc(wx), acc[0]), acc[2]);
     }
     if (K > 1) {
         const Fr r2 = big_r2<8>();
