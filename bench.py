@@ -34,7 +34,7 @@ VALU_PEAK_TOPS = 256 * 4 * 16 * 2.4e9 / 1e12
 # WRITE_SIZE on the kernel alone (python3 bench.py --pmc-probe; summary in profiles/k_open_fold29_pmc_traffic.txt), each
 # counter scaled by what it reads for zk_fr_add over 2^24 elements (1 GiB read, 512 MiB written).  It holds for launches of
 # that size; `traffic` of the in-layer entry, whose launches are of every size, is left null and the algorithmic figure given.
-FOLD_TRAFFIC_BYTES_PER_PAIR_AT_262144 = 618.0
+FOLD_TRAFFIC_BYTES_PER_PAIR_AT_262144 = 764.6      # (53742 KiB x 2.000 fetched + 88253 KiB written) / 262144 pairs, profiles/k_open_fold29_pmc_traffic.txt
 FOLD_ALGO_BYTES_PER_PAIR = 2 * 112 + 112 + 3 * 32      # two points in, one out (affine, 29-bit limbs: 112 B), two scalars in, one out
 MAD_PER_FP_MUL = 300                                   # 2 * 12^2 + 12 limb products of a 381-bit Montgomery product
 MAD_PER_FR_MUL = 136                                   # 2 * 8^2 + 8

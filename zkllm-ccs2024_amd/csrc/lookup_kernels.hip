@@ -514,7 +514,7 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
 #pragma unroll
     for (int i = 0; i < K; ++i) acc[i] = big_zero<8>();
     Fr acc_e = big_zero<8>(), acc_em = big_zero<8>();       // HINTED: sum of E and of E * M over the pairs of unit inverses
-    WideAcc w0 = wide_zero(), w2 = wide_zero(), wx = wide_zero();      // sums of c0, c2 and of the cross products (a0 + da)(s0 + ds) E; HINTED: wx also takes E * M
+    WideAcc w0 = wide_zero(), w2 = wide_zero(), wx = wide_zero();      // sums of c0, c2 and of the cross products (a0 + da)(s0 + ds) E; HINTED: wx alone, the sum of E * M
     for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
         const Fr e = E[t];
         if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table: the top variable summed out
@@ -532,17 +532,12 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
                 // E goes onto a0 and da first, and the middle term comes from (a0 + da)(s0 + ds): five products for the
                 // three weighted terms instead of seven
                 const Fr ea0 = mont_mul(e, a0), eda = mont_mul(e, da);
-                if constexpr (WIDE) {
+                if constexpr (WIDE && !HINTED) {
                     wide_mac(w0, ea0, s0);
                     wide_mac(w2, eda, ds);
-                    if constexpr (HINTED) {
-                        // rare here (a pair whose inverses did not come from the table): its middle term goes in reduced
-                        const Fr c0 = mont_mul(ea0, s0), c2 = mont_mul(eda, ds);
-                        acc[1] = add(acc[1], sub(sub(mont_mul(add(ea0, eda), add(s0, ds)), c0), c2));
-                    } else {
-                        wide_mac(wx, add(ea0, eda), add(s0, ds));
-                    }
+                    wide_mac(wx, add(ea0, eda), add(s0, ds));
                 } else {
+                    // (HINTED: rare, a pair whose inverses did not both come from the table)
                     const Fr c0 = mont_mul(ea0, s0), c2 = mont_mul(eda, ds);
                     acc[0] = add(acc[0], c0);
                     acc[1] = add(acc[1], sub(sub(mont_mul(add(ea0, eda), add(s0, ds)), c0), c2));
@@ -571,11 +566,11 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
             nm[t] = add(m0, mont_mul(v_mont, dm));
         }
     }
-    if constexpr (WIDE) {
-        acc[0] = add(acc[0], wide_redc(w0));
-        acc[2] = add(acc[2], wide_redc(w2));
-        if constexpr (HINTED) acc_em = wide_redc(wx);
-        else acc[1] = add(acc[1], sub(sub(wide_redc(wx), acc[0]), acc[2]));
+    if constexpr (WIDE && HINTED) acc_em = wide_redc(wx);
+    if constexpr (WIDE && !HINTED) {
+        acc[0] = wide_redc(w0);
+        acc[2] = wide_redc(w2);
+        acc[1] = sub(sub(wide_redc(wx), acc[0]), acc[2]);
     }
     if (HINTED) {
         // E is in Montgomery form and the sums carry R^-1: sum(E) * R^-2 through one product with R^-1
