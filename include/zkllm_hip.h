@@ -115,6 +115,13 @@ int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, 
 /* the same for a stack of `batch` products, A [batch][M][N], B [batch][N][P], C [batch][M][P] (the per-head products of
  * zkAttn::compute, zksoftmax.cu:234-238, for all heads at once); the bound check covers the whole stacks, so one path serves all */
 int zk_fr_matmul_batched(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used_host, void* stream);
+/* The right operand of many products (a layer's weight in zkFC::operator(), zkfc.cu:44-58) examined once: its largest magnitude
+ * for the small-integer bound and, when it holds small integers, its int8 digit planes in the GEMM's layout.  No counterpart in
+ * the reference, which converts nothing.  B stays alive and unmodified while the handle is used; zk_fr_matmul_rhs is
+ * zk_fr_matmul(C, A, B, M, N, P, ...) with B's part of the preparation taken from the handle (bit-identical results). */
+int zk_fr_matmul_rhs_prepare(void** prepared, const void* B, uint32_t N, uint32_t P, void* stream);
+int zk_fr_matmul_rhs(void* C, const void* A, const void* prepared, uint32_t M, int mode, int* path_used, void* stream);
+int zk_fr_matmul_rhs_free(void* prepared);
 
 /* ---- inner-product sumcheck (zkip_poly_kernel + 3 sums, zkfc.cu:94-138) ----------------------------- */
 int zk_ip_round(uint32_t* poly3_host, const void* a, const void* b, size_t n_in, size_t n_out, void* stream);

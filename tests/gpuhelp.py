@@ -158,7 +158,7 @@ class Prover:
                      "zkp_g1_from_host", "zkp_g1_from_file", "zkp_g1_devptr", "zkp_commitment_random", "zkp_g1_binop", "zkp_g1_pointop", "zkp_g1_affineop",
                      "zkp_g1_scalar_mul", "zkp_g1_rowwise_sum", "zkp_commit_int", "zkp_commit",
                      "zkp_rescale", "zkp_rescale_prove", "zkp_relu", "zkp_attn", "zkp_zkfc_stacked", "zkp_range_prep", "zkp_batch_inv", "zkp_softmax",
-                     "zkp_layer_create", "zkp_layer_create_random", "zkp_layer_run"):
+                     "zkp_layer_create", "zkp_layer_create_random", "zkp_layer_run", "zkp_fc_forward_over_view"):
             getattr(L, name).restype = c_void_p
         L.zkp_transcript_size.restype = ctypes.c_long
         L.zkp_fr_size.restype = c_uint
@@ -245,6 +245,15 @@ class Prover:
 
     def matmul(self, a, b, M, N, P):
         return self.H(self.lib.zkp_fr_matmul(c_void_p(a.h), c_void_p(b.h), c_uint(M), c_uint(N), c_uint(P)))
+
+    def keep_as_matmul_rhs(self, a):
+        self.check(self.lib.zkp_fr_keep_as_matmul_rhs(c_void_p(a.h)))
+
+    def add_inplace(self, a, b):
+        self.check(self.lib.zkp_fr_add_inplace(c_void_p(a.h), c_void_p(b.h)))
+
+    def fc_forward_over_view(self, w, x, in_dim, out_dim):
+        return self.H(self.lib.zkp_fc_forward_over_view(c_void_p(w.h), c_void_p(x.h), c_uint(in_dim), c_uint(out_dim)))
 
     def matmul_stack(self, a, b, num, M, N, P):
         return self.H(self.lib.zkp_fr_matmul_stack(c_void_p(a.h), c_void_p(b.h), c_uint(num), c_uint(M), c_uint(N), c_uint(P)))

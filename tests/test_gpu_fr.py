@@ -388,6 +388,52 @@ def test_matmul_int8_plane_path_on_ragged_stacks_and_wide_operands(pv):
             os.environ["ZKLLM_MATMUL_PLANES"] = old
 
 
+def test_matmul_with_a_kept_right_operand_and_layers_over_views(pv):
+    """A weight kept as the right operand of matrix products (FrTensor::keep_as_matmul_rhs: largest magnitude and digit planes
+    computed once, zk_fr_matmul_rhs_prepare / zk_fr_matmul_rhs) gives the products of the plain path, on the matrix-core path and
+    on the others; what was kept is dropped when the weight is modified in place; a zkFC over a view of the weight
+    (FrTensor::view) computes with the weight's own elements and leaves them alive."""
+    import os
+    rng = np.random.default_rng(17)
+    pv.lib.zkp_set_matmul_mode(ctypes.c_int(0))
+    old = os.environ.get("ZKLLM_MATMUL_PLANES")
+    try:
+        for planes, (M, N, P), (wlo, whi) in [("1", (70, 130, 50), (-2 ** 13, 2 ** 13)), ("1", (33, 257, 64), (-2 ** 33, 2 ** 33)),
+                                               ("0", (40, 100, 24), (-2 ** 13, 2 ** 13))]:
+            os.environ["ZKLLM_MATMUL_PLANES"] = planes
+            W = rng.integers(wlo, whi, (N, P)).astype(np.int64)
+            D = rng.integers(-50, 50, (N, P)).astype(np.int64)
+            hW, hD = pv.from_i64(W), pv.from_i64(D)
+            pv.keep_as_matmul_rhs(hW)
+            for rep in range(3):                      # first product prepares, the others reuse
+                X = rng.integers(-2 ** 17, 2 ** 17, (M, N)).astype(np.int64)
+                got = pv.matmul(pv.from_i64(X), hW, M, N, P).host()
+                assert pv.lib.zkp_last_matmul_path() == 2
+                assert fr_ints(got) == [int(v) % R_MOD for v in (X.astype(object) @ W.astype(object)).reshape(-1)], (planes, rep)
+            got = pv.fc_forward_over_view(hW, pv.from_i64(X), N, P).host()
+            assert fr_ints(got) == [int(v) % R_MOD for v in (X.astype(object) @ W.astype(object)).reshape(-1)]
+            pv.add_inplace(hW, hD)                    # the weight changes: nothing stale may be used
+            W2 = W + D
+            got = pv.matmul(pv.from_i64(X), hW, M, N, P).host()
+            assert fr_ints(got) == [int(v) % R_MOD for v in (X.astype(object) @ W2.astype(object)).reshape(-1)]
+            assert fr_ints(hW.host()) == [int(v) % R_MOD for v in W2.reshape(-1)]
+        # a right operand of full-width residues: kept, and the generic path still runs
+        Af = mt_random_vec(np.random.RandomState(5), 9 * 20)
+        Bf = mt_random_vec(np.random.RandomState(6), 20 * 7)
+        hB = pv.from_fr(Bf)
+        pv.keep_as_matmul_rhs(hB)
+        for rep in range(2):
+            got = pv.matmul(pv.from_fr(Af), hB, 9, 20, 7).host()
+            assert pv.lib.zkp_last_matmul_path() == 1
+            Ai, Bi = np.array(fr_ints(Af), dtype=object).reshape(9, 20), np.array(fr_ints(Bf), dtype=object).reshape(20, 7)
+            assert fr_ints(got) == [int(v) % R_MOD for v in (Ai @ Bi).reshape(-1)]
+    finally:
+        if old is None:
+            os.environ.pop("ZKLLM_MATMUL_PLANES", None)
+        else:
+            os.environ["ZKLLM_MATMUL_PLANES"] = old
+
+
 def test_stacks_of_matrices_transpose_and_multiply_like_their_members(pv):
     """zk_fr_matmul_batched / zk_fr_transpose_batched on every path of the dispatcher (both operands in 31 bits, wide left
     operand, wide right operand, full-width residues): each product of the stack against big-int arithmetic."""

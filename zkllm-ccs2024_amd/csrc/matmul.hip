@@ -19,6 +19,7 @@
 //    recombined value is the true integer result, below 2^62 by the bound above.
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <mutex>
 #include <utility>
 #include <vector>
@@ -552,8 +553,11 @@ static int digits_for(unsigned long long absmax) {      // planes needed for |x|
     return reach >= absmax ? p : 0;
 }
 // returns ZK status; *done = false when the path does not apply (the caller then takes a VALU kernel)
+// A right operand kept by the caller for many products (a layer's weight): its largest magnitude and, when it is a matrix of
+// small integers, its digit planes in the GEMM's layout -- neither is computed again per product.
+struct MatmulRhs { const void* B = nullptr; uint32_t N = 0, P = 0, Kp = 0; unsigned long long mb = ~0ull; int pb = 0; void* planes = nullptr; };
 static int run_int8_plane_path(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, unsigned long long ma, unsigned long long mb,
-                               hipStream_t st, bool* done) {
+                               hipStream_t st, bool* done, const MatmulRhs* rhs = nullptr) {
     *done = false;
     const int pa = digits_for(ma), pb = digits_for(mb);
     if (!pa || !pb) return 0;
@@ -561,12 +565,13 @@ static int run_int8_plane_path(void* C, const void* A, const void* B, uint32_t b
     if (M > (1u << 30) || P > (1u << 30)) return 0;
     const uint32_t Kp = (N + GBK - 1) / GBK * GBK;
     const size_t rows_a = (size_t)batch * M;
-    Scratch pla(rows_a * pa * Kp, st), plb((size_t)batch * pb * P * Kp, st);
+    const bool have_b = rhs && rhs->planes && rhs->pb == pb && rhs->Kp == Kp && batch == 1;
+    Scratch pla(rows_a * pa * Kp, st), plb(have_b ? 1 : (size_t)batch * pb * P * Kp, st);
     if (pla.rc) return pla.rc;
     if (plb.rc) return plb.rc;
     hipLaunchKernelGGL(k_split_rows, dim3(cdiv(rows_a * (Kp / 4), 256)), dim3(256), 0, st, pla.as<int8_t>(), (const Fr*)A, rows_a, M, N, Kp, pa);
-    hipLaunchKernelGGL(k_split_cols, dim3(cdiv(P, 64), Kp / 64, batch), dim3(256), 0, st, plb.as<int8_t>(), (const Fr*)B, N, P, Kp, pb);
-    const PlaneGemm g{pla.as<int8_t>(), plb.as<int8_t>(), (Fr*)C, M, P, Kp, pa, pb};
+    if (!have_b) hipLaunchKernelGGL(k_split_cols, dim3(cdiv(P, 64), Kp / 64, batch), dim3(256), 0, st, plb.as<int8_t>(), (const Fr*)B, N, P, Kp, pb);
+    const PlaneGemm g{pla.as<int8_t>(), have_b ? (const int8_t*)rhs->planes : plb.as<int8_t>(), (Fr*)C, M, P, Kp, pa, pb};
     hipEvent_t t0 = nullptr, t1 = nullptr;
     if (g_gemm_timer.on) {
         ZK_HIP(hipEventCreate(&t0));
@@ -606,7 +611,8 @@ int zk_fr_matmul_generic(void* C, const void* A, const void* B, uint32_t M, uint
 // path_used (optional, host): 1 generic, 2 small-integer.
 // `batch` products of equally shaped matrices stored one after the other; the bound is taken over the whole stacks, so
 // one path serves every product of the call
-static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv) {
+static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv,
+                           const MatmulRhs* rhs = nullptr) {
     hipStream_t st = (hipStream_t)stv;
     if (batch == 0 || M == 0 || P == 0) return 0;
     ZK_ARG(N > 0, "zk_fr_matmul: inner dimension is 0");
@@ -621,7 +627,7 @@ static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch
         ZK_HIP(hipMemsetAsync(mx.p, 0, 3 * sizeof(unsigned long long), st));
         const size_t na = (size_t)batch * M * N, nb = (size_t)batch * N * P;
         hipLaunchKernelGGL(k_absmax, dim3(absmax_grid(na)), dim3(256), 0, st, mx.as<unsigned long long>(), (const Fr*)A, na);
-        hipLaunchKernelGGL(k_absmax, dim3(absmax_grid(nb)), dim3(256), 0, st, mx.as<unsigned long long>() + 1, (const Fr*)B, nb);
+        if (!rhs) hipLaunchKernelGGL(k_absmax, dim3(absmax_grid(nb)), dim3(256), 0, st, mx.as<unsigned long long>() + 1, (const Fr*)B, nb);
         hipLaunchKernelGGL(k_rowabs, dim3(batch * M), dim3(256), 0, st, mx.as<unsigned long long>() + 2, (const Fr*)A, N);
         ZK_LAUNCH_CHECK();
         void* stage = nullptr;
@@ -629,7 +635,7 @@ static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch
         if (rc) return rc;
         ZK_HIP(hipMemcpyAsync(stage, mx.p, 24, hipMemcpyDeviceToHost, st));
         ZK_HIP(hipStreamSynchronize(st));
-        const unsigned long long ma = ((unsigned long long*)stage)[0], mb = ((unsigned long long*)stage)[1], ra = ((unsigned long long*)stage)[2];
+        const unsigned long long ma = ((unsigned long long*)stage)[0], mb = rhs ? rhs->mb : ((unsigned long long*)stage)[1], ra = ((unsigned long long*)stage)[2];
         if (ma != ~0ull && mb != ~0ull && ra != ~0ull) {
             // |sum_j a_ij b_jk| <= (max_i sum_j |a_ij|) * max|b| must stay below 2^62
             const unsigned __int128 bound = (unsigned __int128)ra * mb;
@@ -653,7 +659,7 @@ static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch
     const int planes_log2 = planes_env ? atoi(planes_env) : 30;
     if (planes_log2 > 0 && (unsigned __int128)batch * M * N * P >= ((unsigned __int128)1 << planes_log2) && M >= 32 && P >= 32) {
         bool done = false;
-        const int rc = run_int8_plane_path(C, A, B, batch, M, N, P, ma_, mb_, st, &done);
+        const int rc = run_int8_plane_path(C, A, B, batch, M, N, P, ma_, mb_, st, &done, rhs);
         if (rc) return rc;
         if (done) return 0;
     }
@@ -685,6 +691,52 @@ int zk_prof_gemm_read(double* total_ms, unsigned long long* launches, double* ma
     *launches = g_gemm_timer.ev.size();
     *macs = g_gemm_timer.macs;
     return 0;
+}
+// B (N x P) examined once for any number of products A * B: its largest magnitude, and its digit planes when it holds
+// small integers.  B must stay alive and unmodified while the handle is in use.
+int zk_fr_matmul_rhs_prepare(void** prepared, const void* B, uint32_t N, uint32_t P, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(prepared != nullptr && B != nullptr && N > 0 && P > 0, "zk_fr_matmul_rhs_prepare: null argument or empty matrix");
+    std::unique_ptr<MatmulRhs> r(new MatmulRhs);
+    r->B = B; r->N = N; r->P = P;
+    r->Kp = (N + GBK - 1) / GBK * GBK;
+    {
+        Scratch mx(sizeof(unsigned long long), st);
+        if (mx.rc) return mx.rc;
+        ZK_HIP(hipMemsetAsync(mx.p, 0, sizeof(unsigned long long), st));
+        const size_t nb = (size_t)N * P;
+        hipLaunchKernelGGL(k_absmax, dim3(absmax_grid(nb)), dim3(256), 0, st, mx.as<unsigned long long>(), (const Fr*)B, nb);
+        ZK_LAUNCH_CHECK();
+        void* stage = nullptr;
+        int rc = staging(&stage, 8);
+        if (rc) return rc;
+        ZK_HIP(hipMemcpyAsync(stage, mx.p, 8, hipMemcpyDeviceToHost, st));
+        ZK_HIP(hipStreamSynchronize(st));
+        r->mb = *(unsigned long long*)stage;
+    }
+    const int pb = r->mb == ~0ull ? 0 : digits_for(r->mb);
+    if (pb && N < (1u << 17) && P <= (1u << 30)) {
+        int rc = pool_alloc(&r->planes, (size_t)pb * P * r->Kp, st);
+        if (rc) return rc;
+        r->pb = pb;
+        hipLaunchKernelGGL(k_split_cols, dim3(cdiv(P, 64), r->Kp / 64, 1), dim3(256), 0, st, (int8_t*)r->planes, (const Fr*)B, N, P, r->Kp, pb);
+        if (hipGetLastError() != hipSuccess) { (void)pool_free(r->planes, st); return hip_fail(hipErrorLaunchFailure, "k_split_cols", __FILE__, __LINE__); }
+    }
+    *prepared = r.release();
+    return 0;
+}
+int zk_fr_matmul_rhs_free(void* prepared) {
+    MatmulRhs* r = (MatmulRhs*)prepared;
+    if (!r) return 0;
+    if (r->planes) (void)pool_free(r->planes, nullptr);
+    delete r;
+    return 0;
+}
+// zk_fr_matmul with a prepared right operand (its shape comes with the handle)
+int zk_fr_matmul_rhs(void* C, const void* A, const void* prepared, uint32_t M, int mode, int* path_used, void* stv) {
+    const MatmulRhs* r = (const MatmulRhs*)prepared;
+    ZK_ARG(r != nullptr, "zk_fr_matmul_rhs: null handle");
+    return matmul_dispatch(C, A, r->B, 1, M, r->N, r->P, mode, path_used, stv, r);
 }
 int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv) {
     return matmul_dispatch(C, A, B, 1, M, N, P, mode, path_used, stv);

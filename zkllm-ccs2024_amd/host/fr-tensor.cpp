@@ -197,13 +197,22 @@ FrTensor::FrTensor(uint size, const double* cpu_data, unsigned long sf) : gpu_da
 FrTensor::FrTensor(const FrTensor& t) : gpu_data(fr_alloc(t.size)), size(t.size) {
     ZKC(zk_memcpy_d2d(gpu_data, t.gpu_data, sizeof(Fr_t) * (size_t)size, nullptr));
 }
-FrTensor::FrTensor(FrTensor&& t) noexcept : gpu_data(t.gpu_data), size(t.size) { t.gpu_data = nullptr; }
+FrTensor::FrTensor(FrTensor&& t) noexcept : gpu_data(t.gpu_data), size(t.size), borrowed(t.borrowed), rhs_cache(std::move(t.rhs_cache)) { t.gpu_data = nullptr; }
+void MatmulRhsCache::reset() {
+    if (prepared) zk_fr_matmul_rhs_free(prepared);
+    prepared = nullptr;
+}
+FrTensor::FrTensor(const FrTensor& t, ViewTag) : gpu_data(t.gpu_data), size(t.size), borrowed(true), rhs_cache(t.rhs_cache) {}
+FrTensor FrTensor::view(const FrTensor& t) { return FrTensor(t, ViewTag{}); }
+void FrTensor::keep_as_matmul_rhs() {
+    if (!rhs_cache) rhs_cache = std::make_shared<MatmulRhsCache>();
+}
 FrTensor::FrTensor(const string& filename) : gpu_data(nullptr), size((uint)(findsize(filename) / sizeof(Fr_t))) {
     gpu_data = fr_alloc(size);
     loadbin(filename, gpu_data, sizeof(Fr_t) * (size_t)size);
 }
 FrTensor::~FrTensor() {
-    if (gpu_data) zk_free(gpu_data);
+    if (gpu_data && !borrowed) zk_free(gpu_data);
     gpu_data = nullptr;
 }
 
@@ -249,21 +258,22 @@ Fr_t FrTensor::operator()(uint idx) const {
 
 FrTensor FrTensor::operator+(const FrTensor& t) const { SAME_SIZE(t); FrTensor out(size); ZKC(zk_fr_add(out.gpu_data, gpu_data, t.gpu_data, size, nullptr)); return out; }
 FrTensor FrTensor::operator+(const Fr_t& x) const { FrTensor out(size); ZKC(zk_fr_add_s(out.gpu_data, gpu_data, x.val, size, nullptr)); return out; }
-FrTensor& FrTensor::operator+=(const FrTensor& t) { SAME_SIZE(t); ZKC(zk_fr_add(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
-FrTensor& FrTensor::operator+=(const Fr_t& x) { ZKC(zk_fr_add_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator+=(const FrTensor& t) { SAME_SIZE(t); if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_add(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator+=(const Fr_t& x) { if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_add_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
 FrTensor FrTensor::operator-() const { FrTensor out(size); ZKC(zk_fr_neg(out.gpu_data, gpu_data, size, nullptr)); return out; }
 FrTensor FrTensor::operator-(const FrTensor& t) const { SAME_SIZE(t); FrTensor out(size); ZKC(zk_fr_sub(out.gpu_data, gpu_data, t.gpu_data, size, nullptr)); return out; }
 FrTensor FrTensor::operator-(const Fr_t& x) const { FrTensor out(size); ZKC(zk_fr_sub_s(out.gpu_data, gpu_data, x.val, size, nullptr)); return out; }
-FrTensor& FrTensor::operator-=(const FrTensor& t) { SAME_SIZE(t); ZKC(zk_fr_sub(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
-FrTensor& FrTensor::operator-=(const Fr_t& x) { ZKC(zk_fr_sub_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
-FrTensor& FrTensor::mont() { ZKC(zk_fr_mont(gpu_data, gpu_data, size, nullptr)); return *this; }
-FrTensor& FrTensor::unmont() { ZKC(zk_fr_unmont(gpu_data, gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator-=(const FrTensor& t) { SAME_SIZE(t); if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_sub(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator-=(const Fr_t& x) { if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_sub_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
+FrTensor& FrTensor::mont() { if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_mont(gpu_data, gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::unmont() { if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_unmont(gpu_data, gpu_data, size, nullptr)); return *this; }
 FrTensor FrTensor::operator*(const FrTensor& t) const { SAME_SIZE(t); FrTensor out(size); ZKC(zk_fr_mul(out.gpu_data, gpu_data, t.gpu_data, size, nullptr)); return out; }
 FrTensor FrTensor::operator*(const Fr_t& x) const { FrTensor out(size); ZKC(zk_fr_mul_s(out.gpu_data, gpu_data, x.val, size, nullptr)); return out; }
-FrTensor& FrTensor::operator*=(const FrTensor& t) { SAME_SIZE(t); ZKC(zk_fr_mul(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
-FrTensor& FrTensor::operator*=(const Fr_t& x) { ZKC(zk_fr_mul_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator*=(const FrTensor& t) { SAME_SIZE(t); if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_mul(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator*=(const Fr_t& x) { if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_mul_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
 FrTensor& FrTensor::operator=(const FrTensor& t) {
     if (size != t.size) throw std::runtime_error("operator=: Incompatible dimensions");
+    if (rhs_cache) rhs_cache->reset();
     ZKC(zk_memcpy_d2d(gpu_data, t.gpu_data, sizeof(Fr_t) * (size_t)size, nullptr));
     return *this;
 }
@@ -415,7 +425,14 @@ FrTensor FrTensor::matmul(const FrTensor& x, const FrTensor& y, uint M, uint N, 
     if (x.size != M * N || y.size != N * P) throw std::runtime_error("matmul: incompatible dimensions");
     FrTensor out(M * P);
     int path = 0;
-    ZKC(zk_fr_matmul(out.gpu_data, x.gpu_data, y.gpu_data, M, N, P, G().matmul_mode, &path, nullptr));
+    MatmulRhsCache* rc = y.rhs_cache.get();
+    if (rc && rc->prepared && (rc->N != N || rc->P != P)) rc->reset();       // the same elements read as another shape
+    if (rc && !rc->prepared) {
+        ZKC(zk_fr_matmul_rhs_prepare(&rc->prepared, y.gpu_data, N, P, nullptr));
+        rc->N = N; rc->P = P;
+    }
+    if (rc) ZKC(zk_fr_matmul_rhs(out.gpu_data, x.gpu_data, rc->prepared, M, G().matmul_mode, &path, nullptr));
+    else ZKC(zk_fr_matmul(out.gpu_data, x.gpu_data, y.gpu_data, M, N, P, G().matmul_mode, &path, nullptr));
     G().last_matmul_path = path;
     return out;
 }

@@ -1,6 +1,7 @@
 // FrTensor: owning device array of BLS12-381 scalars in standard form.  Public interface of the
 // reference class (fr-tensor.cuh:69-177) on top of the gfx950 C ABI (include/zkllm_hip.h).
 #pragma once
+#include <memory>
 #include <iomanip>
 #include <iostream>
 #include <stdexcept>
@@ -64,10 +65,23 @@ void zk_write_proof_file(const std::string& path);
 
 void zk_check(int rc, const char* where);   // throws std::runtime_error on a non-zero C-ABI status
 
+// What a tensor that serves as the right operand of many matrix products keeps between them (FrTensor::keep_as_matmul_rhs):
+// the handle of zk_fr_matmul_rhs_prepare.  Shared by the tensor and its views.
+struct MatmulRhsCache {
+    void* prepared = nullptr;
+    uint N = 0, P = 0;
+    void reset();
+    ~MatmulRhsCache() { reset(); }
+};
+
 class FrTensor {
    public:
     Fr_t* gpu_data;
     const uint size;
+    // additions.  borrowed: the elements belong to another tensor that outlives this one (FrTensor::view); rhs_cache: see
+    // keep_as_matmul_rhs
+    bool borrowed = false;
+    std::shared_ptr<MatmulRhsCache> rhs_cache;
 
     FrTensor(uint size);
     FrTensor(uint size, const Fr_t* cpu_data);
@@ -120,6 +134,16 @@ class FrTensor {
     FrTensor trunc(uint begin_idx, uint end_idx) const;
 
     static FrTensor matmul(const FrTensor& x, const FrTensor& y, uint M, uint N, uint P);
+    // additions.  view: a tensor over t's elements that owns nothing (t must outlive it and stay unmodified); moving it
+    // keeps it a view, copying it makes an owning copy.  For callers such as zkFC that take their weight by value although
+    // it lives elsewhere for the whole proof (the reference copies it, zkfc.cu:7-17).
+    static FrTensor view(const FrTensor& t);
+    struct ViewTag {};
+    FrTensor(const FrTensor& t, ViewTag);          // what view() returns
+    // keep_as_matmul_rhs: from now on matmul(x, *this, ...) examines this tensor once (largest magnitude, int8 digit planes)
+    // and keeps that for later products; for tensors that are not modified afterwards (weights).  The in-place operators
+    // drop what was kept.
+    void keep_as_matmul_rhs();
     // additions for stacks of `num` equally shaped matrices stored one after the other: every M x N matrix transposed,
     // and the num products x_i (M x N) * y_i (N x P)
     FrTensor transpose_stack(uint num, uint M, uint N) const;

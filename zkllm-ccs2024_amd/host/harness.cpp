@@ -152,6 +152,16 @@ void* zkp_fr_scalarop(int op, void* a, const u32* s) {
     throw std::runtime_error("bad op");
     ZKP_END_PTR
 }
+// the additions around a weight tensor: kept as the right operand of matrix products, modified in place (a += b), and a fully
+// connected layer built over a view of it (zkFC(in, out, FrTensor::view(w))): Y = X W through that layer
+int zkp_fr_keep_as_matmul_rhs(void* a) { ZKP_TRY FT(a).keep_as_matmul_rhs(); ZKP_END }
+int zkp_fr_add_inplace(void* a, void* b) { ZKP_TRY FT(a) += FT(b); ZKP_END }
+void* zkp_fc_forward_over_view(void* w, void* x, u32 in_dim, u32 out_dim) {
+    ZKP_TRY
+    zkFC layer(in_dim, out_dim, FrTensor::view(FT(w)));
+    return new FrTensor(layer(FT(x)));
+    ZKP_END_PTR
+}
 int zkp_fr_sum(void* a, u32* out) { ZKP_TRY Fr_t s = FT(a).sum(); memcpy(out, s.val, 32); ZKP_END }
 int zkp_fr_me(void* a, const u32* u, int k, u32* out) { ZKP_TRY Fr_t s = FT(a)(frs(u, k)); memcpy(out, s.val, 32); ZKP_END }
 void* zkp_fr_partial_me(void* a, const u32* u, int k, u32 cur_dim, u32 window) { ZKP_TRY return new FrTensor(FT(a).partial_me(frs(u, k), cur_dim, window)); ZKP_END_PTR }

@@ -85,7 +85,7 @@ void layer_config_from_env(LayerConfig& c) {
 // rmsnorm.cu:26-49
 FrTensor rmsnorm_block(const LayerConfig& c, const Weight& w, const FrTensor& X, const FrTensor& rms_inv) {
     Rescaling rs1(c.sf_linear), rs2(c.sf_linear);
-    zkFC g(1, c.embed_dim, w.weight);
+    zkFC g(1, c.embed_dim, FrTensor::view(w.weight));
     auto g_inv_rms = g(rms_inv);
     auto g_inv_rms_ = rs1(g_inv_rms);
     auto Y = g_inv_rms_ * X;
@@ -103,7 +103,7 @@ FrTensor rmsnorm_block(const LayerConfig& c, const Weight& w, const FrTensor& X,
 
 // self-attn.cu:19-76 (linear mode)
 void attn_linear_block(const LayerConfig& c, const Weight& q, const Weight& k, const Weight& v, const FrTensor& input, FrTensor& Q_, FrTensor& K_, FrTensor& V_) {
-    zkFC q_layer(c.embed_dim, c.embed_dim, q.weight), k_layer(c.embed_dim, c.embed_dim, k.weight), v_layer(c.embed_dim, c.embed_dim, v.weight);
+    zkFC q_layer(c.embed_dim, c.embed_dim, FrTensor::view(q.weight)), k_layer(c.embed_dim, c.embed_dim, FrTensor::view(k.weight)), v_layer(c.embed_dim, c.embed_dim, FrTensor::view(v.weight));
     Rescaling q_rescale(c.sf_linear), k_rescale(c.sf_linear), v_rescale(c.sf_linear);
     auto Q = q_layer(input);
     Q_ = q_rescale(Q);
@@ -301,7 +301,7 @@ FrTensor attn_reference_block(const LayerConfig& c, const FrTensor& Q, const FrT
 }
 
 FrTensor oproj_block(const LayerConfig& c, const Weight& o, const FrTensor& attn_out) {
-    zkFC o_layer(c.embed_dim, c.embed_dim, o.weight);
+    zkFC o_layer(c.embed_dim, c.embed_dim, FrTensor::view(o.weight));
     Rescaling o_rescale(c.sf_linear);
     auto O = o_layer(attn_out);
     auto O_ = o_rescale(O);
@@ -314,7 +314,7 @@ FrTensor oproj_block(const LayerConfig& c, const Weight& o, const FrTensor& attn
 // ffn.cu:44-93
 FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, const Weight& down, const FrTensor& swiglu_values, const FrTensor& input,
                    std::unique_ptr<FrTensor>* down_out_unrescaled) {
-    zkFC up_layer(c.embed_dim, c.hidden_dim, up.weight), gate_layer(c.embed_dim, c.hidden_dim, gate.weight), down_layer(c.hidden_dim, c.embed_dim, down.weight);
+    zkFC up_layer(c.embed_dim, c.hidden_dim, FrTensor::view(up.weight)), gate_layer(c.embed_dim, c.hidden_dim, FrTensor::view(gate.weight)), down_layer(c.hidden_dim, c.embed_dim, FrTensor::view(down.weight));
     Rescaling up_rescale(c.sf_linear), gate_rescale(c.sf_gate), hidden_rescale(c.sf_linear), down_rescale(c.sf_linear);
     tLookupRangeMapping swiglu(c.swiglu_low, c.swiglu_len, swiglu_values);
 
@@ -415,6 +415,7 @@ static Weight random_weight(std::mt19937_64& rng, uint in_dim, uint out_dim, uin
     std::vector<int> wi((size_t)in_dim * out_dim);
     for (auto& x : wi) x = norm ? 65536 : (int)std::nearbyint(nd(rng) * 65536.0);   // scale 2^16 (llama-commit.py:34)
     FrTensor weight((uint)wi.size(), wi.data());
+    if (!norm) weight.keep_as_matmul_rhs();        // the right operand of the layer's projections, run after run
     const bool ragged = in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim));
     std::shared_ptr<const FrTensor> padded = ragged ? std::make_shared<const FrTensor>(weight.pad({in_dim, out_dim})) : nullptr;
     const double t1 = now_ms();

@@ -11,6 +11,10 @@ zkFC::zkFC(uint input_size, uint output_size, const FrTensor& weight)
     : inputSize(input_size), outputSize(output_size), has_bias(false), weights(weight), bias(output_size) {
     if (weight.size != input_size * output_size) throw std::runtime_error("weight size does not match");
 }
+zkFC::zkFC(uint input_size, uint output_size, FrTensor&& weight)
+    : inputSize(input_size), outputSize(output_size), has_bias(false), weights(std::move(weight)), bias(output_size) {
+    if (weights.size != input_size * output_size) throw std::runtime_error("weight size does not match");
+}
 zkFC::zkFC(uint input_size, uint output_size, const FrTensor& weight, const FrTensor& bias)
     : inputSize(input_size), outputSize(output_size), has_bias(true), weights(weight), bias(bias) {
     if (weight.size != input_size * output_size) throw std::runtime_error("weight size does not match");

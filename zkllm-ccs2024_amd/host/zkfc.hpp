@@ -11,6 +11,8 @@ class zkFC {
     FrTensor weights, bias;
 
     zkFC(uint input_size, uint output_size, const FrTensor& weight);
+    // addition: takes the weight over instead of copying it (with FrTensor::view(w) the layer proves against the weight where it lies)
+    zkFC(uint input_size, uint output_size, FrTensor&& weight);
     zkFC(uint input_size, uint output_size, const FrTensor& weight, const FrTensor& bias);
     FrTensor operator()(const FrTensor& X) const;
     vector<Claim> prove(const FrTensor& X, const FrTensor& Y) const;
