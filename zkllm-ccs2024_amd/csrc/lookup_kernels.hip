@@ -1194,7 +1194,25 @@ int zk_hadamard_round(uint32_t* coefs_host, void* const* new_Xs, const void* con
 // ---- whole sumchecks as jobs ---------------------------------------------------------------------------------------------------
 // A job queues every kernel of a sumcheck on one stream without a host round trip (the challenges are known up front),
 // keeps its buffers until the results have been fetched, and can run on a stream of the library's own beside the caller.
+// An eq table that several jobs read: the sumchecks of one softmax proof (its Hadamard argument and every segment's lookup)
+// are all weighted by the same challenges, so the table -- 2 GB for the stacked attention -- is built by the first job that
+// asks and the others wait for its event.  The jobs only read it (a round writes the next, shorter table elsewhere).
+// Freed when the last holder lets go: every job holds it until its own completion has been seen on the host, and the slot
+// below holds the latest one until another table replaces it.
+struct SharedEq {
+    void* p = nullptr;
+    hipEvent_t ready = nullptr;
+    int k = 0;
+    std::vector<uint32_t> key;
+    ~SharedEq() {
+        if (ready) (void)hipEventDestroy(ready);
+        if (p) (void)pool_free(p, nullptr, true);      // every reader has finished (see above)
+    }
+};
+static std::mutex g_eq_mu;
+static std::shared_ptr<SharedEq>& g_eq_latest = *new std::shared_ptr<SharedEq>();      // never destroyed: no device call after the runtime has gone
 struct SumJob {
+    std::shared_ptr<SharedEq> eq;
     Arena arena;
     hipStream_t st = nullptr;
     Fr* sums = nullptr;          // rounds x per_round values
@@ -1439,6 +1457,27 @@ static void lookup_fix_sums(Fr* s, int rounds, int n1) {
             if (r < n1 && i >= 5) x = big_zero<8>();
         }
 }
+// the eq table of k challenges for a job on stream st: the latest one when it was built from the same challenges, else a new one
+static int shared_eq_get(std::shared_ptr<SharedEq>& out, const uint32_t* u, int k, Arena& arena, hipStream_t st) {
+    std::lock_guard<std::mutex> lk(g_eq_mu);
+    if (g_eq_latest && g_eq_latest->k == k && memcmp(g_eq_latest->key.data(), u, sizeof(uint32_t) * 8 * (size_t)k) == 0) {
+        out = g_eq_latest;
+        ZK_HIP(hipStreamWaitEvent(st, out->ready, 0));
+        return 0;
+    }
+    std::shared_ptr<SharedEq> e(new SharedEq);
+    e->k = k;
+    e->key.assign(u, u + 8 * (size_t)k);
+    int rc = pool_alloc(&e->p, sizeof(Fr) * ((size_t)1 << k), st);
+    if (rc) return rc;
+    rc = eq_table_queue((Fr*)e->p, u, k, arena, st);
+    if (rc) { (void)hipStreamSynchronize(st); return rc; }
+    ZK_HIP(hipEventCreateWithFlags(&e->ready, hipEventDisableTiming));
+    ZK_HIP(hipEventRecord(e->ready, st));
+    g_eq_latest = e;
+    out = e;
+    return 0;
+}
 static int lookup_args_ok(size_t D, size_t N, int rounds) {
     ZK_ARG(D >= 2 && N >= 1 && D % N == 0 && ((D / N) & (D / N - 1)) == 0, "lookup sumcheck: D must be N times a power of two");
     ZK_ARG((D & (D - 1)) == 0, "lookup sumcheck: D must be a power of two");
@@ -1499,9 +1538,8 @@ static int lookup_prove_begin(void** handle, const void* S, const void* T, const
     if (rc) { sumjob_abort(job); return rc; }
     hipStream_t st = job->st;
     Scratch& B = job->arena.add(sizeof(Fr) * N);
-    Scratch& E = job->arena.add(sizeof(Fr) * (D / 2));
     Scratch& dp = job->arena.add(sizeof(Fr) * (reduce_grid(N) + 1));
-    if (B.rc || E.rc || dp.rc) { rc = B.rc ? B.rc : (E.rc ? E.rc : dp.rc); sumjob_abort(job); return rc; }
+    if (B.rc || dp.rc) { rc = B.rc ? B.rc : dp.rc; sumjob_abort(job); return rc; }
     const Fr b = load_fr(beta);
     rc = batch_inv_queue(B.as<Fr>(), (const Fr*)T, b, N, job->arena, st);
     const Fr* Aptr = nullptr;
@@ -1523,9 +1561,9 @@ static int lookup_prove_begin(void** handle, const void* S, const void* T, const
     hipLaunchKernelGGL(k_dot_part, dim3(nb), dim3(TPB), 0, st, dp.as<Fr>() + 1, B.as<Fr>(), (const Fr*)m, N);
     hipLaunchKernelGGL(k_finish, dim3(1), dim3(TPB), 0, st, dp.as<Fr>(), dp.as<Fr>() + 1, nb);
     job->extra = dp.as<Fr>();
-    rc = eq_table_queue(E.as<Fr>(), u_eq, rounds - 1, job->arena, st);
+    rc = shared_eq_get(job->eq, u_eq, rounds - 1, job->arena, st);
     if (rc) { sumjob_abort(job); return rc; }
-    rc = lookup_queue(*job, Aptr, (const Fr*)S, B.as<Fr>(), (const Fr*)T, (const Fr*)m, E.as<Fr>(), b, v, D, N, rounds, hint ? &hs : nullptr);
+    rc = lookup_queue(*job, Aptr, (const Fr*)S, B.as<Fr>(), (const Fr*)T, (const Fr*)m, (const Fr*)job->eq->p, b, v, D, N, rounds, hint ? &hs : nullptr);
     if (rc == 0) rc = sumjob_queue_results(*job);
     if (rc) { sumjob_abort(job); return rc; }
     *handle = job;
@@ -1615,13 +1653,11 @@ int zk_hadamard_prove_begin(void** handle, const void* const* Xs, int K, const u
     SumJob* job = new SumJob;
     int rc = sumjob_on_side_stream(*job, (hipStream_t)stv);
     if (rc) { sumjob_abort(job); return rc; }
-    Scratch& E = job->arena.add(sizeof(Fr) * (N / 2));
-    if (E.rc) { rc = E.rc; sumjob_abort(job); return rc; }
     int k = 0;
     while (((size_t)1 << k) < N) ++k;
-    rc = eq_table_queue(E.as<Fr>(), u_eq, k - 1, job->arena, job->st);
+    rc = shared_eq_get(job->eq, u_eq, k - 1, job->arena, job->st);
     if (rc) { sumjob_abort(job); return rc; }
-    rc = hadamard_queue(*job, (const Fr* const*)Xs, K, E.as<Fr>(), v, N);
+    rc = hadamard_queue(*job, (const Fr* const*)Xs, K, (const Fr*)job->eq->p, v, N);
     if (rc == 0) rc = sumjob_queue_results(*job);
     if (rc) { sumjob_abort(job); return rc; }
     *handle = job;
