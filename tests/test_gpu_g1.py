@@ -283,7 +283,7 @@ def test_open_batch_over_prepared_generators_matches_single_openings(orc):
     import ctypes
     from gpuhelp import Hip, c_void_p, c_size_t, c_int
     hip = Hip()
-    for n, count in ((9001, 3), (600, 2), (4096, 8)):
+    for n, count in ((9001, 3), (600, 2), (4096, 8), (2049, 2)):
         k = (n - 1).bit_length()
         npts = 3 * k + 1
         gens, dG, dS, us, preps = [], [], [], [], []

@@ -42,6 +42,25 @@ def test_host_fr_ops_match_bigint_and_oracle():
     assert (got[:64] == exp[:64]).all()
 
 
+def test_unreduced_sums_of_products_reduce_to_the_sum_of_montgomery_products():
+    """wide_mac / wide_redc (the sumcheck rounds' accumulator: products added as 512-bit integers, one reduction at the end)
+    against big integers: sum a_i b_i / R mod r for operands below r, for arbitrary 256-bit operands (the accumulator does
+    not ask for reduced inputs), for the extremes, and for sums long enough to reach the seventeenth limb."""
+    lib = _lib()
+    rng = random.Random(21)
+    rinv = pow(FR_R, -1, R_MOD)
+    top = (1 << 256) - 1
+    cases = [([0], [0]), ([1], [1]), ([R_MOD - 1], [R_MOD - 1]), ([top], [top]), ([top] * 70000, [top] * 70000),
+             ([rng.randrange(R_MOD) for _ in range(300)], [rng.randrange(R_MOD) for _ in range(300)]),
+             ([rng.randrange(1 << 256) for _ in range(1000)], [rng.randrange(1 << 256) for _ in range(1000)])]
+    for a, b in cases:
+        A = np.array([[(x >> (32 * k)) & 0xFFFFFFFF for k in range(8)] for x in a], dtype=np.uint32)
+        B = np.array([[(x >> (32 * k)) & 0xFFFFFFFF for k in range(8)] for x in b], dtype=np.uint32)
+        got = np.zeros((1, 8), dtype=np.uint32)
+        assert lib.zkp_host_fr_wide_dot(_np_ptr(A), _np_ptr(B), _np_ptr(got), ctypes.c_long(len(a))) == 0
+        assert fr_ints(got)[0] == sum(x * y for x, y in zip(a, b)) * rinv % R_MOD
+
+
 def test_host_fp_ops_match_bigint_and_oracle():
     lib, orc = _lib(), load_oracle()
     rng = random.Random(12)

@@ -76,6 +76,21 @@ int zkp_host_fr_op(int op, const u32* a, const u32* b, u32* out, long n) {
     }
     ZKP_END
 }
+// sum_i a_i b_i R^-1 through the unreduced accumulator of the sumcheck kernels (wide_mac / wide_redc, csrc/field.hpp); operands
+// may be any 256-bit values
+int zkp_host_fr_wide_dot(const u32* a, const u32* b, u32* out, long n) {
+    ZKP_TRY
+    zk::WideAcc w = zk::wide_zero();
+    for (long i = 0; i < n; ++i) {
+        zk::Fr x, y;
+        memcpy(x.v, a + 8 * i, 32);
+        memcpy(y.v, b + 8 * i, 32);
+        zk::wide_mac(w, x, y);
+    }
+    const zk::Fr r = zk::wide_redc(w);
+    memcpy(out, r.v, 32);
+    ZKP_END
+}
 int zkp_host_fp_op(int op, const u32* a, const u32* b, u32* out, long n) {
     ZKP_TRY
     for (long i = 0; i < n; ++i) {
