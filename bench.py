@@ -430,7 +430,11 @@ def main():
                                         "frac": l_bytes / (l_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": l_ms / l_launches, "pairs": int(l_pairs),
                                         "whole_proof_ms": look_total_ms,
                                         "note": "algorithmic 240 B per pair (two queries of two tensors, eq weight, two folded values out, next eq table); the kernel also gathers "
-                                                "a 64-byte record (table entry and its inverse) per query from a 64 MiB table, and does six field products per pair"}
+                                                "a 64-byte record (table entry and its inverse) per query from a 64 MiB table and does five field products and one unreduced "
+                                                "one per pair: 2478 lane instructions per pair, 55 % of the VALU issue slots, 25 GB moved with the gathers = 3.3 TB/s "
+                                                "(SQ_INSTS_VALU, FETCH_SIZE, WRITE_SIZE of this launch in profiles/fr_mul_fold_msm_pmc.txt) -- bound by neither unit alone; "
+                                                "a range table's first round (one query tensor, table in L2) runs at 2.6 TB/s algorithmic, the later rounds at 3.6 TB/s "
+                                                "and 79 % of the VALU slots (instruction issue binds there)"}
     del keep, look
 
     # ---- CPU baseline: the oracle's restatement of the reference's algorithm on this host's cores ---------------------------------------
