@@ -13,8 +13,7 @@ namespace zk {
 enum : int {
     ZK_OK = 0,
     ZK_ERR_ARG = 10001,      // bad argument (shape mismatch, null pointer, size over a stated limit)
-    ZK_ERR_NO_DEVICE = 10002,
-    ZK_ERR_BLAS = 10003      // a rocBLAS call failed (the integer GEMMs of large matrix products)
+    ZK_ERR_NO_DEVICE = 10002
 };
 
 void set_error(int code, const std::string& msg);
