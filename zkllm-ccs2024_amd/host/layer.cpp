@@ -352,25 +352,23 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
         ou = std::move(ahead[0]); og = std::move(ahead[1]); od = std::move(ahead[2]);
     }
 
-    {
-        auto pd = down_rescale.prove_begin(down_out, down_out_, ch_dr);
-        down_rescale.prove_end(pd);
-    }
-    auto cd = down_layer.prove(down_in_, down_out, ch_d);
-    if (c.open_weights) verifyWeightClaim(down, cd[0], od);
-    // three lookup proofs in a row with nothing between them: all begun, then collected in order
+    // The five lookup proofs of the block (four rescalings, the activation table) need only the forward pass and their
+    // challenges: all are begun here, on the library's streams, and each is collected where the reference proves it, so
+    // the matrix-product proofs on the caller's stream run beside them and the transcript keeps its order.
+    auto pd = down_rescale.prove_begin(down_out, down_out_, ch_dr);
     auto ph = hidden_rescale.prove_begin(down_in, down_in_, ch_hr);
     auto ps = swiglu.prove_begin(gate_out_, swiglu_out, swiglu_m, temp_rand[0], temp_rand[1], temp_rand[2], swiglu_u, swiglu_v);
     auto pg = gate_rescale.prove_begin(gate_out, gate_out_, ch_gr);
+    auto pu = up_rescale.prove_begin(up_out, up_out_, ch_ur);
+    down_rescale.prove_end(pd);
+    auto cd = down_layer.prove(down_in_, down_out, ch_d);
+    if (c.open_weights) verifyWeightClaim(down, cd[0], od);
     hidden_rescale.prove_end(ph);
     tLookup::prove_end(ps);
     gate_rescale.prove_end(pg);
     auto cg = gate_layer.prove(input, gate_out, ch_g);
     if (c.open_weights) verifyWeightClaim(gate, cg[0], og);
-    {
-        auto pu = up_rescale.prove_begin(up_out, up_out_, ch_ur);
-        up_rescale.prove_end(pu);
-    }
+    up_rescale.prove_end(pu);
     auto cu = up_layer.prove(input, up_out, ch_u);
     if (c.open_weights) verifyWeightClaim(up, cu[0], ou);
     // the reference's executable saves the unrescaled down_out (ffn.cu:81); the rescaled tensor is what the next block consumes
