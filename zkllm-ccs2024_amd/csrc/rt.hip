@@ -62,7 +62,7 @@ static bool is_persistent_stream(hipStream_t s) {
 // Makes `stream` wait for what `blk`'s last user had queued when it let the block go.  Called with the pool locked.
 static void order_behind_last_user(Pool& P, const Block& blk, hipStream_t stream) {
     if (blk.idle || blk.last == stream) return;
-    if (blk.ev_set) {                                             // recorded at free time on a caller's stream
+    if (blk.ev_set) {                                             // recorded at free time (any stream but the default one)
         if (hipStreamWaitEvent(stream, blk.ev, 0) != hipSuccess) { (void)hipGetLastError(); (void)hipDeviceSynchronize(); }
         return;
     }
@@ -129,10 +129,14 @@ int pool_free(void* p, hipStream_t stream, bool idle) {
     b.idle = idle;
     b.freed_tick = ++P.tick;
     b.ev_set = false;
-    if (!idle && !persistent) {
+    // Any stream but the default one: the event is recorded now.  Recorded later, when another stream takes the block,
+    // it would sit behind everything the freeing stream has been given since -- a whole opening or sumcheck job of the
+    // library's own streams -- and the taker would wait for all of that, not for the block's last use.
+    if (!idle && (!persistent || stream != nullptr)) {
         if (!b.ev && hipEventCreateWithFlags(&b.ev, hipEventDisableTiming) != hipSuccess) { (void)hipGetLastError(); b.ev = nullptr; }
         if (b.ev && hipEventRecord(b.ev, stream) == hipSuccess) b.ev_set = true;
-        else { (void)hipGetLastError(); (void)hipStreamSynchronize(stream); b.idle = true; }
+        else if (!persistent) { (void)hipGetLastError(); (void)hipStreamSynchronize(stream); b.idle = true; }
+        else (void)hipGetLastError();      // a stream of the library's own: the wait is placed when the block is taken, as for the default stream
     }
     P.free_lists[it->second.size].push_back(p);
     P.cached_bytes += it->second.size;
