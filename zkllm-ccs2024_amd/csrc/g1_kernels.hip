@@ -843,7 +843,7 @@ k_open_fold29(const FoldBatch fb, size_t old_size, size_t new_size) {
 // COMB_W doublings and at most 2 COMB_W mixed additions instead of 129 doublings and ~65 additions, and no inversion for a
 // table.  Every lane of the launch uses the same indices, so the table is laid out entry-major ([m][pair]): the lanes of a
 // wave read consecutive points.
-static constexpr int COMB_A = 6, COMB_W = 22, COMB_N = (1 << COMB_A) - 1;
+static constexpr int COMB_A = 8, COMB_W = 16, COMB_N = (1 << COMB_A) - 1;
 static_assert(COMB_A * COMB_W >= 128, "the comb must cover 128-bit half scalars");
 struct CombK { uint8_t m1[COMB_W + 2], m2[COMB_W + 2]; };
 // No pair is special here: the table holds multiples of D whatever D is (infinity when the two generators are equal, a
