@@ -34,7 +34,7 @@ VALU_PEAK_TOPS = 256 * 4 * 16 * 2.4e9 / 1e12
 # WRITE_SIZE on the kernel alone (python3 bench.py --pmc-probe; summary in profiles/k_open_fold29_pmc_traffic.txt), each
 # counter scaled by what it reads for zk_fr_add over 2^24 elements (1 GiB read, 512 MiB written).  It holds for launches of
 # that size; `traffic` of the in-layer entry, whose launches are of every size, is left null and the algorithmic figure given.
-FOLD_TRAFFIC_BYTES_PER_PAIR_AT_262144 = 764.6      # (53742 KiB x 2.000 fetched + 88253 KiB written) / 262144 pairs, profiles/k_open_fold29_pmc_traffic.txt
+FOLD_TRAFFIC_BYTES_PER_PAIR_AT_262144 = 763.5      # (53674 KiB x 2.000 fetched + 88108 KiB written) / 262144 pairs, profiles/k_open_fold29_pmc_traffic.txt
 FOLD_ALGO_BYTES_PER_PAIR = 2 * 112 + 112 + 3 * 32      # two points in, one out (affine, 29-bit limbs: 112 B), two scalars in, one out
 MAD_PER_FP_MUL = 300                                   # 2 * 12^2 + 12 limb products of a 381-bit Montgomery product
 MAD_PER_FR_MUL = 136                                   # 2 * 8^2 + 8
@@ -113,8 +113,8 @@ def main():
         n_big, gens_big, bufs, fold_round = fold_probe_setup()
         for _ in range(3):
             fold_round()
-        # a whole opening over the same generators in their prepared form: the first round's comb fold on 262144 pairs,
-        # then k_open_fold29 on 131072, 65536, ... pairs
+        # a whole opening over the same generators in their prepared form: the comb folds of the first two rounds on
+        # 262144 and 131072 pairs, then k_open_fold29 on 65536, 32768, ... pairs
         prep_open = prepared_opening(n_big, gens_big, bufs[0])
         prep_open()
         n = 1 << 24
@@ -262,7 +262,7 @@ def main():
     # Fp multiplication is 2*12^2+12 = 300 of them.  Durations are HIP events around every launch inside the timed
     # region above, on the launch stream.
     fold_tops = fold_mults * MAD_PER_FP_MUL / (fold_ms * 1e-3) / 1e12 if fold_ms > 0 else 0.0
-    out["roofline"] = {"kernel": "k_open_fold29 and, in an opening's first round, k_open_fold_comb (g' = g1 + [u](g0 - g1) per generator pair, 128-bit split scalars; "
+    out["roofline"] = {"kernel": "k_open_fold29 and, in an opening's first two rounds over prepared generators, k_open_fold_comb<1> / <2> (g' = g1 + [u](g0 - g1) per generator pair, 128-bit split scalars; "
                                  "one launch per round for all openings of a size)",
                        "bound": "valu-int", "achieved": fold_tops, "peak": VALU_PEAK_TOPS, "unit": "T MAD32/s", "frac": fold_tops / VALU_PEAK_TOPS,
                        "traffic": None, "algorithmic_bytes_per_launch": FOLD_ALGO_BYTES_PER_PAIR * fold_pairs / max(1, fold_launches),
@@ -298,8 +298,8 @@ def main():
                                   "avg_launch_ms": f_ms / max(1, f_launches), "fp_mul_per_s": f_mults / (f_ms * 1e-3),
                                   "note": "4096 waves on 2048 wave slots (two per SIMD: 256 registers, most of the walk's table in LDS): two full turns.  traffic: "
                                           "FETCH_SIZE + WRITE_SIZE of this launch from profiles/k_open_fold29_pmc_traffic.txt"}
-    # the fold kernels of one whole opening over the same generators prepared: the comb fold of the first round
-    # (262144 pairs) and k_open_fold29 on the later rounds down to the batched last rounds
+    # the fold kernels of one whole opening over the same generators prepared: the comb folds of the first two rounds
+    # (262144 and 131072 pairs) and k_open_fold29 on the later rounds down to the batched last rounds
     prep_open = prepared_opening(n_big, gens_big, bufs[0])
     prep_open()
     hip.check(lib.zk_prof_fold_begin())
@@ -308,7 +308,7 @@ def main():
     open_alone_s = time.perf_counter() - t0
     o_ms, o_launches, o_mults, o_pairs = read_fold_timer()
     o_tops = o_mults * MAD_PER_FP_MUL / (o_ms * 1e-3) / 1e12
-    out["roofline_fold_opening_alone"] = {"kernel": "k_open_fold_comb (first round, 262144 pairs) + k_open_fold29 (later rounds) of one opening over 2^19 prepared generators, "
+    out["roofline_fold_opening_alone"] = {"kernel": "k_open_fold_comb<1> / <2> (first two rounds, 262144 and 131072 pairs) + k_open_fold29 (later rounds) of one opening over 2^19 prepared generators, "
                                                     "beside that opening's own bucket sums only", "bound": "valu-int", "achieved": o_tops, "peak": VALU_PEAK_TOPS,
                                           "unit": "T MAD32/s", "frac": o_tops / VALU_PEAK_TOPS, "traffic": None, "launches": int(o_launches), "pairs": int(o_pairs),
                                           "total_ms": o_ms, "fp_mul_per_pair": o_mults / max(1, o_pairs), "opening_wall_s": open_alone_s}

@@ -849,8 +849,14 @@ struct CombK { uint8_t m1[COMB_W + 2], m2[COMB_W + 2]; };
 // No pair is special here: the table holds multiples of D whatever D is (infinity when the two generators are equal, a
 // doubling when they are opposite), an entry at infinity is skipped, and the mixed addition itself handles a sum that
 // meets its own operand.
-struct CombItem { Fr* ns; A29* ng; const Fr* s; const A29* g; const A29* tab; Fr u_mont; CombK ck; };
+// NT = 2 (the second round): the pair difference of that round is itself a fixed combination of prepared points,
+//     g'_2j - g'_2j+1 = F_j + [u1] H_j,   F_j = g_4j+1 - g_4j+3,  H_j = (g_4j - g_4j+1) - (g_4j+2 - g_4j+3)
+// (g'_i = g_2i+1 + [u1](g_2i - g_2i+1) are the first round's results, a missing generator is the point at infinity), so
+//     g''_j = g'_2j+1 + [u2] F_j + [u1 u2] H_j:
+// two combs that share their doublings, COMB_W doublings and at most 4 COMB_W additions instead of the 129-step walk.
+struct CombItem { Fr* ns; A29* ng; const Fr* s; const A29* g; const A29* tab; const A29* tab2; Fr u_mont; CombK ck, ck2; };
 struct CombBatch { CombItem it[OB_MAX]; };
+template <int NT>
 __global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 k_open_fold_comb(const CombBatch cb, size_t old_size, size_t new_size) {
     __shared__ int32_t inv_lds[14][2 * GT];
@@ -859,8 +865,10 @@ k_open_fold_comb(const CombBatch cb, size_t old_size, size_t new_size) {
     const Fr* __restrict__ scalars = cb.it[blockIdx.y].s;
     const A29* __restrict__ A = cb.it[blockIdx.y].g;
     const A29* __restrict__ tab = cb.it[blockIdx.y].tab;
+    const A29* __restrict__ tab2 = cb.it[blockIdx.y].tab2;
     const Fr u_mont = cb.it[blockIdx.y].u_mont;
     const CombK& ck = cb.it[blockIdx.y].ck;
+    const CombK& ck2 = cb.it[blockIdx.y].ck2;
     const size_t g = (size_t)blockIdx.x * GT + threadIdx.x;
     const bool live = g < new_size;
     const size_t g0 = 2 * g, g1 = 2 * g + 1;
@@ -879,16 +887,20 @@ k_open_fold_comb(const CombBatch cb, size_t old_size, size_t new_size) {
         const Fq29 beta = fq29_from_fp(glv_beta());
         for (int b = COMB_W - 1; b >= 0; --b) {
             w = j29_double(w);
-            const uint32_t m1 = ck.m1[b], m2 = ck.m2[b];          // the same for every lane
-            if (m1) {
-                const A29 t = tab[(size_t)(m1 - 1) * new_size + g];
-                if (!a29_is_inf(t)) w = j29_add_mixed(w, t);
-            }
-            if (m2) {
-                A29 t = tab[(size_t)(m2 - 1) * new_size + g];
-                if (!a29_is_inf(t)) {
-                    t.x = fq29_mul(t.x, beta);
-                    w = j29_add_mixed(w, t);
+#pragma unroll
+            for (int ti = 0; ti < NT; ++ti) {
+                const A29* __restrict__ tb = ti ? tab2 : tab;
+                const uint32_t m1 = ti ? ck2.m1[b] : ck.m1[b], m2 = ti ? ck2.m2[b] : ck.m2[b];          // the same for every lane
+                if (m1) {
+                    const A29 t = tb[(size_t)(m1 - 1) * new_size + g];
+                    if (!a29_is_inf(t)) w = j29_add_mixed(w, t);
+                }
+                if (m2) {
+                    A29 t = tb[(size_t)(m2 - 1) * new_size + g];
+                    if (!a29_is_inf(t)) {
+                        t.x = fq29_mul(t.x, beta);
+                        w = j29_add_mixed(w, t);
+                    }
                 }
             }
         }
@@ -957,6 +969,18 @@ __global__ void __launch_bounds__(GT) k_open_pair_points(G1Jac* __restrict__ pj,
         if (!aff_is_inf(b)) p = g1_add_mixed(p, b);
     }
     pj[i] = p;
+}
+// out[j] = V[2j] - V[2j+1] over the points V[i] = A[off + i * stride], i < cnt (a missing one is the point at infinity)
+__global__ void __launch_bounds__(GT) k_open_pair_diff(G1Jac* __restrict__ out, const G1Affine* __restrict__ A, size_t off, size_t stride, size_t cnt, size_t n_out) {
+    const size_t j = (size_t)blockIdx.x * GT + threadIdx.x;
+    if (j >= n_out) return;
+    G1Jac p = g1_infinity();
+    if (2 * j < cnt) p = aff_to_jac(A[off + 2 * j * stride]);
+    if (2 * j + 1 < cnt) {
+        const G1Affine b = g1_neg(A[off + (2 * j + 1) * stride]);
+        if (!aff_is_inf(b)) p = g1_add_mixed(p, b);
+    }
+    out[j] = p;
 }
 struct PairBatch { Fr* ps[OB_MAX]; const Fr* s[OB_MAX]; };
 __global__ void __launch_bounds__(256) k_open_pair_scalars(const PairBatch pb, size_t old_size, size_t half_up) {
@@ -1175,11 +1199,13 @@ __global__ void __launch_bounds__(64) k_open_t_fix(G1Jac* __restrict__ wsum0, ui
     wsum[w] = g1_add(g1_add(wsum[w], g1_neg(wsum[MW + w])), g1_neg(wsum[2 * MW + w]));
 }
 // One round of `count` openings of equal size (count <= OB_MAX): one launch of each kernel covers all of them.
-struct RoundItem { Fr* new_scalars; A29* new_gens; const Fr* scalars; const A29* gens; Fr u; const A29* comb = nullptr; };
+// comb: the first round's table; comb2 (second round): the tables of F and H one after the other, u_prev the first round's challenge
+struct RoundItem { Fr* new_scalars; A29* new_gens; const Fr* scalars; const A29* gens; Fr u; const A29* comb = nullptr; const A29* comb2 = nullptr; Fr u_prev = Fr(); };
 // Fp multiplications of one pair of the comb fold by the formulas' count
-static double comb_fp_mults_per_pair(const CombK& ck) {
+static double comb_fp_mults_per_pair(const CombK& ck, const CombK* ck2 = nullptr) {
     int adds = 0, phis = 0;
     for (int b = 0; b < COMB_W; ++b) { adds += (ck.m1[b] ? 1 : 0) + (ck.m2[b] ? 1 : 0); phis += ck.m2[b] ? 1 : 0; }
+    if (ck2) for (int b = 0; b < COMB_W; ++b) { adds += (ck2->m1[b] ? 1 : 0) + (ck2->m2[b] ? 1 : 0); phis += ck2->m2[b] ? 1 : 0; }
     // doublings (7 each), mixed additions (11 each), the endomorphism's product, final addition (11), its share of one batched inversion (3) and the way back to affine (5)
     return 7.0 * COMB_W + 11.0 * adds + phis + 11.0 + 3.0 + 5.0;
 }
@@ -1279,8 +1305,8 @@ static int open_round_launch(const RoundItem* items, int count, size_t old_size,
     const size_t sp_stride = 1 + new_size;
     Scratch& special = arena.add(sizeof(uint32_t) * sp_stride * count);
     if (special.rc) return special.rc;
-    bool use_comb = with_T;
-    for (int i = 0; i < count; ++i) use_comb = use_comb && items[i].comb != nullptr;
+    bool use_comb = with_T, use_comb2 = !with_T;
+    for (int i = 0; i < count; ++i) { use_comb = use_comb && items[i].comb != nullptr; use_comb2 = use_comb2 && items[i].comb2 != nullptr; }
     FoldBatch fb;
     CombBatch cbt;
     SpecialBatch sb;
@@ -1289,13 +1315,21 @@ static int open_round_launch(const RoundItem* items, int count, size_t old_size,
         const int k = i < count ? i : 0;
         const GlvK ku = glv_split(items[k].u);
         uint32_t* sp = special.as<uint32_t>() + sp_stride * k;
-        if (use_comb) {
+        if (use_comb || use_comb2) {
             CombItem& f = cbt.it[i];
             f.ns = items[k].new_scalars; f.ng = items[k].new_gens; f.s = items[k].scalars; f.g = items[k].gens;
-            f.tab = items[k].comb;
             f.u_mont = to_mont(items[k].u);
             f.ck = comb_of(ku);
-            if (i < count) fp_mults += comb_fp_mults_per_pair(f.ck) * (double)new_size;
+            if (use_comb) {
+                f.tab = items[k].comb; f.tab2 = items[k].comb;
+                f.ck2 = f.ck;
+                if (i < count) fp_mults += comb_fp_mults_per_pair(f.ck) * (double)new_size;
+            } else {
+                f.tab = items[k].comb2; f.tab2 = items[k].comb2 + (size_t)COMB_N * new_size;
+                // [u2] of [u1] H is [u1 u2 mod r] H: the generators have order r
+                f.ck2 = comb_of(glv_split(from_mont(mont_mul(to_mont(items[k].u_prev), to_mont(items[k].u)))));
+                if (i < count) fp_mults += comb_fp_mults_per_pair(f.ck, &f.ck2) * (double)new_size;
+            }
         } else {
             FoldItem& f = fb.it[i];
             f.ns = items[k].new_scalars; f.ng = items[k].new_gens; f.s = items[k].scalars; f.g = items[k].gens; f.special = sp;
@@ -1312,7 +1346,8 @@ static int open_round_launch(const RoundItem* items, int count, size_t old_size,
         ZK_HIP(hipEventCreate(&t1));
         ZK_HIP(hipEventRecord(t0, st));
     }
-    if (use_comb) hipLaunchKernelGGL(k_open_fold_comb, dim3(cdiv(new_size, GT), count), dim3(GT), 0, st, cbt, old_size, new_size);
+    if (use_comb) hipLaunchKernelGGL(k_open_fold_comb<1>, dim3(cdiv(new_size, GT), count), dim3(GT), 0, st, cbt, old_size, new_size);
+    else if (use_comb2) hipLaunchKernelGGL(k_open_fold_comb<2>, dim3(cdiv(new_size, GT), count), dim3(GT), 0, st, cbt, old_size, new_size);
     else hipLaunchKernelGGL(k_open_fold29, dim3(cdiv(new_size, GT), count), dim3(GT), 0, st, fb, old_size, new_size);
     if (g_fold_timer.on) {
         ZK_HIP(hipEventRecord(t1, st));
@@ -1620,7 +1655,7 @@ struct OpenJob {
 };
 // One opening of the batch: its scalars, its challenges (rounds x 8 limbs) and its generators -- Jacobian, or null when
 // `prep` (their prepared form, open_prep_build) is given
-struct OpenItem { const void* scalars; const void* gens; const A29* prep; const uint32_t* u; const A29* comb = nullptr; };
+struct OpenItem { const void* scalars; const void* gens; const A29* prep; const uint32_t* u; const A29* comb = nullptr; const A29* comb2 = nullptr; };
 static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, int rounds, hipStream_t st, hipStream_t aux) {
     ZK_ARG(n >= 1, "zk_g1_open: empty input");
     ZK_ARG(count >= 1 && count <= OB_MAX, "zk_g1_open: a batch holds 1 to 8 openings");
@@ -1683,6 +1718,7 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
         for (int i = 0; i < count; ++i) {
             ri[i] = RoundItem{s2.as<Fr>() + ns * i, g2.as<A29>() + ns * i, cs[i], cg[i], load_fr(items[i].u + 8 * r)};
             if (r == 0) ri[i].comb = items[i].comb;
+            if (r == 1) { ri[i].comb2 = items[i].comb2; ri[i].u_prev = load_fr(items[i].u + 8 * (r - 1)); }
         }
         int rc = open_round_launch(ri, count, size, r == 0, wsum.as<G1Jac>() + (size_t)3 * MW * r, wstride, job.arena, st, aux, job.events);
         if (rc) return rc;
@@ -1764,7 +1800,7 @@ int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_
 // Generators prepared once for any number of openings against them: their affine 29-bit-limb form and the pair sums of
 // the first round (weight-independent; 1.5 n points of 112 bytes).  The handle is freed with zk_g1_open_prepared_free
 // once no opening that uses it is pending.
-struct OpenPrepared { void* a29 = nullptr; size_t n = 0; void* comb = nullptr; };
+struct OpenPrepared { void* a29 = nullptr; size_t n = 0; void* comb = nullptr; void* comb2 = nullptr; };
 int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stv) {
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(prepared != nullptr && n >= 1, "zk_g1_open_prepare: null handle or no generators");
@@ -1780,33 +1816,50 @@ int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stv) {
         // (an addition of an array to itself), entry m = entry (m without its lowest bit) + entry (that bit).
         if (rc == 0 && n > (size_t)TAIL_N) {
             const size_t np = (n + 1) / 2, ne = np * COMB_N;
+            const size_t nq = (np + 1) / 2, ne2 = nq * COMB_N;        // second round: two tables over the pairs of pairs
+            const bool second = np > (size_t)TAIL_N;                  // that round is a fold too
             rc = pool_alloc(&pr->comb, sizeof(A29) * ne, st);
+            if (rc == 0 && second) rc = pool_alloc(&pr->comb2, sizeof(A29) * 2 * ne2, st);
             Scratch& aff = arena.add(sizeof(G1Affine) * n);
-            Scratch& tj = arena.add(sizeof(G1Jac) * ne);
-            Scratch& ta = arena.add(sizeof(G1Affine) * ne);
+            Scratch& tj = arena.add(sizeof(G1Jac) * std::max(ne, 2 * ne2));
+            Scratch& ta = arena.add(sizeof(G1Affine) * std::max(ne, 2 * ne2));
             Scratch& tmp = arena.add(sizeof(G1Jac) * np);
             if (rc == 0) rc = aff.rc ? aff.rc : (tj.rc ? tj.rc : (ta.rc ? ta.rc : tmp.rc));
             if (rc == 0) {
-                G1Jac* T = tj.as<G1Jac>();
-                auto entry = [&](int m) { return T + (size_t)(m - 1) * np; };
-                hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(n, CH), GT)), dim3(GT), 0, st, aff.p, (const G1Jac*)gens, n);
-                hipLaunchKernelGGL(k_open_pair_points, dim3(cdiv(np, GT)), dim3(GT), 0, st, entry(1), aff.as<G1Affine>(), n, np, 1);
                 static_assert(COMB_W % 2 == 0, "the doublings alternate between two buffers and must end in the table");
-                for (int j = 1; j < COMB_A; ++j) {
-                    const G1Jac* src = entry(1 << (j - 1));
-                    for (int k = 0; k < COMB_W; ++k) {          // no launch writes what it reads
-                        G1Jac* dst = (k & 1) ? entry(1 << j) : tmp.as<G1Jac>();
-                        hipLaunchKernelGGL(k_g1_add, dim3(cdiv(np, GT)), dim3(GT), 0, st, dst, src, src, np, np, 0);
-                        src = dst;
+                // T[0 .. cnt) holds entry 1 (the points themselves); fills the other COMB_N - 1 entries, cnt points each
+                auto fill = [&](G1Jac* T, size_t cnt) {
+                    auto entry = [&](int m) { return T + (size_t)(m - 1) * cnt; };
+                    for (int t = 1; t < COMB_A; ++t) {
+                        const G1Jac* src = entry(1 << (t - 1));
+                        for (int k = 0; k < COMB_W; ++k) {          // no launch writes what it reads
+                            G1Jac* dst = (k & 1) ? entry(1 << t) : tmp.as<G1Jac>();
+                            hipLaunchKernelGGL(k_g1_add, dim3(cdiv(cnt, GT)), dim3(GT), 0, st, dst, src, src, cnt, cnt, 0);
+                            src = dst;
+                        }
                     }
-                }
-                for (int m = 3; m <= COMB_N; ++m) {
-                    const int prev = m & (m - 1);
-                    if (!prev) continue;
-                    hipLaunchKernelGGL(k_g1_add, dim3(cdiv(np, GT)), dim3(GT), 0, st, entry(m), entry(prev), entry(m ^ prev), np, np, 0);
-                }
+                    for (int m = 3; m <= COMB_N; ++m) {
+                        const int prev = m & (m - 1);
+                        if (!prev) continue;
+                        hipLaunchKernelGGL(k_g1_add, dim3(cdiv(cnt, GT)), dim3(GT), 0, st, entry(m), entry(prev), entry(m ^ prev), cnt, cnt, 0);
+                    }
+                };
+                G1Jac* T = tj.as<G1Jac>();
+                hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(n, CH), GT)), dim3(GT), 0, st, aff.p, (const G1Jac*)gens, n);
+                hipLaunchKernelGGL(k_open_pair_points, dim3(cdiv(np, GT)), dim3(GT), 0, st, T, aff.as<G1Affine>(), n, np, 1);
+                fill(T, np);
                 hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(ne, CH), GT)), dim3(GT), 0, st, ta.p, tj.as<G1Jac>(), ne);
                 hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(ne, 256)), dim3(256), 0, st, (A29*)pr->comb, ta.as<G1Affine>(), ne);
+                if (second) {
+                    // F from the odd-numbered generators, H from the first round's differences (entry 1 of its table, affine in ta);
+                    // both are read before the buffers they sit in are written again
+                    hipLaunchKernelGGL(k_open_pair_diff, dim3(cdiv(nq, GT)), dim3(GT), 0, st, T, aff.as<G1Affine>(), (size_t)1, (size_t)2, n / 2, nq);
+                    hipLaunchKernelGGL(k_open_pair_diff, dim3(cdiv(nq, GT)), dim3(GT), 0, st, T + ne2, ta.as<G1Affine>(), (size_t)0, (size_t)1, np, nq);
+                    fill(T, nq);
+                    fill(T + ne2, nq);
+                    hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(2 * ne2, CH), GT)), dim3(GT), 0, st, ta.p, tj.as<G1Jac>(), 2 * ne2);
+                    hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(2 * ne2, 256)), dim3(256), 0, st, (A29*)pr->comb2, ta.as<G1Affine>(), 2 * ne2);
+                }
                 if (rc == 0 && hipGetLastError() != hipSuccess) rc = hip_fail(hipErrorLaunchFailure, "comb build", __FILE__, __LINE__);
             }
         }
@@ -1819,6 +1872,7 @@ int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stv) {
         (void)hipStreamSynchronize(st);
         pool_free(pr->a29, st, true);
         if (pr->comb) pool_free(pr->comb, st, true);
+        if (pr->comb2) pool_free(pr->comb2, st, true);
         return rc;
     }
     *prepared = pr.release();
@@ -1829,13 +1883,14 @@ int zk_g1_open_prepared_free(void* prepared) {
     OpenPrepared* pr = (OpenPrepared*)prepared;
     int rc = pool_free(pr->a29, nullptr);
     if (pr->comb) (void)pool_free(pr->comb, nullptr);
+    if (pr->comb2) (void)pool_free(pr->comb2, nullptr);
     delete pr;
     return rc;
 }
 int zk_g1_open_begin_prepared(void** handle, const void* scalars, const void* prepared, const uint32_t* u, int rounds, void* stv) {
     ZK_ARG(prepared != nullptr, "zk_g1_open_begin_prepared: null generators");
     const OpenPrepared* pr = (const OpenPrepared*)prepared;
-    const OpenItem item{scalars, nullptr, (const A29*)pr->a29, u, (const A29*)pr->comb};
+    const OpenItem item{scalars, nullptr, (const A29*)pr->a29, u, (const A29*)pr->comb, (const A29*)pr->comb2};
     return open_begin_impl(handle, &item, 1, pr->n, rounds, stv);
 }
 // `count` (1 to 8) openings against prepared generator sets of one size and with one round count, as ONE job: every
@@ -1852,7 +1907,7 @@ int zk_g1_open_begin_batch(void** handle, int count, const void* const* scalars,
         const OpenPrepared* pr = (const OpenPrepared*)prepared[i];
         if (i == 0) n = pr->n;
         ZK_ARG(pr->n == n, "zk_g1_open_begin_batch: the generator sets differ in size");
-        items[i] = OpenItem{scalars[i], nullptr, (const A29*)pr->a29, u + (size_t)i * rounds * 8, (const A29*)pr->comb};
+        items[i] = OpenItem{scalars[i], nullptr, (const A29*)pr->a29, u + (size_t)i * rounds * 8, (const A29*)pr->comb, (const A29*)pr->comb2};
     }
     return open_begin_impl(handle, items, count, n, rounds, stv);
 }
