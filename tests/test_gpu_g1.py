@@ -278,8 +278,9 @@ def test_open_begin_end_matches_open_through_the_c_abi(orc):
 def test_open_batch_over_prepared_generators_matches_single_openings(orc):
     """zk_g1_open_begin_batch (openings of one size as ONE job: every round's kernels launched once for all of them) over
     generators prepared with zk_g1_open_prepare delivers, opening by opening, the bytes of zk_g1_open.  Sizes on both
-    sides of the batched last rounds, a ragged one (odd halves), special generators (equal, opposite, infinite) in one
-    member of the batch, and zk_g1_open_begin_prepared alone."""
+    sides of the batched last rounds, a ragged one (odd halves: its first two rounds run on the prepared tables), special
+    generators (equal, opposite, infinite, also among the second round's prepared points) in one member of the batch,
+    and zk_g1_open_begin_prepared alone."""
     import ctypes
     from gpuhelp import Hip, c_void_p, c_size_t, c_int
     hip = Hip()
@@ -299,6 +300,13 @@ def test_open_batch_over_prepared_generators_matches_single_openings(orc):
                 g[6] = 0
                 g[7] = 0
                 g[9] = 0
+                # special among the points of the second round's tables (pairs of pairs g_4j .. g_4j+3): equal odd members
+                # (their difference is infinity), equal pair differences (infinity again), opposite odd members (a doubling)
+                g[15] = g[13]
+                g[18] = g[16]
+                g[19] = g[17]
+                orc_check(orc.orc_g1_op(4, g[21:22].copy(), g[21:22].copy(), neg, 1))
+                g[23] = neg[0]
             S = mt_random_vec(np.random.RandomState(50 + i), n)
             u = mt_random_vec(np.random.RandomState(70 + i), k)
             gens.append(g); us.append(u)
