@@ -1811,9 +1811,11 @@ int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stv) {
     {
         Arena arena(st);
         rc = open_prep_build((A29*)pr->a29, (const G1Jac*)gens, n, arena, st);
-        // The first round's comb, when that round is a fold (more generators than the batched last rounds take): entry-major
-        // table of the subset sums of 2^(j COMB_W) D, built from elementwise point kernels -- the teeth by repeated doubling
-        // (an addition of an array to itself), entry m = entry (m without its lowest bit) + entry (that bit).
+        // The combs of the first two rounds, for each round that is a fold (more generators than the batched last rounds
+        // take): entry-major tables of the subset sums of 2^(j COMB_W) P over the round's prepared points P (the pair
+        // differences D; for the second round F and H, see k_open_fold_comb), built from elementwise point kernels -- the
+        // teeth by repeated doubling (an addition of an array to itself), entry m = entry (m without its lowest bit) + entry
+        // (that bit).
         if (rc == 0 && n > (size_t)TAIL_N) {
             const size_t np = (n + 1) / 2, ne = np * COMB_N;
             const size_t nq = (np + 1) / 2, ne2 = nq * COMB_N;        // second round: two tables over the pairs of pairs
