@@ -1816,18 +1816,27 @@ int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stv) {
         // differences D; for the second round F and H, see k_open_fold_comb), built from elementwise point kernels -- the
         // teeth by repeated doubling (an addition of an array to itself), entry m = entry (m without its lowest bit) + entry
         // (that bit).
-        if (rc == 0 && n > (size_t)TAIL_N) {
+        // The tables only make the folds cheaper: ZKLLM_OPEN_TABLES = 0 or 1 keeps none or the first round's alone (28 KB
+        // per generator pair and round), and when the device has no room for them or for their construction the handle
+        // is made without them -- those rounds then walk (k_open_fold29), the results are the same.
+        static const int table_rounds = [] { const char* e = getenv("ZKLLM_OPEN_TABLES"); return e ? atoi(e) : 2; }();
+        if (rc == 0 && n > (size_t)TAIL_N && table_rounds >= 1) {
             const size_t np = (n + 1) / 2, ne = np * COMB_N;
             const size_t nq = (np + 1) / 2, ne2 = nq * COMB_N;        // second round: two tables over the pairs of pairs
-            const bool second = np > (size_t)TAIL_N;                  // that round is a fold too
-            rc = pool_alloc(&pr->comb, sizeof(A29) * ne, st);
-            if (rc == 0 && second) rc = pool_alloc(&pr->comb2, sizeof(A29) * 2 * ne2, st);
+            bool second = np > (size_t)TAIL_N && table_rounds >= 2;   // that round is a fold too
+            int trc = pool_alloc(&pr->comb, sizeof(A29) * ne, st);
+            if (trc == 0 && second && pool_alloc(&pr->comb2, sizeof(A29) * 2 * ne2, st) != 0) { pr->comb2 = nullptr; second = false; }
+            const size_t nt = second ? std::max(ne, 2 * ne2) : ne;
             Scratch& aff = arena.add(sizeof(G1Affine) * n);
-            Scratch& tj = arena.add(sizeof(G1Jac) * std::max(ne, 2 * ne2));
-            Scratch& ta = arena.add(sizeof(G1Affine) * std::max(ne, 2 * ne2));
+            Scratch& tj = arena.add(sizeof(G1Jac) * nt);
+            Scratch& ta = arena.add(sizeof(G1Affine) * nt);
             Scratch& tmp = arena.add(sizeof(G1Jac) * np);
-            if (rc == 0) rc = aff.rc ? aff.rc : (tj.rc ? tj.rc : (ta.rc ? ta.rc : tmp.rc));
-            if (rc == 0) {
+            if (trc == 0) trc = aff.rc ? aff.rc : (tj.rc ? tj.rc : (ta.rc ? ta.rc : tmp.rc));
+            if (trc) {                                                // nothing has been queued on the tables yet
+                if (pr->comb) (void)pool_free(pr->comb, st, true);
+                if (pr->comb2) (void)pool_free(pr->comb2, st, true);
+                pr->comb = pr->comb2 = nullptr;
+            } else {
                 static_assert(COMB_W % 2 == 0, "the doublings alternate between two buffers and must end in the table");
                 // T[0 .. cnt) holds entry 1 (the points themselves); fills the other COMB_N - 1 entries, cnt points each
                 auto fill = [&](G1Jac* T, size_t cnt) {
