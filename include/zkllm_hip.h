@@ -186,6 +186,15 @@ int zk_g1_open_begin_prepared(void** handle, const void* scalars, const void* pr
  * are independent of each other).  scalars[i] / prepared[i]: opening i; u: its challenges at u + i * rounds * 8.  end
  * delivers opening i's points at proof_host + i * (3 rounds + 1) * 36 and its folded scalar at final_scalar_host + i * 8. */
 int zk_g1_open_begin_batch(void** handle, int count, const void* const* scalars, const void* const* prepared, const uint32_t* u, int rounds, void* stream);
+/* zk_g1_open_begin_batch for openings as Commitment::open makes them (commitment.cu:133-141): the opened vector is the
+ * tensor's rows folded at u_out, and the reference evaluates the row commitments there too (com(u_out), :137).  rows[i]:
+ * tensor i's nrows[i] row commitments (Jacobian, 36 limbs each, on the device, alive until end); u_rows[i]: the
+ * k_rows[i] challenges the rows were folded with, lowest row bit first, 2^k_rows >= nrows.  The first round's T is then
+ * sum_r eq(u_rows, r) rows[r] instead of a sum over all generators: the same group element whenever rows are the
+ * commitments of the tensor's rows under these generators -- the caller's statement; with other rows the T of the
+ * halving rounds (each follows from the round before) differ from zk_g1_open_begin_batch's, nothing else does. */
+int zk_g1_open_begin_batch_rows(void** handle, int count, const void* const* scalars, const void* const* prepared, const uint32_t* u, int rounds,
+                                const void* const* rows, const uint32_t* nrows, const uint32_t* const* u_rows, const int* k_rows, void* stream);
 int zk_g1_open_end_batch(void* handle, uint32_t* proof_host, uint32_t* final_scalar_host);
 
 /* ---- lookup argument (tlookup.cu) ------------------------------------------------------------------------ */

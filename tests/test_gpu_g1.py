@@ -342,6 +342,75 @@ def test_open_batch_over_prepared_generators_matches_single_openings(orc):
             hip.free(x)
 
 
+def test_open_batch_with_row_commitments_delivers_the_points_of_the_plain_opening(pv):
+    """zk_g1_open_begin_batch_rows takes the first round's T from the tensors' row commitments (sum_r eq(u_rows, r) C_r)
+    instead of summing over all generators: for commitments made by commit_int of the same tensors every point of the
+    proof, T of the first round included, equals zk_g1_open's on the row-folded vector.  One tensor with a number of
+    rows that is no power of two, one with a single row (no row challenge), more generators than the batched last
+    rounds take; and with another tensor's commitments only the T of the halving rounds change."""
+    import ctypes
+    from gpuhelp import Hip, c_void_p, c_size_t, c_int
+    hip = Hip()
+    pv.lib.zkp_g1_devptr.restype = ctypes.c_void_p
+    n = 5000
+    k = (n - 1).bit_length()
+    npts = 3 * k + 1
+    pv.seed(77)
+    gens = pv.commitment_random(n)
+    dG = pv.lib.zkp_g1_devptr(c_void_p(gens.h))
+    prep = c_void_p()
+    hip.call("zk_g1_open_prepare", ctypes.byref(prep), c_void_p(dG), c_size_t(n), None)
+    rng = np.random.default_rng(5)
+    keep, folded, coms, urows, us = [], [], [], [], []
+    exp_p = np.zeros((2, npts, 36), np.uint32)
+    exp_v = np.zeros((2, 8), np.uint32)
+    for i, nrows in enumerate((5, 1)):
+        W = pv.from_i32(rng.integers(-30000, 30000, nrows * n).astype(np.int32))
+        com = pv.commit_int(gens, W)
+        assert com.size == nrows
+        kr = (nrows - 1).bit_length()
+        ur = mt_random_vec(np.random.RandomState(40 + i), max(kr, 1))[:kr]
+        f = pv.partial_me_window(W, ur, n) if kr else W
+        assert f.size == n
+        u = mt_random_vec(np.random.RandomState(60 + i), k)
+        print(f"rows={nrows}: zk_g1_open", flush=True)
+        hip.call("zk_g1_open", exp_p[i], exp_v[i], c_void_p(f.devptr), c_void_p(dG), c_size_t(n), u, c_int(k), None)
+        keep += [W, com, f]
+        folded.append(f); coms.append(com); urows.append(np.ascontiguousarray(ur, dtype=np.uint32)); us.append(u)
+
+    def run(com_order):
+        h = c_void_p()
+        sc = (c_void_p * 2)(*[c_void_p(f.devptr) for f in folded])
+        pp = (c_void_p * 2)(prep, prep)
+        rows = (c_void_p * 2)(*[c_void_p(pv.lib.zkp_g1_devptr(c_void_p(coms[j].h))) for j in com_order])
+        nr = np.array([coms[j].size for j in com_order], np.uint32)
+        ur = (c_void_p * 2)(*[c_void_p(urows[j].ctypes.data if urows[j].size else None) for j in com_order])
+        kr = np.array([urows[j].shape[0] for j in com_order], np.int32)
+        uall = np.ascontiguousarray(np.concatenate(us), dtype=np.uint32)
+        print(f"zk_g1_open_begin_batch_rows, commitments {com_order}", flush=True)
+        hip.call("zk_g1_open_begin_batch_rows", ctypes.byref(h), c_int(2), sc, pp, uall, c_int(k), rows, nr, ur, kr, None)
+        got_p = np.zeros_like(exp_p)
+        got_v = np.zeros_like(exp_v)
+        hip.call("zk_g1_open_end_batch", h, got_p, got_v)
+        return got_p, got_v
+
+    got_p, got_v = run((0, 1))
+    assert (got_v == exp_v).all()
+    assert (got_p == exp_p).all()
+    # the statement "these are the tensor's row commitments" is the caller's: with the other tensor's, T of the first round
+    # is what those commitments give, and with it T of the second halving round, which follows from the first round's three
+    # points (5000 -> 2500 -> 1250 generators, then the batched last rounds, which sum over the generators); T0, T1 of
+    # every round, the folded generator and the value do not depend on them
+    got_p, got_v = run((1, 0))
+    assert (got_v == exp_v).all()
+    same = np.ones(npts, bool)
+    same[[0, 3]] = False
+    assert (got_p[:, same] == exp_p[:, same]).all()
+    for i in range(2):
+        assert not (got_p[i, 0] == exp_p[i, 0]).all() and not (got_p[i, 3] == exp_p[i, 3]).all()
+    hip.call("zk_g1_open_prepared_free", prep)
+
+
 def test_fixed_base_multiplication_equals_the_generic_one_and_big_integer_arithmetic(orc):
     """zk_g1_fixed_base_mul (what Commitment::random runs on) against zk_g1_scalar_mul on the same base and, for the
     small cases, against affine big-integer arithmetic: digits at the signed-window boundaries (127, 128, 129, bytes of

@@ -119,6 +119,20 @@ def test_full_shape_layer_gives_one_output_head_by_head_and_stacked(pv):
     assert pv.transcript().shape[0] == sizes[1] + 9
     assert (out.host() == outs[0]).all()
     del out
+    # That run opened each weight where the reference does, every T as a sum over all generators.  The next one starts the
+    # nine openings with the layer, batched, the first two rounds on the prepared tables and T of the first round from the
+    # weights' row commitments: it must deliver the same field elements and the same G1 points.
+    first_t, first_g1 = pv.transcript().copy(), pv.transcript_g1().copy()
+    assert pv.lib.zkp_layer_planned_openings(ctypes.c_void_p(layer)) == 9
+    pv.seed(5)
+    pv.transcript_begin()
+    out, _ = pv.layer_run(layer, X)
+    pv.lib.zkp_transcript_end()
+    assert (out.host() == outs[0]).all()
+    del out
+    again_t, again_g1 = pv.transcript(), pv.transcript_g1()
+    assert again_t.shape == first_t.shape and (again_t == first_t).all()
+    assert again_g1.shape == first_g1.shape and first_g1.shape[0] > 9 * 30 and (again_g1 == first_g1).all()
     pv.layer_free(layer)
     assert (outs[0] == outs[1]).all() and (outs[0] == outs[2]).all()
     assert np.unique(outs[0], axis=0).shape[0] > 1000

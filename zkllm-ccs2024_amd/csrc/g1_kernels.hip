@@ -674,6 +674,32 @@ __global__ void __launch_bounds__(GT) k_open_chain(G1Jac* __restrict__ pts0, con
         pts[3 * r] = tot;
     }
 }
+// T of an opening's first round from the tensor's row commitments: the opened vector is the row fold of the committed tensor,
+// s = sum_r e_r W[r], e_r = prod_j (bit_j(r) ? u_j : 1 - u_j) over the row challenges, so sum_i s_i g_i = sum_r e_r C_r with
+// C_r = sum_i W[r][i] g_i the commitment of row r: a sum over the rows (a hundred points) instead of a bucket sum over all
+// generators.  Holds exactly when `rows` are the commitments of the tensor's rows under these generators -- what the caller
+// states by passing them.  Writes the window sums of T as k_open_horner reads them: the point in window 0, infinity above.
+// blockIdx.x: the opening.  u: the row challenges, Montgomery form, the lowest row bit first (as the row fold takes them).
+struct T0Batch { G1Jac* wsum[OB_MAX]; const G1Jac* rows[OB_MAX]; const Fr* u[OB_MAX]; uint32_t nrows[OB_MAX]; uint32_t k[OB_MAX]; };
+__global__ void __launch_bounds__(MT) k_open_t0_rows(const T0Batch tb) {
+    __shared__ uint32_t pool[36 * MT];
+    const uint32_t t = threadIdx.x, y = blockIdx.x;
+    const G1Jac* __restrict__ rows = tb.rows[y];
+    const Fr* __restrict__ u = tb.u[y];
+    const uint32_t nrows = tb.nrows[y], k = tb.k[y];
+    const Fr one = big_one_mont<8>();
+    G1Jac acc = g1_infinity();
+    for (uint32_t r = t; r < nrows; r += MT) {
+        Fr c = one;
+        for (uint32_t j = 0; j < k; ++j) c = mont_mul(c, ((r >> j) & 1u) ? u[j] : sub(one, u[j]));
+        const G1Jac P = rows[r];
+        if (!is_zero(P.z) && !is_zero(c)) acc = g1_add(acc, g1_mul_glv_lane(P, glv_split_device(from_mont(c))));
+    }
+    const G1Jac tot = msm_block_sum(pool, acc, t);
+    G1Jac* __restrict__ W = tb.wsum[y];
+    if (t == 0) W[0] = tot;
+    else if (t < (uint32_t)MW) W[t] = g1_infinity();
+}
 // ---- the fold on 29-bit-limb affine points ----------------------------------------------------------------------------------
 // The rounds of an opening keep the generators in ONE form: affine, 29-bit limbs (A29; all-zero limbs = infinity), canonical
 // limbs.  The bucket sums add out of it, the fold reads it and writes the next round's generators in it -- no
@@ -1200,7 +1226,8 @@ __global__ void __launch_bounds__(64) k_open_t_fix(G1Jac* __restrict__ wsum0, ui
 }
 // One round of `count` openings of equal size (count <= OB_MAX): one launch of each kernel covers all of them.
 // comb: the first round's table; comb2 (second round): the tables of F and H one after the other, u_prev the first round's challenge
-struct RoundItem { Fr* new_scalars; A29* new_gens; const Fr* scalars; const A29* gens; Fr u; const A29* comb = nullptr; const A29* comb2 = nullptr; Fr u_prev = Fr(); };
+struct RoundItem { Fr* new_scalars; A29* new_gens; const Fr* scalars; const A29* gens; Fr u; const A29* comb = nullptr; const A29* comb2 = nullptr; Fr u_prev = Fr();
+                   const G1Jac* rows = nullptr; uint32_t nrows = 0, k_rows = 0; const Fr* u_rows = nullptr; };      // first round: T from the row commitments (k_open_t0_rows)
 // Fp multiplications of one pair of the comb fold by the formulas' count
 static double comb_fp_mults_per_pair(const CombK& ck, const CombK* ck2 = nullptr) {
     int adds = 0, phis = 0;
@@ -1226,7 +1253,9 @@ static int open_round_launch(const RoundItem* items, int count, size_t old_size,
     ZK_ARG(old_size < (1ull << 31), "opening: more than 2^31 generators");
     ZK_ARG(count >= 1 && count <= OB_MAX, "opening: bad batch size");
     const size_t new_size = (old_size + 1) / 2;
-    const bool chained = !with_T;
+    bool t_given = with_T;                    // the first round's T comes from row commitments: no pair sums
+    for (int i = 0; i < count; ++i) t_given = t_given && items[i].rows != nullptr;
+    const bool chained = !with_T || t_given;
     const size_t dig_bytes = (size_t)(MW + 1) * old_size;
     Scratch& dig = arena.add(dig_bytes * count);
     if (dig.rc) return dig.rc;
@@ -1300,6 +1329,14 @@ static int open_round_launch(const RoundItem* items, int count, size_t old_size,
         hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, aux, wsum, cur, ns, n_per, wsum_item_stride);
     }
     if (!chained) hipLaunchKernelGGL(k_open_t_fix, dim3(count), dim3(64), 0, aux, wsum, wsum_item_stride);
+    if (t_given) {
+        T0Batch tb;
+        for (int i = 0; i < OB_MAX; ++i) {
+            const int k = i < count ? i : 0;
+            tb.wsum[i] = wsum_round + (size_t)wsum_item_stride * k; tb.rows[i] = items[k].rows; tb.u[i] = items[k].u_rows; tb.nrows[i] = items[k].nrows; tb.k[i] = items[k].k_rows;
+        }
+        hipLaunchKernelGGL(k_open_t0_rows, dim3(count), dim3(MT), 0, aux, tb);
+    }
     ZK_LAUNCH_CHECK();
     // ---- critical chain (st): the fold ----
     const size_t sp_stride = 1 + new_size;
@@ -1655,7 +1692,8 @@ struct OpenJob {
 };
 // One opening of the batch: its scalars, its challenges (rounds x 8 limbs) and its generators -- Jacobian, or null when
 // `prep` (their prepared form, open_prep_build) is given
-struct OpenItem { const void* scalars; const void* gens; const A29* prep; const uint32_t* u; const A29* comb = nullptr; const A29* comb2 = nullptr; };
+struct OpenItem { const void* scalars; const void* gens; const A29* prep; const uint32_t* u; const A29* comb = nullptr; const A29* comb2 = nullptr;
+                  const void* rows = nullptr; uint32_t nrows = 0; const uint32_t* u_rows = nullptr; int k_rows = 0; };     // row commitments of the opened tensor (optional)
 static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, int rounds, hipStream_t st, hipStream_t aux) {
     ZK_ARG(n >= 1, "zk_g1_open: empty input");
     ZK_ARG(count >= 1 && count <= OB_MAX, "zk_g1_open: a batch holds 1 to 8 openings");
@@ -1673,7 +1711,9 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
     if (pts.rc) return pts.rc;
     if (wsum.rc) return wsum.rc;
     job.pts = pts.as<G1Jac>();
-    ZK_ARG(sizeof(Fr) * (size_t)rounds * count <= JOB_U_BYTES, "zk_g1_open: too many rounds for the batch");
+    size_t n_urows = 0;
+    for (int i = 0; i < count; ++i) n_urows += items[i].rows ? (size_t)items[i].k_rows : 0;
+    ZK_ARG(sizeof(Fr) * ((size_t)rounds * count + n_urows) <= JOB_U_BYTES, "zk_g1_open: too many rounds for the batch");
     Scratch& jdev = job.arena.add(JOB_U_BYTES + JOB_DESC_BYTES);
     if (jdev.rc) return jdev.rc;
     {
@@ -1682,9 +1722,18 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
         Fr* hu = (Fr*)job.pin;
         for (int i = 0; i < count; ++i)
             for (int r = 0; r < rounds; ++r) hu[(size_t)i * rounds + r] = to_mont(load_fr(items[i].u + 8 * r));
-        if (rounds) ZK_HIP(hipMemcpyAsync(jdev.p, job.pin, sizeof(Fr) * (size_t)rounds * count, hipMemcpyHostToDevice, st));
+        size_t at = (size_t)rounds * count;           // the row challenges follow
+        for (int i = 0; i < count; ++i)
+            if (items[i].rows)
+                for (int j = 0; j < items[i].k_rows; ++j) hu[at++] = to_mont(load_fr(items[i].u_rows + 8 * j));
+        if (at) ZK_HIP(hipMemcpyAsync(jdev.p, job.pin, sizeof(Fr) * at, hipMemcpyHostToDevice, st));
     }
     const Fr* U_dev = jdev.as<Fr>();
+    const Fr* urow_dev[OB_MAX];
+    {
+        size_t at = (size_t)rounds * count;
+        for (int i = 0; i < count; ++i) { urow_dev[i] = U_dev + at; if (items[i].rows) at += (size_t)items[i].k_rows; }
+    }
     const Fr* cs[OB_MAX];
     const A29* cg[OB_MAX];
     for (int i = 0; i < count; ++i) {
@@ -1717,7 +1766,10 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
         RoundItem ri[OB_MAX];
         for (int i = 0; i < count; ++i) {
             ri[i] = RoundItem{s2.as<Fr>() + ns * i, g2.as<A29>() + ns * i, cs[i], cg[i], load_fr(items[i].u + 8 * r)};
-            if (r == 0) ri[i].comb = items[i].comb;
+            if (r == 0) {
+                ri[i].comb = items[i].comb;
+                if (items[i].rows) { ri[i].rows = (const G1Jac*)items[i].rows; ri[i].nrows = items[i].nrows; ri[i].k_rows = (uint32_t)items[i].k_rows; ri[i].u_rows = urow_dev[i]; }
+            }
             if (r == 1) { ri[i].comb2 = items[i].comb2; ri[i].u_prev = load_fr(items[i].u + 8 * (r - 1)); }
         }
         int rc = open_round_launch(ri, count, size, r == 0, wsum.as<G1Jac>() + (size_t)3 * MW * r, wstride, job.arena, st, aux, job.events);
@@ -1919,6 +1971,26 @@ int zk_g1_open_begin_batch(void** handle, int count, const void* const* scalars,
         if (i == 0) n = pr->n;
         ZK_ARG(pr->n == n, "zk_g1_open_begin_batch: the generator sets differ in size");
         items[i] = OpenItem{scalars[i], nullptr, (const A29*)pr->a29, u + (size_t)i * rounds * 8, (const A29*)pr->comb, (const A29*)pr->comb2};
+    }
+    return open_begin_impl(handle, items, count, n, rounds, stv);
+}
+// zk_g1_open_begin_batch for vectors that are row folds of committed tensors: rows[i] holds tensor i's nrows[i] row
+// commitments under the same generators, u_rows[i] the k_rows[i] challenges its rows were folded with (lowest row bit
+// first, 2^k_rows >= nrows).  T of the first round is then the same combination of the row commitments -- equal as a group
+// element to the sum over all generators that zk_g1_open_begin_batch computes, provided the commitments are the tensor's.
+int zk_g1_open_begin_batch_rows(void** handle, int count, const void* const* scalars, const void* const* prepared, const uint32_t* u, int rounds,
+                                const void* const* rows, const uint32_t* nrows, const uint32_t* const* u_rows, const int* k_rows, void* stv) {
+    ZK_ARG(count >= 1 && count <= OB_MAX, "zk_g1_open_begin_batch_rows: 1 to 8 openings");
+    ZK_ARG(scalars != nullptr && prepared != nullptr && u != nullptr && rows != nullptr && nrows != nullptr && u_rows != nullptr && k_rows != nullptr, "zk_g1_open_begin_batch_rows: null argument");
+    OpenItem items[OB_MAX];
+    size_t n = 0;
+    for (int i = 0; i < count; ++i) {
+        ZK_ARG(prepared[i] != nullptr && scalars[i] != nullptr && rows[i] != nullptr, "zk_g1_open_begin_batch_rows: null opening");
+        ZK_ARG(nrows[i] >= 1 && k_rows[i] >= 0 && k_rows[i] <= 31 && ((uint64_t)1 << k_rows[i]) >= nrows[i] && (k_rows[i] == 0 || u_rows[i] != nullptr), "zk_g1_open_begin_batch_rows: rows and row challenges do not fit");
+        const OpenPrepared* pr = (const OpenPrepared*)prepared[i];
+        if (i == 0) n = pr->n;
+        ZK_ARG(pr->n == n, "zk_g1_open_begin_batch_rows: the generator sets differ in size");
+        items[i] = OpenItem{scalars[i], nullptr, (const A29*)pr->a29, u + (size_t)i * rounds * 8, (const A29*)pr->comb, (const A29*)pr->comb2, rows[i], nrows[i], u_rows[i], k_rows[i]};
     }
     return open_begin_impl(handle, items, count, n, rounds, stv);
 }

@@ -76,7 +76,7 @@ Fr_t Commitment::open(const FrTensor& t, const G1TensorJacobian& com, const vect
     }
     return me_open(folded, *this, u_in.begin(), u_in.end(), proof);
 }
-Commitment::Pending Commitment::open_fold(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u) const {
+Commitment::Pending Commitment::open_fold(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u, bool rows_commit) const {
     const uint k_out = ceilLog2(com.size);
     if (u.size() < k_out) throw std::runtime_error("Commitment::open - too few challenges");
     const vector<Fr_t> u_out(u.end() - k_out, u.end());
@@ -84,6 +84,7 @@ Commitment::Pending Commitment::open_fold(const FrTensor& t, const G1TensorJacob
     p.u_in.assign(u.begin(), u.end() - k_out);
     p.folded.reset(new FrTensor(u_out.empty() ? FrTensor(t) : t.partial_me(u_out, t.size / com.size)));
     if (p.folded->size != size) throw std::runtime_error("Commitment::me_open - Incompatible dimensions " + std::to_string(p.folded->size) + " " + std::to_string(size));
+    if (rows_commit) { p.row_com = &com; p.u_out = u_out; }
     return p;
 }
 void Commitment::open_start(Pending& p) const {
@@ -134,7 +135,23 @@ void Commitment::open_start_batch(const std::vector<std::pair<const Commitment*,
             pr.push_back(ops[group[k]].first->prepared.get());
             for (int r = 0; r < b->rounds; ++r) memcpy(&uu[((size_t)k * b->rounds + r) * 8], q->u_in[r].val, 32);
         }
-        ZKC(zk_g1_open_begin_batch(&b->handle, b->count, sc.data(), pr.data(), uu.data(), b->rounds, nullptr));
+        bool with_rows = true;
+        for (size_t k = 0; k < group.size(); ++k) with_rows = with_rows && ops[group[k]].second->row_com != nullptr;
+        if (with_rows) {
+            std::vector<const void*> rows;
+            std::vector<uint32_t> nrows;
+            std::vector<const uint32_t*> urows;
+            std::vector<int> krows;
+            for (size_t k = 0; k < group.size(); ++k) {
+                Pending* q = ops[group[k]].second;
+                rows.push_back(q->row_com->gpu_data);
+                nrows.push_back(q->row_com->size);
+                urows.push_back(q->u_out.empty() ? nullptr : q->u_out[0].val);
+                krows.push_back((int)q->u_out.size());
+            }
+            ZKC(zk_g1_open_begin_batch_rows(&b->handle, b->count, sc.data(), pr.data(), uu.data(), b->rounds, rows.data(), nrows.data(), urows.data(), krows.data(), nullptr));
+        } else
+            ZKC(zk_g1_open_begin_batch(&b->handle, b->count, sc.data(), pr.data(), uu.data(), b->rounds, nullptr));
         for (size_t k = 0; k < group.size(); ++k) {
             Pending* q = ops[group[k]].second;
             q->rounds = b->rounds;

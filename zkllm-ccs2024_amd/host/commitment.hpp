@@ -36,6 +36,8 @@ class Commitment : public G1TensorJacobian {
         int rounds = 0;
         Fr_t value{{0, 0, 0, 0, 0, 0, 0, 0}};
         vector<Fr_t> u_in;                  // between open_fold and open_start: the challenges of the G1 recursion
+        const G1TensorJacobian* row_com = nullptr;      // open_fold(..., rows_commit = true): the tensor's row commitments and the
+        vector<Fr_t> u_out;                             // challenges its rows were folded with (open_start_batch takes T of the first round from them)
         struct Batch;                       // openings started as one job (open_start_batch) share its handle and results
         std::shared_ptr<Batch> batch;
         int batch_index = 0;
@@ -44,7 +46,10 @@ class Commitment : public G1TensorJacobian {
     // open_begin in its two steps: open_fold reduces the rows to the vector that is opened (a pass over the whole tensor
     // on the caller's stream), open_start queues the G1 recursion.  Several openings started together fold first and
     // start afterwards: a fold queued behind another opening's G1 kernels waits for the registers they hold.
-    Pending open_fold(const FrTensor& t, const G1TensorJacobian& c, const vector<Fr_t>& u) const;
+    // rows_commit: the caller states that c holds the commitments of t's rows under these generators (what create_weight
+    // loads and verifyWeightClaim opens against; commitment.cu:137 evaluates them at u_out as well): a batched start may
+    // then take the first round's T from them.  c must outlive the pending opening.
+    Pending open_fold(const FrTensor& t, const G1TensorJacobian& c, const vector<Fr_t>& u, bool rows_commit = false) const;
     void open_start(Pending& p) const;
     // open_start for several folded openings at once: those whose generators are prepared and agree in size and round
     // count run as one device job each group (zk_g1_open_begin_batch), the rest one by one
