@@ -84,6 +84,10 @@ int zk_fr_transpose(void* out, const void* in, uint32_t M, uint32_t N, void* str
 /* the same for a stack of `batch` M x N matrices stored one after the other (per-head K^T of zkAttn::compute, zksoftmax.cu:234) */
 int zk_fr_transpose_batched(void* out, const void* in, uint32_t batch, uint32_t M, uint32_t N, void* stream);
 int zk_fr_gather(void* out, const void* table, const void* idx_u32, size_t n, void* stream);
+/* dst[i] = src[offset + i * stride], i < count, for elements of elem_bytes (a multiple of 16: field elements, G1 points):
+ * every 2^k-th column of a row-major tensor or generator vector (no counterpart in the reference; the cross commitments
+ * of zk_g1_open_begin_batch_rows are commitments of such parts). */
+int zk_copy_strided(void* dst, const void* src, size_t elem_bytes, size_t count, size_t stride, size_t offset, void* stream);
 
 /* ---- reductions and folds ------------------------------------------------------------------------ */
 /* FrTensor::sum (fr-tensor.cu:382-434) */
@@ -187,14 +191,20 @@ int zk_g1_open_begin_prepared(void** handle, const void* scalars, const void* pr
  * delivers opening i's points at proof_host + i * (3 rounds + 1) * 36 and its folded scalar at final_scalar_host + i * 8. */
 int zk_g1_open_begin_batch(void** handle, int count, const void* const* scalars, const void* const* prepared, const uint32_t* u, int rounds, void* stream);
 /* zk_g1_open_begin_batch for openings as Commitment::open makes them (commitment.cu:133-141): the opened vector is the
- * tensor's rows folded at u_out, and the reference evaluates the row commitments there too (com(u_out), :137).  rows[i]:
- * tensor i's nrows[i] row commitments (Jacobian, 36 limbs each, on the device, alive until end); u_rows[i]: the
- * k_rows[i] challenges the rows were folded with, lowest row bit first, 2^k_rows >= nrows.  The first round's T is then
- * sum_r eq(u_rows, r) rows[r] instead of a sum over all generators: the same group element whenever rows are the
- * commitments of the tensor's rows under these generators -- the caller's statement; with other rows the T of the
- * halving rounds (each follows from the round before) differ from zk_g1_open_begin_batch's, nothing else does. */
+ * tensor's rows folded at u_out, and the reference evaluates the row commitments there too (com(u_out), :137).
+ * rows[i]: commitments of tensor i's nrows[i] rows (Jacobian, 36 limbs each, on the device, alive until end), laid out
+ * [pattern][row]: pattern 0 the row commitments C_r = sum_i W[r][i] g_i; with cross_rounds = R > 0 they are followed, for
+ * q = 0 .. R-1, by the 4^q patterns p = a 2^q + b of T0_q, X[r] = sum_j W[r][2^(q+1) j + a] g_(2^(q+1) j + 2^q + b), and the
+ * 4^q of T1_q, X[r] = sum_j W[r][2^(q+1) j + 2^q + a] g_(2^(q+1) j + b): 1 + 2 (4^R - 1) / 3 patterns in all (the host
+ * layer's Commitment::cross_commitments makes them with commit_int over strided parts).  u_rows[i]: the k_rows[i] challenges
+ * the rows were folded with, lowest row bit first, 2^k_rows >= nrows.
+ * T of the first round is then sum_r eq(u_rows, r) C_r, and T0, T1 of the first R halving rounds are the combinations
+ * of the cross patterns with the products of the earlier rounds' challenges -- sums over rows x patterns points instead
+ * of bucket sums over all generators; those rounds then consist of their fold alone.  The points equal the sums over the
+ * generators whenever rows[i] are such commitments of the tensor under these generators -- the caller's statement;
+ * with other points T, T0, T1 of the halving rounds differ from zk_g1_open_begin_batch's, nothing else does. */
 int zk_g1_open_begin_batch_rows(void** handle, int count, const void* const* scalars, const void* const* prepared, const uint32_t* u, int rounds,
-                                const void* const* rows, const uint32_t* nrows, const uint32_t* const* u_rows, const int* k_rows, void* stream);
+                                const void* const* rows, const uint32_t* nrows, const uint32_t* const* u_rows, const int* k_rows, int cross_rounds, void* stream);
 int zk_g1_open_end_batch(void* handle, uint32_t* proof_host, uint32_t* final_scalar_host);
 
 /* ---- lookup argument (tlookup.cu) ------------------------------------------------------------------------ */

@@ -388,7 +388,7 @@ def test_open_batch_with_row_commitments_delivers_the_points_of_the_plain_openin
         kr = np.array([urows[j].shape[0] for j in com_order], np.int32)
         uall = np.ascontiguousarray(np.concatenate(us), dtype=np.uint32)
         print(f"zk_g1_open_begin_batch_rows, commitments {com_order}", flush=True)
-        hip.call("zk_g1_open_begin_batch_rows", ctypes.byref(h), c_int(2), sc, pp, uall, c_int(k), rows, nr, ur, kr, None)
+        hip.call("zk_g1_open_begin_batch_rows", ctypes.byref(h), c_int(2), sc, pp, uall, c_int(k), rows, nr, ur, kr, c_int(0), None)
         got_p = np.zeros_like(exp_p)
         got_v = np.zeros_like(exp_v)
         hip.call("zk_g1_open_end_batch", h, got_p, got_v)
@@ -409,6 +409,72 @@ def test_open_batch_with_row_commitments_delivers_the_points_of_the_plain_openin
     for i in range(2):
         assert not (got_p[i, 0] == exp_p[i, 0]).all() and not (got_p[i, 3] == exp_p[i, 3]).all()
     hip.call("zk_g1_open_prepared_free", prep)
+
+
+def test_open_batch_with_cross_commitments_needs_no_sum_over_the_generators(pv):
+    """With the cross commitments of its first two rounds -- commitments of every 2nd / 4th column of the tensor's rows
+    under every 2nd / 4th generator, made here with commit_int on slices -- zk_g1_open_begin_batch_rows forms T, T0 and T1
+    of those rounds from rows x patterns points; 8192 generators are halved twice before the batched last rounds, so no
+    round sums over its generators.  Every point of the proof equals zk_g1_open's on the row-folded vector."""
+    import ctypes
+    from gpuhelp import Hip, c_void_p, c_size_t, c_int
+    hip = Hip()
+    pv.lib.zkp_g1_devptr.restype = ctypes.c_void_p
+    n, R = 8192, 2
+    k = (n - 1).bit_length()
+    npts = 3 * k + 1
+    pv.seed(78)
+    gens = pv.commitment_random(n)
+    gens_host = gens.host()
+    dG = pv.lib.zkp_g1_devptr(c_void_p(gens.h))
+    prep = c_void_p()
+    hip.call("zk_g1_open_prepare", ctypes.byref(prep), c_void_p(dG), c_size_t(n), None)
+    rng = np.random.default_rng(6)
+    keep, folded, cross, urows, us = [], [], [], [], []
+    exp_p = np.zeros((2, npts, 36), np.uint32)
+    exp_v = np.zeros((2, 8), np.uint32)
+    for i, nrows in enumerate((3, 4)):
+        Wi = rng.integers(-30000, 30000, (nrows, n)).astype(np.int32)
+        W = pv.from_i32(Wi.ravel())
+        pats = [pv.commit_int(gens, W).host()]
+        for q in range(R):
+            half, L = 1 << q, 2 << q
+            for side in (0, 1):
+                for a in range(half):
+                    for b in range(half):
+                        s_off, g_off = (half if side else 0) + a, (0 if side else half) + b
+                        sub_g = pv.g1_from_host(np.ascontiguousarray(gens_host[g_off::L]))
+                        sub_w = pv.from_i32(np.ascontiguousarray(Wi[:, s_off::L]).ravel())
+                        pats.append(pv.commit_int(sub_g, sub_w).host())
+        assert len(pats) == 1 + 2 + 8 and all(x.shape == (nrows, 36) for x in pats)
+        cross.append(hip.upload(np.ascontiguousarray(np.concatenate(pats))))
+        kr = (nrows - 1).bit_length()
+        ur = mt_random_vec(np.random.RandomState(45 + i), kr)
+        f = pv.partial_me_window(W, ur, n)
+        u = mt_random_vec(np.random.RandomState(65 + i), k)
+        print(f"rows={nrows}: zk_g1_open", flush=True)
+        hip.call("zk_g1_open", exp_p[i], exp_v[i], c_void_p(f.devptr), c_void_p(dG), c_size_t(n), u, c_int(k), None)
+        keep += [W, f]
+        folded.append(f); urows.append(np.ascontiguousarray(ur, dtype=np.uint32)); us.append(u)
+    for cr in (2, 1):
+        h = c_void_p()
+        sc = (c_void_p * 2)(*[c_void_p(f.devptr) for f in folded])
+        pp = (c_void_p * 2)(prep, prep)
+        rows = (c_void_p * 2)(*[c_void_p(x) for x in cross])
+        nr = np.array([3, 4], np.uint32)
+        ur = (c_void_p * 2)(*[c_void_p(x.ctypes.data) for x in urows])
+        kr = np.array([x.shape[0] for x in urows], np.int32)
+        uall = np.ascontiguousarray(np.concatenate(us), dtype=np.uint32)
+        print(f"zk_g1_open_begin_batch_rows with {cr} rounds of cross commitments", flush=True)
+        hip.call("zk_g1_open_begin_batch_rows", ctypes.byref(h), c_int(2), sc, pp, uall, c_int(k), rows, nr, ur, kr, c_int(cr), None)
+        got_p = np.zeros_like(exp_p)
+        got_v = np.zeros_like(exp_v)
+        hip.call("zk_g1_open_end_batch", h, got_p, got_v)
+        assert (got_v == exp_v).all(), cr
+        assert (got_p == exp_p).all(), cr
+    hip.call("zk_g1_open_prepared_free", prep)
+    for x in cross:
+        hip.free(x)
 
 
 def test_fixed_base_multiplication_equals_the_generic_one_and_big_integer_arithmetic(orc):

@@ -550,6 +550,21 @@ int zk_fr_transpose_batched(void* out, const void* in, uint32_t batch, uint32_t 
     return 0;
 }
 int zk_fr_transpose(void* out, const void* in, uint32_t M, uint32_t N, void* st) { return zk_fr_transpose_batched(out, in, 1, M, N, st); }
+// dst[i] = src[offset + i * stride] for elements of `words` 16-byte words (a field element 2, a Jacobian point 9)
+__global__ void __launch_bounds__(TPB) k_copy_strided(uint4* __restrict__ dst, const uint4* __restrict__ src, uint32_t words, size_t count, size_t stride, size_t offset) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= count * words) return;
+    const size_t e = i / words, w = i - e * words;
+    dst[i] = src[(offset + e * stride) * words + w];
+}
+int zk_copy_strided(void* dst, const void* src, size_t elem_bytes, size_t count, size_t stride, size_t offset, void* st) {
+    ZK_ARG(elem_bytes >= 16 && elem_bytes % 16 == 0 && elem_bytes <= 1024, "zk_copy_strided: elements of 16 to 1024 bytes, a multiple of 16");
+    ZK_ARG(dst != src, "zk_copy_strided: in place");
+    if (count == 0) return 0;
+    const uint32_t words = (uint32_t)(elem_bytes / 16);
+    LAUNCH1D(k_copy_strided, count * words, st, (uint4*)dst, (const uint4*)src, words, count, stride, offset);
+    return 0;
+}
 int zk_fr_gather(void* out, const void* table, const void* idx, size_t n, void* st) {
     LAUNCH1D(k_gather, n, st, (Fr*)out, (const Fr*)table, (const uint32_t*)idx, n);
     return 0;

@@ -674,31 +674,70 @@ __global__ void __launch_bounds__(GT) k_open_chain(G1Jac* __restrict__ pts0, con
         pts[3 * r] = tot;
     }
 }
-// T of an opening's first round from the tensor's row commitments: the opened vector is the row fold of the committed tensor,
-// s = sum_r e_r W[r], e_r = prod_j (bit_j(r) ? u_j : 1 - u_j) over the row challenges, so sum_i s_i g_i = sum_r e_r C_r with
-// C_r = sum_i W[r][i] g_i the commitment of row r: a sum over the rows (a hundred points) instead of a bucket sum over all
-// generators.  Holds exactly when `rows` are the commitments of the tensor's rows under these generators -- what the caller
-// states by passing them.  Writes the window sums of T as k_open_horner reads them: the point in window 0, infinity above.
-// blockIdx.x: the opening.  u: the row challenges, Montgomery form, the lowest row bit first (as the row fold takes them).
-struct T0Batch { G1Jac* wsum[OB_MAX]; const G1Jac* rows[OB_MAX]; const Fr* u[OB_MAX]; uint32_t nrows[OB_MAX]; uint32_t k[OB_MAX]; };
-__global__ void __launch_bounds__(MT) k_open_t0_rows(const T0Batch tb) {
+// Sums of an opening's first rounds from commitments of the opened tensor's rows.  The opened vector is the row fold of a
+// tensor W, s = sum_r e_r W[r] with e_r = prod_j (bit_j(r) ? v_j : 1 - v_j) over the row challenges v, so every sum of the
+// form  sum_j s_(L j + x) g_(L j + y)  equals  sum_r e_r X[r]  with  X[r] = sum_j W[r][L j + x] g_(L j + y),  a point that
+// depends on the tensor and the generators alone and can be made in advance (a commitment of a strided part of the row
+// under a strided part of the generators).  T0 and T1 of round q are combinations of 4^q such sums each: with u_0 .. u_(q-1)
+// the challenges of the rounds before,
+//   s^(q)_m = sum_{a < 2^q} s_(2^q m + a) prod_k (bit_k(a) ? u_k : 1 - u_k),   g^(q)_m = sum_{b < 2^q} g_(2^q m + b) prod_k (bit_k(b) ? 1 - u_k : u_k),
+//   T0_q = sum_j s^(q)_(2j) g^(q)_(2j+1) = sum_{a,b} c(a,b) sum_j s_(2^(q+1) j + a) g_(2^(q+1) j + 2^q + b),   T1_q likewise with the halves exchanged,
+// and T of round 0 is the same combination of the row commitments themselves.  `pts`: [pattern][row] points, pattern 0 the row
+// commitments, then for q = 0 .. cross_rounds - 1 the 4^q patterns (a 2^q + b) of T0_q followed by those of T1_q.
+// Target t of an opening: 0 = T of round 0, 1 + 2q + side = T0_q / T1_q.  The results go where k_open_horner reads the window
+// sums of those points: the point in window 0, infinity above.  They equal the sums over all generators exactly when `pts`
+// are such commitments of the opened tensor -- what the caller states by passing them.
+struct CrossItem { G1Jac* wsum; G1Jac* part; const G1Jac* pts; const Fr* u_rows; const Fr* u; uint32_t nrows, k_rows; };
+struct CrossBatch { CrossItem it[OB_MAX]; };
+__device__ __forceinline__ void cross_target(uint32_t t, uint32_t& q, uint32_t& first_pattern, uint32_t& npat, uint32_t& slot) {
+    if (t == 0) { q = 0; first_pattern = 0; npat = 1; slot = 0; return; }
+    q = (t - 1) >> 1;
+    const uint32_t side = (t - 1) & 1u, four_q = 1u << (2 * q);
+    npat = four_q;
+    first_pattern = 1 + 2 * (four_q - 1) / 3 + side * four_q;
+    slot = (3 * q + 1 + side) * (uint32_t)MW;
+}
+// grid (chunks, targets, openings): chunk c of a target sums its terms [c MT, (c+1) MT) into part[(t chunks + c)]
+__global__ void __launch_bounds__(MT) k_open_cross_part(const CrossBatch cb) {
     __shared__ uint32_t pool[36 * MT];
-    const uint32_t t = threadIdx.x, y = blockIdx.x;
-    const G1Jac* __restrict__ rows = tb.rows[y];
-    const Fr* __restrict__ u = tb.u[y];
-    const uint32_t nrows = tb.nrows[y], k = tb.k[y];
-    const Fr one = big_one_mont<8>();
+    const CrossItem& it = cb.it[blockIdx.z];
+    const uint32_t t = blockIdx.y, c = blockIdx.x, lane = threadIdx.x;
+    uint32_t q, p0, npat, slot;
+    cross_target(t, q, p0, npat, slot);
+    const uint32_t nrows = it.nrows, terms = npat * nrows, idx = c * MT + lane;
     G1Jac acc = g1_infinity();
-    for (uint32_t r = t; r < nrows; r += MT) {
-        Fr c = one;
-        for (uint32_t j = 0; j < k; ++j) c = mont_mul(c, ((r >> j) & 1u) ? u[j] : sub(one, u[j]));
-        const G1Jac P = rows[r];
-        if (!is_zero(P.z) && !is_zero(c)) acc = g1_add(acc, g1_mul_glv_lane(P, glv_split_device(from_mont(c))));
+    if (idx < terms) {
+        const uint32_t pl = idx / nrows, row = idx - pl * nrows;
+        const Fr one = big_one_mont<8>();
+        Fr coef = one;
+        for (uint32_t j = 0; j < it.k_rows; ++j) coef = mont_mul(coef, ((row >> j) & 1u) ? it.u_rows[j] : sub(one, it.u_rows[j]));
+        if (t != 0) {
+            const uint32_t a = pl >> q, b = pl & ((1u << q) - 1u);
+            for (uint32_t k = 0; k < q; ++k) {
+                const Fr uk = it.u[k], nk = sub(one, uk);
+                coef = mont_mul(coef, mont_mul(((a >> k) & 1u) ? uk : nk, ((b >> k) & 1u) ? nk : uk));
+            }
+        }
+        const G1Jac P = it.pts[(size_t)(p0 + pl) * nrows + row];
+        if (!is_zero(P.z) && !is_zero(coef)) acc = g1_mul_glv_lane(P, glv_split_device(from_mont(coef)));
     }
-    const G1Jac tot = msm_block_sum(pool, acc, t);
-    G1Jac* __restrict__ W = tb.wsum[y];
-    if (t == 0) W[0] = tot;
-    else if (t < (uint32_t)MW) W[t] = g1_infinity();
+    const G1Jac tot = msm_block_sum(pool, acc, lane);
+    if (lane == 0) it.part[(size_t)t * gridDim.x + c] = tot;
+}
+// grid (targets, openings): the chunks of a target summed, the point written as window sums
+__global__ void __launch_bounds__(MT) k_open_cross_finish(const CrossBatch cb, uint32_t chunks) {
+    __shared__ uint32_t pool[36 * MT];
+    const CrossItem& it = cb.it[blockIdx.y];
+    const uint32_t t = blockIdx.x, lane = threadIdx.x;
+    uint32_t q, p0, npat, slot;
+    cross_target(t, q, p0, npat, slot);
+    const uint32_t used = (npat * it.nrows + MT - 1) / MT;            // chunks of this target that hold terms
+    G1Jac acc = g1_infinity();
+    for (uint32_t c = lane; c < used && c < chunks; c += MT) acc = g1_add(acc, it.part[(size_t)t * chunks + c]);
+    const G1Jac tot = msm_block_sum(pool, acc, lane);
+    G1Jac* __restrict__ W = it.wsum + slot;
+    if (lane == 0) W[0] = tot;
+    else if (lane < (uint32_t)MW) W[lane] = g1_infinity();
 }
 // ---- the fold on 29-bit-limb affine points ----------------------------------------------------------------------------------
 // The rounds of an opening keep the generators in ONE form: affine, 29-bit limbs (A29; all-zero limbs = infinity), canonical
@@ -1226,8 +1265,7 @@ __global__ void __launch_bounds__(64) k_open_t_fix(G1Jac* __restrict__ wsum0, ui
 }
 // One round of `count` openings of equal size (count <= OB_MAX): one launch of each kernel covers all of them.
 // comb: the first round's table; comb2 (second round): the tables of F and H one after the other, u_prev the first round's challenge
-struct RoundItem { Fr* new_scalars; A29* new_gens; const Fr* scalars; const A29* gens; Fr u; const A29* comb = nullptr; const A29* comb2 = nullptr; Fr u_prev = Fr();
-                   const G1Jac* rows = nullptr; uint32_t nrows = 0, k_rows = 0; const Fr* u_rows = nullptr; };      // first round: T from the row commitments (k_open_t0_rows)
+struct RoundItem { Fr* new_scalars; A29* new_gens; const Fr* scalars; const A29* gens; Fr u; const A29* comb = nullptr; const A29* comb2 = nullptr; Fr u_prev = Fr(); };
 // Fp multiplications of one pair of the comb fold by the formulas' count
 static double comb_fp_mults_per_pair(const CombK& ck, const CombK* ck2 = nullptr) {
     int adds = 0, phis = 0;
@@ -1248,14 +1286,15 @@ static CombK comb_of(const GlvK& k) {
         }
     return ck;
 }
-static int open_round_launch(const RoundItem* items, int count, size_t old_size, bool with_T, G1Jac* wsum_round, uint32_t wsum_item_stride, Arena& arena, hipStream_t st,
-                             hipStream_t aux, std::vector<hipEvent_t>& events) {
+// given: what of this round's sums comes from commitments of the tensor's rows (k_open_cross_part) and is not summed here:
+// 0 nothing, 1 T of the first round (no pair sums), 2 T0 and T1 as well (no bucket sums at all: the round is its fold)
+static int open_round_launch(const RoundItem* items, int count, size_t old_size, bool with_T, int given, G1Jac* wsum_round, uint32_t wsum_item_stride, Arena& arena,
+                             hipStream_t st, hipStream_t aux, std::vector<hipEvent_t>& events) {
     ZK_ARG(old_size < (1ull << 31), "opening: more than 2^31 generators");
     ZK_ARG(count >= 1 && count <= OB_MAX, "opening: bad batch size");
     const size_t new_size = (old_size + 1) / 2;
-    bool t_given = with_T;                    // the first round's T comes from row commitments: no pair sums
-    for (int i = 0; i < count; ++i) t_given = t_given && items[i].rows != nullptr;
-    const bool chained = !with_T || t_given;
+    const bool chained = !with_T || given >= 1;
+    if (given < 2) {
     const size_t dig_bytes = (size_t)(MW + 1) * old_size;
     Scratch& dig = arena.add(dig_bytes * count);
     if (dig.rc) return dig.rc;
@@ -1329,15 +1368,8 @@ static int open_round_launch(const RoundItem* items, int count, size_t old_size,
         hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, aux, wsum, cur, ns, n_per, wsum_item_stride);
     }
     if (!chained) hipLaunchKernelGGL(k_open_t_fix, dim3(count), dim3(64), 0, aux, wsum, wsum_item_stride);
-    if (t_given) {
-        T0Batch tb;
-        for (int i = 0; i < OB_MAX; ++i) {
-            const int k = i < count ? i : 0;
-            tb.wsum[i] = wsum_round + (size_t)wsum_item_stride * k; tb.rows[i] = items[k].rows; tb.u[i] = items[k].u_rows; tb.nrows[i] = items[k].nrows; tb.k[i] = items[k].k_rows;
-        }
-        hipLaunchKernelGGL(k_open_t0_rows, dim3(count), dim3(MT), 0, aux, tb);
-    }
     ZK_LAUNCH_CHECK();
+    }
     // ---- critical chain (st): the fold ----
     const size_t sp_stride = 1 + new_size;
     Scratch& special = arena.add(sizeof(uint32_t) * sp_stride * count);
@@ -1659,7 +1691,7 @@ int zk_g1_open_round(void* new_scalars, void* new_gens, uint32_t* sums_host, con
     if (rc) return rc;
     std::vector<hipEvent_t> evs;
     const RoundItem item{(Fr*)new_scalars, n29.as<A29>(), (const Fr*)scalars, g29.as<A29>(), load_fr(u), nullptr};
-    rc = open_round_launch(&item, 1, old_size, true, wsum.as<G1Jac>(), 0u, arena, st, st, evs);
+    rc = open_round_launch(&item, 1, old_size, true, 0, wsum.as<G1Jac>(), 0u, arena, st, st, evs);
     (void)evs;
     if (rc) return rc;
     hipLaunchKernelGGL(k_a29_to_jac, dim3(cdiv(new_size, GT)), dim3(GT), 0, st, (G1Jac*)new_gens, n29.as<A29>(), new_size);
@@ -1693,7 +1725,9 @@ struct OpenJob {
 // One opening of the batch: its scalars, its challenges (rounds x 8 limbs) and its generators -- Jacobian, or null when
 // `prep` (their prepared form, open_prep_build) is given
 struct OpenItem { const void* scalars; const void* gens; const A29* prep; const uint32_t* u; const A29* comb = nullptr; const A29* comb2 = nullptr;
-                  const void* rows = nullptr; uint32_t nrows = 0; const uint32_t* u_rows = nullptr; int k_rows = 0; };     // row commitments of the opened tensor (optional)
+                  const void* rows = nullptr; uint32_t nrows = 0; const uint32_t* u_rows = nullptr; int k_rows = 0; int cross_rounds = 0; };
+// rows (optional): commitments of the opened tensor's rows, [pattern][row] as k_open_cross_part takes them -- the row
+// commitments alone (cross_rounds = 0) or with the cross patterns of the first cross_rounds rounds
 static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, int rounds, hipStream_t st, hipStream_t aux) {
     ZK_ARG(n >= 1, "zk_g1_open: empty input");
     ZK_ARG(count >= 1 && count <= OB_MAX, "zk_g1_open: a batch holds 1 to 8 openings");
@@ -1747,6 +1781,44 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
             cg[i] = g29.as<A29>();
         }
     }
+    // commitments of the tensors' rows: which sums they replace (all openings of the batch must bring them)
+    bool with_rows = true;
+    int cross_r = 64;
+    for (int i = 0; i < count; ++i) { with_rows = with_rows && items[i].rows != nullptr; cross_r = std::min(cross_r, items[i].cross_rounds); }
+    if (!with_rows) cross_r = 0;
+    int rounds_from_rows = 0;                 // halving rounds that take sums from the row commitments
+    if (with_rows) {
+        int halving = 0;
+        size_t sz = n;
+        for (int r = 0; r < rounds && !(sz <= (size_t)TAIL_N && rounds - r <= TAIL_LEVELS); ++r) { ++halving; sz = (sz + 1) / 2; }
+        rounds_from_rows = std::min(halving, std::max(cross_r, 1));
+    }
+    if (rounds_from_rows > 0) {
+        // targets: T of round 0, then T0, T1 of every round whose bucket sums were left out
+        const int full = std::min(rounds_from_rows, cross_r);
+        const uint32_t ntargets = 1u + 2u * (uint32_t)full;
+        uint32_t max_terms = 0;
+        for (int i = 0; i < count; ++i) max_terms = std::max(max_terms, (full ? (1u << (2 * (full - 1))) : 1u) * items[i].nrows);
+        const uint32_t chunks = cdiv(max_terms, MT);
+        Scratch& part = job.arena.add(sizeof(G1Jac) * (size_t)ntargets * chunks * count);
+        if (part.rc) return part.rc;
+        CrossBatch cb;
+        for (int i = 0; i < OB_MAX; ++i) {
+            const int k = i < count ? i : 0;
+            cb.it[i] = CrossItem{wsum.as<G1Jac>() + (size_t)wstride * k, part.as<G1Jac>() + (size_t)ntargets * chunks * k, (const G1Jac*)items[k].rows, urow_dev[k],
+                                 U_dev + (size_t)k * rounds, items[k].nrows, (uint32_t)items[k].k_rows};
+        }
+        if (aux != st) {          // the challenges travel on st
+            hipEvent_t up;
+            ZK_HIP(hipEventCreateWithFlags(&up, hipEventDisableTiming));
+            job.events.push_back(up);
+            ZK_HIP(hipEventRecord(up, st));
+            ZK_HIP(hipStreamWaitEvent(aux, up, 0));
+        }
+        hipLaunchKernelGGL(k_open_cross_part, dim3(chunks, ntargets, count), dim3(MT), 0, aux, cb);
+        hipLaunchKernelGGL(k_open_cross_finish, dim3(ntargets, count), dim3(MT), 0, aux, cb, chunks);
+        ZK_LAUNCH_CHECK();
+    }
     size_t size = n;
     int halving_rounds = rounds;
     bool tail_done = false;
@@ -1766,13 +1838,11 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
         RoundItem ri[OB_MAX];
         for (int i = 0; i < count; ++i) {
             ri[i] = RoundItem{s2.as<Fr>() + ns * i, g2.as<A29>() + ns * i, cs[i], cg[i], load_fr(items[i].u + 8 * r)};
-            if (r == 0) {
-                ri[i].comb = items[i].comb;
-                if (items[i].rows) { ri[i].rows = (const G1Jac*)items[i].rows; ri[i].nrows = items[i].nrows; ri[i].k_rows = (uint32_t)items[i].k_rows; ri[i].u_rows = urow_dev[i]; }
-            }
+            if (r == 0) ri[i].comb = items[i].comb;
             if (r == 1) { ri[i].comb2 = items[i].comb2; ri[i].u_prev = load_fr(items[i].u + 8 * (r - 1)); }
         }
-        int rc = open_round_launch(ri, count, size, r == 0, wsum.as<G1Jac>() + (size_t)3 * MW * r, wstride, job.arena, st, aux, job.events);
+        const int given = !with_rows ? 0 : (r < cross_r ? 2 : (r == 0 ? 1 : 0));
+        int rc = open_round_launch(ri, count, size, r == 0, given, wsum.as<G1Jac>() + (size_t)3 * MW * r, wstride, job.arena, st, aux, job.events);
         if (rc) return rc;
         for (int i = 0; i < count; ++i) { cs[i] = ri[i].new_scalars; cg[i] = ri[i].new_gens; }
         size = ns;
@@ -1979,7 +2049,8 @@ int zk_g1_open_begin_batch(void** handle, int count, const void* const* scalars,
 // first, 2^k_rows >= nrows).  T of the first round is then the same combination of the row commitments -- equal as a group
 // element to the sum over all generators that zk_g1_open_begin_batch computes, provided the commitments are the tensor's.
 int zk_g1_open_begin_batch_rows(void** handle, int count, const void* const* scalars, const void* const* prepared, const uint32_t* u, int rounds,
-                                const void* const* rows, const uint32_t* nrows, const uint32_t* const* u_rows, const int* k_rows, void* stv) {
+                                const void* const* rows, const uint32_t* nrows, const uint32_t* const* u_rows, const int* k_rows, int cross_rounds, void* stv) {
+    ZK_ARG(cross_rounds >= 0 && cross_rounds <= 4, "zk_g1_open_begin_batch_rows: 0 to 4 rounds of cross commitments");
     ZK_ARG(count >= 1 && count <= OB_MAX, "zk_g1_open_begin_batch_rows: 1 to 8 openings");
     ZK_ARG(scalars != nullptr && prepared != nullptr && u != nullptr && rows != nullptr && nrows != nullptr && u_rows != nullptr && k_rows != nullptr, "zk_g1_open_begin_batch_rows: null argument");
     OpenItem items[OB_MAX];
@@ -1990,7 +2061,7 @@ int zk_g1_open_begin_batch_rows(void** handle, int count, const void* const* sca
         const OpenPrepared* pr = (const OpenPrepared*)prepared[i];
         if (i == 0) n = pr->n;
         ZK_ARG(pr->n == n, "zk_g1_open_begin_batch_rows: the generator sets differ in size");
-        items[i] = OpenItem{scalars[i], nullptr, (const A29*)pr->a29, u + (size_t)i * rounds * 8, (const A29*)pr->comb, (const A29*)pr->comb2, rows[i], nrows[i], u_rows[i], k_rows[i]};
+        items[i] = OpenItem{scalars[i], nullptr, (const A29*)pr->a29, u + (size_t)i * rounds * 8, (const A29*)pr->comb, (const A29*)pr->comb2, rows[i], nrows[i], u_rows[i], k_rows[i], cross_rounds};
     }
     return open_begin_impl(handle, items, count, n, rounds, stv);
 }

@@ -76,7 +76,39 @@ Fr_t Commitment::open(const FrTensor& t, const G1TensorJacobian& com, const vect
     }
     return me_open(folded, *this, u_in.begin(), u_in.end(), proof);
 }
-Commitment::Pending Commitment::open_fold(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u, bool rows_commit) const {
+G1TensorJacobian Commitment::cross_commitments(const FrTensor& t, const G1TensorJacobian& com, int rounds) const {
+    if (rounds < 0 || rounds > 4) throw std::runtime_error("Commitment::cross_commitments - 0 to 4 rounds");
+    if (t.size % size != 0 || t.size / size != com.size) throw std::runtime_error("Commitment::cross_commitments - Incompatible dimensions");
+    if (rounds > 0 && (size & (size - 1))) throw std::runtime_error("Commitment::cross_commitments - the generator count has to be a power of 2");
+    const uint rows = com.size;
+    uint patterns = 1;
+    for (int q = 0; q < rounds; ++q) patterns += 2u << (2 * q);
+    G1TensorJacobian out(patterns * rows);
+    ZKC(zk_copy_strided(out.gpu_data, com.gpu_data, sizeof(G1Jacobian_t), rows, 1, 0, nullptr));
+    uint base = 1;
+    for (int q = 0; q < rounds; ++q) {
+        const uint half = 1u << q, L = 2 * half, cnt = size / L;
+        if (cnt == 0) throw std::runtime_error("Commitment::cross_commitments - more rounds than the generators have");
+        for (uint side = 0; side < 2; ++side) {
+            // the scalars of every a at once: [a][row][j] = t[row][L j + (side ? half : 0) + a]
+            FrTensor ws(half * rows * cnt);
+            for (uint a = 0; a < half; ++a)
+                ZKC(zk_copy_strided(ws.gpu_data + (size_t)a * rows * cnt, t.gpu_data, sizeof(Fr_t), (size_t)rows * cnt, L, (side ? half : 0) + a, nullptr));
+            for (uint b = 0; b < half; ++b) {
+                Commitment gs(cnt);         // g_(L j + (side ? 0 : half) + b)
+                ZKC(zk_copy_strided(gs.gpu_data, gpu_data, sizeof(G1Jacobian_t), cnt, L, (side ? 0 : half) + b, nullptr));
+                G1TensorJacobian x = gs.commit_int(ws);           // [a][row]
+                for (uint a = 0; a < half; ++a)
+                    ZKC(zk_copy_strided(out.gpu_data + (size_t)(base + side * half * half + a * half + b) * rows, x.gpu_data + (size_t)a * rows, sizeof(G1Jacobian_t), rows, 1, 0, nullptr));
+            }
+        }
+        base += 2 * half * half;
+    }
+    return out;
+}
+
+Commitment::Pending Commitment::open_fold(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u, bool rows_commit, const G1TensorJacobian* cross,
+                                          int cross_rounds) const {
     const uint k_out = ceilLog2(com.size);
     if (u.size() < k_out) throw std::runtime_error("Commitment::open - too few challenges");
     const vector<Fr_t> u_out(u.end() - k_out, u.end());
@@ -84,7 +116,12 @@ Commitment::Pending Commitment::open_fold(const FrTensor& t, const G1TensorJacob
     p.u_in.assign(u.begin(), u.end() - k_out);
     p.folded.reset(new FrTensor(u_out.empty() ? FrTensor(t) : t.partial_me(u_out, t.size / com.size)));
     if (p.folded->size != size) throw std::runtime_error("Commitment::me_open - Incompatible dimensions " + std::to_string(p.folded->size) + " " + std::to_string(size));
-    if (rows_commit) { p.row_com = &com; p.u_out = u_out; }
+    if (rows_commit) {
+        p.row_com = cross ? cross : &com;
+        p.cross_rounds = cross ? cross_rounds : 0;
+        p.n_rows = com.size;
+        p.u_out = u_out;
+    }
     return p;
 }
 void Commitment::open_start(Pending& p) const {
@@ -136,7 +173,11 @@ void Commitment::open_start_batch(const std::vector<std::pair<const Commitment*,
             for (int r = 0; r < b->rounds; ++r) memcpy(&uu[((size_t)k * b->rounds + r) * 8], q->u_in[r].val, 32);
         }
         bool with_rows = true;
-        for (size_t k = 0; k < group.size(); ++k) with_rows = with_rows && ops[group[k]].second->row_com != nullptr;
+        int cross_rounds = 64;
+        for (size_t k = 0; k < group.size(); ++k) {
+            with_rows = with_rows && ops[group[k]].second->row_com != nullptr;
+            cross_rounds = std::min(cross_rounds, ops[group[k]].second->cross_rounds);
+        }
         if (with_rows) {
             std::vector<const void*> rows;
             std::vector<uint32_t> nrows;
@@ -145,11 +186,11 @@ void Commitment::open_start_batch(const std::vector<std::pair<const Commitment*,
             for (size_t k = 0; k < group.size(); ++k) {
                 Pending* q = ops[group[k]].second;
                 rows.push_back(q->row_com->gpu_data);
-                nrows.push_back(q->row_com->size);
+                nrows.push_back(q->n_rows);
                 urows.push_back(q->u_out.empty() ? nullptr : q->u_out[0].val);
                 krows.push_back((int)q->u_out.size());
             }
-            ZKC(zk_g1_open_begin_batch_rows(&b->handle, b->count, sc.data(), pr.data(), uu.data(), b->rounds, rows.data(), nrows.data(), urows.data(), krows.data(), nullptr));
+            ZKC(zk_g1_open_begin_batch_rows(&b->handle, b->count, sc.data(), pr.data(), uu.data(), b->rounds, rows.data(), nrows.data(), urows.data(), krows.data(), cross_rounds, nullptr));
         } else
             ZKC(zk_g1_open_begin_batch(&b->handle, b->count, sc.data(), pr.data(), uu.data(), b->rounds, nullptr));
         for (size_t k = 0; k < group.size(); ++k) {
@@ -204,6 +245,25 @@ Fr_t Commitment::open_end(Pending& p, vector<G1Jacobian_t>& proof) {
 Fr_t Commitment::open(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u) const {
     vector<G1Jacobian_t> proof;
     return open(t, com, u, proof);
+}
+
+void prepare_weight_cross(Weight& w, int rounds) {
+    if (const char* e = getenv("ZKLLM_OPEN_CROSS_ROUNDS")) rounds = atoi(e);
+    int most = 0;
+    for (uint n = w.generator.size; n > 2048 && !(n & 1u); n >>= 1) ++most;       // halving rounds of an opening over these generators
+    rounds = std::max(0, std::min(std::min(rounds, most), 4));
+    if (rounds == 0 || (w.generator.size & (w.generator.size - 1))) { w.cross.reset(); w.cross_rounds = 0; return; }
+    const bool ragged = w.in_dim != (1u << ceilLog2(w.in_dim)) || w.out_dim != (1u << ceilLog2(w.out_dim));
+    try {
+        std::unique_ptr<FrTensor> local;
+        if (ragged && !w.padded) local.reset(new FrTensor(w.weight.pad({w.in_dim, w.out_dim})));
+        const FrTensor& t = !ragged ? w.weight : (w.padded ? *w.padded : *local);
+        w.cross = std::make_shared<const G1TensorJacobian>(w.generator.cross_commitments(t, w.com, rounds));
+        w.cross_rounds = rounds;
+    } catch (const std::exception&) {
+        w.cross.reset();
+        w.cross_rounds = 0;
+    }
 }
 
 Weight create_weight(string generator_filename, string weight_filename, string com_filename, uint in_dim, uint out_dim) {

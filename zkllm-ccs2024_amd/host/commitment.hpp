@@ -38,18 +38,28 @@ class Commitment : public G1TensorJacobian {
         vector<Fr_t> u_in;                  // between open_fold and open_start: the challenges of the G1 recursion
         const G1TensorJacobian* row_com = nullptr;      // open_fold(..., rows_commit = true): the tensor's row commitments and the
         vector<Fr_t> u_out;                             // challenges its rows were folded with (open_start_batch takes T of the first round from them)
+        uint n_rows = 0;                                // rows of the tensor (row_com holds them once per pattern)
+        int cross_rounds = 0;                           // row_com is cross_commitments(t, c, cross_rounds)
         struct Batch;                       // openings started as one job (open_start_batch) share its handle and results
         std::shared_ptr<Batch> batch;
         int batch_index = 0;
     };
     Pending open_begin(const FrTensor& t, const G1TensorJacobian& c, const vector<Fr_t>& u) const;
+    // Commitments of strided parts of t's rows under strided parts of these generators, in the layout
+    // zk_g1_open_begin_batch_rows takes ([pattern][row]; pattern 0 is c itself, then the cross patterns of the first
+    // `rounds` halving rounds of an opening): with them T, T0 and T1 of those rounds are sums over rows x patterns
+    // points.  Depends on the tensor and the generators alone -- made once per weight, like its commitment (seven times
+    // its work for three rounds).  t in the committed (padded) form with fixed-point entries; size a power of two.
+    G1TensorJacobian cross_commitments(const FrTensor& t, const G1TensorJacobian& c, int rounds) const;
     // open_begin in its two steps: open_fold reduces the rows to the vector that is opened (a pass over the whole tensor
     // on the caller's stream), open_start queues the G1 recursion.  Several openings started together fold first and
     // start afterwards: a fold queued behind another opening's G1 kernels waits for the registers they hold.
     // rows_commit: the caller states that c holds the commitments of t's rows under these generators (what create_weight
     // loads and verifyWeightClaim opens against; commitment.cu:137 evaluates them at u_out as well): a batched start may
     // then take the first round's T from them.  c must outlive the pending opening.
-    Pending open_fold(const FrTensor& t, const G1TensorJacobian& c, const vector<Fr_t>& u, bool rows_commit = false) const;
+    // cross (with rows_commit): cross_commitments(t, c, cross_rounds), used in c's place.
+    Pending open_fold(const FrTensor& t, const G1TensorJacobian& c, const vector<Fr_t>& u, bool rows_commit = false, const G1TensorJacobian* cross = nullptr,
+                      int cross_rounds = 0) const;
     void open_start(Pending& p) const;
     // open_start for several folded openings at once: those whose generators are prepared and agree in size and round
     // count run as one device job each group (zk_g1_open_begin_batch), the rest one by one
@@ -77,7 +87,15 @@ struct Weight {
     // (proof.cu:3-10 pads at every opening).  Set where the weight is loaded or made when a dimension is not a power of
     // two; verifyWeightClaim pads on the spot when it is needed and absent.
     std::shared_ptr<const FrTensor> padded;
+    // addition: generator.cross_commitments(committed form of weight, com, cross_rounds), made by prepare_weight_cross:
+    // the planned openings of a layer take T, T0 and T1 of the first cross_rounds halving rounds from them
+    std::shared_ptr<const G1TensorJacobian> cross;
+    int cross_rounds = 0;
 };
+// Makes w.cross for up to `rounds` rounds (fewer when the generators run out before: a round counts while more than 2048
+// generators are left; ZKLLM_OPEN_CROSS_ROUNDS overrides `rounds`, 0 = none).  A weight whose entries are not fixed-point
+// integers is left without (commit_int refuses them).
+void prepare_weight_cross(Weight& w, int rounds = 3);
 
 Weight create_weight(string generator_filename, string weight_filename, string com_filename, uint in_dim, uint out_dim);
 

@@ -504,7 +504,9 @@ void* zkp_layer_create(const u32* cu, const double* cf, const int32_t* norm1, co
         Commitment gen = Commitment::random(1u << ceilLog2(pp));
         G1TensorJacobian com = gen.commit_int(weight.pad({in_dim, out_dim}));
         gen.prepare_openings();
-        return Weight{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim};
+        Weight w{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim};
+        prepare_weight_cross(w);
+        return w;
     };
     // same order of generator draws as the oracle: norm1, q, k, v, o, norm2, up, gate, down
     Weight n1 = mk(norm1, 1, E, E), q = mk(wq, E, E, E << log_off_factor), k = mk(wk, E, E, E << log_off_factor), v = mk(wv, E, E, E << log_off_factor),
@@ -525,6 +527,7 @@ void zkp_layer_set_head_group(void* h, u32 g) { reinterpret_cast<LayerState*>(h)
 void zkp_layer_set_open_weights(void* h, int on) { reinterpret_cast<LayerState*>(h)->cfg.open_weights = on != 0; }
 // setup times of the last zkp_layer_create_random (ms): weights, generators, commitments, prepared generators
 void zkp_layer_setup_times(double* out4) { const LayerSetupTimes& t = layer_setup_times(); out4[0] = t.weights; out4[1] = t.generators; out4[2] = t.commitments; out4[3] = t.prepare; }
+double zkp_layer_setup_cross_ms() { return layer_setup_times().cross; }      // the cross commitments of the nine weights (prepare_weight_cross)
 // the nine commitments of the layer computed once more (ms); negative on error
 double zkp_layer_recommit_ms(void* h) {
     try { return layer_recommit_ms(reinterpret_cast<LayerState*>(h)->w); } catch (const std::exception& e) { g_err = e.what(); return -1.0; }

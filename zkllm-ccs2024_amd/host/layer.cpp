@@ -423,8 +423,13 @@ static Weight random_weight(std::mt19937_64& rng, uint in_dim, uint out_dim, uin
     const double t3 = now_ms();
     gen.prepare_openings();
     const double t4 = now_ms();
+    Weight w{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim, std::move(padded)};
+    prepare_weight_cross(w);
+    zk_check(zk_sync(nullptr), "zk_sync");
+    const double t5 = now_ms();
     g_setup_times.weights += t1 - t0; g_setup_times.generators += t2 - t1; g_setup_times.commitments += t3 - t2; g_setup_times.prepare += t4 - t3;
-    return Weight{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim, std::move(padded)};
+    g_setup_times.cross += t5 - t4;
+    return w;
 }
 double layer_recommit_ms(const LayerWeights& w) {
     const Weight* all[9] = {&w.input_norm, &w.q, &w.k, &w.v, &w.o, &w.post_norm, &w.up, &w.gate, &w.down};

@@ -86,7 +86,7 @@ FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor
 // how long make_random_layer_weights last spent on each part of the setup (ms, device idle at both ends of every part):
 // the random fixed-point weights (host generator + upload + padding), the generator sets, the nine commitments, the
 // generators' prepared form for openings
-struct LayerSetupTimes { double weights = 0, generators = 0, commitments = 0, prepare = 0; };
+struct LayerSetupTimes { double weights = 0, generators = 0, commitments = 0, prepare = 0, cross = 0; };      // cross: prepare_weight_cross
 const LayerSetupTimes& layer_setup_times();
 // commits the nine weights again (the results are dropped): the commitment cost of a layer, in ms
 double layer_recommit_ms(const LayerWeights& w);

@@ -37,7 +37,7 @@ DeferredOpenings::DeferredOpenings(OpeningPlan* pl) : prev(g_deferred), plan(pl)
             std::unique_ptr<FrTensor> local;
             // a Weight's com is the commitment of its (padded) rows: the batched start may use it for the first round's T
             static const bool t_from_rows = [] { const char* v = getenv("ZKLLM_OPEN_T_FROM_COM"); return !(v && v[0] == '0'); }();
-            a->op = e.w->generator.open_fold(padded_form(*e.w, local), e.w->com, a->u_cat, t_from_rows);
+            a->op = e.w->generator.open_fold(padded_form(*e.w, local), e.w->com, a->u_cat, t_from_rows, e.w->cross.get(), e.w->cross_rounds);
         }
         // the longest recursions first; openings of one size run as one job
         std::vector<Ahead*> order(ahead);
