@@ -182,6 +182,8 @@ def main():
     setup_s = time.perf_counter() - t0
     setup4 = np.zeros(4)
     pv.lib.zkp_layer_setup_times(setup4.ctypes.data_as(ctypes.POINTER(ctypes.c_double)))
+    pv.lib.zkp_layer_setup_cross_ms.restype = ctypes.c_double
+    setup_cross_ms = pv.lib.zkp_layer_setup_cross_ms()
     X = np.round(np.random.default_rng(11).normal(0, 1, (seq, 4096)) * 65536).astype(np.int32)
     hX = pv.from_i32(X)
     devnull = os.open(os.devnull, os.O_WRONLY)
@@ -203,8 +205,18 @@ def main():
         fold_ms, fold_launches, fold_mults, fold_pairs = read_fold_timer()
         lk_ms, lk_launches, lk_pairs, lk_bytes = read_lookup_timer()
         # the same layer without its nine openings (the G1 part of verifyWeightClaim switched off), and the nine commitments alone
-        noopen_s = commit_ms = None
+        noopen_s = commit_ms = nocross_s = None
         if not args.skip_extras:
+            # the layer with its openings summing over the generators in every round (no cross commitments of the weights)
+            pv.lib.zkp_openings_use_cross_commitments(c_int(0))
+            pv.layer_run(layer, hX)
+            pv.sync()
+            t1 = time.perf_counter()
+            for _ in range(2):
+                pv.layer_run(layer, hX)
+            pv.sync()
+            nocross_s = (time.perf_counter() - t1) / 2
+            pv.lib.zkp_openings_use_cross_commitments(c_int(1))
             pv.layer_set(layer, open_weights=False)
             pv.layer_run(layer, hX)
             pv.sync()
@@ -248,15 +260,24 @@ def main():
                    "device_pool_gib": round(pool_gib, 1),
                    "setup_s_untimed": round(setup_s, 3),
                    "setup_parts_s": {"random_weights_host_and_upload": round(setup4[0] / 1e3, 3), "generators": round(setup4[1] / 1e3, 3),
-                                     "commitments": round(setup4[2] / 1e3, 3), "generators_prepared_for_openings": round(setup4[3] / 1e3, 3)},
+                                     "commitments": round(setup4[2] / 1e3, 3), "generators_prepared_for_openings": round(setup4[3] / 1e3, 3),
+                                     "cross_commitments_of_the_weights": round(setup_cross_ms / 1e3, 3)},
+                   "setup_note": "all of it is made once per model and kept: the commitments are the public ones; the prepared generators (fixed-base tables of the "
+                                 "first two fold rounds) depend on the generators alone; the cross commitments (commitments of every 2nd / 4th / 8th column of a "
+                                 "weight's rows under every 2nd / 4th / 8th generator) depend on weights and generators alone and let the first three rounds of an "
+                                 "opening take T, T0, T1 from sums over rows x patterns points instead of bucket sums over all generators",
                    "parts_ms": {k: round(float(v), 1) for k, v in zip(["rmsnorm1", "qkv", "attention", "oproj", "rmsnorm2", "ffn", "total", "open_wait"], parts)},
                    "parts_note": "host-side block times; the openings run on the library's streams from the start of the layer, so the first blocks' "
                                  "figures include the time their kernels share the device with them"},
     }
     if noopen_s is not None:
         out["layer_without_openings_s"] = noopen_s
-        out["commitments_s"] = commit_ms / 1e3
-        out["layer_with_commitments_s"] = ms_per_step / 1e3 + commit_ms / 1e3
+        # what is made of the weights once, at commit time: the nine public commitments and their cross commitments
+        out["commitments_s"] = commit_ms / 1e3 + setup_cross_ms / 1e3
+        out["commitments_parts_s"] = {"row_commitments": commit_ms / 1e3, "cross_commitments": setup_cross_ms / 1e3}
+        out["layer_with_commitments_s"] = ms_per_step / 1e3 + commit_ms / 1e3 + setup_cross_ms / 1e3
+        out["layer_without_cross_commitments_s"] = nocross_s
+        out["layer_without_cross_commitments_with_row_commitments_s"] = nocross_s + commit_ms / 1e3
     # roofline of the kernel with the largest share of the layer's GPU time: the generator fold of the openings
     # (one endomorphism-split scalar multiplication per pair).  It is bound by 32-bit integer multiply-adds: an
     # Fp multiplication is 2*12^2+12 = 300 of them.  Durations are HIP events around every launch inside the timed

@@ -527,6 +527,7 @@ void zkp_layer_set_head_group(void* h, u32 g) { reinterpret_cast<LayerState*>(h)
 void zkp_layer_set_open_weights(void* h, int on) { reinterpret_cast<LayerState*>(h)->cfg.open_weights = on != 0; }
 // setup times of the last zkp_layer_create_random (ms): weights, generators, commitments, prepared generators
 void zkp_layer_setup_times(double* out4) { const LayerSetupTimes& t = layer_setup_times(); out4[0] = t.weights; out4[1] = t.generators; out4[2] = t.commitments; out4[3] = t.prepare; }
+void zkp_openings_use_cross_commitments(int on) { zk_openings_use_cross_commitments(on != 0); }
 double zkp_layer_setup_cross_ms() { return layer_setup_times().cross; }      // the cross commitments of the nine weights (prepare_weight_cross)
 // the nine commitments of the layer computed once more (ms); negative on error
 double zkp_layer_recommit_ms(void* h) {

@@ -19,6 +19,8 @@ struct DeferredOpenings::Ahead {
     vector<Fr_t> u_cat;
 };
 static thread_local DeferredOpenings* g_deferred = nullptr;
+static bool g_use_cross = true;
+void zk_openings_use_cross_commitments(bool on) { g_use_cross = on; }
 static const FrTensor& padded_form(const Weight& w, std::unique_ptr<FrTensor>& local);
 DeferredOpenings::DeferredOpenings() : prev(g_deferred) { g_deferred = this; }
 DeferredOpenings::DeferredOpenings(OpeningPlan* pl) : prev(g_deferred), plan(pl) {
@@ -37,7 +39,8 @@ DeferredOpenings::DeferredOpenings(OpeningPlan* pl) : prev(g_deferred), plan(pl)
             std::unique_ptr<FrTensor> local;
             // a Weight's com is the commitment of its (padded) rows: the batched start may use it for the first round's T
             static const bool t_from_rows = [] { const char* v = getenv("ZKLLM_OPEN_T_FROM_COM"); return !(v && v[0] == '0'); }();
-            a->op = e.w->generator.open_fold(padded_form(*e.w, local), e.w->com, a->u_cat, t_from_rows, e.w->cross.get(), e.w->cross_rounds);
+            const bool cross = g_use_cross && e.w->cross;
+            a->op = e.w->generator.open_fold(padded_form(*e.w, local), e.w->com, a->u_cat, t_from_rows, cross ? e.w->cross.get() : nullptr, cross ? e.w->cross_rounds : 0);
         }
         // the longest recursions first; openings of one size run as one job
         std::vector<Ahead*> order(ahead);

@@ -71,6 +71,9 @@ class DeferredOpenings {
     friend void verifyWeightClaim(const Weight& w, const Claim& c, WeightOpeningAhead& ahead);
 };
 
+// planned openings (DeferredOpenings with a learned plan) use a weight's cross commitments when it has them; off: they sum
+// over the generators in every round (measurements compare the two)
+void zk_openings_use_cross_commitments(bool on);
 vector<Fr_t> inner_product_sumcheck(const FrTensor& a, const FrTensor& b, vector<Fr_t> u);
 vector<Fr_t> hadamard_product_sumcheck(const FrTensor& a, const FrTensor& b, vector<Fr_t> u, vector<Fr_t> v);
 vector<Fr_t> binary_sumcheck(const FrTensor& a, vector<Fr_t> u, vector<Fr_t> v);
