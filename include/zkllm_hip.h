@@ -183,6 +183,12 @@ int zk_g1_open_end(void* handle, uint32_t* proof_host, uint32_t* final_scalar_ho
  * such generators; the handle must outlive every opening started with it and is released with
  * zk_g1_open_prepared_free. */
 int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stream);
+/* zk_g1_open_prepare with the choice of tables: 0 none, 1 / 2 those of the first / first two fold rounds (2 is what
+ * zk_g1_open_prepare makes), 3 the tables of a fold that takes three rounds at once (seven differences per eight
+ * generators; as large as the other two together, made in their place).  The three-round fold serves openings started with
+ * zk_g1_open_begin_batch_rows and cross_rounds >= 3, whose first three rounds read no folded generators; any other opening
+ * over such a handle folds by the walk.  Needs a power of two of at least 16384 generators, else 3 means 2. */
+int zk_g1_open_prepare_tables(void** prepared, const void* gens, size_t n, int tables, void* stream);
 int zk_g1_open_prepared_free(void* prepared);
 int zk_g1_open_begin_prepared(void** handle, const void* scalars, const void* prepared, const uint32_t* u, int rounds, void* stream);
 /* `count` (1..8) openings against prepared generator sets of ONE size with ONE round count as a single job: every kernel

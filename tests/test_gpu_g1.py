@@ -411,16 +411,18 @@ def test_open_batch_with_row_commitments_delivers_the_points_of_the_plain_openin
     hip.call("zk_g1_open_prepared_free", prep)
 
 
-def test_open_batch_with_cross_commitments_needs_no_sum_over_the_generators(pv):
-    """With the cross commitments of its first two rounds -- commitments of every 2nd / 4th column of the tensor's rows
-    under every 2nd / 4th generator, made here with commit_int on slices -- zk_g1_open_begin_batch_rows forms T, T0 and T1
-    of those rounds from rows x patterns points; 8192 generators are halved twice before the batched last rounds, so no
-    round sums over its generators.  Every point of the proof equals zk_g1_open's on the row-folded vector."""
+@pytest.mark.parametrize("n,R,tables", [(8192, 2, 2), (16384, 3, 3), (32768, 3, 3)])
+def test_open_batch_with_cross_commitments_needs_no_sum_over_the_generators(pv, n, R, tables):
+    """With the cross commitments of its first R rounds -- commitments of every 2nd / 4th / 8th column of the tensor's rows
+    under every 2nd / 4th / 8th generator, made here with commit_int on slices -- zk_g1_open_begin_batch_rows forms T, T0 and
+    T1 of those rounds from rows x patterns points: 8192 generators are halved twice before the batched last rounds, so no
+    round sums over its generators.  With three rounds of them and the tables of zk_g1_open_prepare_tables(.., 3) the three
+    rounds are one fold (16384 generators: nothing but that fold and the batched last rounds; 32768: one ordinary round
+    behind it).  Every point of the proof equals zk_g1_open's on the row-folded vector."""
     import ctypes
     from gpuhelp import Hip, c_void_p, c_size_t, c_int
     hip = Hip()
     pv.lib.zkp_g1_devptr.restype = ctypes.c_void_p
-    n, R = 8192, 2
     k = (n - 1).bit_length()
     npts = 3 * k + 1
     pv.seed(78)
@@ -428,7 +430,7 @@ def test_open_batch_with_cross_commitments_needs_no_sum_over_the_generators(pv):
     gens_host = gens.host()
     dG = pv.lib.zkp_g1_devptr(c_void_p(gens.h))
     prep = c_void_p()
-    hip.call("zk_g1_open_prepare", ctypes.byref(prep), c_void_p(dG), c_size_t(n), None)
+    hip.call("zk_g1_open_prepare_tables", ctypes.byref(prep), c_void_p(dG), c_size_t(n), c_int(tables), None)
     rng = np.random.default_rng(6)
     keep, folded, cross, urows, us = [], [], [], [], []
     exp_p = np.zeros((2, npts, 36), np.uint32)
@@ -446,7 +448,7 @@ def test_open_batch_with_cross_commitments_needs_no_sum_over_the_generators(pv):
                         sub_g = pv.g1_from_host(np.ascontiguousarray(gens_host[g_off::L]))
                         sub_w = pv.from_i32(np.ascontiguousarray(Wi[:, s_off::L]).ravel())
                         pats.append(pv.commit_int(sub_g, sub_w).host())
-        assert len(pats) == 1 + 2 + 8 and all(x.shape == (nrows, 36) for x in pats)
+        assert len(pats) == 1 + 2 * (4 ** R - 1) // 3 and all(x.shape == (nrows, 36) for x in pats)
         cross.append(hip.upload(np.ascontiguousarray(np.concatenate(pats))))
         kr = (nrows - 1).bit_length()
         ur = mt_random_vec(np.random.RandomState(45 + i), kr)
@@ -456,7 +458,7 @@ def test_open_batch_with_cross_commitments_needs_no_sum_over_the_generators(pv):
         hip.call("zk_g1_open", exp_p[i], exp_v[i], c_void_p(f.devptr), c_void_p(dG), c_size_t(n), u, c_int(k), None)
         keep += [W, f]
         folded.append(f); urows.append(np.ascontiguousarray(ur, dtype=np.uint32)); us.append(u)
-    for cr in (2, 1):
+    for cr in (R, 1):
         h = c_void_p()
         sc = (c_void_p * 2)(*[c_void_p(f.devptr) for f in folded])
         pp = (c_void_p * 2)(prep, prep)

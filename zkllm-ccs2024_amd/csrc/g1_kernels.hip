@@ -984,6 +984,74 @@ k_open_fold_comb(const CombBatch cb, size_t old_size, size_t new_size) {
         new_gens[g] = o;
     }
 }
+// ---- three rounds in one: the generators after the third fold straight from the prepared ones -------------------------------------
+// When T0 and T1 of the first three rounds come from cross commitments of the opened tensor, nothing reads the generators of
+// the second and third round but the next fold.  With c_b = prod_{k<3} (bit_k(b) ? 1 - u_k : u_k) (u_0 .. u_2 the three
+// challenges; the c_b sum to one) the generators after three folds are
+//     g^(3)_m = sum_{b<8} c_b g_(8m+b) = g_(8m+7) + sum_{b<7} [c_b] P_b,m,     P_b,m = g_(8m+b) - g_(8m+7),
+// seven fixed-base combs that share their COMB_W doublings: at most 14 COMB_W additions per eight generators, where the
+// three rounds one after the other take a comb per pair, a double comb per four and a 129-step walk per eight.
+// Tables: [b][entry][m], built like the first round's.  The scalars are folded three times on the way.
+static constexpr int JUMP_ROUNDS = 3, JUMP_SPAN = 1 << JUMP_ROUNDS, JUMP_TABS = JUMP_SPAN - 1;
+struct JumpItem { Fr* ns; A29* ng; const Fr* s; const A29* g; const A29* tab; Fr u_mont[JUMP_ROUNDS]; CombK ck[JUMP_TABS]; };
+struct JumpBatch { JumpItem it[OB_MAX]; };
+__global__ void __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+k_open_fold_jump(const JumpBatch jb, size_t new_size) {
+    __shared__ int32_t inv_lds[14][2 * GT];
+    const JumpItem& it = jb.it[blockIdx.y];
+    const size_t g = (size_t)blockIdx.x * GT + threadIdx.x;
+    const bool live = g < new_size;
+    A29 a1;
+    a1.x = a1.y = fq29_zero();
+    if (live) {
+        a1 = it.g[JUMP_SPAN * g + JUMP_SPAN - 1];
+        // the scalars, level by level as the rounds would fold them
+        Fr v[JUMP_SPAN];
+#pragma unroll
+        for (int i = 0; i < JUMP_SPAN; ++i) v[i] = it.s[JUMP_SPAN * g + i];
+#pragma unroll
+        for (int k = 0; k < JUMP_ROUNDS; ++k)
+#pragma unroll
+            for (int i = 0; i < (JUMP_SPAN >> (k + 1)); ++i) v[i] = add(v[2 * i], mont_mul(it.u_mont[k], sub(v[2 * i + 1], v[2 * i])));
+        it.ns[g] = v[0];
+    }
+    const bool inf1 = !live || a29_is_inf(a1);
+    J29 w = j29_infinity();
+    if (live) {
+        const Fq29 beta = fq29_from_fp(glv_beta());
+        for (int b = COMB_W - 1; b >= 0; --b) {
+            w = j29_double(w);
+            for (int ti = 0; ti < JUMP_TABS; ++ti) {
+                const A29* __restrict__ tb = it.tab + (size_t)ti * COMB_N * new_size;
+                const uint32_t m1 = it.ck[ti].m1[b], m2 = it.ck[ti].m2[b];          // the same for every lane
+                if (m1) {
+                    const A29 t = tb[(size_t)(m1 - 1) * new_size + g];
+                    if (!a29_is_inf(t)) w = j29_add_mixed(w, t);
+                }
+                if (m2) {
+                    A29 t = tb[(size_t)(m2 - 1) * new_size + g];
+                    if (!a29_is_inf(t)) {
+                        t.x = fq29_mul(t.x, beta);
+                        w = j29_add_mixed(w, t);
+                    }
+                }
+            }
+        }
+        if (!inf1) w = j29_add_mixed(w, a1);
+    }
+    const bool has_z = live && !w.inf;
+    const Fq29 zi = block_inv64_29(has_z ? w.z : fq29_one(), inv_lds);
+    if (live) {
+        A29 o;
+        o.x = o.y = fq29_zero();
+        if (has_z) {
+            const Fq29 zi2 = fq29_sqr(zi);
+            o.x = fq29_canon(fq29_mul(w.x, zi2));
+            o.y = fq29_canon(fq29_mul(fq29_mul(w.y, zi2), zi));
+        }
+        it.ng[g] = o;
+    }
+}
 // the pairs k_open_fold29 left out, by the general Jacobian route in 32-bit limbs (one lane per pair, an inversion each)
 __device__ __forceinline__ G1Affine a29_to_affine(const A29& p) {
     G1Affine r;
@@ -1046,6 +1114,15 @@ __global__ void __launch_bounds__(GT) k_open_pair_diff(G1Jac* __restrict__ out, 
         if (!aff_is_inf(b)) p = g1_add_mixed(p, b);
     }
     out[j] = p;
+}
+// out[m] = A[m * span + b] - A[m * span + span - 1], m < n_out (the points of k_open_fold_jump's tables)
+__global__ void __launch_bounds__(GT) k_open_span_diff(G1Jac* __restrict__ out, const G1Affine* __restrict__ A, uint32_t span, uint32_t b, size_t n_out) {
+    const size_t m = (size_t)blockIdx.x * GT + threadIdx.x;
+    if (m >= n_out) return;
+    G1Jac p = aff_to_jac(A[m * span + b]);
+    const G1Affine last = g1_neg(A[m * span + span - 1]);
+    if (!aff_is_inf(last)) p = g1_add_mixed(p, last);
+    out[m] = p;
 }
 struct PairBatch { Fr* ps[OB_MAX]; const Fr* s[OB_MAX]; };
 __global__ void __launch_bounds__(256) k_open_pair_scalars(const PairBatch pb, size_t old_size, size_t half_up) {
@@ -1725,7 +1802,8 @@ struct OpenJob {
 // One opening of the batch: its scalars, its challenges (rounds x 8 limbs) and its generators -- Jacobian, or null when
 // `prep` (their prepared form, open_prep_build) is given
 struct OpenItem { const void* scalars; const void* gens; const A29* prep; const uint32_t* u; const A29* comb = nullptr; const A29* comb2 = nullptr;
-                  const void* rows = nullptr; uint32_t nrows = 0; const uint32_t* u_rows = nullptr; int k_rows = 0; int cross_rounds = 0; };
+                  const void* rows = nullptr; uint32_t nrows = 0; const uint32_t* u_rows = nullptr; int k_rows = 0; int cross_rounds = 0;
+                  const A29* comb3 = nullptr; };
 // rows (optional): commitments of the opened tensor's rows, [pattern][row] as k_open_cross_part takes them -- the row
 // commitments alone (cross_rounds = 0) or with the cross patterns of the first cross_rounds rounds
 static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, int rounds, hipStream_t st, hipStream_t aux) {
@@ -1822,7 +1900,56 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
     size_t size = n;
     int halving_rounds = rounds;
     bool tail_done = false;
-    for (int r = 0; r < rounds; ++r) {
+    int r_first = 0;
+    // three rounds as one fold: every opening brings the jump tables and cross commitments for those rounds, and all
+    // three are halving rounds
+    {
+        bool jump = with_rows && cross_r >= JUMP_ROUNDS && rounds_from_rows >= JUMP_ROUNDS && rounds >= JUMP_ROUNDS && !(n & (n - 1));
+        for (int i = 0; i < count; ++i) jump = jump && items[i].comb3 != nullptr;
+        if (jump) {
+            const size_t ns = n >> JUMP_ROUNDS;
+            Scratch& s2 = job.arena.add(sizeof(Fr) * ns * count);
+            Scratch& g2 = job.arena.add(sizeof(A29) * ns * count);
+            if (s2.rc) return s2.rc;
+            if (g2.rc) return g2.rc;
+            JumpBatch jb;
+            double fp_mults = 0;
+            const Fr one = big_one_mont<8>();
+            for (int i = 0; i < OB_MAX; ++i) {
+                const int k = i < count ? i : 0;
+                JumpItem& f = jb.it[i];
+                f.ns = s2.as<Fr>() + ns * k; f.ng = g2.as<A29>() + ns * k; f.s = cs[k]; f.g = cg[k]; f.tab = items[k].comb3;
+                Fr um[JUMP_ROUNDS];
+                for (int q = 0; q < JUMP_ROUNDS; ++q) um[q] = f.u_mont[q] = to_mont(load_fr(items[k].u + 8 * q));
+                for (int b = 0; b < JUMP_TABS; ++b) {
+                    Fr c = one;           // c_b = prod_q (bit_q(b) ? 1 - u_q : u_q)
+                    for (int q = 0; q < JUMP_ROUNDS; ++q) c = mont_mul(c, ((b >> q) & 1) ? sub(one, um[q]) : um[q]);
+                    f.ck[b] = comb_of(glv_split(from_mont(c)));
+                    if (i < count) fp_mults += (comb_fp_mults_per_pair(f.ck[b]) - 7.0 * COMB_W - 19.0) * (double)ns;
+                }
+                if (i < count) fp_mults += (7.0 * COMB_W + 19.0) * (double)ns;
+            }
+            hipEvent_t t0 = nullptr, t1 = nullptr;
+            if (g_fold_timer.on) {
+                ZK_HIP(hipEventCreate(&t0));
+                ZK_HIP(hipEventCreate(&t1));
+                ZK_HIP(hipEventRecord(t0, st));
+            }
+            hipLaunchKernelGGL(k_open_fold_jump, dim3(cdiv(ns, GT), count), dim3(GT), 0, st, jb, ns);
+            ZK_LAUNCH_CHECK();
+            if (g_fold_timer.on) {
+                ZK_HIP(hipEventRecord(t1, st));
+                std::lock_guard<std::mutex> lk(g_fold_timer.mu);
+                g_fold_timer.ev.emplace_back(t0, t1);
+                g_fold_timer.fp_mults += fp_mults;
+                g_fold_timer.pairs += ns * (size_t)count * (JUMP_SPAN - 1);       // pairs the three rounds fold: 4 + 2 + 1 per result
+            }
+            for (int i = 0; i < count; ++i) { cs[i] = s2.as<Fr>() + ns * i; cg[i] = g2.as<A29>() + ns * i; }
+            size = ns;
+            r_first = JUMP_ROUNDS;
+        }
+    }
+    for (int r = r_first; r < rounds; ++r) {
         if (size <= (size_t)TAIL_N && rounds - r <= TAIL_LEVELS) {
             int rc = open_tail_launch(cs, cg, count, size, rounds - r, r, rounds, pts.as<G1Jac>(), U_dev, job.pin, (char*)jdev.p + JOB_U_BYTES, job.arena, st);
             if (rc) return rc;
@@ -1922,8 +2049,14 @@ int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_
 // Generators prepared once for any number of openings against them: their affine 29-bit-limb form and the pair sums of
 // the first round (weight-independent; 1.5 n points of 112 bytes).  The handle is freed with zk_g1_open_prepared_free
 // once no opening that uses it is pending.
-struct OpenPrepared { void* a29 = nullptr; size_t n = 0; void* comb = nullptr; void* comb2 = nullptr; };
-int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stv) {
+struct OpenPrepared { void* a29 = nullptr; size_t n = 0; void* comb = nullptr; void* comb2 = nullptr; void* comb3 = nullptr; };      // comb3: k_open_fold_jump's tables (instead of the other two)
+static int open_prepare_impl(void** prepared, const void* gens, size_t n, int table_mode, void* stv);
+int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stv) { return open_prepare_impl(prepared, gens, n, 2, stv); }
+int zk_g1_open_prepare_tables(void** prepared, const void* gens, size_t n, int tables, void* stv) {
+    ZK_ARG(tables >= 0 && tables <= 3, "zk_g1_open_prepare_tables: tables 0 to 3");
+    return open_prepare_impl(prepared, gens, n, tables, stv);
+}
+static int open_prepare_impl(void** prepared, const void* gens, size_t n, int table_mode, void* stv) {
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(prepared != nullptr && n >= 1, "zk_g1_open_prepare: null handle or no generators");
     std::unique_ptr<OpenPrepared> pr(new OpenPrepared);
@@ -1941,8 +2074,49 @@ int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stv) {
         // The tables only make the folds cheaper: ZKLLM_OPEN_TABLES = 0 or 1 keeps none or the first round's alone (28 KB
         // per generator pair and round), and when the device has no room for them or for their construction the handle
         // is made without them -- those rounds then walk (k_open_fold29), the results are the same.
-        static const int table_rounds = [] { const char* e = getenv("ZKLLM_OPEN_TABLES"); return e ? atoi(e) : 2; }();
-        if (rc == 0 && n > (size_t)TAIL_N && table_rounds >= 1) {
+        static const int env_rounds = [] { const char* e = getenv("ZKLLM_OPEN_TABLES"); return e ? atoi(e) : -1; }();
+        const int table_rounds = env_rounds >= 0 ? env_rounds : table_mode;
+        // mode 3: the seven tables of k_open_fold_jump in place of those two (as large as both together); only for a power of
+        // two of generators that leaves more than the batched last rounds take after three folds
+        const bool jump = table_rounds >= 3 && !(n & (n - 1)) && (n >> JUMP_ROUNDS) >= (size_t)TAIL_N;
+        if (rc == 0 && jump) {
+            const size_t no = n >> JUMP_ROUNDS, ne = no * COMB_N * JUMP_TABS;
+            int trc = pool_alloc(&pr->comb3, sizeof(A29) * ne, st);
+            Scratch& aff = arena.add(sizeof(G1Affine) * n);
+            Scratch& tj = arena.add(sizeof(G1Jac) * ne);
+            Scratch& ta = arena.add(sizeof(G1Affine) * ne);
+            Scratch& tmp = arena.add(sizeof(G1Jac) * no);
+            if (trc == 0) trc = aff.rc ? aff.rc : (tj.rc ? tj.rc : (ta.rc ? ta.rc : tmp.rc));
+            if (trc) {
+                if (pr->comb3) (void)pool_free(pr->comb3, st, true);
+                pr->comb3 = nullptr;
+            } else {
+                static_assert(COMB_W % 2 == 0, "the doublings alternate between two buffers and must end in the table");
+                hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(n, CH), GT)), dim3(GT), 0, st, aff.p, (const G1Jac*)gens, n);
+                for (int b = 0; b < JUMP_TABS; ++b) {
+                    G1Jac* T = tj.as<G1Jac>() + (size_t)b * COMB_N * no;
+                    auto entry = [&](int m) { return T + (size_t)(m - 1) * no; };
+                    hipLaunchKernelGGL(k_open_span_diff, dim3(cdiv(no, GT)), dim3(GT), 0, st, T, aff.as<G1Affine>(), (uint32_t)JUMP_SPAN, (uint32_t)b, no);
+                    for (int t = 1; t < COMB_A; ++t) {
+                        const G1Jac* src = entry(1 << (t - 1));
+                        for (int k = 0; k < COMB_W; ++k) {          // no launch writes what it reads
+                            G1Jac* dst = (k & 1) ? entry(1 << t) : tmp.as<G1Jac>();
+                            hipLaunchKernelGGL(k_g1_add, dim3(cdiv(no, GT)), dim3(GT), 0, st, dst, src, src, no, no, 0);
+                            src = dst;
+                        }
+                    }
+                    for (int m = 3; m <= COMB_N; ++m) {
+                        const int prev = m & (m - 1);
+                        if (!prev) continue;
+                        hipLaunchKernelGGL(k_g1_add, dim3(cdiv(no, GT)), dim3(GT), 0, st, entry(m), entry(prev), entry(m ^ prev), no, no, 0);
+                    }
+                }
+                hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(ne, CH), GT)), dim3(GT), 0, st, ta.p, tj.as<G1Jac>(), ne);
+                hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(ne, 256)), dim3(256), 0, st, (A29*)pr->comb3, ta.as<G1Affine>(), ne);
+                if (hipGetLastError() != hipSuccess) rc = hip_fail(hipErrorLaunchFailure, "jump table build", __FILE__, __LINE__);
+            }
+        }
+        if (rc == 0 && n > (size_t)TAIL_N && table_rounds >= 1 && !pr->comb3) {
             const size_t np = (n + 1) / 2, ne = np * COMB_N;
             const size_t nq = (np + 1) / 2, ne2 = nq * COMB_N;        // second round: two tables over the pairs of pairs
             bool second = np > (size_t)TAIL_N && table_rounds >= 2;   // that round is a fold too
@@ -2006,6 +2180,7 @@ int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stv) {
         pool_free(pr->a29, st, true);
         if (pr->comb) pool_free(pr->comb, st, true);
         if (pr->comb2) pool_free(pr->comb2, st, true);
+        if (pr->comb3) pool_free(pr->comb3, st, true);
         return rc;
     }
     *prepared = pr.release();
@@ -2017,13 +2192,15 @@ int zk_g1_open_prepared_free(void* prepared) {
     int rc = pool_free(pr->a29, nullptr);
     if (pr->comb) (void)pool_free(pr->comb, nullptr);
     if (pr->comb2) (void)pool_free(pr->comb2, nullptr);
+    if (pr->comb3) (void)pool_free(pr->comb3, nullptr);
     delete pr;
     return rc;
 }
 int zk_g1_open_begin_prepared(void** handle, const void* scalars, const void* prepared, const uint32_t* u, int rounds, void* stv) {
     ZK_ARG(prepared != nullptr, "zk_g1_open_begin_prepared: null generators");
     const OpenPrepared* pr = (const OpenPrepared*)prepared;
-    const OpenItem item{scalars, nullptr, (const A29*)pr->a29, u, (const A29*)pr->comb, (const A29*)pr->comb2};
+    OpenItem item{scalars, nullptr, (const A29*)pr->a29, u, (const A29*)pr->comb, (const A29*)pr->comb2};
+    item.comb3 = (const A29*)pr->comb3;
     return open_begin_impl(handle, &item, 1, pr->n, rounds, stv);
 }
 // `count` (1 to 8) openings against prepared generator sets of one size and with one round count, as ONE job: every
@@ -2061,7 +2238,8 @@ int zk_g1_open_begin_batch_rows(void** handle, int count, const void* const* sca
         const OpenPrepared* pr = (const OpenPrepared*)prepared[i];
         if (i == 0) n = pr->n;
         ZK_ARG(pr->n == n, "zk_g1_open_begin_batch_rows: the generator sets differ in size");
-        items[i] = OpenItem{scalars[i], nullptr, (const A29*)pr->a29, u + (size_t)i * rounds * 8, (const A29*)pr->comb, (const A29*)pr->comb2, rows[i], nrows[i], u_rows[i], k_rows[i], cross_rounds};
+        items[i] = OpenItem{scalars[i], nullptr, (const A29*)pr->a29, u + (size_t)i * rounds * 8, (const A29*)pr->comb, (const A29*)pr->comb2, rows[i], nrows[i], u_rows[i], k_rows[i], cross_rounds,
+                            (const A29*)pr->comb3};
     }
     return open_begin_impl(handle, items, count, n, rounds, stv);
 }

@@ -203,10 +203,10 @@ void Commitment::open_start_batch(const std::vector<std::pair<const Commitment*,
         }
     }
 }
-void Commitment::prepare_openings() const {
+void Commitment::prepare_openings(int tables) const {
     if (prepared || size == 0) return;
     void* h = nullptr;
-    ZKC(zk_g1_open_prepare(&h, gpu_data, size, nullptr));
+    ZKC(zk_g1_open_prepare_tables(&h, gpu_data, size, tables, nullptr));
     prepared = std::shared_ptr<void>(h, [](void* q) { (void)zk_g1_open_prepared_free(q); });
 }
 Commitment::Pending Commitment::open_begin(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u) const {

@@ -69,7 +69,10 @@ class Commitment : public G1TensorJacobian {
     // The generators' form for openings (zk_g1_open_prepare), made once and kept with this object: openings started
     // afterwards skip the normalisation and conversion of the generators.  Anything that changes the points must not
     // be applied afterwards (the prepared form would no longer match); copies share it.
-    void prepare_openings() const;
+    // tables (zk_g1_open_prepare_tables): 0 none, 1 / 2 fixed-base tables of the first / first two fold rounds, 3 the tables
+    // that fold three rounds at once -- for openings that bring cross commitments of three rounds (prepare_weight_cross);
+    // without them such generators fold by the walk
+    void prepare_openings(int tables = 2) const;
     bool openings_prepared() const { return (bool)prepared; }
 
     static Commitment random(uint size);

@@ -503,9 +503,9 @@ void* zkp_layer_create(const u32* cu, const double* cf, const int32_t* norm1, co
         FrTensor weight(in_dim * out_dim, (const int*)p);
         Commitment gen = Commitment::random(1u << ceilLog2(pp));
         G1TensorJacobian com = gen.commit_int(weight.pad({in_dim, out_dim}));
-        gen.prepare_openings();
         Weight w{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim};
         prepare_weight_cross(w);
+        w.generator.prepare_openings(w.cross_rounds >= 3 ? 3 : 2);
         return w;
     };
     // same order of generator draws as the oracle: norm1, q, k, v, o, norm2, up, gate, down

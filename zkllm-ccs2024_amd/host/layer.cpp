@@ -421,14 +421,15 @@ static Weight random_weight(std::mt19937_64& rng, uint in_dim, uint out_dim, uin
     const double t2 = now_ms();
     G1TensorJacobian com = gen.commit_int(ragged ? *padded : weight);
     const double t3 = now_ms();
-    gen.prepare_openings();
-    const double t4 = now_ms();
     Weight w{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim, std::move(padded)};
     prepare_weight_cross(w);
     zk_check(zk_sync(nullptr), "zk_sync");
+    const double t4 = now_ms();
+    w.generator.prepare_openings(w.cross_rounds >= 3 ? 3 : 2);        // with three rounds of cross commitments the openings fold three rounds at once
+    zk_check(zk_sync(nullptr), "zk_sync");
     const double t5 = now_ms();
-    g_setup_times.weights += t1 - t0; g_setup_times.generators += t2 - t1; g_setup_times.commitments += t3 - t2; g_setup_times.prepare += t4 - t3;
-    g_setup_times.cross += t5 - t4;
+    g_setup_times.weights += t1 - t0; g_setup_times.generators += t2 - t1; g_setup_times.commitments += t3 - t2; g_setup_times.cross += t4 - t3;
+    g_setup_times.prepare += t5 - t4;
     return w;
 }
 double layer_recommit_ms(const LayerWeights& w) {
