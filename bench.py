@@ -97,6 +97,26 @@ def main():
             hip.call("zk_g1_open_end", h, pts, fin)
         return run
 
+    def jump_opening(n_big, gens_big, scalars):
+        """one opening whose first three rounds are one fold (k_open_fold_jump): generators prepared with the three-round tables,
+        started through zk_g1_open_begin_batch_rows.  The points that stand in for the cross commitments are infinities: they only
+        feed the sums T, T0, T1 of those rounds, which are not what is timed here; the folds do not read them."""
+        gp = pv.lib.zkp_g1_devptr(c_void_p(gens_big.h))
+        prep = c_void_p()
+        hip.call("zk_g1_open_prepare_tables", ctypes.byref(prep), c_void_p(gp), c_size_t(n_big), c_int(3), None)
+        k = (n_big - 1).bit_length()
+        uk = mt_random_vec(np.random.RandomState(10), k)
+        pts, fin = np.zeros((3 * k + 1, 36), np.uint32), np.zeros(8, np.uint32)
+        rows = hip.upload(np.zeros((43, 36), np.uint32))
+        sc, pp, rr = (c_void_p * 1)(c_void_p(scalars)), (c_void_p * 1)(prep), (c_void_p * 1)(c_void_p(rows))
+        nr, ur, kr = np.array([1], np.uint32), (c_void_p * 1)(c_void_p(None)), np.array([0], np.int32)
+
+        def run():
+            h = c_void_p()
+            hip.call("zk_g1_open_begin_batch_rows", ctypes.byref(h), c_int(1), sc, pp, uk, c_int(k), rr, nr, ur, kr, c_int(3), None)
+            hip.call("zk_g1_open_end_batch", h, pts, fin)
+        return run
+
     def lookup_probe(logD=27, logN=20):
         """one mapping-table lookup proof (tLookupRangeMapping::prove) over 2^logD uniformly spread queries into 2^logN entries"""
         D, N = 1 << logD, 1 << logN
@@ -117,6 +137,9 @@ def main():
         # 262144 and 131072 pairs, then k_open_fold29 on 65536, 32768, ... pairs
         prep_open = prepared_opening(n_big, gens_big, bufs[0])
         prep_open()
+        # and one whose first three rounds are one fold (k_open_fold_jump on 65536 results, then k_open_fold29 on 32768, ... pairs)
+        jump_open = jump_opening(n_big, gens_big, bufs[0])
+        jump_open()
         n = 1 << 24
         dA, dB, dO = hip.malloc(32 * n), hip.malloc(32 * n), hip.malloc(32 * n)
         hip.call("zk_fr_add", c_void_p(dO), c_void_p(dA), c_void_p(dB), c_size_t(n), None)
@@ -207,16 +230,6 @@ def main():
         # the same layer without its nine openings (the G1 part of verifyWeightClaim switched off), and the nine commitments alone
         noopen_s = commit_ms = nocross_s = None
         if not args.skip_extras:
-            # the layer with its openings summing over the generators in every round (no cross commitments of the weights)
-            pv.lib.zkp_openings_use_cross_commitments(c_int(0))
-            pv.layer_run(layer, hX)
-            pv.sync()
-            t1 = time.perf_counter()
-            for _ in range(2):
-                pv.layer_run(layer, hX)
-            pv.sync()
-            nocross_s = (time.perf_counter() - t1) / 2
-            pv.lib.zkp_openings_use_cross_commitments(c_int(1))
             pv.layer_set(layer, open_weights=False)
             pv.layer_run(layer, hX)
             pv.sync()
@@ -238,6 +251,20 @@ def main():
     pool_gib = (live_b.value + cached_b.value) / 2 ** 30      # the allocator keeps what it once needed: live + cached = the layer's peak
     pv.layer_free(layer)
     lib.zk_pool_trim()
+    # The layer with its openings summing over the generators in every round: no cross commitments of the weights, and the
+    # generators prepared with the tables of the first two rounds (the three-round fold needs the cross commitments).  Another
+    # set of prepared generators does not fit beside this one, so a child process measures it, now that this one's memory has gone back.
+    if not args.skip_extras:
+        import subprocess
+        env = dict(os.environ, ZKLLM_OPEN_CROSS_ROUNDS="0")
+        try:
+            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--skip-cpu", "--skip-extras", "--steps", "2", "--warmup", "1", "--seq", str(args.seq),
+                                "--head-group", str(args.head_group)], env=env, capture_output=True, text=True, timeout=300)
+            for line in r.stdout.splitlines():
+                if line.startswith("{"):
+                    nocross_s = json.loads(line)["value"]
+        except Exception:
+            nocross_s = None
 
     out = {
         "metric": "layer prove time (s), 7B shape seq 2048; G1 MSM points/s; Fr mul/s",
@@ -277,13 +304,13 @@ def main():
         out["commitments_parts_s"] = {"row_commitments": commit_ms / 1e3, "cross_commitments": setup_cross_ms / 1e3}
         out["layer_with_commitments_s"] = ms_per_step / 1e3 + commit_ms / 1e3 + setup_cross_ms / 1e3
         out["layer_without_cross_commitments_s"] = nocross_s
-        out["layer_without_cross_commitments_with_row_commitments_s"] = nocross_s + commit_ms / 1e3
+        out["layer_without_cross_commitments_with_row_commitments_s"] = None if nocross_s is None else nocross_s + commit_ms / 1e3
     # roofline of the kernel with the largest share of the layer's GPU time: the generator fold of the openings
     # (one endomorphism-split scalar multiplication per pair).  It is bound by 32-bit integer multiply-adds: an
     # Fp multiplication is 2*12^2+12 = 300 of them.  Durations are HIP events around every launch inside the timed
     # region above, on the launch stream.
     fold_tops = fold_mults * MAD_PER_FP_MUL / (fold_ms * 1e-3) / 1e12 if fold_ms > 0 else 0.0
-    out["roofline"] = {"kernel": "k_open_fold29 and, in an opening's first two rounds over prepared generators, k_open_fold_comb<1> / <2> (g' = g1 + [u](g0 - g1) per generator pair, 128-bit split scalars; "
+    out["roofline"] = {"kernel": "k_open_fold29, k_open_fold_comb<1> / <2> (first two rounds over prepared generators) and k_open_fold_jump (first three rounds at once, openings with cross commitments): g' = g1 + [u](g0 - g1) per generator pair, 128-bit split scalars, "
                                  "one launch per round for all openings of a size)",
                        "bound": "valu-int", "achieved": fold_tops, "peak": VALU_PEAK_TOPS, "unit": "T MAD32/s", "frac": fold_tops / VALU_PEAK_TOPS,
                        "traffic": None, "algorithmic_bytes_per_launch": FOLD_ALGO_BYTES_PER_PAIR * fold_pairs / max(1, fold_launches),
