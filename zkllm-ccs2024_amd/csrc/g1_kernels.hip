@@ -293,7 +293,6 @@ static constexpr int OB_SUMS = 3 * OB_MAX;
 template <int NMAX> struct MsmDescs { MsmDesc d[NMAX]; };
 static constexpr int TAIL_N = 2048;        // generators at which the remaining rounds are computed in one batch (work grows with it, latency shrinks)
 static constexpr int TAIL_LEVELS = 20;     // most rounds the batch takes
-static constexpr int TAIL_SUMS = 3 * TAIL_LEVELS + 1;
 struct GlvK { uint32_t k1[4], k2[4]; };
 
 __device__ __forceinline__ bool aff_is_inf(const G1Affine& p) { return is_zero(p.x) && is_zero(p.y); }   // normalised infinity: all-zero limbs
@@ -414,7 +413,7 @@ template <int NT = MT> __device__ __forceinline__ G1Jac msm_block_sum(uint32_t* 
 }
 
 // One segment's share of sum over elements of digit_w(s) * base: the segment's MT raw buckets,
-// partial[((sum * MW + w) * nseg + seg) * MT + b] for bucket magnitude b + 1 (k_msm_bucket_fold / k_msm_buckets reduce them).
+// partial[((sum * MW + w) * nseg + seg) * MT + b] for bucket magnitude b + 1 (k_msm_bucket_fold / k_msm_point reduce them).
 // One wave per workgroup.  Per chunk of MSEG elements:
 //  1. the bucket sizes are counted (one LDS atomic per element) and the elements are sorted by bucket into one list in
 //     LDS (counting sort: 12-bit position in the chunk + sign);
@@ -539,26 +538,37 @@ __global__ void __launch_bounds__(MT) k_msm_bucket_fold(G1Jac* __restrict__ out,
     for (uint32_t sg = s0 + 1; sg < s1; ++sg) acc = g1_add(acc, b[(size_t)sg * MT + t]);
     out[((size_t)row * gridDim.y + grp) * MT + t] = acc;
 }
-// wsum[(sum * MW + w)] from the raw buckets of nseg segments: lane t adds up bucket t+1 over the segments, weights it,
-// and the lanes are summed.  One workgroup per (sum, window).
-// Row z * MW + w (sum z, window w) goes to wsum[(z / n_per) * item_stride + (z % n_per) * MW + w]: the sums of one opening lie
-// together, the openings of a batch item_stride apart (one opening: n_per = all sums, stride 0).
-__global__ void __launch_bounds__(MT) k_msm_buckets(G1Jac* __restrict__ wsum, const G1Jac* __restrict__ buckets, uint32_t nseg, uint32_t n_per, uint32_t item_stride) {
+// The whole sum from the raw buckets of all its windows, one workgroup per sum: lane t first combines bucket t+1 over the
+// windows, sum_w 2^(8w) B[w][t+1] (one Horner walk of 248 doublings, the segments of a window added on the way), and only
+// then weights it by t+1 -- one weighting and one lane sum per sum instead of one per window, and no Horner pass of a
+// single lane over window sums afterwards.  Raw buckets: buckets[((z MW + w) nseg + seg) MT + t].  wsum != nullptr: the point
+// goes where k_open_horner expects the window sums of sum z, wsum[(z / n_per) item_stride + (z % n_per) MW + w] (the sums of one
+// opening lie together, the openings of a batch item_stride apart): the point as window 0, infinity above; else into
+// pts[descs[z].slot].
+__global__ void __launch_bounds__(MT) k_msm_point(G1Jac* __restrict__ wsum, G1Jac* __restrict__ pts, const MsmDesc* __restrict__ descs, const G1Jac* __restrict__ buckets,
+                                                  uint32_t nseg, uint32_t n_per, uint32_t item_stride) {
     __shared__ uint32_t pool[36 * MT];
-    const uint32_t t = threadIdx.x;
-    const G1Jac* b = buckets + (size_t)blockIdx.x * nseg * MT;
-    G1Jac acc = b[t];
-    for (uint32_t sg = 1; sg < nseg; ++sg) acc = g1_add(acc, b[(size_t)sg * MT + t]);
+    const uint32_t t = threadIdx.x, z = blockIdx.x;
     G1Jac r = g1_infinity();
+    for (int w = MW - 1; w >= 0; --w) {
+        if (w != MW - 1)
+            for (int k = 0; k < 8; ++k) r = g1_double(r);
+        const G1Jac* b = buckets + ((size_t)z * MW + (uint32_t)w) * nseg * MT;
+        G1Jac acc = b[t];
+        for (uint32_t sg = 1; sg < nseg; ++sg) acc = g1_add(acc, b[(size_t)sg * MT + t]);
+        r = g1_add(r, acc);
+    }
+    G1Jac q = g1_infinity();
     for (int bit = 7; bit >= 0; --bit) {
-        r = g1_double(r);
-        if (((t + 1) >> bit) & 1u) r = g1_add(r, acc);
+        q = g1_double(q);
+        if (((t + 1) >> bit) & 1u) q = g1_add(q, r);
     }
-    const G1Jac tot = msm_block_sum(pool, r, t);
-    if (t == 0) {
-        const uint32_t z = blockIdx.x / MW, w = blockIdx.x % MW;
-        wsum[(size_t)(z / n_per) * item_stride + (size_t)(z % n_per) * MW + w] = tot;
-    }
+    const G1Jac tot = msm_block_sum(pool, q, t);
+    if (wsum) {
+        G1Jac* __restrict__ W = wsum + (size_t)(z / n_per) * item_stride + (size_t)(z % n_per) * MW;
+        if (t == 0) W[0] = tot;
+        else if (t < (uint32_t)MW) W[t] = g1_infinity();
+    } else if (t == 0) pts[descs[z].slot] = tot;
 }
 
 // ---- the single points of the halving rounds, once per opening ---------------------------------------------------------
@@ -1199,18 +1209,6 @@ __global__ void __launch_bounds__(256) k_tail_coeffs(Fr* __restrict__ C0, const 
     }
     C[(size_t)(3 * levels) * n0 + k] = from_mont(W);
 }
-// one workgroup per sum: lane 0 assembles sum_w 2^(8w) W[w] into pts[slot]
-__global__ void __launch_bounds__(GT) k_msm_horner(G1Jac* __restrict__ pts, const G1Jac* __restrict__ Wsum, const MsmDesc* __restrict__ descs) {
-    if (threadIdx.x != 0) return;
-    const G1Jac* W = Wsum + (size_t)blockIdx.x * MW;
-    G1Jac r = W[MW - 1];
-    for (int w = MW - 2; w >= 0; --w) {
-        for (int k = 0; k < 8; ++k) r = g1_double(r);
-        r = g1_add(r, W[w]);
-    }
-    pts[descs[blockIdx.x].slot] = r;
-}
-
 __global__ void __launch_bounds__(64) k_u32_zero(uint32_t* __restrict__ p, uint32_t n, size_t stride) {      // p[i * stride] = 0, i < n
     for (uint32_t i = threadIdx.x; i < n; i += 64) p[(size_t)i * stride] = 0u;
 }
@@ -1442,7 +1440,7 @@ static int open_round_launch(const RoundItem* items, int count, size_t old_size,
             cur = nxt.as<G1Jac>();
             ns = ng;
         }
-        hipLaunchKernelGGL(k_msm_buckets, dim3(n_msm * MW), dim3(MT), 0, aux, wsum, cur, ns, n_per, wsum_item_stride);
+        hipLaunchKernelGGL(k_msm_point, dim3(n_msm), dim3(MT), 0, aux, wsum, (G1Jac*)nullptr, (const MsmDesc*)nullptr, cur, ns, n_per, wsum_item_stride);
     }
     if (!chained) hipLaunchKernelGGL(k_open_t_fix, dim3(count), dim3(64), 0, aux, wsum, wsum_item_stride);
     ZK_LAUNCH_CHECK();
@@ -1525,12 +1523,10 @@ static int open_tail_launch(const Fr** scalars, const A29* const* gens, int coun
     const size_t ncoef = (size_t)n_msm * n0 * count;
     Scratch& coef = arena.add(sizeof(Fr) * ncoef);
     Scratch& partial = arena.add(sizeof(G1Jac) * total * MW * (size_t)nseg * MT);
-    Scratch& wsum = arena.add(sizeof(G1Jac) * (size_t)total * MW);
     Scratch& dig = arena.add((size_t)(MW + 1) * ncoef);
     if (sl.rc) return sl.rc;
     if (coef.rc) return coef.rc;
     if (partial.rc) return partial.rc;
-    if (wsum.rc) return wsum.rc;
     if (dig.rc) return dig.rc;
     ZK_ARG(ncoef < (1ull << 32), "opening: batched last rounds too large");
     TailPtrs tp;
@@ -1551,8 +1547,7 @@ static int open_tail_launch(const Fr** scalars, const A29* const* gens, int coun
     ZK_HIP(hipMemcpyAsync(desc_dev, hd, sizeof(MsmDesc) * (size_t)total, hipMemcpyHostToDevice, st));
     const MsmDesc* dd = (const MsmDesc*)desc_dev;
     hipLaunchKernelGGL(k_msm_seg<1>, dim3(nseg, MW, total), dim3(MSL), 0, st, partial.as<G1Jac>(), MsmDescs<1>(), dd, nseg, cps);
-    hipLaunchKernelGGL(k_msm_buckets, dim3(total * MW), dim3(MT), 0, st, wsum.as<G1Jac>(), partial.as<G1Jac>(), nseg, (uint32_t)total, 0u);
-    hipLaunchKernelGGL(k_msm_horner, dim3(total), dim3(GT), 0, st, pts, wsum.as<G1Jac>(), dd);
+    hipLaunchKernelGGL(k_msm_point, dim3(total), dim3(MT), 0, st, (G1Jac*)nullptr, pts, dd, partial.as<G1Jac>(), nseg, 1u, 0u);
     ZK_LAUNCH_CHECK();
     // the folded scalar is the single element of the last level
     size_t off = 0, nn = n0;
