@@ -545,15 +545,20 @@ __global__ void __launch_bounds__(MT) k_msm_bucket_fold(G1Jac* __restrict__ out,
 // goes where k_open_horner expects the window sums of sum z, wsum[(z / n_per) item_stride + (z % n_per) MW + w] (the sums of one
 // opening lie together, the openings of a batch item_stride apart): the point as window 0, infinity above; else into
 // pts[descs[z].slot].
+// list != nullptr: sum z is list[z] -- its raw buckets, their segment count and where its window sums go (the sums of
+// several rounds of a job in one launch, behind the last round's bucket accumulation).
+struct PointDesc { const G1Jac* buckets; G1Jac* W; uint32_t nseg, pad; };
 __global__ void __launch_bounds__(MT) k_msm_point(G1Jac* __restrict__ wsum, G1Jac* __restrict__ pts, const MsmDesc* __restrict__ descs, const G1Jac* __restrict__ buckets,
-                                                  uint32_t nseg, uint32_t n_per, uint32_t item_stride) {
+                                                  uint32_t nseg, uint32_t n_per, uint32_t item_stride, const PointDesc* __restrict__ list) {
     __shared__ uint32_t pool[36 * MT];
     const uint32_t t = threadIdx.x, z = blockIdx.x;
+    if (list) { buckets = list[z].buckets; nseg = list[z].nseg; }
+    const size_t zb = list ? 0 : z;
     G1Jac r = g1_infinity();
     for (int w = MW - 1; w >= 0; --w) {
         if (w != MW - 1)
             for (int k = 0; k < 8; ++k) r = g1_double(r);
-        const G1Jac* b = buckets + ((size_t)z * MW + (uint32_t)w) * nseg * MT;
+        const G1Jac* b = buckets + (zb * MW + (uint32_t)w) * nseg * MT;
         G1Jac acc = b[t];
         for (uint32_t sg = 1; sg < nseg; ++sg) acc = g1_add(acc, b[(size_t)sg * MT + t]);
         r = g1_add(r, acc);
@@ -564,8 +569,8 @@ __global__ void __launch_bounds__(MT) k_msm_point(G1Jac* __restrict__ wsum, G1Ja
         if (((t + 1) >> bit) & 1u) q = g1_add(q, r);
     }
     const G1Jac tot = msm_block_sum(pool, q, t);
-    if (wsum) {
-        G1Jac* __restrict__ W = wsum + (size_t)(z / n_per) * item_stride + (size_t)(z % n_per) * MW;
+    if (wsum || list) {
+        G1Jac* __restrict__ W = list ? list[z].W : wsum + (size_t)(z / n_per) * item_stride + (size_t)(z % n_per) * MW;
         if (t == 0) W[0] = tot;
         else if (t < (uint32_t)MW) W[t] = g1_infinity();
     } else if (t == 0) pts[descs[z].slot] = tot;
@@ -1363,8 +1368,10 @@ static CombK comb_of(const GlvK& k) {
 }
 // given: what of this round's sums comes from commitments of the tensor's rows (k_open_cross_part) and is not summed here:
 // 0 nothing, 1 T of the first round (no pair sums), 2 T0 and T1 as well (no bucket sums at all: the round is its fold)
+// later (optional): the reductions of this round's raw buckets are appended to it instead of launched (the caller runs them
+// all at once behind its last round); a round whose T comes from the pair sums (k_open_t_fix) reduces at once
 static int open_round_launch(const RoundItem* items, int count, size_t old_size, bool with_T, int given, G1Jac* wsum_round, uint32_t wsum_item_stride, Arena& arena,
-                             hipStream_t st, hipStream_t aux, std::vector<hipEvent_t>& events) {
+                             hipStream_t st, hipStream_t aux, std::vector<hipEvent_t>& events, std::vector<PointDesc>* later = nullptr) {
     ZK_ARG(old_size < (1ull << 31), "opening: more than 2^31 generators");
     ZK_ARG(count >= 1 && count <= OB_MAX, "opening: bad batch size");
     const size_t new_size = (old_size + 1) / 2;
@@ -1440,7 +1447,10 @@ static int open_round_launch(const RoundItem* items, int count, size_t old_size,
             cur = nxt.as<G1Jac>();
             ns = ng;
         }
-        hipLaunchKernelGGL(k_msm_point, dim3(n_msm), dim3(MT), 0, aux, wsum, (G1Jac*)nullptr, (const MsmDesc*)nullptr, cur, ns, n_per, wsum_item_stride);
+        if (later && chained) {
+            for (uint32_t z = 0; z < n_msm; ++z)
+                later->push_back(PointDesc{cur + (size_t)z * MW * ns * MT, wsum + (size_t)(z / n_per) * wsum_item_stride + (size_t)(z % n_per) * MW, ns, 0u});
+        } else hipLaunchKernelGGL(k_msm_point, dim3(n_msm), dim3(MT), 0, aux, wsum, (G1Jac*)nullptr, (const MsmDesc*)nullptr, cur, ns, n_per, wsum_item_stride, (const PointDesc*)nullptr);
     }
     if (!chained) hipLaunchKernelGGL(k_open_t_fix, dim3(count), dim3(64), 0, aux, wsum, wsum_item_stride);
     ZK_LAUNCH_CHECK();
@@ -1547,7 +1557,7 @@ static int open_tail_launch(const Fr** scalars, const A29* const* gens, int coun
     ZK_HIP(hipMemcpyAsync(desc_dev, hd, sizeof(MsmDesc) * (size_t)total, hipMemcpyHostToDevice, st));
     const MsmDesc* dd = (const MsmDesc*)desc_dev;
     hipLaunchKernelGGL(k_msm_seg<1>, dim3(nseg, MW, total), dim3(MSL), 0, st, partial.as<G1Jac>(), MsmDescs<1>(), dd, nseg, cps);
-    hipLaunchKernelGGL(k_msm_point, dim3(total), dim3(MT), 0, st, (G1Jac*)nullptr, pts, dd, partial.as<G1Jac>(), nseg, 1u, 0u);
+    hipLaunchKernelGGL(k_msm_point, dim3(total), dim3(MT), 0, st, (G1Jac*)nullptr, pts, dd, partial.as<G1Jac>(), nseg, 1u, 0u, (const PointDesc*)nullptr);
     ZK_LAUNCH_CHECK();
     // the folded scalar is the single element of the last level
     size_t off = 0, nn = n0;
@@ -1792,7 +1802,8 @@ struct OpenJob {
     hipStream_t aux = nullptr;     // second stream of the job (bucket sums beside the folds); equals st when the job has one stream
     std::vector<hipEvent_t> events;
     void* pin = nullptr;           // pinned host buffer behind the job's challenges and descriptors
-    ~OpenJob() { pinned_release(pin); }
+    void* pin2 = nullptr;          // and behind the list of its rounds' bucket reductions
+    ~OpenJob() { pinned_release(pin); pinned_release(pin2); }
 };
 // One opening of the batch: its scalars, its challenges (rounds x 8 limbs) and its generators -- Jacobian, or null when
 // `prep` (their prepared form, open_prep_build) is given
@@ -1944,6 +1955,7 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
             r_first = JUMP_ROUNDS;
         }
     }
+    std::vector<PointDesc> later;        // the bucket reductions of the halving rounds: one launch behind the last of them
     for (int r = r_first; r < rounds; ++r) {
         if (size <= (size_t)TAIL_N && rounds - r <= TAIL_LEVELS) {
             int rc = open_tail_launch(cs, cg, count, size, rounds - r, r, rounds, pts.as<G1Jac>(), U_dev, job.pin, (char*)jdev.p + JOB_U_BYTES, job.arena, st);
@@ -1964,10 +1976,22 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
             if (r == 1) { ri[i].comb2 = items[i].comb2; ri[i].u_prev = load_fr(items[i].u + 8 * (r - 1)); }
         }
         const int given = !with_rows ? 0 : (r < cross_r ? 2 : (r == 0 ? 1 : 0));
-        int rc = open_round_launch(ri, count, size, r == 0, given, wsum.as<G1Jac>() + (size_t)3 * MW * r, wstride, job.arena, st, aux, job.events);
+        int rc = open_round_launch(ri, count, size, r == 0, given, wsum.as<G1Jac>() + (size_t)3 * MW * r, wstride, job.arena, st, aux, job.events, aux != st ? &later : nullptr);
         if (rc) return rc;
         for (int i = 0; i < count; ++i) { cs[i] = ri[i].new_scalars; cg[i] = ri[i].new_gens; }
         size = ns;
+    }
+    if (!later.empty()) {
+        ZK_ARG(sizeof(PointDesc) * later.size() <= 65536, "zk_g1_open: too many sums");
+        int prc = pinned_acquire(&job.pin2);
+        if (prc) return prc;
+        memcpy(job.pin2, later.data(), sizeof(PointDesc) * later.size());
+        Scratch& ld = job.arena.add(sizeof(PointDesc) * later.size());
+        if (ld.rc) return ld.rc;
+        ZK_HIP(hipMemcpyAsync(ld.p, job.pin2, sizeof(PointDesc) * later.size(), hipMemcpyHostToDevice, aux));
+        hipLaunchKernelGGL(k_msm_point, dim3((unsigned)later.size()), dim3(MT), 0, aux, (G1Jac*)nullptr, (G1Jac*)nullptr, (const MsmDesc*)nullptr, (const G1Jac*)nullptr, 0u, 1u, 0u,
+                           (const PointDesc*)ld.p);
+        ZK_LAUNCH_CHECK();
     }
     // the single points of the halving rounds, behind the last bucket sums
     if (halving_rounds > 0) {
