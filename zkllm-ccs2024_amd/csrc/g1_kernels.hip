@@ -1436,10 +1436,11 @@ static int open_round_launch(const RoundItem* items, int count, size_t old_size,
     G1Jac* wsum = wsum_round + (size_t)(3 - n_per) * MW;
     hipLaunchKernelGGL(k_msm_seg<OB_SUMS>, dim3(nseg, MW, n_msm), dim3(MSL), 0, aux, partial.as<G1Jac>(), descs, (const MsmDesc*)nullptr, nseg, cps);
     {
-        // sum the segments' raw buckets eight at a time, then weight and total
+        // sum the segments' raw buckets eight at a time (a lane per bucket and window: the reduction, one workgroup per sum,
+        // then walks single buckets), then weight and total
         const G1Jac* cur = partial.as<G1Jac>();
         uint32_t ns = nseg;
-        while (ns > 8) {
+        while (ns > 1) {
             const uint32_t ng = (ns + 7) / 8;
             Scratch& nxt = arena.add(sizeof(G1Jac) * n_msm * MW * (size_t)ng * MT);
             if (nxt.rc) return nxt.rc;
