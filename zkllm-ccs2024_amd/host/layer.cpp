@@ -91,11 +91,17 @@ FrTensor rmsnorm_block(const LayerConfig& c, const Weight& w, const FrTensor& X,
     auto Y = g_inv_rms_ * X;
     auto Y_ = rs2(Y);
 
-    rs2.prove(Y, Y_);
+    // The challenges in the order the proofs below draw them, so that both range proofs can be begun side by side on the
+    // library's streams; each is collected where the reference proves it and the product's sumcheck runs beside the second.
+    const auto ch2 = Rescaling::draw(Y.size);
     auto hu = random_vec(ceilLog2(Y.size));
     auto hv = random_vec(ceilLog2(Y.size));
+    const auto ch1 = Rescaling::draw(g_inv_rms.size);
+    auto p2 = rs2.prove_begin(Y, Y_, ch2);
+    auto p1 = rs1.prove_begin(g_inv_rms, g_inv_rms_, ch1);
+    rs2.prove_end(p2);
     hadamard_product_sumcheck(g_inv_rms_, X, hu, hv);
-    rs1.prove(g_inv_rms, g_inv_rms_);
+    rs1.prove_end(p1);
     auto claims = g.prove(rms_inv, g_inv_rms);
     if (c.open_weights) verifyWeightClaim(w, claims[0]);
     return Y_;
