@@ -106,6 +106,17 @@ int zk_fr_dot(uint32_t* out_host, const void* a, const void* b, size_t n, void* 
 /* 1..3 levels of Fr_multi_dim_partial_me_step / Fr_me_step / Fr_partial_me_step in one pass over
  * in[other][cur][window] (fr-tensor.cu:518-560, :588-641).  u: `levels` standard-form challenges. */
 int zk_fr_fold_axis(void* out, const void* in, const uint32_t* u, int levels, size_t other, uint32_t cur, size_t window, void* stream);
+/* A tensor that is folded again and again at new points and never changes (a layer's weight: the multilinear evaluations
+ * of zkFC::prove, zkfc.cu:77-78, and the fold over the committed rows at the head of Commitment::me_open, commitment.cu:
+ * 118-123), examined once: when every element is a 32-bit signed integer (fixed-point weights are) the handle keeps the int32
+ * form, an eighth of the bytes, and *prepared is non-null; otherwise *prepared is left null (not an error) and the caller
+ * folds the tensor itself.  No counterpart in the reference, which re-reads the field elements each time.  Synchronises.
+ * zk_fr_fold_axis_prepared is all `levels` (1..24) levels of zk_fr_fold_axis at once for such a tensor read as
+ * in[other][cur][window] with cur <= 2^levels (elements beyond cur count as zero):
+ * out[o][w] = sum_j eq(u, j) in[o][j][w], u[0] on the lowest bit of j; bit-identical to the level-by-level fold. */
+int zk_fr_fold_prepare(void** prepared, const void* t, size_t n, void* stream);
+int zk_fr_fold_axis_prepared(void* out, const void* prepared, const uint32_t* u, int levels, size_t other, uint32_t cur, size_t window, void* stream);
+int zk_fr_fold_prepared_free(void* prepared);
 /* FrTensor::operator()(u) / Fr_me (fr-tensor.cu:437-442, :602-609): whole evaluation, fused */
 int zk_fr_me(uint32_t* out_host, const void* a, size_t n, const uint32_t* u, int k, void* stream);
 /* zkip_reduce_kernel / tLookup reduce kernels / hadamard_reduce_kernel on one tensor */

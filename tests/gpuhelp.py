@@ -249,6 +249,12 @@ class Prover:
     def keep_as_matmul_rhs(self, a):
         self.check(self.lib.zkp_fr_keep_as_matmul_rhs(c_void_p(a.h)))
 
+    def keep_for_folds(self, a):
+        self.check(self.lib.zkp_fr_keep_for_folds(c_void_p(a.h)))
+
+    def folds_from_ints(self, a):
+        return int(self.lib.zkp_fr_folds_from_ints(c_void_p(a.h)))
+
     def add_inplace(self, a, b):
         self.check(self.lib.zkp_fr_add_inplace(c_void_p(a.h), c_void_p(b.h)))
 

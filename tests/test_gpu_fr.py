@@ -434,6 +434,61 @@ def test_matmul_with_a_kept_right_operand_and_layers_over_views(pv):
             os.environ["ZKLLM_MATMUL_PLANES"] = old
 
 
+@pytest.mark.parametrize("other,cur,win", [(1, 128, 4096), (3, 100, 64), (37, 1000, 1), (16, 4096, 1), (9, 11008, 1), (5, 63, 1), (2, 2, 8), (1, 512, 1024), (6, 7, 5),
+                                           (1, 70000, 1)])
+def test_folds_of_a_tensor_kept_for_folds_read_its_int32_form_and_give_the_same_elements(pv, orc, other, cur, win):
+    """A tensor of 32-bit integers kept for folds (FrTensor::keep_for_folds -> zk_fr_fold_prepare / zk_fr_fold_axis_prepared:
+    unreduced ten-limb sums of entry x integer products, one reduction per output) folds to the elements the oracle's
+    level-by-level fold gives, for the row folds of the openings (long windows), the column folds of zkFC::prove (window 1:
+    one wave per four rows), ragged axes and the extreme integers; a change in place drops the kept form; a tensor with an
+    element outside 32 bits keeps none and folds as before."""
+    print("case", other, cur, win, flush=True)
+    rng = np.random.default_rng(cur * 31 + win)
+    n = other * cur * win
+    W = rng.integers(-2 ** 31, 2 ** 31, n).astype(np.int64)
+    W[0], W[1 % n], W[2 % n] = -2 ** 31, 2 ** 31 - 1, 0
+    if n > 8:
+        W[n - 1], W[n - 2] = -2 ** 31, -2 ** 31        # the largest magnitude side by side
+    k = (cur - 1).bit_length()
+    u = mt_random_vec(np.random.RandomState(18), k)
+    A = fr_array([int(v) % R_MOD for v in W])
+    exp = np.zeros((n, 8), np.uint32)
+    out_n = np.zeros(1, np.int64)
+    orc_check(orc.orc_fr_partial_me(A, n, u, k, cur, win, exp, out_n))
+    h = pv.from_i64(W)
+    pv.keep_for_folds(h)
+    assert pv.folds_from_ints(h) == 1
+    for rep in range(2):
+        got = pv.partial_me(h, u, cur, win).host()
+        assert got.shape[0] == out_n[0] == other * win
+        assert (got == exp[:out_n[0]]).all(), rep
+    if other == 1:          # the deprecated window form (the fold at the head of an opening) takes the same path
+        got = pv.partial_me_window(h, u, win).host()
+        assert (got == exp[:out_n[0]]).all()
+    # the tensor changes in place: nothing stale may be read, and the new elements are examined again
+    D = rng.integers(-5, 5, n).astype(np.int64)
+    D[0], D[1 % n] = 1, 0
+    if n > 8:
+        D[n - 1], D[n - 2] = 0, 3
+    pv.add_inplace(h, pv.from_i64(D))
+    W2 = W + D
+    A2 = fr_array([int(v) % R_MOD for v in W2])
+    orc_check(orc.orc_fr_partial_me(A2, n, u, k, cur, win, exp, out_n))
+    got = pv.partial_me(h, u, cur, win).host()
+    assert (got == exp[:out_n[0]]).all()
+    assert pv.folds_from_ints(h) == 1
+    # one element of 33 bits: no int32 form is kept, the fold is the plain one
+    W3 = W2.copy()
+    W3[n // 2] = 2 ** 31
+    h3 = pv.from_i64(W3)
+    pv.keep_for_folds(h3)
+    assert pv.folds_from_ints(h3) == 0
+    A3 = fr_array([int(v) % R_MOD for v in W3])
+    orc_check(orc.orc_fr_partial_me(A3, n, u, k, cur, win, exp, out_n))
+    got = pv.partial_me(h3, u, cur, win).host()
+    assert (got == exp[:out_n[0]]).all()
+
+
 def test_stacks_of_matrices_transpose_and_multiply_like_their_members(pv):
     """zk_fr_matmul_batched / zk_fr_transpose_batched on every path of the dispatcher (both operands in 31 bits, wide left
     operand, wide right operand, full-width residues): each product of the stack against big-int arithmetic."""

@@ -1042,6 +1042,142 @@ static int eq_table_queue(Fr* out, const uint32_t* u, int k, Arena& arena, hipSt
     return 0;
 }
 
+// ---- folds of a tensor of 32-bit integers by eq weights ------------------------------------------------------------------
+// A tensor whose elements are 32-bit signed integers (a weight: fixed-point values) folds from its int32 form: an eighth of
+// the bytes, and a product with an eq entry is eight limb products with no reduction.  The unreduced sum of a whole fold
+// fits ten limbs (entries below 2^255, magnitudes up to 2^31, up to 2^24 terms) and is reduced once: the low 256 bits by
+// one Montgomery product with 1 (the entries carry R), the two limbs above them count R each, which that product cancels.
+struct FoldPrepared { int32_t* ints = nullptr; size_t n = 0; };
+struct EqPair { Fr e, ne; };        // an eq entry and its negative, Montgomery form
+__global__ void __launch_bounds__(TPB) k_fold_ints(int32_t* __restrict__ out, uint32_t* __restrict__ bad, const Fr* __restrict__ in, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    const Fr x = in[i];
+    const int32_t v = fr_to_i32(x);
+    out[i] = v;
+    if (!equal(fr_from_i64((int64_t)v), x)) atomicOr(bad, 1u);
+}
+__global__ void __launch_bounds__(TPB) k_eq_pairs(EqPair* __restrict__ out, const Fr* __restrict__ E, uint32_t cur) {
+    const uint32_t j = blockIdx.x * TPB + threadIdx.x;
+    if (j >= cur) return;
+    EqPair p;
+    p.e = E[j];
+    p.ne = neg(p.e);
+    out[j] = p;
+}
+__device__ __forceinline__ void ifold_mac(uint32_t (&acc)[10], const Fr& e, const Fr& ne, int32_t w) {
+    const bool ng = w < 0;
+    const uint32_t a = ng ? 0u - (uint32_t)w : (uint32_t)w;
+    uint64_t carry = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t s = ng ? ne.v[i] : e.v[i];
+        const uint64_t t = (uint64_t)s * a + acc[i] + carry;       // at most (2^32 - 1)^2 + 2 (2^32 - 1) = 2^64 - 1
+        acc[i] = (uint32_t)t;
+        carry = t >> 32;
+    }
+    const uint64_t t = (uint64_t)acc[8] + carry;
+    acc[8] = (uint32_t)t;
+    acc[9] += (uint32_t)(t >> 32);
+}
+__device__ __forceinline__ Fr ifold_finish(const uint32_t (&acc)[10]) {
+    Fr lo;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) lo.v[i] = acc[i];
+    lo = reduce_once(reduce_once(lo));          // below 2^256 < 3 r
+    Fr one = big_zero<8>(), hi = big_zero<8>();
+    one.v[0] = 1;
+    hi.v[0] = acc[8];
+    hi.v[1] = acc[9];
+    return add(mont_mul(lo, one), hi);
+}
+// the unreduced sums of four waves through LDS: wave 0 adds them up
+__device__ __forceinline__ void ifold_put(uint32_t (*sh)[10][64], uint32_t wv, uint32_t lane, const uint32_t (&acc)[10]) {
+#pragma unroll
+    for (int i = 0; i < 10; ++i) sh[wv][i][lane] = acc[i];
+}
+__device__ __forceinline__ void ifold_gather(uint32_t (&acc)[10], uint32_t (*sh)[10][64], uint32_t lane) {
+#pragma unroll
+    for (int q = 1; q < 4; ++q) {
+        uint32_t c = 0;
+#pragma unroll
+        for (int i = 0; i < 10; ++i) acc[i] = addc32(acc[i], sh[q][i][lane], c);
+    }
+}
+// out[o][w] = sum_j E[j] in[o][j][w].  A workgroup serves 64 consecutive outputs; each of its four waves takes a quarter of
+// the axis (the entries of a step are the same for every lane of a wave), eight loads in flight per lane.
+__global__ void __launch_bounds__(256) k_ifold_window(Fr* __restrict__ out, const int32_t* __restrict__ in, const EqPair* __restrict__ E, size_t n_out, uint32_t cur, size_t window) {
+    __shared__ uint32_t sh[4][10][64];
+    const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;
+    const size_t g = (size_t)blockIdx.x * 64 + lane;
+    const bool live = g < n_out;
+    const size_t gg = live ? g : n_out - 1;
+    const size_t o = gg / window, w = gg % window;
+    const int32_t* p = in + o * (size_t)cur * window + w;
+    const uint32_t per = (cur + 3) / 4;
+    const uint32_t j0 = wv * per < cur ? wv * per : cur, j1 = j0 + per < cur ? j0 + per : cur;
+    uint32_t acc[10];
+#pragma unroll
+    for (int i = 0; i < 10; ++i) acc[i] = 0;
+    uint32_t j = j0;
+    for (; j + 8 <= j1; j += 8) {
+        int32_t x[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) x[t] = p[(size_t)(j + t) * window];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) ifold_mac(acc, E[j + t].e, E[j + t].ne, x[t]);
+    }
+    for (; j < j1; ++j) ifold_mac(acc, E[j].e, E[j].ne, p[(size_t)j * window]);
+    if (wv) ifold_put(sh, wv, lane, acc);
+    __syncthreads();
+    if (wv == 0) {
+        ifold_gather(acc, sh, lane);
+        if (live) out[g] = ifold_finish(acc);
+    }
+}
+// window 1: out[o] = sum_j E[j] in[o][j].  A workgroup serves four rows; each of its four waves takes a quarter of the axis
+// for all four (an entry is loaded once for the four rows), lanes over j, a butterfly over the wave, then the four waves' sums.
+__global__ void __launch_bounds__(256) k_ifold_rows(Fr* __restrict__ out, const int32_t* __restrict__ in, const EqPair* __restrict__ E, size_t other, uint32_t cur) {
+    __shared__ uint32_t sh[4][10][64];          // [wave][limb][row] (rows 0..3 used)
+    const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;
+    const size_t o0 = (size_t)blockIdx.x * 4;
+    const uint32_t per = ((cur + 255) / 256) * 64;          // a quarter of the axis, in whole wave steps
+    const uint32_t j0 = wv * per < cur ? wv * per : cur, j1 = j0 + per < cur ? j0 + per : cur;
+    uint32_t acc[4][10];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int i = 0; i < 10; ++i) acc[r][i] = 0;
+    for (uint32_t j = j0 + lane; j < j1; j += 64) {
+        const EqPair ep = E[j];
+        int32_t x[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) x[r] = o0 + r < other ? in[(o0 + r) * (size_t)cur + j] : 0;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) ifold_mac(acc[r], ep.e, ep.ne, x[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        for (int off = 32; off > 0; off >>= 1) {
+            uint32_t c = 0;
+#pragma unroll
+            for (int i = 0; i < 10; ++i) acc[r][i] = addc32(acc[r][i], (uint32_t)__shfl_xor((int)acc[r][i], off, 64), c);
+        }
+        if (lane == 0 && wv) {
+#pragma unroll
+            for (int i = 0; i < 10; ++i) sh[wv][i][r] = acc[r][i];
+        }
+    }
+    __syncthreads();
+    if (wv == 0 && lane == 0) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            ifold_gather(acc[r], sh, (uint32_t)r);
+            if (o0 + r < other) out[o0 + r] = ifold_finish(acc[r]);
+        }
+    }
+}
+
 extern "C" {
 
 int zk_lookup_index_fr(void* idx_u32, const void* vals, int32_t low, uint32_t table_size, size_t n, void* stv) {
@@ -1105,6 +1241,58 @@ int zk_eq_table(void* out, const uint32_t* u, int k, void* stv) {
     ZK_ARG(k >= 0 && k <= 30, "zk_eq_table: k out of range");
     Arena tmp((hipStream_t)stv);        // the half tables return to the allocator at once: later users are ordered behind these launches on the same stream
     return eq_table_queue((Fr*)out, u, k, tmp, (hipStream_t)stv);
+}
+// ---- folds of a tensor of 32-bit integers by eq weights ------------------------------------------------------------------
+int zk_fr_fold_prepare(void** prepared, const void* t, size_t n, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(prepared != nullptr && t != nullptr && n >= 1, "zk_fr_fold_prepare: null argument or empty tensor");
+    *prepared = nullptr;
+    void* ints = nullptr;
+    int rc = pool_alloc(&ints, sizeof(int32_t) * n, st);
+    if (rc) return rc;
+    uint32_t bad = 0;
+    {
+        Scratch flag(4, st);
+        if (flag.rc) { pool_free(ints, st); return flag.rc; }
+        hipError_t e = hipMemsetAsync(flag.p, 0, 4, st);        // setup call: never part of a captured graph (it ends with a host read)
+        if (e != hipSuccess) { pool_free(ints, st); ZK_HIP(e); }
+        hipLaunchKernelGGL(k_fold_ints, dim3(cdiv(n, TPB)), dim3(TPB), 0, st, (int32_t*)ints, flag.as<uint32_t>(), (const Fr*)t, n);
+        rc = read_flag(flag.as<uint32_t>(), &bad, st);
+    }
+    if (rc || bad) { pool_free(ints, st); return rc; }
+    FoldPrepared* fp = new FoldPrepared;
+    fp->ints = (int32_t*)ints;
+    fp->n = n;
+    *prepared = fp;
+    return 0;
+}
+int zk_fr_fold_prepared_free(void* prepared) {
+    FoldPrepared* fp = (FoldPrepared*)prepared;
+    if (!fp) return 0;
+    pool_free(fp->ints, nullptr);
+    delete fp;
+    return 0;
+}
+int zk_fr_fold_axis_prepared(void* out, const void* prepared, const uint32_t* u, int levels, size_t other, uint32_t cur, size_t window, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    const FoldPrepared* fp = (const FoldPrepared*)prepared;
+    ZK_ARG(fp != nullptr && out != nullptr && u != nullptr, "zk_fr_fold_axis_prepared: null argument");
+    ZK_ARG(levels >= 1 && levels <= 24, "zk_fr_fold_axis_prepared: 1 to 24 levels");
+    ZK_ARG(cur >= 1 && cur <= (1u << levels), "zk_fr_fold_axis_prepared: the axis is longer than 2^levels");
+    ZK_ARG(other >= 1 && window >= 1 && other * (size_t)cur * window == fp->n, "zk_fr_fold_axis_prepared: other * cur * window is not the tensor's size");
+    Arena tmp(st);
+    Scratch& E = tmp.add(sizeof(Fr) * ((size_t)1 << levels));
+    Scratch& P = tmp.add(sizeof(EqPair) * (size_t)cur);
+    if (E.rc) return E.rc;
+    if (P.rc) return P.rc;
+    int rc = eq_table_queue(E.as<Fr>(), u, levels, tmp, st);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_eq_pairs, dim3(cdiv(cur, TPB)), dim3(TPB), 0, st, P.as<EqPair>(), E.as<Fr>(), cur);
+    const size_t n_out = other * window;
+    if (window == 1 && cur >= 64) hipLaunchKernelGGL(k_ifold_rows, dim3(cdiv(other, 4)), dim3(256), 0, st, (Fr*)out, fp->ints, P.as<EqPair>(), other, cur);
+    else hipLaunchKernelGGL(k_ifold_window, dim3(cdiv(n_out, 64)), dim3(256), 0, st, (Fr*)out, fp->ints, P.as<EqPair>(), n_out, cur, window);
+    ZK_LAUNCH_CHECK();
+    return 0;
 }
 // out_host[i] = multilinear extension of Xs[i] (n elements each, zero beyond) at u (k challenges, 2^(k-1) < n <= 2^k)
 int zk_fr_me_multi(uint32_t* out_host, const void* const* Xs, int K, size_t n, const uint32_t* u, int k, void* stv) {

@@ -272,7 +272,12 @@ Weight create_weight(string generator_filename, string weight_filename, string c
     G1TensorJacobian com(com_filename);
     generator.prepare_openings();
     Weight w{generator, weight, com, in_dim, out_dim, nullptr};
-    if (in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim))) w.padded = std::make_shared<const FrTensor>(w.weight.pad({in_dim, out_dim}));
+    w.weight.keep_for_folds();          // proofs and openings fold it at a new point each time
+    if (in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim))) {
+        auto pd = std::make_shared<FrTensor>(w.weight.pad({in_dim, out_dim}));
+        pd->keep_for_folds();
+        w.padded = pd;
+    }
     return w;
 }
 

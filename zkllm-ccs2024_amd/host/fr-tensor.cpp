@@ -197,15 +197,32 @@ FrTensor::FrTensor(uint size, const double* cpu_data, unsigned long sf) : gpu_da
 FrTensor::FrTensor(const FrTensor& t) : gpu_data(fr_alloc(t.size)), size(t.size) {
     ZKC(zk_memcpy_d2d(gpu_data, t.gpu_data, sizeof(Fr_t) * (size_t)size, nullptr));
 }
-FrTensor::FrTensor(FrTensor&& t) noexcept : gpu_data(t.gpu_data), size(t.size), borrowed(t.borrowed), rhs_cache(std::move(t.rhs_cache)) { t.gpu_data = nullptr; }
+FrTensor::FrTensor(FrTensor&& t) noexcept
+    : gpu_data(t.gpu_data), size(t.size), borrowed(t.borrowed), rhs_cache(std::move(t.rhs_cache)), fold_cache(std::move(t.fold_cache)) { t.gpu_data = nullptr; }
 void MatmulRhsCache::reset() {
     if (prepared) zk_fr_matmul_rhs_free(prepared);
     prepared = nullptr;
 }
-FrTensor::FrTensor(const FrTensor& t, ViewTag) : gpu_data(t.gpu_data), size(t.size), borrowed(true), rhs_cache(t.rhs_cache) {}
+FrTensor::FrTensor(const FrTensor& t, ViewTag) : gpu_data(t.gpu_data), size(t.size), borrowed(true), rhs_cache(t.rhs_cache), fold_cache(t.fold_cache) {}
 FrTensor FrTensor::view(const FrTensor& t) { return FrTensor(t, ViewTag{}); }
 void FrTensor::keep_as_matmul_rhs() {
     if (!rhs_cache) rhs_cache = std::make_shared<MatmulRhsCache>();
+}
+void FoldCache::reset() {
+    if (prepared) zk_fr_fold_prepared_free(prepared);
+    prepared = nullptr;
+    tried = false;
+}
+void FrTensor::keep_for_folds() {
+    if (!fold_cache) fold_cache = std::make_shared<FoldCache>();
+    if (!fold_cache->tried) {
+        fold_cache->tried = true;
+        ZKC(zk_fr_fold_prepare(&fold_cache->prepared, gpu_data, size, nullptr));
+    }
+}
+void FrTensor::drop_kept() {
+    if (rhs_cache) rhs_cache->reset();
+    if (fold_cache) fold_cache->reset();
 }
 FrTensor::FrTensor(const string& filename) : gpu_data(nullptr), size((uint)(findsize(filename) / sizeof(Fr_t))) {
     gpu_data = fr_alloc(size);
@@ -258,22 +275,22 @@ Fr_t FrTensor::operator()(uint idx) const {
 
 FrTensor FrTensor::operator+(const FrTensor& t) const { SAME_SIZE(t); FrTensor out(size); ZKC(zk_fr_add(out.gpu_data, gpu_data, t.gpu_data, size, nullptr)); return out; }
 FrTensor FrTensor::operator+(const Fr_t& x) const { FrTensor out(size); ZKC(zk_fr_add_s(out.gpu_data, gpu_data, x.val, size, nullptr)); return out; }
-FrTensor& FrTensor::operator+=(const FrTensor& t) { SAME_SIZE(t); if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_add(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
-FrTensor& FrTensor::operator+=(const Fr_t& x) { if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_add_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator+=(const FrTensor& t) { SAME_SIZE(t); drop_kept(); ZKC(zk_fr_add(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator+=(const Fr_t& x) { drop_kept(); ZKC(zk_fr_add_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
 FrTensor FrTensor::operator-() const { FrTensor out(size); ZKC(zk_fr_neg(out.gpu_data, gpu_data, size, nullptr)); return out; }
 FrTensor FrTensor::operator-(const FrTensor& t) const { SAME_SIZE(t); FrTensor out(size); ZKC(zk_fr_sub(out.gpu_data, gpu_data, t.gpu_data, size, nullptr)); return out; }
 FrTensor FrTensor::operator-(const Fr_t& x) const { FrTensor out(size); ZKC(zk_fr_sub_s(out.gpu_data, gpu_data, x.val, size, nullptr)); return out; }
-FrTensor& FrTensor::operator-=(const FrTensor& t) { SAME_SIZE(t); if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_sub(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
-FrTensor& FrTensor::operator-=(const Fr_t& x) { if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_sub_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
-FrTensor& FrTensor::mont() { if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_mont(gpu_data, gpu_data, size, nullptr)); return *this; }
-FrTensor& FrTensor::unmont() { if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_unmont(gpu_data, gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator-=(const FrTensor& t) { SAME_SIZE(t); drop_kept(); ZKC(zk_fr_sub(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator-=(const Fr_t& x) { drop_kept(); ZKC(zk_fr_sub_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
+FrTensor& FrTensor::mont() { drop_kept(); ZKC(zk_fr_mont(gpu_data, gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::unmont() { drop_kept(); ZKC(zk_fr_unmont(gpu_data, gpu_data, size, nullptr)); return *this; }
 FrTensor FrTensor::operator*(const FrTensor& t) const { SAME_SIZE(t); FrTensor out(size); ZKC(zk_fr_mul(out.gpu_data, gpu_data, t.gpu_data, size, nullptr)); return out; }
 FrTensor FrTensor::operator*(const Fr_t& x) const { FrTensor out(size); ZKC(zk_fr_mul_s(out.gpu_data, gpu_data, x.val, size, nullptr)); return out; }
-FrTensor& FrTensor::operator*=(const FrTensor& t) { SAME_SIZE(t); if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_mul(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
-FrTensor& FrTensor::operator*=(const Fr_t& x) { if (rhs_cache) rhs_cache->reset(); ZKC(zk_fr_mul_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator*=(const FrTensor& t) { SAME_SIZE(t); drop_kept(); ZKC(zk_fr_mul(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
+FrTensor& FrTensor::operator*=(const Fr_t& x) { drop_kept(); ZKC(zk_fr_mul_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
 FrTensor& FrTensor::operator=(const FrTensor& t) {
     if (size != t.size) throw std::runtime_error("operator=: Incompatible dimensions");
-    if (rhs_cache) rhs_cache->reset();
+    drop_kept();
     ZKC(zk_memcpy_d2d(gpu_data, t.gpu_data, sizeof(Fr_t) * (size_t)size, nullptr));
     return *this;
 }
@@ -313,6 +330,17 @@ static FrTensor fold_axis_all(const FrTensor& t, const vector<Fr_t>& u, uint cur
     if (u.empty()) return t;
     if ((size_t)t.size % ((size_t)cur_dim * window) != 0) throw std::runtime_error("t.size % (cur_dim * window_size) != 0");
     const size_t other = (size_t)t.size / ((size_t)cur_dim * window);
+    if (FoldCache* fc = t.fold_cache.get(); fc && u.size() <= 24 && cur_dim <= (1u << u.size())) {
+        if (!fc->tried) {
+            fc->tried = true;
+            ZKC(zk_fr_fold_prepare(&fc->prepared, t.gpu_data, t.size, nullptr));
+        }
+        if (fc->prepared) {
+            FrTensor out((uint)(other * window));
+            ZKC(zk_fr_fold_axis_prepared(out.gpu_data, fc->prepared, u[0].val, (int)u.size(), other, cur_dim, window, nullptr));
+            return out;
+        }
+    }
     const Fr_t* src = t.gpu_data;
     std::vector<FrTensor> keep;   // intermediates stay alive until the last pass has been queued
     size_t done = 0;

@@ -74,6 +74,15 @@ struct MatmulRhsCache {
     ~MatmulRhsCache() { reset(); }
 };
 
+// What a tensor that is folded at many points and never changes keeps (FrTensor::keep_for_folds): the handle of
+// zk_fr_fold_prepare, null when the elements are not 32-bit integers.  Shared by the tensor and its views.
+struct FoldCache {
+    void* prepared = nullptr;
+    bool tried = false;
+    void reset();
+    ~FoldCache() { reset(); }
+};
+
 class FrTensor {
    public:
     Fr_t* gpu_data;
@@ -82,6 +91,7 @@ class FrTensor {
     // keep_as_matmul_rhs
     bool borrowed = false;
     std::shared_ptr<MatmulRhsCache> rhs_cache;
+    std::shared_ptr<FoldCache> fold_cache;      // see keep_for_folds
 
     FrTensor(uint size);
     FrTensor(uint size, const Fr_t* cpu_data);
@@ -144,6 +154,11 @@ class FrTensor {
     // and keeps that for later products; for tensors that are not modified afterwards (weights).  The in-place operators
     // drop what was kept.
     void keep_as_matmul_rhs();
+    // keep_for_folds: from now on partial_me / multi_dim_me of this tensor (and of its views) examine it once and, when it
+    // holds 32-bit integers, fold its int32 form (bit-identical results).  Every operation that changes the elements drops
+    // what was kept.
+    void keep_for_folds();
+    void drop_kept();       // what keep_as_matmul_rhs and keep_for_folds hold, after the elements have changed
     // additions for stacks of `num` equally shaped matrices stored one after the other: every M x N matrix transposed,
     // and the num products x_i (M x N) * y_i (N x P)
     FrTensor transpose_stack(uint num, uint M, uint N) const;

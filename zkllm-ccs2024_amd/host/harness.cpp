@@ -170,6 +170,9 @@ void* zkp_fr_scalarop(int op, void* a, const u32* s) {
 // the additions around a weight tensor: kept as the right operand of matrix products, modified in place (a += b), and a fully
 // connected layer built over a view of it (zkFC(in, out, FrTensor::view(w))): Y = X W through that layer
 int zkp_fr_keep_as_matmul_rhs(void* a) { ZKP_TRY FT(a).keep_as_matmul_rhs(); ZKP_END }
+int zkp_fr_keep_for_folds(void* a) { ZKP_TRY FT(a).keep_for_folds(); ZKP_END }
+// 1 when the tensor's folds read its int32 form, 0 when it keeps none (not asked to, or its elements are not 32-bit integers)
+int zkp_fr_folds_from_ints(void* a) { return FT(a).fold_cache && FT(a).fold_cache->prepared ? 1 : 0; }
 int zkp_fr_add_inplace(void* a, void* b) { ZKP_TRY FT(a) += FT(b); ZKP_END }
 void* zkp_fc_forward_over_view(void* w, void* x, u32 in_dim, u32 out_dim) {
     ZKP_TRY
@@ -501,6 +504,7 @@ void* zkp_layer_create(const u32* cu, const double* cf, const int32_t* norm1, co
     const uint E = c.embed_dim, Hd = c.hidden_dim;
     auto mk = [&](const int32_t* p, uint in_dim, uint out_dim, uint pp) {
         FrTensor weight(in_dim * out_dim, (const int*)p);
+        weight.keep_for_folds();
         Commitment gen = Commitment::random(1u << ceilLog2(pp));
         G1TensorJacobian com = gen.commit_int(weight.pad({in_dim, out_dim}));
         Weight w{std::move(gen), std::move(weight), std::move(com), in_dim, out_dim};

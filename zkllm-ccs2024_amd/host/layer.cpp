@@ -420,8 +420,14 @@ static Weight random_weight(std::mt19937_64& rng, uint in_dim, uint out_dim, uin
     for (auto& x : wi) x = norm ? 65536 : (int)std::nearbyint(nd(rng) * 65536.0);   // scale 2^16 (llama-commit.py:34)
     FrTensor weight((uint)wi.size(), wi.data());
     if (!norm) weight.keep_as_matmul_rhs();        // the right operand of the layer's projections, run after run
+    weight.keep_for_folds();                       // and folded at a new point by every proof and every opening
     const bool ragged = in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim));
-    std::shared_ptr<const FrTensor> padded = ragged ? std::make_shared<const FrTensor>(weight.pad({in_dim, out_dim})) : nullptr;
+    std::shared_ptr<const FrTensor> padded;
+    if (ragged) {
+        auto pd = std::make_shared<FrTensor>(weight.pad({in_dim, out_dim}));
+        pd->keep_for_folds();
+        padded = pd;
+    }
     const double t1 = now_ms();
     Commitment gen = Commitment::random(1u << ceilLog2(pp_size));
     const double t2 = now_ms();
