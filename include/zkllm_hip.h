@@ -117,6 +117,18 @@ int zk_fr_fold_axis(void* out, const void* in, const uint32_t* u, int levels, si
 int zk_fr_fold_prepare(void** prepared, const void* t, size_t n, void* stream);
 int zk_fr_fold_axis_prepared(void* out, const void* prepared, const uint32_t* u, int levels, size_t other, uint32_t cur, size_t window, void* stream);
 int zk_fr_fold_prepared_free(void* prepared);
+/* The same handle for a tensor whose int32 form is written by the kernel that makes the tensor (the digit planes of
+ * zk_softmax_decompose_ints, the outputs of zk_fr_gather_ints), so no pass over the field elements is needed: _new
+ * allocates the handle and its n int32 slots (uninitialised) and returns their device address; the caller must have queued
+ * the kernel that sets ints_dev[i] to element i before the handle is used.  _ints returns that address (null for null). */
+int zk_fr_fold_prepared_new(void** prepared, void** ints_dev, size_t n, void* stream);
+const void* zk_fr_fold_prepared_ints(const void* prepared);
+/* zk_fr_gather (out[i] = table[idx[i]], the mapped values of tLookupRangeMapping::operator(), tlookup.cu:446-470) that
+ * also writes the int32 form of out from the table's own (table_prepared: a handle of zk_fr_fold_prepare over the table) */
+int zk_fr_gather_ints(void* out, void* out_ints, const void* table, const void* table_prepared, const void* idx, size_t n, void* stream);
+/* zk_fr_me_multi where prepareds[i], when non-null, is the int32 form of Xs[i] (same n): such tensors are read from it --
+ * an eighth of the bytes, eight limb products per element instead of a Montgomery product.  Same values. */
+int zk_fr_me_multi_ints(uint32_t* out_host, const void* const* Xs, const void* const* prepareds, int K, size_t n, const uint32_t* u, int k, void* stream);
 /* FrTensor::operator()(u) / Fr_me (fr-tensor.cu:437-442, :602-609): whole evaluation, fused */
 int zk_fr_me(uint32_t* out_host, const void* a, size_t n, const uint32_t* u, int k, void* stream);
 /* zkip_reduce_kernel / tLookup reduce kernels / hadamard_reduce_kernel on one tensor */
@@ -290,6 +302,8 @@ int zk_softmax_shift(void* shift, void* out_shifted, const void* X, uint32_t row
 int zk_softmax_table(void* table, double log_theta, double step, uint32_t len, void* stream);
 /* planes: K device tensors of n elements each (host array of K pointers); plane k receives digit k */
 int zk_softmax_decompose(void* const* planes, const void* X_shifted, const uint32_t* bs_host, int K, size_t n, void* stream);
+/* the same, and int_planes[k] (int32, n each; null entries and a null array allowed) receive digit k once more as int32 */
+int zk_softmax_decompose_ints(void* const* planes, void* const* int_planes, const void* X_shifted, const uint32_t* bs_host, int K, size_t n, void* stream);
 
 /* ---- measurement helpers (no counterpart in the reference) ---------------------------------------- */
 /* v_mad_u64_u32 issue peak of the device: 16 independent chains per lane, no memory traffic */

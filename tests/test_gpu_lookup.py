@@ -424,6 +424,90 @@ def test_mapped_lookup_job_equals_the_plain_one_on_the_combined_queries(k):
         hip.free(p)
 
 
+@pytest.mark.parametrize("n", [3007, 1 << 16])
+def test_int32_forms_written_with_the_tensors_serve_index_gather_and_evaluations(n):
+    """zk_softmax_decompose_ints writes every digit plane as field elements and as int32 (both checked against divmod);
+    zk_fr_gather_ints writes the gathered table values with their int32 form; zk_fr_me_multi_ints, reading the int32 forms
+    where given (five of them and one tensor of full residues: the mix of a softmax proof; then seven with two residue tensors),
+    returns exactly what zk_fr_me_multi returns, which is checked against the brute-force extension at small n."""
+    import ctypes
+    from gpuhelp import Hip, c_void_p, c_size_t, c_int
+    from zkhelp import me_bruteforce
+    hip = Hip()
+    rng = np.random.default_rng(n)
+    bs = np.array([256, 1 << 20, 1 << 20], dtype=np.uint32)
+    mag = rng.integers(0, 1 << 48, n).astype(np.int64)
+    mag[0], mag[1] = 0, (1 << 48) - 1
+    X = fr_array([(-int(v)) % R_MOD for v in mag])
+    dX = hip.upload(X)
+    planes = [hip.malloc(32 * n) for _ in range(3)]
+    handles, ints = [], []
+    for _ in range(3):
+        h, q = c_void_p(), c_void_p()
+        hip.call("zk_fr_fold_prepared_new", ctypes.byref(h), ctypes.byref(q), c_size_t(n), None)
+        handles.append(h)
+        ints.append(q)
+    hip.lib.zk_fr_fold_prepared_ints.restype = c_void_p
+    for h, q in zip(handles, ints):
+        assert hip.lib.zk_fr_fold_prepared_ints(h) == q.value
+    arr = (c_void_p * 3)(*[c_void_p(x) for x in planes])
+    iarr = (c_void_p * 3)(*ints)
+    hip.call("zk_softmax_decompose_ints", arr, iarr, c_void_p(dX), bs, c_int(3), c_size_t(n), None)
+    digits = []
+    t = mag.astype(object)
+    for b in bs:
+        digits.append(np.array([int(v) % int(b) for v in t], dtype=np.int64))
+        t = np.array([int(v) // int(b) for v in t], dtype=object)
+    for k in range(3):
+        got_fr = hip.download(planes[k], (n, 8), np.uint32)
+        got_i = hip.download(ints[k].value, (n,), np.int32)
+        assert (got_i == digits[k]).all(), k
+        assert (got_fr[:, 0] == digits[k]).all() and not got_fr[:, 1:].any(), k
+    # gather by the first plane's digits from a table of 256 integers of up to 22 bits
+    tab_i = rng.integers(0, 1 << 22, 256).astype(np.int64)
+    tab_i[0], tab_i[255] = (1 << 22) - 1, 0
+    dT = hip.upload(fr_array([int(v) for v in tab_i]))
+    th = c_void_p()
+    hip.call("zk_fr_fold_prepare", ctypes.byref(th), c_void_p(dT), c_size_t(256), None)
+    assert th.value
+    idx = digits[0].astype(np.uint32)
+    dI = hip.upload(idx)
+    dG = hip.malloc(32 * n)
+    gh, gq = c_void_p(), c_void_p()
+    hip.call("zk_fr_fold_prepared_new", ctypes.byref(gh), ctypes.byref(gq), c_size_t(n), None)
+    hip.call("zk_fr_gather_ints", c_void_p(dG), gq, c_void_p(dT), th, c_void_p(dI), c_size_t(n), None)
+    got_fr = hip.download(dG, (n, 8), np.uint32)
+    got_i = hip.download(gq.value, (n,), np.int32)
+    assert (got_i == tab_i[idx]).all() and (got_fr[:, 0] == tab_i[idx]).all() and not got_fr[:, 1:].any()
+    # evaluations: int32 forms where there are some, full residues elsewhere
+    k = (n - 1).bit_length()
+    u = ch(71, k)
+    R1, R2 = ch(72, n), ch(73, n)
+    dR1, dR2 = hip.upload(R1), hip.upload(R2)
+    for Xs, hs in [([planes[0], planes[1], dR1, planes[2], dG, planes[0]], [handles[0], handles[1], None, handles[2], gh, handles[0]]),
+                   ([dR1, planes[0], planes[1], planes[2], dG, planes[1], planes[2], dR2], [None, handles[0], handles[1], handles[2], gh, handles[1], handles[2], None]),
+                   ([planes[1]], [handles[1]]), ([dR1, dR2], [None, None])]:
+        K = len(Xs)
+        xa = (c_void_p * K)(*[c_void_p(x) for x in Xs])
+        ha = (c_void_p * K)(*[h if h is not None else c_void_p(None) for h in hs])
+        want, got = np.zeros((K, 8), np.uint32), np.zeros((K, 8), np.uint32)
+        hip.call("zk_fr_me_multi", want, xa, c_int(K), c_size_t(n), u, c_int(k), None)
+        hip.call("zk_fr_me_multi_ints", got, xa, ha, c_int(K), c_size_t(n), u, c_int(k), None)
+        assert (got == want).all(), K
+    if n < 5000:
+        ui = fr_ints(u)
+        assert fr_ints(got[:1])[0] == me_bruteforce(fr_ints(R1), ui)
+        xa = (c_void_p * 1)(c_void_p(planes[1]))
+        ha = (c_void_p * 1)(handles[1])
+        one = np.zeros((1, 8), np.uint32)
+        hip.call("zk_fr_me_multi_ints", one, xa, ha, c_int(1), c_size_t(n), u, c_int(k), None)
+        assert fr_ints(one)[0] == me_bruteforce([int(v) for v in digits[1]], ui)
+    for h in handles + [gh, th]:
+        hip.call("zk_fr_fold_prepared_free", h)
+    for q in planes + [dX, dT, dI, dG, dR1, dR2]:
+        hip.free(q)
+
+
 def test_config4_full_size_range_lookup_and_softmax_of_one_head(pv):
     """One attention head at sequence length 2048: 2^22 scores uniform in [-2^15, 2^15), a range table of 2^16 entries.
     Beyond what the oracle can follow, so checked through what the protocol fixes: the multiplicities are numpy's

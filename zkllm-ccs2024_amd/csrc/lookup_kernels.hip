@@ -984,18 +984,25 @@ __global__ void __launch_bounds__(TPB) k_softmax_table(Fr* __restrict__ table, d
 // negation does not fit 64 bits raise the flag (the reference leaves their planes unwritten).
 struct U32Pack8 { uint32_t v[8]; };
 struct PlanePtrs { Fr* p[8]; };
-__global__ void __launch_bounds__(TPB) k_softmax_decompose(const PlanePtrs planes, uint32_t* __restrict__ flag, const Fr* __restrict__ X, const U32Pack8 bs, int K, size_t n) {
+struct IntPlanePtrs { int32_t* p[8]; };       // optional: the digits once more as int32 (a plane whose radix passes 2^31 gets none)
+__global__ void __launch_bounds__(TPB) k_softmax_decompose(const PlanePtrs planes, const IntPlanePtrs ints, uint32_t* __restrict__ flag, const Fr* __restrict__ X, const U32Pack8 bs,
+                                                           int K, size_t n) {
     const size_t g = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (g >= n) return;
     const Fr mx = neg(X[g]);
     if (mx.v[2] | mx.v[3] | mx.v[4] | mx.v[5] | mx.v[6] | mx.v[7]) {
         atomicOr(flag, 1u);
-        for (int k = 0; k < K; ++k) planes.p[k][g] = big_zero<8>();
+        for (int k = 0; k < K; ++k) {
+            planes.p[k][g] = big_zero<8>();
+            if (ints.p[k]) ints.p[k][g] = 0;
+        }
         return;
     }
     unsigned long long tmp = ((unsigned long long)mx.v[1] << 32) | mx.v[0];
     for (int k = 0; k < K; ++k) {
-        planes.p[k][g] = fr_from_u64(tmp % bs.v[k]);
+        const unsigned long long digit = tmp % bs.v[k];
+        planes.p[k][g] = fr_from_u64(digit);
+        if (ints.p[k]) ints.p[k][g] = (int32_t)digit;
         tmp /= bs.v[k];
     }
     if (tmp != 0) atomicOr(flag, 2u);   // more digits than the radices cover
@@ -1178,6 +1185,43 @@ __global__ void __launch_bounds__(256) k_ifold_rows(Fr* __restrict__ out, const 
     }
 }
 
+// out[i] = table[idx[i]] with the int32 form of the same elements beside it (table_ints: the table's own int32 form)
+__global__ void __launch_bounds__(TPB) k_gather_ints(Fr* __restrict__ out, int32_t* __restrict__ out_ints, const Fr* __restrict__ table, const int32_t* __restrict__ table_ints,
+                                                     const uint32_t* __restrict__ idx, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    const uint32_t j = idx[i];
+    out[i] = table[j];
+    out_ints[i] = table_ints[j];
+}
+// Multilinear evaluations at one point of KF (0 or 1) tensors of field elements and KI tensors given in int32 form, in one
+// pass over the point's eq table: an int32 element costs eight limb products into the lane's unreduced sum.
+struct MeIntPtrs { const int32_t* x[6]; };
+template <int KF, int KI> __global__ void __launch_bounds__(TPB) k_me_mixed(Fr* __restrict__ partials, const Fr* __restrict__ XF, const MeIntPtrs pi, const Fr* __restrict__ E, size_t n) {
+    Fr accf = big_zero<8>();
+    uint32_t acc[KI][10];
+#pragma unroll
+    for (int k = 0; k < KI; ++k)
+#pragma unroll
+        for (int i = 0; i < 10; ++i) acc[k][i] = 0;
+    const size_t stride = (size_t)gridDim.x * TPB;          // at most 2^27 / stride terms per lane: far below the 2^24 that fit
+    for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n; t += stride) {
+        const Fr e = E[t];
+        const Fr ne = neg(e);
+        int32_t x[KI];
+#pragma unroll
+        for (int k = 0; k < KI; ++k) x[k] = pi.x[k][t];
+        if constexpr (KF == 1) accf = add(accf, mont_mul(e, XF[t]));
+#pragma unroll
+        for (int k = 0; k < KI; ++k) ifold_mac(acc[k], e, ne, x[k]);
+    }
+    Fr out[KF + KI];
+    if constexpr (KF == 1) out[0] = accf;
+#pragma unroll
+    for (int k = 0; k < KI; ++k) out[KF + k] = ifold_finish(acc[k]);
+    block_reduce_store<KF + KI>(out, partials);
+}
+
 extern "C" {
 
 int zk_lookup_index_fr(void* idx_u32, const void* vals, int32_t low, uint32_t table_size, size_t n, void* stv) {
@@ -1271,6 +1315,72 @@ int zk_fr_fold_prepared_free(void* prepared) {
     if (!fp) return 0;
     pool_free(fp->ints, nullptr);
     delete fp;
+    return 0;
+}
+int zk_fr_fold_prepared_new(void** prepared, void** ints_dev, size_t n, void* stv) {
+    ZK_ARG(prepared != nullptr && ints_dev != nullptr && n >= 1, "zk_fr_fold_prepared_new: null argument or empty tensor");
+    *prepared = nullptr;
+    void* ints = nullptr;
+    int rc = pool_alloc(&ints, sizeof(int32_t) * n, (hipStream_t)stv);
+    if (rc) return rc;
+    FoldPrepared* fp = new FoldPrepared;
+    fp->ints = (int32_t*)ints;
+    fp->n = n;
+    *prepared = fp;
+    *ints_dev = ints;
+    return 0;
+}
+const void* zk_fr_fold_prepared_ints(const void* prepared) { return prepared ? ((const FoldPrepared*)prepared)->ints : nullptr; }
+int zk_fr_gather_ints(void* out, void* out_ints, const void* table, const void* table_prepared, const void* idx, size_t n, void* stv) {
+    const FoldPrepared* tp = (const FoldPrepared*)table_prepared;
+    ZK_ARG(out != nullptr && out_ints != nullptr && table != nullptr && tp != nullptr && idx != nullptr, "zk_fr_gather_ints: null argument");
+    LAUNCH1D(k_gather_ints, n, stv, (Fr*)out, (int32_t*)out_ints, (const Fr*)table, tp->ints, (const uint32_t*)idx, n);
+    return 0;
+}
+int zk_fr_me_multi_ints(uint32_t* out_host, const void* const* Xs, const void* const* prepareds, int K, size_t n, const uint32_t* u, int k, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(K >= 1 && K <= 8, "zk_fr_me_multi_ints: 1..8 tensors");
+    ZK_ARG(k >= 0 && k <= 30 && n >= 1 && n <= ((size_t)1 << k) && (k == 0 || n > ((size_t)1 << (k - 1))), "zk_fr_me_multi_ints: n does not match the number of challenges");
+    // tensors with an int32 form go through the mixed kernel, up to six at a time and one tensor of field elements with
+    // them; what is left over is evaluated as zk_fr_me_multi does
+    int ints_at[8], n_ints = 0, fr_at[8], n_fr = 0;
+    for (int i = 0; i < K; ++i) {
+        const FoldPrepared* fp = prepareds ? (const FoldPrepared*)prepareds[i] : nullptr;
+        ZK_ARG(!fp || fp->n == n, "zk_fr_me_multi_ints: an int32 form of another size");
+        if (fp && n_ints < 6) ints_at[n_ints++] = i;
+        else fr_at[n_fr++] = i;
+    }
+    if (n_ints == 0) return zk_fr_me_multi(out_host, Xs, K, n, u, k, stv);
+    Arena tmp(st);
+    Scratch& E = tmp.add(sizeof(Fr) * ((size_t)1 << k));
+    if (E.rc) return E.rc;
+    int rc = eq_table_queue(E.as<Fr>(), u, k, tmp, st);
+    if (rc) return rc;
+    const unsigned nb = reduce_grid(n);
+    const int KF = n_fr ? 1 : 0, KT = KF + n_ints;
+    Scratch& part = tmp.add(sizeof(Fr) * KT * nb);
+    if (part.rc) return part.rc;
+    MeIntPtrs pi;
+    for (int i = 0; i < 6; ++i) pi.x[i] = ((const FoldPrepared*)prepareds[ints_at[i < n_ints ? i : 0]])->ints;
+    const Fr* XF = KF ? (const Fr*)Xs[fr_at[0]] : nullptr;
+#define MEI_CASE(F, I) if (KF == F && n_ints == I) hipLaunchKernelGGL((k_me_mixed<F, I>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), XF, pi, E.as<Fr>(), n);
+    MEI_CASE(0, 1) MEI_CASE(0, 2) MEI_CASE(0, 3) MEI_CASE(0, 4) MEI_CASE(0, 5) MEI_CASE(0, 6)
+    MEI_CASE(1, 1) MEI_CASE(1, 2) MEI_CASE(1, 3) MEI_CASE(1, 4) MEI_CASE(1, 5) MEI_CASE(1, 6)
+#undef MEI_CASE
+    ZK_LAUNCH_CHECK();
+    Fr s8[8];
+    rc = finish_sums(part.as<Fr>(), nb, KT, 0, s8, st);
+    if (rc) return rc;
+    if (KF) memcpy(out_host + 8 * fr_at[0], &s8[0], sizeof(Fr));
+    for (int i = 0; i < n_ints; ++i) memcpy(out_host + 8 * ints_at[i], &s8[KF + i], sizeof(Fr));
+    if (n_fr > 1) {         // the other tensors of field elements
+        const void* rest[8];
+        for (int i = 1; i < n_fr; ++i) rest[i - 1] = Xs[fr_at[i]];
+        Fr r8[8];
+        rc = zk_fr_me_multi((uint32_t*)r8, rest, n_fr - 1, n, u, k, stv);
+        if (rc) return rc;
+        for (int i = 1; i < n_fr; ++i) memcpy(out_host + 8 * fr_at[i], &r8[i - 1], sizeof(Fr));
+    }
     return 0;
 }
 int zk_fr_fold_axis_prepared(void* out, const void* prepared, const uint32_t* u, int levels, size_t other, uint32_t cur, size_t window, void* stv) {
@@ -1923,6 +2033,9 @@ int zk_softmax_table(void* table, double log_theta, double step, uint32_t len, v
 }
 // planes: K device tensors of n elements, plane k = digit k of -X in the mixed radix bs_host[0..K)
 int zk_softmax_decompose(void* const* planes, const void* X_shifted, const uint32_t* bs_host, int K, size_t n, void* stv) {
+    return zk_softmax_decompose_ints(planes, nullptr, X_shifted, bs_host, K, n, stv);
+}
+int zk_softmax_decompose_ints(void* const* planes, void* const* int_planes, const void* X_shifted, const uint32_t* bs_host, int K, size_t n, void* stv) {
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(K >= 1 && K <= 8, "zk_softmax_decompose: K must be 1..8");
     if (n == 0) return 0;
@@ -1935,7 +2048,10 @@ int zk_softmax_decompose(void* const* planes, const void* X_shifted, const uint3
     PlanePtrs pp;
     for (int i = 0; i < 8; ++i) pp.p[i] = i < K ? (Fr*)planes[i] : nullptr;
     for (int i = 0; i < K; ++i) ZK_ARG(pp.p[i] != nullptr, "zk_softmax_decompose: null plane");
-    LAUNCH1D(k_softmax_decompose, n, st, pp, flag.as<uint32_t>(), (const Fr*)X_shifted, bs, K, n);
+    IntPlanePtrs ip;
+    for (int i = 0; i < 8; ++i) ip.p[i] = (int_planes && i < K) ? (int32_t*)int_planes[i] : nullptr;
+    for (int i = 0; i < K; ++i) ZK_ARG(!ip.p[i] || bs.v[i] <= 0x80000000u, "zk_softmax_decompose_ints: a radix above 2^31 has no int32 plane");
+    LAUNCH1D(k_softmax_decompose, n, st, pp, ip, flag.as<uint32_t>(), (const Fr*)X_shifted, bs, K, n);
     uint32_t f = 0;
     int rc = read_flag(flag.as<uint32_t>(), &f, st);
     if (rc) return rc;

@@ -220,6 +220,14 @@ void FrTensor::keep_for_folds() {
         ZKC(zk_fr_fold_prepare(&fold_cache->prepared, gpu_data, size, nullptr));
     }
 }
+void* FrTensor::ints_for_producer() {
+    if (!fold_cache) fold_cache = std::make_shared<FoldCache>();
+    fold_cache->reset();
+    void* ints = nullptr;
+    ZKC(zk_fr_fold_prepared_new(&fold_cache->prepared, &ints, size, nullptr));
+    fold_cache->tried = true;
+    return ints;
+}
 void FrTensor::drop_kept() {
     if (rhs_cache) rhs_cache->reset();
     if (fold_cache) fold_cache->reset();
@@ -318,9 +326,11 @@ vector<Fr_t> FrTensor::me_batch(const vector<const FrTensor*>& ts, const vector<
     for (auto* t : ts) if (t->size != n) throw std::runtime_error("me_batch: tensors of different sizes");
     for (size_t i0 = 0; i0 < ts.size(); i0 += 8) {
         const int K = (int)std::min<size_t>(8, ts.size() - i0);
-        const void* ptrs[8];
-        for (int i = 0; i < K; ++i) ptrs[i] = ts[i0 + i]->gpu_data;
-        ZKC(zk_fr_me_multi(out[i0].val, ptrs, K, n, u.empty() ? nullptr : u[0].val, (int)log_dim, nullptr));
+        const void *ptrs[8], *ints[8];
+        bool any = false;
+        for (int i = 0; i < K; ++i) { ptrs[i] = ts[i0 + i]->gpu_data; ints[i] = ts[i0 + i]->kept_ints(); any = any || ints[i]; }
+        if (any) ZKC(zk_fr_me_multi_ints(out[i0].val, ptrs, ints, K, n, u.empty() ? nullptr : u[0].val, (int)log_dim, nullptr));
+        else ZKC(zk_fr_me_multi(out[i0].val, ptrs, K, n, u.empty() ? nullptr : u[0].val, (int)log_dim, nullptr));
     }
     return out;
 }

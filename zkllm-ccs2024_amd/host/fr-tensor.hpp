@@ -159,6 +159,10 @@ class FrTensor {
     // what was kept.
     void keep_for_folds();
     void drop_kept();       // what keep_as_matmul_rhs and keep_for_folds hold, after the elements have changed
+    // A tensor whose int32 form is written by the kernel that writes the tensor: allocates that form (zk_fr_fold_prepared_new)
+    // and keeps it as keep_for_folds would; returns its device address for the kernel.  Call before the kernel is queued.
+    void* ints_for_producer();
+    const void* kept_ints() const { return fold_cache && fold_cache->prepared ? fold_cache->prepared : nullptr; }       // the handle, or null
     // additions for stacks of `num` equally shaped matrices stored one after the other: every M x N matrix transposed,
     // and the num products x_i (M x N) * y_i (N x P)
     FrTensor transpose_stack(uint num, uint M, uint N) const;

@@ -35,9 +35,14 @@ FrTensor tLookupRange::prep(const int* vals, const uint D) {
     ZKC(zk_lookup_index_i32(idx.p, vals, low, len, D, nullptr));
     return counts_to_m(idx.p, D, table.size);
 }
+// table positions of the values: from their int32 form when the tensor keeps one
+static void index_of(void* idx, const FrTensor& vals, int low, uint len) {
+    if (const void* h = vals.kept_ints()) ZKC(zk_lookup_index_i32(idx, zk_fr_fold_prepared_ints(h), low, len, vals.size, nullptr));
+    else ZKC(zk_lookup_index_fr(idx, vals.gpu_data, low, len, vals.size, nullptr));
+}
 FrTensor tLookupRange::prep(const FrTensor& vals) {
     DevBuf idx(sizeof(uint) * (size_t)vals.size);
-    ZKC(zk_lookup_index_fr(idx.p, vals.gpu_data, low, len, vals.size, nullptr));
+    index_of(idx.p, vals, low, len);
     return counts_to_m(idx.p, vals.size, table.size);
 }
 
@@ -48,7 +53,9 @@ static FrTensor make_mapped(uint len, const FrTensor& mvals) {
     ZKC(zk_memcpy_d2d(out.gpu_data, mvals.gpu_data, sizeof(Fr_t) * (size_t)mvals.size, nullptr));
     return out;
 }
-tLookupRangeMapping::tLookupRangeMapping(int low, uint len, const FrTensor& mvals) : tLookupRange(low, len), mapped_vals(make_mapped(len, mvals)) {}
+tLookupRangeMapping::tLookupRangeMapping(int low, uint len, const FrTensor& mvals) : tLookupRange(low, len), mapped_vals(make_mapped(len, mvals)) {
+    mapped_vals.keep_for_folds();          // examined once: outputs of operator() carry an int32 form when these are 32-bit integers
+}
 
 pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const int* vals, const uint D) {
     DevBuf idx(sizeof(uint) * (size_t)D);
@@ -61,10 +68,12 @@ pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const int* vals, const 
 }
 pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const FrTensor& vals) {
     DevBuf idx(sizeof(uint) * (size_t)vals.size);
-    ZKC(zk_lookup_index_fr(idx.p, vals.gpu_data, low, len, vals.size, nullptr));
+    index_of(idx.p, vals, low, len);
     FrTensor m = counts_to_m(idx.p, vals.size, table.size);
     FrTensor y(vals.size);
-    ZKC(zk_fr_gather(y.gpu_data, mapped_vals.gpu_data, idx.p, vals.size, nullptr));
+    // mapped values that are 32-bit integers: the outputs get their int32 form with them
+    if (const void* th = mapped_vals.kept_ints()) ZKC(zk_fr_gather_ints(y.gpu_data, y.ints_for_producer(), mapped_vals.gpu_data, th, idx.p, vals.size, nullptr));
+    else ZKC(zk_fr_gather(y.gpu_data, mapped_vals.gpu_data, idx.p, vals.size, nullptr));
     ZKC(zk_sync(nullptr));
     return {std::move(y), std::move(m)};
 }

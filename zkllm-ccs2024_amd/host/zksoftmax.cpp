@@ -55,12 +55,15 @@ FrTensor zkSoftmax::compute_rows(uint m, const FrTensor& X, FrTensor& shift, FrT
 
     const size_t N = (size_t)m * n;
     X_segments.reserve(K);
-    std::vector<void*> planes(K);
+    // every digit plane is written twice: as field elements and, an eighth of their bytes, as int32 -- the form the index
+    // pass of the lookups and the evaluations of the proof read
+    std::vector<void*> planes(K), int_planes(K, nullptr);
     for (uint i = 0; i < K; ++i) {
         X_segments.emplace_back((uint)N);
         planes[i] = X_segments[i].gpu_data;
+        if (bs[i] <= 0x80000000u) int_planes[i] = X_segments[i].ints_for_producer();
     }
-    ZKC(zk_softmax_decompose(planes.data(), X_shifted.gpu_data, bs.data(), (int)K, N, nullptr));
+    ZKC(zk_softmax_decompose_ints(planes.data(), int_planes.data(), X_shifted.gpu_data, bs.data(), (int)K, N, nullptr));
 
     for (uint i = 0; i < L; ++i) m_segments.push_back(least_significant_segments[i].prep(X_segments[i]));
     for (uint i = L; i < K; ++i) {
