@@ -285,6 +285,17 @@ int zk_lookup_prove_begin_hinted(void** handle, const void* S, const void* T, co
  * T[S_in[i] - low], T = table + r * mapped values; the combined queries are formed inside the first round instead of being written out */
 int zk_lookup_prove_begin_mapped(void** handle, const void* S_in, const void* S_out, const uint32_t* r, const void* T, const void* m, int32_t low, const uint32_t* beta,
                                  const uint32_t* u_eq, const uint32_t* v, size_t D, size_t N, int rounds, void* stream);
+/* The two jobs above for queries that keep an int32 form (handles of zk_fr_fold_prepare / zk_fr_fold_prepared_new; the
+ * tensors of field elements are given as well and serve the jobs too small for a fused first round).  _hinted_ints: the
+ * queries S are their own hints (a range table's case, tLookupRange::prove, tlookup.cu:404-412).  _mapped_ints: S_in, S_out
+ * and the table's mapped values (mapped_prepared: N integers, the padded mapped_vals of tLookupRangeMapping).  The first
+ * round reads 4 bytes per query and tensor instead of 32 and takes query and inverse from the table wherever the table entry
+ * at S_in[i] - low is what the integers say (checked per table entry on the device, so any T is safe); same results. */
+int zk_lookup_prove_begin_hinted_ints(void** handle, const void* S, const void* S_prepared, const void* T, const void* m, int32_t low, const uint32_t* beta,
+                                      const uint32_t* u_eq, const uint32_t* v, size_t D, size_t N, int rounds, void* stream);
+int zk_lookup_prove_begin_mapped_ints(void** handle, const void* S_in, const void* S_in_prepared, const void* S_out, const void* S_out_prepared, const void* mapped_prepared,
+                                      const uint32_t* r, const void* T, const void* m, int32_t low, const uint32_t* beta, const uint32_t* u_eq, const uint32_t* v, size_t D,
+                                      size_t N, int rounds, void* stream);
 int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host);
 /* hadamard_product_sumcheck (Fr_hp_sc, proof.cu:66-109): adjacent-pair folding, first challenge first.  a, b: n elements,
  * 2^(k-1) < n <= 2^k; u, v: k challenges each.  proof_host: 3k + 2 values (per round the three terms evaluated at the

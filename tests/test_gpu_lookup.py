@@ -424,6 +424,100 @@ def test_mapped_lookup_job_equals_the_plain_one_on_the_combined_queries(k):
         hip.free(p)
 
 
+@pytest.mark.parametrize("k", [13, 17, 19])
+def test_lookup_jobs_that_read_int32_forms_equal_the_plain_one(k):
+    """zk_lookup_prove_begin_mapped_ints / _hinted_ints (the first round of a large job reads the queries' int32 forms and
+    takes query and inverse from the table where the entry is what the integers say) against zk_lookup_prove_begin on the
+    combined queries computed here with big integers: inputs outside the table, outputs that are not the mapped value,
+    the extreme integers, a table entry that is NOT low + j + r * mapped[j] (its queries must not be read from it) and one
+    whose inverse does not exist.  2^13: the small-job path (the field elements serve); 2^17 / 2^19: the fused first round."""
+    import ctypes
+    from gpuhelp import Hip, c_void_p, c_size_t, c_int
+    hip = Hip()
+    D, N, low = 1 << k, 64, -9
+    rng = np.random.default_rng(1000 + k)
+    mapped = [int(x) for x in rng.integers(-2 ** 31, 2 ** 31, N)]
+    mapped[5], mapped[6] = -2 ** 31, 2 ** 31 - 1
+    r_fr, beta = ch(62, 1)[0], ch(63, 1)[0]
+    r, b = fr_ints(r_fr.reshape(1, 8))[0], fr_ints(beta.reshape(1, 8))[0]
+    pos = rng.integers(0, N, D)
+    pos[:N] = np.arange(N)                                        # every entry is queried
+    s_in = [int(p) + low for p in pos]
+    s_out = [mapped[int(p)] for p in pos]
+    odd = rng.choice(np.arange(N, D), 300, replace=False)
+    for i in odd[:100]:
+        s_out[i] = int(np.int32((s_out[i] + 1 + int(i)) & 0x7FFFFFFF))      # not the mapped value
+    for i in odd[100:200]:
+        s_in[i] = low + N + 3 + int(i)                                      # outside the table (above)
+    for i in odd[200:250]:
+        s_in[i] = low - 1 - int(i)                                          # outside the table (below)
+    s_in[int(odd[250])], s_in[int(odd[251])] = -2 ** 31, 2 ** 31 - 1
+    s_out[int(odd[252])] = -2 ** 31
+    Tl = [((low + j) + r * mapped[j]) % R_MOD for j in range(N)]
+    Tl[9] = (Tl[9] + 1) % R_MOD                                   # an entry that is something else: queries at position 9 are no entries
+    Tl[11] = (-b) % R_MOD                                         # T + beta == 0 (and not what the integers say)
+    m_counts = np.zeros(N, np.int64)
+    S_com_l = [(a + r * o) % R_MOD for a, o in zip(s_in, s_out)]
+    index_of = {}
+    for j, t in enumerate(Tl):
+        index_of.setdefault(t, j)
+    for q in S_com_l:
+        if q in index_of:
+            m_counts[index_of[q]] += 1
+    T, S_com = fr_array(Tl), fr_array(S_com_l)
+    m = fr_array([int(c) for c in m_counts])
+    u, v = ch(64, k - 1), ch(65, k)
+    Si, So, Mp = fr_array([x % R_MOD for x in s_in]), fr_array([x % R_MOD for x in s_out]), fr_array([x % R_MOD for x in mapped])
+    dS, dT, dm, dSi, dSo, dMp = hip.upload(S_com), hip.upload(T), hip.upload(m), hip.upload(Si), hip.upload(So), hip.upload(Mp)
+    hs = []
+    for dev, n in ((dSi, D), (dSo, D), (dMp, N)):
+        h = c_void_p()
+        hip.call("zk_fr_fold_prepare", ctypes.byref(h), c_void_p(dev), c_size_t(n), None)
+        assert h.value
+        hs.append(h)
+    res = []
+    for job in ("plain", "mapped_ints"):
+        h = c_void_p()
+        if job == "plain":
+            hip.call("zk_lookup_prove_begin", ctypes.byref(h), c_void_p(dS), c_void_p(dT), c_void_p(dm), beta, u, v, c_size_t(D), c_size_t(N), c_int(k), None)
+        else:
+            hip.call("zk_lookup_prove_begin_mapped_ints", ctypes.byref(h), c_void_p(dSi), hs[0], c_void_p(dSo), hs[1], hs[2], r_fr, c_void_p(dT), c_void_p(dm), c_int(low),
+                     beta, u, v, c_size_t(D), c_size_t(N), c_int(k), None)
+        bm, sums = np.zeros(8, np.uint32), np.zeros((k * 11, 8), np.uint32)
+        hip.call("zk_lookup_prove_end", h, bm, sums)
+        res.append((bm, sums))
+    assert (res[0][0] == res[1][0]).all() and (res[0][1] == res[1][1]).all()
+    assert res[0][1].any()
+    # a range table: the queries are their own hints
+    Tr = [(low + j) % R_MOD for j in range(N)]
+    Tr[13] = (Tr[13] + 5) % R_MOD                                 # not a range entry any more
+    dTr = hip.upload(fr_array(Tr))
+    index_of = {}
+    for j, t in enumerate(Tr):
+        index_of.setdefault(t, j)
+    m_counts = np.zeros(N, np.int64)
+    for q in s_in:
+        if q % R_MOD in index_of:
+            m_counts[index_of[q % R_MOD]] += 1
+    dmr = hip.upload(fr_array([int(c) for c in m_counts]))
+    res = []
+    for job in ("plain", "hinted_ints"):
+        h = c_void_p()
+        if job == "plain":
+            hip.call("zk_lookup_prove_begin", ctypes.byref(h), c_void_p(dSi), c_void_p(dTr), c_void_p(dmr), beta, u, v, c_size_t(D), c_size_t(N), c_int(k), None)
+        else:
+            hip.call("zk_lookup_prove_begin_hinted_ints", ctypes.byref(h), c_void_p(dSi), hs[0], c_void_p(dTr), c_void_p(dmr), c_int(low), beta, u, v,
+                     c_size_t(D), c_size_t(N), c_int(k), None)
+        bm, sums = np.zeros(8, np.uint32), np.zeros((k * 11, 8), np.uint32)
+        hip.call("zk_lookup_prove_end", h, bm, sums)
+        res.append((bm, sums))
+    assert (res[0][0] == res[1][0]).all() and (res[0][1] == res[1][1]).all()
+    for h in hs:
+        hip.call("zk_fr_fold_prepared_free", h)
+    for q in (dS, dT, dm, dSi, dSo, dMp, dTr, dmr):
+        hip.free(q)
+
+
 @pytest.mark.parametrize("n", [3007, 1 << 16])
 def test_int32_forms_written_with_the_tensors_serve_index_gather_and_evaluations(n):
     """zk_softmax_decompose_ints writes every digit plane as field elements and as int32 (both checked against divmod);

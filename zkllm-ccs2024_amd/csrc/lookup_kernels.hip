@@ -452,7 +452,13 @@ template <int K> __global__ void __launch_bounds__(TPB) k_me_multi(Fr* __restric
 // query, r_mont = r in Montgomery form) and is formed where it is needed.
 // TB: table entry j and its inverse side by side, TB[2j] = T[j], TB[2j+1] = 1 / (T[j] + beta): the comparison and the
 // inverse of one query come out of one 64-byte line (two gathers into separate arrays fetched two).
-struct HintSrc { const Fr* TB; const Fr* hint; Fr low; Fr beta; uint32_t N; const Fr* S_out = nullptr; Fr r_mont; };
+// hint_ints != nullptr (first round of a large job only): the queries are given by their int32 forms -- query i is
+// hint_ints[i] (+ r * sout_ints[i] for a mapping table) and is never formed: where entry j = hint_ints[i] - low of the table
+// is what these integers say (want[j], written by k_lookup_ints_check: the mapped integer of a consistent entry, 0 for a
+// consistent entry of a plain table, INTS_POISON for an entry that is something else), query and inverse are TB[2j], TB[2j+1].
+struct HintSrc { const Fr* TB; const Fr* hint; Fr low; Fr beta; uint32_t N; const Fr* S_out = nullptr; Fr r_mont;
+                 const int32_t* hint_ints = nullptr; const int32_t* sout_ints = nullptr; const int32_t* want = nullptr; int32_t low_int = 0; };
+static constexpr int32_t INTS_POISON = (int32_t)0x80000000;
 __device__ __forceinline__ Fr hinted_query(const Fr* __restrict__ S, size_t i, const HintSrc& h) {
     return h.S_out ? add(h.hint[i], mont_mul(h.r_mont, h.S_out[i])) : S[i];
 }
@@ -480,6 +486,35 @@ __device__ __forceinline__ Fr inv_by_hint(const Fr& sv, size_t i, const HintSrc&
     }
     if (unit) *unit = false;
     return inv_plus_beta_alone(sv, h.beta);
+}
+// want[j] for the int32 path of the first round: TB[2j] must be low + j (+ r * mapped[j])
+__global__ void __launch_bounds__(TPB) k_lookup_ints_check(int32_t* __restrict__ want, const Fr* __restrict__ TB, const int32_t* __restrict__ mapped_ints, const Fr r_mont,
+                                                           int32_t low, uint32_t N) {
+    const uint32_t j = blockIdx.x * TPB + threadIdx.x;
+    if (j >= N) return;
+    Fr q = fr_from_i64((int64_t)low + (int64_t)j);
+    if (mapped_ints) q = add(q, mont_mul(r_mont, fr_from_i64((int64_t)mapped_ints[j])));
+    const bool ok = equal(q, TB[2 * (size_t)j]) && (!mapped_ints || mapped_ints[j] != INTS_POISON);
+    want[j] = ok ? (mapped_ints ? mapped_ints[j] : 0) : INTS_POISON;
+}
+// query i and 1 / (query + beta) from the int32 forms (HintSrc); unit as in inv_by_hint
+__device__ __forceinline__ Fr query_inv_ints(size_t i, const HintSrc& h, Fr& a, bool& unit) {
+    const int32_t hi = h.hint_ints[i];
+    const int32_t so = h.sout_ints ? h.sout_ints[i] : 0;
+    const int64_t d = (int64_t)hi - (int64_t)h.low_int;
+    const bool in_table = d >= 0 && d < (int64_t)h.N;
+    const uint32_t j = in_table ? (uint32_t)d : 0u;
+    const int32_t w = h.want[j];
+    if (in_table && w != INTS_POISON && so == w) {
+        a = h.TB[2 * (size_t)j + 1];
+        unit = !is_zero(a);
+        return h.TB[2 * (size_t)j];
+    }
+    Fr sv = fr_from_i64((int64_t)hi);
+    if (h.sout_ints) sv = add(sv, mont_mul(h.r_mont, fr_from_i64((int64_t)so)));
+    a = inv_plus_beta_alone(sv, h.beta);
+    unit = false;
+    return sv;
 }
 __global__ void __launch_bounds__(TPB) k_interleave(Fr* __restrict__ out, const Fr* __restrict__ a, const Fr* __restrict__ b, size_t n) {
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
@@ -519,9 +554,17 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
         const Fr e = E[t];
         if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table: the top variable summed out
         {
-            const Fr s0r = HINTED ? hinted_query(S, t, hs) : S[t], s1 = HINTED ? hinted_query(S, t + n_out, hs) : S[t + n_out];
+            Fr s0r, s1, a0, a1;
             bool unit0 = false, unit1 = false;
-            const Fr a0 = HINTED ? inv_by_hint(s0r, t, hs, &unit0) : A[t], a1 = HINTED ? inv_by_hint(s1, t + n_out, hs, &unit1) : A[t + n_out];
+            if (HINTED && hs.hint_ints) {
+                s0r = query_inv_ints(t, hs, a0, unit0);
+                s1 = query_inv_ints(t + n_out, hs, a1, unit1);
+            } else {
+                s0r = HINTED ? hinted_query(S, t, hs) : S[t];
+                s1 = HINTED ? hinted_query(S, t + n_out, hs) : S[t + n_out];
+                a0 = HINTED ? inv_by_hint(s0r, t, hs, &unit0) : A[t];
+                a1 = HINTED ? inv_by_hint(s1, t + n_out, hs, &unit1) : A[t + n_out];
+            }
             const Fr da = sub(a1, a0), ds = sub(s1, s0r), s0 = add(s0r, beta);
             if (HINTED && unit0 && unit1) {
                 const Fr M = mont_mul(add(a0, a1), add(s0, add(s1, beta)));
@@ -1630,7 +1673,9 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
                 g_round_timer.pairs += half;
                 // per pair: two queries (32 B each; a mapping table's query is two tensors), the eq weight (32 B), two folded values
                 // written (64 B), the next round's eq table (16 B)
-                g_round_timer.bytes += (double)half * ((hs->S_out ? 128.0 : 64.0) + 32.0 + 64.0 + (nE ? 16.0 : 0.0));
+                // (queries read from their int32 forms: 4 B each)
+                const double q = hs->hint_ints ? (hs->sout_ints ? 16.0 : 8.0) : (hs->S_out ? 128.0 : 64.0);
+                g_round_timer.bytes += (double)half * (q + 32.0 + 64.0 + (nE ? 16.0 : 0.0));
             }
         }
         else
@@ -1826,11 +1871,19 @@ int zk_lookup_sumcheck(uint32_t* sums_host, const void* A, const void* S, const 
 // B = 1/(T + beta), <B, m>, the eq table of u_eq (rounds - 1 challenges), then every round.  S: D elements; T, m: N.
 // begin returns at once; S, T, m must stay alive and unmodified until end, which waits and delivers <B, m>
 // (standard form) and the rounds x 11 sums.  Every handle must be ended exactly once.
+// int32 forms (handles of zk_fr_fold_prepare / _new) of the hinted queries, of a mapping table's outputs and of its mapped values
+struct LookupInts { const void* queries = nullptr; const void* out = nullptr; const void* mapped = nullptr; };
 static int lookup_prove_begin(void** handle, const void* S, const void* T, const void* m, const void* hint, int32_t low, const uint32_t* beta, const uint32_t* u_eq,
-                              const uint32_t* v, size_t D, size_t N, int rounds, void* stv, const void* S_out = nullptr, const uint32_t* r = nullptr) {
+                              const uint32_t* v, size_t D, size_t N, int rounds, void* stv, const void* S_out = nullptr, const uint32_t* r = nullptr,
+                              const LookupInts* ints = nullptr) {
     ZK_ARG(handle != nullptr, "zk_lookup_prove_begin: null handle");
     int rc = lookup_args_ok(D, N, rounds);
     if (rc) return rc;
+    if (ints) {
+        const FoldPrepared *q = (const FoldPrepared*)ints->queries, *o = (const FoldPrepared*)ints->out, *mp = (const FoldPrepared*)ints->mapped;
+        ZK_ARG(q != nullptr && q->n == D, "lookup sumcheck: the queries' int32 form has another size");
+        ZK_ARG(!S_out || (o != nullptr && o->n == D && mp != nullptr && mp->n == N), "lookup sumcheck: a mapping table's int32 forms are missing or of another size");
+    }
     SumJob* job = new SumJob;
     rc = sumjob_on_side_stream(*job, (hipStream_t)stv);
     if (rc) { sumjob_abort(job); return rc; }
@@ -1848,6 +1901,16 @@ static int lookup_prove_begin(void** handle, const void* S, const void* T, const
         hipLaunchKernelGGL(k_interleave, dim3(cdiv(N, TPB)), dim3(TPB), 0, st, TB.as<Fr>(), (const Fr*)T, B.as<Fr>(), N);
         hs.TB = TB.as<Fr>(); hs.hint = (const Fr*)hint; hs.low = fr_from_i64((int64_t)low); hs.beta = b; hs.N = (uint32_t)N;
         if (S_out) { hs.S_out = (const Fr*)S_out; hs.r_mont = to_mont(load_fr(r)); }
+        if (ints) {
+            Scratch& want = job->arena.add(sizeof(int32_t) * N);
+            if (want.rc) { rc = want.rc; sumjob_abort(job); return rc; }
+            const int32_t* mi = S_out ? ((const FoldPrepared*)ints->mapped)->ints : nullptr;
+            hipLaunchKernelGGL(k_lookup_ints_check, dim3(cdiv(N, TPB)), dim3(TPB), 0, st, want.as<int32_t>(), TB.as<Fr>(), mi, hs.r_mont, low, (uint32_t)N);
+            hs.hint_ints = ((const FoldPrepared*)ints->queries)->ints;
+            hs.sout_ints = S_out ? ((const FoldPrepared*)ints->out)->ints : nullptr;
+            hs.want = want.as<int32_t>();
+            hs.low_int = low;
+        }
     } else if (rc == 0) {
         Scratch& A = job->arena.add(sizeof(Fr) * D);
         rc = A.rc;
@@ -1886,6 +1949,22 @@ int zk_lookup_prove_begin_mapped(void** handle, const void* S_in, const void* S_
                                  const uint32_t* u_eq, const uint32_t* v, size_t D, size_t N, int rounds, void* stv) {
     ZK_ARG(S_in != nullptr && S_out != nullptr && r != nullptr, "zk_lookup_prove_begin_mapped: null queries or challenge");
     return lookup_prove_begin(handle, nullptr, T, m, S_in, low, beta, u_eq, v, D, N, rounds, stv, S_out, r);
+}
+int zk_lookup_prove_begin_hinted_ints(void** handle, const void* S, const void* S_prepared, const void* T, const void* m, int32_t low, const uint32_t* beta,
+                                      const uint32_t* u_eq, const uint32_t* v, size_t D, size_t N, int rounds, void* stv) {
+    ZK_ARG(S != nullptr && S_prepared != nullptr, "zk_lookup_prove_begin_hinted_ints: null queries");
+    LookupInts li;
+    li.queries = S_prepared;
+    return lookup_prove_begin(handle, S, T, m, S, low, beta, u_eq, v, D, N, rounds, stv, nullptr, nullptr, &li);
+}
+int zk_lookup_prove_begin_mapped_ints(void** handle, const void* S_in, const void* S_in_prepared, const void* S_out, const void* S_out_prepared, const void* mapped_prepared,
+                                      const uint32_t* r, const void* T, const void* m, int32_t low, const uint32_t* beta, const uint32_t* u_eq, const uint32_t* v, size_t D,
+                                      size_t N, int rounds, void* stv) {
+    ZK_ARG(S_in != nullptr && S_out != nullptr && r != nullptr, "zk_lookup_prove_begin_mapped_ints: null queries or challenge");
+    ZK_ARG(S_in_prepared != nullptr && S_out_prepared != nullptr && mapped_prepared != nullptr, "zk_lookup_prove_begin_mapped_ints: null int32 form");
+    LookupInts li;
+    li.queries = S_in_prepared; li.out = S_out_prepared; li.mapped = mapped_prepared;
+    return lookup_prove_begin(handle, nullptr, T, m, S_in, low, beta, u_eq, v, D, N, rounds, stv, S_out, r, &li);
 }
 int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host) {
     ZK_ARG(handle != nullptr, "zk_lookup_prove_end: null handle");

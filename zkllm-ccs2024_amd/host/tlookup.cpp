@@ -102,13 +102,14 @@ LookupPending& LookupPending::operator=(LookupPending&& o) noexcept {
 // derives the next claim.
 // S_out / r given: S0 holds the input queries of a mapping table, the combined query S0 + r * S_out is formed on the device
 static LookupPending sumcheck_begin(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0, const Fr_t& alpha0, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v,
-                                    const FrTensor* hint, int low, const FrTensor* S_out, const Fr_t* r);
+                                    const FrTensor* hint, int low, const FrTensor* S_out, const Fr_t* r, const void* mapped_ints = nullptr);
 LookupPending tLookup_sumcheck_begin(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0, const Fr_t& alpha0, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v,
                                      const FrTensor* hint, int low) {
     return sumcheck_begin(S0, T0, m0, alpha0, beta, u, v, hint, low, nullptr, nullptr);
 }
+// mapped_ints: the int32 form of the mapping table's (padded) mapped values, when it keeps one
 static LookupPending sumcheck_begin(const FrTensor& S0, const FrTensor& T0, const FrTensor& m0, const Fr_t& alpha0, const Fr_t& beta, const vector<Fr_t>& u, const vector<Fr_t>& v,
-                                    const FrTensor* hint, int low, const FrTensor* S_out, const Fr_t* r) {
+                                    const FrTensor* hint, int low, const FrTensor* S_out, const Fr_t* r, const void* mapped_ints) {
     const uint D = S0.size, N = m0.size;
     if (S_out && S_out->size != D) throw std::runtime_error("lookup: input and output queries differ in size");
     if (m0.size != T0.size) throw std::runtime_error("m.size != table.size");
@@ -124,7 +125,14 @@ static LookupPending sumcheck_begin(const FrTensor& S0, const FrTensor& T0, cons
     std::vector<Fr_t> vs(k);
     for (uint r = 0; r < k; ++r) vs[r] = r >= n1 ? v[k - 1 - (r - n1)] : v[n1 - 1 - r];
     if (hint && hint->size != D) throw std::runtime_error("lookup hint must have one entry per query");
-    if (S_out) ZKC(zk_lookup_prove_begin_mapped(&p.handle, S0.gpu_data, S_out->gpu_data, r->val, T0.gpu_data, m0.gpu_data, low, beta.val, u[0].val, vs[0].val, D, N, (int)k, nullptr));
+    // queries that keep an int32 form (the digit planes of a softmax, the outputs of a mapping table) are read from it
+    const void *qi = S0.kept_ints(), *oi = S_out ? S_out->kept_ints() : nullptr;
+    if (S_out && qi && oi && mapped_ints)
+        ZKC(zk_lookup_prove_begin_mapped_ints(&p.handle, S0.gpu_data, qi, S_out->gpu_data, oi, mapped_ints, r->val, T0.gpu_data, m0.gpu_data, low, beta.val, u[0].val, vs[0].val,
+                                              D, N, (int)k, nullptr));
+    else if (S_out) ZKC(zk_lookup_prove_begin_mapped(&p.handle, S0.gpu_data, S_out->gpu_data, r->val, T0.gpu_data, m0.gpu_data, low, beta.val, u[0].val, vs[0].val, D, N, (int)k, nullptr));
+    else if (hint == &S0 && qi)
+        ZKC(zk_lookup_prove_begin_hinted_ints(&p.handle, S0.gpu_data, qi, T0.gpu_data, m0.gpu_data, low, beta.val, u[0].val, vs[0].val, D, N, (int)k, nullptr));
     else if (hint) ZKC(zk_lookup_prove_begin_hinted(&p.handle, S0.gpu_data, T0.gpu_data, m0.gpu_data, hint->gpu_data, low, beta.val, u[0].val, vs[0].val, D, N, (int)k, nullptr));
     else ZKC(zk_lookup_prove_begin(&p.handle, S0.gpu_data, T0.gpu_data, m0.gpu_data, beta.val, u[0].val, vs[0].val, D, N, (int)k, nullptr));
     return p;
@@ -219,7 +227,7 @@ LookupPending tLookupRangeMapping::prove_begin(const FrTensor& S_in, const FrTen
     // S_com = S_in + r * S_out (tlookup.cu:517) is formed by the job itself; T_com is small
     keep.emplace_back(new FrTensor(table + mapped_vals * r));
     const FrTensor* T_com = keep.back().get();
-    LookupPending p = sumcheck_begin(*si, *T_com, *mm, alpha, beta, u, v, si, low, so, &r);
+    LookupPending p = sumcheck_begin(*si, *T_com, *mm, alpha, beta, u, v, si, low, so, &r, mapped_vals.kept_ints());
     p.keep = std::move(keep);
     return p;
 }
