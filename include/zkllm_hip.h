@@ -302,6 +302,9 @@ int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host);
  * remaining u, then the folded a and b).  The three term tensors of the reference's step kernel are never materialised. */
 int zk_hadamard_product_sumcheck(uint32_t* proof_host, const void* a, const void* b, const uint32_t* u, const uint32_t* v, size_t n, int k, void* stream);
 int zk_hadamard_prove_begin(void** handle, const void* const* Xs, int K, const uint32_t* u_eq, const uint32_t* v, size_t N, void* stream);
+/* the same where prepareds[i], when non-null, is the int32 form of Xs[i] (N elements): two tensors that both have one (the
+ * mapped outputs of a softmax's segments, zksoftmax.cu:177-180) are read from it in the first round; same sums */
+int zk_hadamard_prove_begin_ints(void** handle, const void* const* Xs, const void* const* prepareds, int K, const uint32_t* u_eq, const uint32_t* v, size_t N, void* stream);
 int zk_hadamard_prove_end(void* handle, uint32_t* coefs_host);
 
 /* ---- rescaling / softmax ------------------------------------------------------------------------------------------ */

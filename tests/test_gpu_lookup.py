@@ -208,6 +208,37 @@ def test_multi_hadamard(pv, orc, nX, n):
     assert (proof == e_proof).all() and (fin == e_fin).all()
 
 
+@pytest.mark.parametrize("n,kept", [(4096, (True, True)), (1 << 17, (True, True)), (1 << 17, (True, False)), (1 << 15, (False, True))])
+def test_multi_hadamard_of_two_tensors_that_keep_an_int32_form(pv, orc, n, kept):
+    """Two tensors of 32-bit integers, the extremes included, kept for folds: the job's first round reads their int32 forms
+    (k_hadamard_round2_ints: exact 64-bit products weighted into unreduced twelve-limb sums) and the proof is the oracle's;
+    with only one of them kept the plain round runs."""
+    rng = np.random.default_rng(n + 7 * kept[0] + 3 * kept[1])
+    Ws = [rng.integers(-2 ** 31, 2 ** 31, n).astype(np.int64) for _ in range(2)]
+    half = n // 2
+    for W in Ws:
+        W[0], W[half] = -2 ** 31, 2 ** 31 - 1                  # the widest difference of a pair, both signs
+        W[1], W[1 + half] = 2 ** 31 - 1, -2 ** 31
+        W[2], W[2 + half] = -2 ** 31, -2 ** 31
+        W[3] = 0
+    Xs = [fr_array([int(v) % R_MOD for v in W]) for W in Ws]
+    k = (n - 1).bit_length()
+    u, v = ch(32, k), ch(33, k)
+    prod = np.zeros_like(Xs[0])
+    orc_check(orc.orc_fr_op(7, Xs[0], Xs[1], prod, n))
+    claim = np.zeros(8, np.uint32)
+    orc_check(orc.orc_fr_me(prod, n, u, k, claim))
+    e_proof, e_fin = np.zeros((k * 3, 8), np.uint32), np.zeros(8, np.uint32)
+    orc_check(orc.orc_multi_hadamard(claim, np.ascontiguousarray(np.concatenate(Xs)), 2, n, u, v, k, e_proof, e_fin))
+    hs = [pv.from_i64(W) for W in Ws]
+    for h, kp in zip(hs, kept):
+        if kp:
+            pv.keep_for_folds(h)
+            assert pv.folds_from_ints(h) == 1
+    proof, fin = pv.multi_hadamard(claim, hs, u, v)
+    assert (proof == e_proof).all() and (fin == e_fin).all()
+
+
 # 70001: several workgroups per round and odd lengths on the way down (70001, 35001, 17501, 8751, 4376, ...)
 @pytest.mark.parametrize("n", [2, 3, 5, 64, 1000, 70001])
 def test_deprecated_hadamard_product_sumcheck(pv, orc, n):

@@ -726,6 +726,79 @@ k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __rest
     block_reduce_store<K + 1>(acc, partials);
 }
 
+// The first round for two tensors given by their int32 forms (the mapped outputs of a softmax's segments): 4 bytes per
+// element instead of 32, and the three weighted coefficients are E times an exact 64-bit integer (x0 y0, dx dy, x1 y1) --
+// sixteen limb products into an unreduced twelve-limb sum each, one reduction per lane -- instead of Montgomery products.
+// The sums come out as k_hadamard_round<2> leaves them (standard form, no factor of R).
+__device__ __forceinline__ void imac64(uint32_t (&acc)[12], const Fr& e, const Fr& ne, int64_t a, int64_t b) {
+    const uint64_t ma = a < 0 ? 0ull - (uint64_t)a : (uint64_t)a, mb = b < 0 ? 0ull - (uint64_t)b : (uint64_t)b;      // both below 2^32
+    const uint64_t mag = ma * mb;
+    const bool ng = (a < 0) != (b < 0);
+    const uint32_t m0 = (uint32_t)mag, m1 = (uint32_t)(mag >> 32);
+    uint32_t s[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s[i] = ng ? ne.v[i] : e.v[i];
+    uint64_t carry = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint64_t t = (uint64_t)s[i] * m0 + acc[i] + carry;
+        acc[i] = (uint32_t)t;
+        carry = t >> 32;
+    }
+#pragma unroll
+    for (int i = 8; i < 12; ++i) {
+        const uint64_t t = (uint64_t)acc[i] + carry;
+        acc[i] = (uint32_t)t;
+        carry = t >> 32;
+    }
+    carry = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint64_t t = (uint64_t)s[i] * m1 + acc[i + 1] + carry;
+        acc[i + 1] = (uint32_t)t;
+        carry = t >> 32;
+    }
+#pragma unroll
+    for (int i = 9; i < 12; ++i) {
+        const uint64_t t = (uint64_t)acc[i] + carry;
+        acc[i] = (uint32_t)t;
+        carry = t >> 32;
+    }
+}
+__device__ __forceinline__ Fr imac64_finish(const uint32_t (&acc)[12]) {
+    Fr lo, hi = big_zero<8>(), one = big_zero<8>();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) lo.v[i] = acc[i];
+    lo = reduce_once(reduce_once(lo));
+    one.v[0] = 1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) hi.v[i] = acc[8 + i];
+    return add(mont_mul(lo, one), hi);
+}
+__global__ void __launch_bounds__(TPB) k_hadamard_round2_ints(Fr* __restrict__ partials, const int32_t* __restrict__ X, const int32_t* __restrict__ Y, Fr* __restrict__ outx,
+                                                              Fr* __restrict__ outy, const Fr* __restrict__ E, const Fr v_mont, size_t n_out, Fr* __restrict__ nE) {
+    uint32_t a0[12], a2[12], ax[12];
+#pragma unroll
+    for (int i = 0; i < 12; ++i) a0[i] = a2[i] = ax[i] = 0;
+    for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
+        const int64_t x0 = X[t], x1 = X[t + n_out], y0 = Y[t], y1 = Y[t + n_out];
+        const int64_t dx = x1 - x0, dy = y1 - y0;
+        outx[t] = add(fr_from_i64(x0), mont_mul(v_mont, fr_from_i64(dx)));
+        outy[t] = add(fr_from_i64(y0), mont_mul(v_mont, fr_from_i64(dy)));
+        const Fr e = E[t];
+        const Fr ne = neg(e);
+        if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);
+        imac64(a0, e, ne, x0, y0);
+        imac64(a2, e, ne, dx, dy);
+        imac64(ax, e, ne, x1, y1);
+    }
+    Fr acc[3];
+    acc[0] = imac64_finish(a0);
+    acc[2] = imac64_finish(a2);
+    acc[1] = sub(sub(imac64_finish(ax), acc[0]), acc[2]);
+    block_reduce_store<3>(acc, partials);
+}
+
 // ---- the last rounds of a sumcheck in one launch ---------------------------------------------------------------------------------
 // Once the tensors are short, a round is a few microseconds of arithmetic between two host round trips.  The
 // challenges of these sumchecks are fixed before the first round (tLookup::prove and multi_hadamard_sumchecks take u and
@@ -1690,7 +1763,7 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
     }
     return 0;
 }
-static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, const uint32_t* v, size_t N) {
+static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, const uint32_t* v, size_t N, const int32_t* const* ints = nullptr) {
     hipStream_t st = job.st;
     int rounds = 0;
     while (((size_t)1 << rounds) < N) ++rounds;
@@ -1751,7 +1824,10 @@ static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, 
         hipLaunchKernelGGL(k_hadamard_round<KK>, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), p, cE, vm, half, nE);                  \
         break;                                                                                                                    \
     }
-        switch (K) { HADS_ROUND(1) HADS_ROUND(2) HADS_ROUND(3) HADS_ROUND(4) }
+        if (r == 0 && K == 2 && ints && ints[0] && ints[1])
+            hipLaunchKernelGGL(k_hadamard_round2_ints, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), ints[0], ints[1], w, w + half, cE, vm, half, nE);
+        else
+            switch (K) { HADS_ROUND(1) HADS_ROUND(2) HADS_ROUND(3) HADS_ROUND(4) }
 #undef HADS_ROUND
         hipLaunchKernelGGL(k_finish, dim3(K + 1), dim3(TPB), 0, st, sums.as<Fr>() + (size_t)r * (K + 1), part.as<Fr>(), nb);
         ZK_LAUNCH_CHECK();
@@ -2024,7 +2100,17 @@ int zk_hadamard_sumcheck(uint32_t* coefs_host, const void* const* Xs, int K, con
 // The same beside the caller's stream, eq table of u_eq (log2(N) - 1 challenges) included.  Xs must stay alive and
 // unmodified until end; every handle must be ended exactly once.
 int zk_hadamard_prove_begin(void** handle, const void* const* Xs, int K, const uint32_t* u_eq, const uint32_t* v, size_t N, void* stv) {
+    return zk_hadamard_prove_begin_ints(handle, Xs, nullptr, K, u_eq, v, N, stv);
+}
+int zk_hadamard_prove_begin_ints(void** handle, const void* const* Xs, const void* const* prepareds, int K, const uint32_t* u_eq, const uint32_t* v, size_t N, void* stv) {
     ZK_ARG(handle != nullptr, "zk_hadamard_prove_begin: null handle");
+    const int32_t* ints[4] = {nullptr, nullptr, nullptr, nullptr};
+    if (prepareds)
+        for (int i = 0; i < K && i < 4; ++i)
+            if (const FoldPrepared* fp = (const FoldPrepared*)prepareds[i]) {
+                ZK_ARG(fp->n == N, "zk_hadamard_prove_begin_ints: an int32 form of another size");
+                ints[i] = fp->ints;
+            }
     ZK_ARG(K >= 1 && K <= 4, "zk_hadamard_prove_begin: K must be 1..4");
     ZK_ARG(N >= 2 && (N & (N - 1)) == 0, "zk_hadamard_prove_begin: N must be a power of two >= 2");
     SumJob* job = new SumJob;
@@ -2034,7 +2120,7 @@ int zk_hadamard_prove_begin(void** handle, const void* const* Xs, int K, const u
     while (((size_t)1 << k) < N) ++k;
     rc = shared_eq_get(job->eq, u_eq, k - 1, job->arena, job->st);
     if (rc) { sumjob_abort(job); return rc; }
-    rc = hadamard_queue(*job, (const Fr* const*)Xs, K, (const Fr*)job->eq->p, v, N);
+    rc = hadamard_queue(*job, (const Fr* const*)Xs, K, (const Fr*)job->eq->p, v, N, prepareds ? ints : nullptr);
     if (rc == 0) rc = sumjob_queue_results(*job);
     if (rc) { sumjob_abort(job); return rc; }
     *handle = job;

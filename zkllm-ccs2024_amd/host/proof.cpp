@@ -233,7 +233,11 @@ HadamardPending multi_hadamard_begin(const Fr_t& claim0, const vector<FrTensor>&
     for (uint i = 0; i < p.K; ++i) cur[i] = Xs[i].gpu_data;
     std::vector<Fr_t> vs(k);
     for (uint r = 0; r < k; ++r) vs[r] = v[k - 1 - r];
-    ZKC(zk_hadamard_prove_begin(&p.handle, cur.data(), (int)p.K, u[0].val, vs[0].val, N, nullptr));
+    std::vector<const void*> ints(p.K);
+    bool any = false;
+    for (uint i = 0; i < p.K; ++i) { ints[i] = Xs[i].kept_ints(); any = any || ints[i]; }
+    if (any) ZKC(zk_hadamard_prove_begin_ints(&p.handle, cur.data(), ints.data(), (int)p.K, u[0].val, vs[0].val, N, nullptr));
+    else ZKC(zk_hadamard_prove_begin(&p.handle, cur.data(), (int)p.K, u[0].val, vs[0].val, N, nullptr));
     return p;
 }
 Fr_t multi_hadamard_end(HadamardPending& pd, vector<Polynomial>& proof) {
