@@ -128,6 +128,9 @@ const void* zk_fr_fold_prepared_ints(const void* prepared);
 int zk_fr_gather_ints(void* out, void* out_ints, const void* table, const void* table_prepared, const void* idx, size_t n, void* stream);
 /* zk_fr_me_multi where prepareds[i], when non-null, is the int32 form of Xs[i] (same n): such tensors are read from it --
  * an eighth of the bytes, eight limb products per element instead of a Montgomery product.  Same values. */
+/* zk_fr_mul (out = a * b element by element) for two tensors given by their int32 forms: the products are exact 64-bit
+ * integers, no field multiplication and an eighth of the bytes read */
+int zk_fr_mul_ints(void* out, const void* a_prepared, const void* b_prepared, size_t n, void* stream);
 int zk_fr_me_multi_ints(uint32_t* out_host, const void* const* Xs, const void* const* prepareds, int K, size_t n, const uint32_t* u, int k, void* stream);
 /* FrTensor::operator()(u) / Fr_me (fr-tensor.cu:437-442, :602-609): whole evaluation, fused */
 int zk_fr_me(uint32_t* out_host, const void* a, size_t n, const uint32_t* u, int k, void* stream);

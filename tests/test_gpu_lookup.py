@@ -604,6 +604,27 @@ def test_int32_forms_written_with_the_tensors_serve_index_gather_and_evaluations
     got_fr = hip.download(dG, (n, 8), np.uint32)
     got_i = hip.download(gq.value, (n,), np.int32)
     assert (got_i == tab_i[idx]).all() and (got_fr[:, 0] == tab_i[idx]).all() and not got_fr[:, 1:].any()
+    # the product of two tensors from their int32 forms (negative factors through a table of signed integers)
+    sg_i = rng.integers(-2 ** 31, 2 ** 31, 256).astype(np.int64)
+    sg_i[0], sg_i[1] = -2 ** 31, 2 ** 31 - 1
+    dT2 = hip.upload(fr_array([int(v) % R_MOD for v in sg_i]))
+    th2 = c_void_p()
+    hip.call("zk_fr_fold_prepare", ctypes.byref(th2), c_void_p(dT2), c_size_t(256), None)
+    dG2 = hip.malloc(32 * n)
+    g2h, g2q = c_void_p(), c_void_p()
+    hip.call("zk_fr_fold_prepared_new", ctypes.byref(g2h), ctypes.byref(g2q), c_size_t(n), None)
+    hip.call("zk_fr_gather_ints", c_void_p(dG2), g2q, c_void_p(dT2), th2, c_void_p(dI), c_size_t(n), None)
+    dP = hip.malloc(32 * n)
+    hip.call("zk_fr_mul_ints", c_void_p(dP), g2h, g2h, c_size_t(n), None)
+    sq = fr_ints(hip.download(dP, (n, 8), np.uint32))
+    assert sq == [int(v) * int(v) % R_MOD for v in sg_i[idx]]
+    hip.call("zk_fr_mul_ints", c_void_p(dP), g2h, gh, c_size_t(n), None)
+    pr = fr_ints(hip.download(dP, (n, 8), np.uint32))
+    assert pr == [int(a) * int(b) % R_MOD for a, b in zip(sg_i[idx], tab_i[idx])]
+    for h in (th2, g2h):
+        hip.call("zk_fr_fold_prepared_free", h)
+    for q in (dT2, dG2, dP):
+        hip.free(q)
     # evaluations: int32 forms where there are some, full residues elsewhere
     k = (n - 1).bit_length()
     u = ch(71, k)

@@ -1310,6 +1310,11 @@ __global__ void __launch_bounds__(TPB) k_gather_ints(Fr* __restrict__ out, int32
     out[i] = table[j];
     out_ints[i] = table_ints[j];
 }
+// out[i] = a[i] * b[i] for two tensors given by their int32 forms: the product is an exact 64-bit integer
+__global__ void __launch_bounds__(TPB) k_mul_ints(Fr* __restrict__ out, const int32_t* __restrict__ a, const int32_t* __restrict__ b, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) out[i] = fr_from_i64((int64_t)a[i] * (int64_t)b[i]);
+}
 // Multilinear evaluations at one point of KF (0 or 1) tensors of field elements and KI tensors given in int32 form, in one
 // pass over the point's eq table: an int32 element costs eight limb products into the lane's unreduced sum.
 struct MeIntPtrs { const int32_t* x[6]; };
@@ -1451,6 +1456,12 @@ int zk_fr_gather_ints(void* out, void* out_ints, const void* table, const void* 
     const FoldPrepared* tp = (const FoldPrepared*)table_prepared;
     ZK_ARG(out != nullptr && out_ints != nullptr && table != nullptr && tp != nullptr && idx != nullptr, "zk_fr_gather_ints: null argument");
     LAUNCH1D(k_gather_ints, n, stv, (Fr*)out, (int32_t*)out_ints, (const Fr*)table, tp->ints, (const uint32_t*)idx, n);
+    return 0;
+}
+int zk_fr_mul_ints(void* out, const void* a_prepared, const void* b_prepared, size_t n, void* stv) {
+    const FoldPrepared *a = (const FoldPrepared*)a_prepared, *b = (const FoldPrepared*)b_prepared;
+    ZK_ARG(out != nullptr && a != nullptr && b != nullptr && a->n == n && b->n == n, "zk_fr_mul_ints: null argument or int32 forms of another size");
+    LAUNCH1D(k_mul_ints, n, stv, (Fr*)out, a->ints, b->ints, n);
     return 0;
 }
 int zk_fr_me_multi_ints(uint32_t* out_host, const void* const* Xs, const void* const* prepareds, int K, size_t n, const uint32_t* u, int k, void* stv) {

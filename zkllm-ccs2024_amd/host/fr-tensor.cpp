@@ -292,7 +292,13 @@ FrTensor& FrTensor::operator-=(const FrTensor& t) { SAME_SIZE(t); drop_kept(); Z
 FrTensor& FrTensor::operator-=(const Fr_t& x) { drop_kept(); ZKC(zk_fr_sub_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }
 FrTensor& FrTensor::mont() { drop_kept(); ZKC(zk_fr_mont(gpu_data, gpu_data, size, nullptr)); return *this; }
 FrTensor& FrTensor::unmont() { drop_kept(); ZKC(zk_fr_unmont(gpu_data, gpu_data, size, nullptr)); return *this; }
-FrTensor FrTensor::operator*(const FrTensor& t) const { SAME_SIZE(t); FrTensor out(size); ZKC(zk_fr_mul(out.gpu_data, gpu_data, t.gpu_data, size, nullptr)); return out; }
+FrTensor FrTensor::operator*(const FrTensor& t) const {
+    SAME_SIZE(t);
+    FrTensor out(size);
+    if (kept_ints() && t.kept_ints()) ZKC(zk_fr_mul_ints(out.gpu_data, kept_ints(), t.kept_ints(), size, nullptr));      // exact 64-bit products
+    else ZKC(zk_fr_mul(out.gpu_data, gpu_data, t.gpu_data, size, nullptr));
+    return out;
+}
 FrTensor FrTensor::operator*(const Fr_t& x) const { FrTensor out(size); ZKC(zk_fr_mul_s(out.gpu_data, gpu_data, x.val, size, nullptr)); return out; }
 FrTensor& FrTensor::operator*=(const FrTensor& t) { SAME_SIZE(t); drop_kept(); ZKC(zk_fr_mul(gpu_data, gpu_data, t.gpu_data, size, nullptr)); return *this; }
 FrTensor& FrTensor::operator*=(const Fr_t& x) { drop_kept(); ZKC(zk_fr_mul_s(gpu_data, gpu_data, x.val, size, nullptr)); return *this; }

@@ -40,6 +40,11 @@ zkSoftmax::zkSoftmax(const vector<uint>& bs, uint L, uint M, unsigned long scali
     }
 }
 
+// the product of two segments' table values: from their int32 forms (exact 64-bit products) when both keep one
+static void mul_segments(Fr_t* out, const FrTensor& a, const FrTensor& b, size_t N) {
+    if (a.kept_ints() && b.kept_ints()) ZKC(zk_fr_mul_ints(out, a.kept_ints(), b.kept_ints(), N, nullptr));
+    else ZKC(zk_fr_mul(out, a.gpu_data, b.gpu_data, N, nullptr));
+}
 // zksoftmax.cu:112-173
 FrTensor zkSoftmax::compute(const FrTensor& X, FrTensor& shift, FrTensor& X_shifted, vector<FrTensor>& X_segments, vector<FrTensor>& Y_segments, vector<FrTensor>& m_segments) {
     return compute_rows(m, X, shift, X_shifted, X_segments, Y_segments, m_segments);
@@ -75,12 +80,13 @@ FrTensor zkSoftmax::compute_rows(uint m, const FrTensor& X, FrTensor& shift, FrT
     if (into) {
         if (into->size != X.size) throw std::invalid_argument("the result must be the same size as X");
         if (Y_segments.size() == 1) { *into = Y_segments[0]; return FrTensor(0); }
-        ZKC(zk_fr_mul(into->gpu_data, Y_segments[0].gpu_data, Y_segments[1].gpu_data, N, nullptr));
+        mul_segments(into->gpu_data, Y_segments[0], Y_segments[1], N);
         for (size_t i = 2; i < Y_segments.size(); ++i) *into *= Y_segments[i];
         return FrTensor(0);
     }
     if (Y_segments.size() == 1) return FrTensor(Y_segments[0]);
-    FrTensor out = Y_segments[0] * Y_segments[1];
+    FrTensor out((uint)N);
+    mul_segments(out.gpu_data, Y_segments[0], Y_segments[1], N);
     for (size_t i = 2; i < Y_segments.size(); ++i) out *= Y_segments[i];
     return out;
 }
