@@ -632,6 +632,7 @@ def test_int32_forms_written_with_the_tensors_serve_index_gather_and_evaluations
     dR1, dR2 = hip.upload(R1), hip.upload(R2)
     for Xs, hs in [([planes[0], planes[1], dR1, planes[2], dG, planes[0]], [handles[0], handles[1], None, handles[2], gh, handles[0]]),
                    ([dR1, planes[0], planes[1], planes[2], dG, planes[1], planes[2], dR2], [None, handles[0], handles[1], handles[2], gh, handles[1], handles[2], None]),
+                   ([dR1, planes[0], dR2, planes[1]], [None, handles[0], None, handles[1]]), ([dR2, dR1, dG], [None, None, gh]),
                    ([planes[1]], [handles[1]]), ([dR1, dR2], [None, None])]:
         K = len(Xs)
         xa = (c_void_p * K)(*[c_void_p(x) for x in Xs])

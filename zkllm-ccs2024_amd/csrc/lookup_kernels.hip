@@ -1026,7 +1026,8 @@ k_hadamard_tail(Fr* __restrict__ sums, const PtrPack<K> p, Fr* wE, const Fr* E, 
 }
 
 // ---- rescaling (rescaling.cu:8-21) ----------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(TPB) k_rescale(Fr* __restrict__ out, Fr* __restrict__ rem, const Fr* __restrict__ in, int64_t sf, size_t n) {
+// rem_ints (optional): the remainders once more as int32 (they lie in [-sf/2, sf/2))
+__global__ void __launch_bounds__(TPB) k_rescale(Fr* __restrict__ out, Fr* __restrict__ rem, int32_t* __restrict__ rem_ints, const Fr* __restrict__ in, int64_t sf, size_t n) {
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (i >= n) return;
     const int64_t hsf = sf >> 1;
@@ -1036,6 +1037,7 @@ __global__ void __launch_bounds__(TPB) k_rescale(Fr* __restrict__ out, Fr* __res
     const int64_t x_rescaled = (x - x_rem) / sf;
     out[i] = fr_from_i64(x_rescaled);
     rem[i] = fr_from_i64(x_rem);
+    if (rem_ints) rem_ints[i] = (int32_t)x_rem;
 }
 
 // ---- ReLU decomposition (zkrelu.cu:8-29) -----------------------------------------------------------------------------------------
@@ -1318,8 +1320,9 @@ __global__ void __launch_bounds__(TPB) k_mul_ints(Fr* __restrict__ out, const in
 // Multilinear evaluations at one point of KF (0 or 1) tensors of field elements and KI tensors given in int32 form, in one
 // pass over the point's eq table: an int32 element costs eight limb products into the lane's unreduced sum.
 struct MeIntPtrs { const int32_t* x[6]; };
-template <int KF, int KI> __global__ void __launch_bounds__(TPB) k_me_mixed(Fr* __restrict__ partials, const Fr* __restrict__ XF, const MeIntPtrs pi, const Fr* __restrict__ E, size_t n) {
-    Fr accf = big_zero<8>();
+template <int KF, int KI> __global__ void __launch_bounds__(TPB) k_me_mixed(Fr* __restrict__ partials, const Fr* __restrict__ XF, const Fr* __restrict__ XF2, const MeIntPtrs pi,
+                                                                            const Fr* __restrict__ E, size_t n) {
+    Fr accf = big_zero<8>(), accf2 = big_zero<8>();
     uint32_t acc[KI][10];
 #pragma unroll
     for (int k = 0; k < KI; ++k)
@@ -1332,12 +1335,14 @@ template <int KF, int KI> __global__ void __launch_bounds__(TPB) k_me_mixed(Fr* 
         int32_t x[KI];
 #pragma unroll
         for (int k = 0; k < KI; ++k) x[k] = pi.x[k][t];
-        if constexpr (KF == 1) accf = add(accf, mont_mul(e, XF[t]));
+        if constexpr (KF >= 1) accf = add(accf, mont_mul(e, XF[t]));
+        if constexpr (KF == 2) accf2 = add(accf2, mont_mul(e, XF2[t]));
 #pragma unroll
         for (int k = 0; k < KI; ++k) ifold_mac(acc[k], e, ne, x[k]);
     }
     Fr out[KF + KI];
-    if constexpr (KF == 1) out[0] = accf;
+    if constexpr (KF >= 1) out[0] = accf;
+    if constexpr (KF == 2) out[1] = accf2;
 #pragma unroll
     for (int k = 0; k < KI; ++k) out[KF + k] = ifold_finish(acc[k]);
     block_reduce_store<KF + KI>(out, partials);
@@ -1484,29 +1489,31 @@ int zk_fr_me_multi_ints(uint32_t* out_host, const void* const* Xs, const void* c
     int rc = eq_table_queue(E.as<Fr>(), u, k, tmp, st);
     if (rc) return rc;
     const unsigned nb = reduce_grid(n);
-    const int KF = n_fr ? 1 : 0, KT = KF + n_ints;
+    const int KF = n_fr >= 2 && n_ints <= 3 ? 2 : (n_fr ? 1 : 0), KT = KF + n_ints;         // two tensors of field elements ride along with up to three int32 forms
     Scratch& part = tmp.add(sizeof(Fr) * KT * nb);
     if (part.rc) return part.rc;
     MeIntPtrs pi;
     for (int i = 0; i < 6; ++i) pi.x[i] = ((const FoldPrepared*)prepareds[ints_at[i < n_ints ? i : 0]])->ints;
     const Fr* XF = KF ? (const Fr*)Xs[fr_at[0]] : nullptr;
-#define MEI_CASE(F, I) if (KF == F && n_ints == I) hipLaunchKernelGGL((k_me_mixed<F, I>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), XF, pi, E.as<Fr>(), n);
+    const Fr* XF2 = KF == 2 ? (const Fr*)Xs[fr_at[1]] : nullptr;
+#define MEI_CASE(F, I) if (KF == F && n_ints == I) hipLaunchKernelGGL((k_me_mixed<F, I>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), XF, XF2, pi, E.as<Fr>(), n);
     MEI_CASE(0, 1) MEI_CASE(0, 2) MEI_CASE(0, 3) MEI_CASE(0, 4) MEI_CASE(0, 5) MEI_CASE(0, 6)
     MEI_CASE(1, 1) MEI_CASE(1, 2) MEI_CASE(1, 3) MEI_CASE(1, 4) MEI_CASE(1, 5) MEI_CASE(1, 6)
+    MEI_CASE(2, 1) MEI_CASE(2, 2) MEI_CASE(2, 3)
 #undef MEI_CASE
     ZK_LAUNCH_CHECK();
     Fr s8[8];
     rc = finish_sums(part.as<Fr>(), nb, KT, 0, s8, st);
     if (rc) return rc;
-    if (KF) memcpy(out_host + 8 * fr_at[0], &s8[0], sizeof(Fr));
+    for (int i = 0; i < KF; ++i) memcpy(out_host + 8 * fr_at[i], &s8[i], sizeof(Fr));
     for (int i = 0; i < n_ints; ++i) memcpy(out_host + 8 * ints_at[i], &s8[KF + i], sizeof(Fr));
-    if (n_fr > 1) {         // the other tensors of field elements
+    if (n_fr > KF) {         // the other tensors of field elements
         const void* rest[8];
-        for (int i = 1; i < n_fr; ++i) rest[i - 1] = Xs[fr_at[i]];
+        for (int i = KF; i < n_fr; ++i) rest[i - KF] = Xs[fr_at[i]];
         Fr r8[8];
-        rc = zk_fr_me_multi((uint32_t*)r8, rest, n_fr - 1, n, u, k, stv);
+        rc = zk_fr_me_multi((uint32_t*)r8, rest, n_fr - KF, n, u, k, stv);
         if (rc) return rc;
-        for (int i = 1; i < n_fr; ++i) memcpy(out_host + 8 * fr_at[i], &r8[i - 1], sizeof(Fr));
+        for (int i = KF; i < n_fr; ++i) memcpy(out_host + 8 * fr_at[i], &r8[i - KF], sizeof(Fr));
     }
     return 0;
 }
@@ -2188,7 +2195,12 @@ int zk_hadamard_product_sumcheck(uint32_t* proof_host, const void* a, const void
 }
 int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* st) {
     ZK_ARG(scaling_factor >= 1, "zk_rescale: scaling factor is 0");
-    LAUNCH1D(k_rescale, n, st, (Fr*)out, (Fr*)rem, (const Fr*)in, (int64_t)scaling_factor, n);
+    LAUNCH1D(k_rescale, n, st, (Fr*)out, (Fr*)rem, (int32_t*)nullptr, (const Fr*)in, (int64_t)scaling_factor, n);
+    return 0;
+}
+int zk_rescale_ints(void* out, void* rem, void* rem_ints, const void* in, uint32_t scaling_factor, size_t n, void* st) {
+    ZK_ARG(scaling_factor >= 1, "zk_rescale: scaling factor is 0");
+    LAUNCH1D(k_rescale, n, st, (Fr*)out, (Fr*)rem, (int32_t*)rem_ints, (const Fr*)in, (int64_t)scaling_factor, n);
     return 0;
 }
 int zk_relu_decomp(void* res, void* sign, void* mag, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* st) {

@@ -10,7 +10,8 @@ FrTensor Rescaling::operator()(const FrTensor& X) {
     rem_hold = std::make_shared<FrTensor>(X.size);
     rem_tensor_ptr = rem_hold.get();
     FrTensor out(X.size);
-    ZKC(zk_rescale(out.gpu_data, rem_tensor_ptr->gpu_data, X.gpu_data, scaling_factor, X.size, nullptr));
+    // the remainders are written as int32 as well: the range proof's index pass, evaluation and first round read that form
+    ZKC(zk_rescale_ints(out.gpu_data, rem_tensor_ptr->gpu_data, rem_hold->ints_for_producer(), X.gpu_data, scaling_factor, X.size, nullptr));
     return out;
 }
 Rescaling::~Rescaling() {}
