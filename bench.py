@@ -123,6 +123,7 @@ def main():
         rng = np.random.default_rng(1)
         low = -(N // 2)
         S = pv.from_i32((rng.integers(0, N, D, dtype=np.int64) + low).astype(np.int32))
+        pv.keep_for_folds(S)        # as the digit planes of the layer's softmax: the queries keep their int32 form, the outputs get theirs from the table
         mv = pv.from_i32(rng.integers(0, 1 << 22, N, dtype=np.int64).astype(np.int32))
         rs = np.random.RandomState(3)
         r, al, be = mt_random_vec(rs, 1), mt_random_vec(rs, 1), mt_random_vec(rs, 1)

@@ -176,9 +176,10 @@ __global__ void __launch_bounds__(256) k_absmax(unsigned long long* __restrict__
 }
 // max over rows of sum_j |a[row][j]| (saturating): with max |b| it bounds every dot product more tightly than
 // N * max|a| * max|b| does -- rows of a softmax output sum to its scale however long they are.
-__global__ void __launch_bounds__(256) k_rowabs(unsigned long long* __restrict__ out, const Fr* __restrict__ a, uint32_t ncol) {
+// The same pass takes the largest magnitude of the tensor (out_max, as k_absmax delivers it) along.
+__global__ void __launch_bounds__(256) k_rowabs(unsigned long long* __restrict__ out, unsigned long long* __restrict__ out_max, const Fr* __restrict__ a, uint32_t ncol) {
     const Fr* row = a + (size_t)blockIdx.x * ncol;
-    unsigned long long m = 0;
+    unsigned long long m = 0, mx = 0;
     for (uint32_t j = threadIdx.x; j < ncol; j += 256) {
         const Fr x = row[j];
         unsigned long long v;
@@ -188,9 +189,18 @@ __global__ void __launch_bounds__(256) k_rowabs(unsigned long long* __restrict__
             v = (y.v[2] | y.v[3] | y.v[4] | y.v[5] | y.v[6] | y.v[7]) ? ~0ull : ((unsigned long long)y.v[0] | ((unsigned long long)y.v[1] << 32));
         }
         if (v > (1ull << 62)) v = ~0ull;
+        mx = v > mx ? v : mx;
         m = (m == ~0ull || v == ~0ull || m + v > (1ull << 62)) ? ~0ull : m + v;
     }
     __shared__ unsigned long long red[256];
+    red[threadIdx.x] = mx;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if (threadIdx.x < s) red[threadIdx.x] = red[threadIdx.x] > red[threadIdx.x + s] ? red[threadIdx.x] : red[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) atomicMax(out_max, red[0]);
+    __syncthreads();
     red[threadIdx.x] = m;
     __syncthreads();
     for (int s = 128; s > 0; s >>= 1) {
@@ -625,10 +635,9 @@ static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch
         Scratch mx(3 * sizeof(unsigned long long), st);
         if (mx.rc) return mx.rc;
         ZK_HIP(hipMemsetAsync(mx.p, 0, 3 * sizeof(unsigned long long), st));
-        const size_t na = (size_t)batch * M * N, nb = (size_t)batch * N * P;
-        hipLaunchKernelGGL(k_absmax, dim3(absmax_grid(na)), dim3(256), 0, st, mx.as<unsigned long long>(), (const Fr*)A, na);
+        const size_t nb = (size_t)batch * N * P;
         if (!rhs) hipLaunchKernelGGL(k_absmax, dim3(absmax_grid(nb)), dim3(256), 0, st, mx.as<unsigned long long>() + 1, (const Fr*)B, nb);
-        hipLaunchKernelGGL(k_rowabs, dim3(batch * M), dim3(256), 0, st, mx.as<unsigned long long>() + 2, (const Fr*)A, N);
+        hipLaunchKernelGGL(k_rowabs, dim3(batch * M), dim3(256), 0, st, mx.as<unsigned long long>() + 2, mx.as<unsigned long long>(), (const Fr*)A, N);      // one pass over A for both of its figures
         ZK_LAUNCH_CHECK();
         void* stage = nullptr;
         int rc = staging(&stage, 24);
