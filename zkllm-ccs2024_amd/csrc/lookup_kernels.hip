@@ -28,6 +28,22 @@ using namespace zk;
 
 static constexpr int TPB = 256;
 static inline Fr load_fr(const uint32_t* p) { Fr r; memcpy(&r, p, 32); return r; }
+// Streamed operands of a kernel that also gathers from a table: loaded and stored past the caches' retention, so that the
+// table's lines stay (elements are 32 bytes at 32-byte strides from 256-byte aligned blocks)
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ Fr ld_stream(const Fr* p) {
+    const u32x4* q = (const u32x4*)p;
+    const u32x4 a = __builtin_nontemporal_load(q), b = __builtin_nontemporal_load(q + 1);
+    Fr r;
+    r.v[0] = a.x; r.v[1] = a.y; r.v[2] = a.z; r.v[3] = a.w; r.v[4] = b.x; r.v[5] = b.y; r.v[6] = b.z; r.v[7] = b.w;
+    return r;
+}
+__device__ __forceinline__ void st_stream(Fr* p, const Fr& x) {
+    u32x4 a, b;
+    a.x = x.v[0]; a.y = x.v[1]; a.z = x.v[2]; a.w = x.v[3]; b.x = x.v[4]; b.y = x.v[5]; b.z = x.v[6]; b.w = x.v[7];
+    __builtin_nontemporal_store(a, (u32x4*)p);
+    __builtin_nontemporal_store(b, (u32x4*)p + 1);
+}
 
 // ---- block reduction helper (K sums per thread) -------------------------------------------------------
 template <int K> __device__ __forceinline__ void block_reduce_store(Fr (&acc)[K], Fr* __restrict__ partials) {
@@ -499,8 +515,8 @@ __global__ void __launch_bounds__(TPB) k_lookup_ints_check(int32_t* __restrict__
 }
 // query i and 1 / (query + beta) from the int32 forms (HintSrc); unit as in inv_by_hint
 __device__ __forceinline__ Fr query_inv_ints(size_t i, const HintSrc& h, Fr& a, bool& unit) {
-    const int32_t hi = h.hint_ints[i];
-    const int32_t so = h.sout_ints ? h.sout_ints[i] : 0;
+    const int32_t hi = __builtin_nontemporal_load(h.hint_ints + i);
+    const int32_t so = h.sout_ints ? __builtin_nontemporal_load(h.sout_ints + i) : 0;
     const int64_t d = (int64_t)hi - (int64_t)h.low_int;
     const bool in_table = d >= 0 && d < (int64_t)h.N;
     const uint32_t j = in_table ? (uint32_t)d : 0u;
@@ -551,8 +567,11 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
     Fr acc_e = big_zero<8>(), acc_em = big_zero<8>();       // HINTED: sum of E and of E * M over the pairs of unit inverses
     WideAcc w0 = wide_zero(), w2 = wide_zero(), wx = wide_zero();      // sums of c0, c2 and of the cross products (a0 + da)(s0 + ds) E; HINTED: wx alone, the sum of E * M
     for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
-        const Fr e = E[t];
-        if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table: the top variable summed out
+        const Fr e = HINTED ? ld_stream(E + t) : E[t];
+        if (nE && t < n_out / 2) {      // the next round's table: the top variable summed out
+            if (HINTED) st_stream(nE + t, add(e, ld_stream(E + t + n_out / 2)));
+            else nE[t] = add(e, E[t + n_out / 2]);
+        }
         {
             Fr s0r, s1, a0, a1;
             bool unit0 = false, unit1 = false;
@@ -589,8 +608,13 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
             }
             acc[3] = add(acc[3], a0);
             acc[4] = add(acc[4], da);
-            nA[t] = add(a0, mont_mul(v_mont, da));
-            nS[t] = add(s0r, mont_mul(v_mont, ds));
+            if (HINTED) {
+                st_stream(nA + t, add(a0, mont_mul(v_mont, da)));
+                st_stream(nS + t, add(s0r, mont_mul(v_mont, ds)));
+            } else {
+                nA[t] = add(a0, mont_mul(v_mont, da));
+                nS[t] = add(s0r, mont_mul(v_mont, ds));
+            }
         }
         if (PHASE2) {
             const Fr b0 = B[t], b1 = B[t + n_out], t0r = T[t], t1 = T[t + n_out], m0 = m[t], m1 = m[t + n_out];
