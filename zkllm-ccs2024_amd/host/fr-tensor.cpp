@@ -319,6 +319,11 @@ Fr_t FrTensor::operator()(const vector<Fr_t>& u) const {
     uint log_dim = (uint)u.size();
     if (size <= ((1u << log_dim) / 2) || size > (1u << log_dim)) throw std::runtime_error("Incompatible dimensions");
     Fr_t out;
+    if (const void* h = kept_ints()) {          // read from the int32 form
+        const void* x = gpu_data;
+        ZKC(zk_fr_me_multi_ints(out.val, &x, &h, 1, size, u.empty() ? nullptr : u[0].val, (int)log_dim, nullptr));
+        return out;
+    }
     ZKC(zk_fr_me(out.val, gpu_data, size, u.empty() ? nullptr : u[0].val, (int)log_dim, nullptr));
     return out;
 }

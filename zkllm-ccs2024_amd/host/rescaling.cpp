@@ -42,12 +42,21 @@ Rescaling::Pending Rescaling::prove_begin(const FrTensor& X, const FrTensor& X_,
 
     Pending p;
     if (rem_tensor_ptr->size == (1u << ceilLog2(rem_tensor_ptr->size))) p.rem = rem_hold;
-    else p.rem = std::make_shared<FrTensor>(rem_tensor_ptr->pad({rem_tensor_ptr->size}));
+    else {
+        auto padded = std::make_shared<FrTensor>(rem_tensor_ptr->pad({rem_tensor_ptr->size}));
+        if (const void* h = rem_tensor_ptr->kept_ints()) {          // the int32 form is padded with the same zeros
+            char* dst = (char*)padded->ints_for_producer();
+            const size_t have = sizeof(int32_t) * (size_t)rem_tensor_ptr->size, all = sizeof(int32_t) * (size_t)padded->size;
+            ZKC(zk_memcpy_d2d(dst, zk_fr_fold_prepared_ints(h), have, nullptr));
+            ZKC(zk_memset(dst + have, 0, all - have, nullptr));
+        }
+        p.rem = padded;
+    }
     p.m.reset(new FrTensor(tl_rem.prep(*p.rem)));
     // X(u), X_(u), rem(u): one pass over the tensors that have the same length (the remainder is padded to a power of two)
     vector<Fr_t> ev;
     if (p.rem->size == X.size) ev = FrTensor::me_batch({&X, &X_, p.rem.get()}, u);
-    else { ev = FrTensor::me_batch({&X, &X_}, u); ev.push_back((*p.rem)(u)); }
+    else { ev = FrTensor::me_batch({&X, &X_}, u); ev.push_back(FrTensor::me_batch({p.rem.get()}, u)[0]); }
     p.lhs = ev[0];
     if (p.lhs != ev[1] * Fr_t({scaling_factor, 0, 0, 0, 0, 0, 0, 0}) + ev[2]) throw std::runtime_error("Error: the rem is not correct.");
     p.look = tl_rem.prove_begin(*p.rem, *p.m, rand_temp[0], rand_temp[1], u, v);
