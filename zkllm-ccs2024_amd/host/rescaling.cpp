@@ -53,10 +53,10 @@ Rescaling::Pending Rescaling::prove_begin(const FrTensor& X, const FrTensor& X_,
         p.rem = padded;
     }
     p.m.reset(new FrTensor(tl_rem.prep(*p.rem)));
-    // X(u), X_(u), rem(u): one pass over the tensors that have the same length (the remainder is padded to a power of two)
+    // X(u), X_(u), rem(u): one pass over the three tensors
     vector<Fr_t> ev;
-    if (p.rem->size == X.size) ev = FrTensor::me_batch({&X, &X_, p.rem.get()}, u);
-    else { ev = FrTensor::me_batch({&X, &X_}, u); ev.push_back(FrTensor::me_batch({p.rem.get()}, u)[0]); }
+    // (the padding of the remainders is zeros: the unpadded tensor has the same extension and the others' length)
+    ev = FrTensor::me_batch({&X, &X_, rem_tensor_ptr}, u);
     p.lhs = ev[0];
     if (p.lhs != ev[1] * Fr_t({scaling_factor, 0, 0, 0, 0, 0, 0, 0}) + ev[2]) throw std::runtime_error("Error: the rem is not correct.");
     p.look = tl_rem.prove_begin(*p.rem, *p.m, rand_temp[0], rand_temp[1], u, v);
