@@ -57,9 +57,8 @@ DeferredOpenings::DeferredOpenings(OpeningPlan* pl) : prev(g_deferred), plan(pl)
                 order.insert(order.end(), mid.begin(), mid.end());
             }
         }
-        std::vector<std::pair<const Commitment*, Commitment::Pending*>> ops;
-        for (Ahead* a : order) ops.emplace_back(&a->w->generator, &a->op);
-        Commitment::open_start_batch(ops);
+        to_start = order;
+        if (!hold_start) start();
     } catch (...) {
         for (Ahead* a : ahead) { try { vector<G1Jacobian_t> drop; Commitment::open_end(a->op, drop); } catch (...) {} delete a; }
         ahead.clear();
@@ -67,8 +66,26 @@ DeferredOpenings::DeferredOpenings(OpeningPlan* pl) : prev(g_deferred), plan(pl)
         throw;
     }
 }
+// The jobs of the planned openings are queued at the scope's first claim (the end of the layer's first block) unless
+// ZKLLM_OPEN_START_LATE=0 asks for the scope's start: the point kernels take the device from whatever runs beside them, and
+// the first block is a chain of small dependent kernels that each wait for a wave slot behind them (the layer is 2 ms
+// shorter this way; ZKLLM_OPEN_START_AT_CLAIM=k moves the start behind the k-th claim).
+bool DeferredOpenings::hold_start = [] { const char* e = getenv("ZKLLM_OPEN_START_LATE"); return !(e && e[0] == '0'); }();
+void DeferredOpenings::start() {
+    if (to_start.empty()) return;
+    std::vector<std::pair<const Commitment*, Commitment::Pending*>> ops;
+    for (Ahead* a : to_start) ops.emplace_back(&a->w->generator, &a->op);
+    to_start.clear();
+    Commitment::open_start_batch(ops);
+    for (auto& ia : claimed_early) { ia.first->op = std::move(ia.second->op); delete ia.second; }
+    claimed_early.clear();
+}
+int DeferredOpenings::start_at_claim = [] { const char* e = getenv("ZKLLM_OPEN_START_AT_CLAIM"); return e ? atoi(e) : 0; }();
+void zk_openings_start_now() { if (g_deferred) g_deferred->start(); }
 DeferredOpenings::~DeferredOpenings() {
     g_deferred = prev;
+    for (auto& ia : claimed_early) delete ia.second;          // never started: nothing to wait for
+    claimed_early.clear();
     for (Ahead* a : ahead) {          // started from the plan and never claimed
         if (a) { try { vector<G1Jacobian_t> drop; Commitment::open_end(a->op, drop); } catch (...) {} delete a; }
     }
@@ -78,6 +95,7 @@ DeferredOpenings::~DeferredOpenings() {
     }
 }
 void DeferredOpenings::finish() {
+    start();
     if (learning && plan) { plan->learned = true; learning = false; }
     std::vector<Item*> todo;
     todo.swap(items);
@@ -125,15 +143,24 @@ void verifyWeightClaim(const Weight& w, const Claim& c) {
     if (g_deferred) {
         DeferredOpenings& d = *g_deferred;
         const size_t k = d.next++;
+        if ((int)k >= DeferredOpenings::start_at_claim) d.start();
         d.learn(w, c);
         if (k < d.ahead.size() && d.ahead[k]) {
             DeferredOpenings::Ahead* a = d.ahead[k];
-            d.ahead[k] = nullptr;
             if (a->w == &w && a->u_cat == u_cat) {
+                d.ahead[k] = nullptr;
+                if (!d.to_start.empty()) {          // its job is not queued yet: the item takes the opening when it is
+                    DeferredOpenings::Item* it = new DeferredOpenings::Item{Commitment::Pending(), c.claim, zk_record_reserve()};
+                    d.items.push_back(it);
+                    d.claimed_early.emplace_back(it, a);
+                    return;
+                }
                 d.items.push_back(new DeferredOpenings::Item{std::move(a->op), c.claim, zk_record_reserve()});
                 delete a;
                 return;
             }
+            d.start();
+            d.ahead[k] = nullptr;
             try { vector<G1Jacobian_t> drop; Commitment::open_end(a->op, drop); } catch (...) {}      // not the planned opening: dropped
             delete a;
             d.plan->learned = false;          // the plan does not describe this sequence: learn it again next time

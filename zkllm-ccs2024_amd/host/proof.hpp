@@ -51,6 +51,9 @@ class DeferredOpenings {
     explicit DeferredOpenings(OpeningPlan* plan);
     ~DeferredOpenings();
     void finish();
+    // queues the device jobs of the planned openings if that has not happened yet (the constructor does unless hold_start)
+    void start();
+    static bool hold_start;               // planned openings wait for start() or for the first claim (default; ZKLLM_OPEN_START_LATE=0: queued by the constructor)
     DeferredOpenings(const DeferredOpenings&) = delete;
     DeferredOpenings& operator=(const DeferredOpenings&) = delete;
 
@@ -64,12 +67,17 @@ class DeferredOpenings {
     struct Ahead;
     std::vector<Ahead*> ahead;            // openings started from the plan, in the plan's order
     size_t next = 0;                      // index of the next verifyWeightClaim within the scope
+    std::vector<Ahead*> to_start;         // planned openings whose jobs are not queued yet, in starting order
+    std::vector<std::pair<Item*, Ahead*>> claimed_early;      // claimed before their jobs were queued: the item takes the opening at start()
+    static int start_at_claim;            // with hold_start: the number of claims after which the jobs are queued (0: the first claim's start)
     void learn(const Weight& w, const Claim& c);
     friend WeightOpeningAhead openWeightAhead(const Weight& w, const std::vector<Fr_t>& u_input, const std::vector<Fr_t>& u_output);
     friend std::vector<WeightOpeningAhead> openWeightsAhead(const std::vector<const Weight*>&, const std::vector<const std::vector<Fr_t>*>&, const std::vector<const std::vector<Fr_t>*>&);
     friend void verifyWeightClaim(const Weight& w, const Claim& c);
     friend void verifyWeightClaim(const Weight& w, const Claim& c, WeightOpeningAhead& ahead);
 };
+
+void zk_openings_start_now();         // DeferredOpenings::start() of the innermost scope, if there is one
 
 // planned openings (DeferredOpenings with a learned plan) use a weight's cross commitments when it has them; off: they sum
 // over the generators in every round (measurements compare the two)
