@@ -323,6 +323,10 @@ int zk_softmax_table(void* table, double log_theta, double step, uint32_t len, v
 int zk_softmax_decompose(void* const* planes, const void* X_shifted, const uint32_t* bs_host, int K, size_t n, void* stream);
 /* the same, and int_planes[k] (int32, n each; null entries and a null array allowed) receive digit k once more as int32 */
 int zk_softmax_decompose_ints(void* const* planes, void* const* int_planes, const void* X_shifted, const uint32_t* bs_host, int K, size_t n, void* stream);
+/* zk_softmax_shift and zk_softmax_decompose_ints in one pass (zksoftmax.cu:124-140): the shifted scores are decomposed where
+ * they are written, so they are not read again */
+int zk_softmax_shift_decompose(void* shift, void* out_shifted, void* const* planes, void* const* int_planes, const void* X, uint32_t rows, uint32_t cols, double scale,
+                               const uint32_t* bs_host, int K, void* stream);
 
 /* ---- measurement helpers (no counterpart in the reference) ---------------------------------------- */
 /* v_mad_u64_u32 issue peak of the device: 16 independent chains per lane, no memory traffic */

@@ -455,6 +455,42 @@ def test_mapped_lookup_job_equals_the_plain_one_on_the_combined_queries(k):
         hip.free(p)
 
 
+@pytest.mark.parametrize("rows,cols", [(5, 64), (37, 200), (64, 2048)])
+def test_softmax_shift_and_decomposition_in_one_pass_equal_the_two_passes(rows, cols):
+    """zk_softmax_shift_decompose against zk_softmax_shift followed by zk_softmax_decompose_ints: the same shifts, shifted
+    scores, digit planes and int32 planes (ragged rows: 200 columns are three full wave steps and a partial one)."""
+    import ctypes
+    from gpuhelp import Hip, c_void_p, c_size_t, c_int
+    from ctypes import c_uint, c_double
+    hip = Hip()
+    rng = np.random.default_rng(rows * 1000 + cols)
+    n = rows * cols
+    scale = 65536.0 * 8.0
+    X = rng.integers(-(1 << 22), 1 << 22, n).astype(np.int64)
+    dX = hip.upload(fr_array([int(v) % R_MOD for v in X]))
+    bs = np.array([256, 1 << 20, 1 << 20], dtype=np.uint32)
+    out = []
+    for fused in (False, True):
+        dShift, dXs = hip.malloc(32 * rows), hip.malloc(32 * n)
+        planes = [hip.malloc(32 * n) for _ in range(3)]
+        ints = [hip.malloc(4 * n) for _ in range(3)]
+        arr = (c_void_p * 3)(*[c_void_p(x) for x in planes])
+        iarr = (c_void_p * 3)(*[c_void_p(x) for x in ints])
+        if fused:
+            hip.call("zk_softmax_shift_decompose", c_void_p(dShift), c_void_p(dXs), arr, iarr, c_void_p(dX), c_uint(rows), c_uint(cols), c_double(scale), bs, c_int(3), None)
+        else:
+            hip.call("zk_softmax_shift", c_void_p(dShift), c_void_p(dXs), c_void_p(dX), c_uint(rows), c_uint(cols), c_double(scale), None)
+            hip.call("zk_softmax_decompose_ints", arr, iarr, c_void_p(dXs), bs, c_int(3), c_size_t(n), None)
+        out.append([hip.download(dShift, (rows, 8), np.uint32), hip.download(dXs, (n, 8), np.uint32)] + [hip.download(q, (n, 8), np.uint32) for q in planes]
+                   + [hip.download(q, (n,), np.int32) for q in ints])
+        for q in [dShift, dXs] + planes + ints:
+            hip.free(q)
+    for a, b in zip(out[0], out[1]):
+        assert (a == b).all()
+    assert out[0][2].any() and out[0][5].any()
+    hip.free(dX)
+
+
 @pytest.mark.parametrize("k", [13, 17, 19])
 def test_lookup_jobs_that_read_int32_forms_equal_the_plain_one(k):
     """zk_lookup_prove_begin_mapped_ints / _hinted_ints (the first round of a large job reads the queries' int32 forms and

@@ -1087,7 +1087,32 @@ __global__ void __launch_bounds__(TPB) k_relu_decomp(Fr* __restrict__ res, Fr* _
 // loop of zksoftmax.cu:24-26 does: the 64 lanes evaluate 64 consecutive terms side by side, park them in LDS, and every
 // lane then adds them in order (the additions are the same in all lanes, so all end with the same total).
 // shift = round_half_away(scale * log(total)).  out = x - shift.  scale = sf_in * sqrt(d).
-__global__ void __launch_bounds__(TPB) k_softmax_shift(Fr* __restrict__ shift, Fr* __restrict__ out, const Fr* __restrict__ X, uint32_t rows, uint32_t cols, double scale) {
+struct U32Pack8 { uint32_t v[8]; };
+struct PlanePtrs { Fr* p[8]; };
+struct IntPlanePtrs { int32_t* p[8]; };       // optional: the digits once more as int32 (a plane whose radix passes 2^31 gets none)
+// digits of -x in the mixed radix bs[0..K) into position g of the planes (zksoftmax.cu:95-109)
+__device__ __forceinline__ void softmax_digits(const PlanePtrs& planes, const IntPlanePtrs& ints, uint32_t* __restrict__ flag, const Fr& x, const U32Pack8& bs, int K, size_t g) {
+    const Fr mx = neg(x);
+    if (mx.v[2] | mx.v[3] | mx.v[4] | mx.v[5] | mx.v[6] | mx.v[7]) {
+        atomicOr(flag, 1u);
+        for (int k = 0; k < K; ++k) {
+            planes.p[k][g] = big_zero<8>();
+            if (ints.p[k]) ints.p[k][g] = 0;
+        }
+        return;
+    }
+    unsigned long long tmp = ((unsigned long long)mx.v[1] << 32) | mx.v[0];
+    for (int k = 0; k < K; ++k) {
+        const unsigned long long digit = tmp % bs.v[k];
+        planes.p[k][g] = fr_from_u64(digit);
+        if (ints.p[k]) ints.p[k][g] = (int32_t)digit;
+        tmp /= bs.v[k];
+    }
+    if (tmp != 0) atomicOr(flag, 2u);   // more digits than the radices cover
+}
+// K > 0: the shifted scores are decomposed where they are written (k_softmax_decompose's planes without its pass over them)
+__global__ void __launch_bounds__(TPB) k_softmax_shift(Fr* __restrict__ shift, Fr* __restrict__ out, const Fr* __restrict__ X, uint32_t rows, uint32_t cols, double scale,
+                                                       const PlanePtrs planes, const IntPlanePtrs ints, uint32_t* __restrict__ flag, const U32Pack8 bs, int K) {
     __shared__ double term[TPB / 64][64];
     const uint32_t w = threadIdx.x >> 6, lane = threadIdx.x & 63u;
     const uint32_t row = blockIdx.x * (TPB / 64) + w;
@@ -1113,7 +1138,11 @@ __global__ void __launch_bounds__(TPB) k_softmax_shift(Fr* __restrict__ shift, F
     const Fr sh = fr_from_i64(si);
     if (lane == 0) shift[row] = sh;
     Fr* orow = out + (size_t)row * cols;
-    for (uint32_t j = lane; j < cols; j += 64) orow[j] = sub(xr[j], sh);
+    for (uint32_t j = lane; j < cols; j += 64) {
+        const Fr xs = sub(xr[j], sh);
+        orow[j] = xs;
+        if (K > 0) softmax_digits(planes, ints, flag, xs, bs, K, (size_t)row * cols + j);
+    }
 }
 // table[x] = floor(exp(log_theta - step * x) + 0.5)  (zksoftmax.cu:4-14); step = B_k / (sf_in sqrt d)
 __global__ void __launch_bounds__(TPB) k_softmax_table(Fr* __restrict__ table, double log_theta, double step, uint32_t len) {
@@ -1124,30 +1153,10 @@ __global__ void __launch_bounds__(TPB) k_softmax_table(Fr* __restrict__ table, d
 }
 // digits of -x in the mixed radix bs[0..K): plane k holds digit k (zksoftmax.cu:95-109).  Values whose
 // negation does not fit 64 bits raise the flag (the reference leaves their planes unwritten).
-struct U32Pack8 { uint32_t v[8]; };
-struct PlanePtrs { Fr* p[8]; };
-struct IntPlanePtrs { int32_t* p[8]; };       // optional: the digits once more as int32 (a plane whose radix passes 2^31 gets none)
 __global__ void __launch_bounds__(TPB) k_softmax_decompose(const PlanePtrs planes, const IntPlanePtrs ints, uint32_t* __restrict__ flag, const Fr* __restrict__ X, const U32Pack8 bs,
                                                            int K, size_t n) {
     const size_t g = (size_t)blockIdx.x * TPB + threadIdx.x;
-    if (g >= n) return;
-    const Fr mx = neg(X[g]);
-    if (mx.v[2] | mx.v[3] | mx.v[4] | mx.v[5] | mx.v[6] | mx.v[7]) {
-        atomicOr(flag, 1u);
-        for (int k = 0; k < K; ++k) {
-            planes.p[k][g] = big_zero<8>();
-            if (ints.p[k]) ints.p[k][g] = 0;
-        }
-        return;
-    }
-    unsigned long long tmp = ((unsigned long long)mx.v[1] << 32) | mx.v[0];
-    for (int k = 0; k < K; ++k) {
-        const unsigned long long digit = tmp % bs.v[k];
-        planes.p[k][g] = fr_from_u64(digit);
-        if (ints.p[k]) ints.p[k][g] = (int32_t)digit;
-        tmp /= bs.v[k];
-    }
-    if (tmp != 0) atomicOr(flag, 2u);   // more digits than the radices cover
+    if (g < n) softmax_digits(planes, ints, flag, X[g], bs, K, g);
 }
 
 // ---- host side ----------------------------------------------------------------------------------------------------------------------
@@ -1327,14 +1336,14 @@ __global__ void __launch_bounds__(256) k_ifold_rows(Fr* __restrict__ out, const 
     }
 }
 
-// out[i] = table[idx[i]] with the int32 form of the same elements beside it (table_ints: the table's own int32 form)
-__global__ void __launch_bounds__(TPB) k_gather_ints(Fr* __restrict__ out, int32_t* __restrict__ out_ints, const Fr* __restrict__ table, const int32_t* __restrict__ table_ints,
+// out[i] = table[idx[i]] with the int32 form of the same elements beside it, both from the table's own int32 form
+__global__ void __launch_bounds__(TPB) k_gather_ints(Fr* __restrict__ out, int32_t* __restrict__ out_ints, const Fr* __restrict__ /*table*/, const int32_t* __restrict__ table_ints,
                                                      const uint32_t* __restrict__ idx, size_t n) {
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (i >= n) return;
-    const uint32_t j = idx[i];
-    out[i] = table[j];
-    out_ints[i] = table_ints[j];
+    const int32_t v = table_ints[idx[i]];      // the table's int32 form is an eighth of the table: it stays cached where the table does not
+    out[i] = fr_from_i64((int64_t)v);           // the same element as table[idx[i]]
+    out_ints[i] = v;
 }
 // out[i] = a[i] * b[i] for two tensors given by their int32 forms: the product is an exact 64-bit integer
 __global__ void __launch_bounds__(TPB) k_mul_ints(Fr* __restrict__ out, const int32_t* __restrict__ a, const int32_t* __restrict__ b, size_t n) {
@@ -2235,8 +2244,34 @@ int zk_relu_decomp(void* res, void* sign, void* mag, void* rem, const void* in, 
 int zk_softmax_shift(void* shift, void* out_shifted, const void* X, uint32_t rows, uint32_t cols, double scale, void* st) {
     if (rows == 0) return 0;
     ZK_ARG(cols >= 1 && scale > 0.0, "zk_softmax_shift: bad shape or scale");
-    hipLaunchKernelGGL(k_softmax_shift, dim3(cdiv(rows, TPB / 64)), dim3(TPB), 0, (hipStream_t)st, (Fr*)shift, (Fr*)out_shifted, (const Fr*)X, rows, cols, scale);
+    hipLaunchKernelGGL(k_softmax_shift, dim3(cdiv(rows, TPB / 64)), dim3(TPB), 0, (hipStream_t)st, (Fr*)shift, (Fr*)out_shifted, (const Fr*)X, rows, cols, scale, PlanePtrs(),
+                       IntPlanePtrs(), (uint32_t*)nullptr, U32Pack8(), 0);
     ZK_LAUNCH_CHECK();
+    return 0;
+}
+int zk_softmax_shift_decompose(void* shift, void* out_shifted, void* const* planes, void* const* int_planes, const void* X, uint32_t rows, uint32_t cols, double scale,
+                               const uint32_t* bs_host, int K, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    if (rows == 0) return 0;
+    ZK_ARG(cols >= 1 && scale > 0.0, "zk_softmax_shift: bad shape or scale");
+    ZK_ARG(K >= 1 && K <= 8, "zk_softmax_decompose: K must be 1..8");
+    U32Pack8 bs;
+    for (int i = 0; i < 8; ++i) bs.v[i] = i < K ? bs_host[i] : 1u;
+    for (int i = 0; i < K; ++i) ZK_ARG(bs.v[i] >= 1, "zk_softmax_decompose: zero radix");
+    PlanePtrs pp;
+    IntPlanePtrs ip;
+    for (int i = 0; i < 8; ++i) { pp.p[i] = i < K ? (Fr*)planes[i] : nullptr; ip.p[i] = (int_planes && i < K) ? (int32_t*)int_planes[i] : nullptr; }
+    for (int i = 0; i < K; ++i) ZK_ARG(pp.p[i] != nullptr, "zk_softmax_decompose: null plane");
+    for (int i = 0; i < K; ++i) ZK_ARG(!ip.p[i] || bs.v[i] <= 0x80000000u, "zk_softmax_decompose_ints: a radix above 2^31 has no int32 plane");
+    Scratch flag(4, st);
+    if (flag.rc) return flag.rc;
+    ZK_HIP(hipMemsetAsync(flag.p, 0, 4, st));
+    hipLaunchKernelGGL(k_softmax_shift, dim3(cdiv(rows, TPB / 64)), dim3(TPB), 0, st, (Fr*)shift, (Fr*)out_shifted, (const Fr*)X, rows, cols, scale, pp, ip, flag.as<uint32_t>(), bs, K);
+    ZK_LAUNCH_CHECK();
+    uint32_t f = 0;
+    int rc = read_flag(flag.as<uint32_t>(), &f, st);
+    if (rc) return rc;
+    ZK_ARG(f == 0, "softmax: a shifted score is positive or exceeds the digit radices");
     return 0;
 }
 int zk_softmax_table(void* table, double log_theta, double step, uint32_t len, void* st) {

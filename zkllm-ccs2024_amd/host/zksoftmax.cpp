@@ -56,7 +56,6 @@ FrTensor zkSoftmax::compute_rows(uint m, const FrTensor& X, FrTensor& shift, FrT
     if (X_shifted.size != X.size) throw std::invalid_argument("X_shifted must be the same size as X");
 
     const double scale = static_cast<double>(scaling_factor_in) * std::sqrt(static_cast<double>(d));
-    ZKC(zk_softmax_shift(shift.gpu_data, X_shifted.gpu_data, X.gpu_data, m, n, scale, nullptr));
 
     const size_t N = (size_t)m * n;
     X_segments.reserve(K);
@@ -68,7 +67,8 @@ FrTensor zkSoftmax::compute_rows(uint m, const FrTensor& X, FrTensor& shift, FrT
         planes[i] = X_segments[i].gpu_data;
         if (bs[i] <= 0x80000000u) int_planes[i] = X_segments[i].ints_for_producer();
     }
-    ZKC(zk_softmax_decompose_ints(planes.data(), int_planes.data(), X_shifted.gpu_data, bs.data(), (int)K, N, nullptr));
+    // shift and digits in one pass: the shifted scores are decomposed where they are written
+    ZKC(zk_softmax_shift_decompose(shift.gpu_data, X_shifted.gpu_data, planes.data(), int_planes.data(), X.gpu_data, m, n, scale, bs.data(), (int)K, nullptr));
 
     for (uint i = 0; i < L; ++i) m_segments.push_back(least_significant_segments[i].prep(X_segments[i]));
     for (uint i = L; i < K; ++i) {
