@@ -192,25 +192,24 @@ __global__ void __launch_bounds__(256) k_rowabs(unsigned long long* __restrict__
         mx = v > mx ? v : mx;
         m = (m == ~0ull || v == ~0ull || m + v > (1ull << 62)) ? ~0ull : m + v;
     }
-    __shared__ unsigned long long red[256];
-    red[threadIdx.x] = mx;
-    __syncthreads();
-    for (int s = 128; s > 0; s >>= 1) {
-        if (threadIdx.x < s) red[threadIdx.x] = red[threadIdx.x] > red[threadIdx.x + s] ? red[threadIdx.x] : red[threadIdx.x + s];
-        __syncthreads();
+    // both figures through one tree: wave shuffles first, one LDS step for the four waves
+    auto sat_add = [](unsigned long long x, unsigned long long y) { return (x == ~0ull || y == ~0ull || x + y > (1ull << 62)) ? ~0ull : x + y; };
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const unsigned long long om = __shfl_xor(mx, off, 64), os = __shfl_xor(m, off, 64);
+        mx = om > mx ? om : mx;
+        m = sat_add(m, os);
     }
-    if (threadIdx.x == 0) atomicMax(out_max, red[0]);
+    __shared__ unsigned long long red[2][4];
+    const uint32_t wv = threadIdx.x >> 6;
+    if ((threadIdx.x & 63u) == 0) { red[0][wv] = mx; red[1][wv] = m; }
     __syncthreads();
-    red[threadIdx.x] = m;
-    __syncthreads();
-    for (int s = 128; s > 0; s >>= 1) {
-        if (threadIdx.x < s) {
-            const unsigned long long x = red[threadIdx.x], y = red[threadIdx.x + s];
-            red[threadIdx.x] = (x == ~0ull || y == ~0ull || x + y > (1ull << 62)) ? ~0ull : x + y;
-        }
-        __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long gm = red[0][0], gs = red[1][0];
+        for (int i = 1; i < 4; ++i) { gm = red[0][i] > gm ? red[0][i] : gm; gs = sat_add(gs, red[1][i]); }
+        atomicMax(out_max, gm);
+        atomicMax(out, gs);
     }
-    if (threadIdx.x == 0) atomicMax(out, red[0]);
 }
 template <typename T> __global__ void __launch_bounds__(256) k_fr_to_int(T* __restrict__ out, const Fr* __restrict__ a, size_t n) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
