@@ -294,6 +294,9 @@ int zk_lookup_prove_begin_mapped(void** handle, const void* S_in, const void* S_
  * and the table's mapped values (mapped_prepared: N integers, the padded mapped_vals of tLookupRangeMapping).  The first
  * round reads 4 bytes per query and tensor instead of 32 and takes query and inverse from the table wherever the table entry
  * at S_in[i] - low is what the integers say (checked per table entry on the device, so any T is safe); same results. */
+/* 1 when a job of D queries into N entries reads its queries from their int32 forms alone: the tensors of field elements
+ * passed beside them (S, S_in, S_out) are then never read and may be left unfilled (a padded copy need not be made) */
+int zk_lookup_ints_suffice(size_t D, size_t N);
 int zk_lookup_prove_begin_hinted_ints(void** handle, const void* S, const void* S_prepared, const void* T, const void* m, int32_t low, const uint32_t* beta,
                                       const uint32_t* u_eq, const uint32_t* v, size_t D, size_t N, int rounds, void* stream);
 int zk_lookup_prove_begin_mapped_ints(void** handle, const void* S_in, const void* S_in_prepared, const void* S_out, const void* S_out_prepared, const void* mapped_prepared,

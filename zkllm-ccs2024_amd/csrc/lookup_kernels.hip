@@ -1710,7 +1710,7 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
     bool fuse_first = false;
     if (!A) {
         ZK_ARG(hs != nullptr, "lookup sumcheck: neither A nor a hint");
-        fuse_first = D > N && (D >> 1) > (size_t)SPLIT_HALF;       // a phase-1 round that the full-size kernel takes
+        fuse_first = zk_lookup_ints_suffice(D, N) != 0;       // a phase-1 round that the full-size kernel takes
         if (!fuse_first && hs->S_out) {
             Scratch& Sbuf = job.arena.add(sizeof(Fr) * D);
             if (Sbuf.rc) return Sbuf.rc;
@@ -2077,6 +2077,9 @@ int zk_lookup_prove_begin_mapped(void** handle, const void* S_in, const void* S_
     ZK_ARG(S_in != nullptr && S_out != nullptr && r != nullptr, "zk_lookup_prove_begin_mapped: null queries or challenge");
     return lookup_prove_begin(handle, nullptr, T, m, S_in, low, beta, u_eq, v, D, N, rounds, stv, S_out, r);
 }
+// 1 when a job of this shape takes its queries from their int32 forms alone (its first round is the fused one): the
+// field-element tensor given beside them is then never read
+int zk_lookup_ints_suffice(size_t D, size_t N) { return (D > N && (D >> 1) > (size_t)SPLIT_HALF) ? 1 : 0; }
 int zk_lookup_prove_begin_hinted_ints(void** handle, const void* S, const void* S_prepared, const void* T, const void* m, int32_t low, const uint32_t* beta,
                                       const uint32_t* u_eq, const uint32_t* v, size_t D, size_t N, int rounds, void* stv) {
     ZK_ARG(S != nullptr && S_prepared != nullptr, "zk_lookup_prove_begin_hinted_ints: null queries");

@@ -43,7 +43,10 @@ Rescaling::Pending Rescaling::prove_begin(const FrTensor& X, const FrTensor& X_,
     Pending p;
     if (rem_tensor_ptr->size == (1u << ceilLog2(rem_tensor_ptr->size))) p.rem = rem_hold;
     else {
-        auto padded = std::make_shared<FrTensor>(rem_tensor_ptr->pad({rem_tensor_ptr->size}));
+        // with an int32 form that a job of this size reads alone, the padded field elements are never read: not written
+        const uint padded_size = 1u << ceilLog2(rem_tensor_ptr->size);
+        const bool ints_only = rem_tensor_ptr->kept_ints() && zk_lookup_ints_suffice(padded_size, tl_rem.table.size);
+        auto padded = ints_only ? std::make_shared<FrTensor>(padded_size) : std::make_shared<FrTensor>(rem_tensor_ptr->pad({rem_tensor_ptr->size}));
         if (const void* h = rem_tensor_ptr->kept_ints()) {          // the int32 form is padded with the same zeros
             char* dst = (char*)padded->ints_for_producer();
             const size_t have = sizeof(int32_t) * (size_t)rem_tensor_ptr->size, all = sizeof(int32_t) * (size_t)padded->size;
