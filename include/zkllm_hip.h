@@ -317,6 +317,10 @@ int zk_hadamard_prove_end(void* handle, uint32_t* coefs_host);
 int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* stream);       /* rescaling_kernel rescaling.cu:8-21 */
 /* the same, and rem_ints (int32, n) receives the remainders once more: they lie in [-sf/2, sf/2) */
 int zk_rescale_ints(void* out, void* rem, void* rem_ints, const void* in, uint32_t scaling_factor, size_t n, void* stream);
+/* the same, and out_ints receives the rescaled values as int32; synchronises and reports in *out_fits_host whether every one
+ * of them fits (0: out_ints must not be used) */
+int zk_rescale_ints_both(void* out, void* out_ints, int* out_fits_host, void* rem, void* rem_ints, const void* in, uint32_t scaling_factor, size_t n, void* stream);
+int zk_i32_fill(void* dst_i32, int32_t value, size_t n, void* stream);       /* n int32 slots set to value (padding of an int32 form) */
 /* zkrelu_decomp_kernel zkrelu.cu:8-29: the same rescaling, then sign (1 when the rescaled value is >= 0), magnitude and max(., 0) */
 int zk_relu_decomp(void* res, void* sign, void* mag, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* stream);
 /* zksoftmax_shift zksoftmax.cu:20-32 (scale = sf_in*sqrt(d)), zksoftmax_calculate_table :4-14, zksoftmax_decompose_kernel :95-109 */

@@ -1051,7 +1051,9 @@ k_hadamard_tail(Fr* __restrict__ sums, const PtrPack<K> p, Fr* wE, const Fr* E, 
 
 // ---- rescaling (rescaling.cu:8-21) ----------------------------------------------------------------------------------------------
 // rem_ints (optional): the remainders once more as int32 (they lie in [-sf/2, sf/2))
-__global__ void __launch_bounds__(TPB) k_rescale(Fr* __restrict__ out, Fr* __restrict__ rem, int32_t* __restrict__ rem_ints, const Fr* __restrict__ in, int64_t sf, size_t n) {
+// out_ints (optional): the rescaled values as int32 too; *flag is raised when one of them does not fit
+__global__ void __launch_bounds__(TPB) k_rescale(Fr* __restrict__ out, Fr* __restrict__ rem, int32_t* __restrict__ rem_ints, const Fr* __restrict__ in, int64_t sf, size_t n,
+                                                 int32_t* __restrict__ out_ints = nullptr, uint32_t* __restrict__ flag = nullptr) {
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (i >= n) return;
     const int64_t hsf = sf >> 1;
@@ -1062,6 +1064,14 @@ __global__ void __launch_bounds__(TPB) k_rescale(Fr* __restrict__ out, Fr* __res
     out[i] = fr_from_i64(x_rescaled);
     rem[i] = fr_from_i64(x_rem);
     if (rem_ints) rem_ints[i] = (int32_t)x_rem;
+    if (out_ints) {
+        out_ints[i] = (int32_t)x_rescaled;
+        if (x_rescaled != (int64_t)(int32_t)x_rescaled) atomicOr(flag, 1u);
+    }
+}
+__global__ void __launch_bounds__(TPB) k_i32_fill(int32_t* __restrict__ dst, int32_t v, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) dst[i] = v;
 }
 
 // ---- ReLU decomposition (zkrelu.cu:8-29) -----------------------------------------------------------------------------------------
@@ -2237,6 +2247,26 @@ int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, si
 int zk_rescale_ints(void* out, void* rem, void* rem_ints, const void* in, uint32_t scaling_factor, size_t n, void* st) {
     ZK_ARG(scaling_factor >= 1, "zk_rescale: scaling factor is 0");
     LAUNCH1D(k_rescale, n, st, (Fr*)out, (Fr*)rem, (int32_t*)rem_ints, (const Fr*)in, (int64_t)scaling_factor, n);
+    return 0;
+}
+int zk_rescale_ints_both(void* out, void* out_ints, int* out_fits_host, void* rem, void* rem_ints, const void* in, uint32_t scaling_factor, size_t n, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(scaling_factor >= 1, "zk_rescale: scaling factor is 0");
+    ZK_ARG(out_ints != nullptr && out_fits_host != nullptr, "zk_rescale_ints_both: null argument");
+    *out_fits_host = 1;
+    if (n == 0) return 0;
+    Scratch flag(4, st);
+    if (flag.rc) return flag.rc;
+    ZK_HIP(hipMemsetAsync(flag.p, 0, 4, st));
+    LAUNCH1D(k_rescale, n, st, (Fr*)out, (Fr*)rem, (int32_t*)rem_ints, (const Fr*)in, (int64_t)scaling_factor, n, (int32_t*)out_ints, flag.as<uint32_t>());
+    uint32_t f = 0;
+    int rc = read_flag(flag.as<uint32_t>(), &f, st);
+    if (rc) return rc;
+    *out_fits_host = f ? 0 : 1;
+    return 0;
+}
+int zk_i32_fill(void* dst, int32_t value, size_t n, void* st) {
+    LAUNCH1D(k_i32_fill, n, st, (int32_t*)dst, value, n);
     return 0;
 }
 int zk_relu_decomp(void* res, void* sign, void* mag, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* st) {

@@ -341,9 +341,9 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
     WeightOpeningAhead od, og, ou;
 
     auto up_out = up_layer(input);
-    auto up_out_ = up_rescale(up_out);
+    auto up_out_ = up_rescale.rescale(up_out, true);            // int32 forms: the activation lookup and the product below read them
     auto gate_out = gate_layer(input);
-    auto gate_out_ = gate_rescale(gate_out);
+    auto gate_out_ = gate_rescale.rescale(gate_out, true);
     auto p = swiglu(gate_out_);
     auto &swiglu_out = p.first, &swiglu_m = p.second;
 

@@ -6,12 +6,20 @@
 
 Rescaling::Rescaling(uint scaling_factor) : scaling_factor(scaling_factor), tl_rem(-static_cast<int>(scaling_factor >> 1), scaling_factor), rem_tensor_ptr(nullptr) {}
 
-FrTensor Rescaling::operator()(const FrTensor& X) {
+FrTensor Rescaling::operator()(const FrTensor& X) { return rescale(X, false); }
+FrTensor Rescaling::rescale(const FrTensor& X, bool ints_out) {
     rem_hold = std::make_shared<FrTensor>(X.size);
     rem_tensor_ptr = rem_hold.get();
     FrTensor out(X.size);
     // the remainders are written as int32 as well: the range proof's index pass, evaluation and first round read that form
-    ZKC(zk_rescale_ints(out.gpu_data, rem_tensor_ptr->gpu_data, rem_hold->ints_for_producer(), X.gpu_data, scaling_factor, X.size, nullptr));
+    // the rescaled values too, when they fit (activations do): lookups, products and evaluations downstream read that form
+    // (asked for by the caller: whether they fit is read back, a host round trip that a block which shares the device with
+    // the openings' kernels pays with milliseconds)
+    if (ints_out) {
+        int fits = 0;
+        ZKC(zk_rescale_ints_both(out.gpu_data, out.ints_for_producer(), &fits, rem_tensor_ptr->gpu_data, rem_hold->ints_for_producer(), X.gpu_data, scaling_factor, X.size, nullptr));
+        if (!fits) out.drop_kept();
+    } else ZKC(zk_rescale_ints(out.gpu_data, rem_tensor_ptr->gpu_data, rem_hold->ints_for_producer(), X.gpu_data, scaling_factor, X.size, nullptr));
     return out;
 }
 Rescaling::~Rescaling() {}

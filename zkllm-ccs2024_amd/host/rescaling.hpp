@@ -13,6 +13,9 @@ class Rescaling {
 
     Rescaling(uint scaling_factor);
     FrTensor operator()(const FrTensor& X);
+    // addition: operator() that, with ints_out, also gives the rescaled tensor an int32 form when every value fits (one
+    // host round trip): for outputs that go into a table lookup or a product with another such tensor
+    FrTensor rescale(const FrTensor& X, bool ints_out);
     vector<Claim> prove(const FrTensor& X, const FrTensor& X_);
     // prove in two halves: begin draws the challenges, checks X = sf * X_ + rem at u and queues the range proof of the
     // remainder on a side stream; end writes the transcript entries.  Proofs that follow each other without anything

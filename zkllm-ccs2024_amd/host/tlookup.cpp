@@ -212,10 +212,32 @@ LookupPending tLookupRangeMapping::prove_begin(const FrTensor& S_in, const FrTen
     const FrTensor *si = &S_in, *so = &S_out, *mm = &m;
     if (D != (1u << ceilLog2(D))) {
         // pad the queries with the first table entry and account for them in m[0] (tlookup.cu:502-510)
-        keep.emplace_back(new FrTensor(S_in.pad({D}, table(0))));
-        si = keep.back().get();
-        keep.emplace_back(new FrTensor(S_out.pad({D}, mapped_vals(0))));
-        so = keep.back().get();
+        const uint Dp = 1u << ceilLog2(D);
+        const Fr_t t0 = table(0), v0 = mapped_vals(0);
+        // Queries that keep int32 forms are padded in that form; where the job reads nothing else (zk_lookup_ints_suffice) the
+        // padded field elements are not written at all.
+        auto small = [](const Fr_t& x, int32_t& out) {          // x as an int32, if it is one
+            const Fr_t n = Fr_t{{0, 0, 0, 0, 0, 0, 0, 0}} - x;
+            auto one_limb = [](const Fr_t& y) { return !(y.val[1] | y.val[2] | y.val[3] | y.val[4] | y.val[5] | y.val[6] | y.val[7]) && y.val[0] < 0x80000000u; };
+            if (one_limb(x)) { out = (int32_t)x.val[0]; return true; }
+            if (one_limb(n)) { out = -(int32_t)n.val[0]; return true; }
+            return false;
+        };
+        int32_t t0i = 0, v0i = 0;
+        const bool ints = S_in.kept_ints() && S_out.kept_ints() && mapped_vals.kept_ints() && small(t0, t0i) && small(v0, v0i);
+        const bool ints_only = ints && zk_lookup_ints_suffice(Dp, table.size);
+        auto padded = [&](const FrTensor& t, const Fr_t& fill, int32_t fill_i) {
+            FrTensor* p = ints_only ? new FrTensor(Dp) : new FrTensor(t.pad({D}, fill));
+            keep.emplace_back(p);
+            if (ints) {
+                char* dst = (char*)p->ints_for_producer();
+                ZKC(zk_memcpy_d2d(dst, zk_fr_fold_prepared_ints(t.kept_ints()), sizeof(int32_t) * (size_t)D, nullptr));
+                ZKC(zk_i32_fill(dst + sizeof(int32_t) * (size_t)D, fill_i, Dp - D, nullptr));
+            }
+            return p;
+        };
+        si = padded(S_in, t0, t0i);
+        so = padded(S_out, v0, v0i);
         keep.emplace_back(new FrTensor(m));
         FrTensor* m_ = keep.back().get();
         Fr_t m0 = (*m_)(0) + Fr_t{{(1u << ceilLog2(D)) - D, 0, 0, 0, 0, 0, 0, 0}};
