@@ -160,6 +160,7 @@ class Prover:
                      "zkp_rescale", "zkp_rescale_prove", "zkp_relu", "zkp_attn", "zkp_zkfc_stacked", "zkp_range_prep", "zkp_batch_inv", "zkp_softmax",
                      "zkp_layer_create", "zkp_layer_create_random", "zkp_layer_run", "zkp_fc_forward_over_view"):
             getattr(L, name).restype = c_void_p
+        L.zkp_rescale_ints_prove.restype = c_void_p
         L.zkp_transcript_size.restype = ctypes.c_long
         L.zkp_fr_size.restype = c_uint
         L.zkp_g1_size.restype = c_uint
@@ -332,6 +333,9 @@ class Prover:
         parts = (c_void_p * 4)()
         out = self.H(self.lib.zkp_relu(c_void_p(X.h), c_uint(sf), parts))
         return out, [self.H(p) for p in parts]
+
+    def rescale_ints_prove(self, X, sf):
+        return self.H(self.lib.zkp_rescale_ints_prove(c_void_p(X.h), c_uint(sf)))
 
     def rescale_prove(self, X, sf):
         return self.H(self.lib.zkp_rescale_prove(c_void_p(X.h), c_uint(sf)))

@@ -172,6 +172,59 @@ def test_mapping_lookup(pv, orc, D, low, length):
     assert t.shape == e_t.shape and (t == e_t).all()
 
 
+@pytest.mark.parametrize("n,sf,bits,fits", [(5000, 1 << 8, 30, True), (1 << 17, 1 << 8, 38, True), (1 << 17, 1 << 8, 41, False), (70000, 1 << 16, 36, True)])
+def test_rescaling_that_gives_its_output_an_int32_form(pv, orc, n, sf, bits, fits):
+    """Rescaling::rescale(X, true): output and proof transcript are the oracle's; the output keeps an int32 form exactly when
+    every rescaled value fits 32 bits (41-bit inputs over 2^8 do not); the remainders' int32 form serves the proof either way
+    (70000 and 5000 elements: padded; 2^17: read from the int32 form alone)."""
+    x = np.random.default_rng(n + bits).integers(-(1 << bits), 1 << bits, n)
+    x[0], x[1] = (1 << bits) - 1, -(1 << bits)
+    X = fr_array([int(v) % R_MOD for v in x])
+    orc.orc_seed(77)
+    orc.orc_transcript_clear()
+    e_out = np.zeros_like(X)
+    orc_check(orc.orc_rescale_prove(X, n, sf, e_out))
+    e_t = orc_transcript(orc)
+    pv.seed(77)
+    pv.transcript_begin()
+    out = pv.rescale_ints_prove(pv.from_fr(X), sf)
+    pv.lib.zkp_transcript_end()
+    assert (out.host() == e_out).all()
+    assert pv.folds_from_ints(out) == (1 if fits else 0)
+    t = pv.transcript()
+    assert t.shape == e_t.shape and (t == e_t).all()
+
+
+@pytest.mark.parametrize("D,low,length", [(1000, -16, 32), (100000, -16, 32), (1 << 17, -20, 40)])
+def test_mapping_lookup_with_int32_forms(pv, orc, D, low, length):
+    """tLookupRangeMapping with integer mapped values over queries that keep an int32 form: outputs, multiplicities and the
+    proof's transcript are the oracle's.  1000 queries: padded in both forms, the small job reads the field elements; 100000:
+    padded to 2^17 in the int32 form only (the job reads nothing else); 2^17: no padding."""
+    rng = np.random.default_rng(D + 1)
+    vals = rng.integers(low, low + length, D)
+    mvi = rng.integers(-2 ** 31, 2 ** 31, length).astype(np.int64)
+    mvi[0], mvi[1] = -2 ** 31, 2 ** 31 - 1
+    mv = fr_array([int(v) % R_MOD for v in mvi])
+    S = fr_array([int(v) % R_MOD for v in vals])
+    k = (D - 1).bit_length()
+    r, alpha, beta, u, v = ch(7, 1)[0], ch(8, 1)[0], ch(9, 1)[0], ch(10, k), ch(11, k)
+    size = 1 << (length - 1).bit_length()
+    e_y, e_m, e_fin = np.zeros((D, 8), np.uint32), np.zeros((size, 8), np.uint32), np.zeros(8, np.uint32)
+    orc.orc_transcript_clear()
+    orc_check(orc.orc_mapping(S, D, low, length, mv, r, alpha, beta, u, v, e_y, e_m, e_fin))
+    e_t = orc_transcript(orc)
+    hS = pv.from_i64(vals.astype(np.int64))
+    pv.keep_for_folds(hS)
+    assert pv.folds_from_ints(hS) == 1
+    pv.transcript_begin()
+    y, m, fin = pv.mapping(hS, low, length, pv.from_fr(mv), r, alpha, beta, u, v)
+    pv.lib.zkp_transcript_end()
+    assert pv.folds_from_ints(y) == 1
+    assert (y.host() == e_y).all() and (m.host() == e_m).all() and (fin == e_fin).all()
+    t = pv.transcript()
+    assert t.shape == e_t.shape and (t == e_t).all()
+
+
 def test_rescaling_prove_seeded_transcript(pv, orc):
     for n, sf in ((256, 16), (5000, 1 << 8)):
         x = np.random.default_rng(n).integers(-(1 << 30), 1 << 30, n)

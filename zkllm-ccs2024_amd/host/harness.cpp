@@ -313,6 +313,15 @@ void* zkp_rescale(void* X, u32 sf, void** rem_out) {
     return new FrTensor(std::move(out));
     ZKP_END_PTR
 }
+// Rescaling::rescale(X, true) + prove: the rescaled tensor comes back with its int32 form when every value fits
+void* zkp_rescale_ints_prove(void* X, u32 sf) {
+    ZKP_TRY
+    Rescaling rs(sf);
+    FrTensor out = rs.rescale(FT(X), true);
+    rs.prove(FT(X), out);
+    return new FrTensor(std::move(out));
+    ZKP_END_PTR
+}
 // Rescaling::operator() + prove with challenges from the seeded stream
 void* zkp_rescale_prove(void* X, u32 sf) {
     ZKP_TRY
