@@ -126,6 +126,12 @@ const void* zk_fr_fold_prepared_ints(const void* prepared);
 /* zk_fr_gather (out[i] = table[idx[i]], the mapped values of tLookupRangeMapping::operator(), tlookup.cu:446-470) that
  * also writes the int32 form of out from the table's own (table_prepared: a handle of zk_fr_fold_prepare over the table) */
 int zk_fr_gather_ints(void* out, void* out_ints, const void* table, const void* table_prepared, const void* idx, size_t n, void* stream);
+/* the same gather by the queries themselves: out[i] = table[queries[i] - low], queries and table given by their int32 forms,
+ * out_prepared a handle of zk_fr_fold_prepared_new that receives out's int32 form (a query outside the table reads entry 0:
+ * zk_lookup_index_i32, run before, reports those).  The handle remembers what it was gathered from: a mapped lookup job over
+ * these queries, these outputs and this table (zk_lookup_prove_begin_mapped_ints) then knows that every output is its
+ * query's table value and reads neither the outputs nor the per-entry integers in its first round. */
+int zk_fr_gather_by_queries_ints(void* out, void* out_prepared, const void* queries_prepared, int32_t low, const void* table_prepared, size_t n, void* stream);
 /* zk_fr_me_multi where prepareds[i], when non-null, is the int32 form of Xs[i] (same n): such tensors are read from it --
  * an eighth of the bytes, eight limb products per element instead of a Montgomery product.  Same values. */
 /* zk_fr_mul (out = a * b element by element) for two tensors given by their int32 forms: the products are exact 64-bit

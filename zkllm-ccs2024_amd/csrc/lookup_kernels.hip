@@ -473,7 +473,11 @@ template <int K> __global__ void __launch_bounds__(TPB) k_me_multi(Fr* __restric
 // is what these integers say (want[j], written by k_lookup_ints_check: the mapped integer of a consistent entry, 0 for a
 // consistent entry of a plain table, INTS_POISON for an entry that is something else), query and inverse are TB[2j], TB[2j+1].
 struct HintSrc { const Fr* TB; const Fr* hint; Fr low; Fr beta; uint32_t N; const Fr* S_out = nullptr; Fr r_mont;
-                 const int32_t* hint_ints = nullptr; const int32_t* sout_ints = nullptr; const int32_t* want = nullptr; int32_t low_int = 0; };
+                 const int32_t* hint_ints = nullptr; const int32_t* sout_ints = nullptr; const int32_t* want = nullptr; int32_t low_int = 0;
+                 // *any_bad == 0: every table entry is what the integers say (k_lookup_ints_check); trusted_out: the outputs were gathered from
+                 // this table by these queries (zk_fr_gather_by_queries_ints).  With both, a query inside the table needs neither its output
+                 // nor the entry's expected integer: nothing is gathered but the table record.
+                 const uint32_t* any_bad = nullptr; bool trusted_out = false; };
 static constexpr int32_t INTS_POISON = (int32_t)0x80000000;
 __device__ __forceinline__ Fr hinted_query(const Fr* __restrict__ S, size_t i, const HintSrc& h) {
     return h.S_out ? add(h.hint[i], mont_mul(h.r_mont, h.S_out[i])) : S[i];
@@ -504,24 +508,31 @@ __device__ __forceinline__ Fr inv_by_hint(const Fr& sv, size_t i, const HintSrc&
     return inv_plus_beta_alone(sv, h.beta);
 }
 // want[j] for the int32 path of the first round: TB[2j] must be low + j (+ r * mapped[j])
-__global__ void __launch_bounds__(TPB) k_lookup_ints_check(int32_t* __restrict__ want, const Fr* __restrict__ TB, const int32_t* __restrict__ mapped_ints, const Fr r_mont,
-                                                           int32_t low, uint32_t N) {
+__global__ void __launch_bounds__(TPB) k_lookup_ints_check(int32_t* __restrict__ want, uint32_t* __restrict__ any_bad, const Fr* __restrict__ TB,
+                                                           const int32_t* __restrict__ mapped_ints, const Fr r_mont, int32_t low, uint32_t N) {
     const uint32_t j = blockIdx.x * TPB + threadIdx.x;
     if (j >= N) return;
     Fr q = fr_from_i64((int64_t)low + (int64_t)j);
     if (mapped_ints) q = add(q, mont_mul(r_mont, fr_from_i64((int64_t)mapped_ints[j])));
     const bool ok = equal(q, TB[2 * (size_t)j]) && (!mapped_ints || mapped_ints[j] != INTS_POISON);
     want[j] = ok ? (mapped_ints ? mapped_ints[j] : 0) : INTS_POISON;
+    if (!ok) atomicOr(any_bad, 1u);
 }
 // query i and 1 / (query + beta) from the int32 forms (HintSrc); unit as in inv_by_hint
 __device__ __forceinline__ Fr query_inv_ints(size_t i, const HintSrc& h, Fr& a, bool& unit) {
     const int32_t hi = __builtin_nontemporal_load(h.hint_ints + i);
-    const int32_t so = h.sout_ints ? __builtin_nontemporal_load(h.sout_ints + i) : 0;
     const int64_t d = (int64_t)hi - (int64_t)h.low_int;
     const bool in_table = d >= 0 && d < (int64_t)h.N;
     const uint32_t j = in_table ? (uint32_t)d : 0u;
-    const int32_t w = h.want[j];
-    if (in_table && w != INTS_POISON && so == w) {
+    const bool sure = *h.any_bad == 0u && (!h.sout_ints || h.trusted_out);      // the same for every query of the job
+    int32_t so = 0;
+    bool match = in_table;
+    if (!sure || !in_table) {
+        so = h.sout_ints ? __builtin_nontemporal_load(h.sout_ints + i) : 0;
+        const int32_t w = h.want[j];
+        match = in_table && w != INTS_POISON && so == w;
+    }
+    if (match) {
         a = h.TB[2 * (size_t)j + 1];
         unit = !is_zero(a);
         return h.TB[2 * (size_t)j];
@@ -1215,7 +1226,10 @@ static int eq_table_queue(Fr* out, const uint32_t* u, int k, Arena& arena, hipSt
 // the bytes, and a product with an eq entry is eight limb products with no reduction.  The unreduced sum of a whole fold
 // fits ten limbs (entries below 2^255, magnitudes up to 2^31, up to 2^24 terms) and is reduced once: the low 256 bits by
 // one Montgomery product with 1 (the entries carry R), the two limbs above them count R each, which that product cancels.
-struct FoldPrepared { int32_t* ints = nullptr; size_t n = 0; };
+// id: unique per handle (the int32 form never changes once written).  src_*: set by zk_fr_gather_by_queries_ints -- element i
+// is entry (queries[i] - src_low) of the table with that id, for every query inside the table.
+struct FoldPrepared { int32_t* ints = nullptr; size_t n = 0; uint64_t id = 0, src_queries = 0, src_table = 0; int32_t src_low = 0; };
+static uint64_t fold_prepared_id() { static std::mutex mu; static uint64_t next = 0; std::lock_guard<std::mutex> lk(mu); return ++next; }
 struct EqPair { Fr e, ne; };        // an eq entry and its negative, Montgomery form
 __global__ void __launch_bounds__(TPB) k_fold_ints(int32_t* __restrict__ out, uint32_t* __restrict__ bad, const Fr* __restrict__ in, size_t n) {
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
@@ -1360,6 +1374,18 @@ __global__ void __launch_bounds__(TPB) k_mul_ints(Fr* __restrict__ out, const in
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (i < n) out[i] = fr_from_i64((int64_t)a[i] * (int64_t)b[i]);
 }
+// out[i] = table[queries[i] - low] from the int32 forms of queries and table (a query outside the table reads entry 0: the index
+// pass, run before, reports those)
+__global__ void __launch_bounds__(TPB) k_gather_by_queries(Fr* __restrict__ out, int32_t* __restrict__ out_ints, const int32_t* __restrict__ queries, int32_t low,
+                                                           const int32_t* __restrict__ table_ints, uint32_t N, size_t n) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    const int64_t d = (int64_t)queries[i] - (int64_t)low;
+    const uint32_t j = (d >= 0 && d < (int64_t)N) ? (uint32_t)d : 0u;
+    const int32_t v = table_ints[j];
+    out[i] = fr_from_i64((int64_t)v);
+    out_ints[i] = v;
+}
 // Multilinear evaluations at one point of KF (0 or 1) tensors of field elements and KI tensors given in int32 form, in one
 // pass over the point's eq table: an int32 element costs eight limb products into the lane's unreduced sum.
 struct MeIntPtrs { const int32_t* x[6]; };
@@ -1476,6 +1502,7 @@ int zk_fr_fold_prepare(void** prepared, const void* t, size_t n, void* stv) {
     FoldPrepared* fp = new FoldPrepared;
     fp->ints = (int32_t*)ints;
     fp->n = n;
+    fp->id = fold_prepared_id();
     *prepared = fp;
     return 0;
 }
@@ -1495,6 +1522,7 @@ int zk_fr_fold_prepared_new(void** prepared, void** ints_dev, size_t n, void* st
     FoldPrepared* fp = new FoldPrepared;
     fp->ints = (int32_t*)ints;
     fp->n = n;
+    fp->id = fold_prepared_id();
     *prepared = fp;
     *ints_dev = ints;
     return 0;
@@ -1504,6 +1532,17 @@ int zk_fr_gather_ints(void* out, void* out_ints, const void* table, const void* 
     const FoldPrepared* tp = (const FoldPrepared*)table_prepared;
     ZK_ARG(out != nullptr && out_ints != nullptr && table != nullptr && tp != nullptr && idx != nullptr, "zk_fr_gather_ints: null argument");
     LAUNCH1D(k_gather_ints, n, stv, (Fr*)out, (int32_t*)out_ints, (const Fr*)table, tp->ints, (const uint32_t*)idx, n);
+    return 0;
+}
+int zk_fr_gather_by_queries_ints(void* out, void* out_prepared, const void* queries_prepared, int32_t low, const void* table_prepared, size_t n, void* stv) {
+    FoldPrepared* o = (FoldPrepared*)out_prepared;
+    const FoldPrepared *q = (const FoldPrepared*)queries_prepared, *t = (const FoldPrepared*)table_prepared;
+    ZK_ARG(out != nullptr && o != nullptr && q != nullptr && t != nullptr, "zk_fr_gather_by_queries_ints: null argument");
+    ZK_ARG(o->n == n && q->n == n && t->n >= 1 && t->n <= 0xFFFFFFFFu, "zk_fr_gather_by_queries_ints: int32 forms of another size");
+    LAUNCH1D(k_gather_by_queries, n, stv, (Fr*)out, o->ints, q->ints, low, t->ints, (uint32_t)t->n, n);
+    o->src_queries = q->id;
+    o->src_table = t->id;
+    o->src_low = low;
     return 0;
 }
 int zk_fr_mul_ints(void* out, const void* a_prepared, const void* b_prepared, size_t n, void* stv) {
@@ -2039,10 +2078,18 @@ static int lookup_prove_begin(void** handle, const void* S, const void* T, const
         hs.TB = TB.as<Fr>(); hs.hint = (const Fr*)hint; hs.low = fr_from_i64((int64_t)low); hs.beta = b; hs.N = (uint32_t)N;
         if (S_out) { hs.S_out = (const Fr*)S_out; hs.r_mont = to_mont(load_fr(r)); }
         if (ints) {
-            Scratch& want = job->arena.add(sizeof(int32_t) * N);
+            Scratch& want = job->arena.add(sizeof(int32_t) * (N + 1));         // the last slot: any_bad
             if (want.rc) { rc = want.rc; sumjob_abort(job); return rc; }
             const int32_t* mi = S_out ? ((const FoldPrepared*)ints->mapped)->ints : nullptr;
-            hipLaunchKernelGGL(k_lookup_ints_check, dim3(cdiv(N, TPB)), dim3(TPB), 0, st, want.as<int32_t>(), TB.as<Fr>(), mi, hs.r_mont, low, (uint32_t)N);
+            uint32_t* any_bad = (uint32_t*)(want.as<int32_t>() + N);
+            hipError_t me = hipMemsetAsync(any_bad, 0, sizeof(uint32_t), st);
+            if (me != hipSuccess) { sumjob_abort(job); ZK_HIP(me); }
+            hipLaunchKernelGGL(k_lookup_ints_check, dim3(cdiv(N, TPB)), dim3(TPB), 0, st, want.as<int32_t>(), any_bad, TB.as<Fr>(), mi, hs.r_mont, low, (uint32_t)N);
+            hs.any_bad = any_bad;
+            if (S_out) {
+                const FoldPrepared *q = (const FoldPrepared*)ints->queries, *o = (const FoldPrepared*)ints->out, *mp = (const FoldPrepared*)ints->mapped;
+                hs.trusted_out = o->src_queries != 0 && o->src_queries == q->id && o->src_table == mp->id && o->src_low == low;
+            }
             hs.hint_ints = ((const FoldPrepared*)ints->queries)->ints;
             hs.sout_ints = S_out ? ((const FoldPrepared*)ints->out)->ints : nullptr;
             hs.want = want.as<int32_t>();

@@ -72,7 +72,11 @@ pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const FrTensor& vals) {
     FrTensor m = counts_to_m(idx.p, vals.size, table.size);
     FrTensor y(vals.size);
     // mapped values that are 32-bit integers: the outputs get their int32 form with them
-    if (const void* th = mapped_vals.kept_ints()) ZKC(zk_fr_gather_ints(y.gpu_data, y.ints_for_producer(), mapped_vals.gpu_data, th, idx.p, vals.size, nullptr));
+    if (const void* th = mapped_vals.kept_ints(); th && vals.kept_ints()) {
+        // queries with an int32 form: gathered by them, and the outputs' form remembers it (the proof's first round then trusts them)
+        y.ints_for_producer();
+        ZKC(zk_fr_gather_by_queries_ints(y.gpu_data, const_cast<void*>(y.kept_ints()), vals.kept_ints(), low, th, vals.size, nullptr));
+    } else if (th) ZKC(zk_fr_gather_ints(y.gpu_data, y.ints_for_producer(), mapped_vals.gpu_data, th, idx.p, vals.size, nullptr));
     else ZKC(zk_fr_gather(y.gpu_data, mapped_vals.gpu_data, idx.p, vals.size, nullptr));
     ZKC(zk_sync(nullptr));
     return {std::move(y), std::move(m)};
