@@ -165,7 +165,7 @@ def main():
         print(json.dumps({"pmc_probe": {"fold_pairs_per_launch": n_big // 2, "fold_launches": 3, "copy_kernel": "k_ew<0> (zk_fr_add)",
                                         "copy_read_bytes": 64 * n, "copy_write_bytes": 32 * n, "montmul_elements": n,
                                         "fold_axis_elements_in": 2048 * 4096, "msm_pairs": 11008 * 4096,
-                                        "lookup_first_round_pairs": 1 << 26, "lookup_first_round_algorithmic_bytes": (1 << 26) * 128}}))
+                                        "lookup_first_round_pairs": 1 << 26, "lookup_first_round_algorithmic_bytes": (1 << 26) * 120}}))
         return
 
     def ev():
@@ -327,8 +327,8 @@ def main():
             "kernel": "k_lookup_round<false,true> (first round of the hinted lookup sumchecks, every launch of the timed layers)", "bound": "hbm",
             "achieved": lk_bytes / (lk_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": lk_bytes / (lk_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "traffic": None, "launches": int(lk_launches), "pairs": int(lk_pairs), "total_ms_in_timed_region": lk_ms,
-            "note": "algorithmic bytes (per pair: the two queries -- 4 B each, 8 B for a mapping table's two tensors, where they are read from their int32 "
-                    "forms as the softmax planes and rescaling remainders are, else 32 B / 64 B; the eq weight 32 B; two folded values out 64 B; the next "
+            "note": "algorithmic bytes (per pair: the two queries -- 4 B each where they are read from their int32 forms as the softmax planes and rescaling "
+                    "remainders are (a mapping table's outputs are not read when they were gathered by these queries), else 32 B / 64 B; the eq weight 32 B; two folded values out 64 B; the next "
                     "round's eq table 16 B) over the summed launch durations; the launches share the device with each other and with the openings, and "
                     "with int32 queries the kernel is bound by its table gathers and instruction issue, not by these bytes"}
     if args.skip_extras:
@@ -480,11 +480,11 @@ def main():
                                         "bound": "hbm", "achieved": l_bytes / (l_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                         "frac": l_bytes / (l_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": l_ms / l_launches, "pairs": int(l_pairs),
                                         "whole_proof_ms": look_total_ms,
-                                        "note": "algorithmic 128 B per pair (two queries of two tensors read from their int32 forms: 16 B; eq weight, two folded values out, "
-                                                "next eq table); the kernel also gathers a 64-byte record (table entry and its inverse) and the entry's expected integer per "
-                                                "query from a 64 MiB and a 4 MiB table and does three field products and one unreduced one per pair: 1573 lane instructions "
-                                                "per pair, 45 % of the VALU issue slots, 24 GB moved with the gathers = 4 TB/s (SQ_INSTS_VALU, FETCH_SIZE, WRITE_SIZE of "
-                                                "this launch in profiles/fr_mul_fold_msm_pmc.txt) -- bound by the gathers; with the queries read as field elements (240 B per "
+                                        "note": "algorithmic 120 B per pair (two queries read from their int32 form: 8 B; eq weight, two folded values out, "
+                                                "next eq table); the kernel also gathers a 64-byte record (table entry and its inverse) per query from a 64 MiB table (the outputs "
+                                                "were gathered by these queries from this table and every entry is what the integers say, so nothing else is read per query) "
+                                                "and does three field products and one unreduced one per pair (SQ_INSTS_VALU, FETCH_SIZE, WRITE_SIZE of "
+                                                "this launch in profiles/fr_mul_fold_msm_pmc.txt) -- bound by the gathers and instruction issue; with the queries read as field elements (240 B per "
                                                 "pair) the same round took 7.6 ms.  The later rounds run at 3.6 TB/s and 79 % of the VALU slots (instruction issue binds there)"}
     del keep, look
 

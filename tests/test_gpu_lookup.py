@@ -508,6 +508,71 @@ def test_mapped_lookup_job_equals_the_plain_one_on_the_combined_queries(k):
         hip.free(p)
 
 
+@pytest.mark.parametrize("k,bad_entry", [(17, False), (17, True), (13, False)])
+def test_mapped_lookup_over_outputs_gathered_by_their_queries(k, bad_entry):
+    """Outputs made by zk_fr_gather_by_queries_ints carry where they came from; a mapped job over the same queries, outputs and
+    table then reads neither outputs nor per-entry integers for queries inside the table.  Checked against the plain job on
+    the combined queries (big integers), with queries outside the table (their output is entry 0's value and must be read),
+    and with one table entry that is not what the integers say (the job falls back to checking every query)."""
+    import ctypes
+    from gpuhelp import Hip, c_void_p, c_size_t, c_int
+    hip = Hip()
+    D, N, low = 1 << k, 64, -9
+    rng = np.random.default_rng(2000 + k + bad_entry)
+    mapped = [int(x) for x in rng.integers(-2 ** 31, 2 ** 31, N)]
+    r_fr, beta = ch(82, 1)[0], ch(83, 1)[0]
+    r = fr_ints(r_fr.reshape(1, 8))[0]
+    pos = rng.integers(0, N, D)
+    s_in = [int(p) + low for p in pos]
+    outside = rng.choice(D, 200, replace=False)
+    for i in outside[:100]:
+        s_in[i] = low + N + 1 + int(i % 1000)
+    for i in outside[100:]:
+        s_in[i] = low - 1 - int(i % 1000)
+    dSi = hip.upload(fr_array([x % R_MOD for x in s_in]))
+    dMp = hip.upload(fr_array([x % R_MOD for x in mapped]))
+    hq, hm = c_void_p(), c_void_p()
+    hip.call("zk_fr_fold_prepare", ctypes.byref(hq), c_void_p(dSi), c_size_t(D), None)
+    hip.call("zk_fr_fold_prepare", ctypes.byref(hm), c_void_p(dMp), c_size_t(N), None)
+    dSo = hip.malloc(32 * D)
+    ho, hoq = c_void_p(), c_void_p()
+    hip.call("zk_fr_fold_prepared_new", ctypes.byref(ho), ctypes.byref(hoq), c_size_t(D), None)
+    hip.call("zk_fr_gather_by_queries_ints", c_void_p(dSo), ho, hq, c_int(low), hm, c_size_t(D), None)
+    s_out = [mapped[x - low] if 0 <= x - low < N else mapped[0] for x in s_in]
+    assert fr_ints(hip.download(dSo, (D, 8), np.uint32)) == [x % R_MOD for x in s_out]
+    assert (hip.download(hoq.value, (D,), np.int32) == np.array(s_out)).all()
+    Tl = [((low + j) + r * mapped[j]) % R_MOD for j in range(N)]
+    if bad_entry:
+        Tl[17] = (Tl[17] + 3) % R_MOD
+    S_com = fr_array([(a + r * o) % R_MOD for a, o in zip(s_in, s_out)])
+    index_of = {}
+    for j, t in enumerate(Tl):
+        index_of.setdefault(t, j)
+    m_counts = np.zeros(N, np.int64)
+    for q in fr_ints(S_com):
+        if q in index_of:
+            m_counts[index_of[q]] += 1
+    dS, dT, dm = hip.upload(S_com), hip.upload(fr_array(Tl)), hip.upload(fr_array([int(c) for c in m_counts]))
+    u, v = ch(84, k - 1), ch(85, k)
+    res = []
+    for job in ("plain", "mapped_ints"):
+        h = c_void_p()
+        if job == "plain":
+            hip.call("zk_lookup_prove_begin", ctypes.byref(h), c_void_p(dS), c_void_p(dT), c_void_p(dm), beta, u, v, c_size_t(D), c_size_t(N), c_int(k), None)
+        else:
+            hip.call("zk_lookup_prove_begin_mapped_ints", ctypes.byref(h), c_void_p(dSi), hq, c_void_p(dSo), ho, hm, r_fr, c_void_p(dT), c_void_p(dm), c_int(low),
+                     beta, u, v, c_size_t(D), c_size_t(N), c_int(k), None)
+        bm, sums = np.zeros(8, np.uint32), np.zeros((k * 11, 8), np.uint32)
+        hip.call("zk_lookup_prove_end", h, bm, sums)
+        res.append((bm, sums))
+    assert (res[0][0] == res[1][0]).all() and (res[0][1] == res[1][1]).all()
+    assert res[0][1].any()
+    for h in (hq, hm, ho):
+        hip.call("zk_fr_fold_prepared_free", h)
+    for q in (dSi, dMp, dSo, dS, dT, dm):
+        hip.free(q)
+
+
 @pytest.mark.parametrize("rows,cols", [(5, 64), (37, 200), (64, 2048)])
 def test_softmax_shift_and_decomposition_in_one_pass_equal_the_two_passes(rows, cols):
     """zk_softmax_shift_decompose against zk_softmax_shift followed by zk_softmax_decompose_ints: the same shifts, shifted

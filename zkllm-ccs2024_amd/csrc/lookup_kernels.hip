@@ -1847,7 +1847,7 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
                 // per pair: two queries (32 B each; a mapping table's query is two tensors), the eq weight (32 B), two folded values
                 // written (64 B), the next round's eq table (16 B)
                 // (queries read from their int32 forms: 4 B each)
-                const double q = hs->hint_ints ? (hs->sout_ints ? 16.0 : 8.0) : (hs->S_out ? 128.0 : 64.0);
+                const double q = hs->hint_ints ? ((hs->sout_ints && !hs->trusted_out) ? 16.0 : 8.0) : (hs->S_out ? 128.0 : 64.0);      // (trusted outputs are not read)
                 g_round_timer.bytes += (double)half * (q + 32.0 + 64.0 + (nE ? 16.0 : 0.0));
             }
         }
