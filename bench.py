@@ -51,6 +51,8 @@ def main():
                          "0 = head by head, the flow of self-attn.cu per head")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extras", action="store_true", help="only the layer timing (used for profiling runs)")
+    ap.add_argument("--at-claim", action="store_true",
+                    help="the timed layers start every weight opening at its claim (what layer_openings_at_claim_s reports); for profiling runs")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: three launches of the opening's fold kernel at 262144 pairs, one hinted lookup "
                          "sumcheck over 2^27 queries, the Montgomery product, the three-level fold, the commitment of config 3 and one "
@@ -215,6 +217,8 @@ def main():
     os.dup2(devnull, 1)      # the class layer prints the reference's progress lines ("Opening complete", ...)
     try:
         parts = np.zeros(8)
+        if args.at_claim:
+            pv.lib.zkp_openings_set_only_at_claim(1)
         for _ in range(args.warmup):
             pv.layer_run(layer, hX)
         pv.sync()
@@ -230,6 +234,27 @@ def main():
         lk_ms, lk_launches, lk_pairs, lk_bytes = read_lookup_timer()
         # the same layer without its nine openings (the G1 part of verifyWeightClaim switched off), and the nine commitments alone
         noopen_s = commit_ms = nocross_s = None
+        # The same layer with every opening started at its claim or later (no challenge is read before the prover has drawn it in
+        # the reference's order): the openings of a block that are claimed close together run as one batched job, with the
+        # same row / cross commitments and three-round folds as the planned run.
+        at_claim_parts = np.zeros(8)
+        at_claim_s = None
+        if args.at_claim:
+            at_claim_s, at_claim_parts = wall / args.steps, parts / args.steps
+        elif not (args.skip_extras and args.skip_cpu):
+            pv.lib.zkp_openings_set_only_at_claim(1)
+            try:
+                pv.layer_run(layer, hX)
+                pv.sync()
+                t1 = time.perf_counter()
+                for _ in range(3):
+                    _, times = pv.layer_run(layer, hX)
+                    at_claim_parts += times
+                pv.sync()
+                at_claim_s = (time.perf_counter() - t1) / 3
+                at_claim_parts /= 3
+            finally:
+                pv.lib.zkp_openings_set_only_at_claim(0)
         if not args.skip_extras:
             pv.layer_set(layer, open_weights=False)
             pv.layer_run(layer, hX)
@@ -298,6 +323,8 @@ def main():
                    "parts_note": "host-side block times; the openings run on the library's streams from the start of the layer, so the first blocks' "
                                  "figures include the time their kernels share the device with them"},
     }
+    out["layer_openings_at_claim_s"] = at_claim_s
+    out["layer_openings_at_claim_parts_ms"] = {k: round(float(v), 1) for k, v in zip(["rmsnorm1", "qkv", "attention", "oproj", "rmsnorm2", "ffn", "total", "open_wait"], at_claim_parts)}
     if noopen_s is not None:
         out["layer_without_openings_s"] = noopen_s
         # what is made of the weights once, at commit time: the nine public commitments and their cross commitments

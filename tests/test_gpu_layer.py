@@ -87,6 +87,46 @@ def test_layer_run_again_starts_its_openings_ahead_and_proves_the_same(pv):
     pv.layer_free(layer)
 
 
+def test_tiny_layer_with_every_opening_started_at_its_claim(pv):
+    """zkp_openings_set_only_at_claim (ZKLLM_OPEN_AHEAD=0): no plan is learned or used and nothing starts ahead inside a block;
+    the openings of a block start together at its last claim.  Transcript and G1 points are those of the default run."""
+    orc = load_oracle()
+    cu, cf = layercfg.tiny(open_weights=True, head_group=2)
+    ws = layercfg.tiny_weights(23, cu)
+    S, E = int(cu[0]), int(cu[1])
+    X = np.round(np.random.default_rng(33).normal(0, 1, (S, E)) * 256).astype(np.int32)
+    exp = np.zeros((S * E, 8), np.uint32)
+    orc.orc_seed(12)
+    orc.orc_transcript_clear()
+    orc_check(orc.orc_layer(cu, cf, *ws, 1, X, exp, None))
+    exp_t = orc_transcript(orc)
+    pv.seed(12)
+    layer = pv.layer_create(cu, cf, ws, 1)
+    pv.lib.zkp_challenge_position.restype = ctypes.c_ulonglong
+    pv.lib.zkp_challenge_skip.argtypes = [ctypes.c_ulonglong]
+    layer_draws = pv.lib.zkp_challenge_position()
+    g1s = []
+    try:
+        for at_claim in (1, 1, 0, 0):
+            pv.lib.zkp_openings_set_only_at_claim(at_claim)
+            pv.seed(12)
+            pv.lib.zkp_challenge_skip(ctypes.c_ulonglong(layer_draws))
+            pv.transcript_begin()
+            out, _ = pv.layer_run(layer, pv.from_i32(X))
+            pv.lib.zkp_transcript_end()
+            got_t = pv.transcript()
+            assert (out.host() == exp).all()
+            assert got_t.shape == exp_t.shape and (got_t == exp_t).all()
+            g1s.append(pv.transcript_g1().copy())
+            # runs that only open at the claim neither learn nor use a plan
+            assert pv.lib.zkp_layer_planned_openings(ctypes.c_void_p(layer)) == (0 if at_claim or len(g1s) < 3 else 9)
+    finally:
+        pv.lib.zkp_openings_set_only_at_claim(0)
+    pv.layer_free(layer)
+    for g in g1s[1:]:
+        assert g.shape == g1s[0].shape and (g == g1s[0]).all()
+
+
 def test_full_shape_layer_gives_one_output_head_by_head_and_stacked(pv):
     """LLaMa-2-7B shape, seq 2048 (tensors of up to 2^27 elements in the stacked proof, beyond what the oracle can follow):
     every proof of the layer runs through its in-prover identities in both attention variants (a failed identity throws),
@@ -112,27 +152,39 @@ def test_full_shape_layer_gives_one_output_head_by_head_and_stacked(pv):
     pv.seed(2024)
     layer = pv.layer_create_random(cu_o, cf_o, 7, 5)
     pv.layer_set(layer, head_group=32)
-    pv.seed(5)
-    pv.transcript_begin()
-    out, _ = pv.layer_run(layer, X)
-    pv.lib.zkp_transcript_end()
+    # First with neither row nor cross commitments: each weight opened at its claim, every T, T0, T1 a sum over all generators
+    # (commitment.cu:109-129) and every round a fold of its own.
+    pv.lib.zkp_openings_use_row_commitments(0)
+    try:
+        pv.seed(5)
+        pv.transcript_begin()
+        out, _ = pv.layer_run(layer, X)
+        pv.lib.zkp_transcript_end()
+    finally:
+        pv.lib.zkp_openings_use_row_commitments(1)
     assert pv.transcript().shape[0] == sizes[1] + 9
     assert (out.host() == outs[0]).all()
     del out
-    # That run opened each weight where the reference does, every T as a sum over all generators.  The next one starts the
-    # nine openings with the layer, batched, the first two rounds on the prepared tables and T of the first round from the
-    # weights' row commitments: it must deliver the same field elements and the same G1 points.
     first_t, first_g1 = pv.transcript().copy(), pv.transcript_g1().copy()
     assert pv.lib.zkp_layer_planned_openings(ctypes.c_void_p(layer)) == 9
-    pv.seed(5)
-    pv.transcript_begin()
-    out, _ = pv.layer_run(layer, X)
-    pv.lib.zkp_transcript_end()
-    assert (out.host() == outs[0]).all()
-    del out
-    again_t, again_g1 = pv.transcript(), pv.transcript_g1()
-    assert again_t.shape == first_t.shape and (again_t == first_t).all()
-    assert again_g1.shape == first_g1.shape and first_g1.shape[0] > 9 * 30 and (again_g1 == first_g1).all()
+    # The next run starts the nine openings ahead of their claims from the learned plan, batched, T / T0 / T1 of the first three
+    # rounds from the weights' row and cross commitments and those rounds as one fold; the one after it starts every opening
+    # at its claim (the openings of a block as one job, same commitments, same folds).  Both must deliver the field elements and
+    # the G1 points of the first.
+    for at_claim in (0, 1):
+        pv.lib.zkp_openings_set_only_at_claim(at_claim)
+        try:
+            pv.seed(5)
+            pv.transcript_begin()
+            out, _ = pv.layer_run(layer, X)
+            pv.lib.zkp_transcript_end()
+        finally:
+            pv.lib.zkp_openings_set_only_at_claim(0)
+        assert (out.host() == outs[0]).all()
+        del out
+        again_t, again_g1 = pv.transcript(), pv.transcript_g1()
+        assert again_t.shape == first_t.shape and (again_t == first_t).all(), at_claim
+        assert again_g1.shape == first_g1.shape and first_g1.shape[0] > 9 * 30 and (again_g1 == first_g1).all(), at_claim
     pv.layer_free(layer)
     assert (outs[0] == outs[1]).all() and (outs[0] == outs[2]).all()
     assert np.unique(outs[0], axis=0).shape[0] > 1000

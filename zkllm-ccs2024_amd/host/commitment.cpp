@@ -1,9 +1,11 @@
 #include <cstring>
 #include "commitment.hpp"
 
+#include <cstdio>
 #include <cstdlib>
 
 #include "../../include/zkllm_hip.h"
+#include "ioutils.hpp"
 
 #define ZKC(call) zk_check((call), #call)
 
@@ -160,7 +162,8 @@ void Commitment::open_start_batch(const std::vector<std::pair<const Commitment*,
         if (!g_skip_g1 && c->prepared)
             for (size_t j = i + 1; j < ops.size() && group.size() < 8; ++j)
                 if (!done[j] && ops[j].first->prepared && ops[j].first->size == c->size && ops[j].second->u_in.size() == p->u_in.size()) group.push_back(j);
-        if (group.size() == 1) { c->open_start(*p); done[i] = true; continue; }
+        // one opening alone is a job of its own kind only when nothing of the batched path applies to it
+        if (group.size() == 1 && (g_skip_g1 || !c->prepared || !p->row_com)) { c->open_start(*p); done[i] = true; continue; }
         auto b = std::make_shared<Pending::Batch>();
         b->count = (int)group.size();
         b->rounds = (int)p->u_in.size();
@@ -247,12 +250,22 @@ Fr_t Commitment::open(const FrTensor& t, const G1TensorJacobian& com, const vect
     return open(t, com, u, proof);
 }
 
+// how many rounds of cross commitments an opening over `generator_size` generators can use, at most `want`
+static int usable_cross_rounds(uint generator_size, int want) {
+    if (generator_size & (generator_size - 1)) return 0;
+    int most = 0;
+    for (uint n = generator_size; n > 2048 && !(n & 1u); n >>= 1) ++most;       // halving rounds of an opening over these generators
+    return std::max(0, std::min(std::min(want, most), 4));
+}
+static uint cross_patterns(int rounds) {
+    uint patterns = 1;
+    for (int q = 0; q < rounds; ++q) patterns += 2u << (2 * q);
+    return patterns;
+}
 void prepare_weight_cross(Weight& w, int rounds) {
     if (const char* e = getenv("ZKLLM_OPEN_CROSS_ROUNDS")) rounds = atoi(e);
-    int most = 0;
-    for (uint n = w.generator.size; n > 2048 && !(n & 1u); n >>= 1) ++most;       // halving rounds of an opening over these generators
-    rounds = std::max(0, std::min(std::min(rounds, most), 4));
-    if (rounds == 0 || (w.generator.size & (w.generator.size - 1))) { w.cross.reset(); w.cross_rounds = 0; return; }
+    rounds = usable_cross_rounds(w.generator.size, rounds);
+    if (rounds == 0) { w.cross.reset(); w.cross_rounds = 0; return; }
     const bool ragged = w.in_dim != (1u << ceilLog2(w.in_dim)) || w.out_dim != (1u << ceilLog2(w.out_dim));
     try {
         std::unique_ptr<FrTensor> local;
@@ -266,11 +279,41 @@ void prepare_weight_cross(Weight& w, int rounds) {
     }
 }
 
+// The cross commitments of a weight as a file beside its commitment file (an addition: commit_param_file writes it,
+// create_weight reads it when it is there): [pattern][row] points with z = ONE, pattern 0 the commitment itself, 1 + 2 + 8
+// + 32 patterns for three rounds.  The pattern count names the rounds; pattern 0 must equal the commitment file's points,
+// so a side file left over from another commitment is ignored.
+string cross_commitment_filename(const string& com_filename) { return com_filename + ".cross"; }
+static bool load_weight_cross(Weight& w, const string& com_filename) {
+    const string name = cross_commitment_filename(com_filename);
+    FILE* f = fopen(name.c_str(), "rb");
+    if (!f) return false;
+    fclose(f);
+    const size_t bytes = findsize(name);
+    const uint rows = w.com.size;
+    if (rows == 0 || bytes % (sizeof(G1Jacobian_t) * (size_t)rows)) return false;
+    const uint patterns = (uint)(bytes / (sizeof(G1Jacobian_t) * (size_t)rows));
+    int rounds = -1;
+    for (int q = 0; q <= 4; ++q) if (cross_patterns(q) == patterns) rounds = q;
+    if (rounds < 1 || rounds != usable_cross_rounds(w.generator.size, rounds)) return false;
+    if (const char* e = getenv("ZKLLM_OPEN_CROSS_ROUNDS")) if (atoi(e) < rounds) return false;
+    auto x = std::make_shared<G1TensorJacobian>(name);
+    // pattern 0 against the commitment that was loaded (both files hold normalised points; a commitment file in another
+    // Jacobian form is normalised for the comparison)
+    std::vector<G1Jacobian_t> a(rows), b(rows);
+    G1TensorJacobian cn = w.com.normalized();
+    ZKC(zk_memcpy_d2h(a.data(), x->gpu_data, sizeof(G1Jacobian_t) * (size_t)rows, nullptr));
+    ZKC(zk_memcpy_d2h(b.data(), cn.gpu_data, sizeof(G1Jacobian_t) * (size_t)rows, nullptr));
+    if (memcmp(a.data(), b.data(), sizeof(G1Jacobian_t) * (size_t)rows) != 0) return false;
+    w.cross = x;
+    w.cross_rounds = rounds;
+    return true;
+}
+
 Weight create_weight(string generator_filename, string weight_filename, string com_filename, uint in_dim, uint out_dim) {
     Commitment generator(generator_filename);
     FrTensor weight = FrTensor::from_int_bin(weight_filename);
     G1TensorJacobian com(com_filename);
-    generator.prepare_openings();
     Weight w{generator, weight, com, in_dim, out_dim, nullptr};
     w.weight.keep_for_folds();          // proofs and openings fold it at a new point each time
     if (in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim))) {
@@ -278,6 +321,10 @@ Weight create_weight(string generator_filename, string weight_filename, string c
         pd->keep_for_folds();
         w.padded = pd;
     }
+    // with three rounds of cross commitments from the side file the openings fold three rounds at once: the generators get
+    // those tables; otherwise the tables of the first two rounds
+    load_weight_cross(w, com_filename);
+    w.generator.prepare_openings(w.cross_rounds >= 3 ? 3 : 2);
     return w;
 }
 
@@ -290,7 +337,19 @@ uint commit_param_file(const string& generator_filename, const string& param_fil
     FrTensor param = FrTensor::from_int_bin(param_filename);
     if (param.size != in_dim * out_dim) throw std::runtime_error("commit-param: the parameter file does not hold in_dim x out_dim values");
     const bool ragged = in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim));
-    G1TensorJacobian com = ragged ? generator.commit_int(param.pad({in_dim, out_dim})) : generator.commit_int(param);
+    std::unique_ptr<FrTensor> padded;
+    if (ragged) padded.reset(new FrTensor(param.pad({in_dim, out_dim})));
+    const FrTensor& t = ragged ? *padded : param;
+    G1TensorJacobian com = generator.commit_int(t);
     com.normalized().save(output_filename);
+    // addition: the cross commitments of the first three opening rounds beside the commitment (seven times its work; what
+    // create_weight picks up so that verifyWeightClaim needs no sums over all generators in those rounds).
+    // ZKLLM_COMMIT_CROSS=0 leaves the side file out, =k writes k rounds.
+    int rounds = 3;
+    if (const char* e = getenv("ZKLLM_COMMIT_CROSS")) rounds = atoi(e);
+    rounds = usable_cross_rounds(generator.size, rounds);
+    const string side = cross_commitment_filename(output_filename);
+    if (rounds > 0) generator.cross_commitments(t, com, rounds).normalized().save(side);
+    else std::remove(side.c_str());          // never leave a side file of an older commitment behind
     return com.size;
 }

@@ -100,10 +100,14 @@ struct Weight {
 // integers is left without (commit_int refuses them).
 void prepare_weight_cross(Weight& w, int rounds = 3);
 
+// (commitment.cu:143-148) Also prepares the generators for openings and, when the side file cross_commitment_filename(com_filename)
+// is there and belongs to this commitment, takes the weight's cross commitments from it.
 Weight create_weight(string generator_filename, string weight_filename, string com_filename, uint in_dim, uint out_dim);
+string cross_commitment_filename(const string& com_filename);
 
 // The flow of the commit-param executable (commit-param.cu:4-29): loads the generators and the int32 parameter file, pads,
-// commits with commit_int and saves the commitment with z = ONE; returns the number of points written.
+// commits with commit_int and saves the commitment with z = ONE; returns the number of points written.  Addition: writes the
+// weight's cross commitments beside it (cross_commitment_filename; ZKLLM_COMMIT_CROSS=0 turns that off).
 uint commit_param_file(const string& generator_filename, const string& param_filename, const string& output_filename, uint in_dim, uint out_dim);
 
 // When set, Commitment::open skips the G1 part of the opening (whose result the reference computes and

@@ -541,6 +541,10 @@ void zkp_layer_set_open_weights(void* h, int on) { reinterpret_cast<LayerState*>
 // setup times of the last zkp_layer_create_random (ms): weights, generators, commitments, prepared generators
 void zkp_layer_setup_times(double* out4) { const LayerSetupTimes& t = layer_setup_times(); out4[0] = t.weights; out4[1] = t.generators; out4[2] = t.commitments; out4[3] = t.prepare; }
 void zkp_openings_use_cross_commitments(int on) { zk_openings_use_cross_commitments(on != 0); }
+void zkp_openings_use_row_commitments(int on) { zk_openings_use_row_commitments(on != 0); }
+// on: every weight opening starts at its claim or later (no learned plan, nothing started ahead inside a block)
+void zkp_openings_set_only_at_claim(int on) { zk_openings_set_only_at_claim(on != 0); }
+int zkp_openings_only_at_claim() { return zk_openings_only_at_claim() ? 1 : 0; }
 double zkp_layer_setup_cross_ms() { return layer_setup_times().cross; }      // the cross commitments of the nine weights (prepare_weight_cross)
 // the nine commitments of the layer computed once more (ms); negative on error
 double zkp_layer_recommit_ms(void* h) {

@@ -123,12 +123,14 @@ void attn_linear_block(const LayerConfig& c, const Weight& q, const Weight& k, c
     q_rescale.prove_end(pq);
     k_rescale.prove_end(pk);
     v_rescale.prove_end(pv);
+    OpeningGroup together;      // the three openings claimed below run as one device job, queued at the last claim
     auto ck = k_layer.prove(input, K);
     if (c.open_weights) verifyWeightClaim(k, ck[0]);
     auto cq = q_layer.prove(input, Q);
     if (c.open_weights) verifyWeightClaim(q, cq[0]);
     auto cv = v_layer.prove(input, V);
     if (c.open_weights) verifyWeightClaim(v, cv[0]);
+    together.end();
 }
 
 // columns [h*d, (h+1)*d) of a seq x embed tensor as a contiguous seq x d tensor
@@ -372,11 +374,13 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
     hidden_rescale.prove_end(ph);
     tLookup::prove_end(ps);
     gate_rescale.prove_end(pg);
+    OpeningGroup gate_and_up;   // when nothing was started ahead: the two openings over the same generator count as one job, queued at up's claim
     auto cg = gate_layer.prove(input, gate_out, ch_g);
     if (c.open_weights) verifyWeightClaim(gate, cg[0], og);
     up_rescale.prove_end(pu);
     auto cu = up_layer.prove(input, up_out, ch_u);
     if (c.open_weights) verifyWeightClaim(up, cu[0], ou);
+    gate_and_up.end();
     // the reference's executable saves the unrescaled down_out (ffn.cu:81); the rescaled tensor is what the next block consumes
     if (down_out_unrescaled) down_out_unrescaled->reset(new FrTensor(std::move(down_out)));
     return down_out_;
@@ -384,8 +388,9 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
 
 FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor& X, LayerTimes* times) {
     LayerTimes t;
-    static const bool ahead_off = [] { const char* e = getenv("ZKLLM_OPEN_AHEAD"); return e && e[0] == '0'; }();
-    DeferredOpenings openings(c.open_weights && !ahead_off ? w.plan.get() : nullptr);       // the nine weight openings run on the device beside the sumchecks
+    // the nine weight openings run on the device beside the sumchecks; with a learned plan they start ahead of their claims
+    // (not with ZKLLM_OPEN_AHEAD=0 / zk_openings_set_only_at_claim: then each starts at its claim)
+    DeferredOpenings openings(c.open_weights ? w.plan.get() : nullptr, {&w.input_norm, &w.q, &w.k, &w.v, &w.o, &w.post_norm, &w.up, &w.gate, &w.down});
     const double t0 = now_ms();
     FrTensor rms1 = compute_rms_inv(X, c.seq_len, c.embed_dim, c.rms_eps, c.value_scale);
     FrTensor n1 = rmsnorm_block(c, w.input_norm, X, rms1);

@@ -12,6 +12,8 @@ struct DeferredOpenings::Item {
     Commitment::Pending op;
     Fr_t claim;
     size_t slot;
+    const Commitment* gen = nullptr;      // for an item whose job is not queued yet
+    bool started = true;
 };
 struct DeferredOpenings::Ahead {
     Commitment::Pending op;
@@ -21,26 +23,37 @@ struct DeferredOpenings::Ahead {
 static thread_local DeferredOpenings* g_deferred = nullptr;
 static bool g_use_cross = true;
 void zk_openings_use_cross_commitments(bool on) { g_use_cross = on; }
+static bool g_use_rows = [] { const char* v = getenv("ZKLLM_OPEN_T_FROM_COM"); return !(v && v[0] == '0'); }();
+void zk_openings_use_row_commitments(bool on) { g_use_rows = on; }
+static bool g_only_at_claim = [] { const char* e = getenv("ZKLLM_OPEN_AHEAD"); return e && e[0] == '0'; }();
+bool zk_openings_only_at_claim() { return g_only_at_claim; }
+void zk_openings_set_only_at_claim(bool on) { g_only_at_claim = on; }
 static const FrTensor& padded_form(const Weight& w, std::unique_ptr<FrTensor>& local);
+// The rows of a weight folded at an opening's point, with what a batched start may use in place of sums over all
+// generators: the weight's row commitments (Weight::com is the commitment of its padded rows, proof.cu:3-10 /
+// commitment.cu:133-141) and its cross commitments when it carries them.
+static Commitment::Pending fold_weight(const Weight& w, const vector<Fr_t>& u_cat) {
+    std::unique_ptr<FrTensor> local;
+    const bool cross = g_use_rows && g_use_cross && w.cross;
+    return w.generator.open_fold(padded_form(w, local), w.com, u_cat, g_use_rows, cross ? w.cross.get() : nullptr, cross ? w.cross_rounds : 0);
+}
 DeferredOpenings::DeferredOpenings() : prev(g_deferred) { g_deferred = this; }
-DeferredOpenings::DeferredOpenings(OpeningPlan* pl) : prev(g_deferred), plan(pl) {
+DeferredOpenings::DeferredOpenings(OpeningPlan* pl, const std::vector<const Weight*>& ws) : prev(g_deferred), plan(g_only_at_claim ? nullptr : pl), weights(ws) {
     g_deferred = this;
     if (!plan) return;
     base = zk_challenge_position();
-    if (!plan->learned) { learning = true; plan->entries.clear(); return; }
+    bool usable = plan->learned;
+    for (const OpeningPlan::Entry& e : plan->entries) usable = usable && e.which < weights.size();
+    if (!usable) { plan->learned = false; learning = true; plan->entries.clear(); return; }
     // every opening of the plan: rows folded first (the folds are passes over whole weights on the caller's stream), then
     // the G1 recursions queued
     try {
         for (const OpeningPlan::Entry& e : plan->entries) {
             Ahead* a = new Ahead;
             ahead.push_back(a);
-            a->w = e.w;
+            a->w = weights[e.which];
             a->u_cat = concatenate(vector<vector<Fr_t>>({zk_challenge_peek(e.pos[1], e.len[1]), zk_challenge_peek(e.pos[0], e.len[0])}));
-            std::unique_ptr<FrTensor> local;
-            // a Weight's com is the commitment of its (padded) rows: the batched start may use it for the first round's T
-            static const bool t_from_rows = [] { const char* v = getenv("ZKLLM_OPEN_T_FROM_COM"); return !(v && v[0] == '0'); }();
-            const bool cross = g_use_cross && e.w->cross;
-            a->op = e.w->generator.open_fold(padded_form(*e.w, local), e.w->com, a->u_cat, t_from_rows, cross ? e.w->cross.get() : nullptr, cross ? e.w->cross_rounds : 0);
+            a->op = fold_weight(*a->w, a->u_cat);
         }
         // the longest recursions first; openings of one size run as one job
         std::vector<Ahead*> order(ahead);
@@ -82,6 +95,21 @@ void DeferredOpenings::start() {
 }
 int DeferredOpenings::start_at_claim = [] { const char* e = getenv("ZKLLM_OPEN_START_AT_CLAIM"); return e ? atoi(e) : 0; }();
 void zk_openings_start_now() { if (g_deferred) g_deferred->start(); }
+void DeferredOpenings::flush() {
+    if (unstarted.empty()) return;
+    std::vector<std::pair<const Commitment*, Commitment::Pending*>> ops;
+    for (Item* it : unstarted) ops.emplace_back(it->gen, &it->op);
+    Commitment::open_start_batch(ops);          // throws before anything of these is marked: finish() tries again and reports
+    for (Item* it : unstarted) it->started = true;
+    unstarted.clear();
+}
+OpeningGroup::OpeningGroup() : scope(g_deferred) { if (scope) ++scope->group_depth; }
+void OpeningGroup::end() {
+    DeferredOpenings* d = scope;
+    scope = nullptr;
+    if (d && --d->group_depth == 0) d->flush();
+}
+OpeningGroup::~OpeningGroup() { try { end(); } catch (...) {} }
 DeferredOpenings::~DeferredOpenings() {
     g_deferred = prev;
     for (auto& ia : claimed_early) delete ia.second;          // never started: nothing to wait for
@@ -90,12 +118,14 @@ DeferredOpenings::~DeferredOpenings() {
         if (a) { try { vector<G1Jacobian_t> drop; Commitment::open_end(a->op, drop); } catch (...) {} delete a; }
     }
     for (Item* it : items) {          // only reached with pending items when an exception unwinds: release them
-        try { vector<G1Jacobian_t> drop; Commitment::open_end(it->op, drop); } catch (...) {}
+        if (it->started) { try { vector<G1Jacobian_t> drop; Commitment::open_end(it->op, drop); } catch (...) {} }
         delete it;
     }
 }
 void DeferredOpenings::finish() {
     start();
+    group_depth = 0;
+    flush();
     if (learning && plan) { plan->learned = true; learning = false; }
     std::vector<Item*> todo;
     todo.swap(items);
@@ -125,21 +155,29 @@ static const FrTensor& padded_form(const Weight& w, std::unique_ptr<FrTensor>& l
     local.reset(new FrTensor(w.weight.pad({w.in_dim, w.out_dim})));
     return *local;
 }
-// while a plan is being learned: where this opening's point was drawn; a point that is not two recent draws ends the
-// learning (nothing runs ahead then)
+// while a plan is being learned: where this opening's point was drawn; a point that is not two recent draws, or a weight
+// that is not one of the scope's, ends the learning (nothing runs ahead then)
 void DeferredOpenings::learn(const Weight& w, const Claim& c) {
     if (!learning) return;
-    OpeningPlan::Entry e{&w, {0, 0}, {0, 0}};
-    if (c.u.size() == 2 && zk_challenge_find(c.u[0], &e.pos[0]) && zk_challenge_find(c.u[1], &e.pos[1]) && e.pos[0] >= base && e.pos[1] >= base) {
+    uint which = 0;
+    while (which < weights.size() && weights[which] != &w) ++which;
+    OpeningPlan::Entry e{which, {0, 0}, {0, 0}};
+    if (which < weights.size() && c.u.size() == 2 && zk_challenge_find(c.u[0], &e.pos[0]) && zk_challenge_find(c.u[1], &e.pos[1]) && e.pos[0] >= base && e.pos[1] >= base) {
         e.len[0] = (uint)c.u[0].size(); e.len[1] = (uint)c.u[1].size();
         e.pos[0] -= base; e.pos[1] -= base;
         plan->entries.push_back(e);
     } else { learning = false; plan->entries.clear(); }
 }
+// an opening that starts at its claim: rows folded now, the G1 job queued now or when the enclosing OpeningGroup ends
+void DeferredOpenings::claim_here(const Weight& w, const Claim& c, const vector<Fr_t>& u_cat) {
+    Item* it = new Item{fold_weight(w, u_cat), c.claim, 0, &w.generator, false};
+    it->slot = zk_record_reserve();
+    items.push_back(it);
+    unstarted.push_back(it);
+    if (group_depth == 0) flush();
+}
 void verifyWeightClaim(const Weight& w, const Claim& c) {
     vector<Fr_t> u_cat = concatenate(vector<vector<Fr_t>>({c.u[1], c.u[0]}));
-    std::unique_ptr<FrTensor> local;
-    const FrTensor& w_padded = padded_form(w, local);
     if (g_deferred) {
         DeferredOpenings& d = *g_deferred;
         const size_t k = d.next++;
@@ -165,12 +203,14 @@ void verifyWeightClaim(const Weight& w, const Claim& c) {
             delete a;
             d.plan->learned = false;          // the plan does not describe this sequence: learn it again next time
         }
-        DeferredOpenings::Item* it = new DeferredOpenings::Item{w.generator.open_begin(w_padded, w.com, u_cat), c.claim, zk_record_reserve()};
-        d.items.push_back(it);
+        d.claim_here(w, c, u_cat);
         return;
     }
+    // no scope: the same job, waited for here
+    Commitment::Pending op = fold_weight(w, u_cat);
+    Commitment::open_start_batch({{&w.generator, &op}});
     vector<G1Jacobian_t> g1_proof;
-    auto opening = w.generator.open(w_padded, w.com, u_cat, g1_proof);
+    auto opening = Commitment::open_end(op, g1_proof);
     zk_record(opening);
     zk_record_g1(g1_proof);
     if (opening != c.claim) throw std::runtime_error("verifyWeightClaim: opening != c.claim");
@@ -191,22 +231,21 @@ WeightOpeningAhead::~WeightOpeningAhead() {
 }
 WeightOpeningAhead openWeightAhead(const Weight& w, const vector<Fr_t>& u_input, const vector<Fr_t>& u_output) {
     WeightOpeningAhead a;
-    if (!g_deferred || !g_deferred->ahead.empty()) return a;            // nothing runs ahead outside a deferred scope
+    if (!g_deferred || !g_deferred->ahead.empty() || g_only_at_claim) return a;            // nothing runs ahead outside a deferred scope
     a.impl = new WeightOpeningAhead::Impl;
     a.impl->u_cat = concatenate(vector<vector<Fr_t>>({u_output, u_input}));
-    std::unique_ptr<FrTensor> local;
-    a.impl->op = w.generator.open_begin(padded_form(w, local), w.com, a.impl->u_cat);
+    a.impl->op = fold_weight(w, a.impl->u_cat);
+    Commitment::open_start_batch({{&w.generator, &a.impl->op}});
     return a;
 }
 std::vector<WeightOpeningAhead> openWeightsAhead(const std::vector<const Weight*>& ws, const std::vector<const std::vector<Fr_t>*>& u_inputs,
                                                  const std::vector<const std::vector<Fr_t>*>& u_outputs) {
     std::vector<WeightOpeningAhead> out(ws.size());
-    if (!g_deferred || !g_deferred->ahead.empty()) return out;      // a scope that runs from a plan has started them already
+    if (!g_deferred || !g_deferred->ahead.empty() || g_only_at_claim) return out;      // a scope that runs from a plan has started them already
     for (size_t i = 0; i < ws.size(); ++i) {
         out[i].impl = new WeightOpeningAhead::Impl;
         out[i].impl->u_cat = concatenate(vector<vector<Fr_t>>({*u_outputs[i], *u_inputs[i]}));
-        std::unique_ptr<FrTensor> local;
-        out[i].impl->op = ws[i]->generator.open_fold(padded_form(*ws[i], local), ws[i]->com, out[i].impl->u_cat);
+        out[i].impl->op = fold_weight(*ws[i], out[i].impl->u_cat);
     }
     std::vector<std::pair<const Commitment*, Commitment::Pending*>> ops;
     for (size_t i = 0; i < ws.size(); ++i) ops.emplace_back(&ws[i]->generator, &out[i].impl->op);
