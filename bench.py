@@ -572,23 +572,75 @@ def main():
         orc_check(orc.orc_range_prep(S4, D4, -(1 << 15), N4, m4))
         orc_check(orc.orc_range_prove(S4, D4, -(1 << 15), N4, al4, be4, u4, w4, fin4))
         c4_s = time.perf_counter() - t0
+        # C2's proof in full (zkfc.cu:61-151): the evaluation of Y, the two reductions X(u_batch, .) and W(., u_output), the 12-round
+        # inner-product sumcheck over them and the closing evaluations of W and X -- on tensors of the configuration's sizes
+        # (2048 x 4096, 4096 x 4096); the claim of the sumcheck is formed from the reduced vectors
+        def small_fr(seed, n):
+            out = np.zeros((n, 8), np.uint32)
+            orc.orc_fr_from_i64(np.ascontiguousarray(np.random.default_rng(seed).integers(-(1 << 20), 1 << 20, n), dtype=np.int64), out, n)
+            return out
+        Bc, Ic, Oc = 2048, 4096, 4096
+        Xc, Wc, Yc = small_fr(21, Bc * Ic), small_fr(22, Ic * Oc), small_fr(23, Bc * Oc)
+        rs2 = np.random.RandomState(24)
+        u_b, u_i, u_o = mt_random_vec(rs2, 11), mt_random_vec(rs2, 12), mt_random_vec(rs2, 12)
+        lens2, one_fr = np.array([11, 12], np.uint32), np.zeros(8, np.uint32)
+        n_out = ctypes.c_long()
+        t0 = time.perf_counter()
+        orc_check(orc.orc_fr_multi_dim_me(Yc, Bc * Oc, np.concatenate([u_b, u_o]), lens2, np.array([Bc, Oc], np.uint32), 2, one_fr))
+        Xr, Wr = np.zeros((Bc * Ic, 8), np.uint32), np.zeros((Ic * Oc, 8), np.uint32)
+        orc_check(orc.orc_fr_partial_me(Xc, Bc * Ic, u_b, 11, Bc, Ic, Xr, ctypes.byref(n_out)))
+        assert n_out.value == Ic
+        orc_check(orc.orc_fr_partial_me(Wc, Ic * Oc, u_o, 12, Oc, 1, Wr, ctypes.byref(n_out)))
+        assert n_out.value == Ic
+        prod, claim2 = np.zeros((Ic, 8), np.uint32), np.zeros(8, np.uint32)
+        orc_check(orc.orc_fr_op(7, Xr[:Ic].copy(), Wr[:Ic].copy(), prod, Ic))
+        orc_check(orc.orc_fr_sum(prod, Ic, claim2))
+        orc_check(orc.orc_zkip(claim2, Xr[:Ic].copy(), Wr[:Ic].copy(), Ic, u_i, 12, np.zeros((12 * 3, 8), np.uint32), np.zeros(8, np.uint32)))
+        orc_check(orc.orc_fr_multi_dim_me(Wc, Ic * Oc, np.concatenate([u_i, u_o]), np.array([12, 12], np.uint32), np.array([Ic, Oc], np.uint32), 2, one_fr))
+        orc_check(orc.orc_fr_multi_dim_me(Xc, Bc * Ic, np.concatenate([u_b, u_i]), lens2, np.array([Bc, Ic], np.uint32), 2, one_fr))
+        c2_prove_s = time.perf_counter() - t0
+        c2_products = Bc * Oc + 2 * Bc * Ic + 2 * Ic * Oc          # one product per element folded
+        del Xc, Wc, Yc, Xr, Wr
+        # the softmax's Hadamard argument (multi_hadamard_sumchecks over the K = 3 table-value planes, proof.cu:191-241) for ONE
+        # head: 2048 x 2048 elements, 22 rounds
+        nh, kh = 2048 * 2048, 22
+        Hs = np.concatenate([small_fr(31 + j, nh) for j in range(3)])
+        rs3 = np.random.RandomState(34)
+        u_h, v_h = mt_random_vec(rs3, kh), mt_random_vec(rs3, kh)
+        p01, p012, claim3 = np.zeros((nh, 8), np.uint32), np.zeros((nh, 8), np.uint32), np.zeros(8, np.uint32)
+        orc_check(orc.orc_fr_op(7, Hs[:nh], Hs[nh:2 * nh], p01, nh))
+        orc_check(orc.orc_fr_op(7, p01, Hs[2 * nh:], p012, nh))
+        orc_check(orc.orc_fr_me(p012, nh, u_h, kh, claim3))            # the claim the argument starts from (not timed: the prover holds it)
+        del p01, p012
+        t0 = time.perf_counter()
+        orc_check(orc.orc_multi_hadamard(claim3, Hs, 3, nh, u_h, v_h, kh, np.zeros((kh * 4, 8), np.uint32), np.zeros(8, np.uint32)))
+        hadamard_head_s = time.perf_counter() - t0
+        del Hs
         layer_mm = 4.49e11                                     # field multiplications in the layer's matrix products (reference algorithm)
+        # elements folded by the layer's matrix-product proofs (zkFC::prove of the seven projections: B O + 2 B I + 2 I O each) and by
+        # the per-head proofs of out = Y V and X = Q K^T (self-attn.cu:97-119: Y, X of 2048 x 2048, Q, K, V, out of 2048 x 128, 32 heads)
+        fc = lambda B_, I_, O_: B_ * O_ + 2 * B_ * I_ + 2 * I_ * O_
+        layer_fold_products = 4 * fc(2048, 4096, 4096) + 2 * fc(2048, 4096, 11008) + fc(2048, 11008, 4096) + 32 * (2 * 2048 * 2048 + 5 * 2048 * 128)
         layer_gens = 5 * (4096 << 5) + 2 * (1 << 19) + 2 * 4096      # generators of the nine openings (11008 << 5 rounds up to 2^19); pairs over all rounds ~ the same number
         # queries of the layer's lookup arguments: three softmax segments over 32 x 2048 x 2048, the activation table and four rescalings over the
         # padded 2048 x 11008 tensors, nine rescalings over 2048 x 4096, two over 4096
         layer_queries = 3 * (1 << 27) + 4 * (1 << 25) + 9 * (1 << 23) + 2 * 4096
-        parts_cpu = {"matrix_products_s": layer_mm / mm_rate, "openings_s": open_s * layer_gens / n_open, "lookup_arguments_s": c4_s * layer_queries / D4}
+        parts_cpu = {"matrix_products_s": layer_mm / mm_rate, "openings_s": open_s * layer_gens / n_open, "lookup_arguments_s": c4_s * layer_queries / D4,
+                     "matrix_product_proofs_s": c2_prove_s * layer_fold_products / c2_products, "softmax_hadamard_arguments_s": hadamard_head_s * 32}
         cpu_s = sum(parts_cpu.values())
         out["cpu_baseline"] = {"value": cpu_s, "unit": "s", "cores": int(cores), "kind": "port",
                                "sample": f"oracle (reference algorithm, OpenMP, {int(cores)} threads): Fr matmul {rows} x 4096 x 1024 = {rows * 4096 * 1024:.3g} multiplications in {dt:.1f} s, "
                                          f"scaled to the layer's 4.49e11; opening of {n_open} generators in {open_s:.1f} s, scaled to the layer's "
                                          f"{layer_gens} generators; configuration 4 in full (2^22 queries into 2^16 entries: multiplicities, Fermat inversions, 22 rounds) in "
-                                         f"{c4_s:.1f} s, scaled to the layer's {layer_queries:.3g} queries; the sumchecks of the matrix products and the softmax's "
-                                         "Hadamard argument are not included",
+                                         f"{c4_s:.1f} s, scaled to the layer's {layer_queries:.3g} queries; configuration 2's proof in full (five folds of 2048 x 4096 / "
+                                         f"4096 x 4096 tensors and the 12-round inner-product sumcheck, {c2_products:.3g} products) in {c2_prove_s:.1f} s, scaled to the "
+                                         f"{layer_fold_products:.3g} elements the layer's matrix-product proofs fold; the softmax's Hadamard argument of one head "
+                                         f"(three planes of 2048 x 2048, 22 rounds) in {hadamard_head_s:.1f} s, times 32 heads",
                                "parts_s": {k_: round(v_, 1) for k_, v_ in parts_cpu.items()},
-                               "config1_zkfc_toy_s": c1_s, "config4_lookup_s": c4_s,
+                               "config1_zkfc_toy_s": c1_s, "config4_lookup_s": c4_s, "config2_proof_s": c2_prove_s, "softmax_hadamard_one_head_s": hadamard_head_s,
                                "fr_mul_per_s_all_cores": mm_rate}
     print(json.dumps(out))
+    lib.zk_shutdown()
 
 
 if __name__ == "__main__":

@@ -41,6 +41,11 @@ int zk_free(void* p);                                      /* last user: the def
 int zk_free_async(void* p, void* stream);                  /* last user: kernels already queued on `stream` */
 int zk_pool_trim(void);                                    /* return cached blocks to the driver */
 int zk_pool_stats(size_t* live_bytes, size_t* cached_bytes);
+/* No counterpart in the reference (which leaves everything to process exit): waits for the device and releases, in a fixed
+ * order and while the runtime is alive, what the library itself holds -- timing events, the cached eq table, cached blocks
+ * (live blocks stay with their owners), its streams, the allocator's events, idle pinned buffers.  The library stays usable
+ * afterwards.  A host calls it before it exits so that nothing is left to static destruction. */
+int zk_shutdown(void);
 /* replace cudaMemcpy in ctors, operator()(idx), savebin/loadbin (ioutils.cu:3-45) */
 int zk_memcpy_h2d(void* dst, const void* src_host, size_t bytes, void* stream);
 int zk_memcpy_d2h(void* dst_host, const void* src, size_t bytes, void* stream);
@@ -120,9 +125,13 @@ int zk_fr_fold_prepared_free(void* prepared);
 /* The same handle for a tensor whose int32 form is written by the kernel that makes the tensor (the digit planes of
  * zk_softmax_decompose_ints, the outputs of zk_fr_gather_ints), so no pass over the field elements is needed: _new
  * allocates the handle and its n int32 slots (uninitialised) and returns their device address; the caller must have queued
- * the kernel that sets ints_dev[i] to element i before the handle is used.  _ints returns that address (null for null). */
+ * the kernel that sets ints_dev[i] to element i before the handle is used.  _ints returns that address (null for null).
+ * The int32 form must not change once that kernel has written it: other handles may remember what they were gathered from by
+ * this one's identity (zk_fr_gather_by_queries_ints).  A caller that does write ints_dev again calls _touch afterwards: the handle
+ * then counts as a new form and nothing gathered from the old one is trusted any more.  No counterpart in the reference. */
 int zk_fr_fold_prepared_new(void** prepared, void** ints_dev, size_t n, void* stream);
 const void* zk_fr_fold_prepared_ints(const void* prepared);
+int zk_fr_fold_prepared_touch(void* prepared);
 /* zk_fr_gather (out[i] = table[idx[i]], the mapped values of tLookupRangeMapping::operator(), tlookup.cu:446-470) that
  * also writes the int32 form of out from the table's own (table_prepared: a handle of zk_fr_fold_prepare over the table) */
 int zk_fr_gather_ints(void* out, void* out_ints, const void* table, const void* table_prepared, const void* idx, size_t n, void* stream);
@@ -309,6 +318,12 @@ int zk_lookup_prove_begin_mapped_ints(void** handle, const void* S_in, const voi
                                       const uint32_t* r, const void* T, const void* m, int32_t low, const uint32_t* beta, const uint32_t* u_eq, const uint32_t* v, size_t D,
                                       size_t N, int rounds, void* stream);
 int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host);
+/* Diagnostics of the job zk_lookup_prove_end collected last (no counterpart in the reference): *n_ok = how many leading table
+ * entries were what the integers say -- the queries naming one of them took the first round's short path, the others their own
+ * comparison -- and *n_table = the table's size; both 0 when the job had no int32 forms.  A range table of len entries padded to
+ * a power of two by repeating its last value reports len.  ZKLLM_LOOKUP_TRUSTED=0 in the environment makes every job report 0:
+ * each query is then compared on its own (same results; for comparing the two paths). */
+int zk_lookup_last_job_consistent_entries(uint32_t* n_ok, uint32_t* n_table);
 /* hadamard_product_sumcheck (Fr_hp_sc, proof.cu:66-109): adjacent-pair folding, first challenge first.  a, b: n elements,
  * 2^(k-1) < n <= 2^k; u, v: k challenges each.  proof_host: 3k + 2 values (per round the three terms evaluated at the
  * remaining u, then the folded a and b).  The three term tensors of the reference's step kernel are never materialised. */

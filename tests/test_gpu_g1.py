@@ -412,13 +412,15 @@ def test_open_batch_with_row_commitments_delivers_the_points_of_the_plain_openin
 
 
 @pytest.mark.parametrize("n,R,tables", [(8192, 2, 2), (16384, 3, 3), (32768, 3, 3)])
-def test_open_batch_with_cross_commitments_needs_no_sum_over_the_generators(pv, n, R, tables):
+def test_open_batch_with_cross_commitments_needs_no_sum_over_the_generators(pv, orc, n, R, tables):
     """With the cross commitments of its first R rounds -- commitments of every 2nd / 4th / 8th column of the tensor's rows
     under every 2nd / 4th / 8th generator, made here with commit_int on slices -- zk_g1_open_begin_batch_rows forms T, T0 and
     T1 of those rounds from rows x patterns points: 8192 generators are halved twice before the batched last rounds, so no
     round sums over its generators.  With three rounds of them and the tables of zk_g1_open_prepare_tables(.., 3) the three
     rounds are one fold (16384 generators: nothing but that fold and the batched last rounds; 32768: one ordinary round
-    behind it).  Every point of the proof equals zk_g1_open's on the row-folded vector."""
+    behind it).  Every point of the proof equals zk_g1_open's on the row-folded vector, and at 16384 generators also the
+    oracle's own opening of the padded tensor (Commitment::open, commitment.cu:133-141: row fold, then me_open), point by
+    point after normalisation, so the batched path is compared with the reference's algorithm directly."""
     import ctypes
     from gpuhelp import Hip, c_void_p, c_size_t, c_int
     hip = Hip()
@@ -458,6 +460,15 @@ def test_open_batch_with_cross_commitments_needs_no_sum_over_the_generators(pv, 
         hip.call("zk_g1_open", exp_p[i], exp_v[i], c_void_p(f.devptr), c_void_p(dG), c_size_t(n), u, c_int(k), None)
         keep += [W, f]
         folded.append(f); urows.append(np.ascontiguousarray(ur, dtype=np.uint32)); us.append(u)
+        if n == 16384:
+            rows_p = 1 << kr
+            Tp = np.zeros((rows_p * n, 8), np.uint32)
+            Tp[:nrows * n] = fr_array([int(x) % R_MOD for x in Wi.ravel()])
+            o_p, o_v = np.zeros((npts, 36), np.uint32), np.zeros(8, np.uint32)
+            print(f"rows={nrows}: oracle opening over {n} generators", flush=True)
+            orc_check(orc.orc_open(np.ascontiguousarray(gens_host), n, Tp, rows_p * n, rows_p, np.ascontiguousarray(np.concatenate([u, ur]), dtype=np.uint32), k + kr, o_p, o_v))
+            assert (o_v == exp_v[i]).all()
+            assert (norm(orc, o_p) == exp_p[i]).all()          # the product delivers its points normalised
     for cr in (R, 1):
         h = c_void_p()
         sc = (c_void_p * 2)(*[c_void_p(f.devptr) for f in folded])

@@ -565,12 +565,135 @@ def test_mapped_lookup_over_outputs_gathered_by_their_queries(k, bad_entry):
         bm, sums = np.zeros(8, np.uint32), np.zeros((k * 11, 8), np.uint32)
         hip.call("zk_lookup_prove_end", h, bm, sums)
         res.append((bm, sums))
+        n_ok, n_tab = ctypes.c_uint32(7), ctypes.c_uint32(7)
+        hip.call("zk_lookup_last_job_consistent_entries", ctypes.byref(n_ok), ctypes.byref(n_tab))
+        # the entries below the first inconsistent one serve their queries from the table record alone
+        assert (n_ok.value, n_tab.value) == ((0, 0) if job == "plain" else ((17 if bad_entry else N), N))
     assert (res[0][0] == res[1][0]).all() and (res[0][1] == res[1][1]).all()
     assert res[0][1].any()
+    # The queries' int32 form written again and declared so (zk_fr_fold_prepared_touch): the outputs no longer count as gathered
+    # by these queries, every query is compared on its own, and the job equals the plain job on the new combined queries.
+    if not bad_entry:
+        s_in2 = list(s_in)
+        for i in range(0, D, 3):
+            s_in2[i] = low + (s_in[i] - low + 1) % N if 0 <= s_in[i] - low < N else s_in[i]
+        hip.lib.zk_fr_fold_prepared_ints.restype = ctypes.c_void_p
+        q_ints = hip.lib.zk_fr_fold_prepared_ints(hq)
+        new_ints = hip.upload(np.array(s_in2, np.int32))
+        hip.lib.zk_memcpy_d2d(c_void_p(q_ints), c_void_p(new_ints), c_size_t(4 * D), None)
+        hip.call("zk_fr_fold_prepared_touch", hq)
+        dSi2 = hip.upload(fr_array([x % R_MOD for x in s_in2]))
+        S2 = [(a + r * o) % R_MOD for a, o in zip(s_in2, s_out)]
+        m2 = np.zeros(N, np.int64)
+        for q in S2:
+            if q in index_of:
+                m2[index_of[q]] += 1
+        dS2, dm2 = hip.upload(fr_array(S2)), hip.upload(fr_array([int(c) for c in m2]))
+        res2 = []
+        for job in ("plain", "mapped_ints"):
+            h = c_void_p()
+            if job == "plain":
+                hip.call("zk_lookup_prove_begin", ctypes.byref(h), c_void_p(dS2), c_void_p(dT), c_void_p(dm2), beta, u, v, c_size_t(D), c_size_t(N), c_int(k), None)
+            else:
+                hip.call("zk_lookup_prove_begin_mapped_ints", ctypes.byref(h), c_void_p(dSi2), hq, c_void_p(dSo), ho, hm, r_fr, c_void_p(dT), c_void_p(dm2), c_int(low),
+                         beta, u, v, c_size_t(D), c_size_t(N), c_int(k), None)
+            bm, sums = np.zeros(8, np.uint32), np.zeros((k * 11, 8), np.uint32)
+            hip.call("zk_lookup_prove_end", h, bm, sums)
+            res2.append((bm, sums))
+        assert (res2[0][0] == res2[1][0]).all() and (res2[0][1] == res2[1][1]).all()
+        assert not (res2[0][1] == res[0][1]).all()
+        for q in (new_ints, dSi2, dS2, dm2):
+            hip.free(q)
     for h in (hq, hm, ho):
         hip.call("zk_fr_fold_prepared_free", h)
     for q in (dSi, dMp, dSo, dS, dT, dm):
         hip.free(q)
+
+
+@pytest.mark.parametrize("k,length", [(17, 48), (17, 64), (13, 37)])
+def test_range_table_padded_by_repeating_its_last_value_keeps_the_short_first_round(k, length):
+    """A range table of `length` entries padded to 64 by repeating its last value (zk_range_table): the entries below `length` are
+    what the integers say and serve their queries from the table record alone (zk_lookup_last_job_consistent_entries reports
+    `length`), queries that name a padding position or lie outside are compared on their own; the job equals the plain one."""
+    import ctypes
+    from gpuhelp import Hip, c_void_p, c_size_t, c_int, c_uint
+    hip = Hip()
+    D, N, low = 1 << k, 64, -11
+    rng = np.random.default_rng(3000 + k + length)
+    dT = hip.malloc(32 * N)
+    hip.call("zk_range_table", c_void_p(dT), c_int(low), c_uint(length), c_uint(N), None)
+    Tl = fr_ints(hip.download(dT, (N, 8), np.uint32))
+    assert Tl == [(low + min(j, length - 1)) % R_MOD for j in range(N)]
+    s_in = [int(x) + low for x in rng.integers(0, length, D)]
+    odd = rng.choice(D, 120, replace=False)
+    for i in odd[:60]:
+        s_in[i] = low + length + int(i % max(1, N - length)) if length < N else low + N + 2      # a padding position (no table value) / above the table
+    for i in odd[60:]:
+        s_in[i] = low - 1 - int(i % 50)
+    index_of = {}
+    for j, t in enumerate(Tl):
+        index_of.setdefault(t, j)
+    m_counts = np.zeros(N, np.int64)
+    for q in s_in:
+        if q % R_MOD in index_of:
+            m_counts[index_of[q % R_MOD]] += 1
+    dS, dm = hip.upload(fr_array([x % R_MOD for x in s_in])), hip.upload(fr_array([int(c) for c in m_counts]))
+    hq = c_void_p()
+    hip.call("zk_fr_fold_prepare", ctypes.byref(hq), c_void_p(dS), c_size_t(D), None)
+    beta, u, v = ch(91, 1)[0], ch(92, k - 1), ch(93, k)
+    res = []
+    for job in ("plain", "hinted_ints"):
+        h = c_void_p()
+        if job == "plain":
+            hip.call("zk_lookup_prove_begin", ctypes.byref(h), c_void_p(dS), c_void_p(dT), c_void_p(dm), beta, u, v, c_size_t(D), c_size_t(N), c_int(k), None)
+        else:
+            hip.call("zk_lookup_prove_begin_hinted_ints", ctypes.byref(h), c_void_p(dS), hq, c_void_p(dT), c_void_p(dm), c_int(low), beta, u, v,
+                     c_size_t(D), c_size_t(N), c_int(k), None)
+        bm, sums = np.zeros(8, np.uint32), np.zeros((k * 11, 8), np.uint32)
+        hip.call("zk_lookup_prove_end", h, bm, sums)
+        res.append((bm, sums))
+    n_ok, n_tab = ctypes.c_uint32(), ctypes.c_uint32()
+    hip.call("zk_lookup_last_job_consistent_entries", ctypes.byref(n_ok), ctypes.byref(n_tab))
+    assert (n_ok.value, n_tab.value) == (length, N)
+    assert (res[0][0] == res[1][0]).all() and (res[0][1] == res[1][1]).all() and res[0][1].any()
+    hip.call("zk_fr_fold_prepared_free", hq)
+    for q in (dT, dS, dm):
+        hip.free(q)
+
+
+def test_evaluations_of_eight_tensors_that_keep_only_their_int32_form():
+    """zk_fr_me_multi_ints with eight int32 forms: every one is evaluated from that form (six, then two), never from the field
+    elements passed beside it -- which hold other values here, as a tensor that keeps only its int32 form does."""
+    import ctypes
+    from gpuhelp import Hip, c_void_p, c_size_t, c_int
+    hip = Hip()
+    n, k = 5000, 13
+    rng = np.random.default_rng(77)
+    vals = [rng.integers(-2 ** 31, 2 ** 31, n) for _ in range(8)]
+    devs = [hip.upload(fr_array([int(x) % R_MOD for x in v])) for v in vals]
+    hs = []
+    for d in devs:
+        h = c_void_p()
+        hip.call("zk_fr_fold_prepare", ctypes.byref(h), c_void_p(d), c_size_t(n), None)
+        hs.append(h)
+    junk = hip.upload(ch(78, n))
+    u = ch(79, k)
+    exp, got = np.zeros((8, 8), np.uint32), np.zeros((8, 8), np.uint32)
+    hip.call("zk_fr_me_multi", exp, (c_void_p * 8)(*[c_void_p(d) for d in devs]), c_int(8), c_size_t(n), u, c_int(k), None)
+    hip.call("zk_fr_me_multi_ints", got, (c_void_p * 8)(*[c_void_p(junk)] * 8), (c_void_p * 8)(*hs), c_int(8), c_size_t(n), u, c_int(k), None)
+    assert (got == exp).all() and len({tuple(r) for r in exp}) == 8
+    # seven forms and one tensor of field elements in the middle
+    mixed_ptrs = [c_void_p(junk)] * 8
+    mixed_ptrs[3] = c_void_p(devs[3])
+    mixed_hs = list(hs)
+    mixed_hs[3] = c_void_p(None)
+    got2 = np.zeros((8, 8), np.uint32)
+    hip.call("zk_fr_me_multi_ints", got2, (c_void_p * 8)(*mixed_ptrs), (c_void_p * 8)(*mixed_hs), c_int(8), c_size_t(n), u, c_int(k), None)
+    assert (got2 == exp).all()
+    for h in hs:
+        hip.call("zk_fr_fold_prepared_free", h)
+    for d in devs + [junk]:
+        hip.free(d)
 
 
 @pytest.mark.parametrize("rows,cols", [(5, 64), (37, 200), (64, 2048)])

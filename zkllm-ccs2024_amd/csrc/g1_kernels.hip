@@ -1266,6 +1266,12 @@ struct FoldTimer {
     unsigned long long pairs = 0;
 };
 static FoldTimer g_fold_timer;
+static const int g_fold_timer_hook = (at_shutdown([] {
+    std::lock_guard<std::mutex> lk(g_fold_timer.mu);
+    for (auto& e : g_fold_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
+    g_fold_timer.ev.clear();
+    g_fold_timer.on = false;
+}), 0);
 // Fp multiplications of one pair of the fold by the formulas' count (two 8-limb products aside)
 static double fold_fp_mults_per_pair(const JsfK& j) {
     int adds = 0;

@@ -474,10 +474,13 @@ template <int K> __global__ void __launch_bounds__(TPB) k_me_multi(Fr* __restric
 // consistent entry of a plain table, INTS_POISON for an entry that is something else), query and inverse are TB[2j], TB[2j+1].
 struct HintSrc { const Fr* TB; const Fr* hint; Fr low; Fr beta; uint32_t N; const Fr* S_out = nullptr; Fr r_mont;
                  const int32_t* hint_ints = nullptr; const int32_t* sout_ints = nullptr; const int32_t* want = nullptr; int32_t low_int = 0;
-                 // *any_bad == 0: every table entry is what the integers say (k_lookup_ints_check); trusted_out: the outputs were gathered from
-                 // this table by these queries (zk_fr_gather_by_queries_ints).  With both, a query inside the table needs neither its output
-                 // nor the entry's expected integer: nothing is gathered but the table record.
-                 const uint32_t* any_bad = nullptr; bool trusted_out = false; };
+                 // *n_ok: the first table entry that is not what the integers say (k_lookup_ints_check; 0xFFFFFFFF: none) -- every entry
+                 // below it is consistent, whatever lies above (a range table padded by repeating its last value is consistent up
+                 // to its own length).  trusted_out: the outputs were gathered from this table by these queries
+                 // (zk_fr_gather_by_queries_ints).  A query that names an entry below *n_ok then needs neither its output nor the
+                 // entry's expected integer (for a plain table; for a mapping table with trusted outputs): nothing is gathered but
+                 // the table record.
+                 const uint32_t* n_ok = nullptr; bool trusted_out = false; };
 static constexpr int32_t INTS_POISON = (int32_t)0x80000000;
 __device__ __forceinline__ Fr hinted_query(const Fr* __restrict__ S, size_t i, const HintSrc& h) {
     return h.S_out ? add(h.hint[i], mont_mul(h.r_mont, h.S_out[i])) : S[i];
@@ -508,7 +511,7 @@ __device__ __forceinline__ Fr inv_by_hint(const Fr& sv, size_t i, const HintSrc&
     return inv_plus_beta_alone(sv, h.beta);
 }
 // want[j] for the int32 path of the first round: TB[2j] must be low + j (+ r * mapped[j])
-__global__ void __launch_bounds__(TPB) k_lookup_ints_check(int32_t* __restrict__ want, uint32_t* __restrict__ any_bad, const Fr* __restrict__ TB,
+__global__ void __launch_bounds__(TPB) k_lookup_ints_check(int32_t* __restrict__ want, uint32_t* __restrict__ n_ok, const Fr* __restrict__ TB,
                                                            const int32_t* __restrict__ mapped_ints, const Fr r_mont, int32_t low, uint32_t N) {
     const uint32_t j = blockIdx.x * TPB + threadIdx.x;
     if (j >= N) return;
@@ -516,7 +519,7 @@ __global__ void __launch_bounds__(TPB) k_lookup_ints_check(int32_t* __restrict__
     if (mapped_ints) q = add(q, mont_mul(r_mont, fr_from_i64((int64_t)mapped_ints[j])));
     const bool ok = equal(q, TB[2 * (size_t)j]) && (!mapped_ints || mapped_ints[j] != INTS_POISON);
     want[j] = ok ? (mapped_ints ? mapped_ints[j] : 0) : INTS_POISON;
-    if (!ok) atomicOr(any_bad, 1u);
+    if (!ok) atomicMin(n_ok, j);          // *n_ok starts at 0xFFFFFFFF
 }
 // query i and 1 / (query + beta) from the int32 forms (HintSrc); unit as in inv_by_hint
 __device__ __forceinline__ Fr query_inv_ints(size_t i, const HintSrc& h, Fr& a, bool& unit) {
@@ -524,10 +527,10 @@ __device__ __forceinline__ Fr query_inv_ints(size_t i, const HintSrc& h, Fr& a, 
     const int64_t d = (int64_t)hi - (int64_t)h.low_int;
     const bool in_table = d >= 0 && d < (int64_t)h.N;
     const uint32_t j = in_table ? (uint32_t)d : 0u;
-    const bool sure = *h.any_bad == 0u && (!h.sout_ints || h.trusted_out);      // the same for every query of the job
+    const bool sure = in_table && j < *h.n_ok && (!h.sout_ints || h.trusted_out);
     int32_t so = 0;
-    bool match = in_table;
-    if (!sure || !in_table) {
+    bool match = sure;
+    if (!sure) {
         so = h.sout_ints ? __builtin_nontemporal_load(h.sout_ints + i) : 0;
         const int32_t w = h.want[j];
         match = in_table && w != INTS_POISON && so == w;
@@ -1528,6 +1531,17 @@ int zk_fr_fold_prepared_new(void** prepared, void** ints_dev, size_t n, void* st
     return 0;
 }
 const void* zk_fr_fold_prepared_ints(const void* prepared) { return prepared ? ((const FoldPrepared*)prepared)->ints : nullptr; }
+// The int32 form of a handle was written again (by anything but the kernel queued right after zk_fr_fold_prepared_new): the
+// handle becomes a new form -- a fresh id, so that whatever remembered the old one (the outputs gathered by these queries or from
+// this table) no longer counts as gathered from it, and nothing it was itself gathered from.
+int zk_fr_fold_prepared_touch(void* prepared) {
+    FoldPrepared* fp = (FoldPrepared*)prepared;
+    ZK_ARG(fp != nullptr, "zk_fr_fold_prepared_touch: null handle");
+    fp->id = fold_prepared_id();
+    fp->src_queries = fp->src_table = 0;
+    fp->src_low = 0;
+    return 0;
+}
 int zk_fr_gather_ints(void* out, void* out_ints, const void* table, const void* table_prepared, const void* idx, size_t n, void* stv) {
     const FoldPrepared* tp = (const FoldPrepared*)table_prepared;
     ZK_ARG(out != nullptr && out_ints != nullptr && table != nullptr && tp != nullptr && idx != nullptr, "zk_fr_gather_ints: null argument");
@@ -1555,13 +1569,14 @@ int zk_fr_me_multi_ints(uint32_t* out_host, const void* const* Xs, const void* c
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(K >= 1 && K <= 8, "zk_fr_me_multi_ints: 1..8 tensors");
     ZK_ARG(k >= 0 && k <= 30 && n >= 1 && n <= ((size_t)1 << k) && (k == 0 || n > ((size_t)1 << (k - 1))), "zk_fr_me_multi_ints: n does not match the number of challenges");
-    // tensors with an int32 form go through the mixed kernel, up to six at a time and one tensor of field elements with
-    // them; what is left over is evaluated as zk_fr_me_multi does
+    // Every tensor with an int32 form is read from that form and never as field elements (a tensor that keeps only its int32
+    // form may have nothing written there): they go through the mixed kernel six at a time, with up to two tensors of field
+    // elements riding along on the first pass; what is left of those is evaluated as zk_fr_me_multi does.
     int ints_at[8], n_ints = 0, fr_at[8], n_fr = 0;
     for (int i = 0; i < K; ++i) {
         const FoldPrepared* fp = prepareds ? (const FoldPrepared*)prepareds[i] : nullptr;
         ZK_ARG(!fp || fp->n == n, "zk_fr_me_multi_ints: an int32 form of another size");
-        if (fp && n_ints < 6) ints_at[n_ints++] = i;
+        if (fp) ints_at[n_ints++] = i;
         else fr_at[n_fr++] = i;
     }
     if (n_ints == 0) return zk_fr_me_multi(out_host, Xs, K, n, u, k, stv);
@@ -1571,31 +1586,36 @@ int zk_fr_me_multi_ints(uint32_t* out_host, const void* const* Xs, const void* c
     int rc = eq_table_queue(E.as<Fr>(), u, k, tmp, st);
     if (rc) return rc;
     const unsigned nb = reduce_grid(n);
-    const int KF = n_fr >= 2 && n_ints <= 3 ? 2 : (n_fr ? 1 : 0), KT = KF + n_ints;         // two tensors of field elements ride along with up to three int32 forms
-    Scratch& part = tmp.add(sizeof(Fr) * KT * nb);
+    Scratch& part = tmp.add(sizeof(Fr) * 8 * nb);
     if (part.rc) return part.rc;
-    MeIntPtrs pi;
-    for (int i = 0; i < 6; ++i) pi.x[i] = ((const FoldPrepared*)prepareds[ints_at[i < n_ints ? i : 0]])->ints;
-    const Fr* XF = KF ? (const Fr*)Xs[fr_at[0]] : nullptr;
-    const Fr* XF2 = KF == 2 ? (const Fr*)Xs[fr_at[1]] : nullptr;
-#define MEI_CASE(F, I) if (KF == F && n_ints == I) hipLaunchKernelGGL((k_me_mixed<F, I>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), XF, XF2, pi, E.as<Fr>(), n);
-    MEI_CASE(0, 1) MEI_CASE(0, 2) MEI_CASE(0, 3) MEI_CASE(0, 4) MEI_CASE(0, 5) MEI_CASE(0, 6)
-    MEI_CASE(1, 1) MEI_CASE(1, 2) MEI_CASE(1, 3) MEI_CASE(1, 4) MEI_CASE(1, 5) MEI_CASE(1, 6)
-    MEI_CASE(2, 1) MEI_CASE(2, 2) MEI_CASE(2, 3)
+    int fr_done = 0;
+    for (int i0 = 0; i0 < n_ints; i0 += 6) {
+        const int ni = n_ints - i0 < 6 ? n_ints - i0 : 6;
+        const int KF = i0 == 0 ? (n_fr >= 2 && ni <= 3 ? 2 : (n_fr ? 1 : 0)) : 0, KT = KF + ni;         // two tensors of field elements ride along with up to three int32 forms
+        MeIntPtrs pi;
+        for (int i = 0; i < 6; ++i) pi.x[i] = ((const FoldPrepared*)prepareds[ints_at[i0 + (i < ni ? i : 0)]])->ints;
+        const Fr* XF = KF ? (const Fr*)Xs[fr_at[0]] : nullptr;
+        const Fr* XF2 = KF == 2 ? (const Fr*)Xs[fr_at[1]] : nullptr;
+#define MEI_CASE(F, I) if (KF == F && ni == I) hipLaunchKernelGGL((k_me_mixed<F, I>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), XF, XF2, pi, E.as<Fr>(), n);
+        MEI_CASE(0, 1) MEI_CASE(0, 2) MEI_CASE(0, 3) MEI_CASE(0, 4) MEI_CASE(0, 5) MEI_CASE(0, 6)
+        MEI_CASE(1, 1) MEI_CASE(1, 2) MEI_CASE(1, 3) MEI_CASE(1, 4) MEI_CASE(1, 5) MEI_CASE(1, 6)
+        MEI_CASE(2, 1) MEI_CASE(2, 2) MEI_CASE(2, 3)
 #undef MEI_CASE
-    ZK_LAUNCH_CHECK();
-    Fr s8[8];
-    rc = finish_sums(part.as<Fr>(), nb, KT, 0, s8, st);
-    if (rc) return rc;
-    for (int i = 0; i < KF; ++i) memcpy(out_host + 8 * fr_at[i], &s8[i], sizeof(Fr));
-    for (int i = 0; i < n_ints; ++i) memcpy(out_host + 8 * ints_at[i], &s8[KF + i], sizeof(Fr));
-    if (n_fr > KF) {         // the other tensors of field elements
-        const void* rest[8];
-        for (int i = KF; i < n_fr; ++i) rest[i - KF] = Xs[fr_at[i]];
-        Fr r8[8];
-        rc = zk_fr_me_multi((uint32_t*)r8, rest, n_fr - KF, n, u, k, stv);
+        ZK_LAUNCH_CHECK();
+        Fr s8[8];
+        rc = finish_sums(part.as<Fr>(), nb, KT, 0, s8, st);
         if (rc) return rc;
-        for (int i = KF; i < n_fr; ++i) memcpy(out_host + 8 * fr_at[i], &r8[i - KF], sizeof(Fr));
+        for (int i = 0; i < KF; ++i) memcpy(out_host + 8 * fr_at[i], &s8[i], sizeof(Fr));
+        for (int i = 0; i < ni; ++i) memcpy(out_host + 8 * ints_at[i0 + i], &s8[KF + i], sizeof(Fr));
+        fr_done += KF;
+    }
+    if (n_fr > fr_done) {         // the other tensors of field elements
+        const void* rest[8];
+        for (int i = fr_done; i < n_fr; ++i) rest[i - fr_done] = Xs[fr_at[i]];
+        Fr r8[8];
+        rc = zk_fr_me_multi((uint32_t*)r8, rest, n_fr - fr_done, n, u, k, stv);
+        if (rc) return rc;
+        for (int i = fr_done; i < n_fr; ++i) memcpy(out_host + 8 * fr_at[i], &r8[i - fr_done], sizeof(Fr));
     }
     return 0;
 }
@@ -1735,7 +1755,10 @@ struct SumJob {
     hipEvent_t ready = nullptr;
     void* host = nullptr;        // jobs on a side stream: pinned buffer the results are copied to behind the last kernel ...
     hipEvent_t done = nullptr;   // ... and the event behind that copy
+    const uint32_t* n_ok_dev = nullptr;      // lookup jobs over int32 forms: the consistent prefix of the table (HintSrc::n_ok) ...
+    uint32_t n_table = 0;                    // ... and the table's size
 };
+__global__ void __launch_bounds__(64) k_u32_set(uint32_t* __restrict__ p, uint32_t v) { if (threadIdx.x == 0) *p = v; }
 __global__ void __launch_bounds__(TPB) k_dot_part(Fr* __restrict__ partials, const Fr* __restrict__ a, const Fr* __restrict__ b, size_t n) {
     Fr acc[1] = {big_zero<8>()};
     for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (size_t)gridDim.x * TPB) acc[0] = add(acc[0], mont_mul(a[i], b[i]));
@@ -1750,6 +1773,16 @@ struct RoundTimer {
     double bytes = 0;          // algorithmic traffic of the timed launches
 };
 static RoundTimer g_round_timer;
+static const int g_round_timer_hook = (at_shutdown([] {
+    {
+        std::lock_guard<std::mutex> lk(g_round_timer.mu);
+        for (auto& e : g_round_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
+        g_round_timer.ev.clear();
+        g_round_timer.on = false;
+    }
+    std::lock_guard<std::mutex> lk(g_eq_mu);
+    g_eq_latest.reset();          // the eq table kept for the next job with the same challenges goes back to the allocator
+}), 0);
 // all rounds of the lookup sumcheck; sums land in job.sums
 // A == nullptr with a hint source: 1 / (S + beta) has not been written anywhere; a large first round computes it on
 // the fly, anything else writes it out first.
@@ -2078,17 +2111,21 @@ static int lookup_prove_begin(void** handle, const void* S, const void* T, const
         hs.TB = TB.as<Fr>(); hs.hint = (const Fr*)hint; hs.low = fr_from_i64((int64_t)low); hs.beta = b; hs.N = (uint32_t)N;
         if (S_out) { hs.S_out = (const Fr*)S_out; hs.r_mont = to_mont(load_fr(r)); }
         if (ints) {
-            Scratch& want = job->arena.add(sizeof(int32_t) * (N + 1));         // the last slot: any_bad
+            Scratch& want = job->arena.add(sizeof(int32_t) * (N + 1));         // the last slot: n_ok
             if (want.rc) { rc = want.rc; sumjob_abort(job); return rc; }
             const int32_t* mi = S_out ? ((const FoldPrepared*)ints->mapped)->ints : nullptr;
-            uint32_t* any_bad = (uint32_t*)(want.as<int32_t>() + N);
-            hipError_t me = hipMemsetAsync(any_bad, 0, sizeof(uint32_t), st);
-            if (me != hipSuccess) { sumjob_abort(job); ZK_HIP(me); }
-            hipLaunchKernelGGL(k_lookup_ints_check, dim3(cdiv(N, TPB)), dim3(TPB), 0, st, want.as<int32_t>(), any_bad, TB.as<Fr>(), mi, hs.r_mont, low, (uint32_t)N);
-            hs.any_bad = any_bad;
+            uint32_t* n_ok = (uint32_t*)(want.as<int32_t>() + N);
+            // ZKLLM_LOOKUP_TRUSTED=0: no entry counts as checked and no output as gathered from the table -- every query goes
+            // through its own comparison (to compare the two paths)
+            static const bool trust = [] { const char* e = getenv("ZKLLM_LOOKUP_TRUSTED"); return !(e && e[0] == '0'); }();
+            hipLaunchKernelGGL(k_u32_set, dim3(1), dim3(64), 0, st, n_ok, trust ? 0xFFFFFFFFu : 0u);      // a kernel, not a memset node: callers may capture this
+            hipLaunchKernelGGL(k_lookup_ints_check, dim3(cdiv(N, TPB)), dim3(TPB), 0, st, want.as<int32_t>(), n_ok, TB.as<Fr>(), mi, hs.r_mont, low, (uint32_t)N);
+            hs.n_ok = n_ok;
+            job->n_ok_dev = n_ok;
+            job->n_table = (uint32_t)N;
             if (S_out) {
                 const FoldPrepared *q = (const FoldPrepared*)ints->queries, *o = (const FoldPrepared*)ints->out, *mp = (const FoldPrepared*)ints->mapped;
-                hs.trusted_out = o->src_queries != 0 && o->src_queries == q->id && o->src_table == mp->id && o->src_low == low;
+                hs.trusted_out = trust && o->src_queries != 0 && o->src_queries == q->id && o->src_table == mp->id && o->src_low == low;
             }
             hs.hint_ints = ((const FoldPrepared*)ints->queries)->ints;
             hs.sout_ints = S_out ? ((const FoldPrepared*)ints->out)->ints : nullptr;
@@ -2153,11 +2190,24 @@ int zk_lookup_prove_begin_mapped_ints(void** handle, const void* S_in, const voi
     li.queries = S_in_prepared; li.out = S_out_prepared; li.mapped = mapped_prepared;
     return lookup_prove_begin(handle, nullptr, T, m, S_in, low, beta, u_eq, v, D, N, rounds, stv, S_out, r, &li);
 }
+// what the last collected lookup job over int32 forms found: how many leading table entries were what the integers say
+// (the queries that name one of them took the first round's short path), and the table's size; 0, 0 when that job had no int32 forms
+static uint32_t g_last_n_ok = 0, g_last_n_table = 0;
+int zk_lookup_last_job_consistent_entries(uint32_t* n_ok, uint32_t* n_table) {
+    if (n_ok) *n_ok = g_last_n_ok;
+    if (n_table) *n_table = g_last_n_table;
+    return 0;
+}
 int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host) {
     ZK_ARG(handle != nullptr, "zk_lookup_prove_end: null handle");
     SumJob* job = (SumJob*)handle;
     Fr bm = big_zero<8>();
     int rc = sumjob_collect(*job, (Fr*)sums_host, &bm);
+    g_last_n_ok = g_last_n_table = 0;
+    if (!rc && job->n_ok_dev) {          // the job's kernels have finished
+        uint32_t v = 0;
+        if (hipMemcpy(&v, job->n_ok_dev, sizeof(uint32_t), hipMemcpyDeviceToHost) == hipSuccess) { g_last_n_ok = v < job->n_table ? v : job->n_table; g_last_n_table = job->n_table; }
+    }
     if (!rc) {
         lookup_fix_sums((Fr*)sums_host, job->rounds, job->n1);
         bm = to_mont(bm);          // the products carried R^-1

@@ -555,6 +555,12 @@ static bool launch_gemm_all(int pa, int pb, dim3 grid, hipStream_t st, const Pla
 // Measurement: every launch of k_gemm_i8_planes between zk_prof_gemm_begin and zk_prof_gemm_read is timed with events on its stream.
 struct GemmTimer { bool on = false; std::mutex mu; std::vector<std::pair<hipEvent_t, hipEvent_t>> ev; double macs = 0; };
 static GemmTimer g_gemm_timer;
+static const int g_gemm_timer_hook = (at_shutdown([] {
+    std::lock_guard<std::mutex> lk(g_gemm_timer.mu);
+    for (auto& e : g_gemm_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
+    g_gemm_timer.ev.clear();
+    g_gemm_timer.on = false;
+}), 0);
 static int digits_for(unsigned long long absmax) {      // planes needed for |x| <= absmax: p digits reach 127 (256^p - 1) / 255
     int p = 1;
     unsigned __int128 reach = 127;

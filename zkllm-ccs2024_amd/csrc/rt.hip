@@ -66,7 +66,11 @@ static void order_behind_last_user(Pool& P, const Block& blk, hipStream_t stream
         if (hipStreamWaitEvent(stream, blk.ev, 0) != hipSuccess) { (void)hipGetLastError(); (void)hipDeviceSynchronize(); }
         return;
     }
-    uint64_t& covered = P.synced[std::make_pair(blk.last, stream)];
+    // What an earlier wait already covers is remembered only for takers that live as long as the process (the default stream and
+    // the library's own): a caller's stream may be destroyed and its handle value given to a new stream, which has waited for
+    // nothing.  A caller's stream gets its wait every time.
+    uint64_t scratch_covered = 0;
+    uint64_t& covered = is_persistent_stream(stream) ? P.synced[std::make_pair(blk.last, stream)] : scratch_covered;
     if (blk.freed_tick <= covered && covered != 0) return;      // an earlier wait of this stream on that one was placed after this block's free
     const uint64_t now = P.tick;
     hipEvent_t& ev = P.events[P.next_event++ % 32];
@@ -181,6 +185,11 @@ hipStream_t side_stream(int pool) {
     return s;
 }
 
+// hooks are registered by static initialisers of the other files: the list is made on first use and never destroyed
+static std::mutex& shutdown_mu() { static std::mutex* m = new std::mutex; return *m; }
+static std::vector<void (*)()>& shutdown_hooks() { static std::vector<void (*)()>* v = new std::vector<void (*)()>; return *v; }
+void at_shutdown(void (*fn)()) { std::lock_guard<std::mutex> lk(shutdown_mu()); shutdown_hooks().push_back(fn); }
+
 static std::mutex g_pinned_mu;
 static std::vector<void*> g_pinned_free;
 int pinned_acquire(void** host_ptr) {
@@ -243,6 +252,39 @@ int zk_malloc(void** out, size_t bytes) { ZK_ARG(out != nullptr, "zk_malloc: nul
 int zk_free(void* p) { return pool_free(p, nullptr); }
 int zk_free_async(void* p, void* stream) { return pool_free(p, (hipStream_t)stream); }
 int zk_pool_trim(void) { return pool_trim(); }
+// Releases what the library holds on the device and in the runtime, in a fixed order, while the runtime is certainly alive:
+// waits for the device, lets the kernel files drop their timing events, gives the cached blocks back (live blocks stay with
+// their owners), destroys the library's streams and the allocator's events and frees the pinned buffers that are not in use.
+// The library stays usable: streams and buffers are made again on demand.  For a host that wants nothing of this left to
+// static destruction at process exit.
+int zk_shutdown(void) {
+    (void)hipDeviceSynchronize();
+    {
+        std::lock_guard<std::mutex> lk(shutdown_mu());
+        for (void (*fn)() : shutdown_hooks()) fn();
+    }
+    pool_trim();
+    {
+        std::lock_guard<std::mutex> lk(g_side_mu);
+        for (auto& row : g_side_streams)
+            for (hipStream_t& t : row)
+                if (t) { (void)hipStreamDestroy(t); t = nullptr; }
+    }
+    {
+        Pool& P = pool();
+        std::lock_guard<std::mutex> lk(P.mu);
+        for (hipEvent_t& e : P.events) if (e) { (void)hipEventDestroy(e); e = nullptr; }
+        P.synced.clear();
+        for (auto& kv : P.live) if (kv.second.ev) { (void)hipEventDestroy(kv.second.ev); kv.second.ev = nullptr; kv.second.ev_set = false; kv.second.idle = true; }      // the device is idle
+    }
+    {
+        std::lock_guard<std::mutex> lk(g_pinned_mu);
+        for (void* p : g_pinned_free) (void)hipHostFree(p);
+        g_pinned_free.clear();
+    }
+    (void)hipGetLastError();
+    return 0;
+}
 int zk_pool_stats(size_t* live_bytes, size_t* cached_bytes) {
     Pool& P = pool();
     std::lock_guard<std::mutex> lk(P.mu);

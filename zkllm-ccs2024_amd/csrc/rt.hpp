@@ -83,6 +83,10 @@ int staging(void** host_ptr, size_t bytes);
 // by zk_init so that the entry point itself has nothing left to set up.
 int fr_static_scratch_setup();
 
+// fn is called by zk_shutdown (device idle, before the cached blocks are given back): a file drops the events and cached
+// buffers it holds in static objects
+void at_shutdown(void (*fn)());
+
 static inline unsigned cdiv(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
 
 }  // namespace zk

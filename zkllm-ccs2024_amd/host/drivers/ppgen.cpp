@@ -3,6 +3,7 @@
 #include "commitment.hpp"
 
 int main(int argc, char* argv[]) {
+    ZkLibraryScope library;      // releases the library\'s device state when main returns
     if (argc < 3) { std::cerr << "usage: ppgen size output.bin" << std::endl; return 2; }
     const uint size = (uint)std::stoul(argv[1]);
     Commitment::random(1u << ceilLog2(size)).normalized().save(argv[2]);

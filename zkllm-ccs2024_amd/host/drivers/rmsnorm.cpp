@@ -4,6 +4,7 @@
 #include "layer.hpp"
 
 int main(int argc, char* argv[]) {
+    ZkLibraryScope library;      // releases the library\'s device state when main returns
     if (argc < 8) { std::cerr << "usage: rmsnorm which input.bin seq_len embed_dim workdir layer_prefix output.bin" << std::endl; return 2; }
     string which = argv[1];
     string input_file_name = argv[2];

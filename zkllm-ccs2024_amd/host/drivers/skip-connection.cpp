@@ -3,6 +3,7 @@
 #include "fr-tensor.hpp"
 
 int main(int argc, char* argv[]) {
+    ZkLibraryScope library;      // releases the library\'s device state when main returns
     if (argc < 4) { std::cerr << "usage: skip-connection block_input.bin block_output.bin output.bin" << std::endl; return 2; }
     FrTensor x = FrTensor::from_int_bin(argv[1]);
     FrTensor y = FrTensor::from_int_bin(argv[2]);

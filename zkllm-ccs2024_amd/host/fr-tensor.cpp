@@ -70,6 +70,7 @@ void zk_write_proof_file(const std::string& path) {
 const std::vector<Fr_t>& zk_transcript() { return G().transcript; }
 void zk_transcript_end() { G().recording = false; }
 void zk_record(const Fr_t& x) { if (G().recording) G().transcript.push_back(x); }
+ZkLibraryScope::~ZkLibraryScope() { (void)zk_shutdown(); }
 size_t zk_record_reserve() {
     if (!G().recording) return (size_t)-1;
     G().transcript.push_back(Fr_t{{0, 0, 0, 0, 0, 0, 0, 0}});

@@ -65,6 +65,16 @@ void zk_write_proof_file(const std::string& path);
 
 void zk_check(int rc, const char* where);   // throws std::runtime_error on a non-zero C-ABI status
 
+// First object of a program's main(): when main returns, after every tensor declared behind it has been released, the library
+// gives back its streams, events and cached device memory (zk_shutdown) while the runtime is alive, so nothing of that is
+// left to static destruction at process exit.
+struct ZkLibraryScope {
+    ZkLibraryScope() = default;
+    ~ZkLibraryScope();
+    ZkLibraryScope(const ZkLibraryScope&) = delete;
+    ZkLibraryScope& operator=(const ZkLibraryScope&) = delete;
+};
+
 // What a tensor that serves as the right operand of many matrix products keeps between them (FrTensor::keep_as_matmul_rhs):
 // the handle of zk_fr_matmul_rhs_prepare.  Shared by the tensor and its views.
 struct MatmulRhsCache {

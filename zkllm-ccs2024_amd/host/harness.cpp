@@ -541,6 +541,7 @@ void zkp_layer_set_open_weights(void* h, int on) { reinterpret_cast<LayerState*>
 // setup times of the last zkp_layer_create_random (ms): weights, generators, commitments, prepared generators
 void zkp_layer_setup_times(double* out4) { const LayerSetupTimes& t = layer_setup_times(); out4[0] = t.weights; out4[1] = t.generators; out4[2] = t.commitments; out4[3] = t.prepare; }
 void zkp_openings_use_cross_commitments(int on) { zk_openings_use_cross_commitments(on != 0); }
+int zkp_shutdown() { return zk_shutdown(); }
 void zkp_openings_use_row_commitments(int on) { zk_openings_use_row_commitments(on != 0); }
 // on: every weight opening starts at its claim or later (no learned plan, nothing started ahead inside a block)
 void zkp_openings_set_only_at_claim(int on) { zk_openings_set_only_at_claim(on != 0); }
