@@ -40,6 +40,97 @@ MAD_PER_FP_MUL = 300                                   # 2 * 12^2 + 12 limb prod
 MAD_PER_FR_MUL = 136                                   # 2 * 8^2 + 8
 
 
+def drivers_leg(seq):
+    """The drop-in chain at the 7B shape: the per-block executables run as child processes over .bin files with the argument
+    lists of the reference's llama-*.py scripts (README.md:60-80, llama-ppgen.py:21-31, llama-commit.py:31-46, llama-rmsnorm.py:35-45,
+    llama-self-attn.py:41-81, llama-ffn.py:26-43).  Returns wall time per executable and its phases (ZKLLM_TIMING=1)."""
+    import shutil
+    import subprocess
+    import tempfile
+    E, Hd, lof = 4096, 11008, 5
+    exe_dir = os.path.join(ROOT, "zkllm-ccs2024_amd", "host")
+    tmp = tempfile.mkdtemp(prefix="zkllm_drivers_", dir=os.environ.get("TMPDIR", "/tmp"))
+    work = os.path.join(tmp, "zkllm-workdir", "Llama-2-7b")
+    os.makedirs(work)
+    prefix = "layer-0"
+    out = {"shape": f"seq {seq}, hidden {E}, FFN {Hd}, log_off_factor {lof}", "runs": []}
+
+    def run(label, argv, env_extra=None):
+        env = dict(os.environ, ZKLLM_TIMING="1", ZKLLM_SEED="7")
+        env.update(env_extra or {})
+        t0 = time.perf_counter()
+        r = subprocess.run([os.path.join(exe_dir, argv[0])] + [str(a) for a in argv[1:]], cwd=tmp, env=env, capture_output=True, text=True, timeout=600)
+        wall = time.perf_counter() - t0
+        if r.returncode != 0:
+            raise RuntimeError(f"{label}: {argv[0]} exited with {r.returncode}: {r.stderr[-800:]}")
+        phases = {}
+        for line in r.stderr.splitlines():
+            if line.startswith("ZKLLM_TIMES "):
+                phases = {k: round(v, 1) for k, v in json.loads(line[len("ZKLLM_TIMES "):]).items()}
+        rec = {"run": label, "wall_s": round(wall, 3), "phases_ms": phases, "process_start_and_exit_s": round(wall - sum(phases.values()) / 1e3, 3)}
+        out["runs"].append(rec)
+        return rec
+
+    try:
+        rng = np.random.default_rng(7)
+        params = [("input_layernorm.weight", (E,)), ("self_attn.q_proj.weight", (E, E)), ("self_attn.k_proj.weight", (E, E)), ("self_attn.v_proj.weight", (E, E)),
+                  ("post_attention_layernorm.weight", (E,)), ("mlp.up_proj.weight", (E, Hd)), ("mlp.gate_proj.weight", (E, Hd)), ("mlp.down_proj.weight", (Hd, E))]
+        setup = {"ppgen_s": 0.0, "commit_param_s": 0.0, "cross_commitments_ms": 0.0}
+        for name, shape in params:
+            pp, ib, cb = (os.path.join(work, f) for f in (f"{name}-pp.bin", f"{prefix}-{name}-int.bin", f"{prefix}-{name}-commitment.bin"))
+            if len(shape) == 1:
+                w = np.full(shape, 65536, np.int32)
+                pp_size, dims = shape[0], (shape[0], 1)
+            else:
+                w = np.round(rng.normal(0, 0.02, shape) * 65536).astype(np.int32)      # in x out, as llama-commit.py saves w.T
+                pp_size, dims = shape[1] << lof, shape
+            w.tofile(ib)
+            setup["ppgen_s"] += run(f"ppgen {name}", ["ppgen", pp_size, pp])["wall_s"]
+            rec = run(f"commit-param {name}", ["commit-param", pp, ib, cb, dims[0], dims[1]])
+            setup["commit_param_s"] += rec["wall_s"]
+            setup["cross_commitments_ms"] += rec["phases_ms"].get("cross_commitments_ms", 0.0)
+        out["setup_runs"], out["runs"] = out["runs"], []
+        out["setup_s"] = {k: round(v, 3) for k, v in setup.items()}
+        X = np.round(rng.normal(0, 1, (seq, E)) * 65536).astype(np.int32)
+        X.tofile(os.path.join(tmp, "layer_input.bin"))
+
+        def rms_inv_file(x_int):
+            xf = x_int.astype(np.float64) / 65536.0
+            np.rint(1.0 / np.sqrt(np.mean(xf ** 2, axis=1) + 1e-5) * 65536.0).astype(np.int32).tofile(os.path.join(tmp, "rms_inv_temp.bin"))
+        xs = (np.arange(-(1 << 21), 1 << 21, dtype=np.float64)) / 4096.0
+        np.rint(xs / (1.0 + np.exp(-xs)) * 16.0).astype(np.int32).tofile(os.path.join(tmp, "swiglu-table.bin"))      # llama-ffn.py:15-18 (save_int with 16)
+        rms_inv_file(X)
+        t_chain = time.perf_counter()
+        run("rmsnorm input", ["rmsnorm", "input", "layer_input.bin", seq, E, work, prefix, "attn_input.bin"])
+        run("self-attn linear", ["self-attn", "linear", "attn_input.bin", seq, E, work, prefix, "attn_output.bin"])
+        # the attention of all 32 heads as one stack (ZKLLM_ATTN_HEADS / ZKLLM_ATTN_HEAD_GROUP, additions); the reference's attn mode
+        # proves ONE head as wide as the embedding and leaves its output argument alone, so its chain cannot go on from there
+        run("self-attn attn (32 heads, stacked)", ["self-attn", "attn", "attn_input.bin", seq, E, work, prefix, "attn_output.bin"],
+            {"ZKLLM_ATTN_HEADS": "32", "ZKLLM_ATTN_HEAD_GROUP": "32"})
+        run("skip-connection", ["skip-connection", "layer_input.bin", "attn_output.bin", "post_attn_norm_input.bin"])
+        x2 = np.fromfile(os.path.join(tmp, "post_attn_norm_input.bin"), dtype=np.int32).reshape(seq, E)
+        rms_inv_file(x2)
+        run("rmsnorm post_attention", ["rmsnorm", "post_attention", "post_attn_norm_input.bin", seq, E, work, prefix, "ffn_input.bin"])
+        run("ffn", ["ffn", "ffn_input.bin", seq, E, Hd, work, prefix, "ffn_output.bin"], {"ZKLLM_FFN_SAVE_RESCALED": "1"})
+        run("skip-connection", ["skip-connection", "post_attn_norm_input.bin", "ffn_output.bin", "layer_output.bin"])
+        out["chain_wall_s"] = round(time.perf_counter() - t_chain, 3)
+        out["chain_prove_s"] = round(sum(r["phases_ms"].get("prove_ms", 0.0) for r in out["runs"]) / 1e3, 3)
+        chain = list(out["runs"])
+        # the same three blocks that open weights, without the cross-commitment side files (ZKLLM_OPEN_CROSS_ROUNDS=0: create_weight
+        # ignores them): every opening sums over its generators in every round
+        out["runs"] = []
+        for label, argv in (("rmsnorm input", ["rmsnorm", "input", "layer_input.bin", seq, E, work, prefix, "attn_input_2.bin"]),
+                            ("self-attn linear", ["self-attn", "linear", "attn_input.bin", seq, E, work, prefix, "attn_output_2.bin"]),
+                            ("ffn", ["ffn", "ffn_input.bin", seq, E, Hd, work, prefix, "ffn_output_2.bin"])):
+            run(label + " without cross commitments", argv, {"ZKLLM_OPEN_CROSS_ROUNDS": "0", "ZKLLM_FFN_SAVE_RESCALED": "1"})
+        out["runs_without_cross_commitment_files"], out["runs"] = out["runs"], chain
+        out["note"] = ("every run is a fresh process: runtime start-up, files read and uploaded (load_*), generators prepared for openings "
+                       "(prepare_generators_ms: the fixed-base tables of the folds), the block's proof with its openings (prove_ms), outputs written")
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -53,6 +144,9 @@ def main():
     ap.add_argument("--skip-extras", action="store_true", help="only the layer timing (used for profiling runs)")
     ap.add_argument("--at-claim", action="store_true",
                     help="the timed layers start every weight opening at its claim (what layer_openings_at_claim_s reports); for profiling runs")
+    ap.add_argument("--drivers", action="store_true",
+                    help="also run the per-block executables over .bin files at the 7B shape (child processes) and report their wall times")
+    ap.add_argument("--drivers-only", action="store_true", help="only the executables' chain (no in-process layer)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: three launches of the opening's fold kernel at 262144 pairs, one hinted lookup "
                          "sumcheck over 2^27 queries, the Montgomery product, the three-level fold, the commitment of config 3 and one "
@@ -62,6 +156,10 @@ def main():
         print("bench.py: this prover runs on one GPU; every configuration of the benchmark fits a single MI355X, "
               "so --gpus must be 1 (no multi-GPU path exists in this build)", file=sys.stderr)
         sys.exit(2)
+
+    if args.drivers_only:
+        print(json.dumps({"drivers_chain": drivers_leg(args.seq)}))
+        return
 
     from gpuhelp import Hip, Prover, c_int, c_size_t, c_uint, c_void_p
     import layercfg
@@ -639,6 +737,13 @@ def main():
                                "parts_s": {k_: round(v_, 1) for k_, v_ in parts_cpu.items()},
                                "config1_zkfc_toy_s": c1_s, "config4_lookup_s": c4_s, "config2_proof_s": c2_prove_s, "softmax_hadamard_one_head_s": hadamard_head_s,
                                "fr_mul_per_s_all_cores": mm_rate}
+    if args.drivers:
+        del pv, hip
+        lib.zk_shutdown()          # the child processes need the device memory this process held in its pool
+        try:
+            out["drivers_chain"] = drivers_leg(args.seq)
+        except Exception as e:          # never loses the headline line
+            out["drivers_chain"] = {"error": str(e)[:600]}
     print(json.dumps(out))
     lib.zk_shutdown()
 

@@ -200,6 +200,63 @@ def test_executables_chain_over_bin_files_matches_the_oracle_byte_for_byte(tmp_p
     assert (np.fromfile(tmp_path / "layer_output.bin", dtype=np.int32) == x2 + f_out).all()
 
 
+def test_cross_commitment_side_files_change_no_byte_of_outputs_or_proof(tmp_path):
+    """commit-param writes a weight's cross commitments beside its commitment (<commitment>.cross, an addition) and create_weight
+    picks them up: the openings of `self-attn linear` then take T, T0, T1 of their first three rounds from them.  16384 generators
+    per weight, the smallest set with three such rounds.  The block runs with the side files, without them (every sum over all
+    generators), and with the three-round fold tables on top (ZKLLM_OPEN_TABLES=3): the same output files and the same proof
+    file, byte for byte, and that proof is the oracle's (field transcript and normalised G1 points)."""
+    import ctypes
+    orc = load_oracle()
+    orc.dll.orc_g1_transcript_size.restype = ctypes.c_long
+    S, E, lof = 16, 128, 7
+    cu, cf = layercfg.pack(S, E, 2, 256, 1 << 8, 1 << 10, 1 << 7, [1 << 8, 1 << 8, 1 << 8], 1, 0, 1 << 16, [1 << 6, 1 << 8], -512, 1024, 64.0, value_scale=256.0)
+    rng = np.random.default_rng(77)
+    work = tmp_path / "zkllm-workdir"
+    work.mkdir()
+    prefix = "layer-0"
+    W = {}
+    seed = 400
+    for name in ("q", "k", "v"):
+        full = f"self_attn.{name}_proj.weight"
+        w = np.round(rng.normal(0, 0.25, (E, E)) * 256).astype(np.int32)
+        pp, ib, cb = work / f"{full}-pp.bin", work / f"{prefix}-{full}-int.bin", work / f"{prefix}-{full}-commitment.bin"
+        seed += 1
+        run(tmp_path, seed, None, "ppgen", E << lof, pp, config=None)
+        w.tofile(ib)
+        run(tmp_path, seed, None, "commit-param", pp, ib, cb, E, E, config=None)
+        gens, com = g1_file(pp), g1_file(cb)
+        assert gens.shape == (E << lof, 36) and com.shape == (1, 36)
+        cross = g1_file(str(cb) + ".cross")
+        assert cross.shape == (43, 36) and (cross[0] == com[0]).all()          # 1 + 2 + 8 + 32 patterns of one row; pattern 0 is the commitment
+        W[name] = OracleWeight(orc, w, E, E, gens, com)
+    X = np.round(rng.normal(0, 1, (S, E)) * 256).astype(np.int32)
+    X.tofile(tmp_path / "attn_input.bin")
+    results = []
+    for label, env, hide in (("side files", {}, False), ("no side files", {}, True), ("side files and three-round tables", {"ZKLLM_OPEN_TABLES": "3"}, False)):
+        moved = []
+        if hide:
+            for f in work.glob("*.cross"):
+                f.rename(str(f) + ".hidden")
+                moved.append(f)
+        proof = tmp_path / f"linear_{len(results)}.proof"
+        run(tmp_path, 410, proof, "self-attn", "linear", "attn_input.bin", S, E, work, prefix, "unused.bin", extra_env=env)
+        for f in moved:
+            (f.parent / (f.name + ".hidden")).rename(f)
+        results.append((label, open(proof, "rb").read(), [open(tmp_path / f"temp_{n}.bin", "rb").read() for n in "QKV"]))
+    for label, pf, outs in results[1:]:
+        assert pf == results[0][1], label
+        assert outs == results[0][2], label
+    eQ, eK, eV = (np.zeros((S * E, 8), np.uint32) for _ in range(3))
+    orc.orc_seed(410)
+    orc.orc_transcript_clear()
+    orc_check(orc.orc_attn_linear_block(cu, cf, W["q"].h, W["k"].h, W["v"].h, as_fr(X), eQ, eK, eV))
+    n_fr, n_g1 = check_proof(orc, tmp_path / "linear_0.proof", "side files")
+    assert n_g1 == 3 * (3 * 14 + 1)
+    Q = np.fromfile(tmp_path / "temp_Q.bin", dtype=np.int32)
+    assert (Q == fr_to_i64(eQ)).all()
+
+
 def test_self_attn_with_heads_from_the_environment_writes_the_output_file(tmp_path):
     """ZKLLM_ATTN_HEADS / ZKLLM_ATTN_HEAD_GROUP (additions): per-head and stacked attention through the executable, against the
     oracle's attention block for the same head count"""

@@ -311,20 +311,27 @@ static bool load_weight_cross(Weight& w, const string& com_filename) {
 }
 
 Weight create_weight(string generator_filename, string weight_filename, string com_filename, uint in_dim, uint out_dim) {
+    zk_phase_end("other_ms");
     Commitment generator(generator_filename);
+    zk_phase_end("load_generators_ms");
     FrTensor weight = FrTensor::from_int_bin(weight_filename);
     G1TensorJacobian com(com_filename);
-    Weight w{generator, weight, com, in_dim, out_dim, nullptr};
+    Weight w{std::move(generator), std::move(weight), std::move(com), in_dim, out_dim, nullptr};
     w.weight.keep_for_folds();          // proofs and openings fold it at a new point each time
     if (in_dim != (1u << ceilLog2(in_dim)) || out_dim != (1u << ceilLog2(out_dim))) {
         auto pd = std::make_shared<FrTensor>(w.weight.pad({in_dim, out_dim}));
         pd->keep_for_folds();
         w.padded = pd;
     }
-    // with three rounds of cross commitments from the side file the openings fold three rounds at once: the generators get
-    // those tables; otherwise the tables of the first two rounds
+    zk_phase_end("load_weight_and_commitment_ms");
     load_weight_cross(w, com_filename);
-    w.generator.prepare_openings(w.cross_rounds >= 3 ? 3 : 2);
+    zk_phase_end("load_cross_commitments_ms");
+    // No fold tables by default: a weight made here is usually opened once, by the process that loaded it, and building the
+    // fixed-base tables of its generators (25 KB per generator) costs ten times what they save on one opening.  A process that
+    // keeps its weights and opens them many times asks for them with ZKLLM_OPEN_TABLES=3 (three rounds as one fold; needs the
+    // cross commitments) or =2.
+    w.generator.prepare_openings(0);
+    zk_phase_end("prepare_generators_ms");
     return w;
 }
 
@@ -340,8 +347,11 @@ uint commit_param_file(const string& generator_filename, const string& param_fil
     std::unique_ptr<FrTensor> padded;
     if (ragged) padded.reset(new FrTensor(param.pad({in_dim, out_dim})));
     const FrTensor& t = ragged ? *padded : param;
+    zk_phase_end("load_ms");
     G1TensorJacobian com = generator.commit_int(t);
+    zk_phase_end("commit_ms");
     com.normalized().save(output_filename);
+    zk_phase_end("save_ms");
     // addition: the cross commitments of the first three opening rounds beside the commitment (seven times its work; what
     // create_weight picks up so that verifyWeightClaim needs no sums over all generators in those rounds).
     // ZKLLM_COMMIT_CROSS=0 leaves the side file out, =k writes k rounds.
@@ -351,5 +361,6 @@ uint commit_param_file(const string& generator_filename, const string& param_fil
     const string side = cross_commitment_filename(output_filename);
     if (rounds > 0) generator.cross_commitments(t, com, rounds).normalized().save(side);
     else std::remove(side.c_str());          // never leave a side file of an older commitment behind
+    zk_phase_end("cross_commitments_ms");
     return com.size;
 }

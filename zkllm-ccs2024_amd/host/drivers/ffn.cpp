@@ -29,10 +29,13 @@ int main(int argc, char* argv[]) {
     c.swiglu_low = -(int)(swiglu_values.size >> 1);
     FrTensor input = FrTensor::from_int_bin(input_file_name);
     std::unique_ptr<FrTensor> down_out;
+    zk_phase_end("load_inputs_ms");
     FrTensor down_out_ = ffn_block(c, up_proj, gate_proj, down_proj, swiglu_values, input, &down_out);
+    openings.finish();
+    zk_phase_end("prove_ms");
     const char* rescaled = getenv("ZKLLM_FFN_SAVE_RESCALED");
     if (rescaled && rescaled[0] == '1') down_out_.save_int(output_file_name);
     else down_out->save_int(output_file_name);
-    openings.finish();
+    zk_phase_end("save_outputs_ms");
     return 0;
 }

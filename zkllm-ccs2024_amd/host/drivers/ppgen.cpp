@@ -7,5 +7,6 @@ int main(int argc, char* argv[]) {
     if (argc < 3) { std::cerr << "usage: ppgen size output.bin" << std::endl; return 2; }
     const uint size = (uint)std::stoul(argv[1]);
     Commitment::random(1u << ceilLog2(size)).normalized().save(argv[2]);
+    zk_phase_end("generate_and_save_ms");
     return 0;
 }

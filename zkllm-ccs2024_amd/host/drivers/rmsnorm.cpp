@@ -21,8 +21,11 @@ int main(int argc, char* argv[]) {
     FrTensor X = FrTensor::from_int_bin(input_file_name);
     FrTensor rms_inv_temp = FrTensor::from_int_bin("rms_inv_temp.bin");
     DeferredOpenings openings;      // the weight opening runs on the device beside the rest of the proof
+    zk_phase_end("load_inputs_ms");
     FrTensor Y_ = rmsnorm_block(c, rmsnorm_weight, X, rms_inv_temp);
-    Y_.save_int(output_file_name);
     openings.finish();
+    zk_phase_end("prove_ms");
+    Y_.save_int(output_file_name);
+    zk_phase_end("save_outputs_ms");
     return 0;
 }

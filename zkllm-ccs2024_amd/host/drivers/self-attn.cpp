@@ -31,27 +31,36 @@ int main(int argc, char* argv[]) {
         auto q_proj = w("q"), k_proj = w("k"), v_proj = w("v");
         FrTensor input = FrTensor::from_int_bin(input_file_name);
         FrTensor Q_(input.size), K_(input.size), V_(input.size);
+        zk_phase_end("load_inputs_ms");
         attn_linear_block(c, q_proj, k_proj, v_proj, input, Q_, K_, V_);
+        openings.finish();
+        zk_phase_end("prove_ms");
         Q_.save_int("temp_Q.bin");
         K_.save_int("temp_K.bin");
         V_.save_int("temp_V.bin");
+        zk_phase_end("save_outputs_ms");
         cout << "QKV linear proof successfully verified!" << endl;
     } else if (mode == "attn") {
         auto Q = FrTensor::from_int_bin("temp_Q.bin");
         auto K = FrTensor::from_int_bin("temp_K.bin");
         auto V = FrTensor::from_int_bin("temp_V.bin");
+        zk_phase_end("load_inputs_ms");
         const char* heads = getenv("ZKLLM_ATTN_HEADS");
         if (heads && atoi(heads) > 0) {
             c.num_heads = atoi(heads);
             if (const char* g = getenv("ZKLLM_ATTN_HEAD_GROUP")) c.attn_head_group = atoi(g);
             FrTensor out = attn_heads_block(c, Q, K, V);
+            zk_phase_end("prove_ms");
             out.save_int("temp_head_out.bin");
             out.save_int(output_file_name);
+            zk_phase_end("save_outputs_ms");
         } else {
             std::unique_ptr<FrTensor> Y;
             FrTensor out = attn_reference_block(c, Q, K, V, &Y);
+            zk_phase_end("prove_ms");
             Y->save_long("temp_head_Y.bin");
             out.save_int("temp_head_out.bin");
+            zk_phase_end("save_outputs_ms");
         }
         cout << "Self attention proof successfully verified!" << endl;
     }

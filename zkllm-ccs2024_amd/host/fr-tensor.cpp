@@ -1,5 +1,6 @@
 #include <memory>
 #include "fr-tensor.hpp"
+#include <chrono>
 
 #include <climits>
 #include <cstdio>
@@ -70,7 +71,40 @@ void zk_write_proof_file(const std::string& path) {
 const std::vector<Fr_t>& zk_transcript() { return G().transcript; }
 void zk_transcript_end() { G().recording = false; }
 void zk_record(const Fr_t& x) { if (G().recording) G().transcript.push_back(x); }
-ZkLibraryScope::~ZkLibraryScope() { (void)zk_shutdown(); }
+namespace {
+struct PhaseTimes {
+    bool on = false;
+    std::chrono::steady_clock::time_point last;
+    std::vector<std::pair<std::string, double>> ms;
+};
+PhaseTimes& phases() { static PhaseTimes p; return p; }
+}  // namespace
+void zk_phase_end(const char* name) {
+    PhaseTimes& p = phases();
+    if (!p.on) return;
+    (void)zk_sync(nullptr);
+    const auto now = std::chrono::steady_clock::now();
+    const double d = std::chrono::duration<double, std::milli>(now - p.last).count();
+    p.last = now;
+    for (auto& kv : p.ms) if (kv.first == name) { kv.second += d; return; }
+    p.ms.emplace_back(name, d);
+}
+ZkLibraryScope::ZkLibraryScope() {
+    const char* e = getenv("ZKLLM_TIMING");
+    phases().on = e && e[0] == '1';
+    phases().last = std::chrono::steady_clock::now();
+}
+ZkLibraryScope::~ZkLibraryScope() {
+    zk_phase_end("release_ms");
+    (void)zk_shutdown();
+    PhaseTimes& p = phases();
+    if (p.on) {
+        zk_phase_end("shutdown_ms");
+        std::cerr << "ZKLLM_TIMES {";
+        for (size_t i = 0; i < p.ms.size(); ++i) std::cerr << (i ? ", " : "") << "\"" << p.ms[i].first << "\": " << p.ms[i].second;
+        std::cerr << "}" << std::endl;
+    }
+}
 size_t zk_record_reserve() {
     if (!G().recording) return (size_t)-1;
     G().transcript.push_back(Fr_t{{0, 0, 0, 0, 0, 0, 0, 0}});

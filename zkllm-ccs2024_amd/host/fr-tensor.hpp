@@ -65,11 +65,17 @@ void zk_write_proof_file(const std::string& path);
 
 void zk_check(int rc, const char* where);   // throws std::runtime_error on a non-zero C-ABI status
 
+// Phase timing of the executables (no effect unless ZKLLM_TIMING=1): the time since the previous call (or since the
+// ZkLibraryScope was made) is added to the phase `name`; the device is waited for first.
+void zk_phase_end(const char* name);
+
 // First object of a program's main(): when main returns, after every tensor declared behind it has been released, the library
 // gives back its streams, events and cached device memory (zk_shutdown) while the runtime is alive, so nothing of that is
 // left to static destruction at process exit.
+// With ZKLLM_TIMING=1 in the environment it also prints, when main returns, one line "ZKLLM_TIMES {...}" to stderr: the wall
+// time of the program's phases in ms (zk_phase_end calls, each taken with the device idle).
 struct ZkLibraryScope {
-    ZkLibraryScope() = default;
+    ZkLibraryScope();
     ~ZkLibraryScope();
     ZkLibraryScope(const ZkLibraryScope&) = delete;
     ZkLibraryScope& operator=(const ZkLibraryScope&) = delete;
