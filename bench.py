@@ -304,6 +304,17 @@ def main():
     layer = pv.layer_create_random(cu, cf, 7, 5)
     pv.sync()
     setup_s = time.perf_counter() - t0
+
+    def pool_gib():
+        live_b, cached_b = ctypes.c_size_t(), ctypes.c_size_t()
+        hip.check(lib.zk_pool_stats(ctypes.byref(live_b), ctypes.byref(cached_b)))
+        return live_b.value / 2 ** 30, cached_b.value / 2 ** 30
+    # memory: what the setup leaves resident (weights with their int32 forms and digit planes, generators, commitments, cross
+    # commitments, the openings' fold tables) and what its construction used on top and gives back here
+    setup_live_gib, setup_cached_gib = pool_gib()
+    lib.zk_pool_trim()
+    pv.lib.zkp_layer_opening_table_bytes.restype = ctypes.c_double
+    tables_gib = pv.lib.zkp_layer_opening_table_bytes(c_void_p(layer)) / 2 ** 30
     setup4 = np.zeros(4)
     pv.lib.zkp_layer_setup_times(setup4.ctypes.data_as(ctypes.POINTER(ctypes.c_double)))
     pv.lib.zkp_layer_setup_cross_ms.restype = ctypes.c_double
@@ -370,9 +381,8 @@ def main():
         os.dup2(saved_stdout, 1)
     ms_per_step = wall * 1e3 / args.steps
     parts /= args.steps
-    live_b, cached_b = ctypes.c_size_t(), ctypes.c_size_t()
-    hip.check(lib.zk_pool_stats(ctypes.byref(live_b), ctypes.byref(cached_b)))
-    pool_gib = (live_b.value + cached_b.value) / 2 ** 30      # the allocator keeps what it once needed: live + cached = the layer's peak
+    run_live_gib, run_cached_gib = pool_gib()
+    peak_gib = run_live_gib + run_cached_gib      # the allocator keeps what it once needed: live + cached behind the runs = their peak
     pv.layer_free(layer)
     lib.zk_pool_trim()
     # The layer with its openings summing over the generators in every round: no cross commitments of the weights, and the
@@ -408,7 +418,11 @@ def main():
                                "(their points are read ahead from the seeded challenge stream, so all nine run from the start of the layer, batched by "
                                "generator size); attention proved "
                                + (f"{args.head_group} heads at a time as head-major stacks (zkAttnStacked)" if args.head_group else "head by head"),
-                   "device_pool_gib": round(pool_gib, 1),
+                   "device_pool_gib": round(peak_gib, 1),
+                   "memory_gib": {"peak_during_layer_runs": round(peak_gib, 1), "fold_tables_of_the_generators": round(tables_gib, 1),
+                                  "resident_weights_generators_commitments": round(setup_live_gib - tables_gib, 1),
+                                  "proof_working_set": round(peak_gib - setup_live_gib, 1),
+                                  "setup_scratch_given_back_before_the_runs": round(setup_cached_gib, 1)},
                    "setup_s_untimed": round(setup_s, 3),
                    "setup_parts_s": {"random_weights_host_and_upload": round(setup4[0] / 1e3, 3), "generators": round(setup4[1] / 1e3, 3),
                                      "commitments": round(setup4[2] / 1e3, 3), "generators_prepared_for_openings": round(setup4[3] / 1e3, 3),

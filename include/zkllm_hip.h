@@ -230,6 +230,12 @@ int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stream
  * zk_g1_open_begin_batch_rows and cross_rounds >= 3, whose first three rounds read no folded generators; any other opening
  * over such a handle folds by the walk.  Needs a power of two of at least 16384 generators, else 3 means 2. */
 int zk_g1_open_prepare_tables(void** prepared, const void* gens, size_t n, int tables, void* stream);
+/* The same with a byte budget for the tables instead of a fixed choice (no counterpart in the reference): makes the richest
+ * mode <= want whose tables fit max_table_bytes (3: 24990 B per generator, 2: 28560, 1: 14280, 0: none) and reports it in
+ * *tables_made (may be null).  _table_bytes: what a mode would keep for n generators; _prepared_table_bytes: what a handle keeps. */
+int zk_g1_open_prepare_budget(void** prepared, const void* gens, size_t n, int want, size_t max_table_bytes, int* tables_made, void* stream);
+size_t zk_g1_open_table_bytes(size_t n, int tables);
+size_t zk_g1_open_prepared_table_bytes(const void* prepared);
 int zk_g1_open_prepared_free(void* prepared);
 int zk_g1_open_begin_prepared(void** handle, const void* scalars, const void* prepared, const uint32_t* u, int rounds, void* stream);
 /* `count` (1..8) openings against prepared generator sets of ONE size with ONE round count as a single job: every kernel

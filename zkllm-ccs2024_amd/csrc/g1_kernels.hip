@@ -2075,13 +2075,32 @@ int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_
 // Generators prepared once for any number of openings against them: their affine 29-bit-limb form and the pair sums of
 // the first round (weight-independent; 1.5 n points of 112 bytes).  The handle is freed with zk_g1_open_prepared_free
 // once no opening that uses it is pending.
-struct OpenPrepared { void* a29 = nullptr; size_t n = 0; void* comb = nullptr; void* comb2 = nullptr; void* comb3 = nullptr; };      // comb3: k_open_fold_jump's tables (instead of the other two)
+struct OpenPrepared { void* a29 = nullptr; size_t n = 0; void* comb = nullptr; void* comb2 = nullptr; void* comb3 = nullptr; size_t table_bytes = 0; };      // comb3: k_open_fold_jump's tables (instead of the other two)
 static int open_prepare_impl(void** prepared, const void* gens, size_t n, int table_mode, void* stv);
 int zk_g1_open_prepare(void** prepared, const void* gens, size_t n, void* stv) { return open_prepare_impl(prepared, gens, n, 2, stv); }
 int zk_g1_open_prepare_tables(void** prepared, const void* gens, size_t n, int tables, void* stv) {
     ZK_ARG(tables >= 0 && tables <= 3, "zk_g1_open_prepare_tables: tables 0 to 3");
     return open_prepare_impl(prepared, gens, n, tables, stv);
 }
+// bytes of fold tables that zk_g1_open_prepare_tables(.., tables) keeps for n generators (0 where that mode makes none for this n)
+static size_t open_table_bytes(size_t n, int tables) {
+    if (tables >= 3 && !(n & (n - 1)) && (n >> JUMP_ROUNDS) >= (size_t)TAIL_N) return sizeof(A29) * (n >> JUMP_ROUNDS) * COMB_N * JUMP_TABS;
+    if (tables < 1 || n <= (size_t)TAIL_N) return 0;
+    const size_t np = (n + 1) / 2, nq = (np + 1) / 2;
+    size_t b = sizeof(A29) * np * COMB_N;
+    if (tables >= 2 && np > (size_t)TAIL_N) b += sizeof(A29) * 2 * nq * COMB_N;
+    return b;
+}
+size_t zk_g1_open_table_bytes(size_t n, int tables) { return open_table_bytes(n, tables < 0 ? 0 : (tables > 3 ? 3 : tables)); }
+// The richest tables that fit `max_table_bytes`: mode `want` (0..3) if its tables fit, else the next smaller mode, down to none.
+int zk_g1_open_prepare_budget(void** prepared, const void* gens, size_t n, int want, size_t max_table_bytes, int* tables_made, void* stv) {
+    ZK_ARG(want >= 0 && want <= 3, "zk_g1_open_prepare_budget: tables 0 to 3");
+    int mode = want;
+    while (mode > 0 && open_table_bytes(n, mode) > max_table_bytes) --mode;
+    if (tables_made) *tables_made = mode;
+    return open_prepare_impl(prepared, gens, n, mode, stv);
+}
+size_t zk_g1_open_prepared_table_bytes(const void* prepared) { return prepared ? ((const OpenPrepared*)prepared)->table_bytes : 0; }
 static int open_prepare_impl(void** prepared, const void* gens, size_t n, int table_mode, void* stv) {
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(prepared != nullptr && n >= 1, "zk_g1_open_prepare: null handle or no generators");
@@ -2209,6 +2228,9 @@ static int open_prepare_impl(void** prepared, const void* gens, size_t n, int ta
         if (pr->comb3) pool_free(pr->comb3, st, true);
         return rc;
     }
+    if (pr->comb3) pr->table_bytes += sizeof(A29) * (n >> JUMP_ROUNDS) * COMB_N * JUMP_TABS;
+    if (pr->comb) pr->table_bytes += sizeof(A29) * ((n + 1) / 2) * COMB_N;
+    if (pr->comb2) pr->table_bytes += sizeof(A29) * 2 * (((n + 1) / 2 + 1) / 2) * COMB_N;
     *prepared = pr.release();
     return 0;
 }

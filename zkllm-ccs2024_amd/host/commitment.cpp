@@ -206,12 +206,13 @@ void Commitment::open_start_batch(const std::vector<std::pair<const Commitment*,
         }
     }
 }
-void Commitment::prepare_openings(int tables) const {
+void Commitment::prepare_openings(int tables, size_t max_table_bytes) const {
     if (prepared || size == 0) return;
     void* h = nullptr;
-    ZKC(zk_g1_open_prepare_tables(&h, gpu_data, size, tables, nullptr));
+    ZKC(zk_g1_open_prepare_budget(&h, gpu_data, size, tables, max_table_bytes, nullptr, nullptr));
     prepared = std::shared_ptr<void>(h, [](void* q) { (void)zk_g1_open_prepared_free(q); });
 }
+size_t Commitment::opening_table_bytes() const { return zk_g1_open_prepared_table_bytes(prepared.get()); }
 Commitment::Pending Commitment::open_begin(const FrTensor& t, const G1TensorJacobian& com, const vector<Fr_t>& u) const {
     Pending p = open_fold(t, com, u);
     open_start(p);

@@ -72,7 +72,9 @@ class Commitment : public G1TensorJacobian {
     // tables (zk_g1_open_prepare_tables): 0 none, 1 / 2 fixed-base tables of the first / first two fold rounds, 3 the tables
     // that fold three rounds at once -- for openings that bring cross commitments of three rounds (prepare_weight_cross);
     // without them such generators fold by the walk
-    void prepare_openings(int tables = 2) const;
+    // max_table_bytes: a budget for the tables; the richest mode <= tables that fits is made (zk_g1_open_prepare_budget)
+    void prepare_openings(int tables = 2, size_t max_table_bytes = ~(size_t)0) const;
+    size_t opening_table_bytes() const;       // device bytes of the fold tables this object keeps
     bool openings_prepared() const { return (bool)prepared; }
 
     static Commitment random(uint size);

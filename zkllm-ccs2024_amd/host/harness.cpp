@@ -535,6 +535,7 @@ void* zkp_layer_create_random(const u32* cu, const double* cf, u32 seed, u32 log
     return new LayerState{c, make_random_layer_weights(c, seed, log_off_factor)};
     ZKP_END_PTR
 }
+double zkp_layer_opening_table_bytes(void* h) { return (double)layer_opening_table_bytes(reinterpret_cast<LayerState*>(h)->w); }
 void zkp_layer_free(void* h) { delete reinterpret_cast<LayerState*>(h); }
 void zkp_layer_set_head_group(void* h, u32 g) { reinterpret_cast<LayerState*>(h)->cfg.attn_head_group = g; }
 void zkp_layer_set_open_weights(void* h, int on) { reinterpret_cast<LayerState*>(h)->cfg.open_weights = on != 0; }

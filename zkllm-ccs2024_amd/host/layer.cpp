@@ -418,7 +418,7 @@ FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor
 
 static LayerSetupTimes g_setup_times;
 const LayerSetupTimes& layer_setup_times() { return g_setup_times; }
-static Weight random_weight(std::mt19937_64& rng, uint in_dim, uint out_dim, uint pp_size, bool norm) {
+static Weight random_weight(std::mt19937_64& rng, uint in_dim, uint out_dim, uint pp_size, bool norm, size_t table_budget) {
     const double t0 = now_ms();
     std::normal_distribution<double> nd(0.0, 0.02);
     std::vector<int> wi((size_t)in_dim * out_dim);
@@ -442,7 +442,7 @@ static Weight random_weight(std::mt19937_64& rng, uint in_dim, uint out_dim, uin
     prepare_weight_cross(w);
     zk_check(zk_sync(nullptr), "zk_sync");
     const double t4 = now_ms();
-    w.generator.prepare_openings(w.cross_rounds >= 3 ? 3 : 2);        // with three rounds of cross commitments the openings fold three rounds at once
+    w.generator.prepare_openings(w.cross_rounds >= 3 ? 3 : 2, table_budget);        // with three rounds of cross commitments the openings fold three rounds at once
     zk_check(zk_sync(nullptr), "zk_sync");
     const double t5 = now_ms();
     g_setup_times.weights += t1 - t0; g_setup_times.generators += t2 - t1; g_setup_times.commitments += t3 - t2; g_setup_times.cross += t4 - t3;
@@ -463,12 +463,27 @@ LayerWeights make_random_layer_weights(const LayerConfig& c, uint32_t seed, uint
     g_setup_times = LayerSetupTimes();
     std::mt19937_64 rng(seed);
     const uint E = c.embed_dim, Hd = c.hidden_dim;
+    // The fold tables of the nine generator sets share one byte budget (ZKLLM_OPEN_TABLES_GIB, default 64: what the three-round
+    // tables of the 7B shape take is 40 GiB), each set in proportion to its generators; a set whose share is too small for the
+    // richest tables gets the next smaller kind or none -- its openings then walk those rounds, with the same results.
+    double gib = 64.0;
+    if (const char* e = getenv("ZKLLM_OPEN_TABLES_GIB")) gib = atof(e);
+    const double total = gib * 1073741824.0;
+    auto gens_of = [](uint pp) { return (double)(1u << ceilLog2(pp)); };
+    const double all = 2 * gens_of(E) + 5 * gens_of(E << lof) + 2 * gens_of(Hd << lof);
+    auto share = [&](uint pp) { return (size_t)(total * gens_of(pp) / all); };
     // llama-ppgen.py:21-31: 2-D parameters use (HF shape[0] = out_features) << log_off_factor, 1-D their length
     return LayerWeights{
-        random_weight(rng, 1, E, E, true),
-        random_weight(rng, E, E, E << lof, false), random_weight(rng, E, E, E << lof, false), random_weight(rng, E, E, E << lof, false),
-        random_weight(rng, E, E, E << lof, false),
-        random_weight(rng, 1, E, E, true),
-        random_weight(rng, E, Hd, Hd << lof, false), random_weight(rng, E, Hd, Hd << lof, false), random_weight(rng, Hd, E, E << lof, false),
+        random_weight(rng, 1, E, E, true, share(E)),
+        random_weight(rng, E, E, E << lof, false, share(E << lof)), random_weight(rng, E, E, E << lof, false, share(E << lof)), random_weight(rng, E, E, E << lof, false, share(E << lof)),
+        random_weight(rng, E, E, E << lof, false, share(E << lof)),
+        random_weight(rng, 1, E, E, true, share(E)),
+        random_weight(rng, E, Hd, Hd << lof, false, share(Hd << lof)), random_weight(rng, E, Hd, Hd << lof, false, share(Hd << lof)), random_weight(rng, Hd, E, E << lof, false, share(E << lof)),
         make_swiglu_table(c.swiglu_low, c.swiglu_len, c.swiglu_in_scale, c.swiglu_out_scale)};
+}
+size_t layer_opening_table_bytes(const LayerWeights& w) {
+    const Weight* all[9] = {&w.input_norm, &w.q, &w.k, &w.v, &w.o, &w.post_norm, &w.up, &w.gate, &w.down};
+    size_t b = 0;
+    for (const Weight* x : all) b += x->generator.opening_table_bytes();
+    return b;
 }

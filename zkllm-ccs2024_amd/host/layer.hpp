@@ -93,3 +93,5 @@ double layer_recommit_ms(const LayerWeights& w);
 // random-init weights of the configured shape (round(N(0, 0.02) * 2^16), norm weights round(2^16)), generators from the
 // seeded stream sized as llama-ppgen.py does (out_features << log_off_factor, rounded up to a power of two) and commitments
 LayerWeights make_random_layer_weights(const LayerConfig& c, uint32_t seed, uint log_off_factor);
+// device bytes of the fold tables kept with the nine generator sets (Commitment::opening_table_bytes)
+size_t layer_opening_table_bytes(const LayerWeights& w);
