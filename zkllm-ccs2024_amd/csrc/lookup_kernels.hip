@@ -18,6 +18,7 @@
 #include <vector>
 #include "detmath.hpp"
 #include "field.hpp"
+#include "fr29.hpp"
 #include <mutex>
 #include <utility>
 #include <vector>
@@ -665,6 +666,63 @@ k_lookup_round(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ 
         acc[2] = add(acc[2], sub(four, acc_em));
     }
     block_reduce_store<K>(acc, partials);
+}
+
+// ---- the same round with the arithmetic in 29-bit limbs (fr29.hpp) ----------------------------------------------------------
+// sum of up to 2^32 - 1 canonical elements as a plain 288-bit integer (nine words), and its residue
+__device__ __forceinline__ void sum9_add(uint32_t (&acc)[9], const Fr& x) {
+    uint32_t c = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = addc32(acc[i], x.v[i], c);
+    acc[8] += c;
+}
+__device__ __forceinline__ Fr sum9_residue(const uint32_t (&acc)[9]) {
+    Fr lo, hi = big_zero<8>();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) lo.v[i] = acc[i];
+    lo = reduce_once(reduce_once(lo));          // below 2^256 < 3 r
+    hi.v[0] = acc[8];
+    return add(lo, mont_mul(hi, big_r2<8>()));  // hi * 2^256
+}
+// k_lookup_round<false, false> (phase 1, inverses given) for rounds of many pairs: same inputs, same outputs (folded tensors
+// canonical, the five sums as that kernel leaves them), about a quarter fewer vector instructions.  The eq weight e arrives
+// as E 2^256: e a0 and e da come out as E a0 / 32 and E da / 32, the three sums of products are kept unreduced (Wide29),
+// reduced once per lane (another 2^-261) and brought to the factor 2^-256 of the other kernel by one product with 2^271.
+// At most 256 pairs per lane (the unreduced sums hold 2^522): the launch site checks.
+__global__ void __launch_bounds__(TPB) k_lookup_round29(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ nS, const Fr* __restrict__ A, const Fr* __restrict__ S,
+                                                        const Fr* __restrict__ E, const Fr beta, const Fr v_mont, size_t n_out, Fr* __restrict__ nE) {
+    const Fr29 vq = fr29_mul(fr29_repack(v_mont), fr29_2_266());      // v 2^261
+    const Fr29 b29 = fr29_repack(beta);
+    Wide29 w0 = wide29_zero(), w2 = wide29_zero(), wx = wide29_zero();
+    uint32_t sa0[9], sa1[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) sa0[i] = sa1[i] = 0;
+    uint32_t it = 0;
+    for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
+        const Fr e = E[t];
+        if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table: the top variable summed out
+        const Fr a0w = A[t], a1w = A[t + n_out], s0w = S[t], s1w = S[t + n_out];
+        sum9_add(sa0, a0w);
+        sum9_add(sa1, a1w);
+        const Fr29 e29 = fr29_repack(e), a0 = fr29_repack(a0w), s0r = fr29_repack(s0w);
+        const Fr29 da = fr29_sub_plus_r(fr29_repack(a1w), a0), ds = fr29_sub_plus_r(fr29_repack(s1w), s0r);      // + r: non-negative, the same residues
+        const Fr29 s0 = fr29_add(s0r, b29);
+        const Fr29 ea0 = fr29_mul(e29, a0), eda = fr29_mul(e29, da);
+        wide29_mac(w0, ea0, s0);
+        wide29_mac(w2, eda, ds);
+        wide29_mac(wx, fr29_add(ea0, eda), fr29_add(s0, ds));
+        if ((++it & 3u) == 0u) { wide29_carry(w0); wide29_carry(w2); wide29_carry(wx); }
+        nA[t] = fr29_canon_pack(fr29_add(a0, fr29_mul(vq, da)));
+        nS[t] = fr29_canon_pack(fr29_add(s0r, fr29_mul(vq, ds)));
+    }
+    Fr acc[5];
+    const Fr29 fix = fr29_2_271();
+    acc[0] = fr29_canon_pack(fr29_mul(wide29_redc(w0), fix));
+    acc[2] = fr29_canon_pack(fr29_mul(wide29_redc(w2), fix));
+    acc[1] = sub(sub(fr29_canon_pack(fr29_mul(wide29_redc(wx), fix)), acc[0]), acc[2]);
+    acc[3] = sum9_residue(sa0);
+    acc[4] = sub(sum9_residue(sa1), acc[3]);
+    block_reduce_store<5>(acc, partials);
 }
 
 // ---- Hadamard-product sumcheck with adjacent-pair folding (Fr_hp_sc, proof.cu:66-98) -------------------------------------
@@ -1783,6 +1841,8 @@ static const int g_round_timer_hook = (at_shutdown([] {
     std::lock_guard<std::mutex> lk(g_eq_mu);
     g_eq_latest.reset();          // the eq table kept for the next job with the same challenges goes back to the allocator
 }), 0);
+// ZKLLM_FR_LIMBS=32 keeps the round kernels on the 32-bit-limb arithmetic throughout (to compare; the results are the same)
+static bool limbs29() { static const bool on = [] { const char* e = getenv("ZKLLM_FR_LIMBS"); return !(e && atoi(e) == 32); }(); return on; }
 // all rounds of the lookup sumcheck; sums land in job.sums
 // A == nullptr with a hint source: 1 / (S + beta) has not been written anywhere; a large first round computes it on
 // the fly, anything else writes it out first.
@@ -1884,6 +1944,8 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
                 g_round_timer.bytes += (double)half * (q + 32.0 + 64.0 + (nE ? 16.0 : 0.0));
             }
         }
+        else if (limbs29() && half <= (size_t)256 * nb * TPB)       // 29-bit limbs inside the kernel; its unreduced sums hold 256 pairs per lane
+            hipLaunchKernelGGL(k_lookup_round29, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, cA, cS, cE, b, vm, half, nE);
         else
             hipLaunchKernelGGL((k_lookup_round<false, false>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, cA, cS, (const Fr*)nullptr,
                                (const Fr*)nullptr, (const Fr*)nullptr, cE, b, vm, half, nE, HintSrc());
