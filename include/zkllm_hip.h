@@ -379,6 +379,9 @@ int zk_prof_gemm_read(double* total_ms, unsigned long long* launches, double* ma
 /* the same for the first round of the hinted lookup sumchecks (k_lookup_round<false, true>); bytes: their algorithmic traffic */
 int zk_prof_lookup_begin(void);
 int zk_prof_lookup_read(double* total_ms, unsigned long long* launches, unsigned long long* pairs, double* bytes);
+/* and for the large rounds behind the first of every lookup sumcheck (phase 1, one lane per pair: k_lookup_round29), timed since
+ * the same zk_prof_lookup_begin; bytes: 240 per pair (inverses and queries of both halves, eq weight, two folded values, next eq table) */
+int zk_prof_lookup_later_read(double* total_ms, unsigned long long* launches, unsigned long long* pairs, double* bytes);
 
 #ifdef __cplusplus
 }

@@ -320,4 +320,37 @@ FQ29_POINT_FN J29 j29_add_mixed(const J29& a, const A29& b) {
     return r;
 }
 
+// a + b, both Jacobian (add-2007-bl, bls12-381.cu:1431-1464), with the flag and the equal-abscissa cases as above
+FQ29_POINT_FN J29 j29_add(const J29& a, const J29& b) {
+    const Fq29 z1z1 = fq29_sqr(a.z), z2z2 = fq29_sqr(b.z);
+    const Fq29 u1 = fq29_mul(a.x, z2z2), u2 = fq29_mul(b.x, z1z1);
+    Fq29 s1 = fq29_mul(fq29_mul(a.y, b.z), z2z2);
+    const Fq29 s2 = fq29_mul(fq29_mul(b.y, a.z), z1z1);
+    const Fq29 h = fq29_sub(u2, u1), rr0 = fq29_sub(s2, s1);
+    const Fq29 i = fq29_sqr(fq29_dbl(h));
+    const Fq29 j = fq29_mul(h, i);
+    const Fq29 rr = fq29_dbl(rr0);
+    const Fq29 v = fq29_mul(u1, i);
+    J29 r;
+    r.inf = 0u;
+    r.x = fq29_sub(fq29_sub(fq29_sqr(rr), j), fq29_dbl(v));
+    s1 = fq29_dbl(fq29_mul(s1, j));
+    r.y = fq29_sub(fq29_mul(fq29_sub(v, r.x), rr), s1);
+    r.z = fq29_mul(fq29_sub(fq29_sub(fq29_sqr(fq29_add(a.z, b.z)), z1z1), z2z2), h);
+    if (a.inf) r = b;
+    else if (b.inf) r = a;
+    else if (fq29_is_zero_mod_p(h)) {
+        if (fq29_is_zero_mod_p(rr0)) r = j29_double(a);
+        else r = j29_infinity();
+    }
+    return r;
+}
+ZK_HD J29 j29_from_jac(const G1Jac& p) {
+    if (is_zero(p.z)) return j29_infinity();
+    J29 r;
+    r.inf = 0u;
+    r.x = fq29_from_fp(p.x); r.y = fq29_from_fp(p.y); r.z = fq29_from_fp(p.z);
+    return r;
+}
+
 }  // namespace zk

@@ -554,20 +554,24 @@ __global__ void __launch_bounds__(MT) k_msm_point(G1Jac* __restrict__ wsum, G1Ja
     const uint32_t t = threadIdx.x, z = blockIdx.x;
     if (list) { buckets = list[z].buckets; nseg = list[z].nseg; }
     const size_t zb = list ? 0 : z;
-    G1Jac r = g1_infinity();
+    // The walk is one lane's chain of 248 doublings: it runs in 29-bit limbs (two thirds of the instructions of the 32-bit
+    // formulas, and the point stays in registers instead of travelling through private memory at every call).
+    J29 r = j29_infinity();
     for (int w = MW - 1; w >= 0; --w) {
         if (w != MW - 1)
-            for (int k = 0; k < 8; ++k) r = g1_double(r);
+            for (int k = 0; k < 8; ++k) r = j29_double(r);
         const G1Jac* b = buckets + (zb * MW + (uint32_t)w) * nseg * MT;
-        G1Jac acc = b[t];
-        for (uint32_t sg = 1; sg < nseg; ++sg) acc = g1_add(acc, b[(size_t)sg * MT + t]);
-        r = g1_add(r, acc);
+        for (uint32_t sg = 0; sg < nseg; ++sg) {
+            const G1Jac pt = b[(size_t)sg * MT + t];
+            if (!is_zero(pt.z)) r = j29_add(r, j29_from_jac(pt));
+        }
     }
-    G1Jac q = g1_infinity();
+    J29 q29 = j29_infinity();
     for (int bit = 7; bit >= 0; --bit) {
-        q = g1_double(q);
-        if (((t + 1) >> bit) & 1u) q = g1_add(q, r);
+        q29 = j29_double(q29);
+        if (((t + 1) >> bit) & 1u) q29 = j29_add(q29, r);
     }
+    const G1Jac q = j29_to_jac(q29);
     const G1Jac tot = msm_block_sum(pool, q, t);
     if (wsum || list) {
         G1Jac* __restrict__ W = list ? list[z].W : wsum + (size_t)(z / n_per) * item_stride + (size_t)(z % n_per) * MW;
@@ -637,10 +641,42 @@ static __device__ __attribute__((noinline)) G1Jac g1_mul_glv_lane(const G1Jac& P
     }
     return out;
 }
+// the same walk in 29-bit limbs.  P stays in registers; beta x (the abscissa of phi(P)) and P + phi(P) wait in LDS, word-
+// interleaved over the workgroup's GT lanes (tab: 57 x GT words), so the walk fits the register file without spilling.
+static __device__ J29 j29_mul_glv_lane(const J29& P, const GlvK& k, int32_t (*tab)[GT]) {
+    const uint32_t t = threadIdx.x;
+    {
+        J29 Q = P;
+        Q.x = fq29_mul(P.x, fq29_from_fp(glv_beta()));
+        const J29 PQ = j29_add(P, Q);
+#pragma unroll
+        for (int l = 0; l < 14; ++l) { tab[l][t] = Q.x.l[l]; tab[14 + l][t] = PQ.x.l[l]; tab[28 + l][t] = PQ.y.l[l]; tab[42 + l][t] = PQ.z.l[l]; }
+        tab[56][t] = (int32_t)PQ.inf;
+    }
+    J29 out = j29_infinity();
+    for (int i = 127; i >= 0; --i) {
+        out = j29_double(out);
+        const uint32_t b = ((k.k1[i >> 5] >> (i & 31)) & 1u) | (((k.k2[i >> 5] >> (i & 31)) & 1u) << 1);
+        if (b) {
+            J29 a = P;
+            if (b == 2) {
+#pragma unroll
+                for (int l = 0; l < 14; ++l) a.x.l[l] = tab[l][t];
+            } else if (b == 3) {
+#pragma unroll
+                for (int l = 0; l < 14; ++l) { a.x.l[l] = tab[14 + l][t]; a.y.l[l] = tab[28 + l][t]; a.z.l[l] = tab[42 + l][t]; }
+                a.inf = (uint32_t)tab[56][t];
+            }
+            out = j29_add(out, a);
+        }
+    }
+    return out;
+}
 // grid: halving_rounds - 1 workgroups; workgroup x computes T of round x + 1 into pts[3 * (x + 1)].  Needs T_0 and all T0, T1.
 // U: the openings' challenges in Montgomery form, opening y's at U + y * ustride
 __global__ void __launch_bounds__(GT) k_open_chain(G1Jac* __restrict__ pts0, const Fr* __restrict__ U, uint32_t halving_rounds, uint32_t npts, uint32_t ustride) {
     __shared__ uint32_t pool[36 * GT];
+    __shared__ int32_t walk_tab[57][GT];
     G1Jac* __restrict__ pts = pts0 + (size_t)blockIdx.y * npts;
     const Fr* __restrict__ usu = U + (size_t)blockIdx.y * ustride;
     const uint32_t r = blockIdx.x + 1, t = threadIdx.x;
@@ -657,7 +693,7 @@ __global__ void __launch_bounds__(GT) k_open_chain(G1Jac* __restrict__ pts0, con
                 c = mont_mul(c, mont_mul(f, f));
             }
             const G1Jac P = pts[i == 0 ? 0u : 3 * k + 1 + s1];
-            if (!is_zero(P.z)) acc = g1_add(acc, g1_mul_glv_lane(P, glv_split_device(from_mont(c))));
+            if (!is_zero(P.z)) acc = g1_add(acc, j29_to_jac(j29_mul_glv_lane(j29_from_jac(P), glv_split_device(from_mont(c)), walk_tab)));
         }
     }
     // sum over the lanes

@@ -1831,12 +1831,19 @@ struct RoundTimer {
     double bytes = 0;          // algorithmic traffic of the timed launches
 };
 static RoundTimer g_round_timer;
+static RoundTimer g_later_timer;          // the same for the large phase-1 rounds behind the first (k_lookup_round29 / k_lookup_round<false, false>)
 static const int g_round_timer_hook = (at_shutdown([] {
     {
         std::lock_guard<std::mutex> lk(g_round_timer.mu);
         for (auto& e : g_round_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
         g_round_timer.ev.clear();
         g_round_timer.on = false;
+    }
+    {
+        std::lock_guard<std::mutex> lk(g_later_timer.mu);
+        for (auto& e : g_later_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
+        g_later_timer.ev.clear();
+        g_later_timer.on = false;
     }
     std::lock_guard<std::mutex> lk(g_eq_mu);
     g_eq_latest.reset();          // the eq table kept for the next job with the same challenges goes back to the allocator
@@ -1944,11 +1951,27 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
                 g_round_timer.bytes += (double)half * (q + 32.0 + 64.0 + (nE ? 16.0 : 0.0));
             }
         }
-        else if (limbs29() && half <= (size_t)256 * nb * TPB)       // 29-bit limbs inside the kernel; its unreduced sums hold 256 pairs per lane
-            hipLaunchKernelGGL(k_lookup_round29, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, cA, cS, cE, b, vm, half, nE);
-        else
-            hipLaunchKernelGGL((k_lookup_round<false, false>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, cA, cS, (const Fr*)nullptr,
-                               (const Fr*)nullptr, (const Fr*)nullptr, cE, b, vm, half, nE, HintSrc());
+        else {
+            hipEvent_t t0 = nullptr, t1 = nullptr;
+            if (g_later_timer.on) {
+                ZK_HIP(hipEventCreate(&t0));
+                ZK_HIP(hipEventCreate(&t1));
+                ZK_HIP(hipEventRecord(t0, st));
+            }
+            if (limbs29() && half <= (size_t)256 * nb * TPB)       // 29-bit limbs inside the kernel; its unreduced sums hold 256 pairs per lane
+                hipLaunchKernelGGL(k_lookup_round29, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, cA, cS, cE, b, vm, half, nE);
+            else
+                hipLaunchKernelGGL((k_lookup_round<false, false>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, cA, cS, (const Fr*)nullptr,
+                                   (const Fr*)nullptr, (const Fr*)nullptr, cE, b, vm, half, nE, HintSrc());
+            if (g_later_timer.on) {
+                ZK_HIP(hipEventRecord(t1, st));
+                std::lock_guard<std::mutex> lk(g_later_timer.mu);
+                g_later_timer.ev.emplace_back(t0, t1);
+                g_later_timer.pairs += half;
+                // per pair: the inverses and queries of both halves (128 B), the eq weight (32 B), two folded values out (64 B), the next eq table (16 B)
+                g_later_timer.bytes += (double)half * (128.0 + 32.0 + 64.0 + (nE ? 16.0 : 0.0));
+            }
+        }
         hipLaunchKernelGGL(k_finish, dim3(phase2 ? 11 : 5), dim3(TPB), 0, st, sums.as<Fr>() + (size_t)r * 11, part.as<Fr>(), nb);
         ZK_LAUNCH_CHECK();
         cA = w; cS = w + half;
@@ -2280,32 +2303,43 @@ int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host) {
 }
 // Measurement: time every launch of the hinted first round (k_lookup_round<false, true>) between begin and read, with events
 // on the launch stream.  bytes: the algorithmic traffic of those launches.
-int zk_prof_lookup_begin(void) {
-    std::lock_guard<std::mutex> lk(g_round_timer.mu);
-    for (auto& e : g_round_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
-    g_round_timer.ev.clear();
-    g_round_timer.pairs = 0;
-    g_round_timer.bytes = 0;
-    g_round_timer.on = true;
-    return 0;
+static void round_timer_begin(RoundTimer& T) {
+    std::lock_guard<std::mutex> lk(T.mu);
+    for (auto& e : T.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
+    T.ev.clear();
+    T.pairs = 0;
+    T.bytes = 0;
+    T.on = true;
 }
-int zk_prof_lookup_read(double* total_ms, unsigned long long* launches, unsigned long long* pairs, double* bytes) {
-    std::lock_guard<std::mutex> lk(g_round_timer.mu);
-    g_round_timer.on = false;
+static int round_timer_read(RoundTimer& T, double* total_ms, unsigned long long* launches, unsigned long long* pairs, double* bytes) {
+    std::lock_guard<std::mutex> lk(T.mu);
+    T.on = false;
     double tot = 0;
-    for (auto& e : g_round_timer.ev) {
+    for (auto& e : T.ev) {
         ZK_HIP(hipEventSynchronize(e.second));
         float ms = 0;
         ZK_HIP(hipEventElapsedTime(&ms, e.first, e.second));
         tot += ms;
     }
     *total_ms = tot;
-    *launches = g_round_timer.ev.size();
-    *pairs = g_round_timer.pairs;
-    *bytes = g_round_timer.bytes;
-    for (auto& e : g_round_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
-    g_round_timer.ev.clear();
+    *launches = T.ev.size();
+    *pairs = T.pairs;
+    *bytes = T.bytes;
+    for (auto& e : T.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
+    T.ev.clear();
     return 0;
+}
+int zk_prof_lookup_begin(void) {
+    round_timer_begin(g_round_timer);
+    round_timer_begin(g_later_timer);
+    return 0;
+}
+int zk_prof_lookup_read(double* total_ms, unsigned long long* launches, unsigned long long* pairs, double* bytes) {
+    return round_timer_read(g_round_timer, total_ms, launches, pairs, bytes);
+}
+// the large phase-1 rounds behind the first (one lane per pair: k_lookup_round29 or k_lookup_round<false, false>) since zk_prof_lookup_begin
+int zk_prof_lookup_later_read(double* total_ms, unsigned long long* launches, unsigned long long* pairs, double* bytes) {
+    return round_timer_read(g_later_timer, total_ms, launches, pairs, bytes);
 }
 // The whole multi-Hadamard sumcheck (proof.cu:191-241) queued without a host round trip.  Xs: K tensors of N elements
 // (N a power of two), E: N/2 elements (Montgomery form), v: log2(N) fold challenges in round order.  coefs_host:
