@@ -36,6 +36,10 @@ VALU_PEAK_TOPS = 256 * 4 * 16 * 2.4e9 / 1e12
 # that size; `traffic` of the in-layer entry, whose launches are of every size, is left null and the algorithmic figure given.
 FOLD_TRAFFIC_BYTES_PER_PAIR_AT_262144 = 763.5      # (53674 KiB x 2.000 fetched + 88108 KiB written) / 262144 pairs, profiles/k_open_fold29_pmc_traffic.txt
 FOLD_ALGO_BYTES_PER_PAIR = 2 * 112 + 112 + 3 * 32      # two points in, one out (affine, 29-bit limbs: 112 B), two scalars in, one out
+# the same for the table-driven folds, from profiles/fr_mul_fold_msm_pmc.txt (each kernel alone): k_open_fold_comb<1> at 262144 pairs
+# (821668 KiB x 2 fetched + 146433 KiB written) and k_open_fold_jump at 65536 results = 7 x 65536 pairs (862752 KiB x 2 + 38100 KiB)
+COMB_TRAFFIC_BYTES_PER_PAIR = (821668 * 2 + 146433) * 1024 / 262144
+JUMP_TRAFFIC_BYTES_PER_PAIR = (862752 * 2 + 38100) * 1024 / (7 * 65536)
 MAD_PER_FP_MUL = 300                                   # 2 * 12^2 + 12 limb products of a 381-bit Montgomery product
 MAD_PER_FR_MUL = 136                                   # 2 * 8^2 + 8
 
@@ -341,6 +345,13 @@ def main():
         pv.sync()
         wall = time.perf_counter() - t0
         fold_ms, fold_launches, fold_mults, fold_pairs = read_fold_timer()
+        m_ms, m_mults = (ctypes.c_double * 3)(), (ctypes.c_double * 3)()
+        m_launches, m_pairs = (ctypes.c_ulonglong * 3)(), (ctypes.c_ulonglong * 3)()
+        hip.check(lib.zk_prof_fold_methods(m_ms, m_launches, m_pairs, m_mults))
+        fold_methods = {name: {"launches": int(m_launches[i]), "pairs": int(m_pairs[i]), "fp_mults": m_mults[i], "ms": m_ms[i],
+                               "fp_mults_per_pair": m_mults[i] / max(1, m_pairs[i])}
+                        for i, name in enumerate(("walk_k_open_fold29", "comb_k_open_fold_comb", "three_rounds_k_open_fold_jump"))}
+        fold_traffic = (m_pairs[0] * FOLD_TRAFFIC_BYTES_PER_PAIR_AT_262144 + m_pairs[1] * COMB_TRAFFIC_BYTES_PER_PAIR + m_pairs[2] * JUMP_TRAFFIC_BYTES_PER_PAIR)
         lk_ms, lk_launches, lk_pairs, lk_bytes = read_lookup_timer()
         lr_ms, lr_launches, lr_pairs, lr_bytes = read_lookup_timer(later=True)
         # the same layer without its nine openings (the G1 part of verifyWeightClaim switched off), and the nine commitments alone
@@ -455,7 +466,11 @@ def main():
     out["roofline"] = {"kernel": "k_open_fold29, k_open_fold_comb<1> / <2> (first two rounds over prepared generators) and k_open_fold_jump (first three rounds at once, openings with cross commitments): g' = g1 + [u](g0 - g1) per generator pair, 128-bit split scalars, "
                                  "one launch per round for all openings of a size)",
                        "bound": "valu-int", "achieved": fold_tops, "peak": VALU_PEAK_TOPS, "unit": "T MAD32/s", "frac": fold_tops / VALU_PEAK_TOPS,
-                       "traffic": None, "algorithmic_bytes_per_launch": FOLD_ALGO_BYTES_PER_PAIR * fold_pairs / max(1, fold_launches),
+                       "traffic": fold_traffic / max(1, fold_launches), "algorithmic_bytes_per_launch": FOLD_ALGO_BYTES_PER_PAIR * fold_pairs / max(1, fold_launches),
+                       "traffic_note": "bytes per launch from the counters of each kernel ALONE (FETCH_SIZE x 2.000 + WRITE_SIZE per pair: walk 764 B, comb 6991 B, "
+                                       "three-round fold 3937 B -- the table-driven folds read their fixed-base table entries, 112 B each) times the pairs of the "
+                                       "timed launches; counters of a kernel inside the layer cannot be told apart from its neighbours'",
+                       "by_method": fold_methods,
                        "launches": int(fold_launches), "avg_launch_ms": fold_ms / max(1, fold_launches),
                        "total_ms_in_timed_region": fold_ms, "pairs": int(fold_pairs), "fp_mul_per_s": fold_mults / (fold_ms * 1e-3) if fold_ms > 0 else 0.0,
                        "note": "algorithmic work = Fp multiplications of the point formulas x 300 MAD32 (12-limb schoolbook product and reduction; the kernel "

@@ -372,6 +372,9 @@ int zk_bench_copy(void* dst, const void* src, size_t bytes, void* stream);
  * perform by the point formulas' count; pairs: generator pairs folded */
 int zk_prof_fold_begin(void);
 int zk_prof_fold_read(double* total_ms, unsigned long long* launches, double* fp_mults, unsigned long long* pairs);
+/* what the last zk_prof_fold_read counted, split by fold method (three values each: the walk k_open_fold29, the combs
+ * k_open_fold_comb<1> / <2>, the three-round fold k_open_fold_jump) */
+int zk_prof_fold_methods(double* ms3, unsigned long long* launches3, unsigned long long* pairs3, double* fp_mults3);
 /* the same for the int8-plane GEMM of the small-integer matrix products (k_gemm_i8_planes, behind zk_fr_matmul);
  * macs: int8 multiply-accumulates of those launches (rows x contraction x columns x plane pairs) */
 int zk_prof_gemm_begin(void);

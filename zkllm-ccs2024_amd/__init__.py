@@ -27,9 +27,9 @@ def _load(path):
 
 
 def _want_hw_queues():
-    """The library keeps up to nine streams busy (the caller's, six for openings, two for sumcheck jobs).  HIP maps
+    """The library keeps up to seven streams busy (the caller's, four for openings, two for sumcheck jobs).  HIP maps
     streams onto GPU_MAX_HW_QUEUES hardware queues (4 unless set) and streams that share a queue run one after the
-    other, so ask for at least sixteen (measured: the decoder layer takes 0.458 s with 8 and 0.454 s with 16).  The HIP runtime reads the variable when it is loaded: this must run before that.
+    other, so ask for at least sixteen (measured when this was added: the decoder layer took 7 % less time with 8 queues than with 4 and another 1 % less with 16).  The HIP runtime reads the variable when it is loaded: this must run before that.
     ZKLLM_HW_QUEUES=0 leaves the variable alone, ZKLLM_HW_QUEUES=N sets it to N."""
     want = os.environ.get("ZKLLM_HW_QUEUES", "")
     if want == "0":

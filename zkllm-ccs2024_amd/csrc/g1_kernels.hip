@@ -1300,6 +1300,10 @@ struct FoldTimer {
     std::vector<std::pair<hipEvent_t, hipEvent_t>> ev;
     double fp_mults = 0;      // Fp multiplications the timed launches perform by the formulas' count
     unsigned long long pairs = 0;
+    // the same per method: 0 the walk (k_open_fold29), 1 the one- and two-table combs (k_open_fold_comb), 2 the three-round fold (k_open_fold_jump)
+    std::vector<int> method;
+    double m_mults[3] = {0, 0, 0};
+    unsigned long long m_pairs[3] = {0, 0, 0};
 };
 static FoldTimer g_fold_timer;
 static const int g_fold_timer_hook = (at_shutdown([] {
@@ -1552,6 +1556,10 @@ static int open_round_launch(const RoundItem* items, int count, size_t old_size,
         g_fold_timer.ev.emplace_back(t0, t1);
         g_fold_timer.fp_mults += fp_mults;
         g_fold_timer.pairs += new_size * (size_t)count;
+        const int mth = (use_comb || use_comb2) ? 1 : 0;
+        g_fold_timer.method.push_back(mth);
+        g_fold_timer.m_mults[mth] += fp_mults;
+        g_fold_timer.m_pairs[mth] += new_size * (size_t)count;
     }
     hipLaunchKernelGGL(k_open_fold_special, dim3(16, count), dim3(GT), 0, st, sb, old_size);
     ZK_LAUNCH_CHECK();
@@ -1992,6 +2000,9 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
                 g_fold_timer.ev.emplace_back(t0, t1);
                 g_fold_timer.fp_mults += fp_mults;
                 g_fold_timer.pairs += ns * (size_t)count * (JUMP_SPAN - 1);       // pairs the three rounds fold: 4 + 2 + 1 per result
+                g_fold_timer.method.push_back(2);
+                g_fold_timer.m_mults[2] += fp_mults;
+                g_fold_timer.m_pairs[2] += ns * (size_t)count * (JUMP_SPAN - 1);
             }
             for (int i = 0; i < count; ++i) { cs[i] = s2.as<Fr>() + ns * i; cg[i] = g2.as<A29>() + ns * i; }
             size = ns;
@@ -2340,11 +2351,16 @@ int zk_g1_open_end(void* handle, uint32_t* proof_host, uint32_t* final_scalar_ho
 }
 
 // Measurement: time every launch of the opening's fold kernel between begin and read with events on the launch stream.
+static double g_fold_method_ms[3] = {0, 0, 0};
+static unsigned long long g_fold_method_launches[3] = {0, 0, 0}, g_fold_method_pairs[3] = {0, 0, 0};
+static double g_fold_method_mults[3] = {0, 0, 0};
 int zk_prof_fold_begin(void) {
     for (auto& e : g_fold_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
     g_fold_timer.ev.clear();
+    g_fold_timer.method.clear();
     g_fold_timer.fp_mults = 0;
     g_fold_timer.pairs = 0;
+    for (int m = 0; m < 3; ++m) { g_fold_timer.m_mults[m] = 0; g_fold_timer.m_pairs[m] = 0; }
     g_fold_timer.on = true;
     return 0;
 }
@@ -2352,18 +2368,30 @@ int zk_prof_fold_begin(void) {
 int zk_prof_fold_read(double* total_ms, unsigned long long* launches, double* fp_mults, unsigned long long* pairs) {
     g_fold_timer.on = false;
     double tot = 0;
-    for (auto& e : g_fold_timer.ev) {
+    for (int m = 0; m < 3; ++m) { g_fold_method_ms[m] = 0; g_fold_method_launches[m] = 0; }
+    for (size_t i = 0; i < g_fold_timer.ev.size(); ++i) {
+        auto& e = g_fold_timer.ev[i];
         ZK_HIP(hipEventSynchronize(e.second));
         float ms = 0;
         ZK_HIP(hipEventElapsedTime(&ms, e.first, e.second));
         tot += ms;
+        const int m = i < g_fold_timer.method.size() ? g_fold_timer.method[i] : 0;
+        g_fold_method_ms[m] += ms;
+        g_fold_method_launches[m] += 1;
     }
+    for (int m = 0; m < 3; ++m) { g_fold_method_mults[m] = g_fold_timer.m_mults[m]; g_fold_method_pairs[m] = g_fold_timer.m_pairs[m]; }
     *total_ms = tot;
     *launches = g_fold_timer.ev.size();
     *fp_mults = g_fold_timer.fp_mults;
     *pairs = g_fold_timer.pairs;
     for (auto& e : g_fold_timer.ev) { (void)hipEventDestroy(e.first); (void)hipEventDestroy(e.second); }
     g_fold_timer.ev.clear();
+    g_fold_timer.method.clear();
+    return 0;
+}
+// what the last zk_prof_fold_read counted, by method (0 walk, 1 comb, 2 three-round fold): ms, launches, pairs, Fp multiplications
+int zk_prof_fold_methods(double* ms3, unsigned long long* launches3, unsigned long long* pairs3, double* fp_mults3) {
+    for (int m = 0; m < 3; ++m) { ms3[m] = g_fold_method_ms[m]; launches3[m] = g_fold_method_launches[m]; pairs3[m] = g_fold_method_pairs[m]; fp_mults3[m] = g_fold_method_mults[m]; }
     return 0;
 }
 
