@@ -148,8 +148,9 @@ def main():
     ap.add_argument("--skip-extras", action="store_true", help="only the layer timing (used for profiling runs)")
     ap.add_argument("--at-claim", action="store_true",
                     help="the timed layers start every weight opening at its claim (what layer_openings_at_claim_s reports); for profiling runs")
-    ap.add_argument("--drivers", action="store_true",
-                    help="also run the per-block executables over .bin files at the 7B shape (child processes) and report their wall times")
+    ap.add_argument("--drivers", action="store_true", help="(default) also run the per-block executables over .bin files at the 7B shape")
+    ap.add_argument("--no-drivers", action="store_true",
+                    help="skip the leg that runs the per-block executables over .bin files at the 7B shape (child processes; about 8 s and 1.3 GB under TMPDIR)")
     ap.add_argument("--drivers-only", action="store_true", help="only the executables' chain (no in-process layer)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: three launches of the opening's fold kernel at 262144 pairs, one hinted lookup "
@@ -428,8 +429,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"C5: LLaMa-2-7B-shape decoder layer proof, seq {seq}, hidden 4096, 32 heads x 128, FFN 11008, "
                                "random-init fixed-point weights (scale 2^16), generators of size out_features<<5, all nine weight openings included "
-                               "(their points are read ahead from the seeded challenge stream, so all nine run from the start of the layer, batched by "
-                               "generator size); attention proved "
+                               "(value: their points are read ahead from the seeded challenge stream, so all nine run from the start of the layer, batched by "
+                               "generator size; layer_openings_at_claim_s: the same layer with every opening started at its claim, the like-for-like order of work); attention proved "
                                + (f"{args.head_group} heads at a time as head-major stacks (zkAttnStacked)" if args.head_group else "head by head"),
                    "device_pool_gib": round(peak_gib, 1),
                    "memory_gib": {"peak_during_layer_runs": round(peak_gib, 1), "fold_tables_of_the_generators": round(tables_gib, 1),
@@ -780,7 +781,7 @@ def main():
                                "parts_s": {k_: round(v_, 1) for k_, v_ in parts_cpu.items()},
                                "config1_zkfc_toy_s": c1_s, "config4_lookup_s": c4_s, "config2_proof_s": c2_prove_s, "softmax_hadamard_one_head_s": hadamard_head_s,
                                "fr_mul_per_s_all_cores": mm_rate}
-    if args.drivers:
+    if not args.no_drivers:
         del pv, hip
         lib.zk_shutdown()          # the child processes need the device memory this process held in its pool
         try:
