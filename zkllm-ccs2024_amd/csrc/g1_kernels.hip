@@ -642,8 +642,8 @@ static __device__ __attribute__((noinline)) G1Jac g1_mul_glv_lane(const G1Jac& P
     return out;
 }
 // the same walk in 29-bit limbs.  P stays in registers; beta x (the abscissa of phi(P)) and P + phi(P) wait in LDS, word-
-// interleaved over the workgroup's GT lanes (tab: 57 x GT words), so the walk fits the register file without spilling.
-static __device__ J29 j29_mul_glv_lane(const J29& P, const GlvK& k, int32_t (*tab)[GT]) {
+// interleaved over the workgroup's NT lanes (tab: 57 x NT words), so the walk fits the register file without spilling.
+template <int NT> static __device__ J29 j29_mul_glv_lane(const J29& P, const GlvK& k, int32_t (*tab)[NT]) {
     const uint32_t t = threadIdx.x;
     {
         J29 Q = P;
@@ -693,7 +693,7 @@ __global__ void __launch_bounds__(GT) k_open_chain(G1Jac* __restrict__ pts0, con
                 c = mont_mul(c, mont_mul(f, f));
             }
             const G1Jac P = pts[i == 0 ? 0u : 3 * k + 1 + s1];
-            if (!is_zero(P.z)) acc = g1_add(acc, j29_to_jac(j29_mul_glv_lane(j29_from_jac(P), glv_split_device(from_mont(c)), walk_tab)));
+            if (!is_zero(P.z)) acc = g1_add(acc, j29_to_jac(j29_mul_glv_lane<GT>(j29_from_jac(P), glv_split_device(from_mont(c)), walk_tab)));
         }
     }
     // sum over the lanes
@@ -751,6 +751,7 @@ __device__ __forceinline__ void cross_target(uint32_t t, uint32_t& q, uint32_t& 
 // grid (chunks, targets, openings): chunk c of a target sums its terms [c MT, (c+1) MT) into part[(t chunks + c)]
 __global__ void __launch_bounds__(MT) k_open_cross_part(const CrossBatch cb) {
     __shared__ uint32_t pool[36 * MT];
+    __shared__ int32_t walk_tab[57][MT];
     const CrossItem& it = cb.it[blockIdx.z];
     const uint32_t t = blockIdx.y, c = blockIdx.x, lane = threadIdx.x;
     uint32_t q, p0, npat, slot;
@@ -770,7 +771,7 @@ __global__ void __launch_bounds__(MT) k_open_cross_part(const CrossBatch cb) {
             }
         }
         const G1Jac P = it.pts[(size_t)(p0 + pl) * nrows + row];
-        if (!is_zero(P.z) && !is_zero(coef)) acc = g1_mul_glv_lane(P, glv_split_device(from_mont(coef)));
+        if (!is_zero(P.z) && !is_zero(coef)) acc = j29_to_jac(j29_mul_glv_lane<MT>(j29_from_jac(P), glv_split_device(from_mont(coef)), walk_tab));
     }
     const G1Jac tot = msm_block_sum(pool, acc, lane);
     if (lane == 0) it.part[(size_t)t * gridDim.x + c] = tot;
