@@ -42,6 +42,39 @@ def test_tiny_layer_transcript(pv, open_weights, seed, head_group):
     assert times[6] > 0
 
 
+@pytest.mark.parametrize("open_weights,seed", [(True, 13), (False, 14)])
+def test_tiny_layer_blocks_overlapped_and_one_after_the_other(pv, open_weights, seed):
+    """With all heads as one stack every block of the layer runs in three steps, and the layer queues a block's forward pass
+    and proof jobs before it collects the proofs of the block before it (zkp_layer_set_blocks_overlap, on by default).  Both
+    orders of work give the oracle's output and transcript."""
+    orc = load_oracle()
+    cu, cf = layercfg.tiny(open_weights=open_weights, head_group=2)
+    ws = layercfg.tiny_weights(seed, cu)
+    S, E = int(cu[0]), int(cu[1])
+    X = np.round(np.random.default_rng(seed + 10).normal(0, 1, (S, E)) * 256).astype(np.int32)
+    exp = np.zeros((S * E, 8), np.uint32)
+    orc.orc_seed(seed)
+    orc.orc_transcript_clear()
+    orc_check(orc.orc_layer(cu, cf, *ws, 1, X, exp, None))
+    exp_t = orc_transcript(orc)
+    assert pv.lib.zkp_layer_blocks_overlap() == 1
+    try:
+        for overlap in (0, 1):
+            pv.lib.zkp_layer_set_blocks_overlap(overlap)
+            pv.seed(seed)
+            layer = pv.layer_create(cu, cf, ws, 1)
+            pv.transcript_begin()
+            out, times = pv.layer_run(layer, pv.from_i32(X))
+            pv.lib.zkp_transcript_end()
+            got_t = pv.transcript()
+            pv.layer_free(layer)
+            assert (out.host() == exp).all(), overlap
+            assert got_t.shape == exp_t.shape and (got_t == exp_t).all(), overlap
+            assert min(times[:6]) > 0
+    finally:
+        pv.lib.zkp_layer_set_blocks_overlap(1)
+
+
 def test_layer_run_again_starts_its_openings_ahead_and_proves_the_same(pv):
     """The first run over a set of weights learns where the nine opening points sit in the challenge stream; a second run
     starts every opening when the layer starts (batched by generator size) and must deliver the transcript of the first,

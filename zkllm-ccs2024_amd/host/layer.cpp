@@ -4,6 +4,8 @@
 
 #include <chrono>
 #include <cmath>
+#include <functional>
+#include <optional>
 #include <random>
 
 #include "../../include/zkllm_hip.h"
@@ -83,54 +85,91 @@ void layer_config_from_env(LayerConfig& c) {
 }
 
 // rmsnorm.cu:26-49
-FrTensor rmsnorm_block(const LayerConfig& c, const Weight& w, const FrTensor& X, const FrTensor& rms_inv) {
-    Rescaling rs1(c.sf_linear), rs2(c.sf_linear);
-    zkFC g(1, c.embed_dim, FrTensor::view(w.weight));
-    auto g_inv_rms = g(rms_inv);
-    auto g_inv_rms_ = rs1(g_inv_rms);
-    auto Y = g_inv_rms_ * X;
-    auto Y_ = rs2(Y);
-
-    // The challenges in the order the proofs below draw them, so that both range proofs can be begun side by side on the
-    // library's streams; each is collected where the reference proves it and the product's sumcheck runs beside the second.
-    const auto ch2 = Rescaling::draw(Y.size);
-    auto hu = random_vec(ceilLog2(Y.size));
-    auto hv = random_vec(ceilLog2(Y.size));
-    const auto ch1 = Rescaling::draw(g_inv_rms.size);
-    auto p2 = rs2.prove_begin(Y, Y_, ch2);
-    auto p1 = rs1.prove_begin(g_inv_rms, g_inv_rms_, ch1);
+RmsNormBlock::RmsNormBlock(const LayerConfig& c, const Weight& w, const FrTensor& X, const FrTensor& rms_inv)
+    : c(c), w(w), X(X), rms_inv(rms_inv), rs1(c.sf_linear), rs2(c.sf_linear), g(1, c.embed_dim, FrTensor::view(w.weight)) {}
+const FrTensor& RmsNormBlock::forward() {
+    g_inv_rms.emplace(g(rms_inv));
+    g_inv_rms_.emplace(rs1(*g_inv_rms));
+    Y.emplace(*g_inv_rms_ * X);
+    Y_.emplace(rs2(*Y));
+    return *Y_;
+}
+void RmsNormBlock::begin() {
+    // The challenges in the order the proofs of finish() use them (rmsnorm.cu:41-45: the second rescaling, the product, the
+    // first rescaling, the weight's product), so that both range proofs can be begun side by side on the library's streams.
+    ch2 = Rescaling::draw(Y->size);
+    hu = random_vec(ceilLog2(Y->size));
+    hv = random_vec(ceilLog2(Y->size));
+    ch1 = Rescaling::draw(g_inv_rms->size);
+    chg = g.draw(rms_inv.size);
+    p2 = rs2.prove_begin(*Y, *Y_, ch2);
+    p1 = rs1.prove_begin(*g_inv_rms, *g_inv_rms_, ch1);
+}
+void RmsNormBlock::finish() {
     rs2.prove_end(p2);
-    hadamard_product_sumcheck(g_inv_rms_, X, hu, hv);
+    hadamard_product_sumcheck(*g_inv_rms_, X, hu, hv);
     rs1.prove_end(p1);
-    auto claims = g.prove(rms_inv, g_inv_rms);
+    auto claims = g.prove(rms_inv, *g_inv_rms, chg);
     if (c.open_weights) verifyWeightClaim(w, claims[0]);
-    return Y_;
+    p1 = Rescaling::Pending(); p2 = Rescaling::Pending();
+    g_inv_rms.reset(); g_inv_rms_.reset(); Y.reset();
+}
+FrTensor rmsnorm_block(const LayerConfig& c, const Weight& w, const FrTensor& X, const FrTensor& rms_inv) {
+    RmsNormBlock b(c, w, X, rms_inv);
+    b.forward();
+    b.begin();
+    b.finish();
+    return std::move(*b.Y_);
 }
 
 // self-attn.cu:19-76 (linear mode)
-void attn_linear_block(const LayerConfig& c, const Weight& q, const Weight& k, const Weight& v, const FrTensor& input, FrTensor& Q_, FrTensor& K_, FrTensor& V_) {
-    zkFC q_layer(c.embed_dim, c.embed_dim, FrTensor::view(q.weight)), k_layer(c.embed_dim, c.embed_dim, FrTensor::view(k.weight)), v_layer(c.embed_dim, c.embed_dim, FrTensor::view(v.weight));
-    Rescaling q_rescale(c.sf_linear), k_rescale(c.sf_linear), v_rescale(c.sf_linear);
-    auto Q = q_layer(input);
-    Q_ = q_rescale(Q);
-    auto K = k_layer(input);
-    K_ = k_rescale(K);
-    auto V = v_layer(input);
-    V_ = v_rescale(V);
-    auto pq = q_rescale.prove_begin(Q, Q_);      // three range proofs side by side
-    auto pk = k_rescale.prove_begin(K, K_);
-    auto pv = v_rescale.prove_begin(V, V_);
+AttnLinearBlock::AttnLinearBlock(const LayerConfig& c, const Weight& q, const Weight& k, const Weight& v, const FrTensor& input)
+    : c(c), q(q), k(k), v(v), input(input), q_layer(c.embed_dim, c.embed_dim, FrTensor::view(q.weight)), k_layer(c.embed_dim, c.embed_dim, FrTensor::view(k.weight)),
+      v_layer(c.embed_dim, c.embed_dim, FrTensor::view(v.weight)), q_rescale(c.sf_linear), k_rescale(c.sf_linear), v_rescale(c.sf_linear) {}
+void AttnLinearBlock::forward() {
+    Q.emplace(q_layer(input));
+    Q_.emplace(q_rescale(*Q));
+    K.emplace(k_layer(input));
+    K_.emplace(k_rescale(*K));
+    V.emplace(v_layer(input));
+    V_.emplace(v_rescale(*V));
+}
+void AttnLinearBlock::begin() {
+    // challenges in the order of self-attn.cu:58-69: the three rescalings, then the products of K, Q and V
+    ch_qr = Rescaling::draw(Q->size);
+    ch_kr = Rescaling::draw(K->size);
+    ch_vr = Rescaling::draw(V->size);
+    const uint batch = input.size / c.embed_dim;
+    ch_k = k_layer.draw(batch);
+    ch_q = q_layer.draw(batch);
+    ch_v = v_layer.draw(batch);
+    pq = q_rescale.prove_begin(*Q, *Q_, ch_qr);      // three range proofs side by side
+    pk = k_rescale.prove_begin(*K, *K_, ch_kr);
+    pv = v_rescale.prove_begin(*V, *V_, ch_vr);
+}
+void AttnLinearBlock::finish() {
     q_rescale.prove_end(pq);
     k_rescale.prove_end(pk);
     v_rescale.prove_end(pv);
     OpeningGroup together;      // the three openings claimed below run as one device job, queued at the last claim
-    auto ck = k_layer.prove(input, K);
+    auto ck = k_layer.prove(input, *K, ch_k);
     if (c.open_weights) verifyWeightClaim(k, ck[0]);
-    auto cq = q_layer.prove(input, Q);
+    auto cq = q_layer.prove(input, *Q, ch_q);
     if (c.open_weights) verifyWeightClaim(q, cq[0]);
-    auto cv = v_layer.prove(input, V);
+    auto cv = v_layer.prove(input, *V, ch_v);
     if (c.open_weights) verifyWeightClaim(v, cv[0]);
     together.end();
+    pq = Rescaling::Pending(); pk = Rescaling::Pending(); pv = Rescaling::Pending();
+    Q.reset(); K.reset(); V.reset();
+}
+void attn_linear_block(const LayerConfig& c, const Weight& q, const Weight& k, const Weight& v, const FrTensor& input, FrTensor& Q_, FrTensor& K_, FrTensor& V_) {
+    AttnLinearBlock b(c, q, k, v, input);
+    b.forward();
+    b.begin();
+    b.finish();
+    Q_ = std::move(*b.Q_);
+    K_ = std::move(*b.K_);
+    V_ = std::move(*b.V_);
 }
 
 // columns [h*d, (h+1)*d) of a seq x embed tensor as a contiguous seq x d tensor
@@ -153,9 +192,7 @@ static FrTensor attn_stacked_heads(const LayerConfig& c, const FrTensor& Q_, con
     const uint per = g * seq * d;
     for (uint h0 = 0; h0 < H; h0 += g) {
         const uint b = (h0 / g) * per;
-        std::unique_ptr<FrTensor> Qg, Kg, Vg;
-        if (g != H) { Qg.reset(new FrTensor(Qs.trunc(b, b + per))); Kg.reset(new FrTensor(Ks.trunc(b, b + per))); Vg.reset(new FrTensor(Vs.trunc(b, b + per))); }
-        const FrTensor &Q = g != H ? *Qg : Qs, &K = g != H ? *Kg : Ks, &V = g != H ? *Vg : Vs;
+        FrTensor Q = Qs.trunc(b, b + per), K = Ks.trunc(b, b + per), V = Vs.trunc(b, b + per);
         FrTensor sm_in(g * seq * seq), sm_out(g * seq * seq), shift(g * seq), shifted(g * seq * seq);
         vector<FrTensor> in_seg, out_seg, m_seg;
         FrTensor out = attn.compute(Q, K, V, sm_in, sm_out, shift, shifted, in_seg, out_seg, m_seg);
@@ -168,10 +205,62 @@ static FrTensor attn_stacked_heads(const LayerConfig& c, const FrTensor& Q_, con
     return outs.transpose_stack(H, seq, d).transpose(E, seq);   // [head][d][seq] = embed x seq -> seq x embed
 }
 
+// All heads as ONE stack (attn_head_group == num_heads), in three steps.
+AttnStackBlock::AttnStackBlock(const LayerConfig& c, const FrTensor& Q_, const FrTensor& K_, const FrTensor& V_)
+    : c(c), Q_(Q_), K_(K_), V_(V_),
+      attn(c.num_heads, c.softmax_sf_in, 1UL, c.softmax_bs, c.softmax_L, c.softmax_M, c.softmax_thetas, c.seq_len, c.seq_len, c.embed_dim / c.num_heads, 1), rs1(c.sf_attn),
+      rs2(c.sf_attn) {
+    if (c.embed_dim % c.num_heads) throw std::runtime_error("embed_dim must be a multiple of num_heads");
+}
+const FrTensor& AttnStackBlock::forward() {
+    const uint seq = c.seq_len, E = c.embed_dim, H = c.num_heads, d = E / H;
+    // seq x embed -> embed x seq = [head][d][seq] -> [head][seq][d]
+    auto to_stack = [&](const FrTensor& t) { return t.transpose(seq, E).transpose_stack(H, d, seq); };
+    Qs.emplace(to_stack(Q_));
+    Ks.emplace(to_stack(K_));
+    Vs.emplace(to_stack(V_));
+    sm_in.emplace(H * seq * seq);
+    sm_out.emplace(H * seq * seq);
+    shift.emplace(H * seq);
+    {
+        FrTensor shifted(H * seq * seq);       // no proof reads it
+        out.emplace(attn.compute(*Qs, *Ks, *Vs, *sm_in, *sm_out, *shift, shifted, in_seg, out_seg, m_seg));
+    }
+    out_all.emplace(out->transpose_stack(H, seq, d).transpose(E, seq));   // [head][d][seq] = embed x seq -> seq x embed
+    out_.emplace(rs2(*out_all));
+    out__.emplace(rs1(*out_));
+    return *out__;
+}
+void AttnStackBlock::begin() {
+    ch = attn.draw();
+    ch_r1 = Rescaling::draw(out_->size);
+    ch_r2 = Rescaling::draw(out_all->size);
+    pending = attn.prove_jobs_begin(in_seg, out_seg, m_seg, ch.u_matmul_out, ch.v_matmul_out, ch.v_matmul_out_num, ch.v_sm, ch.temp_rand[0], ch.temp_rand[1], ch.temp_rand[2]);
+    p1 = rs1.prove_begin(*out_, *out__, ch_r1);
+    p2 = rs2.prove_begin(*out_all, *out_, ch_r2);
+}
+void AttnStackBlock::finish() {
+    vector<Polynomial> proof;
+    attn.prove_finish(pending, *Qs, *Ks, *Vs, *out, *sm_out, *sm_in, *shift, in_seg, out_seg, ch.u_matmul_out_num, ch.v_matmul_out_num, ch.u_matmul_out, ch.v_matmul_out,
+                      ch.w_matmul_out, ch.v_sm, ch.v_matmul_in_num, ch.v_matmul_in, proof);
+    rs1.prove_end(p1);
+    rs2.prove_end(p2);
+    pending = zkSoftmax::Pending(); p1 = Rescaling::Pending(); p2 = Rescaling::Pending();
+    in_seg.clear(); out_seg.clear(); m_seg.clear();
+    Qs.reset(); Ks.reset(); Vs.reset(); sm_in.reset(); sm_out.reset(); shift.reset(); out.reset(); out_all.reset(); out_.reset();
+}
+
 // Per-head attention following self-attn.cu:78-121 (attn mode) with d = head width.
 FrTensor attn_heads_block(const LayerConfig& c, const FrTensor& Q_, const FrTensor& K_, const FrTensor& V_) {
     const uint seq = c.seq_len, E = c.embed_dim, H = c.num_heads, d = E / H;
     if (E % H) throw std::runtime_error("embed_dim must be a multiple of num_heads");
+    if (c.attn_head_group == H) {
+        AttnStackBlock b(c, Q_, K_, V_);
+        b.forward();
+        b.begin();
+        b.finish();
+        return std::move(*b.out__);
+    }
     if (c.attn_head_group) {
         FrTensor out_all = attn_stacked_heads(c, Q_, K_, V_);
         Rescaling rs1(c.sf_attn), rs2(c.sf_attn);
@@ -308,110 +397,202 @@ FrTensor attn_reference_block(const LayerConfig& c, const FrTensor& Q, const FrT
     return out__;
 }
 
-FrTensor oproj_block(const LayerConfig& c, const Weight& o, const FrTensor& attn_out) {
-    zkFC o_layer(c.embed_dim, c.embed_dim, FrTensor::view(o.weight));
-    Rescaling o_rescale(c.sf_linear);
-    auto O = o_layer(attn_out);
-    auto O_ = o_rescale(O);
-    o_rescale.prove(O, O_);
-    auto co = o_layer.prove(attn_out, O);
+OProjBlock::OProjBlock(const LayerConfig& c, const Weight& o, const FrTensor& attn_out)
+    : c(c), o(o), attn_out(attn_out), o_layer(c.embed_dim, c.embed_dim, FrTensor::view(o.weight)), o_rescale(c.sf_linear) {}
+const FrTensor& OProjBlock::forward() {
+    O.emplace(o_layer(attn_out));
+    O_.emplace(o_rescale(*O));
+    return *O_;
+}
+void OProjBlock::begin() {
+    ch_r = Rescaling::draw(O->size);
+    ch_o = o_layer.draw(attn_out.size / c.embed_dim);
+    p = o_rescale.prove_begin(*O, *O_, ch_r);
+}
+void OProjBlock::finish() {
+    o_rescale.prove_end(p);
+    auto co = o_layer.prove(attn_out, *O, ch_o);
     if (c.open_weights) verifyWeightClaim(o, co[0]);
-    return O_;
+    p = Rescaling::Pending();
+    O.reset();
+}
+FrTensor oproj_block(const LayerConfig& c, const Weight& o, const FrTensor& attn_out) {
+    OProjBlock b(c, o, attn_out);
+    b.forward();
+    b.begin();
+    b.finish();
+    return std::move(*b.O_);
 }
 
 // ffn.cu:44-93
-FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, const Weight& down, const FrTensor& swiglu_values, const FrTensor& input,
-                   std::unique_ptr<FrTensor>* down_out_unrescaled) {
-    zkFC up_layer(c.embed_dim, c.hidden_dim, FrTensor::view(up.weight)), gate_layer(c.embed_dim, c.hidden_dim, FrTensor::view(gate.weight)), down_layer(c.hidden_dim, c.embed_dim, FrTensor::view(down.weight));
-    Rescaling up_rescale(c.sf_linear), gate_rescale(c.sf_gate), hidden_rescale(c.sf_linear), down_rescale(c.sf_linear);
-    tLookupRangeMapping swiglu(c.swiglu_low, c.swiglu_len, swiglu_values);
-
-    // Every challenge of this block, drawn first and in the order ffn.cu draws them (:67-69 the three of the activation
-    // lookup, then inside the proofs of :83-93): the forward pass draws none.  The three weight openings need nothing but
-    // their points, so they start as soon as the forward pass is queued and run beside the whole proof instead of behind it.
+FfnBlock::FfnBlock(const LayerConfig& c, const Weight& up, const Weight& gate, const Weight& down, const FrTensor& swiglu_values, const FrTensor& input)
+    : c(c), up(up), gate(gate), down(down), input(input), up_layer(c.embed_dim, c.hidden_dim, FrTensor::view(up.weight)),
+      gate_layer(c.embed_dim, c.hidden_dim, FrTensor::view(gate.weight)), down_layer(c.hidden_dim, c.embed_dim, FrTensor::view(down.weight)), up_rescale(c.sf_linear),
+      gate_rescale(c.sf_gate), hidden_rescale(c.sf_linear), down_rescale(c.sf_linear), swiglu(c.swiglu_low, c.swiglu_len, swiglu_values) {}
+const FrTensor& FfnBlock::forward() {
+    up_out.emplace(up_layer(input));
+    up_out_.emplace(up_rescale.rescale(*up_out, true));            // int32 forms: the activation lookup and the product below read them
+    gate_out.emplace(gate_layer(input));
+    gate_out_.emplace(gate_rescale.rescale(*gate_out, true));
+    auto p = swiglu(*gate_out_);
+    swiglu_out.emplace(std::move(p.first));
+    swiglu_m.emplace(std::move(p.second));
+    down_in.emplace(*swiglu_out * *up_out_);
+    down_in_.emplace(hidden_rescale(*down_in));
+    down_out.emplace(down_layer(*down_in_));
+    down_out_.emplace(down_rescale(*down_out));
+    return *down_out_;
+}
+void FfnBlock::begin() {
+    // Every challenge of this block in the order ffn.cu draws them (:67-69 the three of the activation lookup, then inside the
+    // proofs of :83-93).  The three weight openings need nothing but their points, so (where openings may start ahead of their
+    // claims) they start here and run beside the whole proof instead of behind it.
     const uint seq = input.size / c.embed_dim;
-    auto temp_rand = random_vec(3);
-    auto swiglu_u = random_vec(ceilLog2(c.seq_len * c.hidden_dim));
-    auto swiglu_v = random_vec(ceilLog2(c.seq_len * c.hidden_dim));
-    const auto ch_dr = Rescaling::draw(seq * c.embed_dim);       // down_out
-    const auto ch_d = down_layer.draw(seq);
-    const auto ch_hr = Rescaling::draw(seq * c.hidden_dim);      // down_in
-    const auto ch_gr = Rescaling::draw(seq * c.hidden_dim);      // gate_out
-    const auto ch_g = gate_layer.draw(seq);
-    const auto ch_ur = Rescaling::draw(seq * c.hidden_dim);      // up_out
-    const auto ch_u = up_layer.draw(seq);
-    WeightOpeningAhead od, og, ou;
-
-    auto up_out = up_layer(input);
-    auto up_out_ = up_rescale.rescale(up_out, true);            // int32 forms: the activation lookup and the product below read them
-    auto gate_out = gate_layer(input);
-    auto gate_out_ = gate_rescale.rescale(gate_out, true);
-    auto p = swiglu(gate_out_);
-    auto &swiglu_out = p.first, &swiglu_m = p.second;
-
-    auto down_in = swiglu_out * up_out_;
-    auto down_in_ = hidden_rescale(down_in);
-    auto down_out = down_layer(down_in_);
-    auto down_out_ = down_rescale(down_out);
+    temp_rand = random_vec(3);
+    swiglu_u = random_vec(ceilLog2(c.seq_len * c.hidden_dim));
+    swiglu_v = random_vec(ceilLog2(c.seq_len * c.hidden_dim));
+    ch_dr = Rescaling::draw(seq * c.embed_dim);       // down_out
+    ch_d = down_layer.draw(seq);
+    ch_hr = Rescaling::draw(seq * c.hidden_dim);      // down_in
+    ch_gr = Rescaling::draw(seq * c.hidden_dim);      // gate_out
+    ch_g = gate_layer.draw(seq);
+    ch_ur = Rescaling::draw(seq * c.hidden_dim);      // up_out
+    ch_u = up_layer.draw(seq);
     if (c.open_weights) {
         // behind the forward pass (the openings are ordered after what is queued here): started before it, their kernels keep
         // the forward pass's matrix products waiting for most of their own duration
         auto ahead = openWeightsAhead({&up, &gate, &down}, {&ch_u.u_input, &ch_g.u_input, &ch_d.u_input}, {&ch_u.u_output, &ch_g.u_output, &ch_d.u_output});   // the two large ones first
         ou = std::move(ahead[0]); og = std::move(ahead[1]); od = std::move(ahead[2]);
     }
-
     // The five lookup proofs of the block (four rescalings, the activation table) need only the forward pass and their
     // challenges: all are begun here, on the library's streams, and each is collected where the reference proves it, so
     // the matrix-product proofs on the caller's stream run beside them and the transcript keeps its order.
-    auto pd = down_rescale.prove_begin(down_out, down_out_, ch_dr);
-    auto ph = hidden_rescale.prove_begin(down_in, down_in_, ch_hr);
-    auto ps = swiglu.prove_begin(gate_out_, swiglu_out, swiglu_m, temp_rand[0], temp_rand[1], temp_rand[2], swiglu_u, swiglu_v);
-    auto pg = gate_rescale.prove_begin(gate_out, gate_out_, ch_gr);
-    auto pu = up_rescale.prove_begin(up_out, up_out_, ch_ur);
+    pd = down_rescale.prove_begin(*down_out, *down_out_, ch_dr);
+    ph = hidden_rescale.prove_begin(*down_in, *down_in_, ch_hr);
+    ps = swiglu.prove_begin(*gate_out_, *swiglu_out, *swiglu_m, temp_rand[0], temp_rand[1], temp_rand[2], swiglu_u, swiglu_v);
+    pg = gate_rescale.prove_begin(*gate_out, *gate_out_, ch_gr);
+    pu = up_rescale.prove_begin(*up_out, *up_out_, ch_ur);
+}
+void FfnBlock::finish() {
     down_rescale.prove_end(pd);
-    auto cd = down_layer.prove(down_in_, down_out, ch_d);
+    auto cd = down_layer.prove(*down_in_, *down_out, ch_d);
     if (c.open_weights) verifyWeightClaim(down, cd[0], od);
     hidden_rescale.prove_end(ph);
     tLookup::prove_end(ps);
     gate_rescale.prove_end(pg);
     OpeningGroup gate_and_up;   // when nothing was started ahead: the two openings over the same generator count as one job, queued at up's claim
-    auto cg = gate_layer.prove(input, gate_out, ch_g);
+    auto cg = gate_layer.prove(input, *gate_out, ch_g);
     if (c.open_weights) verifyWeightClaim(gate, cg[0], og);
     up_rescale.prove_end(pu);
-    auto cu = up_layer.prove(input, up_out, ch_u);
+    auto cu = up_layer.prove(input, *up_out, ch_u);
     if (c.open_weights) verifyWeightClaim(up, cu[0], ou);
     gate_and_up.end();
+    pd = Rescaling::Pending(); ph = Rescaling::Pending(); pg = Rescaling::Pending(); pu = Rescaling::Pending(); ps = LookupPending();
+    up_out.reset(); up_out_.reset(); gate_out.reset(); gate_out_.reset(); swiglu_out.reset(); swiglu_m.reset(); down_in.reset(); down_in_.reset();
+}
+FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, const Weight& down, const FrTensor& swiglu_values, const FrTensor& input,
+                   std::unique_ptr<FrTensor>* down_out_unrescaled) {
+    FfnBlock b(c, up, gate, down, swiglu_values, input);
+    b.forward();
+    b.begin();
+    b.finish();
     // the reference's executable saves the unrescaled down_out (ffn.cu:81); the rescaled tensor is what the next block consumes
-    if (down_out_unrescaled) down_out_unrescaled->reset(new FrTensor(std::move(down_out)));
-    return down_out_;
+    if (down_out_unrescaled) down_out_unrescaled->reset(new FrTensor(std::move(*b.down_out)));
+    return std::move(*b.down_out_);
 }
 
+static bool g_overlap_blocks = [] {
+    const char* e = getenv("ZKLLM_LAYER_OVERLAP");
+    return !(e && e[0] == '0');
+}();
+bool layer_blocks_overlap() { return g_overlap_blocks; }
+void layer_set_blocks_overlap(bool on) { g_overlap_blocks = on; }
+
+// The blocks in the order of the reference's executables.  A block's forward pass draws no challenge and records nothing, and
+// the device jobs of its proof need only that pass and the block's challenges; so, with overlap, the next block's forward pass
+// and jobs are queued BEFORE the host collects this block's proofs: the caller's stream works on the next block while the
+// library's streams still run this block's lookup sumchecks, instead of idling until they are collected.  Challenges are still
+// drawn block after block and every transcript entry is written in the order of a block-by-block run: begin() draws and
+// records nothing, finish() records and draws nothing.
 FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor& X, LayerTimes* times) {
     LayerTimes t;
     // the nine weight openings run on the device beside the sumchecks; with a learned plan they start ahead of their claims
     // (not with ZKLLM_OPEN_AHEAD=0 / zk_openings_set_only_at_claim: then each starts at its claim)
     DeferredOpenings openings(c.open_weights ? w.plan.get() : nullptr, {&w.input_norm, &w.q, &w.k, &w.v, &w.o, &w.post_norm, &w.up, &w.gate, &w.down});
+    const bool overlap = g_overlap_blocks;
     const double t0 = now_ms();
+    // per-block times: with overlap, host clock from the end of the block before to the end of this block's finish() (the blocks
+    // share the device, so no other split exists); without, as before, with the caller's stream idle at both ends
+    double mark = t0;
+    auto lap = [&] {
+        const double n = overlap ? std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now().time_since_epoch()).count() : now_ms();
+        const double d = n - mark;
+        mark = n;
+        return d;
+    };
+    std::function<void()> owed;      // finish() of the block whose proofs are not collected yet
+    double* owed_slot = nullptr;
+    auto settle = [&] {
+        if (!owed) return;
+        auto f = std::move(owed);
+        owed = nullptr;
+        f();
+        *owed_slot += lap();
+    };
+    auto begun = [&](std::function<void()> finish, double& slot) {      // call after the block's forward() and begin()
+        if (overlap) settle();
+        owed = std::move(finish);
+        owed_slot = &slot;
+        if (!overlap) settle();
+    };
+
     FrTensor rms1 = compute_rms_inv(X, c.seq_len, c.embed_dim, c.rms_eps, c.value_scale);
-    FrTensor n1 = rmsnorm_block(c, w.input_norm, X, rms1);
-    const double t1 = now_ms();
-    FrTensor Q_(X.size), K_(X.size), V_(X.size);
-    attn_linear_block(c, w.q, w.k, w.v, n1, Q_, K_, V_);
-    const double t2 = now_ms();
-    FrTensor attn = attn_heads_block(c, Q_, K_, V_);
-    const double t3 = now_ms();
-    FrTensor o = oproj_block(c, w.o, attn);
+    RmsNormBlock norm1(c, w.input_norm, X, rms1);
+    const FrTensor& n1 = norm1.forward();
+    norm1.begin();
+    begun([&] { norm1.finish(); }, t.rmsnorm1);
+
+    AttnLinearBlock qkv(c, w.q, w.k, w.v, n1);
+    qkv.forward();
+    qkv.begin();
+    begun([&] { qkv.finish(); }, t.qkv);
+
+    std::optional<AttnStackBlock> stack;
+    std::optional<FrTensor> attn_loop;          // the other variants prove inside their forward passes: nothing may be owed then
+    if (c.attn_head_group == c.num_heads) {
+        stack.emplace(c, *qkv.Q_, *qkv.K_, *qkv.V_);
+        stack->forward();
+        stack->begin();
+        begun([&] { stack->finish(); }, t.attention);
+    } else {
+        settle();
+        attn_loop.emplace(attn_heads_block(c, *qkv.Q_, *qkv.K_, *qkv.V_));
+        t.attention += lap();
+    }
+    const FrTensor& attn = stack ? *stack->out__ : *attn_loop;
+
+    OProjBlock oproj(c, w.o, attn);
+    const FrTensor& o = oproj.forward();
     FrTensor x2 = X + o;                                   // skip-connection.cu:15-18
-    const double t4 = now_ms();
+    oproj.begin();
+    begun([&] { oproj.finish(); }, t.oproj);
+
     FrTensor rms2 = compute_rms_inv(x2, c.seq_len, c.embed_dim, c.rms_eps, c.value_scale);
-    FrTensor n2 = rmsnorm_block(c, w.post_norm, x2, rms2);
-    const double t5 = now_ms();
-    FrTensor f = ffn_block(c, w.up, w.gate, w.down, w.swiglu_table, n2);
+    RmsNormBlock norm2(c, w.post_norm, x2, rms2);
+    const FrTensor& n2 = norm2.forward();
+    norm2.begin();
+    begun([&] { norm2.finish(); }, t.rmsnorm2);
+
+    FfnBlock ffn(c, w.up, w.gate, w.down, w.swiglu_table, n2);
+    const FrTensor& f = ffn.forward();
     FrTensor out = x2 + f;
+    ffn.begin();
+    begun([&] { ffn.finish(); }, t.ffn);
+    settle();
     const double t6 = now_ms();
     openings.finish();
     const double t7 = now_ms();
-    t.rmsnorm1 = t1 - t0; t.qkv = t2 - t1; t.attention = t3 - t2; t.oproj = t4 - t3; t.rmsnorm2 = t5 - t4; t.ffn = t6 - t5; t.open_wait = t7 - t6; t.total = t7 - t0;
+    t.open_wait = t7 - t6; t.total = t7 - t0;
     if (times) *times = t;
     return out;
 }

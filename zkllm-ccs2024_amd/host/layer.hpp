@@ -17,6 +17,7 @@
 //    mask are left out, the RMS statistic is computed on the host in double precision.
 #pragma once
 #include <memory>
+#include <optional>
 #include "commitment.hpp"
 #include "fr-tensor.hpp"
 #include "rescaling.hpp"
@@ -67,6 +68,88 @@ FrTensor compute_rms_inv(const FrTensor& X, uint seq_len, uint embed_dim, double
 // x = (low + i) / in_scale
 FrTensor make_swiglu_table(int low, uint len, double in_scale, double out_scale);
 
+// Every block in three steps (an addition; the *_block functions below run the three in a row, which is the reference's flow):
+//   forward()  the block's tensors, queued on the caller's stream; draws no challenge, records nothing
+//   begin()    draws ALL of the block's challenges in the order the reference's proofs draw them and queues the device jobs of
+//              its lookup proofs on the library's streams; records nothing
+//   finish()   the rest of the proofs, the transcript entries in the reference's order, the weight claims; draws nothing
+// so a caller may queue the next block's forward() and begin() before this block's finish() (llama_layer does): the jobs run
+// beside that forward pass.  The blocks hold references to their inputs, which must outlive them; finish() frees the block's
+// tensors except its outputs.
+struct RmsNormBlock {
+    RmsNormBlock(const LayerConfig& c, const Weight& w, const FrTensor& X, const FrTensor& rms_inv);
+    const FrTensor& forward();
+    void begin();
+    void finish();
+    const LayerConfig& c; const Weight& w; const FrTensor& X; const FrTensor& rms_inv;
+    Rescaling rs1, rs2;
+    zkFC g;
+    std::optional<FrTensor> g_inv_rms, g_inv_rms_, Y, Y_;      // Y_: the output
+    Rescaling::Challenges ch1, ch2;
+    vector<Fr_t> hu, hv;
+    zkFC::Challenges chg;
+    Rescaling::Pending p1, p2;
+};
+struct AttnLinearBlock {
+    AttnLinearBlock(const LayerConfig& c, const Weight& q, const Weight& k, const Weight& v, const FrTensor& input);
+    void forward();
+    void begin();
+    void finish();
+    const LayerConfig& c; const Weight &q, &k, &v; const FrTensor& input;
+    zkFC q_layer, k_layer, v_layer;
+    Rescaling q_rescale, k_rescale, v_rescale;
+    std::optional<FrTensor> Q, K, V, Q_, K_, V_;               // Q_, K_, V_: the outputs
+    Rescaling::Challenges ch_qr, ch_kr, ch_vr;
+    zkFC::Challenges ch_q, ch_k, ch_v;
+    Rescaling::Pending pq, pk, pv;
+};
+// attention with all heads as one stack (attn_head_group == num_heads) and the two rescalings of its output
+struct AttnStackBlock {
+    AttnStackBlock(const LayerConfig& c, const FrTensor& Q_, const FrTensor& K_, const FrTensor& V_);
+    const FrTensor& forward();
+    void begin();
+    void finish();
+    const LayerConfig& c; const FrTensor &Q_, &K_, &V_;
+    zkAttnStacked attn;
+    Rescaling rs1, rs2;
+    std::optional<FrTensor> Qs, Ks, Vs, sm_in, sm_out, shift, out, out_all, out_, out__;      // out__: the output
+    vector<FrTensor> in_seg, out_seg, m_seg;
+    zkAttnStacked::Challenges ch;
+    Rescaling::Challenges ch_r1, ch_r2;
+    zkSoftmax::Pending pending;
+    Rescaling::Pending p1, p2;
+};
+struct OProjBlock {
+    OProjBlock(const LayerConfig& c, const Weight& o, const FrTensor& attn_out);
+    const FrTensor& forward();
+    void begin();
+    void finish();
+    const LayerConfig& c; const Weight& o; const FrTensor& attn_out;
+    zkFC o_layer;
+    Rescaling o_rescale;
+    std::optional<FrTensor> O, O_;                             // O_: the output
+    Rescaling::Challenges ch_r;
+    zkFC::Challenges ch_o;
+    Rescaling::Pending p;
+};
+struct FfnBlock {
+    FfnBlock(const LayerConfig& c, const Weight& up, const Weight& gate, const Weight& down, const FrTensor& swiglu_values, const FrTensor& input);
+    const FrTensor& forward();
+    void begin();
+    void finish();
+    const LayerConfig& c; const Weight &up, &gate, &down; const FrTensor& input;
+    zkFC up_layer, gate_layer, down_layer;
+    Rescaling up_rescale, gate_rescale, hidden_rescale, down_rescale;
+    tLookupRangeMapping swiglu;
+    std::optional<FrTensor> up_out, up_out_, gate_out, gate_out_, swiglu_out, swiglu_m, down_in, down_in_, down_out, down_out_;   // down_out_: the output; down_out is kept too
+    vector<Fr_t> temp_rand, swiglu_u, swiglu_v;
+    Rescaling::Challenges ch_dr, ch_hr, ch_gr, ch_ur;
+    zkFC::Challenges ch_d, ch_g, ch_u;
+    WeightOpeningAhead od, og, ou;
+    Rescaling::Pending pd, ph, pg, pu;
+    LookupPending ps;
+};
+
 FrTensor rmsnorm_block(const LayerConfig& c, const Weight& w, const FrTensor& X, const FrTensor& rms_inv);
 void attn_linear_block(const LayerConfig& c, const Weight& q, const Weight& k, const Weight& v, const FrTensor& input, FrTensor& Q_, FrTensor& K_, FrTensor& V_);
 FrTensor attn_heads_block(const LayerConfig& c, const FrTensor& Q_, const FrTensor& K_, const FrTensor& V_);
@@ -81,6 +164,11 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
 FrTensor attn_reference_block(const LayerConfig& c, const FrTensor& Q, const FrTensor& K, const FrTensor& V, std::unique_ptr<FrTensor>* softmax_out = nullptr);
 
 // whole layer: x -> x + attn(norm(x)) -> (+ ffn(norm(.)))
+// Each block's forward() and begin() are queued before the finish() of the block before it, unless ZKLLM_LAYER_OVERLAP=0 /
+// layer_set_blocks_overlap(false): then block after block.  Same outputs, same transcript.  (With attn_head_group other than
+// num_heads the attention block proves inside its forward pass and nothing overlaps it.)
+bool layer_blocks_overlap();
+void layer_set_blocks_overlap(bool on);
 FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor& X, LayerTimes* times);
 
 // how long make_random_layer_weights last spent on each part of the setup (ms, device idle at both ends of every part):

@@ -262,8 +262,24 @@ Fr_t zkAttnStacked::prove(const FrTensor& Q, const FrTensor& K, const FrTensor& 
     // The softmax proof's sumcheck jobs need only tensors of the forward pass and challenges, so they are queued first and
     // run on the library's side streams beside the proof of out = Y V; values are recorded in the reference's order.  (Jobs left
     // unfinished by an exception are waited for and dropped by the pending object.)
+    Pending pending = prove_jobs_begin(sm_in_segments, sm_out_segments, sm_m_segments, u_matmul_out, v_matmul_out, v_matmul_out_num, v_sm, r_seg, alpha_seg, beta_seg);
+    return prove_finish(pending, Q, K, V, out, sm_out, sm_in, sm_shift, sm_in_segments, sm_out_segments, u_matmul_out_num, v_matmul_out_num, u_matmul_out, v_matmul_out,
+                        w_matmul_out, v_sm, v_matmul_in_num, v_matmul_in, proof);
+}
+
+zkSoftmax::Pending zkAttnStacked::prove_jobs_begin(const vector<FrTensor>& sm_in_segments, const vector<FrTensor>& sm_out_segments, const vector<FrTensor>& sm_m_segments,
+                                                   const vector<Fr_t>& u_matmul_out, const vector<Fr_t>& v_matmul_out, const vector<Fr_t>& v_matmul_out_num,
+                                                   const vector<Fr_t>& v_sm, const Fr_t& r_seg, const Fr_t& alpha_seg, const Fr_t& beta_seg) {
     const auto u_Y = concatenate<Fr_t>({v_matmul_out, u_matmul_out, v_matmul_out_num});
-    Pending pending = jobs_begin(sm_in_segments, sm_out_segments, sm_m_segments, u_Y, v_sm, r_seg, alpha_seg, beta_seg);
+    return jobs_begin(sm_in_segments, sm_out_segments, sm_m_segments, u_Y, v_sm, r_seg, alpha_seg, beta_seg);
+}
+
+Fr_t zkAttnStacked::prove_finish(Pending& pending, const FrTensor& Q, const FrTensor& K, const FrTensor& V, const FrTensor& out, const FrTensor& sm_out, const FrTensor& sm_in,
+                                 const FrTensor& sm_shift, const vector<FrTensor>& sm_in_segments, const vector<FrTensor>& sm_out_segments,
+                                 const vector<Fr_t>& u_matmul_out_num, const vector<Fr_t>& v_matmul_out_num, const vector<Fr_t>& u_matmul_out, const vector<Fr_t>& v_matmul_out,
+                                 const vector<Fr_t>& w_matmul_out, const vector<Fr_t>& v_sm, const vector<Fr_t>& v_matmul_in_num, const vector<Fr_t>& v_matmul_in,
+                                 vector<Polynomial>& proof) {
+    if (sm_in.size != sm_out.size) throw std::invalid_argument("X and Y must have the same size " + to_string(sm_in.size) + " " + to_string(sm_out.size));
     auto out_claim = out.multi_dim_me({u_matmul_out_num, u_matmul_out, w_matmul_out}, {num, m, d});
     zk_record(out_claim);
     auto sm_out_reduced = sm_out.partial_me(u_matmul_out, m, n);

@@ -82,6 +82,16 @@ class zkAttnStacked : public zkAttn {
                const vector<Fr_t>& u_matmul_out_num, const vector<Fr_t>& v_matmul_out_num, const vector<Fr_t>& u_matmul_out, const vector<Fr_t>& v_matmul_out,
                const vector<Fr_t>& w_matmul_out, const vector<Fr_t>& v_sm, const Fr_t& r_seg, const Fr_t& alpha_seg, const Fr_t& beta_seg,
                const vector<Fr_t>& v_matmul_in_num, const vector<Fr_t>& v_matmul_in, vector<Polynomial>& proof);
+    // Addition: prove() in two steps.  prove_jobs_begin queues the softmax proof's sumcheck jobs on the library's streams and
+    // records nothing; prove_finish does everything else of prove() and collects them.  A caller may queue other device work
+    // between the two (the jobs run beside it); challenges are drawn by neither.
+    Pending prove_jobs_begin(const vector<FrTensor>& sm_in_segments, const vector<FrTensor>& sm_out_segments, const vector<FrTensor>& sm_m_segments,
+                             const vector<Fr_t>& u_matmul_out, const vector<Fr_t>& v_matmul_out, const vector<Fr_t>& v_matmul_out_num, const vector<Fr_t>& v_sm,
+                             const Fr_t& r_seg, const Fr_t& alpha_seg, const Fr_t& beta_seg);
+    Fr_t prove_finish(Pending& pending, const FrTensor& Q, const FrTensor& K, const FrTensor& V, const FrTensor& out, const FrTensor& sm_out, const FrTensor& sm_in,
+                      const FrTensor& sm_shift, const vector<FrTensor>& sm_in_segments, const vector<FrTensor>& sm_out_segments, const vector<Fr_t>& u_matmul_out_num,
+                      const vector<Fr_t>& v_matmul_out_num, const vector<Fr_t>& u_matmul_out, const vector<Fr_t>& v_matmul_out, const vector<Fr_t>& w_matmul_out,
+                      const vector<Fr_t>& v_sm, const vector<Fr_t>& v_matmul_in_num, const vector<Fr_t>& v_matmul_in, vector<Polynomial>& proof);
 
    protected:
     const uint num;
