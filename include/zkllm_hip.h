@@ -46,6 +46,14 @@ int zk_pool_stats(size_t* live_bytes, size_t* cached_bytes);
  * (live blocks stay with their owners), its streams, the allocator's events, idle pinned buffers.  The library stays usable
  * afterwards.  A host calls it before it exits so that nothing is left to static destruction. */
 int zk_shutdown(void);
+/* No counterpart in the reference.  The sumcheck jobs that run beside the caller (zk_lookup_prove_begin*, zk_hadamard_prove_begin*)
+ * are long sequences of launches on a stream of the library's own.  With this on (the default; ZKLLM_ASYNC_JOBS=0 in the
+ * environment turns it off) begin only orders the job behind the caller's stream and hands the launches to a thread of the
+ * library's, so the caller goes on queuing its own work at once; the matching end waits for that thread to be done with the
+ * job before it waits for the device.  Results are the same either way.  An error met while the job's launches are queued is
+ * reported by its end call.  Jobs are launched in the order of their begin calls. */
+int zk_set_async_jobs(int on);
+int zk_async_jobs(void);
 /* replace cudaMemcpy in ctors, operator()(idx), savebin/loadbin (ioutils.cu:3-45) */
 int zk_memcpy_h2d(void* dst, const void* src_host, size_t bytes, void* stream);
 int zk_memcpy_d2h(void* dst_host, const void* src, size_t bytes, void* stream);

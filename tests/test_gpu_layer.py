@@ -45,8 +45,8 @@ def test_tiny_layer_transcript(pv, open_weights, seed, head_group):
 @pytest.mark.parametrize("open_weights,seed", [(True, 13), (False, 14)])
 def test_tiny_layer_blocks_overlapped_and_one_after_the_other(pv, open_weights, seed):
     """With all heads as one stack every block of the layer runs in three steps, and the layer queues a block's forward pass
-    and proof jobs before it collects the proofs of the block before it (zkp_layer_set_blocks_overlap, on by default).  Both
-    orders of work give the oracle's output and transcript."""
+    and proof jobs before it collects the proofs of earlier blocks (zkp_layer_set_blocks_overlap: how many blocks may be
+    begun and not yet collected; on by default).  Every order of work gives the oracle's output and transcript."""
     orc = load_oracle()
     cu, cf = layercfg.tiny(open_weights=open_weights, head_group=2)
     ws = layercfg.tiny_weights(seed, cu)
@@ -57,9 +57,10 @@ def test_tiny_layer_blocks_overlapped_and_one_after_the_other(pv, open_weights, 
     orc.orc_transcript_clear()
     orc_check(orc.orc_layer(cu, cf, *ws, 1, X, exp, None))
     exp_t = orc_transcript(orc)
-    assert pv.lib.zkp_layer_blocks_overlap() == 1
+    default = pv.lib.zkp_layer_blocks_overlap()
+    assert default > 0
     try:
-        for overlap in (0, 1):
+        for overlap in (0, 1, 3, 6):
             pv.lib.zkp_layer_set_blocks_overlap(overlap)
             pv.seed(seed)
             layer = pv.layer_create(cu, cf, ws, 1)
@@ -72,7 +73,7 @@ def test_tiny_layer_blocks_overlapped_and_one_after_the_other(pv, open_weights, 
             assert got_t.shape == exp_t.shape and (got_t == exp_t).all(), overlap
             assert min(times[:6]) > 0
     finally:
-        pv.lib.zkp_layer_set_blocks_overlap(1)
+        pv.lib.zkp_layer_set_blocks_overlap(default)
 
 
 def test_layer_run_again_starts_its_openings_ahead_and_proves_the_same(pv):

@@ -463,6 +463,72 @@ def test_hinted_lookup_job_equals_the_plain_one_whatever_the_hints(k):
         hip.free(p)
 
 
+def test_jobs_launched_by_the_library_thread_equal_those_launched_by_the_caller():
+    """zk_set_async_jobs: with it on, begin hands a job's launches to the library's launch thread and returns; off, the caller
+    queues them itself.  Four lookup jobs and two Hadamard jobs begun back to back (more jobs than streams of that kind, so
+    some share a stream) and ended in another order deliver the same sums both ways; the challenge arrays handed to begin are
+    overwritten right after the call, which the jobs must not notice."""
+    import ctypes
+    from gpuhelp import Hip, c_void_p, c_size_t, c_int
+    hip = Hip()
+    assert hip.lib.zk_async_jobs() == 1
+    k, N, low = 16, 256, -100
+    D = 1 << k
+    rng = np.random.default_rng(5)
+    T = fr_array([(low + j) % R_MOD for j in range(N)])
+    dT = hip.upload(T)
+    jobs = []
+    for j in range(4):
+        pos = rng.integers(0, N, D)
+        S = T[pos].copy()
+        m = fr_array([int(c) for c in np.bincount(pos, minlength=N)])
+        jobs.append((hip.upload(S), hip.upload(m), ch(60 + j, 1)[0], ch(70 + j, k - 1), ch(80 + j, k)))
+    Xs = [hip.upload(ch(90 + j, D)) for j in range(4)]
+    res = {}
+    try:
+        for mode in (1, 0, 1):
+            hip.call("zk_set_async_jobs", c_int(mode))
+            hs = []
+            for j, (dS, dm, beta, u, v) in enumerate(jobs):
+                h = c_void_p()
+                beta_, u_, v_ = beta.copy(), u.copy(), v.copy()
+                if j % 2:
+                    hip.call("zk_lookup_prove_begin_hinted", ctypes.byref(h), c_void_p(dS), c_void_p(dT), c_void_p(dm), c_void_p(dS), c_int(low), beta_, u_, v_, c_size_t(D), c_size_t(N), c_int(k), None)
+                else:
+                    hip.call("zk_lookup_prove_begin", ctypes.byref(h), c_void_p(dS), c_void_p(dT), c_void_p(dm), beta_, u_, v_, c_size_t(D), c_size_t(N), c_int(k), None)
+                beta_[:] = 0xFFFFFFFF; u_[:] = 0xFFFFFFFF; v_[:] = 0xFFFFFFFF
+                hs.append(h)
+            hh = []
+            for j in range(2):
+                h = c_void_p()
+                ptrs = (ctypes.c_void_p * 2)(Xs[2 * j], Xs[2 * j + 1])
+                u_, v_ = ch(95 + j, k - 1), ch(97 + j, k)
+                hip.call("zk_hadamard_prove_begin", ctypes.byref(h), ptrs, c_int(2), u_, v_, c_size_t(D), None)
+                u_[:] = 0xFFFFFFFF; v_[:] = 0xFFFFFFFF
+                hh.append(h)
+            out = []
+            for h in reversed(hh):
+                coefs = np.zeros((k * 3, 8), np.uint32)
+                hip.call("zk_hadamard_prove_end", h, coefs)
+                out.append(coefs)
+            for h in reversed(hs):
+                bm, sums = np.zeros(8, np.uint32), np.zeros((k * 11, 8), np.uint32)
+                hip.call("zk_lookup_prove_end", h, bm, sums)
+                out.append(bm)
+                out.append(sums)
+            if mode in res:
+                assert all((a == b).all() for a, b in zip(res[mode], out))
+            res[mode] = out
+    finally:
+        hip.call("zk_set_async_jobs", c_int(1))
+    assert len(res[0]) == len(res[1]) and all((a == b).all() for a, b in zip(res[0], res[1]))
+    assert all(a.any() for a in res[0])
+    for dS, dm, *_ in jobs:
+        hip.free(dS); hip.free(dm)
+    for p in Xs + [dT]:
+        hip.free(p)
+
+
 @pytest.mark.parametrize("k", [13, 17])
 def test_mapped_lookup_job_equals_the_plain_one_on_the_combined_queries(k):
     """zk_lookup_prove_begin_mapped forms S_in + r * S_out itself (2^13 queries: written out first; 2^17: inside the first

@@ -1815,6 +1815,11 @@ struct SumJob {
     hipEvent_t done = nullptr;   // ... and the event behind that copy
     const uint32_t* n_ok_dev = nullptr;      // lookup jobs over int32 forms: the consistent prefix of the table (HintSrc::n_ok) ...
     uint32_t n_table = 0;                    // ... and the table's size
+    // a job whose launches were handed to the library's launch thread: the ticket to wait for before anything of the job is
+    // read, and what that thread's attempt returned
+    uint64_t ticket = 0;
+    int queue_rc = 0;
+    std::string queue_err;
 };
 __global__ void __launch_bounds__(64) k_u32_set(uint32_t* __restrict__ p, uint32_t v) { if (threadIdx.x == 0) *p = v; }
 __global__ void __launch_bounds__(TPB) k_dot_part(Fr* __restrict__ partials, const Fr* __restrict__ a, const Fr* __restrict__ b, size_t n) {
@@ -2130,9 +2135,28 @@ static int sumjob_on_side_stream(SumJob& job, hipStream_t caller) {
     ZK_HIP(hipEventCreateWithFlags(&job.ready, hipEventDisableTiming));
     ZK_HIP(hipEventRecord(job.ready, caller));
     ZK_HIP(hipStreamWaitEvent(job.st, job.ready, 0));
+    pool_note_wait(caller, job.st);
     return 0;
 }
+// The job's launches: by the launch thread (the caller goes on at once; collecting the job waits for the ticket and reports
+// what `queue` returned), or here and now.  queue must not touch memory of the caller's that is only valid during the call.
+static int sumjob_launch(SumJob* job, std::function<int()> queue) {
+    if (!launcher_enabled()) return queue();
+    job->ticket = launcher_submit([job, queue] {
+        job->queue_rc = queue();
+        if (job->queue_rc) job->queue_err = last_error_text();
+    });
+    return 0;
+}
+// before anything of a job is read or released: its launches are on its stream; returns what queuing them returned
+static int sumjob_queued(SumJob* job) {
+    launcher_wait(job->ticket);
+    job->ticket = 0;
+    if (job->queue_rc) set_error(job->queue_rc, job->queue_err);
+    return job->queue_rc;
+}
 static void sumjob_abort(SumJob* job) {
+    launcher_wait(job->ticket);
     // the job's buffers go back to the allocator: wait for its last use (the whole stream when the job never got as far as its event)
     if (job->done) (void)hipEventSynchronize(job->done);
     else if (job->st) (void)hipStreamSynchronize(job->st);
@@ -2181,23 +2205,32 @@ static int lookup_prove_begin(void** handle, const void* S, const void* T, const
     SumJob* job = new SumJob;
     rc = sumjob_on_side_stream(*job, (hipStream_t)stv);
     if (rc) { sumjob_abort(job); return rc; }
+    // the caller's arrays are only valid during this call: the launches take copies
+    const Fr b = load_fr(beta);
+    const Fr r_val = r ? load_fr(r) : big_zero<8>();
+    const std::vector<uint32_t> u_own(u_eq, u_eq + 8 * (size_t)(rounds - 1)), v_own(v, v + 8 * (size_t)rounds);
+    const bool have_ints = ints != nullptr;
+    const LookupInts li = ints ? *ints : LookupInts();
+    rc = sumjob_launch(job, [=]() -> int {
+    int rc = 0;
+    const uint32_t *u_eq = u_own.data(), *v = v_own.data();
+    const LookupInts* ints = have_ints ? &li : nullptr;
     hipStream_t st = job->st;
     Scratch& B = job->arena.add(sizeof(Fr) * N);
     Scratch& dp = job->arena.add(sizeof(Fr) * (reduce_grid(N) + 1));
-    if (B.rc || dp.rc) { rc = B.rc ? B.rc : dp.rc; sumjob_abort(job); return rc; }
-    const Fr b = load_fr(beta);
+    if (B.rc || dp.rc) return B.rc ? B.rc : dp.rc;
     rc = batch_inv_queue(B.as<Fr>(), (const Fr*)T, b, N, job->arena, st);
     const Fr* Aptr = nullptr;
     HintSrc hs;
     if (rc == 0 && hint) {
         Scratch& TB = job->arena.add(sizeof(Fr) * 2 * N);
-        if (TB.rc) { rc = TB.rc; sumjob_abort(job); return rc; }
+        if (TB.rc) return TB.rc;
         hipLaunchKernelGGL(k_interleave, dim3(cdiv(N, TPB)), dim3(TPB), 0, st, TB.as<Fr>(), (const Fr*)T, B.as<Fr>(), N);
         hs.TB = TB.as<Fr>(); hs.hint = (const Fr*)hint; hs.low = fr_from_i64((int64_t)low); hs.beta = b; hs.N = (uint32_t)N;
-        if (S_out) { hs.S_out = (const Fr*)S_out; hs.r_mont = to_mont(load_fr(r)); }
+        if (S_out) { hs.S_out = (const Fr*)S_out; hs.r_mont = to_mont(r_val); }
         if (ints) {
             Scratch& want = job->arena.add(sizeof(int32_t) * (N + 1));         // the last slot: n_ok
-            if (want.rc) { rc = want.rc; sumjob_abort(job); return rc; }
+            if (want.rc) return want.rc;
             const int32_t* mi = S_out ? ((const FoldPrepared*)ints->mapped)->ints : nullptr;
             uint32_t* n_ok = (uint32_t*)(want.as<int32_t>() + N);
             // ZKLLM_LOOKUP_TRUSTED=0: no entry counts as checked and no output as gathered from the table -- every query goes
@@ -2223,15 +2256,17 @@ static int lookup_prove_begin(void** handle, const void* S, const void* T, const
         if (rc == 0) rc = batch_inv_queue(A.as<Fr>(), (const Fr*)S, b, D, job->arena, st);
         Aptr = A.as<Fr>();
     }
-    if (rc) { sumjob_abort(job); return rc; }
+    if (rc) return rc;
     const unsigned nb = reduce_grid(N);
     hipLaunchKernelGGL(k_dot_part, dim3(nb), dim3(TPB), 0, st, dp.as<Fr>() + 1, B.as<Fr>(), (const Fr*)m, N);
     hipLaunchKernelGGL(k_finish, dim3(1), dim3(TPB), 0, st, dp.as<Fr>(), dp.as<Fr>() + 1, nb);
     job->extra = dp.as<Fr>();
     rc = shared_eq_get(job->eq, u_eq, rounds - 1, job->arena, st);
-    if (rc) { sumjob_abort(job); return rc; }
+    if (rc) return rc;
     rc = lookup_queue(*job, Aptr, (const Fr*)S, B.as<Fr>(), (const Fr*)T, (const Fr*)m, (const Fr*)job->eq->p, b, v, D, N, rounds, hint ? &hs : nullptr);
     if (rc == 0) rc = sumjob_queue_results(*job);
+    return rc;
+    });
     if (rc) { sumjob_abort(job); return rc; }
     *handle = job;
     return 0;
@@ -2287,7 +2322,9 @@ int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host) {
     ZK_ARG(handle != nullptr, "zk_lookup_prove_end: null handle");
     SumJob* job = (SumJob*)handle;
     Fr bm = big_zero<8>();
-    int rc = sumjob_collect(*job, (Fr*)sums_host, &bm);
+    int rc = sumjob_queued(job);
+    if (rc) { sumjob_abort(job); return rc; }
+    rc = sumjob_collect(*job, (Fr*)sums_host, &bm);
     g_last_n_ok = g_last_n_table = 0;
     if (!rc && job->n_ok_dev) {          // the job's kernels have finished
         uint32_t v = 0;
@@ -2375,10 +2412,18 @@ int zk_hadamard_prove_begin_ints(void** handle, const void* const* Xs, const voi
     if (rc) { sumjob_abort(job); return rc; }
     int k = 0;
     while (((size_t)1 << k) < N) ++k;
-    rc = shared_eq_get(job->eq, u_eq, k - 1, job->arena, job->st);
-    if (rc) { sumjob_abort(job); return rc; }
-    rc = hadamard_queue(*job, (const Fr* const*)Xs, K, (const Fr*)job->eq->p, v, N, prepareds ? ints : nullptr);
-    if (rc == 0) rc = sumjob_queue_results(*job);
+    // the caller's arrays are only valid during this call: the launches take copies
+    const std::vector<uint32_t> u_own(u_eq, u_eq + 8 * (size_t)(k - 1)), v_own(v, v + 8 * (size_t)k);
+    const std::vector<const Fr*> xs_own((const Fr* const*)Xs, (const Fr* const*)Xs + K);
+    const std::vector<const int32_t*> ints_own(ints, ints + 4);
+    const bool have_ints = prepareds != nullptr;
+    rc = sumjob_launch(job, [=]() -> int {
+        int rc = shared_eq_get(job->eq, u_own.data(), k - 1, job->arena, job->st);
+        if (rc) return rc;
+        rc = hadamard_queue(*job, xs_own.data(), K, (const Fr*)job->eq->p, v_own.data(), N, have_ints ? ints_own.data() : nullptr);
+        if (rc == 0) rc = sumjob_queue_results(*job);
+        return rc;
+    });
     if (rc) { sumjob_abort(job); return rc; }
     *handle = job;
     return 0;
@@ -2386,7 +2431,9 @@ int zk_hadamard_prove_begin_ints(void** handle, const void* const* Xs, const voi
 int zk_hadamard_prove_end(void* handle, uint32_t* coefs_host) {
     ZK_ARG(handle != nullptr, "zk_hadamard_prove_end: null handle");
     SumJob* job = (SumJob*)handle;
-    int rc = sumjob_collect(*job, (Fr*)coefs_host, nullptr);
+    int rc = sumjob_queued(job);
+    if (rc) { sumjob_abort(job); return rc; }
+    rc = sumjob_collect(*job, (Fr*)coefs_host, nullptr);
     sumjob_abort(job);
     return rc;
 }

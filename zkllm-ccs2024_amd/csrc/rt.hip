@@ -1,7 +1,11 @@
 // Runtime pieces of the C ABI: device selection, the caching allocator, copies, error text.
 #include <cstdlib>
+#include <atomic>
+#include <condition_variable>
+#include <deque>
 #include <map>
 #include <mutex>
+#include <thread>
 #include <unordered_map>
 #include <utility>
 #include <vector>
@@ -82,6 +86,21 @@ static void order_behind_last_user(Pool& P, const Block& blk, hipStream_t stream
     covered = now;
 }
 
+void pool_note_wait(hipStream_t from, hipStream_t to) {
+    if (from == to || !is_persistent_stream(from) || !is_persistent_stream(to)) return;
+    Pool& P = pool();
+    std::lock_guard<std::mutex> lk(P.mu);
+    uint64_t& covered = P.synced[std::make_pair(from, to)];
+    if (covered < P.tick) covered = P.tick;
+}
+// whether `stream` can take the block without another wait (called with the pool locked)
+static bool needs_no_wait(Pool& P, const Block& b, hipStream_t stream) {
+    if (b.idle || b.last == stream) return true;
+    if (b.ev_set) return false;
+    auto it = P.synced.find(std::make_pair(b.last, stream));
+    return it != P.synced.end() && it->second != 0 && b.freed_tick <= it->second;
+}
+
 int pool_alloc(void** out, size_t bytes, hipStream_t stream, const hipStream_t* also) {
     Pool& P = pool();
     const size_t sz = round_size(bytes);
@@ -94,7 +113,7 @@ int pool_alloc(void** out, size_t bytes, hipStream_t stream, const hipStream_t* 
             size_t pick = fl.size() - 1;
             for (size_t k = 0; k < 8 && k < fl.size(); ++k) {
                 const Block& b = P.live[fl[fl.size() - 1 - k]];
-                if (b.idle || b.last == stream) { pick = fl.size() - 1 - k; break; }
+                if (needs_no_wait(P, b, stream)) { pick = fl.size() - 1 - k; break; }
             }
             void* p = fl[pick];
             fl[pick] = fl.back();
@@ -208,6 +227,81 @@ void pinned_release(void* host_ptr) {
     g_pinned_free.push_back(host_ptr);
 }
 
+std::string last_error_text() { return g_err; }
+
+namespace {
+struct Launcher {
+    std::mutex mu;
+    std::condition_variable work, finished;
+    std::deque<std::pair<uint64_t, std::pair<int, std::function<void()>>>> q;      // ticket, (device, closure)
+    uint64_t next = 1, done = 0;
+    bool stop = false, running = false;
+    std::thread th;
+    void loop() {
+        int cur_dev = -1;
+        std::unique_lock<std::mutex> lk(mu);
+        for (;;) {
+            work.wait(lk, [&] { return stop || !q.empty(); });
+            if (q.empty()) return;      // stop, and nothing left
+            auto item = std::move(q.front());
+            q.pop_front();
+            lk.unlock();
+            if (item.second.first != cur_dev) { (void)hipSetDevice(item.second.first); cur_dev = item.second.first; }
+            item.second.second();
+            lk.lock();
+            done = item.first;
+            finished.notify_all();
+        }
+    }
+};
+Launcher& launcher() { static Launcher* L = new Launcher; return *L; }      // never destroyed: its thread may outlive static destruction
+}  // namespace
+static std::atomic<int> g_async_jobs{-1};      // -1: not decided yet (the environment decides at the first question)
+bool launcher_enabled() {
+    int v = g_async_jobs.load();
+    if (v < 0) {
+        const char* e = getenv("ZKLLM_ASYNC_JOBS");
+        v = (e && e[0] == '0') ? 0 : 1;
+        g_async_jobs.store(v);
+    }
+    return v != 0;
+}
+void launcher_set_enabled(bool on) { g_async_jobs.store(on ? 1 : 0); }
+uint64_t launcher_submit(std::function<void()> fn) {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    Launcher& L = launcher();
+    std::lock_guard<std::mutex> lk(L.mu);
+    if (!L.running) {
+        L.stop = false;
+        L.th = std::thread([&L] { L.loop(); });
+        L.running = true;
+    }
+    const uint64_t t = L.next++;
+    L.q.emplace_back(t, std::make_pair(dev, std::move(fn)));
+    L.work.notify_one();
+    return t;
+}
+void launcher_wait(uint64_t ticket) {
+    if (!ticket) return;
+    Launcher& L = launcher();
+    std::unique_lock<std::mutex> lk(L.mu);
+    L.finished.wait(lk, [&] { return L.done >= ticket; });
+}
+void launcher_stop() {
+    Launcher& L = launcher();
+    std::thread th;
+    {
+        std::lock_guard<std::mutex> lk(L.mu);
+        if (!L.running) return;
+        L.stop = true;
+        L.work.notify_all();
+        th = std::move(L.th);
+        L.running = false;
+    }
+    th.join();          // the loop leaves once the queue is empty
+}
+
 int staging(void** host_ptr, size_t bytes) {
     static thread_local void* buf = nullptr;     // one per host thread, kept until the process ends
     static const size_t cap = 64 << 10;
@@ -258,6 +352,7 @@ int zk_pool_trim(void) { return pool_trim(); }
 // The library stays usable: streams and buffers are made again on demand.  For a host that wants nothing of this left to
 // static destruction at process exit.
 int zk_shutdown(void) {
+    launcher_stop();          // whatever was handed to the launch thread is on its streams before the device is waited for
     (void)hipDeviceSynchronize();
     {
         std::lock_guard<std::mutex> lk(shutdown_mu());
@@ -285,6 +380,8 @@ int zk_shutdown(void) {
     (void)hipGetLastError();
     return 0;
 }
+int zk_set_async_jobs(int on) { launcher_set_enabled(on != 0); return 0; }
+int zk_async_jobs(void) { return launcher_enabled() ? 1 : 0; }
 int zk_pool_stats(size_t* live_bytes, size_t* cached_bytes) {
     Pool& P = pool();
     std::lock_guard<std::mutex> lk(P.mu);

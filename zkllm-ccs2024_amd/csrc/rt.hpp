@@ -1,6 +1,7 @@
 // Internal runtime helpers shared by the .hip translation units: error capture, the caching
 // device allocator behind zk_malloc/zk_free, and a pinned staging area for small results.
 #pragma once
+#include <functional>
 #include <memory>
 #include <vector>
 #include <cstddef>
@@ -86,6 +87,22 @@ int fr_static_scratch_setup();
 // fn is called by zk_shutdown (device idle, before the cached blocks are given back): a file drops the events and cached
 // buffers it holds in static objects
 void at_shutdown(void (*fn)());
+
+// The allocator is told that `to` now waits for everything queued on `from` so far (the caller has just recorded an event on
+// `from` and made `to` wait for it): blocks that `from` let go before this call need no further wait when `to` takes them.
+void pool_note_wait(hipStream_t from, hipStream_t to);
+
+// The library's launch thread: closures run there one after the other, in the order of their submission, with the
+// submitting thread's device current.  A job that is a long sequence of launches on a stream of its own hands that sequence
+// over and returns to its caller at once; whoever collects the job waits for its ticket first.  Off with ZKLLM_ASYNC_JOBS=0
+// (launcher_enabled() is false then and the caller runs the closure itself).  Error text set inside a closure belongs to the
+// launch thread: a closure that can fail takes it along with last_error_text().
+bool launcher_enabled();
+void launcher_set_enabled(bool on);
+uint64_t launcher_submit(std::function<void()> fn);
+void launcher_wait(uint64_t ticket);      // 0: nothing to wait for
+void launcher_stop();                     // runs what is queued, then ends the thread (it starts again on demand)
+std::string last_error_text();
 
 static inline unsigned cdiv(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
 

@@ -548,8 +548,8 @@ void zkp_openings_use_row_commitments(int on) { zk_openings_use_row_commitments(
 void zkp_openings_set_only_at_claim(int on) { zk_openings_set_only_at_claim(on != 0); }
 int zkp_openings_only_at_claim() { return zk_openings_only_at_claim() ? 1 : 0; }
 // off: llama_layer finishes every block before it queues the next (ZKLLM_LAYER_OVERLAP=0)
-void zkp_layer_set_blocks_overlap(int on) { layer_set_blocks_overlap(on != 0); }
-int zkp_layer_blocks_overlap() { return layer_blocks_overlap() ? 1 : 0; }
+void zkp_layer_set_blocks_overlap(int depth) { layer_set_blocks_overlap(depth); }
+int zkp_layer_blocks_overlap() { return layer_blocks_overlap(); }
 double zkp_layer_setup_cross_ms() { return layer_setup_times().cross; }      // the cross commitments of the nine weights (prepare_weight_cross)
 // the nine commitments of the layer computed once more (ms); negative on error
 double zkp_layer_recommit_ms(void* h) {

@@ -1,9 +1,11 @@
 #include "layer.hpp"
 
+#include <cstdio>
 #include <cstdlib>
 
 #include <chrono>
 #include <cmath>
+#include <deque>
 #include <functional>
 #include <optional>
 #include <random>
@@ -501,12 +503,12 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
     return std::move(*b.down_out_);
 }
 
-static bool g_overlap_blocks = [] {
+static int g_overlap_blocks = [] {      // how many blocks may be begun and not yet finished when the next is begun
     const char* e = getenv("ZKLLM_LAYER_OVERLAP");
-    return !(e && e[0] == '0');
+    return e ? atoi(e) : 3;
 }();
-bool layer_blocks_overlap() { return g_overlap_blocks; }
-void layer_set_blocks_overlap(bool on) { g_overlap_blocks = on; }
+int layer_blocks_overlap() { return g_overlap_blocks; }
+void layer_set_blocks_overlap(int depth) { g_overlap_blocks = depth < 0 ? 0 : depth; }
 
 // The blocks in the order of the reference's executables.  A block's forward pass draws no challenge and records nothing, and
 // the device jobs of its proof need only that pass and the block's challenges; so, with overlap, the next block's forward pass
@@ -519,10 +521,11 @@ FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor
     // the nine weight openings run on the device beside the sumchecks; with a learned plan they start ahead of their claims
     // (not with ZKLLM_OPEN_AHEAD=0 / zk_openings_set_only_at_claim: then each starts at its claim)
     DeferredOpenings openings(c.open_weights ? w.plan.get() : nullptr, {&w.input_norm, &w.q, &w.k, &w.v, &w.o, &w.post_norm, &w.up, &w.gate, &w.down});
-    const bool overlap = g_overlap_blocks;
+    const int depth = g_overlap_blocks;
+    const bool overlap = depth > 0;
     const double t0 = now_ms();
-    // per-block times: with overlap, host clock from the end of the block before to the end of this block's finish() (the blocks
-    // share the device, so no other split exists); without, as before, with the caller's stream idle at both ends
+    // per-block times: with overlap, host clock from the end of the finish() before to the end of this block's finish() (the
+    // blocks share the device, so no other split exists); without, as before, with the caller's stream idle at both ends
     double mark = t0;
     auto lap = [&] {
         const double n = overlap ? std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now().time_since_epoch()).count() : now_ms();
@@ -530,42 +533,53 @@ FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor
         mark = n;
         return d;
     };
-    std::function<void()> owed;      // finish() of the block whose proofs are not collected yet
-    double* owed_slot = nullptr;
-    auto settle = [&] {
-        if (!owed) return;
-        auto f = std::move(owed);
-        owed = nullptr;
-        f();
-        *owed_slot += lap();
+    std::deque<std::pair<std::function<void()>, double*>> owed;      // finish() of the blocks whose proofs are not collected yet, oldest first
+    auto settle = [&](size_t leave) {
+        while (owed.size() > leave) {
+            auto f = std::move(owed.front());
+            owed.pop_front();
+            f.first();
+            *f.second += lap();
+        }
     };
+    int blocks_begun = 0;
+    static const int start_openings_behind = [] { const char* e = getenv("ZKLLM_OPEN_START_BLOCK"); return e ? atoi(e) : 1; }();
     auto begun = [&](std::function<void()> finish, double& slot) {      // call after the block's forward() and begin()
-        if (overlap) settle();
-        owed = std::move(finish);
-        owed_slot = &slot;
-        if (!overlap) settle();
+        owed.emplace_back(std::move(finish), &slot);
+        if (++blocks_begun == start_openings_behind) zk_openings_start_now();
+        settle((size_t)depth);
     };
 
+    static const bool trace = getenv("ZKLLM_LAYER_TRACE") != nullptr;      // host clock at every step, to stderr
+    auto host_ms = [] { return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now().time_since_epoch()).count(); };
+    auto note = [&](const char* what) { if (trace) fprintf(stderr, "layer %8.3f ms  %s\n", host_ms() - t0, what); };
+    note("start");
     FrTensor rms1 = compute_rms_inv(X, c.seq_len, c.embed_dim, c.rms_eps, c.value_scale);
     RmsNormBlock norm1(c, w.input_norm, X, rms1);
     const FrTensor& n1 = norm1.forward();
+    note("norm1 forward queued");
     norm1.begin();
-    begun([&] { norm1.finish(); }, t.rmsnorm1);
+    note("norm1 begun");
+    begun([&] { norm1.finish(); note("norm1 finished"); }, t.rmsnorm1);
 
     AttnLinearBlock qkv(c, w.q, w.k, w.v, n1);
     qkv.forward();
+    note("qkv forward queued");
     qkv.begin();
-    begun([&] { qkv.finish(); }, t.qkv);
+    note("qkv begun");
+    begun([&] { qkv.finish(); note("qkv finished"); }, t.qkv);
 
     std::optional<AttnStackBlock> stack;
     std::optional<FrTensor> attn_loop;          // the other variants prove inside their forward passes: nothing may be owed then
     if (c.attn_head_group == c.num_heads) {
         stack.emplace(c, *qkv.Q_, *qkv.K_, *qkv.V_);
         stack->forward();
+        note("attention forward queued");
         stack->begin();
-        begun([&] { stack->finish(); }, t.attention);
+        note("attention begun");
+        begun([&] { stack->finish(); note("attention finished"); }, t.attention);
     } else {
-        settle();
+        settle(0);
         attn_loop.emplace(attn_heads_block(c, *qkv.Q_, *qkv.K_, *qkv.V_));
         t.attention += lap();
     }
@@ -574,24 +588,31 @@ FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor
     OProjBlock oproj(c, w.o, attn);
     const FrTensor& o = oproj.forward();
     FrTensor x2 = X + o;                                   // skip-connection.cu:15-18
+    note("oproj forward queued");
     oproj.begin();
-    begun([&] { oproj.finish(); }, t.oproj);
+    note("oproj begun");
+    begun([&] { oproj.finish(); note("oproj finished"); }, t.oproj);
 
     FrTensor rms2 = compute_rms_inv(x2, c.seq_len, c.embed_dim, c.rms_eps, c.value_scale);
     RmsNormBlock norm2(c, w.post_norm, x2, rms2);
     const FrTensor& n2 = norm2.forward();
+    note("norm2 forward queued");
     norm2.begin();
-    begun([&] { norm2.finish(); }, t.rmsnorm2);
+    note("norm2 begun");
+    begun([&] { norm2.finish(); note("norm2 finished"); }, t.rmsnorm2);
 
     FfnBlock ffn(c, w.up, w.gate, w.down, w.swiglu_table, n2);
     const FrTensor& f = ffn.forward();
     FrTensor out = x2 + f;
+    note("ffn forward queued");
     ffn.begin();
-    begun([&] { ffn.finish(); }, t.ffn);
-    settle();
+    note("ffn begun");
+    begun([&] { ffn.finish(); note("ffn finished"); }, t.ffn);
+    settle(0);
     const double t6 = now_ms();
     openings.finish();
     const double t7 = now_ms();
+    note("openings collected");
     t.open_wait = t7 - t6; t.total = t7 - t0;
     if (times) *times = t;
     return out;

@@ -167,8 +167,8 @@ FrTensor attn_reference_block(const LayerConfig& c, const FrTensor& Q, const FrT
 // Each block's forward() and begin() are queued before the finish() of the block before it, unless ZKLLM_LAYER_OVERLAP=0 /
 // layer_set_blocks_overlap(false): then block after block.  Same outputs, same transcript.  (With attn_head_group other than
 // num_heads the attention block proves inside its forward pass and nothing overlaps it.)
-bool layer_blocks_overlap();
-void layer_set_blocks_overlap(bool on);
+int layer_blocks_overlap();
+void layer_set_blocks_overlap(int depth);
 FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor& X, LayerTimes* times);
 
 // how long make_random_layer_weights last spent on each part of the setup (ms, device idle at both ends of every part):
