@@ -727,6 +727,63 @@ def test_range_table_padded_by_repeating_its_last_value_keeps_the_short_first_ro
         hip.free(q)
 
 
+@pytest.mark.parametrize("k,n", [(16, 1 << 16), (17, 70001), (19, (1 << 19) - 3)])
+def test_evaluations_that_never_build_the_points_eq_table_against_big_integers(k, n):
+    """From 2^16 positions on zk_fr_me_multi / zk_fr_me_multi_ints evaluate through the two half tables of the point (a lane
+    multiplies its elements by the high half's entry, sums unreduced, and multiplies by the low half's entry once): field
+    elements through 29-bit-limb sums, int32 forms through 32-bit ones.  Checked against sum_t X[t] eq(u, t) in Python integers
+    for full and ragged lengths, with the extreme values of both kinds of element present."""
+    import ctypes
+    from gpuhelp import Hip, c_void_p, c_size_t, c_int
+    hip = Hip()
+    rng = np.random.default_rng(k)
+    u = ch(300 + k, k)
+    ui = fr_ints(u)
+    E = [1]
+    for j in range(k):
+        E = [e * (1 - ui[j]) % R_MOD for e in E] + [e * ui[j] % R_MOD for e in E]
+    frs = [ch(310 + i, n) for i in range(3)]
+    frs[0][0] = fr_array([R_MOD - 1])[0]
+    frs[0][1] = fr_array([0])[0]
+    frs[1][n - 1] = fr_array([R_MOD - 1])[0]
+    ints = [rng.integers(-2 ** 31, 2 ** 31, n) for _ in range(5)]
+    ints[0][:4] = [-2 ** 31, 2 ** 31 - 1, 0, -1]
+    ints[1][:] = -2 ** 31                                  # every term at the largest magnitude
+    ints[2][:] = 2 ** 31 - 1
+    want_fr = [sum(int(x) * e for x, e in zip(fr_ints(f), E)) % R_MOD for f in frs]
+    want_int = [sum(int(x) * e for x, e in zip(v, E)) % R_MOD for v in ints]
+    d_fr = [hip.upload(f) for f in frs]
+    d_int = [hip.upload(fr_array([int(x) % R_MOD for x in v])) for v in ints]
+    hs = []
+    for d in d_int:
+        h = c_void_p()
+        hip.call("zk_fr_fold_prepare", ctypes.byref(h), c_void_p(d), c_size_t(n), None)
+        hs.append(h)
+    junk = hip.upload(ch(320, n))
+
+    def run(fr_idx, int_idx):
+        K = len(fr_idx) + len(int_idx)
+        ptrs = [c_void_p(d_fr[i]) for i in fr_idx] + [c_void_p(junk)] * len(int_idx)
+        preps = [c_void_p(None)] * len(fr_idx) + [hs[i] for i in int_idx]
+        got = np.zeros((K, 8), np.uint32)
+        hip.call("zk_fr_me_multi_ints", got, (c_void_p * K)(*ptrs), (c_void_p * K)(*preps), c_int(K), c_size_t(n), u, c_int(k), None)
+        exp = fr_array([want_fr[i] for i in fr_idx] + [want_int[i] for i in int_idx])
+        assert (got == exp).all(), (fr_idx, int_idx)
+
+    run([0, 1, 2], [0, 1, 2, 3, 4])       # one tensor of field elements with five forms, then two tensors of field elements
+    run([0, 1], [0, 1, 2])                # two and three in one pass
+    run([2], [4])
+    run([], [3])
+    run([], [0, 1, 2, 3, 4, 0])           # six forms in one pass
+    got = np.zeros((3, 8), np.uint32)
+    hip.call("zk_fr_me_multi", got, (c_void_p * 3)(*[c_void_p(d) for d in d_fr]), c_int(3), c_size_t(n), u, c_int(k), None)
+    assert (got == fr_array(want_fr)).all()
+    for h in hs:
+        hip.call("zk_fr_fold_prepared_free", h)
+    for d in d_fr + d_int + [junk]:
+        hip.free(d)
+
+
 def test_evaluations_of_eight_tensors_that_keep_only_their_int32_form():
     """zk_fr_me_multi_ints with eight int32 forms: every one is evaluated from that form (six, then two), never from the field
     elements passed beside it -- which hold other values here, as a tensor that keeps only its int32 form does."""

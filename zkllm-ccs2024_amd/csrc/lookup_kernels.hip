@@ -1282,6 +1282,11 @@ static int eq_table_queue(Fr* out, const uint32_t* u, int k, Arena& arena, hipSt
     return 0;
 }
 
+// The split evaluation (k_me_split) from this many challenges on; ZKLLM_ME_SPLIT=0 keeps every evaluation on the pass over
+// the full eq table (to compare: the results are the same).
+static constexpr int ME_SPLIT_MIN_K = 16;
+static bool me_split_on() { static const bool on = [] { const char* e = getenv("ZKLLM_ME_SPLIT"); return !(e && e[0] == '0'); }(); return on; }
+
 // ---- folds of a tensor of 32-bit integers by eq weights ------------------------------------------------------------------
 // A tensor whose elements are 32-bit signed integers (a weight: fixed-point values) folds from its int32 form: an eighth of
 // the bytes, and a product with an eq entry is eight limb products with no reduction.  The unreduced sum of a whole fold
@@ -1478,6 +1483,116 @@ template <int KF, int KI> __global__ void __launch_bounds__(TPB) k_me_mixed(Fr* 
     block_reduce_store<KF + KI>(out, partials);
 }
 
+// ---- multilinear evaluations without the point's full eq table --------------------------------------------------------------
+// eq(u, t) = lo[t mod 2^kl] * hi[t div 2^kl], so  sum_t X[t] eq(u, t) = sum_g lo[g] (sum_h X[h 2^kl + g] hi[h]).  A lane owns one
+// g (and one slice of the h range): every step it multiplies its element by hi[h], the SAME value for all lanes of the wave,
+// and adds the product to an unreduced sum -- an int32 element by eight limb products (ifold_mac), a field element by 81
+// limb products on 29-bit limbs (wide29_mac; a carry pass every fourth term) -- and it reduces and multiplies by lo[g] once, at
+// the end.  Against a pass over the full table (k_eq_outer writes it with one field product per entry, k_me_mixed reads it
+// and pays a second one per field element) a field element costs about a sixth of the instructions, an int32 element a
+// tenth, and the table's 64 bytes of traffic per position are gone.
+// Tables: lo and hi as k_eq_halves leaves them (Montgomery form), the negatives of hi, and both with the factor 2^261 on
+// 29-bit limbs (x 2^261 = 32 x R): the sum's reduction and the product with lo each take one 2^-261.
+struct MeSplitTabs { const Fr* lo_m; const Fr* hi_m; const Fr* hi_neg; const Fr29* lo29; const Fr29* hi29; int kl; uint32_t nhi, per_slice; };
+__global__ void __launch_bounds__(TPB) k_me_split_tabs(Fr* __restrict__ hi_neg, Fr29* __restrict__ lo29, Fr29* __restrict__ hi29, const Fr* __restrict__ lo_m,
+                                                       const Fr* __restrict__ hi_m, uint32_t nlo, uint32_t nhi) {
+    const uint32_t g = blockIdx.x * TPB + threadIdx.x;
+    if (g >= nlo + nhi) return;
+    Fr c32 = big_zero<8>();
+    c32.v[0] = 32;
+    c32 = to_mont(c32);
+    if (g < nlo) lo29[g] = fr29_repack(mont_mul(lo_m[g], c32));
+    else {
+        const Fr h = hi_m[g - nlo];
+        hi_neg[g - nlo] = neg(h);
+        hi29[g - nlo] = fr29_repack(mont_mul(h, c32));
+    }
+}
+template <int KF, int KI> __global__ void __launch_bounds__(TPB) k_me_split(Fr* __restrict__ partials, const Fr* __restrict__ XF, const Fr* __restrict__ XF2, const MeIntPtrs pi,
+                                                                            const MeSplitTabs tb, size_t n) {
+    const uint32_t gid = blockIdx.x * TPB + threadIdx.x;
+    const uint32_t g = gid & ((1u << tb.kl) - 1u), slice = gid >> tb.kl;
+    const uint32_t h0 = slice * tb.per_slice, h1 = h0 + tb.per_slice < tb.nhi ? h0 + tb.per_slice : tb.nhi;
+    Wide29 w[KF > 0 ? KF : 1];
+    uint32_t acc[KI > 0 ? KI : 1][10];
+#pragma unroll
+    for (int k = 0; k < KF; ++k) w[k] = wide29_zero();
+#pragma unroll
+    for (int k = 0; k < KI; ++k)
+#pragma unroll
+        for (int i = 0; i < 10; ++i) acc[k][i] = 0;
+    for (uint32_t h = h0; h < h1; ++h) {
+        const size_t t = ((size_t)h << tb.kl) + g;
+        if (t < n) {
+            if constexpr (KI > 0) {
+                const Fr e = tb.hi_m[h], ne = tb.hi_neg[h];
+                int32_t x[KI];
+#pragma unroll
+                for (int k = 0; k < KI; ++k) x[k] = pi.x[k][t];
+#pragma unroll
+                for (int k = 0; k < KI; ++k) ifold_mac(acc[k], e, ne, x[k]);
+            }
+            if constexpr (KF > 0) {
+                const Fr29 e29 = tb.hi29[h];
+                wide29_mac(w[0], fr29_repack(XF[t]), e29);
+                if constexpr (KF == 2) wide29_mac(w[1], fr29_repack(XF2[t]), e29);
+            }
+        }
+        if constexpr (KF > 0) {
+            if (((h - h0) & 3u) == 3u) {
+#pragma unroll
+                for (int k = 0; k < KF; ++k) wide29_carry(w[k]);
+            }
+        }
+    }
+    Fr out[KF + KI];
+    if constexpr (KF > 0) {
+        const Fr29 l29 = tb.lo29[g];
+#pragma unroll
+        for (int k = 0; k < KF; ++k) out[k] = fr29_canon_pack(fr29_mul(wide29_redc(w[k]), l29));
+    }
+    if constexpr (KI > 0) {
+        const Fr l = tb.lo_m[g];
+#pragma unroll
+        for (int k = 0; k < KI; ++k) out[KF + k] = mont_mul(ifold_finish(acc[k]), l);
+    }
+    block_reduce_store<KF + KI>(out, partials);
+}
+// the tables of k_me_split for k challenges and n elements, queued on the stream (they live in the arena); blocks: its grid
+static int me_split_tabs_queue(MeSplitTabs& tb, unsigned& blocks, const uint32_t* u, int k, size_t n, Arena& arena, hipStream_t st) {
+    EqChallenges c;
+    Fr one = big_zero<8>();
+    one.v[0] = 1;
+    for (int j = 0; j < 30; ++j) {
+        const Fr uj = j < k ? load_fr(u + 8 * j) : big_zero<8>();
+        c.u[j] = to_mont(uj);
+        c.omu[j] = to_mont(sub(one, uj));
+    }
+    const int kl = (k + 1) / 2, kh = k - kl;
+    const uint32_t nlo = 1u << kl, nhi_full = 1u << kh;
+    Scratch& half = arena.add(sizeof(Fr) * ((size_t)nlo + 2 * (size_t)nhi_full));
+    Scratch& t29 = arena.add(sizeof(Fr29) * ((size_t)nlo + nhi_full));
+    if (half.rc) return half.rc;
+    if (t29.rc) return t29.rc;
+    Fr* lo = half.as<Fr>();
+    Fr* hi = lo + nlo;
+    Fr* hi_neg = hi + nhi_full;
+    Fr29* lo29 = t29.as<Fr29>();
+    Fr29* hi29 = lo29 + nlo;
+    hipLaunchKernelGGL(k_eq_halves, dim3(cdiv((size_t)nlo + nhi_full, TPB)), dim3(TPB), 0, st, lo, hi, c, kl, kh);
+    hipLaunchKernelGGL(k_me_split_tabs, dim3(cdiv((size_t)nlo + nhi_full, TPB)), dim3(TPB), 0, st, hi_neg, lo29, hi29, lo, hi, nlo, nhi_full);
+    ZK_LAUNCH_CHECK();
+    const uint32_t nhi = (uint32_t)((n + nlo - 1) / nlo);          // rows that hold elements
+    // slices of the h range: at most 1024 terms in a lane's unreduced sums, and 2^17 lanes where the tensor is large enough
+    uint32_t S = 1;
+    while ((nhi + S - 1) / S > 1024 || ((size_t)nlo * S < ((size_t)1 << 17) && S < nhi)) S <<= 1;
+    tb.lo_m = lo; tb.hi_m = hi; tb.hi_neg = hi_neg; tb.lo29 = lo29; tb.hi29 = hi29;
+    tb.kl = kl; tb.nhi = nhi; tb.per_slice = (nhi + S - 1) / S;
+    blocks = (unsigned)(((size_t)nlo * S) / TPB);
+    return 0;
+}
+
+
 extern "C" {
 
 int zk_lookup_index_fr(void* idx_u32, const void* vals, int32_t low, uint32_t table_size, size_t n, void* stv) {
@@ -1639,11 +1754,19 @@ int zk_fr_me_multi_ints(uint32_t* out_host, const void* const* Xs, const void* c
     }
     if (n_ints == 0) return zk_fr_me_multi(out_host, Xs, K, n, u, k, stv);
     Arena tmp(st);
-    Scratch& E = tmp.add(sizeof(Fr) * ((size_t)1 << k));
-    if (E.rc) return E.rc;
-    int rc = eq_table_queue(E.as<Fr>(), u, k, tmp, st);
+    const bool split = me_split_on() && k >= ME_SPLIT_MIN_K;
+    MeSplitTabs tb;
+    unsigned nb = reduce_grid(n);
+    Fr* Eptr = nullptr;
+    int rc = 0;
+    if (split) rc = me_split_tabs_queue(tb, nb, u, k, n, tmp, st);
+    else {
+        Scratch& E = tmp.add(sizeof(Fr) * ((size_t)1 << k));
+        if (E.rc) return E.rc;
+        rc = eq_table_queue(E.as<Fr>(), u, k, tmp, st);
+        Eptr = E.as<Fr>();
+    }
     if (rc) return rc;
-    const unsigned nb = reduce_grid(n);
     Scratch& part = tmp.add(sizeof(Fr) * 8 * nb);
     if (part.rc) return part.rc;
     int fr_done = 0;
@@ -1654,7 +1777,11 @@ int zk_fr_me_multi_ints(uint32_t* out_host, const void* const* Xs, const void* c
         for (int i = 0; i < 6; ++i) pi.x[i] = ((const FoldPrepared*)prepareds[ints_at[i0 + (i < ni ? i : 0)]])->ints;
         const Fr* XF = KF ? (const Fr*)Xs[fr_at[0]] : nullptr;
         const Fr* XF2 = KF == 2 ? (const Fr*)Xs[fr_at[1]] : nullptr;
-#define MEI_CASE(F, I) if (KF == F && ni == I) hipLaunchKernelGGL((k_me_mixed<F, I>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), XF, XF2, pi, E.as<Fr>(), n);
+#define MEI_CASE(F, I)                                                                                                                      \
+    if (KF == F && ni == I) {                                                                                                               \
+        if (split) hipLaunchKernelGGL((k_me_split<F, I>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), XF, XF2, pi, tb, n);                 \
+        else hipLaunchKernelGGL((k_me_mixed<F, I>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), XF, XF2, pi, Eptr, n);                      \
+    }
         MEI_CASE(0, 1) MEI_CASE(0, 2) MEI_CASE(0, 3) MEI_CASE(0, 4) MEI_CASE(0, 5) MEI_CASE(0, 6)
         MEI_CASE(1, 1) MEI_CASE(1, 2) MEI_CASE(1, 3) MEI_CASE(1, 4) MEI_CASE(1, 5) MEI_CASE(1, 6)
         MEI_CASE(2, 1) MEI_CASE(2, 2) MEI_CASE(2, 3)
@@ -1704,6 +1831,26 @@ int zk_fr_me_multi(uint32_t* out_host, const void* const* Xs, int K, size_t n, c
     ZK_ARG(K >= 1 && K <= 8, "zk_fr_me_multi: 1..8 tensors");
     ZK_ARG(k >= 0 && k <= 30 && n >= 1 && n <= ((size_t)1 << k) && (k == 0 || n > ((size_t)1 << (k - 1))), "zk_fr_me_multi: n does not match the number of challenges");
     Arena tmp(st);
+    if (me_split_on() && k >= ME_SPLIT_MIN_K) {          // two tensors a pass, no eq table of the whole point
+        MeSplitTabs tb;
+        unsigned nb = 0;
+        int rc = me_split_tabs_queue(tb, nb, u, k, n, tmp, st);
+        if (rc) return rc;
+        Scratch& part = tmp.add(sizeof(Fr) * 2 * nb);
+        if (part.rc) return part.rc;
+        const MeIntPtrs none = {};
+        for (int i = 0; i < K; i += 2) {
+            const int kf = K - i >= 2 ? 2 : 1;
+            if (kf == 2) hipLaunchKernelGGL((k_me_split<2, 0>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), (const Fr*)Xs[i], (const Fr*)Xs[i + 1], none, tb, n);
+            else hipLaunchKernelGGL((k_me_split<1, 0>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), (const Fr*)Xs[i], (const Fr*)nullptr, none, tb, n);
+            ZK_LAUNCH_CHECK();
+            Fr s2[2];
+            rc = finish_sums(part.as<Fr>(), nb, kf, 0, s2, st);
+            if (rc) return rc;
+            memcpy(out_host + 8 * i, s2, sizeof(Fr) * kf);
+        }
+        return 0;
+    }
     Scratch& E = tmp.add(sizeof(Fr) * ((size_t)1 << k));
     if (E.rc) return E.rc;
     int rc = eq_table_queue(E.as<Fr>(), u, k, tmp, st);

@@ -200,7 +200,11 @@ hipStream_t side_stream(int pool) {
     const int q = (pool && !shared) ? 1 : 0;
     const unsigned i = next[q]++ % (unsigned)count[q];
     hipStream_t& s = g_side_streams[q][i];
-    if (!s && hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) { (void)hipGetLastError(); s = nullptr; return nullptr; }
+    // ZKLLM_SIDE_STREAMS_BLOCKING=1 (measurement only): streams that the default stream waits for and that wait for it; with
+    // ZKLLM_SIDE_STREAMS=1,1,1 and a caller on the default stream no two kernels of the library overlap, so a kernel trace
+    // shows what each costs alone
+    static const bool blocking = [] { const char* e = getenv("ZKLLM_SIDE_STREAMS_BLOCKING"); return e && e[0] == '1'; }();
+    if (!s && hipStreamCreateWithFlags(&s, blocking ? hipStreamDefault : hipStreamNonBlocking) != hipSuccess) { (void)hipGetLastError(); s = nullptr; return nullptr; }
     return s;
 }
 
