@@ -147,7 +147,8 @@ int zk_fr_gather_ints(void* out, void* out_ints, const void* table, const void* 
  * out_prepared a handle of zk_fr_fold_prepared_new that receives out's int32 form (a query outside the table reads entry 0:
  * zk_lookup_index_i32, run before, reports those).  The handle remembers what it was gathered from: a mapped lookup job over
  * these queries, these outputs and this table (zk_lookup_prove_begin_mapped_ints) then knows that every output is its
- * query's table value and reads neither the outputs nor the per-entry integers in its first round. */
+ * query's table value and reads neither the outputs nor the per-entry integers in its first round.  out may be null: only the
+ * int32 form is written then (for outputs whose readers all take that form). */
 int zk_fr_gather_by_queries_ints(void* out, void* out_prepared, const void* queries_prepared, int32_t low, const void* table_prepared, size_t n, void* stream);
 /* zk_fr_me_multi where prepareds[i], when non-null, is the int32 form of Xs[i] (same n): such tensors are read from it --
  * an eighth of the bytes, eight limb products per element instead of a Montgomery product.  Same values. */
@@ -346,6 +347,10 @@ int zk_hadamard_prove_begin(void** handle, const void* const* Xs, int K, const u
 /* the same where prepareds[i], when non-null, is the int32 form of Xs[i] (N elements): two tensors that both have one (the
  * mapped outputs of a softmax's segments, zksoftmax.cu:177-180) are read from it in the first round; same sums */
 int zk_hadamard_prove_begin_ints(void** handle, const void* const* Xs, const void* const* prepareds, int K, const uint32_t* u_eq, const uint32_t* v, size_t N, void* stream);
+/* 1 when a job of zk_hadamard_prove_begin_ints over K tensors of N elements that all carry int32 forms reads nothing but those
+ * forms (K == 2 and a job long enough to have a first round of its own): the field elements passed beside them need not hold
+ * anything then.  No counterpart in the reference. */
+int zk_hadamard_ints_suffice(int K, size_t N);
 int zk_hadamard_prove_end(void* handle, uint32_t* coefs_host);
 
 /* ---- rescaling / softmax ------------------------------------------------------------------------------------------ */
@@ -366,7 +371,8 @@ int zk_softmax_decompose(void* const* planes, const void* X_shifted, const uint3
 /* the same, and int_planes[k] (int32, n each; null entries and a null array allowed) receive digit k once more as int32 */
 int zk_softmax_decompose_ints(void* const* planes, void* const* int_planes, const void* X_shifted, const uint32_t* bs_host, int K, size_t n, void* stream);
 /* zk_softmax_shift and zk_softmax_decompose_ints in one pass (zksoftmax.cu:124-140): the shifted scores are decomposed where
- * they are written, so they are not read again */
+ * they are written, so they are not read again.  out_shifted may be null (the shifted scores are not written), and so may
+ * planes[k] where int_planes[k] is given (digit k is written as int32 only). */
 int zk_softmax_shift_decompose(void* shift, void* out_shifted, void* const* planes, void* const* int_planes, const void* X, uint32_t rows, uint32_t cols, double scale,
                                const uint32_t* bs_host, int K, void* stream);
 

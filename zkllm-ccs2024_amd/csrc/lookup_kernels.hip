@@ -1178,7 +1178,7 @@ __device__ __forceinline__ void softmax_digits(const PlanePtrs& planes, const In
     if (mx.v[2] | mx.v[3] | mx.v[4] | mx.v[5] | mx.v[6] | mx.v[7]) {
         atomicOr(flag, 1u);
         for (int k = 0; k < K; ++k) {
-            planes.p[k][g] = big_zero<8>();
+            if (planes.p[k]) planes.p[k][g] = big_zero<8>();
             if (ints.p[k]) ints.p[k][g] = 0;
         }
         return;
@@ -1186,7 +1186,7 @@ __device__ __forceinline__ void softmax_digits(const PlanePtrs& planes, const In
     unsigned long long tmp = ((unsigned long long)mx.v[1] << 32) | mx.v[0];
     for (int k = 0; k < K; ++k) {
         const unsigned long long digit = tmp % bs.v[k];
-        planes.p[k][g] = fr_from_u64(digit);
+        if (planes.p[k]) planes.p[k][g] = fr_from_u64(digit);
         if (ints.p[k]) ints.p[k][g] = (int32_t)digit;
         tmp /= bs.v[k];
     }
@@ -1222,7 +1222,7 @@ __global__ void __launch_bounds__(TPB) k_softmax_shift(Fr* __restrict__ shift, F
     Fr* orow = out + (size_t)row * cols;
     for (uint32_t j = lane; j < cols; j += 64) {
         const Fr xs = sub(xr[j], sh);
-        orow[j] = xs;
+        if (out) orow[j] = xs;
         if (K > 0) softmax_digits(planes, ints, flag, xs, bs, K, (size_t)row * cols + j);
     }
 }
@@ -1449,7 +1449,7 @@ __global__ void __launch_bounds__(TPB) k_gather_by_queries(Fr* __restrict__ out,
     const int64_t d = (int64_t)queries[i] - (int64_t)low;
     const uint32_t j = (d >= 0 && d < (int64_t)N) ? (uint32_t)d : 0u;
     const int32_t v = table_ints[j];
-    out[i] = fr_from_i64((int64_t)v);
+    if (out) out[i] = fr_from_i64((int64_t)v);
     out_ints[i] = v;
 }
 // Multilinear evaluations at one point of KF (0 or 1) tensors of field elements and KI tensors given in int32 form, in one
@@ -1724,7 +1724,7 @@ int zk_fr_gather_ints(void* out, void* out_ints, const void* table, const void* 
 int zk_fr_gather_by_queries_ints(void* out, void* out_prepared, const void* queries_prepared, int32_t low, const void* table_prepared, size_t n, void* stv) {
     FoldPrepared* o = (FoldPrepared*)out_prepared;
     const FoldPrepared *q = (const FoldPrepared*)queries_prepared, *t = (const FoldPrepared*)table_prepared;
-    ZK_ARG(out != nullptr && o != nullptr && q != nullptr && t != nullptr, "zk_fr_gather_by_queries_ints: null argument");
+    ZK_ARG(o != nullptr && q != nullptr && t != nullptr, "zk_fr_gather_by_queries_ints: null argument");      // out may be null: only the int32 form is written
     ZK_ARG(o->n == n && q->n == n && t->n >= 1 && t->n <= 0xFFFFFFFFu, "zk_fr_gather_by_queries_ints: int32 forms of another size");
     LAUNCH1D(k_gather_by_queries, n, stv, (Fr*)out, o->ints, q->ints, low, t->ints, (uint32_t)t->n, n);
     o->src_queries = q->id;
@@ -2540,6 +2540,13 @@ int zk_hadamard_sumcheck(uint32_t* coefs_host, const void* const* Xs, int K, con
 }
 // The same beside the caller's stream, eq table of u_eq (log2(N) - 1 challenges) included.  Xs must stay alive and
 // unmodified until end; every handle must be ended exactly once.
+// 1 when a Hadamard job of K tensors of N elements that all carry int32 forms reads nothing but those forms
+int zk_hadamard_ints_suffice(int K, size_t N) {
+    if (K != 2 || N < 2 || (N & (N - 1))) return 0;
+    int rounds = 0;
+    while (((size_t)1 << rounds) < N) ++rounds;
+    return ((N >> 1) <= (size_t)TAIL_HALF && rounds <= TAIL_ROUNDS) ? 0 : 1;      // a job that is all tail reads the field elements
+}
 int zk_hadamard_prove_begin(void** handle, const void* const* Xs, int K, const uint32_t* u_eq, const uint32_t* v, size_t N, void* stv) {
     return zk_hadamard_prove_begin_ints(handle, Xs, nullptr, K, u_eq, v, N, stv);
 }
@@ -2681,7 +2688,7 @@ int zk_softmax_shift_decompose(void* shift, void* out_shifted, void* const* plan
     PlanePtrs pp;
     IntPlanePtrs ip;
     for (int i = 0; i < 8; ++i) { pp.p[i] = i < K ? (Fr*)planes[i] : nullptr; ip.p[i] = (int_planes && i < K) ? (int32_t*)int_planes[i] : nullptr; }
-    for (int i = 0; i < K; ++i) ZK_ARG(pp.p[i] != nullptr, "zk_softmax_decompose: null plane");
+    for (int i = 0; i < K; ++i) ZK_ARG(pp.p[i] != nullptr || ip.p[i] != nullptr, "zk_softmax_decompose: a digit with neither plane");
     for (int i = 0; i < K; ++i) ZK_ARG(!ip.p[i] || bs.v[i] <= 0x80000000u, "zk_softmax_decompose_ints: a radix above 2^31 has no int32 plane");
     Scratch flag(4, st);
     if (flag.rc) return flag.rc;

@@ -431,7 +431,7 @@ void* zkp_softmax(void* X, u32 m, u32 n, u32 d, const u32* bs, int K, u32 L, u32
     return new FrTensor(std::move(y));
     ZKP_END_PTR
 }
-// zkAttn (stacked = 0: one head, zkAttn::compute + zkAttn::prove) or zkAttnStacked over num heads (its compute + prove);
+// zkAttn (stacked = 0: one head, zkAttn::compute + zkAttn::prove) or zkAttnStacked over num heads (its compute + prove; stacked = 2: with lean_forward);
 // challenges from the seeded stream in the order of the prove function's parameters; returns out, final_claim the returned claim
 void* zkp_attn(void* Q, void* K, void* V, u32 num, u32 m, u32 n, u32 d, int stacked, const u32* bs, int nb, u32 L, u32 M, uint64_t sf_Q, uint64_t sf_K,
                const double* thetas, int nth, u32* final_claim) {
@@ -453,7 +453,8 @@ void* zkp_attn(void* Q, void* K, void* V, u32 num, u32 m, u32 n, u32 d, int stac
         return new FrTensor(std::move(out));
     }
     zkAttnStacked at(num, (unsigned long)sf_Q, (unsigned long)sf_K, bsv, L, M, th, m, n, d, 1);
-    FrTensor sm_in(num * m * n), sm_out(num * m * n), shift(num * m), xs(num * m * n);
+    at.lean_forward = stacked == 2;      // stacked == 2: digit planes and mapped values in their int32 forms only where the proof reads nothing else
+    FrTensor sm_in(num * m * n), sm_out(num * m * n), shift(num * m), xs(stacked == 2 ? 0 : num * m * n);
     FrTensor out = at.compute(FT(Q), FT(K), FT(V), sm_in, sm_out, shift, xs, xseg, yseg, mseg);
     auto c = at.draw();
     fin = at.prove(FT(Q), FT(K), FT(V), out, sm_out, sm_in, shift, xs, xseg, yseg, mseg, c.u_matmul_out_num, c.v_matmul_out_num, c.u_matmul_out, c.v_matmul_out,
@@ -462,6 +463,7 @@ void* zkp_attn(void* Q, void* K, void* V, u32 num, u32 m, u32 n, u32 d, int stac
     return new FrTensor(std::move(out));
     ZKP_END_PTR
 }
+int zkp_softmax_lean_tensors_last() { return (int)zkSoftmax::lean_tensors_last; }
 // zkFCStacked over num layers: X [num][batch][in], W [num][in][out], b [num][out] or null; forward per layer, then prove
 void* zkp_zkfc_stacked(void* X, void* W, void* b, u32 num, u32 batch, u32 in, u32 out) {
     ZKP_TRY

@@ -225,7 +225,9 @@ const FrTensor& AttnStackBlock::forward() {
     sm_out.emplace(H * seq * seq);
     shift.emplace(H * seq);
     {
-        FrTensor shifted(H * seq * seq);       // no proof reads it
+        // no proof reads the shifted scores, and of the digit planes and mapped values the proofs read the int32 forms
+        attn.lean_forward = true;
+        FrTensor shifted(0);
         out.emplace(attn.compute(*Qs, *Ks, *Vs, *sm_in, *sm_out, *shift, shifted, in_seg, out_seg, m_seg));
     }
     out_all.emplace(out->transpose_stack(H, seq, d).transpose(E, seq));   // [head][d][seq] = embed x seq -> seq x embed

@@ -66,7 +66,8 @@ pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const int* vals, const 
     ZKC(zk_sync(nullptr));
     return {std::move(y), std::move(m)};
 }
-pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const FrTensor& vals) {
+pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const FrTensor& vals) { return map(vals, false); }
+pair<FrTensor, FrTensor> tLookupRangeMapping::map(const FrTensor& vals, bool ints_only_out) {
     DevBuf idx(sizeof(uint) * (size_t)vals.size);
     index_of(idx.p, vals, low, len);
     FrTensor m = counts_to_m(idx.p, vals.size, table.size);
@@ -75,7 +76,7 @@ pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const FrTensor& vals) {
     if (const void* th = mapped_vals.kept_ints(); th && vals.kept_ints()) {
         // queries with an int32 form: gathered by them, and the outputs' form remembers it (the proof's first round then trusts them)
         y.ints_for_producer();
-        ZKC(zk_fr_gather_by_queries_ints(y.gpu_data, const_cast<void*>(y.kept_ints()), vals.kept_ints(), low, th, vals.size, nullptr));
+        ZKC(zk_fr_gather_by_queries_ints(ints_only_out ? nullptr : y.gpu_data, const_cast<void*>(y.kept_ints()), vals.kept_ints(), low, th, vals.size, nullptr));
     } else if (th) ZKC(zk_fr_gather_ints(y.gpu_data, y.ints_for_producer(), mapped_vals.gpu_data, th, idx.p, vals.size, nullptr));
     else ZKC(zk_fr_gather(y.gpu_data, mapped_vals.gpu_data, idx.p, vals.size, nullptr));
     ZKC(zk_sync(nullptr));

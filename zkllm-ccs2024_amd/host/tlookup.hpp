@@ -65,6 +65,10 @@ class tLookupRangeMapping : public tLookupRange {
 
     pair<FrTensor, FrTensor> operator()(const int* vals, const uint D);   // vals: device pointer
     pair<FrTensor, FrTensor> operator()(const FrTensor& vals);
+    // operator() that, with ints_only_out and where queries and mapped values keep int32 forms, writes the outputs in that form
+    // alone: their field elements stay unwritten.  For a caller whose every reader of the outputs takes the int32 form (the
+    // proof of a large lookup does: zk_lookup_ints_suffice; evaluations do; products of two such tensors do).
+    pair<FrTensor, FrTensor> map(const FrTensor& vals, bool ints_only_out);
 
     Fr_t prove(const FrTensor& S_in, const FrTensor& S_out, const FrTensor& m, const Fr_t& r, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u,
                const vector<Fr_t>& v, vector<Polynomial>& proof);

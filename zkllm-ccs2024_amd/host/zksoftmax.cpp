@@ -45,6 +45,7 @@ static void mul_segments(Fr_t* out, const FrTensor& a, const FrTensor& b, size_t
     if (a.kept_ints() && b.kept_ints()) ZKC(zk_fr_mul_ints(out, a.kept_ints(), b.kept_ints(), N, nullptr));
     else ZKC(zk_fr_mul(out, a.gpu_data, b.gpu_data, N, nullptr));
 }
+uint zkSoftmax::lean_tensors_last = 0;
 // zksoftmax.cu:112-173
 FrTensor zkSoftmax::compute(const FrTensor& X, FrTensor& shift, FrTensor& X_shifted, vector<FrTensor>& X_segments, vector<FrTensor>& Y_segments, vector<FrTensor>& m_segments) {
     return compute_rows(m, X, shift, X_shifted, X_segments, Y_segments, m_segments);
@@ -53,26 +54,39 @@ FrTensor zkSoftmax::compute_rows(uint m, const FrTensor& X, FrTensor& shift, FrT
                                  vector<FrTensor>& m_segments, FrTensor* into) {
     if ((size_t)X.size != (size_t)m * n) throw std::invalid_argument("X must be m * n");
     if (shift.size != m) throw std::invalid_argument("shift must be m");
-    if (X_shifted.size != X.size) throw std::invalid_argument("X_shifted must be the same size as X");
+    if (X_shifted.size != X.size && !(lean_forward && X_shifted.size == 0)) throw std::invalid_argument("X_shifted must be the same size as X");
 
     const double scale = static_cast<double>(scaling_factor_in) * std::sqrt(static_cast<double>(d));
 
     const size_t N = (size_t)m * n;
     X_segments.reserve(K);
     // every digit plane is written twice: as field elements and, an eighth of their bytes, as int32 -- the form the index
-    // pass of the lookups and the evaluations of the proof read
+    // pass of the lookups and the evaluations of the proof read.  With lean_forward a plane whose lookup proof reads the
+    // int32 form alone is written in that form only, and the mapped values of two such segments likewise when their product's
+    // proof reads nothing else: the field elements of those tensors stay unwritten (nothing in this class reads them).
     std::vector<void*> planes(K), int_planes(K, nullptr);
+    std::vector<char> ints_only(K, 0);
     for (uint i = 0; i < K; ++i) {
         X_segments.emplace_back((uint)N);
         planes[i] = X_segments[i].gpu_data;
         if (bs[i] <= 0x80000000u) int_planes[i] = X_segments[i].ints_for_producer();
+        const FrTensor& table = i < L ? least_significant_segments[i].table : other_segments[i - L].table;
+        const bool mapped_has_ints = i < L || other_segments[i - L].mapped_vals.kept_ints();
+        // a power of two (no padded copies on the way to the proof), and a lookup job of that size reads int32 forms alone
+        ints_only[i] = lean_forward && int_planes[i] && mapped_has_ints && N == ((size_t)1 << ceilLog2((uint)N)) && zk_lookup_ints_suffice(N, table.size);
+        if (ints_only[i]) planes[i] = nullptr;
     }
     // shift and digits in one pass: the shifted scores are decomposed where they are written
-    ZKC(zk_softmax_shift_decompose(shift.gpu_data, X_shifted.gpu_data, planes.data(), int_planes.data(), X.gpu_data, m, n, scale, bs.data(), (int)K, nullptr));
+    ZKC(zk_softmax_shift_decompose(shift.gpu_data, X_shifted.size ? X_shifted.gpu_data : nullptr, planes.data(), int_planes.data(), X.gpu_data, m, n, scale, bs.data(), (int)K,
+                                   nullptr));
 
+    bool lean_out = lean_forward && K - L == 2 && zk_hadamard_ints_suffice(2, N);
+    for (uint i = L; i < K; ++i) lean_out = lean_out && ints_only[i];
+    lean_tensors_last = lean_out ? K - L : 0;
+    for (uint i = 0; i < K; ++i) lean_tensors_last += ints_only[i] ? 1 : 0;
     for (uint i = 0; i < L; ++i) m_segments.push_back(least_significant_segments[i].prep(X_segments[i]));
     for (uint i = L; i < K; ++i) {
-        auto p = other_segments[i - L](X_segments[i]);
+        auto p = other_segments[i - L].map(X_segments[i], lean_out);
         Y_segments.push_back(std::move(p.first));
         m_segments.push_back(std::move(p.second));
     }
@@ -232,7 +246,8 @@ FrTensor zkAttnStacked::compute(const FrTensor& Q, const FrTensor& K, const FrTe
     if ((size_t)Q.size != (size_t)num * m * d) throw std::invalid_argument("Q must be m * d");
     if ((size_t)K.size != (size_t)num * n * d) throw std::invalid_argument("K must be n * d");
     if ((size_t)V.size != (size_t)num * n * d) throw std::invalid_argument("V must be n * d");
-    if ((size_t)sm_in.size != (size_t)num * m * n || sm_out.size != sm_in.size || sm_in_shifted.size != sm_in.size || sm_shift.size != num * m)
+    if ((size_t)sm_in.size != (size_t)num * m * n || sm_out.size != sm_in.size || (sm_in_shifted.size != sm_in.size && !(lean_forward && sm_in_shifted.size == 0)) ||
+        sm_shift.size != num * m)
         throw std::invalid_argument("softmax tensors must be num * m * n (shift: num * m)");
     FrTensor::matmul_stack_into(sm_in, Q, K.transpose_stack(num, n, d), num, m, d, n);
     compute_rows(num * m, sm_in, sm_shift, sm_in_shifted, sm_in_segments, sm_out_segments, sm_m_segments, &sm_out);
