@@ -507,7 +507,7 @@ FrTensor ffn_block(const LayerConfig& c, const Weight& up, const Weight& gate, c
 
 static int g_overlap_blocks = [] {      // how many blocks may be begun and not yet finished when the next is begun
     const char* e = getenv("ZKLLM_LAYER_OVERLAP");
-    return e ? atoi(e) : 3;
+    return e ? atoi(e) : 2;
 }();
 int layer_blocks_overlap() { return g_overlap_blocks; }
 void layer_set_blocks_overlap(int depth) { g_overlap_blocks = depth < 0 ? 0 : depth; }

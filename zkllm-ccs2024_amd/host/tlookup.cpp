@@ -66,12 +66,13 @@ pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const int* vals, const 
     ZKC(zk_sync(nullptr));
     return {std::move(y), std::move(m)};
 }
-pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const FrTensor& vals) { return map(vals, false); }
-pair<FrTensor, FrTensor> tLookupRangeMapping::map(const FrTensor& vals, bool ints_only_out) {
+pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const FrTensor& vals) { return map(vals, nullptr); }
+pair<FrTensor, FrTensor> tLookupRangeMapping::map(const FrTensor& vals, const FrTensor* unwritten) {
     DevBuf idx(sizeof(uint) * (size_t)vals.size);
     index_of(idx.p, vals, low, len);
     FrTensor m = counts_to_m(idx.p, vals.size, table.size);
-    FrTensor y(vals.size);
+    const bool ints_only_out = unwritten && unwritten->size == vals.size && mapped_vals.kept_ints() && vals.kept_ints();
+    FrTensor y = ints_only_out ? FrTensor::view(*unwritten) : FrTensor(vals.size);
     // mapped values that are 32-bit integers: the outputs get their int32 form with them
     if (const void* th = mapped_vals.kept_ints(); th && vals.kept_ints()) {
         // queries with an int32 form: gathered by them, and the outputs' form remembers it (the proof's first round then trusts them)

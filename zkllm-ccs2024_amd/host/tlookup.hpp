@@ -65,10 +65,11 @@ class tLookupRangeMapping : public tLookupRange {
 
     pair<FrTensor, FrTensor> operator()(const int* vals, const uint D);   // vals: device pointer
     pair<FrTensor, FrTensor> operator()(const FrTensor& vals);
-    // operator() that, with ints_only_out and where queries and mapped values keep int32 forms, writes the outputs in that form
-    // alone: their field elements stay unwritten.  For a caller whose every reader of the outputs takes the int32 form (the
-    // proof of a large lookup does: zk_lookup_ints_suffice; evaluations do; products of two such tensors do).
-    pair<FrTensor, FrTensor> map(const FrTensor& vals, bool ints_only_out);
+    // operator() that, given `unwritten` (a tensor of vals' size that nothing writes) and where queries and mapped values keep
+    // int32 forms, writes the outputs in that form alone: the returned tensor is a view of `unwritten` (which must outlive
+    // it) with an int32 form of its own.  For a caller whose every reader of the outputs takes the int32 form (the proof of a
+    // large lookup does: zk_lookup_ints_suffice; evaluations do; products of two such tensors do).
+    pair<FrTensor, FrTensor> map(const FrTensor& vals, const FrTensor* unwritten);
 
     Fr_t prove(const FrTensor& S_in, const FrTensor& S_out, const FrTensor& m, const Fr_t& r, const Fr_t& alpha, const Fr_t& beta, const vector<Fr_t>& u,
                const vector<Fr_t>& v, vector<Polynomial>& proof);

@@ -67,14 +67,17 @@ FrTensor zkSoftmax::compute_rows(uint m, const FrTensor& X, FrTensor& shift, FrT
     std::vector<void*> planes(K), int_planes(K, nullptr);
     std::vector<char> ints_only(K, 0);
     for (uint i = 0; i < K; ++i) {
-        X_segments.emplace_back((uint)N);
-        planes[i] = X_segments[i].gpu_data;
-        if (bs[i] <= 0x80000000u) int_planes[i] = X_segments[i].ints_for_producer();
         const FrTensor& table = i < L ? least_significant_segments[i].table : other_segments[i - L].table;
         const bool mapped_has_ints = i < L || other_segments[i - L].mapped_vals.kept_ints();
         // a power of two (no padded copies on the way to the proof), and a lookup job of that size reads int32 forms alone
-        ints_only[i] = lean_forward && int_planes[i] && mapped_has_ints && N == ((size_t)1 << ceilLog2((uint)N)) && zk_lookup_ints_suffice(N, table.size);
-        if (ints_only[i]) planes[i] = nullptr;
+        ints_only[i] = lean_forward && bs[i] <= 0x80000000u && mapped_has_ints && N == ((size_t)1 << ceilLog2((uint)N)) && zk_lookup_ints_suffice(N, table.size);
+        if (ints_only[i]) {
+            // the tensors that stay unwritten share one buffer that nothing writes (each is a view of it with an int32 form of its own)
+            if (!unwritten || unwritten->size != N) unwritten = std::make_shared<FrTensor>((uint)N);
+            X_segments.push_back(FrTensor::view(*unwritten));
+        } else X_segments.emplace_back((uint)N);
+        planes[i] = ints_only[i] ? nullptr : X_segments[i].gpu_data;
+        if (bs[i] <= 0x80000000u) int_planes[i] = X_segments[i].ints_for_producer();
     }
     // shift and digits in one pass: the shifted scores are decomposed where they are written
     ZKC(zk_softmax_shift_decompose(shift.gpu_data, X_shifted.size ? X_shifted.gpu_data : nullptr, planes.data(), int_planes.data(), X.gpu_data, m, n, scale, bs.data(), (int)K,
@@ -86,7 +89,7 @@ FrTensor zkSoftmax::compute_rows(uint m, const FrTensor& X, FrTensor& shift, FrT
     for (uint i = 0; i < K; ++i) lean_tensors_last += ints_only[i] ? 1 : 0;
     for (uint i = 0; i < L; ++i) m_segments.push_back(least_significant_segments[i].prep(X_segments[i]));
     for (uint i = L; i < K; ++i) {
-        auto p = other_segments[i - L].map(X_segments[i], lean_out);
+        auto p = other_segments[i - L].map(X_segments[i], lean_out ? unwritten.get() : nullptr);
         Y_segments.push_back(std::move(p.first));
         m_segments.push_back(std::move(p.second));
     }

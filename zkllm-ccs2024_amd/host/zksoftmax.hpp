@@ -1,5 +1,6 @@
 // Softmax by digit decomposition and exp lookup tables (zksoftmax.cuh:7-72), plus the attention wrappers.
 #pragma once
+#include <memory>
 #include "tlookup.hpp"
 #include "zkfc.hpp"
 
@@ -8,9 +9,10 @@ class zkSoftmax {
     // Addition.  compute() writes every digit plane and every mapped value as field elements and, where it fits, as int32 too.
     // With lean_forward set, a tensor among them whose every reader in prove() takes the int32 form (a lookup job large enough
     // to read nothing else, the evaluations, the product of two mapped segments) is written in that form ONLY: its field
-    // elements stay unwritten, and X_shifted may be passed with size 0 and is not written either.  For a caller that hands the
-    // tensors to prove() and reads none of them itself.
+    // elements stay unwritten (the tensor is a view of one buffer shared by all of them), and X_shifted may be passed with size 0
+    // and is not written either.  For a caller that hands the tensors to prove() and reads none of them itself.
     bool lean_forward = false;
+    std::shared_ptr<FrTensor> unwritten;      // the buffer those tensors are views of: it must outlive every use of them (it lives as long as this object)
     static uint lean_tensors_last;      // how many digit planes and mapped-value tensors the last compute() left in int32 form only
     zkSoftmax(const vector<uint>& bs, uint L, uint M, unsigned long scaling_factor_in, const vector<double>& thetas, uint m, uint n, uint d, uint E);
 
