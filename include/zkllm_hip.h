@@ -54,6 +54,18 @@ int zk_shutdown(void);
  * reported by its end call.  Jobs are launched in the order of their begin calls. */
 int zk_set_async_jobs(int on);
 int zk_async_jobs(void);
+/* No counterpart in the reference.  Deferred results: between zk_defer_begin and zk_defer_end (same host thread), the entry points
+ * that hand a few field elements back to the host -- zk_fr_me, zk_fr_me_multi(_ints), zk_ip_round, zk_ip_sumcheck_small -- queue
+ * their kernels and the copy of their results and return WITHOUT waiting and WITHOUT writing their host output arguments;
+ * zk_defer_end records an event on `stream` (the stream those calls were given) and zk_defer_wait waits for it and writes every
+ * result, in the order of the calls and with each call's own layout, to out_host (n_fr: how many field elements; at most 2048
+ * per batch).  For a caller that knows all its challenges and wants a chain of such calls queued in one go, e.g. the device
+ * side of a whole zkFC proof (zkfc.cu:61-87), and collects the values where the transcript needs them.  Other entry points are
+ * not affected.  zk_defer_free releases the batch (waiting for its copies first); one open batch per thread. */
+int zk_defer_begin(void** batch);
+int zk_defer_end(void* batch, void* stream);
+int zk_defer_wait(void* batch, uint32_t* out_host, size_t max_fr, size_t* n_fr);
+int zk_defer_free(void* batch);
 /* replace cudaMemcpy in ctors, operator()(idx), savebin/loadbin (ioutils.cu:3-45) */
 int zk_memcpy_h2d(void* dst, const void* src_host, size_t bytes, void* stream);
 int zk_memcpy_d2h(void* dst_host, const void* src, size_t bytes, void* stream);

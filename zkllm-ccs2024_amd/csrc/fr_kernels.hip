@@ -656,15 +656,11 @@ int zk_fr_me(uint32_t* out_host, const void* a, size_t n, const uint32_t* u, int
         for (int i = 0; i < 12; ++i) p.x[i] = (i < rest) ? to_mont(load_fr(u + 8 * (done + i))) : big_zero<8>();
         Scratch fin(sizeof(Fr), st);
         rc = fin.rc;
-        void* stage = nullptr;
-        if (!rc) rc = staging(&stage, sizeof(Fr));
         if (!rc) {
             hipLaunchKernelGGL(k_me_small, dim3(1), dim3(TPB), 0, st, fin.as<Fr>(), cur_ptr, p, (uint32_t)cur, (uint32_t)rest);
             hipError_t e = hipGetLastError();
-            if (e == hipSuccess) e = hipMemcpyAsync(stage, fin.p, sizeof(Fr), hipMemcpyDeviceToHost, st);
-            if (e == hipSuccess) e = hipStreamSynchronize(st);
             if (e != hipSuccess) rc = hip_fail(e, "zk_fr_me", __FILE__, __LINE__);
-            else memcpy(out_host, stage, 32);
+            else rc = deliver(st, fin.p, out_host, 1, 0);
         }
     }
     for (int i = 0; i < 2; ++i) if (bufs[i]) pool_free(bufs[i], st);
@@ -685,12 +681,11 @@ int zk_ip_round(uint32_t* poly3_host, const void* a, const void* b, size_t n_in,
     if (part.rc) return part.rc;
     hipLaunchKernelGGL(k_ip_round, dim3(nb), dim3(TPB), 0, (hipStream_t)stv, part.as<Fr>(), (const Fr*)a, (const Fr*)b, n_in, n_out);
     ZK_LAUNCH_CHECK();
-    Fr s[3];
-    int rc = finish_to_host<3>(part.as<Fr>(), nb, s, (hipStream_t)stv);
-    if (rc) return rc;
-    for (int i = 0; i < 3; ++i) s[i] = to_mont(s[i]);
-    memcpy(poly3_host, s, 96);
-    return 0;
+    Scratch fin(sizeof(Fr) * 3, (hipStream_t)stv);
+    if (fin.rc) return fin.rc;
+    hipLaunchKernelGGL(k_finish_sums, dim3(3), dim3(TPB), 0, (hipStream_t)stv, fin.as<Fr>(), part.as<Fr>(), nb);
+    ZK_LAUNCH_CHECK();
+    return deliver((hipStream_t)stv, fin.p, poly3_host, 3, 3);
 }
 
 // Stacked round over [N][D] tensors: rows_in = N, rows_out = 2^ceil(log2 N) / 2, E = eq table over the
@@ -727,13 +722,12 @@ int zk_ip_sumcheck_small(uint32_t* polys_host, uint32_t* fin_host, const void* a
     Fr* fin = polys + 3 * k;
     hipLaunchKernelGGL(k_ip_small, dim3(1), dim3(1024), 0, st, polys, fin, w, (const Fr*)a, (const Fr*)b, p, n, (uint32_t)k);
     ZK_LAUNCH_CHECK();
-    void* stage = nullptr;
-    int rc = staging(&stage, sizeof(Fr) * (3 * k + 2));
+    // one delivery of 3k + 2 values: the round polynomials, then the two fully folded values
+    Fr both[3 * 13 + 2];
+    int rc = deliver(st, polys, both, 3 * (size_t)k + 2, 0);
     if (rc) return rc;
-    ZK_HIP(hipMemcpyAsync(stage, polys, sizeof(Fr) * (3 * k + 2), hipMemcpyDeviceToHost, st));
-    ZK_HIP(hipStreamSynchronize(st));
-    memcpy(polys_host, stage, sizeof(Fr) * 3 * k);
-    memcpy(fin_host, (char*)stage + sizeof(Fr) * 3 * k, sizeof(Fr) * 2);
+    memcpy(polys_host, both, sizeof(Fr) * 3 * k);           // (while results are deferred these two are not what the kernel wrote: see zk_defer_begin)
+    memcpy(fin_host, both + 3 * k, sizeof(Fr) * 2);
     return 0;
 }
 

@@ -97,11 +97,8 @@ static int finish_sums(Fr* partials, unsigned nb, int K, int n_mont, Fr* host_ou
     if (fin.rc) return fin.rc;
     hipLaunchKernelGGL(k_finish, dim3(K), dim3(TPB), 0, st, fin.as<Fr>(), partials, nb);
     ZK_LAUNCH_CHECK();
-    ZK_HIP(hipMemcpyAsync(stage, fin.p, sizeof(Fr) * K, hipMemcpyDeviceToHost, st));
-    ZK_HIP(hipStreamSynchronize(st));
-    memcpy(host_out, stage, sizeof(Fr) * K);
-    for (int i = 0; i < n_mont; ++i) host_out[i] = to_mont(host_out[i]);
-    return 0;
+    (void)stage;
+    return deliver(st, fin.p, host_out, (size_t)K, n_mont);
 }
 
 // ---- table index / histogram ---------------------------------------------------------------------------------

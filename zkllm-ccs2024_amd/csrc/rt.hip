@@ -12,6 +12,7 @@
 #include <cstdio>
 #include <cstring>
 #include "rt.hpp"
+#include "field.hpp"
 #include "../../include/zkllm_hip.h"
 
 namespace zk {
@@ -234,6 +235,36 @@ void pinned_release(void* host_ptr) {
 std::string last_error_text() { return g_err; }
 
 namespace {
+struct DeferBatch {
+    void* pinned = nullptr;            // 64 KiB
+    size_t used = 0;                   // field elements delivered so far
+    std::vector<std::pair<size_t, int>> monts;      // (first element, count) to multiply by 2^256 on the way out
+    hipEvent_t ev = nullptr;
+    bool open = true;
+};
+thread_local DeferBatch* g_defer = nullptr;
+}  // namespace
+int deliver(hipStream_t st, const void* dev_src, void* host_dst, size_t count_fr, int n_mont) {
+    using Fr = Big<8>;
+    if (DeferBatch* b = g_defer) {
+        ZK_ARG((b->used + count_fr) * sizeof(Fr) <= ((size_t)64 << 10), "deferred results: more than 64 KiB in one batch");
+        ZK_HIP(hipMemcpyAsync((Fr*)b->pinned + b->used, dev_src, sizeof(Fr) * count_fr, hipMemcpyDeviceToHost, st));
+        if (n_mont > 0) b->monts.emplace_back(b->used, n_mont);
+        b->used += count_fr;
+        return 0;
+    }
+    void* stage = nullptr;
+    int rc = staging(&stage, sizeof(Fr) * count_fr);
+    if (rc) return rc;
+    ZK_HIP(hipMemcpyAsync(stage, dev_src, sizeof(Fr) * count_fr, hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipStreamSynchronize(st));
+    Fr* out = (Fr*)host_dst;
+    memcpy(out, stage, sizeof(Fr) * count_fr);
+    for (int i = 0; i < n_mont; ++i) out[i] = to_mont(out[i]);
+    return 0;
+}
+
+namespace {
 struct Launcher {
     std::mutex mu;
     std::condition_variable work, finished;
@@ -382,6 +413,48 @@ int zk_shutdown(void) {
         g_pinned_free.clear();
     }
     (void)hipGetLastError();
+    return 0;
+}
+int zk_defer_begin(void** batch) {
+    ZK_ARG(batch != nullptr, "zk_defer_begin: null argument");
+    ZK_ARG(g_defer == nullptr, "zk_defer_begin: this thread already has a batch open");
+    DeferBatch* b = new DeferBatch;
+    int rc = pinned_acquire(&b->pinned);
+    if (rc) { delete b; return rc; }
+    g_defer = b;
+    *batch = b;
+    return 0;
+}
+int zk_defer_end(void* batch, void* stream) {
+    DeferBatch* b = (DeferBatch*)batch;
+    ZK_ARG(b != nullptr && b == g_defer && b->open, "zk_defer_end: not this thread's open batch");
+    g_defer = nullptr;
+    b->open = false;
+    ZK_HIP(hipEventCreateWithFlags(&b->ev, hipEventDisableTiming));
+    ZK_HIP(hipEventRecord(b->ev, (hipStream_t)stream));
+    return 0;
+}
+int zk_defer_wait(void* batch, uint32_t* out_host, size_t max_fr, size_t* n_fr) {
+    using Fr = Big<8>;
+    DeferBatch* b = (DeferBatch*)batch;
+    ZK_ARG(b != nullptr && !b->open && b->ev != nullptr, "zk_defer_wait: the batch has not been ended");
+    ZK_ARG(b->used <= max_fr, "zk_defer_wait: more results than the buffer holds");
+    ZK_HIP(hipEventSynchronize(b->ev));
+    Fr* out = (Fr*)out_host;
+    memcpy(out, b->pinned, sizeof(Fr) * b->used);
+    for (auto& m : b->monts)
+        for (int i = 0; i < m.second; ++i) out[m.first + i] = to_mont(out[m.first + i]);
+    if (n_fr) *n_fr = b->used;
+    return 0;
+}
+int zk_defer_free(void* batch) {
+    DeferBatch* b = (DeferBatch*)batch;
+    if (!b) return 0;
+    if (b == g_defer) g_defer = nullptr;
+    if (b->ev) { (void)hipEventSynchronize(b->ev); (void)hipEventDestroy(b->ev); }      // the copies into the pinned buffer have landed
+    else if (b->used) (void)hipDeviceSynchronize();                                   // never ended: wait for whatever was queued
+    pinned_release(b->pinned);
+    delete b;
     return 0;
 }
 int zk_set_async_jobs(int on) { launcher_set_enabled(on != 0); return 0; }

@@ -80,6 +80,13 @@ void pinned_release(void* host_ptr);
 // Pinned host buffer (64 KiB, one per host thread) for device->host results of reductions.
 int staging(void** host_ptr, size_t bytes);
 
+// Small results of an entry point (a few field elements: sums, round polynomials) on their way to the host.
+// Normally: copied through the staging buffer, the stream waited for, host_dst filled; the first n_mont elements multiplied by
+// 2^256 mod r there (sums that left the device with a factor R^-1).  While the calling thread has a batch of deferred results
+// open (zk_defer_begin): the copy goes into the batch's pinned buffer behind what is queued on the stream, nothing is waited for,
+// host_dst is NOT written, and zk_defer_wait hands the values out later, in the order of the deliver calls.
+int deliver(hipStream_t st, const void* dev_src, void* host_dst, size_t count_fr, int n_mont);
+
 // Looks up, for the current device, the address of the device array behind zk_fr_sum_static (fr_kernels.hip); called
 // by zk_init so that the entry point itself has nothing left to set up.
 int fr_static_scratch_setup();

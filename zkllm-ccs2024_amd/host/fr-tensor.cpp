@@ -363,6 +363,37 @@ Fr_t FrTensor::operator()(const vector<Fr_t>& u) const {
     return out;
 }
 
+DeferredResults& DeferredResults::operator=(DeferredResults&& o) noexcept {
+    if (this != &o) {
+        if (batch) zk_defer_free(batch);
+        batch = o.batch; open = o.open;
+        o.batch = nullptr; o.open = false;
+    }
+    return *this;
+}
+DeferredResults::~DeferredResults() { if (batch) zk_defer_free(batch); }
+void DeferredResults::begin() {
+    if (batch) throw std::runtime_error("DeferredResults::begin: already begun");
+    ZKC(zk_defer_begin(&batch));
+    open = true;
+}
+void DeferredResults::end() {
+    if (!batch || !open) throw std::runtime_error("DeferredResults::end: nothing open");
+    open = false;
+    ZKC(zk_defer_end(batch, nullptr));
+}
+std::vector<Fr_t> DeferredResults::wait() {
+    if (!batch || open) throw std::runtime_error("DeferredResults::wait: not ended");
+    std::vector<Fr_t> out(2048);
+    size_t n = 0;
+    const int rc = zk_defer_wait(batch, out[0].val, out.size(), &n);
+    zk_defer_free(batch);
+    batch = nullptr;
+    zk_check(rc, "zk_defer_wait");
+    out.resize(n);
+    return out;
+}
+
 vector<Fr_t> FrTensor::me_batch(const vector<const FrTensor*>& ts, const vector<Fr_t>& u) {
     vector<Fr_t> out(ts.size());
     if (ts.empty()) return out;

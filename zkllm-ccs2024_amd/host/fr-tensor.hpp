@@ -190,6 +190,26 @@ class FrTensor {
     static FrTensor filled(uint size, const Fr_t& x);
 };
 
+// Results that arrive later (zk_defer_begin / _end / _wait of the C ABI).  Between begin() and end() the calling thread's
+// evaluations and inner-product rounds (FrTensor::operator()(u), multi_dim_me, zk_ip_round, zk_ip_sumcheck_small) only queue
+// their kernels: what they return is NOT their result.  wait() delivers the results of those calls in call order, each with
+// the layout of its C entry point.  For proofs whose challenges are all known up front: the device side is queued in one go,
+// the host side (checks, transcript entries) runs when the values are collected.
+struct DeferredResults {
+    DeferredResults() = default;
+    DeferredResults(DeferredResults&& o) noexcept : batch(o.batch), open(o.open) { o.batch = nullptr; o.open = false; }
+    DeferredResults& operator=(DeferredResults&& o) noexcept;
+    DeferredResults(const DeferredResults&) = delete;
+    DeferredResults& operator=(const DeferredResults&) = delete;
+    ~DeferredResults();
+    void begin();
+    void end();                        // on the default stream, where the class layer queues its work
+    std::vector<Fr_t> wait();          // also releases the batch
+    explicit operator bool() const { return batch != nullptr; }
+    void* batch = nullptr;
+    bool open = false;
+};
+
 ostream& operator<<(ostream& os, const FrTensor& A);
 FrTensor catTensors(const vector<FrTensor>& vec);
 

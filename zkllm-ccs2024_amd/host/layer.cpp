@@ -148,17 +148,21 @@ void AttnLinearBlock::begin() {
     pq = q_rescale.prove_begin(*Q, *Q_, ch_qr);      // three range proofs side by side
     pk = k_rescale.prove_begin(*K, *K_, ch_kr);
     pv = v_rescale.prove_begin(*V, *V_, ch_vr);
+    // the device side of the three matrix-product proofs, queued behind them: finish() only collects values
+    fk = k_layer.prove_begin(input, *K, ch_k);
+    fq = q_layer.prove_begin(input, *Q, ch_q);
+    fv = v_layer.prove_begin(input, *V, ch_v);
 }
 void AttnLinearBlock::finish() {
     q_rescale.prove_end(pq);
     k_rescale.prove_end(pk);
     v_rescale.prove_end(pv);
     OpeningGroup together;      // the three openings claimed below run as one device job, queued at the last claim
-    auto ck = k_layer.prove(input, *K, ch_k);
+    auto ck = k_layer.prove_end(fk);
     if (c.open_weights) verifyWeightClaim(k, ck[0]);
-    auto cq = q_layer.prove(input, *Q, ch_q);
+    auto cq = q_layer.prove_end(fq);
     if (c.open_weights) verifyWeightClaim(q, cq[0]);
-    auto cv = v_layer.prove(input, *V, ch_v);
+    auto cv = v_layer.prove_end(fv);
     if (c.open_weights) verifyWeightClaim(v, cv[0]);
     together.end();
     pq = Rescaling::Pending(); pk = Rescaling::Pending(); pv = Rescaling::Pending();
@@ -412,10 +416,11 @@ void OProjBlock::begin() {
     ch_r = Rescaling::draw(O->size);
     ch_o = o_layer.draw(attn_out.size / c.embed_dim);
     p = o_rescale.prove_begin(*O, *O_, ch_r);
+    fo = o_layer.prove_begin(attn_out, *O, ch_o);
 }
 void OProjBlock::finish() {
     o_rescale.prove_end(p);
-    auto co = o_layer.prove(attn_out, *O, ch_o);
+    auto co = o_layer.prove_end(fo);
     if (c.open_weights) verifyWeightClaim(o, co[0]);
     p = Rescaling::Pending();
     O.reset();
@@ -476,19 +481,23 @@ void FfnBlock::begin() {
     ps = swiglu.prove_begin(*gate_out_, *swiglu_out, *swiglu_m, temp_rand[0], temp_rand[1], temp_rand[2], swiglu_u, swiglu_v);
     pg = gate_rescale.prove_begin(*gate_out, *gate_out_, ch_gr);
     pu = up_rescale.prove_begin(*up_out, *up_out_, ch_ur);
+    // the device side of the three matrix-product proofs, queued behind them in the order finish() collects them
+    fd = down_layer.prove_begin(*down_in_, *down_out, ch_d);
+    fg = gate_layer.prove_begin(input, *gate_out, ch_g);
+    fu = up_layer.prove_begin(input, *up_out, ch_u);
 }
 void FfnBlock::finish() {
     down_rescale.prove_end(pd);
-    auto cd = down_layer.prove(*down_in_, *down_out, ch_d);
+    auto cd = down_layer.prove_end(fd);
     if (c.open_weights) verifyWeightClaim(down, cd[0], od);
     hidden_rescale.prove_end(ph);
     tLookup::prove_end(ps);
     gate_rescale.prove_end(pg);
     OpeningGroup gate_and_up;   // when nothing was started ahead: the two openings over the same generator count as one job, queued at up's claim
-    auto cg = gate_layer.prove(input, *gate_out, ch_g);
+    auto cg = gate_layer.prove_end(fg);
     if (c.open_weights) verifyWeightClaim(gate, cg[0], og);
     up_rescale.prove_end(pu);
-    auto cu = up_layer.prove(input, *up_out, ch_u);
+    auto cu = up_layer.prove_end(fu);
     if (c.open_weights) verifyWeightClaim(up, cu[0], ou);
     gate_and_up.end();
     pd = Rescaling::Pending(); ph = Rescaling::Pending(); pg = Rescaling::Pending(); pu = Rescaling::Pending(); ps = LookupPending();

@@ -102,6 +102,7 @@ struct AttnLinearBlock {
     Rescaling::Challenges ch_qr, ch_kr, ch_vr;
     zkFC::Challenges ch_q, ch_k, ch_v;
     Rescaling::Pending pq, pk, pv;
+    zkFC::Pending fq, fk, fv;
 };
 // attention with all heads as one stack (attn_head_group == num_heads) and the two rescalings of its output
 struct AttnStackBlock {
@@ -131,6 +132,7 @@ struct OProjBlock {
     Rescaling::Challenges ch_r;
     zkFC::Challenges ch_o;
     Rescaling::Pending p;
+    zkFC::Pending fo;
 };
 struct FfnBlock {
     FfnBlock(const LayerConfig& c, const Weight& up, const Weight& gate, const Weight& down, const FrTensor& swiglu_values, const FrTensor& input);
@@ -148,6 +150,7 @@ struct FfnBlock {
     WeightOpeningAhead od, og, ou;
     Rescaling::Pending pd, ph, pg, pu;
     LookupPending ps;
+    zkFC::Pending fd, fg, fu;
 };
 
 FrTensor rmsnorm_block(const LayerConfig& c, const Weight& w, const FrTensor& X, const FrTensor& rms_inv);

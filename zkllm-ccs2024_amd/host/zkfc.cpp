@@ -54,6 +54,12 @@ vector<Claim> zkFC::prove(const FrTensor& X, const FrTensor& Y) const {
 }
 vector<Claim> zkFC::prove(const FrTensor& X, const FrTensor& Y, const Challenges& ch) const {
     if (has_bias) throw std::runtime_error("Cleaned-up version not implemented for zkFC with bias. Use zkFCStacked instead.");
+    if (inputSize < 2) return prove_at_once(X, Y, ch);      // no inner-product rounds: nothing to queue ahead
+    Pending p = prove_begin(X, Y, ch);
+    return prove_end(p);
+}
+// the proof with every value fetched where it is used (zkfc.cu:61-87 as written)
+vector<Claim> zkFC::prove_at_once(const FrTensor& X, const FrTensor& Y, const Challenges& ch) const {
     uint batchSize = X.size / inputSize;
     const vector<Fr_t>&u_batch = ch.u_batch, &u_input = ch.u_input, &u_output = ch.u_output;
     if (u_batch.size() != ceilLog2(batchSize) || u_input.size() != ceilLog2(inputSize) || u_output.size() != ceilLog2(outputSize))
@@ -70,6 +76,85 @@ vector<Claim> zkFC::prove(const FrTensor& X, const FrTensor& Y, const Challenges
     // pass over the full tensors (zkfc.cu:77-78), so the large tensors are not streamed again.
     auto claim_X = X_reduced(u_input);
     auto claim_W = W_reduced(u_input);
+    zk_record(final_claim);
+    zk_record(claim_X);
+    zk_record(claim_W);
+    if (claim_X * claim_W != final_claim) throw std::runtime_error("Claim does not match");
+    vector<Claim> claims;
+    claims.push_back({claim_W, vector<vector<Fr_t>>({u_input, u_output}), vector<uint>({inputSize, outputSize})});
+    return claims;
+}
+zkFC::Pending zkFC::prove_begin(const FrTensor& X, const FrTensor& Y, const Challenges& ch) const {
+    if (has_bias) throw std::runtime_error("Cleaned-up version not implemented for zkFC with bias. Use zkFCStacked instead.");
+    if (inputSize < 2) throw std::runtime_error("zkFC::prove_begin: needs an input axis of at least two");
+    Pending p;
+    p.ch = ch;
+    p.batchSize = X.size / inputSize;
+    const vector<Fr_t>&u_batch = ch.u_batch, &u_input = ch.u_input, &u_output = ch.u_output;
+    if (u_batch.size() != ceilLog2(p.batchSize) || u_input.size() != ceilLog2(inputSize) || u_output.size() != ceilLog2(outputSize))
+        throw std::runtime_error("zkFC::prove: challenges do not match the shapes");
+    if (Y.size != p.batchSize * outputSize) throw std::runtime_error("zkFC::prove: Y does not match the shapes");
+    p.keep.reserve(2 * u_input.size() + 4);
+    p.results.begin();
+    try {
+        // result 0: Y at (u_batch, u_output)
+        (void)Y.multi_dim_me({u_batch, u_output}, {p.batchSize, outputSize});
+        p.keep.push_back(X.partial_me(u_batch, p.batchSize, inputSize));
+        p.keep.push_back(weights.partial_me(u_output, outputSize, 1));
+        const FrTensor* a = &p.keep[0];
+        const FrTensor* b = &p.keep[1];
+        if (a->size != b->size) throw std::runtime_error("a.size != b.size");
+        // the rounds of zkip (zkfc.cu:129-151): the most significant index bit first, challenges from the back of u_input
+        size_t k = u_input.size();
+        while (k > 0) {
+            const uint n_in = a->size;
+            const uint bits = ceilLog2(n_in);
+            if (bits != k) throw std::runtime_error("zkFC::prove_begin: the reduced vectors do not match the input challenges");
+            if (bits <= 13) {
+                Fr_t unused_polys[3 * 13], unused_fin[2];
+                ZKC(zk_ip_sumcheck_small(unused_polys[0].val, unused_fin[0].val, a->gpu_data, b->gpu_data, n_in, u_input[0].val, (int)k, nullptr));
+                p.small_rounds = (uint)k;
+                break;
+            }
+            const uint n_out = (1u << bits) >> 1;
+            Fr_t unused[3];
+            ZKC(zk_ip_round(unused[0].val, a->gpu_data, b->gpu_data, n_in, n_out, nullptr));
+            p.round_sizes.push_back(n_out);
+            p.keep.emplace_back(n_out);
+            p.keep.emplace_back(n_out);
+            FrTensor& na = p.keep[p.keep.size() - 2];
+            FrTensor& nb = p.keep[p.keep.size() - 1];
+            ZKC(zk_fr_fold_halves(na.gpu_data, a->gpu_data, u_input[k - 1].val, n_in, n_out, nullptr));
+            ZKC(zk_fr_fold_halves(nb.gpu_data, b->gpu_data, u_input[k - 1].val, n_in, n_out, nullptr));
+            a = &na;
+            b = &nb;
+            --k;
+        }
+        if (p.small_rounds == 0) throw std::runtime_error("zkFC::prove_begin: no rounds left for the closing kernel");
+    } catch (...) {
+        p.results.end();
+        throw;
+    }
+    p.results.end();
+    return p;
+}
+vector<Claim> zkFC::prove_end(Pending& p) const {
+    const vector<Fr_t>&u_input = p.ch.u_input, &u_output = p.ch.u_output;
+    const vector<Fr_t> r = p.results.wait();
+    p.keep.clear();
+    const size_t expect = 1 + 3 * p.round_sizes.size() + 3 * (size_t)p.small_rounds + 2;
+    if (r.size() != expect) throw std::runtime_error("zkFC::prove_end: unexpected number of results");
+    Fr_t claim = r[0];
+    zk_record(claim);
+    size_t at = 1, k = u_input.size();
+    for (size_t round = 0; round < p.round_sizes.size() + p.small_rounds; ++round) {
+        Polynomial poly({r[at], r[at + 1], r[at + 2]});
+        at += 3;
+        zk_record(poly.coefficients());
+        if (claim != poly(TEMP_ZERO) + poly(TEMP_ONE)) throw std::runtime_error("claim != p(0) + p(1)");
+        claim = poly(u_input[--k]);
+    }
+    const Fr_t final_claim = claim, claim_X = r[at], claim_W = r[at + 1];
     zk_record(final_claim);
     zk_record(claim_X);
     zk_record(claim_W);

@@ -21,6 +21,22 @@ class zkFC {
     struct Challenges { vector<Fr_t> u_batch, u_input, u_output; };
     Challenges draw(uint batchSize) const;
     vector<Claim> prove(const FrTensor& X, const FrTensor& Y, const Challenges& ch) const;
+    // Addition: prove(X, Y, ch) in two halves.  prove_begin queues the whole device side of the proof on the default stream -- Y
+    // at (u_batch, u_output), the two reduced vectors, every round of the inner-product sumcheck -- without waiting for any of
+    // it and records nothing; prove_end collects the values, runs the checks and writes the transcript entries in prove's
+    // order.  X and Y must stay alive and unmodified in between.  The two fully folded vectors of the sumcheck ARE X and W at the
+    // proof's point, so they are not evaluated a second time (prove() does the same now: it is the two halves in a row).
+    struct Pending {
+        Challenges ch;
+        uint batchSize = 0;
+        vector<uint> round_sizes;          // inner-product rounds that ran as launches of their own (3 values each), then ...
+        uint small_rounds = 0;             // ... the rounds of the single-workgroup kernel (3 each, and the two folded values)
+        std::vector<FrTensor> keep;        // reduced and folded vectors the queued kernels read
+        DeferredResults results;
+    };
+    Pending prove_begin(const FrTensor& X, const FrTensor& Y, const Challenges& ch) const;
+    vector<Claim> prove_end(Pending& p) const;
+    vector<Claim> prove_at_once(const FrTensor& X, const FrTensor& Y, const Challenges& ch) const;      // every value fetched where it is used
 
     // weight_ptr / bias_ptr are device pointers to float data
     static zkFC from_float_gpu_ptr(uint input_size, uint output_size, unsigned long scaling_factor, float* weight_ptr, float* bias_ptr);
