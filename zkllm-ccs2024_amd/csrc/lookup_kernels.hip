@@ -722,6 +722,67 @@ __global__ void __launch_bounds__(TPB) k_lookup_round29(Fr* __restrict__ partial
     block_reduce_store<5>(acc, partials);
 }
 
+// k_lookup_round<false, true> for queries given by their int32 forms (HintSrc::hint_ints), with the arithmetic of the common
+// pair -- both inverses read from the table's records -- in 29-bit limbs: M = (a0 + a1)(s0 + s1') is one product, E M goes into
+// an unreduced sum, the two folds are one product each; the sums of a0, of a1 and of E are plain 288-bit integers.  A pair
+// with an inverse of its own (a query that is no table entry, or -beta) takes the formulas of the other kernel in 32-bit limbs.
+// Same inputs, same outputs (folded tensors canonical, the five sums with the factors that kernel leaves on them).  At most
+// 512 pairs per lane (the unreduced sum holds 2^522): the launch site checks.
+__global__ void __launch_bounds__(TPB) k_lookup_first29(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ nS, const Fr* __restrict__ E, const Fr beta, const Fr v_mont,
+                                                        size_t n_out, Fr* __restrict__ nE, const HintSrc hs) {
+    const Fr29 vq = fr29_mul(fr29_repack(v_mont), fr29_2_266());      // v 2^261
+    const Fr29 b2 = fr29_repack(add(beta, beta));
+    Wide29 wx = wide29_zero();                                         // sum of E M over the pairs of unit inverses, times 2^-5
+    uint32_t se[9], sa0[9], sa1[9];                                    // sums of E (those pairs), of a0 and of a1 (every pair)
+#pragma unroll
+    for (int i = 0; i < 9; ++i) se[i] = sa0[i] = sa1[i] = 0;
+    Fr c0s = big_zero<8>(), c1s = big_zero<8>(), c2s = big_zero<8>();  // the three weighted terms of the other pairs
+    uint32_t it = 0;
+    for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
+        const Fr e = ld_stream(E + t);
+        if (nE && t < n_out / 2) st_stream(nE + t, add(e, ld_stream(E + t + n_out / 2)));      // the next round's table: the top variable summed out
+        Fr s0w, s1w, a0w, a1w;
+        bool unit0 = false, unit1 = false;
+        s0w = query_inv_ints(t, hs, a0w, unit0);
+        s1w = query_inv_ints(t + n_out, hs, a1w, unit1);
+        sum9_add(sa0, a0w);
+        sum9_add(sa1, a1w);
+        if (unit0 && unit1) {
+            const Fr29 a0 = fr29_repack(a0w), a1 = fr29_repack(a1w), s0 = fr29_repack(s0w), s1 = fr29_repack(s1w);
+            sum9_add(se, e);
+            const Fr29 M = fr29_mul(fr29_add(a0, a1), fr29_add(fr29_add(s0, s1), b2));
+            wide29_mac(wx, fr29_repack(e), M);
+            if ((++it & 3u) == 0u) wide29_carry(wx);
+            st_stream(nA + t, fr29_canon_pack(fr29_add(a0, fr29_mul(vq, fr29_sub_plus_r(a1, a0)))));
+            st_stream(nS + t, fr29_canon_pack(fr29_add(s0, fr29_mul(vq, fr29_sub_plus_r(s1, s0)))));
+        } else {
+            const Fr da = sub(a1w, a0w), ds = sub(s1w, s0w), s0 = add(s0w, beta);
+            const Fr ea0 = mont_mul(e, a0w), eda = mont_mul(e, da);
+            const Fr c0 = mont_mul(ea0, s0), c2 = mont_mul(eda, ds);
+            c0s = add(c0s, c0);
+            c1s = add(c1s, sub(sub(mont_mul(add(ea0, eda), add(s0, ds)), c0), c2));
+            c2s = add(c2s, c2);
+            st_stream(nA + t, add(a0w, mont_mul(v_mont, da)));
+            st_stream(nS + t, add(s0w, mont_mul(v_mont, ds)));
+        }
+    }
+    Fr acc[5];
+    // E M 2^-5 summed; reduced (2^-261) and brought to the factor 2^-256 of the other kernel's products by 2^271 (2^-261 again)
+    const Fr acc_em = fr29_canon_pack(fr29_mul(wide29_redc(wx), fr29_2_271()));
+    // E is in Montgomery form and the sums carry R^-1: sum(E) R^-2 through one product with R^-1
+    constexpr uint32_t RINV[8] = {4269129792u, 334977897u, 165441631u, 2876230287u, 1333208682u, 1912866698u, 805346647u, 465471123u};
+    Fr k;
+#pragma unroll
+    for (int l = 0; l < 8; ++l) k.v[l] = RINV[l];
+    const Fr one = mont_mul(sum9_residue(se), k), two = add(one, one), four = add(two, two);
+    acc[0] = add(c0s, one);
+    acc[1] = add(c1s, sub(acc_em, four));
+    acc[2] = add(c2s, sub(four, acc_em));
+    acc[3] = sum9_residue(sa0);
+    acc[4] = sub(sum9_residue(sa1), acc[3]);
+    block_reduce_store<5>(acc, partials);
+}
+
 // ---- Hadamard-product sumcheck with adjacent-pair folding (Fr_hp_sc, proof.cu:66-98) -------------------------------------
 // One round over pairs (2g, 2g+1), zero beyond in_size: the three term tensors of the reference's step kernel
 //   o0 = a0 b0,  o1 = a0 db + b0 da,  o2 = da db      (each product carries R^-1: the reference multiplies standard-form
@@ -2086,8 +2147,11 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
                 ZK_HIP(hipEventCreate(&t1));
                 ZK_HIP(hipEventRecord(t0, st));
             }
-            hipLaunchKernelGGL((k_lookup_round<false, true>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, (const Fr*)nullptr, cS,
-                               (const Fr*)nullptr, (const Fr*)nullptr, (const Fr*)nullptr, cE, b, vm, half, nE, *hs);
+            if (hs->hint_ints && limbs29() && half <= (size_t)512 * nb * TPB)      // queries in int32 form: the common pair in 29-bit limbs
+                hipLaunchKernelGGL(k_lookup_first29, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, cE, b, vm, half, nE, *hs);
+            else
+                hipLaunchKernelGGL((k_lookup_round<false, true>), dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, (Fr*)nullptr, (Fr*)nullptr, (Fr*)nullptr, (const Fr*)nullptr, cS,
+                                   (const Fr*)nullptr, (const Fr*)nullptr, (const Fr*)nullptr, cE, b, vm, half, nE, *hs);
             if (g_round_timer.on) {
                 ZK_HIP(hipEventRecord(t1, st));
                 std::lock_guard<std::mutex> lk(g_round_timer.mu);
