@@ -583,7 +583,7 @@ def test_mapped_lookup_job_equals_the_plain_one_on_the_combined_queries(k):
         hip.free(p)
 
 
-@pytest.mark.parametrize("k,bad_entry", [(17, False), (17, True), (13, False)])
+@pytest.mark.parametrize("k,bad_entry", [(17, False), (17, True), (13, False), (19, False), (19, True)])
 def test_mapped_lookup_over_outputs_gathered_by_their_queries(k, bad_entry):
     """Outputs made by zk_fr_gather_by_queries_ints carry where they came from; a mapped job over the same queries, outputs and
     table then reads neither outputs nor per-entry integers for queries inside the table.  Checked against the plain job on
@@ -685,7 +685,7 @@ def test_mapped_lookup_over_outputs_gathered_by_their_queries(k, bad_entry):
         hip.free(q)
 
 
-@pytest.mark.parametrize("k,length", [(17, 48), (17, 64), (13, 37)])
+@pytest.mark.parametrize("k,length", [(17, 48), (17, 64), (13, 37), (19, 48), (18, 64)])
 def test_range_table_padded_by_repeating_its_last_value_keeps_the_short_first_round(k, length):
     """A range table of `length` entries padded to 64 by repeating its last value (zk_range_table): the entries below `length` are
     what the integers say and serve their queries from the table record alone (zk_lookup_last_job_consistent_entries reports
@@ -870,7 +870,8 @@ def test_lookup_jobs_that_read_int32_forms_equal_the_plain_one(k):
     takes query and inverse from the table where the entry is what the integers say) against zk_lookup_prove_begin on the
     combined queries computed here with big integers: inputs outside the table, outputs that are not the mapped value,
     the extreme integers, a table entry that is NOT low + j + r * mapped[j] (its queries must not be read from it) and one
-    whose inverse does not exist.  2^13: the small-job path (the field elements serve); 2^17 / 2^19: the fused first round."""
+    whose inverse does not exist.  2^13: the small-job path (the field elements serve); 2^17: the fused first round; 2^19: the
+    first two rounds in one pass (k_lookup_first2_29)."""
     import ctypes
     from gpuhelp import Hip, c_void_p, c_size_t, c_int
     hip = Hip()

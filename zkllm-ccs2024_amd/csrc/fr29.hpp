@@ -107,6 +107,19 @@ ZK_HD Fr29 fr29_sub_plus_r(const Fr29& a, const Fr29& b) {
     r.l[8] = a.l[8] - b.l[8] + fr29_p(8) + c;
     return r;
 }
+// a - b + 3 r: non-negative for b < 3 r (operands that are sums of a canonical value and a product, below 2.1 r)
+ZK_HD Fr29 fr29_sub_plus_3r(const Fr29& a, const Fr29& b) {
+    Fr29 r;
+    int32_t c = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int32_t s = a.l[i] - b.l[i] + 3 * fr29_p(i) + c;
+        r.l[i] = (int32_t)((uint32_t)s & R29M);
+        c = s >> 29;
+    }
+    r.l[8] = a.l[8] - b.l[8] + 3 * fr29_p(8) + c;
+    return r;
+}
 // the same integer in 29-bit limbs (any 256-bit value)
 ZK_HD Fr29 fr29_repack(const Big<8>& a) {
     Fr29 r;
@@ -119,11 +132,11 @@ ZK_HD Fr29 fr29_repack(const Big<8>& a) {
     }
     return r;
 }
-// canonical residue of a non-negative value below 3 r, as 8 x 32-bit words
-ZK_HD Big<8> fr29_canon_pack(const Fr29& a) {
+// canonical residue of a non-negative value below (PASSES + 1) r, as 8 x 32-bit words
+template <int PASSES = 2> ZK_HD Big<8> fr29_canon_pack(const Fr29& a) {
     Fr29 v = a;
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
+    for (int pass = 0; pass < PASSES; ++pass) {
         Fr29 t;
         int32_t c = 0;
 #pragma unroll

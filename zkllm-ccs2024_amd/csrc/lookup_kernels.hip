@@ -783,6 +783,127 @@ __global__ void __launch_bounds__(TPB) k_lookup_first29(Fr* __restrict__ partial
     block_reduce_store<5>(acc, partials);
 }
 
+// The first TWO rounds of such a job in one pass: the folded tensors of the first round are never written or read back.
+// Lane t < h2 (h2 = a quarter of the queries) takes the quad t, t + h2, t + h1, t + h1 + h2 (h1 = 2 h2): the first round's pairs
+// (t, t + h1) and (t + h2, t + h1 + h2) with their eq weights E[t], E[t + h2], exactly as k_lookup_first29 treats a pair; their
+// folds by v1 are the second round's pair (t, t + h2), whose weight is the sum of the two (the top variable summed out), treated
+// as k_lookup_round29 treats a pair except that its three weighted products are reduced one by one (three unreduced sums more
+// would not fit two waves per SIMD, and this kernel is bound by its traffic: 176 bytes per quad instead of 528).  The second
+// round's plain sums follow from four sums of the gathered inverses, one per quarter: sum a' = S_0 + v1 (S_1 - S_0).
+// Writes the second round's folded tensors (h2 each), the third round's eq table (h2 / 2 entries) and both rounds' five sums
+// (partials: round 1 at [0, 5 gridDim), round 2 behind it).  At most 256 quads per lane; the launch site checks.
+// what every lane needs of the challenges, made on the host so that it arrives in scalar registers
+struct First2Consts { Fr29 vq1, vq2, b29, b2, c261; };      // v1 2^261, v2 2^261, beta, 2 beta, 2^261 mod r (a product with it leaves the value, reduced)
+static First2Consts first2_consts(const Fr& beta, const Fr& v1_mont, const Fr& v2_mont) {
+    First2Consts c;
+    c.vq1 = fr29_mul(fr29_repack(v1_mont), fr29_2_266());
+    c.vq2 = fr29_mul(fr29_repack(v2_mont), fr29_2_266());
+    c.b29 = fr29_repack(beta);
+    c.b2 = fr29_repack(add(beta, beta));
+    Fr29 one29 = fr29_zero();
+    one29.l[0] = 1;
+    c.c261 = fr29_mul(fr29_2_522(), one29);
+    return c;
+}
+__global__ void __launch_bounds__(TPB) k_lookup_first2_29(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ nS, const Fr* __restrict__ E, const Fr beta,
+                                                          const Fr v1_mont, const First2Consts cs, size_t h2, Fr* __restrict__ nE3, const HintSrc hs) {
+    __shared__ uint32_t rare[3][8][TPB];                               // round 1: the three weighted terms of the pairs with an inverse of their own, per lane
+    const size_t h1 = 2 * h2;
+    const Fr29 vq1 = cs.vq1, vq2 = cs.vq2, b29 = cs.b29, b2 = cs.b2, c261 = cs.c261;
+    Wide29 wx = wide29_zero();                                         // round 1: sum of E M over the pairs of unit inverses, times 2^-5
+    uint32_t se[9], q00[9], q01[9], q10[9], q11[9];                    // sums of E (those pairs) and of the inverses of the four quarters
+#pragma unroll
+    for (int i = 0; i < 9; ++i) se[i] = q00[i] = q01[i] = q10[i] = q11[i] = 0;
+#pragma unroll
+    for (int k = 0; k < 3; ++k)
+#pragma unroll
+        for (int l = 0; l < 8; ++l) rare[k][l][threadIdx.x] = 0;
+    Fr29 t0 = fr29_zero(), t2 = fr29_zero(), tx = fr29_zero();         // round 2: the three weighted sums, times 2^-266
+    uint32_t it = 0;
+    for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < h2; t += (size_t)gridDim.x * TPB) {
+        const Fr eA = ld_stream(E + t), eB = ld_stream(E + t + h2);
+        if (nE3 && t < h2 / 2) st_stream(nE3 + t, add(add(eA, eB), add(ld_stream(E + t + h2 / 2), ld_stream(E + t + h2 + h2 / 2))));      // two variables summed out
+        Fr29 fa[2], fs[2];                                             // the first round's folds: the second round's pair
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const size_t i = t + (half ? h2 : 0);
+            const Fr e = half ? eB : eA;
+            Fr s0w, s1w, a0w, a1w;
+            bool unit0 = false, unit1 = false;
+            s0w = query_inv_ints(i, hs, a0w, unit0);
+            s1w = query_inv_ints(i + h1, hs, a1w, unit1);
+            if (half) { sum9_add(q01, a0w); sum9_add(q11, a1w); }
+            else { sum9_add(q00, a0w); sum9_add(q10, a1w); }
+            if (unit0 && unit1) {
+                const Fr29 a0 = fr29_repack(a0w), a1 = fr29_repack(a1w), s0 = fr29_repack(s0w), s1 = fr29_repack(s1w);
+                sum9_add(se, e);
+                const Fr29 M = fr29_mul(fr29_add(a0, a1), fr29_add(fr29_add(s0, s1), b2));
+                wide29_mac(wx, fr29_repack(e), M);
+                fa[half] = fr29_add(a0, fr29_mul(vq1, fr29_sub_plus_r(a1, a0)));
+                fs[half] = fr29_add(s0, fr29_mul(vq1, fr29_sub_plus_r(s1, s0)));
+            } else {
+                const Fr da = sub(a1w, a0w), ds = sub(s1w, s0w), s0 = add(s0w, beta);
+                const Fr ea0 = mont_mul(e, a0w), eda = mont_mul(e, da);
+                const Fr c0 = mont_mul(ea0, s0), c2 = mont_mul(eda, ds);
+                const Fr c1 = sub(sub(mont_mul(add(ea0, eda), add(s0, ds)), c0), c2);
+                Fr r0, r1, r2;
+#pragma unroll
+                for (int l = 0; l < 8; ++l) { r0.v[l] = rare[0][l][threadIdx.x]; r1.v[l] = rare[1][l][threadIdx.x]; r2.v[l] = rare[2][l][threadIdx.x]; }
+                r0 = add(r0, c0); r1 = add(r1, c1); r2 = add(r2, c2);
+#pragma unroll
+                for (int l = 0; l < 8; ++l) { rare[0][l][threadIdx.x] = r0.v[l]; rare[1][l][threadIdx.x] = r1.v[l]; rare[2][l][threadIdx.x] = r2.v[l]; }
+                fa[half] = fr29_repack(add(a0w, mont_mul(v1_mont, da)));
+                fs[half] = fr29_repack(add(s0w, mont_mul(v1_mont, ds)));
+            }
+        }
+        if ((++it & 1u) == 0u) wide29_carry(wx);                       // two terms a quad: a carry pass every fourth term
+        // the second round over (fa[0], fa[1]), (fs[0], fs[1]); the folds are below 2.03 r, differences are taken with 3 r added
+        const Fr29 e2 = fr29_add(fr29_repack(eA), fr29_repack(eB));
+        const Fr29 da = fr29_sub_plus_3r(fa[1], fa[0]), ds = fr29_sub_plus_3r(fs[1], fs[0]);
+        const Fr29 s0 = fr29_add(fs[0], b29);
+        const Fr29 ea0 = fr29_mul(e2, fa[0]), eda = fr29_mul(e2, da);
+        t0 = fr29_add(t0, fr29_mul(ea0, s0));
+        t2 = fr29_add(t2, fr29_mul(eda, ds));
+        tx = fr29_add(tx, fr29_mul(fr29_add(ea0, eda), fr29_add(s0, ds)));
+        if ((it & 31u) == 0u) { t0 = fr29_mul(t0, c261); t2 = fr29_mul(t2, c261); tx = fr29_mul(tx, c261); }      // the top limbs stay below 2^30
+        st_stream(nA + t, fr29_canon_pack<3>(fr29_add(fa[0], fr29_mul(vq2, da))));
+        st_stream(nS + t, fr29_canon_pack<3>(fr29_add(fs[0], fr29_mul(vq2, ds))));
+    }
+    const Fr29 fix = fr29_2_271();
+    // round 1
+    {
+        Fr acc[5];
+        const Fr acc_em = fr29_canon_pack(fr29_mul(wide29_redc(wx), fix));
+        constexpr uint32_t RINV[8] = {4269129792u, 334977897u, 165441631u, 2876230287u, 1333208682u, 1912866698u, 805346647u, 465471123u};
+        Fr k;
+#pragma unroll
+        for (int l = 0; l < 8; ++l) k.v[l] = RINV[l];
+        const Fr one = mont_mul(sum9_residue(se), k), two = add(one, one), four = add(two, two);
+        Fr c0s, c1s, c2s;
+#pragma unroll
+        for (int l = 0; l < 8; ++l) { c0s.v[l] = rare[0][l][threadIdx.x]; c1s.v[l] = rare[1][l][threadIdx.x]; c2s.v[l] = rare[2][l][threadIdx.x]; }
+        acc[0] = add(c0s, one);
+        acc[1] = add(c1s, sub(acc_em, four));
+        acc[2] = add(c2s, sub(four, acc_em));
+        acc[3] = add(sum9_residue(q00), sum9_residue(q01));
+        acc[4] = sub(add(sum9_residue(q10), sum9_residue(q11)), acc[3]);
+        block_reduce_store<5>(acc, partials);
+    }
+    // round 2
+    {
+        Fr acc[5];
+        acc[0] = fr29_canon_pack(fr29_mul(t0, fix));
+        acc[2] = fr29_canon_pack(fr29_mul(t2, fix));
+        acc[1] = sub(sub(fr29_canon_pack(fr29_mul(tx, fix)), acc[0]), acc[2]);
+        const Fr r00 = sum9_residue(q00), r01 = sum9_residue(q01);
+        const Fr sA = add(r00, mont_mul(v1_mont, sub(sum9_residue(q10), r00)));      // sum of fa[0] over the lane's quads
+        const Fr sB = add(r01, mont_mul(v1_mont, sub(sum9_residue(q11), r01)));      // sum of fa[1]
+        acc[3] = sA;
+        acc[4] = sub(sB, sA);
+        block_reduce_store<5>(acc, partials + 5 * (size_t)gridDim.x);
+    }
+}
+
 // ---- Hadamard-product sumcheck with adjacent-pair folding (Fr_hp_sc, proof.cu:66-98) -------------------------------------
 // One round over pairs (2g, 2g+1), zero beyond in_size: the three term tensors of the reference's step kernel
 //   o0 = a0 b0,  o1 = a0 db + b0 da,  o2 = da db      (each product carries R^-1: the reference multiplies standard-form
@@ -2059,6 +2180,8 @@ static const int g_round_timer_hook = (at_shutdown([] {
     g_eq_latest.reset();          // the eq table kept for the next job with the same challenges goes back to the allocator
 }), 0);
 // ZKLLM_FR_LIMBS=32 keeps the round kernels on the 32-bit-limb arithmetic throughout (to compare; the results are the same)
+// ZKLLM_LOOKUP_TWO_ROUNDS=0: the first two rounds of a lookup job over int32 queries as two passes (to compare)
+static bool two_rounds_on() { static const bool on = [] { const char* e = getenv("ZKLLM_LOOKUP_TWO_ROUNDS"); return !(e && e[0] == '0'); }(); return on; }
 static bool limbs29() { static const bool on = [] { const char* e = getenv("ZKLLM_FR_LIMBS"); return !(e && atoi(e) == 32); }(); return on; }
 // all rounds of the lookup sumcheck; sums land in job.sums
 // A == nullptr with a hint source: 1 / (S + beta) has not been written anywhere; a large first round computes it on
@@ -2112,6 +2235,51 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
                                (uint32_t)rest, (uint32_t)(phase2 ? 0 : n1 - r));
             ZK_LAUNCH_CHECK();
             break;
+        }
+        if (r == 0 && !phase2 && fuse_first && hs->hint_ints && limbs29() && two_rounds_on() && n1 >= 2 && rounds >= 2 && (half >> 1) > (size_t)SPLIT_HALF &&
+            (half >> 1) <= (size_t)256 * reduce_grid(half >> 1) * TPB) {
+            // queries in int32 form, two large phase-1 rounds ahead: both in one pass (k_lookup_first2_29)
+            const size_t h2 = half >> 1;
+            const unsigned nb2 = reduce_grid(h2);
+            Scratch& nx2 = job.arena.add(sizeof(Fr) * h2 * 2);
+            if (nx2.rc) return nx2.rc;
+            Fr* w2 = nx2.as<Fr>();
+            // the third round's eq table goes where the second round would have put it
+            Fr* nE3 = nullptr;
+            if (r + 2 < rounds) {
+                Scratch& e = job.arena.add(sizeof(Fr) * 2 * h2);
+                if (e.rc) return e.rc;
+                eqbuf[0] = e.as<Fr>();
+                eqbuf[1] = eqbuf[0] + h2;
+                nE3 = eqbuf[1];
+            }
+            const Fr vm = to_mont(load_fr(v + 8 * r)), vm2 = to_mont(load_fr(v + 8 * (r + 1)));
+            const First2Consts cs = first2_consts(b, vm, vm2);
+            hipEvent_t t0 = nullptr, t1 = nullptr;
+            if (g_round_timer.on) {
+                ZK_HIP(hipEventCreate(&t0));
+                ZK_HIP(hipEventCreate(&t1));
+                ZK_HIP(hipEventRecord(t0, st));
+            }
+            hipLaunchKernelGGL(k_lookup_first2_29, dim3(nb2), dim3(TPB), 0, st, part.as<Fr>(), w2, w2 + h2, cE, b, vm, cs, h2, nE3, *hs);
+            if (g_round_timer.on) {
+                ZK_HIP(hipEventRecord(t1, st));
+                std::lock_guard<std::mutex> lk(g_round_timer.mu);
+                g_round_timer.ev.emplace_back(t0, t1);
+                g_round_timer.pairs += half;
+                // per quad: four queries in int32 form (and their outputs where those are read), two eq weights, two folded values
+                // written, half a share of the next table (two more weights read, one written)
+                const double q = (hs->sout_ints && !hs->trusted_out) ? 32.0 : 16.0;
+                g_round_timer.bytes += (double)h2 * (q + 64.0 + 64.0 + (nE3 ? 48.0 : 0.0));
+            }
+            hipLaunchKernelGGL(k_finish, dim3(5), dim3(TPB), 0, st, sums.as<Fr>() + (size_t)r * 11, part.as<Fr>(), nb2);
+            hipLaunchKernelGGL(k_finish, dim3(5), dim3(TPB), 0, st, sums.as<Fr>() + (size_t)(r + 1) * 11, part.as<Fr>() + 5 * (size_t)nb2, nb2);
+            ZK_LAUNCH_CHECK();
+            cA = w2; cS = w2 + h2;
+            cur = h2;
+            if (nE3) cE = nE3;
+            ++r;                // two rounds done
+            continue;
         }
         Scratch& nx = job.arena.add(sizeof(Fr) * half * (phase2 ? 5 : 2));
         if (nx.rc) return nx.rc;
