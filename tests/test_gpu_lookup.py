@@ -195,11 +195,12 @@ def test_rescaling_that_gives_its_output_an_int32_form(pv, orc, n, sf, bits, fit
     assert t.shape == e_t.shape and (t == e_t).all()
 
 
-@pytest.mark.parametrize("D,low,length", [(1000, -16, 32), (100000, -16, 32), (1 << 17, -20, 40)])
+@pytest.mark.parametrize("D,low,length", [(1000, -16, 32), (100000, -16, 32), (1 << 17, -20, 40), (1 << 18, -20, 40), (300000, -16, 32)])
 def test_mapping_lookup_with_int32_forms(pv, orc, D, low, length):
     """tLookupRangeMapping with integer mapped values over queries that keep an int32 form: outputs, multiplicities and the
     proof's transcript are the oracle's.  1000 queries: padded in both forms, the small job reads the field elements; 100000:
-    padded to 2^17 in the int32 form only (the job reads nothing else); 2^17: no padding."""
+    padded to 2^17 in the int32 form only (the job reads nothing else); 2^17: no padding; 2^18 and 300000 (padded to 2^19): the
+    job's first two rounds run as one pass (k_lookup_first2_29)."""
     rng = np.random.default_rng(D + 1)
     vals = rng.integers(low, low + length, D)
     mvi = rng.integers(-2 ** 31, 2 ** 31, length).astype(np.int64)
@@ -221,6 +222,31 @@ def test_mapping_lookup_with_int32_forms(pv, orc, D, low, length):
     pv.lib.zkp_transcript_end()
     assert pv.folds_from_ints(y) == 1
     assert (y.host() == e_y).all() and (m.host() == e_m).all() and (fin == e_fin).all()
+    t = pv.transcript()
+    assert t.shape == e_t.shape and (t == e_t).all()
+
+
+@pytest.mark.parametrize("D,low,length", [(1 << 17, -(1 << 9), 1 << 10), (1 << 18, -(1 << 7), 1 << 8), (1 << 19, -(1 << 15), 1 << 16)])
+def test_range_lookup_over_an_int32_form_against_the_oracle(pv, orc, D, low, length):
+    """tLookupRange::prove over queries that keep an int32 form, at sizes where the job reads that form alone: 2^17 queries -- the
+    first round on its own --, 2^18 and 2^19 -- the first two rounds in one pass.  Transcript and final claim are the oracle's."""
+    rng = np.random.default_rng(D + length)
+    vals = rng.integers(low, low + length, D)
+    vals[:4] = [low, low + length - 1, low, low + length - 1]
+    S = fr_array([int(v) % R_MOD for v in vals])
+    k = (D - 1).bit_length()
+    alpha, beta, u, v = ch(1, 1)[0], ch(2, 1)[0], ch(3, k), ch(4, k)
+    orc.orc_transcript_clear()
+    e_fin = np.zeros(8, np.uint32)
+    orc_check(orc.orc_range_prove(S, D, low, length, alpha, beta, u, v, e_fin))
+    e_t = orc_transcript(orc)
+    hS = pv.from_i64(vals.astype(np.int64))
+    pv.keep_for_folds(hS)
+    assert pv.folds_from_ints(hS) == 1
+    pv.transcript_begin()
+    fin = pv.range_prove(hS, low, length, alpha, beta, u, v)
+    pv.lib.zkp_transcript_end()
+    assert (fin == e_fin).all()
     t = pv.transcript()
     assert t.shape == e_t.shape and (t == e_t).all()
 
