@@ -811,36 +811,53 @@ __global__ void __launch_bounds__(TPB) k_lookup_first2_29(Fr* __restrict__ parti
     const size_t h1 = 2 * h2;
     const Fr29 vq1 = cs.vq1, vq2 = cs.vq2, b29 = cs.b29, b2 = cs.b2, c261 = cs.c261;
     Wide29 wx = wide29_zero();                                         // round 1: sum of E M over the pairs of unit inverses, times 2^-5
-    uint32_t se[9], q00[9], q01[9], q10[9], q11[9];                    // sums of E (those pairs) and of the inverses of the four quarters
+    __shared__ uint32_t qsum[4][9][TPB];                               // sums of the inverses of the four quarters, per lane (registers are short here)
+    uint32_t se[9];                                                    // sum of E over the pairs of unit inverses
 #pragma unroll
-    for (int i = 0; i < 9; ++i) se[i] = q00[i] = q01[i] = q10[i] = q11[i] = 0;
+    for (int i = 0; i < 9; ++i) se[i] = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int l = 0; l < 9; ++l) qsum[k][l][threadIdx.x] = 0;
 #pragma unroll
     for (int k = 0; k < 3; ++k)
 #pragma unroll
         for (int l = 0; l < 8; ++l) rare[k][l][threadIdx.x] = 0;
+    auto qsum_add = [&](int k, const Fr& x) {
+        uint32_t acc[9];
+#pragma unroll
+        for (int l = 0; l < 9; ++l) acc[l] = qsum[k][l][threadIdx.x];
+        sum9_add(acc, x);
+#pragma unroll
+        for (int l = 0; l < 9; ++l) qsum[k][l][threadIdx.x] = acc[l];
+    };
+    auto qsum_residue = [&](int k) {
+        uint32_t acc[9];
+#pragma unroll
+        for (int l = 0; l < 9; ++l) acc[l] = qsum[k][l][threadIdx.x];
+        return sum9_residue(acc);
+    };
     Fr29 t0 = fr29_zero(), t2 = fr29_zero(), tx = fr29_zero();         // round 2: the three weighted sums, times 2^-266
     uint32_t it = 0;
     for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < h2; t += (size_t)gridDim.x * TPB) {
         const Fr eA = ld_stream(E + t), eB = ld_stream(E + t + h2);
         if (nE3 && t < h2 / 2) st_stream(nE3 + t, add(add(eA, eB), add(ld_stream(E + t + h2 / 2), ld_stream(E + t + h2 + h2 / 2))));      // two variables summed out
-        Fr29 fa[2], fs[2];                                             // the first round's folds: the second round's pair
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const size_t i = t + (half ? h2 : 0);
-            const Fr e = half ? eB : eA;
+        // the first round's folds: the second round's pair (named variables: an array indexed by the half would live in private memory)
+        Fr29 fa0, fs0, fa1, fs1;
+        auto first_round_pair = [&](size_t i, const Fr& e, int qa, int qb, Fr29& fa, Fr29& fs) {
             Fr s0w, s1w, a0w, a1w;
             bool unit0 = false, unit1 = false;
             s0w = query_inv_ints(i, hs, a0w, unit0);
             s1w = query_inv_ints(i + h1, hs, a1w, unit1);
-            if (half) { sum9_add(q01, a0w); sum9_add(q11, a1w); }
-            else { sum9_add(q00, a0w); sum9_add(q10, a1w); }
+            qsum_add(qa, a0w);
+            qsum_add(qb, a1w);
             if (unit0 && unit1) {
                 const Fr29 a0 = fr29_repack(a0w), a1 = fr29_repack(a1w), s0 = fr29_repack(s0w), s1 = fr29_repack(s1w);
                 sum9_add(se, e);
                 const Fr29 M = fr29_mul(fr29_add(a0, a1), fr29_add(fr29_add(s0, s1), b2));
                 wide29_mac(wx, fr29_repack(e), M);
-                fa[half] = fr29_add(a0, fr29_mul(vq1, fr29_sub_plus_r(a1, a0)));
-                fs[half] = fr29_add(s0, fr29_mul(vq1, fr29_sub_plus_r(s1, s0)));
+                fa = fr29_add(a0, fr29_mul(vq1, fr29_sub_plus_r(a1, a0)));
+                fs = fr29_add(s0, fr29_mul(vq1, fr29_sub_plus_r(s1, s0)));
             } else {
                 const Fr da = sub(a1w, a0w), ds = sub(s1w, s0w), s0 = add(s0w, beta);
                 const Fr ea0 = mont_mul(e, a0w), eda = mont_mul(e, da);
@@ -852,22 +869,24 @@ __global__ void __launch_bounds__(TPB) k_lookup_first2_29(Fr* __restrict__ parti
                 r0 = add(r0, c0); r1 = add(r1, c1); r2 = add(r2, c2);
 #pragma unroll
                 for (int l = 0; l < 8; ++l) { rare[0][l][threadIdx.x] = r0.v[l]; rare[1][l][threadIdx.x] = r1.v[l]; rare[2][l][threadIdx.x] = r2.v[l]; }
-                fa[half] = fr29_repack(add(a0w, mont_mul(v1_mont, da)));
-                fs[half] = fr29_repack(add(s0w, mont_mul(v1_mont, ds)));
+                fa = fr29_repack(add(a0w, mont_mul(v1_mont, da)));
+                fs = fr29_repack(add(s0w, mont_mul(v1_mont, ds)));
             }
-        }
+        };
+        first_round_pair(t, eA, 0, 2, fa0, fs0);              // quarters: 0 = [0, h2), 1 = [h2, h1), 2 = [h1, h1 + h2), 3 = the last
+        first_round_pair(t + h2, eB, 1, 3, fa1, fs1);
         if ((++it & 1u) == 0u) wide29_carry(wx);                       // two terms a quad: a carry pass every fourth term
-        // the second round over (fa[0], fa[1]), (fs[0], fs[1]); the folds are below 2.03 r, differences are taken with 3 r added
+        // the second round over (fa0, fa1), (fs0, fs1); the folds are below 2.03 r, differences are taken with 3 r added
         const Fr29 e2 = fr29_add(fr29_repack(eA), fr29_repack(eB));
-        const Fr29 da = fr29_sub_plus_3r(fa[1], fa[0]), ds = fr29_sub_plus_3r(fs[1], fs[0]);
-        const Fr29 s0 = fr29_add(fs[0], b29);
-        const Fr29 ea0 = fr29_mul(e2, fa[0]), eda = fr29_mul(e2, da);
+        const Fr29 da = fr29_sub_plus_3r(fa1, fa0), ds = fr29_sub_plus_3r(fs1, fs0);
+        const Fr29 s0 = fr29_add(fs0, b29);
+        const Fr29 ea0 = fr29_mul(e2, fa0), eda = fr29_mul(e2, da);
         t0 = fr29_add(t0, fr29_mul(ea0, s0));
         t2 = fr29_add(t2, fr29_mul(eda, ds));
         tx = fr29_add(tx, fr29_mul(fr29_add(ea0, eda), fr29_add(s0, ds)));
         if ((it & 31u) == 0u) { t0 = fr29_mul(t0, c261); t2 = fr29_mul(t2, c261); tx = fr29_mul(tx, c261); }      // the top limbs stay below 2^30
-        st_stream(nA + t, fr29_canon_pack<3>(fr29_add(fa[0], fr29_mul(vq2, da))));
-        st_stream(nS + t, fr29_canon_pack<3>(fr29_add(fs[0], fr29_mul(vq2, ds))));
+        st_stream(nA + t, fr29_canon_pack<3>(fr29_add(fa0, fr29_mul(vq2, da))));
+        st_stream(nS + t, fr29_canon_pack<3>(fr29_add(fs0, fr29_mul(vq2, ds))));
     }
     const Fr29 fix = fr29_2_271();
     // round 1
@@ -885,8 +904,8 @@ __global__ void __launch_bounds__(TPB) k_lookup_first2_29(Fr* __restrict__ parti
         acc[0] = add(c0s, one);
         acc[1] = add(c1s, sub(acc_em, four));
         acc[2] = add(c2s, sub(four, acc_em));
-        acc[3] = add(sum9_residue(q00), sum9_residue(q01));
-        acc[4] = sub(add(sum9_residue(q10), sum9_residue(q11)), acc[3]);
+        acc[3] = add(qsum_residue(0), qsum_residue(1));
+        acc[4] = sub(add(qsum_residue(2), qsum_residue(3)), acc[3]);
         block_reduce_store<5>(acc, partials);
     }
     // round 2
@@ -895,9 +914,9 @@ __global__ void __launch_bounds__(TPB) k_lookup_first2_29(Fr* __restrict__ parti
         acc[0] = fr29_canon_pack(fr29_mul(t0, fix));
         acc[2] = fr29_canon_pack(fr29_mul(t2, fix));
         acc[1] = sub(sub(fr29_canon_pack(fr29_mul(tx, fix)), acc[0]), acc[2]);
-        const Fr r00 = sum9_residue(q00), r01 = sum9_residue(q01);
-        const Fr sA = add(r00, mont_mul(v1_mont, sub(sum9_residue(q10), r00)));      // sum of fa[0] over the lane's quads
-        const Fr sB = add(r01, mont_mul(v1_mont, sub(sum9_residue(q11), r01)));      // sum of fa[1]
+        const Fr r00 = qsum_residue(0), r01 = qsum_residue(1);
+        const Fr sA = add(r00, mont_mul(v1_mont, sub(qsum_residue(2), r00)));      // sum of fa0 over the lane's quads
+        const Fr sB = add(r01, mont_mul(v1_mont, sub(qsum_residue(3), r01)));      // sum of fa1
         acc[3] = sA;
         acc[4] = sub(sB, sA);
         block_reduce_store<5>(acc, partials + 5 * (size_t)gridDim.x);
