@@ -367,7 +367,8 @@ int zk_hadamard_prove_end(void* handle, uint32_t* coefs_host);
 
 /* ---- rescaling / softmax ------------------------------------------------------------------------------------------ */
 int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* stream);       /* rescaling_kernel rescaling.cu:8-21 */
-/* the same, and rem_ints (int32, n) receives the remainders once more: they lie in [-sf/2, sf/2) */
+/* the same, and rem_ints (int32, n) receives the remainders once more: they lie in [-sf/2, sf/2).  rem may be null where
+ * rem_ints is given (here and in zk_rescale_ints_both): the remainders are written as int32 only */
 int zk_rescale_ints(void* out, void* rem, void* rem_ints, const void* in, uint32_t scaling_factor, size_t n, void* stream);
 /* the same, and out_ints receives the rescaled values as int32; synchronises and reports in *out_fits_host whether every one
  * of them fits (0: out_ints must not be used) */

@@ -251,6 +251,32 @@ def test_range_lookup_over_an_int32_form_against_the_oracle(pv, orc, D, low, len
     assert t.shape == e_t.shape and (t == e_t).all()
 
 
+@pytest.mark.parametrize("n,sf", [(1 << 17, 1 << 8), (100000, 1 << 10), (1 << 18, 1 << 16)])
+def test_rescaling_whose_remainders_exist_as_int32_only(pv, orc, n, sf):
+    """Rescaling::lean: at these sizes the remainders' range proof reads their int32 form alone, so their field elements are never
+    written (the pool is poisoned first); outputs and transcript are the oracle's.  100000: the proof pads that form to 2^17."""
+    x = np.random.default_rng(n + sf).integers(-(1 << 40), 1 << 40, n)
+    X = fr_array([int(v) % R_MOD for v in x])
+    orc.orc_seed(98)
+    orc.orc_transcript_clear()
+    e_out = np.zeros_like(X)
+    orc_check(orc.orc_rescale_prove(X, n, sf, e_out))
+    e_t = orc_transcript(orc)
+    junk = [pv.from_fr(ch(5, n)) for _ in range(3)]
+    del junk
+    pv.lib.zkp_rescale_set_lean(1)
+    try:
+        pv.seed(98)
+        pv.transcript_begin()
+        out = pv.rescale_prove(pv.from_fr(X), sf)
+        pv.lib.zkp_transcript_end()
+    finally:
+        pv.lib.zkp_rescale_set_lean(0)
+    assert (out.host() == e_out).all()
+    t = pv.transcript()
+    assert t.shape == e_t.shape and (t == e_t).all()
+
+
 def test_rescaling_prove_seeded_transcript(pv, orc):
     for n, sf in ((256, 16), (5000, 1 << 8)):
         x = np.random.default_rng(n).integers(-(1 << 30), 1 << 30, n)

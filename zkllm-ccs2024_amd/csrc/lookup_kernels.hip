@@ -1332,7 +1332,7 @@ __global__ void __launch_bounds__(TPB) k_rescale(Fr* __restrict__ out, Fr* __res
     const int64_t x_rem = (temp < 0 ? temp + sf : temp) - hsf;
     const int64_t x_rescaled = (x - x_rem) / sf;
     out[i] = fr_from_i64(x_rescaled);
-    rem[i] = fr_from_i64(x_rem);
+    if (rem) rem[i] = fr_from_i64(x_rem);
     if (rem_ints) rem_ints[i] = (int32_t)x_rem;
     if (out_ints) {
         out_ints[i] = (int32_t)x_rescaled;
@@ -1390,10 +1390,15 @@ __device__ __forceinline__ void softmax_digits(const PlanePtrs& planes, const In
     }
     if (tmp != 0) atomicOr(flag, 2u);   // more digits than the radices cover
 }
+static constexpr int SHIFT_ROW_CACHE = 2048;
 // K > 0: the shifted scores are decomposed where they are written (k_softmax_decompose's planes without its pass over them)
 __global__ void __launch_bounds__(TPB) k_softmax_shift(Fr* __restrict__ shift, Fr* __restrict__ out, const Fr* __restrict__ X, uint32_t rows, uint32_t cols, double scale,
                                                        const PlanePtrs planes, const IntPlanePtrs ints, uint32_t* __restrict__ flag, const U32Pack8 bs, int K) {
     __shared__ double term[TPB / 64][64];
+    // Rows of up to SHIFT_ROW_CACHE scores are read once: the first pass leaves each score as a 64-bit integer in LDS and the
+    // second takes it from there (a score that is no 64-bit integer raises the flag: its digits could not be formed either).
+    __shared__ int64_t cache[TPB / 64][SHIFT_ROW_CACHE];
+    const bool cached = flag != nullptr && cols <= (uint32_t)SHIFT_ROW_CACHE;      // (the plain shift has no flag to raise: it reads twice)
     const uint32_t w = threadIdx.x >> 6, lane = threadIdx.x & 63u;
     const uint32_t row = blockIdx.x * (TPB / 64) + w;
     const bool live = row < rows;                         // a whole wave is live or idle; idle waves still reach every barrier
@@ -1401,7 +1406,17 @@ __global__ void __launch_bounds__(TPB) k_softmax_shift(Fr* __restrict__ shift, F
     double total = 0.0;
     for (uint32_t j0 = 0; j0 < cols; j0 += 64) {
         const uint32_t j = j0 + lane;
-        term[w][lane] = (live && j < cols) ? zkd::exp_det((double)fr_to_i64(xr[j]) / scale) : 0.0;
+        double tv = 0.0;
+        if (live && j < cols) {
+            const Fr x = xr[j];
+            const int64_t xi = fr_to_i64(x);
+            if (cached) {
+                cache[w][j] = xi;
+                if (!equal(fr_from_i64(xi), x)) atomicOr(flag, 2u);
+            }
+            tv = zkd::exp_det((double)xi / scale);
+        }
+        term[w][lane] = tv;
         __syncthreads();
         const uint32_t cnt = cols - j0 < 64u ? cols - j0 : 64u;
         if (cnt == 64u) {
@@ -1419,7 +1434,7 @@ __global__ void __launch_bounds__(TPB) k_softmax_shift(Fr* __restrict__ shift, F
     if (lane == 0) shift[row] = sh;
     Fr* orow = out + (size_t)row * cols;
     for (uint32_t j = lane; j < cols; j += 64) {
-        const Fr xs = sub(xr[j], sh);
+        const Fr xs = sub(cached ? fr_from_i64(cache[w][j]) : xr[j], sh);
         if (out) orow[j] = xs;
         if (K > 0) softmax_digits(planes, ints, flag, xs, bs, K, (size_t)row * cols + j);
     }
@@ -2888,6 +2903,7 @@ int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, si
 }
 int zk_rescale_ints(void* out, void* rem, void* rem_ints, const void* in, uint32_t scaling_factor, size_t n, void* st) {
     ZK_ARG(scaling_factor >= 1, "zk_rescale: scaling factor is 0");
+    ZK_ARG(rem != nullptr || rem_ints != nullptr, "zk_rescale_ints: the remainders need at least one form");
     LAUNCH1D(k_rescale, n, st, (Fr*)out, (Fr*)rem, (int32_t*)rem_ints, (const Fr*)in, (int64_t)scaling_factor, n);
     return 0;
 }
@@ -2895,6 +2911,7 @@ int zk_rescale_ints_both(void* out, void* out_ints, int* out_fits_host, void* re
     hipStream_t st = (hipStream_t)stv;
     ZK_ARG(scaling_factor >= 1, "zk_rescale: scaling factor is 0");
     ZK_ARG(out_ints != nullptr && out_fits_host != nullptr, "zk_rescale_ints_both: null argument");
+    ZK_ARG(rem != nullptr || rem_ints != nullptr, "zk_rescale_ints_both: the remainders need at least one form");
     *out_fits_host = 1;
     if (n == 0) return 0;
     Scratch flag(4, st);

@@ -323,9 +323,12 @@ void* zkp_rescale_ints_prove(void* X, u32 sf) {
     ZKP_END_PTR
 }
 // Rescaling::operator() + prove with challenges from the seeded stream
+static bool g_rescale_lean = false;
+void zkp_rescale_set_lean(int on) { g_rescale_lean = on != 0; }      // the next zkp_rescale_prove calls run with Rescaling::lean
 void* zkp_rescale_prove(void* X, u32 sf) {
     ZKP_TRY
     Rescaling rs(sf);
+    rs.lean = g_rescale_lean;
     FrTensor out = rs(FT(X));
     rs.prove(FT(X), out);
     return new FrTensor(std::move(out));

@@ -88,7 +88,9 @@ void layer_config_from_env(LayerConfig& c) {
 
 // rmsnorm.cu:26-49
 RmsNormBlock::RmsNormBlock(const LayerConfig& c, const Weight& w, const FrTensor& X, const FrTensor& rms_inv)
-    : c(c), w(w), X(X), rms_inv(rms_inv), rs1(c.sf_linear), rs2(c.sf_linear), g(1, c.embed_dim, FrTensor::view(w.weight)) {}
+    : c(c), w(w), X(X), rms_inv(rms_inv), rs1(c.sf_linear), rs2(c.sf_linear), g(1, c.embed_dim, FrTensor::view(w.weight)) {
+    rs1.lean = rs2.lean = true;      // nothing here reads the remainders but their range proofs
+}
 const FrTensor& RmsNormBlock::forward() {
     g_inv_rms.emplace(g(rms_inv));
     g_inv_rms_.emplace(rs1(*g_inv_rms));
@@ -127,7 +129,9 @@ FrTensor rmsnorm_block(const LayerConfig& c, const Weight& w, const FrTensor& X,
 // self-attn.cu:19-76 (linear mode)
 AttnLinearBlock::AttnLinearBlock(const LayerConfig& c, const Weight& q, const Weight& k, const Weight& v, const FrTensor& input)
     : c(c), q(q), k(k), v(v), input(input), q_layer(c.embed_dim, c.embed_dim, FrTensor::view(q.weight)), k_layer(c.embed_dim, c.embed_dim, FrTensor::view(k.weight)),
-      v_layer(c.embed_dim, c.embed_dim, FrTensor::view(v.weight)), q_rescale(c.sf_linear), k_rescale(c.sf_linear), v_rescale(c.sf_linear) {}
+      v_layer(c.embed_dim, c.embed_dim, FrTensor::view(v.weight)), q_rescale(c.sf_linear), k_rescale(c.sf_linear), v_rescale(c.sf_linear) {
+    q_rescale.lean = k_rescale.lean = v_rescale.lean = true;
+}
 void AttnLinearBlock::forward() {
     Q.emplace(q_layer(input));
     Q_.emplace(q_rescale(*Q));
@@ -217,6 +221,7 @@ AttnStackBlock::AttnStackBlock(const LayerConfig& c, const FrTensor& Q_, const F
       attn(c.num_heads, c.softmax_sf_in, 1UL, c.softmax_bs, c.softmax_L, c.softmax_M, c.softmax_thetas, c.seq_len, c.seq_len, c.embed_dim / c.num_heads, 1), rs1(c.sf_attn),
       rs2(c.sf_attn) {
     if (c.embed_dim % c.num_heads) throw std::runtime_error("embed_dim must be a multiple of num_heads");
+    rs1.lean = rs2.lean = true;
 }
 const FrTensor& AttnStackBlock::forward() {
     const uint seq = c.seq_len, E = c.embed_dim, H = c.num_heads, d = E / H;
@@ -406,7 +411,9 @@ FrTensor attn_reference_block(const LayerConfig& c, const FrTensor& Q, const FrT
 }
 
 OProjBlock::OProjBlock(const LayerConfig& c, const Weight& o, const FrTensor& attn_out)
-    : c(c), o(o), attn_out(attn_out), o_layer(c.embed_dim, c.embed_dim, FrTensor::view(o.weight)), o_rescale(c.sf_linear) {}
+    : c(c), o(o), attn_out(attn_out), o_layer(c.embed_dim, c.embed_dim, FrTensor::view(o.weight)), o_rescale(c.sf_linear) {
+    o_rescale.lean = true;
+}
 const FrTensor& OProjBlock::forward() {
     O.emplace(o_layer(attn_out));
     O_.emplace(o_rescale(*O));
@@ -437,7 +444,9 @@ FrTensor oproj_block(const LayerConfig& c, const Weight& o, const FrTensor& attn
 FfnBlock::FfnBlock(const LayerConfig& c, const Weight& up, const Weight& gate, const Weight& down, const FrTensor& swiglu_values, const FrTensor& input)
     : c(c), up(up), gate(gate), down(down), input(input), up_layer(c.embed_dim, c.hidden_dim, FrTensor::view(up.weight)),
       gate_layer(c.embed_dim, c.hidden_dim, FrTensor::view(gate.weight)), down_layer(c.hidden_dim, c.embed_dim, FrTensor::view(down.weight)), up_rescale(c.sf_linear),
-      gate_rescale(c.sf_gate), hidden_rescale(c.sf_linear), down_rescale(c.sf_linear), swiglu(c.swiglu_low, c.swiglu_len, swiglu_values) {}
+      gate_rescale(c.sf_gate), hidden_rescale(c.sf_linear), down_rescale(c.sf_linear), swiglu(c.swiglu_low, c.swiglu_len, swiglu_values) {
+    up_rescale.lean = gate_rescale.lean = hidden_rescale.lean = down_rescale.lean = true;
+}
 const FrTensor& FfnBlock::forward() {
     up_out.emplace(up_layer(input));
     up_out_.emplace(up_rescale.rescale(*up_out, true));            // int32 forms: the activation lookup and the product below read them

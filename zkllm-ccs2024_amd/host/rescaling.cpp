@@ -15,11 +15,15 @@ FrTensor Rescaling::rescale(const FrTensor& X, bool ints_out) {
     // the rescaled values too, when they fit (activations do): lookups, products and evaluations downstream read that form
     // (asked for by the caller: whether they fit is read back, a host round trip that a block which shares the device with
     // the openings' kernels pays with milliseconds)
+    // lean: the field elements of the remainders are written only where something reads them
+    // (the same condition under which prove_begin pads the int32 form alone and the lookup job reads nothing else)
+    const bool ints_only = lean && zk_lookup_ints_suffice((size_t)1 << ceilLog2(X.size), tl_rem.table.size);
+    void* rem_fr = ints_only ? nullptr : rem_tensor_ptr->gpu_data;
     if (ints_out) {
         int fits = 0;
-        ZKC(zk_rescale_ints_both(out.gpu_data, out.ints_for_producer(), &fits, rem_tensor_ptr->gpu_data, rem_hold->ints_for_producer(), X.gpu_data, scaling_factor, X.size, nullptr));
+        ZKC(zk_rescale_ints_both(out.gpu_data, out.ints_for_producer(), &fits, rem_fr, rem_hold->ints_for_producer(), X.gpu_data, scaling_factor, X.size, nullptr));
         if (!fits) out.drop_kept();
-    } else ZKC(zk_rescale_ints(out.gpu_data, rem_tensor_ptr->gpu_data, rem_hold->ints_for_producer(), X.gpu_data, scaling_factor, X.size, nullptr));
+    } else ZKC(zk_rescale_ints(out.gpu_data, rem_fr, rem_hold->ints_for_producer(), X.gpu_data, scaling_factor, X.size, nullptr));
     return out;
 }
 Rescaling::~Rescaling() {}

@@ -12,6 +12,11 @@ class Rescaling {
     FrTensor* rem_tensor_ptr;   // the remainders of the last operator() call (owned through rem_hold)
 
     Rescaling(uint scaling_factor);
+    // Addition.  With lean set, operator() writes the remainders in their int32 form ONLY where their range proof reads nothing
+    // else (a lookup job large enough at the tensor's padded length, zk_lookup_ints_suffice): the field elements of
+    // *rem_tensor_ptr then stay unwritten.  For a caller that hands the object to prove() and never reads the remainders
+    // itself (the layer's blocks).
+    bool lean = false;
     FrTensor operator()(const FrTensor& X);
     // addition: operator() that, with ints_out, also gives the rescaled tensor an int32 form when every value fits (one
     // host round trip): for outputs that go into a table lookup or a product with another such tensor
