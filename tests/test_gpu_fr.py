@@ -303,6 +303,67 @@ def test_zkfc_forward_and_proof_transcript(pv, orc, B, I, O, mode):
     pv.lib.zkp_set_matmul_mode(ctypes.c_int(0))
 
 
+def test_zkfc_proof_with_an_input_axis_that_needs_rounds_of_their_own(pv, orc):
+    """An input axis of 11008 (the 7B down projection's; 14 index bits): the inner-product sumcheck runs one round as launches of
+    its own before the single-workgroup kernel takes the other thirteen, all queued ahead by zkFC::prove_begin.  Transcript
+    and output are the oracle's."""
+    B, I, O = 4, 11008, 8
+    rng = np.random.default_rng(77)
+    X = np.round(rng.normal(0, 0.02, (B, I)) * 65536).astype(np.int32)
+    W = np.round(rng.normal(0, 0.02, (I, O)) * 65536).astype(np.int32)
+    got_Y, got_t = pv.zkfc_scenario(X, W, seed=777, matmul_mode=0)
+    orc.orc_seed(777)
+    orc.orc_transcript_clear()
+    exp_Y = np.zeros((B * O, 8), np.uint32)
+    orc_check(orc.orc_zkfc(X, W, B, I, O, exp_Y, np.zeros(8, np.uint32)))
+    exp_t = orc_transcript(orc)
+    assert (got_Y == exp_Y).all()
+    assert got_t.shape == exp_t.shape and (got_t == exp_t).all()
+
+
+def test_deferred_results_arrive_in_call_order_with_the_values_of_the_immediate_calls(hip):
+    """zk_defer_begin / _end / _wait: evaluations and inner-product rounds queued without waiting deliver, in call order, what the
+    same calls return when each waits for itself; the host outputs of the deferred calls are left alone."""
+    rng = np.random.default_rng(31)
+    n, k = 5000, 13
+    a = hip.upload(fr_array([int(x) % R_MOD for x in rng.integers(-2 ** 40, 2 ** 40, n)]))
+    b = hip.upload(mt_random_vec(np.random.RandomState(32), n))
+    u = mt_random_vec(np.random.RandomState(33), k)
+    n2 = 20000
+    c = hip.upload(mt_random_vec(np.random.RandomState(34), n2))
+    d = hip.upload(mt_random_vec(np.random.RandomState(35), n2))
+
+    def calls(out):
+        hip.call("zk_fr_me", out[0], ctypes.c_void_p(a), ctypes.c_size_t(n), u, ctypes.c_int(k), None)
+        hip.call("zk_ip_round", out[1], ctypes.c_void_p(c), ctypes.c_void_p(d), ctypes.c_size_t(n2), ctypes.c_size_t(16384), None)
+        hip.call("zk_ip_sumcheck_small", out[2], out[3], ctypes.c_void_p(a), ctypes.c_void_p(b), ctypes.c_uint32(n), u, ctypes.c_int(k), None)
+        hip.call("zk_fr_me", out[4], ctypes.c_void_p(b), ctypes.c_size_t(n), u, ctypes.c_int(k), None)
+
+    shapes = [(1, 8), (3, 8), (3 * k, 8), (2, 8), (1, 8)]
+    want = [np.zeros(sh, np.uint32) for sh in shapes]
+    calls(want)
+    assert all(w.any() for w in want)
+    batch = ctypes.c_void_p()
+    hip.call("zk_defer_begin", ctypes.byref(batch))
+    untouched = [np.full(sh, 0xA5A5A5A5, np.uint32) for sh in shapes]
+    calls(untouched)
+    hip.call("zk_defer_end", batch, None)
+    got = np.zeros((64, 8), np.uint32)
+    cnt = ctypes.c_size_t()
+    hip.call("zk_defer_wait", batch, got, ctypes.c_size_t(64), ctypes.byref(cnt))
+    hip.call("zk_defer_free", batch)
+    # call order: evaluation, round (three sums), small sumcheck (3k polynomials' values, then the two folded values), evaluation
+    flat = np.concatenate([want[0], want[1], want[2], want[3], want[4]])
+    assert cnt.value == flat.shape[0] and (got[:cnt.value] == flat).all()
+    assert (untouched[0] == 0xA5A5A5A5).all() and (untouched[1] == 0xA5A5A5A5).all() and (untouched[4] == 0xA5A5A5A5).all()
+    # a second batch on the same thread after the first was released, and immediate calls work again in between
+    again = [np.zeros(sh, np.uint32) for sh in shapes]
+    calls(again)
+    assert all((x == y).all() for x, y in zip(again, want))
+    for p in (a, b, c, d):
+        hip.free(p)
+
+
 def test_row_sums_of_squares_in_double_follow_a_plain_loop():
     """zk_row_sumsq_f64 must round exactly as `for j: acc += (x[j] / scale) ** 2` does: Python floats are IEEE doubles and
     every operation involved is exactly rounded, so the device result is compared bit for bit."""
