@@ -503,13 +503,15 @@ def main():
                                "the rest of the proof; traffic was measured for the kernel alone at 262144 pairs (roofline_fold_alone)"}
     if lk_launches:
         out["roofline_lookup_round_in_layer"] = {
-            "kernel": "k_lookup_round<false,true> (first round of the hinted lookup sumchecks, every launch of the timed layers)", "bound": "hbm",
+            "kernel": "k_lookup_first2_29 (the first TWO rounds of the lookup sumchecks over int32 queries in one pass, 29-bit limbs; every launch of the timed layers; "
+                      "pairs counts the first round's)", "bound": "hbm",
             "achieved": lk_bytes / (lk_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": lk_bytes / (lk_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "traffic": None, "launches": int(lk_launches), "pairs": int(lk_pairs), "total_ms_in_timed_region": lk_ms,
-            "note": "algorithmic bytes (per pair: the two queries -- 4 B each where they are read from their int32 forms as the softmax planes and rescaling "
-                    "remainders are (a mapping table's outputs are not read when they were gathered by these queries), else 32 B / 64 B; the eq weight 32 B; two folded values out 64 B; the next "
-                    "round's eq table 16 B) over the summed launch durations; the launches share the device with each other and with the openings, and "
-                    "with int32 queries the kernel is bound by its table gathers and instruction issue, not by these bytes"}
+            "note": "algorithmic bytes (per quad of queries, i.e. two first-round pairs: four queries in int32 form 16 B -- a mapping table's outputs are not read when "
+                    "they were gathered by these queries --, two eq weights 64 B, the second round's two folded values out 64 B, a half share of the third "
+                    "round's eq table 48 B; the first round's folded values are never written) over the summed launch durations; the launches share the device "
+                    "with each other, with the openings and with the main stream; alone the kernel is bound by instruction issue (4 450 lane instructions per "
+                    "quad) and its table gathers, not by these bytes (profiles/layer_c5_seq2048_alone_valu_bytes.txt)"}
     if lr_launches:
         # ~1750 vector instructions per pair (profiles/fr_mul_fold_msm_pmc.txt: SQ_INSTS_VALU of the kernel alone) of which 855 are limb multiply-adds
         lr_tops = lr_pairs * 855.0 / (lr_ms * 1e-3) / 1e12
@@ -667,16 +669,15 @@ def main():
     look_total_ms = (time.perf_counter() - t0) * 1e3
     l_ms, l_launches, l_pairs, l_bytes = read_lookup_timer()
     if l_launches:
-        out["roofline_lookup_round"] = {"kernel": "k_lookup_round<false,true> alone: first round of tLookupRangeMapping::prove, 2^27 queries uniformly spread over 2^20 entries",
+        out["roofline_lookup_round"] = {"kernel": "k_lookup_first2_29 alone: first two rounds of tLookupRangeMapping::prove in one pass, 2^27 queries uniformly spread over 2^20 entries",
                                         "bound": "hbm", "achieved": l_bytes / (l_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                         "frac": l_bytes / (l_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": l_ms / l_launches, "pairs": int(l_pairs),
                                         "whole_proof_ms": look_total_ms,
-                                        "note": "algorithmic 120 B per pair (two queries read from their int32 form: 8 B; eq weight, two folded values out, "
-                                                "next eq table); the kernel also gathers a 64-byte record (table entry and its inverse) per query from a 64 MiB table (the outputs "
-                                                "were gathered by these queries from this table and every entry is what the integers say, so nothing else is read per query) "
-                                                "and does three field products and one unreduced one per pair (SQ_INSTS_VALU, FETCH_SIZE, WRITE_SIZE of "
-                                                "this launch in profiles/fr_mul_fold_msm_pmc.txt) -- bound by the gathers and instruction issue; with the queries read as field elements (240 B per "
-                                                "pair) the same round took 7.6 ms.  The later rounds run at 3.6 TB/s and 79 % of the VALU slots (instruction issue binds there)"}
+                                        "note": "algorithmic 192 B per quad = 96 B per first-round pair (four queries read from their int32 form 16 B, two eq weights 64 B, the second "
+                                                "round's two folded values out 64 B, a half share of the third round's eq table 48 B); the kernel also gathers a 64-byte record (table "
+                                                "entry and its inverse) per query from a 64 MiB table (the outputs were gathered by these queries from this table and every entry is what "
+                                                "the integers say, so nothing else is read per query) and executes about 4 450 lane instructions per quad -- bound by instruction issue and "
+                                                "the gathers; as two passes (first round 4.5 ms, second 2.1 ms) the same work took 6.6 ms"}
     del keep, look
 
     # ---- CPU baseline: the oracle's restatement of the reference's algorithm on this host's cores ---------------------------------------
