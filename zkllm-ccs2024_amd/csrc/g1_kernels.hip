@@ -354,12 +354,8 @@ static __device__ __attribute__((noinline)) G1Jac g1_mul_glv(const G1Jac& P, con
 // small positive ones, instead of r's high bytes in every one of them.  A window byte above 127 becomes byte - 256
 // and carries one into the next window; the top window of a value below 2^254 cannot overflow.
 struct RecodeBatch { int8_t* D[OB_MAX]; const Fr* S[OB_MAX]; };      // blockIdx.y names the pair
-__global__ void __launch_bounds__(256) k_msm_recode(const RecodeBatch rb, size_t n) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    int8_t* __restrict__ D = rb.D[blockIdx.y];
-    const Fr* __restrict__ S = rb.S[blockIdx.y];
-    const Fr sv = S[i];
+// the digits of scalar i of n (standard form)
+__device__ __forceinline__ void msm_recode_store(int8_t* __restrict__ D, size_t n, size_t i, const Fr& sv) {
     Fr ng;
     uint32_t br = 0;
 #pragma unroll
@@ -380,6 +376,11 @@ __global__ void __launch_bounds__(256) k_msm_recode(const RecodeBatch rb, size_t
         }
     }
     D[(size_t)MW * n + i] = flip ? 1 : 0;
+}
+__global__ void __launch_bounds__(256) k_msm_recode(const RecodeBatch rb, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    msm_recode_store(rb.D[blockIdx.y], n, i, rb.S[blockIdx.y][i]);
 }
 
 // sum over the NT lanes of a workgroup through the LDS pool (36 x NT words); every lane returns the total
@@ -740,7 +741,7 @@ __global__ void __launch_bounds__(GT) k_open_chain(G1Jac* __restrict__ pts0, con
 // are such commitments of the opened tensor -- what the caller states by passing them.
 struct CrossItem { G1Jac* wsum; G1Jac* part; const G1Jac* pts; const Fr* u_rows; const Fr* u; uint32_t nrows, k_rows; };
 struct CrossBatch { CrossItem it[OB_MAX]; };
-__device__ __forceinline__ void cross_target(uint32_t t, uint32_t& q, uint32_t& first_pattern, uint32_t& npat, uint32_t& slot) {
+__host__ __device__ __forceinline__ void cross_target(uint32_t t, uint32_t& q, uint32_t& first_pattern, uint32_t& npat, uint32_t& slot) {
     if (t == 0) { q = 0; first_pattern = 0; npat = 1; slot = 0; return; }
     q = (t - 1) >> 1;
     const uint32_t side = (t - 1) & 1u, four_q = 1u << (2 * q);
@@ -790,6 +791,33 @@ __global__ void __launch_bounds__(MT) k_open_cross_finish(const CrossBatch cb, u
     G1Jac* __restrict__ W = it.wsum + slot;
     if (lane == 0) W[0] = tot;
     else if (lane < (uint32_t)MW) W[lane] = g1_infinity();
+}
+// The same sums as bucket multi-scalar multiplications.  Term g = pattern * nrows + row of an opening, in the order `pts`
+// lays the points out, has the coefficient eq(u_rows, row) * c(pattern) -- c = 1 for the row commitments, the product of the
+// earlier rounds' challenges for a cross pattern -- and a target is the sum over a contiguous range of terms: one bucket sum
+// per target over the normalised points, with the digits of all terms written once, as k_msm_recode writes them
+// (D: (MW + 1) x terms bytes).  A term costs 32 mixed additions instead of a 129-step walk of its own.
+struct CrossDigitItem { int8_t* D; const Fr* u_rows; const Fr* u; uint32_t nrows, k_rows; };
+struct CrossDigitBatch { CrossDigitItem it[OB_MAX]; };
+// grid (ceil(most terms / 256), openings)
+__global__ void __launch_bounds__(256) k_open_cross_digits(const CrossDigitBatch cb, uint32_t npatterns) {
+    const CrossDigitItem& it = cb.it[blockIdx.y];
+    const size_t terms = (size_t)npatterns * it.nrows, i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= terms) return;
+    const uint32_t p = (uint32_t)(i / it.nrows), row = (uint32_t)(i - (size_t)p * it.nrows);
+    const Fr one = big_one_mont<8>();
+    Fr coef = one;
+    for (uint32_t j = 0; j < it.k_rows; ++j) coef = mont_mul(coef, ((row >> j) & 1u) ? it.u_rows[j] : sub(one, it.u_rows[j]));
+    if (p != 0) {
+        uint32_t q = 0, first = 1;                      // the patterns of round q: T0's 4^q, then T1's
+        while (p >= first + (2u << (2 * q))) { first += 2u << (2 * q); ++q; }
+        const uint32_t pl = (p - first) & ((1u << (2 * q)) - 1u), a = pl >> q, b = pl & ((1u << q) - 1u);
+        for (uint32_t k = 0; k < q; ++k) {
+            const Fr uk = it.u[k], nk = sub(one, uk);
+            coef = mont_mul(coef, mont_mul(((a >> k) & 1u) ? uk : nk, ((b >> k) & 1u) ? nk : uk));
+        }
+    }
+    msm_recode_store(it.D, terms, i, from_mont(coef));
 }
 // ---- the fold on 29-bit-limb affine points ----------------------------------------------------------------------------------
 // The rounds of an opening keep the generators in ONE form: affine, 29-bit limbs (A29; all-zero limbs = infinity), canonical
@@ -1862,6 +1890,79 @@ struct OpenJob {
 struct OpenItem { const void* scalars; const void* gens; const A29* prep; const uint32_t* u; const A29* comb = nullptr; const A29* comb2 = nullptr;
                   const void* rows = nullptr; uint32_t nrows = 0; const uint32_t* u_rows = nullptr; int k_rows = 0; int cross_rounds = 0;
                   const A29* comb3 = nullptr; };
+// The targets of every opening of a batch (T of round 0, then T0, T1 of the first `full` rounds) as bucket sums over the
+// openings' [pattern][row] points, on aux.  The raw buckets' reductions are appended to `later`: the caller runs them with
+// those of its halving rounds, so the 248 doublings of a reduction are waited for once per job.
+static bool cross_walks() { static const bool on = [] { const char* e = getenv("ZKLLM_OPEN_CROSS_WALKS"); return e && e[0] == '1'; }(); return on; }
+static int open_cross_sums_queue(Arena& arena, const OpenItem* items, int count, int full, G1Jac* wsum, uint32_t wstride, const Fr* const* urow_dev, const Fr* U_dev, int rounds,
+                                 hipStream_t aux, std::vector<PointDesc>& later) {
+    const uint32_t ntargets = 1u + 2u * (uint32_t)full;
+    const uint32_t npatterns = 1u + 2u * (((1u << (2 * full)) - 1u) / 3u);
+    const uint32_t widest = full ? (1u << (2 * (full - 1))) : 1u;           // patterns of the largest target
+    CrossDigitBatch db;
+    const A29* base[OB_MAX];
+    const int8_t* digs[OB_MAX];
+    size_t most_terms = 0, most_count = 0;
+    for (int i = 0; i < count; ++i) {
+        const size_t terms = (size_t)npatterns * items[i].nrows;
+        ZK_ARG(items[i].nrows >= 1 && terms < (1ull << 31), "zk_g1_open: bad row count");
+        most_terms = std::max(most_terms, terms);
+        most_count = std::max(most_count, (size_t)widest * items[i].nrows);
+        Scratch& aff = arena.add(sizeof(G1Affine) * terms);
+        Scratch& a29 = arena.add(sizeof(A29) * terms);
+        Scratch& dg = arena.add((size_t)(MW + 1) * terms);
+        if (aff.rc || a29.rc || dg.rc) return aff.rc ? aff.rc : (a29.rc ? a29.rc : dg.rc);
+        hipLaunchKernelGGL(k_g1_normalize<true>, dim3(cdiv(cdiv(terms, CH), GT)), dim3(GT), 0, aux, aff.p, (const G1Jac*)items[i].rows, terms);
+        hipLaunchKernelGGL(k_g1aff_to_a29, dim3(cdiv(terms, 256)), dim3(256), 0, aux, a29.as<A29>(), aff.as<G1Affine>(), terms);
+        base[i] = a29.as<A29>();
+        digs[i] = dg.as<int8_t>();
+        db.it[i] = CrossDigitItem{dg.as<int8_t>(), urow_dev[i], U_dev + (size_t)i * rounds, items[i].nrows, (uint32_t)items[i].k_rows};
+    }
+    for (int i = count; i < OB_MAX; ++i) db.it[i] = db.it[0];
+    hipLaunchKernelGGL(k_open_cross_digits, dim3(cdiv(most_terms, 256), count), dim3(256), 0, aux, db, npatterns);
+    ZK_LAUNCH_CHECK();
+    const uint32_t chunks = cdiv(most_count, MSEG);
+    const uint32_t cps = (chunks + 255u) / 256u;
+    const uint32_t nseg = (chunks + cps - 1) / cps;
+    const uint32_t n_msm = ntargets * (uint32_t)count;
+    Scratch& partial = arena.add(sizeof(G1Jac) * n_msm * MW * (size_t)nseg * MT);
+    if (partial.rc) return partial.rc;
+    const int per = std::max(1, OB_SUMS / (int)ntargets);                  // openings whose targets fit one launch's descriptors
+    for (int g0 = 0; g0 < count; g0 += per) {
+        const int gc = std::min(per, count - g0);
+        MsmDescs<OB_SUMS> descs;
+        uint32_t z = 0;
+        for (int i = g0; i < g0 + gc; ++i)
+            for (uint32_t t = 0; t < ntargets; ++t) {
+                uint32_t q, p0, npat, slot;
+                cross_target(t, q, p0, npat, slot);
+                const uint32_t terms = npatterns * items[i].nrows, off = p0 * items[i].nrows;
+                descs.d[z++] = MsmDesc{digs[i], base[i], terms, npat * items[i].nrows, 1u, off, 1u, off, 0u};
+            }
+        const uint32_t used = z;
+        for (; z < (uint32_t)OB_SUMS; ++z) descs.d[z] = MsmDesc{digs[0], base[0], 0u, 0u, 1u, 0u, 1u, 0u, 0u};
+        hipLaunchKernelGGL(k_msm_seg<OB_SUMS>, dim3(nseg, MW, used), dim3(MSL), 0, aux, partial.as<G1Jac>() + (size_t)g0 * ntargets * MW * nseg * MT, descs, (const MsmDesc*)nullptr,
+                           nseg, cps);
+    }
+    const G1Jac* cur = partial.as<G1Jac>();
+    uint32_t ns = nseg;
+    while (ns > 1) {
+        const uint32_t ng = (ns + 7) / 8;
+        Scratch& nxt = arena.add(sizeof(G1Jac) * n_msm * MW * (size_t)ng * MT);
+        if (nxt.rc) return nxt.rc;
+        hipLaunchKernelGGL(k_msm_bucket_fold, dim3(n_msm * MW, ng), dim3(MT), 0, aux, nxt.as<G1Jac>(), cur, ns);
+        cur = nxt.as<G1Jac>();
+        ns = ng;
+    }
+    ZK_LAUNCH_CHECK();
+    for (int i = 0; i < count; ++i)
+        for (uint32_t t = 0; t < ntargets; ++t) {
+            uint32_t q, p0, npat, slot;
+            cross_target(t, q, p0, npat, slot);
+            later.push_back(PointDesc{cur + ((size_t)i * ntargets + t) * MW * ns * MT, wsum + (size_t)wstride * i + slot, ns, 0u});
+        }
+    return 0;
+}
 // rows (optional): commitments of the opened tensor's rows, [pattern][row] as k_open_cross_part takes them -- the row
 // commitments alone (cross_rounds = 0) or with the cross patterns of the first cross_rounds rounds
 static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, int rounds, hipStream_t st, hipStream_t aux) {
@@ -1929,7 +2030,18 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
         for (int r = 0; r < rounds && !(sz <= (size_t)TAIL_N && rounds - r <= TAIL_LEVELS); ++r) { ++halving; sz = (sz + 1) / 2; }
         rounds_from_rows = std::min(halving, std::max(cross_r, 1));
     }
-    if (rounds_from_rows > 0) {
+    std::vector<PointDesc> later;        // bucket reductions that nothing waits for before the end: one launch behind the last round
+    if (rounds_from_rows > 0 && !cross_walks()) {
+        if (aux != st) {          // the challenges travel on st
+            hipEvent_t up;
+            ZK_HIP(hipEventCreateWithFlags(&up, hipEventDisableTiming));
+            job.events.push_back(up);
+            ZK_HIP(hipEventRecord(up, st));
+            ZK_HIP(hipStreamWaitEvent(aux, up, 0));
+        }
+        int rc = open_cross_sums_queue(job.arena, items, count, std::min(rounds_from_rows, cross_r), wsum.as<G1Jac>(), wstride, urow_dev, U_dev, rounds, aux, later);
+        if (rc) return rc;
+    } else if (rounds_from_rows > 0) {
         // targets: T of round 0, then T0, T1 of every round whose bucket sums were left out
         const int full = std::min(rounds_from_rows, cross_r);
         const uint32_t ntargets = 1u + 2u * (uint32_t)full;
@@ -2010,7 +2122,6 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
             r_first = JUMP_ROUNDS;
         }
     }
-    std::vector<PointDesc> later;        // the bucket reductions of the halving rounds: one launch behind the last of them
     for (int r = r_first; r < rounds; ++r) {
         if (size <= (size_t)TAIL_N && rounds - r <= TAIL_LEVELS) {
             int rc = open_tail_launch(cs, cg, count, size, rounds - r, r, rounds, pts.as<G1Jac>(), U_dev, job.pin, (char*)jdev.p + JOB_U_BYTES, job.arena, st);

@@ -81,6 +81,21 @@ __global__ void __launch_bounds__(TPB) k_finish(Fr* __restrict__ out, const Fr* 
     for (uint32_t i = threadIdx.x; i < nb; i += TPB) acc[0] = add(acc[0], p[i]);
     block_reduce_store<1>(acc, out);
 }
+// The partial sums of all rounds of a job at once, behind its last round: no round waits for the one before to be summed
+// (the next round needs the fold challenge, not the sums).  Round r's K[r] sums: nb[r] partials each from part + off[r], into
+// sums[r * per_round + k].  grid (most sums of a round, rounds)
+static constexpr int FINISH_ROUNDS_MAX = 64;
+struct FinishRounds { uint32_t off[FINISH_ROUNDS_MAX], nb[FINISH_ROUNDS_MAX]; uint8_t k[FINISH_ROUNDS_MAX]; };
+struct PartSlice { Fr* p; template <class T> T* as() const { return reinterpret_cast<T*>(p); } };      // a round's share of the partial sums
+__global__ void __launch_bounds__(TPB) k_finish_rounds(Fr* __restrict__ sums, const Fr* __restrict__ part, const FinishRounds fr, uint32_t per_round) {
+    const uint32_t r = blockIdx.y;
+    if (blockIdx.x >= fr.k[r]) return;
+    Fr acc[1] = {big_zero<8>()};
+    const uint32_t nb = fr.nb[r];
+    const Fr* p = part + fr.off[r] + (size_t)blockIdx.x * nb;
+    for (uint32_t i = threadIdx.x; i < nb; i += TPB) acc[0] = add(acc[0], p[i]);
+    block_reduce_store<1>(acc, sums + (size_t)r * per_round);
+}
 static inline unsigned reduce_grid(size_t n) {
     size_t b = (n + TPB - 1) / TPB;
     if (b > 1024) b = 1024;
@@ -2247,18 +2262,31 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
     job.rounds = rounds;
     job.per_round = 11;
     job.n1 = n1;
+    ZK_ARG(rounds <= FINISH_ROUNDS_MAX, "lookup sumcheck: too many rounds");
     Scratch& sums = job.arena.add(sizeof(Fr) * 11 * rounds);
-    Scratch& part = job.arena.add(sizeof(Fr) * 11 * reduce_grid(D / 2));
+    // every round keeps its partial sums: one launch sums them all behind the last round
+    size_t part_total = 0;
+    {
+        size_t c = D;
+        for (int r = 0; r < rounds; ++r) { c >>= 1; part_total += 11 * (size_t)reduce_grid(c); }
+    }
+    Scratch& part_all = job.arena.add(sizeof(Fr) * part_total);
     if (sums.rc) return sums.rc;
-    if (part.rc) return part.rc;
+    if (part_all.rc) return part_all.rc;
     job.sums = sums.as<Fr>();
     ZK_HIP(hipMemsetAsync(sums.p, 0, sizeof(Fr) * 11 * rounds, st));
+    FinishRounds fin;
+    memset(&fin, 0, sizeof(fin));
+    size_t part_at = 0;
+    int fin_rounds = 0;              // rounds whose sums come from partials (the rest: the tail kernel's)
+    PartSlice part{nullptr};
     const Fr *cA = A, *cS = S, *cB = B, *cT = T, *cm = m, *cE = E;
     Fr* eqbuf[2] = {nullptr, nullptr};
     size_t cur = D;
     for (int r = 0; r < rounds; ++r) {
         const size_t half = cur >> 1;
         const bool phase2 = r >= n1;
+        part.p = part_all.as<Fr>() + part_at;
         if (half <= (size_t)TAIL_HALF && rounds - r <= TAIL_ROUNDS) {
             const int rest = rounds - r;
             Scratch& work = job.arena.add(sizeof(Fr) * 12 * half);
@@ -2306,9 +2334,11 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
                 const double q = (hs->sout_ints && !hs->trusted_out) ? 32.0 : 16.0;
                 g_round_timer.bytes += (double)h2 * (q + 64.0 + 64.0 + (nE3 ? 48.0 : 0.0));
             }
-            hipLaunchKernelGGL(k_finish, dim3(5), dim3(TPB), 0, st, sums.as<Fr>() + (size_t)r * 11, part.as<Fr>(), nb2);
-            hipLaunchKernelGGL(k_finish, dim3(5), dim3(TPB), 0, st, sums.as<Fr>() + (size_t)(r + 1) * 11, part.as<Fr>() + 5 * (size_t)nb2, nb2);
             ZK_LAUNCH_CHECK();
+            fin.off[r] = (uint32_t)part_at; fin.nb[r] = nb2; fin.k[r] = 5;
+            fin.off[r + 1] = (uint32_t)(part_at + 5 * (size_t)nb2); fin.nb[r + 1] = nb2; fin.k[r + 1] = 5;
+            part_at += 10 * (size_t)nb2;
+            fin_rounds = r + 2;
             cA = w2; cS = w2 + h2;
             cur = h2;
             if (nE3) cE = nE3;
@@ -2387,12 +2417,18 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
                 g_later_timer.bytes += (double)half * (128.0 + 32.0 + 64.0 + (nE ? 16.0 : 0.0));
             }
         }
-        hipLaunchKernelGGL(k_finish, dim3(phase2 ? 11 : 5), dim3(TPB), 0, st, sums.as<Fr>() + (size_t)r * 11, part.as<Fr>(), nb);
         ZK_LAUNCH_CHECK();
+        fin.off[r] = (uint32_t)part_at; fin.nb[r] = nb; fin.k[r] = phase2 ? 11 : 5;
+        part_at += (size_t)(phase2 ? 11 : 5) * nb;
+        fin_rounds = r + 1;
         cA = w; cS = w + half;
         if (phase2) { cB = w + 2 * half; cT = w + 3 * half; cm = w + 4 * half; }
         cur = half;
         if (nE) cE = nE;
+    }
+    if (fin_rounds) {
+        hipLaunchKernelGGL(k_finish_rounds, dim3(11, fin_rounds), dim3(TPB), 0, st, sums.as<Fr>(), part_all.as<Fr>(), fin, 11u);
+        ZK_LAUNCH_CHECK();
     }
     return 0;
 }
@@ -2402,11 +2438,22 @@ static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, 
     while (((size_t)1 << rounds) < N) ++rounds;
     job.rounds = rounds;
     job.per_round = K + 1;
+    ZK_ARG(rounds <= FINISH_ROUNDS_MAX, "Hadamard sumcheck: too many rounds");
     Scratch& sums = job.arena.add(sizeof(Fr) * (K + 1) * rounds);
-    Scratch& part = job.arena.add(sizeof(Fr) * (K + 1) * reduce_grid(N / 2));
+    size_t part_total = 0;            // every round keeps its partial sums: one launch sums them all behind the last round
+    {
+        size_t c = N;
+        for (int r = 0; r < rounds; ++r) { c >>= 1; part_total += (size_t)(K + 1) * reduce_grid(c); }
+    }
+    Scratch& part_all = job.arena.add(sizeof(Fr) * part_total);
     if (sums.rc) return sums.rc;
-    if (part.rc) return part.rc;
+    if (part_all.rc) return part_all.rc;
     job.sums = sums.as<Fr>();
+    FinishRounds fin;
+    memset(&fin, 0, sizeof(fin));
+    size_t part_at = 0;
+    int fin_rounds = 0;
+    PartSlice part{nullptr};
     const Fr* cur[4];
     for (int i = 0; i < K; ++i) cur[i] = Xs[i];
     const Fr* cE = E;
@@ -2414,6 +2461,7 @@ static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, 
     size_t n = N;
     for (int r = 0; r < rounds; ++r) {
         const size_t half = n >> 1;
+        part.p = part_all.as<Fr>() + part_at;
         if (half <= (size_t)TAIL_HALF && rounds - r <= TAIL_ROUNDS) {
             const int rest = rounds - r;
             Scratch& work = job.arena.add(sizeof(Fr) * (K + 1) * half);
@@ -2462,11 +2510,17 @@ static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, 
         else
             switch (K) { HADS_ROUND(1) HADS_ROUND(2) HADS_ROUND(3) HADS_ROUND(4) }
 #undef HADS_ROUND
-        hipLaunchKernelGGL(k_finish, dim3(K + 1), dim3(TPB), 0, st, sums.as<Fr>() + (size_t)r * (K + 1), part.as<Fr>(), nb);
         ZK_LAUNCH_CHECK();
+        fin.off[r] = (uint32_t)part_at; fin.nb[r] = nb; fin.k[r] = (uint8_t)(K + 1);
+        part_at += (size_t)(K + 1) * nb;
+        fin_rounds = r + 1;
         for (int i = 0; i < K; ++i) cur[i] = w + (size_t)i * half;
         n = half;
         if (nE) cE = nE;
+    }
+    if (fin_rounds) {
+        hipLaunchKernelGGL(k_finish_rounds, dim3(K + 1, fin_rounds), dim3(TPB), 0, st, sums.as<Fr>(), part_all.as<Fr>(), fin, (uint32_t)(K + 1));
+        ZK_LAUNCH_CHECK();
     }
     return 0;
 }
@@ -2865,9 +2919,17 @@ int zk_hadamard_product_sumcheck(uint32_t* proof_host, const void* a, const void
     const size_t half = (n + 1) / 2, etab = (size_t)1 << (k - 1);
     Scratch& E = arena.add(sizeof(Fr) * (etab + etab / 2 + 1));          // eq tables, ping-pong
     Scratch& W = arena.add(sizeof(Fr) * 2 * (half + (half + 1) / 2 + 1));   // folded a, b, ping-pong
-    Scratch& part = arena.add(sizeof(Fr) * 3 * reduce_grid(half));
+    size_t part_total = 0;            // every round keeps its partial sums: one launch sums them all behind the last round
+    {
+        size_t c = n;
+        for (int r = 0; r < k; ++r) { c = (c + 1) / 2; part_total += 3 * (size_t)reduce_grid(c); }
+    }
+    Scratch& part = arena.add(sizeof(Fr) * part_total);
     Scratch& sums = arena.add(sizeof(Fr) * (3 * (size_t)k + 2));
     if (E.rc || W.rc || part.rc || sums.rc) return E.rc ? E.rc : (W.rc ? W.rc : (part.rc ? part.rc : sums.rc));
+    FinishRounds fin;
+    memset(&fin, 0, sizeof(fin));
+    size_t part_at = 0;
     int rc = eq_table_queue(E.as<Fr>(), u + 8, k - 1, arena, st);
     if (rc) { (void)hipStreamSynchronize(st); return rc; }
     Fr* ebuf[2] = {E.as<Fr>(), E.as<Fr>() + etab};
@@ -2879,13 +2941,16 @@ int zk_hadamard_product_sumcheck(uint32_t* proof_host, const void* a, const void
     for (int r = 0; r < k; ++r) {
         const size_t out = (cur + 1) / 2;
         const unsigned nb = reduce_grid(out);
-        hipLaunchKernelGGL(k_hp_round, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), wa[r & 1], wb[r & 1], ebuf[(r + 1) & 1], ca, cb, ce, to_mont(load_fr(v + 8 * r)), cur, out, ecur / 2);
-        hipLaunchKernelGGL(k_finish, dim3(3), dim3(TPB), 0, st, sums.as<Fr>() + 3 * (size_t)r, part.as<Fr>(), nb);
+        hipLaunchKernelGGL(k_hp_round, dim3(nb), dim3(TPB), 0, st, part.as<Fr>() + part_at, wa[r & 1], wb[r & 1], ebuf[(r + 1) & 1], ca, cb, ce, to_mont(load_fr(v + 8 * r)), cur, out, ecur / 2);
         ZK_LAUNCH_CHECK();
+        fin.off[r] = (uint32_t)part_at; fin.nb[r] = nb; fin.k[r] = 3;
+        part_at += 3 * (size_t)nb;
         ca = wa[r & 1]; cb = wb[r & 1]; ce = ebuf[(r + 1) & 1];
         cur = out;
         ecur /= 2;
     }
+    hipLaunchKernelGGL(k_finish_rounds, dim3(3, k), dim3(TPB), 0, st, sums.as<Fr>(), part.as<Fr>(), fin, 3u);
+    ZK_LAUNCH_CHECK();
     ZK_HIP(hipMemcpyAsync(sums.as<Fr>() + 3 * (size_t)k, ca, sizeof(Fr), hipMemcpyDeviceToDevice, st));
     ZK_HIP(hipMemcpyAsync(sums.as<Fr>() + 3 * (size_t)k + 1, cb, sizeof(Fr), hipMemcpyDeviceToDevice, st));
     void* stage = nullptr;

@@ -192,7 +192,7 @@ hipStream_t side_stream(int pool) {
     static unsigned next[2] = {0, 0};
     static int count[2] = {0, 0}, shared = 0;
     if (!count[0]) {
-        count[0] = 4; count[1] = 2;       // an opening job takes two consecutive streams of pool 0 (folds / bucket sums); two jobs in flight
+        count[0] = 8; count[1] = 2;       // an opening job takes two consecutive streams of pool 0 (folds / bucket sums); four jobs in flight
         if (const char* e = getenv("ZKLLM_SIDE_STREAMS")) {          // "openings,sumchecks[,shared]" (experiments)
             int a = 0, b2 = 0, c = 0;
             if (sscanf(e, "%d,%d,%d", &a, &b2, &c) >= 2 && a >= 1 && a <= 24 && b2 >= 1 && b2 <= 24) { count[0] = a; count[1] = b2; shared = c; }
