@@ -207,8 +207,11 @@ __global__ void __launch_bounds__(256) k_rowabs(unsigned long long* __restrict__
     if (threadIdx.x == 0) {
         unsigned long long gm = red[0][0], gs = red[1][0];
         for (int i = 1; i < 4; ++i) { gm = red[0][i] > gm ? red[0][i] : gm; gs = sat_add(gs, red[1][i]); }
-        atomicMax(out_max, gm);
-        atomicMax(out, gs);
+        // a row that raises neither figure leaves them alone: with one workgroup per row, tens of thousands of atomics on
+        // the same two words are what the launch would otherwise wait for (the figures only grow, so a stale read costs an
+        // atomic that changes nothing and never drops one that would)
+        if (gm > __atomic_load_n(out_max, __ATOMIC_RELAXED)) atomicMax(out_max, gm);
+        if (gs > __atomic_load_n(out, __ATOMIC_RELAXED)) atomicMax(out, gs);
     }
 }
 template <typename T> __global__ void __launch_bounds__(256) k_fr_to_int(T* __restrict__ out, const Fr* __restrict__ a, size_t n) {
