@@ -355,6 +355,10 @@ int zk_lookup_last_job_consistent_entries(uint32_t* n_ok, uint32_t* n_table);
  * 2^(k-1) < n <= 2^k; u, v: k challenges each.  proof_host: 3k + 2 values (per round the three terms evaluated at the
  * remaining u, then the folded a and b).  The three term tensors of the reference's step kernel are never materialised. */
 int zk_hadamard_product_sumcheck(uint32_t* proof_host, const void* a, const void* b, const uint32_t* u, const uint32_t* v, size_t n, int k, void* stream);
+/* the same in two halves: begin queues the rounds on a stream of the library's own, ordered behind what `stream` holds so far,
+ * and returns at once (u and v are copied; a and b stay alive and unmodified until end); end waits and delivers the values */
+int zk_hadamard_product_sumcheck_begin(void** handle, const void* a, const void* b, const uint32_t* u, const uint32_t* v, size_t n, int k, void* stream);
+int zk_hadamard_product_sumcheck_end(void* handle, uint32_t* proof_host);
 int zk_hadamard_prove_begin(void** handle, const void* const* Xs, int K, const uint32_t* u_eq, const uint32_t* v, size_t N, void* stream);
 /* the same where prepareds[i], when non-null, is the int32 form of Xs[i] (N elements): two tensors that both have one (the
  * mapped outputs of a softmax's segments, zksoftmax.cu:177-180) are read from it in the first round; same sums */

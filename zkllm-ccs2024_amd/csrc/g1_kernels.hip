@@ -739,8 +739,6 @@ __global__ void __launch_bounds__(GT) k_open_chain(G1Jac* __restrict__ pts0, con
 // Target t of an opening: 0 = T of round 0, 1 + 2q + side = T0_q / T1_q.  The results go where k_open_horner reads the window
 // sums of those points: the point in window 0, infinity above.  They equal the sums over all generators exactly when `pts`
 // are such commitments of the opened tensor -- what the caller states by passing them.
-struct CrossItem { G1Jac* wsum; G1Jac* part; const G1Jac* pts; const Fr* u_rows; const Fr* u; uint32_t nrows, k_rows; };
-struct CrossBatch { CrossItem it[OB_MAX]; };
 __host__ __device__ __forceinline__ void cross_target(uint32_t t, uint32_t& q, uint32_t& first_pattern, uint32_t& npat, uint32_t& slot) {
     if (t == 0) { q = 0; first_pattern = 0; npat = 1; slot = 0; return; }
     q = (t - 1) >> 1;
@@ -749,54 +747,11 @@ __host__ __device__ __forceinline__ void cross_target(uint32_t t, uint32_t& q, u
     first_pattern = 1 + 2 * (four_q - 1) / 3 + side * four_q;
     slot = (3 * q + 1 + side) * (uint32_t)MW;
 }
-// grid (chunks, targets, openings): chunk c of a target sums its terms [c MT, (c+1) MT) into part[(t chunks + c)]
-__global__ void __launch_bounds__(MT) k_open_cross_part(const CrossBatch cb) {
-    __shared__ uint32_t pool[36 * MT];
-    __shared__ int32_t walk_tab[57][MT];
-    const CrossItem& it = cb.it[blockIdx.z];
-    const uint32_t t = blockIdx.y, c = blockIdx.x, lane = threadIdx.x;
-    uint32_t q, p0, npat, slot;
-    cross_target(t, q, p0, npat, slot);
-    const uint32_t nrows = it.nrows, terms = npat * nrows, idx = c * MT + lane;
-    G1Jac acc = g1_infinity();
-    if (idx < terms) {
-        const uint32_t pl = idx / nrows, row = idx - pl * nrows;
-        const Fr one = big_one_mont<8>();
-        Fr coef = one;
-        for (uint32_t j = 0; j < it.k_rows; ++j) coef = mont_mul(coef, ((row >> j) & 1u) ? it.u_rows[j] : sub(one, it.u_rows[j]));
-        if (t != 0) {
-            const uint32_t a = pl >> q, b = pl & ((1u << q) - 1u);
-            for (uint32_t k = 0; k < q; ++k) {
-                const Fr uk = it.u[k], nk = sub(one, uk);
-                coef = mont_mul(coef, mont_mul(((a >> k) & 1u) ? uk : nk, ((b >> k) & 1u) ? nk : uk));
-            }
-        }
-        const G1Jac P = it.pts[(size_t)(p0 + pl) * nrows + row];
-        if (!is_zero(P.z) && !is_zero(coef)) acc = j29_to_jac(j29_mul_glv_lane<MT>(j29_from_jac(P), glv_split_device(from_mont(coef)), walk_tab));
-    }
-    const G1Jac tot = msm_block_sum(pool, acc, lane);
-    if (lane == 0) it.part[(size_t)t * gridDim.x + c] = tot;
-}
-// grid (targets, openings): the chunks of a target summed, the point written as window sums
-__global__ void __launch_bounds__(MT) k_open_cross_finish(const CrossBatch cb, uint32_t chunks) {
-    __shared__ uint32_t pool[36 * MT];
-    const CrossItem& it = cb.it[blockIdx.y];
-    const uint32_t t = blockIdx.x, lane = threadIdx.x;
-    uint32_t q, p0, npat, slot;
-    cross_target(t, q, p0, npat, slot);
-    const uint32_t used = (npat * it.nrows + MT - 1) / MT;            // chunks of this target that hold terms
-    G1Jac acc = g1_infinity();
-    for (uint32_t c = lane; c < used && c < chunks; c += MT) acc = g1_add(acc, it.part[(size_t)t * chunks + c]);
-    const G1Jac tot = msm_block_sum(pool, acc, lane);
-    G1Jac* __restrict__ W = it.wsum + slot;
-    if (lane == 0) W[0] = tot;
-    else if (lane < (uint32_t)MW) W[lane] = g1_infinity();
-}
-// The same sums as bucket multi-scalar multiplications.  Term g = pattern * nrows + row of an opening, in the order `pts`
+// These sums are bucket multi-scalar multiplications.  Term g = pattern * nrows + row of an opening, in the order `pts`
 // lays the points out, has the coefficient eq(u_rows, row) * c(pattern) -- c = 1 for the row commitments, the product of the
 // earlier rounds' challenges for a cross pattern -- and a target is the sum over a contiguous range of terms: one bucket sum
 // per target over the normalised points, with the digits of all terms written once, as k_msm_recode writes them
-// (D: (MW + 1) x terms bytes).  A term costs 32 mixed additions instead of a 129-step walk of its own.
+// (D: (MW + 1) x terms bytes).  A term costs 32 mixed additions (a scalar multiplication of its own would cost a 129-step walk).
 struct CrossDigitItem { int8_t* D; const Fr* u_rows; const Fr* u; uint32_t nrows, k_rows; };
 struct CrossDigitBatch { CrossDigitItem it[OB_MAX]; };
 // grid (ceil(most terms / 256), openings)
@@ -1441,7 +1396,7 @@ static CombK comb_of(const GlvK& k) {
         }
     return ck;
 }
-// given: what of this round's sums comes from commitments of the tensor's rows (k_open_cross_part) and is not summed here:
+// given: what of this round's sums comes from commitments of the tensor's rows (open_cross_sums_queue) and is not summed here:
 // 0 nothing, 1 T of the first round (no pair sums), 2 T0 and T1 as well (no bucket sums at all: the round is its fold)
 // later (optional): the reductions of this round's raw buckets are appended to it instead of launched (the caller runs them
 // all at once behind its last round); a round whose T comes from the pair sums (k_open_t_fix) reduces at once
@@ -1883,6 +1838,9 @@ struct OpenJob {
     std::vector<hipEvent_t> events;
     void* pin = nullptr;           // pinned host buffer behind the job's challenges and descriptors
     void* pin2 = nullptr;          // and behind the list of its rounds' bucket reductions
+    uint64_t ticket = 0;           // the launch thread's ticket while it queues the job's kernels
+    int queue_rc = 0;              // what queuing returned, and its message
+    std::string queue_err;
     ~OpenJob() { pinned_release(pin); pinned_release(pin2); }
 };
 // One opening of the batch: its scalars, its challenges (rounds x 8 limbs) and its generators -- Jacobian, or null when
@@ -1893,7 +1851,6 @@ struct OpenItem { const void* scalars; const void* gens; const A29* prep; const 
 // The targets of every opening of a batch (T of round 0, then T0, T1 of the first `full` rounds) as bucket sums over the
 // openings' [pattern][row] points, on aux.  The raw buckets' reductions are appended to `later`: the caller runs them with
 // those of its halving rounds, so the 248 doublings of a reduction are waited for once per job.
-static bool cross_walks() { static const bool on = [] { const char* e = getenv("ZKLLM_OPEN_CROSS_WALKS"); return e && e[0] == '1'; }(); return on; }
 static int open_cross_sums_queue(Arena& arena, const OpenItem* items, int count, int full, G1Jac* wsum, uint32_t wstride, const Fr* const* urow_dev, const Fr* U_dev, int rounds,
                                  hipStream_t aux, std::vector<PointDesc>& later) {
     const uint32_t ntargets = 1u + 2u * (uint32_t)full;
@@ -1963,7 +1920,7 @@ static int open_cross_sums_queue(Arena& arena, const OpenItem* items, int count,
         }
     return 0;
 }
-// rows (optional): commitments of the opened tensor's rows, [pattern][row] as k_open_cross_part takes them -- the row
+// rows (optional): commitments of the opened tensor's rows, [pattern][row] as open_cross_sums_queue takes them -- the row
 // commitments alone (cross_rounds = 0) or with the cross patterns of the first cross_rounds rounds
 static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, int rounds, hipStream_t st, hipStream_t aux) {
     ZK_ARG(n >= 1, "zk_g1_open: empty input");
@@ -2031,7 +1988,7 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
         rounds_from_rows = std::min(halving, std::max(cross_r, 1));
     }
     std::vector<PointDesc> later;        // bucket reductions that nothing waits for before the end: one launch behind the last round
-    if (rounds_from_rows > 0 && !cross_walks()) {
+    if (rounds_from_rows > 0) {
         if (aux != st) {          // the challenges travel on st
             hipEvent_t up;
             ZK_HIP(hipEventCreateWithFlags(&up, hipEventDisableTiming));
@@ -2041,31 +1998,6 @@ static int open_queue(OpenJob& job, const OpenItem* items, int count, size_t n, 
         }
         int rc = open_cross_sums_queue(job.arena, items, count, std::min(rounds_from_rows, cross_r), wsum.as<G1Jac>(), wstride, urow_dev, U_dev, rounds, aux, later);
         if (rc) return rc;
-    } else if (rounds_from_rows > 0) {
-        // targets: T of round 0, then T0, T1 of every round whose bucket sums were left out
-        const int full = std::min(rounds_from_rows, cross_r);
-        const uint32_t ntargets = 1u + 2u * (uint32_t)full;
-        uint32_t max_terms = 0;
-        for (int i = 0; i < count; ++i) max_terms = std::max(max_terms, (full ? (1u << (2 * (full - 1))) : 1u) * items[i].nrows);
-        const uint32_t chunks = cdiv(max_terms, MT);
-        Scratch& part = job.arena.add(sizeof(G1Jac) * (size_t)ntargets * chunks * count);
-        if (part.rc) return part.rc;
-        CrossBatch cb;
-        for (int i = 0; i < OB_MAX; ++i) {
-            const int k = i < count ? i : 0;
-            cb.it[i] = CrossItem{wsum.as<G1Jac>() + (size_t)wstride * k, part.as<G1Jac>() + (size_t)ntargets * chunks * k, (const G1Jac*)items[k].rows, urow_dev[k],
-                                 U_dev + (size_t)k * rounds, items[k].nrows, (uint32_t)items[k].k_rows};
-        }
-        if (aux != st) {          // the challenges travel on st
-            hipEvent_t up;
-            ZK_HIP(hipEventCreateWithFlags(&up, hipEventDisableTiming));
-            job.events.push_back(up);
-            ZK_HIP(hipEventRecord(up, st));
-            ZK_HIP(hipStreamWaitEvent(aux, up, 0));
-        }
-        hipLaunchKernelGGL(k_open_cross_part, dim3(chunks, ntargets, count), dim3(MT), 0, aux, cb);
-        hipLaunchKernelGGL(k_open_cross_finish, dim3(ntargets, count), dim3(MT), 0, aux, cb, chunks);
-        ZK_LAUNCH_CHECK();
     }
     size_t size = n;
     int halving_rounds = rounds;
@@ -2212,18 +2144,49 @@ static int open_begin_impl(void** handle, const OpenItem* items, int count, size
     ZK_ARG(handle != nullptr, "zk_g1_open_begin: null handle");
     hipStream_t side = side_stream(0), aux = side_stream(0);      // consecutive streams of the pool: the folds on one, the bucket sums on the other
     ZK_ARG(side != nullptr && aux != nullptr, "zk_g1_open_begin: could not create a stream");
+    // what open_queue refuses is refused here, before anything is handed to the launch thread
+    ZK_ARG(n >= 1, "zk_g1_open: empty input");
+    ZK_ARG(count >= 1 && count <= OB_MAX, "zk_g1_open: a batch holds 1 to 8 openings");
+    ZK_ARG(rounds >= 0 && rounds <= 64, "zk_g1_open: bad round count");
+    ZK_ARG(sizeof(G1Jac) * (3 * (size_t)rounds + 1) + sizeof(Fr) <= 65536, "zk_g1_open: proof larger than the staging buffer");
     std::unique_ptr<OpenJob> job(new OpenJob);
     ZK_HIP(hipEventCreateWithFlags(&job->ready, hipEventDisableTiming));
     ZK_HIP(hipEventRecord(job->ready, (hipStream_t)stv));
     ZK_HIP(hipStreamWaitEvent(side, job->ready, 0));
-    int rc = open_queue(*job, items, count, n, rounds, side, aux);
-    if (rc) {
-        (void)hipStreamSynchronize(side);
-        (void)hipStreamSynchronize(aux);
-        for (hipEvent_t e : job->events) (void)hipEventDestroy(e);
-        (void)hipEventDestroy(job->ready);
-        return rc;
+    pool_note_wait((hipStream_t)stv, side);
+    if (!launcher_enabled()) {
+        int rc = open_queue(*job, items, count, n, rounds, side, aux);
+        if (rc) {
+            (void)hipStreamSynchronize(side);
+            (void)hipStreamSynchronize(aux);
+            for (hipEvent_t e : job->events) (void)hipEventDestroy(e);
+            (void)hipEventDestroy(job->ready);
+            return rc;
+        }
+        *handle = job.release();
+        return 0;
     }
+    // The launch thread queues the job's few hundred launches (a millisecond of host time an opening) while the caller
+    // goes on; zk_g1_open_end waits for the ticket and reports what queuing returned.  The challenge arrays are the
+    // caller's and only valid during this call: the job takes copies.
+    struct Owned { OpenItem items[OB_MAX]; std::vector<uint32_t> u[OB_MAX], u_rows[OB_MAX]; };
+    std::shared_ptr<Owned> own(new Owned);
+    for (int i = 0; i < count; ++i) {
+        own->items[i] = items[i];
+        own->u[i].assign(items[i].u, items[i].u + 8 * (size_t)rounds);
+        own->items[i].u = own->u[i].data();
+        if (items[i].rows && items[i].k_rows > 0) {
+            own->u_rows[i].assign(items[i].u_rows, items[i].u_rows + 8 * (size_t)items[i].k_rows);
+            own->items[i].u_rows = own->u_rows[i].data();
+        }
+    }
+    OpenJob* j = job.get();
+    j->st = side;
+    j->aux = aux;
+    j->ticket = launcher_submit([j, own, count, n, rounds, side, aux] {
+        j->queue_rc = open_queue(*j, own->items, count, n, rounds, side, aux);
+        if (j->queue_rc) j->queue_err = last_error_text();
+    });
     *handle = job.release();
     return 0;
 }
@@ -2454,7 +2417,11 @@ int zk_g1_open_end_batch(void* handle, uint32_t* proof_host, uint32_t* final_sca
 int zk_g1_open_end(void* handle, uint32_t* proof_host, uint32_t* final_scalar_host) {
     ZK_ARG(handle != nullptr, "zk_g1_open_end: null handle");
     std::unique_ptr<OpenJob> job((OpenJob*)handle);
-    int rc = open_collect(*job, proof_host, final_scalar_host);
+    launcher_wait(job->ticket);
+    job->ticket = 0;
+    int rc = job->queue_rc;
+    if (rc) set_error(rc, job->queue_err);
+    else rc = open_collect(*job, proof_host, final_scalar_host);
     if (rc) { (void)hipStreamSynchronize(job->st); (void)hipStreamSynchronize(job->aux); }
     job->arena.mark_idle();          // both streams have drained behind the job's last kernel
     (void)hipEventDestroy(job->ready);

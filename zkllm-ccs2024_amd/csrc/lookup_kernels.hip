@@ -2911,11 +2911,8 @@ int zk_hadamard_prove_end(void* handle, uint32_t* coefs_host) {
 // hadamard_product_sumcheck (proof.cu:66-109): k rounds over a, b of n elements (2^(k-1) < n <= 2^k), evaluation
 // challenges u and fold challenges v, both in the order the reference consumes them (first challenge first).
 // proof_host: 3k + 2 values -- per round the three evaluated terms, then the fully folded a and b.  Neither input is modified.
-int zk_hadamard_product_sumcheck(uint32_t* proof_host, const void* a, const void* b, const uint32_t* u, const uint32_t* v, size_t n, int k, void* stv) {
-    hipStream_t st = (hipStream_t)stv;
-    ZK_ARG(k >= 1 && k <= 30 && n <= ((size_t)1 << k) && n > ((size_t)1 << (k - 1)), "zk_hadamard_product_sumcheck: n does not match the number of challenges");
-    ZK_ARG(sizeof(Fr) * (3 * (size_t)k + 2) <= 65536, "zk_hadamard_product_sumcheck: too many rounds for the staging buffer");
-    Arena arena(st);
+// the launches of hadamard_product_sumcheck on st, its buffers from `arena`; *sums_out: the 3k + 2 values on the device
+static int hp_sumcheck_queue(Fr** sums_out, Arena& arena, const void* a, const void* b, const uint32_t* u, const uint32_t* v, size_t n, int k, hipStream_t st) {
     const size_t half = (n + 1) / 2, etab = (size_t)1 << (k - 1);
     Scratch& E = arena.add(sizeof(Fr) * (etab + etab / 2 + 1));          // eq tables, ping-pong
     Scratch& W = arena.add(sizeof(Fr) * 2 * (half + (half + 1) / 2 + 1));   // folded a, b, ping-pong
@@ -2931,7 +2928,7 @@ int zk_hadamard_product_sumcheck(uint32_t* proof_host, const void* a, const void
     memset(&fin, 0, sizeof(fin));
     size_t part_at = 0;
     int rc = eq_table_queue(E.as<Fr>(), u + 8, k - 1, arena, st);
-    if (rc) { (void)hipStreamSynchronize(st); return rc; }
+    if (rc) return rc;
     Fr* ebuf[2] = {E.as<Fr>(), E.as<Fr>() + etab};
     Fr* wa[2] = {W.as<Fr>(), W.as<Fr>() + half};
     Fr* wb[2] = {wa[1] + (half + 1) / 2 + 1, nullptr};
@@ -2953,13 +2950,55 @@ int zk_hadamard_product_sumcheck(uint32_t* proof_host, const void* a, const void
     ZK_LAUNCH_CHECK();
     ZK_HIP(hipMemcpyAsync(sums.as<Fr>() + 3 * (size_t)k, ca, sizeof(Fr), hipMemcpyDeviceToDevice, st));
     ZK_HIP(hipMemcpyAsync(sums.as<Fr>() + 3 * (size_t)k + 1, cb, sizeof(Fr), hipMemcpyDeviceToDevice, st));
+    *sums_out = sums.as<Fr>();
+    return 0;
+}
+int zk_hadamard_product_sumcheck(uint32_t* proof_host, const void* a, const void* b, const uint32_t* u, const uint32_t* v, size_t n, int k, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(k >= 1 && k <= 30 && n <= ((size_t)1 << k) && n > ((size_t)1 << (k - 1)), "zk_hadamard_product_sumcheck: n does not match the number of challenges");
+    ZK_ARG(sizeof(Fr) * (3 * (size_t)k + 2) <= 65536, "zk_hadamard_product_sumcheck: too many rounds for the staging buffer");
+    Arena arena(st);
+    Fr* sums = nullptr;
+    int rc = hp_sumcheck_queue(&sums, arena, a, b, u, v, n, k, st);
+    if (rc) { (void)hipStreamSynchronize(st); return rc; }
     void* stage = nullptr;
     rc = staging(&stage, sizeof(Fr) * (3 * (size_t)k + 2));
     if (rc) { (void)hipStreamSynchronize(st); return rc; }
-    ZK_HIP(hipMemcpyAsync(stage, sums.p, sizeof(Fr) * (3 * (size_t)k + 2), hipMemcpyDeviceToHost, st));
+    ZK_HIP(hipMemcpyAsync(stage, sums, sizeof(Fr) * (3 * (size_t)k + 2), hipMemcpyDeviceToHost, st));
     ZK_HIP(hipStreamSynchronize(st));
     memcpy(proof_host, stage, sizeof(Fr) * (3 * (size_t)k + 2));
     return 0;
+}
+// The same in two halves: begin queues the rounds on a stream of the library's own, behind everything queued on `stream` so
+// far, and returns at once; a and b must stay alive and unmodified until end, which waits and delivers the 3k + 2 values.
+int zk_hadamard_product_sumcheck_begin(void** handle, const void* a, const void* b, const uint32_t* u, const uint32_t* v, size_t n, int k, void* stv) {
+    ZK_ARG(handle != nullptr, "zk_hadamard_product_sumcheck_begin: null handle");
+    ZK_ARG(k >= 1 && k <= 30 && n <= ((size_t)1 << k) && n > ((size_t)1 << (k - 1)), "zk_hadamard_product_sumcheck: n does not match the number of challenges");
+    ZK_ARG(sizeof(Fr) * (3 * (size_t)k + 2) <= 65536, "zk_hadamard_product_sumcheck: too many rounds for the staging buffer");
+    SumJob* job = new SumJob;
+    int rc = sumjob_on_side_stream(*job, (hipStream_t)stv);
+    if (rc) { sumjob_abort(job); return rc; }
+    // the caller's arrays are only valid during this call: the launches take copies
+    const std::vector<uint32_t> u_own(u, u + 8 * (size_t)k), v_own(v, v + 8 * (size_t)k);
+    job->rounds = 1;
+    job->per_round = 3 * k + 2;
+    rc = sumjob_launch(job, [=]() -> int {
+        int rc = hp_sumcheck_queue(&job->sums, job->arena, a, b, u_own.data(), v_own.data(), n, k, job->st);
+        if (rc == 0) rc = sumjob_queue_results(*job);
+        return rc;
+    });
+    if (rc) { sumjob_abort(job); return rc; }
+    *handle = job;
+    return 0;
+}
+int zk_hadamard_product_sumcheck_end(void* handle, uint32_t* proof_host) {
+    ZK_ARG(handle != nullptr, "zk_hadamard_product_sumcheck_end: null handle");
+    SumJob* job = (SumJob*)handle;
+    int rc = sumjob_queued(job);
+    if (rc) { sumjob_abort(job); return rc; }
+    rc = sumjob_collect(*job, (Fr*)proof_host, nullptr);
+    sumjob_abort(job);
+    return rc;
 }
 int zk_rescale(void* out, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* st) {
     ZK_ARG(scaling_factor >= 1, "zk_rescale: scaling factor is 0");

@@ -108,10 +108,11 @@ void RmsNormBlock::begin() {
     chg = g.draw(rms_inv.size);
     p2 = rs2.prove_begin(*Y, *Y_, ch2);
     p1 = rs1.prove_begin(*g_inv_rms, *g_inv_rms_, ch1);
+    hp = hadamard_product_sumcheck_begin(*g_inv_rms_, X, hu, hv);      // its rounds beside the caller's stream too
 }
 void RmsNormBlock::finish() {
     rs2.prove_end(p2);
-    hadamard_product_sumcheck(*g_inv_rms_, X, hu, hv);
+    hadamard_product_sumcheck_end(hp);
     rs1.prove_end(p1);
     auto claims = g.prove(rms_inv, *g_inv_rms, chg);
     if (c.open_weights) verifyWeightClaim(w, claims[0]);

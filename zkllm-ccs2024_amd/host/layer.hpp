@@ -89,6 +89,7 @@ struct RmsNormBlock {
     vector<Fr_t> hu, hv;
     zkFC::Challenges chg;
     Rescaling::Pending p1, p2;
+    HadamardProductPending hp;
 };
 struct AttnLinearBlock {
     AttnLinearBlock(const LayerConfig& c, const Weight& q, const Weight& k, const Weight& v, const FrTensor& input);

@@ -379,16 +379,39 @@ vector<Fr_t> inner_product_sumcheck(const FrTensor& a0, const FrTensor& b0, vect
 }
 
 // proof.cu:66-109: every round of the device side in one queue of launches (the challenges are all known), one copy back
-vector<Fr_t> hadamard_product_sumcheck(const FrTensor& a0, const FrTensor& b0, vector<Fr_t> u, vector<Fr_t> v) {
+HadamardProductPending hadamard_product_sumcheck_begin(const FrTensor& a0, const FrTensor& b0, const vector<Fr_t>& u, const vector<Fr_t>& v) {
     if (u.size() != v.size()) throw std::runtime_error("Incompatible dimensions 1");
     uint log_size = (uint)u.size();
     if (a0.size != b0.size) throw std::runtime_error("Incompatible dimensions 2");
     if (log_size == 0 || a0.size <= (1u << (log_size - 1))) throw std::runtime_error("Incompatible dimensions 3");
     if (a0.size > (1u << log_size)) throw std::runtime_error("Incompatible dimensions 4");
-    vector<Fr_t> proof(3 * (size_t)log_size + 2);
-    ZKC(zk_hadamard_product_sumcheck(proof[0].val, a0.gpu_data, b0.gpu_data, u[0].val, v[0].val, a0.size, (int)log_size, nullptr));
+    HadamardProductPending p;
+    p.log_size = log_size;
+    ZKC(zk_hadamard_product_sumcheck_begin(&p.job, a0.gpu_data, b0.gpu_data, u[0].val, v[0].val, a0.size, (int)log_size, nullptr));
+    return p;
+}
+vector<Fr_t> hadamard_product_sumcheck_end(HadamardProductPending& p) {
+    if (!p.job) throw std::runtime_error("hadamard_product_sumcheck_end: nothing pending");
+    vector<Fr_t> proof(3 * (size_t)p.log_size + 2);
+    void* job = p.job;
+    p.job = nullptr;          // end releases the job whatever it returns
+    ZKC(zk_hadamard_product_sumcheck_end(job, proof[0].val));
     zk_record(proof);
     return proof;
+}
+HadamardProductPending& HadamardProductPending::operator=(HadamardProductPending&& o) noexcept {
+    if (this != &o) {
+        if (job) { vector<Fr_t> drop(3 * (size_t)log_size + 2); (void)zk_hadamard_product_sumcheck_end(job, drop[0].val); }
+        job = o.job; log_size = o.log_size; o.job = nullptr;
+    }
+    return *this;
+}
+HadamardProductPending::~HadamardProductPending() {
+    if (job) { vector<Fr_t> drop(3 * (size_t)log_size + 2); (void)zk_hadamard_product_sumcheck_end(job, drop[0].val); }      // waits for the device side and releases it
+}
+vector<Fr_t> hadamard_product_sumcheck(const FrTensor& a0, const FrTensor& b0, vector<Fr_t> u, vector<Fr_t> v) {
+    HadamardProductPending p = hadamard_product_sumcheck_begin(a0, b0, u, v);
+    return hadamard_product_sumcheck_end(p);
 }
 
 // Fr_bin_sc_step (proof.cu:109-120)

@@ -120,6 +120,20 @@ void zk_openings_use_cross_commitments(bool on);
 void zk_openings_use_row_commitments(bool on);
 vector<Fr_t> inner_product_sumcheck(const FrTensor& a, const FrTensor& b, vector<Fr_t> u);
 vector<Fr_t> hadamard_product_sumcheck(const FrTensor& a, const FrTensor& b, vector<Fr_t> u, vector<Fr_t> v);
+// the same in two halves: begin queues the device side beside the caller's stream and records nothing; end collects, records and
+// returns the proof.  a and b stay alive and unmodified in between.
+struct HadamardProductPending {
+    void* job = nullptr;
+    uint log_size = 0;
+    HadamardProductPending() = default;
+    HadamardProductPending(HadamardProductPending&& o) noexcept : job(o.job), log_size(o.log_size) { o.job = nullptr; }
+    HadamardProductPending& operator=(HadamardProductPending&& o) noexcept;
+    HadamardProductPending(const HadamardProductPending&) = delete;
+    HadamardProductPending& operator=(const HadamardProductPending&) = delete;
+    ~HadamardProductPending();
+};
+HadamardProductPending hadamard_product_sumcheck_begin(const FrTensor& a, const FrTensor& b, const vector<Fr_t>& u, const vector<Fr_t>& v);
+vector<Fr_t> hadamard_product_sumcheck_end(HadamardProductPending& p);
 vector<Fr_t> binary_sumcheck(const FrTensor& a, vector<Fr_t> u, vector<Fr_t> v);
 
 Fr_t multi_hadamard_sumchecks(const Fr_t& claim, const vector<FrTensor>& Xs, const vector<Fr_t>& u, const vector<Fr_t>& v, vector<Polynomial>& proof);
