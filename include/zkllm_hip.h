@@ -238,9 +238,9 @@ int zk_g1_open_begin(void** handle, const void* scalars, const void* gens, size_
 int zk_g1_open_end(void* handle, uint32_t* proof_host, uint32_t* final_scalar_host);
 /* The generators of me_open (commitment.cu:109-129 takes the Commitment itself) in the form the rounds work on, made once
  * for any number of openings against them: affine points in 29-bit limbs and the first round's pair sums (1.5 n points
- * of 112 bytes; nothing in it depends on the opened tensor) and, above 2048 generators, the fixed-base tables of the
+ * of 112 bytes; nothing in it depends on the opened tensor) and, above 1024 generators, the fixed-base tables of the
  * first two rounds' folds (255 points per generator pair for the first round, as much again for the second when it
- * folds more than 2048 generators: 28 KB per generator in all, kept until the handle is freed; building them takes
+ * folds more than 1024 generators: 28 KB per generator in all, kept until the handle is freed; building them takes
  * about as much again in temporaries).  zk_g1_open_begin_prepared is zk_g1_open_begin with
  * such generators; the handle must outlive every opening started with it and is released with
  * zk_g1_open_prepared_free. */

@@ -398,16 +398,16 @@ def test_open_batch_with_row_commitments_delivers_the_points_of_the_plain_openin
     assert (got_v == exp_v).all()
     assert (got_p == exp_p).all()
     # the statement "these are the tensor's row commitments" is the caller's: with the other tensor's, T of the first round
-    # is what those commitments give, and with it T of the second halving round, which follows from the first round's three
-    # points (5000 -> 2500 -> 1250 generators, then the batched last rounds, which sum over the generators); T0, T1 of
+    # is what those commitments give, and with it T of the later halving rounds, which follow from the earlier rounds' points
+    # (5000 -> 2500 -> 1250 -> 625 generators, then the batched last rounds, which sum over the generators); T0, T1 of
     # every round, the folded generator and the value do not depend on them
     got_p, got_v = run((1, 0))
     assert (got_v == exp_v).all()
     same = np.ones(npts, bool)
-    same[[0, 3]] = False
+    same[[0, 3, 6]] = False
     assert (got_p[:, same] == exp_p[:, same]).all()
     for i in range(2):
-        assert not (got_p[i, 0] == exp_p[i, 0]).all() and not (got_p[i, 3] == exp_p[i, 3]).all()
+        assert not (got_p[i, 0] == exp_p[i, 0]).all() and not (got_p[i, 3] == exp_p[i, 3]).all() and not (got_p[i, 6] == exp_p[i, 6]).all()
     hip.call("zk_g1_open_prepared_free", prep)
 
 
@@ -415,10 +415,10 @@ def test_open_batch_with_row_commitments_delivers_the_points_of_the_plain_openin
 def test_open_batch_with_cross_commitments_needs_no_sum_over_the_generators(pv, orc, n, R, tables):
     """With the cross commitments of its first R rounds -- commitments of every 2nd / 4th / 8th column of the tensor's rows
     under every 2nd / 4th / 8th generator, made here with commit_int on slices -- zk_g1_open_begin_batch_rows forms T, T0 and
-    T1 of those rounds from rows x patterns points: 8192 generators are halved twice before the batched last rounds, so no
-    round sums over its generators.  With three rounds of them and the tables of zk_g1_open_prepare_tables(.., 3) the three
-    rounds are one fold (16384 generators: nothing but that fold and the batched last rounds; 32768: one ordinary round
-    behind it).  Every point of the proof equals zk_g1_open's on the row-folded vector, and at 16384 generators also the
+    T1 of those rounds from rows x patterns points: of the three halvings of 8192 generators before the batched last rounds
+    only the third sums over its generators.  With three rounds of them and the tables of zk_g1_open_prepare_tables(.., 3) the
+    three rounds are one fold (16384 generators: that fold, one ordinary round and the batched last rounds; 32768: two ordinary
+    rounds behind it).  Every point of the proof equals zk_g1_open's on the row-folded vector, and at 16384 generators also the
     oracle's own opening of the padded tensor (Commitment::open, commitment.cu:133-141: row fold, then me_open), point by
     point after normalisation, so the batched path is compared with the reference's algorithm directly."""
     import ctypes

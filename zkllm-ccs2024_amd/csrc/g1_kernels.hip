@@ -291,7 +291,7 @@ struct MsmDesc { const int8_t* digits; const A29* base; uint32_t dstride, count,
 static constexpr int OB_MAX = 8;           // openings of equal size that share their rounds' launches
 static constexpr int OB_SUMS = 3 * OB_MAX;
 template <int NMAX> struct MsmDescs { MsmDesc d[NMAX]; };
-static constexpr int TAIL_N = 2048;        // generators at which the remaining rounds are computed in one batch (work grows with it, latency shrinks)
+static constexpr int TAIL_N = 1024;        // generators at which the remaining rounds are computed in one batch (work grows with it, latency shrinks)
 static constexpr int TAIL_LEVELS = 20;     // most rounds the batch takes
 struct GlvK { uint32_t k1[4], k2[4]; };
 
