@@ -295,7 +295,7 @@ def test_rescaling_prove_seeded_transcript(pv, orc):
         assert t.shape == e_t.shape and (t == e_t).all()
 
 
-@pytest.mark.parametrize("nX,n", [(1, 8), (1, 2048), (2, 16), (2, 4096), (3, 64), (3, 2048), (4, 32), (4, 2048)])
+@pytest.mark.parametrize("nX,n", [(1, 8), (1, 2048), (2, 16), (2, 4096), (2, 1 << 18), (3, 64), (3, 2048), (4, 32), (4, 2048)])
 def test_multi_hadamard(pv, orc, nX, n):
     Xs = [ch(20 + i, n) for i in range(nX)]
     k = (n - 1).bit_length()

@@ -1035,6 +1035,40 @@ k_hadamard_round(Fr* __restrict__ partials, const PtrPack<K> p, const Fr* __rest
     block_reduce_store<K + 1>(acc, partials);
 }
 
+// k_hadamard_round<2> for rounds of many pairs with the arithmetic in 29-bit limbs, as k_lookup_round29 does it: the weight
+// arrives as E 2^256, e x0 and e dx come out as E x0 / 32 and E dx / 32, the three sums of products stay unreduced, are
+// reduced once per lane (2^-261 again) and brought to standard form by 2^271 (2^-261 once more: R^-1 in all) and R^2.
+// Same inputs, same outputs (folded tensors canonical).  At most 256 pairs per lane: the launch site checks.
+__global__ void __launch_bounds__(TPB) k_hadamard_round29(Fr* __restrict__ partials, Fr* __restrict__ nX, Fr* __restrict__ nY, const Fr* __restrict__ X, const Fr* __restrict__ Y,
+                                                          const Fr* __restrict__ E, const Fr v_mont, size_t n_out, Fr* __restrict__ nE) {
+    const Fr29 vq = fr29_mul(fr29_repack(v_mont), fr29_2_266());      // v 2^261
+    Wide29 w0 = wide29_zero(), w2 = wide29_zero(), wx = wide29_zero();
+    uint32_t it = 0;
+    for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
+        const Fr e = E[t];
+        if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);      // the next round's table: the top variable summed out
+        const Fr29 x0 = fr29_repack(X[t]), y0 = fr29_repack(Y[t]), y1 = fr29_repack(Y[t + n_out]);
+        const Fr29 dx = fr29_sub_plus_r(fr29_repack(X[t + n_out]), x0), dy = fr29_sub_plus_r(y1, y0);      // + r: non-negative, the same residues
+        const Fr29 e29 = fr29_repack(e);
+        const Fr29 ex0 = fr29_mul(e29, x0), edx = fr29_mul(e29, dx);
+        wide29_mac(w0, ex0, y0);
+        wide29_mac(w2, edx, dy);
+        wide29_mac(wx, fr29_add(ex0, edx), y1);                          // x0 dy + y0 dx = x1 y1 - x0 y0 - dx dy
+        if ((++it & 3u) == 0u) { wide29_carry(w0); wide29_carry(w2); wide29_carry(wx); }
+        nX[t] = fr29_canon_pack(fr29_add(x0, fr29_mul(vq, dx)));
+        nY[t] = fr29_canon_pack(fr29_add(y0, fr29_mul(vq, dy)));
+    }
+    Fr acc[3];
+    const Fr29 fix = fr29_2_271();
+    acc[0] = fr29_canon_pack(fr29_mul(wide29_redc(w0), fix));
+    acc[2] = fr29_canon_pack(fr29_mul(wide29_redc(w2), fix));
+    acc[1] = sub(sub(fr29_canon_pack(fr29_mul(wide29_redc(wx), fix)), acc[0]), acc[2]);
+    const Fr r2 = big_r2<8>();
+#pragma unroll
+    for (int j = 0; j < 3; ++j) acc[j] = mont_mul(acc[j], r2);
+    block_reduce_store<3>(acc, partials);
+}
+
 // The first round for two tensors given by their int32 forms (the mapped outputs of a softmax's segments): 4 bytes per
 // element instead of 32, and the three weighted coefficients are E times an exact 64-bit integer (x0 y0, dx dy, x1 y1) --
 // sixteen limb products into an unreduced twelve-limb sum each, one reduction per lane -- instead of Montgomery products.
@@ -2507,6 +2541,8 @@ static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, 
     }
         if (r == 0 && K == 2 && ints && ints[0] && ints[1])
             hipLaunchKernelGGL(k_hadamard_round2_ints, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), ints[0], ints[1], w, w + half, cE, vm, half, nE);
+        else if (K == 2 && limbs29() && half > (size_t)SPLIT_HALF && half <= (size_t)256 * nb * TPB)      // 29-bit limbs inside the kernel; its unreduced sums hold 256 pairs per lane
+            hipLaunchKernelGGL(k_hadamard_round29, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, cur[0], cur[1], cE, vm, half, nE);
         else
             switch (K) { HADS_ROUND(1) HADS_ROUND(2) HADS_ROUND(3) HADS_ROUND(4) }
 #undef HADS_ROUND
