@@ -499,7 +499,7 @@ def main():
                        "note": "algorithmic work = Fp multiplications of the point formulas x 300 MAD32 (12-limb schoolbook product and reduction; the kernel "
                                "itself works on 14 limbs of 29 bits: 392 multiply-adds and ~110 other instructions per product, 301 per square); "
                                "peak = 256 CU x 4 SIMD x 16 lanes x 2.4 GHz.  The launches are of every size (524288 pairs in the first round of the "
-                               "two 2^19 openings down to 2048 in the last halving round) and run beside the bucket sums of their own job and beside "
+                               "two 2^19 openings down to 1024 in the last halving round) and run beside the bucket sums of their own job, beside up to three other opening jobs and beside "
                                "the rest of the proof; traffic was measured for the kernel alone at 262144 pairs (roofline_fold_alone)"}
     if lk_launches:
         out["roofline_lookup_round_in_layer"] = {
