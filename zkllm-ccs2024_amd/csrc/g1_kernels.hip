@@ -1188,14 +1188,17 @@ __global__ void __launch_bounds__(256) k_a29_canon(A29* __restrict__ a, size_t n
 // Folded scalars of all levels: level 0 is S itself, level j >= 1 sits at SL + sum_{1<=i<j} n_i, n_i = ceil(n0 / 2^i).
 struct TailPtrs { Fr* SL[OB_MAX]; const Fr* S[OB_MAX]; };      // per opening of a batch (blockIdx.x of k_tail_scalars, blockIdx.y of k_tail_coeffs)
 // U: the tail's challenges (Montgomery form), opening y's at U + y * ustride
-__global__ void __launch_bounds__(1024) k_tail_scalars(const TailPtrs tp, const Fr* __restrict__ U, uint32_t ustride, uint32_t n0, uint32_t levels) {
+// One workgroup per opening (the levels follow each other behind a barrier) of TAIL_SCALAR_T lanes: four waves find room on
+// a compute unit whose SIMDs each hold a point kernel's waves; the sixteen of a 1024-lane workgroup waited milliseconds for it.
+static constexpr int TAIL_SCALAR_T = 256;
+__global__ void __launch_bounds__(TAIL_SCALAR_T) k_tail_scalars(const TailPtrs tp, const Fr* __restrict__ U, uint32_t ustride, uint32_t n0, uint32_t levels) {
     const Fr* __restrict__ usu = U + (size_t)blockIdx.x * ustride;
     const Fr* cur = tp.S[blockIdx.x];
     Fr* nxt = tp.SL[blockIdx.x];
     uint32_t n = n0;
     for (uint32_t j = 0; j < levels; ++j) {
         const uint32_t ns = (n + 1) / 2;
-        for (uint32_t g = threadIdx.x; g < ns; g += 1024) {
+        for (uint32_t g = threadIdx.x; g < ns; g += TAIL_SCALAR_T) {
             const Fr s0 = cur[2 * g];
             nxt[g] = (2 * g + 1 < n) ? add(s0, mont_mul(usu[j], sub(cur[2 * g + 1], s0))) : sub(s0, mont_mul(usu[j], s0));
         }
@@ -1576,7 +1579,7 @@ static int open_tail_launch(const Fr** scalars, const A29* const* gens, int coun
     ZK_ARG(ncoef < (1ull << 32), "opening: batched last rounds too large");
     TailPtrs tp;
     for (int i = 0; i < OB_MAX; ++i) { const int k = i < count ? i : 0; tp.SL[i] = sl.as<Fr>() + sl_n * k; tp.S[i] = scalars[k]; }
-    hipLaunchKernelGGL(k_tail_scalars, dim3(count), dim3(1024), 0, st, tp, U_dev + r0, (uint32_t)rounds, (uint32_t)n0, (uint32_t)levels);
+    hipLaunchKernelGGL(k_tail_scalars, dim3(count), dim3(TAIL_SCALAR_T), 0, st, tp, U_dev + r0, (uint32_t)rounds, (uint32_t)n0, (uint32_t)levels);
     hipLaunchKernelGGL(k_tail_coeffs, dim3(cdiv(n0, 256), count), dim3(256), 0, st, coef.as<Fr>(), tp, U_dev + r0, (uint32_t)rounds, (uint32_t)n0, (uint32_t)levels);
     {
         RecodeBatch rb;
