@@ -313,6 +313,28 @@ def test_multi_hadamard(pv, orc, nX, n):
     assert (proof == e_proof).all() and (fin == e_fin).all()
 
 
+@pytest.mark.parametrize("special", [1, 0])
+def test_multi_hadamard_with_evaluation_challenges_of_one_and_zero(pv, orc, special):
+    """The rounds of a sumcheck job read the first eq table's prefix and their weighted sums are multiplied by
+    prod 1 / (1 - u_top) when they are collected; a challenge equal to 1 has no such constant (the job then writes every
+    round's table), one equal to 0 makes half of the table zero.  Both against the oracle, 2^16 elements (the large-round
+    kernels, the short rounds and the last-rounds kernel all take part)."""
+    n, nX = 1 << 16, 2
+    Xs = [ch(120 + i, n) for i in range(nX)]
+    k = (n - 1).bit_length()
+    u, v = ch(130, k), ch(131, k)
+    for i in (3, k - 2, k - 1):
+        u[i] = fr_array([special])[0]
+    prod = np.zeros_like(Xs[0])
+    orc_check(orc.orc_fr_op(7, Xs[0], Xs[1], prod, n))
+    claim = np.zeros(8, np.uint32)
+    orc_check(orc.orc_fr_me(prod, n, u, k, claim))
+    e_proof, e_fin = np.zeros((k * (nX + 1), 8), np.uint32), np.zeros(8, np.uint32)
+    orc_check(orc.orc_multi_hadamard(claim, np.ascontiguousarray(np.concatenate(Xs)), nX, n, u, v, k, e_proof, e_fin))
+    proof, fin = pv.multi_hadamard(claim, [pv.from_fr(x) for x in Xs], u, v)
+    assert (proof == e_proof).all() and (fin == e_fin).all()
+
+
 @pytest.mark.parametrize("n,kept", [(4096, (True, True)), (1 << 17, (True, True)), (1 << 17, (True, False)), (1 << 15, (False, True))])
 def test_multi_hadamard_of_two_tensors_that_keep_an_int32_form(pv, orc, n, kept):
     """Two tensors of 32-bit integers, the extremes included, kept for folds: the job's first round reads their int32 forms

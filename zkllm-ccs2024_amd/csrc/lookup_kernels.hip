@@ -2229,7 +2229,39 @@ struct SumJob {
     uint64_t ticket = 0;
     int queue_rc = 0;
     std::string queue_err;
+    // A job whose weights are an eq table of the library's own: summing the top variable out of eq(u, .) leaves its lower half
+    // divided by 1 - u_top, so every round's table is the first table's prefix times a constant and no round writes a table --
+    // the rounds read the prefix, and the E-weighted sums of round r are multiplied by eq_scale[r] when they are collected
+    // (Montgomery form; empty: the rounds write their tables).  tail_from: the round the last-rounds kernel starts at (it
+    // folds its table itself, from the prefix: its rounds share that round's constant).
+    std::vector<Fr> eq_scale;
+    int tail_from = -1;
 };
+// eq_scale of a job over `rounds` rounds whose table is eq(u_eq, .) of rounds - 1 challenges (index bit j <-> u_eq[j]); false
+// (and nothing written) if some challenge is 1
+static bool eq_prefix_scales(std::vector<Fr>& out, const uint32_t* u_eq, int rounds) {
+    const int k = rounds - 1;
+    std::vector<Fr> c((size_t)rounds);
+    const Fr one = big_one_mont<8>();
+    if (rounds >= 1) c[0] = one;
+    for (int r = 1; r < rounds; ++r) {
+        const Fr d = sub(one, to_mont(load_fr(u_eq + 8 * (size_t)(k - r))));
+        if (is_zero(d)) return false;
+        c[r] = mont_mul(c[r - 1], mont_inverse(d));
+    }
+    out.swap(c);
+    return true;
+}
+// the E-weighted entries of collected sums (bit i of `weighted`: entry i of a round's per_round) times their round's constant
+static bool eq_prefix_on() { static const bool on = [] { const char* e = getenv("ZKLLM_EQ_PREFIX"); return !(e && e[0] == '0'); }(); return on; }
+static void eq_prefix_apply(const SumJob& job, Fr* sums, uint32_t weighted) {
+    if (job.eq_scale.empty()) return;
+    for (int r = 0; r < job.rounds; ++r) {
+        const Fr& c = job.eq_scale[(size_t)((job.tail_from >= 0 && r > job.tail_from) ? job.tail_from : r)];
+        for (int i = 0; i < job.per_round; ++i)
+            if ((weighted >> i) & 1u) sums[(size_t)r * job.per_round + i] = mont_mul(sums[(size_t)r * job.per_round + i], c);
+    }
+}
 __global__ void __launch_bounds__(64) k_u32_set(uint32_t* __restrict__ p, uint32_t v) { if (threadIdx.x == 0) *p = v; }
 __global__ void __launch_bounds__(TPB) k_dot_part(Fr* __restrict__ partials, const Fr* __restrict__ a, const Fr* __restrict__ b, size_t n) {
     Fr acc[1] = {big_zero<8>()};
@@ -2314,6 +2346,7 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
     size_t part_at = 0;
     int fin_rounds = 0;              // rounds whose sums come from partials (the rest: the tail kernel's)
     PartSlice part{nullptr};
+    const bool eq_prefix = !job.eq_scale.empty();      // every round reads the first table's prefix
     const Fr *cA = A, *cS = S, *cB = B, *cT = T, *cm = m, *cE = E;
     Fr* eqbuf[2] = {nullptr, nullptr};
     size_t cur = D;
@@ -2330,6 +2363,7 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
             hipLaunchKernelGGL(k_lookup_tail, dim3(1), dim3(TAIL_T), 0, st, sums.as<Fr>() + (size_t)r * 11, work.as<Fr>(), cA, cS, cB, cT, cm, cE, b, vs, (uint32_t)half,
                                (uint32_t)rest, (uint32_t)(phase2 ? 0 : n1 - r));
             ZK_LAUNCH_CHECK();
+            job.tail_from = r;
             break;
         }
         if (r == 0 && !phase2 && fuse_first && hs->hint_ints && limbs29() && two_rounds_on() && n1 >= 2 && rounds >= 2 && (half >> 1) > (size_t)SPLIT_HALF &&
@@ -2342,7 +2376,7 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
             Fr* w2 = nx2.as<Fr>();
             // the third round's eq table goes where the second round would have put it
             Fr* nE3 = nullptr;
-            if (r + 2 < rounds) {
+            if (r + 2 < rounds && !eq_prefix) {
                 Scratch& e = job.arena.add(sizeof(Fr) * 2 * h2);
                 if (e.rc) return e.rc;
                 eqbuf[0] = e.as<Fr>();
@@ -2369,6 +2403,7 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
                 g_round_timer.bytes += (double)h2 * (q + 64.0 + 64.0 + (nE3 ? 48.0 : 0.0));
             }
             ZK_LAUNCH_CHECK();
+            if (eq_prefix) job.eq_scale[(size_t)r + 1] = job.eq_scale[(size_t)r];      // the pass forms the second round's weights from the first round's: the same constant
             fin.off[r] = (uint32_t)part_at; fin.nb[r] = nb2; fin.k[r] = 5;
             fin.off[r + 1] = (uint32_t)(part_at + 5 * (size_t)nb2); fin.nb[r + 1] = nb2; fin.k[r + 1] = 5;
             part_at += 10 * (size_t)nb2;
@@ -2386,7 +2421,7 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
         const Fr vm = to_mont(load_fr(v + 8 * r));
         // the next round's eq table is written by this round's kernel (ping-pong between two buffers of the job)
         Fr* nE = nullptr;
-        if (r + 1 < rounds) {
+        if (r + 1 < rounds && !eq_prefix) {
             const size_t nh = half >> 1;
             if (!eqbuf[0]) {
                 Scratch& e = job.arena.add(sizeof(Fr) * 2 * (nh ? nh : 1));
@@ -2514,6 +2549,7 @@ static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, 
             switch (K) { HADS_TAIL(1) HADS_TAIL(2) HADS_TAIL(3) HADS_TAIL(4) }
 #undef HADS_TAIL
             ZK_LAUNCH_CHECK();
+            job.tail_from = r;
             break;
         }
         Scratch& nx = job.arena.add(sizeof(Fr) * half * K);
@@ -2522,7 +2558,7 @@ static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, 
         const unsigned nb = reduce_grid(half);
         const Fr vm = to_mont(load_fr(v + 8 * r));
         Fr* nE = nullptr;
-        if (r + 1 < rounds) {
+        if (r + 1 < rounds && job.eq_scale.empty()) {      // (with eq_scale every round reads the first table's prefix)
             const size_t nh = half >> 1;
             if (!eqbuf[0]) {
                 Scratch& e = job.arena.add(sizeof(Fr) * 2 * (nh ? nh : 1));
@@ -2763,6 +2799,7 @@ static int lookup_prove_begin(void** handle, const void* S, const void* T, const
     job->extra = dp.as<Fr>();
     rc = shared_eq_get(job->eq, u_eq, rounds - 1, job->arena, st);
     if (rc) return rc;
+    if (eq_prefix_on()) (void)eq_prefix_scales(job->eq_scale, u_eq, rounds);
     rc = lookup_queue(*job, Aptr, (const Fr*)S, B.as<Fr>(), (const Fr*)T, (const Fr*)m, (const Fr*)job->eq->p, b, v, D, N, rounds, hint ? &hs : nullptr);
     if (rc == 0) rc = sumjob_queue_results(*job);
     return rc;
@@ -2831,6 +2868,7 @@ int zk_lookup_prove_end(void* handle, uint32_t* bm_host, uint32_t* sums_host) {
         if (hipMemcpy(&v, job->n_ok_dev, sizeof(uint32_t), hipMemcpyDeviceToHost) == hipSuccess) { g_last_n_ok = v < job->n_table ? v : job->n_table; g_last_n_table = job->n_table; }
     }
     if (!rc) {
+        eq_prefix_apply(*job, (Fr*)sums_host, 0x0E7u);      // sums 0..2 and 5..7: sums 3, 4 and 8..10 carry no eq weight
         lookup_fix_sums((Fr*)sums_host, job->rounds, job->n1);
         bm = to_mont(bm);          // the products carried R^-1
         memcpy(bm_host, &bm, sizeof(Fr));
@@ -2927,6 +2965,7 @@ int zk_hadamard_prove_begin_ints(void** handle, const void* const* Xs, const voi
     rc = sumjob_launch(job, [=]() -> int {
         int rc = shared_eq_get(job->eq, u_own.data(), k - 1, job->arena, job->st);
         if (rc) return rc;
+        if (eq_prefix_on()) (void)eq_prefix_scales(job->eq_scale, u_own.data(), k);
         rc = hadamard_queue(*job, xs_own.data(), K, (const Fr*)job->eq->p, v_own.data(), N, have_ints ? ints_own.data() : nullptr);
         if (rc == 0) rc = sumjob_queue_results(*job);
         return rc;
@@ -2941,6 +2980,7 @@ int zk_hadamard_prove_end(void* handle, uint32_t* coefs_host) {
     int rc = sumjob_queued(job);
     if (rc) { sumjob_abort(job); return rc; }
     rc = sumjob_collect(*job, (Fr*)coefs_host, nullptr);
+    if (!rc) eq_prefix_apply(*job, (Fr*)coefs_host, 0xFFFFFFFFu);      // every coefficient is eq-weighted
     sumjob_abort(job);
     return rc;
 }
