@@ -141,6 +141,8 @@ int zk_fr_fold_axis(void* out, const void* in, const uint32_t* u, int levels, si
  * out[o][w] = sum_j eq(u, j) in[o][j][w], u[0] on the lowest bit of j; bit-identical to the level-by-level fold. */
 int zk_fr_fold_prepare(void** prepared, const void* t, size_t n, void* stream);
 int zk_fr_fold_axis_prepared(void* out, const void* prepared, const uint32_t* u, int levels, size_t other, uint32_t cur, size_t window, void* stream);
+/* the same fold of the elementwise product of two such tensors (handles of equal size): out[o][w] = sum_j eq(u, j) a[o][j][w] b[o][j][w] */
+int zk_fr_fold_axis_prod(void* out, const void* a_prepared, const void* b_prepared, const uint32_t* u, int levels, size_t other, uint32_t cur, size_t window, void* stream);
 int zk_fr_fold_prepared_free(void* prepared);
 /* The same handle for a tensor whose int32 form is written by the kernel that makes the tensor (the digit planes of
  * zk_softmax_decompose_ints, the outputs of zk_fr_gather_ints), so no pass over the field elements is needed: _new
@@ -181,6 +183,12 @@ int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, 
 /* the same for a stack of `batch` products, A [batch][M][N], B [batch][N][P], C [batch][M][P] (the per-head products of
  * zkAttn::compute, zksoftmax.cu:234-238, for all heads at once); the bound check covers the whole stacks, so one path serves all */
 int zk_fr_matmul_batched(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used_host, void* stream);
+/* the same for a left operand that is the elementwise product of two tensors given by their int32 forms (device pointers
+ * to batch * M * N int32 each, zk_fr_fold_prepared_ints): the product, an exact 64-bit integer per element, is read where A
+ * would be and written out as field elements only for the paths that read nothing else.  No counterpart in the reference
+ * (zkSoftmax::compute multiplies the segments' table values into a tensor first, zksoftmax.cu:160-166). */
+int zk_fr_matmul_batched_prod(void* C, const void* a_ints, const void* b_ints, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used_host,
+                              void* stream);
 /* The right operand of many products (a layer's weight in zkFC::operator(), zkfc.cu:44-58) examined once: its largest magnitude
  * for the small-integer bound and, when it holds small integers, its int8 digit planes in the GEMM's layout.  No counterpart in
  * the reference, which converts nothing.  B stays alive and unmodified while the handle is used; zk_fr_matmul_rhs is

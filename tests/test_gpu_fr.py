@@ -575,6 +575,56 @@ def test_stacks_of_matrices_transpose_and_multiply_like_their_members(pv):
     assert fr_ints(got) == [int(v) % R_MOD for v in T.transpose(0, 2, 1).reshape(-1)]
 
 
+@pytest.mark.parametrize("num,M,N,P,abits,bbits,ybits", [(3, 70, 130, 50, 16, 16, 17), (2, 33, 65, 128, 31, 31, 17), (1, 128, 256, 64, 8, 9, 12), (2, 20, 40, 9, 31, 31, 40),
+                                                          (1, 64, 64, 64, 16, 15, 280)])
+def test_a_product_of_two_int32_tensors_multiplies_and_folds_without_being_written(pv, orc, num, M, N, P, abits, bbits, ybits):
+    """zk_fr_matmul_batched_prod / zk_fr_fold_axis_prod (the softmax output as the product of its two segments' table values,
+    zksoftmax.cu:160-166, then Y x V and the fold of Y over its rows, zksoftmax.cu:315-336 in stacked form): the same elements as
+    the product written out first, on every path of the dispatcher (narrow and wide products, wide and full-width right operand)
+    and with the extreme integers in both factors."""
+    print("case", num, M, N, P, abits, bbits, ybits, flush=True)
+    rng = np.random.default_rng(num * 1000 + M + abits)
+    A = rng.integers(-2 ** abits, 2 ** abits, (num, M, N)).astype(np.int64)
+    B = rng.integers(-2 ** bbits, 2 ** bbits, (num, M, N)).astype(np.int64)
+    if abits == 31:
+        A[0, 0, :4], B[0, 0, :4] = [-2 ** 31, -2 ** 31, 2 ** 31 - 1, 2 ** 31 - 1], [-2 ** 31, 2 ** 31 - 1, -2 ** 31, 2 ** 31 - 1]
+        A[-1, -1, -1], B[-1, -1, -1] = -2 ** 31, -2 ** 31
+    A, B = np.clip(A, -2 ** 31, 2 ** 31 - 1), np.clip(B, -2 ** 31, 2 ** 31 - 1)
+    if ybits > 64:
+        Yf = mt_random_vec(np.random.RandomState(5), num * N * P)
+        hY = pv.from_fr(Yf)
+        Yi = np.array(fr_ints(Yf), dtype=object).reshape(num, N, P)
+    else:
+        Y64 = rng.integers(-2 ** ybits, 2 ** ybits, (num, N, P)).astype(np.int64)
+        hY = pv.from_i64(Y64)
+        Yi = Y64.astype(object)
+    hA, hB = pv.from_i64(A), pv.from_i64(B)
+    pv.keep_for_folds(hA)
+    pv.keep_for_folds(hB)
+    assert pv.folds_from_ints(hA) == 1 and pv.folds_from_ints(hB) == 1
+    prod = A.astype(object) * B.astype(object)
+    pv.lib.zkp_set_matmul_mode(ctypes.c_int(0))
+    got = pv.matmul_stack_prod(hA, hB, hY, num, M, N, P).host()
+    want = [int(v) % R_MOD for i in range(num) for v in (prod[i] @ Yi[i]).reshape(-1)]
+    assert fr_ints(got) == want, pv.lib.zkp_last_matmul_path()
+    # the fold over the rows of each matrix (cur = M, window = N, other = num) against the oracle's fold of the written product
+    k = max((M - 1).bit_length(), 1)
+    u = mt_random_vec(np.random.RandomState(19), k)
+    n = num * M * N
+    Pf = fr_array([int(v) % R_MOD for v in prod.reshape(-1)])
+    exp = np.zeros((n, 8), np.uint32)
+    out_n = np.zeros(1, np.int64)
+    orc_check(orc.orc_fr_partial_me(Pf, n, u, k, M, N, exp, out_n))
+    for rep in range(2):
+        got = pv.partial_me_prod(hA, hB, u, M, N).host()
+        assert got.shape[0] == out_n[0] == num * N
+        assert (got == exp[:out_n[0]]).all(), rep
+    # a factor without an int32 form is refused
+    hC = pv.from_i64(A)
+    with pytest.raises(RuntimeError):
+        pv.partial_me_prod(hA, hC, u, M, N)
+
+
 def test_config2_full_size_fully_connected_proof_passes_the_verifier(pv):
     """X 2048 x 4096 times W 4096 x 4096 (fixed point, scale 2^16, N(0, 0.02)), beyond what the oracle can follow: rows
     of the product are compared with int64 arithmetic, and the proof transcript under a seeded stream is checked as a

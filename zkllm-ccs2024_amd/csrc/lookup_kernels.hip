@@ -1645,6 +1645,46 @@ __global__ void __launch_bounds__(256) k_ifold_window(Fr* __restrict__ out, cons
         if (live) out[g] = ifold_finish(acc);
     }
 }
+// the same fold of the elementwise product of two tensors in int32 form (exact 64-bit integers: sixteen limb products into a
+// twelve-limb sum per element): the product is never written
+__global__ void __launch_bounds__(256) k_ifold_window_prod(Fr* __restrict__ out, const int32_t* __restrict__ ina, const int32_t* __restrict__ inb, const EqPair* __restrict__ E,
+                                                           size_t n_out, uint32_t cur, size_t window) {
+    __shared__ uint32_t sh[4][12][64];
+    const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;
+    const size_t g = (size_t)blockIdx.x * 64 + lane;
+    const bool live = g < n_out;
+    const size_t gg = live ? g : n_out - 1;
+    const size_t o = gg / window, w = gg % window;
+    const size_t base = o * (size_t)cur * window + w;
+    const uint32_t per = (cur + 3) / 4;
+    const uint32_t j0 = wv * per < cur ? wv * per : cur, j1 = j0 + per < cur ? j0 + per : cur;
+    uint32_t acc[12];
+#pragma unroll
+    for (int i = 0; i < 12; ++i) acc[i] = 0;
+    uint32_t j = j0;
+    for (; j + 4 <= j1; j += 4) {
+        int32_t x[4], y[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) { x[t] = ina[base + (size_t)(j + t) * window]; y[t] = inb[base + (size_t)(j + t) * window]; }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) imac64(acc, E[j + t].e, E[j + t].ne, (int64_t)x[t], (int64_t)y[t]);
+    }
+    for (; j < j1; ++j) imac64(acc, E[j].e, E[j].ne, (int64_t)ina[base + (size_t)j * window], (int64_t)inb[base + (size_t)j * window]);
+    if (wv) {
+#pragma unroll
+        for (int i = 0; i < 12; ++i) sh[wv][i][lane] = acc[i];
+    }
+    __syncthreads();
+    if (wv == 0) {
+#pragma unroll
+        for (int q = 1; q < 4; ++q) {
+            uint32_t c = 0;
+#pragma unroll
+            for (int i = 0; i < 12; ++i) acc[i] = addc32(acc[i], sh[q][i][lane], c);
+        }
+        if (live) out[g] = imac64_finish(acc);
+    }
+}
 // window 1: out[o] = sum_j E[j] in[o][j].  A workgroup serves four rows; each of its four waves takes a quarter of the axis
 // for all four (an entry is loaded once for the four rows), lanes over j, a butterfly over the wave, then the four waves' sums.
 __global__ void __launch_bounds__(256) k_ifold_rows(Fr* __restrict__ out, const int32_t* __restrict__ in, const EqPair* __restrict__ E, size_t other, uint32_t cur) {
@@ -2084,6 +2124,28 @@ int zk_fr_fold_axis_prepared(void* out, const void* prepared, const uint32_t* u,
     const size_t n_out = other * window;
     if (window == 1 && cur >= 64) hipLaunchKernelGGL(k_ifold_rows, dim3(cdiv(other, 4)), dim3(256), 0, st, (Fr*)out, fp->ints, P.as<EqPair>(), other, cur);
     else hipLaunchKernelGGL(k_ifold_window, dim3(cdiv(n_out, 64)), dim3(256), 0, st, (Fr*)out, fp->ints, P.as<EqPair>(), n_out, cur, window);
+    ZK_LAUNCH_CHECK();
+    return 0;
+}
+// zk_fr_fold_axis_prepared for the elementwise product of two tensors given by their int32 forms (n = other * cur * window
+// elements each): out[o][w] = sum_j eq(u, j) a[o][j][w] b[o][j][w]
+int zk_fr_fold_axis_prod(void* out, const void* a_prepared, const void* b_prepared, const uint32_t* u, int levels, size_t other, uint32_t cur, size_t window, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    const FoldPrepared *fa = (const FoldPrepared*)a_prepared, *fb = (const FoldPrepared*)b_prepared;
+    ZK_ARG(fa != nullptr && fb != nullptr && out != nullptr && u != nullptr, "zk_fr_fold_axis_prod: null argument");
+    ZK_ARG(levels >= 1 && levels <= 24, "zk_fr_fold_axis_prod: 1 to 24 levels");
+    ZK_ARG(cur >= 1 && cur <= (1u << levels), "zk_fr_fold_axis_prod: the axis is longer than 2^levels");
+    ZK_ARG(other >= 1 && window >= 1 && other * (size_t)cur * window == fa->n && fb->n == fa->n, "zk_fr_fold_axis_prod: other * cur * window is not the tensors' size");
+    Arena tmp(st);
+    Scratch& E = tmp.add(sizeof(Fr) * ((size_t)1 << levels));
+    Scratch& P = tmp.add(sizeof(EqPair) * (size_t)cur);
+    if (E.rc) return E.rc;
+    if (P.rc) return P.rc;
+    int rc = eq_table_queue(E.as<Fr>(), u, levels, tmp, st);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_eq_pairs, dim3(cdiv(cur, TPB)), dim3(TPB), 0, st, P.as<EqPair>(), E.as<Fr>(), cur);
+    const size_t n_out = other * window;
+    hipLaunchKernelGGL(k_ifold_window_prod, dim3(cdiv(n_out, 64)), dim3(256), 0, st, (Fr*)out, fa->ints, fb->ints, P.as<EqPair>(), n_out, cur, window);
     ZK_LAUNCH_CHECK();
     return 0;
 }

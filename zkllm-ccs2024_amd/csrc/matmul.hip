@@ -214,6 +214,44 @@ __global__ void __launch_bounds__(256) k_rowabs(unsigned long long* __restrict__
         if (gs > __atomic_load_n(out, __ATOMIC_RELAXED)) atomicMax(out, gs);
     }
 }
+// A left operand that exists as the elementwise product of two tensors in int32 form (a softmax's output: the product of two
+// segments' table values): its elements are exact 64-bit integers, read at 8 bytes each instead of 32.
+struct ProdSrc { const int32_t* a; const int32_t* b; };
+__device__ __forceinline__ long long prod_at(const ProdSrc& s, size_t i) { return (long long)s.a[i] * (long long)s.b[i]; }
+// k_rowabs for such an operand
+__global__ void __launch_bounds__(256) k_rowabs_prod(unsigned long long* __restrict__ out, unsigned long long* __restrict__ out_max, const ProdSrc src, uint32_t ncol) {
+    const size_t base = (size_t)blockIdx.x * ncol;
+    unsigned long long m = 0, mx = 0;
+    for (uint32_t j = threadIdx.x; j < ncol; j += 256) {
+        const long long x = prod_at(src, base + j);
+        unsigned long long v = x < 0 ? 0ull - (unsigned long long)x : (unsigned long long)x;
+        if (v > (1ull << 62)) v = ~0ull;
+        mx = v > mx ? v : mx;
+        m = (m == ~0ull || v == ~0ull || m + v > (1ull << 62)) ? ~0ull : m + v;
+    }
+    auto sat_add = [](unsigned long long x, unsigned long long y) { return (x == ~0ull || y == ~0ull || x + y > (1ull << 62)) ? ~0ull : x + y; };
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const unsigned long long om = __shfl_xor(mx, off, 64), os = __shfl_xor(m, off, 64);
+        mx = om > mx ? om : mx;
+        m = sat_add(m, os);
+    }
+    __shared__ unsigned long long red[2][4];
+    const uint32_t wv = threadIdx.x >> 6;
+    if ((threadIdx.x & 63u) == 0) { red[0][wv] = mx; red[1][wv] = m; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long gm = red[0][0], gs = red[1][0];
+        for (int i = 1; i < 4; ++i) { gm = red[0][i] > gm ? red[0][i] : gm; gs = sat_add(gs, red[1][i]); }
+        if (gm > __atomic_load_n(out_max, __ATOMIC_RELAXED)) atomicMax(out_max, gm);
+        if (gs > __atomic_load_n(out, __ATOMIC_RELAXED)) atomicMax(out, gs);
+    }
+}
+// the operand written out as field elements (for the paths that read nothing else)
+__global__ void __launch_bounds__(256) k_prod_to_fr(Fr* __restrict__ out, const ProdSrc src, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = fr_from_i64(prod_at(src, i));
+}
 template <typename T> __global__ void __launch_bounds__(256) k_fr_to_int(T* __restrict__ out, const Fr* __restrict__ a, size_t n) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) out[i] = (T)fr_to_i64(a[i]);
@@ -344,7 +382,8 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 static constexpr int GBM = 128, GBN = 128, GBK = 128;      // block tile of the GEMM: 4 waves, 64 x 64 outputs each
 static constexpr int GLD = GBK + 16;                       // LDS row stride in bytes: 16-byte aligned rows whose 16-byte reads spread over all banks
 
-__global__ void __launch_bounds__(256) k_split_rows(int8_t* __restrict__ planes, const Fr* __restrict__ a, size_t rows, uint32_t M, uint32_t N, uint32_t Kp, int np) {
+// src: the operand as a product of int32 forms when src.a is set (a is then not read)
+__global__ void __launch_bounds__(256) k_split_rows(int8_t* __restrict__ planes, const Fr* __restrict__ a, const ProdSrc src, size_t rows, uint32_t M, uint32_t N, uint32_t Kp, int np) {
     const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
     const uint32_t groups = Kp / 4;
     const size_t row = gid / groups;
@@ -353,7 +392,7 @@ __global__ void __launch_bounds__(256) k_split_rows(int8_t* __restrict__ planes,
     const size_t b = row / M, m = row % M;
     long long x[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) x[e] = (k + e < N) ? fr_to_i64(a[row * N + k + e]) : 0ll;
+    for (int e = 0; e < 4; ++e) x[e] = (k + e < N) ? (src.a ? prod_at(src, row * N + k + e) : fr_to_i64(a[row * N + k + e])) : 0ll;
     for (int j = 0; j < np; ++j) {
         uint32_t packed = 0;
 #pragma unroll
@@ -575,7 +614,7 @@ static int digits_for(unsigned long long absmax) {      // planes needed for |x|
 // small integers, its digit planes in the GEMM's layout -- neither is computed again per product.
 struct MatmulRhs { const void* B = nullptr; uint32_t N = 0, P = 0, Kp = 0; unsigned long long mb = ~0ull; int pb = 0; void* planes = nullptr; };
 static int run_int8_plane_path(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, unsigned long long ma, unsigned long long mb,
-                               hipStream_t st, bool* done, const MatmulRhs* rhs = nullptr) {
+                               hipStream_t st, bool* done, const MatmulRhs* rhs = nullptr, ProdSrc src = ProdSrc{nullptr, nullptr}) {
     *done = false;
     const int pa = digits_for(ma), pb = digits_for(mb);
     if (!pa || !pb) return 0;
@@ -587,7 +626,7 @@ static int run_int8_plane_path(void* C, const void* A, const void* B, uint32_t b
     Scratch pla(rows_a * pa * Kp, st), plb(have_b ? 1 : (size_t)batch * pb * P * Kp, st);
     if (pla.rc) return pla.rc;
     if (plb.rc) return plb.rc;
-    hipLaunchKernelGGL(k_split_rows, dim3(cdiv(rows_a * (Kp / 4), 256)), dim3(256), 0, st, pla.as<int8_t>(), (const Fr*)A, rows_a, M, N, Kp, pa);
+    hipLaunchKernelGGL(k_split_rows, dim3(cdiv(rows_a * (Kp / 4), 256)), dim3(256), 0, st, pla.as<int8_t>(), (const Fr*)A, src, rows_a, M, N, Kp, pa);
     if (!have_b) hipLaunchKernelGGL(k_split_cols, dim3(cdiv(P, 64), Kp / 64, batch), dim3(256), 0, st, plb.as<int8_t>(), (const Fr*)B, N, P, Kp, pb);
     const PlaneGemm g{pla.as<int8_t>(), have_b ? (const int8_t*)rhs->planes : plb.as<int8_t>(), (Fr*)C, M, P, Kp, pa, pb};
     hipEvent_t t0 = nullptr, t1 = nullptr;
@@ -629,9 +668,22 @@ int zk_fr_matmul_generic(void* C, const void* A, const void* B, uint32_t M, uint
 // path_used (optional, host): 1 generic, 2 small-integer.
 // `batch` products of equally shaped matrices stored one after the other; the bound is taken over the whole stacks, so
 // one path serves every product of the call
+// src.a set: the left operand is the elementwise product of two int32 forms and A is null; the paths that need field elements
+// get them written out first
 static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv,
-                           const MatmulRhs* rhs = nullptr) {
+                           const MatmulRhs* rhs = nullptr, ProdSrc src = ProdSrc{nullptr, nullptr}) {
     hipStream_t st = (hipStream_t)stv;
+    std::unique_ptr<Scratch> a_written;
+    auto write_out = [&]() -> int {          // the product as field elements, once
+        if (!src.a || A) return 0;
+        a_written.reset(new Scratch(sizeof(Fr) * (size_t)batch * M * N, st));
+        if (a_written->rc) return a_written->rc;
+        const size_t na = (size_t)batch * M * N;
+        hipLaunchKernelGGL(k_prod_to_fr, dim3(cdiv(na, 256)), dim3(256), 0, st, a_written->as<Fr>(), src, na);
+        ZK_LAUNCH_CHECK();
+        A = a_written->p;
+        return 0;
+    };
     if (batch == 0 || M == 0 || P == 0) return 0;
     ZK_ARG(N > 0, "zk_fr_matmul: inner dimension is 0");
     ZK_ARG(mode >= 0 && mode <= 2, "zk_fr_matmul: mode must be 0, 1 or 2");
@@ -645,7 +697,8 @@ static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch
         ZK_HIP(hipMemsetAsync(mx.p, 0, 3 * sizeof(unsigned long long), st));
         const size_t nb = (size_t)batch * N * P;
         if (!rhs) hipLaunchKernelGGL(k_absmax, dim3(absmax_grid(nb)), dim3(256), 0, st, mx.as<unsigned long long>() + 1, (const Fr*)B, nb);
-        hipLaunchKernelGGL(k_rowabs, dim3(batch * M), dim3(256), 0, st, mx.as<unsigned long long>() + 2, mx.as<unsigned long long>(), (const Fr*)A, N);      // one pass over A for both of its figures
+        if (src.a) hipLaunchKernelGGL(k_rowabs_prod, dim3(batch * M), dim3(256), 0, st, mx.as<unsigned long long>() + 2, mx.as<unsigned long long>(), src, N);
+        else hipLaunchKernelGGL(k_rowabs, dim3(batch * M), dim3(256), 0, st, mx.as<unsigned long long>() + 2, mx.as<unsigned long long>(), (const Fr*)A, N);      // one pass over A for both of its figures
         ZK_LAUNCH_CHECK();
         void* stage = nullptr;
         int rc = staging(&stage, 24);
@@ -663,6 +716,7 @@ static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch
         }
         if (mode == 2 && !small) { set_error(ZK_ERR_ARG, "zk_fr_matmul: operands do not satisfy the small-integer bound"); return ZK_ERR_ARG; }
     }
+    if (mode == 1 || !small) { int wrc = write_out(); if (wrc) return wrc; }
     if (!small) {
         if (path_used) *path_used = 1;
         hipLaunchKernelGGL(k_matmul, dim3(cdiv(P, TN), cdiv(M, TM), batch), dim3(TM * TN), 0, st, (Fr*)C, (const Fr*)A, (const Fr*)B, M, N, P);
@@ -676,10 +730,11 @@ static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch
     const int planes_log2 = planes_env ? atoi(planes_env) : 30;
     if (planes_log2 > 0 && (unsigned __int128)batch * M * N * P >= ((unsigned __int128)1 << planes_log2) && M >= 32 && P >= 32) {
         bool done = false;
-        const int rc = run_int8_plane_path(C, A, B, batch, M, N, P, ma_, mb_, st, &done, rhs);
+        const int rc = run_int8_plane_path(C, A, B, batch, M, N, P, ma_, mb_, st, &done, rhs, src);
         if (rc) return rc;
         if (done) return 0;
     }
+    { int wrc = write_out(); if (wrc) return wrc; }
     if (fits32) return run_int_path<int>(C, A, B, batch, M, N, P, st);
     if (b_fits32) return run_wide_narrow_path(C, A, B, batch, M, N, P, st);
     return run_int_path<long long>(C, A, B, batch, M, N, P, st);
@@ -760,6 +815,10 @@ int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, 
 }
 int zk_fr_matmul_batched(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv) {
     return matmul_dispatch(C, A, B, batch, M, N, P, mode, path_used, stv);
+}
+int zk_fr_matmul_batched_prod(void* C, const void* a_ints, const void* b_ints, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv) {
+    ZK_ARG(a_ints != nullptr && b_ints != nullptr, "zk_fr_matmul_batched_prod: null int32 form");
+    return matmul_dispatch(C, nullptr, B, batch, M, N, P, mode, path_used, stv, nullptr, ProdSrc{(const int32_t*)a_ints, (const int32_t*)b_ints});
 }
 
 }  // extern "C"

@@ -563,6 +563,24 @@ FrTensor FrTensor::matmul_stack(const FrTensor& x, const FrTensor& y, uint num, 
     matmul_stack_into(out, x, y, num, M, N, P);
     return out;
 }
+FrTensor FrTensor::matmul_stack_prod(const FrTensor& a, const FrTensor& b, const FrTensor& y, uint num, uint M, uint N, uint P) {
+    if ((size_t)a.size != (size_t)num * M * N || b.size != a.size || (size_t)y.size != (size_t)num * N * P) throw std::runtime_error("matmul: incompatible dimensions");
+    if (!a.kept_ints() || !b.kept_ints()) throw std::runtime_error("matmul_stack_prod: both factors need an int32 form");
+    FrTensor out(num * M * P);
+    int path = 0;
+    ZKC(zk_fr_matmul_batched_prod(out.gpu_data, zk_fr_fold_prepared_ints(a.kept_ints()), zk_fr_fold_prepared_ints(b.kept_ints()), y.gpu_data, num, M, N, P, G().matmul_mode, &path, nullptr));
+    G().last_matmul_path = path;
+    return out;
+}
+FrTensor FrTensor::partial_me_prod(const FrTensor& a, const FrTensor& b, const vector<Fr_t>& u, uint cur_dim, uint window_size) {
+    if (a.size != b.size || !a.kept_ints() || !b.kept_ints()) throw std::runtime_error("partial_me_prod: two tensors of one size with int32 forms");
+    if (u.empty() || u.size() > 24 || cur_dim <= ((1u << u.size()) >> 1) || cur_dim > (1u << u.size())) throw std::runtime_error("partial_me_prod: Incompatible dimensions");
+    if ((size_t)a.size % ((size_t)cur_dim * window_size) != 0) throw std::runtime_error("t.size % (cur_dim * window_size) != 0");
+    const size_t other = (size_t)a.size / ((size_t)cur_dim * window_size);
+    FrTensor out((uint)(other * window_size));
+    ZKC(zk_fr_fold_axis_prod(out.gpu_data, a.kept_ints(), b.kept_ints(), u[0].val, (int)u.size(), other, cur_dim, window_size, nullptr));
+    return out;
+}
 void FrTensor::matmul_stack_into(FrTensor& out, const FrTensor& x, const FrTensor& y, uint num, uint M, uint N, uint P) {
     if ((size_t)x.size != (size_t)num * M * N || (size_t)y.size != (size_t)num * N * P || (size_t)out.size != (size_t)num * M * P)
         throw std::runtime_error("matmul: incompatible dimensions");

@@ -184,6 +184,10 @@ class FrTensor {
     FrTensor transpose_stack(uint num, uint M, uint N) const;
     static FrTensor matmul_stack(const FrTensor& x, const FrTensor& y, uint num, uint M, uint N, uint P);
     static void matmul_stack_into(FrTensor& out, const FrTensor& x, const FrTensor& y, uint num, uint M, uint N, uint P);
+    // the same two for a left operand / a tensor that is the elementwise product of a and b, both of which keep an int32 form
+    // (kept_ints): the product itself is never written -- the matrix product reads its exact 64-bit elements, the fold sums them
+    static FrTensor matmul_stack_prod(const FrTensor& a, const FrTensor& b, const FrTensor& y, uint num, uint M, uint N, uint P);
+    static FrTensor partial_me_prod(const FrTensor& a, const FrTensor& b, const vector<Fr_t>& u, uint cur_dim, uint window_size);
     static FrTensor random_int(uint size, uint num_bits);
     static FrTensor random(uint size);
     // all-`x` tensor (replaces the cudaMemset + `+= x` idiom of the reference's callers)

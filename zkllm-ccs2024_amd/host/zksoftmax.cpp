@@ -94,9 +94,11 @@ FrTensor zkSoftmax::compute_rows(uint m, const FrTensor& X, FrTensor& shift, FrT
         m_segments.push_back(std::move(p.second));
     }
     // the product of the segments' table values (the reference multiplies them one by one into a tensor of ones)
+    out_is_product = false;
     if (into) {
         if (into->size != X.size) throw std::invalid_argument("the result must be the same size as X");
         if (Y_segments.size() == 1) { *into = Y_segments[0]; return FrTensor(0); }
+        if (lean_out && product_out_allowed && Y_segments.size() == 2 && Y_segments[0].kept_ints() && Y_segments[1].kept_ints()) { out_is_product = true; return FrTensor(0); }
         mul_segments(into->gpu_data, Y_segments[0], Y_segments[1], N);
         for (size_t i = 2; i < Y_segments.size(); ++i) *into *= Y_segments[i];
         return FrTensor(0);
@@ -253,7 +255,11 @@ FrTensor zkAttnStacked::compute(const FrTensor& Q, const FrTensor& K, const FrTe
         sm_shift.size != num * m)
         throw std::invalid_argument("softmax tensors must be num * m * n (shift: num * m)");
     FrTensor::matmul_stack_into(sm_in, Q, K.transpose_stack(num, n, d), num, m, d, n);
+    // this class reads sm_out in two places, both of which take the product's factors instead (ZKLLM_SOFTMAX_PRODUCT=0 writes it as before)
+    { const char* e = getenv("ZKLLM_SOFTMAX_PRODUCT"); product_out_allowed = !(e && e[0] == '0'); }
     compute_rows(num * m, sm_in, sm_shift, sm_in_shifted, sm_in_segments, sm_out_segments, sm_m_segments, &sm_out);
+    product_out_allowed = false;
+    if (out_is_product) return FrTensor::matmul_stack_prod(sm_out_segments[0], sm_out_segments[1], V, num, m, n, d);
     return FrTensor::matmul_stack(sm_out, V, num, m, n, d);
 }
 
@@ -300,7 +306,7 @@ Fr_t zkAttnStacked::prove_finish(Pending& pending, const FrTensor& Q, const FrTe
     if (sm_in.size != sm_out.size) throw std::invalid_argument("X and Y must have the same size " + to_string(sm_in.size) + " " + to_string(sm_out.size));
     auto out_claim = out.multi_dim_me({u_matmul_out_num, u_matmul_out, w_matmul_out}, {num, m, d});
     zk_record(out_claim);
-    auto sm_out_reduced = sm_out.partial_me(u_matmul_out, m, n);
+    auto sm_out_reduced = out_is_product ? FrTensor::partial_me_prod(sm_out_segments[0], sm_out_segments[1], u_matmul_out, m, n) : sm_out.partial_me(u_matmul_out, m, n);
     auto V_reduced = V.partial_me(w_matmul_out, d, 1);
     auto out_matmul_claim = zkip_stacked(out_claim, sm_out_reduced, V_reduced, u_matmul_out_num, v_matmul_out, v_matmul_out_num, num, n, proof);
 

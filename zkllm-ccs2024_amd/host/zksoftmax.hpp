@@ -10,10 +10,17 @@ class zkSoftmax {
     // With lean_forward set, a tensor among them whose every reader in prove() takes the int32 form (a lookup job large enough
     // to read nothing else, the evaluations, the product of two mapped segments) is written in that form ONLY: its field
     // elements stay unwritten (the tensor is a view of one buffer shared by all of them), and X_shifted may be passed with size 0
-    // and is not written either.  For a caller that hands the tensors to prove() and reads none of them itself.
+    // and is not written either.  zkAttnStacked goes one step further: when both mapped-value tensors are in int32 form only, the
+    // softmax's output (their product, sm_out) is not written either -- the product with V and the fold in the proof read the two
+    // int32 forms (ZKLLM_SOFTMAX_PRODUCT=0 in the environment writes it).  For a caller that hands the tensors to prove() and reads
+    // none of them itself.
     bool lean_forward = false;
     std::shared_ptr<FrTensor> unwritten;      // the buffer those tensors are views of: it must outlive every use of them (it lives as long as this object)
     static uint lean_tensors_last;      // how many digit planes and mapped-value tensors the last compute() left in int32 form only
+    // set by the last compute_rows(..., into) when the output is the product of two mapped-value tensors that exist in int32 form
+    // only: `into` was then NOT written either -- zkAttnStacked multiplies and folds the product from the two int32 forms
+    bool out_is_product = false;
+    bool product_out_allowed = false;      // set by a caller of compute_rows that never reads `into` as field elements
     zkSoftmax(const vector<uint>& bs, uint L, uint M, unsigned long scaling_factor_in, const vector<double>& thetas, uint m, uint n, uint d, uint E);
 
     FrTensor compute(const FrTensor& X, FrTensor& shift, FrTensor& X_shifted, vector<FrTensor>& X_segments, vector<FrTensor>& Y_segments, vector<FrTensor>& m_segments);
