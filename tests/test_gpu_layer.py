@@ -123,7 +123,9 @@ def test_layer_run_again_starts_its_openings_ahead_and_proves_the_same(pv):
 
 def test_tiny_layer_with_every_opening_started_at_its_claim(pv):
     """zkp_openings_set_only_at_claim (ZKLLM_OPEN_AHEAD=0): no plan is learned or used and nothing starts ahead inside a block;
-    the openings of a block start together at its last claim.  Transcript and G1 points are those of the default run."""
+    the openings of a block start together at its last claim, and the stacked attention proof (which opens nothing) is queued
+    and collected behind the last block so that the host reaches those claims early.  Transcript and G1 points are those of
+    the default run and of the oracle, also with the attention proof moved in each of the other ways and in its turn."""
     orc = load_oracle()
     cu, cf = layercfg.tiny(open_weights=True, head_group=2)
     ws = layercfg.tiny_weights(23, cu)
@@ -139,10 +141,11 @@ def test_tiny_layer_with_every_opening_started_at_its_claim(pv):
     pv.lib.zkp_challenge_position.restype = ctypes.c_ulonglong
     pv.lib.zkp_challenge_skip.argtypes = [ctypes.c_ulonglong]
     layer_draws = pv.lib.zkp_challenge_position()
-    g1s = []
+    g1s, learned = [], False
     try:
-        for at_claim in (1, 1, 0, 0):
+        for at_claim, attention in ((1, -1), (1, -1), (0, -1), (0, -1), (1, 0), (1, 1), (1, 2), (0, 3), (0, 1)):
             pv.lib.zkp_openings_set_only_at_claim(at_claim)
+            pv.lib.zkp_layer_set_attention_last(attention)
             pv.seed(12)
             pv.lib.zkp_challenge_skip(ctypes.c_ulonglong(layer_draws))
             pv.transcript_begin()
@@ -152,10 +155,12 @@ def test_tiny_layer_with_every_opening_started_at_its_claim(pv):
             assert (out.host() == exp).all()
             assert got_t.shape == exp_t.shape and (got_t == exp_t).all()
             g1s.append(pv.transcript_g1().copy())
-            # runs that only open at the claim neither learn nor use a plan
-            assert pv.lib.zkp_layer_planned_openings(ctypes.c_void_p(layer)) == (0 if at_claim or len(g1s) < 3 else 9)
+            # runs that only open at the claim neither learn nor use a plan: it is there once a run of the other kind has been
+            learned = learned or not at_claim
+            assert pv.lib.zkp_layer_planned_openings(ctypes.c_void_p(layer)) == (9 if learned else 0)
     finally:
         pv.lib.zkp_openings_set_only_at_claim(0)
+        pv.lib.zkp_layer_set_attention_last(-1)
     pv.layer_free(layer)
     for g in g1s[1:]:
         assert g.shape == g1s[0].shape and (g == g1s[0]).all()

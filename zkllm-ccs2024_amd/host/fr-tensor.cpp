@@ -70,7 +70,15 @@ void zk_write_proof_file(const std::string& path) {
 }
 const std::vector<Fr_t>& zk_transcript() { return G().transcript; }
 void zk_transcript_end() { G().recording = false; }
-void zk_record(const Fr_t& x) { if (G().recording) G().transcript.push_back(x); }
+// entries go to `sink` instead while one is set (a block whose proof is collected out of turn); zk_record_insert puts them in place
+static std::vector<Fr_t>* g_record_sink = nullptr;
+void zk_record_divert(std::vector<Fr_t>* sink) { g_record_sink = sink; }
+void zk_record_insert(size_t pos, const std::vector<Fr_t>& xs) {
+    if (!G().recording || xs.empty()) return;
+    auto& t = G().transcript;
+    t.insert(t.begin() + (pos < t.size() ? pos : t.size()), xs.begin(), xs.end());
+}
+void zk_record(const Fr_t& x) { if (G().recording) (g_record_sink ? *g_record_sink : G().transcript).push_back(x); }
 namespace {
 struct PhaseTimes {
     bool on = false;
@@ -107,11 +115,16 @@ ZkLibraryScope::~ZkLibraryScope() {
 }
 size_t zk_record_reserve() {
     if (!G().recording) return (size_t)-1;
+    if (g_record_sink) throw std::runtime_error("zk_record_reserve: no position can be reserved while the entries are diverted");
     G().transcript.push_back(Fr_t{{0, 0, 0, 0, 0, 0, 0, 0}});
     return G().transcript.size() - 1;
 }
 void zk_record_fill(size_t slot, const Fr_t& x) { if (slot != (size_t)-1 && slot < G().transcript.size()) G().transcript[slot] = x; }
-void zk_record(const std::vector<Fr_t>& xs) { if (G().recording) G().transcript.insert(G().transcript.end(), xs.begin(), xs.end()); }
+void zk_record(const std::vector<Fr_t>& xs) {
+    if (!G().recording) return;
+    auto& t = g_record_sink ? *g_record_sink : G().transcript;
+    t.insert(t.end(), xs.begin(), xs.end());
+}
 
 ostream& operator<<(ostream& os, const Fr_t& x) {
     os << "0x" << std::hex;

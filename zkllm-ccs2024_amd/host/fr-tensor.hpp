@@ -53,6 +53,10 @@ void zk_record(const std::vector<Fr_t>& xs);
 // a transcript position whose value arrives later (an opening that runs beside the prover): reserve keeps the order
 size_t zk_record_reserve();
 void zk_record_fill(size_t slot, const Fr_t& x);
+// a proof collected out of turn: while a sink is set the entries go there (no position can be reserved meanwhile); insert puts
+// them at `pos` of the transcript afterwards -- only once no reserved position is waiting for its value, since it moves those behind
+void zk_record_divert(std::vector<Fr_t>* sink);
+void zk_record_insert(size_t pos, const std::vector<Fr_t>& xs);
 
 // the points of a weight opening (T, T0, T1 per round, then the last generator; z = ONE), kept beside the transcript
 void zk_record_g1(const std::vector<G1Jacobian_t>& points);

@@ -552,6 +552,7 @@ void zkp_openings_use_cross_commitments(int on) { zk_openings_use_cross_commitme
 int zkp_shutdown() { return zk_shutdown(); }
 void zkp_openings_use_row_commitments(int on) { zk_openings_use_row_commitments(on != 0); }
 // on: every weight opening starts at its claim or later (no learned plan, nothing started ahead inside a block)
+void zkp_layer_set_attention_last(int mode) { layer_set_attention_last(mode); }
 void zkp_openings_set_only_at_claim(int on) { zk_openings_set_only_at_claim(on != 0); }
 int zkp_openings_only_at_claim() { return zk_openings_only_at_claim() ? 1 : 0; }
 // off: llama_layer finishes every block before it queues the next (ZKLLM_LAYER_OVERLAP=0)

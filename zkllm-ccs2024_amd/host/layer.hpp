@@ -109,7 +109,9 @@ struct AttnLinearBlock {
 struct AttnStackBlock {
     AttnStackBlock(const LayerConfig& c, const FrTensor& Q_, const FrTensor& K_, const FrTensor& V_);
     const FrTensor& forward();
-    void begin();
+    void begin();      // = draw(); queue();
+    void draw();       // the block's challenges, in the block's turn
+    void queue();      // the device jobs of its proof, any time after draw()
     void finish();
     const LayerConfig& c; const FrTensor &Q_, &K_, &V_;
     zkAttnStacked attn;
@@ -173,6 +175,10 @@ FrTensor attn_reference_block(const LayerConfig& c, const FrTensor& Q, const FrT
 // num_heads the attention block proves inside its forward pass and nothing overlaps it.)
 int layer_blocks_overlap();
 void layer_set_blocks_overlap(int depth);
+// when the stacked attention proof is queued and collected (llama_layer): 0 in its turn, 1 collected last, 2 also queued behind
+// the last block's jobs, 3 queued once the last block is collected; -1 (default): 3 when every opening starts at its claim, else 0.
+// Same transcript in every mode.
+void layer_set_attention_last(int mode);
 FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor& X, LayerTimes* times);
 
 // how long make_random_layer_weights last spent on each part of the setup (ms, device idle at both ends of every part):
