@@ -453,8 +453,8 @@ def test_softmax_compute_and_prove(pv, orc, m, n, d, bs, sf, lim):
 
 
 @pytest.mark.parametrize("num,stacked,m,n,d", [(1, 0, 16, 16, 16), (1, 1, 16, 16, 16), (4, 1, 16, 16, 16), (2, 1, 8, 32, 4), (2, 1, 256, 256, 4), (2, 2, 256, 256, 4),
-                                               (4, 2, 16, 16, 16)])
-def test_attention_forward_and_proof(pv, orc, num, stacked, m, n, d):
+                                               (4, 2, 16, 16, 16), (2, 1, 8, 16, 8)])
+def test_attention_forward_and_proof(pv, orc, monkeypatch, num, stacked, m, n, d):
     """zkAttn (one head) and zkAttnStacked (head-major stacks): forward pass, transcript and returned claim.  stacked == 2:
     zkSoftmax::lean_forward -- at 2 x 256 x 256 scores the lookup and Hadamard jobs read int32 forms alone, so the digit planes
     and the mapped values exist in that form only and the shifted scores are never written (at 4 x 16 x 16 nothing is large
@@ -469,18 +469,23 @@ def test_attention_forward_and_proof(pv, orc, num, stacked, m, n, d):
     orc.orc_transcript_clear()
     orc_check(orc.orc_attn(Q, K, V, num, m, n, d, 1 if stacked else 0, bs, 3, 1, 0, c_u64(16), c_u64(16), thetas, 2, e_out, e_fin))
     e_t = orc_transcript(orc)
-    pv.seed(11)
-    pv.transcript_begin()
-    if stacked == 2:          # poison what the pool hands out next: tensors that stay unwritten must not be read
-        junk = [pv.from_fr(ch(7, num * m * n)) for _ in range(6)]
-        del junk
-    out, fin = pv.attn(pv.from_fr(Q), pv.from_fr(K), pv.from_fr(V), num, m, n, d, stacked, bs, 1, 0, 16, 16, thetas)
-    pv.lib.zkp_transcript_end()
-    assert (out.host() == e_out).all() and (fin == e_fin).all()
-    t = pv.transcript()
-    assert t.shape == e_t.shape and (t == e_t).all()
-    if stacked:          # three digit planes and two mapped-value tensors
-        assert pv.lib.zkp_softmax_lean_tensors_last() == (5 if stacked == 2 and num * m * n >= 1 << 17 else 0)
+    # The stacked proof takes the scores' value at the softmax's point from the folded Q and K instead of reading the scores;
+    # the second run (ZKLLM_CHECK_CLAIMS=1) evaluates the scores as well and throws if the two differ.
+    for check in ((False, True) if stacked else (False,)):
+        if check:
+            monkeypatch.setenv("ZKLLM_CHECK_CLAIMS", "1")
+        pv.seed(11)
+        pv.transcript_begin()
+        if stacked == 2:          # poison what the pool hands out next: tensors that stay unwritten must not be read
+            junk = [pv.from_fr(ch(7, num * m * n)) for _ in range(6)]
+            del junk
+        out, fin = pv.attn(pv.from_fr(Q), pv.from_fr(K), pv.from_fr(V), num, m, n, d, stacked, bs, 1, 0, 16, 16, thetas)
+        pv.lib.zkp_transcript_end()
+        assert (out.host() == e_out).all() and (fin == e_fin).all()
+        t = pv.transcript()
+        assert t.shape == e_t.shape and (t == e_t).all()
+        if stacked:          # three digit planes and two mapped-value tensors
+            assert pv.lib.zkp_softmax_lean_tensors_last() == (5 if stacked == 2 and num * m * n >= 1 << 17 else 0)
 
 
 @pytest.mark.parametrize("num,batch,n_in,n_out,bias", [(1, 4, 8, 8, False), (4, 8, 16, 4, False), (4, 8, 16, 4, True), (3, 5, 6, 7, True)])

@@ -42,6 +42,28 @@ def test_host_fr_ops_match_bigint_and_oracle():
     assert (got[:64] == exp[:64]).all()
 
 
+def test_29_bit_limb_products_match_bigint():
+    """fr29_mul (a b 2^-261 mod r) and fr29_mul_small (a k 2^-58 mod r for a small integer k: the first lookup round of a plain
+    table, whose queries differ by small integers) of the sumcheck kernels, run on the CPU, against big integers: edge operands,
+    random ones, and k at 0, 1, the 32-bit extremes and the routine's own limit."""
+    lib = _lib()
+    rng = random.Random(29)
+    edge = [0, 1, 2, R_MOD - 1, R_MOD - 2, (1 << 29) - 1, 1 << 29, (1 << 232) - 1, 1 << 232, 1 << 254]
+    a = edge + [rng.randrange(R_MOD) for _ in range(600)]
+    b = list(reversed(a))
+    ks = [0, 1, 2, (1 << 29) - 1, 1 << 29, (1 << 32) - 1, 1 << 32, (1 << 33) - 1, (1 << 58) - 1, 12345678901]
+    k = [ks[i % len(ks)] if i < 3 * len(ks) else rng.randrange(1 << rng.choice([8, 16, 31, 32, 33, 58])) for i in range(len(a))]
+    A, B, K = fr_array(a), fr_array(b), np.array(k, dtype=np.uint64)
+    got = np.zeros_like(A)
+    lib.zkp_host_fr29_op.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_long]
+    assert lib.zkp_host_fr29_op(0, _np_ptr(A), _np_ptr(B), K.ctypes.data, _np_ptr(got), len(a)) == 0
+    i261 = pow(1 << 261, -1, R_MOD)
+    assert fr_ints(got) == [x * y * i261 % R_MOD for x, y in zip(a, b)]
+    assert lib.zkp_host_fr29_op(1, _np_ptr(A), _np_ptr(B), K.ctypes.data, _np_ptr(got), len(a)) == 0
+    i58 = pow(1 << 58, -1, R_MOD)
+    assert fr_ints(got) == [x * kk * i58 % R_MOD for x, kk in zip(a, k)]
+
+
 def test_unreduced_sums_of_products_reduce_to_the_sum_of_montgomery_products():
     """wide_mac / wide_redc (the sumcheck rounds' accumulator: products added as 512-bit integers, one reduction at the end)
     against big integers: sum a_i b_i / R mod r for operands below r, for arbitrary 256-bit operands (the accumulator does

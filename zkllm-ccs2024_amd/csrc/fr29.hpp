@@ -81,6 +81,40 @@ ZK_HD Fr29 fr29_mul(const Fr29& a, const Fr29& b) {
         return s;
     });
 }
+// a k 2^-58 mod r for a small k = k0 + k1 2^29 (two limbs: any k below 2^58): a Montgomery product with radix 2^58 -- eighteen
+// limb products for a k and eighteen for the two reduction steps, against 162 of fr29_mul.  a as for fr29_mul (limb 8 below
+// 2^30); the result is non-negative and below a k / 2^58 + r, limbs normalised.
+ZK_HD Fr29 fr29_mul_small(const Fr29& a, uint32_t k0, uint32_t k1) {
+    Fr29 t;
+    auto col = [&](int j) {
+        int64_t s = 0;
+        if (j < 9) s += (int64_t)a.l[j] * (int64_t)k0;
+        if (j >= 1) s += (int64_t)a.l[j - 1] * (int64_t)k1;
+        return s;
+    };
+    int64_t q = col(0);
+    const int32_t m0 = (int32_t)((0u - (uint32_t)q) & R29M);      // r = 1 mod 2^29
+    q += (int64_t)m0;
+    int64_t carry = q >> 29;
+    q = carry + col(1) + (int64_t)m0 * fr29_p(1);
+    const int32_t m1 = (int32_t)((0u - (uint32_t)q) & R29M);
+    q += (int64_t)m1;
+    carry = q >> 29;
+#pragma unroll
+    for (int j = 2; j <= 10; ++j) {
+        q = carry;
+        if (j <= 9) q += col(j);
+        if (j <= 8) q += (int64_t)m0 * fr29_p(j);
+        if (j - 1 <= 8) q += (int64_t)m1 * fr29_p(j - 1);
+        if (j < 10) {
+            t.l[j - 2] = (int32_t)((uint32_t)q & R29M);
+            carry = q >> 29;
+        } else {
+            t.l[8] = (int32_t)q;
+        }
+    }
+    return t;
+}
 // limb-wise with a carry pass; the results are non-negative where the value is
 ZK_HD Fr29 fr29_add(const Fr29& a, const Fr29& b) {
     Fr29 r;

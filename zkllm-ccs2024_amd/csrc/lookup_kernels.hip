@@ -535,8 +535,9 @@ __global__ void __launch_bounds__(TPB) k_lookup_ints_check(int32_t* __restrict__
     if (!ok) atomicMin(n_ok, j);          // *n_ok starts at 0xFFFFFFFF
 }
 // query i and 1 / (query + beta) from the int32 forms (HintSrc); unit as in inv_by_hint
-__device__ __forceinline__ Fr query_inv_ints(size_t i, const HintSrc& h, Fr& a, bool& unit) {
+__device__ __forceinline__ Fr query_inv_ints(size_t i, const HintSrc& h, Fr& a, bool& unit, int32_t* query = nullptr) {
     const int32_t hi = __builtin_nontemporal_load(h.hint_ints + i);
+    if (query) *query = hi;
     const int64_t d = (int64_t)hi - (int64_t)h.low_int;
     const bool in_table = d >= 0 && d < (int64_t)h.N;
     const uint32_t j = in_table ? (uint32_t)d : 0u;
@@ -808,7 +809,9 @@ __global__ void __launch_bounds__(TPB) k_lookup_first29(Fr* __restrict__ partial
 // Writes the second round's folded tensors (h2 each), the third round's eq table (h2 / 2 entries) and both rounds' five sums
 // (partials: round 1 at [0, 5 gridDim), round 2 behind it).  At most 256 quads per lane; the launch site checks.
 // what every lane needs of the challenges, made on the host so that it arrives in scalar registers
-struct First2Consts { Fr29 vq1, vq2, b29, b2, c261; };      // v1 2^261, v2 2^261, beta, 2 beta, 2^261 mod r (a product with it leaves the value, reduced)
+// v1 2^261, v2 2^261, beta, 2 beta, 2^261 mod r (a product with it leaves the value, reduced); v1 2^58 and its negative (for
+// fr29_mul_small: the first fold of a plain table's queries, which differ by a small integer)
+struct First2Consts { Fr29 vq1, vq2, b29, b2, c261, vs1, nvs1; };
 static First2Consts first2_consts(const Fr& beta, const Fr& v1_mont, const Fr& v2_mont) {
     First2Consts c;
     c.vq1 = fr29_mul(fr29_repack(v1_mont), fr29_2_266());
@@ -818,13 +821,21 @@ static First2Consts first2_consts(const Fr& beta, const Fr& v1_mont, const Fr& v
     Fr29 one29 = fr29_zero();
     one29.l[0] = 1;
     c.c261 = fr29_mul(fr29_2_522(), one29);
+    Fr29 two63 = fr29_zero();
+    two63.l[2] = 32;                                                    // 2^63: v1 2^256 2^63 2^-261 = v1 2^58
+    c.vs1 = fr29_mul(fr29_repack(v1_mont), two63);
+    c.nvs1 = fr29_sub_plus_r(fr29_r(), c.vs1);                          // 2 r - v1 2^58: non-negative (the product is below 2 r)
     return c;
 }
-__global__ void __launch_bounds__(TPB) k_lookup_first2_29(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ nS, const Fr* __restrict__ E, const Fr beta,
+template <bool PLAIN> __global__ void __launch_bounds__(TPB) k_lookup_first2_29(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ nS, const Fr* __restrict__ E, const Fr beta,
                                                           const Fr v1_mont, const First2Consts cs, size_t h2, Fr* __restrict__ nE3, const HintSrc hs) {
     __shared__ uint32_t rare[3][8][TPB];                               // round 1: the three weighted terms of the pairs with an inverse of their own, per lane
     const size_t h1 = 2 * h2;
     const Fr29 vq1 = cs.vq1, vq2 = cs.vq2, b29 = cs.b29, b2 = cs.b2, c261 = cs.c261;
+    // A plain table (no mapped values): two queries that are table entries differ by the small integer d = q1 - q0, and with
+    // a0 (s0 + beta) = a1 (s1 + beta) = 1 (as Montgomery products) the pair's M - 4 is (a0 - a1) d (as a Montgomery product).  That product and the fold v1 d are small-operand
+    // products (fr29_mul_small); wx then sums E (M - 4) 2^-58 instead of E M.
+    constexpr bool plain = PLAIN;                                      // the launch site: hs.sout_ints == nullptr
     Wide29 wx = wide29_zero();                                         // round 1: sum of E M over the pairs of unit inverses, times 2^-5
     __shared__ uint32_t qsum[4][9][TPB];                               // sums of the inverses of the four quarters, per lane (registers are short here)
     uint32_t se[9];                                                    // sum of E over the pairs of unit inverses
@@ -862,11 +873,25 @@ __global__ void __launch_bounds__(TPB) k_lookup_first2_29(Fr* __restrict__ parti
         auto first_round_pair = [&](size_t i, const Fr& e, int qa, int qb, Fr29& fa, Fr29& fs) {
             Fr s0w, s1w, a0w, a1w;
             bool unit0 = false, unit1 = false;
-            s0w = query_inv_ints(i, hs, a0w, unit0);
-            s1w = query_inv_ints(i + h1, hs, a1w, unit1);
+            int32_t q0 = 0, q1 = 0;
+            s0w = query_inv_ints(i, hs, a0w, unit0, &q0);
+            s1w = query_inv_ints(i + h1, hs, a1w, unit1, &q1);
             qsum_add(qa, a0w);
             qsum_add(qb, a1w);
-            if (unit0 && unit1) {
+            if constexpr (PLAIN) { if (unit0 && unit1) {
+                const Fr29 a0 = fr29_repack(a0w), a1 = fr29_repack(a1w), s0 = fr29_repack(s0w);
+                sum9_add(se, e);
+                const int64_t d = (int64_t)q1 - (int64_t)q0;
+                const bool ng = d < 0;
+                const uint64_t k = ng ? 0ull - (uint64_t)d : (uint64_t)d;       // below 2^32
+                const uint32_t k0 = (uint32_t)k & R29M, k1 = (uint32_t)(k >> 29);
+                const Fr29 da = fr29_sub_plus_r(a1, a0), nda = fr29_sub_plus_r(a0, a1);
+                wide29_mac(wx, fr29_repack(e), fr29_mul_small(ng ? da : nda, k0, k1));      // (a0 - a1) d 2^-58
+                fa = fr29_add(a0, fr29_mul(vq1, da));
+                fs = fr29_add(s0, fr29_mul_small(ng ? cs.nvs1 : cs.vs1, k0, k1));        // s0 + v1 d
+                return;
+            } }
+            if (!PLAIN && unit0 && unit1) {
                 const Fr29 a0 = fr29_repack(a0w), a1 = fr29_repack(a1w), s0 = fr29_repack(s0w), s1 = fr29_repack(s1w);
                 sum9_add(se, e);
                 const Fr29 M = fr29_mul(fr29_add(a0, a1), fr29_add(fr29_add(s0, s1), b2));
@@ -907,12 +932,20 @@ __global__ void __launch_bounds__(TPB) k_lookup_first2_29(Fr* __restrict__ parti
     // round 1
     {
         Fr acc[5];
-        const Fr acc_em = fr29_canon_pack(fr29_mul(wide29_redc(wx), fix));
+        Fr29 em29 = fr29_mul(wide29_redc(wx), fix);
+        if (plain) {
+            // The inverses are inverses under the Montgomery product, a (s + beta) = 2^256, and M is such a product:
+            // M - 4 = (a0 - a1) d 2^-261 in this file's 29-bit form.  The small products left 2^-58: 2^-203 is missing.
+            Fr29 two58 = fr29_zero();
+            two58.l[2] = 1;
+            em29 = fr29_mul(em29, two58);
+        }
+        const Fr acc_em = fr29_canon_pack(em29);
         constexpr uint32_t RINV[8] = {4269129792u, 334977897u, 165441631u, 2876230287u, 1333208682u, 1912866698u, 805346647u, 465471123u};
         Fr k;
 #pragma unroll
         for (int l = 0; l < 8; ++l) k.v[l] = RINV[l];
-        const Fr one = mont_mul(sum9_residue(se), k), two = add(one, one), four = add(two, two);
+        const Fr one = mont_mul(sum9_residue(se), k), two = add(one, one), four = plain ? big_zero<8>() : add(two, two);      // plain: acc_em is the sum of E (M - 4) already
         Fr c0s, c1s, c2s;
 #pragma unroll
         for (int l = 0; l < 8; ++l) { c0s.v[l] = rare[0][l][threadIdx.x]; c1s.v[l] = rare[1][l][threadIdx.x]; c2s.v[l] = rare[2][l][threadIdx.x]; }
@@ -2453,7 +2486,8 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
                 ZK_HIP(hipEventCreate(&t1));
                 ZK_HIP(hipEventRecord(t0, st));
             }
-            hipLaunchKernelGGL(k_lookup_first2_29, dim3(nb2), dim3(TPB), 0, st, part.as<Fr>(), w2, w2 + h2, cE, b, vm, cs, h2, nE3, *hs);
+            if (hs->sout_ints) hipLaunchKernelGGL(k_lookup_first2_29<false>, dim3(nb2), dim3(TPB), 0, st, part.as<Fr>(), w2, w2 + h2, cE, b, vm, cs, h2, nE3, *hs);
+            else hipLaunchKernelGGL(k_lookup_first2_29<true>, dim3(nb2), dim3(TPB), 0, st, part.as<Fr>(), w2, w2 + h2, cE, b, vm, cs, h2, nE3, *hs);
             if (g_round_timer.on) {
                 ZK_HIP(hipEventRecord(t1, st));
                 std::lock_guard<std::mutex> lk(g_round_timer.mu);

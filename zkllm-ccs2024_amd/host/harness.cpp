@@ -7,6 +7,7 @@
 
 #include "../../include/zkllm_hip.h"
 #include "../csrc/field.hpp"
+#include "../csrc/fr29.hpp"
 #include "fr-tensor.hpp"
 #include "polynomial.hpp"
 #include "proof.hpp"
@@ -89,6 +90,25 @@ int zkp_host_fr_wide_dot(const u32* a, const u32* b, u32* out, long n) {
     }
     const zk::Fr r = zk::wide_redc(w);
     memcpy(out, r.v, 32);
+    ZKP_END
+}
+// the 29-bit-limb routines of the sumcheck kernels (csrc/fr29.hpp) on the CPU; operands canonical, results canonical
+// op 0: a b 2^-261 (fr29_mul)   1: a k 2^-58 for the small integer k[i] below 2^58 (fr29_mul_small)
+int zkp_host_fr29_op(int op, const u32* a, const u32* b, const unsigned long long* k, u32* out, long n) {
+    ZKP_TRY
+    for (long i = 0; i < n; ++i) {
+        zk::Fr x, y;
+        memcpy(x.v, a + 8 * i, 32);
+        memcpy(y.v, b + 8 * i, 32);
+        zk::Fr29 r;
+        switch (op) {
+            case 0: r = zk::fr29_mul(zk::fr29_repack(x), zk::fr29_repack(y)); break;
+            case 1: r = zk::fr29_mul_small(zk::fr29_repack(x), (u32)(k[i] & zk::R29M), (u32)(k[i] >> 29)); break;
+            default: throw std::runtime_error("bad op");
+        }
+        const zk::Fr c = zk::fr29_canon_pack(r);
+        memcpy(out + 8 * i, c.v, 32);
+    }
     ZKP_END
 }
 int zkp_host_fp_op(int op, const u32* a, const u32* b, u32* out, long n) {

@@ -147,7 +147,7 @@ void zkSoftmax::claim_record(Pending& pending, const FrTensor& Y, const vector<F
 }
 
 Fr_t zkSoftmax::prove_end(Pending& pending, const FrTensor& X, const FrTensor& shift, const vector<FrTensor>& X_segments, const vector<FrTensor>& Y_segments,
-                          const vector<Fr_t>& v_Y, vector<Polynomial>& proof, bool evaluate_first) {
+                          const vector<Fr_t>& v_Y, vector<Polynomial>& proof, bool evaluate_first, const Fr_t* X_at_v_Y) {
     // all evaluations at v_Y in one pass over the tensors (zksoftmax.cu:189-196 evaluates them one by one).  They need
     // nothing from the sumcheck jobs: with evaluate_first they run on the caller's stream while the jobs finish on theirs
     // (worth it when the jobs are long, as for a stack of heads; beside short jobs the contention costs more than the
@@ -155,7 +155,9 @@ Fr_t zkSoftmax::prove_end(Pending& pending, const FrTensor& X, const FrTensor& s
     vector<const FrTensor*> at_v;
     for (uint i = L; i < K; ++i) at_v.push_back(&Y_segments[i - L]);
     for (uint i = 0; i < K; ++i) at_v.push_back(&X_segments[i]);
-    at_v.push_back(&X);
+    const char* check_env = getenv("ZKLLM_CHECK_CLAIMS");
+    const bool read_X = !X_at_v_Y || (check_env && check_env[0] == '1');
+    if (read_X) at_v.push_back(&X);
     vector<Fr_t> evals;
     Fr_t shift_const_opening;
     std::string failure;
@@ -182,7 +184,8 @@ Fr_t zkSoftmax::prove_end(Pending& pending, const FrTensor& X, const FrTensor& s
     Fr_t minus_X_shifted_claim = {0, 0, 0, 0, 0, 0, 0, 0};
     for (int i = (int)bs.size() - 1; i >= 0; --i) minus_X_shifted_claim = minus_X_shifted_claim * Fr_t({bs[i], 0, 0, 0, 0, 0, 0, 0}) + X_seg_claims[i];
 
-    auto X_opening = evals.back();
+    if (X_at_v_Y && read_X && evals.back() != *X_at_v_Y) throw std::runtime_error("zkSoftmax::prove_end: the value handed in for X at v_Y is not X's");
+    auto X_opening = X_at_v_Y ? *X_at_v_Y : evals.back();
     zk_record(shift_const_opening);
     zk_record(X_opening);
     if (shift_const_opening - minus_X_shifted_claim != X_opening) throw std::runtime_error("X claim is not correct");
@@ -324,6 +327,16 @@ Fr_t zkAttnStacked::prove_finish(Pending& pending, const FrTensor& Q, const FrTe
     vector<Fr_t> w_matmul_in(v_sm.begin(), v_sm.end() - ceilLog2(num) - ceilLog2(m));
     auto Q_reduced = Q.partial_me(u_matmul_in, m, d);
     auto K_reduced = K.partial_me(w_matmul_in, n, d);
-    auto sm_in_claim = prove_end(pending, sm_in, sm_shift, sm_in_segments, sm_out_segments, v_sm, proof, true);
+    // The scores at v_sm = (w_matmul_in, u_matmul_in, u_matmul_in_num): they are Q K^T head by head, so their extension there is
+    // sum_h eq(u_num, h) sum_k Q_reduced[h][k] K_reduced[h][k] -- the sum the closing inner-product argument starts from.  The
+    // 2^27 scores are not read for it.  (sum_k p[k] = 2^bits times the extension of p at (1/2, ..., 1/2).)
+    Fr_t scores_at_v;
+    {
+        FrTensor prod = Q_reduced * K_reduced;
+        const uint bits = ceilLog2(d);
+        const Fr_t half = inv(Fr_t{{2, 0, 0, 0, 0, 0, 0, 0}});
+        scores_at_v = prod.multi_dim_me({u_matmul_in_num, vector<Fr_t>(bits, half)}, {num, d}) * Fr_t{{1u << bits, 0, 0, 0, 0, 0, 0, 0}};
+    }
+    auto sm_in_claim = prove_end(pending, sm_in, sm_shift, sm_in_segments, sm_out_segments, v_sm, proof, true, &scores_at_v);
     return zkip_stacked(sm_in_claim, Q_reduced, K_reduced, u_matmul_in_num, v_matmul_in, v_matmul_in_num, num, d, proof);
 }

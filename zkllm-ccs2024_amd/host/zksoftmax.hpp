@@ -44,7 +44,9 @@ class zkSoftmax {
                        const vector<Fr_t>& v_Y, const Fr_t& r_seg, const Fr_t& alpha_seg, const Fr_t& beta_seg);
     void claim_record(Pending& pending, const FrTensor& Y, const vector<Fr_t>& u_Y);
     Fr_t prove_end(Pending& pending, const FrTensor& X, const FrTensor& shift, const vector<FrTensor>& X_segments, const vector<FrTensor>& Y_segments,
-                   const vector<Fr_t>& v_Y, vector<Polynomial>& proof, bool evaluate_first = false);
+                   const vector<Fr_t>& v_Y, vector<Polynomial>& proof, bool evaluate_first = false, const Fr_t* X_at_v_Y = nullptr);
+    // X_at_v_Y (addition): the value of X at v_Y when the caller has it from elsewhere -- X is then not read (with
+    // ZKLLM_CHECK_CLAIMS=1 in the environment it is evaluated all the same and compared)
 
    protected:
     // compute() for `rows` rows of n scores (rows = m for one head, num * m for a stack of heads: rows are independent)
