@@ -385,6 +385,9 @@ int zk_rescale_ints(void* out, void* rem, void* rem_ints, const void* in, uint32
 /* the same, and out_ints receives the rescaled values as int32; synchronises and reports in *out_fits_host whether every one
  * of them fits (0: out_ints must not be used) */
 int zk_rescale_ints_both(void* out, void* out_ints, int* out_fits_host, void* rem, void* rem_ints, const void* in, uint32_t scaling_factor, size_t n, void* stream);
+/* the same with the answer left on the device: *bad_flag_dev (4 bytes of device memory) is cleared, then set by the kernel when a
+ * rescaled value does not fit int32; the caller reads it (zk_memcpy_d2h) whenever the kernel is through and a wait costs nothing */
+int zk_rescale_ints_both_flag(void* out, void* out_ints, void* bad_flag_dev, void* rem, void* rem_ints, const void* in, uint32_t scaling_factor, size_t n, void* stream);
 int zk_i32_fill(void* dst_i32, int32_t value, size_t n, void* stream);       /* n int32 slots set to value (padding of an int32 form) */
 /* zkrelu_decomp_kernel zkrelu.cu:8-29: the same rescaling, then sign (1 when the rescaled value is >= 0), magnitude and max(., 0) */
 int zk_relu_decomp(void* res, void* sign, void* mag, void* rem, const void* in, uint32_t scaling_factor, size_t n, void* stream);

@@ -3200,6 +3200,18 @@ int zk_rescale_ints_both(void* out, void* out_ints, int* out_fits_host, void* re
     *out_fits_host = f ? 0 : 1;
     return 0;
 }
+// the same without the round trip: *bad_flag_dev (4 bytes of device memory) is cleared and then raised by the kernel when a
+// rescaled value does not fit; the caller reads it once the kernel is through, whenever that suits it
+int zk_rescale_ints_both_flag(void* out, void* out_ints, void* bad_flag_dev, void* rem, void* rem_ints, const void* in, uint32_t scaling_factor, size_t n, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(scaling_factor >= 1, "zk_rescale: scaling factor is 0");
+    ZK_ARG(out_ints != nullptr && bad_flag_dev != nullptr, "zk_rescale_ints_both_flag: null argument");
+    ZK_ARG(rem != nullptr || rem_ints != nullptr, "zk_rescale_ints_both_flag: the remainders need at least one form");
+    ZK_HIP(hipMemsetAsync(bad_flag_dev, 0, 4, st));
+    if (n == 0) return 0;
+    LAUNCH1D(k_rescale, n, st, (Fr*)out, (Fr*)rem, (int32_t*)rem_ints, (const Fr*)in, (int64_t)scaling_factor, n, (int32_t*)out_ints, (uint32_t*)bad_flag_dev);
+    return 0;
+}
 int zk_i32_fill(void* dst, int32_t value, size_t n, void* st) {
     LAUNCH1D(k_i32_fill, n, st, (int32_t*)dst, value, n);
     return 0;

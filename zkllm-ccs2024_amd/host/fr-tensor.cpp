@@ -260,6 +260,26 @@ void FoldCache::reset() {
     if (prepared) zk_fr_fold_prepared_free(prepared);
     prepared = nullptr;
     tried = false;
+    if (unchecked) zk_free(unchecked);
+    unchecked = nullptr;
+}
+void FoldCache::settle() {
+    if (!unchecked) return;
+    uint32_t bad = 0;
+    const int rc = zk_memcpy_d2h(&bad, unchecked, 4, nullptr);          // waits for the producing kernel
+    zk_free(unchecked);
+    unchecked = nullptr;
+    if (rc || bad) {
+        if (prepared) zk_fr_fold_prepared_free(prepared);
+        prepared = nullptr;          // tried stays set: the elements are known not to be 32-bit integers
+    }
+    zk_check(rc, "zk_memcpy_d2h");
+}
+void* FrTensor::ints_for_producer_unchecked(void** bad_flag_dev) {
+    void* ints = ints_for_producer();
+    ZKC(zk_malloc(&fold_cache->unchecked, 4));
+    *bad_flag_dev = fold_cache->unchecked;
+    return ints;
 }
 void FrTensor::keep_for_folds() {
     if (!fold_cache) fold_cache = std::make_shared<FoldCache>();
@@ -431,6 +451,7 @@ static FrTensor fold_axis_all(const FrTensor& t, const vector<Fr_t>& u, uint cur
     if ((size_t)t.size % ((size_t)cur_dim * window) != 0) throw std::runtime_error("t.size % (cur_dim * window_size) != 0");
     const size_t other = (size_t)t.size / ((size_t)cur_dim * window);
     if (FoldCache* fc = t.fold_cache.get(); fc && u.size() <= 24 && cur_dim <= (1u << u.size())) {
+        if (fc->unchecked) fc->settle();
         if (!fc->tried) {
             fc->tried = true;
             ZKC(zk_fr_fold_prepare(&fc->prepared, t.gpu_data, t.size, nullptr));

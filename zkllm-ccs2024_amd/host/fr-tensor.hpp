@@ -99,6 +99,10 @@ struct MatmulRhsCache {
 struct FoldCache {
     void* prepared = nullptr;
     bool tried = false;
+    // set while nobody has looked yet whether the producer's int32 form holds every element (ints_for_producer_unchecked): 4 bytes
+    // of device memory that the producing kernel raises when one did not fit.  settle() reads it and drops the form if so.
+    void* unchecked = nullptr;
+    void settle();
     void reset();
     ~FoldCache() { reset(); }
 };
@@ -182,7 +186,14 @@ class FrTensor {
     // A tensor whose int32 form is written by the kernel that writes the tensor: allocates that form (zk_fr_fold_prepared_new)
     // and keeps it as keep_for_folds would; returns its device address for the kernel.  Call before the kernel is queued.
     void* ints_for_producer();
-    const void* kept_ints() const { return fold_cache && fold_cache->prepared ? fold_cache->prepared : nullptr; }       // the handle, or null
+    // the same for a producer that finds out on the device whether every element fits: *bad_flag_dev is what the kernel raises
+    // when one does not (the kernel's launch clears it first); it is read at the first question for the form (kept_ints, a
+    // fold), so the producer's caller does not wait for the kernel
+    void* ints_for_producer_unchecked(void** bad_flag_dev);
+    const void* kept_ints() const {       // the handle, or null
+        if (fold_cache && fold_cache->unchecked) fold_cache->settle();
+        return fold_cache && fold_cache->prepared ? fold_cache->prepared : nullptr;
+    }
     // additions for stacks of `num` equally shaped matrices stored one after the other: every M x N matrix transposed,
     // and the num products x_i (M x N) * y_i (N x P)
     FrTensor transpose_stack(uint num, uint M, uint N) const;

@@ -192,7 +192,7 @@ void* zkp_fr_scalarop(int op, void* a, const u32* s) {
 int zkp_fr_keep_as_matmul_rhs(void* a) { ZKP_TRY FT(a).keep_as_matmul_rhs(); ZKP_END }
 int zkp_fr_keep_for_folds(void* a) { ZKP_TRY FT(a).keep_for_folds(); ZKP_END }
 // 1 when the tensor's folds read its int32 form, 0 when it keeps none (not asked to, or its elements are not 32-bit integers)
-int zkp_fr_folds_from_ints(void* a) { return FT(a).fold_cache && FT(a).fold_cache->prepared ? 1 : 0; }
+int zkp_fr_folds_from_ints(void* a) { return FT(a).kept_ints() ? 1 : 0; }
 int zkp_fr_add_inplace(void* a, void* b) { ZKP_TRY FT(a) += FT(b); ZKP_END }
 void* zkp_fc_forward_over_view(void* w, void* x, u32 in_dim, u32 out_dim) {
     ZKP_TRY

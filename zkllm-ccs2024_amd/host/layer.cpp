@@ -90,6 +90,7 @@ void layer_config_from_env(LayerConfig& c) {
 RmsNormBlock::RmsNormBlock(const LayerConfig& c, const Weight& w, const FrTensor& X, const FrTensor& rms_inv)
     : c(c), w(w), X(X), rms_inv(rms_inv), rs1(c.sf_linear), rs2(c.sf_linear), g(1, c.embed_dim, FrTensor::view(w.weight)) {
     rs1.lean = rs2.lean = true;      // nothing here reads the remainders but their range proofs
+    rs2.out_ints_lazy = true;        // the block's output is the left operand of fully connected layers: their proofs fold its int32 form
 }
 const FrTensor& RmsNormBlock::forward() {
     g_inv_rms.emplace(g(rms_inv));
@@ -223,6 +224,7 @@ AttnStackBlock::AttnStackBlock(const LayerConfig& c, const FrTensor& Q_, const F
       rs2(c.sf_attn) {
     if (c.embed_dim % c.num_heads) throw std::runtime_error("embed_dim must be a multiple of num_heads");
     rs1.lean = rs2.lean = true;
+    rs1.out_ints_lazy = true;        // the block's output: folded by the output projection's proof
 }
 const FrTensor& AttnStackBlock::forward() {
     const uint seq = c.seq_len, E = c.embed_dim, H = c.num_heads, d = E / H;
@@ -450,6 +452,7 @@ FfnBlock::FfnBlock(const LayerConfig& c, const Weight& up, const Weight& gate, c
       gate_layer(c.embed_dim, c.hidden_dim, FrTensor::view(gate.weight)), down_layer(c.hidden_dim, c.embed_dim, FrTensor::view(down.weight)), up_rescale(c.sf_linear),
       gate_rescale(c.sf_gate), hidden_rescale(c.sf_linear), down_rescale(c.sf_linear), swiglu(c.swiglu_low, c.swiglu_len, swiglu_values) {
     up_rescale.lean = gate_rescale.lean = hidden_rescale.lean = down_rescale.lean = true;
+    up_rescale.out_ints_lazy = gate_rescale.out_ints_lazy = hidden_rescale.out_ints_lazy = true;      // read by the activation lookup, the product and the down projection's proof
 }
 const FrTensor& FfnBlock::forward() {
     up_out.emplace(up_layer(input));

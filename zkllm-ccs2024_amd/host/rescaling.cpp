@@ -6,7 +6,7 @@
 
 Rescaling::Rescaling(uint scaling_factor) : scaling_factor(scaling_factor), tl_rem(-static_cast<int>(scaling_factor >> 1), scaling_factor), rem_tensor_ptr(nullptr) {}
 
-FrTensor Rescaling::operator()(const FrTensor& X) { return rescale(X, false); }
+FrTensor Rescaling::operator()(const FrTensor& X) { return rescale(X, out_ints_lazy); }
 FrTensor Rescaling::rescale(const FrTensor& X, bool ints_out) {
     rem_hold = std::make_shared<FrTensor>(X.size);
     rem_tensor_ptr = rem_hold.get();
@@ -19,7 +19,11 @@ FrTensor Rescaling::rescale(const FrTensor& X, bool ints_out) {
     // (the same condition under which prove_begin pads the int32 form alone and the lookup job reads nothing else)
     const bool ints_only = lean && zk_lookup_ints_suffice((size_t)1 << ceilLog2(X.size), tl_rem.table.size);
     void* rem_fr = ints_only ? nullptr : rem_tensor_ptr->gpu_data;
-    if (ints_out) {
+    if (ints_out && out_ints_lazy) {
+        void* flag = nullptr;
+        void* oi = out.ints_for_producer_unchecked(&flag);
+        ZKC(zk_rescale_ints_both_flag(out.gpu_data, oi, flag, rem_fr, rem_hold->ints_for_producer(), X.gpu_data, scaling_factor, X.size, nullptr));
+    } else if (ints_out) {
         int fits = 0;
         ZKC(zk_rescale_ints_both(out.gpu_data, out.ints_for_producer(), &fits, rem_fr, rem_hold->ints_for_producer(), X.gpu_data, scaling_factor, X.size, nullptr));
         if (!fits) out.drop_kept();

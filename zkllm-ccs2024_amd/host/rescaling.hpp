@@ -17,6 +17,11 @@ class Rescaling {
     // *rem_tensor_ptr then stay unwritten.  For a caller that hands the object to prove() and never reads the remainders
     // itself (the layer's blocks).
     bool lean = false;
+    // addition.  out_ints_lazy: operator() and rescale(X, true) give the rescaled tensor an int32 form without waiting for the
+    // kernel: whether every value fits is read from the device at the first question for that form (FrTensor::kept_ints, a
+    // fold, an evaluation), which drops it if not.  The folds and evaluations of the proofs downstream then read 4 bytes per
+    // element and multiply by 32-bit integers.
+    bool out_ints_lazy = false;
     FrTensor operator()(const FrTensor& X);
     // addition: operator() that, with ints_out, also gives the rescaled tensor an int32 form when every value fits (one
     // host round trip): for outputs that go into a table lookup or a product with another such tensor
