@@ -172,11 +172,14 @@ def test_mapping_lookup(pv, orc, D, low, length):
     assert t.shape == e_t.shape and (t == e_t).all()
 
 
+@pytest.mark.parametrize("lazy", [0, 1])
 @pytest.mark.parametrize("n,sf,bits,fits", [(5000, 1 << 8, 30, True), (1 << 17, 1 << 8, 38, True), (1 << 17, 1 << 8, 41, False), (70000, 1 << 16, 36, True)])
-def test_rescaling_that_gives_its_output_an_int32_form(pv, orc, n, sf, bits, fits):
+def test_rescaling_that_gives_its_output_an_int32_form(pv, orc, n, sf, bits, fits, lazy):
     """Rescaling::rescale(X, true): output and proof transcript are the oracle's; the output keeps an int32 form exactly when
     every rescaled value fits 32 bits (41-bit inputs over 2^8 do not); the remainders' int32 form serves the proof either way
-    (70000 and 5000 elements: padded; 2^17: read from the int32 form alone)."""
+    (70000 and 5000 elements: padded; 2^17: read from the int32 form alone).  lazy (Rescaling::out_ints_lazy): whether the
+    values fit is read from the device at the first use of the form, not by the rescaling; same results, and a fold of the
+    output afterwards (from the int32 form when it was kept) is the oracle's."""
     x = np.random.default_rng(n + bits).integers(-(1 << bits), 1 << bits, n)
     x[0], x[1] = (1 << bits) - 1, -(1 << bits)
     X = fr_array([int(v) % R_MOD for v in x])
@@ -187,12 +190,22 @@ def test_rescaling_that_gives_its_output_an_int32_form(pv, orc, n, sf, bits, fit
     e_t = orc_transcript(orc)
     pv.seed(77)
     pv.transcript_begin()
-    out = pv.rescale_ints_prove(pv.from_fr(X), sf)
+    pv.lib.zkp_rescale_set_lazy(lazy)
+    try:
+        out = pv.rescale_ints_prove(pv.from_fr(X), sf)
+    finally:
+        pv.lib.zkp_rescale_set_lazy(0)
     pv.lib.zkp_transcript_end()
     assert (out.host() == e_out).all()
     assert pv.folds_from_ints(out) == (1 if fits else 0)
     t = pv.transcript()
     assert t.shape == e_t.shape and (t == e_t).all()
+    k = (n - 1).bit_length()
+    u = mt_random_vec(np.random.RandomState(5), k)
+    exp, out_n = np.zeros((n, 8), np.uint32), np.zeros(1, np.int64)
+    orc_check(orc.orc_fr_partial_me(e_out, n, u, k, n, 1, exp, out_n))
+    got = pv.partial_me(out, u, n, 1).host()
+    assert got.shape[0] == out_n[0] == 1 and (got == exp[:1]).all()
 
 
 @pytest.mark.parametrize("D,low,length", [(1000, -16, 32), (100000, -16, 32), (1 << 17, -20, 40), (1 << 18, -20, 40), (300000, -16, 32)])

@@ -336,9 +336,12 @@ void* zkp_rescale(void* X, u32 sf, void** rem_out) {
     ZKP_END_PTR
 }
 // Rescaling::rescale(X, true) + prove: the rescaled tensor comes back with its int32 form when every value fits
+static bool g_rescale_lazy = false;
+void zkp_rescale_set_lazy(int on) { g_rescale_lazy = on != 0; }      // the next zkp_rescale_ints_prove calls run with Rescaling::out_ints_lazy
 void* zkp_rescale_ints_prove(void* X, u32 sf) {
     ZKP_TRY
     Rescaling rs(sf);
+    rs.out_ints_lazy = g_rescale_lazy;
     FrTensor out = rs.rescale(FT(X), true);
     rs.prove(FT(X), out);
     return new FrTensor(std::move(out));
