@@ -448,7 +448,7 @@ def main():
         "config": {"workload": f"C5: LLaMa-2-7B-shape decoder layer proof, seq {seq}, hidden 4096, 32 heads x 128, FFN 11008, "
                                "random-init fixed-point weights (scale 2^16), generators of size out_features<<5, all nine weight openings included "
                                "(value: their points are read ahead from the seeded challenge stream, so all nine run from the start of the layer, batched by "
-                               "generator size; layer_openings_at_claim_s: the same layer with every opening started at its claim; layer_openings_at_claim_blocks_in_turn_s: that, and every "
+                               "generator size; layer_openings_at_claim_s: the same layer with every opening started at its claim and the attention proof, which opens nothing, queued and collected behind the last block; layer_openings_at_claim_blocks_in_turn_s: that, and every "
                                "block's proofs collected before the next block begins -- the reference's order of work, block by block; in the other two figures a block's forward pass and "
                                "proof jobs are queued while the proofs of the two blocks before it are still being collected, transcript unchanged); attention proved "
                                + (f"{args.head_group} heads at a time as head-major stacks (zkAttnStacked)" if args.head_group else "head by head"),
