@@ -45,7 +45,7 @@ def test_host_fr_ops_match_bigint_and_oracle():
 def test_29_bit_limb_products_match_bigint():
     """fr29_mul (a b 2^-261 mod r) and fr29_mul_small (a k 2^-58 mod r for a small integer k: the first lookup round of a plain
     table, whose queries differ by small integers) of the sumcheck kernels, run on the CPU, against big integers: edge operands,
-    random ones, and k at 0, 1, the 32-bit extremes and the routine's own limit."""
+    random ones, and k at 0, 1, the 32-bit extremes and the routine's own limit; fr29_from_small (a signed integer as a residue)."""
     lib = _lib()
     rng = random.Random(29)
     edge = [0, 1, 2, R_MOD - 1, R_MOD - 2, (1 << 29) - 1, 1 << 29, (1 << 232) - 1, 1 << 232, 1 << 254]
@@ -62,6 +62,11 @@ def test_29_bit_limb_products_match_bigint():
     assert lib.zkp_host_fr29_op(1, _np_ptr(A), _np_ptr(B), K.ctypes.data, _np_ptr(got), len(a)) == 0
     i58 = pow(1 << 58, -1, R_MOD)
     assert fr_ints(got) == [x * kk * i58 % R_MOD for x, kk in zip(a, k)]
+    signed = [0, 1, -1, 2 ** 31 - 1, -2 ** 31, 2 ** 29, -2 ** 29, 2 ** 29 - 1, -(2 ** 29 - 1), 2 ** 58 - 1, -(2 ** 58 - 1)] + [rng.randrange(-2 ** 57, 2 ** 57) for _ in range(200)]
+    Ks = np.array(signed, dtype=np.int64)
+    got = np.zeros((len(signed), 8), np.uint32)
+    assert lib.zkp_host_fr29_op(2, _np_ptr(A), _np_ptr(B), Ks.ctypes.data, _np_ptr(got), len(signed)) == 0
+    assert fr_ints(got) == [v % R_MOD for v in signed]
 
 
 def test_unreduced_sums_of_products_reduce_to_the_sum_of_montgomery_products():

@@ -115,6 +115,26 @@ ZK_HD Fr29 fr29_mul_small(const Fr29& a, uint32_t k0, uint32_t k1) {
     }
     return t;
 }
+// x mod r for an integer of magnitude below 2^58, canonical (x itself, or r - |x|)
+ZK_HD Fr29 fr29_from_small(int64_t x) {
+    Fr29 t = fr29_r();
+    const bool ng = x < 0;
+    const uint64_t y = ng ? 0ull - (uint64_t)x : (uint64_t)x;
+    const int32_t y0 = (int32_t)((uint32_t)y & R29M), y1 = (int32_t)((uint32_t)(y >> 29) & R29M);
+    if (ng) {
+        const int32_t s0 = t.l[0] - y0;
+        t.l[0] = (int32_t)((uint32_t)s0 & R29M);
+        const int32_t s1 = t.l[1] - y1 + (s0 >> 29);
+        t.l[1] = (int32_t)((uint32_t)s1 & R29M);
+        t.l[2] += s1 >> 29;                                 // limb 2 of r is far above 1: no further borrow
+    } else {
+#pragma unroll
+        for (int i = 2; i < 9; ++i) t.l[i] = 0;
+        t.l[0] = y0;
+        t.l[1] = y1;
+    }
+    return t;
+}
 // limb-wise with a carry pass; the results are non-negative where the value is
 ZK_HD Fr29 fr29_add(const Fr29& a, const Fr29& b) {
     Fr29 r;

@@ -809,6 +809,22 @@ __global__ void __launch_bounds__(TPB) k_lookup_first29(Fr* __restrict__ partial
 // Writes the second round's folded tensors (h2 each), the third round's eq table (h2 / 2 entries) and both rounds' five sums
 // (partials: round 1 at [0, 5 gridDim), round 2 behind it).  At most 256 quads per lane; the launch site checks.
 // what every lane needs of the challenges, made on the host so that it arrives in scalar registers
+// v 2^58 and its negative in 29-bit limbs (for fr29_mul_small): what a fold by v of two small integers multiplies by
+struct SmallFold { Fr29 vs, nvs; };
+static SmallFold small_fold_consts(const Fr& v_mont) {
+    SmallFold c;
+    Fr29 two63 = fr29_zero();
+    two63.l[2] = 32;                                                    // 2^63: v 2^256 2^63 2^-261 = v 2^58
+    c.vs = fr29_mul(fr29_repack(v_mont), two63);
+    c.nvs = fr29_sub_plus_r(fr29_r(), c.vs);                            // 2 r - v 2^58: non-negative (the product is below 2 r)
+    return c;
+}
+// x0 + v (x1 - x0) for 32-bit integers, canonical: one small-operand product
+__device__ __forceinline__ Fr fold_small(int64_t x0, int64_t d, const SmallFold& c) {
+    const bool ng = d < 0;
+    const uint64_t k = ng ? 0ull - (uint64_t)d : (uint64_t)d;
+    return fr29_canon_pack(fr29_add(fr29_from_small(x0), fr29_mul_small(ng ? c.nvs : c.vs, (uint32_t)k & R29M, (uint32_t)(k >> 29))));
+}
 // v1 2^261, v2 2^261, beta, 2 beta, 2^261 mod r (a product with it leaves the value, reduced); v1 2^58 and its negative (for
 // fr29_mul_small: the first fold of a plain table's queries, which differ by a small integer)
 struct First2Consts { Fr29 vq1, vq2, b29, b2, c261, vs1, nvs1; };
@@ -821,10 +837,9 @@ static First2Consts first2_consts(const Fr& beta, const Fr& v1_mont, const Fr& v
     Fr29 one29 = fr29_zero();
     one29.l[0] = 1;
     c.c261 = fr29_mul(fr29_2_522(), one29);
-    Fr29 two63 = fr29_zero();
-    two63.l[2] = 32;                                                    // 2^63: v1 2^256 2^63 2^-261 = v1 2^58
-    c.vs1 = fr29_mul(fr29_repack(v1_mont), two63);
-    c.nvs1 = fr29_sub_plus_r(fr29_r(), c.vs1);                          // 2 r - v1 2^58: non-negative (the product is below 2 r)
+    const SmallFold sf = small_fold_consts(v1_mont);
+    c.vs1 = sf.vs;
+    c.nvs1 = sf.nvs;
     return c;
 }
 template <bool PLAIN> __global__ void __launch_bounds__(TPB) k_lookup_first2_29(Fr* __restrict__ partials, Fr* __restrict__ nA, Fr* __restrict__ nS, const Fr* __restrict__ E, const Fr beta,
@@ -1152,15 +1167,15 @@ __device__ __forceinline__ Fr imac64_finish(const uint32_t (&acc)[12]) {
     return add(mont_mul(lo, one), hi);
 }
 __global__ void __launch_bounds__(TPB) k_hadamard_round2_ints(Fr* __restrict__ partials, const int32_t* __restrict__ X, const int32_t* __restrict__ Y, Fr* __restrict__ outx,
-                                                              Fr* __restrict__ outy, const Fr* __restrict__ E, const Fr v_mont, size_t n_out, Fr* __restrict__ nE) {
+                                                              Fr* __restrict__ outy, const Fr* __restrict__ E, const SmallFold vc, size_t n_out, Fr* __restrict__ nE) {
     uint32_t a0[12], a2[12], ax[12];
 #pragma unroll
     for (int i = 0; i < 12; ++i) a0[i] = a2[i] = ax[i] = 0;
     for (size_t t = (size_t)blockIdx.x * TPB + threadIdx.x; t < n_out; t += (size_t)gridDim.x * TPB) {
         const int64_t x0 = X[t], x1 = X[t + n_out], y0 = Y[t], y1 = Y[t + n_out];
         const int64_t dx = x1 - x0, dy = y1 - y0;
-        outx[t] = add(fr_from_i64(x0), mont_mul(v_mont, fr_from_i64(dx)));
-        outy[t] = add(fr_from_i64(y0), mont_mul(v_mont, fr_from_i64(dy)));
+        outx[t] = fold_small(x0, dx, vc);
+        outy[t] = fold_small(y0, dy, vc);
         const Fr e = E[t];
         const Fr ne = neg(e);
         if (nE && t < n_out / 2) nE[t] = add(e, E[t + n_out / 2]);
@@ -2672,7 +2687,7 @@ static int hadamard_queue(SumJob& job, const Fr* const* Xs, int K, const Fr* E, 
         break;                                                                                                                    \
     }
         if (r == 0 && K == 2 && ints && ints[0] && ints[1])
-            hipLaunchKernelGGL(k_hadamard_round2_ints, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), ints[0], ints[1], w, w + half, cE, vm, half, nE);
+            hipLaunchKernelGGL(k_hadamard_round2_ints, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), ints[0], ints[1], w, w + half, cE, small_fold_consts(vm), half, nE);
         else if (K == 2 && limbs29() && half > (size_t)SPLIT_HALF && half <= (size_t)256 * nb * TPB)      // 29-bit limbs inside the kernel; its unreduced sums hold 256 pairs per lane
             hipLaunchKernelGGL(k_hadamard_round29, dim3(nb), dim3(TPB), 0, st, part.as<Fr>(), w, w + half, cur[0], cur[1], cE, vm, half, nE);
         else

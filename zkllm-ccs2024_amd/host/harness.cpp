@@ -93,7 +93,7 @@ int zkp_host_fr_wide_dot(const u32* a, const u32* b, u32* out, long n) {
     ZKP_END
 }
 // the 29-bit-limb routines of the sumcheck kernels (csrc/fr29.hpp) on the CPU; operands canonical, results canonical
-// op 0: a b 2^-261 (fr29_mul)   1: a k 2^-58 for the small integer k[i] below 2^58 (fr29_mul_small)
+// op 0: a b 2^-261 (fr29_mul)   1: a k 2^-58 for the small integer k[i] below 2^58 (fr29_mul_small)   2: the signed integer k[i] (fr29_from_small)
 int zkp_host_fr29_op(int op, const u32* a, const u32* b, const unsigned long long* k, u32* out, long n) {
     ZKP_TRY
     for (long i = 0; i < n; ++i) {
@@ -104,6 +104,7 @@ int zkp_host_fr29_op(int op, const u32* a, const u32* b, const unsigned long lon
         switch (op) {
             case 0: r = zk::fr29_mul(zk::fr29_repack(x), zk::fr29_repack(y)); break;
             case 1: r = zk::fr29_mul_small(zk::fr29_repack(x), (u32)(k[i] & zk::R29M), (u32)(k[i] >> 29)); break;
+            case 2: r = zk::fr29_from_small((long long)k[i]); break;
             default: throw std::runtime_error("bad op");
         }
         const zk::Fr c = zk::fr29_canon_pack(r);
