@@ -195,6 +195,9 @@ int zk_fr_matmul_batched_prod(void* C, const void* a_ints, const void* b_ints, c
  * zk_fr_matmul(C, A, B, M, N, P, ...) with B's part of the preparation taken from the handle (bit-identical results). */
 int zk_fr_matmul_rhs_prepare(void** prepared, const void* B, uint32_t N, uint32_t P, void* stream);
 int zk_fr_matmul_rhs(void* C, const void* A, const void* prepared, uint32_t M, int mode, int* path_used, void* stream);
+/* the same for a left operand given by its int32 form (M * N int32 on the device, zk_fr_fold_prepared_ints): the bound pass and the
+ * digit planes read 4 bytes per element; the paths that read field elements get them written out first.  Same C. */
+int zk_fr_matmul_rhs_ints(void* C, const void* a_ints, const void* prepared, uint32_t M, int mode, int* path_used_host, void* stream);
 int zk_fr_matmul_rhs_free(void* prepared);
 
 /* ---- inner-product sumcheck (zkip_poly_kernel + 3 sums, zkfc.cu:94-138) ----------------------------- */

@@ -473,6 +473,14 @@ def test_matmul_with_a_kept_right_operand_and_layers_over_views(pv):
                 assert fr_ints(got) == [int(v) % R_MOD for v in (X.astype(object) @ W.astype(object)).reshape(-1)], (planes, rep)
             got = pv.fc_forward_over_view(hW, pv.from_i64(X), N, P).host()
             assert fr_ints(got) == [int(v) % R_MOD for v in (X.astype(object) @ W.astype(object)).reshape(-1)]
+            # a left operand that keeps an int32 form is read from it (zk_fr_matmul_rhs_ints), extremes included: same product
+            Xi = rng.integers(-2 ** 31, 2 ** 31, (M, N)).astype(np.int64) if whi <= 2 ** 13 else X.copy()
+            Xi[0, :3] = [-2 ** 31, 2 ** 31 - 1, 0]
+            hXi = pv.from_i64(Xi)
+            pv.keep_for_folds(hXi)
+            assert pv.folds_from_ints(hXi) == 1
+            got = pv.matmul(hXi, hW, M, N, P).host()
+            assert fr_ints(got) == [int(v) % R_MOD for v in (Xi.astype(object) @ W.astype(object)).reshape(-1)], planes
             pv.add_inplace(hW, hD)                    # the weight changes: nothing stale may be used
             W2 = W + D
             got = pv.matmul(pv.from_i64(X), hW, M, N, P).host()

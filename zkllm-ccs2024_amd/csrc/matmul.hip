@@ -216,8 +216,9 @@ __global__ void __launch_bounds__(256) k_rowabs(unsigned long long* __restrict__
 }
 // A left operand that exists as the elementwise product of two tensors in int32 form (a softmax's output: the product of two
 // segments' table values): its elements are exact 64-bit integers, read at 8 bytes each instead of 32.
+// b null: the operand is a itself, a tensor read from its int32 form.
 struct ProdSrc { const int32_t* a; const int32_t* b; };
-__device__ __forceinline__ long long prod_at(const ProdSrc& s, size_t i) { return (long long)s.a[i] * (long long)s.b[i]; }
+__device__ __forceinline__ long long prod_at(const ProdSrc& s, size_t i) { return s.b ? (long long)s.a[i] * (long long)s.b[i] : (long long)s.a[i]; }
 // k_rowabs for such an operand
 __global__ void __launch_bounds__(256) k_rowabs_prod(unsigned long long* __restrict__ out, unsigned long long* __restrict__ out_max, const ProdSrc src, uint32_t ncol) {
     const size_t base = (size_t)blockIdx.x * ncol;
@@ -809,6 +810,12 @@ int zk_fr_matmul_rhs(void* C, const void* A, const void* prepared, uint32_t M, i
     const MatmulRhs* r = (const MatmulRhs*)prepared;
     ZK_ARG(r != nullptr, "zk_fr_matmul_rhs: null handle");
     return matmul_dispatch(C, A, r->B, 1, M, r->N, r->P, mode, path_used, stv, r);
+}
+// the same with the left operand given by its int32 form (M * N int32 on the device): 4 bytes read per element instead of 32
+int zk_fr_matmul_rhs_ints(void* C, const void* a_ints, const void* prepared, uint32_t M, int mode, int* path_used, void* stv) {
+    const MatmulRhs* r = (const MatmulRhs*)prepared;
+    ZK_ARG(r != nullptr && a_ints != nullptr, "zk_fr_matmul_rhs_ints: null argument");
+    return matmul_dispatch(C, nullptr, r->B, 1, M, r->N, r->P, mode, path_used, stv, r, ProdSrc{(const int32_t*)a_ints, nullptr});
 }
 int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv) {
     return matmul_dispatch(C, A, B, 1, M, N, P, mode, path_used, stv);

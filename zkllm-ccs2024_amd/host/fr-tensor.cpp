@@ -580,7 +580,10 @@ FrTensor FrTensor::matmul(const FrTensor& x, const FrTensor& y, uint M, uint N, 
         ZKC(zk_fr_matmul_rhs_prepare(&rc->prepared, y.gpu_data, N, P, nullptr));
         rc->N = N; rc->P = P;
     }
-    if (rc) ZKC(zk_fr_matmul_rhs(out.gpu_data, x.gpu_data, rc->prepared, M, G().matmul_mode, &path, nullptr));
+    // a left operand with an int32 form (a rescaled activation) is read from it, except where the caller asked for the generic product
+    const void* xi = (rc && G().matmul_mode != 1) ? x.kept_ints() : nullptr;
+    if (xi) ZKC(zk_fr_matmul_rhs_ints(out.gpu_data, zk_fr_fold_prepared_ints(xi), rc->prepared, M, G().matmul_mode, &path, nullptr));
+    else if (rc) ZKC(zk_fr_matmul_rhs(out.gpu_data, x.gpu_data, rc->prepared, M, G().matmul_mode, &path, nullptr));
     else ZKC(zk_fr_matmul(out.gpu_data, x.gpu_data, y.gpu_data, M, N, P, G().matmul_mode, &path, nullptr));
     G().last_matmul_path = path;
     return out;
