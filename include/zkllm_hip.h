@@ -189,6 +189,11 @@ int zk_fr_matmul_batched(void* C, const void* A, const void* B, uint32_t batch, 
  * (zkSoftmax::compute multiplies the segments' table values into a tensor first, zksoftmax.cu:160-166). */
 int zk_fr_matmul_batched_prod(void* C, const void* a_ints, const void* b_ints, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used_host,
                               void* stream);
+/* zk_fr_matmul_batched with the products written as 64-bit integers (C64: batch * M * P int64 on the device), for a product whose
+ * only reader takes that form (the attention scores, read once by zk_softmax_shift_decompose_i64).  Only the matrix-core path does
+ * that: *taken_host is 1 when it ran, 0 when the operands or the shape do not allow it -- nothing is written then and the caller
+ * falls back to zk_fr_matmul_batched.  No counterpart in the reference (zkAttn::compute, zksoftmax.cu:237-243, writes field elements). */
+int zk_fr_matmul_batched_i64(void* C64, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int* taken_host, void* stream);
 /* The right operand of many products (a layer's weight in zkFC::operator(), zkfc.cu:44-58) examined once: its largest magnitude
  * for the small-integer bound and, when it holds small integers, its int8 digit planes in the GEMM's layout.  No counterpart in
  * the reference, which converts nothing.  B stays alive and unmodified while the handle is used; zk_fr_matmul_rhs is
@@ -406,6 +411,9 @@ int zk_softmax_decompose_ints(void* const* planes, void* const* int_planes, cons
  * planes[k] where int_planes[k] is given (digit k is written as int32 only). */
 int zk_softmax_shift_decompose(void* shift, void* out_shifted, void* const* planes, void* const* int_planes, const void* X, uint32_t rows, uint32_t cols, double scale,
                                const uint32_t* bs_host, int K, void* stream);
+/* the same over scores given as 64-bit integers (rows * cols int64 on the device) */
+int zk_softmax_shift_decompose_i64(void* shift, void* out_shifted, void* const* planes, void* const* int_planes, const void* X64, uint32_t rows, uint32_t cols, double scale,
+                                   const uint32_t* bs_host, int K, void* stream);
 
 /* ---- measurement helpers (no counterpart in the reference) ---------------------------------------- */
 /* v_mad_u64_u32 issue peak of the device: 16 independent chains per lane, no memory traffic */

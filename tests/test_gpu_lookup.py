@@ -484,9 +484,15 @@ def test_attention_forward_and_proof(pv, orc, monkeypatch, num, stacked, m, n, d
     e_t = orc_transcript(orc)
     # The stacked proof takes the scores' value at the softmax's point from the folded Q and K instead of reading the scores;
     # the second run (ZKLLM_CHECK_CLAIMS=1) evaluates the scores as well and throws if the two differ.
-    for check in ((False, True) if stacked else (False,)):
-        if check:
+    # The third run of the lean variant lowers the matrix-core threshold so that the scores are written as 64-bit integers only
+    # (zk_fr_matmul_batched_i64 -> zk_softmax_shift_decompose_i64; sm_in stays unwritten).
+    for check in ((False, True, "i64") if stacked == 2 else (False, True) if stacked else (False,)):
+        monkeypatch.delenv("ZKLLM_CHECK_CLAIMS", raising=False)
+        monkeypatch.delenv("ZKLLM_MATMUL_PLANES", raising=False)
+        if check is True:
             monkeypatch.setenv("ZKLLM_CHECK_CLAIMS", "1")
+        if check == "i64":
+            monkeypatch.setenv("ZKLLM_MATMUL_PLANES", "1")
         pv.seed(11)
         pv.transcript_begin()
         if stacked == 2:          # poison what the pool hands out next: tensors that stay unwritten must not be read
@@ -499,6 +505,7 @@ def test_attention_forward_and_proof(pv, orc, monkeypatch, num, stacked, m, n, d
         assert t.shape == e_t.shape and (t == e_t).all()
         if stacked:          # three digit planes and two mapped-value tensors
             assert pv.lib.zkp_softmax_lean_tensors_last() == (5 if stacked == 2 and num * m * n >= 1 << 17 else 0)
+            assert pv.lib.zkp_softmax_scores_i64_last() == (1 if check == "i64" and m >= 32 and n >= 32 else 0)
 
 
 @pytest.mark.parametrize("num,batch,n_in,n_out,bias", [(1, 4, 8, 8, False), (4, 8, 16, 4, False), (4, 8, 16, 4, True), (3, 5, 6, 7, True)])

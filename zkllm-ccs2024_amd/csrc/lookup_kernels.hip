@@ -1489,8 +1489,10 @@ __device__ __forceinline__ void softmax_digits(const PlanePtrs& planes, const In
 }
 static constexpr int SHIFT_ROW_CACHE = 2048;
 // K > 0: the shifted scores are decomposed where they are written (k_softmax_decompose's planes without its pass over them)
+// X64 set: the scores are given as 64-bit integers (a matrix product written in that form) and X is not read
 __global__ void __launch_bounds__(TPB) k_softmax_shift(Fr* __restrict__ shift, Fr* __restrict__ out, const Fr* __restrict__ X, uint32_t rows, uint32_t cols, double scale,
-                                                       const PlanePtrs planes, const IntPlanePtrs ints, uint32_t* __restrict__ flag, const U32Pack8 bs, int K) {
+                                                       const PlanePtrs planes, const IntPlanePtrs ints, uint32_t* __restrict__ flag, const U32Pack8 bs, int K,
+                                                       const int64_t* __restrict__ X64 = nullptr) {
     __shared__ double term[TPB / 64][64];
     // Rows of up to SHIFT_ROW_CACHE scores are read once: the first pass leaves each score as a 64-bit integer in LDS and the
     // second takes it from there (a score that is no 64-bit integer raises the flag: its digits could not be formed either).
@@ -1500,16 +1502,23 @@ __global__ void __launch_bounds__(TPB) k_softmax_shift(Fr* __restrict__ shift, F
     const uint32_t row = blockIdx.x * (TPB / 64) + w;
     const bool live = row < rows;                         // a whole wave is live or idle; idle waves still reach every barrier
     const Fr* xr = X + (size_t)(live ? row : 0) * cols;
+    const int64_t* xr64 = X64 ? X64 + (size_t)(live ? row : 0) * cols : nullptr;
     double total = 0.0;
     for (uint32_t j0 = 0; j0 < cols; j0 += 64) {
         const uint32_t j = j0 + lane;
         double tv = 0.0;
         if (live && j < cols) {
-            const Fr x = xr[j];
-            const int64_t xi = fr_to_i64(x);
-            if (cached) {
-                cache[w][j] = xi;
-                if (!equal(fr_from_i64(xi), x)) atomicOr(flag, 2u);
+            int64_t xi;
+            if (xr64) {
+                xi = xr64[j];
+                if (cached) cache[w][j] = xi;
+            } else {
+                const Fr x = xr[j];
+                xi = fr_to_i64(x);
+                if (cached) {
+                    cache[w][j] = xi;
+                    if (!equal(fr_from_i64(xi), x)) atomicOr(flag, 2u);
+                }
             }
             tv = zkd::exp_det((double)xi / scale);
         }
@@ -1531,7 +1540,7 @@ __global__ void __launch_bounds__(TPB) k_softmax_shift(Fr* __restrict__ shift, F
     if (lane == 0) shift[row] = sh;
     Fr* orow = out + (size_t)row * cols;
     for (uint32_t j = lane; j < cols; j += 64) {
-        const Fr xs = sub(cached ? fr_from_i64(cache[w][j]) : xr[j], sh);
+        const Fr xs = sub(cached ? fr_from_i64(cache[w][j]) : (xr64 ? fr_from_i64(xr64[j]) : xr[j]), sh);
         if (out) orow[j] = xs;
         if (K > 0) softmax_digits(planes, ints, flag, xs, bs, K, (size_t)row * cols + j);
     }
@@ -3244,8 +3253,20 @@ int zk_softmax_shift(void* shift, void* out_shifted, const void* X, uint32_t row
     ZK_LAUNCH_CHECK();
     return 0;
 }
+static int softmax_shift_decompose(void* shift, void* out_shifted, void* const* planes, void* const* int_planes, const void* X, const void* X64, uint32_t rows, uint32_t cols,
+                                   double scale, const uint32_t* bs_host, int K, void* stv);
 int zk_softmax_shift_decompose(void* shift, void* out_shifted, void* const* planes, void* const* int_planes, const void* X, uint32_t rows, uint32_t cols, double scale,
                                const uint32_t* bs_host, int K, void* stv) {
+    return softmax_shift_decompose(shift, out_shifted, planes, int_planes, X, nullptr, rows, cols, scale, bs_host, K, stv);
+}
+// the same over scores given as 64-bit integers (rows * cols int64 on the device, zk_fr_matmul_batched_i64)
+int zk_softmax_shift_decompose_i64(void* shift, void* out_shifted, void* const* planes, void* const* int_planes, const void* X64, uint32_t rows, uint32_t cols, double scale,
+                                   const uint32_t* bs_host, int K, void* stv) {
+    ZK_ARG(X64 != nullptr, "zk_softmax_shift_decompose_i64: null scores");
+    return softmax_shift_decompose(shift, out_shifted, planes, int_planes, nullptr, X64, rows, cols, scale, bs_host, K, stv);
+}
+static int softmax_shift_decompose(void* shift, void* out_shifted, void* const* planes, void* const* int_planes, const void* X, const void* X64, uint32_t rows, uint32_t cols,
+                                   double scale, const uint32_t* bs_host, int K, void* stv) {
     hipStream_t st = (hipStream_t)stv;
     if (rows == 0) return 0;
     ZK_ARG(cols >= 1 && scale > 0.0, "zk_softmax_shift: bad shape or scale");
@@ -3261,7 +3282,8 @@ int zk_softmax_shift_decompose(void* shift, void* out_shifted, void* const* plan
     Scratch flag(4, st);
     if (flag.rc) return flag.rc;
     ZK_HIP(hipMemsetAsync(flag.p, 0, 4, st));
-    hipLaunchKernelGGL(k_softmax_shift, dim3(cdiv(rows, TPB / 64)), dim3(TPB), 0, st, (Fr*)shift, (Fr*)out_shifted, (const Fr*)X, rows, cols, scale, pp, ip, flag.as<uint32_t>(), bs, K);
+    hipLaunchKernelGGL(k_softmax_shift, dim3(cdiv(rows, TPB / 64)), dim3(TPB), 0, st, (Fr*)shift, (Fr*)out_shifted, (const Fr*)X, rows, cols, scale, pp, ip, flag.as<uint32_t>(), bs, K,
+                       (const int64_t*)X64);
     ZK_LAUNCH_CHECK();
     uint32_t f = 0;
     int rc = read_flag(flag.as<uint32_t>(), &f, st);

@@ -436,7 +436,12 @@ __global__ void __launch_bounds__(256) k_split_cols(int8_t* __restrict__ planes,
 // Fragments: lane l supplies row (or column) l % 32 and the 16 contraction bytes 16 (l / 32) + 0..15 of a 32-byte step for
 // both operands alike, so whatever order the instruction takes the bytes in, every product pairs equal k.  Outputs:
 // register r of lane l is row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of the 32 x 32 tile.
-struct PlaneGemm { const int8_t* A; const int8_t* B; Fr* C; uint32_t M, P, Kp; int pa, pb; };
+// C64 set: the products are written there as 64-bit integers (8 bytes an element) and C is not written
+struct PlaneGemm { const int8_t* A; const int8_t* B; Fr* C; uint32_t M, P, Kp; int pa, pb; long long* C64; };
+__device__ __forceinline__ void gemm_store(const PlaneGemm& g, size_t at, long long v) {
+    if (g.C64) g.C64[at] = v;
+    else g.C[at] = fr_from_i64(v);
+}
 __global__ void __launch_bounds__(256) k_gemm_i8_planes(const PlaneGemm g) {
     __shared__ __attribute__((aligned(16))) int8_t sA[GBM * GLD];
     __shared__ __attribute__((aligned(16))) int8_t sB[GBN * GLD];
@@ -505,7 +510,7 @@ __global__ void __launch_bounds__(256) k_gemm_i8_planes(const PlaneGemm g) {
         for (int r = 0; r < 16; ++r) {
             const uint32_t row = m0 + wm * 64 + (q >> 1) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
             const uint32_t col = n0 + wn * 64 + (q & 1) * 32 + (lane & 31);
-            if (row < g.M && col < g.P) g.C[(b * g.M + row) * (size_t)g.P + col] = fr_from_i64(tot[q][r]);
+            if (row < g.M && col < g.P) gemm_store(g, (b * g.M + row) * (size_t)g.P + col, tot[q][r]);
         }
 }
 // The same product for up to three planes a side (every projection and attention product of the LLaMa layer): all plane pairs
@@ -576,7 +581,7 @@ template <int PA, int PB> __global__ void __launch_bounds__(256, 2) k_gemm_i8_pl
         for (int s = 0; s < NS; ++s) v += (unsigned long long)(long long)acc[s][r] << (8 * s);
         const uint32_t row = m0 + wm * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         const uint32_t col = n0 + wn * 32 + (lane & 31);
-        if (row < g.M && col < g.P) g.C[(b * g.M + row) * (size_t)g.P + col] = fr_from_i64((long long)v);
+        if (row < g.M && col < g.P) gemm_store(g, (b * g.M + row) * (size_t)g.P + col, (long long)v);
     }
 }
 template <int PA> static bool launch_gemm_all_b(int pb, dim3 grid, hipStream_t st, const PlaneGemm& g) {
@@ -615,7 +620,7 @@ static int digits_for(unsigned long long absmax) {      // planes needed for |x|
 // small integers, its digit planes in the GEMM's layout -- neither is computed again per product.
 struct MatmulRhs { const void* B = nullptr; uint32_t N = 0, P = 0, Kp = 0; unsigned long long mb = ~0ull; int pb = 0; void* planes = nullptr; };
 static int run_int8_plane_path(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, unsigned long long ma, unsigned long long mb,
-                               hipStream_t st, bool* done, const MatmulRhs* rhs = nullptr, ProdSrc src = ProdSrc{nullptr, nullptr}) {
+                               hipStream_t st, bool* done, const MatmulRhs* rhs = nullptr, ProdSrc src = ProdSrc{nullptr, nullptr}, long long* C64 = nullptr) {
     *done = false;
     const int pa = digits_for(ma), pb = digits_for(mb);
     if (!pa || !pb) return 0;
@@ -629,7 +634,7 @@ static int run_int8_plane_path(void* C, const void* A, const void* B, uint32_t b
     if (plb.rc) return plb.rc;
     hipLaunchKernelGGL(k_split_rows, dim3(cdiv(rows_a * (Kp / 4), 256)), dim3(256), 0, st, pla.as<int8_t>(), (const Fr*)A, src, rows_a, M, N, Kp, pa);
     if (!have_b) hipLaunchKernelGGL(k_split_cols, dim3(cdiv(P, 64), Kp / 64, batch), dim3(256), 0, st, plb.as<int8_t>(), (const Fr*)B, N, P, Kp, pb);
-    const PlaneGemm g{pla.as<int8_t>(), have_b ? (const int8_t*)rhs->planes : plb.as<int8_t>(), (Fr*)C, M, P, Kp, pa, pb};
+    const PlaneGemm g{pla.as<int8_t>(), have_b ? (const int8_t*)rhs->planes : plb.as<int8_t>(), (Fr*)C, M, P, Kp, pa, pb, C64};
     hipEvent_t t0 = nullptr, t1 = nullptr;
     if (g_gemm_timer.on) {
         ZK_HIP(hipEventCreate(&t0));
@@ -672,7 +677,8 @@ int zk_fr_matmul_generic(void* C, const void* A, const void* B, uint32_t M, uint
 // src.a set: the left operand is the elementwise product of two int32 forms and A is null; the paths that need field elements
 // get them written out first
 static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv,
-                           const MatmulRhs* rhs = nullptr, ProdSrc src = ProdSrc{nullptr, nullptr}) {
+                           const MatmulRhs* rhs = nullptr, ProdSrc src = ProdSrc{nullptr, nullptr}, long long* C64 = nullptr) {
+    // C64 set: only the matrix-core path writes it; *path_used is 0 and nothing is written when that path does not apply
     hipStream_t st = (hipStream_t)stv;
     std::unique_ptr<Scratch> a_written;
     auto write_out = [&]() -> int {          // the product as field elements, once
@@ -717,6 +723,7 @@ static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch
         }
         if (mode == 2 && !small) { set_error(ZK_ERR_ARG, "zk_fr_matmul: operands do not satisfy the small-integer bound"); return ZK_ERR_ARG; }
     }
+    if (C64 && !small) { if (path_used) *path_used = 0; return 0; }
     if (mode == 1 || !small) { int wrc = write_out(); if (wrc) return wrc; }
     if (!small) {
         if (path_used) *path_used = 1;
@@ -731,10 +738,11 @@ static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch
     const int planes_log2 = planes_env ? atoi(planes_env) : 30;
     if (planes_log2 > 0 && (unsigned __int128)batch * M * N * P >= ((unsigned __int128)1 << planes_log2) && M >= 32 && P >= 32) {
         bool done = false;
-        const int rc = run_int8_plane_path(C, A, B, batch, M, N, P, ma_, mb_, st, &done, rhs, src);
+        const int rc = run_int8_plane_path(C, A, B, batch, M, N, P, ma_, mb_, st, &done, rhs, src, C64);
         if (rc) return rc;
         if (done) return 0;
     }
+    if (C64) { if (path_used) *path_used = 0; return 0; }
     { int wrc = write_out(); if (wrc) return wrc; }
     if (fits32) return run_int_path<int>(C, A, B, batch, M, N, P, st);
     if (b_fits32) return run_wide_narrow_path(C, A, B, batch, M, N, P, st);
@@ -822,6 +830,15 @@ int zk_fr_matmul(void* C, const void* A, const void* B, uint32_t M, uint32_t N, 
 }
 int zk_fr_matmul_batched(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv) {
     return matmul_dispatch(C, A, B, batch, M, N, P, mode, path_used, stv);
+}
+// zk_fr_matmul_batched with the products written as 64-bit integers (C64: batch * M * P int64 on the device).  Only the
+// matrix-core path does that: *taken_host is 1 when it ran, 0 when the operands or the shape do not allow it -- nothing is written then.
+int zk_fr_matmul_batched_i64(void* C64, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int* taken_host, void* stv) {
+    ZK_ARG(C64 != nullptr && taken_host != nullptr, "zk_fr_matmul_batched_i64: null argument");
+    int path = 0;
+    const int rc = matmul_dispatch(nullptr, A, B, batch, M, N, P, 0, &path, stv, nullptr, ProdSrc{nullptr, nullptr}, (long long*)C64);
+    *taken_host = (rc == 0 && path == 2) ? 1 : 0;
+    return rc;
 }
 int zk_fr_matmul_batched_prod(void* C, const void* a_ints, const void* b_ints, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv) {
     ZK_ARG(a_ints != nullptr && b_ints != nullptr, "zk_fr_matmul_batched_prod: null int32 form");

@@ -493,6 +493,7 @@ void* zkp_attn(void* Q, void* K, void* V, u32 num, u32 m, u32 n, u32 d, int stac
     ZKP_END_PTR
 }
 int zkp_softmax_lean_tensors_last() { return (int)zkSoftmax::lean_tensors_last; }
+int zkp_softmax_scores_i64_last() { return zkSoftmax::scores_i64_last ? 1 : 0; }
 // zkFCStacked over num layers: X [num][batch][in], W [num][in][out], b [num][out] or null; forward per layer, then prove
 void* zkp_zkfc_stacked(void* X, void* W, void* b, u32 num, u32 batch, u32 in, u32 out) {
     ZKP_TRY

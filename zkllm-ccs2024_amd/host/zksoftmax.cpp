@@ -45,6 +45,7 @@ static void mul_segments(Fr_t* out, const FrTensor& a, const FrTensor& b, size_t
     if (a.kept_ints() && b.kept_ints()) ZKC(zk_fr_mul_ints(out, a.kept_ints(), b.kept_ints(), N, nullptr));
     else ZKC(zk_fr_mul(out, a.gpu_data, b.gpu_data, N, nullptr));
 }
+bool zkSoftmax::scores_i64_last = false;
 uint zkSoftmax::lean_tensors_last = 0;
 // zksoftmax.cu:112-173
 FrTensor zkSoftmax::compute(const FrTensor& X, FrTensor& shift, FrTensor& X_shifted, vector<FrTensor>& X_segments, vector<FrTensor>& Y_segments, vector<FrTensor>& m_segments) {
@@ -80,8 +81,10 @@ FrTensor zkSoftmax::compute_rows(uint m, const FrTensor& X, FrTensor& shift, FrT
         if (bs[i] <= 0x80000000u) int_planes[i] = X_segments[i].ints_for_producer();
     }
     // shift and digits in one pass: the shifted scores are decomposed where they are written
-    ZKC(zk_softmax_shift_decompose(shift.gpu_data, X_shifted.size ? X_shifted.gpu_data : nullptr, planes.data(), int_planes.data(), X.gpu_data, m, n, scale, bs.data(), (int)K,
-                                   nullptr));
+    if (X_i64) ZKC(zk_softmax_shift_decompose_i64(shift.gpu_data, X_shifted.size ? X_shifted.gpu_data : nullptr, planes.data(), int_planes.data(), X_i64, m, n, scale, bs.data(),
+                                                  (int)K, nullptr));
+    else ZKC(zk_softmax_shift_decompose(shift.gpu_data, X_shifted.size ? X_shifted.gpu_data : nullptr, planes.data(), int_planes.data(), X.gpu_data, m, n, scale, bs.data(), (int)K,
+                                        nullptr));
 
     bool lean_out = lean_forward && K - L == 2 && zk_hadamard_ints_suffice(2, N);
     for (uint i = L; i < K; ++i) lean_out = lean_out && ints_only[i];
@@ -156,7 +159,8 @@ Fr_t zkSoftmax::prove_end(Pending& pending, const FrTensor& X, const FrTensor& s
     for (uint i = L; i < K; ++i) at_v.push_back(&Y_segments[i - L]);
     for (uint i = 0; i < K; ++i) at_v.push_back(&X_segments[i]);
     const char* check_env = getenv("ZKLLM_CHECK_CLAIMS");
-    const bool read_X = !X_at_v_Y || (check_env && check_env[0] == '1');
+    if (X_unwritten && !X_at_v_Y) throw std::runtime_error("zkSoftmax::prove_end: X was left unwritten and its value at v_Y is not given");
+    const bool read_X = !X_at_v_Y || (check_env && check_env[0] == '1' && !X_unwritten);
     if (read_X) at_v.push_back(&X);
     vector<Fr_t> evals;
     Fr_t shift_const_opening;
@@ -257,11 +261,32 @@ FrTensor zkAttnStacked::compute(const FrTensor& Q, const FrTensor& K, const FrTe
     if ((size_t)sm_in.size != (size_t)num * m * n || sm_out.size != sm_in.size || (sm_in_shifted.size != sm_in.size && !(lean_forward && sm_in_shifted.size == 0)) ||
         sm_shift.size != num * m)
         throw std::invalid_argument("softmax tensors must be num * m * n (shift: num * m)");
-    FrTensor::matmul_stack_into(sm_in, Q, K.transpose_stack(num, n, d), num, m, d, n);
+    // The scores have one reader when the proof takes their value at the softmax's point from Q and K (prove_finish): the pass
+    // that shifts and decomposes them.  With lean_forward they are then written as 64-bit integers, 8 bytes an element, where
+    // the matrix-core product applies, and sm_in stays unwritten (not with ZKLLM_CHECK_CLAIMS=1, which evaluates sm_in, nor
+    // with ZKLLM_SCORES_I64=0).
+    std::unique_ptr<FrTensor> scores_i64;          // num * m * n int64 in a tensor's memory
+    {
+        const char* e = getenv("ZKLLM_SCORES_I64");
+        const char* chk = getenv("ZKLLM_CHECK_CLAIMS");
+        const size_t count = (size_t)num * m * n;
+        if (lean_forward && !(e && e[0] == '0') && !(chk && chk[0] == '1') && count % 4 == 0) {
+            scores_i64.reset(new FrTensor((uint)(count / 4)));
+            int taken = 0;
+            FrTensor Kt = K.transpose_stack(num, n, d);
+            ZKC(zk_fr_matmul_batched_i64(scores_i64->gpu_data, Q.gpu_data, Kt.gpu_data, num, m, d, n, &taken, nullptr));
+            if (!taken) scores_i64.reset();
+        }
+    }
+    if (!scores_i64) FrTensor::matmul_stack_into(sm_in, Q, K.transpose_stack(num, n, d), num, m, d, n);
+    X_i64 = scores_i64 ? scores_i64->gpu_data : nullptr;
+    X_unwritten = scores_i64 != nullptr;
+    scores_i64_last = X_unwritten;
     // this class reads sm_out in two places, both of which take the product's factors instead (ZKLLM_SOFTMAX_PRODUCT=0 writes it as before)
     { const char* e = getenv("ZKLLM_SOFTMAX_PRODUCT"); product_out_allowed = !(e && e[0] == '0'); }
     compute_rows(num * m, sm_in, sm_shift, sm_in_shifted, sm_in_segments, sm_out_segments, sm_m_segments, &sm_out);
     product_out_allowed = false;
+    X_i64 = nullptr;
     if (out_is_product) return FrTensor::matmul_stack_prod(sm_out_segments[0], sm_out_segments[1], V, num, m, n, d);
     return FrTensor::matmul_stack(sm_out, V, num, m, n, d);
 }

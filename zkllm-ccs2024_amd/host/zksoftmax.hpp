@@ -16,11 +16,15 @@ class zkSoftmax {
     // none of them itself.
     bool lean_forward = false;
     std::shared_ptr<FrTensor> unwritten;      // the buffer those tensors are views of: it must outlive every use of them (it lives as long as this object)
+    static bool scores_i64_last;        // whether the last zkAttnStacked::compute wrote its scores as 64-bit integers only
     static uint lean_tensors_last;      // how many digit planes and mapped-value tensors the last compute() left in int32 form only
     // set by the last compute_rows(..., into) when the output is the product of two mapped-value tensors that exist in int32 form
     // only: `into` was then NOT written either -- zkAttnStacked multiplies and folds the product from the two int32 forms
     bool out_is_product = false;
     bool product_out_allowed = false;      // set by a caller of compute_rows that never reads `into` as field elements
+    // set by a caller of compute_rows whose X exists as 64-bit integers only (rows * n int64 on the device): X is then not read
+    const void* X_i64 = nullptr;
+    bool X_unwritten = false;      // the last compute left X (the scores) unwritten: prove_end must be given their value at v_Y
     zkSoftmax(const vector<uint>& bs, uint L, uint M, unsigned long scaling_factor_in, const vector<double>& thetas, uint m, uint n, uint d, uint E);
 
     FrTensor compute(const FrTensor& X, FrTensor& shift, FrTensor& X_shifted, vector<FrTensor>& X_segments, vector<FrTensor>& Y_segments, vector<FrTensor>& m_segments);
