@@ -304,6 +304,9 @@ int zk_lookup_index_fr(void* idx_u32, const void* vals_fr, int32_t low, uint32_t
 int zk_lookup_index_i32(void* idx_u32, const void* vals_i32, int32_t low, uint32_t table_size, size_t n, void* stream);
 /* multiplicities (tlookup_kernel :10-15): counts[b] = #{i : idx[i] == b}; counts is cleared first */
 int zk_lookup_hist(void* counts_u32, const void* idx_u32, size_t n, uint32_t nbins, void* stream);
+/* zk_lookup_index_i32 and zk_lookup_hist in one (tLookupRange::prep over queries that keep an int32 form): the counting passes
+ * form the positions value - low themselves and no array of positions is written; a value outside [low, low + len) is an error */
+int zk_lookup_hist_i32(void* counts_u32, const void* vals_i32, int32_t low, uint32_t len, size_t n, uint32_t nbins, void* stream);
 int zk_range_table(void* table_fr, int32_t low, uint32_t len, uint32_t table_size, void* stream);   /* tlookuprange_init_kernel :372-380 */
 /* out[i] = 1/(in[i]+beta) (tlookup_inv_kernel :50-62), by batch inversion */
 int zk_fr_batch_inv(void* out, const void* in, const uint32_t* beta, size_t n, void* stream);

@@ -56,7 +56,13 @@ def test_multiplicities(pv, D, low, length):
     rng = np.random.default_rng(D)
     vals = rng.integers(low, low + length, D)
     vals[: D // 3] = low + length // 2               # a long run of equal values (wave aggregation path)
+    # queries that keep an int32 form are counted from it, positions formed by the counting passes (zk_lookup_hist_i32)
+    hk = pv.from_i64(vals)
+    pv.keep_for_folds(hk)
+    assert pv.folds_from_ints(hk) == 1
+    mk = pv.range_prep(hk, low, length).host()
     m = pv.range_prep(pv.from_i64(vals), low, length).host()
+    assert (mk == m).all()
     size = 1 << max(0, (length - 1).bit_length())
     assert fr_ints(m) == [int(c) for c in np.bincount(vals - low, minlength=size)]
 
@@ -74,11 +80,20 @@ def test_multiplicities_of_many_queries_into_a_large_table(pv, D, low, length, s
     m = pv.range_prep(pv.from_i64(vals), low, length).host()
     want = np.bincount(vals - low, minlength=m.shape[0]).astype(np.uint32)
     assert (m[:, 0] == want).all() and not m[:, 1:].any()
+    hk = pv.from_i64(vals)          # the same from the queries' int32 form
+    pv.keep_for_folds(hk)
+    mk = pv.range_prep(hk, low, length).host()
+    assert (mk[:, 0] == want).all() and not mk[:, 1:].any()
 
 
 def test_lookup_out_of_range_is_an_error(pv):
     with pytest.raises(RuntimeError, match="outside the table"):
         pv.range_prep(pv.from_i64(np.array([0, 1, 99])), 0, 8)
+    for bad in (8, -1, 6):          # from the int32 form too; 6: inside the padded table of 8, outside the range of 6
+        h = pv.from_i64(np.array([0, 1, bad] + [2] * 5000))
+        pv.keep_for_folds(h)
+        with pytest.raises(RuntimeError, match="outside the table"):
+            pv.range_prep(h, 0, 6)
 
 
 def test_range_lookup_rejects_values_in_the_padding_gap(pv):

@@ -135,12 +135,22 @@ __global__ void __launch_bounds__(TPB) k_index_i32(uint32_t* __restrict__ idx, u
     idx[i] = ok ? (uint32_t)d : 0u;
     if (!ok) atomicOr(flag, 1u);
 }
+// Where a counting pass takes its table positions from: an array of them, or the queries themselves in int32 form (position =
+// value - low; a value outside [low, low + len) counts as position 0 and raises *flag in the passes that are asked to check).
+struct KeySrc { const uint32_t* idx; const int32_t* vals; int32_t low; uint32_t len; uint32_t* flag; };
+template <bool CHECK> __device__ __forceinline__ uint32_t key_at(const KeySrc& k, size_t i) {
+    if (k.idx) return k.idx[i];
+    const int64_t d = (int64_t)k.vals[i] - (int64_t)k.low;
+    const bool ok = d >= 0 && d < (int64_t)k.len;
+    if (CHECK && !ok) atomicOr(k.flag, 1u);
+    return ok ? (uint32_t)d : 0u;
+}
 static constexpr uint32_t HIST_LDS_BINS = 16384;
-__global__ void __launch_bounds__(TPB) k_hist_lds(uint32_t* __restrict__ counts, const uint32_t* __restrict__ idx, size_t n, uint32_t nbins) {
+__global__ void __launch_bounds__(TPB) k_hist_lds(uint32_t* __restrict__ counts, const KeySrc idx, size_t n, uint32_t nbins) {
     __shared__ uint32_t h[HIST_LDS_BINS];
     for (uint32_t b = threadIdx.x; b < nbins; b += TPB) h[b] = 0;
     __syncthreads();
-    for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (size_t)gridDim.x * TPB) atomicAdd(&h[idx[i]], 1u);
+    for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (size_t)gridDim.x * TPB) atomicAdd(&h[key_at<true>(idx, i)], 1u);
     __syncthreads();
     for (uint32_t b = threadIdx.x; b < nbins; b += TPB) {
         const uint32_t c = h[b];
@@ -153,7 +163,7 @@ __global__ void __launch_bounds__(TPB) k_hist_lds(uint32_t* __restrict__ counts,
 // bins) then cost a few dozen global atomics per workgroup instead of thousands on the same addresses; spread-out
 // inputs fill the table and pay one global atomic per index, as they must.
 static constexpr uint32_t HH_SLOTS = 1024, HH_PER_LANE = 16, HH_EMPTY = 0xFFFFFFFFu;
-__global__ void __launch_bounds__(TPB) k_hist_global(uint32_t* __restrict__ counts, const uint32_t* __restrict__ idx, size_t n) {
+__global__ void __launch_bounds__(TPB) k_hist_global(uint32_t* __restrict__ counts, const KeySrc idx, size_t n) {
     __shared__ uint32_t keys[HH_SLOTS], cnts[HH_SLOTS];
     for (uint32_t s = threadIdx.x; s < HH_SLOTS; s += TPB) { keys[s] = HH_EMPTY; cnts[s] = 0; }
     __syncthreads();
@@ -162,7 +172,7 @@ __global__ void __launch_bounds__(TPB) k_hist_global(uint32_t* __restrict__ coun
     for (uint32_t k = 0; k < HH_PER_LANE; ++k) {
         const size_t i = base + (size_t)k * TPB + threadIdx.x;
         if (i >= n) break;
-        const uint32_t key = idx[i];
+        const uint32_t key = key_at<true>(idx, i);
         const uint32_t h = (key * 2654435761u) >> 22;          // 10 bits
         bool placed = false;
 #pragma unroll
@@ -189,12 +199,12 @@ static constexpr uint32_t HP_TILE = 65536;                           // queries 
 static constexpr uint32_t HP_SLICE = 32768;                          // queries per workgroup of the counting pass
 static constexpr uint32_t HP_MAXP = 1024;                            // partitions: tables up to 2^22 bins
 static constexpr size_t HP_MIN_QUERIES = (size_t)1 << 20;
-__global__ void __launch_bounds__(TPB) k_hp_sizes(uint32_t* __restrict__ sizes, const uint32_t* __restrict__ idx, size_t n, uint32_t P, uint32_t ntiles) {
+__global__ void __launch_bounds__(TPB) k_hp_sizes(uint32_t* __restrict__ sizes, const KeySrc idx, size_t n, uint32_t P, uint32_t ntiles) {
     __shared__ uint32_t c[HP_MAXP];
     for (uint32_t q = threadIdx.x; q < P; q += TPB) c[q] = 0;
     __syncthreads();
     const size_t base = (size_t)blockIdx.x * HP_TILE, end = base + HP_TILE < n ? base + HP_TILE : n;
-    for (size_t i = base + threadIdx.x; i < end; i += TPB) atomicAdd(&c[idx[i] >> HP_BITS], 1u);
+    for (size_t i = base + threadIdx.x; i < end; i += TPB) atomicAdd(&c[key_at<true>(idx, i) >> HP_BITS], 1u);
     __syncthreads();
     for (uint32_t q = threadIdx.x; q < P; q += TPB) sizes[(size_t)q * ntiles + blockIdx.x] = c[q];
 }
@@ -252,13 +262,13 @@ __global__ void __launch_bounds__(1024) k_hp_slices(uint32_t* __restrict__ slice
     if (t == 1023u) *nslices = part[1023];
 }
 __global__ void __launch_bounds__(TPB) k_hp_scatter(uint16_t* __restrict__ parted, const uint32_t* __restrict__ offs, const uint32_t* __restrict__ part_off,
-                                                    const uint32_t* __restrict__ idx, size_t n, uint32_t P, uint32_t ntiles) {
+                                                    const KeySrc idx, size_t n, uint32_t P, uint32_t ntiles) {
     __shared__ uint32_t cur[HP_MAXP];
     for (uint32_t q = threadIdx.x; q < P; q += TPB) cur[q] = part_off[q] + offs[(size_t)q * ntiles + blockIdx.x];
     __syncthreads();
     const size_t base = (size_t)blockIdx.x * HP_TILE, end = base + HP_TILE < n ? base + HP_TILE : n;
     for (size_t i = base + threadIdx.x; i < end; i += TPB) {
-        const uint32_t key = idx[i];
+        const uint32_t key = key_at<false>(idx, i);
         const uint32_t pos = atomicAdd(&cur[key >> HP_BITS], 1u);
         parted[pos] = (uint16_t)(key & (HP_BINS - 1u));
     }
@@ -279,7 +289,7 @@ __global__ void __launch_bounds__(TPB) k_hp_count(uint32_t* __restrict__ counts,
         if (c && bin < nbins) atomicAdd(&counts[bin], c);
     }
 }
-static int hist_partitioned(uint32_t* counts, const uint32_t* idx, size_t n, uint32_t nbins, hipStream_t st) {
+static int hist_partitioned(uint32_t* counts, const KeySrc idx, size_t n, uint32_t nbins, hipStream_t st) {
     const uint32_t P = (nbins + HP_BINS - 1) / HP_BINS, ntiles = cdiv(n, HP_TILE), M = P * ntiles;
     const uint32_t max_slices = (uint32_t)(n / HP_SLICE) + P + 1;
     Scratch sizes(sizeof(uint32_t) * (size_t)M, st), part_off(sizeof(uint32_t) * (P + 1), st), totals(sizeof(uint32_t) * P, st), slice_tab(sizeof(uint32_t) * max_slices, st),
@@ -1981,21 +1991,40 @@ int zk_lookup_index_i32(void* idx_u32, const void* vals_i32, int32_t low, uint32
     return 0;
 }
 // counts[0..nbins) = number of occurrences of each index (zeroed here first)
-int zk_lookup_hist(void* counts_u32, const void* idx_u32, size_t n, uint32_t nbins, void* stv) {
-    hipStream_t st = (hipStream_t)stv;
-    ZK_ARG(nbins >= 1, "zk_lookup_hist: no bins");
-    ZK_HIP(hipMemsetAsync(counts_u32, 0, sizeof(uint32_t) * (size_t)nbins, st));
+static int hist_queue(uint32_t* counts, const KeySrc src, size_t n, uint32_t nbins, hipStream_t st) {
+    ZK_HIP(hipMemsetAsync(counts, 0, sizeof(uint32_t) * (size_t)nbins, st));
     if (n == 0) return 0;
     if (nbins <= HIST_LDS_BINS) {
         unsigned blocks = cdiv(n, (size_t)TPB * 16);
         if (blocks > 2048) blocks = 2048;
-        hipLaunchKernelGGL(k_hist_lds, dim3(blocks), dim3(TPB), 0, st, (uint32_t*)counts_u32, (const uint32_t*)idx_u32, n, nbins);
+        hipLaunchKernelGGL(k_hist_lds, dim3(blocks), dim3(TPB), 0, st, counts, src, n, nbins);
     } else if (n >= HP_MIN_QUERIES && n < ((size_t)1 << 32) && nbins <= HP_MAXP * HP_BINS) {
-        return hist_partitioned((uint32_t*)counts_u32, (const uint32_t*)idx_u32, n, nbins, st);
+        return hist_partitioned(counts, src, n, nbins, st);
     } else {
-        hipLaunchKernelGGL(k_hist_global, dim3(cdiv(n, (size_t)TPB * HH_PER_LANE)), dim3(TPB), 0, st, (uint32_t*)counts_u32, (const uint32_t*)idx_u32, n);
+        hipLaunchKernelGGL(k_hist_global, dim3(cdiv(n, (size_t)TPB * HH_PER_LANE)), dim3(TPB), 0, st, counts, src, n);
     }
     ZK_LAUNCH_CHECK();
+    return 0;
+}
+int zk_lookup_hist(void* counts_u32, const void* idx_u32, size_t n, uint32_t nbins, void* stv) {
+    ZK_ARG(nbins >= 1, "zk_lookup_hist: no bins");
+    return hist_queue((uint32_t*)counts_u32, KeySrc{(const uint32_t*)idx_u32, nullptr, 0, 0, nullptr}, n, nbins, (hipStream_t)stv);
+}
+// zk_lookup_index_i32 and zk_lookup_hist in one: the counting passes form the positions value - low themselves, no array of
+// them is written.  A value outside [low, low + len) is an error, as there.
+int zk_lookup_hist_i32(void* counts_u32, const void* vals_i32, int32_t low, uint32_t len, size_t n, uint32_t nbins, void* stv) {
+    hipStream_t st = (hipStream_t)stv;
+    ZK_ARG(nbins >= 1 && len >= 1 && len <= nbins, "zk_lookup_hist_i32: need 1 <= len <= nbins");
+    ZK_ARG(vals_i32 != nullptr || n == 0, "zk_lookup_hist_i32: null queries");
+    Scratch flag(4, st);
+    if (flag.rc) return flag.rc;
+    ZK_HIP(hipMemsetAsync(flag.p, 0, 4, st));
+    int rc = hist_queue((uint32_t*)counts_u32, KeySrc{nullptr, (const int32_t*)vals_i32, low, len, flag.as<uint32_t>()}, n, nbins, st);
+    if (rc) return rc;
+    uint32_t f = 0;
+    rc = read_flag(flag.as<uint32_t>(), &f, st);
+    if (rc) return rc;
+    ZK_ARG(f == 0, "lookup: a value lies outside the table range");
     return 0;
 }
 int zk_range_table(void* table, int32_t low, uint32_t len, uint32_t table_size, void* st) {

@@ -21,6 +21,16 @@ static FrTensor counts_to_m(const void* idx, uint D, uint N) {
     return m;
 }
 
+// the same from queries in int32 form: positions value - low formed by the counting passes themselves
+static FrTensor counts_to_m_i32(const void* vals_i32, int low, uint len, uint D, uint N) {
+    DevBuf counts(sizeof(uint) * (size_t)N);
+    ZKC(zk_lookup_hist_i32(counts.p, vals_i32, low, len, D, N, nullptr));
+    FrTensor m(N);
+    ZKC(zk_fr_from_u32(m.gpu_data, counts.p, N, nullptr));
+    ZKC(zk_sync(nullptr));
+    return m;
+}
+
 FrTensor tLookup::prep(const uint* indices, const uint D) { return counts_to_m(indices, D, table.size); }
 
 static FrTensor make_range_table(int low, uint len) {
@@ -30,17 +40,14 @@ static FrTensor make_range_table(int low, uint len) {
 }
 tLookupRange::tLookupRange(int low, uint len) : tLookup(make_range_table(low, len)), low(low), len(len) {}
 
-FrTensor tLookupRange::prep(const int* vals, const uint D) {
-    DevBuf idx(sizeof(uint) * (size_t)D);
-    ZKC(zk_lookup_index_i32(idx.p, vals, low, len, D, nullptr));
-    return counts_to_m(idx.p, D, table.size);
-}
+FrTensor tLookupRange::prep(const int* vals, const uint D) { return counts_to_m_i32(vals, low, len, D, table.size); }
 // table positions of the values: from their int32 form when the tensor keeps one
 static void index_of(void* idx, const FrTensor& vals, int low, uint len) {
     if (const void* h = vals.kept_ints()) ZKC(zk_lookup_index_i32(idx, zk_fr_fold_prepared_ints(h), low, len, vals.size, nullptr));
     else ZKC(zk_lookup_index_fr(idx, vals.gpu_data, low, len, vals.size, nullptr));
 }
 FrTensor tLookupRange::prep(const FrTensor& vals) {
+    if (const void* h = vals.kept_ints()) return counts_to_m_i32(zk_fr_fold_prepared_ints(h), low, len, vals.size, table.size);
     DevBuf idx(sizeof(uint) * (size_t)vals.size);
     index_of(idx.p, vals, low, len);
     return counts_to_m(idx.p, vals.size, table.size);
@@ -68,9 +75,11 @@ pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const int* vals, const 
 }
 pair<FrTensor, FrTensor> tLookupRangeMapping::operator()(const FrTensor& vals) { return map(vals, nullptr); }
 pair<FrTensor, FrTensor> tLookupRangeMapping::map(const FrTensor& vals, const FrTensor* unwritten) {
-    DevBuf idx(sizeof(uint) * (size_t)vals.size);
-    index_of(idx.p, vals, low, len);
-    FrTensor m = counts_to_m(idx.p, vals.size, table.size);
+    // queries and mapped values in int32 form: nothing below needs the array of table positions
+    const bool by_queries = mapped_vals.kept_ints() && vals.kept_ints();
+    DevBuf idx(by_queries ? 4 : sizeof(uint) * (size_t)vals.size);
+    if (!by_queries) index_of(idx.p, vals, low, len);
+    FrTensor m = by_queries ? counts_to_m_i32(zk_fr_fold_prepared_ints(vals.kept_ints()), low, len, vals.size, table.size) : counts_to_m(idx.p, vals.size, table.size);
     const bool ints_only_out = unwritten && unwritten->size == vals.size && mapped_vals.kept_ints() && vals.kept_ints();
     FrTensor y = ints_only_out ? FrTensor::view(*unwritten) : FrTensor(vals.size);
     // mapped values that are 32-bit integers: the outputs get their int32 form with them
