@@ -1013,9 +1013,12 @@ __global__ void __launch_bounds__(TPB) k_hp_round(Fr* __restrict__ partials, Fr*
         const Fr a1 = (2 * g + 1 < in_size) ? A[2 * g + 1] : big_zero<8>(), b1 = (2 * g + 1 < in_size) ? B[2 * g + 1] : big_zero<8>();
         const Fr da = sub(a1, a0), db = sub(b1, b0);
         const Fr e = E[g];
-        acc[0] = add(acc[0], mont_mul(e, mont_mul(a0, b0)));
-        acc[1] = add(acc[1], mont_mul(e, add(mont_mul(a0, db), mont_mul(b0, da))));
-        acc[2] = add(acc[2], mont_mul(e, mont_mul(da, db)));
+        // the eq weight on one factor first: five products instead of seven (a0 db + b0 da = (a0 + da)(b0 + db) - a0 b0 - da db)
+        const Fr ea0 = mont_mul(e, a0), eda = mont_mul(e, da);
+        const Fr c0 = mont_mul(ea0, b0), c2 = mont_mul(eda, db);
+        acc[0] = add(acc[0], c0);
+        acc[1] = add(acc[1], sub(sub(mont_mul(add(ea0, eda), add(b0, db)), c0), c2));
+        acc[2] = add(acc[2], c2);
         nA[g] = add(a0, mont_mul(v_mont, da));
         nB[g] = add(b0, mont_mul(v_mont, db));
         if (g < ne_count) nE[g] = add(E[2 * g], E[2 * g + 1]);
