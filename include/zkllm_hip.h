@@ -108,6 +108,9 @@ int zk_fr_pad(void* out, const void* in, size_t rows, uint32_t last_in, uint32_t
 int zk_fr_transpose(void* out, const void* in, uint32_t M, uint32_t N, void* stream);
 /* the same for a stack of `batch` M x N matrices stored one after the other (per-head K^T of zkAttn::compute, zksoftmax.cu:234) */
 int zk_fr_transpose_batched(void* out, const void* in, uint32_t batch, uint32_t M, uint32_t N, void* stream);
+/* out[b][a][c] = in[a][b][c] (A x B x C elements): what self-attn.cu:80-90 reaches per head through transposes and slices, for
+ * all heads at once -- [token][head][k] to [head][token][k] and back -- in one pass instead of two transposes */
+int zk_fr_swap_axes(void* out, const void* in, uint32_t A, uint32_t B, uint32_t C, void* stream);
 int zk_fr_gather(void* out, const void* table, const void* idx_u32, size_t n, void* stream);
 /* dst[i] = src[offset + i * stride], i < count, for elements of elem_bytes (a multiple of 16: field elements, G1 points):
  * every 2^k-th column of a row-major tensor or generator vector (no counterpart in the reference; the cross commitments

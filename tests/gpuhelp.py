@@ -154,7 +154,7 @@ class Prover:
         L = self.lib
         for name in ("zkp_fr_from_i32", "zkp_fr_from_i64", "zkp_fr_from_fr", "zkp_fr_from_f32", "zkp_fr_from_f64", "zkp_fr_from_file",
                      "zkp_fr_devptr", "zkp_fr_binop", "zkp_fr_scalarop", "zkp_fr_partial_me", "zkp_fr_partial_me_window",
-                     "zkp_fr_pad", "zkp_fr_split", "zkp_fr_transpose", "zkp_fr_matmul", "zkp_fr_matmul_stack", "zkp_fr_transpose_stack", "zkp_fr_matmul_stack_prod", "zkp_fr_partial_me_prod",
+                     "zkp_fr_pad", "zkp_fr_split", "zkp_fr_transpose", "zkp_fr_matmul", "zkp_fr_matmul_stack", "zkp_fr_transpose_stack", "zkp_fr_matmul_stack_prod", "zkp_fr_partial_me_prod", "zkp_fr_swap_axes",
                      "zkp_g1_from_host", "zkp_g1_from_file", "zkp_g1_devptr", "zkp_commitment_random", "zkp_g1_binop", "zkp_g1_pointop", "zkp_g1_affineop",
                      "zkp_g1_scalar_mul", "zkp_g1_rowwise_sum", "zkp_commit_int", "zkp_commit",
                      "zkp_rescale", "zkp_rescale_prove", "zkp_relu", "zkp_attn", "zkp_zkfc_stacked", "zkp_range_prep", "zkp_batch_inv", "zkp_softmax",
@@ -264,6 +264,9 @@ class Prover:
 
     def matmul_stack(self, a, b, num, M, N, P):
         return self.H(self.lib.zkp_fr_matmul_stack(c_void_p(a.h), c_void_p(b.h), c_uint(num), c_uint(M), c_uint(N), c_uint(P)))
+
+    def swap_axes(self, a, A, B, C):
+        return self.H(self.lib.zkp_fr_swap_axes(c_void_p(a.h), c_uint(A), c_uint(B), c_uint(C)))
 
     def matmul_stack_prod(self, a, b, y, num, M, N, P):
         return self.H(self.lib.zkp_fr_matmul_stack_prod(c_void_p(a.h), c_void_p(b.h), c_void_p(y.h), c_uint(num), c_uint(M), c_uint(N), c_uint(P)))

@@ -581,6 +581,13 @@ def test_stacks_of_matrices_transpose_and_multiply_like_their_members(pv):
     T = rng.integers(-2 ** 40, 2 ** 40, (5, 37, 70)).astype(np.int64)
     got = pv.transpose_stack(pv.from_i64(T), 5, 37, 70).host()
     assert fr_ints(got) == [int(v) % R_MOD for v in T.transpose(0, 2, 1).reshape(-1)]
+    # the leading two axes swapped in one pass (zk_fr_swap_axes: tokens x heads x k to heads x tokens x k and back)
+    for A, B, C in ((5, 37, 70), (16, 2, 16), (1, 9, 3), (33, 1, 7)):
+        T3 = rng.integers(-2 ** 40, 2 ** 40, (A, B, C)).astype(np.int64)
+        hT3 = pv.from_i64(T3)
+        got = pv.swap_axes(hT3, A, B, C)
+        assert fr_ints(got.host()) == [int(v) % R_MOD for v in T3.transpose(1, 0, 2).reshape(-1)], (A, B, C)
+        assert (pv.swap_axes(got, B, A, C).host() == hT3.host()).all()
 
 
 @pytest.mark.parametrize("num,M,N,P,abits,bbits,ybits", [(3, 70, 130, 50, 16, 16, 17), (2, 33, 65, 128, 31, 31, 17), (1, 128, 256, 64, 8, 9, 12), (2, 20, 40, 9, 31, 31, 40),

@@ -595,6 +595,12 @@ FrTensor FrTensor::transpose_stack(uint num, uint M, uint N) const {
     ZKC(zk_fr_transpose_batched(out.gpu_data, gpu_data, num, M, N, nullptr));
     return out;
 }
+FrTensor FrTensor::swap_leading_axes(uint A, uint B, uint C) const {
+    if ((size_t)size != (size_t)A * B * C) throw std::runtime_error("swap_leading_axes: incompatible dimensions");
+    FrTensor out(size);
+    ZKC(zk_fr_swap_axes(out.gpu_data, gpu_data, A, B, C, nullptr));
+    return out;
+}
 FrTensor FrTensor::matmul_stack(const FrTensor& x, const FrTensor& y, uint num, uint M, uint N, uint P) {
     FrTensor out(num * M * P);
     matmul_stack_into(out, x, y, num, M, N, P);

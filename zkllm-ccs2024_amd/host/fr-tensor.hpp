@@ -197,6 +197,7 @@ class FrTensor {
     // additions for stacks of `num` equally shaped matrices stored one after the other: every M x N matrix transposed,
     // and the num products x_i (M x N) * y_i (N x P)
     FrTensor transpose_stack(uint num, uint M, uint N) const;
+    FrTensor swap_leading_axes(uint A, uint B, uint C) const;      // addition: [A][B][C] -> [B][A][C]
     static FrTensor matmul_stack(const FrTensor& x, const FrTensor& y, uint num, uint M, uint N, uint P);
     static void matmul_stack_into(FrTensor& out, const FrTensor& x, const FrTensor& y, uint num, uint M, uint N, uint P);
     // the same two for a left operand / a tensor that is the elementwise product of a and b, both of which keep an int32 form

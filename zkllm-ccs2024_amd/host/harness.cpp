@@ -218,6 +218,7 @@ void* zkp_fr_pad(void* a, const u32* shape, int ndim, const u32* pad_val) {
     ZKP_TRY Fr_t pv; memcpy(pv.val, pad_val, 32); return new FrTensor(FT(a).pad(std::vector<uint>(shape, shape + ndim), pv)); ZKP_END_PTR
 }
 void* zkp_fr_transpose(void* a, u32 M, u32 N) { ZKP_TRY return new FrTensor(FT(a).transpose(M, N)); ZKP_END_PTR }
+void* zkp_fr_swap_axes(void* a, u32 A, u32 B, u32 C) { ZKP_TRY return new FrTensor(FT(a).swap_leading_axes(A, B, C)); ZKP_END_PTR }
 void* zkp_fr_matmul_stack_prod(void* a, void* b, void* y, u32 num, u32 M, u32 N, u32 P) { ZKP_TRY return new FrTensor(FrTensor::matmul_stack_prod(FT(a), FT(b), FT(y), num, M, N, P)); ZKP_END_PTR }
 void* zkp_fr_partial_me_prod(void* a, void* b, const u32* u, int k, u32 cur_dim, u32 window) { ZKP_TRY return new FrTensor(FrTensor::partial_me_prod(FT(a), FT(b), frs(u, k), cur_dim, window)); ZKP_END_PTR }
 void* zkp_fr_matmul_stack(void* a, void* b, u32 num, u32 M, u32 N, u32 P) { ZKP_TRY return new FrTensor(FrTensor::matmul_stack(FT(a), FT(b), num, M, N, P)); ZKP_END_PTR }

@@ -197,7 +197,7 @@ static FrTensor attn_stacked_heads(const LayerConfig& c, const FrTensor& Q_, con
     const uint seq = c.seq_len, E = c.embed_dim, H = c.num_heads, d = E / H, g = c.attn_head_group;
     if (H % g) throw std::runtime_error("attn_head_group must divide num_heads");
     // seq x embed -> embed x seq = [head][d][seq] -> [head][seq][d]
-    auto to_stack = [&](const FrTensor& t) { return t.transpose(seq, E).transpose_stack(H, d, seq); };
+    auto to_stack = [&](const FrTensor& t) { return t.swap_leading_axes(seq, H, d); };          // = t.transpose(seq, E).transpose_stack(H, d, seq)
     FrTensor Qs = to_stack(Q_), Ks = to_stack(K_), Vs = to_stack(V_);
     FrTensor outs(H * seq * d);
     zkAttnStacked attn(g, c.softmax_sf_in, 1UL, c.softmax_bs, c.softmax_L, c.softmax_M, c.softmax_thetas, seq, seq, d, 1);
@@ -214,7 +214,7 @@ static FrTensor attn_stacked_heads(const LayerConfig& c, const FrTensor& Q_, con
         attn.prove(Q, K, V, out, sm_out, sm_in, shift, shifted, in_seg, out_seg, m_seg, ch.u_matmul_out_num, ch.v_matmul_out_num, ch.u_matmul_out, ch.v_matmul_out,
                    ch.w_matmul_out, ch.v_sm, ch.temp_rand[0], ch.temp_rand[1], ch.temp_rand[2], ch.v_matmul_in_num, ch.v_matmul_in, proof);
     }
-    return outs.transpose_stack(H, seq, d).transpose(E, seq);   // [head][d][seq] = embed x seq -> seq x embed
+    return outs.swap_leading_axes(H, seq, d);   // [head][seq][d] -> seq x embed (= transpose_stack(H, seq, d).transpose(E, seq))
 }
 
 // All heads as ONE stack (attn_head_group == num_heads), in three steps.
@@ -229,7 +229,7 @@ AttnStackBlock::AttnStackBlock(const LayerConfig& c, const FrTensor& Q_, const F
 const FrTensor& AttnStackBlock::forward() {
     const uint seq = c.seq_len, E = c.embed_dim, H = c.num_heads, d = E / H;
     // seq x embed -> embed x seq = [head][d][seq] -> [head][seq][d]
-    auto to_stack = [&](const FrTensor& t) { return t.transpose(seq, E).transpose_stack(H, d, seq); };
+    auto to_stack = [&](const FrTensor& t) { return t.swap_leading_axes(seq, H, d); };          // = t.transpose(seq, E).transpose_stack(H, d, seq)
     Qs.emplace(to_stack(Q_));
     Ks.emplace(to_stack(K_));
     Vs.emplace(to_stack(V_));
@@ -242,7 +242,7 @@ const FrTensor& AttnStackBlock::forward() {
         FrTensor shifted(0);
         out.emplace(attn.compute(*Qs, *Ks, *Vs, *sm_in, *sm_out, *shift, shifted, in_seg, out_seg, m_seg));
     }
-    out_all.emplace(out->transpose_stack(H, seq, d).transpose(E, seq));   // [head][d][seq] = embed x seq -> seq x embed
+    out_all.emplace(out->swap_leading_axes(H, seq, d));   // [head][seq][d] -> seq x embed (= transpose_stack(H, seq, d).transpose(E, seq))
     out_.emplace(rs2(*out_all));
     out__.emplace(rs1(*out_));
     return *out__;
