@@ -197,6 +197,8 @@ int zk_fr_matmul_batched_prod(void* C, const void* a_ints, const void* b_ints, c
  * that: *taken_host is 1 when it ran, 0 when the operands or the shape do not allow it -- nothing is written then and the caller
  * falls back to zk_fr_matmul_batched.  No counterpart in the reference (zkAttn::compute, zksoftmax.cu:237-243, writes field elements). */
 int zk_fr_matmul_batched_i64(void* C64, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int* taken_host, void* stream);
+/* the same with the right operand given transposed (Bt[b][p][k] = B[b][k][p], batch * P * N elements): Q K^T straight from K */
+int zk_fr_matmul_batched_i64_bt(void* C64, const void* A, const void* Bt, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int* taken_host, void* stream);
 /* The right operand of many products (a layer's weight in zkFC::operator(), zkfc.cu:44-58) examined once: its largest magnitude
  * for the small-integer bound and, when it holds small integers, its int8 digit planes in the GEMM's layout.  No counterpart in
  * the reference, which converts nothing.  B stays alive and unmodified while the handle is used; zk_fr_matmul_rhs is

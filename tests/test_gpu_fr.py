@@ -640,6 +640,44 @@ def test_a_product_of_two_int32_tensors_multiplies_and_folds_without_being_writt
         pv.partial_me_prod(hA, hC, u, M, N)
 
 
+def test_products_written_as_64_bit_integers(monkeypatch):
+    """zk_fr_matmul_batched_i64 / _bt (the attention scores Q K^T for the pass that shifts and decomposes them): the matrix-core
+    path's products as int64 against numpy, the right operand given either way round; a product the path does not take (operands
+    of full width, or too few multiply-adds for it) reports 0 and writes nothing."""
+    from gpuhelp import Hip, c_void_p, c_uint, c_int
+    hip = Hip()
+    rng = np.random.default_rng(64)
+    num, M, N, P = 3, 70, 24, 90
+    A = rng.integers(-2 ** 17, 2 ** 17, (num, M, N)).astype(np.int64)
+    B = rng.integers(-2 ** 17, 2 ** 17, (num, N, P)).astype(np.int64)
+    A[0, 0, :2], B[0, :2, 0] = [2 ** 17 - 1, -2 ** 17], [-2 ** 17, 2 ** 17 - 1]
+    want = np.stack([A[i] @ B[i] for i in range(num)])
+    dA = hip.upload(fr_array([int(v) % R_MOD for v in A.reshape(-1)]))
+    dB = hip.upload(fr_array([int(v) % R_MOD for v in B.reshape(-1)]))
+    dBt = hip.upload(fr_array([int(v) % R_MOD for v in B.transpose(0, 2, 1).reshape(-1)]))
+    dC = hip.malloc(8 * num * M * P)
+    taken = ctypes.c_int(-1)
+    monkeypatch.setenv("ZKLLM_MATMUL_PLANES", "1")
+    for name, b in (("zk_fr_matmul_batched_i64", dB), ("zk_fr_matmul_batched_i64_bt", dBt)):
+        hip.lib.zk_memset(c_void_p(dC), c_int(0x5A), ctypes.c_size_t(8 * num * M * P), None)
+        hip.call(name, c_void_p(dC), c_void_p(dA), c_void_p(b), c_uint(num), c_uint(M), c_uint(N), c_uint(P), ctypes.byref(taken), None)
+        assert taken.value == 1, name
+        assert (hip.download(dC, (num, M, P), np.int64) == want).all(), name
+    # below the threshold of the matrix-core path: not taken, nothing written
+    monkeypatch.setenv("ZKLLM_MATMUL_PLANES", "40")
+    hip.lib.zk_memset(c_void_p(dC), c_int(0x5A), ctypes.c_size_t(8 * num * M * P), None)
+    hip.call("zk_fr_matmul_batched_i64", c_void_p(dC), c_void_p(dA), c_void_p(dB), c_uint(num), c_uint(M), c_uint(N), c_uint(P), ctypes.byref(taken), None)
+    assert taken.value == 0
+    assert (hip.download(dC, (num * M * P,), np.uint64) == 0x5A5A5A5A5A5A5A5A).all()
+    # a left operand of full-width residues: no small-integer bound, not taken
+    monkeypatch.setenv("ZKLLM_MATMUL_PLANES", "1")
+    dAf = hip.upload(mt_random_vec(np.random.RandomState(3), num * M * N))
+    hip.call("zk_fr_matmul_batched_i64_bt", c_void_p(dC), c_void_p(dAf), c_void_p(dBt), c_uint(num), c_uint(M), c_uint(N), c_uint(P), ctypes.byref(taken), None)
+    assert taken.value == 0
+    for p in (dA, dB, dBt, dC, dAf):
+        hip.free(p)
+
+
 def test_config2_full_size_fully_connected_proof_passes_the_verifier(pv):
     """X 2048 x 4096 times W 4096 x 4096 (fixed point, scale 2^16, N(0, 0.02)), beyond what the oracle can follow: rows
     of the product are compared with int64 arithmetic, and the proof transcript under a seeded stream is checked as a

@@ -620,7 +620,8 @@ static int digits_for(unsigned long long absmax) {      // planes needed for |x|
 // small integers, its digit planes in the GEMM's layout -- neither is computed again per product.
 struct MatmulRhs { const void* B = nullptr; uint32_t N = 0, P = 0, Kp = 0; unsigned long long mb = ~0ull; int pb = 0; void* planes = nullptr; };
 static int run_int8_plane_path(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, unsigned long long ma, unsigned long long mb,
-                               hipStream_t st, bool* done, const MatmulRhs* rhs = nullptr, ProdSrc src = ProdSrc{nullptr, nullptr}, long long* C64 = nullptr) {
+                               hipStream_t st, bool* done, const MatmulRhs* rhs = nullptr, ProdSrc src = ProdSrc{nullptr, nullptr}, long long* C64 = nullptr,
+                               bool b_transposed = false) {
     *done = false;
     const int pa = digits_for(ma), pb = digits_for(mb);
     if (!pa || !pb) return 0;
@@ -633,7 +634,10 @@ static int run_int8_plane_path(void* C, const void* A, const void* B, uint32_t b
     if (pla.rc) return pla.rc;
     if (plb.rc) return plb.rc;
     hipLaunchKernelGGL(k_split_rows, dim3(cdiv(rows_a * (Kp / 4), 256)), dim3(256), 0, st, pla.as<int8_t>(), (const Fr*)A, src, rows_a, M, N, Kp, pa);
-    if (!have_b) hipLaunchKernelGGL(k_split_cols, dim3(cdiv(P, 64), Kp / 64, batch), dim3(256), 0, st, plb.as<int8_t>(), (const Fr*)B, N, P, Kp, pb);
+    // a right operand given transposed ([batch][P][N]) has its planes' layout already: its rows are split like the left operand's
+    if (!have_b && b_transposed)
+        hipLaunchKernelGGL(k_split_rows, dim3(cdiv((size_t)batch * P * (Kp / 4), 256)), dim3(256), 0, st, plb.as<int8_t>(), (const Fr*)B, ProdSrc{nullptr, nullptr}, (size_t)batch * P, P, N, Kp, pb);
+    else if (!have_b) hipLaunchKernelGGL(k_split_cols, dim3(cdiv(P, 64), Kp / 64, batch), dim3(256), 0, st, plb.as<int8_t>(), (const Fr*)B, N, P, Kp, pb);
     const PlaneGemm g{pla.as<int8_t>(), have_b ? (const int8_t*)rhs->planes : plb.as<int8_t>(), (Fr*)C, M, P, Kp, pa, pb, C64};
     hipEvent_t t0 = nullptr, t1 = nullptr;
     if (g_gemm_timer.on) {
@@ -677,7 +681,7 @@ int zk_fr_matmul_generic(void* C, const void* A, const void* B, uint32_t M, uint
 // src.a set: the left operand is the elementwise product of two int32 forms and A is null; the paths that need field elements
 // get them written out first
 static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int mode, int* path_used, void* stv,
-                           const MatmulRhs* rhs = nullptr, ProdSrc src = ProdSrc{nullptr, nullptr}, long long* C64 = nullptr) {
+                           const MatmulRhs* rhs = nullptr, ProdSrc src = ProdSrc{nullptr, nullptr}, long long* C64 = nullptr, bool b_transposed = false) {
     // C64 set: only the matrix-core path writes it; *path_used is 0 and nothing is written when that path does not apply
     hipStream_t st = (hipStream_t)stv;
     std::unique_ptr<Scratch> a_written;
@@ -738,7 +742,7 @@ static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch
     const int planes_log2 = planes_env ? atoi(planes_env) : 30;
     if (planes_log2 > 0 && (unsigned __int128)batch * M * N * P >= ((unsigned __int128)1 << planes_log2) && M >= 32 && P >= 32) {
         bool done = false;
-        const int rc = run_int8_plane_path(C, A, B, batch, M, N, P, ma_, mb_, st, &done, rhs, src, C64);
+        const int rc = run_int8_plane_path(C, A, B, batch, M, N, P, ma_, mb_, st, &done, rhs, src, C64, b_transposed);
         if (rc) return rc;
         if (done) return 0;
     }
@@ -837,6 +841,14 @@ int zk_fr_matmul_batched_i64(void* C64, const void* A, const void* B, uint32_t b
     ZK_ARG(C64 != nullptr && taken_host != nullptr, "zk_fr_matmul_batched_i64: null argument");
     int path = 0;
     const int rc = matmul_dispatch(nullptr, A, B, batch, M, N, P, 0, &path, stv, nullptr, ProdSrc{nullptr, nullptr}, (long long*)C64);
+    *taken_host = (rc == 0 && path == 2) ? 1 : 0;
+    return rc;
+}
+// the same with the right operand given transposed (Bt: batch * P * N elements, Bt[b][p][k] = B[b][k][p]): Q K^T straight from K
+int zk_fr_matmul_batched_i64_bt(void* C64, const void* A, const void* Bt, uint32_t batch, uint32_t M, uint32_t N, uint32_t P, int* taken_host, void* stv) {
+    ZK_ARG(C64 != nullptr && taken_host != nullptr, "zk_fr_matmul_batched_i64_bt: null argument");
+    int path = 0;
+    const int rc = matmul_dispatch(nullptr, A, Bt, batch, M, N, P, 0, &path, stv, nullptr, ProdSrc{nullptr, nullptr}, (long long*)C64, true);
     *taken_host = (rc == 0 && path == 2) ? 1 : 0;
     return rc;
 }

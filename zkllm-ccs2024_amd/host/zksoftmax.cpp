@@ -273,8 +273,7 @@ FrTensor zkAttnStacked::compute(const FrTensor& Q, const FrTensor& K, const FrTe
         if (lean_forward && !(e && e[0] == '0') && !(chk && chk[0] == '1') && count % 4 == 0) {
             scores_i64.reset(new FrTensor((uint)(count / 4)));
             int taken = 0;
-            FrTensor Kt = K.transpose_stack(num, n, d);
-            ZKC(zk_fr_matmul_batched_i64(scores_i64->gpu_data, Q.gpu_data, Kt.gpu_data, num, m, d, n, &taken, nullptr));
+            ZKC(zk_fr_matmul_batched_i64_bt(scores_i64->gpu_data, Q.gpu_data, K.gpu_data, num, m, d, n, &taken, nullptr));      // K is (K^T)^T: no transpose
             if (!taken) scores_i64.reset();
         }
     }
