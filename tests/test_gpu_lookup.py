@@ -305,8 +305,13 @@ def test_rescaling_whose_remainders_exist_as_int32_only(pv, orc, n, sf):
     assert t.shape == e_t.shape and (t == e_t).all()
 
 
-def test_rescaling_prove_seeded_transcript(pv, orc):
-    for n, sf in ((256, 16), (5000, 1 << 8)):
+def test_rescaling_prove_seeded_transcript(pv, orc, monkeypatch):
+    """The proof's first entry, X(u), is formed from X_(u) and rem(u) (X = sf X_ + rem element by element); the oracle evaluates X
+    itself, and so does the prover in the runs with ZKLLM_CHECK_CLAIMS=1, which throw if the two differ."""
+    for n, sf, check in ((256, 16, False), (5000, 1 << 8, False), (256, 16, True), (70000, 1 << 8, True)):
+        monkeypatch.delenv("ZKLLM_CHECK_CLAIMS", raising=False)
+        if check:
+            monkeypatch.setenv("ZKLLM_CHECK_CLAIMS", "1")
         x = np.random.default_rng(n).integers(-(1 << 30), 1 << 30, n)
         X = fr_array([int(v) % R_MOD for v in x])
         orc.orc_seed(99)

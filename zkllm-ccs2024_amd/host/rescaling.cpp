@@ -1,5 +1,7 @@
 #include "rescaling.hpp"
 
+#include <cstdlib>
+
 #include "../../include/zkllm_hip.h"
 
 #define ZKC(call) zk_check((call), #call)
@@ -72,12 +74,15 @@ Rescaling::Pending Rescaling::prove_begin(const FrTensor& X, const FrTensor& X_,
         p.rem = padded;
     }
     p.m.reset(new FrTensor(tl_rem.prep(*p.rem)));
-    // X(u), X_(u), rem(u): one pass over the three tensors
-    vector<Fr_t> ev;
-    // (the padding of the remainders is zeros: the unpadded tensor has the same extension and the others' length)
-    ev = FrTensor::me_batch({&X, &X_, rem_tensor_ptr}, u);
-    p.lhs = ev[0];
-    if (p.lhs != ev[1] * Fr_t({scaling_factor, 0, 0, 0, 0, 0, 0, 0}) + ev[2]) throw std::runtime_error("Error: the rem is not correct.");
+    // X_(u) and rem(u) in one pass over the two tensors (the padding of the remainders is zeros: the unpadded tensor has the same
+    // extension and the others' length).  X = scaling_factor X_ + rem element by element, so X(u) is that combination of the two
+    // values: X itself, 32 bytes an element, is read only with ZKLLM_CHECK_CLAIMS=1, which evaluates it and compares as
+    // rescaling.cu:52-57 does.
+    const char* check_env = getenv("ZKLLM_CHECK_CLAIMS");
+    const bool read_X = check_env && check_env[0] == '1';
+    vector<Fr_t> ev = read_X ? FrTensor::me_batch({&X_, rem_tensor_ptr, &X}, u) : FrTensor::me_batch({&X_, rem_tensor_ptr}, u);
+    p.lhs = ev[0] * Fr_t({scaling_factor, 0, 0, 0, 0, 0, 0, 0}) + ev[1];
+    if (read_X && p.lhs != ev[2]) throw std::runtime_error("Error: the rem is not correct.");
     p.look = tl_rem.prove_begin(*p.rem, *p.m, rand_temp[0], rand_temp[1], u, v);
     return p;
 }
