@@ -572,7 +572,7 @@ FrTensor llama_layer(const LayerConfig& c, const LayerWeights& w, const FrTensor
         }
     };
     int blocks_begun = 0;
-    static const int start_openings_behind = [] { const char* e = getenv("ZKLLM_OPEN_START_BLOCK"); return e ? atoi(e) : 1; }();
+    static const int start_openings_behind = [] { const char* e = getenv("ZKLLM_OPEN_START_BLOCK"); return e ? atoi(e) : 2; }();
     auto begun = [&](std::function<void()> finish, double& slot) {      // call after the block's forward() and begin()
         owed.emplace_back(std::move(finish), &slot);
         if (++blocks_begun == start_openings_behind) zk_openings_start_now();
