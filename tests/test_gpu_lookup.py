@@ -947,10 +947,14 @@ def test_evaluations_of_eight_tensors_that_keep_only_their_int32_form():
         hip.free(d)
 
 
+@pytest.mark.parametrize("radices", [(256, 1 << 20, 1 << 20), (100, 1000003, 999983), (7, 1 << 20, 65537)])
 @pytest.mark.parametrize("rows,cols", [(5, 64), (37, 200), (64, 2048)])
-def test_softmax_shift_and_decomposition_in_one_pass_equal_the_two_passes(rows, cols):
+def test_softmax_shift_and_decomposition_in_one_pass_equal_the_two_passes(rows, cols, radices):
     """zk_softmax_shift_decompose against zk_softmax_shift followed by zk_softmax_decompose_ints: the same shifts, shifted
-    scores, digit planes and int32 planes (ragged rows: 200 columns are three full wave steps and a partial one)."""
+    scores, digit planes and int32 planes (ragged rows: 200 columns are three full wave steps and a partial one).  The one pass
+    forms the digits from 64-bit integers (a radix that is a power of two by mask and shift, any other by division), the two
+    passes from the field elements; radices of both kinds, mixed.  The scores as 64-bit integers
+    (zk_softmax_shift_decompose_i64) give the same again, and the digits recombine to the negated shifted scores."""
     import ctypes
     from gpuhelp import Hip, c_void_p, c_size_t, c_int
     from ctypes import c_uint, c_double
@@ -960,15 +964,18 @@ def test_softmax_shift_and_decomposition_in_one_pass_equal_the_two_passes(rows, 
     scale = 65536.0 * 8.0
     X = rng.integers(-(1 << 22), 1 << 22, n).astype(np.int64)
     dX = hip.upload(fr_array([int(v) % R_MOD for v in X]))
-    bs = np.array([256, 1 << 20, 1 << 20], dtype=np.uint32)
+    bs = np.array(radices, dtype=np.uint32)
+    dX64 = hip.upload(X)
     out = []
-    for fused in (False, True):
+    for fused in (False, True, "i64"):
         dShift, dXs = hip.malloc(32 * rows), hip.malloc(32 * n)
         planes = [hip.malloc(32 * n) for _ in range(3)]
         ints = [hip.malloc(4 * n) for _ in range(3)]
         arr = (c_void_p * 3)(*[c_void_p(x) for x in planes])
         iarr = (c_void_p * 3)(*[c_void_p(x) for x in ints])
-        if fused:
+        if fused == "i64":
+            hip.call("zk_softmax_shift_decompose_i64", c_void_p(dShift), c_void_p(dXs), arr, iarr, c_void_p(dX64), c_uint(rows), c_uint(cols), c_double(scale), bs, c_int(3), None)
+        elif fused:
             hip.call("zk_softmax_shift_decompose", c_void_p(dShift), c_void_p(dXs), arr, iarr, c_void_p(dX), c_uint(rows), c_uint(cols), c_double(scale), bs, c_int(3), None)
         else:
             hip.call("zk_softmax_shift", c_void_p(dShift), c_void_p(dXs), c_void_p(dX), c_uint(rows), c_uint(cols), c_double(scale), None)
@@ -977,10 +984,18 @@ def test_softmax_shift_and_decomposition_in_one_pass_equal_the_two_passes(rows, 
                    + [hip.download(q, (n,), np.int32) for q in ints])
         for q in [dShift, dXs] + planes + ints:
             hip.free(q)
-    for a, b in zip(out[0], out[1]):
-        assert (a == b).all()
+    for other in out[1:]:
+        for a, b in zip(out[0], other):
+            assert (a == b).all()
     assert out[0][2].any() and out[0][5].any()
+    # the digits are those of shift - score: d0 + b0 (d1 + b1 d2)
+    shift = np.array([v if v < R_MOD // 2 else v - R_MOD for v in fr_ints(out[0][0])], dtype=np.int64)
+    neg = np.repeat(shift, cols) - X
+    d0, d1, d2 = (out[0][5 + k].astype(np.int64) for k in range(3))
+    assert (d0 + int(bs[0]) * (d1 + int(bs[1]) * d2) == neg).all()
+    assert (d0 >= 0).all() and (d0 < int(bs[0])).all() and (d1 < int(bs[1])).all() and (d2 < int(bs[2])).all()
     hip.free(dX)
+    hip.free(dX64)
 
 
 @pytest.mark.parametrize("k", [13, 17, 19])

@@ -1500,6 +1500,33 @@ __device__ __forceinline__ void softmax_digits(const PlanePtrs& planes, const In
     }
     if (tmp != 0) atomicOr(flag, 2u);   // more digits than the radices cover
 }
+// the same from the non-negative integer itself (negative: the shifted score was positive, the flag's first bit as above); a
+// radix that is a power of two -- the same for every lane -- takes its digit by mask and shift instead of a 64-bit division
+__device__ __forceinline__ void softmax_digits_u64(const PlanePtrs& planes, const IntPlanePtrs& ints, uint32_t* __restrict__ flag, bool negative, unsigned long long tmp,
+                                                   const U32Pack8& bs, int K, size_t g) {
+    if (negative) {
+        atomicOr(flag, 1u);
+        for (int k = 0; k < K; ++k) {
+            if (planes.p[k]) planes.p[k][g] = big_zero<8>();
+            if (ints.p[k]) ints.p[k][g] = 0;
+        }
+        return;
+    }
+    for (int k = 0; k < K; ++k) {
+        const uint32_t b = bs.v[k];
+        unsigned long long digit;
+        if ((b & (b - 1u)) == 0u) {
+            digit = tmp & (unsigned long long)(b - 1u);
+            tmp >>= (31 - __builtin_clz(b));
+        } else {
+            digit = tmp % b;
+            tmp /= b;
+        }
+        if (planes.p[k]) planes.p[k][g] = fr_from_u64(digit);
+        if (ints.p[k]) ints.p[k][g] = (int32_t)digit;
+    }
+    if (tmp != 0) atomicOr(flag, 2u);   // more digits than the radices cover
+}
 static constexpr int SHIFT_ROW_CACHE = 2048;
 // K > 0: the shifted scores are decomposed where they are written (k_softmax_decompose's planes without its pass over them)
 // X64 set: the scores are given as 64-bit integers (a matrix product written in that form) and X is not read
@@ -1553,7 +1580,15 @@ __global__ void __launch_bounds__(TPB) k_softmax_shift(Fr* __restrict__ shift, F
     if (lane == 0) shift[row] = sh;
     Fr* orow = out + (size_t)row * cols;
     for (uint32_t j = lane; j < cols; j += 64) {
-        const Fr xs = sub(cached ? fr_from_i64(cache[w][j]) : (xr64 ? fr_from_i64(xr64[j]) : xr[j]), sh);
+        if (cached || xr64) {
+            // the score as an integer: its shifted value and the digits of the negative from 64-bit arithmetic
+            const int64_t xi = cached ? cache[w][j] : xr64[j];
+            if (out) orow[j] = sub(fr_from_i64(xi), sh);
+            const int64_t d = si - xi;
+            if (K > 0) softmax_digits_u64(planes, ints, flag, d < 0, (unsigned long long)d, bs, K, (size_t)row * cols + j);
+            continue;
+        }
+        const Fr xs = sub(xr[j], sh);
         if (out) orow[j] = xs;
         if (K > 0) softmax_digits(planes, ints, flag, xs, bs, K, (size_t)row * cols + j);
     }
