@@ -24,7 +24,7 @@ def ch(seed, n):
     return mt_random_vec(np.random.RandomState(seed), n)
 
 
-@pytest.mark.parametrize("n,sf", [(1, 16), (1000, 16), (4096, 1 << 16), (70000, 1 << 20)])
+@pytest.mark.parametrize("n,sf", [(1, 16), (1000, 16), (4096, 1 << 16), (70000, 1 << 20), (5000, 1000), (300, 3), (70000, 65537), (100, 1), (100, 2)])
 def test_rescale(pv, orc, n, sf):
     rng = np.random.default_rng(n)
     x = rng.integers(-(1 << 40), 1 << 40, n)

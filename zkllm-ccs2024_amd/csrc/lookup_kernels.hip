@@ -1438,9 +1438,15 @@ __global__ void __launch_bounds__(TPB) k_rescale(Fr* __restrict__ out, Fr* __res
     if (i >= n) return;
     const int64_t hsf = sf >> 1;
     const int64_t x = fr_to_i64(in[i]);
-    const int64_t temp = (x + hsf) % sf;
-    const int64_t x_rem = (temp < 0 ? temp + sf : temp) - hsf;
-    const int64_t x_rescaled = (x - x_rem) / sf;
+    int64_t x_rem, x_rescaled;
+    if ((sf & (sf - 1)) == 0) {          // a power of two (the same for every lane): the non-negative residue by mask, the exact quotient by shift
+        x_rem = ((x + hsf) & (sf - 1)) - hsf;
+        x_rescaled = (x - x_rem) >> (63 - __builtin_clzll((unsigned long long)sf));
+    } else {
+        const int64_t temp = (x + hsf) % sf;
+        x_rem = (temp < 0 ? temp + sf : temp) - hsf;
+        x_rescaled = (x - x_rem) / sf;
+    }
     out[i] = fr_from_i64(x_rescaled);
     if (rem) rem[i] = fr_from_i64(x_rem);
     if (rem_ints) rem_ints[i] = (int32_t)x_rem;
