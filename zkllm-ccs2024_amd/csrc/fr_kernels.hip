@@ -552,18 +552,18 @@ int zk_fr_transpose_batched(void* out, const void* in, uint32_t batch, uint32_t 
 int zk_fr_transpose(void* out, const void* in, uint32_t M, uint32_t N, void* st) { return zk_fr_transpose_batched(out, in, 1, M, N, st); }
 // out[b][a][c] = in[a][b][c]: the leading two axes of a three-axis tensor swapped, rows of C elements moved whole (what two
 // transposes do to bring [token][head][k] to [head][token][k] and back, in one pass)
+// a workgroup per output row (b, a): the row's position is worked out once, by the scalar unit, and the lanes move its 16-byte words
 __global__ void __launch_bounds__(TPB) k_swap_axes(uint4* __restrict__ out, const uint4* __restrict__ in, uint32_t A, uint32_t B, uint32_t Cw) {
-    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;          // a 16-byte word of the output
-    if (i >= (size_t)A * B * Cw) return;
-    const size_t w = i % Cw, ba = i / Cw, a = ba % A, b = ba / A;
-    out[i] = in[(a * B + b) * Cw + w];
+    const uint32_t ba = blockIdx.x, a = ba % A, b = ba / A;
+    const uint4* __restrict__ src = in + ((size_t)a * B + b) * Cw;
+    uint4* __restrict__ dst = out + (size_t)ba * Cw;
+    for (uint32_t w = threadIdx.x; w < Cw; w += TPB) dst[w] = src[w];
 }
 int zk_fr_swap_axes(void* out, const void* in, uint32_t A, uint32_t B, uint32_t C, void* st) {
     if (A == 0 || B == 0 || C == 0) return 0;
     ZK_ARG(out != in && out != nullptr && in != nullptr, "zk_fr_swap_axes: null or in-place");
-    const size_t words = (size_t)A * B * C * 2;
-    ZK_ARG(cdiv(words, TPB) <= 0x7FFFFFFFull, "zk_fr_swap_axes: too many elements for one launch");
-    hipLaunchKernelGGL(k_swap_axes, dim3((unsigned)cdiv(words, TPB)), dim3(TPB), 0, (hipStream_t)st, (uint4*)out, (const uint4*)in, A, B, C * 2);
+    ZK_ARG((size_t)A * B <= 0x7FFFFFFFull && C <= 0x7FFFFFFFu, "zk_fr_swap_axes: too many rows for one launch");
+    hipLaunchKernelGGL(k_swap_axes, dim3(A * B), dim3(TPB), 0, (hipStream_t)st, (uint4*)out, (const uint4*)in, A, B, C * 2);
     ZK_LAUNCH_CHECK();
     return 0;
 }

@@ -387,10 +387,21 @@ static constexpr int GLD = GBK + 16;                       // LDS row stride in 
 __global__ void __launch_bounds__(256) k_split_rows(int8_t* __restrict__ planes, const Fr* __restrict__ a, const ProdSrc src, size_t rows, uint32_t M, uint32_t N, uint32_t Kp, int np) {
     const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
     const uint32_t groups = Kp / 4;
-    const size_t row = gid / groups;
+    // 32-bit divisions where the launch has fewer than 2^32 lanes (the same for every lane; rows is below 2^31): a 64-bit
+    // division costs more than forming a plane's four digits
+    size_t row;
+    uint32_t k;
+    if (rows * (size_t)groups <= 0xFFFFFFFFull) {
+        const uint32_t g32 = (uint32_t)gid, r32 = g32 / groups;
+        row = r32;
+        k = 4 * (g32 - r32 * groups);
+    } else {
+        row = gid / groups;
+        k = 4 * (uint32_t)(gid % groups);
+    }
     if (row >= rows) return;
-    const uint32_t k = 4 * (uint32_t)(gid % groups);
-    const size_t b = row / M, m = row % M;
+    const uint32_t b32 = (uint32_t)row / M;
+    const size_t b = b32, m = (uint32_t)row - b32 * M;
     long long x[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) x[e] = (k + e < N) ? (src.a ? prod_at(src, row * N + k + e) : fr_to_i64(a[row * N + k + e])) : 0ll;
