@@ -674,6 +674,9 @@ def test_products_written_as_64_bit_integers(monkeypatch):
     dAf = hip.upload(mt_random_vec(np.random.RandomState(3), num * M * N))
     hip.call("zk_fr_matmul_batched_i64_bt", c_void_p(dC), c_void_p(dAf), c_void_p(dBt), c_uint(num), c_uint(M), c_uint(N), c_uint(P), ctypes.byref(taken), None)
     assert taken.value == 0
+    # a null operand is an argument error, not a launch
+    with pytest.raises(RuntimeError, match="null operand"):
+        hip.call("zk_fr_matmul_batched_i64", c_void_p(dC), None, c_void_p(dB), c_uint(num), c_uint(M), c_uint(N), c_uint(P), ctypes.byref(taken), None)
     for p in (dA, dB, dBt, dC, dAf):
         hip.free(p)
 

@@ -14,7 +14,7 @@
 //    nothing is assumed.  This is the case for every matmul of the LLaMa pipeline except softmax(Y)*V.
 //    Large products of this kind (the seven projections of a layer) are plain integer GEMMs and go to the matrix
 //    cores: both operands are split into balanced base-256 digits (int8 planes), every pair of planes is an int8 GEMM
-//    with int32 accumulation (rocBLAS, MFMA), planes of equal weight 2^(8s) accumulate into the same output, and one
+//    with int32 accumulation (k_gemm_i8_planes_all: v_mfma_i32_32x32x32_i8 tiles), planes of equal weight 2^(8s) accumulate into the same output, and one
 //    pass recombines the outputs in int64.  Exact: a dot product of digits stays below 2^31 (checked), the
 //    recombined value is the true integer result, below 2^62 by the bound above.
 #include <cstdlib>
@@ -708,6 +708,7 @@ static int matmul_dispatch(void* C, const void* A, const void* B, uint32_t batch
     };
     if (batch == 0 || M == 0 || P == 0) return 0;
     ZK_ARG(N > 0, "zk_fr_matmul: inner dimension is 0");
+    ZK_ARG((A != nullptr || src.a != nullptr) && B != nullptr && (C != nullptr || C64 != nullptr), "zk_fr_matmul: null operand or result");
     ZK_ARG(mode >= 0 && mode <= 2, "zk_fr_matmul: mode must be 0, 1 or 2");
     ZK_ARG(batch <= 65535, "zk_fr_matmul: at most 65535 products per call");
     ZK_ARG((size_t)batch * M < ((size_t)1 << 31), "zk_fr_matmul: too many rows in one call");
