@@ -506,9 +506,14 @@ def test_attention_forward_and_proof(pv, orc, monkeypatch, num, stacked, m, n, d
     # the second run (ZKLLM_CHECK_CLAIMS=1) evaluates the scores as well and throws if the two differ.
     # The third run of the lean variant lowers the matrix-core threshold so that the scores are written as 64-bit integers only
     # (zk_fr_matmul_batched_i64 -> zk_softmax_shift_decompose_i64; sm_in stays unwritten).
-    for check in ((False, True, "i64") if stacked == 2 else (False, True) if stacked else (False,)):
+    # The fourth run writes the softmax's output as a tensor (ZKLLM_SOFTMAX_PRODUCT=0) instead of leaving it the product of its
+    # two factors: the same bytes either way.
+    for check in ((False, True, "i64", "written") if stacked == 2 else (False, True) if stacked else (False,)):
         monkeypatch.delenv("ZKLLM_CHECK_CLAIMS", raising=False)
         monkeypatch.delenv("ZKLLM_MATMUL_PLANES", raising=False)
+        monkeypatch.delenv("ZKLLM_SOFTMAX_PRODUCT", raising=False)
+        if check == "written":
+            monkeypatch.setenv("ZKLLM_SOFTMAX_PRODUCT", "0")
         if check is True:
             monkeypatch.setenv("ZKLLM_CHECK_CLAIMS", "1")
         if check == "i64":
