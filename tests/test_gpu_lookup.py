@@ -512,6 +512,7 @@ def test_attention_forward_and_proof(pv, orc, monkeypatch, num, stacked, m, n, d
         monkeypatch.delenv("ZKLLM_CHECK_CLAIMS", raising=False)
         monkeypatch.delenv("ZKLLM_MATMUL_PLANES", raising=False)
         monkeypatch.delenv("ZKLLM_SOFTMAX_PRODUCT", raising=False)
+        monkeypatch.delenv("ZKLLM_SCORES_I64", raising=False)
         if check == "written":
             monkeypatch.setenv("ZKLLM_SOFTMAX_PRODUCT", "0")
         if check is True:
