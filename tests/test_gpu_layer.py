@@ -224,6 +224,19 @@ def test_full_shape_layer_gives_one_output_head_by_head_and_stacked(pv):
         again_t, again_g1 = pv.transcript(), pv.transcript_g1()
         assert again_t.shape == first_t.shape and (again_t == first_t).all(), at_claim
         assert again_g1.shape == first_g1.shape and first_g1.shape[0] > 9 * 30 and (again_g1 == first_g1).all(), at_claim
+    # The blocks, their sumcheck jobs and the openings run on streams and host threads of their own; a missing wait between them
+    # would show as a proof that changes from run to run.  Twelve more runs, every third with the openings at their claims.
+    for i in range(12):
+        pv.lib.zkp_openings_set_only_at_claim(1 if i % 3 == 2 else 0)
+        try:
+            pv.seed(5)
+            pv.transcript_begin()
+            out, _ = pv.layer_run(layer, X)
+            pv.lib.zkp_transcript_end()
+        finally:
+            pv.lib.zkp_openings_set_only_at_claim(0)
+        del out
+        assert (pv.transcript() == first_t).all() and (pv.transcript_g1() == first_g1).all(), i
     pv.layer_free(layer)
     assert (outs[0] == outs[1]).all() and (outs[0] == outs[2]).all()
     assert np.unique(outs[0], axis=0).shape[0] > 1000
