@@ -102,6 +102,11 @@ static inline unsigned reduce_grid(size_t n) {
     if (b < 1) b = 1;
     return (unsigned)b;
 }
+// the grid of a round that gives a lane `per_lane` pairs where the round has them: at least 64 workgroups, at most reduce_grid's
+static inline unsigned round_grid(size_t n, unsigned per_lane) {
+    const size_t all = reduce_grid(n), want = n / ((size_t)TPB * per_lane);
+    return (unsigned)std::min(all, std::max<size_t>(64, want));
+}
 // finish K sums (K x nb partials) and copy them to the host, applying the R correction (to_mont)
 // to the first `n_mont` of them
 static int finish_sums(Fr* partials, unsigned nb, int K, int n_mont, Fr* host_out, hipStream_t st) {
@@ -2610,7 +2615,11 @@ static int lookup_queue(SumJob& job, const Fr* A, const Fr* S, const Fr* B, cons
         Scratch& nx = job.arena.add(sizeof(Fr) * half * (phase2 ? 5 : 2));
         if (nx.rc) return nx.rc;
         Fr* w = nx.as<Fr>();
-        const unsigned nb = reduce_grid(half);
+        // A lane ends with a fixed tail -- its unreduced sums reduced, the workgroup's tree over five or eleven sums: what two to three
+        // pairs cost -- so a one-lane-per-pair round with a pair or two per lane pays it per pair.  Those rounds (not the first, whose
+        // grid the fused passes choose) take fewer lanes: eight pairs a lane in phase 1, four in phase 2, where the round has them.
+        unsigned nb = reduce_grid(half);
+        if (half > (size_t)SPLIT_HALF && !(r == 0 && fuse_first)) nb = round_grid(half, phase2 ? 4 : 8);
         const Fr vm = to_mont(load_fr(v + 8 * r));
         // the next round's eq table is written by this round's kernel (ping-pong between two buffers of the job)
         Fr* nE = nullptr;
